@@ -1,0 +1,355 @@
+"""CPU oracle for the gated delta rule (Gated DeltaNet) inference path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product package may import this
+module: it is the checker used by ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py``.  It is a restatement, in plain torch
+CPU ops, of the algorithm in the reference's files (paths relative to the
+reference checkout):
+
+* ``fla/ops/gated_delta_rule/naive.py:13-64``    token recurrence
+* ``fla/ops/gated_delta_rule/naive.py:67-161``   chunked form
+* ``fla/ops/gated_delta_rule/chunk.py:33-123``   stage order of the chunk pipeline
+* ``fla/ops/utils/cumsum.py:33-68``              chunk-local gate cumsum
+* ``fla/ops/gated_delta_rule/chunk_fwd.py:137-291``  gated beta*K*K^T and its unit-lower inverse
+* ``fla/ops/gated_delta_rule/wy_fast.py:72-106`` WY factors w, u
+* ``fla/ops/common/chunk_delta_h.py:174-348``    inter-chunk state recurrence
+* ``fla/ops/common/chunk_o.py:94-153``           output
+* ``fla/ops/gated_delta_rule/fused_recurrent.py:66-181``  decode recurrence and its flags
+* ``fla/ops/utils/index.py:113-172``             varlen chunk tables
+* ``fla/modules/l2norm.py:84-109``, ``fla/ops/gated_delta_rule/gate.py:21-46``  prologues
+* ``fla/utils/_testing.py:19-41``                error metric
+
+Parity pins (all in ``tests/test_oracle.py``): scalar brute force written as
+independent pure-python loops on tiny shapes, closed forms for one decode step
+(beta=0, exact projection), ``torch.linalg.inv`` for the triangular solve,
+recurrent == chunked, split-in-time hand-off, varlen == per-sequence loop,
+GVA == repeat_interleave, state_v_first == transpose, and the committed
+fixtures under ``tests/golden/``.  No function here is "parity unpinned".
+
+Everything is computed in ``dtype`` (float32 by default, float64 for tight
+pins); inputs are upcast first, so bf16 inputs are consumed as their exact
+rounded values.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+RCP_LN2 = 1.4426950216  # fla/ops/utils/constant.py:10
+
+
+# --------------------------------------------------------------------------- #
+# error metric (fla/utils/_testing.py:19-26)
+# --------------------------------------------------------------------------- #
+def get_abs_err(x: torch.Tensor, y: torch.Tensor) -> float:
+    return (x.detach().double() - y.detach().double()).flatten().abs().max().item()
+
+
+def get_err_ratio(x: torch.Tensor, y: torch.Tensor) -> float:
+    x, y = x.detach().double(), y.detach().double()
+    err = (x - y).flatten().square().mean().sqrt().item()
+    base = x.flatten().square().mean().sqrt().item()
+    return err / (base + 1e-8)
+
+
+def max_abs_ratio(ref: torch.Tensor, x: torch.Tensor) -> float:
+    """max|ref - x| / max|ref|, the second tolerance the build is held to."""
+    ref, x = ref.detach().double(), x.detach().double()
+    return (ref - x).abs().max().item() / (ref.abs().max().item() + 1e-12)
+
+
+# --------------------------------------------------------------------------- #
+# prologues
+# --------------------------------------------------------------------------- #
+def l2norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """x / sqrt(sum(x^2) + eps) over the last dim (fla/modules/l2norm.py:105-106)."""
+    xf = x.to(torch.float64 if x.dtype == torch.float64 else torch.float32)
+    return xf / torch.sqrt((xf * xf).sum(-1, keepdim=True) + eps)
+
+
+def gdn_gate(g: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor | None = None) -> torch.Tensor:
+    """g = -exp(A_log) * softplus(g + dt_bias) (fla/ops/gated_delta_rule/gate.py:21-46)."""
+    g = g.float()
+    if dt_bias is not None:
+        g = g + dt_bias.float()
+    return -A_log.float().exp() * F.softplus(g)
+
+
+# --------------------------------------------------------------------------- #
+# varlen chunk tables (fla/ops/utils/index.py:113-172), as plain loops
+# --------------------------------------------------------------------------- #
+def prepare_lens(cu_seqlens) -> list[int]:
+    cu = [int(x) for x in cu_seqlens]
+    return [b - a for a, b in zip(cu[:-1], cu[1:])]
+
+
+def prepare_chunk_indices(cu_seqlens, chunk_size: int) -> list[list[int]]:
+    """[[sequence id, chunk id inside that sequence], ...] in packed order."""
+    out = []
+    for n, L in enumerate(prepare_lens(cu_seqlens)):
+        for c in range((L + chunk_size - 1) // chunk_size):
+            out.append([n, c])
+    return out
+
+
+def prepare_chunk_offsets(cu_seqlens, chunk_size: int) -> list[int]:
+    """Exclusive prefix sum of per-sequence chunk counts, length N+1."""
+    out = [0]
+    for L in prepare_lens(cu_seqlens):
+        out.append(out[-1] + (L + chunk_size - 1) // chunk_size)
+    return out
+
+
+# --------------------------------------------------------------------------- #
+# token recurrence (naive.py:13-64 generalised to GVA / varlen / flags of
+# fused_recurrent.py:114-174)
+# --------------------------------------------------------------------------- #
+def _expand_heads(x: torch.Tensor, HV: int) -> torch.Tensor:
+    """GVA: q/k head h serves v heads h*G .. h*G+G-1 (i_h = i_hv // (HV // H),
+    fused_recurrent.py:69); same as repeat_interleave on the head dim."""
+    H = x.shape[2]
+    if H == HV:
+        return x
+    return x.repeat_interleave(HV // H, dim=2)
+
+
+def recurrent_gated_delta_rule(
+    q, k, v, g=None, beta=None, scale=None, initial_state=None, output_final_state=False,
+    cu_seqlens=None, gk=None, gv=None,
+    use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, A_log=None, dt_bias=None,
+    use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, state_v_first=False,
+    dtype=torch.float32,
+):
+    """Per token:  S *= exp(g);  v' = beta*(v - S^T k);  S += k v'^T;  o = S^T (q*scale).
+
+    q, k: [B,T,H,K]; v: [B,T,HV,V]; g, beta: [B,T,HV] (beta may be [B,T,HV,V]);
+    initial_state: [N,HV,K,V] ([N,HV,V,K] if state_v_first).  With cu_seqlens B
+    must be 1 and sequences are the packed slices.  Returns (o [B,T,HV,V] in
+    ``dtype``, final_state [N,HV,K,V] in ``dtype`` or None).
+    """
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if scale is None:
+        scale = K ** -0.5
+    qf, kf, vf = q.to(dtype), k.to(dtype), v.to(dtype)
+    if use_qk_l2norm_in_kernel:
+        qf = qf / torch.sqrt((qf * qf).sum(-1, keepdim=True) + 1e-6)
+        kf = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + 1e-6)
+    qf, kf = _expand_heads(qf, HV), _expand_heads(kf, HV)
+    if beta is None:
+        bf = torch.ones(B, T, HV, dtype=dtype)
+    else:
+        bf = beta.to(dtype)
+        if use_beta_sigmoid_in_kernel:
+            bf = torch.sigmoid(bf) * (2.0 if allow_neg_eigval else 1.0)
+    if bf.dim() == 3:
+        bf = bf[..., None]                      # headwise beta broadcasts over V
+    gf = None
+    if g is not None:
+        gf = gdn_gate(g, A_log, dt_bias).to(dtype) if use_gate_in_kernel else g.to(dtype)
+    gkf = gk.to(dtype) if gk is not None else None
+    gvf = gv.to(dtype) if gv is not None else None
+
+    if cu_seqlens is None:
+        bounds = [(b, 0, T) for b in range(B)]
+    else:
+        cu = [int(x) for x in cu_seqlens]
+        bounds = [(0, s, e) for s, e in zip(cu[:-1], cu[1:])]
+    N = len(bounds)
+    o = torch.zeros(B, T, HV, V, dtype=dtype)
+    ht = torch.zeros(N, HV, K, V, dtype=dtype)
+    for n, (b, s, e) in enumerate(bounds):
+        S = torch.zeros(HV, K, V, dtype=dtype)
+        if initial_state is not None:
+            S0 = initial_state[n].to(dtype)
+            S = S0.transpose(-1, -2).clone() if state_v_first else S0.clone()
+        for t in range(s, e):
+            if gf is not None:
+                S = S * gf[b, t].exp()[:, None, None]
+            if gkf is not None:
+                S = S * gkf[b, t].exp()[:, :, None]
+            if gvf is not None:
+                S = S * gvf[b, t].exp()[:, None, :]
+            kt, qt = kf[b, t], qf[b, t]                          # [HV,K]
+            vp = bf[b, t] * (vf[b, t] - torch.einsum('hkv,hk->hv', S, kt))
+            S = S + kt[:, :, None] * vp[:, None, :]
+            o[b, t] = torch.einsum('hkv,hk->hv', S, qt * scale)
+        ht[n] = S
+    if not output_final_state:
+        return o, None
+    return o, (ht.transpose(-1, -2).contiguous() if state_v_first else ht)
+
+
+# --------------------------------------------------------------------------- #
+# chunked form, stage by stage
+# --------------------------------------------------------------------------- #
+def chunk_local_cumsum(g: torch.Tensor, chunk_size: int, cu_seqlens=None, scale: float | None = None,
+                       reverse: bool = False) -> torch.Tensor:
+    """Inclusive prefix sum of g [B,T,HV] restarted at every chunk of every
+    sequence, optionally times ``scale`` (cumsum.py:33-68); fp32 result."""
+    B, T, HV = g.shape
+    out = torch.zeros(B, T, HV, dtype=torch.float32)
+    bounds = [(b, 0, T) for b in range(B)] if cu_seqlens is None else \
+        [(0, int(s), int(e)) for s, e in zip(cu_seqlens[:-1], cu_seqlens[1:])]
+    for b, s, e in bounds:
+        for c0 in range(s, e, chunk_size):
+            c1 = min(c0 + chunk_size, e)
+            seg = g[b, c0:c1].float()
+            cs = seg.flip(0).cumsum(0).flip(0) if reverse else seg.cumsum(0)
+            out[b, c0:c1] = cs * scale if scale is not None else cs
+    return out
+
+
+def chunk_stages_one_sequence(q, k, v, g, beta, scale, S0, chunk_size=64, dtype=torch.float32):
+    """Chunk pipeline for ONE sequence and ONE v-head group already expanded:
+    q,k [T,HV,K], v [T,HV,V], g,beta [T,HV], S0 [HV,K,V].  Returns a dict of every
+    intermediate (per chunk lists) plus o [T,HV,V] and final S.
+
+    Stage formulas (rows r of a chunk, G_r = cumsum(g)/ln2, gamma = 2^G):
+      L[i,j] = beta_i (k_i.k_j) 2^(G_i-G_j), i>j;  A=(I+L)^-1     chunk_fwd.py:137-291
+      u = A (beta*v);  w = A (beta*gamma*k)                        wy_fast.py:82-106
+      v_new = u - w S;  S <- gamma_last S + k^T (v_new*2^(G_last-G))   chunk_delta_h.py:210-315
+      o = scale[(q S) gamma + tril(q k^T 2^(G_i-G_j)) v_new]       chunk_o.py:107-153
+    """
+    T, HV, K = k.shape
+    V = v.shape[-1]
+    C = chunk_size
+    q, k, v, g, beta = (x.to(dtype) for x in (q, k, v, g, beta))
+    S = S0.to(dtype).clone()
+    o = torch.zeros(T, HV, V, dtype=dtype)
+    stages = dict(G=[], L=[], A=[], w=[], u=[], h=[], v_new=[])
+    for c0 in range(0, T, C):
+        c1 = min(c0 + C, T)
+        r = c1 - c0
+        kc, qc, vc = (x[c0:c1].transpose(0, 1) for x in (k, q, v))          # [HV,r,*]
+        bc = beta[c0:c1].transpose(0, 1)                                     # [HV,r]
+        G = g[c0:c1].transpose(0, 1).cumsum(-1) * RCP_LN2                    # [HV,r]
+        diff = G[:, :, None] - G[:, None, :]
+        strict = torch.ones(r, r, dtype=torch.bool).tril(-1)
+        incl = torch.ones(r, r, dtype=torch.bool).tril(0)
+        # mask BEFORE exponentiating so the upper triangle cannot overflow
+        dec_strict = torch.where(strict, torch.exp2(torch.where(strict, diff, torch.zeros_like(diff))), torch.zeros_like(diff))
+        dec_incl = torch.where(incl, torch.exp2(torch.where(incl, diff, torch.zeros_like(diff))), torch.zeros_like(diff))
+        L = bc[:, :, None] * (kc @ kc.transpose(-1, -2)) * dec_strict
+        eye = torch.eye(r, dtype=dtype).expand(HV, r, r)
+        A = torch.linalg.solve_triangular(eye + L, eye.clone(), upper=False, unitriangular=True)
+        gamma = torch.exp2(G)
+        u = A @ (vc * bc[:, :, None])
+        w = A @ (kc * (bc * gamma)[:, :, None])
+        v_new = u - w @ S
+        o_c = (qc @ S) * gamma[:, :, None] + ((qc @ kc.transpose(-1, -2)) * dec_incl) @ v_new
+        o[c0:c1] = (o_c * scale).transpose(0, 1)
+        stages['G'].append(G); stages['L'].append(L); stages['A'].append(A)
+        stages['w'].append(w); stages['u'].append(u); stages['h'].append(S.clone()); stages['v_new'].append(v_new)
+        g_last = G[:, -1]
+        S = S * torch.exp2(g_last)[:, None, None] + \
+            (kc * torch.exp2(g_last[:, None] - G)[:, :, None]).transpose(-1, -2) @ v_new
+    stages['o'] = o
+    stages['S'] = S
+    return stages
+
+
+def chunk_gated_delta_rule(
+    q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False,
+    cu_seqlens=None, chunk_size=64,
+    use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, A_log=None, dt_bias=None,
+    use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, state_v_first=False,
+    dtype=torch.float32, return_stages=False,
+):
+    """Chunked gated delta rule with the argument order of
+    fla/ops/gated_delta_rule/chunk.py:397-415 (q, k, v, g, beta).  Returns
+    (o [B,T,HV,V], final_state [N,HV,K,V] or None) in ``dtype``."""
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if scale is None:
+        scale = K ** -0.5
+    qf, kf, vf = q.to(dtype), k.to(dtype), v.to(dtype)
+    if use_qk_l2norm_in_kernel:
+        # chunk.py:279-282 normalises through l2norm_fwd, whose output keeps the input dtype
+        qf = l2norm(q).to(q.dtype).to(dtype)
+        kf = l2norm(k).to(k.dtype).to(dtype)
+    qf, kf = _expand_heads(qf, HV), _expand_heads(kf, HV)
+    bf = beta.to(dtype)
+    if use_beta_sigmoid_in_kernel:
+        bf = torch.sigmoid(bf) * (2.0 if allow_neg_eigval else 1.0)
+    gf = gdn_gate(g, A_log, dt_bias).to(dtype) if use_gate_in_kernel else g.to(dtype)
+
+    if cu_seqlens is None:
+        bounds = [(b, 0, T) for b in range(B)]
+    else:
+        cu = [int(x) for x in cu_seqlens]
+        bounds = [(0, s, e) for s, e in zip(cu[:-1], cu[1:])]
+    N = len(bounds)
+    o = torch.zeros(B, T, HV, V, dtype=dtype)
+    ht = torch.zeros(N, HV, K, V, dtype=dtype)
+    all_stages = []
+    for n, (b, s, e) in enumerate(bounds):
+        S0 = torch.zeros(HV, K, V, dtype=dtype)
+        if initial_state is not None:
+            S0 = initial_state[n].to(dtype)
+            if state_v_first:
+                S0 = S0.transpose(-1, -2)
+        st = chunk_stages_one_sequence(qf[b, s:e], kf[b, s:e], vf[b, s:e], gf[b, s:e], bf[b, s:e],
+                                       scale, S0, chunk_size, dtype)
+        o[b, s:e] = st['o']
+        ht[n] = st['S']
+        all_stages.append(st)
+    fs = None
+    if output_final_state:
+        fs = ht.transpose(-1, -2).contiguous() if state_v_first else ht
+    if return_stages:
+        return o, fs, all_stages
+    return o, fs
+
+
+# --------------------------------------------------------------------------- #
+# one decode step in closed form (used to pin the recurrence and as the CPU
+# baseline of the decode bench): S' = e^g S + k [beta (v - e^g S^T k)]^T, o = scale S'^T q
+# --------------------------------------------------------------------------- #
+def decode_step(q, k, v, g, beta, S, scale=None):
+    """q,k [N,H,K]; v [N,HV,V]; g,beta [N,HV]; S [N,HV,K,V] fp32.  Vectorised over
+    N and HV.  Returns (o [N,HV,V], S' [N,HV,K,V])."""
+    N, H, K = k.shape
+    HV = v.shape[1]
+    if scale is None:
+        scale = K ** -0.5
+    G = HV // H
+    qf = q.float().repeat_interleave(G, dim=1)
+    kf = k.float().repeat_interleave(G, dim=1)
+    S = S.float() * g.float().exp()[:, :, None, None]
+    vp = beta.float()[:, :, None] * (v.float() - torch.einsum('nhkv,nhk->nhv', S, kf))
+    S = S + kf[:, :, :, None] * vp[:, :, None, :]
+    o = torch.einsum('nhkv,nhk->nhv', S, qf * scale)
+    return o, S
+
+
+def make_inputs(B, T, H, HV, K, V, seed=42, gate_div=1.0, h0_std=None, N=None, dtype=torch.float32):
+    """Synthetic inputs in the order q,k,v,g,beta,h0 from one CPU generator:
+    q,k = normalize(randn), v = randn, g = logsigmoid(randn)/gate_div,
+    beta = sigmoid(randn), h0 = h0_std*randn or None.  q,k,v are cast to ``dtype``
+    (g, beta, h0 stay fp32)."""
+    gen = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1)
+    k = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1)
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / gate_div
+    beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
+    h0 = None
+    if h0_std is not None:
+        h0 = h0_std * torch.randn(N if N is not None else B, HV, K, V, generator=gen)
+    return q.to(dtype), k.to(dtype), v.to(dtype), g, beta, h0
+
+
+def make_varlen_lengths(total: int, n_seq: int, lo: int, hi: int, seed: int = 42) -> list[int]:
+    """Lengths ~ U[lo,hi] rescaled (floor) to sum to ``total``; the remainder is
+    handed out one token at a time to the first sequences."""
+    gen = torch.Generator().manual_seed(seed)
+    L = torch.randint(lo, hi + 1, (n_seq,), generator=gen).double()
+    L = torch.floor(L * total / L.sum()).long()
+    rem = total - int(L.sum())
+    for i in range(rem):
+        L[i % n_seq] += 1
+    assert int(L.sum()) == total and int(L.min()) >= 1
+    return [int(x) for x in L]

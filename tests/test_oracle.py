@@ -1,0 +1,206 @@
+"""Pins the CPU oracle (oracle/gdn_oracle.py) without running the reference:
+scalar fixtures, closed forms, library routines and algebraic invariants.
+Each check is chosen so that a plausible slip (dropped term, wrong sign/index,
+transposed operand, swapped g/beta) fails it."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'gdn_scalar_cases.npz'))
+CASES = ['single_T5', 'gva_T70_h0', 'varlen_h0']
+
+
+def _gold(name):
+    t = lambda key: torch.from_numpy(GOLD[f'{name}.{key}'])
+    cu = GOLD[f'{name}.cu'].tolist()
+    h0 = t('h0') if f'{name}.h0' in GOLD.files else None
+    return dict(q=t('q')[None], k=t('k')[None], v=t('v')[None], g=t('g')[None], beta=t('beta')[None],
+                h0=h0, cu=cu, scale=float(GOLD[f'{name}.scale']), o=t('o')[None], ht=t('ht'))
+
+
+@pytest.mark.parametrize('name', CASES)
+def test_recurrent_matches_scalar_fixture(name):
+    c = _gold(name)
+    o, ht = O.recurrent_gated_delta_rule(c['q'], c['k'], c['v'], c['g'], c['beta'], c['scale'], c['h0'], True,
+                                         cu_seqlens=c['cu'], dtype=torch.float64)
+    assert torch.allclose(o, c['o'], atol=1e-12, rtol=1e-10)
+    assert torch.allclose(ht, c['ht'], atol=1e-12, rtol=1e-10)
+
+
+@pytest.mark.parametrize('name', CASES)
+@pytest.mark.parametrize('chunk', [16, 64])
+def test_chunk_matches_scalar_fixture(name, chunk):
+    c = _gold(name)
+    o, ht = O.chunk_gated_delta_rule(c['q'], c['k'], c['v'], c['g'], c['beta'], c['scale'], c['h0'], True,
+                                     cu_seqlens=c['cu'], chunk_size=chunk, dtype=torch.float64)
+    # RCP_LN2 is the reference's fp32-rounded 1/ln2 (relative error 1.3e-8 in every exponent)
+    assert torch.allclose(o, c['o'], atol=1e-6, rtol=1e-6)
+    assert torch.allclose(ht, c['ht'], atol=1e-6, rtol=1e-6)
+
+
+def test_config1_recurrent_equals_chunk():
+    # BASELINE config 1: B=2 T=256 H=2 K=V=64 fp32, zero initial state
+    q, k, v, g, beta, _ = O.make_inputs(2, 256, 2, 2, 64, 64, seed=42)
+    o_r, h_r = O.recurrent_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    o_c, h_c = O.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    assert h_r.shape == (2, 2, 64, 64)
+    assert O.get_err_ratio(o_r, o_c) < 1e-4 and O.get_err_ratio(h_r, h_c) < 1e-4
+    o_d, h_d = O.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, dtype=torch.float64)
+    assert O.get_err_ratio(o_d, o_c) < 1e-5 and O.get_err_ratio(h_d, h_r) < 1e-5
+
+
+def test_one_step_closed_forms():
+    torch.manual_seed(0)
+    N, H, HV, K, V = 3, 2, 4, 8, 5
+    q = torch.randn(N, H, K, dtype=torch.float64)
+    k = F.normalize(torch.randn(N, H, K, dtype=torch.float64), dim=-1)
+    v = torch.randn(N, HV, V, dtype=torch.float64)
+    S = torch.randn(N, HV, K, V, dtype=torch.float64)
+    g = -torch.rand(N, HV, dtype=torch.float64)
+    beta = torch.rand(N, HV, dtype=torch.float64)
+    call = lambda g_, b_: O.recurrent_gated_delta_rule(q[:, None], k[:, None], v[:, None], g_[:, None], b_[:, None],
+                                                        1.0, S, True, dtype=torch.float64)
+    # beta = 0: pure decay, output reads the decayed state
+    o, S1 = call(g, torch.zeros_like(beta))
+    Sd = S * g.exp()[:, :, None, None]
+    assert torch.allclose(S1, Sd)
+    assert torch.allclose(o[:, 0], torch.einsum('nhkv,nhk->nhv', Sd, q.repeat_interleave(2, 1)))
+    # g = 0, beta = 1, |k| = 1: the state is overwritten so that S'^T k = v exactly
+    o, S1 = call(torch.zeros_like(g), torch.ones_like(beta))
+    assert torch.allclose(torch.einsum('nhkv,nhk->nhv', S1, k.repeat_interleave(2, 1)), v)
+    # general closed form  S' = e^g S + k [beta (v - e^g S^T k)]^T
+    o, S1 = call(g, beta)
+    kk = k.repeat_interleave(2, 1)
+    d = beta[..., None] * (v - torch.einsum('nhkv,nhk->nhv', Sd, kk))
+    assert torch.allclose(S1, Sd + kk[..., None] * d[:, :, None, :])
+    # decode_step helper is the same map (fp32)
+    o32, S32 = O.decode_step(q, k, v, g, beta, S, scale=1.0)
+    assert torch.allclose(S32.double(), S1, atol=1e-5) and torch.allclose(o32.double(), o[:, 0], atol=1e-5)
+
+
+def test_argument_order_is_g_then_beta_for_chunk():
+    # swapping g and beta must change the result (guards the (beta, g) vs (g, beta) slip)
+    q, k, v, g, beta, _ = O.make_inputs(1, 40, 1, 1, 4, 4, seed=3)
+    o1, _ = O.chunk_gated_delta_rule(q, k, v, g, beta)
+    o2, _ = O.chunk_gated_delta_rule(q, k, v, beta, g)
+    assert O.get_err_ratio(o1, o2) > 1e-2
+
+
+def test_T_steps_equal_chained_single_steps_and_split_handoff():
+    q, k, v, g, beta, h0 = O.make_inputs(2, 150, 2, 4, 16, 8, seed=5, h0_std=0.3)
+    o, ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True, dtype=torch.float64)
+    S = h0.double()
+    for t in range(150):
+        o_t, S = O.recurrent_gated_delta_rule(q[:, t:t + 1], k[:, t:t + 1], v[:, t:t + 1], g[:, t:t + 1], beta[:, t:t + 1],
+                                              initial_state=S, output_final_state=True, dtype=torch.float64)
+        assert torch.allclose(o_t[:, 0], o[:, t], atol=1e-12)
+    assert torch.allclose(S, ht, atol=1e-12)
+    # chunk op: split T at a non-multiple of the chunk size, hand the state over
+    oc, hc = O.chunk_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True, dtype=torch.float64)
+    o1, h1 = O.chunk_gated_delta_rule(q[:, :70], k[:, :70], v[:, :70], g[:, :70], beta[:, :70], initial_state=h0,
+                                      output_final_state=True, dtype=torch.float64)
+    o2, h2 = O.chunk_gated_delta_rule(q[:, 70:], k[:, 70:], v[:, 70:], g[:, 70:], beta[:, 70:], initial_state=h1,
+                                      output_final_state=True, dtype=torch.float64)
+    assert torch.allclose(torch.cat([o1, o2], 1), oc, atol=1e-10) and torch.allclose(h2, hc, atol=1e-10)
+    assert torch.allclose(oc, o, atol=1e-10) and torch.allclose(hc, ht, atol=1e-10)
+
+
+def test_varlen_equals_per_sequence_loop_and_gva_equals_repeat():
+    cu = [0, 15, 100, 300, 301, 520]
+    q, k, v, g, beta, h0 = O.make_inputs(1, 520, 2, 4, 8, 8, seed=7, h0_std=0.5, N=5)
+    for fn in (O.recurrent_gated_delta_rule, O.chunk_gated_delta_rule):
+        o, ht = fn(q, k, v, g, beta, initial_state=h0, output_final_state=True, cu_seqlens=cu, dtype=torch.float64)
+        for n, (s, e) in enumerate(zip(cu[:-1], cu[1:])):
+            o_n, h_n = fn(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e], initial_state=h0[n:n + 1],
+                          output_final_state=True, dtype=torch.float64)
+            assert torch.equal(o_n[0], o[0, s:e]) and torch.equal(h_n[0], ht[n])
+        qe, ke = q.repeat_interleave(2, 2), k.repeat_interleave(2, 2)
+        o_e, h_e = fn(qe, ke, v, g, beta, initial_state=h0, output_final_state=True, cu_seqlens=cu, dtype=torch.float64)
+        assert torch.equal(o_e, o) and torch.equal(h_e, ht)
+
+
+def test_state_v_first_is_a_transpose():
+    q, k, v, g, beta, h0 = O.make_inputs(2, 70, 1, 2, 8, 4, seed=9, h0_std=0.5)
+    for fn in (O.recurrent_gated_delta_rule, O.chunk_gated_delta_rule):
+        o, ht = fn(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+        o2, ht2 = fn(q, k, v, g, beta, initial_state=h0.transpose(-1, -2).contiguous(), output_final_state=True,
+                     state_v_first=True)
+        assert ht2.shape == (2, 2, 4, 8)
+        assert torch.equal(o, o2) and torch.equal(ht2.transpose(-1, -2), ht)
+
+
+def test_stages_solve_wy_and_scan_invariants():
+    q, k, v, g, beta, h0 = O.make_inputs(1, 150, 1, 2, 16, 8, seed=11, h0_std=0.5)
+    o, ht, st = O.chunk_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                         dtype=torch.float64, return_stages=True)
+    st = st[0]
+    assert [x.shape[-1] for x in st['G']] == [64, 64, 22]           # tail chunk is the leading r x r problem
+    kk = k.double().repeat_interleave(2, 2)[0]
+    for c, (L, A, G, w, u) in enumerate(zip(st['L'], st['A'], st['G'], st['w'], st['u'])):
+        r = L.shape[-1]
+        eye = torch.eye(r, dtype=torch.float64)
+        # library routine + definition: A (I+L) = I, unit lower triangular
+        assert torch.allclose(A, torch.linalg.inv(eye + L), atol=1e-10)
+        assert torch.allclose(A @ (eye + L), eye.expand_as(A), atol=1e-10)
+        assert torch.equal(A.triu(1), torch.zeros_like(A)) and torch.allclose(A.diagonal(dim1=-2, dim2=-1), torch.ones(2, r, dtype=torch.float64))
+        assert torch.equal(L.triu(0), torch.zeros_like(L))
+        # the row-by-row substitution of naive.py:129-131 gives the same inverse
+        attn = -L.clone()
+        for i in range(1, r):
+            attn[..., i, :i] = attn[..., i, :i] + (attn[..., i, :i, None] * attn[..., :i, :i]).sum(-2)
+        assert torch.allclose(attn + eye, A, atol=1e-10)
+        # cumsum closed form, restarted per chunk, in log2 units
+        gc = g[0, c * 64:c * 64 + r].double().transpose(0, 1)
+        assert torch.allclose(G, gc.cumsum(-1) / math.log(2), atol=1e-6)
+        # w,u plain definitions
+        b = beta[0, c * 64:c * 64 + r].double().transpose(0, 1)
+        kc = kk[c * 64:c * 64 + r].transpose(0, 1)
+        vc = v[0, c * 64:c * 64 + r].double().transpose(0, 1)
+        assert torch.allclose(u, A @ (vc * b[..., None]), atol=1e-12)
+        assert torch.allclose(w, A @ (kc * (b * torch.exp2(G))[..., None]), atol=1e-12)
+    assert torch.equal(st['h'][0], h0[0].double())                   # h[0] == h0
+    cs = O.chunk_local_cumsum(g, 64, scale=O.RCP_LN2)
+    assert torch.allclose(cs[0, :64].double(), st['G'][0].transpose(0, 1), atol=1e-5)
+    rev = O.chunk_local_cumsum(g, 64, reverse=True)
+    assert torch.allclose(rev[0, 128:150], g[0, 128:150].flip(0).cumsum(0).flip(0), atol=1e-6)
+
+
+def test_flags_equal_host_side_prologues():
+    torch.manual_seed(1)
+    B, T, H, HV, K, V = 1, 70, 2, 4, 8, 8
+    q, k, v = torch.randn(B, T, H, K), torch.randn(B, T, H, K), torch.randn(B, T, HV, V)
+    graw, braw = torch.randn(B, T, HV), torch.randn(B, T, HV)
+    A_log, dt_bias = torch.randn(HV) * 0.3, torch.randn(HV) * 0.3
+    for fn in (O.recurrent_gated_delta_rule, O.chunk_gated_delta_rule):
+        o1, h1 = fn(q, k, v, graw, braw, output_final_state=True, use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True,
+                    A_log=A_log, dt_bias=dt_bias, use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True)
+        gd = -A_log.exp() * F.softplus(graw + dt_bias)
+        o2, h2 = fn(O.l2norm(q), O.l2norm(k), v, gd, 2 * torch.sigmoid(braw), output_final_state=True)
+        assert O.get_err_ratio(o2, o1) < 1e-5 and O.get_err_ratio(h2, h1) < 1e-5
+    x = torch.randn(5, 7)
+    assert torch.allclose(O.l2norm(x), x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6))
+
+
+def test_index_tables():
+    cu = [0, 1, 65, 192, 193, 400]
+    idx = O.prepare_chunk_indices(cu, 64)
+    assert idx == [[0, 0], [1, 0], [2, 0], [2, 1], [3, 0], [4, 0], [4, 1], [4, 2], [4, 3]]
+    assert O.prepare_chunk_offsets(cu, 64) == [0, 1, 2, 4, 5, 9]
+    assert O.prepare_chunk_offsets([0, 64], 64) == [0, 1]
+
+
+def test_error_metric_definition():
+    x = torch.tensor([3.0, 4.0]); y = torch.tensor([3.0, 5.0])
+    assert abs(O.get_abs_err(x, y) - 1.0) < 1e-12
+    assert abs(O.get_err_ratio(x, y) - (math.sqrt(0.5) / (math.sqrt(12.5) + 1e-8))) < 1e-12
+
+
+def test_varlen_length_recipe():
+    L = O.make_varlen_lengths(65536, 32, 256, 4096, seed=42)
+    assert len(L) == 32 and sum(L) == 65536 and min(L) >= 1
