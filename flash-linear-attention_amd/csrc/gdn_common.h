@@ -1,0 +1,69 @@
+// Shared helpers for the gfx950 gated-delta-rule kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/gdn_hip.h"
+
+namespace gdn {
+
+void set_error(const char* fmt, ...);
+
+#define GDN_CHECK_ARG(cond, code, ...)            \
+    do {                                          \
+        if (!(cond)) {                            \
+            gdn::set_error(__VA_ARGS__);          \
+            return (code);                        \
+        }                                         \
+    } while (0)
+
+inline int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("%s: %s", what, hipGetErrorString(e));
+        return GDN_ERR_LAUNCH;
+    }
+    return GDN_OK;
+}
+
+// ---- element types -------------------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+// g/beta may arrive in any float type; they are tiny, so a run-time switch is enough.
+__device__ __forceinline__ float load_scalar(const void* p, int64_t i, int dtype) {
+    if (dtype == GDN_DTYPE_F32) return ((const float*)p)[i];
+    if (dtype == GDN_DTYPE_BF16) return (float)((const bf16_t*)p)[i];
+    return (float)((const f16_t*)p)[i];
+}
+
+__device__ __forceinline__ int64_t load_index(const void* p, int64_t i, bool is_i32) {
+    return is_i32 ? (int64_t)((const int32_t*)p)[i] : ((const int64_t*)p)[i];
+}
+
+__device__ __forceinline__ float softplus_f(float x) {
+    // log(1 + e^x) with the usual linear tail (torch threshold 20)
+    return x > 20.f ? x : log1pf(__expf(x));
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + __expf(-x)); }
+
+}  // namespace gdn

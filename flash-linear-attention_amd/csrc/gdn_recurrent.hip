@@ -1,0 +1,311 @@
+// Token recurrence of the gated delta rule (decode and short prompts) for gfx950.
+//
+//   S <- e^{g_t} S (and e^{gk}, e^{gv});  d = beta_t (v_t - S^T k_t);  S <- S + k_t d^T;  o_t = scale S^T q_t
+//
+// One workgroup of 256 threads owns the state of one (sequence, v-head) restricted to a
+// block of VB value columns (K-first layout [K,V]) or VB value rows (V-first layout
+// [V,K]).  The fp32 state lives in registers for the whole call: each thread holds R
+// float4 pieces, every global access is a 16-byte piece of a contiguous row, so one wave
+// instruction reads whole rows - the step is a pure HBM stream of the state (read once,
+// written once, in place if the caller aliases ht to h0).
+#include "gdn_common.h"
+
+namespace gdn {
+
+struct RecurrentParams {
+    const void* q; const void* k; const void* v;
+    const void* g; const void* beta; const float* gk; const float* gv;
+    const float* A_log; const float* dt_bias;
+    const float* h0; float* ht; void* o;
+    const void* cu_seqlens;
+    int64_t T; int H, HV, K, V, NVB;
+    float scale; int gb_dtype; uint32_t flags;
+};
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// KMAX: compile-time bound on K (rows padded with zeros), VB: value block per workgroup.
+template <typename T, int KMAX, int VB, bool VFIRST>
+__global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
+    // lanes along the contiguous dim (float4 each), the rest of the 256 threads along rows
+    constexpr int CONT = VFIRST ? KMAX : VB;        // extent of the contiguous dim handled
+    constexpr int TC = CONT / 4;                    // threads along the contiguous dim
+    constexpr int RP = 256 / TC;                    // rows per pass
+    constexpr int ROWS = VFIRST ? VB : KMAX;        // extent of the row dim handled
+    constexpr int R = (ROWS + RP - 1) / RP;         // float4 pieces per thread
+    static_assert(TC <= 64 && (TC & (TC - 1)) == 0, "contiguous extent must map to <= 64 lanes");
+
+    const int tid = threadIdx.x;
+    const int c = tid % TC, r0 = tid / TC;
+    const int wave = tid >> 6;
+    const int ivb = blockIdx.x % p.NVB;
+    const int64_t inh = blockIdx.x / p.NVB;
+    const int64_t in = inh / p.HV;
+    const int ihv = (int)(inh % p.HV);
+    const int ih = ihv / (p.HV / p.H);
+    const int K = p.K, V = p.V, H = p.H, HV = p.HV;
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+
+    int64_t bos, len;
+    if (p.cu_seqlens) {
+        bos = load_index(p.cu_seqlens, in, cu32);
+        len = load_index(p.cu_seqlens, in + 1, cu32) - bos;
+    } else {
+        bos = in * p.T;
+        len = p.T;
+    }
+    const int v0 = ivb * VB;                        // first value index of this block
+
+    // ---- state into registers (issued first: everything else hides behind these loads) ----
+    f32x4 S[R];
+    // K-first: row = k index, cont = v index.  V-first: row = v index, cont = k index.
+    const int cont_idx = (VFIRST ? 0 : v0) + 4 * c;
+    const int cont_lim = VFIRST ? K : V;
+    const int row_lim = VFIRST ? V : K;
+    const int row_base = VFIRST ? v0 : 0;
+    const int64_t row_stride = VFIRST ? K : V;
+    const bool cont_ok = cont_idx < cont_lim;
+    const int64_t state_off = inh * (int64_t)K * V;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int row = row_base + r0 + RP * i;
+        const bool ok = cont_ok && (r0 + RP * i < ROWS) && row < row_lim;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        if (ok && p.h0) s = __builtin_nontemporal_load((const f32x4*)(p.h0 + state_off + row * row_stride + cont_idx));
+        S[i] = s;
+    }
+
+    __shared__ float sh_q[2][KMAX], sh_k[2][KMAX];
+    __shared__ float sh_red[2][4][4];                       // per-wave partial sums for |q|^2, |k|^2, q.k
+    __shared__ float sh_part[2][4][2][VFIRST ? 4 : VB];     // K-first: per-wave column sums for S^T k and S^T q
+
+    const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
+    float a_neg = 0.f, dtb = 0.f;
+    if (p.A_log) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+
+    for (int64_t t = 0; t < len; ++t) {
+        const int pb = (int)(t & 1);
+        const int64_t tok = bos + t;
+        // -- stage q_t, k_t and their three inner products
+        float qv = 0.f, kv = 0.f;
+        if (tid < K) {
+            qv = to_f32(q[(tok * H + ih) * K + tid]);
+            kv = to_f32(k[(tok * H + ih) * K + tid]);
+        }
+        if (tid < KMAX) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
+        float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
+        if ((tid & 63) == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
+        // per-token scalars / per-column vectors (independent of the state)
+        float eg = 1.f;
+        if (p.g) {
+            float gt = load_scalar(p.g, tok * HV + ihv, p.gb_dtype);
+            if (p.A_log) gt = a_neg * softplus_f(gt + dtb);
+            eg = __expf(gt);
+        }
+        __syncthreads();
+        sqq = sh_red[pb][0][0] + sh_red[pb][1][0] + sh_red[pb][2][0] + sh_red[pb][3][0];
+        skk = sh_red[pb][0][1] + sh_red[pb][1][1] + sh_red[pb][2][1] + sh_red[pb][3][1];
+        sqk = sh_red[pb][0][2] + sh_red[pb][1][2] + sh_red[pb][2][2] + sh_red[pb][3][2];
+        float rq = p.scale, rk = 1.f;
+        if (p.flags & GDN_FLAG_QK_L2NORM) {
+            rq *= 1.f / sqrtf(sqq + 1e-6f);
+            rk = 1.f / sqrtf(skk + 1e-6f);
+        }
+        const float qk = sqk * rq * rk;             // (scale q).k after normalisation
+
+        if constexpr (!VFIRST) {
+            // ---------------- K-first: rows are k, this thread owns 4 value columns ----------------
+            float kr[R], qr[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const int row = r0 + RP * i;
+                kr[i] = row < KMAX ? sh_k[pb][row] * rk : 0.f;
+                qr[i] = row < KMAX ? sh_q[pb][row] * rq : 0.f;
+            }
+            f32x4 dgv = {1.f, 1.f, 1.f, 1.f};
+            if (p.gv && cont_ok) {
+                const f32x4 x = *(const f32x4*)(p.gv + (tok * HV + ihv) * V + cont_idx);
+                dgv = f32x4{__expf(x.x), __expf(x.y), __expf(x.z), __expf(x.w)};
+            }
+            dgv *= eg;
+            f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sq = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                f32x4 s = S[i] * dgv;
+                if (p.gk) {
+                    const int row = r0 + RP * i;
+                    if (row < K) s *= __expf(p.gk[(tok * HV + ihv) * K + row]);
+                }
+                S[i] = s;
+                sk += s * kr[i];
+                sq += s * qr[i];
+            }
+            // reduce over the row groups that share this thread's columns: inside the wave, then across waves
+#pragma unroll
+            for (int off = TC; off < 64; off <<= 1) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { sk[j] += __shfl_xor(sk[j], off, 64); sq[j] += __shfl_xor(sq[j], off, 64); }
+            }
+            if ((tid & 63) < TC) {
+                *(f32x4*)&sh_part[pb][wave][0][4 * c] = sk;
+                *(f32x4*)&sh_part[pb][wave][1][4 * c] = sq;
+            }
+            __syncthreads();
+            sk = *(f32x4*)&sh_part[pb][0][0][4 * c] + *(f32x4*)&sh_part[pb][1][0][4 * c] +
+                 *(f32x4*)&sh_part[pb][2][0][4 * c] + *(f32x4*)&sh_part[pb][3][0][4 * c];
+            sq = *(f32x4*)&sh_part[pb][0][1][4 * c] + *(f32x4*)&sh_part[pb][1][1][4 * c] +
+                 *(f32x4*)&sh_part[pb][2][1][4 * c] + *(f32x4*)&sh_part[pb][3][1][4 * c];
+            f32x4 vv = {0.f, 0.f, 0.f, 0.f}, bb = {1.f, 1.f, 1.f, 1.f};
+            if (cont_ok) {
+                const T* pv = v + (tok * HV + ihv) * V + cont_idx;
+                vv = f32x4{to_f32(pv[0]), to_f32(pv[1]), to_f32(pv[2]), to_f32(pv[3])};
+                if (p.beta) {
+                    if (p.flags & GDN_FLAG_BETA_VECTOR) {
+                        const int64_t bi = (tok * HV + ihv) * V + cont_idx;
+                        bb = f32x4{load_scalar(p.beta, bi, p.gb_dtype), load_scalar(p.beta, bi + 1, p.gb_dtype),
+                                   load_scalar(p.beta, bi + 2, p.gb_dtype), load_scalar(p.beta, bi + 3, p.gb_dtype)};
+                    } else {
+                        const float b = load_scalar(p.beta, tok * HV + ihv, p.gb_dtype);
+                        bb = f32x4{b, b, b, b};
+                    }
+                    if (p.flags & GDN_FLAG_BETA_SIGMOID) {
+                        const float m = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+                        bb = f32x4{m * sigmoid_f(bb.x), m * sigmoid_f(bb.y), m * sigmoid_f(bb.z), m * sigmoid_f(bb.w)};
+                    }
+                }
+            }
+            const f32x4 d = bb * (vv - sk);
+#pragma unroll
+            for (int i = 0; i < R; ++i) S[i] += d * kr[i];
+            if (r0 == 0 && cont_ok) {
+                const f32x4 ov = sq + d * qk;
+                T* po = o + (tok * HV + ihv) * V + cont_idx;
+                po[0] = from_f32<T>(ov.x); po[1] = from_f32<T>(ov.y); po[2] = from_f32<T>(ov.z); po[3] = from_f32<T>(ov.w);
+            }
+        } else {
+            // ---------------- V-first: rows are v, this thread owns 4 key columns ----------------
+            f32x4 kc = {0.f, 0.f, 0.f, 0.f}, qc = {0.f, 0.f, 0.f, 0.f};
+            kc = *(f32x4*)&sh_k[pb][4 * c] * rk;
+            qc = *(f32x4*)&sh_q[pb][4 * c] * rq;
+            f32x4 dgk = {eg, eg, eg, eg};
+            if (p.gk && cont_ok) {
+                const f32x4 x = *(const f32x4*)(p.gk + (tok * HV + ihv) * K + cont_idx);
+                dgk *= f32x4{__expf(x.x), __expf(x.y), __expf(x.z), __expf(x.w)};
+            }
+            const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                const int row = v0 + r0 + RP * i;
+                const bool rok = (r0 + RP * i < ROWS) && row < V;
+                f32x4 s = S[i] * dgk;
+                if (p.gv && rok) s *= __expf(p.gv[(tok * HV + ihv) * V + row]);
+                f32x4 a = s * kc, b = s * qc;
+                float sk = a.x + a.y + a.z + a.w, sq = b.x + b.y + b.z + b.w;
+#pragma unroll
+                for (int off = 1; off < TC; off <<= 1) { sk += __shfl_xor(sk, off, 64); sq += __shfl_xor(sq, off, 64); }
+                float vv = 0.f, bb = 1.f;
+                if (rok) {
+                    vv = to_f32(v[(tok * HV + ihv) * V + row]);
+                    if (p.beta) {
+                        bb = (p.flags & GDN_FLAG_BETA_VECTOR) ? load_scalar(p.beta, (tok * HV + ihv) * V + row, p.gb_dtype)
+                                                              : load_scalar(p.beta, tok * HV + ihv, p.gb_dtype);
+                        if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
+                    }
+                }
+                const float d = bb * (vv - sk);
+                S[i] = s + kc * d;
+                if (c == 0 && rok) o[(tok * HV + ihv) * V + row] = from_f32<T>(sq + d * qk);
+            }
+        }
+    }
+
+    if (p.ht) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int row = row_base + r0 + RP * i;
+            const bool ok = cont_ok && (r0 + RP * i < ROWS) && row < row_lim;
+            if (ok) __builtin_nontemporal_store(S[i], (f32x4*)(p.ht + state_off + row * row_stride + cont_idx));
+        }
+    }
+}
+
+template <typename T, int KMAX, bool VFIRST>
+static int launch_vb(const RecurrentParams& p0, int64_t n_states, int vb, hipStream_t stream) {
+    RecurrentParams p = p0;
+    p.NVB = (p.V + vb - 1) / vb;
+    dim3 grid((unsigned)(n_states * p.NVB)), block(256);
+    switch (vb) {
+        case 128: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 128, VFIRST>), grid, block, 0, stream, p); break;
+        case 64: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 64, VFIRST>), grid, block, 0, stream, p); break;
+        default: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 32, VFIRST>), grid, block, 0, stream, p); break;
+    }
+    return check_launch("gdn_recurrent_kernel");
+}
+
+template <typename T>
+static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stream) {
+    const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
+    // Value block per workgroup: whole rows when there are enough (sequence, head) pairs to
+    // fill 256 CUs several times over, narrower blocks otherwise.
+    int vb = 128;
+    while (vb > 32 && (p.V <= vb / 2 || n_states * ((p.V + vb - 1) / vb) < 1024)) vb >>= 1;
+    if (vfirst) vb = p.V >= 64 && n_states >= 1024 ? 64 : 32;   // V-first rows are independent; keep R small
+    const int kmax = p.K <= 64 ? 64 : (p.K <= 128 ? 128 : 256);
+#define GDN_REC_CASE(KM)                                                          \
+    case KM:                                                                      \
+        return vfirst ? launch_vb<T, KM, true>(p, n_states, vb, stream)           \
+                      : launch_vb<T, KM, false>(p, n_states, vb, stream);
+    switch (kmax) {
+        GDN_REC_CASE(64)
+        GDN_REC_CASE(128)
+        GDN_REC_CASE(256)
+    }
+#undef GDN_REC_CASE
+    return GDN_ERR_UNSUPPORTED;
+}
+
+}  // namespace gdn
+
+extern "C" int gdn_fused_recurrent_fwd(
+    const void* q, const void* k, const void* v,
+    const void* g, const void* beta, const float* gk, const float* gv,
+    const float* A_log, const float* dt_bias,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    using namespace gdn;
+    GDN_CHECK_ARG(q && k && v && o, GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: q, k, v, o must not be NULL");
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && K >= 1 && V >= 1 && N >= 1, GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: non-positive dimension");
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: HV=%lld not divisible by H=%lld",
+                  (long long)HV, (long long)H);
+    GDN_CHECK_ARG(cu_seqlens ? B == 1 : N == B, GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: with cu_seqlens B must be 1; without it N must equal B");
+    GDN_CHECK_ARG(K <= 256, GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: K=%lld > 256", (long long)K);
+    GDN_CHECK_ARG(K % 4 == 0 && V % 4 == 0, GDN_ERR_UNSUPPORTED,
+                  "gdn_fused_recurrent_fwd: K=%lld and V=%lld must be multiples of 4", (long long)K, (long long)V);
+    GDN_CHECK_ARG(N * HV * ((V + 31) / 32) < (1ll << 31), GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: grid too large");
+    GDN_CHECK_ARG(((uintptr_t)h0 % 16) == 0 && ((uintptr_t)ht % 16) == 0 && ((uintptr_t)gk % 16) == 0 &&
+                      ((uintptr_t)gv % 16) == 0,
+                  GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: h0/ht/gk/gv must be 16-byte aligned");
+    GDN_CHECK_ARG(!(A_log && !g), GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: A_log given without g");
+    if (T == 0) return GDN_OK;
+    RecurrentParams p;
+    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.gk = gk; p.gv = gv;
+    p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o; p.cu_seqlens = cu_seqlens;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.K = (int)K; p.V = (int)V; p.NVB = 1;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    hipStream_t s = (hipStream_t)stream;
+    switch (qkv_dtype) {
+        case GDN_DTYPE_BF16: return launch_t<bf16_t>(p, N * HV, s);
+        case GDN_DTYPE_F16: return launch_t<f16_t>(p, N * HV, s);
+        case GDN_DTYPE_F32: return launch_t<float>(p, N * HV, s);
+    }
+    set_error("gdn_fused_recurrent_fwd: unknown qkv_dtype %d", qkv_dtype);
+    return GDN_ERR_INVALID;
+}

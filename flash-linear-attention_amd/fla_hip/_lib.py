@@ -1,0 +1,100 @@
+"""ctypes binding of libgdn_hip.so (declarations follow include/gdn_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, '_C', 'libgdn_hip.so')
+
+ABI_VERSION = 1
+
+GDN_OK = 0
+GDN_ERR_INVALID = -1
+GDN_ERR_UNSUPPORTED = -2
+GDN_ERR_LAUNCH = -3
+GDN_ERR_WORKSPACE = -4
+
+DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
+
+FLAG_QK_L2NORM = 1 << 0
+FLAG_BETA_SIGMOID = 1 << 1
+FLAG_NEG_EIGVAL = 1 << 2
+FLAG_STATE_V_FIRST = 1 << 3
+FLAG_BETA_VECTOR = 1 << 4
+FLAG_CU_INT32 = 1 << 5
+
+# name -> (restype, argtypes); one entry per declaration in include/gdn_hip.h
+SIGNATURES = {
+    'gdn_hip_abi_version': (c_int, []),
+    'gdn_last_error': (c_char_p, []),
+    'gdn_fused_recurrent_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p,                      # q k v
+        c_void_p, c_void_p, c_void_p, c_void_p,            # g beta gk gv
+        c_void_p, c_void_p,                                # A_log dt_bias
+        c_void_p, c_void_p, c_void_p,                      # h0 ht o
+        c_void_p,                                          # cu_seqlens
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
+        c_float, c_int, c_int, c_uint32, c_void_p]),
+    'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
+    'gdn_chunk_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k v g beta
+        c_void_p, c_void_p, c_void_p,                      # h0 ht o
+        c_void_p, c_void_p, c_void_p,                      # cu_seqlens chunk_table chunk_offsets
+        c_void_p, c_size_t,                                # workspace, bytes
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V
+        c_int64, c_int64,                                  # N num_chunks
+        c_float, c_int, c_int, c_uint32, c_void_p]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class GDNLibraryError(ImportError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library.  Fails loudly when it has not been built: there is no
+    fallback implementation behind this package."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise GDNLibraryError(
+                f'{LIB_PATH} is missing. Build it with '
+                f'`python {os.path.join(os.path.dirname(_HERE), "build.py")}` (needs hipcc); '
+                'fla_hip has no CPU or eager fallback.')
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)        # AttributeError if the .so is stale
+            fn.restype = res
+            fn.argtypes = args
+        got = lib.gdn_hip_abi_version()
+        if got != ABI_VERSION:
+            raise GDNLibraryError(f'{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}; rebuild it')
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    msg = load().gdn_last_error()
+    return msg.decode() if msg else ''
+
+
+def check(status: int) -> None:
+    """Map C status codes to the exception types the reference raises from Python."""
+    if status == GDN_OK:
+        return
+    msg = last_error()
+    if status == GDN_ERR_INVALID:
+        raise ValueError(msg)
+    if status == GDN_ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(f'libgdn_hip status {status}: {msg}')

@@ -1,0 +1,8 @@
+from fla_hip.ops.gated_delta_rule import (
+    chunk_gated_delta_rule,
+    chunk_gdn,
+    fused_recurrent_gated_delta_rule,
+    fused_recurrent_gdn,
+)
+
+__all__ = ['chunk_gated_delta_rule', 'chunk_gdn', 'fused_recurrent_gated_delta_rule', 'fused_recurrent_gdn']

@@ -1,0 +1,68 @@
+"""Host-side helpers shared by the two operators: dtype codes, pointer extraction,
+argument normalisation.  Nothing here computes on tensors beyond casts/copies."""
+from __future__ import annotations
+
+import torch
+
+from fla_hip import _lib
+
+_DTYPE_CODE = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16, torch.float32: _lib.DTYPE_F32}
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise NotImplementedError(f'dtype {dt} is not supported by the HIP kernels (bf16, fp16, fp32)') from None
+
+
+def ptr(x: torch.Tensor | None) -> int | None:
+    return None if x is None else x.data_ptr()
+
+
+def require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != 'cuda':
+        raise RuntimeError(
+            'fla_hip runs only on a ROCm GPU (tensors must live on a "cuda" device); '
+            'there is no CPU implementation behind this operator.')
+    for t in tensors:
+        if t is not None and t.device != dev:
+            raise ValueError(f'all tensors must be on {dev}, got {t.device}')
+    return dev
+
+
+def as_f32(x: torch.Tensor | None) -> torch.Tensor | None:
+    if x is None:
+        return None
+    return x if x.dtype == torch.float32 else x.float()
+
+
+def aligned16(x: torch.Tensor | None) -> torch.Tensor | None:
+    """The kernels read states with 16-byte vector loads."""
+    if x is None or x.data_ptr() % 16 == 0:
+        return x
+    return x.clone(memory_format=torch.contiguous_format)
+
+
+def unify_qkv(q, k, v):
+    """q, k, v must share one of bf16/fp16/fp32; mixed inputs are cast to q's dtype."""
+    dt = q.dtype
+    if dt not in _DTYPE_CODE:
+        raise NotImplementedError(f'q dtype {dt} is not supported (bf16, fp16, fp32)')
+    return q, k.to(dt), v.to(dt)
+
+
+def unify_gate_beta(g, beta):
+    """g and beta are passed to the kernels with one shared dtype code."""
+    present = [x for x in (g, beta) if x is not None]
+    if not present:
+        return g, beta, _lib.DTYPE_F32
+    dts = {x.dtype for x in present}
+    if len(dts) == 1 and present[0].dtype in _DTYPE_CODE:
+        return g, beta, _DTYPE_CODE[present[0].dtype]
+    return as_f32(g), as_f32(beta), _lib.DTYPE_F32
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

@@ -1,0 +1,245 @@
+"""``chunk_gated_delta_rule``: same signature, defaults, validation and error types as
+fla/ops/gated_delta_rule/chunk.py:397-593.  The reference's five Triton launches
+(chunk.py:33-123) are replaced by one call into libgdn_hip.so (``gdn_chunk_fwd``), which
+runs two HIP kernels: a chunk-parallel one (gate cumsum, gated beta*K*K^T, 64x64 unit-lower
+solve, WY factors w/u, intra-chunk q k^T) and a sequential one (state recurrence fused with
+the output), so per-chunk states are never written to memory."""
+from __future__ import annotations
+
+import warnings
+
+import torch
+
+from fla_hip import _lib
+from fla_hip.ops.backends import dispatch
+from fla_hip.ops.gated_delta_rule._common import (
+    aligned16,
+    as_f32,
+    current_stream_ptr,
+    dtype_code,
+    ptr,
+    require_gpu,
+    unify_gate_beta,
+)
+from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_chunk_offsets
+from fla_hip.utils import input_guard
+
+# The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
+# the chunk size (only rounding does), so chunk_size 16 and 32 are accepted and run with 64.
+_KERNEL_CHUNK = 64
+_KERNEL_DIMS = (64, 128)        # head dims the MFMA kernels are instantiated for
+
+
+def _l2norm_rows(x: torch.Tensor) -> torch.Tensor:
+    """x / sqrt(sum(x^2) + 1e-6) per head vector, result in x's dtype (the reference's
+    l2norm_fwd, fla/modules/l2norm.py:84-109, applied before its chunk pipeline)."""
+    xf = x.float()
+    return (xf * torch.rsqrt((xf * xf).sum(-1, keepdim=True) + 1e-6)).to(x.dtype)
+
+
+def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
+    if x.shape[-1] == size:
+        return x
+    return torch.nn.functional.pad(x, (0, size - x.shape[-1]))
+
+
+def _kernel_dim(d: int) -> int:
+    for s in _KERNEL_DIMS:
+        if d <= s:
+            return s
+    raise NotImplementedError(f'head dim {d} > {_KERNEL_DIMS[-1]} is not supported by the HIP chunk kernels')
+
+
+@input_guard
+def chunk_gated_delta_rule_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    scale: float,
+    initial_state: torch.Tensor | None,
+    output_final_state: bool,
+    state_v_first: bool = False,
+    cu_seqlens: torch.Tensor | None = None,
+    cu_seqlens_cpu: torch.Tensor | None = None,
+    chunk_indices: torch.Tensor | None = None,
+    chunk_size: int = 64,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Forward of the chunked operator on already-activated ``g`` (log space) and ``beta``.
+    Returns ``(o in q's dtype, final_state fp32 or None)``."""
+    dev = require_gpu(q, k, v, g, beta)
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    out_dtype = q.dtype
+
+    # the MFMA kernels take bf16 or fp16 operands; fp32 inputs are rounded to bf16 first
+    work_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    q, k, v = q.to(work_dtype), k.to(work_dtype), v.to(work_dtype)
+    # head dims other than 64/128 are zero-padded: zero key features and zero value columns
+    # change neither the other columns nor the state rows that matter
+    KP, VP = _kernel_dim(K), _kernel_dim(V)
+    KP = VP = max(KP, VP)
+    q, k, v = _pad_last(q, KP), _pad_last(k, KP), _pad_last(v, VP)
+    g, beta, gb_code = unify_gate_beta(g, beta)
+
+    flags = 0
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype not in (torch.int32, torch.int64):
+            cu_seqlens = cu_seqlens.long()
+        if cu_seqlens.device != dev:
+            cu_seqlens = cu_seqlens.to(dev)
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        if chunk_indices is None or chunk_size != _KERNEL_CHUNK:
+            chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        chunk_indices = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        chunk_offsets = prepare_chunk_offsets(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        num_chunks = chunk_indices.shape[0]
+    else:
+        chunk_indices = chunk_offsets = None
+        num_chunks = B * ((T + _KERNEL_CHUNK - 1) // _KERNEL_CHUNK)
+
+    state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+    h0 = initial_state
+    if h0 is not None:
+        if tuple(h0.shape) != state_shape:
+            raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
+        h0 = as_f32(h0)
+        if (KP, VP) != (K, V):
+            h0 = torch.nn.functional.pad(h0, (0, (KP if state_v_first else VP) - h0.shape[-1],
+                                              0, (VP if state_v_first else KP) - h0.shape[-2]))
+        h0 = aligned16(h0.contiguous())
+        flags |= _lib.FLAG_STATE_V_FIRST if state_v_first else 0
+    elif state_v_first:
+        flags |= _lib.FLAG_STATE_V_FIRST
+
+    o = torch.empty(B, T, HV, VP, dtype=work_dtype, device=dev)
+    ht = None
+    if output_final_state:
+        ht = torch.empty((N, HV, VP, KP) if state_v_first else (N, HV, KP, VP), dtype=torch.float32, device=dev)
+
+    lib = _lib.load()
+    ws_bytes = lib.gdn_chunk_workspace_bytes(num_chunks, H, HV, KP, VP)
+    if ws_bytes == 0 and num_chunks > 0:
+        raise NotImplementedError(f'HIP chunk kernels do not cover K={KP}, V={VP}')
+    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    if T > 0:
+        _lib.check(lib.gdn_chunk_fwd(
+            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(ht), ptr(o),
+            ptr(cu_seqlens), ptr(chunk_indices), ptr(chunk_offsets),
+            ptr(workspace), ws_bytes,
+            B, T, H, HV, KP, VP, N, num_chunks,
+            float(scale), dtype_code(work_dtype), gb_code, flags, current_stream_ptr(dev)))
+    elif ht is not None:
+        ht.copy_(h0) if h0 is not None else ht.zero_()
+
+    if VP != V:
+        o = o[..., :V]
+    if ht is not None and (KP, VP) != (K, V):
+        ht = (ht[..., :V, :K] if state_v_first else ht[..., :K, :V]).contiguous()
+    return o.to(out_dtype), ht
+
+
+@dispatch('gated_delta_rule')
+@torch.compiler.disable
+def chunk_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    scale: float | None = None,
+    initial_state: torch.Tensor | None = None,
+    output_final_state: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+    use_beta_sigmoid_in_kernel: bool = False,
+    allow_neg_eigval: bool = False,
+    state_v_first: bool = False,
+    cu_seqlens: torch.LongTensor | None = None,
+    cu_seqlens_cpu: torch.LongTensor | None = None,
+    chunk_indices: torch.LongTensor | None = None,
+    cp_context=None,
+    **kwargs,
+):
+    r"""Chunked gated delta rule (prefill), forward only.
+
+    Args:
+        q, k: ``[B, T, H, K]``.  v: ``[B, T, HV, V]`` with ``HV % H == 0`` (grouped value heads).
+        g: log-space decay ``[B, T, HV]`` (raw pre-activation with ``use_gate_in_kernel=True``,
+            ``A_log`` and optional ``dt_bias`` passed as keywords).
+        beta: ``[B, T, HV]`` (logits with ``use_beta_sigmoid_in_kernel=True``;
+            ``allow_neg_eigval`` doubles the sigmoid).
+        scale: defaults to ``K ** -0.5``.
+        initial_state: ``[N, HV, K, V]`` (``[N, HV, V, K]`` with ``state_v_first``), any float dtype.
+        output_final_state: also return the fp32 final state.
+        use_qk_l2norm_in_kernel: L2-normalise q and k per head first.
+        cu_seqlens: ``[N + 1]`` int32/int64 boundaries of packed sequences (then ``B == 1``);
+            ``cu_seqlens_cpu`` is an optional host copy that avoids a device sync;
+            ``chunk_indices`` optional precomputed chunk table for ``chunk_size``.
+        cp_context: context parallelism is not part of this single-GPU build.
+
+    Returns:
+        ``(o [B, T, HV, V] in q's dtype, final_state or None)``.
+    """
+    if 'transpose_state_layout' in kwargs:
+        if state_v_first:
+            raise ValueError('Cannot pass both `state_v_first` and the deprecated `transpose_state_layout`.')
+        warnings.warn('`transpose_state_layout` is deprecated and renamed to `state_v_first`.',
+                      DeprecationWarning, stacklevel=2)
+        state_v_first = kwargs.pop('transpose_state_layout')
+
+    if q.shape[2] != k.shape[2]:
+        raise ValueError(
+            f'q and k must have the same number of heads, '
+            f'but got q.shape[2]={q.shape[2]} and k.shape[2]={k.shape[2]}')
+    H, HV = q.shape[2], v.shape[2]
+    if HV % H != 0:
+        raise ValueError(
+            f'For GVA, num_v_heads (HV={HV}) must be evenly divisible by '
+            f'num_heads (H={H}), but got HV % H = {HV % H}')
+    if 'head_first' in kwargs:
+        raise DeprecationWarning('head_first has been removed. Inputs must be in `[B, T, H, ...]` format.')
+    chunk_size = kwargs.pop('chunk_size', 64)
+    if chunk_size not in (16, 32, 64):
+        raise ValueError(f'`chunk_size` must be 16, 32, or 64 for Gated Delta Rule, got {chunk_size}.')
+    if cp_context is not None:
+        raise NotImplementedError('context parallelism (cp_context) is outside this single-GPU build')
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(
+                f'The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`.'
+                f'Please flatten variable-length inputs before processing.')
+        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+            raise ValueError(
+                f'The number of initial states is expected to be equal to the number of input sequences, '
+                f'i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.')
+    use_gate_in_kernel = kwargs.get('use_gate_in_kernel', False)
+    A_log = kwargs.get('A_log')
+    dt_bias = kwargs.get('dt_bias')
+    if use_gate_in_kernel:
+        assert A_log is not None, 'A_log must be provided when use_gate_in_kernel=True.'
+    if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
+        raise ValueError('`allow_neg_eigval=True` requires `use_beta_sigmoid_in_kernel=True`.')
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+
+    # prologues the reference runs as separate launches before its chunk pipeline
+    # (chunk.py:278-288 and gate.py:63-106); elementwise, done on the device
+    if use_qk_l2norm_in_kernel:
+        q, k = _l2norm_rows(q), _l2norm_rows(k)
+    if use_beta_sigmoid_in_kernel:
+        beta = torch.sigmoid(beta.float()) * (2.0 if allow_neg_eigval else 1.0)
+    if use_gate_in_kernel:
+        gf = g.float()
+        if dt_bias is not None:
+            gf = gf + dt_bias.float()
+        g = -A_log.float().exp() * torch.nn.functional.softplus(gf)
+
+    return chunk_gated_delta_rule_fwd(
+        q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first,
+        cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size)
+
+
+chunk_gdn = chunk_gated_delta_rule

@@ -1,0 +1,188 @@
+"""``fused_recurrent_gated_delta_rule``: same signature, defaults, validation and error
+types as fla/ops/gated_delta_rule/fused_recurrent.py:309-475; the single Triton launch
+(:184-250) is replaced by one call into libgdn_hip.so (``gdn_fused_recurrent_fwd``)."""
+from __future__ import annotations
+
+import warnings
+
+import torch
+
+from fla_hip import _lib
+from fla_hip.ops.gated_delta_rule._common import (
+    aligned16,
+    as_f32,
+    current_stream_ptr,
+    dtype_code,
+    ptr,
+    require_gpu,
+    unify_gate_beta,
+    unify_qkv,
+)
+from fla_hip.utils import input_guard
+
+
+@input_guard
+def fused_recurrent_gated_delta_rule_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor | None = None,
+    gk: torch.Tensor | None = None,
+    gv: torch.Tensor | None = None,
+    beta: torch.Tensor | None = None,
+    A_log: torch.Tensor | None = None,
+    dt_bias: torch.Tensor | None = None,
+    scale: float = None,
+    initial_state: torch.Tensor = None,
+    output_final_state: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+    use_beta_sigmoid_in_kernel: bool = False,
+    allow_neg_eigval: bool = False,
+    state_v_first: bool = False,
+    cu_seqlens: torch.Tensor | None = None,
+    inplace_final_state: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """Allocates ``o`` (v's dtype) and the fp32 final state, then launches the HIP kernel on
+    the current stream.  With ``inplace_final_state`` the final state is written over
+    ``initial_state`` (which must then be fp32 and contiguous) and that tensor is returned."""
+    dev = require_gpu(q, k, v)
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    q, k, v = unify_qkv(q, k, v)
+    g, beta, gb_code = unify_gate_beta(g, beta)
+    gk, gv, A_log, dt_bias = as_f32(gk), as_f32(gv), as_f32(A_log), as_f32(dt_bias)
+
+    flags = 0
+    if use_qk_l2norm_in_kernel:
+        flags |= _lib.FLAG_QK_L2NORM
+    if use_beta_sigmoid_in_kernel:
+        flags |= _lib.FLAG_BETA_SIGMOID
+    if allow_neg_eigval:
+        flags |= _lib.FLAG_NEG_EIGVAL
+    if state_v_first:
+        flags |= _lib.FLAG_STATE_V_FIRST
+    if beta is not None and beta.ndim == v.ndim:
+        flags |= _lib.FLAG_BETA_VECTOR
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        elif cu_seqlens.dtype != torch.int64:
+            cu_seqlens = cu_seqlens.long()
+        if cu_seqlens.device != dev:
+            cu_seqlens = cu_seqlens.to(dev)
+
+    state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+    h0 = initial_state
+    if h0 is not None:
+        if tuple(h0.shape) != state_shape:
+            raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
+        if inplace_final_state:
+            if h0.dtype != torch.float32 or h0.data_ptr() % 16 != 0:
+                raise ValueError('inplace_final_state needs a contiguous, 16-byte aligned fp32 initial_state')
+        else:
+            h0 = aligned16(as_f32(h0))
+
+    o = torch.empty_like(v)
+    final_state = None
+    if inplace_final_state:
+        if initial_state is None:
+            raise ValueError('inplace_final_state=True requires initial_state')
+        final_state = h0
+    elif output_final_state:
+        final_state = torch.empty(state_shape, dtype=torch.float32, device=dev)
+
+    lib = _lib.load()
+    _lib.check(lib.gdn_fused_recurrent_fwd(
+        ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(gk), ptr(gv), ptr(A_log), ptr(dt_bias),
+        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens),
+        B, T, H, HV, K, V, N, float(scale), dtype_code(q.dtype), gb_code, flags,
+        current_stream_ptr(dev)))
+    return o, final_state
+
+
+def fused_recurrent_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor | None = None,
+    gk: torch.Tensor | None = None,
+    gv: torch.Tensor | None = None,
+    beta: torch.Tensor | None = None,
+    scale: float = None,
+    initial_state: torch.Tensor = None,
+    output_final_state: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+    use_gate_in_kernel: bool = False,
+    A_log: torch.Tensor | None = None,
+    dt_bias: torch.Tensor | None = None,
+    use_beta_sigmoid_in_kernel: bool = False,
+    allow_neg_eigval: bool = False,
+    state_v_first: bool = False,
+    cu_seqlens: torch.LongTensor | None = None,
+    **kwargs,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    r"""Token-by-token gated delta rule (decode / short prompts).
+
+    Args:
+        q, k: ``[B, T, H, K]``.  v: ``[B, T, HV, V]`` (``HV % H == 0``; each q/k head serves
+            ``HV // H`` consecutive v heads).
+        g: log-space decay ``[B, T, HV]``; raw pre-activation when ``use_gate_in_kernel``
+            (then ``g = -exp(A_log) * softplus(g + dt_bias)`` is applied per step).
+        gk / gv: optional per-key / per-value log decays ``[B, T, HV, K]`` / ``[B, T, HV, V]``.
+        beta: ``[B, T, HV]`` (or ``[B, T, HV, V]``); ones when omitted; logits when
+            ``use_beta_sigmoid_in_kernel`` (``allow_neg_eigval`` doubles the sigmoid).
+        scale: defaults to ``K ** -0.5``.
+        initial_state: ``[N, HV, K, V]`` (``[N, HV, V, K]`` when ``state_v_first``).
+        output_final_state: also return the fp32 final state.
+        cu_seqlens: ``[N + 1]`` int32/int64 boundaries of packed sequences (then ``B == 1``).
+        inplace_final_state (keyword only, extension): write the final state over
+            ``initial_state`` instead of allocating a new tensor.
+
+    Returns:
+        ``(o [B, T, HV, V] in v's dtype, final_state or None)``.
+    """
+    if 'transpose_state_layout' in kwargs:
+        if state_v_first:
+            raise ValueError('Cannot pass both `state_v_first` and the deprecated `transpose_state_layout`.')
+        warnings.warn('`transpose_state_layout` is deprecated and renamed to `state_v_first`.',
+                      DeprecationWarning, stacklevel=2)
+        state_v_first = kwargs.pop('transpose_state_layout')
+    inplace_final_state = bool(kwargs.pop('inplace_final_state', False))
+
+    if q.shape[2] != k.shape[2]:
+        raise ValueError(f'q and k must have the same number of heads, got {q.shape[2]} and {k.shape[2]}')
+    if v.shape[2] % q.shape[2] != 0:
+        raise ValueError(f'num_v_heads (HV={v.shape[2]}) must be divisible by num_heads (H={q.shape[2]})')
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(
+                f'The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`.'
+                f'Please flatten variable-length inputs before processing.')
+        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+            raise ValueError(
+                f'The number of initial states is expected to be equal to the number of input sequences, '
+                f'i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.')
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    if use_gate_in_kernel:
+        if A_log is None:
+            raise ValueError('`A_log` must be provided when `use_gate_in_kernel=True`.')
+        if g is None:
+            raise ValueError('`g` (raw pre-activation) must be provided when `use_gate_in_kernel=True`.')
+    else:
+        A_log = None
+        dt_bias = None
+    if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
+        raise ValueError('`allow_neg_eigval=True` requires `use_beta_sigmoid_in_kernel=True`.')
+    if inplace_final_state and (initial_state is None or not initial_state.is_contiguous()
+                                or initial_state.dtype != torch.float32):
+        raise ValueError('`inplace_final_state=True` requires a contiguous fp32 `initial_state`.')
+
+    return fused_recurrent_gated_delta_rule_fwd(
+        q, k, v, g, gk, gv, beta, A_log, dt_bias, scale, initial_state, output_final_state,
+        use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, cu_seqlens,
+        inplace_final_state)
+
+
+fused_recurrent_gdn = fused_recurrent_gated_delta_rule

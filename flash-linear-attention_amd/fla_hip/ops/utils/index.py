@@ -1,0 +1,43 @@
+"""Varlen chunk tables: same results as ``prepare_lens`` / ``prepare_chunk_indices`` /
+``prepare_chunk_offsets`` of fla/ops/utils/index.py:41-43,156-172.
+
+The tables are tiny integer arrays; they are built on the HOST from ``cu_seqlens_cpu`` when
+the caller supplies it (no device sync), otherwise from one device-to-host copy of
+``cu_seqlens``, and then uploaded.  Results are memoised by tensor identity."""
+from __future__ import annotations
+
+import torch
+
+from fla_hip.utils import tensor_cache
+
+
+def prepare_lens(cu_seqlens: torch.Tensor) -> torch.Tensor:
+    return cu_seqlens[1:] - cu_seqlens[:-1]
+
+
+def _host_lens(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None) -> torch.Tensor:
+    src = cu_seqlens_cpu if cu_seqlens_cpu is not None else cu_seqlens
+    src = src.detach().to('cpu', torch.int64)
+    return src[1:] - src[:-1]
+
+
+@tensor_cache
+def prepare_chunk_indices(cu_seqlens: torch.Tensor, chunk_size: int,
+                          cu_seqlens_cpu: torch.Tensor | None = None) -> torch.Tensor:
+    """[num_chunks, 2] rows (sequence id, chunk id inside that sequence), packed order;
+    dtype and device of ``cu_seqlens``."""
+    counts = (_host_lens(cu_seqlens, cu_seqlens_cpu) + (chunk_size - 1)) // chunk_size
+    seq_id = torch.repeat_interleave(torch.arange(counts.numel(), dtype=torch.int64), counts)
+    first = torch.cumsum(counts, 0) - counts                    # first packed chunk of each sequence
+    within = torch.arange(seq_id.numel(), dtype=torch.int64) - first[seq_id]
+    return torch.stack([seq_id, within], 1).to(device=cu_seqlens.device, dtype=cu_seqlens.dtype)
+
+
+@tensor_cache
+def prepare_chunk_offsets(cu_seqlens: torch.Tensor, chunk_size: int,
+                          cu_seqlens_cpu: torch.Tensor | None = None) -> torch.Tensor:
+    """[N+1] exclusive prefix sum of the number of chunks per sequence."""
+    counts = (_host_lens(cu_seqlens, cu_seqlens_cpu) + (chunk_size - 1)) // chunk_size
+    out = torch.zeros(counts.numel() + 1, dtype=torch.int64)
+    out[1:] = torch.cumsum(counts, 0)
+    return out.to(device=cu_seqlens.device, dtype=cu_seqlens.dtype)

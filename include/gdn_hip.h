@@ -1,0 +1,113 @@
+/*
+ * gdn_hip.h - C ABI of libgdn_hip.so: the gated delta rule (Gated DeltaNet)
+ * inference path as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The reference (fla-org/flash-linear-attention) is Python + Triton and has no
+ * FFI of its own; its boundary for this path is two Python functions.  Each
+ * entry point below is what a binding for one of them calls, and cites the
+ * reference interface it replaces.  All pointers are DEVICE pointers unless
+ * stated otherwise; all tensors are contiguous, token-major, exactly as the
+ * reference's `input_guard` hands them to its kernels
+ * (fla/utils/_decorators.py:99-165).  Calls only enqueue work on `stream`
+ * (a hipStream_t passed as void*, NULL = the null stream); they never
+ * synchronise.  Return value: 0 on success, negative GDN_ERR_* otherwise;
+ * gdn_last_error() then returns a message for the calling thread.
+ */
+#ifndef GDN_HIP_H
+#define GDN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GDN_OK                 0
+#define GDN_ERR_INVALID       -1   /* bad argument (Python shim raises ValueError)            */
+#define GDN_ERR_UNSUPPORTED   -2   /* shape/dtype outside the kernels (NotImplementedError)   */
+#define GDN_ERR_LAUNCH        -3   /* HIP runtime error at launch (RuntimeError)              */
+#define GDN_ERR_WORKSPACE     -4   /* workspace too small                                     */
+
+/* element types of q/k/v/o and of g/beta */
+#define GDN_DTYPE_BF16 0
+#define GDN_DTYPE_F16  1
+#define GDN_DTYPE_F32  2
+
+/* flag bits (the reference's keyword switches) */
+#define GDN_FLAG_QK_L2NORM      (1u << 0)  /* use_qk_l2norm_in_kernel                           */
+#define GDN_FLAG_BETA_SIGMOID   (1u << 1)  /* use_beta_sigmoid_in_kernel                        */
+#define GDN_FLAG_NEG_EIGVAL     (1u << 2)  /* allow_neg_eigval (beta = 2*sigmoid)               */
+#define GDN_FLAG_STATE_V_FIRST  (1u << 3)  /* state_v_first: states are [N,HV,V,K]              */
+#define GDN_FLAG_BETA_VECTOR    (1u << 4)  /* beta is [B,T,HV,V] instead of [B,T,HV]            */
+#define GDN_FLAG_CU_INT32       (1u << 5)  /* cu_seqlens / chunk tables are int32, else int64   */
+
+/* Library ABI version (bumped on any signature change). */
+int gdn_hip_abi_version(void);
+
+/* Message describing the last error raised on the calling thread ("" if none). */
+const char* gdn_last_error(void);
+
+/*
+ * Token recurrence, used for decode and short prompts.
+ * Replaces fused_recurrent_gated_delta_rule_fwd
+ * (fla/ops/gated_delta_rule/fused_recurrent.py:184-250, kernel :30-181).
+ *
+ *   q, k   [B,T,H,K]   qkv_dtype          v, o  [B,T,HV,V]  qkv_dtype
+ *   g      [B,T,HV]    gb_dtype or NULL   beta  [B,T,HV] (or [B,T,HV,V] with GDN_FLAG_BETA_VECTOR), gb_dtype, or NULL (=1)
+ *   gk     [B,T,HV,K]  fp32 or NULL       gv    [B,T,HV,V]  fp32 or NULL
+ *   A_log, dt_bias [HV] fp32 or NULL: when A_log != NULL, g is raw and the gate
+ *          g = -exp(A_log)*softplus(g + dt_bias) is applied per step (use_gate_in_kernel)
+ *   h0     [N,HV,K,V] fp32 or NULL (zero state)
+ *   ht     [N,HV,K,V] fp32 or NULL (final state not stored); ht MAY alias h0 (in-place update)
+ *   cu_seqlens [N+1] or NULL; when given B must be 1 and T is the packed length
+ *   N = B when cu_seqlens == NULL.  Requires K <= 256, K % 4 == 0, V % 4 == 0, HV % H == 0.
+ */
+int gdn_fused_recurrent_fwd(
+    const void* q, const void* k, const void* v,
+    const void* g, const void* beta, const float* gk, const float* gv,
+    const float* A_log, const float* dt_bias,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
+ * Bytes of device workspace gdn_chunk_fwd needs for `num_chunks` 64-token
+ * chunks (dense: B*ceil(T/64); packed: sum over sequences of ceil(len/64)).
+ * Returns 0 for unsupported (K,V).
+ */
+size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V);
+
+/*
+ * Chunked prefill, chunk size 64.  Replaces chunk_gated_delta_rule_fwd
+ * (fla/ops/gated_delta_rule/chunk.py:33-123), i.e. the five launches
+ * chunk_local_cumsum (fla/ops/utils/cumsum.py:243-277),
+ * chunk_gated_delta_rule_fwd_intra (fla/ops/gated_delta_rule/chunk_fwd.py:332-428),
+ * recompute_w_u_fwd (fla/ops/gated_delta_rule/wy_fast.py:255-294),
+ * chunk_gated_delta_rule_fwd_h (fla/ops/common/chunk_delta_h.py:687-743) and
+ * chunk_fwd_o (fla/ops/common/chunk_o.py:544-586).
+ *
+ *   q, k [B,T,H,K], v, o [B,T,HV,V] qkv_dtype (bf16 or f16); g, beta [B,T,HV] gb_dtype
+ *   h0 [N,HV,K,V] fp32 or NULL; ht [N,HV,K,V] fp32 or NULL
+ *   cu_seqlens [N+1] (device) or NULL
+ *   chunk_table [num_chunks][2] (device; sequence id, chunk id inside the sequence) -
+ *         prepare_chunk_indices of fla/ops/utils/index.py:156-164; NULL for dense input
+ *   chunk_offsets [N+1] (device; exclusive prefix sum of chunks per sequence) -
+ *         prepare_chunk_offsets of fla/ops/utils/index.py:167-172; NULL for dense input
+ *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
+ *   Requires K == V == 128 (or 64), HV % H == 0.
+ */
+int gdn_chunk_fwd(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GDN_HIP_H */

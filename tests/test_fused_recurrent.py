@@ -1,0 +1,175 @@
+"""GPU parity of fused_recurrent_gated_delta_rule (HIP, through the C ABI) against the CPU
+oracle on the same seeded inputs.  Shapes follow the reference's own matrix
+(tests/ops/test_gdn.py:48-105, :450-517) plus the decode configuration."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# tolerance on o and on the final state: relative RMSE <= 2e-3 (the reference's own bar for
+# this kernel, tests/ops/test_gdn.py:104-105) and max-abs-error ratio <= 1e-2
+RATIO, MAXABS = 2e-3, 1e-2
+
+
+def _ops():
+    from fla_hip.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    return fused_recurrent_gated_delta_rule
+
+
+def _check(name, ref, got, ratio=RATIO):
+    got = got.detach().float().cpu()
+    assert not torch.isnan(got).any(), f'{name}: NaN'
+    r, m = O.get_err_ratio(ref, got), O.max_abs_ratio(ref, got)
+    assert r <= ratio and m <= MAXABS, f'{name}: rel-rmse {r:.3e} max-abs ratio {m:.3e}'
+
+
+def _inputs(B, T, H, HV, D, dtype, seed=42, gate_norm=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    k = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    v = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    g = F.logsigmoid(torch.rand(B, T, HV, generator=gen)) / gate_norm
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    return q, k, v, g, beta, h0
+
+
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_norm,dtype', [
+    (1, 63, 1, 1, 64, 1.0, 1.0, torch.float32),
+    (2, 200, 4, 4, 60, 1.0, 1.0, torch.float32),
+    (2, 300, 2, 8, 128, 1.0, 0.1, torch.float32),
+    (3, 256, 2, 2, 128, 0.1, 1.0, torch.float32),
+    (2, 128, 3, 3, 100, 1.0, 10.0, torch.float32),
+    (2, 256, 4, 4, 128, 0.1, 1.0, torch.float16),
+    (2, 256, 4, 8, 128, 1.0, 10.0, torch.float16),
+    (2, 256, 2, 4, 128, 1.0, 1.0, torch.bfloat16),
+    (1, 64, 2, 2, 256, 1.0, 1.0, torch.float32),
+])
+def test_fused_recurrent_vs_oracle(B, T, H, HV, D, scale, gate_norm, dtype):
+    op = _ops()
+    q, k, v, g, beta, h0 = _inputs(B, T, H, HV, D, dtype, gate_norm=gate_norm)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, scale, h0, True, use_qk_l2norm_in_kernel=True)
+    dev = 'cuda'
+    o, ht = op(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), scale=scale,
+               initial_state=h0.to(dev), output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o.dtype == v.dtype and ht.dtype == torch.float32 and ht.shape == (B, HV, D, D)
+    ratio = RATIO if dtype == torch.float32 else 5e-3      # o itself is rounded to 16 bits
+    _check('o', ref_o, o, ratio)
+    _check('ht', ref_ht, ht)
+
+
+def test_decode_shape_inplace_and_chained_steps():
+    """N=64 decode steps with Hqk=16, Hv=32, K=V=128 (the decode configuration at a quarter
+    of its batch): three chained single-token calls, state updated in place, must equal the
+    oracle's three-token recurrence."""
+    op = _ops()
+    N, H, HV, D = 64, 16, 32, 128
+    gen = torch.Generator().manual_seed(1)
+    q = F.normalize(torch.randn(N, 3, H, D, generator=gen), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(N, 3, H, D, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(N, 3, HV, D, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(N, 3, HV, generator=gen))
+    beta = torch.sigmoid(torch.randn(N, 3, HV, generator=gen))
+    h0 = 0.1 * torch.randn(N, HV, D, D, generator=gen)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    dev = 'cuda'
+    state = h0.to(dev)
+    ptr0 = state.data_ptr()
+    outs = []
+    for t in range(3):
+        o, st = op(q[:, t:t + 1].to(dev), k[:, t:t + 1].to(dev), v[:, t:t + 1].to(dev), g[:, t:t + 1].to(dev),
+                   beta=beta[:, t:t + 1].to(dev), initial_state=state, output_final_state=True, inplace_final_state=True)
+        assert st.data_ptr() == ptr0
+        outs.append(o)
+    _check('o', ref_o, torch.cat(outs, 1), 5e-3)
+    _check('ht', ref_ht, state)
+    # one 3-token call gives the same state as the three chained calls, bit for bit
+    o3, st3 = op(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=h0.to(dev),
+                 output_final_state=True)
+    assert torch.equal(st3, state) and torch.equal(o3, torch.cat(outs, 1))
+
+
+@pytest.mark.parametrize('cu,H,HV,D', [
+    ([0, 15], 2, 2, 64),
+    ([0, 1, 100, 101, 300], 2, 4, 64),
+    ([0, 15, 100, 300, 1200, 1500], 2, 8, 100),
+])
+@pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
+def test_varlen_ownership_is_bit_exact(cu, H, HV, D, idx_dtype):
+    """Packed call == each sequence run alone, bit for bit, and both match the oracle."""
+    op = _ops()
+    T, N = cu[-1], len(cu) - 1
+    q, k, v, g, beta, _ = _inputs(1, T, H, HV, D, torch.float16, seed=3)
+    h0 = torch.randn(N, HV, D, D, generator=torch.Generator().manual_seed(4))
+    dev = 'cuda'
+    a = [x.to(dev) for x in (q, k, v, g, beta)]
+    o, ht = op(a[0], a[1], a[2], a[3], beta=a[4], initial_state=h0.to(dev), output_final_state=True,
+               use_qk_l2norm_in_kernel=True, cu_seqlens=torch.tensor(cu, dtype=idx_dtype, device=dev))
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu,
+                                                 use_qk_l2norm_in_kernel=True)
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht)
+    for n, (s, e) in enumerate(zip(cu[:-1], cu[1:])):
+        o_n, h_n = op(a[0][:, s:e], a[1][:, s:e], a[2][:, s:e], a[3][:, s:e], beta=a[4][:, s:e],
+                      initial_state=h0[n:n + 1].to(dev), output_final_state=True, use_qk_l2norm_in_kernel=True)
+        assert torch.equal(o_n[0], o[0, s:e]), f'sequence {n}: o differs'
+        assert torch.equal(h_n[0], ht[n]), f'sequence {n}: state differs'
+
+
+def test_flags_gate_sigmoid_vector_beta_gk_gv_vfirst():
+    op = _ops()
+    B, T, H, HV, D = 2, 70, 2, 4, 64
+    gen = torch.Generator().manual_seed(5)
+    q, k = torch.randn(B, T, H, D, generator=gen), torch.randn(B, T, H, D, generator=gen)
+    v = torch.randn(B, T, HV, D, generator=gen)
+    graw, braw = torch.randn(B, T, HV, generator=gen), torch.randn(B, T, HV, D, generator=gen)
+    gk = -0.1 * torch.rand(B, T, HV, D, generator=gen)
+    gv = -0.1 * torch.rand(B, T, HV, D, generator=gen)
+    A_log, dt_bias = 0.3 * torch.randn(HV, generator=gen), 0.3 * torch.randn(HV, generator=gen)
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, A_log=A_log, dt_bias=dt_bias,
+              use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, graw, braw, None, h0, True, gk=gk, gv=gv, **kw)
+    dev = 'cuda'
+    kwd = dict(kw, A_log=A_log.to(dev), dt_bias=dt_bias.to(dev))
+    o, ht = op(q.to(dev), k.to(dev), v.to(dev), graw.to(dev), gk=gk.to(dev), gv=gv.to(dev), beta=braw.to(dev),
+               initial_state=h0.to(dev), output_final_state=True, **kwd)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    # V-first layout is the transpose of the default one
+    o2, ht2 = op(q.to(dev), k.to(dev), v.to(dev), graw.to(dev), gk=gk.to(dev), gv=gv.to(dev), beta=braw.to(dev),
+                 initial_state=h0.transpose(-1, -2).contiguous().to(dev), output_final_state=True,
+                 state_v_first=True, **kwd)
+    _check('o (v-first)', ref_o, o2)
+    _check('ht (v-first)', ref_ht.transpose(-1, -2), ht2)
+    # no gate, no beta: plain delta rule with beta = 1
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(O.l2norm(q), O.l2norm(k), v, None, None, None, None, True)
+    o, ht = op(O.l2norm(q).to(dev), O.l2norm(k).to(dev), v.to(dev), output_final_state=True)
+    _check('o (no g/beta)', ref_o, o)
+    _check('ht (no g/beta)', ref_ht, ht)
+    o, none = op(q.to(dev), k.to(dev), v.to(dev), graw.to(dev) * 0 - 0.1)
+    assert none is None
+
+
+def test_host_validation_errors():
+    op = _ops()
+    dev = 'cuda'
+    q = torch.randn(2, 4, 2, 64, device=dev)
+    v = torch.randn(2, 4, 4, 64, device=dev)
+    g = torch.zeros(2, 4, 4, device=dev)
+    with pytest.raises(ValueError):
+        op(q, q, v, g, cu_seqlens=torch.tensor([0, 4, 8], device=dev))          # batch must be 1
+    with pytest.raises(ValueError):
+        op(q[:1], q[:1], v[:1], g[:1], initial_state=torch.zeros(3, 4, 64, 64, device=dev),
+           cu_seqlens=torch.tensor([0, 2, 4], device=dev))                       # len(h0) != N
+    with pytest.raises(ValueError):
+        op(q, q, v, g, allow_neg_eigval=True)
+    with pytest.raises(ValueError):
+        op(q, q, v, g, use_gate_in_kernel=True)
+    with pytest.raises(ValueError):
+        op(q, q, v, g, state_v_first=True, transpose_state_layout=True)
+    with pytest.raises(RuntimeError):
+        op(q.cpu(), q.cpu(), v.cpu(), g.cpu())                                   # no CPU path
