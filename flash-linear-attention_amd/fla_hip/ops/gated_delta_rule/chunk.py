@@ -27,7 +27,7 @@ from fla_hip.utils import input_guard
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
 # the chunk size (only rounding does), so chunk_size 16 and 32 are accepted and run with 64.
 _KERNEL_CHUNK = 64
-_KERNEL_DIMS = (64, 128)        # head dims the MFMA kernels are instantiated for
+_KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 
 def _l2norm_rows(x: torch.Tensor) -> torch.Tensor:

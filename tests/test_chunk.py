@@ -1,0 +1,180 @@
+"""GPU parity of chunk_gated_delta_rule (HIP, through the C ABI) against the fp32 CPU oracle
+on the same seeded inputs.  Cases follow the reference's matrix for this operator
+(tests/ops/test_gdn.py:108-200, :712-878, :1350-1478; tests/ops/test_gdn_kernels.py:587-627)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# o and final state: relative RMSE <= 5e-3 and max-abs-error ratio <= 1e-2 vs the fp32 oracle
+RATIO, MAXABS = 5e-3, 1e-2
+
+
+def _op():
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    return chunk_gated_delta_rule
+
+
+def _check(name, ref, got, ratio=RATIO, maxabs=MAXABS):
+    got = got.detach().float().cpu()
+    assert got.shape == ref.shape, f'{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}'
+    assert not torch.isnan(got).any(), f'{name}: NaN'
+    r, m = O.get_err_ratio(ref, got), O.max_abs_ratio(ref, got)
+    assert r <= ratio and m <= maxabs, f'{name}: rel-rmse {r:.3e} max-abs ratio {m:.3e}'
+    return r, m
+
+
+def _run(q, k, v, g, beta, h0=None, cu=None, **kw):
+    dev = 'cuda'
+    cu_t = None if cu is None else torch.tensor(cu, dtype=kw.pop('idx_dtype', torch.int64), device=dev)
+    return _op()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta.to(dev),
+                 initial_state=None if h0 is None else h0.to(dev), output_final_state=True, cu_seqlens=cu_t, **kw)
+
+
+@pytest.mark.parametrize('B,T,H,HV,D,gate_div,with_h0,dtype', [
+    (1, 64, 1, 1, 128, 1.0, False, torch.bfloat16),
+    (2, 256, 2, 2, 128, 1.0, False, torch.bfloat16),
+    (1, 130, 2, 4, 128, 16.0, True, torch.bfloat16),       # GVA, ragged tail chunk, non-zero h0
+    (2, 1000, 2, 8, 128, 16.0, True, torch.bfloat16),
+    (2, 75, 2, 2, 128, 1.0, True, torch.float16),
+    (1, 1024, 4, 4, 128, 16.0, True, torch.float16),
+    (2, 512, 2, 2, 64, 1.0, True, torch.bfloat16),         # padded to 128 on the host
+    (2, 500, 2, 4, 60, 16.0, True, torch.float16),
+    (1, 300, 3, 3, 100, 1.0, False, torch.bfloat16),
+    (2, 256, 2, 2, 64, 1.0, False, torch.float32),         # config 1 shape; fp32 inputs run as bf16
+])
+def test_chunk_vs_oracle(B, T, H, HV, D, gate_div, with_h0, dtype):
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, D, D, seed=42, gate_div=gate_div,
+                                         h0_std=0.5 if with_h0 else None, dtype=dtype)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    o, ht = _run(q, k, v, g, beta, h0)
+    assert o.dtype == q.dtype and ht.dtype == torch.float32
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+def test_against_token_recurrence_and_decode_handoff():
+    """Prefill with the chunk op, continue with the recurrent op: equals one long recurrence."""
+    from fla_hip.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = O.make_inputs(2, 300, 2, 4, 128, 128, seed=7, gate_div=4.0, h0_std=0.3, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    dev = 'cuda'
+    a = [x.to(dev) for x in (q, k, v, g, beta)]
+    o1, h1 = _op()(*(x[:, :290] for x in a), initial_state=h0.to(dev), output_final_state=True)
+    o2, h2 = fused_recurrent_gated_delta_rule(a[0][:, 290:], a[1][:, 290:], a[2][:, 290:], a[3][:, 290:], beta=a[4][:, 290:],
+                                              initial_state=h1, output_final_state=True)
+    _check('o', ref_o, torch.cat([o1, o2], 1))
+    _check('ht', ref_ht, h2)
+
+
+@pytest.mark.parametrize('cu,H,HV,D', [
+    ([0, 15], 2, 2, 128),
+    ([0, 256, 500, 1000], 2, 4, 128),
+    ([0, 1, 100, 101, 300, 1200, 2000], 2, 8, 128),
+    ([0, 15, 100, 300, 1200, 2000], 2, 4, 64),
+])
+@pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
+def test_varlen_vs_oracle_and_bit_exact_ownership(cu, H, HV, D, idx_dtype):
+    T, N = cu[-1], len(cu) - 1
+    q, k, v, g, beta, h0 = O.make_inputs(1, T, H, HV, D, D, seed=11, gate_div=2.0, h0_std=0.5, N=N, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)
+    o, ht = _run(q, k, v, g, beta, h0, cu, idx_dtype=idx_dtype)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    # every sequence run alone through the same kernels reproduces the packed result bit for bit
+    for n, (s, e) in enumerate(zip(cu[:-1], cu[1:])):
+        o_n, h_n = _run(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e], h0[n:n + 1])
+        assert torch.equal(o_n[0], o[0, s:e]), f'sequence {n}: o differs'
+        assert torch.equal(h_n[0], ht[n]), f'sequence {n}: state differs'
+
+
+def test_many_documents_equals_two_halves():
+    """More (document, head) pairs than a 16-bit grid dimension holds
+    (tests/ops/test_gdn_kernels.py:587-627): 2050 documents of 16 tokens, HV = 32."""
+    ND, L, H, D = 2050, 16, 32, 128
+    T = ND * L
+    gen = torch.Generator().manual_seed(0)
+    q = F.normalize(torch.randn(1, T, H, D, generator=gen), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(1, T, H, D, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(1, T, H, generator=gen))
+    beta = torch.sigmoid(torch.randn(1, T, H, generator=gen))
+    cu = list(range(0, T + 1, L))
+    o, ht = _run(q, k, v, g, beta, None, cu)
+    half = (ND // 2) * L
+    o1, h1 = _run(q[:, :half], k[:, :half], v[:, :half], g[:, :half], beta[:, :half], None, cu[:ND // 2 + 1])
+    o2, h2 = _run(q[:, half:], k[:, half:], v[:, half:], g[:, half:], beta[:, half:], None,
+                  [c - half for c in cu[ND // 2:]])
+    assert torch.equal(torch.cat([o1, o2], 1), o) and torch.equal(torch.cat([h1, h2], 0), ht)
+    # spot-check a few documents against the oracle
+    for n in (0, 1024, 2049):
+        s, e = cu[n], cu[n + 1]
+        ref_o, ref_h = O.recurrent_gated_delta_rule(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e], None, None, True)
+        _check(f'o[{n}]', ref_o[0], o[0, s:e])
+        _check(f'ht[{n}]', ref_h[0], ht[n])
+
+
+def test_flags_and_state_layout():
+    B, T, H, HV, D = 2, 200, 2, 4, 128
+    gen = torch.Generator().manual_seed(5)
+    q, k = torch.randn(B, T, H, D, generator=gen).bfloat16(), torch.randn(B, T, H, D, generator=gen).bfloat16()
+    v = torch.randn(B, T, HV, D, generator=gen).bfloat16()
+    graw, braw = torch.randn(B, T, HV, generator=gen), torch.randn(B, T, HV, generator=gen)
+    A_log, dt_bias = 0.3 * torch.randn(HV, generator=gen), 0.3 * torch.randn(HV, generator=gen)
+    h0 = 0.5 * torch.randn(B, HV, D, D, generator=gen)
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, use_beta_sigmoid_in_kernel=True, allow_neg_eigval=False)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, graw, braw, None, h0, True, A_log=A_log, dt_bias=dt_bias, **kw)
+    o, ht = _run(q, k, v, graw, braw, h0, A_log=A_log.cuda(), dt_bias=dt_bias.cuda(), **kw)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    o2, ht2 = _run(q, k, v, graw, braw, h0.transpose(-1, -2).contiguous(), A_log=A_log.cuda(), dt_bias=dt_bias.cuda(),
+                   state_v_first=True, **kw)
+    assert ht2.shape == (B, HV, D, D)
+    assert torch.equal(o2, o) and torch.equal(ht2.transpose(-1, -2), ht)      # same kernels, transposed I/O only
+    for cs in (16, 32):
+        o3, ht3 = _run(q, k, v, graw, braw, h0, A_log=A_log.cuda(), dt_bias=dt_bias.cuda(), chunk_size=cs, **kw)
+        _check(f'o chunk_size={cs}', ref_o, o3)
+
+
+def test_outputs_fully_written_and_deterministic():
+    """Two runs agree bit for bit and every output element is written (no NaN survives from
+    poisoned allocations: the workspace and outputs come from torch.empty)."""
+    q, k, v, g, beta, h0 = O.make_inputs(2, 333, 2, 4, 128, 128, seed=3, gate_div=8.0, h0_std=0.2, dtype=torch.bfloat16)
+    junk = torch.full((64, 1024, 1024), float('nan'), device='cuda')      # poison the caching allocator's pool
+    del junk
+    o1, h1 = _run(q, k, v, g, beta, h0)
+    junk = torch.full((64, 1024, 1024), float('nan'), device='cuda')
+    del junk
+    o2, h2 = _run(q, k, v, g, beta, h0)
+    assert not torch.isnan(o1).any() and not torch.isnan(h1).any()
+    assert torch.equal(o1, o2) and torch.equal(h1, h2)
+
+
+def test_host_validation_errors():
+    op = _op()
+    dev = 'cuda'
+    q = torch.randn(2, 64, 2, 128, device=dev, dtype=torch.bfloat16)
+    v = torch.randn(2, 64, 4, 128, device=dev, dtype=torch.bfloat16)
+    g = torch.zeros(2, 64, 4, device=dev)
+    with pytest.raises(ValueError):
+        op(q, q[:, :, :1], v, g, g)                                              # q/k head mismatch
+    with pytest.raises(ValueError):
+        op(q, q, v[:, :, :3], g[:, :, :3], g[:, :, :3])                          # HV % H
+    with pytest.raises(ValueError):
+        op(q, q, v, g, g, chunk_size=48)
+    with pytest.raises(ValueError):
+        op(q, q, v, g, g, cu_seqlens=torch.tensor([0, 64, 128], device=dev))     # batch must be 1
+    with pytest.raises(ValueError):
+        op(q[:1], q[:1], v[:1], g[:1], g[:1], initial_state=torch.zeros(3, 4, 128, 128, device=dev),
+           cu_seqlens=torch.tensor([0, 32, 64], device=dev))
+    with pytest.raises(ValueError):
+        op(q, q, v, g, g, allow_neg_eigval=True)
+    with pytest.raises(AssertionError):
+        op(q, q, v, g, g, use_gate_in_kernel=True)
+    with pytest.raises(DeprecationWarning):
+        op(q, q, v, g, g, head_first=True)
+    with pytest.raises(RuntimeError):
+        op(q.cpu(), q.cpu(), v.cpu(), g.cpu(), g.cpu())                          # no CPU path
