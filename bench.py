@@ -1,0 +1,262 @@
+"""Benchmark of the gated delta rule inference path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode]
+
+Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
+K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
+configuration the >= 50 %-of-MFMA-roofline target is quoted on.  A step is one call of
+chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries, under
+"other_workloads", the decode step (B=256: us/step and state GB/s) and the other prefill
+configurations, and:
+  roofline      dominant kernel, algorithmic FLOPs (or bytes) per launch / its mean duration
+                measured with HIP events on the launch stream
+  cpu_baseline  the CPU oracle (torch fp32, all host cores) on a bounded sample of the workload
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, 'flash-linear-attention_amd')):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+import torch.nn.functional as F  # noqa: E402
+
+C, K, V = 64, 128, 128
+# algorithmic FLOPs per (token, v-head): 2*(3CK + 2CV + 3KV); the scan kernel does w*S, k^T*v_new,
+# q*S (3KV) and P*v_new (CV), the prepare kernel K K^T, q k^T, w (3CK) and u (CV)
+F_SCAN = 2 * (3 * K * V + C * V)
+F_PREP = 2 * (3 * C * K + C * V)
+F_TOTAL = F_SCAN + F_PREP                      # 180224
+PEAK_BF16_TFLOPS = 2500.0                      # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0                          # MI355X HBM3E, published
+
+WORKLOADS = {
+    'prefill': dict(kind='prefill', B=1, T=32768, H=16, HV=32, h0=True, varlen=False,
+                    name='configs[2]: GDN chunk prefill B=1 T=32768 Hqk=16 Hv=32 K=V=128 bf16, fp32 state'),
+    'prefill_b4': dict(kind='prefill', B=4, T=4096, H=16, HV=16, h0=False, varlen=False,
+                       name='configs[1]: GDN chunk prefill B=4 T=4096 H=16 K=V=128 bf16, fp32 state'),
+    'varlen': dict(kind='prefill', B=1, T=65536, H=16, HV=32, h0=True, varlen=True,
+                   name='configs[3]: GDN varlen prefill 65536 tokens in 32 sequences Hqk=16 Hv=32 K=V=128 bf16'),
+    'decode': dict(kind='decode', N=256, H=16, HV=32,
+                   name='configs[4]: GDN single-token decode batch=256 Hqk=16 Hv=32 K=V=128 bf16, fp32 states in place'),
+}
+
+
+def _ensure_built():
+    from fla_hip import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+
+
+def make_prefill_inputs(w, device):
+    from oracle import gdn_oracle as O
+    gen = torch.Generator().manual_seed(42)
+    B, T, H, HV = w['B'], w['T'], w['H'], w['HV']
+    q = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1).bfloat16()
+    k = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1).bfloat16()
+    v = torch.randn(B, T, HV, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / 16
+    beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
+    cu = None
+    N = B
+    if w['varlen']:
+        lens = O.make_varlen_lengths(T, 32, 256, 4096, seed=42)
+        cu = [0]
+        for x in lens:
+            cu.append(cu[-1] + x)
+        N = 32
+    h0 = 0.1 * torch.randn(N, HV, K, V, generator=gen) if w['h0'] else None
+    cpu = dict(q=q, k=k, v=v, g=g, beta=beta, h0=h0, cu=cu)
+    dev = {key: (val.to(device) if isinstance(val, torch.Tensor) else val) for key, val in cpu.items()}
+    dev['cu_t'] = None if cu is None else torch.tensor(cu, dtype=torch.int64, device=device)
+    dev['cu_cpu'] = None if cu is None else torch.tensor(cu, dtype=torch.int64)
+    return cpu, dev
+
+
+def bench_prefill(w, steps, warmup, device, with_cpu):
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
+    cpu, d = make_prefill_inputs(w, device)
+    tokens = w['B'] * w['T']
+
+    def step():
+        return chunk_gated_delta_rule(d['q'], d['k'], d['v'], d['g'], d['beta'], initial_state=d['h0'],
+                                      output_final_state=True, cu_seqlens=d['cu_t'], cu_seqlens_cpu=d['cu_cpu'])
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / steps * 1e3
+
+    # per-kernel durations: the same work issued as its two stages with HIP events in between
+    call = ChunkLaunch(d['q'], d['k'], d['v'], d['g'], d['beta'], K ** -0.5, d['h0'], True, False,
+                       d['cu_t'], d['cu_cpu'], None, 64)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for i in range(steps):
+        ev[i][0].record()
+        call.run('prepare')
+        ev[i][1].record()
+        call.run('scan')
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    t_prep = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e-3
+    t_scan = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e-3
+    units = tokens * w['HV']
+    dom = ('gdn_chunk_scan_kernel', F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_prepare_kernel', F_PREP, t_prep)
+    achieved = units * dom[1] / dom[2] / 1e12
+    roofline = dict(bound='mfma', achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit='TFLOP/s',
+                    frac=round(achieved / PEAK_BF16_TFLOPS, 5), traffic=None, kernel=dom[0],
+                    kernel_us=round(dom[2] * 1e6, 1), flops_per_launch=units * dom[1],
+                    kernels_us=dict(gdn_chunk_prepare_kernel=round(t_prep * 1e6, 1), gdn_chunk_scan_kernel=round(t_scan * 1e6, 1)),
+                    whole_op=dict(flops=units * F_TOTAL, achieved=round(units * F_TOTAL / (elapsed / steps) / 1e12, 2),
+                                  frac=round(units * F_TOTAL / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 5)))
+    out = dict(value=tokens * steps / elapsed, ms_per_step=ms_per_step, roofline=roofline)
+
+    if with_cpu:
+        out['cpu_baseline'] = cpu_baseline_prefill(w, cpu)
+        # parity of this very workload's head of the sequence against the oracle
+    return out
+
+
+def cpu_baseline_prefill(w, cpu):
+    """Oracle (torch fp32 chunked form) on the first tokens of the same inputs; the sample
+    length is chosen from a short calibration run so that the timed run takes ~10-20 s."""
+    from oracle import gdn_oracle as O
+    torch.set_num_threads(os.cpu_count() or 1)
+
+    def run(T_s):
+        sl = slice(0, T_s)
+        h0 = None if cpu['h0'] is None else cpu['h0'][:cpu['q'].shape[0]]
+        t0 = time.perf_counter()
+        O.chunk_gated_delta_rule(cpu['q'][:, sl], cpu['k'][:, sl], cpu['v'][:, sl], cpu['g'][:, sl], cpu['beta'][:, sl],
+                                 None, h0, True)
+        return time.perf_counter() - t0
+
+    t_cal = run(512)
+    rate = 512 * cpu['q'].shape[0] / t_cal
+    T_s = int(min(cpu['q'].shape[1], max(1024, (rate * 12 / cpu['q'].shape[0]) // 64 * 64)))
+    t = run(T_s)
+    toks = T_s * cpu['q'].shape[0]
+    return dict(value=round(toks / t, 1), unit='tokens/s', cores=torch.get_num_threads(), kind='port',
+                sample=f'oracle chunk_gated_delta_rule (torch fp32 CPU) on the first {T_s} tokens per sequence of the same '
+                       f'inputs, {t:.1f} s wall, dense (not packed) layout', seconds=round(t, 2))
+
+
+def bench_decode(w, steps, warmup, device, with_cpu):
+    from fla_hip.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    N, H, HV = w['N'], w['H'], w['HV']
+    gen = torch.Generator().manual_seed(42)
+    q = F.normalize(torch.randn(N, 1, H, K, generator=gen), p=2, dim=-1).bfloat16()
+    k = F.normalize(torch.randn(N, 1, H, K, generator=gen), p=2, dim=-1).bfloat16()
+    v = torch.randn(N, 1, HV, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(N, 1, HV, generator=gen))
+    beta = torch.sigmoid(torch.randn(N, 1, HV, generator=gen))
+    h0 = 0.1 * torch.randn(N, HV, K, V, generator=gen)
+    dq, dk, dv, dg, db = (x.to(device) for x in (q, k, v, g, beta))
+    # two state pools used alternately: each step streams 2 x 512 MiB, more than the 256 MB Infinity Cache
+    states = [h0.to(device), h0.to(device)]
+
+    def step(i):
+        return fused_recurrent_gated_delta_rule(dq, dk, dv, dg, beta=db, initial_state=states[i & 1],
+                                                output_final_state=True, inplace_final_state=True)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    t_kernel = statistics.mean(ev[i].elapsed_time(ev[i + 1]) for i in range(steps)) * 1e-3
+    state_bytes = 2 * N * HV * K * V * 4
+    achieved = state_bytes / t_kernel / 1e9
+    roofline = dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
+                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None, kernel='gdn_recurrent_kernel',
+                    kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=state_bytes)
+    out = dict(value=elapsed / steps * 1e6, ms_per_step=elapsed / steps * 1e3, roofline=roofline)
+    if with_cpu:
+        from oracle import gdn_oracle as O
+        torch.set_num_threads(os.cpu_count() or 1)
+        S = h0.clone()
+        reps = 3
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            o_ref, S = O.decode_step(q[:, 0], k[:, 0], v[:, 0], g[:, 0], beta[:, 0], S)
+        t = (time.perf_counter() - t0) / reps
+        out['cpu_baseline'] = dict(value=round(t * 1e6, 1), unit='us/step', cores=torch.get_num_threads(), kind='port',
+                                   sample=f'oracle decode_step (torch fp32 CPU), full batch of {N}, mean of {reps} steps',
+                                   seconds=round(t * reps, 2))
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS))
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this build measures ONE GPU only (every sequence and v-head is independent, so more GPUs '
+              'shard them with no communication); run it with --gpus 1.', file=sys.stderr)
+        sys.exit(2)
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    _ensure_built()
+    device = 'cuda:0'
+    torch.cuda.set_device(0)
+
+    w = WORKLOADS[args.workload]
+    fn = bench_prefill if w['kind'] == 'prefill' else bench_decode
+    res = fn(w, args.steps, args.warmup, device, not args.no_cpu_baseline)
+    if w['kind'] == 'prefill':
+        line = dict(metric='gdn_chunk_prefill_tokens_per_s', value=round(res['value'], 1), unit='tokens/s', higher_is_better=True)
+    else:
+        line = dict(metric='gdn_decode_us_per_step', value=round(res['value'], 2), unit='us/step', higher_is_better=False)
+    line.update(n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(res['ms_per_step'], 4), scaling='weak',
+                vs_baseline=None, dtype='bf16', data='synthetic', config=dict(workload=w['name'], chunk_size=64),
+                roofline=res['roofline'])
+    if 'cpu_baseline' in res:
+        line['cpu_baseline'] = res['cpu_baseline']
+    if not args.no_extra:
+        extra = {}
+        for name, ww in WORKLOADS.items():
+            if name == args.workload:
+                continue
+            f2 = bench_prefill if ww['kind'] == 'prefill' else bench_decode
+            r = f2(ww, args.steps, args.warmup, device, ww['kind'] == 'decode' and not args.no_cpu_baseline)
+            e = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), roofline=r['roofline'])
+            if ww['kind'] == 'prefill':
+                e['tokens_per_s'] = round(r['value'], 1)
+            else:
+                e['us_per_step'] = round(r['value'], 2)
+                e['state_GBps'] = r['roofline']['achieved']
+            if 'cpu_baseline' in r:
+                e['cpu_baseline'] = r['cpu_baseline']
+            extra[name] = e
+            torch.cuda.empty_cache()
+        line['other_workloads'] = extra
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

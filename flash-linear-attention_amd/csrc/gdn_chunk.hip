@@ -84,6 +84,17 @@ struct ChunkParams {
     int nslab; int64_t NH;
 };
 
+// Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains
+// the vector-memory counter, which would serialise the global prefetch of the next chunk
+// behind every barrier of the current one.
+#ifndef GDN_EXP
+#define GDN_EXP 0
+#endif
+__device__ __forceinline__ void lds_barrier() {
+    if (GDN_EXP == 3) return;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // 16x16 product of fp32 matrices held in LDS on the fp32 matrix cores:
 // C = A[16 x 4*nk] * B[4*nk x 16]; result in C/D layout.
 __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* B, int ldb, int nk, int c16, int g) {
@@ -456,7 +467,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             V4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (trow < f.valid) {
+            if (trow < f.valid && GDN_EXP != 2) {
                 a = *(const V4*)(qrow + 32 * s);
                 b = *(const V4*)(qrow + 32 * s + 16);
             }
@@ -483,7 +494,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
     if (nt > 0) load_frags(0, cur);
     nxt = cur;
     for (int64_t it = 0; it < nt; ++it) {
-        if (it + 1 < nt) load_frags(it + 1, nxt);
+        if (it + 1 < nt && GDN_EXP != 4) load_frags(it + 1, nxt);
         // (a) publish the state of this chunk as bf16/f16 B-operand fragments
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn) {
@@ -495,7 +506,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
             }
             sSb[(w * NV + nn) * 64 + lane] = f;
         }
-        __syncthreads();
+        lds_barrier();
         // (b,c) w S and q S for t-tile w
         f32x4 accv[NV], acco[NV];
 #pragma unroll
@@ -530,7 +541,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
             sVn[(((0 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = plain;
             sVn[(((1 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = gated;
         }
-        __syncthreads();
+        lds_barrier();
         // (e,f) state update and output
         const float gl2 = exp2f(glast);
         const V8* sVn8 = (const V8*)sVn;
@@ -551,7 +562,11 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = 16 * w + 4 * g + r;
+#if GDN_EXP != 1
                 if (t < cur.valid) og[((tok0 + t) * HV + hv) * 128 + v0 + 16 * nn + c16] = from_f32<T>(ao[r] * p.scale);
+#else
+                if (ao[r] == 12345.f) og[((tok0 + t) * HV + hv) * 128 + v0 + 16 * nn + c16] = from_f32<T>(ao[r] * p.scale);
+#endif
             }
         }
         cur = nxt;
@@ -589,9 +604,11 @@ static int launch_scan(const ChunkParams& p0, hipStream_t stream) {
     return check_launch("gdn_chunk_scan_kernel");
 }
 
+constexpr int STAGE_PREPARE = 1, STAGE_SCAN = 2;
+
 template <typename T>
-static int launch_chunk(const ChunkParams& p, int64_t num_chunks, hipStream_t stream) {
-    {
+static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hipStream_t stream) {
+    if (stages & STAGE_PREPARE) {
         auto kern = gdn_chunk_prepare_kernel<T>;
         static bool attr_done = false;       // per instantiation
         if (!attr_done) {
@@ -604,6 +621,7 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, hipStream_t st
         int rc = check_launch("gdn_chunk_prepare_kernel");
         if (rc) return rc;
     }
+    if (!(stages & STAGE_SCAN)) return GDN_OK;
     // widest value slab that still gives every CU a workgroup
     if (p.NH >= 256) return launch_scan<T, 8>(p, stream);
     if (p.NH * 2 >= 256) return launch_scan<T, 4>(p, stream);
@@ -618,7 +636,8 @@ extern "C" size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64
     return gdn::ws_layout(num_chunks, H, HV, nullptr, nullptr);
 }
 
-extern "C" int gdn_chunk_fwd(
+static int chunk_entry(
+    const char* who, int stages,
     const void* q, const void* k, const void* v, const void* g, const void* beta,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
@@ -627,33 +646,56 @@ extern "C" int gdn_chunk_fwd(
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "gdn_chunk_fwd: q, k, v, g, beta, o must not be NULL");
-    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "gdn_chunk_fwd: non-positive dimension");
-    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "gdn_chunk_fwd: HV=%lld not divisible by H=%lld", (long long)HV, (long long)H);
-    GDN_CHECK_ARG(K == 128 && V == 128, GDN_ERR_UNSUPPORTED, "gdn_chunk_fwd: only K = V = 128 is built (got K=%lld V=%lld)",
+    GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "%s: non-positive dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
+    GDN_CHECK_ARG(K == 128 && V == 128, GDN_ERR_UNSUPPORTED, "%s: only K = V = 128 is built (got K=%lld V=%lld)", who,
                   (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
-                  "gdn_chunk_fwd: q/k/v must be bf16 or f16");
-    GDN_CHECK_ARG(HV <= 65535, GDN_ERR_UNSUPPORTED, "gdn_chunk_fwd: HV > 65535");
+                  "%s: q/k/v must be bf16 or f16", who);
+    GDN_CHECK_ARG(HV <= 65535, GDN_ERR_UNSUPPORTED, "%s: HV > 65535", who);
     if (cu_seqlens) {
-        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "gdn_chunk_fwd: with cu_seqlens B must be 1");
-        GDN_CHECK_ARG(chunk_table && chunk_offsets, GDN_ERR_INVALID, "gdn_chunk_fwd: packed input needs chunk_table and chunk_offsets");
+        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
+        GDN_CHECK_ARG(chunk_table && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
     } else {
-        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "gdn_chunk_fwd: without cu_seqlens N must equal B");
-        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "gdn_chunk_fwd: num_chunks does not match B and T");
+        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
+        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
     }
     GDN_CHECK_ARG(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0 && ((uintptr_t)h0 % 16) == 0 &&
                       ((uintptr_t)ht % 16) == 0 && ((uintptr_t)workspace % 256) == 0,
-                  GDN_ERR_INVALID, "gdn_chunk_fwd: q/k/v/h0/ht must be 16-byte and the workspace 256-byte aligned");
+                  GDN_ERR_INVALID, "%s: q/k/v/h0/ht must be 16-byte and the workspace 256-byte aligned", who);
     if (T == 0 || num_chunks == 0) return GDN_OK;
     ChunkParams p;
     const size_t need = ws_layout(num_chunks, H, HV, (char*)workspace, &p.ws);
-    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "gdn_chunk_fwd: workspace of %zu bytes needed, %zu given",
+    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.nslab = 1; p.NH = N * HV;
     hipStream_t s = (hipStream_t)stream;
-    return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, s) : launch_chunk<f16_t>(p, num_chunks, s);
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, stages, s)
+                                       : launch_chunk<f16_t>(p, num_chunks, stages, s);
+}
+
+#define GDN_CHUNK_ARGS                                                                          \
+    const void *q, const void *k, const void *v, const void *g, const void *beta,               \
+    const float *h0, float *ht, void *o,                                                        \
+    const void *cu_seqlens, const void *chunk_table, const void *chunk_offsets,                 \
+    void *workspace, size_t workspace_bytes,                                                    \
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,                          \
+    int64_t N, int64_t num_chunks,                                                              \
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void *stream
+#define GDN_CHUNK_PASS                                                                          \
+    q, k, v, g, beta, h0, ht, o, cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, \
+    B, T, H, HV, K, V, N, num_chunks, scale, qkv_dtype, gb_dtype, flags, stream
+
+extern "C" int gdn_chunk_fwd(GDN_CHUNK_ARGS) {
+    return chunk_entry("gdn_chunk_fwd", gdn::STAGE_PREPARE | gdn::STAGE_SCAN, GDN_CHUNK_PASS);
+}
+extern "C" int gdn_chunk_fwd_prepare(GDN_CHUNK_ARGS) {
+    return chunk_entry("gdn_chunk_fwd_prepare", gdn::STAGE_PREPARE, GDN_CHUNK_PASS);
+}
+extern "C" int gdn_chunk_fwd_scan(GDN_CHUNK_ARGS) {
+    return chunk_entry("gdn_chunk_fwd_scan", gdn::STAGE_SCAN, GDN_CHUNK_PASS);
 }

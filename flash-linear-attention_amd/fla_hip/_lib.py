@@ -7,7 +7,7 @@ import threading
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, '_C', 'libgdn_hip.so')
+LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
 ABI_VERSION = 1
 
@@ -39,15 +39,17 @@ SIGNATURES = {
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
         c_float, c_int, c_int, c_uint32, c_void_p]),
     'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
-    'gdn_chunk_fwd': (c_int, [
-        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k v g beta
-        c_void_p, c_void_p, c_void_p,                      # h0 ht o
-        c_void_p, c_void_p, c_void_p,                      # cu_seqlens chunk_table chunk_offsets
-        c_void_p, c_size_t,                                # workspace, bytes
-        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V
-        c_int64, c_int64,                                  # N num_chunks
-        c_float, c_int, c_int, c_uint32, c_void_p]),
 }
+_CHUNK_ARGS = [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # q k v g beta
+    c_void_p, c_void_p, c_void_p,                          # h0 ht o
+    c_void_p, c_void_p, c_void_p,                          # cu_seqlens chunk_table chunk_offsets
+    c_void_p, c_size_t,                                    # workspace, bytes
+    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,  # B T H HV K V
+    c_int64, c_int64,                                      # N num_chunks
+    c_float, c_int, c_int, c_uint32, c_void_p]
+for _name in ('gdn_chunk_fwd', 'gdn_chunk_fwd_prepare', 'gdn_chunk_fwd_scan'):
+    SIGNATURES[_name] = (c_int, _CHUNK_ARGS)
 
 _lib = None
 _lock = threading.Lock()

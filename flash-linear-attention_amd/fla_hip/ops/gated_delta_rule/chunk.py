@@ -50,6 +50,102 @@ def _kernel_dim(d: int) -> int:
     raise NotImplementedError(f'head dim {d} > {_KERNEL_DIMS[-1]} is not supported by the HIP chunk kernels')
 
 
+class ChunkLaunch:
+    """Everything one forward call hands to the C ABI: normalised inputs, freshly allocated
+    outputs and workspace, and the argument tuple of ``gdn_chunk_fwd``.  ``run()`` launches the
+    whole operator; ``run('prepare')`` / ``run('scan')`` launch its two stages separately (same
+    arguments), which is how the benchmark attributes time to each kernel."""
+
+    _ENTRY = {None: 'gdn_chunk_fwd', 'prepare': 'gdn_chunk_fwd_prepare', 'scan': 'gdn_chunk_fwd_scan'}
+
+    def __init__(self, q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first=False,
+                 cu_seqlens=None, cu_seqlens_cpu=None, chunk_indices=None, chunk_size=64):
+        dev = require_gpu(q, k, v, g, beta)
+        B, T, H, K = k.shape
+        HV, V = v.shape[2], v.shape[3]
+        N = B if cu_seqlens is None else len(cu_seqlens) - 1
+        self.out_dtype = q.dtype
+        self.dims = (B, T, H, HV, K, V, N)
+        self.state_v_first = state_v_first
+
+        # the MFMA kernels take bf16 or fp16 operands; fp32 inputs are rounded to bf16 first
+        work_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+        q, k, v = q.to(work_dtype), k.to(work_dtype), v.to(work_dtype)
+        # head dims below 128 are zero-padded: zero key features and zero value columns change
+        # neither the other columns of the output nor the state entries that are kept
+        KP, VP = _kernel_dim(K), _kernel_dim(V)
+        KP = VP = max(KP, VP)
+        self.padded = (KP, VP)
+        q, k, v = _pad_last(q, KP), _pad_last(k, KP), _pad_last(v, VP)
+        g, beta, gb_code = unify_gate_beta(g, beta)
+
+        flags = _lib.FLAG_STATE_V_FIRST if state_v_first else 0
+        if cu_seqlens is not None:
+            if cu_seqlens.dtype not in (torch.int32, torch.int64):
+                cu_seqlens = cu_seqlens.long()
+            if cu_seqlens.device != dev:
+                cu_seqlens = cu_seqlens.to(dev)
+            if cu_seqlens.dtype == torch.int32:
+                flags |= _lib.FLAG_CU_INT32
+            if chunk_indices is None or chunk_size != _KERNEL_CHUNK:
+                chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+            chunk_indices = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+            chunk_offsets = prepare_chunk_offsets(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+            num_chunks = chunk_indices.shape[0]
+        else:
+            chunk_indices = chunk_offsets = None
+            num_chunks = B * ((T + _KERNEL_CHUNK - 1) // _KERNEL_CHUNK)
+
+        state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+        h0 = initial_state
+        if h0 is not None:
+            if tuple(h0.shape) != state_shape:
+                raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
+            h0 = as_f32(h0)
+            if (KP, VP) != (K, V):
+                h0 = torch.nn.functional.pad(h0, (0, (KP if state_v_first else VP) - h0.shape[-1],
+                                                  0, (VP if state_v_first else KP) - h0.shape[-2]))
+            h0 = aligned16(h0.contiguous())
+
+        self.o = torch.empty(B, T, HV, VP, dtype=work_dtype, device=dev)
+        self.ht = None
+        if output_final_state:
+            self.ht = torch.empty((N, HV, VP, KP) if state_v_first else (N, HV, KP, VP), dtype=torch.float32, device=dev)
+        self.h0 = h0
+
+        self.lib = _lib.load()
+        ws_bytes = self.lib.gdn_chunk_workspace_bytes(num_chunks, H, HV, KP, VP)
+        if ws_bytes == 0 and num_chunks > 0:
+            raise NotImplementedError(f'HIP chunk kernels do not cover K={KP}, V={VP}')
+        self.workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+        self.keep = (q, k, v, g, beta, cu_seqlens, chunk_indices, chunk_offsets)     # keep the buffers alive
+        self.device = dev
+        self.args = (
+            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(self.ht), ptr(self.o),
+            ptr(cu_seqlens), ptr(chunk_indices), ptr(chunk_offsets),
+            ptr(self.workspace), ws_bytes,
+            B, T, H, HV, KP, VP, N, num_chunks,
+            float(scale), dtype_code(work_dtype), gb_code, flags)
+
+    def run(self, stage: str | None = None) -> None:
+        B, T = self.dims[0], self.dims[1]
+        if T > 0:
+            fn = getattr(self.lib, self._ENTRY[stage])
+            _lib.check(fn(*self.args, current_stream_ptr(self.device)))
+        elif self.ht is not None:
+            self.ht.copy_(self.h0) if self.h0 is not None else self.ht.zero_()
+
+    def results(self) -> tuple[torch.Tensor, torch.Tensor | None]:
+        B, T, H, HV, K, V, N = self.dims
+        KP, VP = self.padded
+        o, ht = self.o, self.ht
+        if VP != V:
+            o = o[..., :V]
+        if ht is not None and (KP, VP) != (K, V):
+            ht = (ht[..., :V, :K] if self.state_v_first else ht[..., :K, :V]).contiguous()
+        return o.to(self.out_dtype), ht
+
+
 @input_guard
 def chunk_gated_delta_rule_fwd(
     q: torch.Tensor,
@@ -68,78 +164,10 @@ def chunk_gated_delta_rule_fwd(
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Forward of the chunked operator on already-activated ``g`` (log space) and ``beta``.
     Returns ``(o in q's dtype, final_state fp32 or None)``."""
-    dev = require_gpu(q, k, v, g, beta)
-    B, T, H, K = k.shape
-    HV, V = v.shape[2], v.shape[3]
-    N = B if cu_seqlens is None else len(cu_seqlens) - 1
-    out_dtype = q.dtype
-
-    # the MFMA kernels take bf16 or fp16 operands; fp32 inputs are rounded to bf16 first
-    work_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-    q, k, v = q.to(work_dtype), k.to(work_dtype), v.to(work_dtype)
-    # head dims other than 64/128 are zero-padded: zero key features and zero value columns
-    # change neither the other columns nor the state rows that matter
-    KP, VP = _kernel_dim(K), _kernel_dim(V)
-    KP = VP = max(KP, VP)
-    q, k, v = _pad_last(q, KP), _pad_last(k, KP), _pad_last(v, VP)
-    g, beta, gb_code = unify_gate_beta(g, beta)
-
-    flags = 0
-    if cu_seqlens is not None:
-        if cu_seqlens.dtype not in (torch.int32, torch.int64):
-            cu_seqlens = cu_seqlens.long()
-        if cu_seqlens.device != dev:
-            cu_seqlens = cu_seqlens.to(dev)
-        if cu_seqlens.dtype == torch.int32:
-            flags |= _lib.FLAG_CU_INT32
-        if chunk_indices is None or chunk_size != _KERNEL_CHUNK:
-            chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
-        chunk_indices = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
-        chunk_offsets = prepare_chunk_offsets(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
-        num_chunks = chunk_indices.shape[0]
-    else:
-        chunk_indices = chunk_offsets = None
-        num_chunks = B * ((T + _KERNEL_CHUNK - 1) // _KERNEL_CHUNK)
-
-    state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
-    h0 = initial_state
-    if h0 is not None:
-        if tuple(h0.shape) != state_shape:
-            raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
-        h0 = as_f32(h0)
-        if (KP, VP) != (K, V):
-            h0 = torch.nn.functional.pad(h0, (0, (KP if state_v_first else VP) - h0.shape[-1],
-                                              0, (VP if state_v_first else KP) - h0.shape[-2]))
-        h0 = aligned16(h0.contiguous())
-        flags |= _lib.FLAG_STATE_V_FIRST if state_v_first else 0
-    elif state_v_first:
-        flags |= _lib.FLAG_STATE_V_FIRST
-
-    o = torch.empty(B, T, HV, VP, dtype=work_dtype, device=dev)
-    ht = None
-    if output_final_state:
-        ht = torch.empty((N, HV, VP, KP) if state_v_first else (N, HV, KP, VP), dtype=torch.float32, device=dev)
-
-    lib = _lib.load()
-    ws_bytes = lib.gdn_chunk_workspace_bytes(num_chunks, H, HV, KP, VP)
-    if ws_bytes == 0 and num_chunks > 0:
-        raise NotImplementedError(f'HIP chunk kernels do not cover K={KP}, V={VP}')
-    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    if T > 0:
-        _lib.check(lib.gdn_chunk_fwd(
-            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(ht), ptr(o),
-            ptr(cu_seqlens), ptr(chunk_indices), ptr(chunk_offsets),
-            ptr(workspace), ws_bytes,
-            B, T, H, HV, KP, VP, N, num_chunks,
-            float(scale), dtype_code(work_dtype), gb_code, flags, current_stream_ptr(dev)))
-    elif ht is not None:
-        ht.copy_(h0) if h0 is not None else ht.zero_()
-
-    if VP != V:
-        o = o[..., :V]
-    if ht is not None and (KP, VP) != (K, V):
-        ht = (ht[..., :V, :K] if state_v_first else ht[..., :K, :V]).contiguous()
-    return o.to(out_dtype), ht
+    call = ChunkLaunch(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first,
+                       cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size)
+    call.run()
+    return call.results()
 
 
 @dispatch('gated_delta_rule')

@@ -96,9 +96,36 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  *   chunk_offsets [N+1] (device; exclusive prefix sum of chunks per sequence) -
  *         prepare_chunk_offsets of fla/ops/utils/index.py:167-172; NULL for dense input
  *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
- *   Requires K == V == 128 (or 64), HV % H == 0.
+ *   Requires K == V == 128, HV % H == 0 (the Python host zero-pads smaller head dims).
  */
 int gdn_chunk_fwd(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
+ * The two stages of gdn_chunk_fwd as separate calls with the same argument list, so that a
+ * caller can time or overlap them.  gdn_chunk_fwd(...) == gdn_chunk_fwd_prepare(...) followed
+ * by gdn_chunk_fwd_scan(...) on the same stream and workspace.
+ *   prepare: the chunk-parallel part - chunk_local_cumsum, chunk_gated_delta_rule_fwd_intra
+ *            (gated beta*K*K^T, its unit-lower inverse, w, u) and the intra-chunk q*k^T of
+ *            chunk_fwd_o (fla/ops/common/chunk_o.py:107-139); fills the workspace.
+ *   scan:    chunk_gated_delta_rule_fwd_h fused with the rest of chunk_fwd_o; reads the
+ *            workspace, writes o and ht.
+ */
+int gdn_chunk_fwd_prepare(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+int gdn_chunk_fwd_scan(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,

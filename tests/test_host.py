@@ -1,0 +1,238 @@
+"""CPU-only tests: the C ABI library loads and exports what include/gdn_hip.h declares, and
+the host logic (index tables, caches, guards, dispatch registry, argument validation, naive
+torch forms) behaves like the reference's (tests/ops/utils/test_index.py, tests/ops/test_backends.py)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import gdn_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from fla_hip import _lib
+    header = open(os.path.join(ROOT, 'include', 'gdn_hip.h')).read()
+    header = re.sub(r'/\*.*?\*/', '', header, flags=re.S)
+    declared = set(re.findall(r'\b(gdn_[a-z0-9_]+)\s*\(', header))
+    assert declared == set(_lib.SIGNATURES), (declared, set(_lib.SIGNATURES))
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip('libgdn_hip.so not built in this checkout')
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f'{name} is declared in gdn_hip.h but missing from the library'
+    assert _lib.load().gdn_hip_abi_version() == _lib.ABI_VERSION
+    # pure host-side entry points can be called without a GPU
+    l = _lib.load()
+    assert l.gdn_chunk_workspace_bytes(8, 2, 4, 128, 128) > 0
+    assert l.gdn_chunk_workspace_bytes(8, 2, 4, 96, 128) == 0
+    # argument errors are reported before any launch
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None,
+                                   1, 1, 2, 3, 64, 64, 1, 1.0, 0, 2, 0, None)
+    assert rc == _lib.GDN_ERR_INVALID and 'divisible' in _lib.last_error()
+    with pytest.raises(ValueError):
+        _lib.check(rc)
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None,
+                                   1, 1, 1, 1, 512, 64, 1, 1.0, 0, 2, 0, None)
+    assert rc == _lib.GDN_ERR_UNSUPPORTED
+    with pytest.raises(NotImplementedError):
+        _lib.check(rc)
+
+
+@pytest.mark.parametrize('cu', [[0, 15], [0, 64], [0, 1, 65, 192, 193, 400], [0, 256, 500, 1000], [0, 100, 100, 164]])
+@pytest.mark.parametrize('dtype', [torch.int64, torch.int32])
+def test_chunk_tables_match_loop_reference(cu, dtype):
+    from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_chunk_offsets
+    t = torch.tensor(cu, dtype=dtype)
+    for cs in (16, 64):
+        idx = prepare_chunk_indices(t, cs)
+        assert idx.dtype == dtype and idx.tolist() == O.prepare_chunk_indices(cu, cs)
+        off = prepare_chunk_offsets(t, cs)
+        assert off.dtype == dtype and off.tolist() == O.prepare_chunk_offsets(cu, cs)
+        # host copy gives the same table
+        assert prepare_chunk_indices(t, cs, cu_seqlens_cpu=t.clone()).tolist() == idx.tolist()
+
+
+def test_tensor_cache_is_by_identity():
+    from fla_hip.utils import tensor_cache
+    calls = []
+
+    @tensor_cache
+    def f(x, n):
+        calls.append(1)
+        return x * n
+
+    a = torch.ones(3)
+    r1 = f(a, 2)
+    assert f(a, 2) is r1 and len(calls) == 1
+    f(a.clone(), 2)                      # equal values, different object: recomputed
+    assert len(calls) == 2
+    f(a, n=2)                            # different call shape: recomputed
+    assert len(calls) == 3
+
+
+def test_input_guard_makes_contiguous():
+    from fla_hip.utils import input_guard
+    seen = {}
+
+    @input_guard
+    def f(x, y=None):
+        seen['x'], seen['y'] = x.is_contiguous(), y.is_contiguous()
+        return x
+
+    @input_guard(no_guard_contiguous=['y'])
+    def g(x, y=None):
+        seen['x'], seen['y'] = x.is_contiguous(), y.is_contiguous()
+
+    a = torch.randn(4, 6).t()
+    f(a, y=a)
+    assert seen == {'x': True, 'y': True}
+    g(a, y=a)
+    assert seen == {'x': True, 'y': False}
+
+
+def test_dispatch_registry_priority_verifier_and_fallthrough(monkeypatch):
+    from fla_hip.ops.backends import BackendRegistry, BaseBackend, dispatch
+    reg = BackendRegistry('unit_test_op')
+    BackendRegistry._initialized.add('unit_test_op')
+    log = []
+
+    @dispatch('unit_test_op')
+    def op(x, flag=False):
+        log.append('default')
+        return x
+
+    class Low(BaseBackend):
+        backend_type, priority = 'low', 7
+
+        def op(self, x, flag=False):
+            log.append('low')
+            return x + 1
+
+    class High(BaseBackend):
+        backend_type, priority = 'high', 2
+
+        def op_verifier(self, x, flag=False):
+            if flag:
+                raise RuntimeError('boom')       # a raising verifier is a rejection
+            return x < 10, 'x too large'
+
+        def op(self, x, flag=False):
+            log.append('high')
+            return x + 100
+
+    class Gated(BaseBackend):
+        backend_type, priority, env_var, default_enable = 'gated', 0, 'UNIT_TEST_GATED', False
+
+        def op(self, x, flag=False):
+            log.append('gated')
+            return -1
+
+    class Missing(BaseBackend):
+        backend_type, priority, package_name = 'missing', 0, 'surely_not_an_installed_package_xyz'
+
+        def op(self, x, flag=False):
+            return -2
+
+    for b in (Low(), High(), Gated(), Missing()):
+        reg.register(b)
+    assert op(1) == 101 and log[-1] == 'high'             # lowest priority number wins
+    assert op(50) == 51 and log[-1] == 'low'              # verifier rejects -> next backend
+    assert op(1, flag=True) == 2 and log[-1] == 'low'     # verifier raised -> rejected, not an error
+    monkeypatch.setenv('UNIT_TEST_GATED', '1')
+    assert op(1) == -1 and log[-1] == 'gated'             # env var opts the gated backend in
+    monkeypatch.delenv('UNIT_TEST_GATED')
+    assert reg.get_active().backend_type == 'high'
+    # an operation without backends falls through to the decorated default
+    @dispatch('unit_test_op_without_backends')
+    def op2(x):
+        return x * 2
+    assert op2(4) == 8
+    from fla_hip.ops.gated_delta_rule.backends import gated_delta_rule_registry
+    assert gated_delta_rule_registry.operation_name == 'gated_delta_rule'
+
+
+def test_public_surface_and_signatures():
+    import inspect
+    import importlib
+    pkg = importlib.import_module('flash-linear-attention_amd')
+    import fla_hip.ops.gated_delta_rule as m
+    assert m.__all__ == ['chunk_gated_delta_rule', 'chunk_gdn', 'fused_recurrent_gated_delta_rule', 'fused_recurrent_gdn',
+                         'naive_chunk_gated_delta_rule', 'naive_recurrent_gated_delta_rule']
+    assert pkg.chunk_gdn is m.chunk_gated_delta_rule and m.fused_recurrent_gdn is m.fused_recurrent_gated_delta_rule
+    # parameter names are ABI (callers filter keyword arguments by name)
+    assert list(inspect.signature(m.chunk_gated_delta_rule).parameters) == [
+        'q', 'k', 'v', 'g', 'beta', 'scale', 'initial_state', 'output_final_state', 'use_qk_l2norm_in_kernel',
+        'use_beta_sigmoid_in_kernel', 'allow_neg_eigval', 'state_v_first', 'cu_seqlens', 'cu_seqlens_cpu',
+        'chunk_indices', 'cp_context', 'kwargs']
+    assert list(inspect.signature(m.fused_recurrent_gated_delta_rule).parameters) == [
+        'q', 'k', 'v', 'g', 'gk', 'gv', 'beta', 'scale', 'initial_state', 'output_final_state',
+        'use_qk_l2norm_in_kernel', 'use_gate_in_kernel', 'A_log', 'dt_bias', 'use_beta_sigmoid_in_kernel',
+        'allow_neg_eigval', 'state_v_first', 'cu_seqlens', 'kwargs']
+    assert list(inspect.signature(m.naive_recurrent_gated_delta_rule).parameters)[:5] == ['q', 'k', 'v', 'beta', 'g']
+    assert list(inspect.signature(m.naive_chunk_gated_delta_rule).parameters)[:5] == ['q', 'k', 'v', 'g', 'beta']
+
+
+def test_validation_happens_on_the_host_and_cpu_tensors_are_refused():
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
+    q = torch.randn(2, 8, 2, 16)
+    v = torch.randn(2, 8, 4, 16)
+    g = torch.zeros(2, 8, 4)
+    with pytest.raises(ValueError, match='same number of heads'):
+        chunk_gated_delta_rule(q, q[:, :, :1], v, g, g)
+    with pytest.raises(ValueError, match='divisible'):
+        chunk_gated_delta_rule(q, q, v[:, :, :3], g[:, :, :3], g[:, :, :3])
+    with pytest.raises(ValueError, match='chunk_size'):
+        chunk_gated_delta_rule(q, q, v, g, g, chunk_size=128)
+    with pytest.raises(ValueError, match='batch size'):
+        chunk_gated_delta_rule(q, q, v, g, g, cu_seqlens=torch.tensor([0, 8, 16]))
+    with pytest.raises(ValueError, match='initial states'):
+        chunk_gated_delta_rule(q[:1], q[:1], v[:1], g[:1], g[:1], initial_state=torch.zeros(3, 4, 16, 16),
+                               cu_seqlens=torch.tensor([0, 4, 8]))
+    with pytest.raises(ValueError, match='allow_neg_eigval'):
+        chunk_gated_delta_rule(q, q, v, g, g, allow_neg_eigval=True)
+    with pytest.raises(AssertionError, match='A_log'):
+        chunk_gated_delta_rule(q, q, v, g, g, use_gate_in_kernel=True)
+    with pytest.raises(DeprecationWarning):
+        chunk_gated_delta_rule(q, q, v, g, g, head_first=False)
+    with pytest.raises(ValueError, match='transpose_state_layout'):
+        chunk_gated_delta_rule(q, q, v, g, g, state_v_first=True, transpose_state_layout=True)
+    with pytest.raises(NotImplementedError):
+        chunk_gated_delta_rule(q, q, v, g, g, cp_context=object())
+    with pytest.raises(ValueError, match='A_log'):
+        fused_recurrent_gated_delta_rule(q, q, v, g, use_gate_in_kernel=True)
+    with pytest.raises(ValueError, match='inplace_final_state'):
+        fused_recurrent_gated_delta_rule(q, q, v, g, inplace_final_state=True)
+    # no CPU or eager fallback exists: CPU tensors are an error, not a slow path
+    with pytest.raises(RuntimeError, match='ROCm GPU'):
+        chunk_gated_delta_rule(q, q, v, g, g)
+    with pytest.raises(RuntimeError, match='ROCm GPU'):
+        fused_recurrent_gated_delta_rule(q, q, v, g)
+
+
+def test_naive_forms_match_oracle():
+    from fla_hip.ops.gated_delta_rule import naive_chunk_gated_delta_rule, naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = O.make_inputs(2, 150, 2, 2, 16, 8, seed=13, h0_std=0.5)
+    ref_o, ref_h = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, dtype=torch.float64)
+    o1, h1 = naive_recurrent_gated_delta_rule(q, k, v, beta, g, initial_state=h0, output_final_state=True)
+    o2, h2 = naive_chunk_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    for o, h in ((o1, h1), (o2, h2)):
+        assert o.shape == ref_o.shape
+        assert O.get_err_ratio(ref_o, o) < 1e-5 and O.get_err_ratio(ref_h, h) < 1e-5
+    o3, h3 = naive_chunk_gated_delta_rule(q, k, v, g, beta, chunk_size=16, scale=0.3)
+    ref_o3, _ = O.recurrent_gated_delta_rule(q, k, v, g, beta, 0.3, dtype=torch.float64)
+    assert h3 is None and O.get_err_ratio(ref_o3, o3) < 1e-5
+
+
+def test_assert_close_metric():
+    from fla_hip.utils import assert_close, get_abs_err, get_err_ratio
+    x = torch.tensor([3.0, 4.0]); y = torch.tensor([3.0, 5.0])
+    assert get_abs_err(x, y) == 1.0 and abs(get_err_ratio(x, y) - O.get_err_ratio(x, y)) < 1e-6
+    assert_close('ok', x, x + 1e-7, 1e-6)
+    with pytest.raises(AssertionError):
+        assert_close('bad', x, y, 0.01)
+    with pytest.warns(UserWarning):
+        assert_close('warn', x, y, 0.01, warning=True)
