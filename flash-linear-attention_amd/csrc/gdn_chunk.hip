@@ -23,11 +23,16 @@
 // exactly how a C/D result is spread over lanes, so an accumulator can be converted in
 // place into the B operand of the next product.
 #include "gdn_common.h"
+#include <type_traits>
 
 namespace gdn {
 
 constexpr int CH = 64;                       // chunk length
 constexpr float RCP_LN2_F = 1.4426950216f;   // fla/ops/utils/constant.py:10
+
+typedef bf16x4 __attribute__((address_space(3)))* lds_bf16x4_ptr;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef s16x4 __attribute__((address_space(3)))* lds_s16x4_ptr;
 
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
@@ -36,6 +41,11 @@ template <> struct Mma<bf16_t> {
     static __device__ __forceinline__ f32x4 run(V8 a, V8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
+    // LDS transpose read: the 16 lanes of a group each pass the address of 4 consecutive
+    // elements; lane L receives element L%4 of the runs addressed by lanes L/4, L/4+4, L/4+8, L/4+12.
+    static __device__ __forceinline__ V4 tr_read(const bf16_t* p) {
+        return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4_ptr)p);
+    }
 };
 template <> struct Mma<f16_t> {
     typedef f16x8 V8;
@@ -43,34 +53,48 @@ template <> struct Mma<f16_t> {
     static __device__ __forceinline__ f32x4 run(V8 a, V8 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ V4 tr_read(const f16_t* p) {
+        return __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p));
+    }
 };
 
+template <typename V8, typename V4>
+__device__ __forceinline__ V8 join(V4 a, V4 b) {
+    return V8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+}
+
+// 2^x as a single v_exp_f32 (results below 2^-126 flush to zero, which is what a decay wants)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // Per-chunk workspace written by the prepare kernel (element counts for K = V = 128):
-//   G   fp32 [NC][HV][64]                   chunk-local gate cumsum in log2 units
+//   Tab fp32 [NC][HV][192]                  [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128] G_last (log2 units)
 //   Wf  T    [NC][HV][4 tt][4 s][64][8]     w rows of t-tile tt, key tiles (2s, 2s+1)
 //   Uf  T    [NC][HV][8 n ][4 tt][64][4]    u, C/D layout of tile (t-tile tt, value tile n)
+//   Pf  T    [NC][HV][4 tt][2 s][64][8]     scale*P rows of t-tile tt, t-tiles (2s, 2s+1) as columns
 //   KTf T    [NC][H ][8 m ][2 s][64][8]     k^T rows of key tile m, t-tiles (2s, 2s+1)
-//   Pf  T    [NC][HV][4 tt][2 s][64][8]     P rows of t-tile tt, t-tiles (2s, 2s+1) as columns
+//   Qf  T    [NC][H ][4 tt][4 s][64][8]     q rows of t-tile tt, key tiles (2s, 2s+1)
 struct ChunkWs {
-    float* G;
+    float* Tab;
     void* Wf;
     void* Uf;
-    void* KTf;
     void* Pf;
+    void* KTf;
+    void* Qf;
 };
-constexpr int64_t WS_W = 8192, WS_U = 8192, WS_KT = 8192, WS_P = 4096;   // elements per (chunk, head)
+constexpr int64_t WS_TAB = 192, WS_W = 8192, WS_U = 8192, WS_P = 4096, WS_KT = 8192, WS_Q = 8192;   // elements per (chunk, head)
 
 static size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 static size_t ws_layout(int64_t NC, int64_t H, int64_t HV, char* base, ChunkWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
-    void* G = take((size_t)NC * HV * CH * 4);
+    void* Tab = take((size_t)NC * HV * WS_TAB * 4);
     void* Wf = take((size_t)NC * HV * WS_W * 2);
     void* Uf = take((size_t)NC * HV * WS_U * 2);
-    void* KTf = take((size_t)NC * H * WS_KT * 2);
     void* Pf = take((size_t)NC * HV * WS_P * 2);
-    if (ws) { ws->G = (float*)G; ws->Wf = Wf; ws->Uf = Uf; ws->KTf = KTf; ws->Pf = Pf; }
+    void* KTf = take((size_t)NC * H * WS_KT * 2);
+    void* Qf = take((size_t)NC * H * WS_Q * 2);
+    if (ws) { ws->Tab = (float*)Tab; ws->Wf = Wf; ws->Uf = Uf; ws->Pf = Pf; ws->KTf = KTf; ws->Qf = Qf; }
     return off;
 }
 
@@ -85,20 +109,30 @@ struct ChunkParams {
 };
 
 // Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains
-// the vector-memory counter, which would serialise the global prefetch of the next chunk
+// the vector-memory counter, which would serialise the global prefetch of later chunks
 // behind every barrier of the current one.
 #ifndef GDN_EXP
 #define GDN_EXP 0
 #endif
 __device__ __forceinline__ void lds_barrier() {
-    if (GDN_EXP == 3) return;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// 8-byte global store issued from inline assembly.  The compiler's wait-count bookkeeping
+// does not see it, so the prefetched loads of the scan loop stay the only operations it
+// counts and it can wait for "all but the newest N loads" instead of draining the queue
+// (loads and stores share one hardware counter, and once both are pending the compiler
+// falls back to waiting for everything).  The extra, uncounted stores only make the
+// hardware counter larger than the compiler assumes, i.e. its waits err on the late side.
+__device__ __forceinline__ void store_b64_uncounted(void* ptr, u32x2 data) {
+    asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(ptr), "v"(data) : "memory");
 }
 
 // 16x16 product of fp32 matrices held in LDS on the fp32 matrix cores:
 // C = A[16 x 4*nk] * B[4*nk x 16]; result in C/D layout.
 __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* B, int ldb, int nk, int c16, int g) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
     for (int kk = 0; kk < nk; ++kk) {
         const float a = A[c16 * lda + 4 * kk + g];
         const float b = B[(4 * kk + g) * ldb + c16];
@@ -113,6 +147,20 @@ __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* 
 constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 272 B rows, conflict-free 16 B reads
 constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
 constexpr size_t PREP_SMEM = 3 * CH * NP * 2 + CH * LP * 4 + 3 * CH * 4;
+
+// Transposed MFMA operand from a token-major tile: lane (c16, g) gets column fb + c16 of the
+// 8 rows r0 .. r0+7 (two transpose reads of 4 rows each).
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V8 tr_frag8(const T* tile, int r0, int fb, int c16) {
+    const T* a = tile + (r0 + (c16 >> 2)) * NP + fb + 4 * (c16 & 3);
+    return join<typename Mma<T>::V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * NP));
+}
+// Same for two separate groups of 4 rows starting at ra and rb.
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V8 tr_frag44(const T* tile, int ra, int rb, int fb, int c16) {
+    const int o = (c16 >> 2) * NP + fb + 4 * (c16 & 3);
+    return join<typename Mma<T>::V8>(Mma<T>::tr_read(tile + ra * NP + o), Mma<T>::tr_read(tile + rb * NP + o));
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
@@ -133,6 +181,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
     const int hv = blockIdx.y;
     const int H = p.H, HV = p.HV;
     const int h = hv / (HV / H);
+    const bool first_of_group = hv % (HV / H) == 0;      // writes the per-q/k-head fragments
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
 
     int64_t tok0;
@@ -177,10 +226,15 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
             if (lane >= off) x += y;
         }
         x *= RCP_LN2_F;
+        const float xl = __shfl(x, 63, 64);      // rows past the end carry the last valid sum
+        const float ex = fast_exp2(x);
         sG[lane] = x;
         sB[lane] = b;
-        sBG[lane] = b * exp2f(x);
-        p.ws.G[(ci * HV + hv) * CH + lane] = x;
+        sBG[lane] = b * ex;
+        float* tab = p.ws.Tab + (ci * HV + hv) * WS_TAB;
+        tab[lane] = fast_exp2(xl - x);
+        tab[64 + lane] = p.scale * ex;
+        if (lane == 63) tab[128] = x;
     }
 #pragma unroll
     for (int ps = 0; ps < 4; ++ps) {
@@ -190,12 +244,16 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         *(u32x4*)(v_nat + row * NP + col) = rv[ps];
     }
     __syncthreads();
+#if GDN_EXP == 5
+    return;
+#endif
 
     // ---- L tiles of row-tile w (K K^T, gated, beta-scaled, strictly lower) ----
     {
         V8 ka[4];
 #pragma unroll
         for (int s = 0; s < 4; ++s) ka[s] = *(const V8*)(k_nat + (16 * w + c16) * NP + 32 * s + 8 * g);
+        const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g), bi = *(const f32x4*)(sB + 16 * w + 4 * g);
         for (int tj = 0; tj < 4; ++tj) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
             if (tj <= w) {
@@ -211,8 +269,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
             for (int r = 0; r < 4; ++r) {
                 const int i = 16 * w + 4 * g + r;
                 // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
-                const float val = (i > j) ? sB[i] * acc[r] * exp2f(sG[i] - gj) : 0.f;
-                sL[i * LP + j] = val;
+                sL[i * LP + j] = (i > j) ? bi[r] * acc[r] * fast_exp2(gi[r] - gj) : 0.f;
             }
         }
     }
@@ -225,7 +282,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         const int t = 16 * tt + c16;
         const float gt = sG[t];
         T* pf = (T*)p.ws.Pf + (ci * HV + hv) * WS_P;
-        for (int sp = 0; sp <= tt / 2; ++sp) {
+        for (int sp = 0; sp < 2; ++sp) {
             V8 frag;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
@@ -238,17 +295,30 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
                         acc = Mma<T>::run(ka, qb[s], acc);
                     }
                 }
+                const f32x4 gj = *(const f32x4*)(sG + 16 * tj + 4 * g);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = 16 * tj + 4 * g + r;
-                    const float val = (t >= j) ? acc[r] * exp2f(gt - sG[j]) : 0.f;
+                    const float val = (t >= j) ? p.scale * acc[r] * fast_exp2(gt - gj[r]) : 0.f;
                     frag[half * 4 + r] = from_f32<T>(val);
                 }
             }
             *(V8*)(pf + ((tt * 2 + sp) * 64 + lane) * 8) = frag;
         }
+        // q rows of t-tile tt as A operands over key tiles (2s, 2s+1), one copy per q/k head
+        if (first_of_group) {
+            T* qf = (T*)p.ws.Qf + (ci * H + h) * WS_Q;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const T* src = q_nat + (16 * tt + c16) * NP + 32 * s + 4 * g;
+                *(V8*)(qf + ((tt * 4 + s) * 64 + lane) * 8) = join<V8>(*(const V4*)src, *(const V4*)(src + 16));
+            }
+        }
     }
     __syncthreads();     // L complete; q_nat is dead from here on and becomes X
+#if GDN_EXP == 6
+    return;
+#endif
 
     // ---- X = (I+L)^-1: 16x16 diagonal blocks by forward substitution (column c16 per lane) ----
     {
@@ -295,7 +365,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         const int a = w >> 1, b = w & 1;
         float* tmp2 = sX + 32;                              // rows 0..31, columns 32..63
         f32x4 y = mm16_f32(sL + (32 + 16 * a) * LP, LP, sX + 16 * b, LP, 8, c16, g);
-        __syncthreads();                                    // level-1 temporaries (same region) fully consumed
 #pragma unroll
         for (int r = 0; r < 4; ++r) tmp2[(16 * a + 4 * g + r) * LP + 16 * b + c16] = y[r];
         __syncthreads();
@@ -305,6 +374,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
     }
     __syncthreads();
 
+#if GDN_EXP == 7
+    return;
+#endif
     // ---- w^T = k^T (diag(beta 2^G) X^T) and u = (X diag(beta)) v for t-tile w ----
     const int ns = (w >= 2) ? 2 : 1;         // X is lower triangular: columns >= 32 matter only for rows >= 32
     V8 fw[2], fu[2];
@@ -326,6 +398,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
     }
     {
         T* wf = (T*)p.ws.Wf + (ci * HV + hv) * WS_W;
+#pragma unroll
         for (int sp = 0; sp < 4; ++sp) {
             V8 frag;
 #pragma unroll
@@ -333,31 +406,20 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
                 const int m = 2 * sp + half;
                 f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    if (s < ns) {
-                        V8 ka;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) ka[e] = k_nat[(32 * s + 8 * g + e) * NP + 16 * m + c16];
-                        acc = Mma<T>::run(ka, fw[s], acc);
-                    }
-                }
+                for (int s = 0; s < 2; ++s)
+                    if (s < ns) acc = Mma<T>::run(tr_frag8<T>(k_nat, 32 * s + 8 * g, 16 * m, c16), fw[s], acc);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) frag[half * 4 + r] = from_f32<T>(acc[r]);
             }
             *(V8*)(wf + ((w * 4 + sp) * 64 + lane) * 8) = frag;
         }
         T* uf = (T*)p.ws.Uf + (ci * HV + hv) * WS_U;
+#pragma unroll
         for (int n = 0; n < 8; ++n) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (s < ns) {
-                    V8 vb;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) vb[e] = v_nat[(32 * s + 8 * g + e) * NP + 16 * n + c16];
-                    acc = Mma<T>::run(fu[s], vb, acc);
-                }
-            }
+            for (int s = 0; s < 2; ++s)
+                if (s < ns) acc = Mma<T>::run(fu[s], tr_frag8<T>(v_nat, 32 * s + 8 * g, 16 * n, c16), acc);
             V4 o4;
 #pragma unroll
             for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
@@ -365,21 +427,14 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         }
     }
     // ---- k^T fragments for the state update (one copy per q/k head) ----
-    if (hv % (HV / H) == 0) {
+    if (first_of_group) {
         T* ktf = (T*)p.ws.KTf + (ci * H + h) * WS_KT;
 #pragma unroll
         for (int mm = 0; mm < 2; ++mm) {
             const int m = 2 * w + mm;
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                V8 frag;
-#pragma unroll
-                for (int half = 0; half < 2; ++half)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        frag[half * 4 + r] = k_nat[(32 * s + 16 * half + 4 * g + r) * NP + 16 * m + c16];
-                *(V8*)(ktf + ((m * 2 + s) * 64 + lane) * 8) = frag;
-            }
+            for (int s = 0; s < 2; ++s)
+                *(V8*)(ktf + ((m * 2 + s) * 64 + lane) * 8) = tr_frag44<T>(k_nat, 32 * s + 4 * g, 32 * s + 16 + 4 * g, 16 * m, c16);
         }
     }
 }
@@ -391,8 +446,9 @@ template <typename T, int NV>
 struct ScanFrags {
     typename Mma<T>::V8 wf[4], qf[4], kt[2][2], pf[2];
     typename Mma<T>::V4 uf[NV];
-    f32x4 grow;
-    float glast;
+    f32x4 dec;          // 2^(G_last-G_t) for the 4 rows of this lane's C/D fragment
+    float gam;          // scale*2^G_t for the column of this lane's transposed output fragment
+    float glast;        // G_last in log2 units
     int valid;
 };
 
@@ -448,128 +504,180 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
             S[i][nn] = s;
         }
 
+    // Make the initial state arrive before the prefetch queue is started: a wait for these
+    // registers inside the loop (their first use) would be executed on every trip and would
+    // drain the prefetched loads with it.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int nn = 0; nn < NV; ++nn) asm volatile("" : "+v"(S[i][nn]) : : "memory");
+
     const T* Wf = (const T*)p.ws.Wf;
     const T* Uf = (const T*)p.ws.Uf;
     const T* KTf = (const T*)p.ws.KTf;
     const T* Pf = (const T*)p.ws.Pf;
-    const T* qg = (const T*)p.q;
+    const T* Qf = (const T*)p.ws.Qf;
     T* og = (T*)p.o;
 
-    auto load_frags = [&](int64_t it, ScanFrags<T, NV>& f) {
+    // All loads are unconditional and there is no data-dependent control flow around memory
+    // operations in the main loop: the compiler can then count outstanding loads exactly and
+    // wait only for the buffer it is about to use, instead of draining the queue.
+    auto load_a = [&](int64_t it, ScanFrags<T, NV>& f) {        // operands of the first half of a step
         const int64_t ci = boh + it;
-        const int64_t chv = ci * HV + hv;
-        const int64_t tok0 = bos + it * CH;
-        f.valid = (int)min((int64_t)CH, len - it * CH);
+        const int64_t chv = ci * HV + hv, ch = ci * H + h;
 #pragma unroll
         for (int s = 0; s < 4; ++s) f.wf[s] = *(const V8*)(Wf + chv * WS_W + ((w * 4 + s) * 64 + lane) * 8);
-        const int trow = 16 * w + c16;
-        const T* qrow = qg + ((tok0 + trow) * H + h) * 128 + 4 * g;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            V4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (trow < f.valid && GDN_EXP != 2) {
-                a = *(const V4*)(qrow + 32 * s);
-                b = *(const V4*)(qrow + 32 * s + 16);
-            }
-            f.qf[s] = V8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-        }
+        for (int s = 0; s < 4; ++s) f.qf[s] = *(const V8*)(Qf + ch * WS_Q + ((w * 4 + s) * 64 + lane) * 8);
+    };
+    auto load_b = [&](int64_t it, ScanFrags<T, NV>& f) {        // everything else
+        const int64_t ci = boh + it;
+        const int64_t chv = ci * HV + hv, ch = ci * H + h;
+        f.valid = (int)min((int64_t)CH, len - it * CH);
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int s = 0; s < 2; ++s)
-                f.kt[i][s] = *(const V8*)(KTf + (ci * H + h) * WS_KT + (((2 * w + i) * 2 + s) * 64 + lane) * 8);
+                f.kt[i][s] = *(const V8*)(KTf + ch * WS_KT + (((2 * w + i) * 2 + s) * 64 + lane) * 8);
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            // P rows of t-tile w only reach t-tiles <= w: the second column pair exists for w >= 2
-            if (s == 0 || w >= 2) f.pf[s] = *(const V8*)(Pf + chv * WS_P + ((w * 2 + s) * 64 + lane) * 8);
-        }
+        for (int s = 0; s < 2; ++s) f.pf[s] = *(const V8*)(Pf + chv * WS_P + ((w * 2 + s) * 64 + lane) * 8);
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn)
             f.uf[nn] = *(const V4*)(Uf + chv * WS_U + (((v0 / 16 + nn) * 4 + w) * 64 + lane) * 4);
-        f.grow = *(const f32x4*)(p.ws.G + chv * CH + 16 * w + 4 * g);
-        f.glast = p.ws.G[chv * CH + CH - 1];
+        const float* tab = p.ws.Tab + chv * WS_TAB;
+        f.dec = *(const f32x4*)(tab + 16 * w + 4 * g);
+        f.gam = tab[64 + 16 * w + c16];
+        f.glast = tab[128];
     };
 
-    ScanFrags<T, NV> cur, nxt;
-    if (nt > 0) load_frags(0, cur);
-    nxt = cur;
-    for (int64_t it = 0; it < nt; ++it) {
-        if (it + 1 < nt && GDN_EXP != 4) load_frags(it + 1, nxt);
-        // (a) publish the state of this chunk as bf16/f16 B-operand fragments
+    // The registers hold Shat = S / Gamma with one scalar Gamma = 2^lg per workgroup, so the
+    // decay of the whole state by 2^G_last per chunk costs nothing: products with S are
+    // rescaled by Gamma (folded into multiplies that exist anyway) and the update is divided
+    // by the new Gamma (folded into the decay factors of v_new).  When Gamma gets small the
+    // state is rescaled once and Gamma restarts at 1.  f16 operands have too little range for
+    // Shat, so there the state is rescaled on every chunk.
+    constexpr float LG_MIN = std::is_same<T, bf16_t>::value ? -60.f : 1.f;
+    float lg = 0.f;                                              // log2 Gamma
+
+    auto step = [&](int64_t it, ScanFrags<T, NV>& f, int64_t refill, auto masked) {
+        // (a) publish the state at the start of this chunk as bf16/f16 B-operand fragments
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn) {
-            V8 f;
+            V8 sb;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                f[r] = from_f32<T>(S[0][nn][r]);
-                f[4 + r] = from_f32<T>(S[1][nn][r]);
+                sb[r] = from_f32<T>(S[0][nn][r]);
+                sb[4 + r] = from_f32<T>(S[1][nn][r]);
             }
-            sSb[(w * NV + nn) * 64 + lane] = f;
+            sSb[(w * NV + nn) * 64 + lane] = sb;
         }
+        const float gamma = fast_exp2(lg);
+        const float lg_try = lg + f.glast;
+        const bool lazy = lg_try >= LG_MIN;                      // same value in every lane of the workgroup
+        const float vscale = lazy ? fast_exp2(-lg_try) : 1.f;
+        const f32x4 dec = f.dec * vscale;
+        const float ogam = f.gam * gamma;
         lds_barrier();
-        // (b,c) w S and q S for t-tile w
-        f32x4 accv[NV], acco[NV];
+        // (b,c) w S (rows of t-tile w) and (q S)^T (columns of t-tile w)
+        f32x4 acco[NV];
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn) {
             f32x4 av = {0.f, 0.f, 0.f, 0.f}, ao = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const V8 sb = sSb[(s * NV + nn) * 64 + lane];
-                av = Mma<T>::run(cur.wf[s], sb, av);
-                ao = Mma<T>::run(cur.qf[s], sb, ao);
+                av = Mma<T>::run(f.wf[s], sb, av);
+                ao = Mma<T>::run(sb, f.qf[s], ao);      // operands swapped: result is the transposed tile
             }
-            accv[nn] = av;
-            acco[nn] = ao;
-        }
-        // (d) v_new = u - w S; publish it plain (for the output) and decayed to the chunk end (for the state)
-        const float glast = cur.glast;
-        f32x4 dec, grow2;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            dec[r] = exp2f(glast - cur.grow[r]);
-            grow2[r] = exp2f(cur.grow[r]);
-        }
-#pragma unroll
-        for (int nn = 0; nn < NV; ++nn) {
+            acco[nn] = ao * ogam;
+            // (d) v_new = u - w S; publish it plain (for the output) and decayed to the chunk end (for the state)
             V4 plain, gated;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float vn = to_f32(cur.uf[nn][r]) - accv[nn][r];
+                const float vn = to_f32(f.uf[nn][r]) - gamma * av[r];
                 plain[r] = from_f32<T>(vn);
                 gated[r] = from_f32<T>(vn * dec[r]);
             }
             sVn[(((0 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = plain;
             sVn[(((1 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = gated;
         }
+        if (!decltype(masked)::value) load_a(refill, f);
+        if (!lazy) {
+            const float fold = fast_exp2(lg_try);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int nn = 0; nn < NV; ++nn) S[i][nn] *= fold;
+        }
+        lg = lazy ? lg_try : 0.f;
         lds_barrier();
         // (e,f) state update and output
-        const float gl2 = exp2f(glast);
         const V8* sVn8 = (const V8*)sVn;
+        const int trow = 16 * w + c16;
+        T* orow = og + ((bos + it * CH + trow) * HV + hv) * 128 + v0 + 4 * g;
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn) {
             const V8 vg0 = sVn8[((1 * 2 + 0) * NV + nn) * 64 + lane], vg1 = sVn8[((1 * 2 + 1) * NV + nn) * 64 + lane];
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                f32x4 s = S[i][nn] * gl2;
-                s = Mma<T>::run(cur.kt[i][0], vg0, s);
-                s = Mma<T>::run(cur.kt[i][1], vg1, s);
+                f32x4 s = S[i][nn];
+                s = Mma<T>::run(f.kt[i][0], vg0, s);
+                s = Mma<T>::run(f.kt[i][1], vg1, s);
                 S[i][nn] = s;
             }
-            f32x4 ao = acco[nn] * grow2;
-            ao = Mma<T>::run(cur.pf[0], sVn8[((0 * 2 + 0) * NV + nn) * 64 + lane], ao);
-            if (w >= 2) ao = Mma<T>::run(cur.pf[1], sVn8[((0 * 2 + 1) * NV + nn) * 64 + lane], ao);
-            const int64_t tok0 = bos + it * CH;
+            // P rows of t-tile w reach t-tiles <= w only; the fragments above the diagonal are zero
+            f32x4 ao = Mma<T>::run(sVn8[((0 * 2 + 0) * NV + nn) * 64 + lane], f.pf[0], acco[nn]);
+            ao = Mma<T>::run(sVn8[((0 * 2 + 1) * NV + nn) * 64 + lane], f.pf[1], ao);
+            // transposed tile: this lane holds 4 consecutive value columns of token row trow
+            V4 o4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int t = 16 * w + 4 * g + r;
-#if GDN_EXP != 1
-                if (t < cur.valid) og[((tok0 + t) * HV + hv) * 128 + v0 + 16 * nn + c16] = from_f32<T>(ao[r] * p.scale);
-#else
-                if (ao[r] == 12345.f) og[((tok0 + t) * HV + hv) * 128 + v0 + 16 * nn + c16] = from_f32<T>(ao[r] * p.scale);
-#endif
-            }
+            for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(ao[r]);
+            if (!decltype(masked)::value) store_b64_uncounted(orow + 16 * nn, __builtin_bit_cast(u32x2, o4));
+            else if (trow < f.valid) *(V4*)(orow + 16 * nn) = o4;
         }
-        cur = nxt;
+        if (!decltype(masked)::value) load_b(refill, f);
+    };
+    std::integral_constant<bool, false> full_chunk;
+    std::integral_constant<bool, true> tail_chunk;
+
+    // Three fragment buffers; a buffer is refilled while and right after its chunk is consumed,
+    // so every load has two full steps to arrive.  Refills past the end re-read the last chunk.
+    ScanFrags<T, NV> f0, f1, f2;
+    const int64_t last = nt - 1;
+    const int64_t nfast = (len / CH) / 3 * 3;       // chunks handled three at a time; all of them are full
+    if (nt > 0) {
+        // compiler fences keep the groups in issue order, as inside the loop: the waits in the
+        // loop are sized for the entry path too
+        load_a(0, f0);
+        asm volatile("" ::: "memory");
+        load_b(0, f0);
+        asm volatile("" ::: "memory");
+        load_a(min((int64_t)1, last), f1);
+        asm volatile("" ::: "memory");
+        load_b(min((int64_t)1, last), f1);
+        asm volatile("" ::: "memory");
+        load_a(min((int64_t)2, last), f2);
+        asm volatile("" ::: "memory");
+        load_b(min((int64_t)2, last), f2);
+        asm volatile("" ::: "memory");
+    }
+    for (int64_t it = 0; it < nfast; it += 3) {
+        step(it, f0, min(it + 3, last), full_chunk);
+        step(it + 1, f1, min(it + 4, last), full_chunk);
+        step(it + 2, f2, min(it + 5, last), full_chunk);
+    }
+    // at most three chunks remain (two full ones and a ragged tail)
+    if (nfast < nt) step(nfast, f0, 0, tail_chunk);
+    if (nfast + 1 < nt) step(nfast + 1, f1, 0, tail_chunk);
+    if (nfast + 2 < nt) step(nfast + 2, f2, 0, tail_chunk);
+
+    // back to the true state
+    {
+        const float gamma = fast_exp2(lg);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int nn = 0; nn < NV; ++nn) S[i][nn] *= gamma;
     }
 
     if (p.ht) {
