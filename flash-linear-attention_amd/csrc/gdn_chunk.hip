@@ -559,7 +559,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
     constexpr float LG_MIN = std::is_same<T, bf16_t>::value ? -60.f : 1.f;
     float lg = 0.f;                                              // log2 Gamma
 
-    auto step = [&](int64_t it, ScanFrags<T, NV>& f, int64_t refill, auto masked) {
+    // `f` holds the chunk being processed; `fr` is the buffer consumed one step earlier, which is
+    // refilled with chunk `refill` while this step computes (its loads are interleaved with the
+    // matrix instructions so that the memory pipeline never sees a burst).
+    auto step = [&](int64_t it, ScanFrags<T, NV>& f, ScanFrags<T, NV>& fr, int64_t refill, auto masked) {
         // (a) publish the state at the start of this chunk as bf16/f16 B-operand fragments
 #pragma unroll
         for (int nn = 0; nn < NV; ++nn) {
@@ -601,7 +604,14 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
             sVn[(((0 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = plain;
             sVn[(((1 * 2 + (w >> 1)) * NV + nn) * 64 + lane) * 2 + (w & 1)] = gated;
         }
-        if (!decltype(masked)::value) load_a(refill, f);
+        if (!decltype(masked)::value) {
+            load_a(refill, fr);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                __builtin_amdgcn_sched_group_barrier(0x008, NV, 0);      // NV matrix instructions
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);       // then one global load
+            }
+        }
         if (!lazy) {
             const float fold = fast_exp2(lg_try);
 #pragma unroll
@@ -635,41 +645,50 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
             if (!decltype(masked)::value) store_b64_uncounted(orow + 16 * nn, __builtin_bit_cast(u32x2, o4));
             else if (trow < f.valid) *(V4*)(orow + 16 * nn) = o4;
         }
-        if (!decltype(masked)::value) load_b(refill, f);
+        if (!decltype(masked)::value) {
+            load_b(refill, fr);
+#pragma unroll
+            for (int j = 0; j < 6; ++j) {
+                __builtin_amdgcn_sched_group_barrier(0x008, NV, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+            }
+        }
     };
     std::integral_constant<bool, false> full_chunk;
     std::integral_constant<bool, true> tail_chunk;
 
-    // Three fragment buffers; a buffer is refilled while and right after its chunk is consumed,
-    // so every load has two full steps to arrive.  Refills past the end re-read the last chunk.
-    ScanFrags<T, NV> f0, f1, f2;
+    // NB fragment buffers in rotation: step `it` computes from buffer it%NB and refills buffer
+    // (it-1)%NB (consumed in the previous step) with chunk it+NB-1, so every load has NB-2 full
+    // steps to arrive.  A wave can have 63 loads in flight, 18 per buffer, hence NB = 4.
+    // Refills past the end re-read the last chunk and are never used.
+    constexpr int NB = NV >= 8 ? 3 : 4;          // the widest slab has no registers to spare and is compute-bound anyway
+    ScanFrags<T, NV> fb[NB];
     const int64_t last = nt - 1;
-    const int64_t nfast = (len / CH) / 3 * 3;       // chunks handled three at a time; all of them are full
+    const int64_t nfast = (len / CH) / NB * NB;     // chunks handled NB at a time; all of them are full
     if (nt > 0) {
         // compiler fences keep the groups in issue order, as inside the loop: the waits in the
         // loop are sized for the entry path too
-        load_a(0, f0);
-        asm volatile("" ::: "memory");
-        load_b(0, f0);
-        asm volatile("" ::: "memory");
-        load_a(min((int64_t)1, last), f1);
-        asm volatile("" ::: "memory");
-        load_b(min((int64_t)1, last), f1);
-        asm volatile("" ::: "memory");
-        load_a(min((int64_t)2, last), f2);
-        asm volatile("" ::: "memory");
-        load_b(min((int64_t)2, last), f2);
-        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < NB - 1; ++j) {
+            load_a(min((int64_t)j, last), fb[j]);
+            asm volatile("" ::: "memory");
+            load_b(min((int64_t)j, last), fb[j]);
+            asm volatile("" ::: "memory");
+        }
     }
-    for (int64_t it = 0; it < nfast; it += 3) {
-        step(it, f0, min(it + 3, last), full_chunk);
-        step(it + 1, f1, min(it + 4, last), full_chunk);
-        step(it + 2, f2, min(it + 5, last), full_chunk);
+    for (int64_t it = 0; it < nfast; it += NB) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) step(it + j, fb[j], fb[(j + NB - 1) % NB], min(it + j + NB - 1, last), full_chunk);
     }
-    // at most three chunks remain (two full ones and a ragged tail)
-    if (nfast < nt) step(nfast, f0, 0, tail_chunk);
-    if (nfast + 1 < nt) step(nfast + 1, f1, 0, tail_chunk);
-    if (nfast + 2 < nt) step(nfast + 2, f2, 0, tail_chunk);
+    // at most NB chunks remain (NB-1 full ones and a ragged tail): buffers 0..NB-2 already hold
+    // the first of them
+    if (nfast + NB - 1 < nt) {
+        load_a(nfast + NB - 1, fb[NB - 1]);
+        load_b(nfast + NB - 1, fb[NB - 1]);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+        if (nfast + j < nt) step(nfast + j, fb[j], fb[j], 0, tail_chunk);
 
     // back to the true state
     {
