@@ -146,7 +146,7 @@ __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* 
 // ============================================================================================
 constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 272 B rows, conflict-free 16 B reads
 constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
-constexpr size_t PREP_SMEM = 3 * CH * NP * 2 + CH * LP * 4 + 3 * CH * 4;
+constexpr size_t PREP_SMEM = 3 * CH * NP * 2 + 3 * CH * 4;     // 52 992 B: three workgroups per CU
 
 // Transposed MFMA operand from a token-major tile: lane (c16, g) gets column fb + c16 of the
 // 8 rows r0 .. r0+7 (two transpose reads of 4 rows each).
@@ -169,10 +169,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
     extern __shared__ __align__(16) char smem[];
     T* k_nat = (T*)smem;                        // [64][NP] keys, token-major
     T* q_nat = k_nat + CH * NP;                 // [64][NP] queries; the region is reused for X below
-    T* v_nat = q_nat + CH * NP;                 // [64][NP] values
-    float* sL = (float*)(v_nat + CH * NP);      // [64][LP] L (strictly lower)
-    float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1, same bytes as q_nat (64*136*2 == 64*68*4)
-    float* sG = sL + CH * LP;                   // [64] cumulative gate (log2)
+    T* v_nat = q_nat + CH * NP;                 // [64][NP] values; staged only after the solve (same bytes as L)
+    float* sL = (float*)v_nat;                  // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
+    float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1, same bytes as q_nat
+    float* sG = (float*)(v_nat + CH * NP);      // [64] cumulative gate (log2)
     float* sB = sG + CH;                        // [64] beta
     float* sBG = sB + CH;                       // [64] beta * 2^G
 
@@ -241,7 +241,6 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
         *(u32x4*)(k_nat + row * NP + col) = rk[ps];
         *(u32x4*)(q_nat + row * NP + col) = rq[ps];
-        *(u32x4*)(v_nat + row * NP + col) = rv[ps];
     }
     __syncthreads();
 #if GDN_EXP == 5
@@ -371,6 +370,13 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         f32x4 z = mm16_f32(sX + (32 + 16 * a) * LP + 32, LP, tmp2 + 16 * b, LP, 8, c16, g);
 #pragma unroll
         for (int r = 0; r < 4; ++r) sX[(32 + 16 * a + 4 * g + r) * LP + 16 * b + c16] = -z[r];
+    }
+    __syncthreads();
+    // L is dead: its bytes now take the value tile, which has been waiting in registers
+#pragma unroll
+    for (int ps = 0; ps < 4; ++ps) {
+        const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
+        *(u32x4*)(v_nat + row * NP + col) = rv[ps];
     }
     __syncthreads();
 
