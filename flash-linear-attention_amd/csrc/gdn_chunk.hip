@@ -14,6 +14,32 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
         if (rc) return rc;
     }
     if (!(stages & STAGE_SCAN)) return GDN_OK;
+    // Which form of the sequential stage:
+    //   wide      one workgroup per (sequence, head): enough pairs to fill the CUs
+    //   segments  few pairs but long dense sequences: cut time into segments (3 wide passes + merge)
+    //   slab      otherwise: split the value columns of each head over several workgroups
+    const bool dense = p.cu_seqlens == nullptr;
+    int nseg = 0;
+    if (dense && p.NH > 0) {
+        nseg = (int)std::min<int64_t>((256 + p.NH / 2) / p.NH, p.NT / 4);
+        if ((int64_t)nseg * p.NH > SEG_SLOTS_MAX || (int64_t)nseg * p.NH > (num_chunks * p.HV + 3) / 4) nseg = 0;
+    }
+    int mode = p.NH >= 192 ? 1 : (nseg >= 2 ? 2 : 0);
+    if (p.flags & GDN_FLAG_SCAN_SLAB) mode = 0;
+    if (p.flags & GDN_FLAG_SCAN_WIDE) mode = 1;
+    if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) mode = 2;
+    if (mode == 1) return launch_scan_wide<T>(p, stream);
+    if (mode == 2) {
+        SegmentPlan sp;
+        sp.kind = 0;
+        sp.nseg = nseg;
+        sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
+        const size_t slots = (size_t)p.NH * nseg;
+        sp.sloc = p.ws.Seg;
+        sp.mseg = p.ws.Seg + slots * 16384;
+        sp.sin = p.ws.Seg + 2 * slots * 16384;
+        return launch_scan_segments<T>(p, sp, stream);
+    }
     return launch_scan_slab<T>(p, stream);
 }
 

@@ -12,6 +12,7 @@
 #pragma once
 #include "gdn_common.h"
 #include <type_traits>
+#include <algorithm>
 
 namespace gdn {
 
@@ -55,13 +56,14 @@ __device__ __forceinline__ V8 join(V4 a, V4 b) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Per-chunk workspace written by the prepare kernel (element counts for K = V = 128):
-//   Tab fp32 [NC][HV][192]                  [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128] G_last (log2 units)
+//   Tab fp32 [NC][HV][256]                  [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128] G_last (log2 units)
 //   Wf  T    [NC][HV][4 tt][4 s][64][8]     w rows of t-tile tt, key tiles (2s, 2s+1)
 //   Uf  T    [NC][HV][8 n ][4 tt][64][4]    u, C/D layout of tile (t-tile tt, value tile n)
 //   Pf  T    [NC][HV][4 tt][2 s][64][8]     scale*P rows of t-tile tt, t-tiles (2s, 2s+1) as columns
 //   KTf T    [NC][H ][8 m ][2 s][64][8]     k^T rows of key tile m, t-tiles (2s, 2s+1)
 //   Qf  T    [NC][H ][4 tt][4 s][64][8]     q rows of t-tile tt, key tiles (2s, 2s+1)
 struct ChunkWs {
+    float* Seg;          // 3 * seg_slots 128x128 fp32 matrices for the segment-parallel scan
     float* Tab;
     void* Wf;
     void* Uf;
@@ -69,20 +71,24 @@ struct ChunkWs {
     void* KTf;
     void* Qf;
 };
-constexpr int64_t WS_TAB = 192, WS_W = 8192, WS_U = 8192, WS_P = 4096, WS_KT = 8192, WS_Q = 8192;   // elements per (chunk, head)
+constexpr int64_t WS_TAB = 256, WS_W = 8192, WS_U = 8192, WS_P = 4096, WS_KT = 8192, WS_Q = 8192;   // elements per (chunk, head)
+
+constexpr int64_t SEG_SLOTS_MAX = 640;            // upper bound on (sequences * heads * segments) when segmenting
 
 inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 inline size_t ws_layout(int64_t NC, int64_t H, int64_t HV, char* base, ChunkWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
+    const size_t seg_slots = (size_t)std::min<int64_t>((NC * HV + 3) / 4, SEG_SLOTS_MAX);
+    void* Seg = take(3 * seg_slots * 16384 * 4);
     void* Tab = take((size_t)NC * HV * WS_TAB * 4);
     void* Wf = take((size_t)NC * HV * WS_W * 2);
     void* Uf = take((size_t)NC * HV * WS_U * 2);
     void* Pf = take((size_t)NC * HV * WS_P * 2);
     void* KTf = take((size_t)NC * H * WS_KT * 2);
     void* Qf = take((size_t)NC * H * WS_Q * 2);
-    if (ws) { ws->Tab = (float*)Tab; ws->Wf = Wf; ws->Uf = Uf; ws->Pf = Pf; ws->KTf = KTf; ws->Qf = Qf; }
+    if (ws) { ws->Seg = (float*)Seg; ws->Tab = (float*)Tab; ws->Wf = Wf; ws->Uf = Uf; ws->Pf = Pf; ws->KTf = KTf; ws->Qf = Qf; }
     return off;
 }
 
@@ -127,8 +133,23 @@ __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* 
 }
 
 
+// Segment-parallel evaluation of long dense sequences: every sequence is cut into `nseg`
+// segments of `seg_chunks` chunks; per (sequence, head, segment) the buffers hold 128x128 fp32
+// matrices ([K][V], K-first): sloc = state reached from a zero state (segment 0: from the true
+// initial state), mseg = transition matrix, sin = merged state at the start of the segment.
+struct SegmentPlan {
+    int kind;
+    int nseg;
+    int seg_chunks;
+    float* sloc;
+    float* mseg;
+    float* sin;
+};
+
 // launchers defined next to their kernels
 template <typename T> int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream);
 template <typename T> int launch_scan_slab(const ChunkParams& p, hipStream_t stream);
+template <typename T> int launch_scan_wide(const ChunkParams& p, hipStream_t stream);
+template <typename T> int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
 
 }  // namespace gdn

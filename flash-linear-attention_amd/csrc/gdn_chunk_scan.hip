@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkParams p) {
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);       // then one global load
             }
         }
-        if (!lazy) {
+        if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {       // scalar branch: rare, must not be if-converted
             const float fold = fast_exp2(lg_try);
 #pragma unroll
             for (int i = 0; i < 2; ++i)

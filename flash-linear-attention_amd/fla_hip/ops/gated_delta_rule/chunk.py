@@ -6,6 +6,7 @@ solve, WY factors w/u, intra-chunk q k^T) and a sequential one (state recurrence
 the output), so per-chunk states are never written to memory."""
 from __future__ import annotations
 
+import os
 import warnings
 
 import torch
@@ -27,6 +28,8 @@ from fla_hip.utils import input_guard
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
 # the chunk size (only rounding does), so chunk_size 16 and 32 are accepted and run with 64.
 _KERNEL_CHUNK = 64
+# FLA_HIP_SCAN_MODE=slab|wide|segments forces one form of the sequential kernel (default: automatic)
+_SCAN_MODE_FLAGS = {'slab': _lib.FLAG_SCAN_SLAB, 'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS}
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 
@@ -80,6 +83,7 @@ class ChunkLaunch:
         g, beta, gb_code = unify_gate_beta(g, beta)
 
         flags = _lib.FLAG_STATE_V_FIRST if state_v_first else 0
+        flags |= _SCAN_MODE_FLAGS.get(os.environ.get('FLA_HIP_SCAN_MODE', 'auto'), 0)
         if cu_seqlens is not None:
             if cu_seqlens.dtype not in (torch.int32, torch.int64):
                 cu_seqlens = cu_seqlens.long()

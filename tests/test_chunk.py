@@ -56,6 +56,39 @@ def test_chunk_vs_oracle(B, T, H, HV, D, gate_div, with_h0, dtype):
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('mode', ['slab', 'wide', 'segments'])
+@pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
+    (2, 1000, 2, 4, True, False),
+    (1, 2100, 2, 2, True, True),          # ragged tail, V-first state layout
+    (3, 512, 1, 2, False, False),
+])
+def test_every_form_of_the_sequential_stage(monkeypatch, mode, B, T, H, HV, with_h0, vfirst):
+    """The three forms of the sequential kernel (value slabs, whole head per workgroup, time
+    segments with fp32 merge) are interchangeable: each must meet the oracle on its own."""
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, 128, 128, seed=21, gate_div=16.0,
+                                         h0_std=0.5 if with_h0 else None, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    if vfirst:
+        o, ht = _run(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), state_v_first=True)
+        ht = ht.transpose(-1, -2)
+    else:
+        o, ht = _run(q, k, v, g, beta, h0)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+@pytest.mark.parametrize('mode', ['slab', 'wide'])
+def test_varlen_every_form(monkeypatch, mode):
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
+    cu = [0, 1, 100, 101, 300, 1200, 2000]
+    q, k, v, g, beta, h0 = O.make_inputs(1, cu[-1], 2, 4, 128, 128, seed=23, gate_div=2.0, h0_std=0.5, N=6, dtype=torch.float16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)
+    o, ht = _run(q, k, v, g, beta, h0, cu)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 def test_against_token_recurrence_and_decode_handoff():
     """Prefill with the chunk op, continue with the recurrent op: equals one long recurrence."""
     from fla_hip.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
@@ -77,7 +110,11 @@ def test_against_token_recurrence_and_decode_handoff():
     ([0, 15, 100, 300, 1200, 2000], 2, 4, 64),
 ])
 @pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
-def test_varlen_vs_oracle_and_bit_exact_ownership(cu, H, HV, D, idx_dtype):
+@pytest.mark.parametrize('mode', ['slab', 'wide'])
+def test_varlen_vs_oracle_and_bit_exact_ownership(monkeypatch, cu, H, HV, D, idx_dtype, mode):
+    # the form of the sequential kernel is pinned so that the packed call and the single-sequence
+    # calls run the very same code: any difference is then a token or state given to the wrong sequence
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
     T, N = cu[-1], len(cu) - 1
     q, k, v, g, beta, h0 = O.make_inputs(1, T, H, HV, D, D, seed=11, gate_div=2.0, h0_std=0.5, N=N, dtype=torch.bfloat16)
     ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)
