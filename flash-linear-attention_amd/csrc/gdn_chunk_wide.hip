@@ -5,8 +5,9 @@
 // lanes, C/D layout == operand layout), so the dependent chain S -> w S -> v_new -> k^T v_new
 // -> S runs in registers with no barrier.  What the waves share are the A operands (w, q,
 // k^T, P, u fragments and the gate tables, 73 KB per chunk): they are copied verbatim from the
-// workspace into a double-buffered LDS stage, one chunk ahead, by asynchronous global->LDS
-// loads that use no registers; publishing that stage is the only barrier per chunk.
+// workspace into a double-buffered LDS stage by asynchronous global->LDS loads that use no
+// registers and are issued one and a half steps before their data is needed; two barriers per
+// chunk publish the two halves of a stage.
 //
 // The same kernel serves the segment-parallel evaluation of long sequences
 // (S_out = M S_in + S_loc per segment):
@@ -36,9 +37,13 @@ constexpr int WIDE_PASS2 = 2;     // per segment: from merged S_in -> o (last se
 // wave-uniform byte offset `lds_off` (+ 16 * lane).  Issued from inline assembly on purpose:
 // the compiler then does not order later LDS reads of the OTHER stage behind it; completion
 // is awaited explicitly (s_waitcnt vmcnt(0)) before the barrier that publishes the stage.
-__device__ __forceinline__ void copy_1k_to_lds(const char* gsrc_lane, uint32_t lds_off) {
-    lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make it a scalar
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_off), "v"(gsrc_lane));
+// `gsrc` is the wave-uniform source of the 1 KB piece (scalar base), `lane_off` = 16 * lane.
+__device__ __forceinline__ void copy_1k_to_lds(const char* gsrc, uint32_t lane_off, uint32_t lds_off) {
+    lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make them scalars
+    const uint64_t g = (uint64_t)gsrc;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+    const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(lane_off), "s"(gs));
 }
 
 template <typename T, bool FULL>
@@ -112,39 +117,54 @@ __global__ __launch_bounds__(256) void gdn_chunk_wide_kernel(ChunkParams p, Segm
     T* og = (T*)p.o;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 
-    // Every wave copies a quarter of the 1-KB pieces of a stage.  The copies are issued in four
-    // groups spread over a step (a burst of ~20 would block the issuing wave while the memory
-    // pipeline accepts them).
-    auto copy_group = [&](int64_t it, int stage, int grp) {
+    // Every wave copies a quarter of the 1-KB pieces of a stage.  A stage has two parts with
+    // separate lifetimes: the operands of the first half of a step (w, u, q, P, tables) and k^T,
+    // the operand of the state update in the second half.
+    auto copy_first = [&](int64_t it, int stage) {
         const int64_t ci = boh + it;
         const int64_t chv = ci * HV + hv, ch = ci * H + h;
         const uint32_t base = lds0 + stage * STG_BYTES;
-        const int l16 = lane * 16;
-        if (grp == 0) {
+        const uint32_t l16 = lane * 16;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) copy_1k_to_lds(Wf + chv * (WS_W * 2) + (4 * j + w) * 1024 + l16, base + STG_W + (4 * j + w) * 1024);
-            if (w == 0) copy_1k_to_lds(Tab + chv * (WS_TAB * 4) + l16, base + STG_TAB);
-        } else if (grp == 1) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) copy_1k_to_lds(Uf + chv * (WS_U * 2) + (4 * j + w) * 1024 + l16, base + STG_U + (4 * j + w) * 1024);
-        } else if (grp == 2) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) copy_1k_to_lds(KTf + ch * (WS_KT * 2) + (4 * j + w) * 1024 + l16, base + STG_KT + (4 * j + w) * 1024);
-        } else if constexpr (FULL) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) copy_1k_to_lds(Qf + ch * (WS_Q * 2) + (4 * j + w) * 1024 + l16, base + STG_Q + (4 * j + w) * 1024);
+        for (int j = 0; j < 4; ++j) {
+            const int pc = (4 * j + w) * 1024;
+            copy_1k_to_lds(Wf + chv * (WS_W * 2) + pc, l16, base + STG_W + pc);
+            copy_1k_to_lds(Uf + chv * (WS_U * 2) + pc, l16, base + STG_U + pc);
+            if constexpr (FULL) copy_1k_to_lds(Qf + ch * (WS_Q * 2) + pc, l16, base + STG_Q + pc);
+        }
+        if constexpr (FULL) {
             // P: workspace pieces 0,2,4,5,6,7 (the others are zero); wave w takes slot w, waves 0/1 also slots 4/5
             const int src0 = w < 2 ? 2 * w : w + 2;
-            copy_1k_to_lds(Pf + chv * (WS_P * 2) + src0 * 1024 + l16, base + STG_P + w * 1024);
-            if (w < 2) copy_1k_to_lds(Pf + chv * (WS_P * 2) + (6 + w) * 1024 + l16, base + STG_P + (4 + w) * 1024);
+            copy_1k_to_lds(Pf + chv * (WS_P * 2) + src0 * 1024, l16, base + STG_P + w * 1024);
+            if (w < 2) copy_1k_to_lds(Pf + chv * (WS_P * 2) + (6 + w) * 1024, l16, base + STG_P + (4 + w) * 1024);
+        }
+        if (w == 0) copy_1k_to_lds(Tab + chv * (WS_TAB * 4), l16, base + STG_TAB);
+    };
+    auto copy_kt = [&](int64_t it, int stage) {
+        const int64_t ch = (boh + it) * H + h;
+        const uint32_t base = lds0 + stage * STG_BYTES;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int pc = (4 * j + w) * 1024;
+            copy_1k_to_lds(KTf + ch * (WS_KT * 2) + pc, lane * 16, base + STG_KT + pc);
         }
     };
-    auto copy_stage = [&](int64_t it, int stage) {
-#pragma unroll
-        for (int grp = 0; grp < 4; ++grp) copy_group(it, stage, grp);
+    // A wave issues at least FIRST_MIN copies per copy_first and exactly 4 per copy_kt.  Loads
+    // complete in issue order, so "at most FIRST_MIN + 4 operations outstanding" proves that
+    // everything older than the last copy_first + copy_kt pair has landed (outstanding stores only
+    // make the wait longer).
+    auto wait_all_but_newest_pair = [&]() {
+        if constexpr (FULL) asm volatile("s_waitcnt vmcnt(17)" ::: "memory");      // 4 w + 4 u + 4 q + 1 P, + 4 k^T
+        else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");                     // 4 w + 4 u, + 4 k^T
     };
 
-    if (nsteps > 0) copy_stage(it0, 0);      // travels while the state is loaded
+    const int64_t lastc = it1 - 1;
+    if (nsteps > 0) {                         // these travel while the state is loaded
+        copy_first(it0, 0);
+        copy_kt(it0, 0);
+        copy_first(min(it0 + 1, lastc), 1);
+    }
+
 
     // ---- state: all key rows, value columns 32w .. 32w+31 (tiles n = 2w, 2w+1), C/D layout ----
     f32x4 S[8][2];
@@ -183,10 +203,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_wide_kernel(ChunkParams p, Segm
         }
     };
 
-    auto compute = [&](int64_t it, const char* st, int64_t it_next, int stage_next) {
+    V8 Vg[2][2];          // v_new decayed to the chunk end, B operand of the state update (first half -> second half)
+    auto first_half = [&](int64_t it, const char* st) {
         const V8* sW = (const V8*)(st + STG_W);
         const V8* sQ = (const V8*)(st + STG_Q);
-        const V8* sKT = (const V8*)(st + STG_KT);
         const V8* sP = (const V8*)(st + STG_P);
         const V4* sU = (const V4*)(st + STG_U);
         const float* sTab = (const float*)(st + STG_TAB);
@@ -205,12 +225,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_wide_kernel(ChunkParams p, Segm
         const float lg_try = lg + sTab[128];
         const bool lazy = lg_try >= LG_MIN;
         const float vscale = lazy ? fast_exp2(-lg_try) : 1.f;
-        V8 Vn[2][2], Vg[2][2];
-        copy_group(it_next, stage_next, 0);
+        V8 Vn[2][2];
         // two t-tiles at a time: w S -> v_new, and the output rows of those tiles
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            copy_group(it_next, stage_next, 1 + hf);
             f32x4 av[2][2], ao[2][2];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
@@ -278,10 +296,12 @@ __global__ __launch_bounds__(256) void gdn_chunk_wide_kernel(ChunkParams p, Segm
                 for (int nn = 0; nn < 2; ++nn) S[m][nn] *= fold;
         }
         lg = lazy ? lg_try : 0.f;
-        // S += k^T (v_new decayed)
+    };
+    // S += k^T (v_new decayed)
+    auto second_half = [&](const char* st) {
+        const V8* sKT = (const V8*)(st + STG_KT);
 #pragma unroll
         for (int mh = 0; mh < 4; ++mh) {
-            if (mh == 1) copy_group(it_next, stage_next, 3);
             V8 ak[2][2];
 #pragma unroll
             for (int mm = 0; mm < 2; ++mm)
@@ -297,19 +317,24 @@ __global__ __launch_bounds__(256) void gdn_chunk_wide_kernel(ChunkParams p, Segm
         }
     };
     if (nsteps > 0) {
-        const int64_t lastc = it1 - 1;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // first stage (and the state) have arrived
+        // (the loads of the initial state are older than the copies and complete before them)
+        wait_all_but_newest_pair();                             // the first half of stage 0 has landed
         __syncthreads();
         for (int64_t i = 0; i < nsteps; ++i) {
             const int64_t it = it0 + i;
             const int cur = (int)(i & 1);
-            // the next chunk's operands travel while this chunk is computed (the target stage was
-            // last read in the previous step, which every wave has left through the barrier)
+            char* st = smem + cur * STG_BYTES;
+            copy_kt(min(it + 1, lastc), cur ^ 1);               // that k^T region was last read before the previous barrier
             if constexpr (FULL) { if (i > 0) store_pending(it - 1); }
-            compute(it, smem + cur * STG_BYTES, min(it + 1, lastc), cur ^ 1);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // my copies have landed ...
-            lds_barrier();                                      // ... and so have everybody else's
+            first_half(it, st);
+            wait_all_but_newest_pair();                         // k^T of this chunk has landed ...
+            lds_barrier();                                      // ... everywhere, and nobody reads the first-half operands any more
+            copy_first(min(it + 2, lastc), cur);
+            second_half(st);
+            wait_all_but_newest_pair();                         // the first-half operands of the next chunk have landed ...
+            lds_barrier();                                      // ... everywhere, and nobody reads this k^T any more
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // no copy may land in LDS after this workgroup has gone
         if constexpr (FULL) store_pending(it1 - 1);
     }
 
