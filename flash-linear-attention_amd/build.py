@@ -21,7 +21,7 @@ OBJ_DIR = os.path.join(HERE, 'build', 'obj')
 
 HIPCC = os.environ.get('HIPCC', '/opt/rocm/bin/hipcc')
 FLAGS = [
-    '--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-fvisibility=default',
+    '--offload-arch=gfx950', '-O3', '-std=c++20', '-fPIC', '-fvisibility=default',
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
     # keep MFMA accumulators in ordinary VGPRs: the state and the products are read by vector ALU
     # instructions every chunk, and the AGPR form costs a copy per register each time
