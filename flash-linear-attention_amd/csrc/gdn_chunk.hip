@@ -1,6 +1,6 @@
 // C entry points of the chunked prefill (64-token chunks, K = V = 128): argument checks,
 // workspace layout and the choice of kernels.  The kernels live in gdn_chunk_prepare.hip
-// (chunk-parallel stage) and gdn_chunk_scan.hip (sequential stage).
+// (chunk-parallel stage) and gdn_chunk_wide.hip (sequential stage).
 #include "gdn_chunk_common.h"
 
 namespace gdn {
@@ -14,33 +14,28 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
         if (rc) return rc;
     }
     if (!(stages & STAGE_SCAN)) return GDN_OK;
-    // Which form of the sequential stage:
-    //   wide      one workgroup per (sequence, head): enough pairs to fill the CUs
-    //   segments  few pairs but long dense sequences: cut time into segments (3 wide passes + merge)
-    //   slab      otherwise: split the value columns of each head over several workgroups
+    // One workgroup per (sequence, head) walks the chunks of the sequence ("wide").  With few
+    // such pairs and long dense sequences, time is cut into segments instead so that every CU
+    // has a workgroup: two passes over 1/nseg of the chunks each plus a small merge.
     const bool dense = p.cu_seqlens == nullptr;
     int nseg = 0;
     if (dense && p.NH > 0) {
         nseg = (int)std::min<int64_t>((256 + p.NH / 2) / p.NH, p.NT / 4);
         if ((int64_t)nseg * p.NH > SEG_SLOTS_MAX || (int64_t)nseg * p.NH > (num_chunks * p.HV + 3) / 4) nseg = 0;
     }
-    int mode = p.NH >= 192 ? 1 : (nseg >= 2 ? 2 : 0);
-    if (p.flags & GDN_FLAG_SCAN_SLAB) mode = 0;
-    if (p.flags & GDN_FLAG_SCAN_WIDE) mode = 1;
-    if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) mode = 2;
-    if (mode == 1) return launch_scan_wide<T>(p, stream);
-    if (mode == 2) {
-        SegmentPlan sp;
-        sp.kind = 0;
-        sp.nseg = nseg;
-        sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
-        const size_t slots = (size_t)p.NH * nseg;
-        sp.sloc = p.ws.Seg;
-        sp.mseg = p.ws.Seg + slots * 16384;
-        sp.sin = p.ws.Seg + 2 * slots * 16384;
-        return launch_scan_segments<T>(p, sp, stream);
-    }
-    return launch_scan_slab<T>(p, stream);
+    bool segments = nseg >= 3;           // two passes of NT/nseg steps each must beat one pass of NT steps
+    if (p.flags & GDN_FLAG_SCAN_WIDE) segments = false;
+    if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
+    if (!segments) return launch_scan_wide<T>(p, stream);
+    SegmentPlan sp;
+    sp.kind = 0;
+    sp.nseg = nseg;
+    sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
+    const size_t slots = (size_t)p.NH * nseg;
+    sp.sloc = p.ws.Seg;
+    sp.mseg = p.ws.Seg + slots * 16384;
+    sp.sin = p.ws.Seg + 2 * slots * 16384;
+    return launch_scan_segments<T>(p, sp, stream);
 }
 
 }  // namespace gdn
@@ -86,7 +81,7 @@ static int chunk_entry(
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
-    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.nslab = 1; p.NH = N * HV;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.NH = N * HV;
     hipStream_t s = (hipStream_t)stream;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, stages, s)
                                        : launch_chunk<f16_t>(p, num_chunks, stages, s);

@@ -5,7 +5,7 @@
 //   B operand (32 x N): lane holds column c16, the same 8 contraction indices;
 //   C/D (16 x 16):      lane holds column c16, rows 4g..4g+3.
 // Any assignment of contraction indices to (g, element) is valid as long as A and B agree.
-// The scan kernels use {16a+4g+r} U {16b+4g+r} for a pair of 16-row tiles (a, b): that is
+// The scan kernel uses {16a+4g+r} U {16b+4g+r} for a pair of 16-row tiles (a, b): that is
 // exactly how a C/D result is spread over lanes, so an accumulator can be converted in
 // place into the B operand of the next product, and swapping the two operands of an MFMA
 // yields the transposed tile.
@@ -55,40 +55,36 @@ __device__ __forceinline__ V8 join(V4 a, V4 b) {
 // 2^x as a single v_exp_f32 (results below 2^-126 flush to zero, which is what a decay wants)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Per-chunk workspace written by the prepare kernel (element counts for K = V = 128):
-//   Tab fp32 [NC][HV][256]                  [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128] G_last (log2 units)
-//   Wf  T    [NC][HV][4 tt][4 s][64][8]     w rows of t-tile tt, key tiles (2s, 2s+1)
-//   Uf  T    [NC][HV][8 n ][4 tt][64][4]    u, C/D layout of tile (t-tile tt, value tile n)
-//   Pf  T    [NC][HV][4 tt][2 s][64][8]     scale*P rows of t-tile tt, t-tiles (2s, 2s+1) as columns
-//   KTf T    [NC][H ][8 m ][2 s][64][8]     k^T rows of key tile m, t-tiles (2s, 2s+1)
-//   Qf  T    [NC][H ][4 tt][4 s][64][8]     q rows of t-tile tt, key tiles (2s, 2s+1)
+// Workspace record written by the prepare kernel per (chunk, v-head): 13 KB that the scan
+// copies verbatim into LDS.  Xb and P are stored as matrix-core operand fragments
+// ([slot][lane][8]): rows of t-tile tt, columns t' in {32sp+4g+r} U {32sp+16+4g+r}.  Both are
+// lower triangular, so the fragments (tt, sp) = (0,1), (1,1) are identically zero and are not
+// stored; the other six live in slot p_slot(tt, sp).
+//   Xb  T    [6][64][8]   (I+L)^-1 diag(beta)
+//   P   T    [6][64][8]   scale * tril(q k^T 2^(G_t-G_t'))
+//   tab fp32 [256]        [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units)
+constexpr int REC_X = 0, REC_P = 6144, REC_TAB = 12288;
+constexpr int64_t REC_BYTES = 13312;
+constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
+__host__ __device__ constexpr int p_slot(int tt, int sp) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp; }
+
 struct ChunkWs {
     float* Seg;          // 3 * seg_slots 128x128 fp32 matrices for the segment-parallel scan
-    float* Tab;
-    void* Wf;
-    void* Uf;
-    void* Pf;
-    void* KTf;
-    void* Qf;
+    char* Rec;           // [NC][HV] records
 };
-constexpr int64_t WS_TAB = 256, WS_W = 8192, WS_U = 8192, WS_P = 4096, WS_KT = 8192, WS_Q = 8192;   // elements per (chunk, head)
 
 constexpr int64_t SEG_SLOTS_MAX = 640;            // upper bound on (sequences * heads * segments) when segmenting
 
 inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 inline size_t ws_layout(int64_t NC, int64_t H, int64_t HV, char* base, ChunkWs* ws) {
+    (void)H;
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
     const size_t seg_slots = (size_t)std::min<int64_t>((NC * HV + 3) / 4, SEG_SLOTS_MAX);
     void* Seg = take(3 * seg_slots * 16384 * 4);
-    void* Tab = take((size_t)NC * HV * WS_TAB * 4);
-    void* Wf = take((size_t)NC * HV * WS_W * 2);
-    void* Uf = take((size_t)NC * HV * WS_U * 2);
-    void* Pf = take((size_t)NC * HV * WS_P * 2);
-    void* KTf = take((size_t)NC * H * WS_KT * 2);
-    void* Qf = take((size_t)NC * H * WS_Q * 2);
-    if (ws) { ws->Seg = (float*)Seg; ws->Tab = (float*)Tab; ws->Wf = Wf; ws->Uf = Uf; ws->Pf = Pf; ws->KTf = KTf; ws->Qf = Qf; }
+    void* Rec = take((size_t)NC * HV * REC_BYTES);
+    if (ws) { ws->Seg = (float*)Seg; ws->Rec = (char*)Rec; }
     return off;
 }
 
@@ -99,7 +95,7 @@ struct ChunkParams {
     ChunkWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;       // NT: chunks per sequence (dense input)
     float scale; int gb_dtype; uint32_t flags;
-    int nslab; int64_t NH;
+    int64_t NH;
 };
 
 // Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains
@@ -107,16 +103,6 @@ struct ChunkParams {
 // behind every barrier of the current one.
 __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-// 8-byte global store issued from inline assembly.  The compiler's wait-count bookkeeping
-// does not see it, so the prefetched loads of the scan loop stay the only operations it
-// counts and it can wait for "all but the newest N loads" instead of draining the queue
-// (loads and stores share one hardware counter, and once both are pending the compiler
-// falls back to waiting for everything).  The extra, uncounted stores only make the
-// hardware counter larger than the compiler assumes, i.e. its waits err on the late side.
-__device__ __forceinline__ void store_b64_uncounted(void* ptr, u32x2 data) {
-    asm volatile("global_store_dwordx2 %0, %1, off" : : "v"(ptr), "v"(data) : "memory");
 }
 
 // 16x16 product of fp32 matrices held in LDS on the fp32 matrix cores:
@@ -148,7 +134,6 @@ struct SegmentPlan {
 
 // launchers defined next to their kernels
 template <typename T> int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream);
-template <typename T> int launch_scan_slab(const ChunkParams& p, hipStream_t stream);
 template <typename T> int launch_scan_wide(const ChunkParams& p, hipStream_t stream);
 template <typename T> int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
 

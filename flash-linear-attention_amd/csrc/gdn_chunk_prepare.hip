@@ -1,31 +1,18 @@
 // Chunk-parallel stage of the chunked prefill: one workgroup per (chunk, v-head) computes
-// everything that does not depend on the running state:
-//   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  A = (I+L)^-1 in fp32 (16x16 forward
-//   substitution on the diagonal blocks, fp32-MFMA block merges),  w = A (beta*2^G*k),
-//   u = A (beta*v),  P = scale*tril(q k^T * 2^(G_i-G_j)).
-// Results are written in the exact register order ("fragments") in which the scan kernels
-// feed them to the matrix cores, so those kernels need no transposes.
+// what does not depend on the running state and is not a plain copy of the inputs:
+//   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  X = (I+L)^-1 in fp32 (16x16 forward
+//   substitution on the diagonal blocks, fp32-MFMA block merges),  Xb = X diag(beta),
+//   P = scale*tril(q k^T * 2^(G_i-G_j)),  and the per-token gate tables.
+// Xb and P are written in the exact register order ("fragments") in which the scan kernel
+// feeds them to the matrix cores; the scan forms v_new = Xb (v - 2^G (k S)) itself from the
+// raw k and v, so neither w = Xb 2^G k nor u = Xb v is ever materialised.
 #include "gdn_chunk_common.h"
 
 namespace gdn {
 
 constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 272 B rows, conflict-free 16 B reads
 constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
-constexpr size_t PREP_SMEM = 3 * CH * NP * 2 + 3 * CH * 4;     // 52 992 B: three workgroups per CU
-
-// Transposed MFMA operand from a token-major tile: lane (c16, g) gets column fb + c16 of the
-// 8 rows r0 .. r0+7 (two transpose reads of 4 rows each).
-template <typename T>
-__device__ __forceinline__ typename Mma<T>::V8 tr_frag8(const T* tile, int r0, int fb, int c16) {
-    const T* a = tile + (r0 + (c16 >> 2)) * NP + fb + 4 * (c16 & 3);
-    return join<typename Mma<T>::V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * NP));
-}
-// Same for two separate groups of 4 rows starting at ra and rb.
-template <typename T>
-__device__ __forceinline__ typename Mma<T>::V8 tr_frag44(const T* tile, int ra, int rb, int fb, int c16) {
-    const int o = (c16 >> 2) * NP + fb + 4 * (c16 & 3);
-    return join<typename Mma<T>::V8>(Mma<T>::tr_read(tile + ra * NP + o), Mma<T>::tr_read(tile + rb * NP + o));
-}
+constexpr size_t PREP_SMEM = 3 * CH * NP * 2 + 2 * CH * 4;     // 52 736 B: three workgroups per CU
 
 template <typename T>
 __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
@@ -34,19 +21,16 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
     extern __shared__ __align__(16) char smem[];
     T* k_nat = (T*)smem;                        // [64][NP] keys, token-major
     T* q_nat = k_nat + CH * NP;                 // [64][NP] queries; the region is reused for X below
-    T* v_nat = q_nat + CH * NP;                 // [64][NP] values; staged only after the solve (same bytes as L)
-    float* sL = (float*)v_nat;                  // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
+    float* sL = (float*)(q_nat + CH * NP);      // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
     float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1, same bytes as q_nat
-    float* sG = (float*)(v_nat + CH * NP);      // [64] cumulative gate (log2)
+    float* sG = sL + CH * LP;                   // [64] cumulative gate (log2)
     float* sB = sG + CH;                        // [64] beta
-    float* sBG = sB + CH;                       // [64] beta * 2^G
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     const int64_t ci = blockIdx.x;
     const int hv = blockIdx.y;
     const int H = p.H, HV = p.HV;
     const int h = hv / (HV / H);
-    const bool first_of_group = hv % (HV / H) == 0;      // writes the per-q/k-head fragments
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
 
     int64_t tok0;
@@ -62,22 +46,21 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
 
-    // ---- stage k, q, v (rows past the end of the sequence are zero) ----
+    // ---- stage k, q (rows past the end of the sequence are zero) ----
     const T* kg = (const T*)p.k + (tok0 * H + h) * 128;
     const T* qg = (const T*)p.q + (tok0 * H + h) * 128;
-    const T* vg = (const T*)p.v + (tok0 * HV + hv) * 128;
-    u32x4 rk[4], rq[4], rv[4];
+    u32x4 rk[4], rq[4];
 #pragma unroll
     for (int ps = 0; ps < 4; ++ps) {
         const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
         const u32x4 z = {0u, 0u, 0u, 0u};
-        rk[ps] = rq[ps] = rv[ps] = z;
+        rk[ps] = rq[ps] = z;
         if (row < valid) {
             rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * 128 + col);
             rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * 128 + col);
-            rv[ps] = *(const u32x4*)(vg + (int64_t)row * HV * 128 + col);
         }
     }
+    char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
     // ---- gates: inclusive scan over the chunk (wave 0, one token per lane) ----
     if (w == 0) {
         float x = 0.f, b = 0.f;
@@ -95,11 +78,11 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         const float ex = fast_exp2(x);
         sG[lane] = x;
         sB[lane] = b;
-        sBG[lane] = b * ex;
-        float* tab = p.ws.Tab + (ci * HV + hv) * WS_TAB;
-        tab[lane] = fast_exp2(xl - x);
-        tab[64 + lane] = p.scale * ex;
-        if (lane == 63) tab[128] = x;
+        float* tab = (float*)(rec + REC_TAB);
+        tab[TAB_DEC + lane] = fast_exp2(xl - x);
+        tab[TAB_SG + lane] = p.scale * ex;
+        tab[TAB_EG + lane] = ex;
+        if (lane == 63) tab[TAB_GLAST] = x;
     }
 #pragma unroll
     for (int ps = 0; ps < 4; ++ps) {
@@ -142,8 +125,9 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         for (int s = 0; s < 4; ++s) qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
         const int t = 16 * tt + c16;
         const float gt = sG[t];
-        T* pf = (T*)p.ws.Pf + (ci * HV + hv) * WS_P;
+        T* pf = (T*)(rec + REC_P);
         for (int sp = 0; sp < 2; ++sp) {
+            if (tt < 2 && sp == 1) continue;        // identically zero, not stored
             V8 frag;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
@@ -164,16 +148,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
                     frag[half * 4 + r] = from_f32<T>(val);
                 }
             }
-            *(V8*)(pf + ((tt * 2 + sp) * 64 + lane) * 8) = frag;
-        }
-        // q rows of t-tile tt as A operands over key tiles (2s, 2s+1), one copy per q/k head
-        if (first_of_group) {
-            T* qf = (T*)p.ws.Qf + (ci * H + h) * WS_Q;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const T* src = q_nat + (16 * tt + c16) * NP + 32 * s + 4 * g;
-                *(V8*)(qf + ((tt * 4 + s) * 64 + lane) * 8) = join<V8>(*(const V4*)src, *(const V4*)(src + 16));
-            }
+            *(V8*)(pf + (p_slot(tt, sp) * 64 + lane) * 8) = frag;
         }
     }
     __syncthreads();     // L complete; q_nat is dead from here on and becomes X
@@ -231,72 +206,21 @@ __global__ __launch_bounds__(256) void gdn_chunk_prepare_kernel(ChunkParams p) {
         for (int r = 0; r < 4; ++r) sX[(32 + 16 * a + 4 * g + r) * LP + 16 * b + c16] = -z[r];
     }
     __syncthreads();
-    // L is dead: its bytes now take the value tile, which has been waiting in registers
-#pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-        const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
-        *(u32x4*)(v_nat + row * NP + col) = rv[ps];
-    }
-    __syncthreads();
-
-    // ---- w^T = k^T (diag(beta 2^G) X^T) and u = (X diag(beta)) v for t-tile w ----
-    const int ns = (w >= 2) ? 2 : 1;         // X is lower triangular: columns >= 32 matter only for rows >= 32
-    V8 fw[2], fu[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        if (s < ns) {
-            const float* xr = sX + (16 * w + c16) * LP + 32 * s + 8 * g;
-            const f32x4 x0 = *(const f32x4*)xr, x1 = *(const f32x4*)(xr + 4);
-            const f32x4 bg0 = *(const f32x4*)(sBG + 32 * s + 8 * g), bg1 = *(const f32x4*)(sBG + 32 * s + 8 * g + 4);
-            const f32x4 b0 = *(const f32x4*)(sB + 32 * s + 8 * g), b1 = *(const f32x4*)(sB + 32 * s + 8 * g + 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                fw[s][e] = from_f32<T>(x0[e] * bg0[e]);
-                fw[s][4 + e] = from_f32<T>(x1[e] * bg1[e]);
-                fu[s][e] = from_f32<T>(x0[e] * b0[e]);
-                fu[s][4 + e] = from_f32<T>(x1[e] * b1[e]);
-            }
-        }
-    }
+    // ---- Xb = X diag(beta) rows of t-tile w as A-operand fragments ----
     {
-        T* wf = (T*)p.ws.Wf + (ci * HV + hv) * WS_W;
-#pragma unroll
-        for (int sp = 0; sp < 4; ++sp) {
+        T* xf = (T*)(rec + REC_X);
+        const int ns = (w >= 2) ? 2 : 1;         // X is lower triangular: columns >= 32 matter only for rows >= 32
+        for (int sp = 0; sp < ns; ++sp) {
+            const float* xr = sX + (16 * w + c16) * LP + 32 * sp + 4 * g;
+            const f32x4 x0 = *(const f32x4*)xr, x1 = *(const f32x4*)(xr + 16);
+            const f32x4 b0 = *(const f32x4*)(sB + 32 * sp + 4 * g), b1 = *(const f32x4*)(sB + 32 * sp + 16 + 4 * g);
             V8 frag;
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int m = 2 * sp + half;
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    if (s < ns) acc = Mma<T>::run(tr_frag8<T>(k_nat, 32 * s + 8 * g, 16 * m, c16), fw[s], acc);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) frag[half * 4 + r] = from_f32<T>(acc[r]);
+            for (int e = 0; e < 4; ++e) {
+                frag[e] = from_f32<T>(x0[e] * b0[e]);
+                frag[4 + e] = from_f32<T>(x1[e] * b1[e]);
             }
-            *(V8*)(wf + ((w * 4 + sp) * 64 + lane) * 8) = frag;
-        }
-        T* uf = (T*)p.ws.Uf + (ci * HV + hv) * WS_U;
-#pragma unroll
-        for (int n = 0; n < 8; ++n) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-                if (s < ns) acc = Mma<T>::run(fu[s], tr_frag8<T>(v_nat, 32 * s + 8 * g, 16 * n, c16), acc);
-            V4 o4;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
-            *(V4*)(uf + ((n * 4 + w) * 64 + lane) * 4) = o4;
-        }
-    }
-    // ---- k^T fragments for the state update (one copy per q/k head) ----
-    if (first_of_group) {
-        T* ktf = (T*)p.ws.KTf + (ci * H + h) * WS_KT;
-#pragma unroll
-        for (int mm = 0; mm < 2; ++mm) {
-            const int m = 2 * w + mm;
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-                *(V8*)(ktf + ((m * 2 + s) * 64 + lane) * 8) = tr_frag44<T>(k_nat, 32 * s + 4 * g, 32 * s + 16 + 4 * g, 16 * m, c16);
+            *(V8*)(xf + (p_slot(w, sp) * 64 + lane) * 8) = frag;
         }
     }
 }

@@ -1,55 +1,67 @@
-// Sequential stage of the chunked prefill, "wide" form: one workgroup per (sequence, v-head,
-// segment of consecutive chunks) holds the WHOLE fp32 state S[128, 128] in registers.
+// Sequential stage of the chunked prefill: one workgroup per (sequence, v-head, segment of
+// consecutive chunks) holds the WHOLE fp32 state S[128, 128] in registers and walks the
+// chunks in order.  Per chunk, with Xb = (I+L)^-1 diag(beta), P and the gate tables from the
+// prepare kernel and the raw q, k, v tiles:
+//   D     = v - 2^G (k S)                      (the delta-rule residual of every token)
+//   v_new = Xb D                               (== u - w S of the WY form)
+//   o     = scale 2^G (q S) + P v_new
+//   S     = 2^G_last S + k^T (v_new 2^(G_last-G))
 //
-// Ten waves.  Eight compute waves: wave w owns value columns 16w .. 16w+15 for all key rows.
-// Nothing of the recurrence crosses waves: bf16(S) and bf16(v_new) are the B operands of this
-// wave's own next products (same lanes, C/D layout == operand layout), so the dependent chain
-// S -> w S -> v_new -> k^T v_new -> S runs in registers.  Two waves per SIMD let one wave's
-// vector-ALU work overlap the other's matrix instructions.  The compute waves issue no global
-// memory instruction inside the loop.
-// Two copy waves move everything else: what the compute waves share are the A operands (w, q,
-// k^T, P, u fragments and the gate tables, 71 KB per chunk); they are copied verbatim from the
-// workspace into a double-buffered LDS stage by asynchronous global->LDS loads that use no
-// registers, and the output tile of a chunk goes LDS -> registers -> global in 256-byte rows.
-// Two barriers per chunk (after each half of a step) are the only synchronisation.
+// Twelve waves.  Eight compute waves: wave w owns value columns 16w .. 16w+15 for all key
+// rows.  Nothing of the recurrence crosses waves: bf16(S), bf16(D) and bf16(v_new) are the B
+// operands of this wave's own next products (same lanes, C/D layout == operand layout), so
+// the dependent chain runs in registers.  Two compute waves per SIMD let one wave's vector-ALU
+// work overlap the other's matrix instructions.  The compute waves issue no global memory
+// instruction inside the loop.
+// Four copy waves move everything else.  Three of them fill a double-buffered LDS stage with
+// asynchronous global->LDS loads that use no registers: the prepare record verbatim, and the
+// q, k, v tiles gathered straight from the user's tensors in 16-byte pieces, placed so that
+// the matrix-core operands are conflict-free 16-byte LDS reads (q, k rows) or LDS transpose
+// reads (k^T, v).  The fourth moves the output tile of a chunk LDS -> registers -> global in
+// 256-byte rows.  Two barriers per chunk (after each half of a step) are the only
+// synchronisation.
+//
+// State rows are permuted inside the registers so that the 8 contraction indices a lane
+// feeds to the matrix core are 8 CONSECUTIVE key features (one 16-byte piece of a q or k
+// row): tile m, row 4g+r holds key feature 32*(m/2) + 8g + 4*(m%2) + r.
 //
 // The same kernel serves the segment-parallel evaluation of long sequences
 // (S_out = M S_in + S_loc per segment):
 //   pass 1  state only (no q / P / output), started from the true initial state (first
-//           segment), from zero (S_loc) or from the identity with u = 0 (the transition M);
+//           segment), from zero (S_loc) or from the identity with v = 0 (the transition M);
 //   merge   S_in[j+1] = M_j S_in[j] + S_loc,j in fp32 (gdn_segment_merge_kernel);
 //   pass 2  full evaluation of every segment from its merged initial state.
 #include "gdn_chunk_common.h"
 
 namespace gdn {
 
-// LDS stage = verbatim copy of one chunk's workspace fragments
-constexpr int STG_W = 0, STG_Q = 16384, STG_KT = 32768, STG_P = 49152, STG_U = 55296, STG_TAB = 71680;
-constexpr int STG_BYTES = 72704;                  // W 16K, Q 16K, k^T 16K, P 6K (the 6 non-zero pieces), u 16K, tables 1K
+// LDS stage of one chunk.  q, k, v: [4 tt][4 s][64 lanes][16 B], piece (tt, s, 16g+c16) = bytes
+// [64s+16g, +16) of token row 16tt+c16.
+constexpr int STG_K = 0, STG_Q = 16384, STG_V = 32768, STG_REC = 49152;
+constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB;
+constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 62 464
 constexpr int OT_PITCH = 272;                     // bytes per token row of the output tile (256 B + pad: conflict-free 8-byte writes)
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
-constexpr size_t WIDE_SMEM = 2 * STG_BYTES + OT_BYTES;       // 162 816 B of the CU's 163 840: one workgroup per CU
+constexpr size_t WIDE_SMEM = 2 * STG_BYTES + OT_BYTES;       // 142 336 B: one workgroup per CU
 constexpr int CW = 8;                             // compute waves
-constexpr int WIDE_THREADS = (CW + 2) * 64;
-// P pieces (t-tile tt, column pair sp2) -> slot in the stage; (0,1) and (1,1) are identically zero and not staged
-__host__ __device__ constexpr int p_slot(int tt, int sp2) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp2; }
+constexpr int WIDE_THREADS = (CW + 4) * 64;
 
 // kind of run
 constexpr int WIDE_WHOLE = 0;     // whole sequences, user h0 -> o, ht
 constexpr int WIDE_PASS1 = 1;     // per segment: S_loc / M into the segment buffers
 constexpr int WIDE_PASS2 = 2;     // per segment: from merged S_in -> o (last segment also ht)
 
-// Asynchronous copy of 1 KB (16 bytes per lane) from global memory straight into LDS at the
-// wave-uniform byte offset `lds_off` (+ 16 * lane).  Issued from inline assembly on purpose:
-// the compiler then keeps no account of it, and completion is awaited explicitly with
-// s_waitcnt vmcnt before the barrier that publishes the data.
-// `gsrc` is the wave-uniform source of the 1 KB piece (scalar base), `lane_off` = 16 * lane.
-__device__ __forceinline__ void copy_1k_to_lds(const char* gsrc, uint32_t lane_off, uint32_t lds_off) {
+// Asynchronous copy of 64 x 16 bytes from global memory straight into LDS: lane l fetches the
+// 16 bytes at gbase + voff (gbase wave-uniform, voff per lane) and they land at the
+// wave-uniform LDS byte offset `lds_off` + 16 l.  Issued from inline assembly on purpose: the
+// compiler then keeps no account of it, and completion is awaited explicitly with s_waitcnt
+// vmcnt before the barrier that publishes the data.
+__device__ __forceinline__ void gather_1k_to_lds(const char* gbase, uint32_t voff, uint32_t lds_off) {
     lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make them scalars
-    const uint64_t g = (uint64_t)gsrc;
+    const uint64_t g = (uint64_t)gbase;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
     const uint64_t gs = ((uint64_t)hi << 32) | lo;
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(lane_off), "s"(gs));
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(voff), "s"(gs));
 }
 
 template <int N>
@@ -74,7 +86,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     int64_t inh;
     int seg;
     int init = 0;                 // 0: from `src` (NULL = zero state), 1: identity, 2: zero
-    bool u_zero = false, src_user = false, dst_user = false;
+    bool v_zero = false, src_user = false, dst_user = false;
     const float* src = nullptr;
     float* dst = nullptr;
     if (sp.kind == WIDE_WHOLE) {
@@ -92,7 +104,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             dst = sp.sloc + (inh * sp.nseg + seg) * 16384;
         } else {
             seg = idx - (sp.nseg - 1) + 1;
-            init = 1; u_zero = true;
+            init = 1; v_zero = true;
             dst = sp.mseg + (inh * sp.nseg + seg) * 16384;
         }
     } else {
@@ -126,76 +138,94 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // =====================================================================================
     // Copy waves.  Step i (chunk it = it0 + i, stage cur = i & 1) has two phases, separated by
     // the workgroup barriers B1 (after the first half) and B2 (after the second half):
-    //   phase A  compute waves read w, q, P, u, tables of stage cur and write the output tile
-    //   phase B  compute waves read k^T of stage cur
-    // Loads complete in issue order, so "at most N operations outstanding" proves that all but
-    // the N newest have landed; outstanding stores only make such a wait longer.
+    //   phase A  compute waves read everything of stage cur and write the output tile
+    //   phase B  compute waves read k of stage cur (transposed)
+    // so the q / v / record part of a stage is free from B1 on and its k part from B2 on; all of
+    // chunk it+1 must be in the other stage at B2.  Loads complete in issue order, so "at most
+    // N operations outstanding" proves that all but the N newest have landed.
     // =====================================================================================
     if (w >= CW) {
         if (nsteps <= 0) return;
-        const char* Wf = (const char*)p.ws.Wf;
-        const char* Uf = (const char*)p.ws.Uf;
-        const char* KTf = (const char*)p.ws.KTf;
-        const char* Pf = (const char*)p.ws.Pf;
-        const char* Qf = (const char*)p.ws.Qf;
-        const char* Tab = (const char*)p.ws.Tab;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-        const uint32_t l16 = lane * 16;
+        // Row gather: the four 1-KB pieces (s = 0..3) of t-tile tt of a [token][head][128] tensor.
+        // Rows past the end of the sequence re-read its last row: whatever they hold is finite and
+        // is multiplied by the zero columns of Xb, the zero rows of v_new and the causal zeros of P.
+        auto gather_tile = [&](const T* tensor, int heads, int head, int64_t it, int tt, uint32_t lds_tile) {
+            const int64_t tok0 = bos + it * CH;
+            const int valid = (int)min((int64_t)CH, len - it * CH);
+            const int row = min(16 * tt + c16, valid - 1);
+            const uint32_t voff = (uint32_t)row * (uint32_t)(heads * 256) + 16 * g;
+            const char* base = (const char*)(tensor + (tok0 * heads + head) * 128);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) gather_1k_to_lds(base + 64 * s, voff, lds_tile + (tt * 4 + s) * 1024);
+        };
+        auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage) {
+            const char* rec = p.ws.Rec + ((boh + it) * HV + hv) * REC_BYTES;
+#pragma unroll
+            for (int j = 0; j < 13; ++j)
+                if (j >= from && j < to) gather_1k_to_lds(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024);
+        };
         if (w == CW) {
-            // ---- first-half operands: NOPS one-KB pieces per chunk, pieces [0, XA) are issued in
-            // phase B of step c-2 and the rest in phase A of step c-1 (their LDS region is free from
-            // B1 of step c-2 on); all must have landed at B2 of step c-1.
-            constexpr int NOPS = FULL ? 55 : 33;
-            constexpr int XA = 16;
-            auto piece = [&](auto op_c, int64_t it, int stage) {
-                constexpr int op = decltype(op_c)::value;
-                const int64_t ci = boh + it;
-                const int64_t chv = ci * HV + hv, ch = ci * H + h;
-                const uint32_t base = lds0 + stage * STG_BYTES;
-                if constexpr (op < 16) copy_1k_to_lds(Wf + chv * (WS_W * 2) + op * 1024, l16, base + STG_W + op * 1024);
-                else if constexpr (op < 32) copy_1k_to_lds(Uf + chv * (WS_U * 2) + (op - 16) * 1024, l16, base + STG_U + (op - 16) * 1024);
-                else if constexpr (op == 32) copy_1k_to_lds(Tab + chv * (WS_TAB * 4), l16, base + STG_TAB);
-                else if constexpr (op < 49) copy_1k_to_lds(Qf + ch * (WS_Q * 2) + (op - 33) * 1024, l16, base + STG_Q + (op - 33) * 1024);
-                else {
-                    // P: workspace pieces 0,2,4,5,6,7 (the others are zero) go to slots 0..5
-                    constexpr int slot = op - 49, srcp = slot < 2 ? 2 * slot : slot + 2;
-                    copy_1k_to_lds(Pf + chv * (WS_P * 2) + srcp * 1024, l16, base + STG_P + slot * 1024);
+            // ---- k: issued at the start of a step for the next chunk, awaited at its end ----
+            auto issue_k = [&](int64_t it, int stage) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) gather_tile((const T*)p.k, H, h, it, tt, lds0 + stage * STG_BYTES + STG_K);
+            };
+            issue_k(it0, 0);
+            wait_vm_at_most<0>();
+            lds_barrier();                                                  // B0: stage 0 is complete
+            for (int64_t i = 0; i < nsteps; ++i) {
+                issue_k(min(it0 + i + 1, lastc), (int)((i & 1) ^ 1));
+                lds_barrier();                                              // B1
+                wait_vm_at_most<0>();
+                lds_barrier();                                              // B2
+            }
+        } else if (w <= CW + 2) {
+            // ---- q + Xb + tables (wave CW+1) and v + P (wave CW+2): NOPS pieces per chunk.  Pieces
+            // [0, XB) of chunk c are issued in phase B of step c-2, the rest in phase A of step c-1.
+            const bool qside = (w == CW + 1);
+            constexpr int XB = 8;
+            auto issue = [&](int64_t it, int stage, bool early) {
+                const uint32_t st = lds0 + stage * STG_BYTES;
+                if (qside) {
+                    if constexpr (FULL) {
+                        // 16 q pieces, then Xb (6) and the tables (1)
+                        if (early) { gather_tile((const T*)p.q, H, h, it, 0, st + STG_Q); gather_tile((const T*)p.q, H, h, it, 1, st + STG_Q); }
+                        else { gather_tile((const T*)p.q, H, h, it, 2, st + STG_Q); gather_tile((const T*)p.q, H, h, it, 3, st + STG_Q); copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }
+                    } else {
+                        if (early) { copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }      // all 7 pieces
+                    }
+                } else {
+                    if (early) { gather_tile((const T*)p.v, HV, hv, it, 0, st + STG_V); gather_tile((const T*)p.v, HV, hv, it, 1, st + STG_V); }
+                    else {
+                        gather_tile((const T*)p.v, HV, hv, it, 2, st + STG_V); gather_tile((const T*)p.v, HV, hv, it, 3, st + STG_V);
+                        if constexpr (FULL) copy_rec(it, 6, 12, st);
+                    }
                 }
             };
-            auto issue = [&](auto from_c, auto to_c, int64_t it, int stage) {
-                constexpr int from = decltype(from_c)::value, to = decltype(to_c)::value;
-                [&]<int... I>(std::integer_sequence<int, I...>) {
-                    (piece(std::integral_constant<int, from + I>{}, it, stage), ...);
-                }(std::make_integer_sequence<int, to - from>{});
+            // number of pieces issued early: 8, except 7 for the q side of a state-only run
+            auto wait_early_only = [&]() {
+                if (!FULL && qside) wait_vm_at_most<7>();
+                else wait_vm_at_most<XB>();
             };
-            std::integral_constant<int, 0> c0;
-            std::integral_constant<int, XA> cx;
-            std::integral_constant<int, NOPS> cn;
-            issue(c0, cn, it0, 0);
-            issue(c0, cx, min(it0 + 1, lastc), 1);
-            wait_vm_at_most<XA>();
-            lds_barrier();                                                  // B0: stage 0 is complete
+            issue(it0, 0, true);
+            issue(it0, 0, false);
+            issue(min(it0 + 1, lastc), 1, true);
+            wait_early_only();
+            lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 const int64_t it = it0 + i;
                 const int cur = (int)(i & 1);
-                issue(cx, cn, min(it + 1, lastc), cur ^ 1);
+                issue(min(it + 1, lastc), cur ^ 1, false);
                 lds_barrier();                                              // B1
-                issue(c0, cx, min(it + 2, lastc), cur);
-                wait_vm_at_most<XA>();                                      // the first-half operands of chunk it+1 have landed
+                issue(min(it + 2, lastc), cur, true);
+                wait_early_only();                                          // chunk it+1 is complete
                 lds_barrier();                                              // B2
             }
-            wait_vm_at_most<0>();                                           // no copy may land in LDS after this workgroup has gone
         } else {
-            // ---- k^T (16 pieces per chunk, issued in phase A one step ahead) and the output rows
+            // ---- output rows: one instruction stores 4 token rows of 256 bytes ----
             T* og = (T*)p.o;
             u32x4 orow[16];                                                 // output tile of the previous chunk
-            auto issue_kt = [&](int64_t it, int stage) {
-                const int64_t ch = (boh + it) * H + h;
-                const uint32_t base = lds0 + stage * STG_BYTES;
-#pragma unroll
-                for (int j = 0; j < 16; ++j) copy_1k_to_lds(KTf + ch * (WS_KT * 2) + j * 1024, l16, base + STG_KT + j * 1024);
-            };
-            // one instruction stores 4 token rows of 256 bytes
             auto store_rows = [&](int64_t it) {
                 const int valid = (int)min((int64_t)CH, len - it * CH);
                 int64_t stride = (int64_t)HV * 128 * 4;                     // elements between rows 4 apart
@@ -207,22 +237,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                     dstp += stride;
                 }
             };
-            issue_kt(it0, 0);
-            wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                const int64_t it = it0 + i;
-                const int cur = (int)(i & 1);
-                issue_kt(min(it + 1, lastc), cur ^ 1);                      // that region was last read before B2 of the previous step
-                if constexpr (FULL) {
-                    if (i > 0) store_rows(it - 1);
-                    // k^T of this chunk was issued one step ago; newer than it are the stores of chunks
-                    // it-2 and it-1 (16 each, all rows of those chunks are valid) and the k^T just issued
-                    if (i >= 2) wait_vm_at_most<48>();
-                    else if (i == 1) wait_vm_at_most<32>();
-                } else {
-                    wait_vm_at_most<16>();
-                }
+                if constexpr (FULL) { if (i > 0) store_rows(it0 + i - 1); }
                 lds_barrier();                                              // B1
                 if constexpr (FULL) {
 #pragma unroll
@@ -231,19 +248,19 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 lds_barrier();                                              // B2 (waits for the tile reads)
             }
             if constexpr (FULL) store_rows(lastc);
-            wait_vm_at_most<0>();
         }
+        wait_vm_at_most<0>();                               // no copy may land in LDS after this workgroup has gone
         return;
     }
 
     // =====================================================================================
     // Compute waves
     // =====================================================================================
-    // ---- state: all key rows, value columns 16w .. 16w+15, C/D layout ----
+    // ---- state: all key rows (permuted, see above), value columns 16w .. 16w+15, C/D layout ----
     f32x4 S[8];
 #pragma unroll
     for (int m = 0; m < 8; ++m) {
-        const int kk = 16 * m + 4 * g, vc = 16 * w + c16;
+        const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * w + c16;
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
         if (init == 1) {
 #pragma unroll
@@ -255,18 +272,29 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         S[m] = s;
     }
 
-    // Lazy decay: registers hold S / Gamma, Gamma = 2^lg one scalar per workgroup (see the slab kernel).
+    // Lazy decay: the registers hold Shat = S / Gamma with one scalar Gamma = 2^lg per workgroup,
+    // so the decay of the whole state by 2^G_last per chunk costs nothing: products with S are
+    // rescaled by Gamma (folded into multiplies that exist anyway) and the update is divided by
+    // the new Gamma (folded into the decay factors of v_new).  When Gamma gets small the state
+    // is rescaled once and Gamma restarts at 1.  f16 operands have too little range for Shat, so
+    // there the state is rescaled on every chunk.
     constexpr float LG_MIN = std::is_same<T, bf16_t>::value ? -60.f : 1.f;
     float lg = 0.f;
 
+    // element offsets of this lane's LDS transpose reads (i = row within a 4-row run, j = column group)
+    const int tr_i = c16 >> 2, tr_j = c16 & 3;
+    const int v_tr = (((w >> 1) * 64 + (2 * (w & 1) + (tr_j >> 1)) * 16 + 4 * g + tr_i) * 8) + 4 * (tr_j & 1);     // + tt * 2048
+    const int k_tr = ((tr_j * 16 + 4 * g + tr_i) * 8);                                                             // + ((tt*4 + m/2)*64)*8 + 4*(m&1)
+
     V8 Vg[2];              // v_new decayed to the chunk end, B operand of the state update (first half -> second half)
     auto first_half = [&](const char* st) {
-        const V8* sW = (const V8*)(st + STG_W);
+        const V8* sK = (const V8*)(st + STG_K);
         const V8* sQ = (const V8*)(st + STG_Q);
+        const T* sV = (const T*)(st + STG_V);
+        const V8* sX = (const V8*)(st + STG_X);
         const V8* sP = (const V8*)(st + STG_P);
-        const V4* sU = (const V4*)(st + STG_U);
         const float* sTab = (const float*)(st + STG_TAB);
-        // (a) the state as B operand: pairs of key tiles (2s, 2s+1)
+        // (a) the state as B operand: pairs of key tiles (2s, 2s+1) = key features 32s + 8g + e
         V8 Sb[4];
 #pragma unroll
         for (int s = 0; s < 4; ++s)
@@ -276,43 +304,56 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 Sb[s][4 + r] = from_f32<T>(S[2 * s + 1][r]);
             }
         const float gamma = fast_exp2(lg);
-        const float lg_try = lg + sTab[128];
+        const float lg_try = lg + sTab[TAB_GLAST];
         const bool lazy = lg_try >= LG_MIN;
         const float vscale = lazy ? fast_exp2(-lg_try) : 1.f;
-        V8 Vn[2];
-        // two t-tiles at a time: w S -> v_new, and the output rows of those tiles
+        V8 Db[2], Vn[2];
+        // two t-tiles at a time
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            f32x4 av[2], ao[2];
+            f32x4 ks[2], ao[2];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
                 const int tt = 2 * hf + t2;
-                av[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
+                ks[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
                 ao[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
-                V8 aw[4], aq[4];
+                V8 ak[4], aq[4];
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-                    aw[s] = sW[(tt * 4 + s) * 64 + lane];
+                    ak[s] = sK[(tt * 4 + s) * 64 + lane];
                     if constexpr (FULL) aq[s] = sQ[(tt * 4 + s) * 64 + lane];
                 }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-                    av[t2] = Mma<T>::run(aw[s], Sb[s], av[t2]);
+                    ks[t2] = Mma<T>::run(ak[s], Sb[s], ks[t2]);
                     if constexpr (FULL) ao[t2] = Mma<T>::run(Sb[s], aq[s], ao[t2]);     // transposed tile
                 }
             }
-            // v_new = u - w S, plain (for the output) and decayed to the chunk end (for the state)
+            // D = v - 2^G (k S) for the token rows of these tiles
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
                 const int tt = 2 * hf + t2;
-                const f32x4 dec = *(const f32x4*)(sTab + 16 * tt + 4 * g) * vscale;
-                const V4 u4 = sU[(w * 4 + tt) * 64 + lane];
+                const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
+                const V4 v4 = Mma<T>::tr_read(sV + tt * 2048 + v_tr);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float uu = u_zero ? 0.f : to_f32(u4[r]);
-                    const float vn = uu - gamma * av[t2][r];
-                    Vn[hf][t2 * 4 + r] = from_f32<T>(vn);
-                    Vg[hf][t2 * 4 + r] = from_f32<T>(vn * dec[r]);
+                    const float vv = v_zero ? 0.f : to_f32(v4[r]);
+                    Db[hf][t2 * 4 + r] = from_f32<T>(vv - eg[r] * ks[t2][r]);
+                }
+            }
+            // v_new = Xb D (Xb is lower triangular: t-tile pairs up to this one), plain for the
+            // output and decayed to the chunk end for the state
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const int tt = 2 * hf + t2;
+                f32x4 vn = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int sp2 = 0; sp2 <= hf; ++sp2) vn = Mma<T>::run(sX[p_slot(tt, sp2) * 64 + lane], Db[sp2], vn);
+                const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    Vn[hf][t2 * 4 + r] = from_f32<T>(vn[r]);
+                    Vg[hf][t2 * 4 + r] = from_f32<T>(vn[r] * dec[r]);
                 }
             }
             // o^T = scale 2^G (q S)^T + (P v_new)^T; each lane holds 4 consecutive value columns of a token row
@@ -320,7 +361,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) {
                     const int tt = 2 * hf + t2;
-                    const float gam = sTab[64 + 16 * tt + c16] * gamma;
+                    const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
                     f32x4 acc = ao[t2] * gam;
 #pragma unroll
                     for (int sp2 = 0; sp2 <= hf; ++sp2) acc = Mma<T>::run(Vn[sp2], sP[p_slot(tt, sp2) * 64 + lane], acc);
@@ -338,13 +379,17 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         }
         lg = lazy ? lg_try : 0.f;
     };
-    // S += k^T (v_new decayed)
+    // S += k^T (v_new decayed): rows of tile m are key features 32*(m/2) + 8*(c16/4) + 4*(m%2) + c16%4
     auto second_half = [&](const char* st) {
-        const V8* sKT = (const V8*)(st + STG_KT);
+        const T* sK = (const T*)(st + STG_K);
 #pragma unroll
         for (int m = 0; m < 8; ++m)
 #pragma unroll
-            for (int sp2 = 0; sp2 < 2; ++sp2) S[m] = Mma<T>::run(sKT[(m * 2 + sp2) * 64 + lane], Vg[sp2], S[m]);
+            for (int sp2 = 0; sp2 < 2; ++sp2) {
+                const T* a = sK + (((2 * sp2) * 4 + (m >> 1)) * 64) * 8 + 4 * (m & 1) + k_tr;
+                const V8 kt = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * 64 * 8));
+                S[m] = Mma<T>::run(kt, Vg[sp2], S[m]);
+            }
     };
     if (nsteps > 0) {
         lds_barrier();                                          // B0: the copy waves have filled stage 0
@@ -361,7 +406,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const float gamma = fast_exp2(lg);
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
-            const int kk = 16 * m + 4 * g, vc = 16 * w + c16;
+            const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * w + c16;
             const f32x4 s = S[m] * gamma;
             if (dst_user && vfirst) *(f32x4*)(dst + vc * 128 + kk) = s;
             else {

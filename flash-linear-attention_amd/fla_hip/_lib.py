@@ -25,7 +25,6 @@ FLAG_NEG_EIGVAL = 1 << 2
 FLAG_STATE_V_FIRST = 1 << 3
 FLAG_BETA_VECTOR = 1 << 4
 FLAG_CU_INT32 = 1 << 5
-FLAG_SCAN_SLAB = 1 << 16
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
 

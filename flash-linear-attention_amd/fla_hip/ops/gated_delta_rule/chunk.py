@@ -28,8 +28,8 @@ from fla_hip.utils import input_guard
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
 # the chunk size (only rounding does), so chunk_size 16 and 32 are accepted and run with 64.
 _KERNEL_CHUNK = 64
-# FLA_HIP_SCAN_MODE=slab|wide|segments forces one form of the sequential kernel (default: automatic)
-_SCAN_MODE_FLAGS = {'slab': _lib.FLAG_SCAN_SLAB, 'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS}
+# FLA_HIP_SCAN_MODE=wide|segments forces one form of the sequential kernel (default: automatic)
+_SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS}
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 

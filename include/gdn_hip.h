@@ -43,7 +43,6 @@ extern "C" {
 #define GDN_FLAG_CU_INT32       (1u << 5)  /* cu_seqlens / chunk tables are int32, else int64   */
 /* gdn_chunk_fwd only: force one form of the sequential stage instead of the automatic choice
  * (all forms give the same result up to rounding; used by tests and for tuning)                */
-#define GDN_FLAG_SCAN_SLAB      (1u << 16) /* value columns of a head split over workgroups     */
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
 #define GDN_FLAG_SCAN_SEGMENTS  (1u << 18) /* time cut into segments (dense input, >= 8 chunks) */
 
