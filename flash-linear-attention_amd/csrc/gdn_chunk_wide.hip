@@ -7,12 +7,11 @@
 //   o     = scale 2^G (q S) + P v_new
 //   S     = 2^G_last S + k^T (v_new 2^(G_last-G))
 //
-// Twelve waves.  Eight compute waves: wave w owns value columns 16w .. 16w+15 for all key
-// rows.  Nothing of the recurrence crosses waves: bf16(S), bf16(D) and bf16(v_new) are the B
+// Eight waves.  Four compute waves, one per SIMD: wave w owns value columns 32w .. 32w+31 for all key
+// rows, so every operand fragment read from LDS feeds two matrix instructions.  Nothing of the recurrence crosses waves: bf16(S), bf16(D) and bf16(v_new) are the B
 // operands of this wave's own next products (same lanes, C/D layout == operand layout), so
-// the dependent chain runs in registers.  Two compute waves per SIMD let one wave's vector-ALU
-// work overlap the other's matrix instructions.  The compute waves issue no global memory
-// instruction inside the loop.
+// the dependent chain runs in registers.  The compute waves issue no global memory instruction
+// inside the loop.
 // Four copy waves move everything else.  Three of them fill a double-buffered LDS stage with
 // asynchronous global->LDS loads that use no registers: the prepare record verbatim, and the
 // q, k, v tiles gathered straight from the user's tensors in 16-byte pieces, placed so that
@@ -43,7 +42,8 @@ constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 62 464
 constexpr int OT_PITCH = 272;                     // bytes per token row of the output tile (256 B + pad: conflict-free 8-byte writes)
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
 constexpr size_t WIDE_SMEM = 2 * STG_BYTES + OT_BYTES;       // 142 336 B: one workgroup per CU
-constexpr int CW = 8;                             // compute waves
+constexpr int WIDE_NN = 2;                        // 16-column tiles per compute wave
+constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
 
 // kind of run
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         auto gather_tile = [&](const T* tensor, int heads, int head, int64_t it, int tt, uint32_t lds_tile) {
             const int64_t tok0 = bos + it * CH;
             const int valid = (int)min((int64_t)CH, len - it * CH);
-            const int row = min(16 * tt + c16, valid - 1);
+            const int row = min(16 * tt + ((c16 - 4 * g) & 15), valid - 1);      // this lane's slot holds that row's piece
             const uint32_t voff = (uint32_t)row * (uint32_t)(heads * 256) + 16 * g;
             const char* base = (const char*)(tensor + (tok0 * heads + head) * 128);
 #pragma unroll
@@ -257,10 +257,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // Compute waves
     // =====================================================================================
     // ---- state: all key rows (permuted, see above), value columns 16w .. 16w+15, C/D layout ----
-    f32x4 S[8];
+    constexpr int NN = WIDE_NN;
+    f32x4 S[8][NN];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-        const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * w + c16;
+    for (int m = 0; m < 8; ++m)
+#pragma unroll
+    for (int nn = 0; nn < NN; ++nn) {
+        const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * (NN * w + nn) + c16;
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
         if (init == 1) {
 #pragma unroll
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             if (src_user && vfirst) s = *(const f32x4*)(src + vc * 128 + kk);
             else s = f32x4{src[kk * 128 + vc], src[(kk + 1) * 128 + vc], src[(kk + 2) * 128 + vc], src[(kk + 3) * 128 + vc]};
         }
-        S[m] = s;
+        S[m][nn] = s;
     }
 
     // Lazy decay: the registers hold Shat = S / Gamma with one scalar Gamma = 2^lg per workgroup,
@@ -281,12 +284,20 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     constexpr float LG_MIN = std::is_same<T, bf16_t>::value ? -60.f : 1.f;
     float lg = 0.f;
 
-    // element offsets of this lane's LDS transpose reads (i = row within a 4-row run, j = column group)
+    // element offsets of this lane's LDS reads.  A transpose read hands lane 4j+e element e of the
+    // four 4-element runs addressed by lanes j, j+4, j+8, j+12 of its 16-lane group: this lane
+    // addresses row i = c16/4 of the 4-row run and column group j = c16%4.
     const int tr_i = c16 >> 2, tr_j = c16 & 3;
-    const int v_tr = (((w >> 1) * 64 + (2 * (w & 1) + (tr_j >> 1)) * 16 + 4 * g + tr_i) * 8) + 4 * (tr_j & 1);     // + tt * 2048
-    const int k_tr = ((tr_j * 16 + 4 * g + tr_i) * 8);                                                             // + ((tt*4 + m/2)*64)*8 + 4*(m&1)
+    const int a_slot = 16 * g + ((c16 + 4 * g) & 15);                             // operand piece (g, c16) of a block
+    const int k_tr = (16 * tr_j + ((4 * g + tr_i + 4 * tr_j) & 15)) * 8;          // piece (g_p = j, row 4g+i); + block, + 4*(m&1)
+    int v_tr[NN];                                                                 // piece (s, g_p) = column group of tile nn, row 4g+i
+#pragma unroll
+    for (int nn = 0; nn < NN; ++nn) {
+        const int cgrp = 2 * (NN * w + nn) + (tr_j >> 1), gp = cgrp & 3;
+        v_tr[nn] = ((cgrp >> 2) * 64 + 16 * gp + ((4 * g + tr_i + 4 * gp) & 15)) * 8 + 4 * (tr_j & 1);     // + tt * 2048
+    }
 
-    V8 Vg[2];              // v_new decayed to the chunk end, B operand of the state update (first half -> second half)
+    V8 Vg[2][NN];          // v_new decayed to the chunk end, B operand of the state update (first half -> second half)
     auto first_half = [&](const char* st) {
         const V8* sK = (const V8*)(st + STG_K);
         const V8* sQ = (const V8*)(st + STG_Q);
@@ -295,50 +306,60 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const V8* sP = (const V8*)(st + STG_P);
         const float* sTab = (const float*)(st + STG_TAB);
         // (a) the state as B operand: pairs of key tiles (2s, 2s+1) = key features 32s + 8g + e
-        V8 Sb[4];
+        V8 Sb[4][NN];
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                Sb[s][r] = from_f32<T>(S[2 * s][r]);
-                Sb[s][4 + r] = from_f32<T>(S[2 * s + 1][r]);
-            }
+            for (int nn = 0; nn < NN; ++nn)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    Sb[s][nn][r] = from_f32<T>(S[2 * s][nn][r]);
+                    Sb[s][nn][4 + r] = from_f32<T>(S[2 * s + 1][nn][r]);
+                }
         const float gamma = fast_exp2(lg);
         const float lg_try = lg + sTab[TAB_GLAST];
         const bool lazy = lg_try >= LG_MIN;
         const float vscale = lazy ? fast_exp2(-lg_try) : 1.f;
-        V8 Db[2], Vn[2];
+        V8 Db[2][NN], Vn[2][NN];
         // two t-tiles at a time
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            f32x4 ks[2], ao[2];
+            f32x4 ks[2][NN], ao[2][NN];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
                 const int tt = 2 * hf + t2;
-                ks[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
-                ao[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
                 V8 ak[4], aq[4];
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-                    ak[s] = sK[(tt * 4 + s) * 64 + lane];
-                    if constexpr (FULL) aq[s] = sQ[(tt * 4 + s) * 64 + lane];
+                    ak[s] = sK[(tt * 4 + s) * 64 + a_slot];
+                    if constexpr (FULL) aq[s] = sQ[(tt * 4 + s) * 64 + a_slot];
                 }
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    ks[t2] = Mma<T>::run(ak[s], Sb[s], ks[t2]);
-                    if constexpr (FULL) ao[t2] = Mma<T>::run(Sb[s], aq[s], ao[t2]);     // transposed tile
+                for (int nn = 0; nn < NN; ++nn) {
+                    ks[t2][nn] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    ao[t2][nn] = f32x4{0.f, 0.f, 0.f, 0.f};
                 }
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int nn = 0; nn < NN; ++nn) {
+                        ks[t2][nn] = Mma<T>::run(ak[s], Sb[s][nn], ks[t2][nn]);
+                        if constexpr (FULL) ao[t2][nn] = Mma<T>::run(Sb[s][nn], aq[s], ao[t2][nn]);     // transposed tile
+                    }
             }
             // D = v - 2^G (k S) for the token rows of these tiles
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
                 const int tt = 2 * hf + t2;
                 const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
-                const V4 v4 = Mma<T>::tr_read(sV + tt * 2048 + v_tr);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float vv = v_zero ? 0.f : to_f32(v4[r]);
-                    Db[hf][t2 * 4 + r] = from_f32<T>(vv - eg[r] * ks[t2][r]);
+                for (int nn = 0; nn < NN; ++nn) {
+                    const V4 v4 = Mma<T>::tr_read(sV + tt * 2048 + v_tr[nn]);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float vv = v_zero ? 0.f : to_f32(v4[r]);
+                        Db[hf][nn][t2 * 4 + r] = from_f32<T>(vv - eg[r] * ks[t2][nn][r]);
+                    }
                 }
             }
             // v_new = Xb D (Xb is lower triangular: t-tile pairs up to this one), plain for the
@@ -346,14 +367,20 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
                 const int tt = 2 * hf + t2;
-                f32x4 vn = {0.f, 0.f, 0.f, 0.f};
+                V8 ax[2];
 #pragma unroll
-                for (int sp2 = 0; sp2 <= hf; ++sp2) vn = Mma<T>::run(sX[p_slot(tt, sp2) * 64 + lane], Db[sp2], vn);
+                for (int sp2 = 0; sp2 <= hf; ++sp2) ax[sp2] = sX[p_slot(tt, sp2) * 64 + lane];
                 const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    Vn[hf][t2 * 4 + r] = from_f32<T>(vn[r]);
-                    Vg[hf][t2 * 4 + r] = from_f32<T>(vn[r] * dec[r]);
+                for (int nn = 0; nn < NN; ++nn) {
+                    f32x4 vn = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int sp2 = 0; sp2 <= hf; ++sp2) vn = Mma<T>::run(ax[sp2], Db[sp2][nn], vn);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        Vn[hf][nn][t2 * 4 + r] = from_f32<T>(vn[r]);
+                        Vg[hf][nn][t2 * 4 + r] = from_f32<T>(vn[r] * dec[r]);
+                    }
                 }
             }
             // o^T = scale 2^G (q S)^T + (P v_new)^T; each lane holds 4 consecutive value columns of a token row
@@ -362,20 +389,28 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 for (int t2 = 0; t2 < 2; ++t2) {
                     const int tt = 2 * hf + t2;
                     const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
-                    f32x4 acc = ao[t2] * gam;
+                    V8 ap[2];
 #pragma unroll
-                    for (int sp2 = 0; sp2 <= hf; ++sp2) acc = Mma<T>::run(Vn[sp2], sP[p_slot(tt, sp2) * 64 + lane], acc);
-                    V4 o4;
+                    for (int sp2 = 0; sp2 <= hf; ++sp2) ap[sp2] = sP[p_slot(tt, sp2) * 64 + lane];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
-                    *(V4*)(otile + (16 * tt + c16) * OT_PITCH + (16 * w + 4 * g) * 2) = o4;
+                    for (int nn = 0; nn < NN; ++nn) {
+                        f32x4 acc = ao[t2][nn] * gam;
+#pragma unroll
+                        for (int sp2 = 0; sp2 <= hf; ++sp2) acc = Mma<T>::run(Vn[sp2][nn], ap[sp2], acc);
+                        V4 o4;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
+                        *(V4*)(otile + (16 * tt + c16) * OT_PITCH + (16 * (NN * w + nn) + 4 * g) * 2) = o4;
+                    }
                 }
             }
         }
         if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {       // scalar branch: rare, must not be if-converted
             const float fold = fast_exp2(lg_try);
 #pragma unroll
-            for (int m = 0; m < 8; ++m) S[m] *= fold;
+            for (int m = 0; m < 8; ++m)
+#pragma unroll
+                for (int nn = 0; nn < NN; ++nn) S[m][nn] *= fold;
         }
         lg = lazy ? lg_try : 0.f;
     };
@@ -388,7 +423,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             for (int sp2 = 0; sp2 < 2; ++sp2) {
                 const T* a = sK + (((2 * sp2) * 4 + (m >> 1)) * 64) * 8 + 4 * (m & 1) + k_tr;
                 const V8 kt = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * 64 * 8));
-                S[m] = Mma<T>::run(kt, Vg[sp2], S[m]);
+#pragma unroll
+                for (int nn = 0; nn < NN; ++nn) S[m][nn] = Mma<T>::run(kt, Vg[sp2][nn], S[m][nn]);
             }
     };
     if (nsteps > 0) {
@@ -405,9 +441,11 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (dst) {
         const float gamma = fast_exp2(lg);
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * w + c16;
-            const f32x4 s = S[m] * gamma;
+        for (int m = 0; m < 8; ++m)
+#pragma unroll
+        for (int nn = 0; nn < NN; ++nn) {
+            const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * (NN * w + nn) + c16;
+            const f32x4 s = S[m][nn] * gamma;
             if (dst_user && vfirst) *(f32x4*)(dst + vc * 128 + kk) = s;
             else {
 #pragma unroll
