@@ -297,16 +297,107 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         v_tr[nn] = ((cgrp >> 2) * 64 + 16 * gp + ((4 * g + tr_i + 4 * gp) & 15)) * 8 + 4 * (tr_j & 1);     // + tt * 2048
     }
 
-    V8 Vg[2][NN];          // v_new decayed to the chunk end, B operand of the state update (first half -> second half)
-    auto first_half = [&](const char* st) {
+    // One step, written as a fixed sequence of small scheduling regions (the compiler may reorder
+    // inside a region, not across `fence`).  A lone wave per SIMD has nobody to hide LDS latency
+    // behind, so every LDS read is issued two or more regions before its first use (a rolling
+    // window of three operand fragments), and the thin, dependent part of a step (D -> v_new ->
+    // output of a pair of t-tiles) is cut into pieces that each share a region with four
+    // independent matrix instructions (products of the next tiles, or the state update).
+    auto step = [&](const char* st) {
         const V8* sK = (const V8*)(st + STG_K);
         const V8* sQ = (const V8*)(st + STG_Q);
         const T* sV = (const T*)(st + STG_V);
+        const T* sKt = (const T*)(st + STG_K);
         const V8* sX = (const V8*)(st + STG_X);
         const V8* sP = (const V8*)(st + STG_P);
         const float* sTab = (const float*)(st + STG_TAB);
-        // (a) the state as B operand: pairs of key tiles (2s, 2s+1) = key features 32s + 8g + e
+        auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+
+        // fragment f = (t-tile f/4, key tiles (2s, 2s+1) with s = f%4) of k and q, ring of three
+        V8 ak[3], aq[3];
+        auto F = [&](int f) {
+            ak[f % 3] = sK[f * 64 + a_slot];
+            if constexpr (FULL) aq[f % 3] = sQ[f * 64 + a_slot];
+        };
+        f32x4 ks[4][NN], ao[4][NN];
         V8 Sb[4][NN];
+        auto M = [&](int f) {                   // (k S) and (q S)^T contributions of fragment f
+            const int tt = f >> 2, sx = f & 3;
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn) {
+                ks[tt][nn] = Mma<T>::run(ak[f % 3], Sb[sx][nn], sx ? ks[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
+                if constexpr (FULL) ao[tt][nn] = Mma<T>::run(Sb[sx][nn], aq[f % 3], sx ? ao[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
+            }
+        };
+        V4 vv[4][NN];                           // v in C/D layout, per t-tile
+        V8 ax[4][2], ap[4][2];                  // Xb and P fragments [t-tile][column pair]
+        auto FV = [&](int tt) {
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn) vv[tt][nn] = Mma<T>::tr_read(sV + tt * 2048 + v_tr[nn]);
+        };
+        auto FX = [&](int tt) {
+#pragma unroll
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = sX[p_slot(tt, sp2) * 64 + lane];
+        };
+        auto FP = [&](int tt) {
+            if constexpr (FULL) {
+#pragma unroll
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = sP[p_slot(tt, sp2) * 64 + lane];
+            }
+        };
+        V8 kt[2][8];                            // k^T rows of key tile m over t-tile pair sp2
+        auto FK = [&](int sp2, int m) {
+            const T* a = sKt + (((2 * sp2) * 4 + (m >> 1)) * 64) * 8 + 4 * (m & 1) + k_tr;
+            kt[sp2][m] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * 64 * 8));
+        };
+        float gamma, vscale;
+        V8 Db[2][NN], Vn[2][NN], Vg[2][NN];
+        auto TD = [&](int tt) {                 // D = v - 2^G (k S), rows of t-tile tt
+            const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float x = v_zero ? 0.f : to_f32(vv[tt][nn][r]);
+                    Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(x - eg[r] * ks[tt][nn][r]);
+                }
+        };
+        auto TX = [&](int tt) {                 // v_new = Xb D (lower triangular), plain and decayed to the chunk end
+            const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn) {
+                f32x4 vn = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) vn = Mma<T>::run(ax[tt][sp2], Db[sp2][nn], vn);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    Vn[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[r]);
+                    Vg[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[r] * dec[r]);
+                }
+            }
+        };
+        auto TP = [&](int tt) {                 // o^T = scale 2^G (q S)^T + (P v_new)^T: 4 consecutive value columns of a token row per lane
+            if constexpr (FULL) {
+                const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
+#pragma unroll
+                for (int nn = 0; nn < NN; ++nn) {
+                    f32x4 acc = ao[tt][nn] * gam;
+#pragma unroll
+                    for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) acc = Mma<T>::run(Vn[sp2][nn], ap[tt][sp2], acc);
+                    V4 o4;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
+                    *(V4*)(otile + (16 * tt + c16) * OT_PITCH + (16 * (NN * w + nn) + 4 * g) * 2) = o4;
+                }
+            }
+        };
+        auto U = [&](int sp2, int m) {          // S += k^T (v_new decayed): key tile m, t-tile pair sp2
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn) S[m][nn] = Mma<T>::run(kt[sp2][m], Vg[sp2][nn], S[m][nn]);
+        };
+
+        // ---- the state as B operand (pairs of key tiles (2s, 2s+1) = key features 32s + 8g + e) ----
+        F(0); F(1);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -316,96 +407,31 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                     Sb[s][nn][r] = from_f32<T>(S[2 * s][nn][r]);
                     Sb[s][nn][4 + r] = from_f32<T>(S[2 * s + 1][nn][r]);
                 }
-        const float gamma = fast_exp2(lg);
+        gamma = fast_exp2(lg);
         const float lg_try = lg + sTab[TAB_GLAST];
         const bool lazy = lg_try >= LG_MIN;
-        const float vscale = lazy ? fast_exp2(-lg_try) : 1.f;
-        V8 Db[2][NN], Vn[2][NN];
-        // two t-tiles at a time
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            f32x4 ks[2][NN], ao[2][NN];
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int tt = 2 * hf + t2;
-                V8 ak[4], aq[4];
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    ak[s] = sK[(tt * 4 + s) * 64 + a_slot];
-                    if constexpr (FULL) aq[s] = sQ[(tt * 4 + s) * 64 + a_slot];
-                }
-#pragma unroll
-                for (int nn = 0; nn < NN; ++nn) {
-                    ks[t2][nn] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    ao[t2][nn] = f32x4{0.f, 0.f, 0.f, 0.f};
-                }
-#pragma unroll
-                for (int s = 0; s < 4; ++s)
-#pragma unroll
-                    for (int nn = 0; nn < NN; ++nn) {
-                        ks[t2][nn] = Mma<T>::run(ak[s], Sb[s][nn], ks[t2][nn]);
-                        if constexpr (FULL) ao[t2][nn] = Mma<T>::run(Sb[s][nn], aq[s], ao[t2][nn]);     // transposed tile
-                    }
-            }
-            // D = v - 2^G (k S) for the token rows of these tiles
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int tt = 2 * hf + t2;
-                const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
-#pragma unroll
-                for (int nn = 0; nn < NN; ++nn) {
-                    const V4 v4 = Mma<T>::tr_read(sV + tt * 2048 + v_tr[nn]);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float vv = v_zero ? 0.f : to_f32(v4[r]);
-                        Db[hf][nn][t2 * 4 + r] = from_f32<T>(vv - eg[r] * ks[t2][nn][r]);
-                    }
-                }
-            }
-            // v_new = Xb D (Xb is lower triangular: t-tile pairs up to this one), plain for the
-            // output and decayed to the chunk end for the state
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int tt = 2 * hf + t2;
-                V8 ax[2];
-#pragma unroll
-                for (int sp2 = 0; sp2 <= hf; ++sp2) ax[sp2] = sX[p_slot(tt, sp2) * 64 + lane];
-                const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
-#pragma unroll
-                for (int nn = 0; nn < NN; ++nn) {
-                    f32x4 vn = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int sp2 = 0; sp2 <= hf; ++sp2) vn = Mma<T>::run(ax[sp2], Db[sp2][nn], vn);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        Vn[hf][nn][t2 * 4 + r] = from_f32<T>(vn[r]);
-                        Vg[hf][nn][t2 * 4 + r] = from_f32<T>(vn[r] * dec[r]);
-                    }
-                }
-            }
-            // o^T = scale 2^G (q S)^T + (P v_new)^T; each lane holds 4 consecutive value columns of a token row
-            if constexpr (FULL) {
-#pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2) {
-                    const int tt = 2 * hf + t2;
-                    const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
-                    V8 ap[2];
-#pragma unroll
-                    for (int sp2 = 0; sp2 <= hf; ++sp2) ap[sp2] = sP[p_slot(tt, sp2) * 64 + lane];
-#pragma unroll
-                    for (int nn = 0; nn < NN; ++nn) {
-                        f32x4 acc = ao[t2][nn] * gam;
-#pragma unroll
-                        for (int sp2 = 0; sp2 <= hf; ++sp2) acc = Mma<T>::run(Vn[sp2][nn], ap[sp2], acc);
-                        V4 o4;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
-                        *(V4*)(otile + (16 * tt + c16) * OT_PITCH + (16 * (NN * w + nn) + 4 * g) * 2) = o4;
-                    }
-                }
-            }
-        }
-        if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {       // scalar branch: rare, must not be if-converted
+        vscale = lazy ? fast_exp2(-lg_try) : 1.f;
+        fence();
+        // ---- t-tiles 0, 1 ----
+        F(2); M(0); fence();
+        F(3); M(1); fence();
+        F(4); M(2); fence();
+        F(5); M(3); fence();
+        F(6); M(4); FV(0); fence();
+        F(7); M(5); FV(1); fence();
+        F(8); M(6); FX(0); fence();
+        F(9); M(7); FX(1); fence();
+        // ---- t-tiles 2, 3, with the tail of tiles 0, 1 ----
+        F(10); M(8); TD(0); fence();
+        F(11); M(9); TD(1); FP(0); fence();
+        F(12); M(10); TX(0); FP(1); fence();
+        F(13); M(11); TX(1); FV(2); fence();
+        F(14); M(12); TP(0); FV(3); fence();
+        F(15); M(13); TP(1); FX(2); fence();
+        M(14); FX(3); FK(0, 0); FK(0, 1); fence();
+        M(15); FK(0, 2); FK(0, 3); fence();
+        // the decay fold: rare, a scalar branch so that it is not if-converted into the common path
+        if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
             const float fold = fast_exp2(lg_try);
 #pragma unroll
             for (int m = 0; m < 8; ++m)
@@ -413,28 +439,24 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 for (int nn = 0; nn < NN; ++nn) S[m][nn] *= fold;
         }
         lg = lazy ? lg_try : 0.f;
-    };
-    // S += k^T (v_new decayed): rows of tile m are key features 32*(m/2) + 8*(c16/4) + 4*(m%2) + c16%4
-    auto second_half = [&](const char* st) {
-        const T* sK = (const T*)(st + STG_K);
+        // ---- state update from tiles 0, 1, with the tail of tiles 2, 3 ----
+        U(0, 0); U(0, 1); TD(2); FK(0, 4); FK(0, 5); fence();
+        U(0, 2); U(0, 3); TD(3); FK(0, 6); FK(0, 7); FP(2); fence();
+        U(0, 4); U(0, 5); TX(2); FK(1, 0); FK(1, 1); FP(3); fence();
+        U(0, 6); U(0, 7); TX(3); FK(1, 2); FK(1, 3); fence();
+        TP(2); FK(1, 4); FK(1, 5); fence();
+        TP(3); FK(1, 6); FK(1, 7); fence();
+        lds_barrier();                                          // B1: q, v, record of this stage are free
+        // ---- state update from tiles 2, 3 ----
 #pragma unroll
-        for (int m = 0; m < 8; ++m)
-#pragma unroll
-            for (int sp2 = 0; sp2 < 2; ++sp2) {
-                const T* a = sK + (((2 * sp2) * 4 + (m >> 1)) * 64) * 8 + 4 * (m & 1) + k_tr;
-                const V8 kt = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * 64 * 8));
-#pragma unroll
-                for (int nn = 0; nn < NN; ++nn) S[m][nn] = Mma<T>::run(kt, Vg[sp2][nn], S[m][nn]);
-            }
+        for (int m = 0; m < 8; ++m) U(1, m);
+        fence();
+        lds_barrier();                                          // B2: k of this stage is free, the other stage is complete
     };
     if (nsteps > 0) {
         lds_barrier();                                          // B0: the copy waves have filled stage 0
         for (int64_t i = 0; i < nsteps; ++i) {
-            const char* st = smem + (i & 1) * STG_BYTES;
-            first_half(st);
-            lds_barrier();                                      // B1
-            second_half(st);
-            lds_barrier();                                      // B2
+            step(smem + (i & 1) * STG_BYTES);
         }
     }
 
