@@ -34,8 +34,11 @@
 
 namespace gdn {
 
-// LDS stage of one chunk.  q, k, v: [4 tt][4 s][64 lanes][16 B], piece (tt, s, 16g+c16) = bytes
-// [64s+16g, +16) of token row 16tt+c16.
+// LDS stage of one chunk.  q, k, v tiles: 64 token rows x 256 B as 16 blocks of 4 rows (1 KB, one
+// asynchronous copy each: 4 whole rows is the access shape the memory pipeline moves fastest).
+// Inside block j the 16-byte piece c of row 4j + r sits in slot 16*(c/4) + ((4*(j%4) + r + 4*(c%4)) & 15):
+// the rotation makes both the 16-byte operand reads (16 rows x one piece) and the LDS transpose
+// reads (4 rows x 4 pieces) of a 16-lane group touch 16 different slots modulo 16, i.e. all banks.
 constexpr int STG_K = 0, STG_Q = 16384, STG_V = 32768, STG_REC = 49152;
 constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB;
 constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 62 464
@@ -147,17 +150,21 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (w >= CW) {
         if (nsteps <= 0) return;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-        // Row gather: the four 1-KB pieces (s = 0..3) of t-tile tt of a [token][head][128] tensor.
-        // Rows past the end of the sequence re-read its last row: whatever they hold is finite and
-        // is multiplied by the zero columns of Xb, the zero rows of v_new and the causal zeros of P.
-        auto gather_tile = [&](const T* tensor, int heads, int head, int64_t it, int tt, uint32_t lds_tile) {
+        // Block gather: rows 4j .. 4j+3 of a [token][head][128] tensor.  Rows past the end of the
+        // sequence re-read its last row: whatever they hold is finite and is multiplied by the zero
+        // columns of Xb, the zero rows of v_new and the causal zeros of P.
+        auto gather_blocks = [&](const T* tensor, int heads, int head, int64_t it, int j0, int j1, uint32_t lds_tile) {
             const int64_t tok0 = bos + it * CH;
             const int valid = (int)min((int64_t)CH, len - it * CH);
-            const int row = min(16 * tt + ((c16 - 4 * g) & 15), valid - 1);      // this lane's slot holds that row's piece
-            const uint32_t voff = (uint32_t)row * (uint32_t)(heads * 256) + 16 * g;
             const char* base = (const char*)(tensor + (tok0 * heads + head) * 128);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) gather_1k_to_lds(base + 64 * s, voff, lds_tile + (tt * 4 + s) * 1024);
+            for (int j = 0; j < 16; ++j) {
+                if (j < j0 || j >= j1) continue;
+                const int x = (c16 - 4 * (j & 3)) & 15;                     // this lane's slot holds piece c of row 4j + r
+                const int r = x & 3, c = 4 * g + (x >> 2);
+                const int row = min(4 * j + r, valid - 1);
+                gather_1k_to_lds(base, (uint32_t)row * (uint32_t)(heads * 256) + 16 * c, lds_tile + j * 1024);
+            }
         };
         auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage) {
             const char* rec = p.ws.Rec + ((boh + it) * HV + hv) * REC_BYTES;
@@ -168,8 +175,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         if (w == CW) {
             // ---- k: issued at the start of a step for the next chunk, awaited at its end ----
             auto issue_k = [&](int64_t it, int stage) {
-#pragma unroll
-                for (int tt = 0; tt < 4; ++tt) gather_tile((const T*)p.k, H, h, it, tt, lds0 + stage * STG_BYTES + STG_K);
+                gather_blocks((const T*)p.k, H, h, it, 0, 16, lds0 + stage * STG_BYTES + STG_K);
             };
             issue_k(it0, 0);
             wait_vm_at_most<0>();
@@ -190,15 +196,15 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 if (qside) {
                     if constexpr (FULL) {
                         // 16 q pieces, then Xb (6) and the tables (1)
-                        if (early) { gather_tile((const T*)p.q, H, h, it, 0, st + STG_Q); gather_tile((const T*)p.q, H, h, it, 1, st + STG_Q); }
-                        else { gather_tile((const T*)p.q, H, h, it, 2, st + STG_Q); gather_tile((const T*)p.q, H, h, it, 3, st + STG_Q); copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }
+                        if (early) gather_blocks((const T*)p.q, H, h, it, 0, 8, st + STG_Q);
+                        else { gather_blocks((const T*)p.q, H, h, it, 8, 16, st + STG_Q); copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }
                     } else {
                         if (early) { copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }      // all 7 pieces
                     }
                 } else {
-                    if (early) { gather_tile((const T*)p.v, HV, hv, it, 0, st + STG_V); gather_tile((const T*)p.v, HV, hv, it, 1, st + STG_V); }
+                    if (early) gather_blocks((const T*)p.v, HV, hv, it, 0, 8, st + STG_V);
                     else {
-                        gather_tile((const T*)p.v, HV, hv, it, 2, st + STG_V); gather_tile((const T*)p.v, HV, hv, it, 3, st + STG_V);
+                        gather_blocks((const T*)p.v, HV, hv, it, 8, 16, st + STG_V);
                         if constexpr (FULL) copy_rec(it, 6, 12, st);
                     }
                 }
@@ -288,13 +294,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // four 4-element runs addressed by lanes j, j+4, j+8, j+12 of its 16-lane group: this lane
     // addresses row i = c16/4 of the 4-row run and column group j = c16%4.
     const int tr_i = c16 >> 2, tr_j = c16 & 3;
-    const int a_slot = 16 * g + ((c16 + 4 * g) & 15);                             // operand piece (g, c16) of a block
-    const int k_tr = (16 * tr_j + ((4 * g + tr_i + 4 * tr_j) & 15)) * 8;          // piece (g_p = j, row 4g+i); + block, + 4*(m&1)
-    int v_tr[NN];                                                                 // piece (s, g_p) = column group of tile nn, row 4g+i
+    const int a_off = (c16 >> 2) * 64 + ((c16 + 4 * g) & 15);                    // operand piece of row c16 of a t-tile: + tt*256 + 16*s  (16-byte units)
+    const int k_tr = (g * 64 + ((4 * g + tr_i + 4 * tr_j) & 15)) * 8;            // row 4g+i of a 16-row group, piece 4*(m/2) + j: + (32*sp2 + 16*half)*128 + 128*(m/2) + 4*(m&1)  (elements)
+    int v_tr[NN];                                                                 // row 4g+i, piece = 8-column group of tile nn: + tt*2048
 #pragma unroll
     for (int nn = 0; nn < NN; ++nn) {
-        const int cgrp = 2 * (NN * w + nn) + (tr_j >> 1), gp = cgrp & 3;
-        v_tr[nn] = ((cgrp >> 2) * 64 + 16 * gp + ((4 * g + tr_i + 4 * gp) & 15)) * 8 + 4 * (tr_j & 1);     // + tt * 2048
+        const int c = 2 * (NN * w + nn) + (tr_j >> 1);
+        v_tr[nn] = (g * 64 + 16 * (c >> 2) + ((4 * g + tr_i + 4 * (c & 3)) & 15)) * 8 + 4 * (tr_j & 1);
     }
 
     // One step, written as a fixed sequence of small scheduling regions (the compiler may reorder
@@ -316,8 +322,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         // fragment f = (t-tile f/4, key tiles (2s, 2s+1) with s = f%4) of k and q, ring of three
         V8 ak[3], aq[3];
         auto F = [&](int f) {
-            ak[f % 3] = sK[f * 64 + a_slot];
-            if constexpr (FULL) aq[f % 3] = sQ[f * 64 + a_slot];
+            ak[f % 3] = sK[(f >> 2) * 256 + 16 * (f & 3) + a_off];
+            if constexpr (FULL) aq[f % 3] = sQ[(f >> 2) * 256 + 16 * (f & 3) + a_off];
         };
         f32x4 ks[4][NN], ao[4][NN];
         V8 Sb[4][NN];
@@ -347,8 +353,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         };
         V8 kt[2][8];                            // k^T rows of key tile m over t-tile pair sp2
         auto FK = [&](int sp2, int m) {
-            const T* a = sKt + (((2 * sp2) * 4 + (m >> 1)) * 64) * 8 + 4 * (m & 1) + k_tr;
-            kt[sp2][m] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 4 * 64 * 8));
+            const T* a = sKt + sp2 * 4096 + 128 * (m >> 1) + 4 * (m & 1) + k_tr;
+            kt[sp2][m] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 2048));
         };
         float gamma, vscale;
         V8 Db[2][NN], Vn[2][NN], Vg[2][NN];
