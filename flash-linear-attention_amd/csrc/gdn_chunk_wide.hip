@@ -497,6 +497,17 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp) 
     const int64_t inh = blockIdx.x >> 3;
     const int v0 = (int)(blockIdx.x & 7) * 16;
     const int nseg = sp.nseg;
+    // the next transition matrix travels in registers while the current one is multiplied
+    f32x4 pre[16];
+    auto fetch_M = [&](int j) {
+        const float* M = sp.mseg + (inh * nseg + j) * 16384;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int idx = tid + 256 * i;
+            pre[i] = *(const f32x4*)(M + (idx >> 5) * 128 + (idx & 31) * 4);
+        }
+    };
+    if (nseg > 2) fetch_M(1);
     // S_in[1] = S_loc,0
     for (int idx = tid; idx < 128 * 16; idx += 256) {
         const int kk = idx >> 4, c = idx & 15;
@@ -505,23 +516,35 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp) 
         sp.sin[(inh * nseg + 1) * 16384 + kk * 128 + v0 + c] = x;
     }
     for (int j = 1; j + 1 < nseg; ++j) {
-        const float* M = sp.mseg + (inh * nseg + j) * 16384;
         __syncthreads();                            // previous readers of sM are done; sS is complete
-        for (int idx = tid; idx < 128 * 32; idx += 256) {
-            const int row = idx >> 5, c4 = (idx & 31) * 4;
-            *(f32x4*)(sM + row * MP + c4) = *(const f32x4*)(M + row * 128 + c4);
-        }
-        __syncthreads();
-        f32x4 acc[2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) acc[i] = mm16_f32(sM + (16 * (2 * w + i)) * MP, MP, sS, 16, 32, c16, g);
+        for (int i = 0; i < 16; ++i) {
+            const int idx = tid + 256 * i;
+            *(f32x4*)(sM + (idx >> 5) * MP + (idx & 31) * 4) = pre[i];
+        }
+        if (j + 2 < nseg) fetch_M(j + 1);
+        // this wave's rows of S_loc,j (C/D layout of key tiles 2w, 2w+1)
+        float sl[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                sl[i][r] = sp.sloc[(inh * nseg + j) * 16384 + (16 * (2 * w + i) + 4 * g + r) * 128 + v0 + c16];
+        __syncthreads();
+        // two independent accumulation chains per tile (halves of the contraction)
+        f32x4 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+                acc[i][hh] = mm16_f32(sM + (16 * (2 * w + i)) * MP + 64 * hh, MP, sS + 64 * hh * 16, 16, 16, c16, g);
         __syncthreads();                            // all waves have read sS
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int kk = 16 * (2 * w + i) + 4 * g + r;
-                const float x = acc[i][r] + sp.sloc[(inh * nseg + j) * 16384 + kk * 128 + v0 + c16];
+                const float x = acc[i][0][r] + acc[i][1][r] + sl[i][r];
                 sS[kk * 16 + c16] = x;
                 sp.sin[(inh * nseg + j + 1) * 16384 + kk * 128 + v0 + c16] = x;
             }
