@@ -39,12 +39,15 @@ namespace gdn {
 // Inside block j the 16-byte piece c of row 4j + r sits in slot 16*(c/4) + ((4*(j%4) + r + 4*(c%4)) & 15):
 // the rotation makes both the 16-byte operand reads (16 rows x one piece) and the LDS transpose
 // reads (4 rows x 4 pieces) of a 16-lane group touch 16 different slots modulo 16, i.e. all banks.
-constexpr int STG_K = 0, STG_Q = 16384, STG_V = 32768, STG_REC = 49152;
+// q, v and the record are double-buffered (stage = chunk % 2); k, the one operand that is read until the
+// very end of a step, has three buffers (chunk % 3) so that its copy can be issued two steps ahead.
+constexpr int STG_Q = 0, STG_V = 16384, STG_REC = 32768;
 constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB;
-constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 62 464
+constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 46 080
+constexpr int KBUF = 2 * STG_BYTES;                          // three k tiles of 16 KB follow the two stages
 constexpr int OT_PITCH = 272;                     // bytes per token row of the output tile (256 B + pad: conflict-free 8-byte writes)
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
-constexpr size_t WIDE_SMEM = 2 * STG_BYTES + OT_BYTES;       // 142 336 B: one workgroup per CU
+constexpr size_t WIDE_SMEM = KBUF + 3 * 16384 + OT_BYTES;    // 158 720 B of the CU's 163 840: one workgroup per CU
 constexpr int WIDE_NN = 2;                        // 16-column tiles per compute wave
 constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
@@ -86,6 +89,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which (sequence, head, segment) and what to start from / write to ----
+    // Workgroups that read the same k (and q) rows - the value heads of one q/k head, and in pass 1
+    // also the S and M runs of one segment - form a group.  Workgroups are dealt to the 8 XCDs
+    // round-robin by block index, so a group takes consecutive slots of ONE XCD: its members run at
+    // the same time on CUs that share an L2, and the shared rows come from HBM once.
+    const int G = HV / H;                         // value heads per q/k head
+    const int64_t slot = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
     int64_t inh;
     int seg;
     int init = 0;                 // 0: from `src` (NULL = zero state), 1: identity, 2: zero
@@ -93,26 +103,34 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     const float* src = nullptr;
     float* dst = nullptr;
     if (sp.kind == WIDE_WHOLE) {
-        inh = blockIdx.x; seg = 0;
+        const int64_t group = (slot / G) * 8 + xcd;                 // (sequence, q/k head)
+        if (group >= p.N * H) return;
+        inh = (group / H) * HV + (group % H) * G + slot % G; seg = 0;
         src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true;
         dst = p.ht ? p.ht + inh * 16384 : nullptr; dst_user = true;
     } else if (sp.kind == WIDE_PASS1) {
-        const int per = 2 * sp.nseg - 3;                    // S runs of segments 0..nseg-2, M runs of 1..nseg-2
-        inh = blockIdx.x / per;
-        const int idx = (int)(blockIdx.x % per);
-        if (idx < sp.nseg - 1) {
-            seg = idx;
+        // group = (sequence, q/k head, segment 0 .. nseg-2); members: S runs of its value heads, then M runs
+        const int64_t group = (slot / (2 * G)) * 8 + xcd;
+        if (group >= p.N * H * (sp.nseg - 1)) return;
+        const int member = (int)(slot % (2 * G));
+        const int64_t nh = group / (sp.nseg - 1);
+        seg = (int)(group % (sp.nseg - 1));
+        inh = (nh / H) * HV + (nh % H) * G + member % G;
+        if (member < G) {
             if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
             else init = 2;
             dst = sp.sloc + (inh * sp.nseg + seg) * 16384;
         } else {
-            seg = idx - (sp.nseg - 1) + 1;
+            if (seg == 0) return;                                   // the first segment starts from the true state: no transition needed
             init = 1; v_zero = true;
             dst = sp.mseg + (inh * sp.nseg + seg) * 16384;
         }
     } else {
-        inh = blockIdx.x / sp.nseg;
-        seg = (int)(blockIdx.x % sp.nseg);
+        const int64_t group = (slot / G) * 8 + xcd;                 // (sequence, q/k head, segment)
+        if (group >= p.N * H * sp.nseg) return;
+        const int64_t nh = group / sp.nseg;
+        seg = (int)(group % sp.nseg);
+        inh = (nh / H) * HV + (nh % H) * G + slot % G;
         if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
         else src = sp.sin + (inh * sp.nseg + seg) * 16384;
         if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * 16384; dst_user = true; }
@@ -136,15 +154,15 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     const int64_t it1 = min(nt, it0 + sp.seg_chunks);
     const int64_t nsteps = it1 - it0;                       // may be <= 0 for an empty sequence
     const int64_t lastc = it1 - 1;
-    char* otile = smem + 2 * STG_BYTES;                     // [64 token rows][OT_PITCH]
+    char* otile = smem + KBUF + 3 * 16384;                  // [64 token rows][OT_PITCH]
 
     // =====================================================================================
     // Copy waves.  Step i (chunk it = it0 + i, stage cur = i & 1) has two phases, separated by
     // the workgroup barriers B1 (after the first half) and B2 (after the second half):
     //   phase A  compute waves read everything of stage cur and write the output tile
     //   phase B  compute waves read k of stage cur (transposed)
-    // so the q / v / record part of a stage is free from B1 on and its k part from B2 on; all of
-    // chunk it+1 must be in the other stage at B2.  Loads complete in issue order, so "at most
+    // so the q / v / record part of a stage is free from B1 on and a k buffer from B2 on; all of
+    // chunk it+1 must have landed at B2.  Loads complete in issue order, so "at most
     // N operations outstanding" proves that all but the N newest have landed.
     // =====================================================================================
     if (w >= CW) {
@@ -173,17 +191,19 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 if (j >= from && j < to) gather_1k_to_lds(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024);
         };
         if (w == CW) {
-            // ---- k: issued at the start of a step for the next chunk, awaited at its end ----
-            auto issue_k = [&](int64_t it, int stage) {
-                gather_blocks((const T*)p.k, H, h, it, 0, 16, lds0 + stage * STG_BYTES + STG_K);
+            // ---- k: the copy of chunk i+2 is issued at the start of step i (its buffer was last read
+            // in step i-1) and awaited at the end of step i+1 ----
+            auto issue_k = [&](int64_t i) {                                 // i counts from the first chunk of this run
+                gather_blocks((const T*)p.k, H, h, min(it0 + i, lastc), 0, 16, lds0 + KBUF + (int)(i % 3) * 16384);
             };
-            issue_k(it0, 0);
-            wait_vm_at_most<0>();
-            lds_barrier();                                                  // B0: stage 0 is complete
+            issue_k(0);
+            issue_k(1);
+            wait_vm_at_most<16>();
+            lds_barrier();                                                  // B0: chunk 0 is complete
             for (int64_t i = 0; i < nsteps; ++i) {
-                issue_k(min(it0 + i + 1, lastc), (int)((i & 1) ^ 1));
+                issue_k(i + 2);
                 lds_barrier();                                              // B1
-                wait_vm_at_most<0>();
+                wait_vm_at_most<16>();                                      // all but the newest copy: chunk i+1 has landed
                 lds_barrier();                                              // B2
             }
         } else if (w <= CW + 2) {
@@ -202,9 +222,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                         if (early) { copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }      // all 7 pieces
                     }
                 } else {
-                    if (early) gather_blocks((const T*)p.v, HV, hv, it, 0, 8, st + STG_V);
+                    if (early) { if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 0, 8, st + STG_V); }      // (v is not read when it counts as zero)
                     else {
-                        gather_blocks((const T*)p.v, HV, hv, it, 8, 16, st + STG_V);
+                        if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 8, 16, st + STG_V);
                         if constexpr (FULL) copy_rec(it, 6, 12, st);
                     }
                 }
@@ -309,11 +329,11 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // window of three operand fragments), and the thin, dependent part of a step (D -> v_new ->
     // output of a pair of t-tiles) is cut into pieces that each share a region with four
     // independent matrix instructions (products of the next tiles, or the state update).
-    auto step = [&](const char* st) {
-        const V8* sK = (const V8*)(st + STG_K);
+    auto step = [&](const char* st, const char* kbuf) {
+        const V8* sK = (const V8*)kbuf;
         const V8* sQ = (const V8*)(st + STG_Q);
         const T* sV = (const T*)(st + STG_V);
-        const T* sKt = (const T*)(st + STG_K);
+        const T* sKt = (const T*)kbuf;
         const V8* sX = (const V8*)(st + STG_X);
         const V8* sP = (const V8*)(st + STG_P);
         const float* sTab = (const float*)(st + STG_TAB);
@@ -462,7 +482,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (nsteps > 0) {
         lds_barrier();                                          // B0: the copy waves have filled stage 0
         for (int64_t i = 0; i < nsteps; ++i) {
-            step(smem + (i & 1) * STG_BYTES);
+            step(smem + (i & 1) * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384);
         }
     }
 
@@ -571,14 +591,16 @@ int launch_scan_wide(const ChunkParams& p, hipStream_t stream) {
     sp.kind = WIDE_WHOLE;
     sp.nseg = 1;
     sp.seg_chunks = 1 << 30;
-    return launch_wide_kind<T, true>(p, sp, p.NH, stream);
+    const int64_t G = p.HV / p.H;
+    return launch_wide_kind<T, true>(p, sp, (p.N * p.H + 7) / 8 * 8 * G, stream);
 }
 
 template <typename T>
 int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
     int rc;
     sp.kind = WIDE_PASS1;
-    if ((rc = launch_wide_kind<T, false>(p, sp, p.NH * (2 * sp.nseg - 3), stream))) return rc;
+    const int64_t G = p.HV / p.H;
+    if ((rc = launch_wide_kind<T, false>(p, sp, (p.N * p.H * (sp.nseg - 1) + 7) / 8 * 8 * 2 * G, stream))) return rc;
     if (sp.nseg > 1) {
         static bool attr_done = false;
         if (!attr_done) {
@@ -591,7 +613,7 @@ int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t strea
         if ((rc = check_launch("gdn_segment_merge_kernel"))) return rc;
     }
     sp.kind = WIDE_PASS2;
-    return launch_wide_kind<T, true>(p, sp, p.NH * sp.nseg, stream);
+    return launch_wide_kind<T, true>(p, sp, (p.N * p.H * sp.nseg + 7) / 8 * 8 * G, stream);
 }
 
 template int launch_scan_wide<bf16_t>(const ChunkParams&, hipStream_t);
