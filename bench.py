@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|calib_copy]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -8,9 +8,11 @@ configuration the >= 50 %-of-MFMA-roofline target is quoted on.  A step is one c
 chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries, under
 "other_workloads", the decode step (B=256: us/step and state GB/s) and the other prefill
 configurations, and:
-  roofline      dominant kernel, algorithmic FLOPs (or bytes) per launch / its mean duration
-                measured with HIP events on the launch stream
+  roofline      dominant stage (the launches of one C entry point), algorithmic FLOPs (or bytes)
+                per call / its mean duration measured with HIP events on the launch stream
   cpu_baseline  the CPU oracle (torch fp32, all host cores) on a bounded sample of the workload
+--workload calib_copy runs a plain 1 GiB device copy: the kernel of known size against which the
+FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled.
 """
 from __future__ import annotations
 
@@ -30,11 +32,17 @@ import torch  # noqa: E402
 import torch.nn.functional as F  # noqa: E402
 
 C, K, V = 64, 128, 128
-# algorithmic FLOPs per (token, v-head): 2*(3CK + 2CV + 3KV); the scan kernel does w*S, k^T*v_new,
-# q*S (3KV) and P*v_new (CV), the prepare kernel K K^T, q k^T, w (3CK) and u (CV)
-F_SCAN = 2 * (3 * K * V + C * V)
-F_PREP = 2 * (3 * C * K + C * V)
-F_TOTAL = F_SCAN + F_PREP                      # 180224
+# algorithmic FLOPs per (token, v-head) of the chunked gated delta rule as the reference evaluates
+# it: 2*(3CK + 2CV + 3KV) = 180224 (K K^T, q k^T, w; u, P v_new; w S, k^T v_new, q S).
+# Here the sequential stage does k S, q S, k^T v_new (3KV), Xb D and P v_new (2CV); the rest
+# (K K^T, q k^T, the 64x64 inverse) is the chunk-parallel stage.
+F_TOTAL = 2 * (3 * C * K + 2 * C * V + 3 * K * V)      # 180224
+F_SCAN = 2 * (3 * K * V + 2 * C * V)                   # 131072
+F_PREP = F_TOTAL - F_SCAN                              # 49152
+# HBM bytes per call of the dominant stage on the default workload, from FETCH_SIZE + WRITE_SIZE of
+# a counter run of this file scaled by the calib_copy workload (profiles/ holds the summary); other
+# workloads: not measured
+TRAFFIC_BYTES = {'prefill': 1.67e9}
 PEAK_BF16_TFLOPS = 2500.0                      # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0                          # MI355X HBM3E, published
 
@@ -116,12 +124,13 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     t_prep = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e-3
     t_scan = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e-3
     units = tokens * w['HV']
-    dom = ('gdn_chunk_scan_kernel', F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_prepare_kernel', F_PREP, t_prep)
+    scan_name = 'gdn_chunk_fwd_scan: gdn_chunk_wide_kernel (+ gdn_segment_merge_kernel when time is cut into segments)'
+    dom = (scan_name, F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_fwd_prepare: gdn_chunk_prepare_kernel', F_PREP, t_prep)
     achieved = units * dom[1] / dom[2] / 1e12
     roofline = dict(bound='mfma', achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit='TFLOP/s',
-                    frac=round(achieved / PEAK_BF16_TFLOPS, 5), traffic=None, kernel=dom[0],
+                    frac=round(achieved / PEAK_BF16_TFLOPS, 5), traffic=TRAFFIC_BYTES.get(w['key']), kernel=dom[0],
                     kernel_us=round(dom[2] * 1e6, 1), flops_per_launch=units * dom[1],
-                    kernels_us=dict(gdn_chunk_prepare_kernel=round(t_prep * 1e6, 1), gdn_chunk_scan_kernel=round(t_scan * 1e6, 1)),
+                    kernels_us=dict(gdn_chunk_fwd_prepare=round(t_prep * 1e6, 1), gdn_chunk_fwd_scan=round(t_scan * 1e6, 1)),
                     whole_op=dict(flops=units * F_TOTAL, achieved=round(units * F_TOTAL / (elapsed / steps) / 1e12, 2),
                                   frac=round(units * F_TOTAL / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 5)))
     out = dict(value=tokens * steps / elapsed, ms_per_step=ms_per_step, roofline=roofline)
@@ -149,11 +158,13 @@ def cpu_baseline_prefill(w, cpu):
     t_cal = run(512)
     rate = 512 * cpu['q'].shape[0] / t_cal
     T_s = int(min(cpu['q'].shape[1], max(1024, (rate * 12 / cpu['q'].shape[0]) // 64 * 64)))
-    t = run(T_s)
+    reps = max(1, min(8, int(12 / max(run(T_s), 1e-3))))          # about 10-20 s of CPU work in all
+    ts = [run(T_s) for _ in range(reps)]
+    t = statistics.median(ts)
     toks = T_s * cpu['q'].shape[0]
     return dict(value=round(toks / t, 1), unit='tokens/s', cores=torch.get_num_threads(), kind='port',
                 sample=f'oracle chunk_gated_delta_rule (torch fp32 CPU) on the first {T_s} tokens per sequence of the same '
-                       f'inputs, {t:.1f} s wall, dense (not packed) layout', seconds=round(t, 2))
+                       f'inputs, median of {reps} runs of {t:.1f} s, dense (not packed) layout', seconds=round(sum(ts), 2))
 
 
 def bench_decode(w, steps, warmup, device, with_cpu):
@@ -207,12 +218,29 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     return out
 
 
+def calib_copy(steps, warmup, device):
+    """A plain device-to-device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch)."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    print(json.dumps(dict(metric='calib_copy_GBps', value=round(2 * n / t / 1e9, 1), unit='GB/s', bytes_read=n, bytes_written=n,
+                          steps=steps, warmup=warmup)))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS))
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['calib_copy'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     args = ap.parse_args()
@@ -225,6 +253,11 @@ def main():
     device = 'cuda:0'
     torch.cuda.set_device(0)
 
+    if args.workload == 'calib_copy':
+        calib_copy(args.steps, args.warmup, device)
+        return
+    for key, val in WORKLOADS.items():
+        val['key'] = key
     w = WORKLOADS[args.workload]
     fn = bench_prefill if w['kind'] == 'prefill' else bench_decode
     res = fn(w, args.steps, args.warmup, device, not args.no_cpu_baseline)

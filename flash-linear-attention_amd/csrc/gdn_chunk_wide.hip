@@ -105,7 +105,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (sp.kind == WIDE_WHOLE) {
         const int64_t group = (slot / G) * 8 + xcd;                 // (sequence, q/k head)
         if (group >= p.N * H) return;
-        inh = (group / H) * HV + (group % H) * G + slot % G; seg = 0;
+        int64_t nseq = group / H;
+        if (p.flags & GDN_FLAG_SEQ_ORDER) nseq = load_index(p.chunk_offsets, p.N + 1 + nseq, cu32);     // longest sequences start first
+        inh = nseq * HV + (group % H) * G + slot % G; seg = 0;
         src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true;
         dst = p.ht ? p.ht + inh * 16384 : nullptr; dst_user = true;
     } else if (sp.kind == WIDE_PASS1) {

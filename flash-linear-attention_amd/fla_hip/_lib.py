@@ -27,6 +27,7 @@ FLAG_BETA_VECTOR = 1 << 4
 FLAG_CU_INT32 = 1 << 5
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
+FLAG_SEQ_ORDER = 1 << 19
 
 # name -> (restype, argtypes); one entry per declaration in include/gdn_hip.h
 SIGNATURES = {

@@ -22,7 +22,7 @@ from fla_hip.ops.gated_delta_rule._common import (
     require_gpu,
     unify_gate_beta,
 )
-from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_chunk_offsets
+from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
 from fla_hip.utils import input_guard
 
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
@@ -94,7 +94,9 @@ class ChunkLaunch:
             if chunk_indices is None or chunk_size != _KERNEL_CHUNK:
                 chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
             chunk_indices = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
-            chunk_offsets = prepare_chunk_offsets(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+            # chunk offsets per sequence, followed by the longest-first order of the sequences
+            chunk_offsets = prepare_scan_tables(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+            flags |= _lib.FLAG_SEQ_ORDER
             num_chunks = chunk_indices.shape[0]
         else:
             chunk_indices = chunk_offsets = None

@@ -41,3 +41,17 @@ def prepare_chunk_offsets(cu_seqlens: torch.Tensor, chunk_size: int,
     out = torch.zeros(counts.numel() + 1, dtype=torch.int64)
     out[1:] = torch.cumsum(counts, 0)
     return out.to(device=cu_seqlens.device, dtype=cu_seqlens.dtype)
+
+
+@tensor_cache
+def prepare_scan_tables(cu_seqlens: torch.Tensor, chunk_size: int,
+                        cu_seqlens_cpu: torch.Tensor | None = None) -> torch.Tensor:
+    """``prepare_chunk_offsets`` ([N+1]) followed by [N] sequence ids sorted by decreasing length:
+    the order in which the sequential kernel hands sequences to the CUs (longest first, so that
+    no CU is left with a long sequence at the end).  One tensor, one upload."""
+    lens = _host_lens(cu_seqlens, cu_seqlens_cpu)
+    counts = (lens + (chunk_size - 1)) // chunk_size
+    out = torch.zeros(2 * counts.numel() + 1, dtype=torch.int64)
+    out[1:counts.numel() + 1] = torch.cumsum(counts, 0)
+    out[counts.numel() + 1:] = torch.argsort(counts, descending=True, stable=True)
+    return out.to(device=cu_seqlens.device, dtype=cu_seqlens.dtype)

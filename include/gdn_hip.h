@@ -45,6 +45,7 @@ extern "C" {
  * (all forms give the same result up to rounding; used by tests and for tuning)                */
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
 #define GDN_FLAG_SCAN_SEGMENTS  (1u << 18) /* time cut into segments (dense input, >= 8 chunks) */
+#define GDN_FLAG_SEQ_ORDER      (1u << 19) /* chunk_offsets carries N more entries (see there)   */
 
 /* Library ABI version (bumped on any signature change). */
 int gdn_hip_abi_version(void);
@@ -98,7 +99,9 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  *   chunk_table [num_chunks][2] (device; sequence id, chunk id inside the sequence) -
  *         prepare_chunk_indices of fla/ops/utils/index.py:156-164; NULL for dense input
  *   chunk_offsets [N+1] (device; exclusive prefix sum of chunks per sequence) -
- *         prepare_chunk_offsets of fla/ops/utils/index.py:167-172; NULL for dense input
+ *         prepare_chunk_offsets of fla/ops/utils/index.py:167-172; NULL for dense input.
+ *         With GDN_FLAG_SEQ_ORDER the array has N more entries: the sequence ids in the order in
+ *         which the sequential kernel should start them (longest first keeps the CUs evenly loaded)
  *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
  *   Requires K == V == 128, HV % H == 0 (the Python host zero-pads smaller head dims).
  */

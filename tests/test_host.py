@@ -236,3 +236,20 @@ def test_assert_close_metric():
         assert_close('bad', x, y, 0.01)
     with pytest.warns(UserWarning):
         assert_close('warn', x, y, 0.01, warning=True)
+
+
+def test_scan_tables_offsets_then_longest_first_order():
+    """prepare_scan_tables = prepare_chunk_offsets followed by the sequence ids by decreasing
+    number of chunks (ties keep packed order)."""
+    import torch
+    from fla_hip.ops.utils.index import prepare_chunk_offsets, prepare_scan_tables
+    cu = torch.tensor([0, 5, 300, 301, 1000, 1064, 1064 + 700])
+    t = prepare_scan_tables(cu, 64)
+    n = cu.numel() - 1
+    assert t.dtype == cu.dtype and t.numel() == 2 * n + 1
+    assert torch.equal(t[:n + 1], prepare_chunk_offsets(cu, 64))
+    counts = [(int(b - a) + 63) // 64 for a, b in zip(cu[:-1], cu[1:])]
+    order = t[n + 1:].tolist()
+    assert sorted(order) == list(range(n))
+    assert [counts[i] for i in order] == sorted(counts, reverse=True)
+    assert order == sorted(range(n), key=lambda i: (-counts[i], i))
