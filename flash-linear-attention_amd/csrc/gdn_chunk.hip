@@ -62,7 +62,7 @@ static int chunk_entry(
                   (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
                   "%s: q/k/v must be bf16 or f16", who);
-    GDN_CHECK_ARG(HV <= 65535, GDN_ERR_UNSUPPORTED, "%s: HV > 65535", who);
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * H < (1ll << 31), GDN_ERR_UNSUPPORTED, "%s: too many heads or chunks for one launch", who);
     if (cu_seqlens) {
         GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
         GDN_CHECK_ARG(chunk_table && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);

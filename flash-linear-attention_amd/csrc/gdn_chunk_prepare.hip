@@ -29,9 +29,11 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
     float* sGB = sLd + 4 * 256;                 // [group][2][64] cumulative gate (log2), beta
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t ci = blockIdx.x;
-    const int h = blockIdx.y;
+    // heads vary fastest over the workgroups: those that run at the same time then read whole token rows
+    // (all heads of a token are contiguous in memory) instead of one 256-byte piece of every row
     const int H = p.H, HV = p.HV;
+    const int64_t ci = blockIdx.x / H;
+    const int h = (int)(blockIdx.x % H);
     const int G = HV / H;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
 
@@ -274,7 +276,7 @@ int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream)
             return check_launch("hipFuncSetAttribute(prepare)");
         attr_done = true;
     }
-    dim3 grid((unsigned)num_chunks, (unsigned)p.H), block(256);
+    dim3 grid((unsigned)(num_chunks * p.H)), block(256);
     hipLaunchKernelGGL(kern, grid, block, smem, stream, p);
     return check_launch("gdn_chunk_prepare_kernel");
 }

@@ -49,6 +49,9 @@ constexpr int OT_PITCH = 272;                     // bytes per token row of the 
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
 constexpr size_t WIDE_SMEM = KBUF + 3 * 16384 + OT_BYTES;    // 158 720 B of the CU's 163 840: one workgroup per CU
 constexpr int WIDE_NN = 2;                        // 16-column tiles per compute wave
+#ifndef WIDE_RING
+#define WIDE_RING 3                               // operand fragments in flight per compute wave
+#endif
 constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
 
@@ -341,11 +344,12 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const float* sTab = (const float*)(st + STG_TAB);
         auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
-        // fragment f = (t-tile f/4, key tiles (2s, 2s+1) with s = f%4) of k and q, ring of three
-        V8 ak[3], aq[3];
+        // fragment f = (t-tile f/4, key tiles (2s, 2s+1) with s = f%4) of k and q, in a ring of RING register sets
+        constexpr int RING = WIDE_RING;
+        V8 ak[RING], aq[RING];
         auto F = [&](int f) {
-            ak[f % 3] = sK[(f >> 2) * 256 + 16 * (f & 3) + a_off];
-            if constexpr (FULL) aq[f % 3] = sQ[(f >> 2) * 256 + 16 * (f & 3) + a_off];
+            ak[f % RING] = sK[(f >> 2) * 256 + 16 * (f & 3) + a_off];
+            if constexpr (FULL) aq[f % RING] = sQ[(f >> 2) * 256 + 16 * (f & 3) + a_off];
         };
         f32x4 ks[4][NN], ao[4][NN];
         V8 Sb[4][NN];
@@ -353,8 +357,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             const int tt = f >> 2, sx = f & 3;
 #pragma unroll
             for (int nn = 0; nn < NN; ++nn) {
-                ks[tt][nn] = Mma<T>::run(ak[f % 3], Sb[sx][nn], sx ? ks[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
-                if constexpr (FULL) ao[tt][nn] = Mma<T>::run(Sb[sx][nn], aq[f % 3], sx ? ao[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
+                ks[tt][nn] = Mma<T>::run(ak[f % RING], Sb[sx][nn], sx ? ks[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
+                if constexpr (FULL) ao[tt][nn] = Mma<T>::run(Sb[sx][nn], aq[f % RING], sx ? ao[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
             }
         };
         V4 vv[4][NN];                           // v in C/D layout, per t-tile
@@ -425,7 +429,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         };
 
         // ---- the state as B operand (pairs of key tiles (2s, 2s+1) = key features 32s + 8g + e) ----
-        F(0); F(1);
+#pragma unroll
+        for (int f = 0; f < RING - 1; ++f) F(f);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -440,24 +445,26 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const bool lazy = lg_try >= LG_MIN;
         vscale = lazy ? fast_exp2(-lg_try) : 1.f;
         fence();
-        // ---- t-tiles 0, 1 ----
-        F(2); M(0); fence();
-        F(3); M(1); fence();
-        F(4); M(2); fence();
-        F(5); M(3); fence();
-        F(6); M(4); FV(0); fence();
-        F(7); M(5); FV(1); fence();
-        F(8); M(6); FX(0); fence();
-        F(9); M(7); FX(1); fence();
-        // ---- t-tiles 2, 3, with the tail of tiles 0, 1 ----
-        F(10); M(8); TD(0); fence();
-        F(11); M(9); TD(1); FP(0); fence();
-        F(12); M(10); TX(0); FP(1); fence();
-        F(13); M(11); TX(1); FV(2); fence();
-        F(14); M(12); TP(0); FV(3); fence();
-        F(15); M(13); TP(1); FX(2); fence();
-        M(14); FX(3); FK(0, 0); FK(0, 1); fence();
-        M(15); FK(0, 2); FK(0, 3); fence();
+        // ---- sixteen regions: the products of fragment f, the fetch of fragment f + RING - 1, and beside them
+        // the other fetches (t-tiles 0, 1) and then the tail of tiles 0, 1 while tiles 2, 3 are multiplied ----
+#pragma unroll
+        for (int f = 0; f < 16; ++f) {
+            if (f + RING - 1 < 16) F(f + RING - 1);
+            M(f);
+            if (f == 4) FV(0);
+            if (f == 5) FV(1);
+            if (f == 6) FX(0);
+            if (f == 7) FX(1);
+            if (f == 8) TD(0);
+            if (f == 9) { TD(1); FP(0); }
+            if (f == 10) { TX(0); FP(1); }
+            if (f == 11) { TX(1); FV(2); }
+            if (f == 12) { TP(0); FV(3); }
+            if (f == 13) { TP(1); FX(2); }
+            if (f == 14) { FX(3); FK(0, 0); FK(0, 1); }
+            if (f == 15) { FK(0, 2); FK(0, 3); }
+            fence();
+        }
         // the decay fold: rare, a scalar branch so that it is not if-converted into the common path
         if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
             const float fold = fast_exp2(lg_try);
