@@ -48,6 +48,7 @@ extern "C" size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64
 static int chunk_entry(
     const char* who, int stages,
     const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,
@@ -57,6 +58,8 @@ static int chunk_entry(
     using namespace gdn;
     GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "%s: non-positive dimension", who);
+    GDN_CHECK_ARG(!dt_bias || A_log, GDN_ERR_INVALID, "%s: dt_bias without A_log", who);
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
     GDN_CHECK_ARG(K == 128 && V == 128, GDN_ERR_UNSUPPORTED, "%s: only K = V = 128 is built (got K=%lld V=%lld)", who,
                   (long long)K, (long long)V);
@@ -78,7 +81,7 @@ static int chunk_entry(
     const size_t need = ws_layout(num_chunks, H, HV, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
-    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.ht = ht; p.o = o;
+    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.NH = N * HV;
@@ -89,6 +92,7 @@ static int chunk_entry(
 
 #define GDN_CHUNK_ARGS                                                                          \
     const void *q, const void *k, const void *v, const void *g, const void *beta,               \
+    const float *A_log, const float *dt_bias,                                                   \
     const float *h0, float *ht, void *o,                                                        \
     const void *cu_seqlens, const void *chunk_table, const void *chunk_offsets,                 \
     void *workspace, size_t workspace_bytes,                                                    \
@@ -96,7 +100,7 @@ static int chunk_entry(
     int64_t N, int64_t num_chunks,                                                              \
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void *stream
 #define GDN_CHUNK_PASS                                                                          \
-    q, k, v, g, beta, h0, ht, o, cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, \
+    q, k, v, g, beta, A_log, dt_bias, h0, ht, o, cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, \
     B, T, H, HV, K, V, N, num_chunks, scale, qkv_dtype, gb_dtype, flags, stream
 
 extern "C" int gdn_chunk_fwd(GDN_CHUNK_ARGS) {

@@ -90,6 +90,7 @@ inline size_t ws_layout(int64_t NC, int64_t H, int64_t HV, char* base, ChunkWs* 
 
 struct ChunkParams {
     const void* q; const void* k; const void* v; const void* g; const void* beta;
+    const float* A_log; const float* dt_bias;     // optional gate activation (per value head)
     const float* h0; float* ht; void* o;
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     ChunkWs ws;

@@ -4,6 +4,9 @@
 //   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  X = (I+L)^-1 in fp32 (16x16 forward
 //   substitution on the diagonal blocks, fp32-MFMA block merges),  Xb = X diag(beta),
 //   P = scale*tril(q k^T * 2^(G_i-G_j)),  and the per-token gate tables.
+// Optional prologues of the reference are folded in: the gate and beta activations, and the l2
+// normalisation of q and k as per-row factors 1/|k_t|, 1/|q_t| on L, P and the tables (so the
+// sequential stage reads q and k exactly as the caller gave them).
 // The raw products K K^T and q K^T are formed once and stay in registers; the value heads differ
 // only in their gates.  Xb and P are written in the exact register order ("fragments") in which
 // the scan kernel feeds them to the matrix cores; the scan forms v_new = Xb (v - 2^G (k S)) itself
@@ -14,8 +17,9 @@ namespace gdn {
 
 constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 272 B rows, conflict-free 16 B reads
 constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
-// two tiles (k then L, q then X), the transposed diagonal blocks of L, and gates + beta of every value head of the group
-inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + (size_t)group * 2 * CH * 4; }
+// two tiles (k then L, q then X), the transposed diagonal blocks of L, the row factors of k and q, and gates + beta
+// of every value head of the group
+inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + 2 * CH * 4 + (size_t)group * 2 * CH * 4; }
 
 template <typename T>
 __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p) {
@@ -26,7 +30,8 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
     float* sL = (float*)k_nat;                  // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
     float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1
     float* sLd = (float*)(q_nat + CH * NP);     // [4][16 j][16 i] diagonal blocks of L, transposed (column j contiguous)
-    float* sGB = sLd + 4 * 256;                 // [group][2][64] cumulative gate (log2), beta
+    float* sRN = sLd + 4 * 256;                 // [2][64] 1/|k_t|, 1/|q_t| (ones unless the rows are to be normalised)
+    float* sGB = sRN + 2 * CH;                  // [group][2][64] cumulative gate (log2), beta
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // heads vary fastest over the workgroups: those that run at the same time then read whole token rows
@@ -71,13 +76,28 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
                 rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * 128 + col);
             }
         }
+        const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
 #pragma unroll
         for (int ps = 0; ps < 4; ++ps) {
             const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
             *(u32x4*)(k_nat + row * NP + col) = rk[ps];
             *(u32x4*)(q_nat + row * NP + col) = rq[ps];
+            // l2 normalisation is applied as per-row factors: 16 lanes hold one row
+            float sk = 0.f, sq = 0.f;
+            if (l2) {
+                const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk += a * a; sq += b * b; }
+#pragma unroll
+                for (int off = 1; off < 16; off <<= 1) { sk += __shfl_xor(sk, off, 64); sq += __shfl_xor(sq, off, 64); }
+            }
+            if ((tid & 15) == 0) {
+                sRN[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
+                sRN[CH + row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
+            }
         }
     }
+    __syncthreads();
     // ---- gates of every value head of the group: inclusive scan over the chunk, one token per lane ----
     for (int m = w; m < G; m += 4) {
         const int hv = h * G + m;
@@ -88,6 +108,10 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
                 x = load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype);
                 b = load_scalar(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
             }
+        }
+        if (lane < valid) {                      // optional activations of the raw gate / beta inputs
+            if (p.A_log) x = -__expf(p.A_log[hv]) * softplus_f(x + (p.dt_bias ? p.dt_bias[hv] : 0.f));
+            if (p.flags & GDN_FLAG_BETA_SIGMOID) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
         }
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -100,12 +124,12 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
         sGB[(2 * m) * CH + lane] = x;
         sGB[(2 * m + 1) * CH + lane] = b;
         float* tab = (float*)(p.ws.Rec + (ci * HV + hv) * REC_BYTES + REC_TAB);
-        tab[TAB_DEC + lane] = fast_exp2(xl - x);
-        tab[TAB_SG + lane] = p.scale * ex;
-        tab[TAB_EG + lane] = ex;
+        const float nk = sRN[lane], nq = sRN[CH + lane];
+        tab[TAB_DEC + lane] = fast_exp2(xl - x) * nk;        // multiplies v_new rows on their way into k^T v_new
+        tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
+        tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
         if (lane == 63) tab[TAB_GLAST] = x;
     }
-    __syncthreads();
 
     // ---- raw products, kept in registers: K K^T tiles (row-tile w, column-tiles <= w) and the
     // transposed q K^T tiles of query tile tt = 3 - w (key tiles <= tt) ----
@@ -140,16 +164,17 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
         char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
         // ---- L tiles of row-tile w (gated, beta-scaled, strictly lower) ----
         {
-            const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g), bi = *(const f32x4*)(sB + 16 * w + 4 * g);
+            const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g);
+            const f32x4 bi = *(const f32x4*)(sB + 16 * w + 4 * g) * *(const f32x4*)(sRN + 16 * w + 4 * g);
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
                 const int j = 16 * tj + c16;
-                const float gj = sG[j];
+                const float gj = sG[j], nj = sRN[j];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int i = 16 * w + 4 * g + r;
                     // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
-                    const float val = (i > j && tj <= w) ? bi[r] * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
+                    const float val = (i > j && tj <= w) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
                     sL[i * LP + j] = val;
                     if (tj == w) sLd[(w * 16 + c16) * 16 + 4 * g + r] = val;
                 }
@@ -158,7 +183,7 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
         // ---- P^T tiles of query tile tt (gated, lower incl. diagonal), straight to memory ----
         {
             const int t = 16 * tt + c16;
-            const float gt = sG[t];
+            const float gt = sG[t], st = p.scale * sRN[CH + t];
             T* pf = (T*)(rec + REC_P);
 #pragma unroll
             for (int sp = 0; sp < 2; ++sp) {
@@ -167,11 +192,11 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     const int tj = 2 * sp + half;
-                    const f32x4 gj = *(const f32x4*)(sG + 16 * tj + 4 * g);
+                    const f32x4 gj = *(const f32x4*)(sG + 16 * tj + 4 * g), nj = *(const f32x4*)(sRN + 16 * tj + 4 * g);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int j = 16 * tj + 4 * g + r;
-                        const float val = (t >= j) ? p.scale * qk[tj][r] * fast_exp2(gt - gj[r]) : 0.f;
+                        const float val = (t >= j) ? st * nj[r] * qk[tj][r] * fast_exp2(gt - gj[r]) : 0.f;
                         frag[half * 4 + r] = from_f32<T>(val);
                     }
                 }

@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -45,6 +45,7 @@ SIGNATURES = {
 }
 _CHUNK_ARGS = [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # q k v g beta
+    c_void_p, c_void_p,                                    # A_log dt_bias
     c_void_p, c_void_p, c_void_p,                          # h0 ht o
     c_void_p, c_void_p, c_void_p,                          # cu_seqlens chunk_table chunk_offsets
     c_void_p, c_size_t,                                    # workspace, bytes

@@ -1,9 +1,11 @@
 """``chunk_gated_delta_rule``: same signature, defaults, validation and error types as
 fla/ops/gated_delta_rule/chunk.py:397-593.  The reference's five Triton launches
-(chunk.py:33-123) are replaced by one call into libgdn_hip.so (``gdn_chunk_fwd``), which
-runs two HIP kernels: a chunk-parallel one (gate cumsum, gated beta*K*K^T, 64x64 unit-lower
-solve, WY factors w/u, intra-chunk q k^T) and a sequential one (state recurrence fused with
-the output), so per-chunk states are never written to memory."""
+(chunk.py:33-123) and its optional prologue launches (l2norm of q and k, gate activation,
+beta sigmoid: chunk.py:278-288) are replaced by one call into libgdn_hip.so
+(``gdn_chunk_fwd``), which runs a chunk-parallel HIP kernel (prologues, gate cumsum, gated
+beta*K*K^T, 64x64 unit-lower solve, intra-chunk q k^T) and a sequential one (state
+recurrence fused with the WY step and the output), so neither normalised copies of q and k
+nor w, u or per-chunk states are ever written to memory."""
 from __future__ import annotations
 
 import os
@@ -33,13 +35,6 @@ _SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGM
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 
-def _l2norm_rows(x: torch.Tensor) -> torch.Tensor:
-    """x / sqrt(sum(x^2) + 1e-6) per head vector, result in x's dtype (the reference's
-    l2norm_fwd, fla/modules/l2norm.py:84-109, applied before its chunk pipeline)."""
-    xf = x.float()
-    return (xf * torch.rsqrt((xf * xf).sum(-1, keepdim=True) + 1e-6)).to(x.dtype)
-
-
 def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
     if x.shape[-1] == size:
         return x
@@ -62,7 +57,8 @@ class ChunkLaunch:
     _ENTRY = {None: 'gdn_chunk_fwd', 'prepare': 'gdn_chunk_fwd_prepare', 'scan': 'gdn_chunk_fwd_scan'}
 
     def __init__(self, q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first=False,
-                 cu_seqlens=None, cu_seqlens_cpu=None, chunk_indices=None, chunk_size=64):
+                 cu_seqlens=None, cu_seqlens_cpu=None, chunk_indices=None, chunk_size=64,
+                 A_log=None, dt_bias=None, qk_l2norm=False, beta_sigmoid=False, neg_eigval=False):
         dev = require_gpu(q, k, v, g, beta)
         B, T, H, K = k.shape
         HV, V = v.shape[2], v.shape[3]
@@ -83,6 +79,19 @@ class ChunkLaunch:
         g, beta, gb_code = unify_gate_beta(g, beta)
 
         flags = _lib.FLAG_STATE_V_FIRST if state_v_first else 0
+        # prologues the kernels apply themselves
+        if qk_l2norm:
+            flags |= _lib.FLAG_QK_L2NORM
+        if beta_sigmoid:
+            flags |= _lib.FLAG_BETA_SIGMOID | (_lib.FLAG_NEG_EIGVAL if neg_eigval else 0)
+        if A_log is not None:
+            A_log = A_log.detach().to(device=dev, dtype=torch.float32).contiguous()
+            if A_log.numel() != HV:
+                raise ValueError(f'A_log must have {HV} entries, got {A_log.numel()}')
+        if dt_bias is not None:
+            dt_bias = dt_bias.detach().to(device=dev, dtype=torch.float32).contiguous()
+            if dt_bias.numel() != HV:
+                raise ValueError(f'dt_bias must have {HV} entries, got {dt_bias.numel()}')
         flags |= _SCAN_MODE_FLAGS.get(os.environ.get('FLA_HIP_SCAN_MODE', 'auto'), 0)
         if cu_seqlens is not None:
             if cu_seqlens.dtype not in (torch.int32, torch.int64):
@@ -124,10 +133,10 @@ class ChunkLaunch:
         if ws_bytes == 0 and num_chunks > 0:
             raise NotImplementedError(f'HIP chunk kernels do not cover K={KP}, V={VP}')
         self.workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-        self.keep = (q, k, v, g, beta, cu_seqlens, chunk_indices, chunk_offsets)     # keep the buffers alive
+        self.keep = (q, k, v, g, beta, A_log, dt_bias, cu_seqlens, chunk_indices, chunk_offsets)     # keep the buffers alive
         self.device = dev
         self.args = (
-            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(h0), ptr(self.ht), ptr(self.o),
+            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(A_log), ptr(dt_bias), ptr(h0), ptr(self.ht), ptr(self.o),
             ptr(cu_seqlens), ptr(chunk_indices), ptr(chunk_offsets),
             ptr(self.workspace), ws_bytes,
             B, T, H, HV, KP, VP, N, num_chunks,
@@ -167,11 +176,18 @@ def chunk_gated_delta_rule_fwd(
     cu_seqlens_cpu: torch.Tensor | None = None,
     chunk_indices: torch.Tensor | None = None,
     chunk_size: int = 64,
+    A_log: torch.Tensor | None = None,
+    dt_bias: torch.Tensor | None = None,
+    use_qk_l2norm_in_kernel: bool = False,
+    use_beta_sigmoid_in_kernel: bool = False,
+    allow_neg_eigval: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
-    """Forward of the chunked operator on already-activated ``g`` (log space) and ``beta``.
+    """Forward of the chunked operator.  ``g`` is the log-space decay (raw gate inputs when
+    ``A_log`` is given), ``beta`` the write strength (logits with ``use_beta_sigmoid_in_kernel``).
     Returns ``(o in q's dtype, final_state fp32 or None)``."""
     call = ChunkLaunch(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first,
-                       cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size)
+                       cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size,
+                       A_log, dt_bias, use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)
     call.run()
     return call.results()
 
@@ -259,21 +275,13 @@ def chunk_gated_delta_rule(
     if scale is None:
         scale = k.shape[-1] ** -0.5
 
-    # prologues the reference runs as separate launches before its chunk pipeline
-    # (chunk.py:278-288 and gate.py:63-106); elementwise, done on the device
-    if use_qk_l2norm_in_kernel:
-        q, k = _l2norm_rows(q), _l2norm_rows(k)
-    if use_beta_sigmoid_in_kernel:
-        beta = torch.sigmoid(beta.float()) * (2.0 if allow_neg_eigval else 1.0)
-    if use_gate_in_kernel:
-        gf = g.float()
-        if dt_bias is not None:
-            gf = gf + dt_bias.float()
-        g = -A_log.float().exp() * torch.nn.functional.softplus(gf)
-
+    # the prologues the reference runs as separate launches before its chunk pipeline
+    # (chunk.py:278-288, gate.py:63-106) happen inside the first kernel
     return chunk_gated_delta_rule_fwd(
         q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first,
-        cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size)
+        cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size,
+        A_log if use_gate_in_kernel else None, dt_bias if use_gate_in_kernel else None,
+        use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)
 
 
 chunk_gdn = chunk_gated_delta_rule

@@ -94,6 +94,13 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  * chunk_fwd_o (fla/ops/common/chunk_o.py:544-586).
  *
  *   q, k [B,T,H,K], v, o [B,T,HV,V] qkv_dtype (bf16 or f16); g, beta [B,T,HV] gb_dtype
+ *   A_log [HV] fp32 or NULL: with it, g holds raw gate inputs and the kernel forms
+ *         g = -exp(A_log) * softplus(g + dt_bias) (dt_bias [HV] fp32 or NULL) - use_gate_in_kernel,
+ *         gdn_gate_chunk_cumsum of fla/ops/gated_delta_rule/gate.py:63-106
+ *   flags: GDN_FLAG_QK_L2NORM (q, k rows divided by sqrt(sum x^2 + 1e-6): l2norm_fwd of
+ *         fla/modules/l2norm.py:84-109, applied as per-row factors, q and k are read as given),
+ *         GDN_FLAG_BETA_SIGMOID / GDN_FLAG_NEG_EIGVAL (beta = [2*]sigmoid(beta):
+ *         fla/ops/common/gate.py:19-31), GDN_FLAG_STATE_V_FIRST, GDN_FLAG_CU_INT32, the scan flags
  *   h0 [N,HV,K,V] fp32 or NULL; ht [N,HV,K,V] fp32 or NULL
  *   cu_seqlens [N+1] (device) or NULL
  *   chunk_table [num_chunks][2] (device; sequence id, chunk id inside the sequence) -
@@ -107,6 +114,7 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  */
 int gdn_chunk_fwd(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,
@@ -126,6 +134,7 @@ int gdn_chunk_fwd(
  */
 int gdn_chunk_fwd_prepare(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,
@@ -134,6 +143,7 @@ int gdn_chunk_fwd_prepare(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 int gdn_chunk_fwd_scan(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,

@@ -176,6 +176,45 @@ def test_flags_and_state_layout():
         _check(f'o chunk_size={cs}', ref_o, o3)
 
 
+@pytest.mark.parametrize('kw', [
+    dict(use_qk_l2norm_in_kernel=True),
+    dict(use_gate_in_kernel=True),
+    dict(use_gate_in_kernel=True, dt_bias=None),
+    dict(use_beta_sigmoid_in_kernel=True),
+    dict(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True),
+    dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True),
+])
+def test_each_prologue_inside_the_kernels_packed_input(kw):
+    """l2 normalisation of q and k, gate activation and beta sigmoid are applied by the kernels
+    (as row factors / on the fly); each alone and all together must meet the oracle, here on packed
+    sequences with grouped value heads and ragged tails."""
+    cu = [0, 70, 71, 400, 1000]
+    T, N, H, HV, D = cu[-1], len(cu) - 1, 2, 4, 128
+    gen = torch.Generator().manual_seed(17)
+    q, k = 3 * torch.randn(1, T, H, D, generator=gen).bfloat16(), 0.3 * torch.randn(1, T, H, D, generator=gen).bfloat16()
+    if not kw.get('use_qk_l2norm_in_kernel'):
+        q, k = F.normalize(q.float(), dim=-1).bfloat16(), F.normalize(k.float(), dim=-1).bfloat16()
+    v = torch.randn(1, T, HV, D, generator=gen).bfloat16()
+    g = torch.randn(1, T, HV, generator=gen)
+    if not kw.get('use_gate_in_kernel'):
+        g = F.logsigmoid(g) / 4
+    beta = torch.randn(1, T, HV, generator=gen)
+    if not kw.get('use_beta_sigmoid_in_kernel'):
+        beta = torch.sigmoid(beta)
+    h0 = 0.5 * torch.randn(N, HV, D, D, generator=gen)
+    kw = dict(kw)
+    ref_kw, run_kw = dict(kw), dict(kw)
+    if kw.get('use_gate_in_kernel'):
+        A_log = 0.3 * torch.randn(HV, generator=gen)
+        dt_bias = None if 'dt_bias' in kw else 0.3 * torch.randn(HV, generator=gen)
+        ref_kw.update(A_log=A_log, dt_bias=dt_bias)
+        run_kw.update(A_log=A_log.cuda(), dt_bias=None if dt_bias is None else dt_bias.cuda())
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, **ref_kw)
+    o, ht = _run(q, k, v, g, beta, h0, cu, **run_kw)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 def test_outputs_fully_written_and_deterministic():
     """Two runs agree bit for bit and every output element is written (no NaN survives from
     poisoned allocations: the workspace and outputs come from torch.empty)."""
