@@ -390,7 +390,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             for (int nn = 0; nn < NN; ++nn)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float x = v_zero ? 0.f : to_f32(vv[tt][nn][r]);
+                    const float x = (!FULL && v_zero) ? 0.f : to_f32(vv[tt][nn][r]);      // (full runs always have their v)
                     Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(x - eg[r] * ks[tt][nn][r]);
                 }
         };
