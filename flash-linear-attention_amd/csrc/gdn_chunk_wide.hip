@@ -394,31 +394,46 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                     Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(x - eg[r] * ks[tt][nn][r]);
                 }
         };
-        auto TX = [&](int tt) {                 // v_new = Xb D (lower triangular), plain and decayed to the chunk end
-            const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
+        // The matrix part and the conversion of its result sit in different regions: a vector
+        // instruction that needs the result of a matrix instruction issued just before it stalls
+        // for the whole latency of the matrix pipeline.
+        f32x4 vn[4][NN], oacc[4][NN];
+        auto TXa = [&](int tt) {                // v_new = Xb D (lower triangular)
 #pragma unroll
             for (int nn = 0; nn < NN; ++nn) {
-                f32x4 vn = {0.f, 0.f, 0.f, 0.f};
+                vn[tt][nn] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) vn = Mma<T>::run(ax[tt][sp2], Db[sp2][nn], vn);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    Vn[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[r]);
-                    Vg[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[r] * dec[r]);
-                }
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) vn[tt][nn] = Mma<T>::run(ax[tt][sp2], Db[sp2][nn], vn[tt][nn]);
             }
         };
-        auto TP = [&](int tt) {                 // o^T = scale 2^G (q S)^T + (P v_new)^T: 4 consecutive value columns of a token row per lane
+        auto TXb = [&](int tt) {                // ... as B operands: plain, and decayed to the chunk end
+            const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
+#pragma unroll
+            for (int nn = 0; nn < NN; ++nn)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    Vn[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[tt][nn][r]);
+                    Vg[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(vn[tt][nn][r] * dec[r]);
+                }
+        };
+        auto TPa = [&](int tt) {                // o^T = scale 2^G (q S)^T + (P v_new)^T
             if constexpr (FULL) {
                 const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
 #pragma unroll
                 for (int nn = 0; nn < NN; ++nn) {
-                    f32x4 acc = ao[tt][nn] * gam;
+                    oacc[tt][nn] = ao[tt][nn] * gam;
 #pragma unroll
-                    for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) acc = Mma<T>::run(Vn[sp2][nn], ap[tt][sp2], acc);
+                    for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) oacc[tt][nn] = Mma<T>::run(Vn[sp2][nn], ap[tt][sp2], oacc[tt][nn]);
+                }
+            }
+        };
+        auto TPb = [&](int tt) {                // ... to the output tile: 4 consecutive value columns of a token row per lane
+            if constexpr (FULL) {
+#pragma unroll
+                for (int nn = 0; nn < NN; ++nn) {
                     V4 o4;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(acc[r]);
+                    for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(oacc[tt][nn][r]);
                     *(V4*)(otile + (16 * tt + c16) * OT_PITCH + (16 * (NN * w + nn) + 4 * g) * 2) = o4;
                 }
             }
@@ -457,10 +472,10 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             if (f == 7) FX(1);
             if (f == 8) TD(0);
             if (f == 9) { TD(1); FP(0); }
-            if (f == 10) { TX(0); FP(1); }
-            if (f == 11) { TX(1); FV(2); }
-            if (f == 12) { TP(0); FV(3); }
-            if (f == 13) { TP(1); FX(2); }
+            if (f == 10) { TXa(0); TXa(1); FP(1); }
+            if (f == 11) { TXb(0); TXb(1); FV(2); }
+            if (f == 12) { TPa(0); TPa(1); FV(3); }
+            if (f == 13) { TPb(0); TPb(1); FX(2); }
             if (f == 14) { FX(3); FK(0, 0); FK(0, 1); }
             if (f == 15) { FK(0, 2); FK(0, 3); }
             fence();
@@ -477,14 +492,15 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         // ---- state update from tiles 0, 1, with the tail of tiles 2, 3 ----
         U(0, 0); U(0, 1); TD(2); FK(0, 4); FK(0, 5); fence();
         U(0, 2); U(0, 3); TD(3); FK(0, 6); FK(0, 7); FP(2); fence();
-        U(0, 4); U(0, 5); TX(2); FK(1, 0); FK(1, 1); FP(3); fence();
-        U(0, 6); U(0, 7); TX(3); FK(1, 2); FK(1, 3); fence();
-        TP(2); FK(1, 4); FK(1, 5); fence();
-        TP(3); FK(1, 6); FK(1, 7); fence();
+        U(0, 4); U(0, 5); TXa(2); TXa(3); FK(1, 0); FK(1, 1); FP(3); fence();
+        U(0, 6); U(0, 7); TXb(2); TXb(3); FK(1, 2); FK(1, 3); fence();
+        // ... and the first half of the update from tiles 2, 3
+        U(1, 0); U(1, 1); TPa(2); TPa(3); FK(1, 4); FK(1, 5); fence();
+        U(1, 2); U(1, 3); TPb(2); TPb(3); FK(1, 6); FK(1, 7); fence();
         lds_barrier();                                          // B1: q, v, record of this stage are free
-        // ---- state update from tiles 2, 3 ----
+        // ---- rest of the state update from tiles 2, 3 ----
 #pragma unroll
-        for (int m = 0; m < 8; ++m) U(1, m);
+        for (int m = 4; m < 8; ++m) U(1, m);
         fence();
         lds_barrier();                                          // B2: k of this stage is free, the other stage is complete
     };
