@@ -14,28 +14,44 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
         if (rc) return rc;
     }
     if (!(stages & STAGE_SCAN)) return GDN_OK;
-    // One workgroup per (sequence, head) walks the chunks of the sequence ("wide").  With few
-    // such pairs and long dense sequences, time is cut into segments instead so that every CU
-    // has a workgroup: two passes over 1/nseg of the chunks each plus a small merge.
+    // One workgroup per (sequence, head) walks the chunks of the sequence.  With few such runs and
+    // long dense sequences, time is cut into segments instead so that every CU has a workgroup: two
+    // passes over 1/nseg of the chunks each plus a small merge.
+    // Either way a workgroup can also carry two runs that read the same k rows (two value heads of
+    // a q/k head; in pass 1 the S and M runs of one head).  That halves the number of workgroups and
+    // runs a pair about 1.25 times as fast as two single runs one after the other, so it pays as soon
+    // as the single runs would not all fit on the chip at once.
+    const int64_t G = p.HV / p.H;
     const bool dense = p.cu_seqlens == nullptr;
     int nseg = 0;
     if (dense && p.NH > 0) {
         nseg = (int)std::min<int64_t>((256 + p.NH / 2) / p.NH, p.NT / 4);
-        if ((int64_t)nseg * p.NH > SEG_SLOTS_MAX || (int64_t)nseg * p.NH > (num_chunks * p.HV + 3) / 4) nseg = 0;
+        while (nseg > 0 && ((int64_t)nseg * p.NH > SEG_SLOTS_MAX || (int64_t)nseg * p.NH > (num_chunks * p.HV + 3) / 4)) --nseg;
     }
     bool segments = nseg >= 3;           // two passes of NT/nseg steps each must beat one pass of NT steps
     if (p.flags & GDN_FLAG_SCAN_WIDE) segments = false;
     if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
-    if (!segments) return launch_scan_wide<T>(p, stream);
-    SegmentPlan sp;
-    sp.kind = 0;
+    const bool no_pair = p.flags & GDN_FLAG_SCAN_NO_PAIR, force_pair = p.flags & GDN_FLAG_SCAN_PAIR;
+    auto use_pair = [&](bool possible, int64_t single_workgroups) {
+        return possible && !no_pair && (force_pair || single_workgroups > 256);
+    };
+    SegmentPlan sp = {};
+    if (!segments) {
+        sp.kind = WIDE_WHOLE;
+        return use_pair(G % 2 == 0, p.NH) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
+    }
     sp.nseg = nseg;
     sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
     const size_t slots = (size_t)p.NH * nseg;
     sp.sloc = p.ws.Seg;
     sp.mseg = p.ws.Seg + slots * 16384;
     sp.sin = p.ws.Seg + 2 * slots * 16384;
-    return launch_scan_segments<T>(p, sp, stream);
+    int rc;
+    sp.kind = WIDE_PASS1;
+    if ((rc = use_pair(true, 2 * p.NH * (nseg - 1)) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream))) return rc;
+    if ((rc = launch_segment_merge(p, sp, stream))) return rc;
+    sp.kind = WIDE_PASS2;
+    return use_pair(G % 2 == 0, p.NH * nseg) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
 }
 
 }  // namespace gdn
@@ -60,6 +76,7 @@ static int chunk_entry(
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "%s: non-positive dimension", who);
     GDN_CHECK_ARG(!dt_bias || A_log, GDN_ERR_INVALID, "%s: dt_bias without A_log", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_SCAN_NO_PAIR) || !(flags & GDN_FLAG_SCAN_PAIR), GDN_ERR_INVALID, "%s: GDN_FLAG_SCAN_PAIR and GDN_FLAG_SCAN_NO_PAIR exclude each other", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
     GDN_CHECK_ARG(K == 128 && V == 128, GDN_ERR_UNSUPPORTED, "%s: only K = V = 128 is built (got K=%lld V=%lld)", who,
                   (long long)K, (long long)V);

@@ -106,6 +106,30 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// kind of run
+constexpr int WIDE_WHOLE = 0;     // whole sequences, user h0 -> o, ht
+constexpr int WIDE_PASS1 = 1;     // per segment: S_loc / M into the segment buffers
+constexpr int WIDE_PASS2 = 2;     // per segment: from merged S_in -> o (last segment also ht)
+
+// Asynchronous copy of 64 x 16 bytes from global memory straight into LDS: lane l fetches the
+// 16 bytes at gbase + voff (gbase wave-uniform, voff per lane) and they land at the
+// wave-uniform LDS byte offset `lds_off` + 16 l.  Issued from inline assembly on purpose: the
+// compiler then keeps no account of it, and completion is awaited explicitly with s_waitcnt
+// vmcnt before the barrier that publishes the data.
+__device__ __forceinline__ void gather_1k_to_lds(const char* gbase, uint32_t voff, uint32_t lds_off) {
+    lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make them scalars
+    const uint64_t g = (uint64_t)gbase;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+    const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(voff), "s"(gs));
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm_at_most() {
+    static_assert(N >= 0 && N <= 63, "the vector-memory counter has 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 // 16x16 product of fp32 matrices held in LDS on the fp32 matrix cores:
 // C = A[16 x 4*nk] * B[4*nk x 16]; result in C/D layout.
 __device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* B, int ldb, int nk, int c16, int g) {
@@ -135,7 +159,10 @@ struct SegmentPlan {
 
 // launchers defined next to their kernels
 template <typename T> int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream);
-template <typename T> int launch_scan_wide(const ChunkParams& p, hipStream_t stream);
-template <typename T> int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
+// Sequential stage; sp.kind selects whole sequences, pass 1 or pass 2.  Four compute waves and one
+// run per workgroup (gdn_chunk_wide.hip) or eight compute waves and two runs (gdn_chunk_pair.hip).
+template <typename T> int launch_wide(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
+template <typename T> int launch_pair(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
+int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
 
 }  // namespace gdn

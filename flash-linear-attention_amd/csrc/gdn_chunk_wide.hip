@@ -55,30 +55,6 @@ constexpr int WIDE_NN = 2;                        // 16-column tiles per compute
 constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
 
-// kind of run
-constexpr int WIDE_WHOLE = 0;     // whole sequences, user h0 -> o, ht
-constexpr int WIDE_PASS1 = 1;     // per segment: S_loc / M into the segment buffers
-constexpr int WIDE_PASS2 = 2;     // per segment: from merged S_in -> o (last segment also ht)
-
-// Asynchronous copy of 64 x 16 bytes from global memory straight into LDS: lane l fetches the
-// 16 bytes at gbase + voff (gbase wave-uniform, voff per lane) and they land at the
-// wave-uniform LDS byte offset `lds_off` + 16 l.  Issued from inline assembly on purpose: the
-// compiler then keeps no account of it, and completion is awaited explicitly with s_waitcnt
-// vmcnt before the barrier that publishes the data.
-__device__ __forceinline__ void gather_1k_to_lds(const char* gbase, uint32_t voff, uint32_t lds_off) {
-    lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make them scalars
-    const uint64_t g = (uint64_t)gbase;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
-    const uint64_t gs = ((uint64_t)hi << 32) | lo;
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(voff), "s"(gs));
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vm_at_most() {
-    static_assert(N >= 0 && N <= 63, "the vector-memory counter has 6 bits");
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
 template <typename T, bool FULL>
 __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParams p, SegmentPlan sp) {
     typedef typename Mma<T>::V8 V8;
@@ -610,40 +586,33 @@ static int launch_wide_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t
     return check_launch("gdn_chunk_wide_kernel");
 }
 
+// sp.kind selects the work (whole sequences, pass 1 or pass 2 of the segment-parallel evaluation)
 template <typename T>
-int launch_scan_wide(const ChunkParams& p, hipStream_t stream) {
-    SegmentPlan sp = {};
-    sp.kind = WIDE_WHOLE;
-    sp.nseg = 1;
-    sp.seg_chunks = 1 << 30;
+int launch_wide(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
     const int64_t G = p.HV / p.H;
-    return launch_wide_kind<T, true>(p, sp, (p.N * p.H + 7) / 8 * 8 * G, stream);
-}
-
-template <typename T>
-int launch_scan_segments(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
-    int rc;
-    sp.kind = WIDE_PASS1;
-    const int64_t G = p.HV / p.H;
-    if ((rc = launch_wide_kind<T, false>(p, sp, (p.N * p.H * (sp.nseg - 1) + 7) / 8 * 8 * 2 * G, stream))) return rc;
-    if (sp.nseg > 1) {
-        static bool attr_done = false;
-        if (!attr_done) {
-            if (hipFuncSetAttribute((const void*)gdn_segment_merge_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)MERGE_SMEM) != hipSuccess)
-                return check_launch("hipFuncSetAttribute(merge)");
-            attr_done = true;
-        }
-        hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)(p.NH * 8)), dim3(256), MERGE_SMEM, stream, sp);
-        if ((rc = check_launch("gdn_segment_merge_kernel"))) return rc;
+    if (sp.kind == WIDE_PASS1)
+        return launch_wide_kind<T, false>(p, sp, (p.N * p.H * (sp.nseg - 1) + 7) / 8 * 8 * 2 * G, stream);
+    if (sp.kind == WIDE_WHOLE) {
+        sp.nseg = 1;
+        sp.seg_chunks = 1 << 30;
+        return launch_wide_kind<T, true>(p, sp, (p.N * p.H + 7) / 8 * 8 * G, stream);
     }
-    sp.kind = WIDE_PASS2;
     return launch_wide_kind<T, true>(p, sp, (p.N * p.H * sp.nseg + 7) / 8 * 8 * G, stream);
 }
 
-template int launch_scan_wide<bf16_t>(const ChunkParams&, hipStream_t);
-template int launch_scan_wide<f16_t>(const ChunkParams&, hipStream_t);
-template int launch_scan_segments<bf16_t>(const ChunkParams&, SegmentPlan, hipStream_t);
-template int launch_scan_segments<f16_t>(const ChunkParams&, SegmentPlan, hipStream_t);
+int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (hipFuncSetAttribute((const void*)gdn_segment_merge_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)MERGE_SMEM) != hipSuccess)
+            return check_launch("hipFuncSetAttribute(merge)");
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)(p.NH * 8)), dim3(256), MERGE_SMEM, stream, sp);
+    return check_launch("gdn_segment_merge_kernel");
+}
+
+template int launch_wide<bf16_t>(const ChunkParams&, SegmentPlan, hipStream_t);
+template int launch_wide<f16_t>(const ChunkParams&, SegmentPlan, hipStream_t);
 
 }  // namespace gdn

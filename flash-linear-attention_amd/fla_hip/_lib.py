@@ -28,6 +28,8 @@ FLAG_CU_INT32 = 1 << 5
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
 FLAG_SEQ_ORDER = 1 << 19
+FLAG_SCAN_NO_PAIR = 1 << 20
+FLAG_SCAN_PAIR = 1 << 21
 
 # name -> (restype, argtypes); one entry per declaration in include/gdn_hip.h
 SIGNATURES = {

@@ -30,8 +30,13 @@ from fla_hip.utils import input_guard
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
 # the chunk size (only rounding does), so chunk_size 16 and 32 are accepted and run with 64.
 _KERNEL_CHUNK = 64
-# FLA_HIP_SCAN_MODE=wide|segments forces one form of the sequential kernel (default: automatic)
-_SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS}
+# FLA_HIP_SCAN_MODE forces one form of the sequential kernel (default: automatic): whole sequences
+# ('wide') or time cut into segments, each with one run per workgroup ('-single') or two ('-pair')
+_SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS,
+                    'single': _lib.FLAG_SCAN_NO_PAIR, 'pair': _lib.FLAG_SCAN_PAIR}
+for _form in ('wide', 'segments'):
+    for _runs in ('single', 'pair'):
+        _SCAN_MODE_FLAGS[f'{_form}-{_runs}'] = _SCAN_MODE_FLAGS[_form] | _SCAN_MODE_FLAGS[_runs]
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 

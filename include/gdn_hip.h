@@ -46,6 +46,8 @@ extern "C" {
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
 #define GDN_FLAG_SCAN_SEGMENTS  (1u << 18) /* time cut into segments (dense input, >= 8 chunks) */
 #define GDN_FLAG_SEQ_ORDER      (1u << 19) /* chunk_offsets carries N more entries (see there)   */
+#define GDN_FLAG_SCAN_NO_PAIR   (1u << 20) /* always one run per workgroup                      */
+#define GDN_FLAG_SCAN_PAIR      (1u << 21) /* two runs per workgroup wherever two can share k rows */
 
 /* Library ABI version (bumped on any signature change). */
 int gdn_hip_abi_version(void);

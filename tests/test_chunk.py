@@ -56,15 +56,16 @@ def test_chunk_vs_oracle(B, T, H, HV, D, gate_div, with_h0, dtype):
     _check('ht', ref_ht, ht)
 
 
-@pytest.mark.parametrize('mode', ['wide', 'segments'])
+@pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'wide-pair', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
     (2, 1000, 2, 4, True, False),
     (1, 2100, 2, 2, True, True),          # ragged tail, V-first state layout
     (3, 512, 1, 2, False, False),
 ])
 def test_every_form_of_the_sequential_stage(monkeypatch, mode, B, T, H, HV, with_h0, vfirst):
-    """The two forms of the sequential stage (one workgroup per head for the whole sequence, time
-    segments with fp32 merge) are interchangeable: each must meet the oracle on its own."""
+    """The forms of the sequential stage (one workgroup for the whole sequence or time segments
+    with fp32 merge; two runs per workgroup or one) are interchangeable: each must meet the
+    oracle on its own."""
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
     q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, 128, 128, seed=21, gate_div=16.0,
                                          h0_std=0.5 if with_h0 else None, dtype=torch.bfloat16)
@@ -78,7 +79,7 @@ def test_every_form_of_the_sequential_stage(monkeypatch, mode, B, T, H, HV, with
     _check('ht', ref_ht, ht)
 
 
-@pytest.mark.parametrize('mode', ['wide', 'auto'])
+@pytest.mark.parametrize('mode', ['auto', 'single', 'pair'])
 def test_varlen_every_form(monkeypatch, mode):
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
     cu = [0, 1, 100, 101, 300, 1200, 2000]
@@ -110,7 +111,7 @@ def test_against_token_recurrence_and_decode_handoff():
     ([0, 15, 100, 300, 1200, 2000], 2, 4, 64),
 ])
 @pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
-@pytest.mark.parametrize('mode', ['wide'])
+@pytest.mark.parametrize('mode', ['wide-single', 'wide-pair'])
 def test_varlen_vs_oracle_and_bit_exact_ownership(monkeypatch, cu, H, HV, D, idx_dtype, mode):
     # the form of the sequential kernel is pinned so that the packed call and the single-sequence
     # calls run the very same code: any difference is then a token or state given to the wrong sequence

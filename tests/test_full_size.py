@@ -67,15 +67,17 @@ def test_long_sequence_properties():
     ob, sb = op(dq[:, h:], dk[:, h:], dv[:, h:], dg[:, h:], db[:, h:], initial_state=sa, output_final_state=True)
     _check('o (two calls)', o.float().cpu(), torch.cat([oa, ob], 1))
     _check('ht (two calls)', ht.float().cpu(), sb)
-    # (3) a forced single pass over the sequence (one workgroup per head) agrees with the segmented evaluation
+    # (3) every other form of the sequential stage agrees with the automatic choice: a single pass over
+    # the sequence, and segments with one or two runs per workgroup throughout
     import os
-    os.environ['FLA_HIP_SCAN_MODE'] = 'wide'
-    try:
-        ow, hw = op(dq, dk, dv, dg, db, initial_state=ds, output_final_state=True)
-    finally:
-        del os.environ['FLA_HIP_SCAN_MODE']
-    _check('o (single pass)', o.float().cpu(), ow)
-    _check('ht (single pass)', ht.float().cpu(), hw)
+    for mode in ('wide-single', 'wide-pair', 'segments-single', 'segments-pair'):
+        os.environ['FLA_HIP_SCAN_MODE'] = mode
+        try:
+            ow, hw = op(dq, dk, dv, dg, db, initial_state=ds, output_final_state=True)
+        finally:
+            del os.environ['FLA_HIP_SCAN_MODE']
+        _check(f'o ({mode})', o.float().cpu(), ow)
+        _check(f'ht ({mode})', ht.float().cpu(), hw)
 
 
 def test_packed_65536_tokens_in_32_sequences():
