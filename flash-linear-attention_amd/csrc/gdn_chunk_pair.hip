@@ -168,16 +168,18 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
             gather_1k_to_lds(base, __umul24(row, rowB_v) + v_cb, lds0 + PR_V + w * 4096 + b * 1024);
         }
     };
-    auto issue_rec = [&](int64_t c, int stage, int part) {                           // 2 parts of 2 operations (1 for a state-only run)
+    // The record of (chunk, value head).  A full run needs all 13 KB, a quarter per wave of the team.  A
+    // state-only run needs Xb and the tables (pieces 0..5 and 12), and its two teams work on the same
+    // value head: they share one copy (in the area of team 0), one piece per wave.
+    auto issue_rec = [&](int64_t c, int stage, int part) {                           // 2 parts of 2 operations (state-only: 1 part of 1)
         const char* rec = p.ws.Rec + ((boh + c) * HV + hv) * REC_BYTES;
-        const uint32_t to = lds0 + PR_REC + (tm * 2 + stage) * (uint32_t)REC_BYTES;
+        const uint32_t to = lds0 + PR_REC + ((FULL ? tm : 0) * 2 + stage) * (uint32_t)REC_BYTES;
         auto piece = [&](int j) { gather_1k_to_lds(rec + j * 1024, lane * 16, to + j * 1024); };
         if constexpr (FULL) {
             if (part == 0) { piece(cw); piece(cw + 4); }
             else { piece(cw + 8); piece(cw == 0 ? 12 : cw); }                         // (waves 1..3 fetch one piece twice: equal counts)
         } else {
-            if (part == 0) piece(cw);
-            else piece(cw < 2 ? cw + 4 : cw == 2 ? 12 : cw);                          // Xb (0..5) and the tables (12)
+            if (part == 0) piece(w < 6 ? w : w == 6 ? 12 : 0);                        // (wave 7 fetches piece 0 again: equal counts)
         }
     };
     // everything a barrier publishes, 8 (4) operations, in four parts so that the waves do not all
@@ -188,18 +190,20 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         if (part >= 2) issue_rec(c, stage, part - 2);
     };
     // number of operations a wave issues between ...
-    // (per step, in order: shared 8 (4), in the first four regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
+    // (per step, in order: shared 8 (3), in the first four regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
     constexpr int N_AFTER_SHARED = FULL ? 8 : 4;      // the shared copies of a step and the barrier at its end
-    constexpr int N_AFTER_VLO = FULL ? 14 : 6;        // the first half of v and its use in the next step
-    constexpr int N_AFTER_VHI = FULL ? 12 : 6;        // the second half of v and its use in the next step
+    constexpr int N_AFTER_VLO = FULL ? 14 : 5;        // the first half of v and its use in the next step
+    constexpr int N_AFTER_VHI = FULL ? 12 : 5;        // the second half of v and its use in the next step
 
     if (nsteps > 0 && !active) {
-        // a team with nothing to compute still fetches its share of k
+        // a team with nothing to compute still fetches its share of k and of the record
         issue_kq((const T*)p.k, it0, lds0 + PR_K);
+        issue_rec(it0, 0, 0);
         wait_vm_at_most<0>();
         lds_barrier();
         for (int64_t i = 0; i < nsteps; ++i) {
             issue_kq((const T*)p.k, min(it0 + i + 1, lastc), lds0 + PR_K + (int)((i + 1) & 1) * 16384);
+            issue_rec(min(it0 + i + 1, lastc), (int)((i + 1) & 1), 0);
             wait_vm_at_most<0>();
             lds_barrier();
         }
@@ -253,7 +257,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         const V8* sQ = (const V8*)(smem + PR_Q + cur * 16384);
         const T* sV = (const T*)(smem + PR_V + w * 4096);
         const T* sKt = (const T*)kbuf;
-        const char* rec = smem + PR_REC + (tm * 2 + cur) * REC_BYTES;
+        const char* rec = smem + PR_REC + ((FULL ? tm : 0) * 2 + cur) * REC_BYTES;
         const V8* sX = (const V8*)(rec + REC_X);
         const V8* sP = (const V8*)(rec + REC_P);
         const float* sTab = (const float*)(rec + REC_TAB);

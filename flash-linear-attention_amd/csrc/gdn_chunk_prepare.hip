@@ -22,7 +22,7 @@ constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
 inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + 2 * CH * 4 + (size_t)group * 2 * CH * 4; }
 
 template <typename T>
-__global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p) {
+__global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p) {
     typedef typename Mma<T>::V8 V8;
     extern __shared__ __align__(16) char smem[];
     T* k_nat = (T*)smem;                        // [64][NP] keys, token-major; reused for L once the raw products exist
@@ -157,29 +157,11 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
         }
     }
     __syncthreads();     // k and q are dead from here on: their bytes become L and X
+    // P of every value head first: the raw q K^T tiles then leave the registers before the inversion needs them
     for (int m = 0; m < G; ++m) {
         const int hv = h * G + m;
         const float* sG = sGB + (2 * m) * CH;
-        const float* sB = sG + CH;
         char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
-        // ---- L tiles of row-tile w (gated, beta-scaled, strictly lower) ----
-        {
-            const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g);
-            const f32x4 bi = *(const f32x4*)(sB + 16 * w + 4 * g) * *(const f32x4*)(sRN + 16 * w + 4 * g);
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                const int j = 16 * tj + c16;
-                const float gj = sG[j], nj = sRN[j];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
-                    const float val = (i > j && tj <= w) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
-                    sL[i * LP + j] = val;
-                    if (tj == w) sLd[(w * 16 + c16) * 16 + 4 * g + r] = val;
-                }
-            }
-        }
         // ---- P^T tiles of query tile tt (gated, lower incl. diagonal), straight to memory ----
         {
             const int t = 16 * tt + c16;
@@ -201,6 +183,30 @@ __global__ __launch_bounds__(256, 3) void gdn_chunk_prepare_kernel(ChunkParams p
                     }
                 }
                 *(V8*)(pf + (p_slot(tt, sp) * 64 + lane) * 8) = frag;
+            }
+        }
+    }
+    for (int m = 0; m < G; ++m) {
+        const int hv = h * G + m;
+        const float* sG = sGB + (2 * m) * CH;
+        const float* sB = sG + CH;
+        char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
+        // ---- L tiles of row-tile w (gated, beta-scaled, strictly lower) ----
+        {
+            const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g);
+            const f32x4 bi = *(const f32x4*)(sB + 16 * w + 4 * g) * *(const f32x4*)(sRN + 16 * w + 4 * g);
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                const int j = 16 * tj + c16;
+                const float gj = sG[j], nj = sRN[j];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
+                    const float val = (i > j && tj <= w) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
+                    sL[i * LP + j] = val;
+                    if (tj == w) sLd[(w * 16 + c16) * 16 + 4 * g + r] = val;
+                }
             }
         }
         __syncthreads();     // L complete
