@@ -124,7 +124,8 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     t_prep = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e-3
     t_scan = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e-3
     units = tokens * w['HV']
-    scan_name = 'gdn_chunk_fwd_scan: gdn_chunk_wide_kernel (+ gdn_segment_merge_kernel when time is cut into segments)'
+    scan_name = ('gdn_chunk_fwd_scan: gdn_chunk_wide_kernel / gdn_chunk_pair_kernel '
+                 '(+ gdn_segment_merge_kernel when time is cut into segments)')
     dom = (scan_name, F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_fwd_prepare: gdn_chunk_prepare_kernel', F_PREP, t_prep)
     achieved = units * dom[1] / dom[2] / 1e12
     roofline = dict(bound='mfma', achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit='TFLOP/s',

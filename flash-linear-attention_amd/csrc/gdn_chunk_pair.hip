@@ -129,6 +129,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     // finite and is multiplied by the zero columns of Xb, the zero rows of v_new and the causal
     // zeros of P.
     // =====================================================================================
+    const bool vz = __builtin_amdgcn_readfirstlane((int)v_zero) != 0;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     const uint32_t rowB_qk = (uint32_t)H * 256, rowB_v = (uint32_t)HV * 256;
     // k and q tiles in LDS: 64 token rows x 256 B as 16 blocks of 4 rows (1 KB, one copy each).  In block j
@@ -286,6 +287,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         V4 vv[4][NN];
         V8 ax[4][2], ap[4][2];
         auto FV = [&](int tt) {
+            if (!FULL && vz) return;
 #pragma unroll
             for (int nn = 0; nn < NN; ++nn) vv[tt][nn] = Mma<T>::tr_read(sV + tt * 512 + v_tr + 4 * nn);
         };
@@ -308,13 +310,18 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         V8 Db[2][NN], Vn[2][NN], Vg[2][NN];
         auto TD = [&](int tt) {
             const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
+            if (!FULL && vz) {                  // a transition run has v = 0 (scalar branch: nothing is selected per element)
 #pragma unroll
-            for (int nn = 0; nn < NN; ++nn)
+                for (int nn = 0; nn < NN; ++nn)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float x = (!FULL && v_zero) ? 0.f : to_f32(vv[tt][nn][r]);
-                    Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(x - eg[r] * ks[tt][nn][r]);
-                }
+                    for (int r = 0; r < 4; ++r) Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(-eg[r] * ks[tt][nn][r]);
+            } else {
+#pragma unroll
+                for (int nn = 0; nn < NN; ++nn)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        Db[tt >> 1][nn][(tt & 1) * 4 + r] = from_f32<T>(to_f32(vv[tt][nn][r]) - eg[r] * ks[tt][nn][r]);
+            }
         };
         f32x4 vn[4][NN], oacc[4][NN];
         auto TXa = [&](int tt) {
