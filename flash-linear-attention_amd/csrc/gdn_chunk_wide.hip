@@ -505,20 +505,26 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 }
 
 // S_in[j+1] = M_j S_in[j] + S_loc,j for j = 1 .. nseg-2, with S_in[1] = S_loc,0 (the run of segment 0
-// started from the true initial state).  fp32 throughout (fp32 matrix cores): one workgroup
-// per (sequence, head, slab of 16 value columns); M_j is staged in LDS.
-constexpr int MP = 132;                            // pitch of the staged M rows (floats)
-constexpr size_t MERGE_SMEM = (128 * MP + 128 * 16) * 4;
+// started from the true initial state).  fp32 throughout (fp32 matrix cores): one workgroup per
+// (sequence, head, slab of 16 value columns); M_j is staged in LDS, the next one travels in registers
+// meanwhile (fetched with consecutive lanes on consecutive addresses: read straight into the operand
+// registers, where neighbouring lanes hold different rows, the same bytes take longer).  The 8 slabs
+// of a head sit on one XCD (block index mod 8), so that M_j comes from HBM once.
+// Contraction indices of the 16x16x4 products: step e of block q uses {16q + 4g + e}, so a lane
+// reads its four values of A (a row of M) and of B (a column of S, kept transposed) as one 16-byte
+// LDS read each.
+constexpr int MP = 132;                            // pitch of the staged rows (floats): conflict-free 16-byte reads
+constexpr size_t MERGE_SMEM = (128 * MP + 16 * MP) * 4;
 
-__global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp) {
+__global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, int64_t NH) {
     extern __shared__ __align__(16) char smem[];
-    float* sM = (float*)smem;                      // [128][MP]
-    float* sS = sM + 128 * MP;                     // [128][16] current S_in slab
+    float* sM = (float*)smem;                      // [128 i][MP] M_j
+    float* sSt = sM + 128 * MP;                    // [16 n][MP] current S_in slab, transposed
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t inh = blockIdx.x >> 3;
-    const int v0 = (int)(blockIdx.x & 7) * 16;
+    const int64_t inh = (int64_t)(blockIdx.x >> 6) * 8 + (blockIdx.x & 7);
+    if (inh >= NH) return;
+    const int v0 = (int)((blockIdx.x >> 3) & 7) * 16;
     const int nseg = sp.nseg;
-    // the next transition matrix travels in registers while the current one is multiplied
     f32x4 pre[16];
     auto fetch_M = [&](int j) {
         const float* M = sp.mseg + (inh * nseg + j) * 16384;
@@ -529,46 +535,51 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp) 
         }
     };
     if (nseg > 2) fetch_M(1);
-    // S_in[1] = S_loc,0
-    for (int idx = tid; idx < 128 * 16; idx += 256) {
-        const int kk = idx >> 4, c = idx & 15;
-        const float x = sp.sloc[(inh * nseg + 0) * 16384 + kk * 128 + v0 + c];
-        sS[idx] = x;
-        sp.sin[(inh * nseg + 1) * 16384 + kk * 128 + v0 + c] = x;
-    }
+    // this wave's part of a slab: key tiles 2w, 2w+1 in C/D layout (column c16, rows 4g .. 4g+3)
+    auto slab_rows = [&](const float* base, int j, f32x4 (&x)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) x[i][r] = base[(inh * nseg + j) * 16384 + (16 * (2 * w + i) + 4 * g + r) * 128 + v0 + c16];
+    };
+    auto publish = [&](int j, const f32x4 (&x)[2]) {          // x becomes S_in[j]: to the other waves (transposed) and to memory
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *(f32x4*)(sSt + c16 * MP + 16 * (2 * w + i) + 4 * g) = x[i];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sp.sin[(inh * nseg + j) * 16384 + (16 * (2 * w + i) + 4 * g + r) * 128 + v0 + c16] = x[i][r];
+        }
+    };
+    f32x4 x[2];
+    slab_rows(sp.sloc, 0, x);
+    publish(1, x);
     for (int j = 1; j + 1 < nseg; ++j) {
-        __syncthreads();                            // previous readers of sM are done; sS is complete
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int idx = tid + 256 * i;
             *(f32x4*)(sM + (idx >> 5) * MP + (idx & 31) * 4) = pre[i];
         }
         if (j + 2 < nseg) fetch_M(j + 1);
-        // this wave's rows of S_loc,j (C/D layout of key tiles 2w, 2w+1)
-        float sl[2][4];
+        f32x4 sl[2];
+        slab_rows(sp.sloc, j, sl);
+        __syncthreads();                            // M_j and S_in[j] are complete
+        f32x4 acc[2][2];                            // two accumulation chains per tile (even / odd blocks)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 2; ++i) acc[i][0] = acc[i][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                sl[i][r] = sp.sloc[(inh * nseg + j) * 16384 + (16 * (2 * w + i) + 4 * g + r) * 128 + v0 + c16];
-        __syncthreads();
-        // two independent accumulation chains per tile (halves of the contraction)
-        f32x4 acc[2][2];
+        for (int q = 0; q < 8; ++q) {
+            const f32x4 b = *(const f32x4*)(sSt + c16 * MP + 16 * q + 4 * g);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i) {
+                const f32x4 a = *(const f32x4*)(sM + (16 * (2 * w + i) + c16) * MP + 16 * q + 4 * g);
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh)
-                acc[i][hh] = mm16_f32(sM + (16 * (2 * w + i)) * MP + 64 * hh, MP, sS + 64 * hh * 16, 16, 16, c16, g);
-        __syncthreads();                            // all waves have read sS
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int kk = 16 * (2 * w + i) + 4 * g + r;
-                const float x = acc[i][0][r] + acc[i][1][r] + sl[i][r];
-                sS[kk * 16 + c16] = x;
-                sp.sin[(inh * nseg + j + 1) * 16384 + kk * 128 + v0 + c16] = x;
+                for (int e = 0; e < 4; ++e) acc[i][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], acc[i][q & 1], 0, 0, 0);
             }
+        }
+        __syncthreads();                            // all waves have read M_j and S_in[j]
+#pragma unroll
+        for (int i = 0; i < 2; ++i) x[i] = acc[i][0] + acc[i][1] + sl[i];
+        publish(j + 1, x);
     }
 }
 
@@ -608,7 +619,7 @@ int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t strea
             return check_launch("hipFuncSetAttribute(merge)");
         attr_done = true;
     }
-    hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)(p.NH * 8)), dim3(256), MERGE_SMEM, stream, sp);
+    hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)((p.NH + 7) / 8 * 64)), dim3(256), MERGE_SMEM, stream, sp, p.NH);
     return check_launch("gdn_segment_merge_kernel");
 }
 
