@@ -174,6 +174,11 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     const int tj = 2 * sp + half;
+                    if (tj > tt) {              // a key tile after the query tile: zero (tt is scalar: nothing is evaluated)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) frag[half * 4 + r] = from_f32<T>(0.f);
+                        continue;
+                    }
                     const f32x4 gj = *(const f32x4*)(sG + 16 * tj + 4 * g), nj = *(const f32x4*)(sRN + 16 * tj + 4 * g);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
@@ -198,12 +203,19 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
                 const int j = 16 * tj + c16;
+                if (tj > w) {                   // above the diagonal: zero (w is scalar: nothing is evaluated)
+                    if (w < 2 && tj >= 2) {     // only the block that will hold XT is ever read
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) sL[(16 * w + 4 * g + r) * LP + j] = 0.f;
+                    }
+                    continue;
+                }
                 const float gj = sG[j], nj = sRN[j];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int i = 16 * w + 4 * g + r;
                     // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
-                    const float val = (i > j && tj <= w) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
+                    const float val = (i > j) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
                     sL[i * LP + j] = val;
                     if (tj == w) sLd[(w * 16 + c16) * 16 + 4 * g + r] = val;
                 }
@@ -233,6 +245,17 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
 #pragma unroll
                 for (int i = 0; i < 16; ++i) sX[(b0 + i) * LP + b0 + c16] = x[i];
             }
+            // The merges below multiply by X blocks from the left AND from the right.  A right factor is read by
+            // columns, so it is kept transposed as well (one 16-byte LDS read then serves four matrix
+            // instructions): XT, the transposed top-left 32x32 block, lives in the unused upper-right
+            // block of L (zero so far), the transposed X22 in rows 16..31 of the unused upper-right block of X.
+            if (g == 1) {
+                float* xt = (w < 2) ? sL + (b0 + c16) * LP + 32 + b0 : sX + (16 + c16) * LP + 32;
+                if (w != 3) {
+#pragma unroll
+                    for (int i4 = 0; i4 < 4; ++i4) *(f32x4*)(xt + 4 * i4) = f32x4{x[4 * i4], x[4 * i4 + 1], x[4 * i4 + 2], x[4 * i4 + 3]};
+                }
+            }
             // zero tile above the diagonal inside each 32x32 diagonal block
             if ((w & 1) == 0) {
 #pragma unroll
@@ -240,33 +263,43 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             }
         }
         __syncthreads();
-        // ---- merge 16 -> 32: X[hi][lo] = -X[hi][hi] (L[hi][lo] X[lo][lo]); pairs (1,0) and (3,2) ----
-        // (waves 2,3 repeat the work of waves 0,1 so that the barriers stay block-uniform)
-        {
-            const int pr = w & 1, hi = 2 * pr + 1, lo = 2 * pr;
-            float* tmp = sX + 32 + 16 * pr;                     // rows 0..15 of the unused upper-right block
-            f32x4 y = mm16_f32(sL + (16 * hi) * LP + 16 * lo, LP, sX + (16 * lo) * LP + 16 * lo, LP, 4, c16, g);
-            if (w < 2) {
+        // 16x16 products on the fp32 matrix cores, contraction over 16*nq indices: A by rows (pitch LP),
+        // the right factor transposed (Bt[n][k], pitch LP); step e of block q uses the indices {16q + 4g + e}
+        auto mm_rt = [&](const float* A, const float* Bt, int nq) {
+            f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-                for (int r = 0; r < 4; ++r) tmp[(4 * g + r) * LP + c16] = y[r];
-            }
-            __syncthreads();
-            f32x4 z = mm16_f32(sX + (16 * hi) * LP + 16 * hi, LP, tmp, LP, 4, c16, g);
-            if (w < 2) {
+            for (int q = 0; q < 2; ++q) {
+                if (q >= nq) break;
+                const f32x4 a = *(const f32x4*)(A + c16 * LP + 16 * q + 4 * g);
+                const f32x4 bt = *(const f32x4*)(Bt + c16 * LP + 16 * q + 4 * g);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) sX[(16 * hi + 4 * g + r) * LP + 16 * lo + c16] = -z[r];
+                for (int e = 0; e < 4; ++e) acc[q] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], bt[e], acc[q], 0, 0, 0);
             }
+            return acc[0] + acc[1];
+        };
+        // ---- merge 16 -> 32: X[hi][lo] = -X[hi][hi] (L[hi][lo] X[lo][lo]); pairs (1,0) and (3,2) by waves 0 and 1.
+        // A wave only reads back what it has written itself (LDS operations of a wave execute in order), so
+        // there is no barrier between the two products; waves 2 and 3 leave their SIMDs to other workgroups.
+        if (w < 2) {
+            const int hi = 2 * w + 1, lo = 2 * w;
+            float* tmpT = sX + 32 + 16 * w;                     // rows 0..15 of the unused upper-right block: (L X)^T
+            const float* xlo_t = w ? sX + 16 * LP + 32 : sL + 32;
+            const f32x4 y = mm_rt(sL + (16 * hi) * LP + 16 * lo, xlo_t, 1);
+            *(f32x4*)(tmpT + c16 * LP + 4 * g) = y;
+            const f32x4 z = mm_rt(sX + (16 * hi) * LP + 16 * hi, tmpT, 1);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sX[(16 * hi + 4 * g + r) * LP + 16 * lo + c16] = -z[r];
+            if (w == 0) *(f32x4*)(sL + c16 * LP + 32 + 16 + 4 * g) = -z;             // X10 into XT
         }
         __syncthreads();
         // ---- merge 32 -> 64: X[32:64][0:32] = -X[32:64][32:64] (L[32:64][0:32] X[0:32][0:32]) ----
         {
             const int a = w >> 1, b = w & 1;
-            float* tmp2 = sX + 32;                              // rows 0..31, columns 32..63
-            f32x4 y = mm16_f32(sL + (32 + 16 * a) * LP, LP, sX + 16 * b, LP, 8, c16, g);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) tmp2[(16 * a + 4 * g + r) * LP + 16 * b + c16] = y[r];
+            float* tmp2T = sX + 32;                             // rows 0..31, columns 32..63: (L X)^T
+            const f32x4 y = mm_rt(sL + (32 + 16 * a) * LP, sL + (16 * b) * LP + 32, 2);
+            *(f32x4*)(tmp2T + (16 * b + c16) * LP + 16 * a + 4 * g) = y;
             __syncthreads();
-            f32x4 z = mm16_f32(sX + (32 + 16 * a) * LP + 32, LP, tmp2 + 16 * b, LP, 8, c16, g);
+            const f32x4 z = mm_rt(sX + (32 + 16 * a) * LP + 32, tmp2T + (16 * b) * LP, 2);
 #pragma unroll
             for (int r = 0; r < 4; ++r) sX[(32 + 16 * a + 4 * g + r) * LP + 16 * b + c16] = -z[r];
         }
