@@ -130,20 +130,6 @@ __device__ __forceinline__ void wait_vm_at_most() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// 16x16 product of fp32 matrices held in LDS on the fp32 matrix cores:
-// C = A[16 x 4*nk] * B[4*nk x 16]; result in C/D layout.
-__device__ __forceinline__ f32x4 mm16_f32(const float* A, int lda, const float* B, int ldb, int nk, int c16, int g) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < nk; ++kk) {
-        const float a = A[c16 * lda + 4 * kk + g];
-        const float b = B[(4 * kk + g) * ldb + c16];
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc, 0, 0, 0);
-    }
-    return acc;
-}
-
-
 // Segment-parallel evaluation of long dense sequences: every sequence is cut into `nseg`
 // segments of `seg_chunks` chunks; per (sequence, head, segment) the buffers hold 128x128 fp32
 // matrices ([K][V], K-first): sloc = state reached from a zero state (segment 0: from the true
