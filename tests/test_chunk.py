@@ -79,6 +79,42 @@ def test_every_form_of_the_sequential_stage(monkeypatch, mode, B, T, H, HV, with
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('mode', ['wide-pair', 'segments-pair'])
+@pytest.mark.parametrize('B,T,H,HV,dtype,gate_div', [
+    (1, 1991, 1, 4, torch.float16, 16.0),       # f16 (state rescaled every chunk), four value heads per q/k head, ragged tail
+    (2, 1300, 3, 6, torch.bfloat16, 1.0),       # strong decay: the lazy rescaling of the state fires
+    (1, 4160, 2, 2, torch.bfloat16, 16.0),      # one value head per q/k head: only pass 1 can pair its runs
+])
+def test_two_runs_per_workgroup(monkeypatch, mode, B, T, H, HV, dtype, gate_div):
+    """Shapes that stress what only the two-run kernel has: its own copies and counted waits over many
+    chunks, the masked output stores of a partial last chunk, teams with different value heads or with
+    the S / M runs of one head, and the idle team of the first segment."""
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, 128, 128, seed=5, gate_div=gate_div, h0_std=0.5, dtype=dtype)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    o, ht = _run(q, k, v, g, beta, h0)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    # rows past the end of a sequence are never written: guard rows behind the output keep their value
+    if B == 1:
+        from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
+        from fla_hip.ops.gated_delta_rule._common import ptr
+        dev = 'cuda'
+        Tm = T - 13
+        a = [x[:, :Tm].to(dev).contiguous() for x in (q, k, v, g, beta)]
+        call = ChunkLaunch(*a, 128 ** -0.5, h0.to(dev), True)
+        big = torch.full((1, Tm + 64, HV, 128), 7.0, dtype=dtype, device=dev)
+        args = list(call.args)
+        assert args[9] == ptr(call.o)
+        args[9] = ptr(big)
+        call.args = tuple(args)
+        call.run()
+        torch.cuda.synchronize()
+        assert torch.all(big[:, Tm:] == 7.0), 'tokens past the end of the sequence were written'
+        ref_m = O.chunk_gated_delta_rule(q[:, :Tm], k[:, :Tm], v[:, :Tm], g[:, :Tm], beta[:, :Tm], None, h0, True)[0]
+        _check('o (shorter call)', ref_m, big[:, :Tm])
+
+
 @pytest.mark.parametrize('mode', ['auto', 'single', 'pair'])
 def test_varlen_every_form(monkeypatch, mode):
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
