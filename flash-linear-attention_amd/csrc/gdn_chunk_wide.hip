@@ -36,9 +36,11 @@ namespace gdn {
 
 // LDS stage of one chunk.  q, k, v tiles: 64 token rows x 256 B as 16 blocks of 4 rows (1 KB, one
 // asynchronous copy each: 4 whole rows is the access shape the memory pipeline moves fastest).
-// Inside block j the 16-byte piece c of row 4j + r sits in slot 16*(c/4) + ((4*(j%4) + r + 4*(c%4)) & 15):
-// the rotation makes both the 16-byte operand reads (16 rows x one piece) and the LDS transpose
-// reads (4 rows x 4 pieces) of a 16-lane group touch 16 different slots modulo 16, i.e. all banks.
+// Inside block j the 16-byte piece c of row 4j + r sits in slot 16*(c/4) + 4r + ((c + j) & 3): four consecutive
+// lanes of a copy fetch 64 contiguous bytes of one row (neighbouring lanes on different rows would go through
+// the memory pipeline one lane at a time), and the rotation makes both the 16-byte operand reads (16 rows x
+// one piece) and the LDS transpose reads (4 rows x 4 pieces) of a 16-lane group touch 16 different slots
+// modulo 16, i.e. all banks.
 // q, v and the record are double-buffered (stage = chunk % 2); k, the one operand that is read until the
 // very end of a step, has three buffers (chunk % 3) so that its copy can be issued two steps ahead.
 constexpr int STG_Q = 0, STG_V = 16384, STG_REC = 32768;
@@ -159,8 +161,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 if (j < j0 || j >= j1) continue;
-                const int x = (c16 - 4 * (j & 3)) & 15;                     // this lane's slot holds piece c of row 4j + r
-                const int r = x & 3, c = 4 * g + (x >> 2);
+                const int r = c16 >> 2, c = 4 * g + ((c16 - j) & 3);        // this lane's slot holds piece c of row 4j + r
                 const int row = min(4 * j + r, valid - 1);
                 gather_1k_to_lds(base, (uint32_t)row * (uint32_t)(heads * 256) + 16 * c, lds_tile + j * 1024);
             }
@@ -295,13 +296,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // four 4-element runs addressed by lanes j, j+4, j+8, j+12 of its 16-lane group: this lane
     // addresses row i = c16/4 of the 4-row run and column group j = c16%4.
     const int tr_i = c16 >> 2, tr_j = c16 & 3;
-    const int a_off = (c16 >> 2) * 64 + ((c16 + 4 * g) & 15);                    // operand piece of row c16 of a t-tile: + tt*256 + 16*s  (16-byte units)
-    const int k_tr = (g * 64 + ((4 * g + tr_i + 4 * tr_j) & 15)) * 8;            // row 4g+i of a 16-row group, piece 4*(m/2) + j: + (32*sp2 + 16*half)*128 + 128*(m/2) + 4*(m&1)  (elements)
+    const int a_off = (c16 >> 2) * 64 + 4 * (c16 & 3) + ((g + (c16 >> 2)) & 3);  // operand piece 4s + g of row c16 of a t-tile: + tt*256 + 16*s  (16-byte units)
+    const int k_tr = (g * 64 + 4 * tr_i + ((tr_j + g) & 3)) * 8;                 // row 4g+i of a 16-row group, piece 4*(m/2) + j: + (32*sp2 + 16*half)*128 + 128*(m/2) + 4*(m&1)  (elements)
     int v_tr[NN];                                                                 // row 4g+i, piece = 8-column group of tile nn: + tt*2048
 #pragma unroll
     for (int nn = 0; nn < NN; ++nn) {
         const int c = 2 * (NN * w + nn) + (tr_j >> 1);
-        v_tr[nn] = (g * 64 + 16 * (c >> 2) + ((4 * g + tr_i + 4 * (c & 3)) & 15)) * 8 + 4 * (tr_j & 1);
+        v_tr[nn] = (g * 64 + 16 * (c >> 2) + 4 * tr_i + ((c + g) & 3)) * 8 + 4 * (tr_j & 1);
     }
 
     // One step, written as a fixed sequence of small scheduling regions (the compiler may reorder
