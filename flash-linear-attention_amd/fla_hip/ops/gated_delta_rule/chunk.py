@@ -190,6 +190,48 @@ def chunk_gated_delta_rule_fwd(
     """Forward of the chunked operator.  ``g`` is the log-space decay (raw gate inputs when
     ``A_log`` is given), ``beta`` the write strength (logits with ``use_beta_sigmoid_in_kernel``).
     Returns ``(o in q's dtype, final_state fp32 or None)``."""
+    K, V = k.shape[-1], v.shape[-1]
+    assert K <= 256, 'current kernel does not support head dimension larger than 256.'     # (chunk_delta_h.py:712)
+    if K > _KERNEL_DIMS[-1]:
+        # The chunk kernels hold a [K <= 128, 128] state per workgroup.  Wider keys take the token
+        # recurrence instead (same operator, same HIP library, state [K <= 256, V] in registers):
+        # correct for every shape the reference accepts, without the chunk path's throughput.
+        from fla_hip.ops.gated_delta_rule.fused_recurrent import fused_recurrent_gated_delta_rule_fwd
+        o, ht = fused_recurrent_gated_delta_rule_fwd(
+            q, k, v, g=g, beta=beta, A_log=A_log, dt_bias=dt_bias, scale=scale, initial_state=initial_state,
+            output_final_state=output_final_state, use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel,
+            use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel, allow_neg_eigval=allow_neg_eigval,
+            state_v_first=state_v_first, cu_seqlens=cu_seqlens)
+        return o.to(q.dtype), ht
+    nb = (V + _KERNEL_DIMS[-1] - 1) // _KERNEL_DIMS[-1]
+    if nb > 1:
+        # The value columns of the recurrence are independent: a head with V > 128 is nb heads of 128
+        # columns that share the head's k, q, gate and beta (grouped value heads do exactly that).
+        D = _KERNEL_DIMS[-1]
+        B, T, HV = v.shape[:3]
+        N = B if cu_seqlens is None else len(cu_seqlens) - 1
+        v2 = _pad_last(v, nb * D).reshape(B, T, HV * nb, D)
+        g2, beta2 = g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2)
+        A2 = None if A_log is None else A_log.reshape(-1).repeat_interleave(nb)
+        dt2 = None if dt_bias is None else dt_bias.reshape(-1).repeat_interleave(nb)
+        h2 = None
+        if initial_state is not None:
+            if state_v_first:       # [N, HV, V, K] -> [N, HV*nb, D, K]
+                h2 = torch.nn.functional.pad(initial_state, (0, 0, 0, nb * D - V)).reshape(N, HV * nb, D, K)
+            else:                   # [N, HV, K, V] -> [N, HV*nb, K, D]
+                h2 = _pad_last(initial_state, nb * D).reshape(N, HV, K, nb, D).permute(0, 1, 3, 2, 4).reshape(N, HV * nb, K, D)
+        o2, ht2 = chunk_gated_delta_rule_fwd(
+            q, k, v2, g2, beta2, scale, h2, output_final_state, state_v_first, cu_seqlens, cu_seqlens_cpu,
+            chunk_indices, chunk_size, A2, dt2, use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)
+        o = o2.reshape(B, T, HV, nb * D)[..., :V]
+        ht = None
+        if ht2 is not None:
+            if state_v_first:
+                ht = ht2.reshape(N, HV, nb * D, K)[:, :, :V]
+            else:
+                ht = ht2.reshape(N, HV, nb, K, D).permute(0, 1, 3, 2, 4).reshape(N, HV, K, nb * D)[..., :V]
+            ht = ht.contiguous()
+        return o.contiguous() if nb * D != V else o, ht
     call = ChunkLaunch(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first,
                        cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size,
                        A_log, dt_bias, use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)

@@ -115,6 +115,35 @@ def test_two_runs_per_workgroup(monkeypatch, mode, B, T, H, HV, dtype, gate_div)
         _check('o (shorter call)', ref_m, big[:, :Tm])
 
 
+@pytest.mark.parametrize('B,T,H,HV,K,V,vfirst,cu', [
+    (2, 300, 2, 2, 128, 256, False, None),      # wide values: split into two 128-column heads
+    (1, 500, 2, 4, 64, 200, True, None),        # ... padded, V-first state layout
+    (1, 700, 1, 2, 100, 384, False, [0, 130, 131, 700]),
+    (2, 150, 2, 2, 256, 128, False, None),      # wide keys: the token recurrence takes over
+    (1, 200, 1, 2, 192, 192, True, [0, 77, 200]),
+])
+def test_head_dims_above_128(B, T, H, HV, K, V, vfirst, cu):
+    """Every shape the reference accepts (K <= 256, any V) gives the right answer through the chunk entry
+    point, also where the chunk kernels themselves do not apply (fla/ops/common/chunk_delta_h.py:712)."""
+    N = B if cu is None else len(cu) - 1
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=31, gate_div=8.0, h0_std=0.5, N=N, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)
+    if vfirst:
+        o, ht = _run(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), cu, state_v_first=True)
+        ht = ht.transpose(-1, -2)
+    else:
+        o, ht = _run(q, k, v, g, beta, h0, cu)
+    assert o.shape == (B, T, HV, V) and o.dtype == q.dtype
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+def test_key_dim_above_256_is_rejected():
+    q, k, v, g, beta, _ = O.make_inputs(1, 64, 1, 1, 320, 64, seed=1, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        _run(q, k, v, g, beta)
+
+
 @pytest.mark.parametrize('mode', ['auto', 'single', 'pair'])
 def test_varlen_every_form(monkeypatch, mode):
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
