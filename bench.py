@@ -42,7 +42,7 @@ F_PREP = F_TOTAL - F_SCAN                              # 49152
 # HBM bytes per call of the dominant stage on the default workload, from FETCH_SIZE + WRITE_SIZE of
 # a counter run of this file scaled by the calib_copy workload (profiles/ holds the summary); other
 # workloads: not measured
-TRAFFIC_BYTES = {'prefill': 1.57e9}
+TRAFFIC_BYTES = {'prefill': 1.52e9}
 PEAK_BF16_TFLOPS = 2500.0                      # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0                          # MI355X HBM3E, published
 

@@ -55,18 +55,41 @@ __device__ __forceinline__ V8 join(V4 a, V4 b) {
 // 2^x as a single v_exp_f32 (results below 2^-126 flush to zero, which is what a decay wants)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Workspace record written by the prepare kernel per (chunk, v-head): 13 KB that the scan
+// Workspace record written by the prepare kernel per (chunk, v-head): 11 KB that the scan
 // copies verbatim into LDS.  Xb and P are stored as matrix-core operand fragments
-// ([slot][lane][8]): rows of t-tile tt, columns t' in {32sp+4g+r} U {32sp+16+4g+r}.  Both are
-// lower triangular, so the fragments (tt, sp) = (0,1), (1,1) are identically zero and are not
-// stored; the other six live in slot p_slot(tt, sp).
-//   Xb  T    [6][64][8]   (I+L)^-1 diag(beta)
-//   P   T    [6][64][8]   scale * tril(q k^T 2^(G_t-G_t'))
+// ([lane][8]): rows of t-tile tt, columns t' in {32sp+4g+r} U {32sp+16+4g+r}.  Both are
+// lower triangular: the fragments (tt, sp) = (0,1), (1,1) are identically zero and are not
+// stored, and of (0,0), (2,1) only the first half (4 values per lane) is.
+//   Xb  T    5 KB         (I+L)^-1 diag(beta)
+//   P   T    5 KB         scale * tril(q k^T 2^(G_t-G_t'))
 //   tab fp32 [256]        [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units)
-constexpr int REC_X = 0, REC_P = 6144, REC_TAB = 12288;
-constexpr int64_t REC_BYTES = 13312;
+constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240;
+constexpr int64_t REC_BYTES = 11264;
+constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10
 constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
 __host__ __device__ constexpr int p_slot(int tt, int sp) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp; }
+__host__ __device__ constexpr bool frag_half(int tt, int sp) { return (tt == 0 && sp == 0) || (tt == 2 && sp == 1); }
+__host__ __device__ constexpr int frag_off(int tt, int sp) {          // bytes from the start of Xb or P
+    return p_slot(tt, sp) == 0 ? 0 : p_slot(tt, sp) == 1 ? 512 : p_slot(tt, sp) == 2 ? 1536 : p_slot(tt, sp) == 3 ? 2560
+         : p_slot(tt, sp) == 4 ? 3072 : 4096;
+}
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V8 load_frag(const char* m, int tt, int sp, int lane) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    if (frag_half(tt, sp)) {
+        const V4 a = *(const V4*)(m + frag_off(tt, sp) + lane * 8);
+        const T z = (T)0.f;
+        return V8{a[0], a[1], a[2], a[3], z, z, z, z};
+    }
+    return *(const V8*)(m + frag_off(tt, sp) + lane * 16);
+}
+template <typename T>
+__device__ __forceinline__ void store_frag(char* m, int tt, int sp, int lane, typename Mma<T>::V8 f) {
+    typedef typename Mma<T>::V4 V4;
+    if (frag_half(tt, sp)) *(V4*)(m + frag_off(tt, sp) + lane * 8) = V4{f[0], f[1], f[2], f[3]};
+    else *(typename Mma<T>::V8*)(m + frag_off(tt, sp) + lane * 16) = f;
+}
 
 struct ChunkWs {
     float* Seg;          // 3 * seg_slots 128x128 fp32 matrices for the segment-parallel scan

@@ -28,7 +28,7 @@ namespace gdn {
 // per wave (each half of the rows is fetched again as soon as the wave has consumed it).
 constexpr int PR_K = 0, PR_Q = 32768, PR_V = 65536, PR_REC = 98304;
 constexpr int PR_OT = PR_REC + 4 * (int)REC_BYTES;            // 8 x 1 KB: per wave, one 16-token tile of its output columns on its way out
-constexpr size_t PAIR_SMEM = PR_OT + 8 * 1024;                // 159 744 B
+constexpr size_t PAIR_SMEM = PR_OT + 8 * 1024;                // 151 552 B
 constexpr int PAIR_THREADS = 512;
 
 // One 16-byte store per lane at sbase + voff, for the lanes named by `mask` only.  Written in
@@ -169,21 +169,21 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
             gather_1k_to_lds(base, __umul24(row, rowB_v) + v_cb, lds0 + PR_V + w * 4096 + b * 1024);
         }
     };
-    // The record of (chunk, value head).  A full run needs all 13 KB, a quarter per wave of the team.  A
-    // state-only run needs Xb and the tables (pieces 0..5 and 12), and its two teams work on the same
-    // value head: they share one copy (in the area of team 0), one piece per wave.
-    auto issue_rec = [&](int64_t c, int stage, int part) {                           // 2 parts of 2 operations (state-only: 1 part of 1)
+    // The record of (chunk, value head), in 1 KB pieces.  A full run needs all 11, three per wave of the
+    // team.  A state-only run needs Xb and the tables (pieces 0..4 and 10), and its two teams work on the
+    // same value head: they share one copy (in the area of team 0), one piece per wave.
+    auto issue_rec = [&](int64_t c, int stage, int part) {                           // parts of 2 and 1 operations (state-only: 1 part of 1)
         const char* rec = p.ws.Rec + ((boh + c) * HV + hv) * REC_BYTES;
         const uint32_t to = lds0 + PR_REC + ((FULL ? tm : 0) * 2 + stage) * (uint32_t)REC_BYTES;
         auto piece = [&](int j) { gather_1k_to_lds(rec + j * 1024, lane * 16, to + j * 1024); };
         if constexpr (FULL) {
             if (part == 0) { piece(cw); piece(cw + 4); }
-            else { piece(cw + 8); piece(cw == 0 ? 12 : cw); }                         // (waves 1..3 fetch one piece twice: equal counts)
+            else piece(cw < 3 ? cw + 8 : cw);                                         // (wave 3 fetches a piece twice: equal counts)
         } else {
-            if (part == 0) piece(w < 6 ? w : w == 6 ? 12 : 0);                        // (wave 7 fetches piece 0 again: equal counts)
+            if (part == 0) piece(w < REC_PIECES_X ? w : w == REC_PIECES_X ? REC_PIECE_TAB : 0);      // (waves 6, 7 fetch piece 0 again: equal counts)
         }
     };
-    // everything a barrier publishes, 8 (4) operations, in four parts so that the waves do not all
+    // everything a barrier publishes, 7 (3) operations, in four parts so that the waves do not all
     // queue at the memory pipeline at once
     auto issue_shared = [&](int64_t c, int stage, int part) {
         if (part == 0) issue_kq((const T*)p.k, c, lds0 + PR_K + stage * 16384);
@@ -191,10 +191,10 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         if (part >= 2) issue_rec(c, stage, part - 2);
     };
     // number of operations a wave issues between ...
-    // (per step, in order: shared 8 (3), in the first four regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
+    // (per step, in order: shared 7 (3), in the first four regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
     constexpr int N_AFTER_SHARED = FULL ? 8 : 4;      // the shared copies of a step and the barrier at its end
-    constexpr int N_AFTER_VLO = FULL ? 14 : 5;        // the first half of v and its use in the next step
-    constexpr int N_AFTER_VHI = FULL ? 12 : 5;        // the second half of v and its use in the next step
+    constexpr int N_AFTER_VLO = FULL ? 13 : 5;        // the first half of v and its use in the next step
+    constexpr int N_AFTER_VHI = FULL ? 11 : 5;        // the second half of v and its use in the next step
 
     if (nsteps > 0 && !active) {
         // a team with nothing to compute still fetches its share of k and of the record
@@ -259,8 +259,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         const T* sV = (const T*)(smem + PR_V + w * 4096);
         const T* sKt = (const T*)kbuf;
         const char* rec = smem + PR_REC + ((FULL ? tm : 0) * 2 + cur) * REC_BYTES;
-        const V8* sX = (const V8*)(rec + REC_X);
-        const V8* sP = (const V8*)(rec + REC_P);
+        const char* sX = rec + REC_X;
+        const char* sP = rec + REC_P;
         const float* sTab = (const float*)(rec + REC_TAB);
         const char* obase = (const char*)p.o + ((bos + it * CH) * HV + hv) * 256;
         const int valid = (int)min((int64_t)CH, len - it * CH);
@@ -293,12 +293,12 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         };
         auto FX = [&](int tt) {
 #pragma unroll
-            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = sX[p_slot(tt, sp2) * 64 + lane];
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = load_frag<T>(sX, tt, sp2, lane);
         };
         auto FP = [&](int tt) {
             if constexpr (FULL) {
 #pragma unroll
-                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = sP[p_slot(tt, sp2) * 64 + lane];
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
             }
         };
         V8 kt[2][8];

@@ -166,7 +166,6 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         {
             const int t = 16 * tt + c16;
             const float gt = sG[t], st = p.scale * sRN[CH + t];
-            T* pf = (T*)(rec + REC_P);
 #pragma unroll
             for (int sp = 0; sp < 2; ++sp) {
                 if (tt < 2 && sp == 1) continue;        // identically zero, not stored
@@ -187,7 +186,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
                         frag[half * 4 + r] = from_f32<T>(val);
                     }
                 }
-                *(V8*)(pf + (p_slot(tt, sp) * 64 + lane) * 8) = frag;
+                store_frag<T>(rec + REC_P, tt, sp, lane, frag);
             }
         }
     }
@@ -306,7 +305,6 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         __syncthreads();
         // ---- Xb = X diag(beta) rows of t-tile w as A-operand fragments ----
         {
-            T* xf = (T*)(rec + REC_X);
             const int ns = (w >= 2) ? 2 : 1;         // X is lower triangular: columns >= 32 matter only for rows >= 32
             for (int sp = 0; sp < ns; ++sp) {
                 const float* xr = sX + (16 * w + c16) * LP + 32 * sp + 4 * g;
@@ -318,7 +316,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
                     frag[e] = from_f32<T>(x0[e] * b0[e]);
                     frag[4 + e] = from_f32<T>(x1[e] * b1[e]);
                 }
-                *(V8*)(xf + (p_slot(w, sp) * 64 + lane) * 8) = frag;
+                store_frag<T>(rec + REC_X, w, sp, lane, frag);
             }
         }
         if (m + 1 < G) __syncthreads();          // the next value head overwrites L and X

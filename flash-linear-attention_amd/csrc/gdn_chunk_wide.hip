@@ -45,11 +45,11 @@ namespace gdn {
 // very end of a step, has three buffers (chunk % 3) so that its copy can be issued two steps ahead.
 constexpr int STG_Q = 0, STG_V = 16384, STG_REC = 32768;
 constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB;
-constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 46 080
+constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 44 032
 constexpr int KBUF = 2 * STG_BYTES;                          // three k tiles of 16 KB follow the two stages
 constexpr int OT_PITCH = 272;                     // bytes per token row of the output tile (256 B + pad: conflict-free 8-byte writes)
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
-constexpr size_t WIDE_SMEM = KBUF + 3 * 16384 + OT_BYTES;    // 158 720 B of the CU's 163 840: one workgroup per CU
+constexpr size_t WIDE_SMEM = KBUF + 3 * 16384 + OT_BYTES;    // 154 624 B of the CU's 163 840: one workgroup per CU
 constexpr int WIDE_NN = 2;                        // 16-column tiles per compute wave
 #ifndef WIDE_RING
 #define WIDE_RING 3                               // operand fragments in flight per compute wave
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage) {
             const char* rec = p.ws.Rec + ((boh + it) * HV + hv) * REC_BYTES;
 #pragma unroll
-            for (int j = 0; j < 13; ++j)
+            for (int j = 0; j < (int)(REC_BYTES / 1024); ++j)
                 if (j >= from && j < to) gather_1k_to_lds(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024);
         };
         if (w == CW) {
@@ -197,23 +197,23 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 const uint32_t st = lds0 + stage * STG_BYTES;
                 if (qside) {
                     if constexpr (FULL) {
-                        // 16 q pieces, then Xb (6) and the tables (1)
+                        // 16 q pieces, then Xb (5) and the tables (1)
                         if (early) gather_blocks((const T*)p.q, H, h, it, 0, 8, st + STG_Q);
-                        else { gather_blocks((const T*)p.q, H, h, it, 8, 16, st + STG_Q); copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }
+                        else { gather_blocks((const T*)p.q, H, h, it, 8, 16, st + STG_Q); copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }
                     } else {
-                        if (early) { copy_rec(it, 0, 6, st); copy_rec(it, 12, 13, st); }      // all 7 pieces
+                        if (early) { copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }      // all 6 pieces
                     }
                 } else {
                     if (early) { if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 0, 8, st + STG_V); }      // (v is not read when it counts as zero)
                     else {
                         if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 8, 16, st + STG_V);
-                        if constexpr (FULL) copy_rec(it, 6, 12, st);
+                        if constexpr (FULL) copy_rec(it, REC_PIECES_X, REC_PIECES_X + REC_PIECES_P, st);
                     }
                 }
             };
-            // number of pieces issued early: 8, except 7 for the q side of a state-only run
+            // number of pieces issued early: 8, except 6 for the q side of a state-only run
             auto wait_early_only = [&]() {
-                if (!FULL && qside) wait_vm_at_most<7>();
+                if (!FULL && qside) wait_vm_at_most<REC_PIECES_X + 1>();
                 else wait_vm_at_most<XB>();
             };
             issue(it0, 0, true);
@@ -316,8 +316,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const V8* sQ = (const V8*)(st + STG_Q);
         const T* sV = (const T*)(st + STG_V);
         const T* sKt = (const T*)kbuf;
-        const V8* sX = (const V8*)(st + STG_X);
-        const V8* sP = (const V8*)(st + STG_P);
+        const char* sX = st + STG_X;
+        const char* sP = st + STG_P;
         const float* sTab = (const float*)(st + STG_TAB);
         auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
@@ -346,12 +346,12 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         };
         auto FX = [&](int tt) {
 #pragma unroll
-            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = sX[p_slot(tt, sp2) * 64 + lane];
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = load_frag<T>(sX, tt, sp2, lane);
         };
         auto FP = [&](int tt) {
             if constexpr (FULL) {
 #pragma unroll
-                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = sP[p_slot(tt, sp2) * 64 + lane];
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
             }
         };
         V8 kt[2][8];                            // k^T rows of key tile m over t-tile pair sp2
