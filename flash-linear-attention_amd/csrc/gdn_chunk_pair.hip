@@ -459,12 +459,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
 template <typename T, bool FULL>
 static int launch_pair_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
     auto kern = gdn_chunk_pair_kernel<T, FULL>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)PAIR_SMEM) != hipSuccess)
-            return check_launch("hipFuncSetAttribute(pair)");
-        attr_done = true;
-    }
+    static SmemAttrDone attr_done;       // per instantiation
+    if (int rc = ensure_dynamic_smem((const void*)kern, PAIR_SMEM, attr_done, "hipFuncSetAttribute(pair)")) return rc;
     if (blocks <= 0) return GDN_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(PAIR_THREADS), PAIR_SMEM, stream, p, sp);
     return check_launch("gdn_chunk_pair_kernel");

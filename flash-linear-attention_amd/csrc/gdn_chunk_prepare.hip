@@ -332,12 +332,8 @@ int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream)
         set_error("gdn_chunk_fwd: %d value heads per q/k head exceed what the prepare kernel stages", G);
         return GDN_ERR_UNSUPPORTED;
     }
-    static bool attr_done = false;       // per instantiation
-    if (!attr_done) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024) != hipSuccess)
-            return check_launch("hipFuncSetAttribute(prepare)");
-        attr_done = true;
-    }
+    static SmemAttrDone attr_done;       // per instantiation
+    if (int rc = ensure_dynamic_smem((const void*)kern, 64 * 1024, attr_done, "hipFuncSetAttribute(prepare)")) return rc;
     dim3 grid((unsigned)(num_chunks * p.H)), block(256);
     hipLaunchKernelGGL(kern, grid, block, smem, stream, p);
     return check_launch("gdn_chunk_prepare_kernel");

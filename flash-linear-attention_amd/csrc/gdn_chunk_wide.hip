@@ -587,12 +587,8 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, 
 template <typename T, bool FULL>
 static int launch_wide_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
     auto kern = gdn_chunk_wide_kernel<T, FULL>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)WIDE_SMEM) != hipSuccess)
-            return check_launch("hipFuncSetAttribute(wide)");
-        attr_done = true;
-    }
+    static SmemAttrDone attr_done;       // per instantiation
+    if (int rc = ensure_dynamic_smem((const void*)kern, WIDE_SMEM, attr_done, "hipFuncSetAttribute(wide)")) return rc;
     if (blocks <= 0) return GDN_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WIDE_THREADS), WIDE_SMEM, stream, p, sp);
     return check_launch("gdn_chunk_wide_kernel");
@@ -613,13 +609,8 @@ int launch_wide(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
 }
 
 int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute((const void*)gdn_segment_merge_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)MERGE_SMEM) != hipSuccess)
-            return check_launch("hipFuncSetAttribute(merge)");
-        attr_done = true;
-    }
+    static SmemAttrDone attr_done;
+    if (int rc = ensure_dynamic_smem((const void*)gdn_segment_merge_kernel, MERGE_SMEM, attr_done, "hipFuncSetAttribute(merge)")) return rc;
     hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)((p.NH + 7) / 8 * 64)), dim3(256), MERGE_SMEM, stream, sp, p.NH);
     return check_launch("gdn_segment_merge_kernel");
 }

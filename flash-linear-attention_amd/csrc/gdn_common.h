@@ -29,6 +29,19 @@ inline int check_launch(const char* what) {
     return GDN_OK;
 }
 
+// Raises the dynamic LDS limit of a kernel once per device (the attribute belongs to the function on
+// the current device; a process may drive several).  `done` is a per-kernel table owned by the caller.
+struct SmemAttrDone { bool dev[64] = {}; };
+inline int ensure_dynamic_smem(const void* kernel, size_t bytes, SmemAttrDone& done, const char* what) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return check_launch(what);
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && done.dev[dev]) return GDN_OK;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return check_launch(what);
+    if (tracked) done.dev[dev] = true;
+    return GDN_OK;
+}
+
 // ---- element types -------------------------------------------------------
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;
