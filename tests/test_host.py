@@ -42,6 +42,19 @@ def test_library_exports_every_declared_symbol():
         _lib.check(rc)
 
 
+def test_flag_and_status_constants_match_the_header():
+    """The Python binding repeats the header's constants by value: they must agree, and no two flags
+    may share a bit."""
+    from fla_hip import _lib
+    header = open(os.path.join(ROOT, 'include', 'gdn_hip.h')).read()
+    flags = {n: (1 << int(b)) for n, b in re.findall(r'#define\s+GDN_FLAG_(\w+)\s+\(1u\s*<<\s*(\d+)\)', header)}
+    assert len(flags) >= 11 and len(set(flags.values())) == len(flags)
+    for name, value in flags.items():
+        assert getattr(_lib, 'FLAG_' + name) == value, name
+    for name, value in re.findall(r'#define\s+(GDN_ERR_\w+|GDN_OK)\s+\(?(-?\d+)\)?', header):
+        assert getattr(_lib, name) == int(value), name
+
+
 @pytest.mark.parametrize('cu', [[0, 15], [0, 64], [0, 1, 65, 192, 193, 400], [0, 256, 500, 1000], [0, 100, 100, 164]])
 @pytest.mark.parametrize('dtype', [torch.int64, torch.int32])
 def test_chunk_tables_match_loop_reference(cu, dtype):
