@@ -17,7 +17,7 @@ struct RecurrentParams {
     const void* g; const void* beta; const float* gk; const float* gv;
     const float* A_log; const float* dt_bias;
     const float* h0; float* ht; void* o;
-    const void* cu_seqlens;
+    const void* cu_seqlens; const void* state_slots;
     int64_t T; int H, HV, K, V, NVB;
     float scale; int gb_dtype; uint32_t flags;
 };
@@ -69,7 +69,9 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
     const int row_base = VFIRST ? v0 : 0;
     const int64_t row_stride = VFIRST ? K : V;
     const bool cont_ok = cont_idx < cont_lim;
-    const int64_t state_off = inh * (int64_t)K * V;
+    // the state lives at sequence n of the state tensors, or at the slot of a pool that the caller names for n
+    const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
+    const int64_t state_off = (slot * HV + ihv) * (int64_t)K * V;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int row = row_base + r0 + RP * i;
@@ -275,7 +277,7 @@ extern "C" int gdn_fused_recurrent_fwd(
     const void* g, const void* beta, const float* gk, const float* gv,
     const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
-    const void* cu_seqlens,
+    const void* cu_seqlens, const void* state_slots,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
@@ -297,7 +299,7 @@ extern "C" int gdn_fused_recurrent_fwd(
     if (T == 0) return GDN_OK;
     RecurrentParams p;
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.gk = gk; p.gv = gv;
-    p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o; p.cu_seqlens = cu_seqlens;
+    p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o; p.cu_seqlens = cu_seqlens; p.state_slots = state_slots;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.K = (int)K; p.V = (int)V; p.NVB = 1;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
     hipStream_t s = (hipStream_t)stream;

@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -25,6 +25,7 @@ FLAG_NEG_EIGVAL = 1 << 2
 FLAG_STATE_V_FIRST = 1 << 3
 FLAG_BETA_VECTOR = 1 << 4
 FLAG_CU_INT32 = 1 << 5
+FLAG_SLOT_INT32 = 1 << 6
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
 FLAG_SEQ_ORDER = 1 << 19
@@ -40,7 +41,7 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p,            # g beta gk gv
         c_void_p, c_void_p,                                # A_log dt_bias
         c_void_p, c_void_p, c_void_p,                      # h0 ht o
-        c_void_p,                                          # cu_seqlens
+        c_void_p, c_void_p,                                # cu_seqlens state_slots
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
         c_float, c_int, c_int, c_uint32, c_void_p]),
     'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),

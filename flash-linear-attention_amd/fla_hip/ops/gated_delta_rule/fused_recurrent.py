@@ -41,10 +41,13 @@ def fused_recurrent_gated_delta_rule_fwd(
     state_v_first: bool = False,
     cu_seqlens: torch.Tensor | None = None,
     inplace_final_state: bool = False,
+    ssm_state_indices: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Allocates ``o`` (v's dtype) and the fp32 final state, then launches the HIP kernel on
     the current stream.  With ``inplace_final_state`` the final state is written over
-    ``initial_state`` (which must then be fp32 and contiguous) and that tensor is returned."""
+    ``initial_state`` (which must then be fp32 and contiguous) and that tensor is returned.
+    With ``ssm_state_indices`` ``[N]`` the states are slots of the pool ``initial_state
+    [num_slots, HV, K, V]``, updated in place."""
     dev = require_gpu(q, k, v)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
@@ -74,6 +77,19 @@ def fused_recurrent_gated_delta_rule_fwd(
 
     state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
     h0 = initial_state
+    slots = None
+    if ssm_state_indices is not None:
+        if not inplace_final_state or h0 is None:
+            raise ValueError('ssm_state_indices needs the state pool as initial_state and inplace_final_state=True')
+        if ssm_state_indices.ndim != 1 or ssm_state_indices.shape[0] != N:
+            raise ValueError(f'ssm_state_indices must have shape ({N},), got {tuple(ssm_state_indices.shape)}')
+        slots = ssm_state_indices.to(dev)
+        if slots.dtype == torch.int32:
+            flags |= _lib.FLAG_SLOT_INT32
+        elif slots.dtype != torch.int64:
+            slots = slots.long()
+        slots = slots.contiguous()
+        state_shape = (h0.shape[0],) + state_shape[1:]            # the pool has its own number of slots
     if h0 is not None:
         if tuple(h0.shape) != state_shape:
             raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
@@ -95,7 +111,7 @@ def fused_recurrent_gated_delta_rule_fwd(
     lib = _lib.load()
     _lib.check(lib.gdn_fused_recurrent_fwd(
         ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(gk), ptr(gv), ptr(A_log), ptr(dt_bias),
-        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens),
+        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots),
         B, T, H, HV, K, V, N, float(scale), dtype_code(q.dtype), gb_code, flags,
         current_stream_ptr(dev)))
     return o, final_state
@@ -138,6 +154,10 @@ def fused_recurrent_gated_delta_rule(
         cu_seqlens: ``[N + 1]`` int32/int64 boundaries of packed sequences (then ``B == 1``).
         inplace_final_state (keyword only, extension): write the final state over
             ``initial_state`` instead of allocating a new tensor.
+        ssm_state_indices (keyword only, extension; the sibling KDA operator's argument,
+            fla/ops/kda/fused_recurrent.py:248-326): ``[N]`` int32/int64 slot of every sequence in the
+            state pool ``initial_state [num_slots, HV, K, V]``; needs ``inplace_final_state=True``.
+            Slots must be distinct; slots that are not named keep their contents.
 
     Returns:
         ``(o [B, T, HV, V] in v's dtype, final_state or None)``.
@@ -149,6 +169,7 @@ def fused_recurrent_gated_delta_rule(
                       DeprecationWarning, stacklevel=2)
         state_v_first = kwargs.pop('transpose_state_layout')
     inplace_final_state = bool(kwargs.pop('inplace_final_state', False))
+    ssm_state_indices = kwargs.pop('ssm_state_indices', None)
 
     if q.shape[2] != k.shape[2]:
         raise ValueError(f'q and k must have the same number of heads, got {q.shape[2]} and {k.shape[2]}')
@@ -159,7 +180,7 @@ def fused_recurrent_gated_delta_rule(
             raise ValueError(
                 f'The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`.'
                 f'Please flatten variable-length inputs before processing.')
-        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+        if initial_state is not None and ssm_state_indices is None and initial_state.shape[0] != len(cu_seqlens) - 1:
             raise ValueError(
                 f'The number of initial states is expected to be equal to the number of input sequences, '
                 f'i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.')
@@ -182,7 +203,7 @@ def fused_recurrent_gated_delta_rule(
     return fused_recurrent_gated_delta_rule_fwd(
         q, k, v, g, gk, gv, beta, A_log, dt_bias, scale, initial_state, output_final_state,
         use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, cu_seqlens,
-        inplace_final_state)
+        inplace_final_state, ssm_state_indices)
 
 
 fused_recurrent_gdn = fused_recurrent_gated_delta_rule

@@ -41,6 +41,7 @@ extern "C" {
 #define GDN_FLAG_STATE_V_FIRST  (1u << 3)  /* state_v_first: states are [N,HV,V,K]              */
 #define GDN_FLAG_BETA_VECTOR    (1u << 4)  /* beta is [B,T,HV,V] instead of [B,T,HV]            */
 #define GDN_FLAG_CU_INT32       (1u << 5)  /* cu_seqlens / chunk tables are int32, else int64   */
+#define GDN_FLAG_SLOT_INT32     (1u << 6)  /* state_slots is int32, else int64                  */
 /* gdn_chunk_fwd only: force one form of the sequential stage instead of the automatic choice
  * (all forms give the same result up to rounding; used by tests and for tuning)                */
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
@@ -68,6 +69,10 @@ const char* gdn_last_error(void);
  *   h0     [N,HV,K,V] fp32 or NULL (zero state)
  *   ht     [N,HV,K,V] fp32 or NULL (final state not stored); ht MAY alias h0 (in-place update)
  *   cu_seqlens [N+1] or NULL; when given B must be 1 and T is the packed length
+ *   state_slots [N] or NULL: sequence n then keeps its state in slot state_slots[n] of a pool, i.e. h0 and ht
+ *          are [num_slots,HV,K,V] and are addressed through the slot instead of n (continuous batching; the
+ *          sibling KDA operator's ssm_state_indices, fla/ops/kda/fused_recurrent.py:27,75-91,145-159).  Slots
+ *          must be distinct; other slots are not touched.
  *   N = B when cu_seqlens == NULL.  Requires K <= 256, K % 4 == 0, V % 4 == 0, HV % H == 0.
  */
 int gdn_fused_recurrent_fwd(
@@ -75,7 +80,7 @@ int gdn_fused_recurrent_fwd(
     const void* g, const void* beta, const float* gk, const float* gv,
     const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
-    const void* cu_seqlens,
+    const void* cu_seqlens, const void* state_slots,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 

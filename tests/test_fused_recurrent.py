@@ -154,6 +154,40 @@ def test_flags_gate_sigmoid_vector_beta_gk_gv_vfirst():
     assert none is None
 
 
+@pytest.mark.parametrize('idx_dtype', [torch.int32, torch.int64])
+@pytest.mark.parametrize('vfirst,cu', [(False, None), (True, None), (False, [0, 3, 4, 9])])
+def test_state_pool_addressed_by_slot(idx_dtype, vfirst, cu):
+    """Continuous batching: every sequence names its slot in a state pool; the step reads and writes
+    that slot in place and touches no other (fla/ops/kda/fused_recurrent.py:75-91,145-159 for the
+    sibling operator; the GDN reference has no such argument)."""
+    H, HV, D, slots_total = 2, 4, 128, 11
+    N = 3
+    if cu is None:
+        q, k, v, g, beta, _ = _inputs(N, 2, H, HV, D, torch.bfloat16, seed=9)
+    else:
+        q, k, v, g, beta, _ = _inputs(1, cu[-1], H, HV, D, torch.bfloat16, seed=9)
+    gen = torch.Generator().manual_seed(10)
+    pool = torch.randn(slots_total, HV, D, D, generator=gen)
+    slots = [7, 0, 4]
+    ref_o, ref_h = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, pool[slots], True, cu_seqlens=cu)
+    dev = 'cuda'
+    dpool = (pool.transpose(-1, -2) if vfirst else pool).contiguous().to(dev)
+    before = dpool.clone()
+    o, out = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=dpool,
+                    output_final_state=True, inplace_final_state=True, state_v_first=vfirst,
+                    cu_seqlens=None if cu is None else torch.tensor(cu, device=dev),
+                    ssm_state_indices=torch.tensor(slots, dtype=idx_dtype, device=dev))
+    assert out.data_ptr() == dpool.data_ptr()
+    _check('o', ref_o, o)
+    got = dpool[slots].transpose(-1, -2) if vfirst else dpool[slots]
+    _check('slots', ref_h, got)
+    rest = [i for i in range(slots_total) if i not in slots]
+    assert torch.equal(dpool[rest], before[rest]), 'a slot that no sequence named was modified'
+    with pytest.raises(ValueError):
+        _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=dpool,
+               output_final_state=True, ssm_state_indices=torch.tensor(slots, device=dev))
+
+
 def test_host_validation_errors():
     op = _ops()
     dev = 'cuda'

@@ -30,12 +30,12 @@ def test_library_exports_every_declared_symbol():
     assert l.gdn_chunk_workspace_bytes(8, 2, 4, 128, 128) > 0
     assert l.gdn_chunk_workspace_bytes(8, 2, 4, 96, 128) == 0
     # argument errors are reported before any launch
-    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None,
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None,
                                    1, 1, 2, 3, 64, 64, 1, 1.0, 0, 2, 0, None)
     assert rc == _lib.GDN_ERR_INVALID and 'divisible' in _lib.last_error()
     with pytest.raises(ValueError):
         _lib.check(rc)
-    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None,
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None,
                                    1, 1, 1, 1, 512, 64, 1, 1.0, 0, 2, 0, None)
     assert rc == _lib.GDN_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):
