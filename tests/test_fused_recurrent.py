@@ -188,6 +188,39 @@ def test_state_pool_addressed_by_slot(idx_dtype, vfirst, cu):
                output_final_state=True, ssm_state_indices=torch.tensor(slots, device=dev))
 
 
+def test_decode_and_prefill_replay_from_a_captured_graph():
+    """Serving loops replay captured graphs: the entry points only enqueue kernels on the given
+    stream (no allocation, no memset, no synchronisation of their own), so a captured decode step
+    and a captured prefill reproduce the eager results on every replay, with eager work and
+    synchronisations in between."""
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    dev = 'cuda'
+    H, HV, D, N = 2, 4, 128, 8
+    q, k, v, g, beta, h0 = _inputs(N, 1, H, HV, D, torch.bfloat16, seed=5)
+    dq, dk, dv, dg, db = (x.to(dev) for x in (q, k, v, g, beta))
+    state = h0.to(dev).contiguous()
+    eager_state = state.clone()
+    pq, pk, pv, pg, pb, ph = (x.to(dev) for x in O.make_inputs(1, 700, H, HV, D, D, seed=6, gate_div=8.0, h0_std=0.5, dtype=torch.bfloat16))
+    # warm up outside the capture (library load, kernel attributes)
+    _ops()(dq, dk, dv, dg, beta=db, initial_state=state.clone(), output_final_state=True, inplace_final_state=True)
+    po_eager, ph_eager = chunk_gated_delta_rule(pq, pk, pv, pg, pb, initial_state=ph, output_final_state=True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_static, _ = _ops()(dq, dk, dv, dg, beta=db, initial_state=state, output_final_state=True, inplace_final_state=True)
+        po_static, ph_static = chunk_gated_delta_rule(pq, pk, pv, pg, pb, initial_state=ph, output_final_state=True)
+    state.copy_(h0.to(dev))                      # (the capture itself did not run anything)
+    for step in range(3):
+        graph.replay()
+        o_eager, _ = _ops()(dq, dk, dv, dg, beta=db, initial_state=eager_state, output_final_state=True, inplace_final_state=True)
+        torch.cuda.synchronize()
+        assert torch.equal(o_static, o_eager), f'decode output differs on replay {step}'
+        assert torch.equal(state, eager_state), f'decode state differs on replay {step}'
+        assert not torch.isnan(po_eager).any()
+        assert torch.equal(po_static, po_eager) and torch.equal(ph_static, ph_eager), f'prefill differs on replay {step}'
+        po_static.zero_(); ph_static.zero_()     # the next replay has to write everything again
+
+
 def test_host_validation_errors():
     op = _ops()
     dev = 'cuda'
