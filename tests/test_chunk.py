@@ -56,6 +56,43 @@ def test_chunk_vs_oracle(B, T, H, HV, D, gate_div, with_h0, dtype):
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_logit_normalizer,mask_p,l2norm_in_kernel', [
+    (4, 1024, 4, 4, 128, 0.1, 1, 1.0, False),
+    (2, 75, 4, 4, 64, 1, 0.01, 0, False),
+    (2, 500, 3, 3, 60, 1, 1, 0, False),
+    (2, 1000, 3, 3, 64, 0.1, 1, 0.5, False),
+    (3, 1024, 4, 4, 100, 1, 0.1, 0, False),
+    (4, 1024, 4, 4, 128, 0.1, 1, 0, True),
+    (2, 1500, 4, 4, 128, 0.1, 10, 0, False),
+    (4, 2048, 8, 8, 64, 0.1, 1, 0, False),
+    (2, 256, 2, 4, 64, 1, 1, 0, False),
+    (2, 512, 2, 8, 64, 1, 0.1, 0, True),
+    (2, 1024, 4, 8, 128, 0.1, 1, 0, False),
+])
+def test_reference_matrix_with_the_reference_input_recipe(B, T, H, HV, D, scale, gate_logit_normalizer, mask_p, l2norm_in_kernel):
+    """The reference's own parameter matrix and input recipe for this operator (tests/ops/test_gdn.py:108-200):
+    fp16, q/k/v uniform in [0, 1) (strongly correlated keys), gates divided by the normaliser (0.01 = decay
+    by e^-69 per token), a fraction mask_p of the gates set to zero, zero initial state, custom scale, l2
+    normalisation outside or inside the kernels.  Its bar: error ratio 0.005 on o and ht."""
+    gen = torch.Generator().manual_seed(42)
+    dtype = torch.float16
+    q = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    k = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    v = torch.rand(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    g = F.logsigmoid(torch.rand(B, T, HV, generator=gen)) / gate_logit_normalizer
+    g = g * (torch.rand(B, T, HV, generator=gen) > mask_p)
+    h0 = torch.zeros(B, HV, D, D)
+    qn, kn = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(qn, kn, v, g, beta, scale, h0, True)
+    dev = 'cuda'
+    o, ht = _op()((q if l2norm_in_kernel else qn).to(dev), (k if l2norm_in_kernel else kn).to(dev), v.to(dev), g.to(dev),
+                  beta.to(dev), scale=scale, initial_state=h0.to(dev), output_final_state=True,
+                  use_qk_l2norm_in_kernel=l2norm_in_kernel)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 @pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'wide-pair', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
     (2, 1000, 2, 4, True, False),
