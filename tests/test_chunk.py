@@ -93,6 +93,37 @@ def test_reference_matrix_with_the_reference_input_recipe(B, T, H, HV, D, scale,
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('H,HV,D,mask_p,cu', [
+    (4, 4, 60, 0, [0, 15]),
+    (4, 4, 64, 0, [0, 256, 500, 1000]),
+    (4, 4, 64, 0.5, [0, 256, 500, 1000]),
+    (4, 4, 100, 0, [0, 15, 100, 300, 1200, 2000]),
+    (2, 4, 64, 0, [0, 256, 500, 1000]),
+    (2, 8, 64, 0, [0, 256, 500, 1000]),
+])
+def test_reference_varlen_matrix_with_the_reference_input_recipe(H, HV, D, mask_p, cu):
+    """The reference's packed-input matrix and recipe (tests/ops/test_gdn.py:712-800): fp16, q NOT
+    normalised, k normalised, fp16 gates with a masked fraction, fp16 initial states of unit variance;
+    every sequence is checked against the token recurrence run on it alone.  Bar 0.005."""
+    gen = torch.Generator().manual_seed(42)
+    dtype = torch.float16
+    T, N = cu[-1], len(cu) - 1
+    q = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    k = F.normalize(torch.randn(1, T, H, D, generator=gen), p=2, dim=-1).to(dtype)
+    v = torch.randn(1, T, HV, D, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.rand(1, T, HV, generator=gen)).to(dtype)
+    g = g * (torch.rand(1, T, HV, generator=gen) > mask_p)
+    beta = torch.rand(1, T, HV, generator=gen).sigmoid()
+    h0 = torch.randn(N, HV, D, D, generator=gen).to(dtype)
+    refs = [O.recurrent_gated_delta_rule(q[:, a:b], k[:, a:b], v[:, a:b], g[:, a:b].float(), beta[:, a:b], None,
+                                         h0[i:i + 1].float(), True) for i, (a, b) in enumerate(zip(cu[:-1], cu[1:]))]
+    ref_o, ref_ht = torch.cat([r[0] for r in refs], 1), torch.cat([r[1] for r in refs], 0)
+    o, ht = _run(q, k, v, g, beta, h0, cu)
+    assert ht.dtype == torch.float32
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 @pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'wide-pair', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
     (2, 1000, 2, 4, True, False),
