@@ -61,6 +61,36 @@ def test_fused_recurrent_vs_oracle(B, T, H, HV, D, scale, gate_norm, dtype):
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_logit_normalizer,dtype', [
+    (1, 63, 1, 1, 64, 1, 1, torch.float),
+    (2, 500, 4, 4, 60, 1, 1, torch.float),
+    (2, 1000, 2, 8, 128, 1, 0.1, torch.float),
+    (3, 1024, 2, 2, 128, 0.1, 1, torch.float),
+    (4, 1024, 3, 3, 128, 1, 10, torch.float),
+    (4, 2048, 4, 4, 64, 0.1, 1, torch.float),
+    (2, 1024, 4, 4, 128, 1, 0.1, torch.float16),
+    (2, 1024, 4, 8, 128, 1, 10, torch.float16),
+])
+def test_reference_matrix_with_the_reference_input_recipe(B, T, H, HV, D, scale, gate_logit_normalizer, dtype):
+    """The reference's own matrix and recipe for this operator (tests/ops/test_gdn.py:48-105): q and k in
+    fp32 and NOT normalised (the kernel does it), v and beta in the test dtype, unit-variance fp32 initial
+    state, full sequence lengths.  Its bar: error ratio 0.002 on o and ht."""
+    gen = torch.Generator().manual_seed(42)
+    q = torch.randn(B, T, H, D, generator=gen)
+    k = torch.randn(B, T, H, D, generator=gen)
+    v = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).to(dtype).sigmoid()
+    g = F.logsigmoid(torch.rand(B, T, HV, generator=gen)) / gate_logit_normalizer
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(F.normalize(q, p=2, dim=-1).to(dtype), F.normalize(k, p=2, dim=-1).to(dtype),
+                                                 v, g, beta, scale, h0, True)
+    dev = 'cuda'
+    o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), scale=scale,
+                   initial_state=h0.to(dev), output_final_state=True, use_qk_l2norm_in_kernel=True)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 def test_decode_shape_inplace_and_chained_steps():
     """N=64 decode steps with Hqk=16, Hv=32, K=V=128 (the decode configuration at a quarter
     of its batch): three chained single-token calls, state updated in place, must equal the
