@@ -124,6 +124,25 @@ def test_reference_varlen_matrix_with_the_reference_input_recipe(H, HV, D, mask_
     _check('ht', ref_ht, ht)
 
 
+@torch.inference_mode()
+def test_reference_varlen_prefill_case_under_inference_mode():
+    """tests/ops/test_gdn.py:806-876, its largest case: one packed sequence of 8192 tokens, D = 60, fp16
+    everywhere (q unnormalised, gates, beta and initial state in fp16), called under inference mode."""
+    gen = torch.Generator().manual_seed(42)
+    dtype, H, D, cu = torch.float16, 4, 60, [0, 8192]
+    T = cu[-1]
+    q = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    k = F.normalize(torch.randn(1, T, H, D, generator=gen), p=2, dim=-1).to(dtype)
+    v = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.rand(1, T, H, generator=gen)).to(dtype)
+    beta = torch.rand(1, T, H, generator=gen).to(dtype).sigmoid()
+    h0 = torch.randn(1, H, D, D, generator=gen).to(dtype)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g.float(), beta.float(), None, h0.float(), True)
+    o, ht = _run(q, k, v, g, beta, h0, cu)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 @pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'wide-pair', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
     (2, 1000, 2, 4, True, False),
