@@ -124,6 +124,44 @@ def test_reference_varlen_matrix_with_the_reference_input_recipe(H, HV, D, mask_
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('B,T,H,HV,D,scale,has_dt_bias,l2norm_in_kernel', [
+    (2, 75, 4, 4, 64, 1, True, True),
+    (2, 500, 3, 3, 60, 1, False, False),
+    (2, 1000, 3, 3, 64, 0.1, True, False),
+    (3, 1024, 4, 4, 100, 1, True, True),
+    (4, 1024, 4, 4, 128, 0.1, False, True),
+    (4, 2048, 8, 8, 64, 0.1, True, False),
+    (2, 256, 2, 4, 64, 1, True, False),             # grouped value heads (:1000-1104)
+    (2, 512, 1, 4, 64, 0.1, False, False),
+    (2, 512, 2, 8, 64, 1, True, False),
+    (2, 1024, 4, 8, 128, 0.1, True, False),
+])
+def test_reference_gate_in_kernel_matrix_with_the_reference_input_recipe(B, T, H, HV, D, scale, has_dt_bias, l2norm_in_kernel):
+    """tests/ops/test_gdn.py:878-1104: raw gate inputs ~ N(0,1), A_log ~ N(0,1) per value head (decays up to
+    e^-20 and more per token), optional dt_bias, fp16 uniform q/k/v, zero initial state; the gate activation
+    -exp(A_log)*softplus(g + dt_bias) happens inside the first kernel.  Bar 0.005."""
+    gen = torch.Generator().manual_seed(42)
+    dtype = torch.float16
+    q = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    k = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    v = torch.rand(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    g_raw = torch.randn(B, T, HV, generator=gen)
+    A_log = torch.randn(HV, generator=gen)
+    dt_bias = torch.randn(HV, generator=gen) if has_dt_bias else None
+    h0 = torch.zeros(B, HV, D, D)
+    qn, kn = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    g_ref = -A_log.exp() * F.softplus(g_raw + (dt_bias if has_dt_bias else 0.0))        # gate.py:21-46
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(qn, kn, v, g_ref, beta, scale, h0, True)
+    dev = 'cuda'
+    o, ht = _op()((q if l2norm_in_kernel else qn).to(dev), (k if l2norm_in_kernel else kn).to(dev), v.to(dev),
+                  g_raw.to(dev), beta.to(dev), scale=scale, initial_state=h0.to(dev), output_final_state=True,
+                  use_qk_l2norm_in_kernel=l2norm_in_kernel, use_gate_in_kernel=True, A_log=A_log.to(dev),
+                  dt_bias=None if dt_bias is None else dt_bias.to(dev))
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
 @torch.inference_mode()
 def test_reference_varlen_prefill_case_under_inference_mode():
     """tests/ops/test_gdn.py:806-876, its largest case: one packed sequence of 8192 tokens, D = 60, fp16
