@@ -91,6 +91,39 @@ def test_reference_matrix_with_the_reference_input_recipe(B, T, H, HV, D, scale,
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('B,T,H,HV,D,scale,has_dt_bias,neg_eigval,dtype', [
+    (1, 64, 1, 1, 64, 1, False, False, torch.float),
+    (2, 256, 2, 2, 64, 1, True, False, torch.float),
+    (2, 512, 2, 4, 64, 0.1, True, True, torch.float16),
+    (3, 1000, 2, 8, 128, 1, False, True, torch.float16),
+    (4, 1024, 4, 4, 128, 0.1, True, False, torch.float16),
+])
+def test_reference_in_kernel_gate_and_beta_matrices(B, T, H, HV, D, scale, has_dt_bias, neg_eigval, dtype):
+    """tests/ops/test_gdn.py:520-657: raw gates with A_log = log U(1, 16) and optional dt_bias activated in
+    the kernel, and beta logits squashed in the kernel (doubled with allow_neg_eigval), both on top of
+    the in-kernel l2 normalisation, against the oracle fed with the activated values.  Bar 0.002."""
+    gen = torch.Generator().manual_seed(42)
+    q = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    k = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    v = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    beta_logits = torch.randn(B, T, HV, generator=gen).to(dtype)
+    g_raw = torch.randn(B, T, HV, generator=gen)
+    A_log = torch.log(torch.empty(HV).uniform_(1, 16, generator=gen))
+    dt_bias = torch.randn(HV, generator=gen) if has_dt_bias else None
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    g_ref = -A_log.exp() * F.softplus(g_raw + (dt_bias if has_dt_bias else 0.0))
+    beta_ref = beta_logits.float().sigmoid() * (2.0 if neg_eigval else 1.0)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g_ref, beta_ref, scale, h0, True, use_qk_l2norm_in_kernel=True)
+    dev = 'cuda'
+    o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g_raw.to(dev), beta=beta_logits.to(dev), scale=scale,
+                   initial_state=h0.to(dev), output_final_state=True, use_qk_l2norm_in_kernel=True,
+                   use_gate_in_kernel=True, A_log=A_log.to(dev), dt_bias=None if dt_bias is None else dt_bias.to(dev),
+                   use_beta_sigmoid_in_kernel=True, allow_neg_eigval=neg_eigval)
+    ratio = RATIO if dtype == torch.float32 else 5e-3      # o itself is rounded to 16 bits
+    _check('o', ref_o, o, ratio)
+    _check('ht', ref_ht, ht)
+
+
 def test_decode_shape_inplace_and_chained_steps():
     """N=64 decode steps with Hqk=16, Hv=32, K=V=128 (the decode configuration at a quarter
     of its batch): three chained single-token calls, state updated in place, must equal the
