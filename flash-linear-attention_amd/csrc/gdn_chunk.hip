@@ -32,13 +32,16 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
     if (p.flags & GDN_FLAG_SCAN_WIDE) segments = false;
     if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
     const bool no_pair = p.flags & GDN_FLAG_SCAN_NO_PAIR, force_pair = p.flags & GDN_FLAG_SCAN_PAIR;
+    // (full runs in pairs: an even number of value heads per q/k head, and all 128 value columns real: the two-run
+    // kernel counts its output stores, which every wave must therefore have)
+    const bool pair_full_ok = G % 2 == 0 && p.V == 128;
     auto use_pair = [&](bool possible, int64_t single_workgroups) {
         return possible && !no_pair && (force_pair || single_workgroups > 256);
     };
     SegmentPlan sp = {};
     if (!segments) {
         sp.kind = WIDE_WHOLE;
-        return use_pair(G % 2 == 0, p.NH) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
+        return use_pair(pair_full_ok, p.NH) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
     }
     sp.nseg = nseg;
     sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
@@ -51,13 +54,13 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
     if ((rc = use_pair(true, 2 * p.NH * (nseg - 1)) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream))) return rc;
     if ((rc = launch_segment_merge(p, sp, stream))) return rc;
     sp.kind = WIDE_PASS2;
-    return use_pair(G % 2 == 0, p.NH * nseg) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
+    return use_pair(pair_full_ok, p.NH * nseg) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
 }
 
 }  // namespace gdn
 
 extern "C" size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V) {
-    if (K != 128 || V != 128 || num_chunks < 0 || H < 1 || HV < 1) return 0;
+    if (K < 8 || V < 8 || K > 128 || V > 128 || K % 8 || V % 8 || num_chunks < 0 || H < 1 || HV < 1) return 0;
     return gdn::ws_layout(num_chunks, H, HV, nullptr, nullptr);
 }
 
@@ -78,8 +81,8 @@ static int chunk_entry(
     GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_SCAN_NO_PAIR) || !(flags & GDN_FLAG_SCAN_PAIR), GDN_ERR_INVALID, "%s: GDN_FLAG_SCAN_PAIR and GDN_FLAG_SCAN_NO_PAIR exclude each other", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
-    GDN_CHECK_ARG(K == 128 && V == 128, GDN_ERR_UNSUPPORTED, "%s: only K = V = 128 is built (got K=%lld V=%lld)", who,
-                  (long long)K, (long long)V);
+    GDN_CHECK_ARG(K >= 8 && V >= 8 && K <= 128 && V <= 128 && K % 8 == 0 && V % 8 == 0, GDN_ERR_UNSUPPORTED,
+                  "%s: head dims must be multiples of 8 up to 128 (got K=%lld V=%lld)", who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
                   "%s: q/k/v must be bf16 or f16", who);
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * H < (1ll << 31), GDN_ERR_UNSUPPORTED, "%s: too many heads or chunks for one launch", who);
@@ -100,7 +103,7 @@ static int chunk_entry(
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
-    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH; p.K = (int)K; p.V = (int)V;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.NH = N * HV;
     hipStream_t s = (hipStream_t)stream;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, stages, s)

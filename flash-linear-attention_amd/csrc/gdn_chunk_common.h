@@ -118,6 +118,7 @@ struct ChunkParams {
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     ChunkWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;       // NT: chunks per sequence (dense input)
+    int K, V;                                          // head dims of the caller's tensors (multiples of 8, <= 128)
     float scale; int gb_dtype; uint32_t flags;
     int64_t NH;
 };
@@ -145,6 +146,21 @@ __device__ __forceinline__ void gather_1k_to_lds(const char* gbase, uint32_t vof
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
     const uint64_t gs = ((uint64_t)hi << 32) | lo;
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(voff), "s"(gs));
+}
+
+// The same copy for the lanes named by `mask` only (the others leave their 16 bytes of LDS as they are).
+// The instruction is issued whatever the mask, so counts of outstanding operations do not depend on it.
+__device__ __forceinline__ void gather_1k_to_lds_masked(const char* gbase, uint32_t voff, uint32_t lds_off, uint64_t mask) {
+    lds_off = __builtin_amdgcn_readfirstlane(lds_off);
+    const uint64_t g = (uint64_t)gbase;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+    const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    uint64_t saved;
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_and_saveexec_b64 %0, %4\n\t"
+                 "global_load_lds_dwordx4 %2, %3\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved) : "s"(lds_off), "v"(voff), "s"(gs), "s"(mask) : "scc");
 }
 
 template <int N>

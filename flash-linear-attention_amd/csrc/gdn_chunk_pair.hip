@@ -46,8 +46,11 @@ __device__ __forceinline__ void store16_masked(const char* sbase, uint32_t voff,
                  : "=&s"(saved) : "s"(mask), "v"(voff), "v"(d), "s"(gs) : "memory", "scc");
 }
 
-template <typename T, bool FULL>
+template <typename T, bool FULL, bool DIMS128>
 __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParams p, SegmentPlan sp) {
+    // Head dims: DIMS128 fixes K = V = 128 at compile time (every copy is whole, nothing is masked); otherwise they
+    // are the caller's multiples of 8 and the tiles' features past them are zero (q, k) or never stored (v, o, state).
+    const int K = DIMS128 ? 128 : p.K, V = DIMS128 ? 128 : p.V;
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
@@ -77,8 +80,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         if (p.flags & GDN_FLAG_SEQ_ORDER) n = load_index(p.chunk_offsets, p.N + 1 + n, cu32);
         h = (int)(group % H); hv = h * G + 2 * (int)(slot % mem) + tm; seg = 0;
         const int64_t inh = n * HV + hv;
-        src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true;
-        dst = p.ht ? p.ht + inh * 16384 : nullptr; dst_user = true;
+        src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true;
+        dst = p.ht ? p.ht + inh * (int64_t)(K * V) : nullptr; dst_user = true;
     } else if (sp.kind == WIDE_PASS1) {
         const int64_t group = (slot / G) * 8 + xcd;                   // (sequence, q/k head, segment 0 .. nseg-2)
         if (group >= p.N * H * (sp.nseg - 1)) return;
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         n = nh / H; h = (int)(nh % H); hv = h * G + (int)(slot % G);
         const int64_t inh = n * HV + hv;
         if (tm == 0) {
-            if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
+            if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
             else init = 2;
             dst = sp.sloc + (inh * sp.nseg + seg) * 16384;
         } else {
@@ -103,9 +106,9 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         seg = (int)(group % sp.nseg);
         n = nh / H; h = (int)(nh % H); hv = h * G + 2 * (int)(slot % mem) + tm;
         const int64_t inh = n * HV + hv;
-        if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
+        if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
         else src = sp.sin + (inh * sp.nseg + seg) * 16384;
-        if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * 16384; dst_user = true; }
+        if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * (int64_t)(K * V); dst_user = true; }
     }
 
     int64_t bos, len, boh;
@@ -131,7 +134,11 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     // =====================================================================================
     const bool vz = __builtin_amdgcn_readfirstlane((int)v_zero) != 0;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-    const uint32_t rowB_qk = (uint32_t)H * 256, rowB_v = (uint32_t)HV * 256;
+    // rows of the caller's tensors hold K (q, k) or V (v, o) elements, multiples of 8 up to 128.  Pieces of q and k
+    // past K stay zero in LDS (the tiles are cleared once, those lanes copy nothing); pieces of v past V re-read
+    // valid ones: value columns never mix, and the padded ones are never stored.
+    const uint32_t rowB_qk = (uint32_t)H * K * 2, rowB_v = (uint32_t)HV * V * 2;
+    const int k_pieces = K >> 3, v_pieces = V >> 3;
     // k and q tiles in LDS: 64 token rows x 256 B as 16 blocks of 4 rows (1 KB, one copy each).  In block j
     // the 16-byte piece c of row 4j + r sits in slot 16*(c/4) + 4r + ((c + j) & 3): four consecutive lanes
     // fetch 64 contiguous bytes of one row, and both the operand reads (16 rows x one piece) and the
@@ -145,23 +152,27 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         kq_row[e] = 4 * j + (c16 >> 2);
         kq_cb[e] = 16 * (4 * g + ((c16 - j) & 3));
     }
+    uint64_t kq_mask[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) kq_mask[e] = __builtin_amdgcn_ballot_w64((int)(kq_cb[e] >> 4) < k_pieces);
     auto issue_kq = [&](const T* tensor, int64_t c, uint32_t lds_tile) {            // 2 operations
         const int valid = (int)min((int64_t)CH, len - c * CH);
-        const char* base = (const char*)(tensor + ((bos + c * CH) * H + h) * 128);
+        const char* base = (const char*)(tensor + ((bos + c * CH) * H + h) * K);
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint32_t row = (uint32_t)min(kq_row[e], valid - 1);
-            gather_1k_to_lds(base, __umul24(row, rowB_qk) + kq_cb[e], lds_tile + (2 * w + e) * 1024);
+            if constexpr (DIMS128) gather_1k_to_lds(base, __umul24(row, rowB_qk) + kq_cb[e], lds_tile + (2 * w + e) * 1024);
+            else gather_1k_to_lds_masked(base, __umul24(row, rowB_qk) + kq_cb[e], lds_tile + (2 * w + e) * 1024, kq_mask[e]);
         }
     };
     // private v area: block b = rows 16b .. 16b+15 x this wave's 4 pieces (64 bytes of a row are
     // fetched by 4 consecutive lanes); piece pc of row r sits in slot 4r + pc, so the transpose reads
     // of a 16-lane group (4 rows x 4 pieces) cover 16 consecutive slots
     const int v_r16 = lane >> 2;
-    const uint32_t v_cb = 16 * (4 * cw + (lane & 3));
+    const uint32_t v_cb = 16 * ((4 * cw + (lane & 3)) % v_pieces);
     auto issue_v = [&](int64_t c, int half) {                                        // 2 operations
         const int valid = v_zero ? 1 : (int)min((int64_t)CH, len - c * CH);         // (a transition run reads no v: one row, from cache)
-        const char* base = (const char*)((const T*)p.v + ((bos + c * CH) * HV + hv) * 128);
+        const char* base = (const char*)((const T*)p.v + ((bos + c * CH) * HV + hv) * V);
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int b = 2 * half + e;
@@ -196,6 +207,11 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     constexpr int N_AFTER_VLO = FULL ? 13 : 5;        // the first half of v and its use in the next step
     constexpr int N_AFTER_VHI = FULL ? 11 : 5;        // the second half of v and its use in the next step
 
+    if (K < 128 && nsteps > 0) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int i = tid; i < (PR_V - PR_K) / 16; i += PAIR_THREADS) *(u32x4*)(smem + PR_K + i * 16) = z;
+        lds_barrier();
+    }
     if (nsteps > 0 && !active) {
         // a team with nothing to compute still fetches its share of k and of the record
         issue_kq((const T*)p.k, it0, lds0 + PR_K);
@@ -225,8 +241,13 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[r] = (kk + r == vc) ? 1.f : 0.f;
         } else if (init == 0 && src) {
-            if (src_user && vfirst) s = *(const f32x4*)(src + vc * 128 + kk);
-            else s = f32x4{src[kk * 128 + vc], src[(kk + 1) * 128 + vc], src[(kk + 2) * 128 + vc], src[(kk + 3) * 128 + vc]};
+            // the caller's state is [K][V] or [V][K] with rows and columns past K, V counting as zero; the buffers
+            // of the segment passes are [128][128]: one strided form serves all three
+            const int sk = src_user ? (vfirst ? 1 : V) : 128, sv = src_user ? (vfirst ? K : 1) : 1;
+            if (kk < (src_user ? K : 128) && vc < (src_user ? V : 128)) {
+                const float* e = src + kk * sk + vc * sv;
+                s = f32x4{e[0], e[sk], e[2 * sk], e[3 * sk]};
+            }
         }
         S[m][nn] = s;
     }
@@ -247,7 +268,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     char* ot = smem + PR_OT + w * 1024;
     const int ot_w = (4 * c16 + ((g + (c16 >> 2)) & 3)) * 16;
     const int o_row = lane >> 2;
-    const uint32_t o_voff = (uint32_t)o_row * rowB_v + 64 * cw + 16 * (((lane & 3) - (o_row >> 2)) & 3);
+    const int o_piece = 4 * cw + (((lane & 3) - (o_row >> 2)) & 3);        // 16-byte piece of the output row this lane stores
+    const uint32_t o_voff = (uint32_t)o_row * rowB_v + 16 * o_piece;
 
     // One step: the regions of the four-wave kernel, plus this wave's copies and stores.
     auto step = [&](int64_t i) {
@@ -262,7 +284,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         const char* sX = rec + REC_X;
         const char* sP = rec + REC_P;
         const float* sTab = (const float*)(rec + REC_TAB);
-        const char* obase = (const char*)p.o + ((bos + it * CH) * HV + hv) * 256;
+        const char* obase = (const char*)p.o + ((bos + it * CH) * HV + hv) * (int64_t)(V * 2);
         const int valid = (int)min((int64_t)CH, len - it * CH);
         auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
@@ -364,7 +386,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
                 const u32x2 lo = __builtin_bit_cast(u32x2, o4[0]), hi = __builtin_bit_cast(u32x2, o4[1]);
                 *(u32x4*)(ot + ot_w) = u32x4{lo[0], lo[1], hi[0], hi[1]};
                 const u32x4 orow = *(const u32x4*)(ot + lane * 16);       // (LDS operations of a wave execute in order)
-                store16_masked(ob, o_voff, orow, __builtin_amdgcn_ballot_w64(16 * tt + o_row < valid));
+                store16_masked(ob, o_voff, orow, __builtin_amdgcn_ballot_w64(16 * tt + o_row < valid && o_piece < v_pieces));
             }
         };
         auto U = [&](int sp2, int m) {
@@ -447,23 +469,30 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         for (int nn = 0; nn < NN; ++nn) {
             const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 32 * cw + 8 * (c16 >> 2) + 4 * nn + (c16 & 3);
             const f32x4 s = S[m][nn] * gamma;
-            if (dst_user && vfirst) *(f32x4*)(dst + vc * 128 + kk) = s;
-            else {
+            const int sk = dst_user ? (vfirst ? 1 : V) : 128, sv = dst_user ? (vfirst ? K : 1) : 1;
+            if (kk < (dst_user ? K : 128) && vc < (dst_user ? V : 128)) {
+                float* e = dst + kk * sk + vc * sv;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) dst[(kk + r) * 128 + vc] = s[r];
+                for (int r = 0; r < 4; ++r) e[r * sk] = s[r];
             }
         }
     }
 }
 
-template <typename T, bool FULL>
-static int launch_pair_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
-    auto kern = gdn_chunk_pair_kernel<T, FULL>;
+template <typename T, bool FULL, bool DIMS128>
+static int launch_pair_dims(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
+    auto kern = gdn_chunk_pair_kernel<T, FULL, DIMS128>;
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, PAIR_SMEM, attr_done, "hipFuncSetAttribute(pair)")) return rc;
     if (blocks <= 0) return GDN_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(PAIR_THREADS), PAIR_SMEM, stream, p, sp);
     return check_launch("gdn_chunk_pair_kernel");
+}
+
+template <typename T, bool FULL>
+static int launch_pair_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
+    return p.K == 128 && p.V == 128 ? launch_pair_dims<T, FULL, true>(p, sp, blocks, stream)
+                                    : launch_pair_dims<T, FULL, false>(p, sp, blocks, stream);
 }
 
 // sp.kind selects the work: whole sequences and pass 2 need an even number of value heads per

@@ -63,17 +63,19 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         rb = load_scalar(p.beta, (tok0 + lane) * HV + h * G + w, p.gb_dtype);
     }
     {
-        const T* kg = (const T*)p.k + (tok0 * H + h) * 128;
-        const T* qg = (const T*)p.q + (tok0 * H + h) * 128;
+        // (key features past K are zero, like the rows past the end: the tiles are always 64 x 128)
+        const int K = p.K;
+        const T* kg = (const T*)p.k + (tok0 * H + h) * K;
+        const T* qg = (const T*)p.q + (tok0 * H + h) * K;
         u32x4 rk[4], rq[4];
 #pragma unroll
         for (int ps = 0; ps < 4; ++ps) {
             const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
             const u32x4 z = {0u, 0u, 0u, 0u};
             rk[ps] = rq[ps] = z;
-            if (row < valid) {
-                rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * 128 + col);
-                rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * 128 + col);
+            if (row < valid && col < K) {
+                rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * K + col);
+                rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
             }
         }
         const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;

@@ -57,8 +57,11 @@ constexpr int WIDE_NN = 2;                        // 16-column tiles per compute
 constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
 
-template <typename T, bool FULL>
+template <typename T, bool FULL, bool DIMS128>
 __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParams p, SegmentPlan sp) {
+    // Head dims: DIMS128 fixes K = V = 128 at compile time (every copy is whole, nothing is masked); otherwise they
+    // are the caller's multiples of 8 and the tiles' features past them are zero (q, k) or never stored (v, o, state).
+    const int K = DIMS128 ? 128 : p.K, V = DIMS128 ? 128 : p.V;
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
@@ -89,8 +92,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         int64_t nseq = group / H;
         if (p.flags & GDN_FLAG_SEQ_ORDER) nseq = load_index(p.chunk_offsets, p.N + 1 + nseq, cu32);     // longest sequences start first
         inh = nseq * HV + (group % H) * G + slot % G; seg = 0;
-        src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true;
-        dst = p.ht ? p.ht + inh * 16384 : nullptr; dst_user = true;
+        src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true;
+        dst = p.ht ? p.ht + inh * (int64_t)(K * V) : nullptr; dst_user = true;
     } else if (sp.kind == WIDE_PASS1) {
         // group = (sequence, q/k head, segment 0 .. nseg-2); members: S runs of its value heads, then M runs
         const int64_t group = (slot / (2 * G)) * 8 + xcd;
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         seg = (int)(group % (sp.nseg - 1));
         inh = (nh / H) * HV + (nh % H) * G + member % G;
         if (member < G) {
-            if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
+            if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
             else init = 2;
             dst = sp.sloc + (inh * sp.nseg + seg) * 16384;
         } else {
@@ -114,9 +117,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const int64_t nh = group / sp.nseg;
         seg = (int)(group % sp.nseg);
         inh = (nh / H) * HV + (nh % H) * G + slot % G;
-        if (seg == 0) { src = p.h0 ? p.h0 + inh * 16384 : nullptr; src_user = true; }
+        if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
         else src = sp.sin + (inh * sp.nseg + seg) * 16384;
-        if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * 16384; dst_user = true; }
+        if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * (int64_t)(K * V); dst_user = true; }
     }
     const int64_t n = inh / HV;
     const int hv = (int)(inh % HV);
@@ -148,22 +151,48 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // chunk it+1 must have landed at B2.  Loads complete in issue order, so "at most
     // N operations outstanding" proves that all but the N newest have landed.
     // =====================================================================================
+    if (K < 128 && nsteps > 0) {
+        // key features past K: clear the q and k tiles once; the copies never touch those pieces
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int i = tid; i < (2 * 16384) / 16; i += WIDE_THREADS) {
+            *(u32x4*)(smem + (i >> 10) * STG_BYTES + STG_Q + (i & 1023) * 16) = z;
+        }
+        for (int i = tid; i < (3 * 16384) / 16; i += WIDE_THREADS) *(u32x4*)(smem + KBUF + i * 16) = z;
+        lds_barrier();
+    }
     if (w >= CW) {
         if (nsteps <= 0) return;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
         // Block gather: rows 4j .. 4j+3 of a [token][head][128] tensor.  Rows past the end of the
         // sequence re-read its last row: whatever they hold is finite and is multiplied by the zero
         // columns of Xb, the zero rows of v_new and the causal zeros of P.
-        auto gather_blocks = [&](const T* tensor, int heads, int head, int64_t it, int j0, int j1, uint32_t lds_tile) {
+        // A copy wave moves one tensor: k (wave CW), q (CW+1) or v (CW+2), whose rows hold `dim` = K or V elements
+        // (a multiple of 8, <= 128).  Pieces of q and k past K stay zero in LDS (the tiles were cleared once and those
+        // lanes copy nothing); pieces of v past V re-read valid ones: value columns never mix, and the padded ones
+        // are never stored.  What a lane fetches depends on the block only through j % 4: prepared once.
+        const bool is_v = (w == CW + 2);
+        const int dim = is_v ? V : K, pieces = dim >> 3;
+        const int heads = is_v ? HV : H, head = is_v ? hv : h;
+        const uint32_t row_bytes = (uint32_t)(heads * dim * 2);
+        uint32_t piece_off[4];
+        uint64_t piece_mask[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int c = 4 * g + ((c16 - jj) & 3);                         // this lane's slot holds piece c of row 4j + r
+            piece_off[jj] = 16 * (is_v ? c % pieces : c);
+            piece_mask[jj] = __builtin_amdgcn_ballot_w64(is_v || c < pieces);
+        }
+        auto gather_blocks = [&](const T* tensor, int64_t it, int j0, int j1, uint32_t lds_tile) {
             const int64_t tok0 = bos + it * CH;
             const int valid = (int)min((int64_t)CH, len - it * CH);
-            const char* base = (const char*)(tensor + (tok0 * heads + head) * 128);
+            const char* base = (const char*)(tensor + (tok0 * heads + head) * dim);
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 if (j < j0 || j >= j1) continue;
-                const int r = c16 >> 2, c = 4 * g + ((c16 - j) & 3);        // this lane's slot holds piece c of row 4j + r
-                const int row = min(4 * j + r, valid - 1);
-                gather_1k_to_lds(base, (uint32_t)row * (uint32_t)(heads * 256) + 16 * c, lds_tile + j * 1024);
+                const int row = min(4 * j + (c16 >> 2), valid - 1);
+                const uint32_t voff = (uint32_t)row * row_bytes + piece_off[j & 3];
+                if constexpr (DIMS128) gather_1k_to_lds(base, voff, lds_tile + j * 1024);
+                else gather_1k_to_lds_masked(base, voff, lds_tile + j * 1024, piece_mask[j & 3]);
             }
         };
         auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage) {
@@ -176,7 +205,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             // ---- k: the copy of chunk i+2 is issued at the start of step i (its buffer was last read
             // in step i-1) and awaited at the end of step i+1 ----
             auto issue_k = [&](int64_t i) {                                 // i counts from the first chunk of this run
-                gather_blocks((const T*)p.k, H, h, min(it0 + i, lastc), 0, 16, lds0 + KBUF + (int)(i % 3) * 16384);
+                gather_blocks((const T*)p.k, min(it0 + i, lastc), 0, 16, lds0 + KBUF + (int)(i % 3) * 16384);
             };
             issue_k(0);
             issue_k(1);
@@ -198,15 +227,15 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 if (qside) {
                     if constexpr (FULL) {
                         // 16 q pieces, then Xb (5) and the tables (1)
-                        if (early) gather_blocks((const T*)p.q, H, h, it, 0, 8, st + STG_Q);
-                        else { gather_blocks((const T*)p.q, H, h, it, 8, 16, st + STG_Q); copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }
+                        if (early) gather_blocks((const T*)p.q, it, 0, 8, st + STG_Q);
+                        else { gather_blocks((const T*)p.q, it, 8, 16, st + STG_Q); copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }
                     } else {
                         if (early) { copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }      // all 6 pieces
                     }
                 } else {
-                    if (early) { if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 0, 8, st + STG_V); }      // (v is not read when it counts as zero)
+                    if (early) { if (!v_zero) gather_blocks((const T*)p.v, it, 0, 8, st + STG_V); }      // (v is not read when it counts as zero)
                     else {
-                        if (!v_zero) gather_blocks((const T*)p.v, HV, hv, it, 8, 16, st + STG_V);
+                        if (!v_zero) gather_blocks((const T*)p.v, it, 8, 16, st + STG_V);
                         if constexpr (FULL) copy_rec(it, REC_PIECES_X, REC_PIECES_X + REC_PIECES_P, st);
                     }
                 }
@@ -236,12 +265,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             u32x4 orow[16];                                                 // output tile of the previous chunk
             auto store_rows = [&](int64_t it) {
                 const int valid = (int)min((int64_t)CH, len - it * CH);
-                int64_t stride = (int64_t)HV * 128 * 4;                     // elements between rows 4 apart
+                int64_t stride = (int64_t)HV * V * 4;                     // elements between rows 4 apart
                 asm volatile("" : "+s"(stride));                            // keep the 16 row addresses out of long-lived registers
-                T* dstp = og + ((bos + it * CH + g) * HV + hv) * 128 + c16 * 8;
+                T* dstp = og + ((bos + it * CH + g) * HV + hv) * V + c16 * 8;
+                const bool col_ok = c16 * 8 < V;                          // (value columns past V exist in the tile only)
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
-                    if (4 * j + g < valid) *(u32x4*)dstp = orow[j];
+                    if (4 * j + g < valid && col_ok) *(u32x4*)dstp = orow[j];
                     dstp += stride;
                 }
             };
@@ -277,8 +307,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[r] = (kk + r == vc) ? 1.f : 0.f;
         } else if (init == 0 && src) {
-            if (src_user && vfirst) s = *(const f32x4*)(src + vc * 128 + kk);
-            else s = f32x4{src[kk * 128 + vc], src[(kk + 1) * 128 + vc], src[(kk + 2) * 128 + vc], src[(kk + 3) * 128 + vc]};
+            // the caller's state is [K][V] or [V][K] with rows and columns past K, V counting as zero; the buffers
+            // of the segment passes are [128][128]: one strided form serves all three
+            const int sk = src_user ? (vfirst ? 1 : V) : 128, sv = src_user ? (vfirst ? K : 1) : 1;
+            if (kk < (src_user ? K : 128) && vc < (src_user ? V : 128)) {
+                const float* e = src + kk * sk + vc * sv;
+                s = f32x4{e[0], e[sk], e[2 * sk], e[3 * sk]};
+            }
         }
         S[m][nn] = s;
     }
@@ -496,10 +531,11 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         for (int nn = 0; nn < NN; ++nn) {
             const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * (NN * w + nn) + c16;
             const f32x4 s = S[m][nn] * gamma;
-            if (dst_user && vfirst) *(f32x4*)(dst + vc * 128 + kk) = s;
-            else {
+            const int sk = dst_user ? (vfirst ? 1 : V) : 128, sv = dst_user ? (vfirst ? K : 1) : 1;
+            if (kk < (dst_user ? K : 128) && vc < (dst_user ? V : 128)) {
+                float* e = dst + kk * sk + vc * sv;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) dst[(kk + r) * 128 + vc] = s[r];
+                for (int r = 0; r < 4; ++r) e[r * sk] = s[r];
             }
         }
     }
@@ -584,14 +620,20 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, 
     }
 }
 
-template <typename T, bool FULL>
-static int launch_wide_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
-    auto kern = gdn_chunk_wide_kernel<T, FULL>;
+template <typename T, bool FULL, bool DIMS128>
+static int launch_wide_dims(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
+    auto kern = gdn_chunk_wide_kernel<T, FULL, DIMS128>;
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, WIDE_SMEM, attr_done, "hipFuncSetAttribute(wide)")) return rc;
     if (blocks <= 0) return GDN_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WIDE_THREADS), WIDE_SMEM, stream, p, sp);
     return check_launch("gdn_chunk_wide_kernel");
+}
+
+template <typename T, bool FULL>
+static int launch_wide_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
+    return p.K == 128 && p.V == 128 ? launch_wide_dims<T, FULL, true>(p, sp, blocks, stream)
+                                    : launch_wide_dims<T, FULL, false>(p, sp, blocks, stream);
 }
 
 // sp.kind selects the work (whole sequences, pass 1 or pass 2 of the segment-parallel evaluation)

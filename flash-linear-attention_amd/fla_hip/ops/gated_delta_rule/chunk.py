@@ -75,10 +75,14 @@ class ChunkLaunch:
         # the MFMA kernels take bf16 or fp16 operands; fp32 inputs are rounded to bf16 first
         work_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
         q, k, v = q.to(work_dtype), k.to(work_dtype), v.to(work_dtype)
-        # head dims below 128 are zero-padded: zero key features and zero value columns change
-        # neither the other columns of the output nor the state entries that are kept
+        # The kernels take head dims that are multiples of 8 up to 128 as they are.  Others are
+        # zero-padded to 128 here: zero key features and zero value columns change neither the
+        # other columns of the output nor the state entries that are kept.
         KP, VP = _kernel_dim(K), _kernel_dim(V)
-        KP = VP = max(KP, VP)
+        if K % 8 == 0 and V % 8 == 0:
+            KP, VP = K, V
+        else:
+            KP = VP = max(KP, VP)
         self.padded = (KP, VP)
         q, k, v = _pad_last(q, KP), _pad_last(k, KP), _pad_last(v, VP)
         g, beta, gb_code = unify_gate_beta(g, beta)

@@ -117,7 +117,9 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  *         With GDN_FLAG_SEQ_ORDER the array has N more entries: the sequence ids in the order in
  *         which the sequential kernel should start them (longest first keeps the CUs evenly loaded)
  *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
- *   Requires K == V == 128, HV % H == 0 (the Python host zero-pads smaller head dims).
+ *   Requires K, V multiples of 8 up to 128 and HV % H == 0.  The kernels work on 128 x 128 states: key features past K
+ *   count as zero and value columns past V are not stored (same time as K = V = 128; the Python host zero-pads
+ *   head dims that are not multiples of 8).
  */
 int gdn_chunk_fwd(
     const void* q, const void* k, const void* v, const void* g, const void* beta,

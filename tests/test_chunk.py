@@ -162,6 +162,45 @@ def test_reference_gate_in_kernel_matrix_with_the_reference_input_recipe(B, T, H
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('mode', ['auto', 'wide-single', 'wide-pair', 'segments-single', 'segments-pair'])
+@pytest.mark.parametrize('B,T,H,HV,K,V,vfirst,cu', [
+    (2, 1100, 2, 4, 64, 64, False, None),
+    (1, 1300, 2, 2, 32, 96, True, None),
+    (2, 900, 1, 2, 128, 64, False, None),
+    (1, 2000, 2, 4, 64, 128, True, [0, 15, 100, 300, 1200, 2000]),
+    (1, 777, 2, 4, 8, 8, False, None),
+])
+def test_head_dims_that_are_multiples_of_8_go_to_the_kernels_as_they_are(monkeypatch, mode, B, T, H, HV, K, V, vfirst, cu):
+    """No padded copies on the host: the kernels read rows of K or V elements, keep key features past K at
+    zero and never store value columns past V.  Guard rows and columns around the outputs stay untouched."""
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
+    N = B if cu is None else len(cu) - 1
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=17, gate_div=8.0, h0_std=0.5, N=N, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)
+    from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
+    from fla_hip.ops.gated_delta_rule._common import ptr
+    dev = 'cuda'
+    hs = (h0.transpose(-1, -2) if vfirst else h0).contiguous().to(dev)
+    cu_t = None if cu is None else torch.tensor(cu, device=dev)
+    call = ChunkLaunch(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta.to(dev), K ** -0.5, hs, True, vfirst, cu_t)
+    assert call.padded == (K, V)
+    # the outputs sit inside larger buffers filled with a guard value
+    o_big = torch.full((B * T * HV * V + 256,), 7.0, dtype=torch.bfloat16, device=dev)
+    h_big = torch.full((N * HV * K * V + 256,), 7.0, dtype=torch.float32, device=dev)
+    args = list(call.args)
+    assert args[9] == ptr(call.o) and args[8] == ptr(call.ht)
+    args[9], args[8] = o_big.data_ptr() + 128 * 2, h_big.data_ptr() + 128 * 4
+    call.args = tuple(args)
+    call.run()
+    torch.cuda.synchronize()
+    o = o_big[128:128 + B * T * HV * V].view(B, T, HV, V)
+    ht = h_big[128:128 + N * HV * K * V].view((N, HV, V, K) if vfirst else (N, HV, K, V))
+    assert torch.all(o_big[:128] == 7.0) and torch.all(o_big[-128:] == 7.0), 'output guard overwritten'
+    assert torch.all(h_big[:128] == 7.0) and torch.all(h_big[-128:] == 7.0), 'state guard overwritten'
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht.transpose(-1, -2) if vfirst else ht)
+
+
 @torch.inference_mode()
 def test_reference_varlen_prefill_case_under_inference_mode():
     """tests/ops/test_gdn.py:806-876, its largest case: one packed sequence of 8192 tokens, D = 60, fp16
