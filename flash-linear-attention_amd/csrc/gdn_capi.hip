@@ -11,5 +11,5 @@ void set_error(const char* fmt, ...) {
 }
 }  // namespace gdn
 
-extern "C" int gdn_hip_abi_version(void) { return 3; }
+extern "C" int gdn_hip_abi_version(void) { return 4; }
 extern "C" const char* gdn_last_error(void) { return gdn::g_err; }

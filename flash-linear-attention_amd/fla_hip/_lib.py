@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -32,6 +32,8 @@ FLAG_SEQ_ORDER = 1 << 19
 FLAG_SCAN_NO_PAIR = 1 << 20
 FLAG_SCAN_PAIR = 1 << 21
 
+ACT_NONE, ACT_SILU, ACT_SIGMOID = 0, 1, 2
+
 # name -> (restype, argtypes); one entry per declaration in include/gdn_hip.h
 SIGNATURES = {
     'gdn_hip_abi_version': (c_int, []),
@@ -45,6 +47,20 @@ SIGNATURES = {
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
         c_float, c_int, c_int, c_uint32, c_void_p]),
     'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
+    'gdn_causal_conv1d_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # x weight bias residual initial_state
+        c_void_p, c_void_p, c_void_p,                      # y final_state cu_seqlens
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T D W N stride_x_n stride_x_t
+        c_int, c_int, c_int, c_int, c_uint32, c_void_p]),  # x_dtype w_dtype state_dtype activation flags stream
+    'gdn_causal_conv1d_update': (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # x cache residual weight bias y
+        c_int64, c_int64, c_int64, c_int64, c_int64,       # N D W stride_x_n stride_y_n
+        c_int, c_int, c_int, c_int, c_void_p]),            # x_dtype w_dtype cache_dtype activation stream
+    'gdn_norm_gated_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # x g weight bias residual
+        c_void_p, c_void_p, c_void_p, c_void_p,            # y residual_out mean rstd
+        c_int64, c_int64, c_float,                         # T D eps
+        c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),   # x/w/res/res_out dtype, activation, is_rms_norm, stream
 }
 _CHUNK_ARGS = [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # q k v g beta

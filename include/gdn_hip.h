@@ -50,6 +50,11 @@ extern "C" {
 #define GDN_FLAG_SCAN_NO_PAIR   (1u << 20) /* always one run per workgroup                      */
 #define GDN_FLAG_SCAN_PAIR      (1u << 21) /* two runs per workgroup wherever two can share k rows */
 
+/* activation codes of the convolution and normalisation entry points */
+#define GDN_ACT_NONE    0
+#define GDN_ACT_SILU    1   /* swish / silu: x * sigmoid(x)                                  */
+#define GDN_ACT_SIGMOID 2   /* gate of the normalisation only                                */
+
 /* Library ABI version (bumped on any signature change). */
 int gdn_hip_abi_version(void);
 
@@ -159,6 +164,62 @@ int gdn_chunk_fwd_scan(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
+ * The two memory-bound steps either side of the operator in the layer
+ * (fla/layers/gated_deltanet.py:246-300 and :355-359).
+ *
+ * Causal depthwise convolution over [token][channel] rows, prefill form.  Replaces causal_conv1d_fwd
+ * (fla/modules/conv/triton/ops.py:37-96: kernel fla/modules/conv/triton/kernels.py:37-139 and, for
+ * final_state, causal_conv1d_update_states, kernels.py:520-631).
+ *
+ *   y[t,d] = act(sum_{j<W} weight[d,j] * x[t-(W-1)+j, d] + bias[d]) + residual[t,d]
+ *
+ *   x        [B,T,D] x_dtype, rows stride_x_t elements apart, batches stride_x_n apart, channels adjacent
+ *            (a slice of a wider projection is read in place)
+ *   weight   [D,W] w_dtype; bias [D] w_dtype or NULL; residual [B,T,D] x_dtype contiguous or NULL
+ *   initial_state [N,D,W] state_dtype or NULL: inputs before the start of each sequence (entry W-1 is the newest;
+ *            entry 0 is never read, as in the reference)
+ *   y        [B,T,D] x_dtype contiguous, or NULL (only the state is wanted: weight may then be NULL too);
+ *            final_state [N,D,W] x_dtype or NULL (not stored): the last W inputs of
+ *            each sequence, reaching back into initial_state (or zero) when the sequence is shorter
+ *   cu_seqlens [N+1] or NULL (int64, or int32 with GDN_FLAG_CU_INT32); with it B must be 1; tokens outside
+ *            [cu_seqlens[0], cu_seqlens[N]) are not written
+ *   activation GDN_ACT_NONE or GDN_ACT_SILU.  Requires 1 <= W <= 8.
+ */
+int gdn_causal_conv1d_fwd(
+    const void* x, const void* weight, const void* bias, const void* residual, const void* initial_state,
+    void* y, void* final_state, const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t D, int64_t W, int64_t N, int64_t stride_x_n, int64_t stride_x_t,
+    int x_dtype, int w_dtype, int state_dtype, int activation, uint32_t flags, void* stream);
+
+/*
+ * The same convolution for one new token per sequence (decode).  Replaces causal_conv1d_update
+ * (fla/modules/conv/triton/ops.py:301-363, kernel fla/modules/conv/triton/kernels.py:356-421).
+ *   x, y   N rows of D channels, rows stride_x_n / stride_y_n elements apart, x_dtype
+ *   cache  [N,D,W] cache_dtype, updated IN PLACE: entries move one place towards 0 and x becomes entry W-1.
+ *          NULL: the window counts as zero (x included), as in the reference kernel without a cache
+ *   weight [D,W] w_dtype or NULL (taps of 1); bias [D] w_dtype or NULL; residual [N,D] x_dtype or NULL
+ */
+int gdn_causal_conv1d_update(
+    const void* x, void* cache, const void* residual, const void* weight, const void* bias, void* y,
+    int64_t N, int64_t D, int64_t W, int64_t stride_x_n, int64_t stride_y_n,
+    int x_dtype, int w_dtype, int cache_dtype, int activation, void* stream);
+
+/*
+ * Layer / RMS normalisation of rows of D features with an output gate.  Replaces layer_norm_gated_fwd
+ * (fla/modules/fused_norm_gate.py:456-538, kernels :36-108 and :125-189).
+ *   r = x + residual ; y = (r - mean) * rstd * weight + bias ; y *= g * sigmoid(g) (GDN_ACT_SILU) or sigmoid(g)
+ *   with rstd = 1/sqrt(var + eps); is_rms_norm != 0: mean = 0 and var = mean(r^2)
+ *   x, g, y [T,D] x_dtype contiguous; weight, bias [D] w_dtype or NULL; residual [T,D] res_dtype or NULL;
+ *   residual_out [T,D] res_out_dtype or NULL (r is not stored); mean, rstd [T] fp32 or NULL (not stored)
+ *   Requires D * sizeof(element) < 64 KB.
+ */
+int gdn_norm_gated_fwd(
+    const void* x, const void* g, const void* weight, const void* bias, const void* residual,
+    void* y, void* residual_out, float* mean, float* rstd,
+    int64_t T, int64_t D, float eps,
+    int x_dtype, int w_dtype, int res_dtype, int res_out_dtype, int activation, int is_rms_norm, void* stream);
 
 #ifdef __cplusplus
 }
