@@ -1,17 +1,18 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|calib_copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|layer_steps|calib_copy]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
 configuration the >= 50 %-of-MFMA-roofline target is quoted on.  A step is one call of
 chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries, under
-"other_workloads", the decode step (B=256: us/step and state GB/s) and the other prefill
-configurations, and:
+"other_workloads", the decode step (B=256: us/step and state GB/s), the other prefill
+configurations and the layer's two memory-bound steps either side of the operator (causal
+convolution, gated norm), and:
   roofline      dominant stage (the launches of one C entry point), algorithmic FLOPs (or bytes)
                 per call / its mean duration measured with HIP events on the launch stream
   cpu_baseline  the CPU oracle (torch fp32, all host cores) on a bounded sample of the workload
---workload calib_copy runs a plain 1 GiB device copy: the kernel of known size against which the
+--workload layer_steps runs only the convolution and the gated norm; --workload calib_copy runs a plain 1 GiB device copy: the kernel of known size against which the
 FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled.
 """
 from __future__ import annotations
@@ -42,7 +43,7 @@ F_PREP = F_TOTAL - F_SCAN                              # 49152
 # HBM bytes per call of the dominant stage on the default workload, from FETCH_SIZE + WRITE_SIZE of
 # a counter run of this file scaled by the calib_copy workload (profiles/ holds the summary); other
 # workloads: not measured
-TRAFFIC_BYTES = {'prefill': 1.52e9}
+TRAFFIC_BYTES = {'prefill': 1.52e9, 'conv_qkv': 1.0743e9, 'norm_gate': 0.8097e9}
 PEAK_BF16_TFLOPS = 2500.0                      # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0                          # MI355X HBM3E, published
 
@@ -219,6 +220,67 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     return out
 
 
+def _time_calls(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    return elapsed / steps, statistics.mean(ev[i].elapsed_time(ev[i + 1]) for i in range(steps)) * 1e-3
+
+
+def bench_layer_steps(steps, warmup, device, with_cpu):
+    """The two memory-bound steps either side of the operator in the layer at the default prefill size: the causal
+    convolution (+ SiLU) over the joined q|k|v projection (8192 channels, kernel size 4) and the gated RMS norm over
+    the 32 value heads of 128 features.  Algorithmic bytes: every input element read once, every output written once."""
+    from fla_hip.modules import causal_conv1d, rms_norm_gated
+    T, H, HV, W = 32768, 16, 32, 4
+    D = 2 * H * K + HV * V
+    gen = torch.Generator(device=device).manual_seed(42)
+    x = torch.randn(1, T, D, generator=gen, device=device).bfloat16()
+    wt = torch.randn(D, W, generator=gen, device=device).bfloat16()
+    o = torch.randn(T * HV, V, generator=gen, device=device).bfloat16()
+    gate = torch.randn(T * HV, V, generator=gen, device=device).bfloat16()
+    wn = torch.randn(V, generator=gen, device=device).bfloat16()
+    out = {}
+    cases = (('conv_qkv', 'causal_conv1d_fwd_kernel', 2 * T * D * 2,
+              f'causal conv + SiLU, T={T}, {D} channels (q|k|v), kernel size {W}, bf16',
+              lambda: causal_conv1d(x, wt, activation='silu')),
+             ('norm_gate', 'norm_gated_rows_kernel', 3 * T * HV * V * 2,
+              f'gated RMS norm (swish), {T}x{HV} rows of {V} features, bf16',
+              lambda: rms_norm_gated(o, gate, wn, None, 'swish', eps=1e-5)))
+    for key, kernel, nbytes, name, fn in cases:
+        wall, t_kernel = _time_calls(fn, steps, warmup)
+        achieved = nbytes / t_kernel / 1e9
+        out[key] = dict(workload=name, ms_per_step=round(wall * 1e3, 4), tokens_per_s=round(T / wall, 1),
+                        roofline=dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
+                                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=TRAFFIC_BYTES[key], kernel=kernel,
+                                      kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=nbytes))
+    if with_cpu:
+        from oracle import modules_oracle as MO
+        torch.set_num_threads(os.cpu_count() or 1)
+        Ts = 2048                                      # bounded sample: the first 2048 tokens
+        xs, ws = x[:, :Ts].cpu(), wt.cpu()
+        t0 = time.perf_counter()
+        MO.causal_conv1d(xs, ws, activation='silu')
+        t = time.perf_counter() - t0
+        out['conv_qkv']['cpu_baseline'] = dict(value=round(Ts / t, 1), unit='tokens/s', cores=torch.get_num_threads(), kind='port',
+                                               sample=f'oracle causal_conv1d (torch fp32 CPU) on the first {Ts} tokens', seconds=round(t, 2))
+        os_, gs = o[:Ts * HV].cpu(), gate[:Ts * HV].cpu()
+        t0 = time.perf_counter()
+        MO.norm_gated(os_, gs, wn.cpu(), None, None, 1e-5, 'swish', True)
+        t = time.perf_counter() - t0
+        out['norm_gate']['cpu_baseline'] = dict(value=round(Ts / t, 1), unit='tokens/s', cores=torch.get_num_threads(), kind='port',
+                                                sample=f'oracle norm_gated (torch fp32 CPU) on the first {Ts} tokens', seconds=round(t, 2))
+    return out
+
+
 def calib_copy(steps, warmup, device):
     """A plain device-to-device copy of 1 GiB (reads 1 GiB, writes 1 GiB per launch)."""
     n = 1 << 30
@@ -241,7 +303,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=20)
     ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['calib_copy'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['layer_steps', 'calib_copy'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     args = ap.parse_args()
@@ -256,6 +318,10 @@ def main():
 
     if args.workload == 'calib_copy':
         calib_copy(args.steps, args.warmup, device)
+        return
+    if args.workload == 'layer_steps':
+        print(json.dumps(dict(metric='gdn_layer_steps', steps=args.steps, warmup=args.warmup, dtype='bf16', data='synthetic',
+                              **bench_layer_steps(args.steps, args.warmup, device, not args.no_cpu_baseline))))
         return
     for key, val in WORKLOADS.items():
         val['key'] = key
@@ -288,6 +354,7 @@ def main():
                 e['cpu_baseline'] = r['cpu_baseline']
             extra[name] = e
             torch.cuda.empty_cache()
+        extra.update(bench_layer_steps(args.steps, args.warmup, device, not args.no_cpu_baseline))
         line['other_workloads'] = extra
     print(json.dumps(line))
 

@@ -7,14 +7,14 @@
 // for pos = -1 .. -(W-1)) or zero.  Three kernels: prefill (causal_conv1d_fwd_kernel,
 // fla/modules/conv/triton/kernels.py:37-139), the state left behind by a prefill
 // (causal_conv1d_states_fwd_kernel, :520-582) and the one-token update of that state for decode
-// (causal_conv1d_update_kernel, :356-421).  All three stream memory once: a thread owns 16 bytes of
-// channels and walks down the tokens with the last W-1 rows in registers.
+// (causal_conv1d_update_kernel, :356-421).  All three stream memory once.
 #include "gdn_common.h"
 
 namespace gdn {
 
-constexpr int CONV_TOKENS = 32;        // tokens a thread walks through
-constexpr int CONV_MAX_W = 8;          // widest kernel held in registers
+constexpr int CONV_TOKENS = 8;         // tokens per thread (measured against 4 and 16: best)
+constexpr int CONV_BX = 64, CONV_BY = 4;     // a workgroup: 64 channel groups x 4 token tiles (against 128 x 2, 256 x 1: best)
+constexpr int CONV_MAX_W = 8;          // widest kernel
 
 struct ConvParams {
     const void* x; const void* weight; const void* bias; const void* residual; const void* initial_state;
@@ -22,35 +22,8 @@ struct ConvParams {
     int64_t B, T, D, N, total;         // total = B*T tokens
     int64_t stride_n, stride_t;        // of x, in elements (channel stride is 1)
     int W, w_dtype, state_dtype, act;
-    bool cu32, vec_ok;
+    bool cu32;
 };
-
-template <typename T, int VEC>
-__device__ __forceinline__ void load_row(const T* p, int c0, int D, bool vec_ok, float (&out)[VEC]) {
-    if (vec_ok) {
-        typedef T vec_t __attribute__((ext_vector_type(VEC)));
-        const vec_t v = *(const vec_t*)p;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) out[e] = (float)v[e];
-    } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) out[e] = c0 + e < D ? (float)p[e] : 0.f;
-    }
-}
-
-template <typename T, int VEC>
-__device__ __forceinline__ void store_row(T* p, int c0, int D, bool vec_ok, const float (&in)[VEC]) {
-    if (vec_ok) {
-        typedef T vec_t __attribute__((ext_vector_type(VEC)));
-        vec_t v;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] = (T)in[e];
-        *(vec_t*)p = v;
-    } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) if (c0 + e < D) p[e] = (T)in[e];
-    }
-}
 
 // Sequence that holds global token `gt` (packed input): the last n with cu[n] <= gt.
 __device__ __forceinline__ int64_t find_sequence(const void* cu, int64_t N, int64_t gt, bool cu32) {
@@ -62,12 +35,23 @@ __device__ __forceinline__ int64_t find_sequence(const void* cu, int64_t N, int6
     return lo;
 }
 
-// blockDim = (64 channel pieces, 4 token tiles); grid = (pieces / 64, tiles / 4)
-template <typename T, int W>
+template <typename T> struct dtype_of { static constexpr int value = GDN_DTYPE_F32; };
+template <> struct dtype_of<bf16_t> { static constexpr int value = GDN_DTYPE_BF16; };
+template <> struct dtype_of<f16_t> { static constexpr int value = GDN_DTYPE_F16; };
+
+// A thread owns VEC adjacent channels (16 bytes when VECTOR, else one channel) and CONV_TOKENS consecutive
+// tokens.  blockDim = (64 channel groups, 4 token tiles); grid = (groups / 64, tiles / 4).
+//
+// Tiles that lie inside one sequence, W-1 tokens or more after its start, take the short way: the
+// CONV_TOKENS + W-1 rows are requested at once (neighbouring tiles share W-1 of them through the caches)
+// and contracted from registers.  Other tiles (sequence starts, ends of the input) go token by token and
+// tap by tap, reading the initial state where a tap reaches in front of the sequence.
+template <typename T, int W, bool VECTOR>
 __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(ConvParams p) {
-    constexpr int VEC = 16 / sizeof(T);
-    const int c0 = (blockIdx.x * 64 + threadIdx.x) * VEC;
-    int64_t gt0 = ((int64_t)blockIdx.y * 4 + threadIdx.y) * CONV_TOKENS;
+    constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
+    const int c0 = (blockIdx.x * CONV_BX + threadIdx.x) * VEC;
+    int64_t gt0 = ((int64_t)blockIdx.y * CONV_BY + threadIdx.y) * CONV_TOKENS;
     int64_t gt_end = min(gt0 + CONV_TOKENS, p.total);
     const int D = (int)p.D;
     const bool varlen = p.cu_seqlens != nullptr;
@@ -77,16 +61,24 @@ __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(ConvParams p) {
     }
     if (c0 >= D || gt0 >= gt_end) return;
 
+    // taps and bias of this thread's channels: weight rows are adjacent, VEC * W elements in one run
     float wgt[W][VEC], bias[VEC];
+    if (VECTOR && p.w_dtype == dtype_of<T>::value && ((uintptr_t)p.weight & 15) == 0) {
+        vec_t wraw[W];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-        const bool ok = c0 + e < D;
+        for (int j = 0; j < W; ++j) wraw[j] = *(const vec_t*)((const T*)p.weight + (int64_t)c0 * W + j * VEC);
 #pragma unroll
-        for (int j = 0; j < W; ++j) wgt[j][e] = ok ? load_scalar(p.weight, (int64_t)(c0 + e) * W + j, p.w_dtype) : 0.f;
-        bias[e] = ok && p.bias ? load_scalar(p.bias, c0 + e, p.w_dtype) : 0.f;
+        for (int i = 0; i < W * VEC; ++i) wgt[i % W][i / W] = (float)wraw[i / VEC][i % VEC];
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+#pragma unroll
+            for (int j = 0; j < W; ++j) wgt[j][e] = load_scalar(p.weight, (int64_t)(c0 + e) * W + j, p.w_dtype);
     }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) bias[e] = p.bias ? load_scalar(p.bias, c0 + e, p.w_dtype) : 0.f;
 
-    // the sequence of the first token, its bounds in global token numbers, and where its rows start
+    // the sequence of the first token and its bounds in global token numbers
     int64_t n, bos, eos;
     if (varlen) {
         n = find_sequence(p.cu_seqlens, p.N, gt0, p.cu32);
@@ -98,60 +90,65 @@ __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(ConvParams p) {
     auto row_of = [&](int64_t gt) -> const T* {      // x row of global token gt of the current sequence
         return (const T*)p.x + (varlen ? gt * p.stride_t : n * p.stride_n + (gt - bos) * p.stride_t) + c0;
     };
-    // rows before position 0 of the current sequence: its initial state or zero
-    auto before_start = [&](int back, float (&out)[VEC]) {        // position -back, back = 1 .. W-1
+    auto finish = [&](int64_t gt, float (&acc)[VEC], vec_t res) {
+        vec_t out;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-            out[e] = p.initial_state && c0 + e < D
-                ? load_scalar(p.initial_state, (n * D + c0 + e) * (int64_t)p.W + (p.W - back), p.state_dtype) : 0.f;
+        for (int e = 0; e < VEC; ++e) {
+            float a = acc[e] + bias[e];
+            if (p.act) a = a * sigmoid_stream(a);
+            if (p.residual) a += (float)res[e];
+            out[e] = (T)a;
+        }
+        *(vec_t*)((T*)p.y + gt * D + c0) = out;
     };
 
-    // win[j] = row at (current token) - (W-1) + j for j < W-1; filled for the first token
-    float win[W > 1 ? W - 1 : 1][VEC];
+    if (gt0 + CONV_TOKENS == gt_end && gt_end <= eos && gt0 - (W - 1) >= bos) {
+        vec_t raw[CONV_TOKENS + W - 1];
+        const T* first = row_of(gt0 - (W - 1));
 #pragma unroll
-    for (int j = 0; j < W - 1; ++j) {
-        const int back = W - 1 - j;
-        if (gt0 - back >= bos) load_row<T, VEC>(row_of(gt0 - back), c0, D, p.vec_ok, win[j]);
-        else before_start((int)(bos - (gt0 - back)), win[j]);
+        for (int i = 0; i < CONV_TOKENS + W - 1; ++i) raw[i] = *(const vec_t*)(first + i * p.stride_t);
+#pragma unroll
+        for (int u = 0; u < CONV_TOKENS; ++u) {
+            float acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float a = 0.f;
+#pragma unroll
+                for (int j = 0; j < W; ++j) a += (float)raw[u + j][e] * wgt[j][e];
+                acc[e] = a;
+            }
+            vec_t res = {};
+            if (p.residual) res = *(const vec_t*)((const T*)p.residual + (gt0 + u) * D + c0);
+            finish(gt0 + u, acc, res);
+        }
+        return;
     }
 
     for (int64_t gt = gt0; gt < gt_end; ++gt) {
-        if (gt >= eos) {                             // first token of the next sequence (empty ones are skipped)
-            do {
-                ++n;
-                bos = eos;
-                eos = varlen ? load_index(p.cu_seqlens, n + 1, p.cu32) : bos + p.T;
-            } while (gt >= eos);
-#pragma unroll
-            for (int j = 0; j < W - 1; ++j) before_start(W - 1 - j, win[j]);
+        while (gt >= eos) {                          // first token of the next sequence (empty ones are skipped)
+            ++n;
+            bos = eos;
+            eos = varlen ? load_index(p.cu_seqlens, n + 1, p.cu32) : bos + p.T;
         }
-        float cur[VEC], acc[VEC];
-        load_row<T, VEC>(row_of(gt), c0, D, p.vec_ok, cur);
+        float acc[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            float a = 0.f;
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
 #pragma unroll
-            for (int j = 0; j < W - 1; ++j) a += win[j][e] * wgt[j][e];
-            a += cur[e] * wgt[W - 1][e];
-            a += bias[e];
-            if (p.act) a = a * sigmoid_f(a);
-            acc[e] = a;
+        for (int j = 0; j < W; ++j) {
+            const int64_t src = gt - (W - 1) + j;
+            if (src >= bos) {
+                const vec_t v = *(const vec_t*)row_of(src);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] += (float)v[e] * wgt[j][e];
+            } else if (p.initial_state) {            // position src - bos = -1 .. -(W-1): state entry W + position
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    acc[e] += load_scalar(p.initial_state, (n * D + c0 + e) * (int64_t)W + (W + (src - bos)), p.state_dtype) * wgt[j][e];
+            }
         }
-        if (p.residual) {
-            float r[VEC];
-            load_row<T, VEC>((const T*)p.residual + gt * D + c0, c0, D, p.vec_ok, r);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) acc[e] += r[e];
-        }
-        store_row<T, VEC>((T*)p.y + gt * D + c0, c0, D, p.vec_ok, acc);
-#pragma unroll
-        for (int j = 0; j + 1 < W - 1; ++j)
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) win[j][e] = win[j + 1][e];
-        if (W > 1) {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) win[W - 2][e] = cur[e];
-        }
+        vec_t res = {};
+        if (p.residual) res = *(const vec_t*)((const T*)p.residual + gt * D + c0);
+        finish(gt, acc, res);
     }
 }
 
@@ -220,24 +217,29 @@ __global__ __launch_bounds__(256) void causal_conv1d_update_kernel(ConvUpdatePar
         }
     }
     if (p.bias) acc += load_scalar(p.bias, d, p.w_dtype);
-    if (p.act) acc = acc * sigmoid_f(acc);
+    if (p.act) acc = acc * sigmoid_stream(acc);
     if (p.residual) acc += (float)((const T*)p.residual)[n * p.D + d];
     ((T*)p.y)[n * p.stride_y_n + d] = (T)acc;
 }
 
-template <typename T>
-static int launch_conv_fwd(const ConvParams& p, hipStream_t stream) {
-    constexpr int VEC = 16 / sizeof(T);
-    const int64_t pieces = (p.D + VEC - 1) / VEC, tiles = (p.total + CONV_TOKENS - 1) / CONV_TOKENS;
-    if (p.total > 0 && p.y) {
-        const dim3 grid((unsigned)((pieces + 63) / 64), (unsigned)((tiles + 3) / 4)), block(64, 4);
-        switch (p.W) {
-#define GDN_CONV_CASE(w) case w: hipLaunchKernelGGL((causal_conv1d_fwd_kernel<T, w>), grid, block, 0, stream, p); break;
-            GDN_CONV_CASE(1) GDN_CONV_CASE(2) GDN_CONV_CASE(3) GDN_CONV_CASE(4)
-            GDN_CONV_CASE(5) GDN_CONV_CASE(6) GDN_CONV_CASE(7) GDN_CONV_CASE(8)
+template <typename T, bool VECTOR>
+static int launch_conv_fwd_w(const ConvParams& p, hipStream_t stream) {
+    constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
+    const int64_t groups = (p.D + VEC - 1) / VEC, tiles = (p.total + CONV_TOKENS - 1) / CONV_TOKENS;
+    const dim3 grid((unsigned)((groups + CONV_BX - 1) / CONV_BX), (unsigned)((tiles + CONV_BY - 1) / CONV_BY)), block(CONV_BX, CONV_BY);
+    switch (p.W) {
+#define GDN_CONV_CASE(w) case w: hipLaunchKernelGGL((causal_conv1d_fwd_kernel<T, w, VECTOR>), grid, block, 0, stream, p); break;
+        GDN_CONV_CASE(1) GDN_CONV_CASE(2) GDN_CONV_CASE(3) GDN_CONV_CASE(4)
+        GDN_CONV_CASE(5) GDN_CONV_CASE(6) GDN_CONV_CASE(7) GDN_CONV_CASE(8)
 #undef GDN_CONV_CASE
-        }
-        if (int rc = check_launch("causal_conv1d_fwd_kernel")) return rc;
+    }
+    return check_launch("causal_conv1d_fwd_kernel");
+}
+
+template <typename T>
+static int launch_conv_fwd(const ConvParams& p, bool vec_ok, hipStream_t stream) {
+    if (p.total > 0 && p.y) {
+        if (int rc = vec_ok ? launch_conv_fwd_w<T, true>(p, stream) : launch_conv_fwd_w<T, false>(p, stream)) return rc;
     }
     if (p.final_state && p.N * p.D > 0) {
         hipLaunchKernelGGL(causal_conv1d_states_kernel<T>, dim3((unsigned)((p.N * p.D + 255) / 256)), dim3(256), 0, stream, p);
@@ -276,11 +278,12 @@ extern "C" int gdn_causal_conv1d_fwd(
     p.cu32 = (flags & GDN_FLAG_CU_INT32) != 0;
     const int64_t vec = x_dtype == GDN_DTYPE_F32 ? 4 : 8;
     auto aligned = [](const void* q) { return ((uintptr_t)q & 15) == 0; };
-    p.vec_ok = D % vec == 0 && stride_x_t % vec == 0 && stride_x_n % vec == 0 && aligned(x) && aligned(y) && aligned(residual);
+    // 16 bytes of channels per thread need every row to start on a 16-byte boundary
+    const bool vec_ok = D % vec == 0 && stride_x_t % vec == 0 && stride_x_n % vec == 0 && aligned(x) && aligned(y) && aligned(residual);
     hipStream_t s = (hipStream_t)stream;
-    if (x_dtype == GDN_DTYPE_BF16) return launch_conv_fwd<bf16_t>(p, s);
-    if (x_dtype == GDN_DTYPE_F16) return launch_conv_fwd<f16_t>(p, s);
-    return launch_conv_fwd<float>(p, s);
+    if (x_dtype == GDN_DTYPE_BF16) return launch_conv_fwd<bf16_t>(p, vec_ok, s);
+    if (x_dtype == GDN_DTYPE_F16) return launch_conv_fwd<f16_t>(p, vec_ok, s);
+    return launch_conv_fwd<float>(p, vec_ok, s);
 }
 
 extern "C" int gdn_causal_conv1d_update(

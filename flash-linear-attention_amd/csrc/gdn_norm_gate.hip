@@ -29,7 +29,7 @@ __device__ __forceinline__ void store_typed(void* p, int64_t i, int dtype, float
 }
 
 __device__ __forceinline__ float gate_of(float y, float g, int act) {
-    const float s = sigmoid_f(g);
+    const float s = sigmoid_stream(g);
     return act == GDN_ACT_SILU ? y * g * s : y * s;
 }
 
@@ -41,76 +41,116 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-// A group of LANES lanes holds one row: lane l owns elements [(l + LANES * i) * VEC, +VEC) for i < PIECES.
-template <typename T, int LANES, int PIECES>
+// Weights and biases of one 16-byte piece as fp32 (one vector load when they have the rows' element type).
+template <typename T, int VEC>
+__device__ __forceinline__ void load_params(const void* w, int c, int w_dtype, float fill, float (&out)[VEC]) {
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
+    constexpr int own = sizeof(T) == 4 ? GDN_DTYPE_F32 : (__is_same(T, bf16_t) ? GDN_DTYPE_BF16 : GDN_DTYPE_F16);
+    if (!w) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out[e] = fill;
+    } else if (w_dtype == own && (((uintptr_t)w) & 15) == 0) {
+        const vec_t v = *(const vec_t*)((const T*)w + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out[e] = (float)v[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out[e] = load_scalar(w, c + e, w_dtype);
+    }
+}
+
+// A group of LANES lanes holds ROWS rows at a time: lane l owns elements [(l + LANES * i) * VEC, +VEC) for
+// i < PIECES of each.  All loads of the ROWS rows are issued before anything is reduced.
+template <typename T, int LANES, int PIECES, int ROWS>
 __global__ __launch_bounds__(256) void norm_gated_rows_kernel(NormGateParams p) {
     constexpr int VEC = 16 / sizeof(T);
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int l = threadIdx.x % LANES;
-    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / LANES;
-    const bool live = row < p.T;
+    // rows of a workgroup: round r covers 256 / LANES consecutive rows, one per group, so a wave's load is contiguous
+    constexpr int GROUPS = 256 / LANES;
+    const int64_t row0 = (int64_t)blockIdx.x * (GROUPS * ROWS) + threadIdx.x / LANES;
     const int D = (int)p.D;
-    const int64_t base = (live ? row : 0) * D;               // dead groups shadow row 0 and store nothing
 
-    float v[PIECES][VEC];
-    float sum = 0.f, sq = 0.f;
+    vec_t xv[ROWS][PIECES], gv[ROWS][PIECES];
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-        const int c = (l + LANES * i) * VEC;
-        if (c < D) {
-            const vec_t xv = *(const vec_t*)((const T*)p.x + base + c);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) v[i][e] = (float)xv[e];
-            if (p.residual) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) v[i][e] += load_scalar(p.residual, base + c + e, p.res_dtype);
-            }
-            if (p.residual_out && live) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) store_typed(p.residual_out, base + c + e, p.res_out_dtype, v[i][e]);
-            }
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) { sum += v[i][e]; sq += v[i][e] * v[i][e]; }
-        } else {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
-        }
-    }
-    float mean = 0.f, var;
-    if (p.rms) {
-        var = group_sum<LANES>(sq) / D;
-    } else {
-        mean = group_sum<LANES>(sum) / D;
-        float d2 = 0.f;
+    for (int r = 0; r < ROWS; ++r) {
+        const int64_t base = min(row0 + r * GROUPS, p.T - 1) * D;     // rows past the end shadow the last row and store nothing
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            if ((l + LANES * i) * VEC < D) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) { const float d = v[i][e] - mean; d2 += d * d; }
+            const int c = (l + LANES * i) * VEC;
+            if (c < D) {
+                xv[r][i] = *(const vec_t*)((const T*)p.x + base + c);
+                gv[r][i] = *(const vec_t*)((const T*)p.g + base + c);
             }
         }
-        var = group_sum<LANES>(d2) / D;
     }
-    const float rstd = 1.f / sqrtf(var + p.eps);
-    if (live && l == 0) {
-        if (p.rstd) p.rstd[row] = rstd;
-        if (p.mean && !p.rms) p.mean[row] = mean;
+    float v[ROWS][PIECES][VEC];
+    float sum[ROWS], sq[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const bool live = row0 + r * GROUPS < p.T;
+        const int64_t base = min(row0 + r * GROUPS, p.T - 1) * D;
+        sum[r] = 0.f; sq[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int c = (l + LANES * i) * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[r][i][e] = c < D ? (float)xv[r][i][e] : 0.f;
+            if (c < D && p.residual) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) v[r][i][e] += load_scalar(p.residual, base + c + e, p.res_dtype);
+            }
+            if (c < D && p.residual_out && live) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) store_typed(p.residual_out, base + c + e, p.res_out_dtype, v[r][i][e]);
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) { sum[r] += v[r][i][e]; sq[r] += v[r][i][e] * v[r][i][e]; }
+        }
     }
-    if (!live) return;
+    float mean[ROWS], rstd[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        float var;
+        if (p.rms) {
+            mean[r] = 0.f;
+            var = group_sum<LANES>(sq[r]) / D;
+        } else {
+            mean[r] = group_sum<LANES>(sum[r]) / D;
+            float d2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                if ((l + LANES * i) * VEC < D) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) { const float d = v[r][i][e] - mean[r]; d2 += d * d; }
+                }
+            }
+            var = group_sum<LANES>(d2) / D;
+        }
+        rstd[r] = 1.f / sqrtf(var + p.eps);
+        if (l == 0 && row0 + r * GROUPS < p.T) {
+            if (p.rstd) p.rstd[row0 + r * GROUPS] = rstd[r];
+            if (p.mean && !p.rms) p.mean[row0 + r * GROUPS] = mean[r];
+        }
+    }
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
         const int c = (l + LANES * i) * VEC;
         if (c >= D) continue;
-        const vec_t gv = *(const vec_t*)((const T*)p.g + base + c);
-        vec_t out;
+        float wv[VEC], bv[VEC];
+        load_params<T, VEC>(p.weight, c, p.w_dtype, 1.f, wv);
+        load_params<T, VEC>(p.bias, c, p.w_dtype, 0.f, bv);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            float y = (v[i][e] - mean) * rstd;
-            if (p.weight) y *= load_scalar(p.weight, c + e, p.w_dtype);
-            if (p.bias) y += load_scalar(p.bias, c + e, p.w_dtype);
-            out[e] = (T)gate_of(y, (float)gv[e], p.act);
+        for (int r = 0; r < ROWS; ++r) {
+            if (row0 + r * GROUPS >= p.T) continue;
+            vec_t out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float y = (v[r][i][e] - mean[r]) * rstd[r] * wv[e] + bv[e];
+                out[e] = (T)gate_of(y, (float)gv[r][i][e], p.act);
+            }
+            *(vec_t*)((T*)p.y + (row0 + r * GROUPS) * D + c) = out;
         }
-        *(vec_t*)((T*)p.y + base + c) = out;
     }
 }
 
@@ -160,10 +200,10 @@ __global__ __launch_bounds__(256) void norm_gated_long_kernel(NormGateParams p) 
     }
 }
 
-template <typename T, int LANES, int PIECES>
+template <typename T, int LANES, int PIECES, int ROWS>
 static void launch_rows(const NormGateParams& p, hipStream_t stream) {
-    const int64_t rows_per_block = 256 / LANES;
-    hipLaunchKernelGGL((norm_gated_rows_kernel<T, LANES, PIECES>), dim3((unsigned)((p.T + rows_per_block - 1) / rows_per_block)),
+    const int64_t rows_per_block = (256 / LANES) * ROWS;
+    hipLaunchKernelGGL((norm_gated_rows_kernel<T, LANES, PIECES, ROWS>), dim3((unsigned)((p.T + rows_per_block - 1) / rows_per_block)),
                        dim3(256), 0, stream, p);
 }
 
@@ -173,13 +213,13 @@ static int launch_norm_gate(const NormGateParams& p, bool aligned, hipStream_t s
     if (p.T == 0) return GDN_OK;
     const int64_t pieces = p.D / VEC;                         // 16-byte pieces per row (when D % VEC == 0)
     if (aligned && p.D % VEC == 0 && pieces <= 64 * 8) {
-        if (pieces <= 8) launch_rows<T, 8, 1>(p, stream);
-        else if (pieces <= 16) launch_rows<T, 16, 1>(p, stream);
-        else if (pieces <= 32) launch_rows<T, 32, 1>(p, stream);
-        else if (pieces <= 64) launch_rows<T, 64, 1>(p, stream);
-        else if (pieces <= 128) launch_rows<T, 64, 2>(p, stream);
-        else if (pieces <= 256) launch_rows<T, 64, 4>(p, stream);
-        else launch_rows<T, 64, 8>(p, stream);
+        if (pieces <= 8) launch_rows<T, 8, 1, 4>(p, stream);
+        else if (pieces <= 16) launch_rows<T, 16, 1, 4>(p, stream);
+        else if (pieces <= 32) launch_rows<T, 32, 1, 4>(p, stream);
+        else if (pieces <= 64) launch_rows<T, 64, 1, 4>(p, stream);
+        else if (pieces <= 128) launch_rows<T, 64, 2, 2>(p, stream);
+        else if (pieces <= 256) launch_rows<T, 64, 4, 1>(p, stream);
+        else launch_rows<T, 64, 8, 1>(p, stream);
     } else {
         hipLaunchKernelGGL(norm_gated_long_kernel<T>, dim3((unsigned)p.T), dim3(256), 0, stream, p);
     }
