@@ -267,3 +267,78 @@ def test_scan_tables_offsets_then_longest_first_order():
     assert sorted(order) == list(range(n))
     assert [counts[i] for i in order] == sorted(counts, reverse=True)
     assert order == sorted(range(n), key=lambda i: (-counts[i], i))
+
+
+def test_upstream_backends_follow_the_plugin_interface():
+    # the backends for an unmodified upstream fla, exercised through this package's mirror of the registry:
+    # CPU tensors are rejected by the verifier, so the decorated default runs
+    import torch
+    from fla_hip.ops.backends import BackendRegistry, BaseBackend, dispatch
+    from fla_hip.upstream import make_backends
+    op_cls, mod_cls = make_backends(BaseBackend)
+    assert issubclass(op_cls, BaseBackend) and op_cls.priority < 3 and op_cls.package_name == 'fla_hip'
+    assert op_cls.is_available() and op_cls.is_enabled()
+    reg = BackendRegistry('upstream_test_cpu')
+    reg.register(op_cls())
+    calls = []
+
+    @dispatch('upstream_test_cpu')
+    def chunk_gated_delta_rule(q, k, v, g, beta, **kwargs):
+        calls.append('default')
+        return 'default'
+
+    x = torch.zeros(1, 4, 1, 8)
+    assert chunk_gated_delta_rule(x, x, x, x[..., 0], x[..., 0]) == 'default' and calls == ['default']
+    be = mod_cls()
+    for name in ('causal_conv1d_fwd', 'causal_conv1d_update_states', 'causal_conv1d_update', 'layer_norm_gated_fwd'):
+        assert callable(getattr(be, name)) and callable(getattr(be, name + '_verifier'))
+    assert be.verify('causal_conv1d_fwd', x[0], torch.zeros(8, 4))[0] is False
+    assert be.verify('layer_norm_gated_fwd', x[0, :, 0], x[0, :, 0], None, None)[0] is False
+    os.environ['FLA_HIP_GFX950'] = '0'
+    try:
+        assert not op_cls.is_enabled()
+    finally:
+        del os.environ['FLA_HIP_GFX950']
+
+
+@pytest.mark.gpu
+def test_upstream_backends_take_gpu_inference_calls_and_leave_the_rest():
+    import torch
+    from fla_hip.ops.backends import BackendRegistry, BaseBackend, dispatch
+    from fla_hip.upstream import make_backends
+    from oracle import gdn_oracle as O
+    op_cls, mod_cls = make_backends(BaseBackend)
+    BackendRegistry('upstream_test_gpu').register(op_cls())
+    BackendRegistry('upstream_test_modules').register(mod_cls())
+
+    @dispatch('upstream_test_gpu')
+    def chunk_gated_delta_rule(q, k, v, g, beta, **kwargs):
+        return 'default', None
+
+    @dispatch('upstream_test_modules')
+    def causal_conv1d_fwd(x, weight, bias, residual, initial_state=None, output_final_state=False, activation=None, **kwargs):
+        return 'default', None
+
+    @dispatch('upstream_test_modules')
+    def layer_norm_gated_fwd(x, g, weight, bias, activation='swish', eps=1e-5, residual=None, out_dtype=None,
+                             residual_dtype=None, is_rms_norm=False):
+        return 'default'
+
+    q, k, v, g, beta, _ = O.make_inputs(1, 130, 2, 4, 64, 64, seed=3, dtype=torch.bfloat16)
+    ref, _ = O.chunk_gated_delta_rule(q, k, v, g, beta, None, None, False)
+    dq, dk, dv, dg, db = (t.cuda() for t in (q, k, v, g, beta))
+    o, ht = chunk_gated_delta_rule(dq, dk, dv, dg, db, output_final_state=False)
+    assert isinstance(o, torch.Tensor) and ht is None and O.get_err_ratio(ref, o.float().cpu()) < 5e-3
+    assert chunk_gated_delta_rule(dq.requires_grad_(), dk, dv, dg, db)[0] == 'default'           # training stays upstream
+    assert chunk_gated_delta_rule(q, k, v, g, beta)[0] == 'default'                               # CPU stays upstream
+    with torch.no_grad():
+        assert isinstance(chunk_gated_delta_rule(dq, dk, dv, dg, db)[0], torch.Tensor)
+    x = torch.randn(2, 40, 64, device='cuda', dtype=torch.bfloat16)
+    w = torch.randn(64, 4, device='cuda', dtype=torch.bfloat16)
+    y, st = causal_conv1d_fwd(x, w, None, None, activation='silu', output_final_state=True)
+    assert y.shape == x.shape and st.shape == (2, 64, 4)
+    assert causal_conv1d_fwd(x, torch.randn(64, 9, device='cuda', dtype=torch.bfloat16), None, None)[0] == 'default'
+    assert causal_conv1d_fwd(x, w, None, None, activation='gelu')[0] == 'default'
+    out = layer_norm_gated_fwd(x[0], x[1], None, None, is_rms_norm=True)
+    assert len(out) == 4 and out[0].shape == x[0].shape and out[1] is None
+    assert layer_norm_gated_fwd(x[0], x[1], None, None, activation='relu') == 'default'
