@@ -40,7 +40,7 @@ template <> struct dtype_of<bf16_t> { static constexpr int value = GDN_DTYPE_BF1
 template <> struct dtype_of<f16_t> { static constexpr int value = GDN_DTYPE_F16; };
 
 // A thread owns VEC adjacent channels (16 bytes when VECTOR, else one channel) and CONV_TOKENS consecutive
-// tokens.  blockDim = (64 channel groups, 4 token tiles); grid = (groups / 64, tiles / 4).
+// tokens.  blockDim = (64 channel groups, 4 token tiles); the grid is flat: (groups / 64) x (tiles / 4) workgroups.
 //
 // Tiles that lie inside one sequence, W-1 tokens or more after its start, take the short way: the
 // CONV_TOKENS + W-1 rows are requested at once (neighbouring tiles share W-1 of them through the caches)
@@ -50,8 +50,10 @@ template <typename T, int W, bool VECTOR>
 __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(ConvParams p) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
-    const int c0 = (blockIdx.x * CONV_BX + threadIdx.x) * VEC;
-    int64_t gt0 = ((int64_t)blockIdx.y * CONV_BY + threadIdx.y) * CONV_TOKENS;
+    // workgroups are numbered channel block first, so those that run together cover whole rows of the same tokens
+    const int64_t cblocks = (p.D + (int64_t)CONV_BX * VEC - 1) / ((int64_t)CONV_BX * VEC);
+    const int c0 = (int)((blockIdx.x % cblocks) * CONV_BX + threadIdx.x) * VEC;
+    int64_t gt0 = ((int64_t)(blockIdx.x / cblocks) * CONV_BY + threadIdx.y) * CONV_TOKENS;
     int64_t gt_end = min(gt0 + CONV_TOKENS, p.total);
     const int D = (int)p.D;
     const bool varlen = p.cu_seqlens != nullptr;
@@ -226,7 +228,12 @@ template <typename T, bool VECTOR>
 static int launch_conv_fwd_w(const ConvParams& p, hipStream_t stream) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     const int64_t groups = (p.D + VEC - 1) / VEC, tiles = (p.total + CONV_TOKENS - 1) / CONV_TOKENS;
-    const dim3 grid((unsigned)((groups + CONV_BX - 1) / CONV_BX), (unsigned)((tiles + CONV_BY - 1) / CONV_BY)), block(CONV_BX, CONV_BY);
+    const int64_t blocks = ((groups + CONV_BX - 1) / CONV_BX) * ((tiles + CONV_BY - 1) / CONV_BY);
+    if (blocks >= (1ll << 31)) {
+        set_error("gdn_causal_conv1d_fwd: %lld workgroups exceed the grid limit", (long long)blocks);
+        return GDN_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)blocks), block(CONV_BX, CONV_BY);
     switch (p.W) {
 #define GDN_CONV_CASE(w) case w: hipLaunchKernelGGL((causal_conv1d_fwd_kernel<T, w, VECTOR>), grid, block, 0, stream, p); break;
         GDN_CONV_CASE(1) GDN_CONV_CASE(2) GDN_CONV_CASE(3) GDN_CONV_CASE(4)

@@ -258,6 +258,16 @@ def test_conv_full_width_prefill_spot_checks():
     assert torch.equal(state[0].T, x[0, T - W:])
 
 
+def test_conv_many_tokens_few_channels():
+    # more than 65535 * 32 tokens: the launch must not depend on the y extent of the grid
+    B, T, D, W, dtype = 3, 740000, 8, 4, torch.bfloat16
+    x, w, b, _, _ = _inputs(B, T, D, W, dtype, True, False)
+    ref, ref_state = M.causal_conv1d(x, w, b, None, None, True, 'silu')
+    tri, state = _mods().causal_conv1d(x.to(DEV), w.to(DEV), b.to(DEV), activation='silu', output_final_state=True)
+    _close('y', ref, tri, dtype)
+    assert torch.equal(state.cpu().float(), ref_state)
+
+
 def test_conv_errors():
     mods = _mods()
     x = torch.randn(2, 8, 16, device=DEV)
