@@ -489,3 +489,53 @@ def test_host_validation_errors():
         op(q, q, v, g, g, head_first=True)
     with pytest.raises(RuntimeError):
         op(q.cpu(), q.cpu(), v.cpu(), g.cpu(), g.cpu())                          # no CPU path
+
+
+@pytest.mark.parametrize('B,T,H,HV,D,dtype', [
+    (1, 1024, 4, 4, 128, torch.bfloat16),
+    (2, 2048, 8, 8, 128, torch.bfloat16),
+    (1, 4096, 16, 16, 128, torch.bfloat16),
+    (1, 1024, 4, 4, 128, torch.float16),
+    (2, 2048, 8, 8, 128, torch.float16),
+    (1, 1024, 2, 8, 128, torch.bfloat16),           # grouped value heads
+    (2, 2048, 4, 16, 128, torch.bfloat16),
+])
+def test_reference_whole_operator_backend_matrix(B, T, H, HV, D, dtype):
+    """The matrix and recipe with which the reference checks a whole-operator backend (its closest analogue of this
+    library; tests/ops/test_gdn.py:1350-1403): everything `randn`, unit-variance fp32 initial states, l2 norm in
+    the kernel, scale D^-0.5, against the token recurrence on normalised q, k.  The reference's bar is 0.008."""
+    gen = torch.Generator().manual_seed(42)
+    q = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    k = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    v = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen))
+    beta = torch.randn(B, T, HV, generator=gen).sigmoid()
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(O.l2norm(q.float()), O.l2norm(k.float()), v, g, beta, D ** -0.5, h0, True)
+    o, ht = _run(q, k, v, g, beta, h0, scale=D ** -0.5, use_qk_l2norm_in_kernel=True)
+    _check('o', ref_o, o, ratio=0.008)
+    _check('ht', ref_ht, ht, ratio=0.008)
+
+
+@pytest.mark.parametrize('H,D,cu', [
+    (4, 128, [0, 256, 500, 1000]),
+    (8, 128, [0, 100, 300, 1200, 2000]),
+    (16, 128, [0, 101, 303, 1205, 3007, 4096]),
+])
+def test_reference_whole_operator_backend_matrix_packed(H, D, cu):
+    """The packed-input half of the same check (tests/ops/test_gdn.py:1406-1478): bf16, every sequence against the
+    token recurrence run on it alone."""
+    gen = torch.Generator().manual_seed(42)
+    dtype, T, N = torch.bfloat16, cu[-1], len(cu) - 1
+    q = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    k = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    v = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.randn(1, T, H, generator=gen))
+    beta = torch.randn(1, T, H, generator=gen).sigmoid()
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    refs = [O.recurrent_gated_delta_rule(O.l2norm(q[:, a:b].float()), O.l2norm(k[:, a:b].float()), v[:, a:b], g[:, a:b],
+                                         beta[:, a:b], D ** -0.5, h0[i:i + 1], True) for i, (a, b) in enumerate(zip(cu[:-1], cu[1:]))]
+    ref_o, ref_ht = torch.cat([r[0] for r in refs], 1), torch.cat([r[1] for r in refs], 0)
+    o, ht = _run(q, k, v, g, beta, h0, cu, scale=D ** -0.5, use_qk_l2norm_in_kernel=True)
+    _check('o', ref_o, o, ratio=0.008)
+    _check('ht', ref_ht, ht, ratio=0.008)
