@@ -382,3 +382,67 @@ def test_norm_gated_errors():
         mods.layer_norm_gated_fwd(torch.randn(2, 40000, device=DEV), torch.randn(2, 40000, device=DEV), None, None)
     with pytest.raises(RuntimeError):
         mods.rms_norm_gated(x.cpu(), x.cpu(), None, None)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# seeded random combinations
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('seed', range(64))
+def test_conv_random_configuration(seed):
+    import random
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+    W = rnd.choice([1, 2, 3, 4, 4, 5, 8])
+    D = rnd.choice([4, 8, 24, 64, 100, 128, 520, 1032])
+    packed = rnd.random() < 0.5
+    if packed:
+        lens = [rnd.choice([0, 1, 2, 3, 8, 9, 31, 32, 33, 100]) for _ in range(rnd.choice([1, 2, 4, 7]))]
+        if sum(lens) == 0:
+            lens[0] = 5
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        B, T, N = 1, cu[-1], len(lens)
+    else:
+        B, T, cu = rnd.choice([1, 2, 3]), rnd.choice([1, 2, 7, 8, 9, 40, 257]), None
+        N = B
+    has_bias, has_res, has_state = rnd.random() < 0.5, rnd.random() < 0.4, rnd.random() < 0.5
+    act = rnd.choice([None, 'silu', 'swish'])
+    x, w, b, r, s = _inputs(B, T, D, W, dtype, has_bias, has_res, seed=seed, N=N, state=has_state)
+    ref, ref_state = M.causal_conv1d(x, w, b, r, s, True, act, cu_seqlens=cu)
+    gx, gw, gb, gr, gs = _gpu(x, w, b, r, s)
+    if rnd.random() < 0.4:                                      # x as a column block of a wider tensor
+        pad = rnd.choice([8, 3])
+        wide = torch.zeros(B, T, D + 2 * pad, device=DEV, dtype=dtype)
+        wide[..., pad:pad + D] = gx
+        gx = wide[..., pad:pad + D]
+    cu_t = None if cu is None else torch.tensor(cu, device=DEV, dtype=rnd.choice([torch.int32, torch.int64]))
+    tri, state = _mods().causal_conv1d(gx, gw, gb, residual=gr, initial_state=gs, output_final_state=True, activation=act,
+                                       cu_seqlens=cu_t)
+    _close('y', ref, tri, dtype)
+    assert torch.equal(state.cpu().float(), ref_state)
+
+
+@pytest.mark.parametrize('seed', range(48))
+def test_norm_gated_random_configuration(seed):
+    import random
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+    T = rnd.choice([1, 3, 17, 64, 255, 1000])
+    D = rnd.choice([8, 16, 50, 64, 96, 128, 256, 384, 512, 640, 1024, 2048, 3000, 4096])
+    is_rms, act = rnd.random() < 0.6, rnd.choice(['swish', 'silu', 'sigmoid'])
+    gen = torch.Generator().manual_seed(seed)
+    x, g = torch.randn(T, D, generator=gen).to(dtype), torch.randn(T, D, generator=gen).to(dtype)
+    w = torch.randn(D, generator=gen).to(rnd.choice([dtype, torch.float32])) if rnd.random() < 0.8 else None
+    b = torch.randn(D, generator=gen).to(w.dtype) if w is not None and rnd.random() < 0.4 else None
+    res = torch.randn(T, D, generator=gen).to(rnd.choice([dtype, torch.float32])) if rnd.random() < 0.3 else None
+    eps = rnd.choice([1e-5, 1e-6])
+    ref, r, mean, rstd = M.norm_gated(x, g, w, b, res, eps, act, is_rms)
+    gx, gg, gw, gb, gres = _gpu(x, g, w, b, res)
+    y, tmean, trstd, rout = _mods().layer_norm_gated_fwd(gx, gg, gw, gb, act, eps, residual=gres, is_rms_norm=is_rms)
+    _close('y', ref, y, dtype)
+    assert get_err_ratio(rstd, trstd.cpu()) < 2e-6
+    if res is not None:
+        _close('residual_out', r, rout, res.dtype)
+    else:
+        assert rout is gx or rout.data_ptr() == gx.data_ptr()
