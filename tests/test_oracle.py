@@ -45,7 +45,7 @@ def test_chunk_matches_scalar_fixture(name, chunk):
 
 
 def test_config1_recurrent_equals_chunk():
-    # BASELINE config 1: B=2 T=256 H=2 K=V=64 fp32, zero initial state
+    # the CPU-runnable configuration: B=2 T=256 H=2 K=V=64 fp32, zero initial state
     q, k, v, g, beta, _ = O.make_inputs(2, 256, 2, 2, 64, 64, seed=42)
     o_r, h_r = O.recurrent_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
     o_c, h_c = O.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
