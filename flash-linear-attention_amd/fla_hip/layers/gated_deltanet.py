@@ -164,11 +164,17 @@ class GatedDeltaNet(nn.Module):
 
         recurrent_state = last_state['recurrent_state'] if last_state is not None else None
         op = chunk_gated_delta_rule if mode == 'chunk' else fused_recurrent_gated_delta_rule
+        extra = {}
+        if (mode == 'fused_recurrent' and use_cache and recurrent_state is not None and recurrent_state.dtype == torch.float32
+                and recurrent_state.is_contiguous()):
+            # decode: the cached state is updated where it is - no allocation per step, and a step captured in a
+            # HIP graph keeps reading and writing the same buffers on every replay
+            extra['inplace_final_state'] = True
         o, recurrent_state = op(
             q=q, k=k, v=v, g=self.a_proj(hidden_states), beta=self.b_proj(hidden_states),
             A_log=self.A_log, dt_bias=self.dt_bias, initial_state=recurrent_state, output_final_state=use_cache,
             use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, use_beta_sigmoid_in_kernel=True,
-            allow_neg_eigval=self.allow_neg_eigval, state_v_first=True, cu_seqlens=cu_seqlens)
+            allow_neg_eigval=self.allow_neg_eigval, state_v_first=True, cu_seqlens=cu_seqlens, **extra)
 
         if past_key_values is not None:
             past_key_values.update(layer_idx=self.layer_idx, recurrent_state=recurrent_state,

@@ -129,3 +129,39 @@ def test_layer_refuses_training_and_missing_layer_idx():
         layer(x, past_key_values=LayerCache())
     with pytest.raises(ValueError):
         GatedDeltaNet(hidden_size=64, head_dim=16, num_heads=2, num_v_heads=3)
+
+
+def test_decode_step_replayed_from_a_captured_graph():
+    """A decode step of the layer captured once and replayed per token: the conv caches and the recurrent state are
+    updated in place, so every replay continues from the previous one.  Checked against the same steps run eagerly."""
+    from fla_hip.layers import LayerCache
+    layer = _layer(seed=6)
+    T, n = 100, 5
+    x = torch.randn(2, T + n, 256, generator=torch.Generator().manual_seed(8)).to(BF).to(DEV)
+    eager_cache = LayerCache()
+    layer(x[:, :T], past_key_values=eager_cache, use_cache=True)
+    eager = [layer(x[:, T + i:T + i + 1], past_key_values=eager_cache, use_cache=True)[0].clone() for i in range(n)]
+
+    cache = LayerCache()
+    layer(x[:, :T], past_key_values=cache, use_cache=True)
+    state_ptr = cache[0]['recurrent_state'].data_ptr()
+    token = x[:, T:T + 1].clone()                                # static input buffer of the graph
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                                # warm-up outside the capture, on a copy of the cache
+        warm = LayerCache()
+        warm.update(layer_idx=0, recurrent_state=cache[0]['recurrent_state'].clone(),
+                    conv_state=tuple(c.clone() for c in cache[0]['conv_state']), offset=T)
+        layer(token, past_key_values=warm, use_cache=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = layer(token, past_key_values=cache, use_cache=True)[0]
+    # the capture itself does not run the step: the cache still holds the state after the prompt
+    for i in range(n):
+        token.copy_(x[:, T + i:T + i + 1])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert O.get_err_ratio(eager[i].float().cpu(), out.float().cpu()) < 1e-3, i
+    assert cache[0]['recurrent_state'].data_ptr() == state_ptr
+    assert torch.equal(cache[0]['recurrent_state'], eager_cache[0]['recurrent_state'])
