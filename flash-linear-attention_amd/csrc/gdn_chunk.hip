@@ -14,23 +14,14 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
         if (rc) return rc;
     }
     if (!(stages & STAGE_SCAN)) return GDN_OK;
-    // One workgroup per (sequence, head) walks the chunks of the sequence.  With few such runs and
-    // long dense sequences, time is cut into segments instead so that every CU has a workgroup: two
-    // passes over 1/nseg of the chunks each plus a small merge.
-    // Either way a workgroup can also carry two runs that read the same k rows (two value heads of
+    // One workgroup per (sequence, head) walks the chunks of the sequence, or time is cut into
+    // segments (plan_segments).  Either way a workgroup can also carry two runs that read the same k rows (two value heads of
     // a q/k head; in pass 1 the S and M runs of one head).  That halves the number of workgroups and
     // runs a pair about 1.25 times as fast as two single runs one after the other, so it pays as soon
     // as the single runs would not all fit on the chip at once.
     const int64_t G = p.HV / p.H;
-    const bool dense = p.cu_seqlens == nullptr;
-    int nseg = 0;
-    if (dense && p.NH > 0) {
-        nseg = (int)std::min<int64_t>((256 + p.NH / 2) / p.NH, p.NT / 4);
-        while (nseg > 0 && ((int64_t)nseg * p.NH > SEG_SLOTS_MAX || (int64_t)nseg * p.NH > (num_chunks * p.HV + 3) / 4)) --nseg;
-    }
-    bool segments = nseg >= 3;           // two passes of NT/nseg steps each must beat one pass of NT steps
-    if (p.flags & GDN_FLAG_SCAN_WIDE) segments = false;
-    if ((p.flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
+    const int nseg = plan_segments(p.N, p.HV, p.NT, num_chunks, p.cu_seqlens == nullptr, p.flags);
+    const bool segments = nseg > 0;
     const bool no_pair = p.flags & GDN_FLAG_SCAN_NO_PAIR, force_pair = p.flags & GDN_FLAG_SCAN_PAIR;
     // (full runs in pairs: an even number of value heads per q/k head, and all 128 value columns real: the two-run
     // kernel counts its output stores, which every wave must therefore have)
@@ -59,9 +50,20 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
 
 }  // namespace gdn
 
-extern "C" size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V) {
-    if (K < 8 || V < 8 || K > 128 || V > 128 || K % 8 || V % 8 || num_chunks < 0 || H < 1 || HV < 1) return 0;
-    return gdn::ws_layout(num_chunks, H, HV, nullptr, nullptr);
+static bool chunk_dims_ok(int64_t K, int64_t V) { return K >= 8 && V >= 8 && K <= 128 && V <= 128 && K % 8 == 0 && V % 8 == 0; }
+
+// bytes of workspace for the plan that launch_chunk will choose
+static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int64_t HV, bool packed, uint32_t flags,
+                                   char* base, gdn::ChunkWs* ws) {
+    using namespace gdn;
+    const int nseg = plan_segments(N, HV, (T + CH - 1) / CH, num_chunks, !packed, flags);
+    return ws_layout(num_chunks, HV, (int64_t)nseg * N * HV, base, ws);
+}
+
+extern "C" size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V,
+                                            int packed, uint32_t flags) {
+    if (!chunk_dims_ok(K, V) || num_chunks < 0 || N < 1 || T < 0 || H < 1 || HV < 1) return 0;
+    return chunk_workspace_need(N, T, num_chunks, HV, packed != 0, flags, nullptr, nullptr);
 }
 
 static int chunk_entry(
@@ -75,13 +77,13 @@ static int chunk_entry(
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
+    GDN_CHECK_ARG(T == 0 || (q && k && v && g && beta && o), GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "%s: non-positive dimension", who);
     GDN_CHECK_ARG(!dt_bias || A_log, GDN_ERR_INVALID, "%s: dt_bias without A_log", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_SCAN_NO_PAIR) || !(flags & GDN_FLAG_SCAN_PAIR), GDN_ERR_INVALID, "%s: GDN_FLAG_SCAN_PAIR and GDN_FLAG_SCAN_NO_PAIR exclude each other", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
-    GDN_CHECK_ARG(K >= 8 && V >= 8 && K <= 128 && V <= 128 && K % 8 == 0 && V % 8 == 0, GDN_ERR_UNSUPPORTED,
+    GDN_CHECK_ARG(chunk_dims_ok(K, V), GDN_ERR_UNSUPPORTED,
                   "%s: head dims must be multiples of 8 up to 128 (got K=%lld V=%lld)", who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
                   "%s: q/k/v must be bf16 or f16", who);
@@ -96,16 +98,20 @@ static int chunk_entry(
     GDN_CHECK_ARG(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0 && ((uintptr_t)h0 % 16) == 0 &&
                       ((uintptr_t)ht % 16) == 0 && ((uintptr_t)workspace % 256) == 0,
                   GDN_ERR_INVALID, "%s: q/k/v/h0/ht must be 16-byte and the workspace 256-byte aligned", who);
-    if (T == 0 || num_chunks == 0) return GDN_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0 || num_chunks == 0) {
+        // no token anywhere: the final states are the initial ones
+        if (ht && (stages & gdn::STAGE_SCAN)) return launch_state_copy(h0, ht, N * HV * K * V, s);
+        return GDN_OK;
+    }
     ChunkParams p;
-    const size_t need = ws_layout(num_chunks, H, HV, (char*)workspace, &p.ws);
+    const size_t need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH; p.K = (int)K; p.V = (int)V;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.NH = N * HV;
-    hipStream_t s = (hipStream_t)stream;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, stages, s)
                                        : launch_chunk<f16_t>(p, num_chunks, stages, s);
 }

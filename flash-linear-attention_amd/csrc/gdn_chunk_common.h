@@ -100,12 +100,29 @@ constexpr int64_t SEG_SLOTS_MAX = 640;            // upper bound on (sequences *
 
 inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
-inline size_t ws_layout(int64_t NC, int64_t H, int64_t HV, char* base, ChunkWs* ws) {
-    (void)H;
+// Number of time segments the sequential stage cuts every sequence into (0: whole sequences, one
+// workgroup per sequence and head).  With few (sequence, head) runs and long dense sequences, time is
+// cut so that every CU has a workgroup: two passes over 1/nseg of the chunks each plus a small merge,
+// which must beat one pass over all chunks (nseg >= 3).  Shared by the workspace size and the launch.
+inline int plan_segments(int64_t N, int64_t HV, int64_t NT, int64_t num_chunks, bool dense, uint32_t flags) {
+    const int64_t NH = N * HV;
+    int nseg = 0;
+    if (dense && NH > 0) {
+        nseg = (int)std::min<int64_t>((256 + NH / 2) / NH, NT / 4);
+        while (nseg > 0 && ((int64_t)nseg * NH > SEG_SLOTS_MAX || (int64_t)nseg * NH > (num_chunks * HV + 3) / 4)) --nseg;
+    }
+    bool segments = nseg >= 3;
+    if (flags & GDN_FLAG_SCAN_WIDE) segments = false;
+    if ((flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
+    return segments ? nseg : 0;
+}
+
+// Workspace: the segment matrices (S_loc, M, S_in per (sequence, head, segment); none without segments),
+// then the records.
+inline size_t ws_layout(int64_t NC, int64_t HV, int64_t seg_slots, char* base, ChunkWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
-    const size_t seg_slots = (size_t)std::min<int64_t>((NC * HV + 3) / 4, SEG_SLOTS_MAX);
-    void* Seg = take(3 * seg_slots * 16384 * 4);
+    void* Seg = take(3 * (size_t)seg_slots * 16384 * 4);
     void* Rec = take((size_t)NC * HV * REC_BYTES);
     if (ws) { ws->Seg = (float*)Seg; ws->Rec = (char*)Rec; }
     return off;

@@ -11,6 +11,8 @@
 namespace gdn {
 
 void set_error(const char* fmt, ...);
+// dst = src, or zero when src is NULL (`count` floats), as a kernel on `stream`
+int launch_state_copy(const float* src, float* dst, int64_t count, hipStream_t stream);
 
 #define GDN_CHECK_ARG(cond, code, ...)            \
     do {                                          \

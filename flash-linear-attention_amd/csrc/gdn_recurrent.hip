@@ -17,7 +17,8 @@ struct RecurrentParams {
     const void* g; const void* beta; const float* gk; const float* gv;
     const float* A_log; const float* dt_bias;
     const float* h0; float* ht; void* o;
-    const void* cu_seqlens; const void* state_slots;
+    const void* cu_seqlens; const void* state_slots; const void* num_accepted;
+    int64_t slots_stride;
     int64_t T; int H, HV, K, V, NVB;
     float scale; int gb_dtype; uint32_t flags;
 };
@@ -69,9 +70,19 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
     const int row_base = VFIRST ? v0 : 0;
     const int64_t row_stride = VFIRST ? K : V;
     const bool cont_ok = cont_idx < cont_lim;
-    // the state lives at sequence n of the state tensors, or at the slot of a pool that the caller names for n
-    const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
-    const int64_t state_off = (slot * HV + ihv) * (int64_t)K * V;
+    // The state lives at sequence n of the state tensors, or at the slot of a pool that the caller names for n.
+    // With a slot per token (speculative decoding) the sequence starts from the slot of its last accepted token
+    // (the first one without num_accepted) and leaves the state after token t in slot (n, t).
+    const bool slot32 = p.flags & GDN_FLAG_SLOT_INT32;
+    const bool slot_per_token = p.flags & GDN_FLAG_SLOT_PER_TOKEN, state_per_token = p.flags & GDN_FLAG_STATE_PER_TOKEN;
+    int64_t slot = in;
+    if (p.state_slots) {
+        int64_t first = 0;
+        if (slot_per_token && p.num_accepted) first = load_index(p.num_accepted, in, slot32) - 1;
+        slot = load_index(p.state_slots, slot_per_token ? in * p.slots_stride + first : in, slot32);
+    }
+    const int64_t head_off = (int64_t)ihv * K * V, state_stride = (int64_t)HV * K * V;
+    const int64_t state_off = slot * state_stride + head_off;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int row = row_base + r0 + RP * i;
@@ -80,6 +91,15 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
         if (ok && p.h0) s = __builtin_nontemporal_load((const f32x4*)(p.h0 + state_off + row * row_stride + cont_idx));
         S[i] = s;
     }
+
+    auto store_state = [&](float* dst) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int row = row_base + r0 + RP * i;
+            const bool ok = cont_ok && (r0 + RP * i < ROWS) && row < row_lim;
+            if (ok) __builtin_nontemporal_store(S[i], (f32x4*)(dst + row * row_stride + cont_idx));
+        }
+    };
 
     __shared__ float sh_q[2][KMAX], sh_k[2][KMAX];
     __shared__ float sh_red[2][4][4];                       // per-wave partial sums for |q|^2, |k|^2, q.k
@@ -165,6 +185,7 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
             if (cont_ok) {
                 const T* pv = v + (tok * HV + ihv) * V + cont_idx;
                 vv = f32x4{to_f32(pv[0]), to_f32(pv[1]), to_f32(pv[2]), to_f32(pv[3])};
+                // (a missing beta counts as ones BEFORE the activation, fla/ops/gated_delta_rule/fused_recurrent.py:443)
                 if (p.beta) {
                     if (p.flags & GDN_FLAG_BETA_VECTOR) {
                         const int64_t bi = (tok * HV + ihv) * V + cont_idx;
@@ -174,10 +195,10 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
                         const float b = load_scalar(p.beta, tok * HV + ihv, p.gb_dtype);
                         bb = f32x4{b, b, b, b};
                     }
-                    if (p.flags & GDN_FLAG_BETA_SIGMOID) {
-                        const float m = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
-                        bb = f32x4{m * sigmoid_f(bb.x), m * sigmoid_f(bb.y), m * sigmoid_f(bb.z), m * sigmoid_f(bb.w)};
-                    }
+                }
+                if (p.flags & GDN_FLAG_BETA_SIGMOID) {
+                    const float m = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+                    bb = f32x4{m * sigmoid_f(bb.x), m * sigmoid_f(bb.y), m * sigmoid_f(bb.z), m * sigmoid_f(bb.w)};
                 }
             }
             const f32x4 d = bb * (vv - sk);
@@ -215,24 +236,22 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
                     if (p.beta) {
                         bb = (p.flags & GDN_FLAG_BETA_VECTOR) ? load_scalar(p.beta, (tok * HV + ihv) * V + row, p.gb_dtype)
                                                               : load_scalar(p.beta, tok * HV + ihv, p.gb_dtype);
-                        if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
                     }
+                    if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
                 }
                 const float d = bb * (vv - sk);
                 S[i] = s + kc * d;
                 if (c == 0 && rok) o[(tok * HV + ihv) * V + row] = from_f32<T>(sq + d * qk);
             }
         }
-    }
-
-    if (p.ht) {
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int row = row_base + r0 + RP * i;
-            const bool ok = cont_ok && (r0 + RP * i < ROWS) && row < row_lim;
-            if (ok) __builtin_nontemporal_store(S[i], (f32x4*)(p.ht + state_off + row * row_stride + cont_idx));
+        // a state per token: into the slot named for (n, t), or into entry `tok` of a per-token state tensor
+        if (p.ht && (slot_per_token || state_per_token)) {
+            const int64_t dst = state_per_token ? tok : load_index(p.state_slots, in * p.slots_stride + t, slot32);
+            store_state(p.ht + dst * state_stride + head_off);
         }
     }
+
+    if (p.ht && !slot_per_token && !state_per_token) store_state(p.ht + state_off);
 }
 
 template <typename T, int KMAX, bool VFIRST>
@@ -277,11 +296,11 @@ extern "C" int gdn_fused_recurrent_fwd(
     const void* g, const void* beta, const float* gk, const float* gv,
     const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
-    const void* cu_seqlens, const void* state_slots,
+    const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    GDN_CHECK_ARG(q && k && v && o, GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: q, k, v, o must not be NULL");
+    GDN_CHECK_ARG(T == 0 || (q && k && v && o), GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: q, k, v, o must not be NULL");
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && K >= 1 && V >= 1 && N >= 1, GDN_ERR_INVALID,
                   "gdn_fused_recurrent_fwd: non-positive dimension");
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: HV=%lld not divisible by H=%lld",
@@ -296,13 +315,26 @@ extern "C" int gdn_fused_recurrent_fwd(
                       ((uintptr_t)gv % 16) == 0,
                   GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: h0/ht/gk/gv must be 16-byte aligned");
     GDN_CHECK_ARG(!(A_log && !g), GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: A_log given without g");
-    if (T == 0) return GDN_OK;
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_SLOT_PER_TOKEN) || (state_slots && h0 && slots_stride >= 1), GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: GDN_FLAG_SLOT_PER_TOKEN needs state_slots, the pool as h0 and slots_stride >= 1");
+    GDN_CHECK_ARG(!num_accepted || (flags & GDN_FLAG_SLOT_PER_TOKEN), GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: num_accepted needs GDN_FLAG_SLOT_PER_TOKEN");
+    GDN_CHECK_ARG(!((flags & GDN_FLAG_SLOT_PER_TOKEN) && (flags & GDN_FLAG_STATE_PER_TOKEN)), GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: GDN_FLAG_SLOT_PER_TOKEN and GDN_FLAG_STATE_PER_TOKEN exclude each other");
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_PER_TOKEN) || (ht && ht != h0), GDN_ERR_INVALID,
+                  "gdn_fused_recurrent_fwd: GDN_FLAG_STATE_PER_TOKEN needs ht [tokens,HV,K,V] distinct from h0");
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0) {
+        // no token: the final states are the initial ones (nothing to do for pools and per-token states)
+        if (ht && !state_slots && !(flags & GDN_FLAG_STATE_PER_TOKEN)) return launch_state_copy(h0, ht, N * HV * K * V, s);
+        return GDN_OK;
+    }
     RecurrentParams p;
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.gk = gk; p.gv = gv;
     p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o; p.cu_seqlens = cu_seqlens; p.state_slots = state_slots;
+    p.num_accepted = num_accepted; p.slots_stride = slots_stride;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.K = (int)K; p.V = (int)V; p.NVB = 1;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
-    hipStream_t s = (hipStream_t)stream;
     switch (qkv_dtype) {
         case GDN_DTYPE_BF16: return launch_t<bf16_t>(p, N * HV, s);
         case GDN_DTYPE_F16: return launch_t<f16_t>(p, N * HV, s);

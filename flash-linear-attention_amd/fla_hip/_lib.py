@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -26,6 +26,8 @@ FLAG_STATE_V_FIRST = 1 << 3
 FLAG_BETA_VECTOR = 1 << 4
 FLAG_CU_INT32 = 1 << 5
 FLAG_SLOT_INT32 = 1 << 6
+FLAG_SLOT_PER_TOKEN = 1 << 7
+FLAG_STATE_PER_TOKEN = 1 << 8
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
 FLAG_SEQ_ORDER = 1 << 19
@@ -43,10 +45,10 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p,            # g beta gk gv
         c_void_p, c_void_p,                                # A_log dt_bias
         c_void_p, c_void_p, c_void_p,                      # h0 ht o
-        c_void_p, c_void_p,                                # cu_seqlens state_slots
+        c_void_p, c_void_p, c_void_p, c_int64,             # cu_seqlens state_slots num_accepted slots_stride
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
         c_float, c_int, c_int, c_uint32, c_void_p]),
-    'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64]),
+    'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_uint32]),
     'gdn_causal_conv1d_fwd': (c_int, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # x weight bias residual initial_state
         c_void_p, c_void_p, c_void_p,                      # y final_state cu_seqlens

@@ -138,7 +138,7 @@ class ChunkLaunch:
         self.h0 = h0
 
         self.lib = _lib.load()
-        ws_bytes = self.lib.gdn_chunk_workspace_bytes(num_chunks, H, HV, KP, VP)
+        ws_bytes = self.lib.gdn_chunk_workspace_bytes(N, T, num_chunks, H, HV, KP, VP, int(cu_seqlens is not None), flags)
         if ws_bytes == 0 and num_chunks > 0:
             raise NotImplementedError(f'HIP chunk kernels do not cover K={KP}, V={VP}')
         self.workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -152,12 +152,8 @@ class ChunkLaunch:
             float(scale), dtype_code(work_dtype), gb_code, flags)
 
     def run(self, stage: str | None = None) -> None:
-        B, T = self.dims[0], self.dims[1]
-        if T > 0:
-            fn = getattr(self.lib, self._ENTRY[stage])
-            _lib.check(fn(*self.args, current_stream_ptr(self.device)))
-        elif self.ht is not None:
-            self.ht.copy_(self.h0) if self.h0 is not None else self.ht.zero_()
+        fn = getattr(self.lib, self._ENTRY[stage])          # (without tokens the library copies h0 into ht)
+        _lib.check(fn(*self.args, current_stream_ptr(self.device)))
 
     def results(self) -> tuple[torch.Tensor, torch.Tensor | None]:
         B, T, H, HV, K, V, N = self.dims

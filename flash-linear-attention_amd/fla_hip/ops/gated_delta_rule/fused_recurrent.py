@@ -42,12 +42,16 @@ def fused_recurrent_gated_delta_rule_fwd(
     cu_seqlens: torch.Tensor | None = None,
     inplace_final_state: bool = False,
     ssm_state_indices: torch.Tensor | None = None,
+    num_accepted_tokens: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Allocates ``o`` (v's dtype) and the fp32 final state, then launches the HIP kernel on
     the current stream.  With ``inplace_final_state`` the final state is written over
     ``initial_state`` (which must then be fp32 and contiguous) and that tensor is returned.
-    With ``ssm_state_indices`` ``[N]`` the states are slots of the pool ``initial_state
-    [num_slots, HV, K, V]``, updated in place."""
+    With ``ssm_state_indices`` the states are slots of the pool ``initial_state
+    [num_slots, HV, K, V]``: ``[N]`` names one slot per sequence, updated in place; ``[N, T]`` names
+    a slot per token (the state after token t goes to slot ``[n, t]``, and the sequence starts from
+    slot ``[n, num_accepted_tokens[n] - 1]``, or ``[n, 0]``).  Without ``inplace_final_state`` the
+    pool is only read and the states after every token are returned as ``[B * T, HV, K, V]``."""
     dev = require_gpu(q, k, v)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
@@ -55,6 +59,22 @@ def fused_recurrent_gated_delta_rule_fwd(
     q, k, v = unify_qkv(q, k, v)
     g, beta, gb_code = unify_gate_beta(g, beta)
     gk, gv, A_log, dt_bias = as_f32(gk), as_f32(gv), as_f32(A_log), as_f32(dt_bias)
+
+    # The kernel moves 16-byte pieces of state rows.  Head dims that are not multiples of 4 are zero-padded
+    # here (zero key features and zero value columns change nothing else) and the results cut back.
+    KP, VP = (K + 3) // 4 * 4, (V + 3) // 4 * 4
+    padded = (KP, VP) != (K, V)
+    if padded:
+        if inplace_final_state or ssm_state_indices is not None:
+            raise NotImplementedError('in-place and pooled states need head dims that are multiples of 4')
+        pad = torch.nn.functional.pad
+        q, k, v = pad(q, (0, KP - K)), pad(k, (0, KP - K)), pad(v, (0, VP - V))
+        gk = None if gk is None else pad(gk, (0, KP - K))
+        gv = None if gv is None else pad(gv, (0, VP - V))
+        if beta is not None and beta.ndim == v.ndim:
+            beta = pad(beta, (0, VP - V))
+        if initial_state is not None:
+            initial_state = pad(initial_state, (0, KP - K, 0, VP - V) if state_v_first else (0, VP - V, 0, KP - K))
 
     flags = 0
     if use_qk_l2norm_in_kernel:
@@ -75,20 +95,51 @@ def fused_recurrent_gated_delta_rule_fwd(
         if cu_seqlens.device != dev:
             cu_seqlens = cu_seqlens.to(dev)
 
-    state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+    state_shape = (N, HV, VP, KP) if state_v_first else (N, HV, KP, VP)
     h0 = initial_state
-    slots = None
+    slots = accepted = None
+    slots_stride = 1
+    per_token_out = False
+    if num_accepted_tokens is not None and (ssm_state_indices is None or ssm_state_indices.ndim != 2):
+        raise ValueError('num_accepted_tokens needs ssm_state_indices of shape (N, T)')
     if ssm_state_indices is not None:
-        if not inplace_final_state or h0 is None:
-            raise ValueError('ssm_state_indices needs the state pool as initial_state and inplace_final_state=True')
-        if ssm_state_indices.ndim != 1 or ssm_state_indices.shape[0] != N:
-            raise ValueError(f'ssm_state_indices must have shape ({N},), got {tuple(ssm_state_indices.shape)}')
+        if h0 is None:
+            raise ValueError('ssm_state_indices needs the state pool as initial_state')
+        if ssm_state_indices.ndim == 1:
+            if not inplace_final_state:
+                raise ValueError('ssm_state_indices of shape (N,) needs inplace_final_state=True')
+            if ssm_state_indices.shape[0] != N:
+                raise ValueError(f'ssm_state_indices must have shape ({N},), got {tuple(ssm_state_indices.shape)}')
+        elif ssm_state_indices.ndim == 2:
+            if ssm_state_indices.shape[0] != N:
+                raise ValueError(f'ssm_state_indices must have {N} rows, got {tuple(ssm_state_indices.shape)}')
+            if cu_seqlens is None and ssm_state_indices.shape[1] < T:
+                raise ValueError(f'ssm_state_indices needs a slot for each of the {T} tokens of a sequence, '
+                                 f'got {tuple(ssm_state_indices.shape)}')
+            if inplace_final_state:
+                flags |= _lib.FLAG_SLOT_PER_TOKEN
+            slots_stride = ssm_state_indices.shape[1]
+        else:
+            raise ValueError('ssm_state_indices must have one or two dimensions')
         slots = ssm_state_indices.to(dev)
         if slots.dtype == torch.int32:
             flags |= _lib.FLAG_SLOT_INT32
         elif slots.dtype != torch.int64:
             slots = slots.long()
         slots = slots.contiguous()
+        if num_accepted_tokens is not None:
+            if num_accepted_tokens.shape != (N,):
+                raise ValueError(f'num_accepted_tokens must have shape ({N},), got {tuple(num_accepted_tokens.shape)}')
+            accepted = num_accepted_tokens.to(device=dev, dtype=slots.dtype).contiguous()
+        if not inplace_final_state:
+            # read-only pool; the kernel finds the first slot the same way and returns a state per token
+            per_token_out = True
+            flags |= _lib.FLAG_STATE_PER_TOKEN
+            if ssm_state_indices.ndim == 2:
+                # (the start slot is picked on the host side of the kernel argument list: a gather of N indices)
+                first = (accepted - 1) if accepted is not None else torch.zeros(N, dtype=slots.dtype, device=dev)
+                slots = slots.gather(1, first.long()[:, None])[:, 0].to(slots.dtype).contiguous()
+                accepted, slots_stride = None, 1
         state_shape = (h0.shape[0],) + state_shape[1:]            # the pool has its own number of slots
     if h0 is not None:
         if tuple(h0.shape) != state_shape:
@@ -105,15 +156,21 @@ def fused_recurrent_gated_delta_rule_fwd(
         if initial_state is None:
             raise ValueError('inplace_final_state=True requires initial_state')
         final_state = h0
+    elif per_token_out:
+        final_state = torch.empty((B * T,) + state_shape[1:], dtype=torch.float32, device=dev)
     elif output_final_state:
         final_state = torch.empty(state_shape, dtype=torch.float32, device=dev)
 
     lib = _lib.load()
     _lib.check(lib.gdn_fused_recurrent_fwd(
         ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(gk), ptr(gv), ptr(A_log), ptr(dt_bias),
-        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots),
-        B, T, H, HV, K, V, N, float(scale), dtype_code(q.dtype), gb_code, flags,
+        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots), ptr(accepted), slots_stride,
+        B, T, H, HV, KP, VP, N, float(scale), dtype_code(q.dtype), gb_code, flags,
         current_stream_ptr(dev)))
+    if padded:
+        o = o[..., :V].contiguous()
+        if final_state is not None:
+            final_state = (final_state[..., :V, :K] if state_v_first else final_state[..., :K, :V]).contiguous()
     return o, final_state
 
 
@@ -157,7 +214,12 @@ def fused_recurrent_gated_delta_rule(
         ssm_state_indices (keyword only, extension; the sibling KDA operator's argument,
             fla/ops/kda/fused_recurrent.py:248-326): ``[N]`` int32/int64 slot of every sequence in the
             state pool ``initial_state [num_slots, HV, K, V]``; needs ``inplace_final_state=True``.
-            Slots must be distinct; slots that are not named keep their contents.
+            Slots must be distinct; slots that are not named keep their contents.  ``[N, T]`` names a slot
+            per token (speculative decoding, fla/ops/kda/fused_recurrent.py:131-145,203-219): the state after
+            token t of sequence n goes to slot ``[n, t]``; without ``inplace_final_state`` the pool is only read
+            and the states after every token are returned as ``[B * T, HV, K, V]``.
+        num_accepted_tokens (keyword only, extension): ``[N]``; with ``ssm_state_indices [N, T]`` sequence n
+            starts from slot ``[n, num_accepted_tokens[n] - 1]`` instead of ``[n, 0]``.
 
     Returns:
         ``(o [B, T, HV, V] in v's dtype, final_state or None)``.
@@ -170,6 +232,7 @@ def fused_recurrent_gated_delta_rule(
         state_v_first = kwargs.pop('transpose_state_layout')
     inplace_final_state = bool(kwargs.pop('inplace_final_state', False))
     ssm_state_indices = kwargs.pop('ssm_state_indices', None)
+    num_accepted_tokens = kwargs.pop('num_accepted_tokens', None)
 
     if q.shape[2] != k.shape[2]:
         raise ValueError(f'q and k must have the same number of heads, got {q.shape[2]} and {k.shape[2]}')
@@ -203,7 +266,7 @@ def fused_recurrent_gated_delta_rule(
     return fused_recurrent_gated_delta_rule_fwd(
         q, k, v, g, gk, gv, beta, A_log, dt_bias, scale, initial_state, output_final_state,
         use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, cu_seqlens,
-        inplace_final_state, ssm_state_indices)
+        inplace_final_state, ssm_state_indices, num_accepted_tokens)
 
 
 fused_recurrent_gdn = fused_recurrent_gated_delta_rule

@@ -41,7 +41,9 @@ extern "C" {
 #define GDN_FLAG_STATE_V_FIRST  (1u << 3)  /* state_v_first: states are [N,HV,V,K]              */
 #define GDN_FLAG_BETA_VECTOR    (1u << 4)  /* beta is [B,T,HV,V] instead of [B,T,HV]            */
 #define GDN_FLAG_CU_INT32       (1u << 5)  /* cu_seqlens / chunk tables are int32, else int64   */
-#define GDN_FLAG_SLOT_INT32     (1u << 6)  /* state_slots is int32, else int64                  */
+#define GDN_FLAG_SLOT_INT32     (1u << 6)  /* state_slots / num_accepted are int32, else int64  */
+#define GDN_FLAG_SLOT_PER_TOKEN (1u << 7)  /* state_slots is [N, slots_stride]: a slot per token */
+#define GDN_FLAG_STATE_PER_TOKEN (1u << 8) /* ht is [tokens,HV,K,V]: the state after every token */
 /* gdn_chunk_fwd only: force one form of the sequential stage instead of the automatic choice
  * (all forms give the same result up to rounding; used by tests and for tuning)                */
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
@@ -78,23 +80,31 @@ const char* gdn_last_error(void);
  *          are [num_slots,HV,K,V] and are addressed through the slot instead of n (continuous batching; the
  *          sibling KDA operator's ssm_state_indices, fla/ops/kda/fused_recurrent.py:27,75-91,145-159).  Slots
  *          must be distinct; other slots are not touched.
+ *          With GDN_FLAG_SLOT_PER_TOKEN (speculative decoding, fla/ops/kda/fused_recurrent.py:131-145,203-219)
+ *          state_slots is [N][slots_stride] (slots_stride >= tokens of the longest sequence): sequence n starts
+ *          from slot state_slots[n][num_accepted[n]-1] (num_accepted [N], same integer type as state_slots; NULL:
+ *          entry 0) and the state after its token t is written to slot state_slots[n][t] of ht.
+ *   GDN_FLAG_STATE_PER_TOKEN: ht is [B*T,HV,K,V] and receives the state after every token (the reference's
+ *          continuous-batching form without inplace_final_state, fused_recurrent.py:212-213); h0 as usual.
  *   N = B when cu_seqlens == NULL.  Requires K <= 256, K % 4 == 0, V % 4 == 0, HV % H == 0.
+ *   T == 0: ht = h0 (zeros without h0).
  */
 int gdn_fused_recurrent_fwd(
     const void* q, const void* k, const void* v,
     const void* g, const void* beta, const float* gk, const float* gv,
     const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
-    const void* cu_seqlens, const void* state_slots,
+    const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
- * Bytes of device workspace gdn_chunk_fwd needs for `num_chunks` 64-token
- * chunks (dense: B*ceil(T/64); packed: sum over sequences of ceil(len/64)).
- * Returns 0 for unsupported (K,V).
+ * Bytes of device workspace gdn_chunk_fwd needs for the same N, T, num_chunks (64-token chunks; dense:
+ * B*ceil(T/64); packed: sum over sequences of ceil(len/64)), head counts, packed (cu_seqlens given) and flags
+ * (the scan flags change the plan and with it the size).  Returns 0 for unsupported (K,V).
  */
-size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V);
+size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V,
+                                 int packed, uint32_t flags);
 
 /*
  * Chunked prefill, chunk size 64.  Replaces chunk_gated_delta_rule_fwd
@@ -122,6 +132,7 @@ size_t gdn_chunk_workspace_bytes(int64_t num_chunks, int64_t H, int64_t HV, int6
  *         With GDN_FLAG_SEQ_ORDER the array has N more entries: the sequence ids in the order in
  *         which the sequential kernel should start them (longest first keeps the CUs evenly loaded)
  *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
+ *   T == 0 (or no chunk at all): ht = h0 (zeros without h0), nothing else is written.
  *   Requires K, V multiples of 8 up to 128 and HV % H == 0.  The kernels work on 128 x 128 states: key features past K
  *   count as zero and value columns past V are not stored (same time as K = V = 128; the Python host zero-pads
  *   head dims that are not multiples of 8).

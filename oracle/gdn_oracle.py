@@ -24,7 +24,9 @@ independent pure-python loops on tiny shapes, closed forms for one decode step
 (beta=0, exact projection), ``torch.linalg.inv`` for the triangular solve,
 recurrent == chunked, split-in-time hand-off, varlen == per-sequence loop,
 GVA == repeat_interleave, state_v_first == transpose, and the committed
-fixtures under ``tests/golden/``.  No function here is "parity unpinned".
+fixtures under ``tests/golden/`` (a second set of scalar fixtures pins the
+optional arguments gk, gv, beta per value column and the pooled states of
+speculative decoding).  No function here is "parity unpinned".
 
 Everything is computed in ``dtype`` (float32 by default, float64 for tight
 pins); inputs are upcast first, so bf16 inputs are consumed as their exact
@@ -180,6 +182,44 @@ def recurrent_gated_delta_rule(
     if not output_final_state:
         return o, None
     return o, (ht.transpose(-1, -2).contiguous() if state_v_first else ht)
+
+
+def recurrent_gated_delta_rule_pooled(
+    q, k, v, g, beta, scale, pool, ssm_state_indices, num_accepted_tokens=None, cu_seqlens=None,
+    dtype=torch.float32, **flags,
+):
+    """Token recurrence over states kept in a pool [num_slots,HV,K,V] (continuous batching and
+    speculative decoding, fla/ops/kda/fused_recurrent.py:131-145,203-219).
+
+    ssm_state_indices [N]: sequence n reads and finally rewrites slot [n].
+    ssm_state_indices [N,Tmax]: sequence n starts from slot [n, num_accepted_tokens[n]-1] (entry 0
+    without num_accepted_tokens) and the state after its token t is written to slot [n, t].
+    Returns (o, pool after the call, states after every token [tokens,HV,K,V]).  Built on
+    recurrent_gated_delta_rule, one token at a time, chained through its final state."""
+    B, T = k.shape[:2]
+    idx = torch.as_tensor(ssm_state_indices).long()
+    bounds = [(b, 0, T) for b in range(B)] if cu_seqlens is None else \
+        [(0, int(s), int(e)) for s, e in zip(cu_seqlens[:-1], cu_seqlens[1:])]
+    pool_after = pool.to(dtype).clone()
+    HV, V = v.shape[2], v.shape[3]
+    o = torch.zeros(B, T, HV, V, dtype=dtype)
+    per_token = torch.zeros((B * T,) + tuple(pool.shape[1:]), dtype=dtype)
+    for n, (b, s, e) in enumerate(bounds):
+        if idx.dim() == 1:
+            first = int(idx[n])
+        else:
+            first = int(idx[n, int(num_accepted_tokens[n]) - 1 if num_accepted_tokens is not None else 0])
+        S = pool[first:first + 1].to(dtype)
+        for t in range(s, e):
+            sl = lambda x: None if x is None else x[b:b + 1, t:t + 1]
+            o1, S = recurrent_gated_delta_rule(sl(q), sl(k), sl(v), sl(g), sl(beta), scale, S, True, dtype=dtype, **flags)
+            o[b, t] = o1[0, 0]
+            per_token[b * T + t] = S[0]
+            if idx.dim() == 2:
+                pool_after[int(idx[n, t - s])] = S[0]
+        if idx.dim() == 1 and e > s:
+            pool_after[first] = S[0]
+    return o, pool_after, per_token
 
 
 # --------------------------------------------------------------------------- #

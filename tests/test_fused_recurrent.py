@@ -251,6 +251,136 @@ def test_state_pool_addressed_by_slot(idx_dtype, vfirst, cu):
                output_final_state=True, ssm_state_indices=torch.tensor(slots, device=dev))
 
 
+@pytest.mark.parametrize('idx_dtype', [torch.int32, torch.int64])
+@pytest.mark.parametrize('vfirst,cu', [(False, None), (True, None), (False, [0, 3, 4, 6])])
+def test_speculative_decoding_slot_per_token(idx_dtype, vfirst, cu):
+    """ssm_state_indices [N, T] with num_accepted_tokens (fla/ops/kda/fused_recurrent.py:131-145,203-219):
+    each sequence starts from the slot of its last accepted token and leaves the state after draft
+    token t in slot [n, t]; slots nobody writes keep their contents."""
+    H, HV, D, slots_total, N, TMAX = 2, 4, 128, 16, 3, 3
+    gen = torch.Generator().manual_seed(21)
+    pool = torch.randn(slots_total, HV, D, D, generator=gen)
+    idx = torch.randperm(slots_total, generator=gen)[:N * TMAX].view(N, TMAX)
+    accepted = torch.tensor([2, 1, 3])
+    if cu is None:
+        q, k, v, g, beta, _ = _inputs(N, TMAX, H, HV, D, torch.bfloat16, seed=11)
+        lens = [TMAX] * N
+    else:
+        q, k, v, g, beta, _ = _inputs(1, cu[-1], H, HV, D, torch.bfloat16, seed=11)
+        lens = [b - a for a, b in zip(cu[:-1], cu[1:])]
+        accepted = torch.tensor([2, 1, 2])
+    ref_o, ref_pool, ref_tok = O.recurrent_gated_delta_rule_pooled(q, k, v, g, beta, None, pool, idx, accepted, cu_seqlens=cu)
+    dev = 'cuda'
+    lay = (lambda x: x.transpose(-1, -2).contiguous()) if vfirst else (lambda x: x.contiguous())
+    dpool = lay(pool).to(dev)
+    before = dpool.clone()
+    kw = dict(beta=beta.to(dev), state_v_first=vfirst, cu_seqlens=None if cu is None else torch.tensor(cu, device=dev),
+              ssm_state_indices=idx.to(device=dev, dtype=idx_dtype), num_accepted_tokens=accepted.to(dev))
+    # read-only pool: a state per token comes back
+    o, per_tok = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), initial_state=dpool, **kw)
+    assert torch.equal(dpool, before)
+    _check('o', ref_o, o)
+    _check('per-token states', lay(ref_tok), per_tok)
+    # in place: slot [n, t] receives the state after token t
+    o2, out = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), initial_state=dpool, inplace_final_state=True, **kw)
+    assert out.data_ptr() == dpool.data_ptr() and torch.equal(o2, o)
+    written = sorted({int(idx[n, t]) for n in range(N) for t in range(lens[n])})
+    rest = [i for i in range(slots_total) if i not in written]
+    _check('pool', lay(ref_pool)[written], dpool[written])
+    assert torch.equal(dpool[rest], before[rest]), 'a slot that no token named was modified'
+    with pytest.raises(ValueError):
+        _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), initial_state=dpool, beta=beta.to(dev),
+               ssm_state_indices=idx[:, 0].to(dev), num_accepted_tokens=accepted.to(dev), inplace_final_state=True)
+
+
+def test_spec_pool_scalar_fixture_on_the_gpu():
+    import os
+    import numpy as np
+    gold = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'gdn_scalar_cases_ext.npz'))
+    t = lambda key: torch.from_numpy(gold[f'spec_pool.{key}'])
+    dev = 'cuda'
+    pool = t('pool').float().to(dev)
+    o, _ = _ops()(t('q')[None].float().to(dev), t('k')[None].float().to(dev), t('v')[None].float().to(dev),
+                  t('g')[None].float().to(dev), beta=t('beta')[None].float().to(dev), scale=float(gold['spec_pool.scale']),
+                  initial_state=pool, inplace_final_state=True, cu_seqlens=t('cu').to(dev),
+                  ssm_state_indices=t('idx').to(dev), num_accepted_tokens=t('accepted').to(dev))
+    _check('o', t('o')[None].float(), o, 1e-5)
+    _check('pool', t('pool_after').float(), pool, 1e-5)
+
+
+@pytest.mark.parametrize('name', ['gk_gv_vbeta', 'gk_only_varlen', 'gv_vbeta_varlen'])
+@pytest.mark.parametrize('vfirst', [False, True])
+def test_optional_decay_scalar_fixtures_on_the_gpu(name, vfirst):
+    """gk, gv and beta per value column against the scalar fixtures directly (K and V are 2 or 3 there:
+    the host pads head dims that are not multiples of 4)."""
+    import os
+    import numpy as np
+    gold = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'gdn_scalar_cases_ext.npz'))
+    dev = 'cuda'
+    t = lambda key: torch.from_numpy(gold[f'{name}.{key}'])[None].float().to(dev) if f'{name}.{key}' in gold.files else None
+    h0 = torch.from_numpy(gold[f'{name}.h0']).float()
+    o, ht = _ops()(t('q'), t('k'), t('v'), t('g'), gk=t('gk'), gv=t('gv'), beta=t('beta'), scale=float(gold[f'{name}.scale']),
+                   initial_state=(h0.transpose(-1, -2).contiguous() if vfirst else h0).to(dev), output_final_state=True,
+                   state_v_first=vfirst, cu_seqlens=torch.from_numpy(gold[f'{name}.cu']).to(dev))
+    _check('o', torch.from_numpy(gold[f'{name}.o'])[None].float(), o, 1e-5)
+    ref_ht = torch.from_numpy(gold[f'{name}.ht']).float()
+    _check('ht', ref_ht.transpose(-1, -2) if vfirst else ref_ht, ht, 1e-5)
+
+
+@pytest.mark.parametrize('K,V', [(50, 30), (6, 130), (129, 3)])
+def test_head_dims_that_are_not_multiples_of_four(K, V):
+    # the reference takes any K <= 256 (BK = next_power_of_2(K), fla/ops/gated_delta_rule/fused_recurrent.py:206-208)
+    gen = torch.Generator().manual_seed(K * 1000 + V)
+    B, T, H, HV = 2, 5, 1, 2
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g, beta = -torch.rand(B, T, HV, generator=gen), torch.rand(B, T, HV, generator=gen)
+    h0 = torch.randn(B, HV, K, V, generator=gen)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, use_qk_l2norm_in_kernel=True)
+    dev = 'cuda'
+    o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=h0.to(dev),
+                   output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o.shape == ref_o.shape and ht.shape == ref_ht.shape
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+@pytest.mark.parametrize('vfirst', [False, True])
+def test_missing_beta_counts_as_ones_before_the_sigmoid(vfirst):
+    # fla/ops/gated_delta_rule/fused_recurrent.py:443: beta = ones, then the in-kernel sigmoid still applies
+    q, k, v, g, _, h0 = _inputs(2, 3, 2, 4, 64, torch.float32, seed=3)
+    dev = 'cuda'
+    for neg in (False, True):
+        ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, torch.ones(2, 3, 4), None, h0, True,
+                                                     use_beta_sigmoid_in_kernel=True, allow_neg_eigval=neg,
+                                                     use_qk_l2norm_in_kernel=True)
+        st = h0.transpose(-1, -2).contiguous() if vfirst else h0
+        o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), initial_state=st.to(dev), output_final_state=True,
+                       use_beta_sigmoid_in_kernel=True, allow_neg_eigval=neg, use_qk_l2norm_in_kernel=True, state_v_first=vfirst)
+        _check('o', ref_o, o)
+        _check('ht', ref_ht.transpose(-1, -2) if vfirst else ref_ht, ht)
+
+
+def test_no_tokens_returns_the_initial_state():
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    dev = 'cuda'
+    h0 = torch.randn(2, 4, 64, 64, device=dev)
+    e = lambda *shape: torch.empty(*shape, device=dev, dtype=torch.bfloat16)
+    for op in (_ops(), chunk_gated_delta_rule):
+        poison = torch.full((1 << 20,), float('nan'), device=dev); del poison       # what torch.empty may hand back
+        o, ht = op(e(2, 0, 2, 64), e(2, 0, 2, 64), e(2, 0, 4, 64), e(2, 0, 4).float(), beta=e(2, 0, 4).float(),
+                   initial_state=h0, output_final_state=True)
+        assert o.shape == (2, 0, 4, 64) and torch.equal(ht, h0) and ht.data_ptr() != h0.data_ptr()
+        o, ht = op(e(2, 0, 2, 64), e(2, 0, 2, 64), e(2, 0, 4, 64), e(2, 0, 4).float(), beta=e(2, 0, 4).float(),
+                   output_final_state=True)
+        assert torch.equal(ht, torch.zeros_like(h0))
+    # packed input whose sequences are all empty
+    cu = torch.zeros(3, dtype=torch.long, device=dev)
+    o, ht = chunk_gated_delta_rule(e(1, 0, 2, 64), e(1, 0, 2, 64), e(1, 0, 4, 64), e(1, 0, 4).float(), e(1, 0, 4).float(),
+                                   initial_state=h0, output_final_state=True, cu_seqlens=cu)
+    assert torch.equal(ht, h0)
+
+
 def test_decode_and_prefill_replay_from_a_captured_graph():
     """Serving loops replay captured graphs: the entry points only enqueue kernels on the given
     stream (no allocation, no memset, no synchronisation of their own), so a captured decode step

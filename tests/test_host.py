@@ -27,16 +27,23 @@ def test_library_exports_every_declared_symbol():
     assert _lib.load().gdn_hip_abi_version() == _lib.ABI_VERSION
     # pure host-side entry points can be called without a GPU
     l = _lib.load()
-    assert l.gdn_chunk_workspace_bytes(8, 2, 4, 128, 128) > 0
-    assert l.gdn_chunk_workspace_bytes(8, 2, 4, 64, 96) > 0          # multiples of 8 up to 128 are taken as they are
-    assert l.gdn_chunk_workspace_bytes(8, 2, 4, 100, 128) == 0
+    ws = lambda N, T, NC, H, HV, K, V, packed=0, flags=0: l.gdn_chunk_workspace_bytes(N, T, NC, H, HV, K, V, packed, flags)
+    assert ws(1, 512, 8, 2, 4, 128, 128) > 0
+    assert ws(1, 512, 8, 2, 4, 64, 96) > 0          # multiples of 8 up to 128 are taken as they are
+    assert ws(1, 512, 8, 2, 4, 100, 128) == 0
+    # the segment matrices are reserved only when the plan cuts time into segments: long dense input with few heads
+    rec = 11264
+    assert ws(1, 32768, 512, 16, 32, 128, 128) == 512 * 32 * rec + 3 * 8 * 32 * 65536
+    assert ws(1, 32768, 512, 16, 32, 128, 128, 0, _lib.FLAG_SCAN_WIDE) == 512 * 32 * rec
+    assert ws(32, 65536, 1040, 16, 32, 128, 128, 1) == 1040 * 32 * rec                 # packed input never does
+    assert ws(64, 4096, 64 * 64, 16, 32, 128, 128) == 64 * 64 * 32 * rec               # enough runs already
     # argument errors are reported before any launch
-    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None,
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None, None, 1,
                                    1, 1, 2, 3, 64, 64, 1, 1.0, 0, 2, 0, None)
     assert rc == _lib.GDN_ERR_INVALID and 'divisible' in _lib.last_error()
     with pytest.raises(ValueError):
         _lib.check(rc)
-    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None,
+    rc = l.gdn_fused_recurrent_fwd(1, 1, 1, None, None, None, None, None, None, None, None, 1, None, None, None, 1,
                                    1, 1, 1, 1, 512, 64, 1, 1.0, 0, 2, 0, None)
     assert rc == _lib.GDN_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):

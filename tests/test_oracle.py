@@ -44,6 +44,55 @@ def test_chunk_matches_scalar_fixture(name, chunk):
     assert torch.allclose(ht, c['ht'], atol=1e-6, rtol=1e-6)
 
 
+GOLD_EXT = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'gdn_scalar_cases_ext.npz'))
+
+
+def _ext(name, key):
+    return torch.from_numpy(GOLD_EXT[f'{name}.{key}']) if f'{name}.{key}' in GOLD_EXT.files else None
+
+
+@pytest.mark.parametrize('name', ['gk_gv_vbeta', 'gk_only_varlen', 'gv_vbeta_varlen'])
+def test_optional_decays_and_vector_beta_match_scalar_fixture(name):
+    # pins the gk / gv / beta-per-value-column branches of the oracle against the independent scalar loop
+    b1 = lambda x: None if x is None else x[None]
+    o, ht = O.recurrent_gated_delta_rule(
+        b1(_ext(name, 'q')), b1(_ext(name, 'k')), b1(_ext(name, 'v')), b1(_ext(name, 'g')), b1(_ext(name, 'beta')),
+        float(GOLD_EXT[f'{name}.scale']), _ext(name, 'h0'), True, cu_seqlens=GOLD_EXT[f'{name}.cu'].tolist(),
+        gk=b1(_ext(name, 'gk')), gv=b1(_ext(name, 'gv')), dtype=torch.float64)
+    assert torch.allclose(o[0], _ext(name, 'o'), atol=1e-12, rtol=1e-10)
+    assert torch.allclose(ht, _ext(name, 'ht'), atol=1e-12, rtol=1e-10)
+    # a slip that swaps gk and gv (or drops one) must not pass: the fixture has K != V or only one of them
+    assert _ext(name, 'gk') is None or _ext(name, 'gv') is None or _ext(name, 'gk').shape != _ext(name, 'gv').shape
+
+
+def test_pooled_states_of_speculative_decoding_match_scalar_fixture():
+    n = 'spec_pool'
+    o, pool_after, _ = O.recurrent_gated_delta_rule_pooled(
+        _ext(n, 'q')[None], _ext(n, 'k')[None], _ext(n, 'v')[None], _ext(n, 'g')[None], _ext(n, 'beta')[None],
+        float(GOLD_EXT[f'{n}.scale']), _ext(n, 'pool'), _ext(n, 'idx'), _ext(n, 'accepted'),
+        cu_seqlens=GOLD_EXT[f'{n}.cu'].tolist(), dtype=torch.float64)
+    assert torch.allclose(o[0], _ext(n, 'o'), atol=1e-12, rtol=1e-10)
+    assert torch.allclose(pool_after, _ext(n, 'pool_after'), atol=1e-12, rtol=1e-10)
+    # slots nobody names keep their contents; named ones changed
+    named = set(_ext(n, 'idx').flatten().tolist())
+    lens = np.diff(GOLD_EXT[f'{n}.cu'])
+    written = {int(_ext(n, 'idx')[i, t]) for i in range(len(lens)) for t in range(lens[i])}
+    for slot in range(_ext(n, 'pool').shape[0]):
+        same = torch.equal(pool_after[slot], _ext(n, 'pool')[slot])
+        assert same == (slot not in written), (slot, slot in named)
+
+
+def test_pooled_one_slot_per_sequence_equals_plain_call():
+    q, k, v, g, beta, h0 = O.make_inputs(3, 4, 1, 2, 4, 4, seed=5, h0_std=1.0, N=7)
+    idx = torch.tensor([5, 0, 3])
+    o, pool_after, per_tok = O.recurrent_gated_delta_rule_pooled(q, k, v, g, beta, None, h0, idx)
+    o2, ht2 = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0[idx], True)
+    assert torch.allclose(o, o2, atol=1e-6) and torch.allclose(pool_after[idx], ht2, atol=1e-6)
+    assert torch.allclose(per_tok.view(3, 4, 2, 4, 4)[:, -1], ht2, atol=1e-6)
+    keep = [i for i in range(7) if i not in idx.tolist()]
+    assert torch.equal(pool_after[keep], h0[keep])
+
+
 def test_config1_recurrent_equals_chunk():
     # the CPU-runnable configuration: B=2 T=256 H=2 K=V=64 fp32, zero initial state
     q, k, v, g, beta, _ = O.make_inputs(2, 256, 2, 2, 64, 64, seed=42)
