@@ -90,7 +90,7 @@ static int chunk_entry(
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * H < (1ll << 31), GDN_ERR_UNSUPPORTED, "%s: too many heads or chunks for one launch", who);
     if (cu_seqlens) {
         GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
-        GDN_CHECK_ARG(chunk_table && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
+        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
     } else {
         GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
         GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
