@@ -138,3 +138,58 @@ extern "C" int gdn_chunk_fwd_prepare(GDN_CHUNK_ARGS) {
 extern "C" int gdn_chunk_fwd_scan(GDN_CHUNK_ARGS) {
     return chunk_entry("gdn_chunk_fwd_scan", gdn::STAGE_SCAN, GDN_CHUNK_PASS);
 }
+
+// ---------------------------------------------------------------------------------------------
+// gdn_chunk_fwd without any allocation: the workspace is a fixed array in device memory that
+// belongs to the library (one copy per GPU, held until the process ends).
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[GDN_CHUNK_STATIC_WORKSPACE_BYTES];
+
+// Device address of `scratch` on the current device.  The array's name is only a handle on the host:
+// its address on each GPU comes from hipGetSymbolAddress, asked once per device with that device current.
+static int static_workspace(const char* who, void** out) {
+    static void* addr[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return gdn::check_launch(who);
+    GDN_CHECK_ARG(dev >= 0 && dev < 64, GDN_ERR_UNSUPPORTED, "%s: device index %d not supported", who, dev);
+    void* p = __atomic_load_n(&addr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            gdn::set_error("%s: hipGetSymbolAddress(scratch): %s", who, hipGetErrorString(e));
+            (void)hipGetLastError();
+            return GDN_ERR_LAUNCH;
+        }
+        __atomic_store_n(&addr[dev], p, __ATOMIC_RELEASE);      // (every thread that asks gets the same address)
+    }
+    *out = p;
+    return GDN_OK;
+}
+
+extern "C" int gdn_chunk_fwd_static(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    const char* who = "gdn_chunk_fwd_static";
+    GDN_CHECK_ARG(chunk_dims_ok(K, V) && N >= 1 && T >= 0 && HV >= 1 && num_chunks >= 0, GDN_ERR_INVALID,
+                  "%s: bad dimensions", who);
+    // The plan with time segments needs room for their matrices; when only that does not fit, whole sequences do.
+    size_t need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, nullptr, nullptr);
+    if (need > GDN_CHUNK_STATIC_WORKSPACE_BYTES && !(flags & GDN_FLAG_SCAN_SEGMENTS)) {
+        flags |= GDN_FLAG_SCAN_WIDE;
+        need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, nullptr, nullptr);
+    }
+    GDN_CHECK_ARG(need <= GDN_CHUNK_STATIC_WORKSPACE_BYTES, GDN_ERR_WORKSPACE,
+                  "%s: this input needs %zu bytes of workspace, the built-in one holds %zu (%lld records of one chunk and "
+                  "value head); use gdn_chunk_fwd with a workspace of the caller",
+                  who, need, (size_t)GDN_CHUNK_STATIC_WORKSPACE_BYTES,
+                  (long long)(GDN_CHUNK_STATIC_WORKSPACE_BYTES / gdn::REC_BYTES));
+    void* workspace = nullptr;
+    if (int rc = static_workspace(who, &workspace)) return rc;
+    const size_t workspace_bytes = GDN_CHUNK_STATIC_WORKSPACE_BYTES;
+    return chunk_entry(who, gdn::STAGE_PREPARE | gdn::STAGE_SCAN, GDN_CHUNK_PASS);
+}

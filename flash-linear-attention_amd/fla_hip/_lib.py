@@ -76,6 +76,9 @@ _CHUNK_ARGS = [
 for _name in ('gdn_chunk_fwd', 'gdn_chunk_fwd_prepare', 'gdn_chunk_fwd_scan'):
     SIGNATURES[_name] = (c_int, _CHUNK_ARGS)
 
+SIGNATURES['gdn_chunk_fwd_static'] = (c_int, _CHUNK_ARGS[:13] + _CHUNK_ARGS[15:])     # no workspace, no size
+CHUNK_STATIC_WORKSPACE_BYTES = 64 << 20
+
 _lib = None
 _lock = threading.Lock()
 

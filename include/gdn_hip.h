@@ -177,6 +177,27 @@ int gdn_chunk_fwd_scan(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * gdn_chunk_fwd minus the workspace: the kernels use a fixed array of GDN_CHUNK_STATIC_WORKSPACE_BYTES that the
+ * library keeps in device memory (one per GPU it runs on, until the process ends).  The call allocates and frees
+ * nothing.  Inputs whose workspace (gdn_chunk_workspace_bytes) exceeds the array are refused with
+ * GDN_ERR_WORKSPACE; when only the plan with time segments is too large, whole sequences are scanned instead
+ * (same result up to rounding).  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * two threads) race, so serialise them.  The first call on a device looks up the array's address; make it
+ * outside a graph capture.
+ */
+#define GDN_CHUNK_STATIC_WORKSPACE_BYTES (64u << 20)
+int gdn_chunk_fwd_static(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* A_log, const float* dt_bias,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * The two memory-bound steps either side of the operator in the layer
  * (fla/layers/gated_deltanet.py:246-300 and :355-359).
  *

@@ -59,6 +59,8 @@ def test_flag_and_status_constants_match_the_header():
     assert len(flags) >= 11 and len(set(flags.values())) == len(flags)
     for name, value in flags.items():
         assert getattr(_lib, 'FLAG_' + name) == value, name
+    m = re.search(r'#define\s+GDN_CHUNK_STATIC_WORKSPACE_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)', header)
+    assert int(m.group(1)) << int(m.group(2)) == _lib.CHUNK_STATIC_WORKSPACE_BYTES
     for name, value in re.findall(r'#define\s+(GDN_ERR_\w+|GDN_OK)\s+\(?(-?\d+)\)?', header):
         assert getattr(_lib, name) == int(value), name
 
