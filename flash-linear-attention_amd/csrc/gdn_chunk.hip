@@ -77,7 +77,8 @@ static int chunk_entry(
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    GDN_CHECK_ARG(T == 0 || (q && k && v && g && beta && o), GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
+    GDN_CHECK_ARG(T == 0 || (q && k && v && beta && o), GDN_ERR_INVALID, "%s: q, k, v, beta, o must not be NULL", who);
+    GDN_CHECK_ARG(g || !A_log, GDN_ERR_INVALID, "%s: A_log given without g", who);
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1, GDN_ERR_INVALID, "%s: non-positive dimension", who);
     GDN_CHECK_ARG(!dt_bias || A_log, GDN_ERR_INVALID, "%s: dt_bias without A_log", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
     // (rows past the end of the sequence are zero) ----
     float rg = 0.f, rb = 0.f;
     if (w < G && lane < valid) {
-        rg = load_scalar(p.g, (tok0 + lane) * HV + h * G + w, p.gb_dtype);
+        rg = p.g ? load_scalar(p.g, (tok0 + lane) * HV + h * G + w, p.gb_dtype) : 0.f;      // (no gate: the plain delta rule)
         rb = load_scalar(p.beta, (tok0 + lane) * HV + h * G + w, p.gb_dtype);
     }
     {
@@ -107,12 +107,12 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         if (m >= 4) {                            // beyond the four fetched up front
             x = b = 0.f;
             if (lane < valid) {
-                x = load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype);
+                x = p.g ? load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype) : 0.f;
                 b = load_scalar(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
             }
         }
         if (lane < valid) {                      // optional activations of the raw gate / beta inputs
-            if (p.A_log) x = -__expf(p.A_log[hv]) * softplus_f(x + (p.dt_bias ? p.dt_bias[hv] : 0.f));
+            if (p.A_log && p.g) x = -__expf(p.A_log[hv]) * softplus_f(x + (p.dt_bias ? p.dt_bias[hv] : 0.f));
             if (p.flags & GDN_FLAG_BETA_SIGMOID) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
         }
 #pragma unroll

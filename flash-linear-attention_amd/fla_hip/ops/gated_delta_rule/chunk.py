@@ -37,6 +37,7 @@ _SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGM
 for _form in ('wide', 'segments'):
     for _runs in ('single', 'pair'):
         _SCAN_MODE_FLAGS[f'{_form}-{_runs}'] = _SCAN_MODE_FLAGS[_form] | _SCAN_MODE_FLAGS[_runs]
+_WARNED_WIDE_KEYS = False
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 
@@ -64,7 +65,7 @@ class ChunkLaunch:
     def __init__(self, q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first=False,
                  cu_seqlens=None, cu_seqlens_cpu=None, chunk_indices=None, chunk_size=64,
                  A_log=None, dt_bias=None, qk_l2norm=False, beta_sigmoid=False, neg_eigval=False):
-        dev = require_gpu(q, k, v, g, beta)
+        dev = require_gpu(q, k, v, beta) if g is None else require_gpu(q, k, v, g, beta)
         B, T, H, K = k.shape
         HV, V = v.shape[2], v.shape[3]
         N = B if cu_seqlens is None else len(cu_seqlens) - 1
@@ -197,6 +198,11 @@ def chunk_gated_delta_rule_fwd(
         # recurrence instead (same operator, same HIP library, state [K <= 256, V] in registers):
         # correct for every shape the reference accepts, without the chunk path's throughput.
         from fla_hip.ops.gated_delta_rule.fused_recurrent import fused_recurrent_gated_delta_rule_fwd
+        global _WARNED_WIDE_KEYS
+        if not _WARNED_WIDE_KEYS and q.shape[1] > 4 * _KERNEL_CHUNK:
+            _WARNED_WIDE_KEYS = True
+            warnings.warn(f'fla_hip: chunk_gated_delta_rule with K={K} > {_KERNEL_DIMS[-1]} runs the token recurrence '
+                          f'(one dependent step per token, no matrix cores); long prompts will be slow.', stacklevel=3)
         o, ht = fused_recurrent_gated_delta_rule_fwd(
             q, k, v, g=g, beta=beta, A_log=A_log, dt_bias=dt_bias, scale=scale, initial_state=initial_state,
             output_final_state=output_final_state, use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel,
@@ -211,7 +217,7 @@ def chunk_gated_delta_rule_fwd(
         B, T, HV = v.shape[:3]
         N = B if cu_seqlens is None else len(cu_seqlens) - 1
         v2 = _pad_last(v, nb * D).reshape(B, T, HV * nb, D)
-        g2, beta2 = g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2)
+        g2, beta2 = None if g is None else g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2)
         A2 = None if A_log is None else A_log.reshape(-1).repeat_interleave(nb)
         dt2 = None if dt_bias is None else dt_bias.reshape(-1).repeat_interleave(nb)
         h2 = None

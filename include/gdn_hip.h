@@ -116,6 +116,7 @@ size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64
  * chunk_fwd_o (fla/ops/common/chunk_o.py:544-586).
  *
  *   q, k [B,T,H,K], v, o [B,T,HV,V] qkv_dtype (bf16 or f16); g, beta [B,T,HV] gb_dtype
+ *   g == NULL: no decay, i.e. the delta rule without gates (chunk_delta_rule_fwd, fla/ops/delta_rule/chunk.py:25-70)
  *   A_log [HV] fp32 or NULL: with it, g holds raw gate inputs and the kernel forms
  *         g = -exp(A_log) * softplus(g + dt_bias) (dt_bias [HV] fp32 or NULL) - use_gate_in_kernel,
  *         gdn_gate_chunk_cumsum of fla/ops/gated_delta_rule/gate.py:63-106
