@@ -40,12 +40,22 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
     sp.sloc = p.ws.Seg;
     sp.mseg = p.ws.Seg + slots * 16384;
     sp.sin = p.ws.Seg + 2 * slots * 16384;
+    // Segments start warm where the decay allows it (see WARM_LOG2); the first pass and the merge then only serve
+    // the heads that need exact start states, and their workgroups for the other heads return at once.  Not with two
+    // runs per workgroup in pass 2: the two heads would want different starts.
+    const bool pass2_pairs = use_pair(pair_full_ok, p.NH * nseg);
+    if (!(p.flags & GDN_FLAG_SCAN_NO_WARM) && !pass2_pairs) {
+        sp.bound = p.ws.Bound;
+        // a warm-up of w chunks costs w more steps; the exact start costs about 1.2 steps per chunk of the segment
+        // (first pass) plus the merge
+        sp.warm_cap = std::min(WARM_CAP_MAX, sp.seg_chunks + sp.seg_chunks / 4 + 6);
+    }
     int rc;
     sp.kind = WIDE_PASS1;
     if ((rc = use_pair(true, 2 * p.NH * (nseg - 1)) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream))) return rc;
     if ((rc = launch_segment_merge(p, sp, stream))) return rc;
     sp.kind = WIDE_PASS2;
-    return use_pair(pair_full_ok, p.NH * nseg) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
+    return pass2_pairs ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
 }
 
 }  // namespace gdn

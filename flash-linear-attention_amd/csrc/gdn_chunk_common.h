@@ -67,6 +67,14 @@ constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240;
 constexpr int64_t REC_BYTES = 11264;
 constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10
 constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
+// Besides the records the prepare kernel leaves one number per (chunk, v-head): an upper bound, in log2 units, on how much
+// the chunk's transition S -> 2^G_last S - k~^T (Xb 2^G k) S can stretch any state:
+//   bound = sum_t [ log2 gamma_t + log2 max(1, |1 - beta_t |k_t|^2|) ]      (each token's factor gamma_t (I - beta_t k_t k_t^T))
+// A run of chunks whose bounds add up to at most WARM_LOG2 forgets what came before it to within 2^WARM_LOG2 of that
+// state's size - far below the rounding of the fp32 state itself - so a time segment may start from a ZERO state that
+// many chunks early instead of from the exact state that a first pass and a merge would have to compute.
+constexpr float WARM_LOG2 = -64.f;
+constexpr int WARM_CAP_MAX = 64;
 __host__ __device__ constexpr int p_slot(int tt, int sp) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp; }
 __host__ __device__ constexpr bool frag_half(int tt, int sp) { return (tt == 0 && sp == 0) || (tt == 2 && sp == 1); }
 __host__ __device__ constexpr int frag_off(int tt, int sp) {          // bytes from the start of Xb or P
@@ -93,6 +101,7 @@ __device__ __forceinline__ void store_frag(char* m, int tt, int sp, int lane, ty
 
 struct ChunkWs {
     float* Seg;          // 3 * seg_slots 128x128 fp32 matrices for the segment-parallel scan
+    float* Bound;        // [NC][HV] log2 bound on the norm of every chunk's transition
     char* Rec;           // [NC][HV] records
 };
 
@@ -118,13 +127,14 @@ inline int plan_segments(int64_t N, int64_t HV, int64_t NT, int64_t num_chunks, 
 }
 
 // Workspace: the segment matrices (S_loc, M, S_in per (sequence, head, segment); none without segments),
-// then the records.
+// the transition bounds, then the records.
 inline size_t ws_layout(int64_t NC, int64_t HV, int64_t seg_slots, char* base, ChunkWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
     void* Seg = take(3 * (size_t)seg_slots * 16384 * 4);
+    void* Bound = take((size_t)NC * HV * 4);
     void* Rec = take((size_t)NC * HV * REC_BYTES);
-    if (ws) { ws->Seg = (float*)Seg; ws->Rec = (char*)Rec; }
+    if (ws) { ws->Seg = (float*)Seg; ws->Bound = (float*)Bound; ws->Rec = (char*)Rec; }
     return off;
 }
 
@@ -197,7 +207,36 @@ struct SegmentPlan {
     float* sloc;
     float* mseg;
     float* sin;
+    const float* bound;     // non-NULL: segments may start early from a zero state where the bounds allow it
+    int warm_cap;           // ... at most this many chunks early (<= WARM_CAP_MAX)
 };
+
+// How many chunks before chunk it0 a run of (sequence, head) must start from a zero state so that at it0 it has
+// forgotten the difference to the true state: the shortest run of chunks ending at it0 - 1 whose bounds add up to
+// WARM_LOG2 or less.  When the start of the sequence comes first (within `cap` chunks) the answer is it0: the run
+// starts at chunk 0 from the true initial state and is exact.  -1: not within `cap` chunks.  `bound` points at the
+// entry of chunk 0 of the sequence for this head; entries of consecutive chunks are HV apart.  Lane l looks at
+// chunk it0 - 1 - l; the result is the same in every lane.
+__device__ __forceinline__ int warm_chunks(const float* bound, int HV, int64_t it0, int cap, int lane) {
+    const bool in = lane < cap && lane < it0;
+    float x = in ? bound[(it0 - 1 - lane) * HV] : 0.f;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float y = __shfl_up(x, off, 64);
+        if (lane >= off) x += y;
+    }
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(in && x <= WARM_LOG2);
+    if (hit) return __builtin_ctzll(hit) + 1;
+    return it0 <= cap ? (int)it0 : -1;
+}
+
+// Whether the segments of this (sequence, head) need the exact start states of the first pass and the merge:
+// true when some segment cannot be warm-started within the cap.
+__device__ __forceinline__ bool needs_exact_segments(const SegmentPlan& sp, const float* bound, int HV, int lane) {
+    bool exact = false;
+    for (int j = 1; j < sp.nseg; ++j) exact |= warm_chunks(bound, HV, (int64_t)j * sp.seg_chunks, sp.warm_cap, lane) < 0;
+    return exact;
+}
 
 // launchers defined next to their kernels
 template <typename T> int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream);

@@ -89,6 +89,8 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         seg = (int)(group % (sp.nseg - 1));
         n = nh / H; h = (int)(nh % H); hv = h * G + (int)(slot % G);
         const int64_t inh = n * HV + hv;
+        // (a head whose segments all start warm needs no exact start states)
+        if (sp.bound && !needs_exact_segments(sp, sp.bound + n * p.NT * HV + hv, HV, lane)) return;
         if (tm == 0) {
             if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
             else init = 2;

@@ -19,7 +19,7 @@ constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 
 constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
 // two tiles (k then L, q then X), the transposed diagonal blocks of L, the row factors of k and q, and gates + beta
 // of every value head of the group
-inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + 2 * CH * 4 + (size_t)group * 2 * CH * 4; }
+inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + 3 * CH * 4 + (size_t)group * 2 * CH * 4; }
 
 template <typename T>
 __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p) {
@@ -30,8 +30,8 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
     float* sL = (float*)k_nat;                  // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
     float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1
     float* sLd = (float*)(q_nat + CH * NP);     // [4][16 j][16 i] diagonal blocks of L, transposed (column j contiguous)
-    float* sRN = sLd + 4 * 256;                 // [2][64] 1/|k_t|, 1/|q_t| (ones unless the rows are to be normalised)
-    float* sGB = sRN + 2 * CH;                  // [group][2][64] cumulative gate (log2), beta
+    float* sRN = sLd + 4 * 256;                 // [3][64] 1/|k_t|, 1/|q_t| (ones unless the rows are to be normalised), |k_t|^2 as given
+    float* sGB = sRN + 3 * CH;                  // [group][2][64] cumulative gate (log2), beta
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // heads vary fastest over the workgroups: those that run at the same time then read whole token rows
@@ -85,8 +85,9 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             *(u32x4*)(k_nat + row * NP + col) = rk[ps];
             *(u32x4*)(q_nat + row * NP + col) = rq[ps];
             // l2 normalisation is applied as per-row factors: 16 lanes hold one row
+            // (|k_t|^2 is needed in any case: it enters the bound on the chunk's transition)
             float sk = 0.f, sq = 0.f;
-            if (l2) {
+            {
                 const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk += a * a; sq += b * b; }
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             if ((tid & 15) == 0) {
                 sRN[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
                 sRN[CH + row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
+                sRN[2 * CH + row] = sk;
             }
         }
     }
@@ -131,6 +133,13 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
         tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
         if (lane == 63) tab[TAB_GLAST] = x;
+        // bound on the chunk's transition: every token contributes gamma_t * max(1, |1 - beta_t |k~_t|^2|)
+        // (rows past the end have beta = 0 and g = 0)
+        float lb = fabsf(1.f - b * sRN[2 * CH + lane] * nk * nk);
+        lb = lb > 1.f ? __log2f(lb) : 0.f;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) lb += __shfl_xor(lb, off, 64);
+        if (lane == 63) p.ws.Bound[ci * HV + hv] = xl + lb;
     }
 
     // ---- raw products, kept in registers: K K^T tiles (row-tile w, column-tiles <= w) and the

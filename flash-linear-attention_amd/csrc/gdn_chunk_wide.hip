@@ -83,6 +83,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     int64_t inh;
     int seg;
     int init = 0;                 // 0: from `src` (NULL = zero state), 1: identity, 2: zero
+    int warm = 0;                 // chunks run before the segment proper, without output
     bool v_zero = false, src_user = false, dst_user = false;
     const float* src = nullptr;
     float* dst = nullptr;
@@ -102,6 +103,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const int64_t nh = group / (sp.nseg - 1);
         seg = (int)(group % (sp.nseg - 1));
         inh = (nh / H) * HV + (nh % H) * G + member % G;
+        // (a head whose segments all start warm needs no exact start states)
+        if (sp.bound && !needs_exact_segments(sp, sp.bound + (inh / HV) * p.NT * HV + inh % HV, HV, lane)) return;
         if (member < G) {
             if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
             else init = 2;
@@ -118,7 +121,19 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         seg = (int)(group % sp.nseg);
         inh = (nh / H) * HV + (nh % H) * G + slot % G;
         if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
-        else src = sp.sin + (inh * sp.nseg + seg) * 16384;
+        else {
+            // Warm start: begin `warm` chunks early from a zero state (from the true initial state when that reaches
+            // the start of the sequence) and produce no output until the segment proper.  Heads with a segment that
+            // cannot be started this way take the exact start states of the first pass and the merge.
+            const float* bnd = sp.bound ? sp.bound + (inh / HV) * p.NT * HV + inh % HV : nullptr;
+            if (bnd && !needs_exact_segments(sp, bnd, HV, lane)) {
+                warm = __builtin_amdgcn_readfirstlane(warm_chunks(bnd, HV, (int64_t)seg * sp.seg_chunks, sp.warm_cap, lane));
+                if ((int64_t)seg * sp.seg_chunks - warm == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
+                else init = 2;
+            } else {
+                src = sp.sin + (inh * sp.nseg + seg) * 16384;
+            }
+        }
         if (seg == sp.nseg - 1 && p.ht) { dst = p.ht + inh * (int64_t)(K * V); dst_user = true; }
     }
     const int64_t n = inh / HV;
@@ -136,8 +151,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         boh = n * p.NT;
     }
     const int64_t nt = (len + CH - 1) / CH;
-    const int64_t it0 = (int64_t)seg * sp.seg_chunks;
-    const int64_t it1 = min(nt, it0 + sp.seg_chunks);
+    const int64_t it0 = (int64_t)seg * sp.seg_chunks - warm;
+    const int64_t it1 = min(nt, (int64_t)seg * sp.seg_chunks + sp.seg_chunks);
     const int64_t nsteps = it1 - it0;                       // may be <= 0 for an empty sequence
     const int64_t lastc = it1 - 1;
     char* otile = smem + KBUF + 3 * 16384;                  // [64 token rows][OT_PITCH]
@@ -277,7 +292,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             };
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                if constexpr (FULL) { if (i > 0) store_rows(it0 + i - 1); }
+                if constexpr (FULL) { if (i > warm) store_rows(it0 + i - 1); }
                 lds_barrier();                                              // B1
                 if constexpr (FULL) {
 #pragma unroll
@@ -285,7 +300,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 }
                 lds_barrier();                                              // B2 (waits for the tile reads)
             }
-            if constexpr (FULL) store_rows(lastc);
+            if constexpr (FULL) { if (nsteps > warm) store_rows(lastc); }
         }
         wait_vm_at_most<0>();                               // no copy may land in LDS after this workgroup has gone
         return;
@@ -553,13 +568,14 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 constexpr int MP = 132;                            // pitch of the staged rows (floats): conflict-free 16-byte reads
 constexpr size_t MERGE_SMEM = (128 * MP + 16 * MP) * 4;
 
-__global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, int64_t NH) {
+__global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, int64_t NH, int HV, int64_t NT) {
     extern __shared__ __align__(16) char smem[];
     float* sM = (float*)smem;                      // [128 i][MP] M_j
     float* sSt = sM + 128 * MP;                    // [16 n][MP] current S_in slab, transposed
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     const int64_t inh = (int64_t)(blockIdx.x >> 6) * 8 + (blockIdx.x & 7);
     if (inh >= NH) return;
+    if (sp.bound && !needs_exact_segments(sp, sp.bound + (inh / HV) * NT * HV + inh % HV, HV, lane)) return;      // all segments start warm
     const int v0 = (int)((blockIdx.x >> 3) & 7) * 16;
     const int nseg = sp.nseg;
     f32x4 pre[16];
@@ -653,7 +669,7 @@ int launch_wide(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
 int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t stream) {
     static SmemAttrDone attr_done;
     if (int rc = ensure_dynamic_smem((const void*)gdn_segment_merge_kernel, MERGE_SMEM, attr_done, "hipFuncSetAttribute(merge)")) return rc;
-    hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)((p.NH + 7) / 8 * 64)), dim3(256), MERGE_SMEM, stream, sp, p.NH);
+    hipLaunchKernelGGL(gdn_segment_merge_kernel, dim3((unsigned)((p.NH + 7) / 8 * 64)), dim3(256), MERGE_SMEM, stream, sp, p.NH, p.HV, p.NT);
     return check_launch("gdn_segment_merge_kernel");
 }
 

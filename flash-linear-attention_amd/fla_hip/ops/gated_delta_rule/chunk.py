@@ -33,10 +33,13 @@ _KERNEL_CHUNK = 64
 # FLA_HIP_SCAN_MODE forces one form of the sequential kernel (default: automatic): whole sequences
 # ('wide') or time cut into segments, each with one run per workgroup ('-single') or two ('-pair')
 _SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS,
-                    'single': _lib.FLAG_SCAN_NO_PAIR, 'pair': _lib.FLAG_SCAN_PAIR}
+                    'single': _lib.FLAG_SCAN_NO_PAIR, 'pair': _lib.FLAG_SCAN_PAIR,
+                    'segments-exact': _lib.FLAG_SCAN_SEGMENTS | _lib.FLAG_SCAN_NO_WARM}
 for _form in ('wide', 'segments'):
     for _runs in ('single', 'pair'):
         _SCAN_MODE_FLAGS[f'{_form}-{_runs}'] = _SCAN_MODE_FLAGS[_form] | _SCAN_MODE_FLAGS[_runs]
+        if _form == 'segments':
+            _SCAN_MODE_FLAGS[f'segments-exact-{_runs}'] = _SCAN_MODE_FLAGS['segments-exact'] | _SCAN_MODE_FLAGS[_runs]
 _WARNED_WIDE_KEYS = False
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 

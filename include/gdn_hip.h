@@ -51,6 +51,7 @@ extern "C" {
 #define GDN_FLAG_SEQ_ORDER      (1u << 19) /* chunk_offsets carries N more entries (see there)   */
 #define GDN_FLAG_SCAN_NO_PAIR   (1u << 20) /* always one run per workgroup                      */
 #define GDN_FLAG_SCAN_PAIR      (1u << 21) /* two runs per workgroup wherever two can share k rows */
+#define GDN_FLAG_SCAN_NO_WARM   (1u << 22) /* time segments always start from exact states (first pass + merge) */
 
 /* activation codes of the convolution and normalisation entry points */
 #define GDN_ACT_NONE    0

@@ -162,7 +162,7 @@ def test_reference_gate_in_kernel_matrix_with_the_reference_input_recipe(B, T, H
     _check('ht', ref_ht, ht)
 
 
-@pytest.mark.parametrize('mode', ['auto', 'wide-single', 'wide-pair', 'segments-single', 'segments-pair'])
+@pytest.mark.parametrize('mode', ['auto', 'wide-single', 'wide-pair', 'segments-single', 'segments-exact-single', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,K,V,vfirst,cu', [
     (2, 1100, 2, 4, 64, 64, False, None),
     (1, 1300, 2, 2, 32, 96, True, None),
@@ -220,7 +220,7 @@ def test_reference_varlen_prefill_case_under_inference_mode():
     _check('ht', ref_ht, ht)
 
 
-@pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'wide-pair', 'segments-pair'])
+@pytest.mark.parametrize('mode', ['wide-single', 'segments-single', 'segments-exact-single', 'wide-pair', 'segments-pair'])
 @pytest.mark.parametrize('B,T,H,HV,with_h0,vfirst', [
     (2, 1000, 2, 4, True, False),
     (1, 2100, 2, 2, True, True),          # ragged tail, V-first state layout
@@ -241,6 +241,69 @@ def test_every_form_of_the_sequential_stage(monkeypatch, mode, B, T, H, HV, with
         o, ht = _run(q, k, v, g, beta, h0)
     _check('o', ref_o, o)
     _check('ht', ref_ht, ht)
+
+
+def _gates_per_head(B, T, HV, per_token, seed):
+    """log-decays of size `per_token[hv]` (times a random factor in [0.5, 1.5]) per value head"""
+    gen = torch.Generator().manual_seed(seed)
+    return -(0.5 + torch.rand(B, T, HV, generator=gen)) * torch.tensor(per_token)
+
+
+@pytest.mark.parametrize('case', ['fast', 'slow', 'mixed', 'expanding', 'boundary'])
+def test_segments_that_start_warm(monkeypatch, case):
+    """Time segments start from a zero state a few chunks early where the decay over those chunks makes
+    the true state irrelevant (bound 2^-64), and from the exact merged state otherwise - decided per head
+    on the device.  Heads that decay slowly, or whose keys are long enough to stretch the state
+    (beta |k|^2 > 2), must take the exact path and then equal it bit for bit."""
+    B, T, H, HV, D = 1, 8192, 4, 16, 128          # 16 segments of 8 chunks; up to 16 chunks of warm-up
+    q, k, v, _, beta, h0 = O.make_inputs(B, T, H, HV, D, D, seed=31, h0_std=0.5, dtype=torch.bfloat16)
+    per_token = {'fast': [0.05] * 16, 'slow': [1e-4] * 16, 'mixed': [0.05, 1e-4, 0.2, 0.01] * 4,
+                 'expanding': [0.05] * 16, 'boundary': [0.0875] * 16}[case]
+    g = _gates_per_head(B, T, HV, per_token, seed=32)
+    if case == 'expanding':
+        k = (k.float() * 1.6).bfloat16()          # beta |k|^2 up to 2.56: some tokens stretch the state
+        beta = torch.ones_like(beta)
+        g = g * 4                                   # (keeps the recurrence itself stable)
+    if case == 'boundary':
+        # constant decay chosen so that 8 chunks give 2^-64.6 and 7 do not: the warm-up length is exactly 8
+        g = torch.full_like(g, -0.0875)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    out = {}
+    for mode in ('segments-single', 'segments-exact-single'):
+        monkeypatch.setenv('FLA_HIP_SCAN_MODE', mode)
+        out[mode] = _run(q, k, v, g, beta, h0)
+        _check(f'o {mode}', ref_o, out[mode][0])
+        _check(f'ht {mode}', ref_ht, out[mode][1])
+    (o_w, h_w), (o_e, h_e) = out['segments-single'], out['segments-exact-single']
+    same = torch.equal(o_w, o_e) and torch.equal(h_w, h_e)
+    if case in ('slow', 'expanding'):
+        assert same, 'heads that cannot start warm must take the exact path unchanged'
+    else:
+        # a different (and equally good) start state: close; with a decay that varies it is not identical
+        # (with the constant decay of 'boundary' what a warm start drops is below the rounding of the fp32 state)
+        assert case == 'boundary' or not same
+        assert O.get_err_ratio(o_e.float().cpu(), o_w.float().cpu()) < 2e-3
+    if case == 'mixed':
+        # per head: value heads 1 and 3 decay too slowly (1e-4, 0.01 per token) and are bitwise those of the exact path
+        assert torch.equal(o_w[:, :, 1::2], o_e[:, :, 1::2]) and torch.equal(h_w[:, 1::2], h_e[:, 1::2])
+        # (heads 2, 6, ... decay so fast that a warm start reproduces the exact fp32 state: nothing to tell apart)
+        for hv in range(0, 16, 4):
+            assert not torch.equal(o_w[:, :, hv], o_e[:, :, hv]), hv
+
+
+def test_warm_start_forgets_an_enormous_state(monkeypatch):
+    """What a warm start drops is bounded by 2^-64 of the state BEFORE the warm-up chunks, whatever its size:
+    a huge initial state and huge early values must leave the later output as accurate as the exact path."""
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'segments-single')
+    B, T, H, HV, D = 1, 8192, 4, 16, 128
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, D, D, seed=33, gate_div=4.0, h0_std=1e6, dtype=torch.bfloat16)
+    v = v.float()
+    v[:, :512] *= 1e6
+    v = v.bfloat16()
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, dtype=torch.float64)
+    o, ht = _run(q, k, v, g, beta, h0)
+    _check('ht', ref_ht.float(), ht)
+    _check('o (late tokens)', ref_o[:, 4096:].float(), o[:, 4096:])
 
 
 @pytest.mark.parametrize('mode', ['wide-pair', 'segments-pair'])
@@ -445,7 +508,7 @@ def test_each_prologue_inside_the_kernels_packed_input(kw):
     _check('ht', ref_ht, ht)
 
 
-@pytest.mark.parametrize('mode,T', [('auto', 333), ('wide-single', 2100), ('wide-pair', 2100), ('segments-single', 4200), ('segments-pair', 4200)])
+@pytest.mark.parametrize('mode,T', [('auto', 333), ('wide-single', 2100), ('wide-pair', 2100), ('segments-single', 4200), ('segments-exact-single', 4200), ('segments-pair', 4200)])
 def test_outputs_fully_written_and_deterministic(monkeypatch, mode, T):
     """Two runs agree bit for bit and every output element is written (no NaN survives from
     poisoned allocations: the workspace and outputs come from torch.empty).  Every form of the

@@ -47,14 +47,18 @@ def _records(call, num_chunks, HV):
     (1, 256, 4, 4, 32, torch.float16, 1.0, False),
     (2, 200, 2, 4, 128, torch.bfloat16, 16.0, True),           # ragged last chunk, row factors of the l2 norm
     (1, 63, 1, 1, 16, torch.float16, 4.0, False),              # tests/ops/test_solve_tril.py:22
+    (1, 128, 1, 2, 32, torch.bfloat16, 2.0, 'long'),           # keys of length 1.7: beta |k|^2 > 2 stretches the state
 ])
 def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2):
     from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
     gen = torch.Generator().manual_seed(7)
     q = torch.randn(B, T, H, K, generator=gen)
     k = torch.randn(B, T, H, K, generator=gen)
+    long_keys, l2 = l2 == 'long', l2 is True
     if not l2:
         q, k = F.normalize(q, dim=-1), F.normalize(k, dim=-1)
+    if long_keys:
+        k = 1.7 * k
     q, k = q.to(dtype), k.to(dtype)
     v = torch.randn(B, T, HV, K, generator=gen).to(dtype)
     g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / gate_div
@@ -65,6 +69,10 @@ def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2)
     torch.cuda.synchronize()
     NT = (T + 63) // 64
     recs = _records(call, B * NT, HV)
+    # the transition bounds sit in front of the records (one float per chunk and value head, padded to 256 bytes)
+    ws = call.workspace.cpu()
+    nb = (B * NT * HV * 4 + 255) // 256 * 256
+    bounds = ws[ws.numel() - B * NT * HV * REC_BYTES - nb:][:B * NT * HV * 4].view(torch.float32).view(B * NT, HV).double()
     qn, kn = (O.l2norm(q.double()), O.l2norm(k.double())) if l2 else (q.double(), k.double())
     G = HV // H
     for b in range(B):
@@ -92,6 +100,15 @@ def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2)
                 assert torch.allclose(tab[128:128 + n], torch.exp2(gc) * rk, rtol=2e-5, atol=1e-30)          # 2^G (k rows)
                 assert torch.allclose(tab[64:64 + n], scale * torch.exp2(gc) * rq, rtol=2e-5, atol=1e-30)    # scale 2^G (q rows)
                 assert torch.allclose(tab[0:n], torch.exp2(gc[-1] - gc) * rk, rtol=2e-5, atol=1e-30)         # 2^(G_last - G)
+                # the bound: its closed form, and that it does bound the chunk's transition prod_t gamma_t (I - beta_t k_t k_t^T)
+                k2 = (kk * kk).sum(-1)
+                closed = gc[-1] + torch.log2(torch.clamp((1 - bt * k2).abs(), min=1.0)).sum()
+                got = bounds[b * NT + it, hv].item()
+                assert abs(got - closed.item()) < 1e-3 * max(1.0, abs(closed.item())), (got, closed.item())
+                M = torch.eye(K, dtype=torch.float64)
+                for t in range(n):
+                    M = math.exp(g[b, 64 * it + t, hv].item()) * (M - bt[t] * torch.outer(kk[t], kk[t] @ M))
+                assert math.log2(torch.linalg.matrix_norm(M, 2).item() + 1e-300) <= got + 1e-3
 
 
 @pytest.mark.parametrize('B,T,H,HV', [(2, 300, 2, 4), (1, 4200, 1, 2)])

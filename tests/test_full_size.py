@@ -70,7 +70,7 @@ def test_long_sequence_properties():
     # (3) every other form of the sequential stage agrees with the automatic choice: a single pass over
     # the sequence, and segments with one or two runs per workgroup throughout
     import os
-    for mode in ('wide-single', 'wide-pair', 'segments-single', 'segments-pair'):
+    for mode in ('wide-single', 'wide-pair', 'segments-single', 'segments-exact-single', 'segments-pair'):
         os.environ['FLA_HIP_SCAN_MODE'] = mode
         try:
             ow, hw = op(dq, dk, dv, dg, db, initial_state=ds, output_final_state=True)

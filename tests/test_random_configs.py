@@ -39,7 +39,7 @@ def _case(seed, recurrent):
     flags = dict(l2=rnd.random() < 0.5, gate=rnd.random() < 0.4, sig=rnd.random() < 0.4, neg=False,
                  vfirst=rnd.random() < 0.5, h0=rnd.random() < 0.7, scale=rnd.choice([None, 0.1, 1.0]))
     flags['neg'] = flags['sig'] and rnd.random() < 0.5
-    mode = rnd.choice(['auto', 'wide-single', 'wide-pair', 'segments-single', 'segments-pair'])
+    mode = rnd.choice(['auto', 'wide-single', 'wide-pair', 'segments-single', 'segments-pair', 'segments-exact-single'])
     return dict(dtype=dtype, H=H, HV=H * G, K=K, V=V, B=B, T=T, N=N, cu=cu, mode=mode, **flags)
 
 
