@@ -85,9 +85,8 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             *(u32x4*)(k_nat + row * NP + col) = rk[ps];
             *(u32x4*)(q_nat + row * NP + col) = rq[ps];
             // l2 normalisation is applied as per-row factors: 16 lanes hold one row
-            // (|k_t|^2 is needed in any case: it enters the bound on the chunk's transition)
             float sk = 0.f, sq = 0.f;
-            {
+            if (l2) {
                 const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk += a * a; sq += b * b; }
@@ -97,7 +96,6 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             if ((tid & 15) == 0) {
                 sRN[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
                 sRN[CH + row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
-                sRN[2 * CH + row] = sk;
             }
         }
     }
@@ -133,13 +131,6 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
         tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
         if (lane == 63) tab[TAB_GLAST] = x;
-        // bound on the chunk's transition: every token contributes gamma_t * max(1, |1 - beta_t |k~_t|^2|)
-        // (rows past the end have beta = 0 and g = 0)
-        float lb = fabsf(1.f - b * sRN[2 * CH + lane] * nk * nk);
-        lb = lb > 1.f ? __log2f(lb) : 0.f;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) lb += __shfl_xor(lb, off, 64);
-        if (lane == 63) p.ws.Bound[ci * HV + hv] = xl + lb;
     }
 
     // ---- raw products, kept in registers: K K^T tiles (row-tile w, column-tiles <= w) and the
@@ -167,7 +158,27 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             }
         }
     }
+    // |k_t|^2 is the diagonal of K K^T: lane (c16, g) of the diagonal tile holds rows 4g .. 4g+3 of column c16
+    {
+        float d = 0.f;
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (tj == w && r == (c16 & 3)) d = kk[tj][r];
+        if ((c16 >> 2) == g) sRN[2 * CH + 16 * w + c16] = d;
+    }
     __syncthreads();     // k and q are dead from here on: their bytes become L and X
+    // ---- bound on the chunk's transition, per value head: every token contributes gamma_t max(1, |1 - beta_t |k~_t|^2|)
+    // (rows past the end have beta = 0 and g = 0) ----
+    for (int m = w; m < G; m += 4) {
+        const float nk = sRN[lane];
+        float lb = fabsf(1.f - sGB[(2 * m + 1) * CH + lane] * sRN[2 * CH + lane] * nk * nk);
+        lb = lb > 1.f ? __log2f(lb) : 0.f;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) lb += __shfl_xor(lb, off, 64);
+        if (lane == 63) p.ws.Bound[ci * HV + h * G + m] = sGB[(2 * m) * CH + 63] + lb;
+    }
     // P of every value head first: the raw q K^T tiles then leave the registers before the inversion needs them
     for (int m = 0; m < G; ++m) {
         const int hv = h * G + m;
