@@ -8,12 +8,9 @@ namespace gdn {
 constexpr int STAGE_PREPARE = 1, STAGE_SCAN = 2;
 
 template <typename T>
-static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hipStream_t stream) {
-    if (stages & STAGE_PREPARE) {
-        int rc = launch_prepare<T>(p, num_chunks, stream);
-        if (rc) return rc;
-    }
-    if (!(stages & STAGE_SCAN)) return GDN_OK;
+static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, hipStream_t stream) {
+    ChunkParams p = p0;
+    // The plan of the sequential stage first: the prepare kernel writes P only for the kernel that reads it.
     // One workgroup per (sequence, head) walks the chunks of the sequence, or time is cut into
     // segments (plan_segments).  Either way a workgroup can also carry two runs that read the same k rows (two value heads of
     // a q/k head; in pass 1 the S and M runs of one head).  That halves the number of workgroups and
@@ -29,10 +26,18 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
     auto use_pair = [&](bool possible, int64_t single_workgroups) {
         return possible && !no_pair && (force_pair || single_workgroups > 256);
     };
+    const bool pass2_pairs = segments && use_pair(pair_full_ok, p.NH * nseg);
+    const bool whole_pairs = !segments && use_pair(pair_full_ok, p.NH);
+    p.want_P = pass2_pairs || whole_pairs;
+    if (stages & STAGE_PREPARE) {
+        int rc = launch_prepare<T>(p, num_chunks, stream);
+        if (rc) return rc;
+    }
+    if (!(stages & STAGE_SCAN)) return GDN_OK;
     SegmentPlan sp = {};
     if (!segments) {
         sp.kind = WIDE_WHOLE;
-        return use_pair(pair_full_ok, p.NH) ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
+        return whole_pairs ? launch_pair<T>(p, sp, stream) : launch_wide<T>(p, sp, stream);
     }
     sp.nseg = nseg;
     sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
@@ -43,7 +48,6 @@ static int launch_chunk(const ChunkParams& p, int64_t num_chunks, int stages, hi
     // Segments start warm where the decay allows it (see WARM_LOG2); the first pass and the merge then only serve
     // the heads that need exact start states, and their workgroups for the other heads return at once.  Not with two
     // runs per workgroup in pass 2: the two heads would want different starts.
-    const bool pass2_pairs = use_pair(pair_full_ok, p.NH * nseg);
     if (!(p.flags & GDN_FLAG_SCAN_NO_WARM) && !pass2_pairs) {
         sp.bound = p.ws.Bound;
         // a warm-up of w chunks costs w more steps; the exact start costs about 1.2 steps per chunk of the segment

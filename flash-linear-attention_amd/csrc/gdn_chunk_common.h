@@ -55,18 +55,22 @@ __device__ __forceinline__ V8 join(V4 a, V4 b) {
 // 2^x as a single v_exp_f32 (results below 2^-126 flush to zero, which is what a decay wants)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Workspace record written by the prepare kernel per (chunk, v-head): 11 KB that the scan
+// Workspace record written by the prepare kernel per (chunk, v-head): 12 KB in 1 KB pieces that the scan
 // copies verbatim into LDS.  Xb and P are stored as matrix-core operand fragments
 // ([lane][8]): rows of t-tile tt, columns t' in {32sp+4g+r} U {32sp+16+4g+r}.  Both are
 // lower triangular: the fragments (tt, sp) = (0,1), (1,1) are identically zero and are not
 // stored, and of (0,0), (2,1) only the first half (4 values per lane) is.
-//   Xb  T    5 KB         (I+L)^-1 diag(beta)
-//   P   T    5 KB         scale * tril(q k^T 2^(G_t-G_t'))
-//   tab fp32 [256]        [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units)
-constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240;
-constexpr int64_t REC_BYTES = 11264;
-constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10
+//   Xb   T    5 KB        (I+L)^-1 diag(beta)
+//   P    T    5 KB        scale * tril(q k^T 2^(G_t-G_t')); written only for the scan kernel that reads it (two runs per
+//                         workgroup); the one-run kernel forms P itself from its q and k tiles and the second table
+//   tab  fp32 [256]       [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units),
+//                         the first three times the row factors 1/|k_t|, 1/|q_t|, 1/|k_t| of the l2 normalisation
+//   tab2 fp32 [256]       [0..63] G_t (log2 units), [64..127] scale/|q_t|, [128..191] 1/|k_t|: what P needs
+constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240, REC_TAB2 = 11264;
+constexpr int64_t REC_BYTES = 12288;
+constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10, REC_PIECE_TAB2 = 11;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10, tab2 = 11
 constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
+constexpr int TAB2_G = 0, TAB2_NQS = 64, TAB2_NK = 128;
 // Besides the records the prepare kernel leaves one number per (chunk, v-head): an upper bound, in log2 units, on how much
 // the chunk's transition S -> 2^G_last S - k~^T (Xb 2^G k) S can stretch any state:
 //   bound = sum_t [ log2 gamma_t + log2 max(1, |1 - beta_t |k_t|^2|) ]      (each token's factor gamma_t (I - beta_t k_t k_t^T))
@@ -148,6 +152,7 @@ struct ChunkParams {
     int K, V;                                          // head dims of the caller's tensors (multiples of 8, <= 128)
     float scale; int gb_dtype; uint32_t flags;
     int64_t NH;
+    int want_P;                                        // the scan will read P from the records (two runs per workgroup)
 };
 
 // Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains
@@ -182,6 +187,8 @@ __device__ __forceinline__ void gather_1k_to_lds_masked(const char* gbase, uint3
     const uint64_t g = (uint64_t)gbase;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
     const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    const uint32_t mlo = __builtin_amdgcn_readfirstlane((uint32_t)mask), mhi = __builtin_amdgcn_readfirstlane((uint32_t)(mask >> 32));
+    mask = ((uint64_t)mhi << 32) | mlo;                         // wave-uniform by construction; make it scalar registers
     uint64_t saved;
     asm volatile("s_mov_b32 m0, %1\n\t"
                  "s_and_saveexec_b64 %0, %4\n\t"

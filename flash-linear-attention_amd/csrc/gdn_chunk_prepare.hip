@@ -55,6 +55,9 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
 
+    // q is needed for its row norms (l2 normalisation) and for P, when the scan wants P from the records
+    const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
+    const bool want_P = p.want_P != 0, need_q = l2 || want_P;
     // ---- all global loads first: the gate inputs of value head w of the group, then the k, q rows
     // (rows past the end of the sequence are zero) ----
     float rg = 0.f, rb = 0.f;
@@ -75,15 +78,14 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
             rk[ps] = rq[ps] = z;
             if (row < valid && col < K) {
                 rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * K + col);
-                rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
+                if (need_q) rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
             }
         }
-        const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
 #pragma unroll
         for (int ps = 0; ps < 4; ++ps) {
             const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
             *(u32x4*)(k_nat + row * NP + col) = rk[ps];
-            *(u32x4*)(q_nat + row * NP + col) = rq[ps];
+            if (want_P) *(u32x4*)(q_nat + row * NP + col) = rq[ps];
             // l2 normalisation is applied as per-row factors: 16 lanes hold one row
             float sk = 0.f, sq = 0.f;
             if (l2) {
@@ -131,6 +133,10 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
         tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
         if (lane == 63) tab[TAB_GLAST] = x;
+        float* tab2 = (float*)(p.ws.Rec + (ci * HV + hv) * REC_BYTES + REC_TAB2);
+        tab2[TAB2_G + lane] = x;
+        tab2[TAB2_NQS + lane] = p.scale * nq;
+        tab2[TAB2_NK + lane] = nk;
     }
 
     // ---- raw products, kept in registers: K K^T tiles (row-tile w, column-tiles <= w) and the
@@ -142,18 +148,18 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             ka[s] = *(const V8*)(k_nat + (16 * w + c16) * NP + 32 * s + 8 * g);
-            qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
+            if (want_P) qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
         }
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             kk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
             qk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (tj <= w || tj <= tt) {
+            if (tj <= w || (want_P && tj <= tt)) {
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     const V8 kb = *(const V8*)(k_nat + (16 * tj + c16) * NP + 32 * s + 8 * g);
                     if (tj <= w) kk[tj] = Mma<T>::run(ka[s], kb, kk[tj]);          // rows: tokens of tile w, column: token 16tj + c16
-                    if (tj <= tt) qk[tj] = Mma<T>::run(kb, qb[s], qk[tj]);         // rows: key tokens of tile tj, column: query token 16tt + c16
+                    if (want_P && tj <= tt) qk[tj] = Mma<T>::run(kb, qb[s], qk[tj]);         // rows: key tokens of tile tj, column: query token 16tt + c16
                 }
             }
         }
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         if (lane == 63) p.ws.Bound[ci * HV + h * G + m] = sGB[(2 * m) * CH + 63] + lb;
     }
     // P of every value head first: the raw q K^T tiles then leave the registers before the inversion needs them
-    for (int m = 0; m < G; ++m) {
+    for (int m = 0; want_P && m < G; ++m) {
         const int hv = h * G + m;
         const float* sG = sGB + (2 * m) * CH;
         char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;

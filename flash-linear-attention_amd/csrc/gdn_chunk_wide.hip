@@ -44,12 +44,13 @@ namespace gdn {
 // q, v and the record are double-buffered (stage = chunk % 2); k, the one operand that is read until the
 // very end of a step, has three buffers (chunk % 3) so that its copy can be issued two steps ahead.
 constexpr int STG_Q = 0, STG_V = 16384, STG_REC = 32768;
-constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB;
-constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 44 032
+constexpr int STG_X = STG_REC + REC_X, STG_P = STG_REC + REC_P, STG_TAB = STG_REC + REC_TAB, STG_TAB2 = STG_REC + REC_TAB2;
+constexpr int STG_BYTES = STG_REC + (int)REC_BYTES;          // 45 056
 constexpr int KBUF = 2 * STG_BYTES;                          // three k tiles of 16 KB follow the two stages
 constexpr int OT_PITCH = 272;                     // bytes per token row of the output tile (256 B + pad: conflict-free 8-byte writes)
 constexpr int OT_BYTES = 64 * OT_PITCH;           // 17 408 B
-constexpr size_t WIDE_SMEM = KBUF + 3 * 16384 + OT_BYTES;    // 154 624 B of the CU's 163 840: one workgroup per CU
+constexpr int PCOUNT_OFF = KBUF + 3 * 16384 + OT_BYTES;       // one counter: P fragments published so far
+constexpr size_t WIDE_SMEM = PCOUNT_OFF + 16;                // 156 688 B of the CU's 163 840: one workgroup per CU
 constexpr int WIDE_NN = 2;                        // 16-column tiles per compute wave
 #ifndef WIDE_RING
 #define WIDE_RING 3                               // operand fragments in flight per compute wave
@@ -156,6 +157,11 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     const int64_t nsteps = it1 - it0;                       // may be <= 0 for an empty sequence
     const int64_t lastc = it1 - 1;
     char* otile = smem + KBUF + 3 * 16384;                  // [64 token rows][OT_PITCH]
+    // The copy waves form P of a chunk while the compute waves are busy with the first products of its step and
+    // announce it by adding to this counter (4 per step); a compute wave looks at the counter before it fetches P.
+    // No barrier: one in the middle of a step costs the compute waves the slack between them.
+    volatile int* pcount = (volatile int*)(smem + PCOUNT_OFF);
+    if (tid == 0) *pcount = 0;                              // (published by the barrier B0)
 
     // =====================================================================================
     // Copy waves.  Step i (chunk it = it0 + i, stage cur = i & 1) has two phases, separated by
@@ -178,6 +184,61 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (w >= CW) {
         if (nsteps <= 0) return;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+        // ---- P = scale tril(q k^T 2^(G_t - G_t')) of a chunk, formed here from the q and k tiles of its stage while
+        // the compute waves multiply by the state: the four copy waves share the 10 non-zero 16 x 16 tiles (tile
+        // (tt, tj): query tokens of t-tile tt, key tokens of tile tj <= tt), as the transposed product so that a result
+        // is spread over the lanes exactly like the operand fragment the compute waves read.  A counter in LDS announces it
+        // (announce_P). ----
+        auto produce_P = [&](const char* st, const char* kbuf) {
+            if constexpr (FULL) {
+                __builtin_amdgcn_s_setprio(3);
+                const int pw = w - CW;
+                const V8* sK = (const V8*)kbuf;
+                const V8* sQ = (const V8*)(st + STG_Q);
+                const float* t2 = (const float*)(st + STG_TAB2);
+                const int a_off = (c16 >> 2) * 64 + 4 * (c16 & 3) + ((g + (c16 >> 2)) & 3);
+                auto frag = [&](int tt, int sp) {
+                    V8 qb[4];
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) qb[s4] = sQ[tt * 256 + 16 * s4 + a_off];
+                    const int t = 16 * tt + c16;
+                    const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                    V8 out;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const int tj = 2 * sp + half;
+                        if (tj > tt) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) out[half * 4 + r] = from_f32<T>(0.f);
+                            continue;
+                        }
+                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int s4 = 0; s4 < 4; ++s4) acc = Mma<T>::run(sK[tj * 256 + 16 * s4 + a_off], qb[s4], acc);
+                        const f32x4 gj = *(const f32x4*)(t2 + TAB2_G + 16 * tj + 4 * g), nj = *(const f32x4*)(t2 + TAB2_NK + 16 * tj + 4 * g);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int j = 16 * tj + 4 * g + r;
+                            // select, never multiply by a mask: 2^(G_t - G_j) may overflow above the diagonal
+                            out[half * 4 + r] = from_f32<T>((t >= j) ? st_ * nj[r] * acc[r] * fast_exp2(gt - gj[r]) : 0.f);
+                        }
+                    }
+                    store_frag<T>((char*)st + STG_P, tt, sp, lane, out);
+                };
+                if (pw == 0) frag(3, 0);
+                else if (pw == 1) frag(3, 1);
+                else if (pw == 2) { frag(2, 0); frag(0, 0); }
+                else { frag(1, 0); frag(2, 1); }
+            }
+        };
+        // ... and announces it: this wave's fragments of step i are in LDS (its LDS operations complete in order)
+        auto announce_P = [&]() {
+            if constexpr (FULL) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (lane == 0) __hip_atomic_fetch_add((int*)pcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __builtin_amdgcn_s_setprio(0);
+            }
+        };
         // Block gather: rows 4j .. 4j+3 of a [token][head][128] tensor.  Rows past the end of the
         // sequence re-read its last row: whatever they hold is finite and is multiplied by the zero
         // columns of Xb, the zero rows of v_new and the causal zeros of P.
@@ -197,24 +258,37 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             piece_off[jj] = 16 * (is_v ? c % pieces : c);
             piece_mask[jj] = __builtin_amdgcn_ballot_w64(is_v || c < pieces);
         }
-        auto gather_blocks = [&](const T* tensor, int64_t it, int j0, int j1, uint32_t lds_tile) {
+        // `skip`: the copy is issued with no lane enabled (nothing moves, the count of operations in flight is the same):
+        // for what only the output needs (q, P) in the chunks of a warm-up, whose output nobody wants.
+        auto gather_blocks = [&](const T* tensor, int64_t it, int j0, int j1, uint32_t lds_tile, bool skip = false) {
             const int64_t tok0 = bos + it * CH;
             const int valid = (int)min((int64_t)CH, len - it * CH);
             const char* base = (const char*)(tensor + (tok0 * heads + head) * dim);
+            const uint32_t keep32 = __builtin_amdgcn_readfirstlane(skip ? 0u : ~0u);      // (scalar registers, never a literal)
+            const uint64_t keep = ((uint64_t)keep32 << 32) | keep32;
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 if (j < j0 || j >= j1) continue;
                 const int row = min(4 * j + (c16 >> 2), valid - 1);
                 const uint32_t voff = (uint32_t)row * row_bytes + piece_off[j & 3];
-                if constexpr (DIMS128) gather_1k_to_lds(base, voff, lds_tile + j * 1024);
-                else gather_1k_to_lds_masked(base, voff, lds_tile + j * 1024, piece_mask[j & 3]);
+                if constexpr (DIMS128) {
+                    if (FULL && warm > 0) gather_1k_to_lds_masked(base, voff, lds_tile + j * 1024, keep);
+                    else gather_1k_to_lds(base, voff, lds_tile + j * 1024);
+                } else {
+                    gather_1k_to_lds_masked(base, voff, lds_tile + j * 1024, piece_mask[j & 3] & keep);
+                }
             }
         };
-        auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage) {
+        auto copy_rec = [&](int64_t it, int from, int to, uint32_t lds_stage, bool skip = false) {
             const char* rec = p.ws.Rec + ((boh + it) * HV + hv) * REC_BYTES;
+            const uint32_t keep32 = __builtin_amdgcn_readfirstlane(skip ? 0u : ~0u);
+            const uint64_t keep = ((uint64_t)keep32 << 32) | keep32;
 #pragma unroll
             for (int j = 0; j < (int)(REC_BYTES / 1024); ++j)
-                if (j >= from && j < to) gather_1k_to_lds(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024);
+                if (j >= from && j < to) {
+                    if (FULL && warm > 0) gather_1k_to_lds_masked(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024, keep);
+                    else gather_1k_to_lds(rec + j * 1024, lane * 16, lds_stage + STG_REC + j * 1024);
+                }
         };
         if (w == CW) {
             // ---- k: the copy of chunk i+2 is issued at the start of step i (its buffer was last read
@@ -227,23 +301,26 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             wait_vm_at_most<16>();
             lds_barrier();                                                  // B0: chunk 0 is complete
             for (int64_t i = 0; i < nsteps; ++i) {
+                if (i >= warm) produce_P(smem + (i & 1) * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384);
+                announce_P();
                 issue_k(i + 2);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<16>();                                      // all but the newest copy: chunk i+1 has landed
                 lds_barrier();                                              // B2
             }
         } else if (w <= CW + 2) {
-            // ---- q + Xb + tables (wave CW+1) and v + P (wave CW+2): NOPS pieces per chunk.  Pieces
+            // ---- q + Xb + tables (wave CW+1) and v (wave CW+2).  Pieces
             // [0, XB) of chunk c are issued in phase B of step c-2, the rest in phase A of step c-1.
             const bool qside = (w == CW + 1);
             constexpr int XB = 8;
             auto issue = [&](int64_t it, int stage, bool early) {
                 const uint32_t st = lds0 + stage * STG_BYTES;
+                const bool warming = it - it0 < warm;               // a chunk of the warm-up: no output, so neither q nor P
                 if (qside) {
                     if constexpr (FULL) {
-                        // 16 q pieces, then Xb (5) and the tables (1)
-                        if (early) gather_blocks((const T*)p.q, it, 0, 8, st + STG_Q);
-                        else { gather_blocks((const T*)p.q, it, 8, 16, st + STG_Q); copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }
+                        // 16 q pieces, then Xb (5) and the tables (2)
+                        if (early) gather_blocks((const T*)p.q, it, 0, 8, st + STG_Q, warming);
+                        else { gather_blocks((const T*)p.q, it, 8, 16, st + STG_Q, warming); copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); copy_rec(it, REC_PIECE_TAB2, REC_PIECE_TAB2 + 1, st, warming); }
                     } else {
                         if (early) { copy_rec(it, 0, REC_PIECES_X, st); copy_rec(it, REC_PIECE_TAB, REC_PIECE_TAB + 1, st); }      // all 6 pieces
                     }
@@ -251,7 +328,6 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                     if (early) { if (!v_zero) gather_blocks((const T*)p.v, it, 0, 8, st + STG_V); }      // (v is not read when it counts as zero)
                     else {
                         if (!v_zero) gather_blocks((const T*)p.v, it, 8, 16, st + STG_V);
-                        if constexpr (FULL) copy_rec(it, REC_PIECES_X, REC_PIECES_X + REC_PIECES_P, st);
                     }
                 }
             };
@@ -268,6 +344,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             for (int64_t i = 0; i < nsteps; ++i) {
                 const int64_t it = it0 + i;
                 const int cur = (int)(i & 1);
+                if (i >= warm) produce_P(smem + cur * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384);
+                announce_P();
                 issue(min(it + 1, lastc), cur ^ 1, false);
                 lds_barrier();                                              // B1
                 issue(min(it + 2, lastc), cur, true);
@@ -292,6 +370,8 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             };
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
+                if (i >= warm) produce_P(smem + (i & 1) * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384);
+                announce_P();
                 if constexpr (FULL) { if (i > warm) store_rows(it0 + i - 1); }
                 lds_barrier();                                              // B1
                 if constexpr (FULL) {
@@ -361,7 +441,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // window of three operand fragments), and the thin, dependent part of a step (D -> v_new ->
     // output of a pair of t-tiles) is cut into pieces that each share a region with four
     // independent matrix instructions (products of the next tiles, or the state update).
-    auto step = [&](const char* st, const char* kbuf) {
+    auto step = [&](const char* st, const char* kbuf, int p_target) {
         const V8* sK = (const V8*)kbuf;
         const V8* sQ = (const V8*)(st + STG_Q);
         const T* sV = (const T*)(st + STG_V);
@@ -498,8 +578,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             if (f == 6) FX(0);
             if (f == 7) FX(1);
             if (f == 8) TD(0);
-            if (f == 9) { TD(1); FP(0); }
-            if (f == 10) { TXa(0); TXa(1); FP(1); }
+            if (f == 9) { TD(1); }
+            if (f == 10) { TXa(0); TXa(1); }
+            if (f == 11) {
+                // P of this chunk: normally long there (the copy waves form it first thing in a step, at raised priority)
+                if constexpr (FULL) { while (*pcount < p_target) __builtin_amdgcn_s_sleep(1); }
+                FP(0); FP(1);
+            }
             if (f == 11) { TXb(0); TXb(1); FV(2); }
             if (f == 12) { TPa(0); TPa(1); FV(3); }
             if (f == 13) { TPb(0); TPb(1); FX(2); }
@@ -534,7 +619,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     if (nsteps > 0) {
         lds_barrier();                                          // B0: the copy waves have filled stage 0
         for (int64_t i = 0; i < nsteps; ++i) {
-            step(smem + (i & 1) * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384);
+            step(smem + (i & 1) * STG_BYTES, smem + KBUF + (int)(i % 3) * 16384, 4 * ((int)i + 1));
         }
     }
 

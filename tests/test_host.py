@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
     assert ws(1, 512, 8, 2, 4, 64, 96) > 0          # multiples of 8 up to 128 are taken as they are
     assert ws(1, 512, 8, 2, 4, 100, 128) == 0
     # the segment matrices are reserved only when the plan cuts time into segments: long dense input with few heads
-    rec = 11264 + 4                                 # a record and a transition bound per (chunk, value head)
+    rec = 12288 + 4                                 # a record and a transition bound per (chunk, value head)
     assert ws(1, 32768, 512, 16, 32, 128, 128) == 512 * 32 * rec + 3 * 8 * 32 * 65536
     assert ws(1, 32768, 512, 16, 32, 128, 128, 0, _lib.FLAG_SCAN_WIDE) == 512 * 32 * rec
     assert ws(32, 65536, 1040, 16, 32, 128, 128, 1) == 1040 * 32 * rec                 # packed input never does
