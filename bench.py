@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|layer_steps|calib_copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -15,7 +15,8 @@ convolution, gated norm), and:
 Before the W warm-up steps of a workload the GPU is kept busy with the same step for 80 ms (untimed), so that the timed
 steps run at the clocks of sustained load and not at those of the first milliseconds after an idle period.
 --workload layer_steps runs only the convolution and the gated norm; --workload calib_copy runs a plain 1 GiB device copy: the kernel of known size against which the
-FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled.
+FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled; --workload calib_rmw an in-place read-modify-write of the decode states' 2 x 512 MiB
+with torch's elementwise kernel: the stream the decode step is compared with.
 """
 from __future__ import annotations
 
@@ -333,12 +334,35 @@ def calib_copy(steps, warmup, device):
                           steps=steps, warmup=warmup)))
 
 
+def calib_rmw(steps, warmup, device):
+    """The decode step's traffic without its arithmetic: every fp32 element of two alternating 512 MiB pools (the size
+    of the B = 256 decode states) read, changed and written back in place by torch's elementwise kernel.  What this
+    reaches is what a read-modify-write stream of that size reaches on the machine."""
+    n = 256 * 32 * 128 * 128
+    pools = [torch.zeros(n, dtype=torch.float32, device=device) for _ in range(2)]
+    spin_up(lambda i: pools[i & 1].add_(1.0))
+    for i in range(warmup):
+        pools[i & 1].add_(1.0)
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        pools[i & 1].add_(1.0)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e-3 for i in range(steps))
+    t = statistics.mean(ts)
+    print(json.dumps(dict(metric='calib_rmw_GBps', value=round(2 * n * 4 / t / 1e9, 1), unit='GB/s', us_per_pass=round(t * 1e6, 1),
+                          us_median=round(ts[len(ts) // 2] * 1e6, 1), bytes_read=n * 4, bytes_written=n * 4, steps=steps, warmup=warmup,
+                          frac_of_peak=round(2 * n * 4 / t / 1e9 / PEAK_HBM_GBS, 4))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['layer_steps', 'calib_copy'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     args = ap.parse_args()
@@ -353,6 +377,9 @@ def main():
 
     if args.workload == 'calib_copy':
         calib_copy(args.steps, args.warmup, device)
+        return
+    if args.workload == 'calib_rmw':
+        calib_rmw(args.steps, args.warmup, device)
         return
     if args.workload == 'layer_steps':
         print(json.dumps(dict(metric='gdn_layer_steps', steps=args.steps, warmup=args.warmup, dtype='bf16', data='synthetic',

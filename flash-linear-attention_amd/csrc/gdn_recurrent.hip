@@ -21,7 +21,22 @@ struct RecurrentParams {
     int64_t slots_stride;
     int64_t T; int H, HV, K, V, NVB;
     float scale; int gb_dtype; uint32_t flags;
+    int xcd_group; int64_t nblocks;      // see xcd_block()
 };
+
+// Workgroups are dealt to the chip's 8 XCDs round-robin by block index.  With xcd_group = g > 0 the work items (state
+// blocks, consecutive in memory) are handed out so that every XCD works on runs of g consecutive items instead of
+// every eighth one: an XCD then touches an eighth of the pages the launch touches, not all of them.  The grid is
+// rounded up to whole rounds of 8 groups; -1 = nothing to do for this workgroup.
+__device__ __forceinline__ int64_t xcd_block(const RecurrentParams& p) {
+    int64_t blk = blockIdx.x;
+    if (p.xcd_group > 0) {
+        const int64_t s = blk >> 3;
+        blk = ((s / p.xcd_group) * 8 + (blk & 7)) * p.xcd_group + s % p.xcd_group;
+        if (blk >= p.nblocks) return -1;
+    }
+    return blk;
+}
 
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
@@ -43,8 +58,10 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
     const int tid = threadIdx.x;
     const int c = tid % TC, r0 = tid / TC;
     const int wave = tid >> 6;
-    const int ivb = blockIdx.x % p.NVB;
-    const int64_t inh = blockIdx.x / p.NVB;
+    const int64_t blk = xcd_block(p);
+    if (blk < 0) return;
+    const int ivb = (int)(blk % p.NVB);
+    const int64_t inh = blk / p.NVB;
     const int64_t in = inh / p.HV;
     const int ihv = (int)(inh % p.HV);
     const int ih = ihv / (p.HV / p.H);
@@ -254,22 +271,161 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
     if (p.ht && !slot_per_token && !state_per_token) store_state(p.ht + state_off);
 }
 
+
+// The common decode shape on its own: K = V = 128, K-first states [K][V], one gate and one beta per head, states
+// per sequence or per slot.  Same arithmetic as gdn_recurrent_kernel with the decay e^g applied after the reductions,
+//   S' = e^g S + k d^T,   d = beta (v - e^g S^T k),   o = scale (e^g S^T q + (q.k) d),
+// k and q of a token read from LDS where they are used instead of being held per row.  The token's own rows (q, k,
+// v, gate, beta) are requested BEFORE the state: loads return in issue order, so their norms and the LDS staging are
+// done while the 64 KB of state are still on their way, and what follows the state's arrival is only the two
+// reductions and the update.  Thread (c = tid % 32, r0 = tid / 32) owns value columns 4c .. 4c+3 of key rows r0 + 8i.
+// Launched with enough unused LDS that two workgroups share a CU: more resident workgroups widen the window of
+// memory the chip works on at one time, and the read-modify-write stream gets slower (measured: 1, 2, 3+ workgroups
+// per CU = 208, 183, 191 us for 1 GiB of state traffic).
+constexpr size_t DECODE_LDS_PAD = 64 * 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = tid & 31, r0 = tid >> 5;
+    const int64_t inh = xcd_block(p);
+    if (inh < 0) return;
+    const int64_t in = inh / p.HV;
+    const int ihv = (int)(inh % p.HV);
+    const int H = p.H, HV = p.HV;
+    const int ih = ihv / (HV / H);
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    int64_t bos, len;
+    if (p.cu_seqlens) {
+        bos = load_index(p.cu_seqlens, in, cu32);
+        len = load_index(p.cu_seqlens, in + 1, cu32) - bos;
+    } else {
+        bos = in * p.T;
+        len = p.T;
+    }
+    const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
+    const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 4 * c;
+    const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
+    // what a token brings, as it comes from memory
+    struct Token { T q, k; T v[4]; float g, b; };
+    auto fetch = [&](int64_t tok) {
+        Token x;
+        x.q = x.k = from_f32<T>(0.f);
+        if (tid < 128) { x.q = q[(tok * H + ih) * 128 + tid]; x.k = k[(tok * H + ih) * 128 + tid]; }
+        const T* pv = v + (tok * HV + ihv) * 128 + 4 * c;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x.v[j] = pv[j];
+        x.g = p.g ? load_scalar(p.g, tok * HV + ihv, p.gb_dtype) : 0.f;
+        x.b = p.beta ? load_scalar(p.beta, tok * HV + ihv, p.gb_dtype) : 1.f;
+        return x;
+    };
+    Token cur = {};
+    if (len > 0) cur = fetch(bos);
+    float a_neg = 0.f, dtb = 0.f;
+    if (p.A_log) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+    // ---- the state: 16 requests of 16 bytes per thread, a wave instruction covers two whole rows ----
+    f32x4 S[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (p.h0) S[i] = __builtin_nontemporal_load((const f32x4*)(p.h0 + state_off + (r0 + 8 * i) * 128));
+    }
+    __shared__ float sh_q[2][128], sh_k[2][128];
+    __shared__ float sh_red[2][4][4];
+    __shared__ f32x4 sh_part[2][4][2][32];
+    const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+
+    for (int64_t t = 0; t < len; ++t) {
+        const int pb = (int)(t & 1);
+        const int64_t tok = bos + t;
+        const float qv = to_f32(cur.q), kv = to_f32(cur.k);
+        if (tid < 128) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
+        float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
+        if (lane == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
+        float eg = 1.f;
+        if (p.g) {
+            float gt = cur.g;
+            if (p.A_log) gt = a_neg * softplus_f(gt + dtb);
+            eg = __expf(gt);
+        }
+        float bb = cur.b;
+        if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
+        const f32x4 vv = {to_f32(cur.v[0]), to_f32(cur.v[1]), to_f32(cur.v[2]), to_f32(cur.v[3])};
+        if (t + 1 < len) cur = fetch(tok + 1);          // the next token's rows travel during this one's arithmetic
+        __syncthreads();
+        sqq = sh_red[pb][0][0] + sh_red[pb][1][0];      // (q and k live in waves 0 and 1)
+        skk = sh_red[pb][0][1] + sh_red[pb][1][1];
+        sqk = sh_red[pb][0][2] + sh_red[pb][1][2];
+        float rq = p.scale, rk = 1.f;
+        if (p.flags & GDN_FLAG_QK_L2NORM) {
+            rq *= 1.f / sqrtf(sqq + 1e-6f);
+            rk = 1.f / sqrtf(skk + 1e-6f);
+        }
+        const float qk = sqk * rq * rk;
+        // S^T k and S^T q over this thread's rows (k, q unscaled: the row factors come after the reduction)
+        f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sq = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            sk += S[i] * sh_k[pb][r0 + 8 * i];
+            sq += S[i] * sh_q[pb][r0 + 8 * i];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { sk[j] += __shfl_xor(sk[j], 32, 64); sq[j] += __shfl_xor(sq[j], 32, 64); }
+        if (lane < 32) { sh_part[pb][wave][0][c] = sk; sh_part[pb][wave][1][c] = sq; }
+        __syncthreads();
+        sk = (sh_part[pb][0][0][c] + sh_part[pb][1][0][c] + sh_part[pb][2][0][c] + sh_part[pb][3][0][c]) * (eg * rk);
+        sq = (sh_part[pb][0][1][c] + sh_part[pb][1][1][c] + sh_part[pb][2][1][c] + sh_part[pb][3][1][c]) * (eg * rq);
+        const f32x4 d = bb * (vv - sk);
+        const f32x4 dk = d * rk;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = S[i] * eg + dk * sh_k[pb][r0 + 8 * i];
+        if (r0 == 0) {
+            const f32x4 ov = sq + d * qk;
+            T* po = o + (tok * HV + ihv) * 128 + 4 * c;
+            po[0] = from_f32<T>(ov.x); po[1] = from_f32<T>(ov.y); po[2] = from_f32<T>(ov.z); po[3] = from_f32<T>(ov.w);
+        }
+    }
+    if (p.ht) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) __builtin_nontemporal_store(S[i], (f32x4*)(p.ht + state_off + (r0 + 8 * i) * 128));
+    }
+}
+
+// Grid for xcd_block(): launches that cover the chip several times over hand every XCD runs of `group` consecutive
+// work items (the states of one sequence); smaller ones keep the plain order.
+static int64_t place(RecurrentParams& p, int64_t nblocks, int64_t group) {
+    p.nblocks = nblocks;
+    p.xcd_group = 0;
+    if (nblocks < 2048 || group >= (1 << 20)) return nblocks;
+    p.xcd_group = (int)group;
+    const int64_t ngroups = (nblocks + group - 1) / group;
+    return (ngroups + 7) / 8 * 8 * group;
+}
+
 template <typename T, int KMAX, bool VFIRST>
 static int launch_vb(const RecurrentParams& p0, int64_t n_states, int vb, hipStream_t stream) {
     RecurrentParams p = p0;
     p.NVB = (p.V + vb - 1) / vb;
-    dim3 grid((unsigned)(n_states * p.NVB)), block(256);
-    switch (vb) {
-        case 128: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 128, VFIRST>), grid, block, 0, stream, p); break;
-        case 64: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 64, VFIRST>), grid, block, 0, stream, p); break;
-        default: hipLaunchKernelGGL((gdn_recurrent_kernel<T, KMAX, 32, VFIRST>), grid, block, 0, stream, p); break;
-    }
+    dim3 grid((unsigned)place(p, n_states * p.NVB, (int64_t)p.HV * p.NVB)), block(256);
+    void (*kern)(RecurrentParams) = vb == 128 ? gdn_recurrent_kernel<T, KMAX, 128, VFIRST>
+                                   : vb == 64 ? gdn_recurrent_kernel<T, KMAX, 64, VFIRST> : gdn_recurrent_kernel<T, KMAX, 32, VFIRST>;
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, p);
     return check_launch("gdn_recurrent_kernel");
 }
 
 template <typename T>
 static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stream) {
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
+    // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
+    if (p.K == 128 && p.V == 128 && !vfirst && !p.gk && !p.gv && n_states >= 1024 &&
+        !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
+        RecurrentParams pd = p;
+        const int64_t grid = place(pd, n_states, p.HV);
+        static SmemAttrDone attr_done;                   // per instantiation
+        if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T>, DECODE_LDS_PAD, attr_done, "hipFuncSetAttribute(decode)")) return rc;
+        hipLaunchKernelGGL(gdn_decode_kernel<T>, dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        return check_launch("gdn_decode_kernel");
+    }
     // Value block per workgroup: whole rows when there are enough (sequence, head) pairs to
     // fill 256 CUs several times over, narrower blocks otherwise.
     int vb = 128;
@@ -310,7 +466,7 @@ extern "C" int gdn_fused_recurrent_fwd(
     GDN_CHECK_ARG(K <= 256, GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: K=%lld > 256", (long long)K);
     GDN_CHECK_ARG(K % 4 == 0 && V % 4 == 0, GDN_ERR_UNSUPPORTED,
                   "gdn_fused_recurrent_fwd: K=%lld and V=%lld must be multiples of 4", (long long)K, (long long)V);
-    GDN_CHECK_ARG(N * HV * ((V + 31) / 32) < (1ll << 31), GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: grid too large");
+    GDN_CHECK_ARG((N + 8) * HV * ((V + 31) / 32) < (1ll << 31), GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: grid too large");
     GDN_CHECK_ARG(((uintptr_t)h0 % 16) == 0 && ((uintptr_t)ht % 16) == 0 && ((uintptr_t)gk % 16) == 0 &&
                       ((uintptr_t)gv % 16) == 0,
                   GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: h0/ht/gk/gv must be 16-byte aligned");

@@ -386,6 +386,70 @@ def test_no_tokens_returns_the_initial_state():
     assert torch.equal(ht, h0)
 
 
+@pytest.mark.parametrize('case', ['plain', 'flags', 'packed', 'slots', 'f16', 'fp32'])
+def test_decode_kernel_for_the_common_shape(case):
+    """K = V = 128, K-first states, 1024 or more (sequence, head) states: the decode kernel written for that shape."""
+    H, HV, D = 8, 32, 128
+    dtype = {'f16': torch.float16, 'fp32': torch.float32}.get(case, torch.bfloat16)
+    kw, okw = {}, {}
+    cu = None
+    if case == 'packed':
+        lens = [1, 3, 2, 1] * 8
+        cu = [0]
+        for x in lens:
+            cu.append(cu[-1] + x)
+        q, k, v, g, beta, _ = _inputs(1, cu[-1], H, HV, D, dtype, seed=17)
+        N = len(lens)
+    else:
+        N, T = 32, 2 if case != 'slots' else 1
+        q, k, v, g, beta, _ = _inputs(N, T, H, HV, D, dtype, seed=17)
+    gen = torch.Generator().manual_seed(18)
+    h0 = torch.randn(N, HV, D, D, generator=gen)
+    if case == 'flags':
+        A_log, dt_bias = 0.3 * torch.randn(HV, generator=gen), 0.3 * torch.randn(HV, generator=gen)
+        g, beta = torch.randn(g.shape, generator=gen), torch.randn(beta.shape, generator=gen)
+        okw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, A_log=A_log, dt_bias=dt_bias,
+                   use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True)
+        kw = dict(okw, A_log=A_log.cuda(), dt_bias=dt_bias.cuda())
+    else:
+        okw = kw = dict(use_qk_l2norm_in_kernel=True)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, **okw)
+    dev = 'cuda'
+    cu_t = None if cu is None else torch.tensor(cu, device=dev)
+    if case == 'slots':
+        pool = torch.randn(N + 5, HV, D, D, generator=gen)
+        idx = torch.randperm(N + 5, generator=gen)[:N]
+        pool[idx] = h0
+        dpool = pool.to(dev)
+        o, _ = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=dpool, inplace_final_state=True,
+                      ssm_state_indices=idx.to(dev), **kw)
+        ht = dpool[idx.to(dev)]
+        rest = [i for i in range(N + 5) if i not in idx.tolist()]
+        assert torch.equal(dpool[rest].cpu(), pool[rest])
+    else:
+        o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=h0.to(dev),
+                       output_final_state=True, cu_seqlens=cu_t, **kw)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+@pytest.mark.parametrize('N,HV,D,vfirst', [(65, 32, 128, False), (67, 32, 128, True), (75, 32, 64, False), (69, 32, 32, False)])
+def test_workgroup_placement_with_sequence_counts_that_are_not_multiples_of_8(N, HV, D, vfirst):
+    """Launches of 2048 or more workgroups hand every XCD runs of consecutive states; the grid is rounded up to whole
+    rounds of 8 runs and the surplus workgroups must do nothing: every state is updated exactly once."""
+    H = 8
+    q, k, v, g, beta, _ = _inputs(N, 1, H, HV, D, torch.bfloat16, seed=23)
+    gen = torch.Generator().manual_seed(24)
+    h0 = torch.randn(N, HV, D, D, generator=gen)
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, use_qk_l2norm_in_kernel=True)
+    dev = 'cuda'
+    dh0 = (h0.transpose(-1, -2).contiguous() if vfirst else h0).to(dev)
+    o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=dh0, output_final_state=True,
+                   use_qk_l2norm_in_kernel=True, state_v_first=vfirst)
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht.transpose(-1, -2) if vfirst else ht)
+
+
 def test_decode_and_prefill_replay_from_a_captured_graph():
     """Serving loops replay captured graphs: the entry points only enqueue kernels on the given
     stream (no allocation, no memset, no synchronisation of their own), so a captured decode step
