@@ -36,17 +36,28 @@ import torch  # noqa: E402
 import torch.nn.functional as F  # noqa: E402
 
 C, K, V = 64, 128, 128
-# algorithmic FLOPs per (token, v-head) of the chunked gated delta rule as the reference evaluates
-# it: 2*(3CK + 2CV + 3KV) = 180224 (K K^T, q k^T, w; u, P v_new; w S, k^T v_new, q S).
-# Here the sequential stage does k S, q S, k^T v_new (3KV), Xb D and P v_new (2CV); the rest
-# (K K^T, q k^T, the 64x64 inverse) is the chunk-parallel stage.
-F_TOTAL = 2 * (3 * C * K + 2 * C * V + 3 * K * V)      # 180224
-F_SCAN = 2 * (3 * K * V + 2 * C * V)                   # 131072
-F_PREP = F_TOTAL - F_SCAN                              # 49152
-# HBM bytes per call of the dominant stage on the default workload, from FETCH_SIZE + WRITE_SIZE of
-# a counter run of this file scaled by the calib_copy workload (profiles/ holds the summary); other
-# workloads: not measured
-TRAFFIC_BYTES = {'prefill': 1.52e9, 'conv_qkv': 1.0743e9, 'norm_gate': 0.8097e9}
+
+
+def flops_per_unit(k, v):
+    """Algorithmic FLOPs per (token, v-head) of the chunked gated delta rule as the reference evaluates it:
+    2*(3CK + 2CV + 3KV) (K K^T, q k^T, w; u, P v_new; w S, k^T v_new, q S) = 180224 at K = V = 128.
+    Here the sequential stage does k S, q S, k^T v_new (3KV), Xb D and P v_new (2CV); the rest (K K^T, q k^T, the
+    64x64 inverse) is the chunk-parallel stage.  Returns (whole operator, sequential stage)."""
+    return 2 * (3 * C * k + 2 * C * v + 3 * k * v), 2 * (3 * k * v + 2 * C * v)
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of a workload's dominant stage as a profiler run of this file measured them (FETCH_SIZE +
+    WRITE_SIZE scaled by the calib_copy workload): read from profiles/hbm_traffic.json, which names the run; None for
+    workloads that have no such run.  Nothing is measured in the run that prints it."""
+    try:
+        with open(os.path.join(ROOT, 'profiles', 'hbm_traffic.json')) as fh:
+            rec = json.load(fh)['workloads'].get(key)
+        return None if rec is None else rec['dominant_stage_bytes']
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 PEAK_BF16_TFLOPS = 2500.0                      # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0                          # MI355X HBM3E, published
 
@@ -62,6 +73,24 @@ WORKLOADS = {
 }
 
 
+def _published(B, T, H, D):
+    return dict(kind='prefill', B=B, T=T, H=H, HV=H, K=D, V=D, h0=False, varlen=False, final=False, l2norm=True, raw_qk=True,
+                name=f"the reference's published shape B={B} T={T} H={H} D={D} bf16: q, k not normalised, "
+                     'use_qk_l2norm_in_kernel, no initial state, no final state')
+
+
+# The shapes the reference publishes forward times for (benchmarks/ops/registry.py:323-335: H == HV, in-kernel l2 norm of
+# raw q and k, no initial and no final state; README.md:566-580 adds D = 64 and D = 256): context rows, never `value`.
+PUBLISHED = {
+    'ref_b1_t8192_h96_d128': _published(1, 8192, 96, 128),
+    'ref_b2_t16384_h16_d128': _published(2, 16384, 16, 128),
+    'ref_b4_t2048_h16_d128': _published(4, 2048, 16, 128),
+    'ref_b4_t4096_h64_d128': _published(4, 4096, 64, 128),
+    'ref_b8_t1024_h8_d64': _published(8, 1024, 8, 64),
+    'ref_b8_t2048_h32_d256': _published(8, 2048, 32, 256),
+}
+
+
 def _ensure_built():
     from fla_hip import _lib
     if not os.path.exists(_lib.LIB_PATH):
@@ -73,8 +102,11 @@ def make_prefill_inputs(w, device):
     from oracle import gdn_oracle as O
     gen = torch.Generator().manual_seed(42)
     B, T, H, HV = w['B'], w['T'], w['H'], w['HV']
-    q = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1).bfloat16()
-    k = F.normalize(torch.randn(B, T, H, K, generator=gen), p=2, dim=-1).bfloat16()
+    K, V = w.get('K', 128), w.get('V', 128)
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    if not w.get('raw_qk'):
+        q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    q, k = q.bfloat16(), k.bfloat16()
     v = torch.randn(B, T, HV, V, generator=gen).bfloat16()
     g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / 16
     beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
@@ -118,10 +150,15 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
     cpu, d = make_prefill_inputs(w, device)
     tokens = w['B'] * w['T']
+    K, V = w.get('K', 128), w.get('V', 128)
+    final, l2norm = w.get('final', True), w.get('l2norm', False)
+    F_TOTAL, F_SCAN = flops_per_unit(K, V)
+    F_PREP = F_TOTAL - F_SCAN
 
     def step():
         return chunk_gated_delta_rule(d['q'], d['k'], d['v'], d['g'], d['beta'], initial_state=d['h0'],
-                                      output_final_state=True, cu_seqlens=d['cu_t'], cu_seqlens_cpu=d['cu_cpu'])
+                                      output_final_state=final, use_qk_l2norm_in_kernel=l2norm,
+                                      cu_seqlens=d['cu_t'], cu_seqlens_cpu=d['cu_cpu'])
 
     spin_up(step)
     for _ in range(warmup):
@@ -145,9 +182,18 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     per_call = sorted(a.elapsed_time(b) for a, b in evq)
     quant = {f'p{int(100 * f)}': round(per_call[min(len(per_call) - 1, int(f * len(per_call)))], 4) for f in (0.2, 0.5, 0.8)}
 
+    units = tokens * w['HV']
+    whole = dict(flops=units * F_TOTAL, achieved=round(units * F_TOTAL / (elapsed / steps) / 1e12, 2),
+                 frac=round(units * F_TOTAL / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 5))
+    if not w.get('stages', True):
+        # context rows: the whole call against the matrix-core peak for the operator's algorithmic FLOPs
+        roofline = dict(bound='mfma', achieved=whole['achieved'], peak=PEAK_BF16_TFLOPS, unit='TFLOP/s', frac=whole['frac'],
+                        traffic=None, kernel='whole operator (all launches of one call)', kernel_us=round(ms_per_step * 1e3, 1),
+                        flops_per_launch=whole['flops'])
+        return dict(value=tokens * steps / elapsed, ms_per_step=ms_per_step, roofline=roofline, call_ms_quantiles=quant)
     # per-kernel durations: the same work issued as its two stages with HIP events in between
-    call = ChunkLaunch(d['q'], d['k'], d['v'], d['g'], d['beta'], K ** -0.5, d['h0'], True, False,
-                       d['cu_t'], d['cu_cpu'], None, 64)
+    call = ChunkLaunch(d['q'], d['k'], d['v'], d['g'], d['beta'], K ** -0.5, d['h0'], final, False,
+                       d['cu_t'], d['cu_cpu'], None, 64, qk_l2norm=l2norm)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     for i in range(steps):
         ev[i][0].record()
@@ -158,17 +204,15 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     torch.cuda.synchronize()
     t_prep = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e-3
     t_scan = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e-3
-    units = tokens * w['HV']
     scan_name = ('gdn_chunk_fwd_scan: gdn_chunk_wide_kernel / gdn_chunk_pair_kernel '
                  '(+ gdn_segment_merge_kernel when time is cut into segments)')
     dom = (scan_name, F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_fwd_prepare: gdn_chunk_prepare_kernel', F_PREP, t_prep)
     achieved = units * dom[1] / dom[2] / 1e12
     roofline = dict(bound='mfma', achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit='TFLOP/s',
-                    frac=round(achieved / PEAK_BF16_TFLOPS, 5), traffic=TRAFFIC_BYTES.get(w['key']), kernel=dom[0],
+                    frac=round(achieved / PEAK_BF16_TFLOPS, 5), traffic=measured_traffic(w['key']), kernel=dom[0],
                     kernel_us=round(dom[2] * 1e6, 1), flops_per_launch=units * dom[1],
                     kernels_us=dict(gdn_chunk_fwd_prepare=round(t_prep * 1e6, 1), gdn_chunk_fwd_scan=round(t_scan * 1e6, 1)),
-                    whole_op=dict(flops=units * F_TOTAL, achieved=round(units * F_TOTAL / (elapsed / steps) / 1e12, 2),
-                                  frac=round(units * F_TOTAL / (elapsed / steps) / 1e12 / PEAK_BF16_TFLOPS, 5)))
+                    whole_op=whole)
     out = dict(value=tokens * steps / elapsed, ms_per_step=ms_per_step, roofline=roofline, call_ms_quantiles=quant)
 
     if with_cpu:
@@ -237,7 +281,7 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     state_bytes = 2 * N * HV * K * V * 4
     achieved = state_bytes / t_kernel / 1e9
     roofline = dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
-                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None, kernel='gdn_recurrent_kernel',
+                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=measured_traffic(w['key']), kernel='gdn_decode_kernel',
                     kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=state_bytes)
     out = dict(value=elapsed / steps * 1e6, ms_per_step=elapsed / steps * 1e3, roofline=roofline)
     if with_cpu:
@@ -296,7 +340,7 @@ def bench_layer_steps(steps, warmup, device, with_cpu):
         achieved = nbytes / t_kernel / 1e9
         out[key] = dict(workload=name, ms_per_step=round(wall * 1e3, 4), tokens_per_s=round(T / wall, 1),
                         roofline=dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
-                                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=TRAFFIC_BYTES[key], kernel=kernel,
+                                      frac=round(achieved / PEAK_HBM_GBS, 4), traffic=measured_traffic(key), kernel=kernel,
                                       kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=nbytes))
     if with_cpu:
         from oracle import modules_oracle as MO
@@ -362,7 +406,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + ['layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     args = ap.parse_args()
@@ -387,6 +431,14 @@ def main():
         return
     for key, val in WORKLOADS.items():
         val['key'] = key
+    if args.workload in PUBLISHED:
+        w = dict(PUBLISHED[args.workload], key=args.workload, stages=False)
+        r = bench_prefill(w, args.steps, args.warmup, device, False)
+        print(json.dumps(dict(metric='gdn_chunk_prefill_tokens_per_s', value=round(r['value'], 1), unit='tokens/s', higher_is_better=True,
+                              n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(r['ms_per_step'], 4), dtype='bf16',
+                              data='synthetic', config=dict(workload=w['name'], chunk_size=64), roofline=r['roofline'],
+                              call_ms_quantiles=r['call_ms_quantiles'])))
+        return
     w = WORKLOADS[args.workload]
     fn = bench_prefill if w['kind'] == 'prefill' else bench_decode
     res = fn(w, args.steps, args.warmup, device, not args.no_cpu_baseline)
@@ -420,6 +472,11 @@ def main():
             extra[name] = e
             torch.cuda.empty_cache()
         extra.update(bench_layer_steps(args.steps, args.warmup, device, not args.no_cpu_baseline))
+        for name, ww in PUBLISHED.items():
+            r = bench_prefill(dict(ww, key=name, stages=False), max(10, args.steps // 2), max(3, args.warmup // 2), device, False)
+            extra[name] = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), tokens_per_s=round(r['value'], 1),
+                               call_ms_quantiles=r['call_ms_quantiles'], roofline=r['roofline'])
+            torch.cuda.empty_cache()
         line['other_workloads'] = extra
     print(json.dumps(line))
 

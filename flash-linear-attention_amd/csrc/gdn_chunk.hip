@@ -16,6 +16,14 @@ static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, h
     // a q/k head; in pass 1 the S and M runs of one head).  That halves the number of workgroups and
     // runs a pair about 1.25 times as fast as two single runs one after the other, so it pays as soon
     // as the single runs would not all fit on the chip at once.
+    if (p.K > 128) {
+        // wide keys: whole sequences, a workgroup per 64 value columns; the scan forms P itself
+        p.want_P = 0;
+        if (stages & STAGE_PREPARE) {
+            if (int rc = launch_prepare<T>(p, num_chunks, stream)) return rc;
+        }
+        return (stages & STAGE_SCAN) ? launch_wide256<T>(p, stream) : GDN_OK;
+    }
     const int64_t G = p.HV / p.H;
     const int nseg = plan_segments(p.N, p.HV, p.NT, num_chunks, p.cu_seqlens == nullptr, p.flags);
     const bool segments = nseg > 0;
@@ -64,12 +72,16 @@ static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, h
 
 }  // namespace gdn
 
-static bool chunk_dims_ok(int64_t K, int64_t V) { return K >= 8 && V >= 8 && K <= 128 && V <= 128 && K % 8 == 0 && V % 8 == 0; }
+// K, V multiples of 8: both up to 128, or wide keys (128 < K <= 256) with any number of value columns
+static bool chunk_dims_ok(int64_t K, int64_t V) {
+    return K >= 8 && V >= 8 && K % 8 == 0 && V % 8 == 0 && (K <= 128 ? V <= 128 : (K <= 256 && V <= 8192));
+}
 
 // bytes of workspace for the plan that launch_chunk will choose
-static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int64_t HV, bool packed, uint32_t flags,
+static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int64_t HV, int64_t K, bool packed, uint32_t flags,
                                    char* base, gdn::ChunkWs* ws) {
     using namespace gdn;
+    if (K > 128) flags = (flags & ~GDN_FLAG_SCAN_SEGMENTS) | GDN_FLAG_SCAN_WIDE;       // wide keys: no time segments
     const int nseg = plan_segments(N, HV, (T + CH - 1) / CH, num_chunks, !packed, flags);
     return ws_layout(num_chunks, HV, (int64_t)nseg * N * HV, base, ws);
 }
@@ -77,7 +89,7 @@ static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int
 extern "C" size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V,
                                             int packed, uint32_t flags) {
     if (!chunk_dims_ok(K, V) || num_chunks < 0 || N < 1 || T < 0 || H < 1 || HV < 1) return 0;
-    return chunk_workspace_need(N, T, num_chunks, HV, packed != 0, flags, nullptr, nullptr);
+    return chunk_workspace_need(N, T, num_chunks, HV, K, packed != 0, flags, nullptr, nullptr);
 }
 
 static int chunk_entry(
@@ -99,7 +111,7 @@ static int chunk_entry(
     GDN_CHECK_ARG(!(flags & GDN_FLAG_SCAN_NO_PAIR) || !(flags & GDN_FLAG_SCAN_PAIR), GDN_ERR_INVALID, "%s: GDN_FLAG_SCAN_PAIR and GDN_FLAG_SCAN_NO_PAIR exclude each other", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
     GDN_CHECK_ARG(chunk_dims_ok(K, V), GDN_ERR_UNSUPPORTED,
-                  "%s: head dims must be multiples of 8 up to 128 (got K=%lld V=%lld)", who, (long long)K, (long long)V);
+                  "%s: head dims must be multiples of 8, K, V <= 128 or 128 < K <= 256 (got K=%lld V=%lld)", who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
                   "%s: q/k/v must be bf16 or f16", who);
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * H < (1ll << 31), GDN_ERR_UNSUPPORTED, "%s: too many heads or chunks for one launch", who);
@@ -120,7 +132,7 @@ static int chunk_entry(
         return GDN_OK;
     }
     ChunkParams p;
-    const size_t need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, (char*)workspace, &p.ws);
+    const size_t need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
@@ -193,10 +205,10 @@ extern "C" int gdn_chunk_fwd_static(
     GDN_CHECK_ARG(chunk_dims_ok(K, V) && N >= 1 && T >= 0 && HV >= 1 && num_chunks >= 0, GDN_ERR_INVALID,
                   "%s: bad dimensions", who);
     // The plan with time segments needs room for their matrices; when only that does not fit, whole sequences do.
-    size_t need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, nullptr, nullptr);
+    size_t need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, nullptr, nullptr);
     if (need > GDN_CHUNK_STATIC_WORKSPACE_BYTES && !(flags & GDN_FLAG_SCAN_SEGMENTS)) {
         flags |= GDN_FLAG_SCAN_WIDE;
-        need = chunk_workspace_need(N, T, num_chunks, HV, cu_seqlens != nullptr, flags, nullptr, nullptr);
+        need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, nullptr, nullptr);
     }
     GDN_CHECK_ARG(need <= GDN_CHUNK_STATIC_WORKSPACE_BYTES, GDN_ERR_WORKSPACE,
                   "%s: this input needs %zu bytes of workspace, the built-in one holds %zu (%lld records of one chunk and "

@@ -149,7 +149,7 @@ struct ChunkParams {
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     ChunkWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;       // NT: chunks per sequence (dense input)
-    int K, V;                                          // head dims of the caller's tensors (multiples of 8, <= 128)
+    int K, V;                                          // head dims of the caller's tensors (multiples of 8; K, V <= 128, or 128 < K <= 256 with any V)
     float scale; int gb_dtype; uint32_t flags;
     int64_t NH;
     int want_P;                                        // the scan will read P from the records (two runs per workgroup)
@@ -252,5 +252,7 @@ template <typename T> int launch_prepare(const ChunkParams& p, int64_t num_chunk
 template <typename T> int launch_wide(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
 template <typename T> int launch_pair(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
 int launch_segment_merge(const ChunkParams& p, SegmentPlan sp, hipStream_t stream);
+// Sequential stage for 128 < K <= 256 (gdn_chunk_wide256.hip): whole sequences, any V that is a multiple of 8.
+template <typename T> int launch_wide256(const ChunkParams& p, hipStream_t stream);
 
 }  // namespace gdn

@@ -58,50 +58,84 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
     // q is needed for its row norms (l2 normalisation) and for P, when the scan wants P from the records
     const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
     const bool want_P = p.want_P != 0, need_q = l2 || want_P;
-    // ---- all global loads first: the gate inputs of value head w of the group, then the k, q rows
-    // (rows past the end of the sequence are zero) ----
+    // ---- all global loads first: the gate inputs of value head w of the group, then the k, q rows ----
     float rg = 0.f, rb = 0.f;
     if (w < G && lane < valid) {
         rg = p.g ? load_scalar(p.g, (tok0 + lane) * HV + h * G + w, p.gb_dtype) : 0.f;      // (no gate: the plain delta rule)
         rb = load_scalar(p.beta, (tok0 + lane) * HV + h * G + w, p.gb_dtype);
     }
+    // ---- k (and q) rows, 128 key features at a time (K <= 128: one round): into LDS, their squared norms, and the raw
+    // products, which stay in registers: K K^T tiles (row-tile w, column-tiles <= w) and the transposed q K^T tiles
+    // of query tile tt = 3 - w (key tiles <= tt).  Rows past the end of the sequence and key features past K are zero.
+    const int tt = 3 - w;
+    f32x4 kk[4], qk[4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) kk[tj] = qk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
     {
-        // (key features past K are zero, like the rows past the end: the tiles are always 64 x 128)
         const int K = p.K;
         const T* kg = (const T*)p.k + (tok0 * H + h) * K;
         const T* qg = (const T*)p.q + (tok0 * H + h) * K;
-        u32x4 rk[4], rq[4];
+        float sk[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int k0 = 0; k0 < K; k0 += 128) {
+            if (k0) __syncthreads();                 // the products of the previous round have read the tiles
+            u32x4 rk[4], rq[4];
 #pragma unroll
-        for (int ps = 0; ps < 4; ++ps) {
-            const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
-            const u32x4 z = {0u, 0u, 0u, 0u};
-            rk[ps] = rq[ps] = z;
-            if (row < valid && col < K) {
-                rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * K + col);
-                if (need_q) rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
+            for (int ps = 0; ps < 4; ++ps) {
+                const int row = ps * 16 + (tid >> 4), col = k0 + (tid & 15) * 8;
+                const u32x4 z = {0u, 0u, 0u, 0u};
+                rk[ps] = rq[ps] = z;
+                if (row < valid && col < K) {
+                    rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * K + col);
+                    if (need_q) rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
+                }
             }
-        }
 #pragma unroll
-        for (int ps = 0; ps < 4; ++ps) {
-            const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
-            *(u32x4*)(k_nat + row * NP + col) = rk[ps];
-            if (want_P) *(u32x4*)(q_nat + row * NP + col) = rq[ps];
-            // l2 normalisation is applied as per-row factors: 16 lanes hold one row
-            float sk = 0.f, sq = 0.f;
-            if (l2) {
-                const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
+            for (int ps = 0; ps < 4; ++ps) {
+                const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
+                *(u32x4*)(k_nat + row * NP + col) = rk[ps];
+                if (want_P) *(u32x4*)(q_nat + row * NP + col) = rq[ps];
+                // l2 normalisation is applied as per-row factors: 16 lanes hold one row
+                if (l2) {
+                    const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk += a * a; sq += b * b; }
-#pragma unroll
-                for (int off = 1; off < 16; off <<= 1) { sk += __shfl_xor(sk, off, 64); sq += __shfl_xor(sq, off, 64); }
+                    for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk[ps] += a * a; sq[ps] += b * b; }
+                }
             }
-            if ((tid & 15) == 0) {
-                sRN[row] = l2 ? rsqrtf(sk + 1e-6f) : 1.f;
-                sRN[CH + row] = l2 ? rsqrtf(sq + 1e-6f) : 1.f;
+            if (k0 + 128 >= K) {
+#pragma unroll
+                for (int ps = 0; ps < 4; ++ps) {
+                    float a = sk[ps], b = sq[ps];
+                    if (l2) {
+#pragma unroll
+                        for (int off = 1; off < 16; off <<= 1) { a += __shfl_xor(a, off, 64); b += __shfl_xor(b, off, 64); }
+                    }
+                    if ((tid & 15) == 0) {
+                        const int row = ps * 16 + (tid >> 4);
+                        sRN[row] = l2 ? rsqrtf(a + 1e-6f) : 1.f;
+                        sRN[CH + row] = l2 ? rsqrtf(b + 1e-6f) : 1.f;
+                    }
+                }
+            }
+            __syncthreads();
+            V8 ka[4], qb[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                ka[s] = *(const V8*)(k_nat + (16 * w + c16) * NP + 32 * s + 8 * g);
+                if (want_P) qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
+            }
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                if (tj <= w || (want_P && tj <= tt)) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 kb = *(const V8*)(k_nat + (16 * tj + c16) * NP + 32 * s + 8 * g);
+                        if (tj <= w) kk[tj] = Mma<T>::run(ka[s], kb, kk[tj]);          // rows: tokens of tile w, column: token 16tj + c16
+                        if (want_P && tj <= tt) qk[tj] = Mma<T>::run(kb, qb[s], qk[tj]);         // rows: key tokens of tile tj, column: query token 16tt + c16
+                    }
+                }
             }
         }
     }
-    __syncthreads();
     // ---- gates of every value head of the group: inclusive scan over the chunk, one token per lane ----
     for (int m = w; m < G; m += 4) {
         const int hv = h * G + m;
@@ -139,31 +173,6 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tab2[TAB2_NK + lane] = nk;
     }
 
-    // ---- raw products, kept in registers: K K^T tiles (row-tile w, column-tiles <= w) and the
-    // transposed q K^T tiles of query tile tt = 3 - w (key tiles <= tt) ----
-    const int tt = 3 - w;
-    f32x4 kk[4], qk[4];
-    {
-        V8 ka[4], qb[4];
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            ka[s] = *(const V8*)(k_nat + (16 * w + c16) * NP + 32 * s + 8 * g);
-            if (want_P) qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
-        }
-#pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            kk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
-            qk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (tj <= w || (want_P && tj <= tt)) {
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const V8 kb = *(const V8*)(k_nat + (16 * tj + c16) * NP + 32 * s + 8 * g);
-                    if (tj <= w) kk[tj] = Mma<T>::run(ka[s], kb, kk[tj]);          // rows: tokens of tile w, column: token 16tj + c16
-                    if (want_P && tj <= tt) qk[tj] = Mma<T>::run(kb, qb[s], qk[tj]);         // rows: key tokens of tile tj, column: query token 16tt + c16
-                }
-            }
-        }
-    }
     // |k_t|^2 is the diagonal of K K^T: lane (c16, g) of the diagonal tile holds rows 4g .. 4g+3 of column c16
     {
         float d = 0.f;

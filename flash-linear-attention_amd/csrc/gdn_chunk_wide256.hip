@@ -1,0 +1,453 @@
+// Sequential stage of the chunked prefill for WIDE keys, 128 < K <= 256 (the reference's scan holds up to four
+// [64, BV] state tiles, i.e. K <= 256: fla/ops/common/chunk_delta_h.py:108-114, 210-315).  Same step as
+// gdn_chunk_wide.hip,
+//   D = v - 2^G (k S),  v_new = Xb D,  o = scale 2^G (q S) + P v_new,  S = 2^G_last S + k^T (v_new 2^(G_last-G)),
+// with the state of one workgroup cut along the VALUE columns instead: a workgroup owns 64 value columns of one
+// (sequence, value head) for all 256 key rows (the value columns of the recurrence never mix), compute wave w the
+// columns 16w .. 16w+15: 16 state tiles of 16 x 16 per wave, the same 64 registers as the 128 x 32 slab of the
+// narrow kernel.  A head with V value columns takes ceil(V / 64) workgroups, which share the head's record and, with
+// the other value heads of the q/k head, its k and q rows (consecutive slots of one XCD: one L2).
+//
+// k and q tiles are two 128-feature halves, each laid out exactly like the narrow kernel's tile, so every operand
+// address is the narrow kernel's plus a half offset.  What differs is the LDS budget: 64 tokens x 512 B of k and of
+// q are 32 KB each.  k has two buffers (read until the very end of a step, copied one step ahead), v and the record
+// have two, q and P have ONE: q of the next chunk is copied after the barrier that ends this chunk's last read of
+// it, while the compute waves finish the state update.
+#include "gdn_chunk_common.h"
+
+namespace gdn {
+
+constexpr int W2_KB = 0;                                  // two k buffers: [half][16 KB tile]
+constexpr int W2_Q = 65536;                               // q: [half][16 KB tile]
+constexpr int W2_V = 98304;                               // two v tiles, 64 rows of 256 B of which the first 128 B are used
+constexpr int W2_REC = 131072;                            // two records without P
+constexpr int W2_RX = 0, W2_RTAB = 5120, W2_RTAB2 = 6144, W2_REC_BYTES = 7168;
+constexpr int W2_P = W2_REC + 2 * W2_REC_BYTES;           // P of the current chunk, formed here
+constexpr int W2_OT = W2_P + 5120;                        // output tile [64 tokens][W2_OT_PITCH]
+constexpr int W2_OT_PITCH = 144;                          // 128 B of a row + pad
+constexpr int W2_PCOUNT = W2_OT + 64 * W2_OT_PITCH;
+constexpr size_t W2_SMEM = W2_PCOUNT + 16;                // 159 760 B
+constexpr int W2_CW = 4;                                  // compute waves
+constexpr int W2_THREADS = (W2_CW + 4) * 64;
+constexpr int W2_VB = 64;                                 // value columns per workgroup
+
+template <typename T>
+__global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkParams p, int NVB) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    const int K = p.K, V = p.V;
+    const int tid = threadIdx.x, lane = tid & 63, c16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int H = p.H, HV = p.HV;
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
+
+    // ---- which (sequence, value head, block of value columns): the workgroups that read the same k and q rows take
+    // consecutive slots of one XCD (block index mod 8) ----
+    const int G = HV / H, GV = G * NVB;
+    const int64_t slot = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
+    const int64_t group = (slot / GV) * 8 + xcd;                     // (sequence, q/k head)
+    if (group >= p.N * H) return;
+    int64_t n = group / H;
+    if (p.flags & GDN_FLAG_SEQ_ORDER) n = load_index(p.chunk_offsets, p.N + 1 + n, cu32);
+    const int h = (int)(group % H);
+    const int member = (int)(slot % GV);
+    const int hv = h * G + member / NVB;
+    const int v0 = (member % NVB) * W2_VB;
+    const int64_t inh = n * HV + hv;
+    const float* src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr;
+    float* dst = p.ht ? p.ht + inh * (int64_t)(K * V) : nullptr;
+
+    int64_t bos, len, boh;
+    if (p.cu_seqlens) {
+        bos = load_index(p.cu_seqlens, n, cu32);
+        len = load_index(p.cu_seqlens, n + 1, cu32) - bos;
+        boh = load_index(p.chunk_offsets, n, cu32);
+    } else {
+        bos = n * p.T;
+        len = p.T;
+        boh = n * p.NT;
+    }
+    const int64_t nsteps = (len + CH - 1) / CH;
+    const int64_t lastc = nsteps - 1;
+    char* otile = smem + W2_OT;
+    volatile int* pcount = (volatile int*)(smem + W2_PCOUNT);
+    if (tid == 0) *pcount = 0;
+    // Key features past K and value columns past V are never copied: the tiles are cleared once.
+    if (nsteps > 0) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int i = tid; i < W2_REC / 16; i += W2_THREADS) *(u32x4*)(smem + i * 16) = z;
+    }
+    lds_barrier();
+
+    const int a_off = (c16 >> 2) * 64 + 4 * (c16 & 3) + ((g + (c16 >> 2)) & 3);   // operand piece 4s + g of row c16 of a t-tile (16-byte units)
+
+    // =====================================================================================
+    // Copy waves.  Step i reads stage i & 1 of k, v and the record; barrier B1 ends the reads of q, v, the record and
+    // the writes of the output tile, barrier B2 the reads of k.
+    // =====================================================================================
+    if (w >= W2_CW) {
+        if (nsteps <= 0) return;
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+        // P = scale tril(q k^T 2^(G_t - G_t')) of a chunk from its q and k tiles (see gdn_chunk_wide.hip), contraction
+        // over both halves of the key features
+        auto produce_P = [&](const char* kbuf, const char* rec) {
+            __builtin_amdgcn_s_setprio(3);
+            const int pw = w - W2_CW;
+            const V8* sK = (const V8*)kbuf;
+            const V8* sQ = (const V8*)(smem + W2_Q);
+            const float* t2 = (const float*)(rec + W2_RTAB2);
+            auto frag = [&](int tt, int sp) {
+                V8 qb[8];
+#pragma unroll
+                for (int s8 = 0; s8 < 8; ++s8) qb[s8] = sQ[(s8 >> 2) * 1024 + tt * 256 + 16 * (s8 & 3) + a_off];
+                const int t = 16 * tt + c16;
+                const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                V8 out;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int tj = 2 * sp + half;
+                    if (tj > tt) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) out[half * 4 + r] = from_f32<T>(0.f);
+                        continue;
+                    }
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s8 = 0; s8 < 8; ++s8) acc = Mma<T>::run(sK[(s8 >> 2) * 1024 + tj * 256 + 16 * (s8 & 3) + a_off], qb[s8], acc);
+                    const f32x4 gj = *(const f32x4*)(t2 + TAB2_G + 16 * tj + 4 * g), nj = *(const f32x4*)(t2 + TAB2_NK + 16 * tj + 4 * g);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = 16 * tj + 4 * g + r;
+                        out[half * 4 + r] = from_f32<T>((t >= j) ? st_ * nj[r] * acc[r] * fast_exp2(gt - gj[r]) : 0.f);
+                    }
+                }
+                store_frag<T>(smem + W2_P, tt, sp, lane, out);
+            };
+            if (pw == 0) frag(3, 0);
+            else if (pw == 1) frag(3, 1);
+            else if (pw == 2) { frag(2, 0); frag(0, 0); }
+            else { frag(1, 0); frag(2, 1); }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_fetch_add((int*)pcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __builtin_amdgcn_s_setprio(0);
+        };
+        // Rows 4j .. 4j+3 of a [token][head][K] tensor, 128 features of them (`half`), into block j of a 16 KB tile:
+        // lane (g, c16) holds piece c = 4g + ((c16 - j) & 3) of row 4j + c16 / 4.  Rows past the end of the sequence
+        // re-read its last row (finite, and multiplied by zeros everywhere).
+        auto gather_qk = [&](const T* tensor, int64_t it, uint32_t lds_tile) {
+            const int valid = (int)min((int64_t)CH, len - it * CH);
+            const char* base = (const char*)(tensor + ((bos + it * CH) * H + h) * K);
+            const uint32_t row_bytes = (uint32_t)(H * K * 2);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int c = 4 * g + ((c16 - j) & 3);
+                    const uint64_t mask = __builtin_amdgcn_ballot_w64(128 * half + 8 * c < K);
+                    const int row = min(4 * j + (c16 >> 2), valid - 1);
+                    gather_1k_to_lds_masked(base, (uint32_t)row * row_bytes + 256 * half + 16 * c, lds_tile + half * 16384 + j * 1024, mask);
+                }
+        };
+        auto copy_rec = [&](int64_t it, uint32_t lds_rec) {
+            const char* rec = p.ws.Rec + ((boh + it) * HV + hv) * REC_BYTES;
+#pragma unroll
+            for (int j = 0; j < REC_PIECES_X; ++j) gather_1k_to_lds(rec + REC_X + j * 1024, lane * 16, lds_rec + W2_RX + j * 1024);
+            gather_1k_to_lds(rec + REC_TAB, lane * 16, lds_rec + W2_RTAB);
+            gather_1k_to_lds(rec + REC_TAB2, lane * 16, lds_rec + W2_RTAB2);
+        };
+        if (w == W2_CW) {
+            // ---- k: chunk i+1 is copied during step i (its buffer was last read in step i-1) ----
+            gather_qk((const T*)p.k, 0, lds0 + W2_KB);
+            wait_vm_at_most<0>();
+            lds_barrier();                                                  // B0
+            for (int64_t i = 0; i < nsteps; ++i) {
+                gather_qk((const T*)p.k, min(i + 1, lastc), lds0 + W2_KB + (int)((i + 1) & 1) * 32768);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                lds_barrier();                                              // B1
+                wait_vm_at_most<0>();
+                lds_barrier();                                              // B2
+            }
+        } else if (w == W2_CW + 1) {
+            // ---- q (one buffer: copied between B1 and B2) and the record (two) ----
+            gather_qk((const T*)p.q, 0, lds0 + W2_Q);
+            copy_rec(0, lds0 + W2_REC);
+            wait_vm_at_most<0>();
+            lds_barrier();                                                  // B0
+            for (int64_t i = 0; i < nsteps; ++i) {
+                copy_rec(min(i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                lds_barrier();                                              // B1
+                gather_qk((const T*)p.q, min(i + 1, lastc), lds0 + W2_Q);
+                wait_vm_at_most<0>();
+                lds_barrier();                                              // B2
+            }
+        } else if (w == W2_CW + 2) {
+            // ---- v: the 64 columns of this workgroup, 4 rows per copy (lanes g < 2 hold the 8 pieces of a row) ----
+            auto gather_v = [&](int64_t it, uint32_t lds_tile) {
+                const int valid = (int)min((int64_t)CH, len - it * CH);
+                const char* base = (const char*)((const T*)p.v + ((bos + it * CH) * HV + hv) * V + v0);
+                const uint32_t row_bytes = (uint32_t)(HV * V * 2);
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int c = 4 * g + ((c16 - j) & 3);
+                    const uint64_t mask = __builtin_amdgcn_ballot_w64(c < 8 && v0 + 8 * c < V);
+                    const int row = min(4 * j + (c16 >> 2), valid - 1);
+                    gather_1k_to_lds_masked(base, (uint32_t)row * row_bytes + 16 * c, lds_tile + j * 1024, mask);
+                }
+            };
+            gather_v(0, lds0 + W2_V);
+            wait_vm_at_most<0>();
+            lds_barrier();                                                  // B0
+            for (int64_t i = 0; i < nsteps; ++i) {
+                gather_v(min(i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                lds_barrier();                                              // B1
+                wait_vm_at_most<0>();
+                lds_barrier();                                              // B2
+            }
+        } else {
+            // ---- output rows: one instruction stores 8 token rows of 128 bytes ----
+            T* og = (T*)p.o;
+            u32x4 orow[8];
+            const int orow_r = lane >> 3, opiece = lane & 7;
+            auto store_rows = [&](int64_t it) {
+                const int valid = (int)min((int64_t)CH, len - it * CH);
+                const bool col_ok = v0 + 8 * opiece < V;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int row = 8 * j + orow_r;
+                    if (row < valid && col_ok) *(u32x4*)(og + ((bos + it * CH + row) * HV + hv) * V + v0 + 8 * opiece) = orow[j];
+                }
+            };
+            lds_barrier();                                                  // B0
+            for (int64_t i = 0; i < nsteps; ++i) {
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                if (i > 0) store_rows(i - 1);
+                lds_barrier();                                              // B1
+#pragma unroll
+                for (int j = 0; j < 8; ++j) orow[j] = *(const u32x4*)(otile + (8 * j + orow_r) * W2_OT_PITCH + opiece * 16);
+                lds_barrier();                                              // B2 (waits for the tile reads)
+            }
+            store_rows(lastc);
+        }
+        wait_vm_at_most<0>();                               // no copy may land in LDS after this workgroup has gone
+        return;
+    }
+
+    // =====================================================================================
+    // Compute waves
+    // =====================================================================================
+    // state tile m (0..15), row 4g + r: key feature 32 (m/2) + 8g + 4 (m%2) + r; column: value v0 + 16w + c16
+    f32x4 S[16];
+    const int vc = v0 + 16 * w + c16;
+    const int sk = vfirst ? 1 : V, sv = vfirst ? K : 1;
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+        const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        if (src && kk < K && vc < V) {
+            const float* e = src + (int64_t)kk * sk + (int64_t)vc * sv;
+            s = f32x4{e[0], e[sk], e[2 * sk], e[3 * sk]};
+        }
+        S[m] = s;
+    }
+    // lazy decay, as in the narrow kernel: the registers hold S / 2^lg
+    constexpr float LG_MIN = std::is_same<T, bf16_t>::value ? -60.f : 1.f;
+    float lg = 0.f;
+
+    const int tr_i = c16 >> 2, tr_j = c16 & 3;
+    const int k_tr = (g * 64 + 4 * tr_i + ((tr_j + g) & 3)) * 8;
+    int v_tr;
+    {
+        const int c = 2 * w + (tr_j >> 1);
+        v_tr = (g * 64 + 16 * (c >> 2) + 4 * tr_i + ((c + g) & 3)) * 8 + 4 * (tr_j & 1);
+    }
+
+    auto step = [&](const char* kbuf, const char* vbuf, const char* rec, int p_target) {
+        const V8* sK = (const V8*)kbuf;
+        const V8* sQ = (const V8*)(smem + W2_Q);
+        const T* sV = (const T*)vbuf;
+        const T* sKt = (const T*)kbuf;
+        const char* sX = rec + W2_RX;
+        const char* sP = smem + W2_P;
+        const float* sTab = (const float*)(rec + W2_RTAB);
+        auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+
+        // fragment f = (t-tile f/8, key features 32s .. 32s+31 with s = f%8) of k and q, in a ring of register sets
+        constexpr int RING = 3;
+        V8 ak[RING], aq[RING];
+        auto F = [&](int f) {
+            const int idx = ((f & 7) >> 2) * 1024 + (f >> 3) * 256 + 16 * (f & 3) + a_off;
+            ak[f % RING] = sK[idx];
+            aq[f % RING] = sQ[idx];
+        };
+        f32x4 ks[4], ao[4];
+        V8 Sb[8];
+        auto M = [&](int f) {
+            const int tt = f >> 3, sx = f & 7;
+            ks[tt] = Mma<T>::run(ak[f % RING], Sb[sx], sx ? ks[tt] : f32x4{0.f, 0.f, 0.f, 0.f});
+            ao[tt] = Mma<T>::run(Sb[sx], aq[f % RING], sx ? ao[tt] : f32x4{0.f, 0.f, 0.f, 0.f});
+        };
+        V4 vv[4];
+        V8 ax[4][2], ap[4][2];
+        auto FV = [&](int tt) { vv[tt] = Mma<T>::tr_read(sV + tt * 2048 + v_tr); };
+        auto FX = [&](int tt) {
+#pragma unroll
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = load_frag<T>(sX, tt, sp2, lane);
+        };
+        auto FP = [&](int tt) {
+#pragma unroll
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
+        };
+        // k^T operands of the state update, u = 16 sp2 + m (t-tile pair sp2, key tile m), in a ring of 8
+        V8 kt[8];
+        auto FK = [&](int u) {
+            const int sp2 = u >> 4, m = u & 15;
+            const T* a = sKt + (m >> 3) * 8192 + sp2 * 4096 + 128 * ((m & 7) >> 1) + 4 * (m & 1) + k_tr;
+            kt[u & 7] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 2048));
+        };
+        float gamma, vscale;
+        V8 Db[2], Vn[2], Vg[2];
+        auto TD = [&](int tt) {
+            const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) Db[tt >> 1][(tt & 1) * 4 + r] = from_f32<T>(to_f32(vv[tt][r]) - eg[r] * ks[tt][r]);
+        };
+        f32x4 vn[4], oacc[4];
+        auto TXa = [&](int tt) {
+            vn[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) vn[tt] = Mma<T>::run(ax[tt][sp2], Db[sp2], vn[tt]);
+        };
+        auto TXb = [&](int tt) {
+            const f32x4 dec = *(const f32x4*)(sTab + TAB_DEC + 16 * tt + 4 * g) * vscale;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                Vn[tt >> 1][(tt & 1) * 4 + r] = from_f32<T>(vn[tt][r]);
+                Vg[tt >> 1][(tt & 1) * 4 + r] = from_f32<T>(vn[tt][r] * dec[r]);
+            }
+        };
+        auto TPa = [&](int tt) {
+            const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
+            oacc[tt] = ao[tt] * gam;
+#pragma unroll
+            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) oacc[tt] = Mma<T>::run(Vn[sp2], ap[tt][sp2], oacc[tt]);
+        };
+        auto TPb = [&](int tt) {
+            V4 o4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(oacc[tt][r]);
+            *(V4*)(otile + (16 * tt + c16) * W2_OT_PITCH + (16 * w + 4 * g) * 2) = o4;
+        };
+        auto U = [&](int u) { S[u & 15] = Mma<T>::run(kt[u & 7], Vg[u >> 4], S[u & 15]); };
+
+#pragma unroll
+        for (int f = 0; f < RING - 1; ++f) F(f);
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                Sb[s][r] = from_f32<T>(S[2 * s][r]);
+                Sb[s][4 + r] = from_f32<T>(S[2 * s + 1][r]);
+            }
+        gamma = fast_exp2(lg);
+        const float lg_try = lg + sTab[TAB_GLAST];
+        const bool lazy = lg_try >= LG_MIN;
+        vscale = lazy ? fast_exp2(-lg_try) : 1.f;
+        fence();
+        // ---- 32 regions: the products of fragment f and the fetch of fragment f + 2; beside them the fetches of
+        // v and Xb, then the tail of t-tiles 0, 1 while tiles 2, 3 are multiplied ----
+#pragma unroll
+        for (int f = 0; f < 32; ++f) {
+            if (f + RING - 1 < 32) F(f + RING - 1);
+            M(f);
+            if (f == 8) FV(0);
+            if (f == 9) FV(1);
+            if (f == 10) FX(0);
+            if (f == 11) FX(1);
+            if (f == 16) TD(0);
+            if (f == 17) TD(1);
+            if (f == 18) { TXa(0); TXa(1); }
+            if (f == 19) {
+                while (*pcount < p_target) __builtin_amdgcn_s_sleep(1);      // P of this chunk (normally long there)
+                FP(0); FP(1);
+                TXb(0); TXb(1); FV(2);
+            }
+            if (f == 20) { TPa(0); TPa(1); FV(3); }
+            if (f == 21) { TPb(0); TPb(1); FX(2); }
+            if (f == 22) FX(3);
+            if (f == 24) { FP(2); FP(3); }
+            if (f >= 29) { FK(2 * (f - 29)); FK(2 * (f - 29) + 1); }          // u = 0 .. 5
+            fence();
+        }
+        if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
+            const float fold = fast_exp2(lg_try);
+#pragma unroll
+            for (int m = 0; m < 16; ++m) S[m] *= fold;
+        }
+        lg = lazy ? lg_try : 0.f;
+        // ---- state update from t-tiles 0, 1 (16 products) beside the tail of tiles 2, 3; the k^T operands are fetched
+        // six products ahead ----
+#pragma unroll
+        for (int r8 = 0; r8 < 8; ++r8) {
+            U(2 * r8); U(2 * r8 + 1);
+            FK(2 * r8 + 6); FK(2 * r8 + 7);
+            if (r8 == 0) TD(2);
+            if (r8 == 1) TD(3);
+            if (r8 == 2) { TXa(2); TXa(3); }
+            if (r8 == 3) { TXb(2); TXb(3); }
+            if (r8 == 4) { TPa(2); TPa(3); }
+            if (r8 == 5) { TPb(2); TPb(3); }
+            fence();
+        }
+        lds_barrier();                                          // B1: q, v, the record and P are free, the output tile is complete
+        // ---- state update from t-tiles 2, 3 ----
+#pragma unroll
+        for (int r8 = 0; r8 < 8; ++r8) {
+            U(16 + 2 * r8); U(16 + 2 * r8 + 1);
+            if (r8 < 5) { FK(16 + 2 * r8 + 6); FK(16 + 2 * r8 + 7); }
+            fence();
+        }
+        lds_barrier();                                          // B2: k of this stage is free, the next chunk is complete
+    };
+    if (nsteps > 0) {
+        lds_barrier();                                          // B0
+        for (int64_t i = 0; i < nsteps; ++i)
+            step(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_V + (int)(i & 1) * 16384, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES,
+                 4 * ((int)i + 1));
+    }
+
+    if (dst) {
+        const float gamma = fast_exp2(lg);
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
+            const f32x4 s = S[m] * gamma;
+            if (kk < K && vc < V) {
+                float* e = dst + (int64_t)kk * sk + (int64_t)vc * sv;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) e[r * sk] = s[r];
+            }
+        }
+    }
+}
+
+template <typename T>
+int launch_wide256(const ChunkParams& p, hipStream_t stream) {
+    auto kern = gdn_chunk_wide256_kernel<T>;
+    static SmemAttrDone attr_done;       // per instantiation
+    if (int rc = ensure_dynamic_smem((const void*)kern, W2_SMEM, attr_done, "hipFuncSetAttribute(wide256)")) return rc;
+    const int NVB = (p.V + W2_VB - 1) / W2_VB;
+    const int64_t blocks = (p.N * p.H + 7) / 8 * 8 * (p.HV / p.H) * NVB;
+    if (blocks >= (1ll << 31)) { set_error("gdn_chunk_fwd: too many workgroups for one launch"); return GDN_ERR_UNSUPPORTED; }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(W2_THREADS), W2_SMEM, stream, p, NVB);
+    return check_launch("gdn_chunk_wide256_kernel");
+}
+
+template int launch_wide256<bf16_t>(const ChunkParams&, hipStream_t);
+template int launch_wide256<f16_t>(const ChunkParams&, hipStream_t);
+
+}  // namespace gdn

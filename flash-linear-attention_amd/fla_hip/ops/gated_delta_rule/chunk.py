@@ -40,7 +40,6 @@ for _form in ('wide', 'segments'):
         _SCAN_MODE_FLAGS[f'{_form}-{_runs}'] = _SCAN_MODE_FLAGS[_form] | _SCAN_MODE_FLAGS[_runs]
         if _form == 'segments':
             _SCAN_MODE_FLAGS[f'segments-exact-{_runs}'] = _SCAN_MODE_FLAGS['segments-exact'] | _SCAN_MODE_FLAGS[_runs]
-_WARNED_WIDE_KEYS = False
 _KERNEL_DIMS = (128,)           # head dim the MFMA kernels are instantiated for (smaller dims are zero-padded)
 
 
@@ -48,13 +47,6 @@ def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
     if x.shape[-1] == size:
         return x
     return torch.nn.functional.pad(x, (0, size - x.shape[-1]))
-
-
-def _kernel_dim(d: int) -> int:
-    for s in _KERNEL_DIMS:
-        if d <= s:
-            return s
-    raise NotImplementedError(f'head dim {d} > {_KERNEL_DIMS[-1]} is not supported by the HIP chunk kernels')
 
 
 class ChunkLaunch:
@@ -79,14 +71,10 @@ class ChunkLaunch:
         # the MFMA kernels take bf16 or fp16 operands; fp32 inputs are rounded to bf16 first
         work_dtype = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
         q, k, v = q.to(work_dtype), k.to(work_dtype), v.to(work_dtype)
-        # The kernels take head dims that are multiples of 8 up to 128 as they are.  Others are
-        # zero-padded to 128 here: zero key features and zero value columns change neither the
+        # The kernels take head dims that are multiples of 8 as they are.  Others are zero-padded
+        # to the next one here: zero key features and zero value columns change neither the
         # other columns of the output nor the state entries that are kept.
-        KP, VP = _kernel_dim(K), _kernel_dim(V)
-        if K % 8 == 0 and V % 8 == 0:
-            KP, VP = K, V
-        else:
-            KP = VP = max(KP, VP)
+        KP, VP = (K + 7) // 8 * 8, (V + 7) // 8 * 8
         self.padded = (KP, VP)
         q, k, v = _pad_last(q, KP), _pad_last(k, KP), _pad_last(v, VP)
         g, beta, gb_code = unify_gate_beta(g, beta)
@@ -196,23 +184,8 @@ def chunk_gated_delta_rule_fwd(
     Returns ``(o in q's dtype, final_state fp32 or None)``."""
     K, V = k.shape[-1], v.shape[-1]
     assert K <= 256, 'current kernel does not support head dimension larger than 256.'     # (chunk_delta_h.py:712)
-    if K > _KERNEL_DIMS[-1]:
-        # The chunk kernels hold a [K <= 128, 128] state per workgroup.  Wider keys take the token
-        # recurrence instead (same operator, same HIP library, state [K <= 256, V] in registers):
-        # correct for every shape the reference accepts, without the chunk path's throughput.
-        from fla_hip.ops.gated_delta_rule.fused_recurrent import fused_recurrent_gated_delta_rule_fwd
-        global _WARNED_WIDE_KEYS
-        if not _WARNED_WIDE_KEYS and q.shape[1] > 4 * _KERNEL_CHUNK:
-            _WARNED_WIDE_KEYS = True
-            warnings.warn(f'fla_hip: chunk_gated_delta_rule with K={K} > {_KERNEL_DIMS[-1]} runs the token recurrence '
-                          f'(one dependent step per token, no matrix cores); long prompts will be slow.', stacklevel=3)
-        o, ht = fused_recurrent_gated_delta_rule_fwd(
-            q, k, v, g=g, beta=beta, A_log=A_log, dt_bias=dt_bias, scale=scale, initial_state=initial_state,
-            output_final_state=output_final_state, use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel,
-            use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel, allow_neg_eigval=allow_neg_eigval,
-            state_v_first=state_v_first, cu_seqlens=cu_seqlens)
-        return o.to(q.dtype), ht
-    nb = (V + _KERNEL_DIMS[-1] - 1) // _KERNEL_DIMS[-1]
+    # Wide keys (128 < K <= 256) have a scan kernel of their own that takes any number of value columns, 64 per workgroup.
+    nb = (V + _KERNEL_DIMS[-1] - 1) // _KERNEL_DIMS[-1] if K <= _KERNEL_DIMS[-1] else 1
     if nb > 1:
         # The value columns of the recurrence are independent: a head with V > 128 is nb heads of 128
         # columns that share the head's k, q, gate and beta (grouped value heads do exactly that).

@@ -44,9 +44,8 @@ def make_backends(BaseBackend):
                 return False, 'forward only: a tensor requires grad'
             if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
                 return False, f'dtype {q.dtype}'
-            if k.shape[-1] > 128:
-                # wider keys would run this package's token recurrence: upstream's chunk kernels are the better choice
-                return False, 'key head dim above 128 has no chunk kernel here'
+            if k.shape[-1] > 256:
+                return False, 'key head dim above 256'           # (upstream asserts the same: chunk_delta_h.py:712)
             return True, None
 
         def chunk_gated_delta_rule(self, *args, **kwargs):

@@ -346,12 +346,12 @@ def test_two_runs_per_workgroup(monkeypatch, mode, B, T, H, HV, dtype, gate_div)
     (2, 300, 2, 2, 128, 256, False, None),      # wide values: split into two 128-column heads
     (1, 500, 2, 4, 64, 200, True, None),        # ... padded, V-first state layout
     (1, 700, 1, 2, 100, 384, False, [0, 130, 131, 700]),
-    (2, 150, 2, 2, 256, 128, False, None),      # wide keys: the token recurrence takes over
+    (2, 150, 2, 2, 256, 128, False, None),      # wide keys: the scan kernel with 64 value columns per workgroup
     (1, 200, 1, 2, 192, 192, True, [0, 77, 200]),
 ])
 def test_head_dims_above_128(B, T, H, HV, K, V, vfirst, cu):
-    """Every shape the reference accepts (K <= 256, any V) gives the right answer through the chunk entry
-    point, also where the chunk kernels themselves do not apply (fla/ops/common/chunk_delta_h.py:712)."""
+    """Every shape the reference accepts (K <= 256, any V: fla/ops/common/chunk_delta_h.py:712) gives the right answer
+    through the chunk entry point."""
     N = B if cu is None else len(cu) - 1
     q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=31, gate_div=8.0, h0_std=0.5, N=N, dtype=torch.bfloat16)
     ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu)

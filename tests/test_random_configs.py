@@ -75,10 +75,17 @@ def _compare(c, ref, got, tol):
         assert err <= tol and m <= 2 * tol, f'{name}: rel-rmse {err:.2e} max-abs {m:.2e} for {c}'
 
 
-@pytest.mark.parametrize('seed', range(48))
+@pytest.mark.parametrize('seed', list(range(48)) + [f'wide{i}' for i in range(24)])
 def test_chunk_random_configuration(seed, monkeypatch):
     from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
-    c = _case(seed, recurrent=False)
+    if isinstance(seed, str):
+        # the same combinations with wide keys (128 < K <= 256) and any number of value columns
+        seed = 500 + int(seed[4:])
+        c = _case(seed, recurrent=False)
+        rnd = random.Random(seed + 7)
+        c['K'], c['V'] = rnd.choice([136, 160, 192, 250, 256]), rnd.choice([16, 64, 72, 128, 200, 320])
+    else:
+        c = _case(seed, recurrent=False)
     if c['mode'] != 'auto':
         monkeypatch.setenv('FLA_HIP_SCAN_MODE', c['mode'])
     q, k, v, g, beta, A_log, dt_bias, h0 = _inputs(c, 1000 + seed)
