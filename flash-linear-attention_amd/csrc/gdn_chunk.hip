@@ -27,7 +27,9 @@ static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, h
     const int64_t G = p.HV / p.H;
     const int nseg = plan_segments(p.N, p.HV, p.NT, num_chunks, p.cu_seqlens == nullptr, p.flags);
     const bool segments = nseg > 0;
-    const bool no_pair = p.flags & GDN_FLAG_SCAN_NO_PAIR, force_pair = p.flags & GDN_FLAG_SCAN_PAIR;
+    // (head dims up to 64 have a one-run kernel with a quarter-size state; the two-run kernel would do the full 128 x 128 work)
+    const bool small = p.K <= 64 && p.V <= 64;
+    const bool no_pair = (p.flags & GDN_FLAG_SCAN_NO_PAIR) || small, force_pair = (p.flags & GDN_FLAG_SCAN_PAIR) && !small;
     // (full runs in pairs: an even number of value heads per q/k head, and all 128 value columns real: the two-run
     // kernel counts its output stores, which every wave must therefore have)
     const bool pair_full_ok = G % 2 == 0 && p.V == 128;

@@ -116,12 +116,14 @@ inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 // Number of time segments the sequential stage cuts every sequence into (0: whole sequences, one
 // workgroup per sequence and head).  With few (sequence, head) runs and long dense sequences, time is
 // cut so that every CU has a workgroup: two passes over 1/nseg of the chunks each plus a small merge,
-// which must beat one pass over all chunks (nseg >= 3).  Shared by the workspace size and the launch.
+// which must beat one pass over all chunks (nseg >= 3, and segments of 8 chunks or more: every pass also pays for filling
+// and draining its pipeline and for a launch).  Shared by the workspace size and the launch.
 inline int plan_segments(int64_t N, int64_t HV, int64_t NT, int64_t num_chunks, bool dense, uint32_t flags) {
     const int64_t NH = N * HV;
     int nseg = 0;
     if (dense && NH > 0) {
-        nseg = (int)std::min<int64_t>((256 + NH / 2) / NH, NT / 4);
+        // (GDN_FLAG_SCAN_SEGMENTS asks for segments wherever they are possible at all: segments of 4 chunks)
+        nseg = (int)std::min<int64_t>((256 + NH / 2) / NH, NT / ((flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
         while (nseg > 0 && ((int64_t)nseg * NH > SEG_SLOTS_MAX || (int64_t)nseg * NH > (num_chunks * HV + 3) / 4)) --nseg;
     }
     bool segments = nseg >= 3;

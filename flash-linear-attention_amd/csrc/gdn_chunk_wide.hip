@@ -58,11 +58,15 @@ constexpr int WIDE_NN = 2;                        // 16-column tiles per compute
 constexpr int CW = 8 / WIDE_NN;                   // compute waves
 constexpr int WIDE_THREADS = (CW + 4) * 64;
 
-template <typename T, bool FULL, bool DIMS128>
+template <typename T, bool FULL, bool DIMS128, bool SMALL>
 __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParams p, SegmentPlan sp) {
     // Head dims: DIMS128 fixes K = V = 128 at compile time (every copy is whole, nothing is masked); otherwise they
     // are the caller's multiples of 8 and the tiles' features past them are zero (q, k) or never stored (v, o, state).
+    // SMALL (K, V <= 64, e.g. the reference's D = 64 shapes): a quarter of the state - 64 key rows, 16 value columns
+    // per compute wave - with the LDS layout unchanged, so that nothing is multiplied by the zero features.
+    static_assert(!(DIMS128 && SMALL), "one or the other");
     const int K = DIMS128 ? 128 : p.K, V = DIMS128 ? 128 : p.V;
+    constexpr int KS = SMALL ? 2 : 4;                 // pairs of 16-row key tiles (32 key features each)
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
@@ -198,9 +202,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 const float* t2 = (const float*)(st + STG_TAB2);
                 const int a_off = (c16 >> 2) * 64 + 4 * (c16 & 3) + ((g + (c16 >> 2)) & 3);
                 auto frag = [&](int tt, int sp) {
-                    V8 qb[4];
+                    V8 qb[KS];
 #pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4) qb[s4] = sQ[tt * 256 + 16 * s4 + a_off];
+                    for (int s4 = 0; s4 < KS; ++s4) qb[s4] = sQ[tt * 256 + 16 * s4 + a_off];
                     const int t = 16 * tt + c16;
                     const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
                     V8 out;
@@ -214,7 +218,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                         }
                         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int s4 = 0; s4 < 4; ++s4) acc = Mma<T>::run(sK[tj * 256 + 16 * s4 + a_off], qb[s4], acc);
+                        for (int s4 = 0; s4 < KS; ++s4) acc = Mma<T>::run(sK[tj * 256 + 16 * s4 + a_off], qb[s4], acc);
                         const f32x4 gj = *(const f32x4*)(t2 + TAB2_G + 16 * tj + 4 * g), nj = *(const f32x4*)(t2 + TAB2_NK + 16 * tj + 4 * g);
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
@@ -390,10 +394,10 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     // Compute waves
     // =====================================================================================
     // ---- state: all key rows (permuted, see above), value columns 16w .. 16w+15, C/D layout ----
-    constexpr int NN = WIDE_NN;
-    f32x4 S[8][NN];
+    constexpr int NN = SMALL ? 1 : WIDE_NN;           // 16-column tiles per compute wave
+    f32x4 S[2 * KS][NN];
 #pragma unroll
-    for (int m = 0; m < 8; ++m)
+    for (int m = 0; m < 2 * KS; ++m)
 #pragma unroll
     for (int nn = 0; nn < NN; ++nn) {
         const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * (NN * w + nn) + c16;
@@ -455,13 +459,13 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         constexpr int RING = WIDE_RING;
         V8 ak[RING], aq[RING];
         auto F = [&](int f) {
-            ak[f % RING] = sK[(f >> 2) * 256 + 16 * (f & 3) + a_off];
-            if constexpr (FULL) aq[f % RING] = sQ[(f >> 2) * 256 + 16 * (f & 3) + a_off];
+            ak[f % RING] = sK[(f / KS) * 256 + 16 * (f % KS) + a_off];
+            if constexpr (FULL) aq[f % RING] = sQ[(f / KS) * 256 + 16 * (f % KS) + a_off];
         };
         f32x4 ks[4][NN], ao[4][NN];
-        V8 Sb[4][NN];
+        V8 Sb[KS][NN];
         auto M = [&](int f) {                   // (k S) and (q S)^T contributions of fragment f
-            const int tt = f >> 2, sx = f & 3;
+            const int tt = f / KS, sx = f % KS;
 #pragma unroll
             for (int nn = 0; nn < NN; ++nn) {
                 ks[tt][nn] = Mma<T>::run(ak[f % RING], Sb[sx][nn], sx ? ks[tt][nn] : f32x4{0.f, 0.f, 0.f, 0.f});
@@ -484,7 +488,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
                 for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
             }
         };
-        V8 kt[2][8];                            // k^T rows of key tile m over t-tile pair sp2
+        V8 kt[2][2 * KS];                       // k^T rows of key tile m over t-tile pair sp2
         auto FK = [&](int sp2, int m) {
             const T* a = sKt + sp2 * 4096 + 128 * (m >> 1) + 4 * (m & 1) + k_tr;
             kt[sp2][m] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 2048));
@@ -554,7 +558,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
 #pragma unroll
         for (int f = 0; f < RING - 1; ++f) F(f);
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int s = 0; s < KS; ++s)
 #pragma unroll
             for (int nn = 0; nn < NN; ++nn)
 #pragma unroll
@@ -567,54 +571,82 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
         const bool lazy = lg_try >= LG_MIN;
         vscale = lazy ? fast_exp2(-lg_try) : 1.f;
         fence();
-        // ---- sixteen regions: the products of fragment f, the fetch of fragment f + RING - 1, and beside them
-        // the other fetches (t-tiles 0, 1) and then the tail of tiles 0, 1 while tiles 2, 3 are multiplied ----
+        auto wait_P = [&]() {
+            // P of this chunk: normally long there (the copy waves form it first thing in a step, at raised priority)
+            if constexpr (FULL) { while (*pcount < p_target) __builtin_amdgcn_s_sleep(1); }
+        };
+        auto fold = [&]() {                     // the decay fold: rare, a scalar branch so that it is not if-converted into the common path
+            if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
+                const float fo = fast_exp2(lg_try);
 #pragma unroll
-        for (int f = 0; f < 16; ++f) {
-            if (f + RING - 1 < 16) F(f + RING - 1);
-            M(f);
-            if (f == 4) FV(0);
-            if (f == 5) FV(1);
-            if (f == 6) FX(0);
-            if (f == 7) FX(1);
-            if (f == 8) TD(0);
-            if (f == 9) { TD(1); }
-            if (f == 10) { TXa(0); TXa(1); }
-            if (f == 11) {
-                // P of this chunk: normally long there (the copy waves form it first thing in a step, at raised priority)
-                if constexpr (FULL) { while (*pcount < p_target) __builtin_amdgcn_s_sleep(1); }
-                FP(0); FP(1);
+                for (int m = 0; m < 2 * KS; ++m)
+#pragma unroll
+                    for (int nn = 0; nn < NN; ++nn) S[m][nn] *= fo;
             }
-            if (f == 11) { TXb(0); TXb(1); FV(2); }
-            if (f == 12) { TPa(0); TPa(1); FV(3); }
-            if (f == 13) { TPb(0); TPb(1); FX(2); }
-            if (f == 14) { FX(3); FK(0, 0); FK(0, 1); }
-            if (f == 15) { FK(0, 2); FK(0, 3); }
+            lg = lazy ? lg_try : 0.f;
+        };
+        if constexpr (SMALL) {
+            // ---- eight fragments (two per t-tile), four state tiles per wave.  The chain that the next step waits for
+            // is M(7) -> D, v_new of t-tiles 2, 3 -> their state update; the tail of tiles 0, 1 and everything of the
+            // output fill its gaps ----
+            F(2); M(0); FV(0); FV(1); fence();
+            F(3); M(1); FX(0); FX(1); fence();
+            F(4); M(2); FV(2); FV(3); fence();
+            F(5); M(3); FX(2); FX(3); fence();
+            F(6); M(4); TD(0); TD(1); FK(0, 0); FK(0, 1); fence();
+            F(7); M(5); TXa(0); TXa(1); FK(0, 2); FK(0, 3); fence();
+            M(6); TXb(0); TXb(1); FK(1, 0); FK(1, 1); fence();
+            M(7); FK(1, 2); FK(1, 3); fence();
+            fold();
+            TD(2); TD(3); U(0, 0); U(0, 1); U(0, 2); U(0, 3); fence();
+            TXa(2); TXa(3); wait_P(); FP(0); FP(1); FP(2); FP(3); fence();
+            TXb(2); TXb(3); TPa(0); TPa(1); fence();
+            U(1, 0); U(1, 1); TPb(0); TPb(1); TPa(2); TPa(3); fence();
+            TPb(2); TPb(3); fence();
+            lds_barrier();                                          // B1
+            U(1, 2); U(1, 3); fence();
+            lds_barrier();                                          // B2
+        } else {
+            // ---- sixteen regions: the products of fragment f, the fetch of fragment f + RING - 1, and beside them
+            // the other fetches (t-tiles 0, 1) and then the tail of tiles 0, 1 while tiles 2, 3 are multiplied ----
+    #pragma unroll
+            for (int f = 0; f < 16; ++f) {
+                if (f + RING - 1 < 16) F(f + RING - 1);
+                M(f);
+                if (f == 4) FV(0);
+                if (f == 5) FV(1);
+                if (f == 6) FX(0);
+                if (f == 7) FX(1);
+                if (f == 8) TD(0);
+                if (f == 9) { TD(1); }
+                if (f == 10) { TXa(0); TXa(1); }
+                if (f == 11) {
+                    wait_P();
+                    FP(0); FP(1);
+                }
+                if (f == 11) { TXb(0); TXb(1); FV(2); }
+                if (f == 12) { TPa(0); TPa(1); FV(3); }
+                if (f == 13) { TPb(0); TPb(1); FX(2); }
+                if (f == 14) { FX(3); FK(0, 0); FK(0, 1); }
+                if (f == 15) { FK(0, 2); FK(0, 3); }
+                fence();
+            }
+            fold();
+            // ---- state update from tiles 0, 1, with the tail of tiles 2, 3 ----
+            U(0, 0); U(0, 1); TD(2); FK(0, 4); FK(0, 5); fence();
+            U(0, 2); U(0, 3); TD(3); FK(0, 6); FK(0, 7); FP(2); fence();
+            U(0, 4); U(0, 5); TXa(2); TXa(3); FK(1, 0); FK(1, 1); FP(3); fence();
+            U(0, 6); U(0, 7); TXb(2); TXb(3); FK(1, 2); FK(1, 3); fence();
+            // ... and the first half of the update from tiles 2, 3
+            U(1, 0); U(1, 1); TPa(2); TPa(3); FK(1, 4); FK(1, 5); fence();
+            U(1, 2); U(1, 3); TPb(2); TPb(3); FK(1, 6); FK(1, 7); fence();
+            lds_barrier();                                          // B1: q, v, record of this stage are free
+            // ---- rest of the state update from tiles 2, 3 ----
+    #pragma unroll
+            for (int m = 4; m < 8; ++m) U(1, m);
             fence();
+            lds_barrier();                                          // B2: k of this stage is free, the other stage is complete
         }
-        // the decay fold: rare, a scalar branch so that it is not if-converted into the common path
-        if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
-            const float fold = fast_exp2(lg_try);
-#pragma unroll
-            for (int m = 0; m < 8; ++m)
-#pragma unroll
-                for (int nn = 0; nn < NN; ++nn) S[m][nn] *= fold;
-        }
-        lg = lazy ? lg_try : 0.f;
-        // ---- state update from tiles 0, 1, with the tail of tiles 2, 3 ----
-        U(0, 0); U(0, 1); TD(2); FK(0, 4); FK(0, 5); fence();
-        U(0, 2); U(0, 3); TD(3); FK(0, 6); FK(0, 7); FP(2); fence();
-        U(0, 4); U(0, 5); TXa(2); TXa(3); FK(1, 0); FK(1, 1); FP(3); fence();
-        U(0, 6); U(0, 7); TXb(2); TXb(3); FK(1, 2); FK(1, 3); fence();
-        // ... and the first half of the update from tiles 2, 3
-        U(1, 0); U(1, 1); TPa(2); TPa(3); FK(1, 4); FK(1, 5); fence();
-        U(1, 2); U(1, 3); TPb(2); TPb(3); FK(1, 6); FK(1, 7); fence();
-        lds_barrier();                                          // B1: q, v, record of this stage are free
-        // ---- rest of the state update from tiles 2, 3 ----
-#pragma unroll
-        for (int m = 4; m < 8; ++m) U(1, m);
-        fence();
-        lds_barrier();                                          // B2: k of this stage is free, the other stage is complete
     };
     if (nsteps > 0) {
         lds_barrier();                                          // B0: the copy waves have filled stage 0
@@ -624,9 +656,18 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     }
 
     if (dst) {
+        if constexpr (SMALL) {
+            // the buffers of the segment passes are [128][128] and the merge reads all of them: zero what this state leaves out
+            if (!dst_user) {
+                for (int i = tid; i < 4096; i += CW * 64) {
+                    const int row = i >> 5, c4 = (i & 31) * 4;
+                    if (row >= 64 || c4 >= 64) *(f32x4*)(dst + row * 128 + c4) = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
         const float gamma = fast_exp2(lg);
 #pragma unroll
-        for (int m = 0; m < 8; ++m)
+        for (int m = 0; m < 2 * KS; ++m)
 #pragma unroll
         for (int nn = 0; nn < NN; ++nn) {
             const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1), vc = 16 * (NN * w + nn) + c16;
@@ -721,9 +762,9 @@ __global__ __launch_bounds__(256) void gdn_segment_merge_kernel(SegmentPlan sp, 
     }
 }
 
-template <typename T, bool FULL, bool DIMS128>
+template <typename T, bool FULL, bool DIMS128, bool SMALL>
 static int launch_wide_dims(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
-    auto kern = gdn_chunk_wide_kernel<T, FULL, DIMS128>;
+    auto kern = gdn_chunk_wide_kernel<T, FULL, DIMS128, SMALL>;
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, WIDE_SMEM, attr_done, "hipFuncSetAttribute(wide)")) return rc;
     if (blocks <= 0) return GDN_OK;
@@ -733,8 +774,9 @@ static int launch_wide_dims(const ChunkParams& p, const SegmentPlan& sp, int64_t
 
 template <typename T, bool FULL>
 static int launch_wide_kind(const ChunkParams& p, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
-    return p.K == 128 && p.V == 128 ? launch_wide_dims<T, FULL, true>(p, sp, blocks, stream)
-                                    : launch_wide_dims<T, FULL, false>(p, sp, blocks, stream);
+    if (p.K == 128 && p.V == 128) return launch_wide_dims<T, FULL, true, false>(p, sp, blocks, stream);
+    if (p.K <= 64 && p.V <= 64) return launch_wide_dims<T, FULL, false, true>(p, sp, blocks, stream);
+    return launch_wide_dims<T, FULL, false, false>(p, sp, blocks, stream);
 }
 
 // sp.kind selects the work (whole sequences, pass 1 or pass 2 of the segment-parallel evaluation)
