@@ -380,25 +380,38 @@ def calib_copy(steps, warmup, device):
 
 def calib_rmw(steps, warmup, device):
     """The decode step's traffic without its arithmetic: every fp32 element of two alternating 512 MiB pools (the size
-    of the B = 256 decode states) read, changed and written back in place by torch's elementwise kernel.  What this
-    reaches is what a read-modify-write stream of that size reaches on the machine."""
+    of the B = 256 decode states) read, changed and written back in place - by torch's elementwise kernel (the headline
+    of this workload), and by the library's calibration kernel gdn_calib_rmw, which has the decode step's shape (64 KB
+    per workgroup, a workgroup-wide reduction between the reads and the writes) with the placement of the workgroups as
+    parameters.  What these reach is what a read-modify-write stream of that size reaches on the machine."""
+    from fla_hip import _lib
+    lib = _lib.load()
     n = 256 * 32 * 128 * 128
     pools = [torch.zeros(n, dtype=torch.float32, device=device) for _ in range(2)]
-    spin_up(lambda i: pools[i & 1].add_(1.0))
-    for i in range(warmup):
-        pools[i & 1].add_(1.0)
-    torch.cuda.synchronize()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    ev[0].record()
-    for i in range(steps):
-        pools[i & 1].add_(1.0)
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    ts = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e-3 for i in range(steps))
-    t = statistics.mean(ts)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn):
+        spin_up(fn)
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        ev[0].record()
+        for i in range(steps):
+            fn(i)
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ts = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e-3 for i in range(steps))
+        return statistics.mean(ts), ts[len(ts) // 2]
+
+    t, tm = timed(lambda i: pools[i & 1].add_(1.0))
+    shapes = {}
+    for run, per_cu in ((0, 0), (32, 0), (32, 1), (32, 2), (32, 3), (1024, 0), (1024, 2)):
+        ts, _ = timed(lambda i: _lib.check(lib.gdn_calib_rmw(pools[i & 1].data_ptr(), n, run, per_cu, stream)))
+        shapes[f'xcd_run={run},workgroups_per_cu={per_cu}'] = dict(us_per_pass=round(ts * 1e6, 1), GBps=round(2 * n * 4 / ts / 1e9, 1))
     print(json.dumps(dict(metric='calib_rmw_GBps', value=round(2 * n * 4 / t / 1e9, 1), unit='GB/s', us_per_pass=round(t * 1e6, 1),
-                          us_median=round(ts[len(ts) // 2] * 1e6, 1), bytes_read=n * 4, bytes_written=n * 4, steps=steps, warmup=warmup,
-                          frac_of_peak=round(2 * n * 4 / t / 1e9 / PEAK_HBM_GBS, 4))))
+                          us_median=round(tm * 1e6, 1), bytes_read=n * 4, bytes_written=n * 4, steps=steps, warmup=warmup,
+                          frac_of_peak=round(2 * n * 4 / t / 1e9 / PEAK_HBM_GBS, 4), gdn_calib_rmw=shapes)))
 
 
 def main():

@@ -255,6 +255,15 @@ int gdn_norm_gated_fwd(
     int64_t T, int64_t D, float eps,
     int x_dtype, int w_dtype, int res_dtype, int res_out_dtype, int activation, int is_rms_norm, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference (bench.py --workload calib_rmw): the memory traffic and the
+ * dependency of a decode step without its arithmetic.  Every 64 KB block of `data` (n_floats a multiple of 16384)
+ * is read, reduced across its workgroup and written back in place.  xcd_run > 0: every XCD works on runs of that
+ * many consecutive blocks (0: block b on XCD b % 8); workgroups_per_cu 1..8 caps the workgroups that share a CU
+ * (0: no cap).  The decode kernel of gdn_fused_recurrent_fwd uses the shape (HV, 2).
+ */
+int gdn_calib_rmw(float* data, int64_t n_floats, int xcd_run, int workgroups_per_cu, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
