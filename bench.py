@@ -135,6 +135,8 @@ def spin_up(fn):
     per call falling to 0.48 ms over the first 60 calls of the default workload - and a handful of warm-up steps
     does not cover that.  The W warm-up steps and the K timed steps follow as usual."""
     torch.cuda.synchronize()
+    if SPIN_UP_MS <= 0:
+        return
     t0 = time.perf_counter()
     i = 0
     while (time.perf_counter() - t0) * 1e3 < SPIN_UP_MS:
@@ -422,7 +424,11 @@ def main():
     ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
+    ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
     args = ap.parse_args()
+    if args.no_spin_up:
+        global SPIN_UP_MS
+        SPIN_UP_MS = 0.0
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py: this build measures ONE GPU only (every sequence and v-head is independent, so more GPUs '
               'shard them with no communication); run it with --gpus 1.', file=sys.stderr)
