@@ -135,9 +135,11 @@ size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64
  *         which the sequential kernel should start them (longest first keeps the CUs evenly loaded)
  *   workspace: at least gdn_chunk_workspace_bytes(...) bytes, 256-byte aligned
  *   T == 0 (or no chunk at all): ht = h0 (zeros without h0), nothing else is written.
- *   Requires K, V multiples of 8 up to 128 and HV % H == 0.  The kernels work on 128 x 128 states: key features past K
- *   count as zero and value columns past V are not stored (same time as K = V = 128; the Python host zero-pads
- *   head dims that are not multiples of 8).
+ *   Requires HV % H == 0 and K, V multiples of 8: both up to 128, or 128 < K <= 256 (the reference's limit,
+ *   fla/ops/common/chunk_delta_h.py:712) with V up to 8192.  State shapes of the kernels: 128 x 128 (key features
+ *   past K count as zero, value columns past V are not stored), 64 x 64 for K, V <= 64, and 256 x 64-column blocks
+ *   for wide keys; the Python host zero-pads head dims that are not multiples of 8 and splits V > 128 with K <= 128
+ *   into value heads of 128 columns.
  */
 int gdn_chunk_fwd(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
