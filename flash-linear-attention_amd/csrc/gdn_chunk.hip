@@ -10,7 +10,6 @@ constexpr int STAGE_PREPARE = 1, STAGE_SCAN = 2;
 template <typename T>
 static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, hipStream_t stream) {
     ChunkParams p = p0;
-    // The plan of the sequential stage first: the prepare kernel writes P only for the kernel that reads it.
     // One workgroup per (sequence, head) walks the chunks of the sequence, or time is cut into
     // segments (plan_segments).  Either way a workgroup can also carry two runs that read the same k rows (two value heads of
     // a q/k head; in pass 1 the S and M runs of one head).  That halves the number of workgroups and
@@ -18,7 +17,7 @@ static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, h
     // as the single runs would not all fit on the chip at once.
     if (p.K > 128) {
         // wide keys: whole sequences, a workgroup per 64 value columns; the scan forms P itself
-        p.want_P = 0;
+        p.want_P = (p.flags & GDN_FLAG_RECORD_P) != 0;
         if (stages & STAGE_PREPARE) {
             if (int rc = launch_prepare<T>(p, num_chunks, stream)) return rc;
         }
@@ -38,7 +37,7 @@ static int launch_chunk(const ChunkParams& p0, int64_t num_chunks, int stages, h
     };
     const bool pass2_pairs = segments && use_pair(pair_full_ok, p.NH * nseg);
     const bool whole_pairs = !segments && use_pair(pair_full_ok, p.NH);
-    p.want_P = pass2_pairs || whole_pairs;
+    p.want_P = (p.flags & GDN_FLAG_RECORD_P) != 0;       // every scan kernel forms P itself
     if (stages & STAGE_PREPARE) {
         int rc = launch_prepare<T>(p, num_chunks, stream);
         if (rc) return rc;

@@ -61,8 +61,9 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // lower triangular: the fragments (tt, sp) = (0,1), (1,1) are identically zero and are not
 // stored, and of (0,0), (2,1) only the first half (4 values per lane) is.
 //   Xb   T    5 KB        (I+L)^-1 diag(beta)
-//   P    T    5 KB        scale * tril(q k^T 2^(G_t-G_t')); written only for the scan kernel that reads it (two runs per
-//                         workgroup); the one-run kernel forms P itself from its q and k tiles and the second table
+//   P    T    5 KB        scale * tril(q k^T 2^(G_t-G_t')): room only.  Every scan kernel forms P itself, from its q and k
+//                         tiles and the second table, into this place of its LDS copy; the prepare kernel writes it to
+//                         memory on request (GDN_FLAG_RECORD_P), for callers that look at the records
 //   tab  fp32 [256]       [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units),
 //                         the first three times the row factors 1/|k_t|, 1/|q_t|, 1/|k_t| of the l2 normalisation
 //   tab2 fp32 [256]       [0..63] G_t (log2 units), [64..127] scale/|q_t|, [128..191] 1/|k_t|: what P needs
@@ -154,7 +155,7 @@ struct ChunkParams {
     int K, V;                                          // head dims of the caller's tensors (multiples of 8; K, V <= 128, or 128 < K <= 256 with any V)
     float scale; int gb_dtype; uint32_t flags;
     int64_t NH;
-    int want_P;                                        // the scan will read P from the records (two runs per workgroup)
+    int want_P;                                        // the prepare kernel also writes P (GDN_FLAG_RECORD_P)
 };
 
 // Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains

@@ -28,7 +28,8 @@ namespace gdn {
 // per wave (each half of the rows is fetched again as soon as the wave has consumed it).
 constexpr int PR_K = 0, PR_Q = 32768, PR_V = 65536, PR_REC = 98304;
 constexpr int PR_OT = PR_REC + 4 * (int)REC_BYTES;            // 8 x 1 KB: per wave, one 16-token tile of its output columns on its way out
-constexpr size_t PAIR_SMEM = PR_OT + 8 * 1024;                // 151 552 B
+constexpr int PR_PCOUNT = PR_OT + 8 * 1024;                   // per team: P fragments published so far
+constexpr size_t PAIR_SMEM = PR_PCOUNT + 16;                  // 151 568 B
 constexpr int PAIR_THREADS = 512;
 
 // One 16-byte store per lane at sbase + voff, for the lanes named by `mask` only.  Written in
@@ -136,6 +137,10 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     // =====================================================================================
     const bool vz = __builtin_amdgcn_readfirstlane((int)v_zero) != 0;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    // P = scale tril(q k^T 2^(G_t - G_t')) of a chunk is formed by the four waves of a team from the q and k tiles at the
+    // start of its step (see gdn_chunk_wide.hip); a counter per team in LDS tells when its fragments are complete.
+    volatile int* pcount = (volatile int*)(smem + PR_PCOUNT) + tm;
+    if (tid == 0) { ((volatile int*)(smem + PR_PCOUNT))[0] = 0; ((volatile int*)(smem + PR_PCOUNT))[1] = 0; }      // (published by the first barrier)
     // rows of the caller's tensors hold K (q, k) or V (v, o) elements, multiples of 8 up to 128.  Pieces of q and k
     // past K stay zero in LDS (the tiles are cleared once, those lanes copy nothing); pieces of v past V re-read
     // valid ones: value columns never mix, and the padded ones are never stored.
@@ -182,32 +187,32 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
             gather_1k_to_lds(base, __umul24(row, rowB_v) + v_cb, lds0 + PR_V + w * 4096 + b * 1024);
         }
     };
-    // The record of (chunk, value head), in 1 KB pieces.  A full run needs all 11, three per wave of the
-    // team.  A state-only run needs Xb and the tables (pieces 0..4 and 10), and its two teams work on the
-    // same value head: they share one copy (in the area of team 0), one piece per wave.
-    auto issue_rec = [&](int64_t c, int stage, int part) {                           // parts of 2 and 1 operations (state-only: 1 part of 1)
+    // The record of (chunk, value head), in 1 KB pieces.  A full run needs Xb and the two tables (pieces 0..4, 10, 11: P is
+    // formed here), two per wave of the team.  A state-only run needs Xb and the first table (pieces 0..4 and 10), and its two
+    // teams work on the same value head: they share one copy (in the area of team 0), one piece per wave.
+    auto issue_rec = [&](int64_t c, int stage) {                                     // 2 operations (state-only: 1)
         const char* rec = p.ws.Rec + ((boh + c) * HV + hv) * REC_BYTES;
         const uint32_t to = lds0 + PR_REC + ((FULL ? tm : 0) * 2 + stage) * (uint32_t)REC_BYTES;
         auto piece = [&](int j) { gather_1k_to_lds(rec + j * 1024, lane * 16, to + j * 1024); };
         if constexpr (FULL) {
-            if (part == 0) { piece(cw); piece(cw + 4); }
-            else piece(cw < 3 ? cw + 8 : cw);                                         // (wave 3 fetches a piece twice: equal counts)
+            piece(cw);                                                                // Xb 0..3
+            piece(cw == 0 ? REC_PIECES_X - 1 : cw == 1 ? REC_PIECE_TAB : cw == 2 ? REC_PIECE_TAB2 : 0);      // (wave 3 fetches piece 0 again: equal counts)
         } else {
-            if (part == 0) piece(w < REC_PIECES_X ? w : w == REC_PIECES_X ? REC_PIECE_TAB : 0);      // (waves 6, 7 fetch piece 0 again: equal counts)
+            piece(w < REC_PIECES_X ? w : w == REC_PIECES_X ? REC_PIECE_TAB : 0);      // (waves 6, 7 fetch piece 0 again: equal counts)
         }
     };
-    // everything a barrier publishes, 7 (3) operations, in four parts so that the waves do not all
+    // everything a barrier publishes, 6 (3) operations, in three parts so that the waves do not all
     // queue at the memory pipeline at once
     auto issue_shared = [&](int64_t c, int stage, int part) {
         if (part == 0) issue_kq((const T*)p.k, c, lds0 + PR_K + stage * 16384);
         if (part == 1) { if constexpr (FULL) issue_kq((const T*)p.q, c, lds0 + PR_Q + stage * 16384); }
-        if (part >= 2) issue_rec(c, stage, part - 2);
+        if (part == 2) issue_rec(c, stage);
     };
     // number of operations a wave issues between ...
-    // (per step, in order: shared 7 (3), in the first four regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
+    // (per step, in order: shared 6 (3), in the first three regions | v rows 0..31: 2 | output tiles 0, 1: 2 | v rows 32..63: 2 | output tiles 2, 3: 2)
     constexpr int N_AFTER_SHARED = FULL ? 8 : 4;      // the shared copies of a step and the barrier at its end
-    constexpr int N_AFTER_VLO = FULL ? 13 : 5;        // the first half of v and its use in the next step
-    constexpr int N_AFTER_VHI = FULL ? 11 : 5;        // the second half of v and its use in the next step
+    constexpr int N_AFTER_VLO = FULL ? 12 : 5;        // the first half of v and its use in the next step
+    constexpr int N_AFTER_VHI = FULL ? 10 : 5;        // the second half of v and its use in the next step
 
     if (K < 128 && nsteps > 0) {
         const u32x4 z = {0u, 0u, 0u, 0u};
@@ -217,12 +222,12 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     if (nsteps > 0 && !active) {
         // a team with nothing to compute still fetches its share of k and of the record
         issue_kq((const T*)p.k, it0, lds0 + PR_K);
-        issue_rec(it0, 0, 0);
+        issue_rec(it0, 0);
         wait_vm_at_most<0>();
         lds_barrier();
         for (int64_t i = 0; i < nsteps; ++i) {
             issue_kq((const T*)p.k, min(it0 + i + 1, lastc), lds0 + PR_K + (int)((i + 1) & 1) * 16384);
-            issue_rec(min(it0 + i + 1, lastc), (int)((i + 1) & 1), 0);
+            issue_rec(min(it0 + i + 1, lastc), (int)((i + 1) & 1));
             wait_vm_at_most<0>();
             lds_barrier();
         }
@@ -291,6 +296,47 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
         const int64_t nxt = min(it + 1, lastc);                 // (its buffers were released by the barrier that ended the previous step)
+
+        if constexpr (FULL) {
+            // ---- this wave's share of P (transposed product, so that a result is spread over the lanes like the operand
+            // fragment that is read back), gated with its team's tables ----
+            const float* t2 = (const float*)(rec + REC_TAB2);
+            auto frag = [&](int tt, int sp) {
+                V8 qb[4];
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4) qb[s4] = sQ[tt * 256 + 16 * s4 + a_off];
+                const int t = 16 * tt + c16;
+                const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                V8 out;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int tj = 2 * sp + half;
+                    if (tj > tt) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) out[half * 4 + r] = from_f32<T>(0.f);
+                        continue;
+                    }
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) acc = Mma<T>::run(sK[tj * 256 + 16 * s4 + a_off], qb[s4], acc);
+                    const f32x4 gj = *(const f32x4*)(t2 + TAB2_G + 16 * tj + 4 * g), nj = *(const f32x4*)(t2 + TAB2_NK + 16 * tj + 4 * g);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = 16 * tj + 4 * g + r;
+                        // select, never multiply by a mask: 2^(G_t - G_j) may overflow above the diagonal
+                        out[half * 4 + r] = from_f32<T>((t >= j) ? st_ * nj[r] * acc[r] * fast_exp2(gt - gj[r]) : 0.f);
+                    }
+                }
+                store_frag<T>((char*)rec + REC_P, tt, sp, lane, out);
+            };
+            if (cw == 0) frag(3, 0);
+            else if (cw == 1) frag(3, 1);
+            else if (cw == 2) { frag(2, 0); frag(0, 0); }
+            else { frag(1, 0); frag(2, 1); }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_fetch_add((int*)pcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            fence();
+        }
 
         constexpr int RING = 2;
         V8 ak[RING], aq[RING];
@@ -416,13 +462,16 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
         for (int f = 0; f < 16; ++f) {
             if (f + RING - 1 < 16) F(f + RING - 1);
             M(f);
-            if (f < 4) issue_shared(nxt, cur ^ 1, f);
+            if (f < 3) issue_shared(nxt, cur ^ 1, f);
             if (f == 4) { wait_vm_at_most<N_AFTER_VLO>(); FV(0); }
             if (f == 5) FV(1);
             if (f == 6) FX(0);
             if (f == 7) FX(1);
             if (f == 8) TD(0);
-            if (f == 9) { TD(1); FP(0); }
+            if (f == 9) {
+                if constexpr (FULL) { while (*pcount < 4 * ((int)i + 1)) __builtin_amdgcn_s_sleep(1); }       // the team's P (long there)
+                TD(1); FP(0);
+            }
             if (f == 10) { TXa(0); TXa(1); FP(1); issue_v(nxt, 0); }     // (v rows 0..31 are in registers since region 9)
             if (f == 11) { TXb(0); TXb(1); wait_vm_at_most<N_AFTER_VHI>(); FV(2); }
             if (f == 12) { TPa(0); TPa(1); FV(3); }
@@ -454,7 +503,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
 
     if (nsteps > 0) {
 #pragma unroll
-        for (int part = 0; part < 4; ++part) issue_shared(it0, 0, part);
+        for (int part = 0; part < 3; ++part) issue_shared(it0, 0, part);
         issue_v(it0, 0);
         issue_v(it0, 1);
         wait_vm_at_most<0>();

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
 
-    // q is needed for its row norms (l2 normalisation) and for P, when the scan wants P from the records
+    // q is needed for its row norms (l2 normalisation) and for P, when P is asked for
     const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
     const bool want_P = p.want_P != 0, need_q = l2 || want_P;
     // ---- all global loads first: the gate inputs of value head w of the group, then the k, q rows ----

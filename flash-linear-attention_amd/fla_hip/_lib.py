@@ -34,6 +34,7 @@ FLAG_SEQ_ORDER = 1 << 19
 FLAG_SCAN_NO_PAIR = 1 << 20
 FLAG_SCAN_PAIR = 1 << 21
 FLAG_SCAN_NO_WARM = 1 << 22
+FLAG_RECORD_P = 1 << 23
 
 ACT_NONE, ACT_SILU, ACT_SIGMOID = 0, 1, 2
 

@@ -34,7 +34,8 @@ _KERNEL_CHUNK = 64
 # ('wide') or time cut into segments, each with one run per workgroup ('-single') or two ('-pair')
 _SCAN_MODE_FLAGS = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS,
                     'single': _lib.FLAG_SCAN_NO_PAIR, 'pair': _lib.FLAG_SCAN_PAIR,
-                    'segments-exact': _lib.FLAG_SCAN_SEGMENTS | _lib.FLAG_SCAN_NO_WARM}
+                    'segments-exact': _lib.FLAG_SCAN_SEGMENTS | _lib.FLAG_SCAN_NO_WARM,
+                    'record-p': _lib.FLAG_RECORD_P}       # (the prepare stage also writes P: for looking at its records)
 for _form in ('wide', 'segments'):
     for _runs in ('single', 'pair'):
         _SCAN_MODE_FLAGS[f'{_form}-{_runs}'] = _SCAN_MODE_FLAGS[_form] | _SCAN_MODE_FLAGS[_runs]

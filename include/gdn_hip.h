@@ -52,6 +52,7 @@ extern "C" {
 #define GDN_FLAG_SCAN_NO_PAIR   (1u << 20) /* always one run per workgroup                      */
 #define GDN_FLAG_SCAN_PAIR      (1u << 21) /* two runs per workgroup wherever two can share k rows */
 #define GDN_FLAG_SCAN_NO_WARM   (1u << 22) /* time segments always start from exact states (first pass + merge) */
+#define GDN_FLAG_RECORD_P       (1u << 23) /* the chunk-parallel stage also leaves P in its records (the scan forms P itself and never reads it) */
 
 /* activation codes of the convolution and normalisation entry points */
 #define GDN_ACT_NONE    0

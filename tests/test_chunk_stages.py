@@ -51,10 +51,9 @@ def _records(call, num_chunks, HV):
 ])
 def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2, monkeypatch):
     from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
-    # P is part of the records only for the scan kernel that reads it from there: two runs per workgroup, which needs
-    # an even number of value heads per q/k head and 128 value columns (the other kernel forms P itself)
-    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'wide-pair')
-    has_P = (HV // H) % 2 == 0 and K == 128
+    # the scan kernels form P themselves; the chunk-parallel stage leaves it in its records only on request
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'record-p')
+    has_P = True
     gen = torch.Generator().manual_seed(7)
     q = torch.randn(B, T, H, K, generator=gen)
     k = torch.randn(B, T, H, K, generator=gen)
