@@ -116,18 +116,21 @@ inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Number of time segments the sequential stage cuts every sequence into (0: whole sequences, one
 // workgroup per sequence and head).  With few (sequence, head) runs and long dense sequences, time is
-// cut so that every CU has a workgroup: two passes over 1/nseg of the chunks each plus a small merge,
-// which must beat one pass over all chunks (nseg >= 3, and segments of 8 chunks or more: every pass also pays for filling
-// and draining its pipeline and for a launch).  Shared by the workspace size and the launch.
+// cut so that every CU has a workgroup - never more workgroups than CUs: a second round of workgroups
+// costs more than longer segments do.  Segments hold 8 chunks or more each (every pass also pays for
+// filling and draining its pipeline and for a launch).  Two segments pay where they may start warm
+// (one pass over half the chunks plus the warm-up); with exact start states only (first pass, merge,
+// second pass) it takes three.  Either way the steps saved per workgroup must outweigh a warm-up of typical
+// length plus the two launches that find nothing to do: 24 chunks or more.  Shared by the workspace size and the launch.
 inline int plan_segments(int64_t N, int64_t HV, int64_t NT, int64_t num_chunks, bool dense, uint32_t flags) {
     const int64_t NH = N * HV;
     int nseg = 0;
     if (dense && NH > 0) {
         // (GDN_FLAG_SCAN_SEGMENTS asks for segments wherever they are possible at all: segments of 4 chunks)
-        nseg = (int)std::min<int64_t>((256 + NH / 2) / NH, NT / ((flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
+        nseg = (int)std::min<int64_t>(256 / NH, NT / ((flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
         while (nseg > 0 && ((int64_t)nseg * NH > SEG_SLOTS_MAX || (int64_t)nseg * NH > (num_chunks * HV + 3) / 4)) --nseg;
     }
-    bool segments = nseg >= 3;
+    bool segments = nseg >= ((flags & GDN_FLAG_SCAN_NO_WARM) ? 3 : 2) && NT - NT / std::max(nseg, 1) >= 24;
     if (flags & GDN_FLAG_SCAN_WIDE) segments = false;
     if ((flags & GDN_FLAG_SCAN_SEGMENTS) && nseg >= 2) segments = true;
     return segments ? nseg : 0;
