@@ -450,19 +450,20 @@ def test_workgroup_placement_with_sequence_counts_that_are_not_multiples_of_8(N,
     _check('ht', ref_ht, ht.transpose(-1, -2) if vfirst else ht)
 
 
-def test_decode_and_prefill_replay_from_a_captured_graph():
+@pytest.mark.parametrize('H,HV,D,N,K_prefill', [(2, 4, 128, 8, 128), (8, 32, 128, 40, 256)])
+def test_decode_and_prefill_replay_from_a_captured_graph(H, HV, D, N, K_prefill):
     """Serving loops replay captured graphs: the entry points only enqueue kernels on the given
     stream (no allocation, no memset, no synchronisation of their own), so a captured decode step
     and a captured prefill reproduce the eager results on every replay, with eager work and
-    synchronisations in between."""
+    synchronisations in between.  (Second case: the decode kernel of the common shape with its placement
+    on the XCDs, and the wide-key prefill kernel.)"""
     from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
     dev = 'cuda'
-    H, HV, D, N = 2, 4, 128, 8
     q, k, v, g, beta, h0 = _inputs(N, 1, H, HV, D, torch.bfloat16, seed=5)
     dq, dk, dv, dg, db = (x.to(dev) for x in (q, k, v, g, beta))
     state = h0.to(dev).contiguous()
     eager_state = state.clone()
-    pq, pk, pv, pg, pb, ph = (x.to(dev) for x in O.make_inputs(1, 700, H, HV, D, D, seed=6, gate_div=8.0, h0_std=0.5, dtype=torch.bfloat16))
+    pq, pk, pv, pg, pb, ph = (x.to(dev) for x in O.make_inputs(1, 700, 2, 4, K_prefill, D, seed=6, gate_div=8.0, h0_std=0.5, dtype=torch.bfloat16))
     # warm up outside the capture (library load, kernel attributes)
     _ops()(dq, dk, dv, dg, beta=db, initial_state=state.clone(), output_final_state=True, inplace_final_state=True)
     po_eager, ph_eager = chunk_gated_delta_rule(pq, pk, pv, pg, pb, initial_state=ph, output_final_state=True)
