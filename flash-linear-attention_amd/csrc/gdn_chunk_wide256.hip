@@ -11,8 +11,9 @@
 // k and q tiles are two 128-feature halves, each laid out exactly like the narrow kernel's tile, so every operand
 // address is the narrow kernel's plus a half offset.  What differs is the LDS budget: 64 tokens x 512 B of k and of
 // q are 32 KB each.  k has two buffers (read until the very end of a step, copied one step ahead), v and the record
-// have two, q and P have ONE: q of the next chunk is copied after the barrier that ends this chunk's last read of
-// it, while the compute waves finish the state update.
+// have two, q and P have ONE: q of the next chunk is requested after the barrier that ends this chunk's last read of
+// it and awaited in the middle of the next step - a step multiplies by k first (the products that head the chain to the
+// next state) and turns to q, P and the output when an LDS counter says that q has landed.
 #include "gdn_chunk_common.h"
 
 namespace gdn {
@@ -73,8 +74,9 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     const int64_t nsteps = (len + CH - 1) / CH;
     const int64_t lastc = nsteps - 1;
     char* otile = smem + W2_OT;
-    volatile int* pcount = (volatile int*)(smem + W2_PCOUNT);
-    if (tid == 0) *pcount = 0;
+    volatile int* pcount = (volatile int*)(smem + W2_PCOUNT);           // copy waves whose share of P of step i is in LDS: 4 (i + 1)
+    volatile int* qcount = pcount + 1;                                   // chunks whose q tile has landed
+    if (tid == 0) { *pcount = 0; *qcount = 0; }
     // Key features past K and value columns past V are never copied: the tiles are cleared once.
     if (nsteps > 0) {
         const u32x4 z = {0u, 0u, 0u, 0u};
@@ -93,7 +95,9 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
         // P = scale tril(q k^T 2^(G_t - G_t')) of a chunk from its q and k tiles (see gdn_chunk_wide.hip), contraction
         // over both halves of the key features
-        auto produce_P = [&](const char* kbuf, const char* rec) {
+        auto produce_P = [&](const char* kbuf, const char* rec, int q_target) {
+            while (*qcount < q_target) __builtin_amdgcn_s_sleep(1);          // q of this chunk has landed
+            asm volatile("" ::: "memory");
             __builtin_amdgcn_s_setprio(3);
             const int pw = w - W2_CW;
             const V8* sK = (const V8*)kbuf;
@@ -165,23 +169,27 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 gather_qk((const T*)p.k, min(i + 1, lastc), lds0 + W2_KB + (int)((i + 1) & 1) * 32768);
-                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();
                 lds_barrier();                                              // B2
             }
         } else if (w == W2_CW + 1) {
-            // ---- q (one buffer: copied between B1 and B2) and the record (two) ----
+            // ---- q (one buffer) and the record (two).  q of chunk i+1 is requested right after the barrier B1 of step i,
+            // which ends the last read of q of chunk i, and is awaited inside step i+1: the compute waves multiply by k
+            // first and turn to q, and the copy waves to P, only when the counter says that it has landed ----
             gather_qk((const T*)p.q, 0, lds0 + W2_Q);
             copy_rec(0, lds0 + W2_REC);
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                copy_rec(min(i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);
-                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                copy_rec(min(i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);      // 7 operations
+                wait_vm_at_most<7>();                                       // everything older than these: q of chunk i
+                if (lane == 0) __hip_atomic_fetch_add((int*)qcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
-                gather_qk((const T*)p.q, min(i + 1, lastc), lds0 + W2_Q);
-                wait_vm_at_most<0>();
+                wait_vm_at_most<0>();                                       // the record of chunk i+1
+                if (i + 1 < nsteps) gather_qk((const T*)p.q, i + 1, lds0 + W2_Q);
                 lds_barrier();                                              // B2
             }
         } else if (w == W2_CW + 2) {
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 gather_v(min(i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
-                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();
                 lds_barrier();                                              // B2
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             };
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES);
+                produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 if (i > 0) store_rows(i - 1);
                 lds_barrier();                                              // B1
 #pragma unroll
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         v_tr = (g * 64 + 16 * (c >> 2) + 4 * tr_i + ((c + g) & 3)) * 8 + 4 * (tr_j & 1);
     }
 
-    auto step = [&](const char* kbuf, const char* vbuf, const char* rec, int p_target) {
+    auto step = [&](const char* kbuf, const char* vbuf, const char* rec, int istep) {
         const V8* sK = (const V8*)kbuf;
         const V8* sQ = (const V8*)(smem + W2_Q);
         const T* sV = (const T*)vbuf;
@@ -276,21 +284,18 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         const float* sTab = (const float*)(rec + W2_RTAB);
         auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
 
-        // fragment f = (t-tile f/8, key features 32s .. 32s+31 with s = f%8) of k and q, in a ring of register sets
-        constexpr int RING = 3;
-        V8 ak[RING], aq[RING];
-        auto F = [&](int f) {
-            const int idx = ((f & 7) >> 2) * 1024 + (f >> 3) * 256 + 16 * (f & 3) + a_off;
-            ak[f % RING] = sK[idx];
-            aq[f % RING] = sQ[idx];
-        };
+        // fragment f = (t-tile f/8, key features 32s .. 32s+31 with s = f%8) of k or of q, each in a ring of four registers
+        // sets: a region multiplies two fragments and fetches the two of the next region
+        auto fidx = [&](int f) { return ((f & 7) >> 2) * 1024 + (f >> 3) * 256 + 16 * (f & 3) + a_off; };
+        V8 ak[4], aq[4];
+        auto Fk = [&](int f) { if (f < 32) ak[f & 3] = sK[fidx(f)]; };
+        auto Fq = [&](int f) { if (f < 32) aq[f & 3] = sQ[fidx(f)]; };
         f32x4 ks[4], ao[4];
         V8 Sb[8];
-        auto M = [&](int f) {
-            const int tt = f >> 3, sx = f & 7;
-            ks[tt] = Mma<T>::run(ak[f % RING], Sb[sx], sx ? ks[tt] : f32x4{0.f, 0.f, 0.f, 0.f});
-            ao[tt] = Mma<T>::run(Sb[sx], aq[f % RING], sx ? ao[tt] : f32x4{0.f, 0.f, 0.f, 0.f});
-        };
+        auto Mk = [&](int f) { ks[f >> 3] = Mma<T>::run(ak[f & 3], Sb[f & 7], (f & 7) ? ks[f >> 3] : f32x4{0.f, 0.f, 0.f, 0.f}); };
+        auto Mq = [&](int f) { ao[f >> 3] = Mma<T>::run(Sb[f & 7], aq[f & 3], (f & 7) ? ao[f >> 3] : f32x4{0.f, 0.f, 0.f, 0.f}); };
+        auto KK = [&](int r) { Fk(2 * r + 2); Fk(2 * r + 3); Mk(2 * r); Mk(2 * r + 1); };       // region r of the k products
+        auto QQ = [&](int r) { Fq(2 * r + 2); Fq(2 * r + 3); Mq(2 * r); Mq(2 * r + 1); };       // region r of the q products
         V4 vv[4];
         V8 ax[4][2], ap[4][2];
         auto FV = [&](int tt) { vv[tt] = Mma<T>::tr_read(sV + tt * 2048 + v_tr); };
@@ -302,9 +307,10 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
 #pragma unroll
             for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
         };
-        // k^T operands of the state update, u = 16 sp2 + m (t-tile pair sp2, key tile m), in a ring of 8
+        // k^T operands of the state update, u = 16 sp2 + m (t-tile pair sp2, key tile m), in a ring of 8, fetched 6 ahead
         V8 kt[8];
         auto FK = [&](int u) {
+            if (u >= 32) return;
             const int sp2 = u >> 4, m = u & 15;
             const T* a = sKt + (m >> 3) * 8192 + sp2 * 4096 + 128 * ((m & 7) >> 1) + 4 * (m & 1) + k_tr;
             kt[u & 7] = join<V8>(Mma<T>::tr_read(a), Mma<T>::tr_read(a + 2048));
@@ -342,10 +348,13 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(oacc[tt][r]);
             *(V4*)(otile + (16 * tt + c16) * W2_OT_PITCH + (16 * w + 4 * g) * 2) = o4;
         };
-        auto U = [&](int u) { S[u & 15] = Mma<T>::run(kt[u & 7], Vg[u >> 4], S[u & 15]); };
+        auto UU = [&](int j) {                   // two products of the state update, and the operands of two later ones
+            FK(2 * j + 6); FK(2 * j + 7);
+            S[(2 * j) & 15] = Mma<T>::run(kt[(2 * j) & 7], Vg[j >> 3], S[(2 * j) & 15]);
+            S[(2 * j + 1) & 15] = Mma<T>::run(kt[(2 * j + 1) & 7], Vg[j >> 3], S[(2 * j + 1) & 15]);
+        };
 
-#pragma unroll
-        for (int f = 0; f < RING - 1; ++f) F(f);
+        Fk(0); Fk(1);
 #pragma unroll
         for (int s = 0; s < 8; ++s)
 #pragma unroll
@@ -357,67 +366,63 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         const float lg_try = lg + sTab[TAB_GLAST];
         const bool lazy = lg_try >= LG_MIN;
         vscale = lazy ? fast_exp2(-lg_try) : 1.f;
-        fence();
-        // ---- 32 regions: the products of fragment f and the fetch of fragment f + 2; beside them the fetches of
-        // v and Xb, then the tail of t-tiles 0, 1 while tiles 2, 3 are multiplied ----
-#pragma unroll
-        for (int f = 0; f < 32; ++f) {
-            if (f + RING - 1 < 32) F(f + RING - 1);
-            M(f);
-            if (f == 8) FV(0);
-            if (f == 9) FV(1);
-            if (f == 10) FX(0);
-            if (f == 11) FX(1);
-            if (f == 16) TD(0);
-            if (f == 17) TD(1);
-            if (f == 18) { TXa(0); TXa(1); }
-            if (f == 19) {
-                while (*pcount < p_target) __builtin_amdgcn_s_sleep(1);      // P of this chunk (normally long there)
-                FP(0); FP(1);
-                TXb(0); TXb(1); FV(2);
-            }
-            if (f == 20) { TPa(0); TPa(1); FV(3); }
-            if (f == 21) { TPb(0); TPb(1); FX(2); }
-            if (f == 22) FX(3);
-            if (f == 24) { FP(2); FP(3); }
-            if (f >= 29) { FK(2 * (f - 29)); FK(2 * (f - 29) + 1); }          // u = 0 .. 5
-            fence();
-        }
+        // the decay fold (rare; a scalar branch): the products below read the bf16 copy made above, the update the folded state
         if (__builtin_amdgcn_readfirstlane((int)lazy) == 0) {
             const float fold = fast_exp2(lg_try);
 #pragma unroll
             for (int m = 0; m < 16; ++m) S[m] *= fold;
         }
         lg = lazy ? lg_try : 0.f;
-        // ---- state update from t-tiles 0, 1 (16 products) beside the tail of tiles 2, 3; the k^T operands are fetched
-        // six products ahead ----
-#pragma unroll
-        for (int r8 = 0; r8 < 8; ++r8) {
-            U(2 * r8); U(2 * r8 + 1);
-            FK(2 * r8 + 6); FK(2 * r8 + 7);
-            if (r8 == 0) TD(2);
-            if (r8 == 1) TD(3);
-            if (r8 == 2) { TXa(2); TXa(3); }
-            if (r8 == 3) { TXb(2); TXb(3); }
-            if (r8 == 4) { TPa(2); TPa(3); }
-            if (r8 == 5) { TPb(2); TPb(3); }
-            fence();
-        }
+        fence();
+        // ---- The products with k come first: they head the chain that the next step waits for (k S -> D -> v_new -> state
+        // update), and q of this chunk may still be on its way.  The update from t-tiles 0, 1 starts while tiles 2, 3 are
+        // still being multiplied; the products with q, P and the output fill the second half of the step. ----
+        KK(0); FV(0); fence();
+        KK(1); FV(1); fence();
+        KK(2); FX(0); fence();
+        KK(3); FX(1); fence();
+        KK(4); TD(0); FK(0); FK(1); fence();
+        KK(5); FV(2); FK(2); FK(3); fence();
+        KK(6); FV(3); FK(4); FK(5); fence();
+        KK(7); fence();
+        KK(8); TD(1); fence();
+        KK(9); TXa(0); TXa(1); fence();
+        KK(10); TXb(0); TXb(1); fence();
+        KK(11); UU(0); fence();
+        while (*qcount < istep + 1) __builtin_amdgcn_s_sleep(1);      // q of this chunk (normally long there)
+        asm volatile("" ::: "memory");                                // (no read of the tile may move in front of the poll)
+        Fq(0); Fq(1);
+        KK(12); UU(1); TD(2); FX(2); fence();
+        KK(13); UU(2); QQ(0); fence();
+        KK(14); UU(3); QQ(1); FX(3); fence();
+        KK(15); UU(4); QQ(2); fence();
+        TD(3); UU(5); QQ(3); fence();
+        TXa(2); TXa(3); UU(6); QQ(4); fence();
+        TXb(2); TXb(3); UU(7); QQ(5); fence();
+        while (*pcount < 4 * (istep + 1)) __builtin_amdgcn_s_sleep(1);      // P of this chunk
+        asm volatile("" ::: "memory");
+        FP(0); FP(1);
+        UU(8); QQ(6); fence();
+        UU(9); QQ(7); TPa(0); fence();
+        UU(10); QQ(8); TPa(1); TPb(0); FP(2); fence();
+        UU(11); QQ(9); TPb(1); FP(3); fence();
+        UU(12); QQ(10); fence();
+        QQ(11); TPa(2); fence();
+        QQ(12); TPb(2); fence();
+        QQ(13); fence();
+        QQ(14); fence();
+        QQ(15); fence();
+        TPa(3); fence();
+        TPb(3); fence();
         lds_barrier();                                          // B1: q, v, the record and P are free, the output tile is complete
-        // ---- state update from t-tiles 2, 3 ----
-#pragma unroll
-        for (int r8 = 0; r8 < 8; ++r8) {
-            U(16 + 2 * r8); U(16 + 2 * r8 + 1);
-            if (r8 < 5) { FK(16 + 2 * r8 + 6); FK(16 + 2 * r8 + 7); }
-            fence();
-        }
-        lds_barrier();                                          // B2: k of this stage is free, the next chunk is complete
+        UU(13); UU(14); UU(15); fence();
+        lds_barrier();                                          // B2: k of this stage is free, k, v and the record of the next chunk are complete
     };
     if (nsteps > 0) {
         lds_barrier();                                          // B0
         for (int64_t i = 0; i < nsteps; ++i)
             step(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_V + (int)(i & 1) * 16384, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES,
-                 4 * ((int)i + 1));
+                 (int)i);
     }
 
     if (dst) {
