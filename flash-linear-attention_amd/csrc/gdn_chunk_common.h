@@ -76,9 +76,10 @@ constexpr int TAB2_G = 0, TAB2_NQS = 64, TAB2_NK = 128;
 // the chunk's transition S -> 2^G_last S - k~^T (Xb 2^G k) S can stretch any state:
 //   bound = sum_t [ log2 gamma_t + log2 max(1, |1 - beta_t |k_t|^2|) ]      (each token's factor gamma_t (I - beta_t k_t k_t^T))
 // A run of chunks whose bounds add up to at most WARM_LOG2 forgets what came before it to within 2^WARM_LOG2 of that
-// state's size - far below the rounding of the fp32 state itself - so a time segment may start from a ZERO state that
-// many chunks early instead of from the exact state that a first pass and a merge would have to compute.
-constexpr float WARM_LOG2 = -64.f;
+// state's size: the state in front of the run would have to be 2^24 times the size of the state behind it for the
+// dropped part to reach the rounding of the fp32 state (2^-24 of its own size).  So a time segment may start from a
+// ZERO state that many chunks early instead of from the exact state that a first pass and a merge would have to compute.
+constexpr float WARM_LOG2 = -48.f;
 constexpr int WARM_CAP_MAX = 64;
 __host__ __device__ constexpr int p_slot(int tt, int sp) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp; }
 __host__ __device__ constexpr bool frag_half(int tt, int sp) { return (tt == 0 && sp == 0) || (tt == 2 && sp == 1); }

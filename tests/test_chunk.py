@@ -252,7 +252,7 @@ def _gates_per_head(B, T, HV, per_token, seed):
 @pytest.mark.parametrize('case', ['fast', 'slow', 'mixed', 'expanding', 'boundary'])
 def test_segments_that_start_warm(monkeypatch, case):
     """Time segments start from a zero state a few chunks early where the decay over those chunks makes
-    the true state irrelevant (bound 2^-64), and from the exact merged state otherwise - decided per head
+    the true state irrelevant (bound 2^-48), and from the exact merged state otherwise - decided per head
     on the device.  Heads that decay slowly, or whose keys are long enough to stretch the state
     (beta |k|^2 > 2), must take the exact path and then equal it bit for bit."""
     B, T, H, HV, D = 1, 8192, 4, 16, 128          # 16 segments of 8 chunks; up to 16 chunks of warm-up
@@ -265,7 +265,7 @@ def test_segments_that_start_warm(monkeypatch, case):
         beta = torch.ones_like(beta)
         g = g * 4                                   # (keeps the recurrence itself stable)
     if case == 'boundary':
-        # constant decay chosen so that 8 chunks give 2^-64.6 and 7 do not: the warm-up length is exactly 8
+        # constant decay: 8.08 in log2 units per chunk, so 6 chunks give 2^-48.5 and 5 do not: the warm-up length is exactly 6
         g = torch.full_like(g, -0.0875)
     ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
     out = {}
@@ -280,9 +280,11 @@ def test_segments_that_start_warm(monkeypatch, case):
         assert same, 'heads that cannot start warm must take the exact path unchanged'
     else:
         # a different (and equally good) start state: close; with a decay that varies it is not identical
-        # (with the constant decay of 'boundary' what a warm start drops is below the rounding of the fp32 state)
+        # (with the constant decay of 'boundary' what a warm start drops may lie below the rounding of the fp32 state)
         assert case == 'boundary' or not same
-        assert O.get_err_ratio(o_e.float().cpu(), o_w.float().cpu()) < 2e-3
+        # (bf16 rounding of the operands: two EXACT evaluations - whole sequences and segments from merged states - differ
+        # by 2.1e-3 from each other on these inputs, each 3.7e-3 from the fp32 oracle)
+        assert O.get_err_ratio(o_e.float().cpu(), o_w.float().cpu()) < 3e-3
     if case == 'mixed':
         # per head: value heads 1 and 3 decay too slowly (1e-4, 0.01 per token) and are bitwise those of the exact path
         assert torch.equal(o_w[:, :, 1::2], o_e[:, :, 1::2]) and torch.equal(h_w[:, 1::2], h_e[:, 1::2])
@@ -292,7 +294,7 @@ def test_segments_that_start_warm(monkeypatch, case):
 
 
 def test_warm_start_forgets_an_enormous_state(monkeypatch):
-    """What a warm start drops is bounded by 2^-64 of the state BEFORE the warm-up chunks, whatever its size:
+    """What a warm start drops is bounded by 2^-48 of the state BEFORE the warm-up chunks, whatever its size:
     a huge initial state and huge early values must leave the later output as accurate as the exact path."""
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'segments-single')
     B, T, H, HV, D = 1, 8192, 4, 16, 128
