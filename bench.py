@@ -88,6 +88,12 @@ PUBLISHED = {
     'ref_b4_t4096_h64_d128': _published(4, 4096, 64, 128),
     'ref_b8_t1024_h8_d64': _published(8, 1024, 8, 64),
     'ref_b8_t2048_h32_d256': _published(8, 2048, 32, 256),
+    # one long prompt through the reference layer's default head shape (fla/layers/gated_deltanet.py:91-92: head_dim 256, expand_v 2;
+    # hidden size 2048 -> 6 heads): wide keys, time segments that start warm
+    'layer_default_b1_t32768_h6_k256_v512': dict(kind='prefill', B=1, T=32768, H=6, HV=6, K=256, V=512, h0=False, varlen=False, final=True,
+                                                 l2norm=True, raw_qk=True,
+                                                 name="one prompt of 32768 tokens in the reference layer's default head shape: H=6 K=256 V=512 bf16, "
+                                                      'use_qk_l2norm_in_kernel, final state returned'),
 }
 
 

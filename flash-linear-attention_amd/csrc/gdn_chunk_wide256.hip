@@ -33,7 +33,7 @@ constexpr int W2_THREADS = (W2_CW + 4) * 64;
 constexpr int W2_VB = 64;                                 // value columns per workgroup
 
 template <typename T>
-__global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkParams p, int NVB) {
+__global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkParams p, int NVB, SegmentPlan sp) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
@@ -49,17 +49,32 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     const int G = HV / H, GV = G * NVB;
     const int64_t slot = blockIdx.x >> 3;
     const int xcd = blockIdx.x & 7;
-    const int64_t group = (slot / GV) * 8 + xcd;                     // (sequence, q/k head)
-    if (group >= p.N * H) return;
-    int64_t n = group / H;
+    const int64_t group = (slot / GV) * 8 + xcd;                     // (sequence, q/k head, time segment)
+    const int nseg = sp.nseg;                                        // 1: whole sequences
+    if (group >= p.N * H * nseg) return;
+    const int seg = (int)(group % nseg);
+    int64_t n = (group / nseg) / H;
     if (p.flags & GDN_FLAG_SEQ_ORDER) n = load_index(p.chunk_offsets, p.N + 1 + n, cu32);
-    const int h = (int)(group % H);
+    const int h = (int)((group / nseg) % H);
     const int member = (int)(slot % GV);
     const int hv = h * G + member / NVB;
     const int v0 = (member % NVB) * W2_VB;
     const int64_t inh = n * HV + hv;
-    const float* src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr;
-    float* dst = p.ht ? p.ht + inh * (int64_t)(K * V) : nullptr;
+    // Time segments (long dense sequences on few heads) start warm: a zero state a few chunks early, where the bound on
+    // the chunks' transitions makes the true state irrelevant (see WARM_LOG2), and no output until the segment proper.
+    // A head with a segment that cannot start this way is evaluated whole by the workgroups of its segment 0; those of
+    // its other segments have nothing to do.
+    int warm = 0;
+    bool whole = nseg == 1;
+    if (nseg > 1) {
+        const float* bnd = sp.bound + n * p.NT * HV + hv;
+        whole = needs_exact_segments(sp, bnd, HV, lane);
+        if (whole && seg > 0) return;
+        if (!whole && seg > 0) warm = __builtin_amdgcn_readfirstlane(warm_chunks(bnd, HV, (int64_t)seg * sp.seg_chunks, sp.warm_cap, lane));
+    }
+    const bool from_start = whole || (int64_t)seg * sp.seg_chunks - warm == 0, to_end = whole || seg == nseg - 1;
+    const float* src = p.h0 && from_start ? p.h0 + inh * (int64_t)(K * V) : nullptr;
+    float* dst = p.ht && to_end ? p.ht + inh * (int64_t)(K * V) : nullptr;
 
     int64_t bos, len, boh;
     if (p.cu_seqlens) {
@@ -71,8 +86,11 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         len = p.T;
         boh = n * p.NT;
     }
-    const int64_t nsteps = (len + CH - 1) / CH;
-    const int64_t lastc = nsteps - 1;
+    const int64_t nt = (len + CH - 1) / CH;
+    const int64_t it0 = whole ? 0 : (int64_t)seg * sp.seg_chunks - warm;           // first chunk of this run (warm-up included)
+    const int64_t it1 = whole ? nt : min(nt, (int64_t)(seg + 1) * sp.seg_chunks);
+    const int64_t nsteps = it1 - it0;                                               // step i works on chunk it0 + i
+    const int64_t lastc = it1 - 1;
     char* otile = smem + W2_OT;
     volatile int* pcount = (volatile int*)(smem + W2_PCOUNT);           // copy waves whose share of P of step i is in LDS: 4 (i + 1)
     volatile int* qcount = pcount + 1;                                   // chunks whose q tile has landed
@@ -164,11 +182,11 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         };
         if (w == W2_CW) {
             // ---- k: chunk i+1 is copied during step i (its buffer was last read in step i-1) ----
-            gather_qk((const T*)p.k, 0, lds0 + W2_KB);
+            gather_qk((const T*)p.k, it0, lds0 + W2_KB);
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                gather_qk((const T*)p.k, min(i + 1, lastc), lds0 + W2_KB + (int)((i + 1) & 1) * 32768);
+                gather_qk((const T*)p.k, min(it0 + i + 1, lastc), lds0 + W2_KB + (int)((i + 1) & 1) * 32768);
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();
@@ -178,18 +196,18 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             // ---- q (one buffer) and the record (two).  q of chunk i+1 is requested right after the barrier B1 of step i,
             // which ends the last read of q of chunk i, and is awaited inside step i+1: the compute waves multiply by k
             // first and turn to q, and the copy waves to P, only when the counter says that it has landed ----
-            gather_qk((const T*)p.q, 0, lds0 + W2_Q);
-            copy_rec(0, lds0 + W2_REC);
+            gather_qk((const T*)p.q, it0, lds0 + W2_Q);
+            copy_rec(it0, lds0 + W2_REC);
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                copy_rec(min(i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);      // 7 operations
+                copy_rec(min(it0 + i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);      // 7 operations
                 wait_vm_at_most<7>();                                       // everything older than these: q of chunk i
                 if (lane == 0) __hip_atomic_fetch_add((int*)qcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();                                       // the record of chunk i+1
-                if (i + 1 < nsteps) gather_qk((const T*)p.q, i + 1, lds0 + W2_Q);
+                if (i + 1 < nsteps) gather_qk((const T*)p.q, it0 + i + 1, lds0 + W2_Q);
                 lds_barrier();                                              // B2
             }
         } else if (w == W2_CW + 2) {
@@ -206,11 +224,11 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
                     gather_1k_to_lds_masked(base, (uint32_t)row * row_bytes + 16 * c, lds_tile + j * 1024, mask);
                 }
             };
-            gather_v(0, lds0 + W2_V);
+            gather_v(it0, lds0 + W2_V);
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                gather_v(min(i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
+                gather_v(min(it0 + i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();
@@ -233,13 +251,13 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
-                if (i > 0) store_rows(i - 1);
+                if (i > warm) store_rows(it0 + i - 1);             // (the chunks of a warm-up leave no output)
                 lds_barrier();                                              // B1
 #pragma unroll
                 for (int j = 0; j < 8; ++j) orow[j] = *(const u32x4*)(otile + (8 * j + orow_r) * W2_OT_PITCH + opiece * 16);
                 lds_barrier();                                              // B2 (waits for the tile reads)
             }
-            store_rows(lastc);
+            if (nsteps > warm) store_rows(lastc);
         }
         wait_vm_at_most<0>();                               // no copy may land in LDS after this workgroup has gone
         return;
@@ -446,9 +464,25 @@ int launch_wide256(const ChunkParams& p, hipStream_t stream) {
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, W2_SMEM, attr_done, "hipFuncSetAttribute(wide256)")) return rc;
     const int NVB = (p.V + W2_VB - 1) / W2_VB;
-    const int64_t blocks = (p.N * p.H + 7) / 8 * 8 * (p.HV / p.H) * NVB;
+    const int64_t GV = (int64_t)(p.HV / p.H) * NVB;
+    // Time segments where whole sequences leave CUs without a workgroup: never more workgroups than CUs, segments of 8
+    // chunks or more, and at least 24 chunks saved per workgroup (a warm-up of typical length must pay)
+    SegmentPlan sp = {};
+    sp.nseg = 1;
+    sp.seg_chunks = 1 << 30;
+    const int64_t runs = p.N * p.H * GV;
+    if (!p.cu_seqlens && !(p.flags & (GDN_FLAG_SCAN_WIDE | GDN_FLAG_SCAN_NO_WARM)) && runs > 0) {
+        const int nseg = (int)std::min<int64_t>(256 / runs, p.NT / ((p.flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
+        if (nseg >= 2 && ((p.flags & GDN_FLAG_SCAN_SEGMENTS) || p.NT - p.NT / nseg >= 24)) {
+            sp.nseg = nseg;
+            sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
+            sp.bound = p.ws.Bound;
+            sp.warm_cap = std::min(WARM_CAP_MAX, sp.seg_chunks + sp.seg_chunks / 4 + 6);
+        }
+    }
+    const int64_t blocks = (p.N * p.H * sp.nseg + 7) / 8 * 8 * GV;
     if (blocks >= (1ll << 31)) { set_error("gdn_chunk_fwd: too many workgroups for one launch"); return GDN_ERR_UNSUPPORTED; }
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(W2_THREADS), W2_SMEM, stream, p, NVB);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(W2_THREADS), W2_SMEM, stream, p, NVB, sp);
     return check_launch("gdn_chunk_wide256_kernel");
 }
 

@@ -122,3 +122,29 @@ def test_wide_keys_outputs_fully_written_and_deterministic():
     assert not torch.isnan(o1.float()).any() and not torch.isnan(h1).any()
     o2, h2 = _run(q, k, v, g, beta, h0)
     assert torch.equal(o1, o2) and torch.equal(h1, h2)
+
+
+@pytest.mark.parametrize('case', ['fast', 'slow', 'mixed'])
+def test_wide_keys_time_segments_that_start_warm(monkeypatch, case):
+    """A long dense sequence on few heads is cut into time segments that start warm (a zero state a few chunks early, decided
+    per head on the device from the bound on the chunks' transitions); a head that decays too slowly for that is evaluated
+    whole by the workgroups of its first segment and equals the run without segments bit for bit."""
+    B, T, H, HV, K, V = 1, 4096, 2, 4, 256, 128                # 16 workgroups per segment: 8 segments of 8 chunks
+    q, k, v, _, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=31, h0_std=0.5, dtype=torch.bfloat16)
+    per_token = {'fast': [0.1] * 4, 'slow': [1e-3] * 4, 'mixed': [0.1, 1e-3, 0.3, 0.005]}[case]
+    gen = torch.Generator().manual_seed(32)
+    g = -(0.5 + torch.rand(B, T, HV, generator=gen)) * torch.tensor(per_token)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    o_s, h_s = _run(q, k, v, g, beta, h0)
+    _check('o', ref_o, o_s)
+    _check('ht', ref_ht, h_s)
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'wide')
+    o_w, h_w = _run(q, k, v, g, beta, h0)
+    slow_heads = {'fast': [], 'slow': [0, 1, 2, 3], 'mixed': [1, 3]}[case]
+    for hv in range(HV):
+        same = torch.equal(o_s[:, :, hv], o_w[:, :, hv]) and torch.equal(h_s[:, hv], h_w[:, hv])
+        if hv in slow_heads:
+            assert same, f'head {hv} cannot start warm and must be evaluated whole'
+        else:
+            # (the first segment starts from the true state either way; the later ones from a different, equally good one)
+            assert torch.equal(o_s[:, :512, hv], o_w[:, :512, hv]) and not same, hv
