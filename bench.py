@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -70,6 +70,9 @@ WORKLOADS = {
                    name='configs[3]: GDN varlen prefill 65536 tokens in 32 sequences Hqk=16 Hv=32 K=V=128 bf16'),
     'decode': dict(kind='decode', N=256, H=16, HV=32,
                    name='configs[4]: GDN single-token decode batch=256 Hqk=16 Hv=32 K=V=128 bf16, fp32 states in place'),
+    'decode_bf16_states': dict(kind='decode', N=256, H=16, HV=32, state_dtype='bf16',
+                               name='the decode step of configs[4] with the states kept in bf16 (an option of this library: '
+                                    'fp32 step, one rounding per step; 2 x 256 MiB of state traffic)'),
 }
 
 
@@ -265,12 +268,16 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     g = F.logsigmoid(torch.randn(N, 1, HV, generator=gen))
     beta = torch.sigmoid(torch.randn(N, 1, HV, generator=gen))
     h0 = 0.1 * torch.randn(N, HV, K, V, generator=gen)
+    bf16_states = w.get('state_dtype') == 'bf16'
+    if bf16_states:
+        h0 = h0.bfloat16()
     dq, dk, dv, dg, db = (x.to(device) for x in (q, k, v, g, beta))
-    # two state pools used alternately: each step streams 2 x 512 MiB, more than the 256 MB Infinity Cache
-    states = [h0.to(device), h0.to(device)]
+    # state pools used in turn: each step streams 2 x 512 MiB, more than the 256 MB Infinity Cache (bf16 states: four
+    # pools of 256 MiB, so that a pool's lines have left the cache when its turn comes again)
+    states = [h0.to(device) for _ in range(4 if bf16_states else 2)]
 
     def step(i):
-        return fused_recurrent_gated_delta_rule(dq, dk, dv, dg, beta=db, initial_state=states[i & 1],
+        return fused_recurrent_gated_delta_rule(dq, dk, dv, dg, beta=db, initial_state=states[i % len(states)],
                                                 output_final_state=True, inplace_final_state=True)
 
     spin_up(step)
@@ -286,16 +293,17 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     t_kernel = statistics.mean(ev[i].elapsed_time(ev[i + 1]) for i in range(steps)) * 1e-3
-    state_bytes = 2 * N * HV * K * V * 4
+    state_bytes = 2 * N * HV * K * V * h0.element_size()
     achieved = state_bytes / t_kernel / 1e9
     roofline = dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
-                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=measured_traffic(w['key']), kernel='gdn_decode_kernel',
+                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=measured_traffic(w['key']),
+                    kernel='gdn_decode_bf16_kernel' if bf16_states else 'gdn_decode_kernel',
                     kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=state_bytes)
     out = dict(value=elapsed / steps * 1e6, ms_per_step=elapsed / steps * 1e3, roofline=roofline)
     if with_cpu:
         from oracle import gdn_oracle as O
         torch.set_num_threads(os.cpu_count() or 1)
-        S = h0.clone()
+        S = h0.float()
         reps = 3
         t0 = time.perf_counter()
         for _ in range(reps):
@@ -484,7 +492,7 @@ def main():
             if name == args.workload:
                 continue
             f2 = bench_prefill if ww['kind'] == 'prefill' else bench_decode
-            r = f2(ww, args.steps, args.warmup, device, ww['kind'] == 'decode' and not args.no_cpu_baseline)
+            r = f2(ww, args.steps, args.warmup, device, name == 'decode' and not args.no_cpu_baseline)
             e = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), roofline=r['roofline'])
             if ww['kind'] == 'prefill':
                 e['tokens_per_s'] = round(r['value'], 1)

@@ -391,6 +391,149 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     }
 }
 
+// The same step with the states held in bf16 in memory (half the traffic of a decode step): K = V = 128, K-first.  The
+// recurrence runs in fp32 registers; the state is rounded (to nearest even) once, when it is written back.  A thread owns
+// 8 value columns (16 bytes of a row) of key rows r0 + 16 i; a wave instruction covers four whole rows.  (Three to five
+// workgroups per CU run at the same speed, two are slower: no cap on the occupancy here.)
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_decode_bf16_kernel(RecurrentParams p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = tid & 15, r0 = tid >> 4;
+    const int64_t inh = xcd_block(p);
+    if (inh < 0) return;
+    const int64_t in = inh / p.HV;
+    const int ihv = (int)(inh % p.HV);
+    const int H = p.H, HV = p.HV;
+    const int ih = ihv / (HV / H);
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    int64_t bos, len;
+    if (p.cu_seqlens) {
+        bos = load_index(p.cu_seqlens, in, cu32);
+        len = load_index(p.cu_seqlens, in + 1, cu32) - bos;
+    } else {
+        bos = in * p.T;
+        len = p.T;
+    }
+    const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
+    const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 8 * c;
+    const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
+    struct Token { T q, k; T v[8]; float g, b; };
+    auto fetch = [&](int64_t tok) {
+        Token x;
+        x.q = x.k = from_f32<T>(0.f);
+        if (tid < 128) { x.q = q[(tok * H + ih) * 128 + tid]; x.k = k[(tok * H + ih) * 128 + tid]; }
+        const T* pv = v + (tok * HV + ihv) * 128 + 8 * c;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x.v[j] = pv[j];
+        x.g = p.g ? load_scalar(p.g, tok * HV + ihv, p.gb_dtype) : 0.f;
+        x.b = p.beta ? load_scalar(p.beta, tok * HV + ihv, p.gb_dtype) : 1.f;
+        return x;
+    };
+    Token cur = {};
+    if (len > 0) cur = fetch(bos);
+    float a_neg = 0.f, dtb = 0.f;
+    if (p.A_log) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+    // ---- the state: 8 requests of 16 bytes (8 bf16) per thread ----
+    const bf16_t* h0 = (const bf16_t*)p.h0;
+    u32x4 raw[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw[i] = __builtin_nontemporal_load((const u32x4*)(h0 + state_off + (r0 + 16 * i) * 128));
+    __shared__ float sh_q[2][128], sh_k[2][128];
+    __shared__ float sh_red[2][4][4];
+    __shared__ float sh_part[2][4][2][128];
+    const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+    float S[8][8];                                       // bf16 -> fp32: the 16 bits become the upper half of the word
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            S[i][2 * j] = __builtin_bit_cast(float, raw[i][j] << 16);
+            S[i][2 * j + 1] = __builtin_bit_cast(float, raw[i][j] & 0xffff0000u);
+        }
+
+    for (int64_t t = 0; t < len; ++t) {
+        const int pb = (int)(t & 1);
+        const int64_t tok = bos + t;
+        const float qv = to_f32(cur.q), kv = to_f32(cur.k);
+        if (tid < 128) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
+        float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
+        if (lane == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
+        float eg = 1.f;
+        if (p.g) {
+            float gt = cur.g;
+            if (p.A_log) gt = a_neg * softplus_f(gt + dtb);
+            eg = __expf(gt);
+        }
+        float bb = cur.b;
+        if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
+        float vv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vv[j] = to_f32(cur.v[j]);
+        if (t + 1 < len) cur = fetch(tok + 1);
+        __syncthreads();
+        sqq = sh_red[pb][0][0] + sh_red[pb][1][0];
+        skk = sh_red[pb][0][1] + sh_red[pb][1][1];
+        sqk = sh_red[pb][0][2] + sh_red[pb][1][2];
+        float rq = p.scale, rk = 1.f;
+        if (p.flags & GDN_FLAG_QK_L2NORM) {
+            rq *= 1.f / sqrtf(sqq + 1e-6f);
+            rk = 1.f / sqrtf(skk + 1e-6f);
+        }
+        const float qk = sqk * rq * rk;
+        float sk[8], sq[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sk[j] = sq[j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float kr = sh_k[pb][r0 + 16 * i], qr = sh_q[pb][r0 + 16 * i];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { sk[j] += S[i][j] * kr; sq[j] += S[i][j] * qr; }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            sk[j] += __shfl_xor(sk[j], 16, 64); sq[j] += __shfl_xor(sq[j], 16, 64);
+            sk[j] += __shfl_xor(sk[j], 32, 64); sq[j] += __shfl_xor(sq[j], 32, 64);
+        }
+        if (lane < 16) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { sh_part[pb][wave][0][8 * c + j] = sk[j]; sh_part[pb][wave][1][8 * c + j] = sq[j]; }
+        }
+        __syncthreads();
+        float d[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int col = 8 * c + j;
+            sk[j] = (sh_part[pb][0][0][col] + sh_part[pb][1][0][col] + sh_part[pb][2][0][col] + sh_part[pb][3][0][col]) * (eg * rk);
+            sq[j] = (sh_part[pb][0][1][col] + sh_part[pb][1][1][col] + sh_part[pb][2][1][col] + sh_part[pb][3][1][col]) * (eg * rq);
+            d[j] = bb * (vv[j] - sk[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float kr = sh_k[pb][r0 + 16 * i] * rk;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) S[i][j] = S[i][j] * eg + d[j] * kr;
+        }
+        if (r0 == 0) {
+            T* po = o + (tok * HV + ihv) * 128 + 8 * c;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) po[j] = from_f32<T>(sq[j] + d[j] * qk);
+        }
+    }
+    if (p.ht) {
+        bf16_t* ht = (bf16_t*)p.ht;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            u32x4 out;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bf16x2 pr = {(bf16_t)S[i][2 * j], (bf16_t)S[i][2 * j + 1]};
+                out[j] = __builtin_bit_cast(uint32_t, pr);
+            }
+            __builtin_nontemporal_store(out, (u32x4*)(ht + state_off + (r0 + 16 * i) * 128));
+        }
+    }
+}
+
 // Grid for xcd_block(): launches that cover the chip several times over hand every XCD runs of `group` consecutive
 // work items (the states of one sequence); smaller ones keep the plain order.
 static int64_t place(RecurrentParams& p, int64_t nblocks, int64_t group) {
@@ -416,6 +559,12 @@ static int launch_vb(const RecurrentParams& p0, int64_t n_states, int vb, hipStr
 template <typename T>
 static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stream) {
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
+    if (p.flags & GDN_FLAG_STATE_BF16) {
+        RecurrentParams pd = p;
+        const int64_t grid = place(pd, n_states, p.HV);
+        hipLaunchKernelGGL(gdn_decode_bf16_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, pd);
+        return check_launch("gdn_decode_bf16_kernel");
+    }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
     if (p.K == 128 && p.V == 128 && !vfirst && !p.gk && !p.gv && n_states >= 1024 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
@@ -477,12 +626,17 @@ extern "C" int gdn_fused_recurrent_fwd(
                   "gdn_fused_recurrent_fwd: num_accepted needs GDN_FLAG_SLOT_PER_TOKEN");
     GDN_CHECK_ARG(!((flags & GDN_FLAG_SLOT_PER_TOKEN) && (flags & GDN_FLAG_STATE_PER_TOKEN)), GDN_ERR_INVALID,
                   "gdn_fused_recurrent_fwd: GDN_FLAG_SLOT_PER_TOKEN and GDN_FLAG_STATE_PER_TOKEN exclude each other");
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_BF16) ||
+                      (h0 && K == 128 && V == 128 && !gk && !gv &&
+                       !(flags & (GDN_FLAG_STATE_V_FIRST | GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))),
+                  GDN_ERR_UNSUPPORTED,
+                  "gdn_fused_recurrent_fwd: bf16 states need h0, K = V = 128, the K-first layout, no gk / gv / beta per column and states per sequence or slot");
     GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_PER_TOKEN) || (ht && ht != h0), GDN_ERR_INVALID,
                   "gdn_fused_recurrent_fwd: GDN_FLAG_STATE_PER_TOKEN needs ht [tokens,HV,K,V] distinct from h0");
     hipStream_t s = (hipStream_t)stream;
     if (T == 0) {
         // no token: the final states are the initial ones (nothing to do for pools and per-token states)
-        if (ht && !state_slots && !(flags & GDN_FLAG_STATE_PER_TOKEN)) return launch_state_copy(h0, ht, N * HV * K * V, s);
+        if (ht && !state_slots && !(flags & GDN_FLAG_STATE_PER_TOKEN)) return launch_state_copy(h0, ht, N * HV * K * V / ((flags & GDN_FLAG_STATE_BF16) ? 2 : 1), s);
         return GDN_OK;
     }
     RecurrentParams p;

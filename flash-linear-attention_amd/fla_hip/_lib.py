@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -28,6 +28,7 @@ FLAG_CU_INT32 = 1 << 5
 FLAG_SLOT_INT32 = 1 << 6
 FLAG_SLOT_PER_TOKEN = 1 << 7
 FLAG_STATE_PER_TOKEN = 1 << 8
+FLAG_STATE_BF16 = 1 << 9
 FLAG_SCAN_WIDE = 1 << 17
 FLAG_SCAN_SEGMENTS = 1 << 18
 FLAG_SEQ_ORDER = 1 << 19

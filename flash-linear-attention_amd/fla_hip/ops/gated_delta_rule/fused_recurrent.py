@@ -46,7 +46,7 @@ def fused_recurrent_gated_delta_rule_fwd(
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Allocates ``o`` (v's dtype) and the fp32 final state, then launches the HIP kernel on
     the current stream.  With ``inplace_final_state`` the final state is written over
-    ``initial_state`` (which must then be fp32 and contiguous) and that tensor is returned.
+    ``initial_state`` (which must then be fp32, or bf16 for states kept in bf16, and contiguous) and that tensor is returned.
     With ``ssm_state_indices`` the states are slots of the pool ``initial_state
     [num_slots, HV, K, V]``: ``[N]`` names one slot per sequence, updated in place; ``[N, T]`` names
     a slot per token (the state after token t goes to slot ``[n, t]``, and the sequence starts from
@@ -145,8 +145,15 @@ def fused_recurrent_gated_delta_rule_fwd(
         if tuple(h0.shape) != state_shape:
             raise ValueError(f'initial_state must have shape {state_shape}, got {tuple(h0.shape)}')
         if inplace_final_state:
-            if h0.dtype != torch.float32 or h0.data_ptr() % 16 != 0:
-                raise ValueError('inplace_final_state needs a contiguous, 16-byte aligned fp32 initial_state')
+            if h0.dtype not in (torch.float32, torch.bfloat16) or h0.data_ptr() % 16 != 0:
+                raise ValueError('inplace_final_state needs a contiguous, 16-byte aligned fp32 (or bf16) initial_state')
+            if h0.dtype == torch.bfloat16:
+                # states kept in bf16 between steps: half the traffic of a decode step; the step itself is fp32
+                if ((K, V) != (128, 128) or state_v_first or gk is not None or gv is not None
+                        or flags & (_lib.FLAG_BETA_VECTOR | _lib.FLAG_SLOT_PER_TOKEN)):
+                    raise NotImplementedError('bf16 states need K = V = 128, the K-first layout, no gk / gv / beta per '
+                                              'column and a state per sequence or per slot')
+                flags |= _lib.FLAG_STATE_BF16
         else:
             h0 = aligned16(as_f32(h0))
 
@@ -210,7 +217,9 @@ def fused_recurrent_gated_delta_rule(
         output_final_state: also return the fp32 final state.
         cu_seqlens: ``[N + 1]`` int32/int64 boundaries of packed sequences (then ``B == 1``).
         inplace_final_state (keyword only, extension): write the final state over
-            ``initial_state`` instead of allocating a new tensor.
+            ``initial_state`` instead of allocating a new tensor.  A bf16 ``initial_state`` (K = V = 128, no
+            ``gk`` / ``gv``) keeps the states in bf16 between calls: the step runs in fp32 and the state is rounded once,
+            when it is written back, so a decode step moves half the bytes.
         ssm_state_indices (keyword only, extension; the sibling KDA operator's argument,
             fla/ops/kda/fused_recurrent.py:248-326): ``[N]`` int32/int64 slot of every sequence in the
             state pool ``initial_state [num_slots, HV, K, V]``; needs ``inplace_final_state=True``.
@@ -260,8 +269,8 @@ def fused_recurrent_gated_delta_rule(
     if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
         raise ValueError('`allow_neg_eigval=True` requires `use_beta_sigmoid_in_kernel=True`.')
     if inplace_final_state and (initial_state is None or not initial_state.is_contiguous()
-                                or initial_state.dtype != torch.float32):
-        raise ValueError('`inplace_final_state=True` requires a contiguous fp32 `initial_state`.')
+                                or initial_state.dtype not in (torch.float32, torch.bfloat16)):
+        raise ValueError('`inplace_final_state=True` requires a contiguous fp32 (or bf16) `initial_state`.')
 
     return fused_recurrent_gated_delta_rule_fwd(
         q, k, v, g, gk, gv, beta, A_log, dt_bias, scale, initial_state, output_final_state,

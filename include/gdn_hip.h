@@ -44,6 +44,7 @@ extern "C" {
 #define GDN_FLAG_SLOT_INT32     (1u << 6)  /* state_slots / num_accepted are int32, else int64  */
 #define GDN_FLAG_SLOT_PER_TOKEN (1u << 7)  /* state_slots is [N, slots_stride]: a slot per token */
 #define GDN_FLAG_STATE_PER_TOKEN (1u << 8) /* ht is [tokens,HV,K,V]: the state after every token */
+#define GDN_FLAG_STATE_BF16     (1u << 9)  /* h0 and ht hold bf16 states (decode at half the state traffic)  */
 /* gdn_chunk_fwd only: force one form of the sequential stage instead of the automatic choice
  * (all forms give the same result up to rounding; used by tests and for tuning)                */
 #define GDN_FLAG_SCAN_WIDE      (1u << 17) /* one workgroup per (sequence, head)                */
@@ -88,6 +89,9 @@ const char* gdn_last_error(void);
  *          entry 0) and the state after its token t is written to slot state_slots[n][t] of ht.
  *   GDN_FLAG_STATE_PER_TOKEN: ht is [B*T,HV,K,V] and receives the state after every token (the reference's
  *          continuous-batching form without inplace_final_state, fused_recurrent.py:212-213); h0 as usual.
+ *   GDN_FLAG_STATE_BF16 (no counterpart in the GDN reference, whose states are fp32): h0 and ht point at bf16 states
+ *          [N or slots,HV,128,128], K-first; the recurrence runs in fp32 registers and the state is rounded once, when
+ *          it is written back.  Needs h0, K = V = 128, no gk / gv / beta per column, states per sequence or per slot.
  *   N = B when cu_seqlens == NULL.  Requires K <= 256, K % 4 == 0, V % 4 == 0, HV % H == 0.
  *   T == 0: ht = h0 (zeros without h0).
  */

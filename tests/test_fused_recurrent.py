@@ -433,6 +433,105 @@ def test_decode_kernel_for_the_common_shape(case):
     _check('ht', ref_ht, ht)
 
 
+@pytest.mark.parametrize('case', ['plain', 'few', 'flags', 'packed', 'slots', 'f16'])
+def test_decode_with_states_kept_in_bf16(case):
+    """A bf16 state updated in place (an option of this library; the reference's GDN states are fp32): the step runs in
+    fp32 from the bf16 values and the state is rounded once on the way back.  Checked against the fp32 oracle started
+    from the same bf16 values: o to the usual bound, the state against the oracle's state rounded to bf16 (at most one
+    unit in the last place apart wherever the fp32 results agree that closely), and over two calls in a row against
+    the oracle with the rounding in between."""
+    H, HV, D = 8, 32, 128
+    dtype = torch.float16 if case == 'f16' else torch.bfloat16
+    kw, okw = {}, {}
+    cu = None
+    N = 3 if case == 'few' else 67                       # 67 x 32 states: placed on the XCDs, the grid rounded up
+    if case == 'packed':
+        lens = [1, 3, 2, 1] * 8
+        cu = [0]
+        for x in lens:
+            cu.append(cu[-1] + x)
+        q, k, v, g, beta, _ = _inputs(1, cu[-1], H, HV, D, dtype, seed=27)
+        N = len(lens)
+    else:
+        q, k, v, g, beta, _ = _inputs(N, 2, H, HV, D, dtype, seed=27)
+    gen = torch.Generator().manual_seed(28)
+    h0 = torch.randn(N, HV, D, D, generator=gen).bfloat16()
+    if case == 'flags':
+        A_log, dt_bias = 0.3 * torch.randn(HV, generator=gen), 0.3 * torch.randn(HV, generator=gen)
+        g, beta = torch.randn(g.shape, generator=gen), torch.randn(beta.shape, generator=gen)
+        okw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, A_log=A_log, dt_bias=dt_bias,
+                   use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True)
+        kw = dict(okw, A_log=A_log.cuda(), dt_bias=dt_bias.cuda())
+    else:
+        okw = kw = dict(use_qk_l2norm_in_kernel=True)
+    dev = 'cuda'
+    cu_t = None if cu is None else torch.tensor(cu, device=dev)
+    dq, dk, dv, dg, db = (x.to(dev) for x in (q, k, v, g, beta))
+
+    def run(state, sl=slice(None)):
+        if case == 'slots':
+            pool = torch.randn(N + 5, HV, D, D, generator=gen).bfloat16()
+            idx = torch.randperm(N + 5, generator=gen)[:N]
+            pool[idx] = state
+            dpool = pool.to(dev)
+            o, ret = _ops()(dq[:, sl], dk[:, sl], dv[:, sl], dg[:, sl], beta=db[:, sl], initial_state=dpool,
+                            inplace_final_state=True, ssm_state_indices=idx.to(dev), **kw)
+            rest = [i for i in range(N + 5) if i not in idx.tolist()]
+            assert torch.equal(dpool[rest].cpu(), pool[rest]), 'slots that are not named must keep their contents'
+            return o, dpool[idx.to(dev)]
+        dstate = state.to(dev)
+        o, ret = _ops()(dq[:, sl], dk[:, sl], dv[:, sl], dg[:, sl], beta=db[:, sl], initial_state=dstate,
+                        inplace_final_state=True, cu_seqlens=cu_t, **kw)
+        assert ret.data_ptr() == dstate.data_ptr() and ret.dtype == torch.bfloat16
+        return o, dstate
+
+    def check_state(name, ref, got):
+        got = got.cpu()
+        assert got.dtype == torch.bfloat16 and not torch.isnan(got.float()).any()
+        want = ref.bfloat16()
+        # one unit in the last place of a bf16 value x is at most 2^-7 |x|
+        off = (got.float() - want.float()).abs() > 2.0 ** -7 * want.float().abs() + 1e-6
+        assert off.float().mean() < 1e-4, f'{name}: {int(off.sum())} of {off.numel()} elements more than one ulp off'
+        assert (got == want).float().mean() > 0.98, f'{name}: only {(got == want).float().mean():.4f} rounded alike'
+        assert O.get_err_ratio(ref, got.float()) <= 3e-3, name
+
+    ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0.float(), True, cu_seqlens=cu, **okw)
+    o, ht = run(h0)
+    _check('o', ref_o, o)
+    check_state('ht', ref_ht, ht)
+    if cu is None:
+        # two calls of one token each: the state passes through bf16 in between
+        r1_o, r1_h = O.recurrent_gated_delta_rule(q[:, :1], k[:, :1], v[:, :1], g[:, :1], beta[:, :1], None, h0.float(), True, **okw)
+        o1, h1 = run(h0, slice(0, 1))
+        check_state('ht after the first call', r1_h, h1)
+        r2_o, r2_h = O.recurrent_gated_delta_rule(q[:, 1:], k[:, 1:], v[:, 1:], g[:, 1:], beta[:, 1:], None,
+                                                  h1.cpu().float(), True, **okw)
+        o2, h2 = run(h1.cpu(), slice(1, 2))
+        _check('o of the second call', r2_o, o2)
+        check_state('ht after the second call', r2_h, h2)
+
+
+def test_bf16_states_are_refused_where_no_kernel_covers_them():
+    dev = 'cuda'
+    q, k, v, g, beta, _ = _inputs(2, 1, 2, 4, 64, torch.bfloat16, seed=1)
+    h0 = torch.zeros(2, 4, 64, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(NotImplementedError, match='bf16 states need'):
+        _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=h0, inplace_final_state=True)
+    # (straight through the C ABI as well)
+    from fla_hip import _lib
+    lib = _lib.load()
+    rc = lib.gdn_fused_recurrent_fwd(*([None] * 9), h0.data_ptr(), h0.data_ptr(), None, None, None, None, 1,
+                                     2, 0, 2, 4, 64, 64, 2, 1.0, 0, 0, _lib.FLAG_STATE_BF16, None)
+    assert rc == _lib.GDN_ERR_UNSUPPORTED and 'bf16 states need' in _lib.last_error()
+    # no token: the states stay as they are
+    q, k, v, g, beta, _ = _inputs(2, 1, 2, 4, 128, torch.bfloat16, seed=1)
+    h0 = torch.randn(2, 4, 128, 128, device=dev).bfloat16()
+    keep = h0.clone()
+    e = lambda x: x[:, :0].to(dev)
+    o, ht = _ops()(e(q), e(k), e(v), e(g), beta=e(beta), initial_state=h0, inplace_final_state=True)
+    assert o.shape == (2, 0, 4, 128) and torch.equal(ht, keep)
+
+
 @pytest.mark.parametrize('N,HV,D,vfirst', [(65, 32, 128, False), (67, 32, 128, True), (75, 32, 64, False), (69, 32, 32, False)])
 def test_workgroup_placement_with_sequence_counts_that_are_not_multiples_of_8(N, HV, D, vfirst):
     """Launches of 2048 or more workgroups hand every XCD runs of consecutive states; the grid is rounded up to whole
