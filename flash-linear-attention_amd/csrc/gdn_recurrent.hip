@@ -22,7 +22,21 @@ struct RecurrentParams {
     int64_t T; int H, HV, K, V, NVB;
     float scale; int gb_dtype; uint32_t flags;
     int xcd_group; int64_t nblocks;      // see xcd_block()
+    // gate per key feature given as a raw input (the KDA operator): 0 = gk is the log decay itself,
+    // 1: gk <- -e^A softplus(gk + bias), 2: gk <- lower sigmoid(e^A (gk + bias)); A = A_log[head] (mode 1 without
+    // A_log: A = 1, mode 2 without: e^A = 1), bias = gk_bias[head][key feature] or 0
+    int gk_act; const float* gk_bias; float gk_lower;
 };
+
+// log decay of key feature `kidx` for token `tok` (see RecurrentParams::gk_act)
+__device__ __forceinline__ float gate_k(const RecurrentParams& p, int64_t tok, int ihv, int kidx, float a_k) {
+    float x = p.gk[(tok * p.HV + ihv) * p.K + kidx];
+    if (p.gk_act) {
+        if (p.gk_bias) x += p.gk_bias[ihv * p.K + kidx];
+        x = p.gk_act == 2 ? p.gk_lower * sigmoid_f(a_k * x) : -a_k * softplus_f(x);
+    }
+    return x;
+}
 
 // Workgroups are dealt to the chip's 8 XCDs round-robin by block index.  With xcd_group = g > 0 the work items (state
 // blocks, consecutive in memory) are handed out so that every XCD works on runs of g consecutive items instead of
@@ -124,7 +138,8 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
 
     const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
     float a_neg = 0.f, dtb = 0.f;
-    if (p.A_log) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+    if (p.A_log && !p.gk_act) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+    const float a_k = p.gk_act ? (p.A_log ? __expf(p.A_log[ihv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
 
     for (int64_t t = 0; t < len; ++t) {
         const int pb = (int)(t & 1);
@@ -142,7 +157,7 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
         float eg = 1.f;
         if (p.g) {
             float gt = load_scalar(p.g, tok * HV + ihv, p.gb_dtype);
-            if (p.A_log) gt = a_neg * softplus_f(gt + dtb);
+            if (p.A_log && !p.gk_act) gt = a_neg * softplus_f(gt + dtb);
             eg = __expf(gt);
         }
         __syncthreads();
@@ -177,7 +192,7 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
                 f32x4 s = S[i] * dgv;
                 if (p.gk) {
                     const int row = r0 + RP * i;
-                    if (row < K) s *= __expf(p.gk[(tok * HV + ihv) * K + row]);
+                    if (row < K) s *= __expf(gate_k(p, tok, ihv, row, a_k));
                 }
                 S[i] = s;
                 sk += s * kr[i];
@@ -233,7 +248,9 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
             qc = *(f32x4*)&sh_q[pb][4 * c] * rq;
             f32x4 dgk = {eg, eg, eg, eg};
             if (p.gk && cont_ok) {
-                const f32x4 x = *(const f32x4*)(p.gk + (tok * HV + ihv) * K + cont_idx);
+                f32x4 x = *(const f32x4*)(p.gk + (tok * HV + ihv) * K + cont_idx);
+                if (p.gk_act) x = f32x4{gate_k(p, tok, ihv, cont_idx, a_k), gate_k(p, tok, ihv, cont_idx + 1, a_k),
+                                        gate_k(p, tok, ihv, cont_idx + 2, a_k), gate_k(p, tok, ihv, cont_idx + 3, a_k)};
                 dgk *= f32x4{__expf(x.x), __expf(x.y), __expf(x.z), __expf(x.w)};
             }
             const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
@@ -596,43 +613,46 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
 
 }  // namespace gdn
 
-extern "C" int gdn_fused_recurrent_fwd(
+// gk_act, gk_bias, gk_lower: see RecurrentParams (0, NULL, 0 for the gated delta rule)
+static int recurrent_entry(
+    const char* who,
     const void* q, const void* k, const void* v,
     const void* g, const void* beta, const float* gk, const float* gv,
     const float* A_log, const float* dt_bias,
     const float* h0, float* ht, void* o,
     const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
-    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream,
+    int gk_act, const float* gk_bias, float gk_lower) {
     using namespace gdn;
-    GDN_CHECK_ARG(T == 0 || (q && k && v && o), GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: q, k, v, o must not be NULL");
+    GDN_CHECK_ARG(T == 0 || (q && k && v && o), GDN_ERR_INVALID, "%s: q, k, v, o must not be NULL", who);
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && K >= 1 && V >= 1 && N >= 1, GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: non-positive dimension");
-    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: HV=%lld not divisible by H=%lld",
+                  "%s: non-positive dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who,
                   (long long)HV, (long long)H);
     GDN_CHECK_ARG(cu_seqlens ? B == 1 : N == B, GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: with cu_seqlens B must be 1; without it N must equal B");
-    GDN_CHECK_ARG(K <= 256, GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: K=%lld > 256", (long long)K);
+                  "%s: with cu_seqlens B must be 1; without it N must equal B", who);
+    GDN_CHECK_ARG(K <= 256, GDN_ERR_UNSUPPORTED, "%s: K=%lld > 256", who, (long long)K);
     GDN_CHECK_ARG(K % 4 == 0 && V % 4 == 0, GDN_ERR_UNSUPPORTED,
-                  "gdn_fused_recurrent_fwd: K=%lld and V=%lld must be multiples of 4", (long long)K, (long long)V);
-    GDN_CHECK_ARG((N + 8) * HV * ((V + 31) / 32) < (1ll << 31), GDN_ERR_UNSUPPORTED, "gdn_fused_recurrent_fwd: grid too large");
+                  "%s: K=%lld and V=%lld must be multiples of 4", who, (long long)K, (long long)V);
+    GDN_CHECK_ARG((N + 8) * HV * ((V + 31) / 32) < (1ll << 31), GDN_ERR_UNSUPPORTED, "%s: grid too large", who);
     GDN_CHECK_ARG(((uintptr_t)h0 % 16) == 0 && ((uintptr_t)ht % 16) == 0 && ((uintptr_t)gk % 16) == 0 &&
                       ((uintptr_t)gv % 16) == 0,
-                  GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: h0/ht/gk/gv must be 16-byte aligned");
-    GDN_CHECK_ARG(!(A_log && !g), GDN_ERR_INVALID, "gdn_fused_recurrent_fwd: A_log given without g");
+                  GDN_ERR_INVALID, "%s: h0/ht/gk/gv must be 16-byte aligned", who);
+    GDN_CHECK_ARG(!(A_log && !g && !gk_act), GDN_ERR_INVALID, "%s: A_log given without g", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_SLOT_PER_TOKEN) || (state_slots && h0 && slots_stride >= 1), GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: GDN_FLAG_SLOT_PER_TOKEN needs state_slots, the pool as h0 and slots_stride >= 1");
+                  "%s: GDN_FLAG_SLOT_PER_TOKEN needs state_slots, the pool as h0 and slots_stride >= 1", who);
     GDN_CHECK_ARG(!num_accepted || (flags & GDN_FLAG_SLOT_PER_TOKEN), GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: num_accepted needs GDN_FLAG_SLOT_PER_TOKEN");
+                  "%s: num_accepted needs GDN_FLAG_SLOT_PER_TOKEN", who);
     GDN_CHECK_ARG(!((flags & GDN_FLAG_SLOT_PER_TOKEN) && (flags & GDN_FLAG_STATE_PER_TOKEN)), GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: GDN_FLAG_SLOT_PER_TOKEN and GDN_FLAG_STATE_PER_TOKEN exclude each other");
+                  "%s: GDN_FLAG_SLOT_PER_TOKEN and GDN_FLAG_STATE_PER_TOKEN exclude each other", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_BF16) ||
                       (h0 && K == 128 && V == 128 && !gk && !gv &&
                        !(flags & (GDN_FLAG_STATE_V_FIRST | GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))),
                   GDN_ERR_UNSUPPORTED,
-                  "gdn_fused_recurrent_fwd: bf16 states need h0, K = V = 128, the K-first layout, no gk / gv / beta per column and states per sequence or slot");
+                  "%s: bf16 states need h0, K = V = 128, the K-first layout, no gk / gv / beta per column and states per sequence or slot", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_PER_TOKEN) || (ht && ht != h0), GDN_ERR_INVALID,
-                  "gdn_fused_recurrent_fwd: GDN_FLAG_STATE_PER_TOKEN needs ht [tokens,HV,K,V] distinct from h0");
+                  "%s: GDN_FLAG_STATE_PER_TOKEN needs ht [tokens,HV,K,V] distinct from h0", who);
     hipStream_t s = (hipStream_t)stream;
     if (T == 0) {
         // no token: the final states are the initial ones (nothing to do for pools and per-token states)
@@ -645,11 +665,42 @@ extern "C" int gdn_fused_recurrent_fwd(
     p.num_accepted = num_accepted; p.slots_stride = slots_stride;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.K = (int)K; p.V = (int)V; p.NVB = 1;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    p.gk_act = gk_act; p.gk_bias = gk_bias; p.gk_lower = gk_lower;
     switch (qkv_dtype) {
         case GDN_DTYPE_BF16: return launch_t<bf16_t>(p, N * HV, s);
         case GDN_DTYPE_F16: return launch_t<f16_t>(p, N * HV, s);
         case GDN_DTYPE_F32: return launch_t<float>(p, N * HV, s);
     }
-    set_error("gdn_fused_recurrent_fwd: unknown qkv_dtype %d", qkv_dtype);
+    set_error("%s: unknown qkv_dtype %d", who, qkv_dtype);
     return GDN_ERR_INVALID;
+}
+
+extern "C" int gdn_fused_recurrent_fwd(
+    const void* q, const void* k, const void* v,
+    const void* g, const void* beta, const float* gk, const float* gv,
+    const float* A_log, const float* dt_bias,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    return recurrent_entry("gdn_fused_recurrent_fwd", q, k, v, g, beta, gk, gv, A_log, dt_bias, h0, ht, o, cu_seqlens, state_slots,
+                           num_accepted, slots_stride, B, T, H, HV, K, V, N, scale, qkv_dtype, gb_dtype, flags, stream, 0, nullptr, 0.f);
+}
+
+// The KDA operator's token recurrence: the gated delta rule with a decay per key feature, g [B,T,HV,K].
+extern "C" int gdn_fused_recurrent_kda_fwd(
+    const void* q, const void* k, const void* v,
+    const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    const char* who = "gdn_fused_recurrent_kda_fwd";
+    GDN_CHECK_ARG(T == 0 || g, GDN_ERR_INVALID, "%s: g must not be NULL", who);
+    GDN_CHECK_ARG(gate_mode >= 0 && gate_mode <= 2, GDN_ERR_INVALID, "%s: gate_mode %d is not 0 (log decays), 1 (softplus) or 2 (bounded sigmoid)", who, gate_mode);
+    GDN_CHECK_ARG(gate_mode != 0 || (!A_log && !dt_bias), GDN_ERR_INVALID, "%s: A_log and dt_bias belong to the gate activation (gate_mode 1 or 2)", who);
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_BF16), GDN_ERR_UNSUPPORTED, "%s: bf16 states are not supported with a decay per key feature", who);
+    return recurrent_entry(who, q, k, v, nullptr, beta, g, nullptr, A_log, nullptr, h0, ht, o, cu_seqlens, state_slots,
+                           num_accepted, slots_stride, B, T, H, HV, K, V, N, scale, qkv_dtype, gb_dtype, flags, stream, gate_mode, dt_bias, lower_bound);
 }

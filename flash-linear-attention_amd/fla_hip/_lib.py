@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -47,6 +47,14 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p,                      # q k v
         c_void_p, c_void_p, c_void_p, c_void_p,            # g beta gk gv
         c_void_p, c_void_p,                                # A_log dt_bias
+        c_void_p, c_void_p, c_void_p,                      # h0 ht o
+        c_void_p, c_void_p, c_void_p, c_int64,             # cu_seqlens state_slots num_accepted slots_stride
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
+        c_float, c_int, c_int, c_uint32, c_void_p]),
+    'gdn_fused_recurrent_kda_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p,                      # q k v
+        c_void_p, c_void_p,                                # g beta
+        c_void_p, c_void_p, c_float, c_int,                # A_log dt_bias lower_bound gate_mode
         c_void_p, c_void_p, c_void_p,                      # h0 ht o
         c_void_p, c_void_p, c_void_p, c_int64,             # cu_seqlens state_slots num_accepted slots_stride
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N

@@ -43,6 +43,8 @@ def fused_recurrent_gated_delta_rule_fwd(
     inplace_final_state: bool = False,
     ssm_state_indices: torch.Tensor | None = None,
     num_accepted_tokens: torch.Tensor | None = None,
+    kda_gate_mode: int | None = None,
+    lower_bound: float = 0.0,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Allocates ``o`` (v's dtype) and the fp32 final state, then launches the HIP kernel on
     the current stream.  With ``inplace_final_state`` the final state is written over
@@ -51,7 +53,10 @@ def fused_recurrent_gated_delta_rule_fwd(
     [num_slots, HV, K, V]``: ``[N]`` names one slot per sequence, updated in place; ``[N, T]`` names
     a slot per token (the state after token t goes to slot ``[n, t]``, and the sequence starts from
     slot ``[n, num_accepted_tokens[n] - 1]``, or ``[n, 0]``).  Without ``inplace_final_state`` the
-    pool is only read and the states after every token are returned as ``[B * T, HV, K, V]``."""
+    pool is only read and the states after every token are returned as ``[B * T, HV, K, V]``.
+    ``kda_gate_mode`` (0, 1, 2) selects the KDA operator's entry point: ``gk`` is then its per-key gate ``g``
+    (mode 0: log decays; 1, 2: raw, activated in the kernel with ``A_log [HV]``, ``dt_bias [HV, K]`` and
+    ``lower_bound``), and ``g``, ``gv`` must be absent."""
     dev = require_gpu(q, k, v)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
@@ -70,6 +75,8 @@ def fused_recurrent_gated_delta_rule_fwd(
         pad = torch.nn.functional.pad
         q, k, v = pad(q, (0, KP - K)), pad(k, (0, KP - K)), pad(v, (0, VP - V))
         gk = None if gk is None else pad(gk, (0, KP - K))
+        if kda_gate_mode and dt_bias is not None:
+            dt_bias = pad(dt_bias.reshape(HV, K), (0, KP - K))
         gv = None if gv is None else pad(gv, (0, VP - V))
         if beta is not None and beta.ndim == v.ndim:
             beta = pad(beta, (0, VP - V))
@@ -169,11 +176,19 @@ def fused_recurrent_gated_delta_rule_fwd(
         final_state = torch.empty(state_shape, dtype=torch.float32, device=dev)
 
     lib = _lib.load()
-    _lib.check(lib.gdn_fused_recurrent_fwd(
-        ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(gk), ptr(gv), ptr(A_log), ptr(dt_bias),
-        ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots), ptr(accepted), slots_stride,
-        B, T, H, HV, KP, VP, N, float(scale), dtype_code(q.dtype), gb_code, flags,
-        current_stream_ptr(dev)))
+    if kda_gate_mode is not None:
+        assert g is None and gv is None and gk is not None
+        _lib.check(lib.gdn_fused_recurrent_kda_fwd(
+            ptr(q), ptr(k), ptr(v), ptr(gk), ptr(beta), ptr(A_log), ptr(dt_bias), float(lower_bound), int(kda_gate_mode),
+            ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots), ptr(accepted), slots_stride,
+            B, T, H, HV, KP, VP, N, float(scale), dtype_code(q.dtype), gb_code, flags,
+            current_stream_ptr(dev)))
+    else:
+        _lib.check(lib.gdn_fused_recurrent_fwd(
+            ptr(q), ptr(k), ptr(v), ptr(g), ptr(beta), ptr(gk), ptr(gv), ptr(A_log), ptr(dt_bias),
+            ptr(h0), ptr(final_state), ptr(o), ptr(cu_seqlens), ptr(slots), ptr(accepted), slots_stride,
+            B, T, H, HV, KP, VP, N, float(scale), dtype_code(q.dtype), gb_code, flags,
+            current_stream_ptr(dev)))
     if padded:
         o = o[..., :V].contiguous()
         if final_state is not None:

@@ -3,10 +3,11 @@
 whole operator and ``fla/modules/backends/triton_ascend`` for module functions).
 
     import fla_hip.upstream
-    fla_hip.upstream.register()        # needs `fla` importable; registers for 'gated_delta_rule' and 'modules'
+    fla_hip.upstream.register()        # needs `fla` importable; registers for 'gated_delta_rule', 'modules' and 'kda'
 
 Upstream's ``@dispatch`` then offers every call of ``chunk_gated_delta_rule``, ``causal_conv1d_fwd``,
-``causal_conv1d_update_states``, ``causal_conv1d_update`` and ``layer_norm_gated_fwd`` to the verifier below first;
+``causal_conv1d_update_states``, ``causal_conv1d_update``, ``layer_norm_gated_fwd`` and ``fused_recurrent_kda_fwd``
+(the KDA operator's token recurrence, ``fla/ops/kda/fused_recurrent.py:236``) to the verifier below first;
 a rejected call (other device, gradients needed, a shape outside the kernels) falls through to upstream's own
 implementation.  The classes are built on whatever ``BaseBackend`` they are given, so the same code serves this
 package's mirror of the registry (used by the tests)."""
@@ -119,9 +120,39 @@ def make_backends(BaseBackend):
     return HipGfx950Backend, HipGfx950ModulesBackend
 
 
+def make_kda_backend(BaseBackend):
+    """Backend for the 'kda' registry: the token recurrence only (the chunked KDA prefill stays upstream)."""
+
+    class HipGfx950KDABackend(BaseBackend):
+        backend_type = 'hip_gfx950'
+        package_name = 'fla_hip'
+        env_var = ENV_VAR
+        default_enable = True
+        priority = 2
+
+        def fused_recurrent_kda_fwd_verifier(self, q, k, v, g, beta, A_log=None, dt_bias=None, initial_state=None, *args, **kwargs):
+            if not _on_gfx950(q):
+                return False, 'not a gfx950 device'
+            if _needs_grad(q, k, v, g, beta, A_log, dt_bias, initial_state):
+                return False, 'forward only: a tensor requires grad'
+            if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+                return False, f'dtype {q.dtype}'
+            if k.shape[-1] > 256:
+                return False, 'key head dim above 256'
+            if initial_state is not None and (initial_state.dtype != torch.float32 or not initial_state.is_contiguous()):
+                return False, 'needs contiguous fp32 states'
+            return True, None
+
+        def fused_recurrent_kda_fwd(self, *args, **kwargs):
+            from fla_hip.ops.kda import fused_recurrent_kda_fwd
+            return fused_recurrent_kda_fwd(*args, **kwargs)
+
+    return HipGfx950KDABackend
+
+
 def register() -> None:
-    """Register both backends with upstream ``fla`` (ImportError when it is not installed).  Importing the two
-    upstream packages first creates their registries (``gdr_registry``, ``modules_registry``)."""
+    """Register the backends with upstream ``fla`` (ImportError when it is not installed).  Importing the two
+    upstream packages first creates their registries (``gdr_registry``, ``modules_registry``, ``kda_registry``)."""
     import importlib
     backends = importlib.import_module('fla.ops.backends')
     gdr = importlib.import_module('fla.ops.gated_delta_rule.backends').gdr_registry
@@ -129,3 +160,5 @@ def register() -> None:
     op_backend, modules_backend = make_backends(backends.BaseBackend)
     gdr.register(op_backend())
     modules.register(modules_backend())
+    kda = importlib.import_module('fla.ops.kda.backends').kda_registry
+    kda.register(make_kda_backend(backends.BaseBackend)())

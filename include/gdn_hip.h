@@ -105,6 +105,26 @@ int gdn_fused_recurrent_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Replaces fla/ops/kda/fused_recurrent.py:236-338 (fused_recurrent_kda_fwd and its kernel :37-233): the token recurrence of
+ * the KDA operator, i.e. the gated delta rule with a decay per key feature,
+ *   S <- diag(e^{g_t}) S;  d = beta_t (v_t - S^T k_t);  S <- S + k_t d^T;  o_t = scale S^T q_t.
+ *   g [B,T,HV,K] fp32.  gate_mode 0: g is the log decay.  gate_mode 1 (use_gate_in_kernel, :168-181): the log decay is
+ *   -exp(A_log[hv]) softplus(g + dt_bias[hv][k]); gate_mode 2 (with a lower bound): lower_bound sigmoid(exp(A_log[hv]) (g + dt_bias[hv][k])).
+ *   A_log [HV] fp32 or NULL (mode 1: exp(1) then, as the reference's kernel; mode 2: factor 1), dt_bias [HV,K] fp32 or NULL.
+ *   Everything else (beta per head or per value column, the flags for the l2 norm of q and k, the beta sigmoid, the V-first
+ *   state layout, packed sequences, state pools with a slot per sequence or per token, states per token) as in
+ *   gdn_fused_recurrent_fwd, on the same kernel; GDN_FLAG_STATE_BF16 is refused.
+ */
+int gdn_fused_recurrent_kda_fwd(
+    const void* q, const void* k, const void* v,
+    const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Bytes of device workspace gdn_chunk_fwd needs for the same N, T, num_chunks (64-token chunks; dense:
  * B*ceil(T/64); packed: sum over sequences of ceil(len/64)), head counts, packed (cu_seqlens given) and flags
  * (the scan flags change the plan and with it the size).  Returns 0 for unsupported (K,V).

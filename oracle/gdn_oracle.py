@@ -18,6 +18,8 @@ reference checkout):
 * ``fla/ops/utils/index.py:113-172``             varlen chunk tables
 * ``fla/modules/l2norm.py:84-109``, ``fla/ops/gated_delta_rule/gate.py:21-46``  prologues
 * ``fla/utils/_testing.py:19-41``                error metric
+* ``fla/ops/kda/naive.py:12-66``, ``fla/ops/kda/gate.py:27-94``, ``fla/ops/kda/fused_recurrent.py:150-181``
+  the KDA operator's token recurrence (a decay per key feature) and its gate activations
 
 Parity pins (all in ``tests/test_oracle.py``): scalar brute force written as
 independent pure-python loops on tiny shapes, closed forms for one decode step
@@ -26,7 +28,9 @@ recurrent == chunked, split-in-time hand-off, varlen == per-sequence loop,
 GVA == repeat_interleave, state_v_first == transpose, and the committed
 fixtures under ``tests/golden/`` (a second set of scalar fixtures pins the
 optional arguments gk, gv, beta per value column and the pooled states of
-speculative decoding).  No function here is "parity unpinned".
+speculative decoding).  The KDA recurrence is the gk branch of the token recurrence (pinned by those
+fixtures); its gate activations are pinned by values that the formulas fix (``test_kda_gate_pins``).
+No function here is "parity unpinned".
 
 Everything is computed in ``dtype`` (float32 by default, float64 for tight
 pins); inputs are upcast first, so bf16 inputs are consumed as their exact
@@ -77,6 +81,24 @@ def gdn_gate(g: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor | None 
     if dt_bias is not None:
         g = g + dt_bias.float()
     return -A_log.float().exp() * F.softplus(g)
+
+
+def kda_gate(g: torch.Tensor, A_log: torch.Tensor | None = None, dt_bias: torch.Tensor | None = None,
+             lower_bound: float | None = None) -> torch.Tensor:
+    """Log decay per key feature from the raw gate g [..., HV, K] (fla/ops/kda/gate.py:27-94): with a bias
+    dt_bias [HV * K] added first, ``-exp(A_log[hv]) * softplus(g)``, or with a lower bound
+    ``lower_bound * sigmoid(exp(A_log[hv]) * g)``.  Without A_log the factor is 1 under the sigmoid and exp(1) in
+    front of the softplus (the recurrent kernel's constant, fla/ops/kda/fused_recurrent.py:168-181)."""
+    HV, K = g.shape[-2:]
+    x = g.float()
+    if dt_bias is not None:
+        x = x + dt_bias.float().reshape(HV, K)
+    if lower_bound is not None:
+        if A_log is not None:
+            x = x * A_log.float().exp().reshape(HV, 1)
+        return lower_bound * torch.sigmoid(x)
+    a = A_log.float().exp().reshape(HV, 1) if A_log is not None else math.e
+    return -a * F.softplus(x)
 
 
 # --------------------------------------------------------------------------- #
@@ -184,9 +206,24 @@ def recurrent_gated_delta_rule(
     return o, (ht.transpose(-1, -2).contiguous() if state_v_first else ht)
 
 
+def recurrent_kda(
+    q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
+    use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, A_log=None, dt_bias=None, lower_bound=None,
+    use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, state_v_first=False, dtype=torch.float32,
+):
+    """Token recurrence of the KDA operator (fla/ops/kda/naive.py:12-66): per token S *= exp(g)[:, None] with
+    g [B,T,HV,K] a decay per key feature, then the delta-rule update and the read-out of the gated delta rule.
+    With use_gate_in_kernel g is the raw gate (kda_gate)."""
+    gk = kda_gate(g, A_log, dt_bias, lower_bound) if use_gate_in_kernel else g
+    return recurrent_gated_delta_rule(
+        q, k, v, None, beta, scale, initial_state, output_final_state, cu_seqlens, gk=gk,
+        use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel,
+        allow_neg_eigval=allow_neg_eigval, state_v_first=state_v_first, dtype=dtype)
+
+
 def recurrent_gated_delta_rule_pooled(
     q, k, v, g, beta, scale, pool, ssm_state_indices, num_accepted_tokens=None, cu_seqlens=None,
-    dtype=torch.float32, **flags,
+    dtype=torch.float32, gk=None, **flags,
 ):
     """Token recurrence over states kept in a pool [num_slots,HV,K,V] (continuous batching and
     speculative decoding, fla/ops/kda/fused_recurrent.py:131-145,203-219).
@@ -212,7 +249,7 @@ def recurrent_gated_delta_rule_pooled(
         S = pool[first:first + 1].to(dtype)
         for t in range(s, e):
             sl = lambda x: None if x is None else x[b:b + 1, t:t + 1]
-            o1, S = recurrent_gated_delta_rule(sl(q), sl(k), sl(v), sl(g), sl(beta), scale, S, True, dtype=dtype, **flags)
+            o1, S = recurrent_gated_delta_rule(sl(q), sl(k), sl(v), sl(g), sl(beta), scale, S, True, dtype=dtype, gk=sl(gk), **flags)
             o[b, t] = o1[0, 0]
             per_token[b * T + t] = S[0]
             if idx.dim() == 2:

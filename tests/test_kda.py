@@ -1,0 +1,218 @@
+"""The KDA operator's token recurrence (fused_recurrent_kda, fused_recurrent_kda_fwd: a decay per key feature) on the
+gated delta rule's HIP recurrence kernel, through gdn_fused_recurrent_kda_fwd, against the CPU oracle.  Shapes, input
+recipes and the 0.005 bar of the reference's own tests (tests/ops/test_kda.py:100-330: fp32, q and k uniform in [0, 1)
+and normalised, g = logsigmoid(randn) / normalizer, beta = sigmoid(randn), random initial state)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+pytestmark = pytest.mark.gpu
+RATIO = 5e-3
+
+
+def _ops():
+    from fla_hip.ops.kda import fused_recurrent_kda, fused_recurrent_kda_fwd
+    return fused_recurrent_kda, fused_recurrent_kda_fwd
+
+
+def _check(name, ref, got, ratio=RATIO):
+    got = got.detach().float().cpu()
+    assert got.shape == ref.shape, f'{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}'
+    assert not torch.isnan(got).any(), f'{name}: NaN'
+    r, m = O.get_err_ratio(ref, got), O.max_abs_ratio(ref, got)
+    assert r <= ratio and m <= 1e-2, f'{name}: rel-rmse {r:.3e} max-abs ratio {m:.3e}'
+
+
+def _inputs(B, T, H, HV, D, dtype=torch.float32, normalizer=1.0, seed=42, raw_gate=False):
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    k = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    v = torch.rand(B, T, HV, D, generator=gen).to(dtype)
+    g = torch.randn(B, T, HV, D, generator=gen)
+    if not raw_gate:
+        g = F.logsigmoid(g) / normalizer
+    beta = torch.randn(B, T, HV, generator=gen).to(dtype).sigmoid()
+    h0 = torch.randn(B, HV, D, D, generator=gen)
+    return q, k, v, g, beta, h0
+
+
+def _cuda(*xs):
+    return [None if x is None else x.cuda() for x in xs]
+
+
+@pytest.mark.parametrize('B,T,H,HV,D,scale,normalizer,l2,dtype', [
+    (1, 64, 1, 1, 64, 1, 1, False, torch.float32),
+    (2, 512, 3, 3, 60, 1, 1, False, torch.float32),
+    (3, 1000, 4, 4, 100, 0.1, 1, True, torch.float32),
+    (4, 1024, 4, 4, 128, 0.1, 1, False, torch.float32),
+    (2, 512, 2, 4, 60, 1, 1, False, torch.float32),
+    (2, 1024, 2, 8, 128, 0.1, 1, True, torch.float32),
+    (2, 300, 2, 4, 128, 0.1, 10, True, torch.bfloat16),
+    (1, 200, 2, 2, 256, 1, 1, False, torch.float16),
+])
+def test_fused_recurrent_kda_reference_matrix(B, T, H, HV, D, scale, normalizer, l2, dtype):
+    q, k, v, g, beta, h0 = _inputs(B, T, H, HV, D, dtype, normalizer)
+    if not l2:
+        q, k = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, scale, h0, True, use_qk_l2norm_in_kernel=l2)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta, h0)
+    keep = dh.clone()
+    o, ht = _ops()[0](dq, dk, dv, dg, db, scale=scale, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and torch.equal(dh, keep)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+
+
+@pytest.mark.parametrize('B,T,H,D,neg', [(2, 256, 4, 64, False), (2, 256, 4, 64, True), (1, 512, 3, 60, True)])
+def test_fused_recurrent_kda_beta_sigmoid_in_kernel(B, T, H, D, neg):
+    q, k, v, g, beta_post, h0 = _inputs(B, T, H, H, D)
+    q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    beta_raw = torch.logit(beta_post.clamp(1e-4, 1 - 1e-4))
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta_post * (2 if neg else 1), None, h0, True)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta_raw, h0)
+    o, ht = _ops()[0](dq, dk, dv, dg, db, initial_state=dh, output_final_state=True,
+                      use_beta_sigmoid_in_kernel=True, allow_neg_eigval=neg)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    with pytest.raises(ValueError, match='allow_neg_eigval'):
+        _ops()[0](dq, dk, dv, dg, db, allow_neg_eigval=True)
+
+
+@pytest.mark.parametrize('B,T,H,D,scale', [(1, 64, 1, 64, 1), (2, 512, 3, 60, 1), (3, 1000, 4, 100, 0.1), (4, 1024, 4, 128, 0.1)])
+def test_fused_recurrent_kda_state_v_first(B, T, H, D, scale):
+    q, k, v, g, beta, h0 = _inputs(B, T, H, H, D)
+    q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, scale, h0, True)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta, h0.transpose(-1, -2).contiguous())
+    o, ht = _ops()[0](dq, dk, dv, dg, db, scale=scale, initial_state=dh, output_final_state=True, state_v_first=True)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht.transpose(-1, -2))
+
+
+@pytest.mark.parametrize('mode', ['softplus', 'softplus-no-bias', 'bounded', 'bounded-no-A', 'softplus-no-A'])
+@pytest.mark.parametrize('H,HV,D,vfirst', [(2, 4, 64, False), (3, 3, 100, True), (2, 2, 128, False)])
+def test_fused_recurrent_kda_gate_in_kernel(mode, H, HV, D, vfirst):
+    """The raw gate activated in the kernel (fla/ops/kda/fused_recurrent.py:168-181): both forms, with and without
+    A_log and the bias [HV * K]; the reference's layer draws A_log = log(U(1, 16)) and a bias of softplus-inverse values."""
+    B, T = 2, 150
+    q, k, v, g, beta, h0 = _inputs(B, T, H, HV, D, raw_gate=True, seed=7)
+    gen = torch.Generator().manual_seed(8)
+    A_log = torch.log(1 + 15 * torch.rand(HV, generator=gen)) if 'no-A' not in mode else None
+    dt_bias = torch.randn(HV * D, generator=gen) if 'no-bias' not in mode else None
+    lower = -5.0 if mode.startswith('bounded') else None
+    if mode == 'softplus':
+        g = g - 4.0                      # (keeps the decay of 150 tokens from wiping the state)
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True, lower_bound=lower)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, A_log=A_log, dt_bias=dt_bias, **kw)
+    kw['state_v_first'] = vfirst
+    dq, dk, dv, dg, db, dh, dA, dbias = _cuda(q, k, v, g, beta, h0.transpose(-1, -2).contiguous() if vfirst else h0, A_log, dt_bias)
+    o, ht = _ops()[0](dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=dh, output_final_state=True, **kw)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht.transpose(-1, -2) if vfirst else ht)
+    # the gate applied on the host and passed as log decays gives the same numbers up to the activation's rounding
+    gk = O.kda_gate(g, A_log, dt_bias, lower).cuda()
+    o2, ht2 = _ops()[0](dq, dk, dv, gk, db, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=True, state_v_first=vfirst)
+    _check('o (host gate)', o2.float().cpu(), o, 1e-4)
+    _check('ht (host gate)', ht2.cpu(), ht, 1e-4)
+
+
+@pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
+def test_fused_recurrent_kda_packed(idx_dtype):
+    cu = [0, 15, 16, 100, 356, 357, 1000]
+    T, N, H, HV, D = cu[-1], len(cu) - 1, 2, 4, 64
+    q, k, v, g, beta, _ = _inputs(1, T, H, HV, D, seed=3)
+    h0 = torch.randn(N, HV, D, D, generator=torch.Generator().manual_seed(4))
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, use_qk_l2norm_in_kernel=True)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta, h0)
+    o, ht = _ops()[0](dq, dk, dv, dg, db, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=True,
+                      cu_seqlens=torch.tensor(cu, dtype=idx_dtype, device='cuda'))
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    with pytest.raises(ValueError, match='number of initial states'):
+        _ops()[0](dq, dk, dv, dg, db, initial_state=dh[:2], cu_seqlens=torch.tensor(cu, device='cuda'))
+    with pytest.raises(ValueError, match='batch size is expected to be 1'):
+        _ops()[0](dq.expand(2, -1, -1, -1), dk, dv, dg, db, cu_seqlens=torch.tensor(cu, device='cuda'))
+
+
+def test_fused_recurrent_kda_fwd_state_pool_and_speculative_decoding():
+    """The serving form (fla/ops/kda/fused_recurrent.py:236-338): states in a pool, in place by default; a slot per
+    sequence, and a slot per token with the start taken from the slot of the last accepted token."""
+    N, H, HV, D, slots = 5, 2, 4, 64, 23
+    fwd = _ops()[1]
+    gen = torch.Generator().manual_seed(11)
+    pool = torch.randn(slots, HV, D, D, generator=gen)
+    # one token per sequence, a slot per sequence, gate activated in the kernel
+    q, k, v, g, beta, _ = _inputs(N, 1, H, HV, D, raw_gate=True, seed=12)
+    A_log, dt_bias = torch.log(1 + 15 * torch.rand(HV, generator=gen)), torch.randn(HV * D, generator=gen)
+    idx = torch.randperm(slots, generator=gen)[:N]
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=True)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, pool[idx], True, A_log=A_log, dt_bias=dt_bias, **kw)
+    dq, dk, dv, dg, db, dpool, dA, dbias = _cuda(q, k, v, g, beta, pool, A_log, dt_bias)
+    o, ret = fwd(dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=dpool, ssm_state_indices=idx.cuda(), **kw)
+    assert ret.data_ptr() == dpool.data_ptr()
+    _check('o', ref_o, o)
+    _check('pool slots', ref_ht, dpool[idx.cuda()])
+    rest = [i for i in range(slots) if i not in idx.tolist()]
+    assert torch.equal(dpool[rest].cpu(), pool[rest])
+    # three draft tokens per sequence, a slot per token, starts from the slot of the last accepted token
+    T = 3
+    q, k, v, g, beta, _ = _inputs(N, T, H, HV, D, seed=13)
+    idx2 = torch.randperm(slots, generator=gen)[:N * T].view(N, T).to(torch.int32)
+    acc = torch.tensor([1, 3, 2, 1, 2], dtype=torch.int32)
+    gk = g
+    ref_o, ref_pool, _ = O.recurrent_gated_delta_rule_pooled(q, k, v, None, beta, D ** -0.5, pool, idx2, acc, gk=gk, use_qk_l2norm_in_kernel=True)
+    dq, dk, dv, dg, db, dpool = _cuda(q, k, v, g, beta, pool)
+    o, _ = fwd(dq, dk, dv, dg, db, initial_state=dpool, ssm_state_indices=idx2.cuda(), num_accepted_tokens=acc.cuda(),
+               use_qk_l2norm_in_kernel=True)
+    _check('o (speculative)', ref_o, o)
+    _check('pool (speculative)', ref_pool, dpool)
+    # `out` receives the result; in-place without a state is refused
+    buf = torch.empty_like(dv)
+    o2, _ = fwd(dq, dk, dv, dg, db, initial_state=dpool.clone(), ssm_state_indices=idx2.cuda(), num_accepted_tokens=acc.cuda(),
+                use_qk_l2norm_in_kernel=True, out=buf)
+    assert o2.data_ptr() == buf.data_ptr()
+    with pytest.raises(ValueError, match='requires `initial_state`'):
+        fwd(dq, dk, dv, dg, db)
+
+
+def test_kda_entry_point_argument_checks():
+    from fla_hip import _lib
+    lib = _lib.load()
+    x = torch.zeros(2, 1, 2, 64, device='cuda')
+    g = torch.zeros(2, 1, 2, 64, device='cuda')
+    b = torch.zeros(2, 1, 2, device='cuda')
+    A = torch.zeros(2, device='cuda')
+    args = lambda A_log, mode, flags: (x.data_ptr(), x.data_ptr(), x.data_ptr(), g.data_ptr(), b.data_ptr(), A_log, None, 0.0, mode,
+                                        None, None, x.data_ptr(), None, None, None, 1, 2, 1, 2, 2, 64, 64, 2, 1.0,
+                                        _lib.DTYPE_F32, _lib.DTYPE_F32, flags, None)
+    assert lib.gdn_fused_recurrent_kda_fwd(*args(None, 3, 0)) == _lib.GDN_ERR_INVALID and 'gate_mode' in _lib.last_error()
+    assert lib.gdn_fused_recurrent_kda_fwd(*args(A.data_ptr(), 0, 0)) == _lib.GDN_ERR_INVALID and 'A_log' in _lib.last_error()
+    assert lib.gdn_fused_recurrent_kda_fwd(*args(None, 0, _lib.FLAG_STATE_BF16)) == _lib.GDN_ERR_UNSUPPORTED
+    assert lib.gdn_fused_recurrent_kda_fwd(*args(A.data_ptr(), 1, 0)) == _lib.GDN_OK
+    torch.cuda.synchronize()
+
+
+def test_upstream_kda_backend_takes_gpu_inference_calls_and_leaves_the_rest():
+    """The backend for upstream's 'kda' registry (fla/ops/kda/backends/__init__.py:14), through this package's mirror of
+    the registry: GPU inference calls of fused_recurrent_kda_fwd run the HIP kernel, everything else the default."""
+    from fla_hip.ops.backends import BackendRegistry, BaseBackend, dispatch
+    from fla_hip.upstream import make_kda_backend
+    BackendRegistry('upstream_test_kda').register(make_kda_backend(BaseBackend)())
+
+    @dispatch('upstream_test_kda')
+    def fused_recurrent_kda_fwd(q, k, v, g, beta, A_log=None, dt_bias=None, initial_state=None, scale=None,
+                                output_final_state=False, inplace_final_state=True, **kwargs):
+        return 'default', None
+
+    q, k, v, g, beta, h0 = _inputs(2, 5, 2, 4, 64)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, use_qk_l2norm_in_kernel=True)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta, h0)
+    o, ht = fused_recurrent_kda_fwd(dq, dk, dv, dg, db, initial_state=dh, use_qk_l2norm_in_kernel=True)
+    assert ht.data_ptr() == dh.data_ptr()                    # in place by default, as upstream
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    assert fused_recurrent_kda_fwd(q, k, v, g, beta, initial_state=h0)[0] == 'default'                       # CPU stays upstream
+    assert fused_recurrent_kda_fwd(dq.requires_grad_(), dk, dv, dg, db, initial_state=dh)[0] == 'default'    # training stays upstream
+    assert fused_recurrent_kda_fwd(dq.detach(), dk, dv, dg, db, initial_state=dh.bfloat16())[0] == 'default'

@@ -65,6 +65,50 @@ def test_optional_decays_and_vector_beta_match_scalar_fixture(name):
     assert _ext(name, 'gk') is None or _ext(name, 'gv') is None or _ext(name, 'gk').shape != _ext(name, 'gv').shape
 
 
+def test_kda_recurrence_matches_scalar_fixture():
+    # the KDA operator's recurrence is the token recurrence with a decay per key feature and no scalar gate: the fixture
+    # of that form, from the independent scalar loop
+    name = 'gk_only_varlen'
+    assert _ext(name, 'g') is None and _ext(name, 'gv') is None
+    b1 = lambda x: x[None]
+    o, ht = O.recurrent_kda(b1(_ext(name, 'q')), b1(_ext(name, 'k')), b1(_ext(name, 'v')), b1(_ext(name, 'gk')), b1(_ext(name, 'beta')),
+                            float(GOLD_EXT[f'{name}.scale']), _ext(name, 'h0'), True, cu_seqlens=GOLD_EXT[f'{name}.cu'].tolist(),
+                            dtype=torch.float64)
+    assert torch.allclose(o[0], _ext(name, 'o'), atol=1e-12, rtol=1e-10)
+    assert torch.allclose(ht, _ext(name, 'ht'), atol=1e-12, rtol=1e-10)
+
+
+def test_kda_gate_pins():
+    """Values that the two gate formulas fix (fla/ops/kda/gate.py:27-94), chosen so that a wrong sign, a bias added
+    after the activation, A applied outside the sigmoid or a bias indexed [K][HV] instead of [HV][K] fails."""
+    HV, K = 2, 3
+    z = torch.zeros(1, 1, HV, K)
+    A = torch.tensor([0.0, math.log(2.0)])
+    # softplus form: -e^A ln 2 at zero input; head 1 decays twice as fast; ~ -e^A x for large x
+    out = O.kda_gate(z, A)
+    assert torch.allclose(out[0, 0, 0], torch.full((K,), -math.log(2.0))) and torch.allclose(out[0, 0, 1], torch.full((K,), -2 * math.log(2.0)))
+    assert torch.allclose(O.kda_gate(z + 30.0, A)[0, 0, :, 0], torch.tensor([-30.0, -60.0]), atol=1e-5)
+    assert (O.kda_gate(torch.randn(2, 5, HV, K), A) < 0).all()
+    # the bias is added before the activation and is laid out [HV][K]
+    bias = torch.zeros(HV * K)
+    bias[1 * K + 2] = 30.0                      # head 1, key feature 2
+    out = O.kda_gate(z, A, bias)
+    assert abs(float(out[0, 0, 1, 2]) + 60.0) < 1e-4
+    rest = out.clone(); rest[0, 0, 1, 2] = O.kda_gate(z, A)[0, 0, 1, 2]
+    assert torch.equal(rest, O.kda_gate(z, A))
+    # without A_log the kernel's constant is exp(1)
+    assert torch.allclose(O.kda_gate(z), torch.full((1, 1, HV, K), -math.e * math.log(2.0)))
+    # bounded form: lower_bound / 2 at zero input, A multiplies inside the sigmoid, the bound is reached for large inputs
+    lb = -5.0
+    assert torch.allclose(O.kda_gate(z, A, None, lb), torch.full((1, 1, HV, K), lb / 2))
+    out = O.kda_gate(z + 1.0, torch.tensor([0.0, math.log(3.0)]), None, lb)
+    assert torch.allclose(out[0, 0, :, 0], torch.tensor([lb / (1 + math.exp(-1.0)), lb / (1 + math.exp(-3.0))]))
+    assert torch.allclose(O.kda_gate(z + 40.0, None, None, lb), torch.full((1, 1, HV, K), lb))
+    assert torch.allclose(O.kda_gate(z - 40.0, None, None, lb), torch.zeros(1, 1, HV, K), atol=1e-6)
+    out = O.kda_gate(z, None, bias, lb)
+    assert abs(float(out[0, 0, 1, 2]) - lb) < 1e-6 and abs(float(out[0, 0, 0, 2]) - lb / 2) < 1e-6
+
+
 def test_pooled_states_of_speculative_decoding_match_scalar_fixture():
     n = 'spec_pool'
     o, pool_after, _ = O.recurrent_gated_delta_rule_pooled(
