@@ -231,9 +231,11 @@ struct SegmentPlan {
 // starts at chunk 0 from the true initial state and is exact.  -1: not within `cap` chunks.  `bound` points at the
 // entry of chunk 0 of the sequence for this head; entries of consecutive chunks are HV apart.  Lane l looks at
 // chunk it0 - 1 - l; the result is the same in every lane.
-__device__ __forceinline__ int warm_chunks(const float* bound, int HV, int64_t it0, int cap, int lane) {
+__device__ __forceinline__ float warm_load(const float* bound, int HV, int64_t it0, int cap, int lane) {
+    return (lane < cap && lane < it0) ? bound[(it0 - 1 - lane) * HV] : 0.f;
+}
+__device__ __forceinline__ int warm_from(float x, int64_t it0, int cap, int lane) {
     const bool in = lane < cap && lane < it0;
-    float x = in ? bound[(it0 - 1 - lane) * HV] : 0.f;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const float y = __shfl_up(x, off, 64);
@@ -243,12 +245,29 @@ __device__ __forceinline__ int warm_chunks(const float* bound, int HV, int64_t i
     if (hit) return __builtin_ctzll(hit) + 1;
     return it0 <= cap ? (int)it0 : -1;
 }
+__device__ __forceinline__ int warm_chunks(const float* bound, int HV, int64_t it0, int cap, int lane) {
+    return warm_from(warm_load(bound, HV, it0, cap, lane), it0, cap, lane);
+}
 
 // Whether the segments of this (sequence, head) need the exact start states of the first pass and the merge:
-// true when some segment cannot be warm-started within the cap.
-__device__ __forceinline__ bool needs_exact_segments(const SegmentPlan& sp, const float* bound, int HV, int lane) {
+// true when some segment cannot be warm-started within the cap.  The bounds of eight segments are requested
+// before the first is looked at (every workgroup of three launches waits for this answer before anything else).
+// `warm_of` (optional) receives warm_chunks() of segment `seg`.
+__device__ __forceinline__ bool needs_exact_segments(const SegmentPlan& sp, const float* bound, int HV, int lane,
+                                                     int seg = -1, int* warm_of = nullptr) {
     bool exact = false;
-    for (int j = 1; j < sp.nseg; ++j) exact |= warm_chunks(bound, HV, (int64_t)j * sp.seg_chunks, sp.warm_cap, lane) < 0;
+    for (int j0 = 1; j0 < sp.nseg; j0 += 8) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = j0 + e < sp.nseg ? warm_load(bound, HV, (int64_t)(j0 + e) * sp.seg_chunks, sp.warm_cap, lane) : 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (j0 + e >= sp.nseg) break;
+            const int wch = warm_from(x[e], (int64_t)(j0 + e) * sp.seg_chunks, sp.warm_cap, lane);
+            exact |= wch < 0;
+            if (warm_of && j0 + e == seg) *warm_of = wch;
+        }
+    }
     return exact;
 }
 

@@ -131,8 +131,9 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
             // the start of the sequence) and produce no output until the segment proper.  Heads with a segment that
             // cannot be started this way take the exact start states of the first pass and the merge.
             const float* bnd = sp.bound ? sp.bound + (inh / HV) * p.NT * HV + inh % HV : nullptr;
-            if (bnd && !needs_exact_segments(sp, bnd, HV, lane)) {
-                warm = __builtin_amdgcn_readfirstlane(warm_chunks(bnd, HV, (int64_t)seg * sp.seg_chunks, sp.warm_cap, lane));
+            int wch = 0;
+            if (bnd && !needs_exact_segments(sp, bnd, HV, lane, seg, &wch)) {
+                warm = __builtin_amdgcn_readfirstlane(wch);
                 if ((int64_t)seg * sp.seg_chunks - warm == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
                 else init = 2;
             } else {

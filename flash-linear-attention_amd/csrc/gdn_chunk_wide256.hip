@@ -68,9 +68,10 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     bool whole = nseg == 1;
     if (nseg > 1) {
         const float* bnd = sp.bound + n * p.NT * HV + hv;
-        whole = needs_exact_segments(sp, bnd, HV, lane);
+        int wch = 0;
+        whole = needs_exact_segments(sp, bnd, HV, lane, seg, &wch);
         if (whole && seg > 0) return;
-        if (!whole && seg > 0) warm = __builtin_amdgcn_readfirstlane(warm_chunks(bnd, HV, (int64_t)seg * sp.seg_chunks, sp.warm_cap, lane));
+        if (!whole && seg > 0) warm = __builtin_amdgcn_readfirstlane(wch);
     }
     const bool from_start = whole || (int64_t)seg * sp.seg_chunks - warm == 0, to_end = whole || seg == nseg - 1;
     const float* src = p.h0 && from_start ? p.h0 + inh * (int64_t)(K * V) : nullptr;
