@@ -1,47 +1,64 @@
-// Chunk-parallel stage of the chunked prefill: one workgroup per (chunk, q/k head) computes
-// what does not depend on the running state and is not a plain copy of the inputs, for every
-// value head of that q/k head:
-//   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  X = (I+L)^-1 in fp32 (16x16 forward
-//   substitution on the diagonal blocks, fp32-MFMA block merges),  Xb = X diag(beta),
-//   P = scale*tril(q k^T * 2^(G_i-G_j)),  and the per-token gate tables.
-// Optional prologues of the reference are folded in: the gate and beta activations, and the l2
-// normalisation of q and k as per-row factors 1/|k_t|, 1/|q_t| on L, P and the tables (so the
-// sequential stage reads q and k exactly as the caller gave them).
-// The raw products K K^T and q K^T are formed once and stay in registers; the value heads differ
-// only in their gates.  Xb and P are written in the exact register order ("fragments") in which
-// the scan kernel feeds them to the matrix cores; the scan forms v_new = Xb (v - 2^G (k S)) itself
-// from the raw k and v, so neither w = Xb 2^G k nor u = Xb v is ever materialised.
+// Chunk-parallel stage of the chunked prefill: one WAVE per (chunk, value head) computes what does not depend on the
+// running state and is not a plain copy of the inputs:
+//   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  X = (I+L)^-1 in fp32,  Xb = X diag(beta),
+//   the per-token gate tables, a bound on the chunk's transition, and on request P = scale*tril(q k^T * 2^(G_i-G_j)).
+// Optional prologues of the reference are folded in: the gate and beta activations, and the l2 normalisation of q and
+// k as per-row factors 1/|k_t|, 1/|q_t| on L, P and the tables (so the sequential stage reads q and k exactly as the
+// caller gave them).  Xb and P are written in the exact register order ("fragments") in which the scan kernel feeds
+// them to the matrix cores; the scan forms v_new = Xb (v - 2^G (k S)) itself from the raw k and v, so neither
+// w = Xb 2^G k nor u = Xb v is ever materialised.
+//
+// A wave shares nothing with the other waves of its workgroup, so there is no workgroup barrier:
+//   * The k rows are loaded straight into matrix-core operand registers (the operand layout of A and of B is the same:
+//     lane (c16, g) holds 8 features of token row c16), so K K^T needs no LDS; the value heads of a q/k head sit in
+//     neighbouring waves and read the same lines.
+//   * Everything is kept TRANSPOSED: the raw tile (a, b), a <= b, holds (k_j . k_i) for rows j of t-tile a and columns i
+//     of t-tile b, gated it is U = L^T, and T = X^T = (I + U)^-1 is upper triangular.  A tile in accumulator layout
+//     (lane (c16, g): rows 4g..4g+3, column c16) serves directly as the RIGHT factor of a product on the fp32 matrix
+//     cores (step e contracts over the indices {4g + e}), the left factor comes from LDS by rows, and the result is
+//     again in accumulator layout.  The transposed X in accumulator layout is also exactly the order of the Xb operand
+//     fragments (row c16, columns 4g + e): results go from registers to memory.
+//   * Diagonal 16x16 blocks: lane group g inverts block g by substitution, one row of X per lane (all 64 lanes busy).
+//     Merges: T(lo,hi) = -(T(lo,lo) U(lo,hi)) T(hi,hi) on 16-tiles, then on 32-blocks with the zero tiles left out: the gated
+//     tiles U are right factors and never leave the registers, only the products T U pass through LDS.
 #include "gdn_chunk_common.h"
 
 namespace gdn {
 
-constexpr int NP = 128 + 8;     // pitch (elements) of the staged 64x128 tiles: 272 B rows, conflict-free 16 B reads
-constexpr int LP = 68;          // pitch (floats) of the 64x64 fp32 matrices
-// two tiles (k then L, q then X), the transposed diagonal blocks of L, the row factors of k and q, and gates + beta
-// of every value head of the group
-inline size_t prep_smem(int group) { return 2 * CH * NP * 2 + 4 * 16 * 16 * 4 + 3 * CH * 4 + (size_t)group * 2 * CH * 4; }
+// LDS per wave: seven 16x16 fp32 tiles that serve as left factors.  The diagonal blocks of L (by rows) and the three gate
+// tables lie where the transposed diagonal blocks of X go afterwards, |k|^2 and 1/|q| where the first products go
+// afterwards: 8.75 KB, four workgroups per CU.
+constexpr int TP = 20;                                       // pitch (floats) of a 16x16 fp32 tile in LDS
+constexpr int PW_FLOATS = 7 * 16 * TP;                       // 2240 floats per wave
+constexpr int PW_WAVES = 4;                                  // waves per workgroup: small workgroups keep the CU's wave slots filled
+constexpr size_t PREP_SMEM = (size_t)PW_WAVES * PW_FLOATS * 4;
 
-template <typename T>
-__global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p) {
+// WANT_P: also the records' P (for callers that look at the records; the scan kernels form P themselves): keeps the q
+// rows in registers beside the k rows, so half as many waves fit.
+template <typename T, bool L2, bool WANT_P>
+__global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void gdn_chunk_prepare_kernel(ChunkParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     extern __shared__ __align__(16) char smem[];
-    T* k_nat = (T*)smem;                        // [64][NP] keys, token-major; reused for L once the raw products exist
-    T* q_nat = k_nat + CH * NP;                 // [64][NP] queries; reused for X
-    float* sL = (float*)k_nat;                  // [64][LP] L (strictly lower); 64*68*4 == 64*136*2 bytes
-    float* sX = (float*)q_nat;                  // [64][LP] (I+L)^-1
-    float* sLd = (float*)(q_nat + CH * NP);     // [4][16 j][16 i] diagonal blocks of L, transposed (column j contiguous)
-    float* sRN = sLd + 4 * 256;                 // [3][64] 1/|k_t|, 1/|q_t| (ones unless the rows are to be normalised), |k_t|^2 as given
-    float* sGB = sRN + 3 * CH;                  // [group][2][64] cumulative gate (log2), beta
+    const int tid = threadIdx.x, lane = tid & 63, c16 = lane & 15, g = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t u = (int64_t)blockIdx.x * PW_WAVES + w;    // (chunk, value head), heads fastest
+    if (u >= units) return;
+    float* base = (float*)smem + w * PW_FLOATS;
+    float* tiles = base;
+    // left factors: the transposed diagonal blocks T(0,0) .. T(3,3) and the intermediate products V = T U; the gated
+    // tiles U themselves stay in registers as right factors
+    constexpr int I_T00 = 0, I_T11 = 1, I_T22 = 2, I_T33 = 3, I_V01 = 4, I_V23 = 5, I_T01 = I_V01;
+    constexpr int I_V02 = I_T22, I_V03 = I_T33, I_V12 = I_V23, I_V13 = 6;      // (T(2,2), T(3,3), V(2,3) are in registers by then)
+    float* sLd = tiles;                                      // [4][16 i][16 j] diagonal blocks of L, by rows (until the T(g,g) are written)
+    float* sG = tiles + 1024; float* sBN = sG + 64; float* sNK = sG + 128;      // gate tables (likewise)
+    float* sK2 = tiles + 4 * 16 * TP; float* sNQ = sK2 + 64; // (until the gated tiles are written)
+    auto tile = [&](int i) { return tiles + i * 16 * TP; };
+    auto lds_sync = [] { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };   // (LDS operations of a wave execute in order)
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    // heads vary fastest over the workgroups: those that run at the same time then read whole token rows
-    // (all heads of a token are contiguous in memory) instead of one 256-byte piece of every row
-    const int H = p.H, HV = p.HV;
-    const int64_t ci = blockIdx.x / H;
-    const int h = (int)(blockIdx.x % H);
-    const int G = HV / H;
+    const int H = p.H, HV = p.HV, G = HV / H, K = p.K;
+    const int64_t ci = u / HV;
+    const int hv = (int)(u % HV), h = hv / G;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-
     int64_t tok0;
     int valid;
     if (p.cu_seqlens) {
@@ -54,99 +71,111 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tok0 = b * p.T + it * CH;
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
+    constexpr bool l2 = L2;                      // q and k are to be l2-normalised (as row factors)
 
-    // q is needed for its row norms (l2 normalisation) and for P, when P is asked for
-    const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
-    const bool want_P = p.want_P != 0, need_q = l2 || want_P;
-    // ---- all global loads first: the gate inputs of value head w of the group, then the k, q rows ----
+    // ---- loads: the gate inputs of token `lane`, then the k rows as operand fragments ----
     float rg = 0.f, rb = 0.f;
-    if (w < G && lane < valid) {
-        rg = p.g ? load_scalar(p.g, (tok0 + lane) * HV + h * G + w, p.gb_dtype) : 0.f;      // (no gate: the plain delta rule)
-        rb = load_scalar(p.beta, (tok0 + lane) * HV + h * G + w, p.gb_dtype);
+    if (lane < valid) {
+        rg = p.g ? load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype) : 0.f;      // (no gate: the plain delta rule)
+        rb = load_scalar(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
     }
-    // ---- k (and q) rows, 128 key features at a time (K <= 128: one round): into LDS, their squared norms, and the raw
-    // products, which stay in registers: K K^T tiles (row-tile w, column-tiles <= w) and the transposed q K^T tiles
-    // of query tile tt = 3 - w (key tiles <= tt).  Rows past the end of the sequence and key features past K are zero.
-    const int tt = 3 - w;
-    f32x4 kk[4], qk[4];
+    f32x4 U[4][4];
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) kk[tj] = qk[tj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = a; b < 4; ++b) U[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float sq[4] = {0.f, 0.f, 0.f, 0.f};
+    f32x4 QK[4][4];                              // (WANT_P) raw k q^T tiles, like U
+    if constexpr (WANT_P) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+            for (int b = a; b < 4; ++b) QK[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     {
-        const int K = p.K;
         const T* kg = (const T*)p.k + (tok0 * H + h) * K;
         const T* qg = (const T*)p.q + (tok0 * H + h) * K;
-        float sk[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        // one 32-bit offset per lane (its row of a t-tile, its 8 features of a 32-feature block); tile and block
+        // select a wave-uniform base
+        const uint32_t lane_off = ((uint32_t)c16 * (uint32_t)(H * K) + 8u * g) * (uint32_t)sizeof(T);
+        auto fragment = [&](const T* rows, int t, int col0) {
+            const char* bp = (const char*)(rows + (int64_t)(16 * t) * H * K + col0);
+            return (16 * t + c16 < valid && col0 + 8 * g < K) ? *(const u32x4*)(bp + lane_off) : z;
+        };
+        // 128 features at a time: all 16 fragments of a round are requested before the first product; the q rows (for
+        // their norms only) follow into the same registers once the products have been issued
         for (int k0 = 0; k0 < K; k0 += 128) {
-            if (k0) __syncthreads();                 // the products of the previous round have read the tiles
-            u32x4 rk[4], rq[4];
+            u32x4 fk[4][4];
 #pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                const int row = ps * 16 + (tid >> 4), col = k0 + (tid & 15) * 8;
-                const u32x4 z = {0u, 0u, 0u, 0u};
-                rk[ps] = rq[ps] = z;
-                if (row < valid && col < K) {
-                    rk[ps] = *(const u32x4*)(kg + (int64_t)row * H * K + col);
-                    if (need_q) rq[ps] = *(const u32x4*)(qg + (int64_t)row * H * K + col);
-                }
-            }
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                const int row = ps * 16 + (tid >> 4), col = (tid & 15) * 8;
-                *(u32x4*)(k_nat + row * NP + col) = rk[ps];
-                if (want_P) *(u32x4*)(q_nat + row * NP + col) = rq[ps];
-                // l2 normalisation is applied as per-row factors: 16 lanes hold one row
-                if (l2) {
-                    const V8 k8 = __builtin_bit_cast(V8, rk[ps]), q8 = __builtin_bit_cast(V8, rq[ps]);
+                for (int s4 = 0; s4 < 4; ++s4) fk[t][s4] = fragment(kg, t, k0 + 32 * s4);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) { const float a = to_f32(k8[e]), b = to_f32(q8[e]); sk[ps] += a * a; sq[ps] += b * b; }
-                }
-            }
-            if (k0 + 128 >= K) {
+            for (int a = 0; a < 4; ++a)
 #pragma unroll
-                for (int ps = 0; ps < 4; ++ps) {
-                    float a = sk[ps], b = sq[ps];
-                    if (l2) {
+                for (int b = a; b < 4; ++b)
 #pragma unroll
-                        for (int off = 1; off < 16; off <<= 1) { a += __shfl_xor(a, off, 64); b += __shfl_xor(b, off, 64); }
+                    for (int s4 = 0; s4 < 4; ++s4)
+                        U[a][b] = Mma<T>::run(__builtin_bit_cast(V8, fk[a][s4]), __builtin_bit_cast(V8, fk[b][s4]), U[a][b]);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (WANT_P) {
+                u32x4 fq[4][4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) fq[t][s4] = fragment(qg, t, k0 + 32 * s4);
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int b = a; b < 4; ++b)
+#pragma unroll
+                        for (int s4 = 0; s4 < 4; ++s4)      // rows: key tokens of tile a, column: query token 16b + c16
+                            QK[a][b] = Mma<T>::run(__builtin_bit_cast(V8, fk[a][s4]), __builtin_bit_cast(V8, fq[b][s4]), QK[a][b]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) {
+                        const V8 q8 = __builtin_bit_cast(V8, fq[t][s4]);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) { const float x = to_f32(q8[e]); sq[t] += x * x; }
                     }
-                    if ((tid & 15) == 0) {
-                        const int row = ps * 16 + (tid >> 4);
-                        sRN[row] = l2 ? rsqrtf(a + 1e-6f) : 1.f;
-                        sRN[CH + row] = l2 ? rsqrtf(b + 1e-6f) : 1.f;
+            } else if constexpr (l2) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) fk[t][s4] = fragment(qg, t, k0 + 32 * s4);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) {
+                        const V8 q8 = __builtin_bit_cast(V8, fk[t][s4]);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) { const float x = to_f32(q8[e]); sq[t] += x * x; }
                     }
-                }
-            }
-            __syncthreads();
-            V8 ka[4], qb[4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                ka[s] = *(const V8*)(k_nat + (16 * w + c16) * NP + 32 * s + 8 * g);
-                if (want_P) qb[s] = *(const V8*)(q_nat + (16 * tt + c16) * NP + 32 * s + 8 * g);
-            }
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                if (tj <= w || (want_P && tj <= tt)) {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const V8 kb = *(const V8*)(k_nat + (16 * tj + c16) * NP + 32 * s + 8 * g);
-                        if (tj <= w) kk[tj] = Mma<T>::run(ka[s], kb, kk[tj]);          // rows: tokens of tile w, column: token 16tj + c16
-                        if (want_P && tj <= tt) qk[tj] = Mma<T>::run(kb, qb[s], qk[tj]);         // rows: key tokens of tile tj, column: query token 16tt + c16
-                    }
-                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
-    // ---- gates of every value head of the group: inclusive scan over the chunk, one token per lane ----
-    for (int m = w; m < G; m += 4) {
-        const int hv = h * G + m;
+    // |k_t|^2 is the diagonal of K K^T; |q_t|^2 is summed over the four lanes that share a row
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        float d = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (r == (c16 & 3)) d = U[t][t][r];
+        if ((c16 >> 2) == g) sK2[16 * t + c16] = d;
+        float a = sq[t];
+        a += __shfl_xor(a, 16, 64);
+        a += __shfl_xor(a, 32, 64);
+        if (g == t) sNQ[16 * t + c16] = l2 ? rsqrtf(a + 1e-6f) : 1.f;
+    }
+    lds_sync();
+    // ---- gates: inclusive scan over the chunk, one token per lane; the tables; the bound on the chunk's transition ----
+    float beta_tok;
+    {
         float x = rg, b = rb;
-        if (m >= 4) {                            // beyond the four fetched up front
-            x = b = 0.f;
-            if (lane < valid) {
-                x = p.g ? load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype) : 0.f;
-                b = load_scalar(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
-            }
-        }
         if (lane < valid) {                      // optional activations of the raw gate / beta inputs
             if (p.A_log && p.g) x = -__expf(p.A_log[hv]) * softplus_f(x + (p.dt_bias ? p.dt_bias[hv] : 0.f));
             if (p.flags & GDN_FLAG_BETA_SIGMOID) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
@@ -159,10 +188,13 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         x *= RCP_LN2_F;
         const float xl = __shfl(x, 63, 64);      // rows past the end carry the last valid sum
         const float ex = fast_exp2(x);
-        sGB[(2 * m) * CH + lane] = x;
-        sGB[(2 * m + 1) * CH + lane] = b;
+        const float k2 = sK2[lane];
+        const float nk = l2 ? rsqrtf(k2 + 1e-6f) : 1.f, nq = sNQ[lane];
+        beta_tok = b;
+        sG[lane] = x;
+        sBN[lane] = b * nk;
+        sNK[lane] = nk;
         float* tab = (float*)(p.ws.Rec + (ci * HV + hv) * REC_BYTES + REC_TAB);
-        const float nk = sRN[lane], nq = sRN[CH + lane];
         tab[TAB_DEC + lane] = fast_exp2(xl - x) * nk;        // multiplies v_new rows on their way into k^T v_new
         tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
         tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
@@ -171,209 +203,153 @@ __global__ __launch_bounds__(256, 4) void gdn_chunk_prepare_kernel(ChunkParams p
         tab2[TAB2_G + lane] = x;
         tab2[TAB2_NQS + lane] = p.scale * nq;
         tab2[TAB2_NK + lane] = nk;
-    }
-
-    // |k_t|^2 is the diagonal of K K^T: lane (c16, g) of the diagonal tile holds rows 4g .. 4g+3 of column c16
-    {
-        float d = 0.f;
-#pragma unroll
-        for (int tj = 0; tj < 4; ++tj)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (tj == w && r == (c16 & 3)) d = kk[tj][r];
-        if ((c16 >> 2) == g) sRN[2 * CH + 16 * w + c16] = d;
-    }
-    __syncthreads();     // k and q are dead from here on: their bytes become L and X
-    // ---- bound on the chunk's transition, per value head: every token contributes gamma_t max(1, |1 - beta_t |k~_t|^2|)
-    // (rows past the end have beta = 0 and g = 0) ----
-    for (int m = w; m < G; m += 4) {
-        const float nk = sRN[lane];
-        float lb = fabsf(1.f - sGB[(2 * m + 1) * CH + lane] * sRN[2 * CH + lane] * nk * nk);
+        // every token contributes gamma_t max(1, |1 - beta_t |k~_t|^2|) (rows past the end have beta = 0 and g = 0)
+        float lb = fabsf(1.f - b * k2 * nk * nk);
         lb = lb > 1.f ? __log2f(lb) : 0.f;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) lb += __shfl_xor(lb, off, 64);
-        if (lane == 63) p.ws.Bound[ci * HV + h * G + m] = sGB[(2 * m) * CH + 63] + lb;
+        if (lane == 63) p.ws.Bound[ci * HV + hv] = x + lb;
     }
-    // P of every value head first: the raw q K^T tiles then leave the registers before the inversion needs them
-    for (int m = 0; want_P && m < G; ++m) {
-        const int hv = h * G + m;
-        const float* sG = sGB + (2 * m) * CH;
+    lds_sync();
+    if constexpr (WANT_P) {
+        // ---- P^T tiles (rows: key tokens j, column: query token t; lower triangle incl. the diagonal), gated, as fragments ----
         char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
-        // ---- P^T tiles of query tile tt (gated, lower incl. diagonal), straight to memory ----
-        {
-            const int t = 16 * tt + c16;
-            const float gt = sG[t], st = p.scale * sRN[CH + t];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const float gt = sG[16 * b + c16], st = p.scale * sNQ[16 * b + c16];
 #pragma unroll
             for (int sp = 0; sp < 2; ++sp) {
-                if (tt < 2 && sp == 1) continue;        // identically zero, not stored
+                if (b < 2 && sp == 1) continue;         // identically zero, not stored
                 V8 frag;
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {
-                    const int tj = 2 * sp + half;
-                    if (tj > tt) {              // a key tile after the query tile: zero (tt is scalar: nothing is evaluated)
+                    const int a = 2 * sp + half;
+                    if (a > b) {                        // a key tile after the query tile: zero
 #pragma unroll
                         for (int r = 0; r < 4; ++r) frag[half * 4 + r] = from_f32<T>(0.f);
                         continue;
                     }
-                    const f32x4 gj = *(const f32x4*)(sG + 16 * tj + 4 * g), nj = *(const f32x4*)(sRN + 16 * tj + 4 * g);
+                    const f32x4 gj = *(const f32x4*)(sG + 16 * a + 4 * g), nj = *(const f32x4*)(sNK + 16 * a + 4 * g);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const int j = 16 * tj + 4 * g + r;
-                        const float val = (t >= j) ? st * nj[r] * qk[tj][r] * fast_exp2(gt - gj[r]) : 0.f;
-                        frag[half * 4 + r] = from_f32<T>(val);
+                        const bool below = a < b || c16 >= 4 * g + r;
+                        frag[half * 4 + r] = from_f32<T>(below ? st * nj[r] * QK[a][b][r] * fast_exp2(gt - gj[r]) : 0.f);
                     }
                 }
-                store_frag<T>(rec + REC_P, tt, sp, lane, frag);
+                store_frag<T>(rec + REC_P, b, sp, lane, frag);
             }
         }
     }
-    for (int m = 0; m < G; ++m) {
-        const int hv = h * G + m;
-        const float* sG = sGB + (2 * m) * CH;
-        const float* sB = sG + CH;
+    // ---- U = L^T: gated, beta-scaled, strictly upper; diagonal blocks to LDS as L by rows, the others as left factors ----
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = a; b < 4; ++b) {
+            const float gi = sG[16 * b + c16], bni = sBN[16 * b + c16];               // column: token i
+            const f32x4 gj = *(const f32x4*)(sG + 16 * a + 4 * g), nj = *(const f32x4*)(sNK + 16 * a + 4 * g);   // rows: tokens j
+            f32x4 val;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // select, never multiply by a mask: 2^(G_i-G_j) may overflow for i < j
+                const bool below = a < b || c16 > 4 * g + r;
+                val[r] = below ? bni * nj[r] * U[a][b][r] * fast_exp2(gi - gj[r]) : 0.f;
+            }
+            if (a == b) *(f32x4*)(sLd + a * 256 + c16 * 16 + 4 * g) = val;             // L[i = c16][j = 4g + r]
+            else U[a][b] = val;                                                        // stays in registers: a right factor
+        }
+    lds_sync();
+    // ---- diagonal blocks: X (I + L) = I by rows, from the right.  Lane c16 of group g owns row c16 of block g; as soon as
+    // x_i is known it is folded into the pending sums of all earlier columns (a dependent chain of 16 short steps) ----
+    {
+        const float* ld = sLd + g * 256;
+        float x[16], acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int i = 15; i >= 0; --i) {
+            x[i] = ((i == c16) ? 1.f : 0.f) - acc[i];
+            float row[16];
+#pragma unroll
+            for (int q4 = 0; q4 < (i + 3) / 4; ++q4) *(f32x4*)(row + 4 * q4) = *(const f32x4*)(ld + i * 16 + 4 * q4);
+#pragma unroll
+            for (int j = 0; j < i; ++j) acc[j] += row[j] * x[i];
+        }
+        // T(g,g) = X_gg^T as a left factor: [row j][column c16]
+        float* tt = tile(I_T00 + g);             // (group g: block g)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) tt[j * TP + c16] = x[j];
+    }
+    lds_sync();
+    auto acc_layout = [&](int i) {               // a tile of LDS in accumulator layout
+        const float* t = tile(i);
+        return f32x4{t[(4 * g) * TP + c16], t[(4 * g + 1) * TP + c16], t[(4 * g + 2) * TP + c16], t[(4 * g + 3) * TP + c16]};
+    };
+    // acc + A B: A a tile of LDS by rows, B in accumulator layout
+    auto mul = [&](int ia, f32x4 B, f32x4 acc) {
+        const f32x4 a = *(const f32x4*)(tile(ia) + c16 * TP + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], B[e], acc, 0, 0, 0);
+        return acc;
+    };
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    auto put = [&](int i, f32x4 v) {             // a tile in accumulator layout to LDS, by rows
+#pragma unroll
+        for (int r = 0; r < 4; ++r) tile(i)[(4 * g + r) * TP + c16] = v[r];
+    };
+    const f32x4 T00 = acc_layout(I_T00), T11 = acc_layout(I_T11), T22 = acc_layout(I_T22), T33 = acc_layout(I_T33);
+    // ---- merge 16 -> 32: T(lo,hi) = -(T(lo,lo) U(lo,hi)) T(hi,hi) ----
+    put(I_V01, mul(I_T00, U[0][1], zero));
+    put(I_V23, mul(I_T22, U[2][3], zero));
+    lds_sync();
+    const f32x4 T01 = -mul(I_V01, T11, zero);
+    const f32x4 T23 = -mul(I_V23, T33, zero);
+    put(I_T01, T01);
+    lds_sync();
+    // ---- merge 32 -> 64: V = T[0:32][0:32] U[0:32][32:64], T[0:32][32:64] = -V T[32:64][32:64] (zero tiles left out) ----
+    put(I_V02, mul(I_T00, U[0][2], mul(I_T01, U[1][2], zero)));
+    put(I_V03, mul(I_T00, U[0][3], mul(I_T01, U[1][3], zero)));
+    put(I_V12, mul(I_T11, U[1][2], zero));
+    put(I_V13, mul(I_T11, U[1][3], zero));
+    lds_sync();
+    const f32x4 T02 = -mul(I_V02, T22, zero), T03 = -mul(I_V03, T33, mul(I_V02, T23, zero));
+    const f32x4 T12 = -mul(I_V12, T22, zero), T13 = -mul(I_V13, T33, mul(I_V12, T23, zero));
+    // ---- Xb = X diag(beta) as operand fragments: rows of t-tile tt, columns {32sp + 4g + e} and {32sp + 16 + 4g + e} ----
+    {
         char* rec = p.ws.Rec + (ci * HV + hv) * REC_BYTES;
-        // ---- L tiles of row-tile w (gated, beta-scaled, strictly lower) ----
-        {
-            const f32x4 gi = *(const f32x4*)(sG + 16 * w + 4 * g);
-            const f32x4 bi = *(const f32x4*)(sB + 16 * w + 4 * g) * *(const f32x4*)(sRN + 16 * w + 4 * g);
+        auto emit = [&](int tt, int sp, f32x4 lo, f32x4 hi, bool has_hi) {
+            V8 frag;
 #pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                const int j = 16 * tj + c16;
-                if (tj > w) {                   // above the diagonal: zero (w is scalar: nothing is evaluated)
-                    if (w < 2 && tj >= 2) {     // only the block that will hold XT is ever read
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) sL[(16 * w + 4 * g + r) * LP + j] = 0.f;
-                    }
-                    continue;
-                }
-                const float gj = sG[j], nj = sRN[j];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    // select, never multiply by a mask: 2^(G_i-G_j) may overflow above the diagonal
-                    const float val = (i > j) ? bi[r] * nj * kk[tj][r] * fast_exp2(gi[r] - gj) : 0.f;
-                    sL[i * LP + j] = val;
-                    if (tj == w) sLd[(w * 16 + c16) * 16 + 4 * g + r] = val;
-                }
+            for (int e = 0; e < 4; ++e) {
+                frag[e] = from_f32<T>(lo[e] * __shfl(beta_tok, 32 * sp + 4 * g + e, 64));
+                frag[4 + e] = from_f32<T>(has_hi ? hi[e] * __shfl(beta_tok, 32 * sp + 16 + 4 * g + e, 64) : 0.f);
             }
-        }
-        __syncthreads();     // L complete
-
-        // ---- X = (I+L)^-1: 16x16 diagonal blocks by forward substitution.  Lane c16 owns column c16 of
-        // the block; as soon as x_j is known it is folded into the pending sums of all later rows, so
-        // the dependent chain is 16 steps of two operations (not the 120 of a row-by-row evaluation).
-        {
-            const int b0 = 16 * w;
-            const float* ld = sLd + w * 256;
-            float x[16], acc[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                x[j] = ((j == c16) ? 1.f : 0.f) - acc[j];
-                float col[16];
-#pragma unroll
-                for (int q4 = (j + 1) / 4; q4 < 4; ++q4) *(f32x4*)(col + 4 * q4) = *(const f32x4*)(ld + j * 16 + 4 * q4);
-#pragma unroll
-                for (int i = j + 1; i < 16; ++i) acc[i] += col[i] * x[j];
-            }
-            if (g == 0) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) sX[(b0 + i) * LP + b0 + c16] = x[i];
-            }
-            // The merges below multiply by X blocks from the left AND from the right.  A right factor is read by
-            // columns, so it is kept transposed as well (one 16-byte LDS read then serves four matrix
-            // instructions): XT, the transposed top-left 32x32 block, lives in the unused upper-right
-            // block of L (zero so far), the transposed X22 in rows 16..31 of the unused upper-right block of X.
-            if (g == 1) {
-                float* xt = (w < 2) ? sL + (b0 + c16) * LP + 32 + b0 : sX + (16 + c16) * LP + 32;
-                if (w != 3) {
-#pragma unroll
-                    for (int i4 = 0; i4 < 4; ++i4) *(f32x4*)(xt + 4 * i4) = f32x4{x[4 * i4], x[4 * i4 + 1], x[4 * i4 + 2], x[4 * i4 + 3]};
-                }
-            }
-            // zero tile above the diagonal inside each 32x32 diagonal block
-            if ((w & 1) == 0) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sX[(b0 + 4 * g + r) * LP + b0 + 16 + c16] = 0.f;
-            }
-        }
-        __syncthreads();
-        // 16x16 products on the fp32 matrix cores, contraction over 16*nq indices: A by rows (pitch LP),
-        // the right factor transposed (Bt[n][k], pitch LP); step e of block q uses the indices {16q + 4g + e}
-        auto mm_rt = [&](const float* A, const float* Bt, int nq) {
-            f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                if (q >= nq) break;
-                const f32x4 a = *(const f32x4*)(A + c16 * LP + 16 * q + 4 * g);
-                const f32x4 bt = *(const f32x4*)(Bt + c16 * LP + 16 * q + 4 * g);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[q] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], bt[e], acc[q], 0, 0, 0);
-            }
-            return acc[0] + acc[1];
+            store_frag<T>(rec + REC_X, tt, sp, lane, frag);
         };
-        // ---- merge 16 -> 32: X[hi][lo] = -X[hi][hi] (L[hi][lo] X[lo][lo]); pairs (1,0) and (3,2) by waves 0 and 1.
-        // A wave only reads back what it has written itself (LDS operations of a wave execute in order), so
-        // there is no barrier between the two products; waves 2 and 3 leave their SIMDs to other workgroups.
-        if (w < 2) {
-            const int hi = 2 * w + 1, lo = 2 * w;
-            float* tmpT = sX + 32 + 16 * w;                     // rows 0..15 of the unused upper-right block: (L X)^T
-            const float* xlo_t = w ? sX + 16 * LP + 32 : sL + 32;
-            const f32x4 y = mm_rt(sL + (16 * hi) * LP + 16 * lo, xlo_t, 1);
-            *(f32x4*)(tmpT + c16 * LP + 4 * g) = y;
-            const f32x4 z = mm_rt(sX + (16 * hi) * LP + 16 * hi, tmpT, 1);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sX[(16 * hi + 4 * g + r) * LP + 16 * lo + c16] = -z[r];
-            if (w == 0) *(f32x4*)(sL + c16 * LP + 32 + 16 + 4 * g) = -z;             // X10 into XT
-        }
-        __syncthreads();
-        // ---- merge 32 -> 64: X[32:64][0:32] = -X[32:64][32:64] (L[32:64][0:32] X[0:32][0:32]) ----
-        {
-            const int a = w >> 1, b = w & 1;
-            float* tmp2T = sX + 32;                             // rows 0..31, columns 32..63: (L X)^T
-            const f32x4 y = mm_rt(sL + (32 + 16 * a) * LP, sL + (16 * b) * LP + 32, 2);
-            *(f32x4*)(tmp2T + (16 * b + c16) * LP + 16 * a + 4 * g) = y;
-            __syncthreads();
-            const f32x4 z = mm_rt(sX + (32 + 16 * a) * LP + 32, tmp2T + (16 * b) * LP, 2);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sX[(32 + 16 * a + 4 * g + r) * LP + 16 * b + c16] = -z[r];
-        }
-        __syncthreads();
-        // ---- Xb = X diag(beta) rows of t-tile w as A-operand fragments ----
-        {
-            const int ns = (w >= 2) ? 2 : 1;         // X is lower triangular: columns >= 32 matter only for rows >= 32
-            for (int sp = 0; sp < ns; ++sp) {
-                const float* xr = sX + (16 * w + c16) * LP + 32 * sp + 4 * g;
-                const f32x4 x0 = *(const f32x4*)xr, x1 = *(const f32x4*)(xr + 16);
-                const f32x4 b0 = *(const f32x4*)(sB + 32 * sp + 4 * g), b1 = *(const f32x4*)(sB + 32 * sp + 16 + 4 * g);
-                V8 frag;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    frag[e] = from_f32<T>(x0[e] * b0[e]);
-                    frag[4 + e] = from_f32<T>(x1[e] * b1[e]);
-                }
-                store_frag<T>(rec + REC_X, w, sp, lane, frag);
-            }
-        }
-        if (m + 1 < G) __syncthreads();          // the next value head overwrites L and X
+        emit(0, 0, T00, zero, false);
+        emit(1, 0, T01, T11, true);
+        emit(2, 0, T02, T12, true);
+        emit(2, 1, T22, zero, false);
+        emit(3, 0, T03, T13, true);
+        emit(3, 1, T23, T33, true);
     }
+}
+
+template <typename T, bool L2, bool WANT_P>
+static int launch_prepare_as(const ChunkParams& p, int64_t units, hipStream_t stream) {
+    auto kern = gdn_chunk_prepare_kernel<T, L2, WANT_P>;
+    static SmemAttrDone attr_done;       // per instantiation
+    if (int rc = ensure_dynamic_smem((const void*)kern, PREP_SMEM, attr_done, "hipFuncSetAttribute(prepare)")) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)((units + PW_WAVES - 1) / PW_WAVES)), dim3(64 * PW_WAVES), PREP_SMEM, stream, p, units);
+    return check_launch("gdn_chunk_prepare_kernel");
 }
 
 template <typename T>
 int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream) {
-    auto kern = gdn_chunk_prepare_kernel<T>;
-    const int G = p.HV / p.H;
-    const size_t smem = prep_smem(G);
-    if (smem > 64 * 1024) {
-        set_error("gdn_chunk_fwd: %d value heads per q/k head exceed what the prepare kernel stages", G);
-        return GDN_ERR_UNSUPPORTED;
-    }
-    static SmemAttrDone attr_done;       // per instantiation
-    if (int rc = ensure_dynamic_smem((const void*)kern, 64 * 1024, attr_done, "hipFuncSetAttribute(prepare)")) return rc;
-    dim3 grid((unsigned)(num_chunks * p.H)), block(256);
-    hipLaunchKernelGGL(kern, grid, block, smem, stream, p);
-    return check_launch("gdn_chunk_prepare_kernel");
+    const int64_t units = num_chunks * p.HV;
+    if (units <= 0) return GDN_OK;
+    const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
+    if (p.want_P) return l2 ? launch_prepare_as<T, true, true>(p, units, stream) : launch_prepare_as<T, false, true>(p, units, stream);
+    return l2 ? launch_prepare_as<T, true, false>(p, units, stream) : launch_prepare_as<T, false, false>(p, units, stream);
 }
 template int launch_prepare<bf16_t>(const ChunkParams&, int64_t, hipStream_t);
 template int launch_prepare<f16_t>(const ChunkParams&, int64_t, hipStream_t);
