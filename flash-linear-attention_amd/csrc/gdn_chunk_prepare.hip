@@ -99,8 +99,10 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
         // one 32-bit offset per lane (its row of a t-tile, its 8 features of a 32-feature block); tile and block
         // select a wave-uniform base
         const uint32_t lane_off = ((uint32_t)c16 * (uint32_t)(H * K) + 8u * g) * (uint32_t)sizeof(T);
+        // (a full chunk with the 32 features in range - the common case - loads without any per-lane condition)
         auto fragment = [&](const T* rows, int t, int col0) {
             const char* bp = (const char*)(rows + (int64_t)(16 * t) * H * K + col0);
+            if (valid == CH && col0 + 32 <= K) return *(const u32x4*)(bp + lane_off);
             return (16 * t + c16 < valid && col0 + 8 * g < K) ? *(const u32x4*)(bp + lane_off) : z;
         };
         // 128 features at a time: all 16 fragments of a round are requested before the first product; the q rows (for
