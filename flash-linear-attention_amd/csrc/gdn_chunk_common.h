@@ -65,13 +65,29 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 //                         tiles and the second table, into this place of its LDS copy; the prepare kernel writes it to
 //                         memory on request (GDN_FLAG_RECORD_P), for callers that look at the records
 //   tab  fp32 [256]       [0..63] 2^(G_last-G_t), [64..127] scale*2^G_t, [128..191] 2^G_t, [192] G_last (log2 units),
-//                         the first three times the row factors 1/|k_t|, 1/|q_t|, 1/|k_t| of the l2 normalisation
-//   tab2 fp32 [256]       [0..63] G_t (log2 units), [64..127] scale/|q_t|, [128..191] 1/|k_t|: what P needs
+//                         the first and the third times the row factor 1/|k_t| of the l2 normalisation
+//   tab2 fp32 [256]       [0..63] G_t (log2 units), [64..127] scale, [128..191] 1/|k_t|: what P needs
+// The row factors 1/|q_t| of the l2 normalisation are not in the records: the prepare kernel does not read q.  The scan
+// kernels take them from the q tiles in LDS where they form P (row_rnorm below), scale P with them and multiply them
+// into [64..127] of their LDS copy of `tab` before anything reads it.  (Head dims up to 64 are the exception: there the
+// prepare kernel reads q for its norms and both tables carry 1/|q_t|, scale/|q_t|.)
 constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240, REC_TAB2 = 11264;
 constexpr int64_t REC_BYTES = 12288;
 constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10, REC_PIECE_TAB2 = 11;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10, tab2 = 11
 constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
 constexpr int TAB2_G = 0, TAB2_NQS = 64, TAB2_NK = 128;
+// 1/|q_t| of the token row that this lane's q fragments belong to (lane (c16, g) holds 8 features per fragment of row c16
+// of a t-tile).  On the matrix cores: the tile's q q^T, whose diagonal element (c16, c16) lands in lane (c16, g = c16 / 4),
+// register c16 % 4, and is handed to the other three lanes of the row by one cross-lane read.
+template <typename T, int N>
+__device__ __forceinline__ float row_rnorm(const typename Mma<T>::V8 (&qb)[N], int c16) {
+    f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < N; ++i) d = Mma<T>::run(qb[i], qb[i], d);
+    const int r = c16 & 3;
+    const float own = r == 0 ? d[0] : r == 1 ? d[1] : r == 2 ? d[2] : d[3];
+    return rsqrtf(__shfl(own, 16 * (c16 >> 2) + c16, 64) + 1e-6f);
+}
 // Besides the records the prepare kernel leaves one number per (chunk, v-head): an upper bound, in log2 units, on how much
 // the chunk's transition S -> 2^G_last S - k~^T (Xb 2^G k) S can stretch any state:
 //   bound = sum_t [ log2 gamma_t + log2 max(1, |1 - beta_t |k_t|^2|) ]      (each token's factor gamma_t (I - beta_t k_t k_t^T))

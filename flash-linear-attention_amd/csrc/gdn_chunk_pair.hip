@@ -61,6 +61,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     const int tm = w >> 2, cw = w & 3;
     const int H = p.H, HV = p.HV;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    const bool l2q = p.flags & GDN_FLAG_QK_L2NORM;        // q is l2-normalised where P is formed (row factors)
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which runs: workgroups that read the same k rows take consecutive slots of one XCD ----
@@ -306,7 +307,12 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
 #pragma unroll
                 for (int s4 = 0; s4 < 4; ++s4) qb[s4] = sQ[tt * 256 + 16 * s4 + a_off];
                 const int t = 16 * tt + c16;
-                const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                if (l2q) {                        // q is normalised here: P, and the table that scales the (q S) rows
+                    const float nq = row_rnorm<T>(qb, c16);
+                    st_ *= nq;
+                    if (sp == 0 && g == 0) ((float*)(rec + REC_TAB))[TAB_SG + t] *= nq;
+                }
                 V8 out;
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {

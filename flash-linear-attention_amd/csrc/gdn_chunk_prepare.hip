@@ -2,9 +2,9 @@
 // running state and is not a plain copy of the inputs:
 //   G = cumsum(g)/ln2,  L = beta*(K K^T)*2^(G_i-G_j) (i>j),  X = (I+L)^-1 in fp32,  Xb = X diag(beta),
 //   the per-token gate tables, a bound on the chunk's transition, and on request P = scale*tril(q k^T * 2^(G_i-G_j)).
-// Optional prologues of the reference are folded in: the gate and beta activations, and the l2 normalisation of q and
-// k as per-row factors 1/|k_t|, 1/|q_t| on L, P and the tables (so the sequential stage reads q and k exactly as the
-// caller gave them).  Xb and P are written in the exact register order ("fragments") in which the scan kernel feeds
+// Optional prologues of the reference are folded in: the gate and beta activations, and the l2 normalisation of k as
+// per-row factors 1/|k_t| on L and the tables (so the sequential stage reads q and k exactly as the caller gave them;
+// q is read here only for P, its row factors 1/|q_t| are applied by the scan where it has q in LDS anyway).  Xb and P are written in the exact register order ("fragments") in which the scan kernel feeds
 // them to the matrix cores; the scan forms v_new = Xb (v - 2^G (k S)) itself from the raw k and v, so neither
 // w = Xb 2^G k nor u = Xb v is ever materialised.
 //
@@ -35,7 +35,7 @@ constexpr size_t PREP_SMEM = (size_t)PW_WAVES * PW_FLOATS * 4;
 
 // WANT_P: also the records' P (for callers that look at the records; the scan kernels form P themselves): keeps the q
 // rows in registers beside the k rows, so half as many waves fit.
-template <typename T, bool L2, bool WANT_P>
+template <typename T, bool WANT_P>
 __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void gdn_chunk_prepare_kernel(ChunkParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     extern __shared__ __align__(16) char smem[];
@@ -71,7 +71,9 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
         tok0 = b * p.T + it * CH;
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
-    constexpr bool l2 = L2;                      // q and k are to be l2-normalised (as row factors)
+    const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;      // k is l2-normalised here, as row factors (q: by the scan, or below for P)
+    // (head dims up to 64: the scan's step is short and P is on its critical path, so 1/|q_t| comes from here, in the tables)
+    const bool q_norms_here = l2 && p.K <= 64 && p.V <= 64;
 
     // ---- loads: the gate inputs of token `lane`, then the k rows as operand fragments ----
     float rg = 0.f, rb = 0.f;
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
 #pragma unroll
                         for (int e = 0; e < 8; ++e) { const float x = to_f32(q8[e]); sq[t] += x * x; }
                     }
-            } else if constexpr (l2) {
+            } else if (q_norms_here) {                       // the q rows into the registers that held k
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
             }
         }
     }
-    // |k_t|^2 is the diagonal of K K^T; |q_t|^2 is summed over the four lanes that share a row
+    // |k_t|^2 is the diagonal of K K^T; |q_t|^2 (for P only) is summed over the four lanes that share a row
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         float d = 0.f;
@@ -168,10 +170,12 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
         for (int r = 0; r < 4; ++r)
             if (r == (c16 & 3)) d = U[t][t][r];
         if ((c16 >> 2) == g) sK2[16 * t + c16] = d;
-        float a = sq[t];
-        a += __shfl_xor(a, 16, 64);
-        a += __shfl_xor(a, 32, 64);
-        if (g == t) sNQ[16 * t + c16] = l2 ? rsqrtf(a + 1e-6f) : 1.f;
+        if (WANT_P || q_norms_here) {
+            float a = sq[t];
+            a += __shfl_xor(a, 16, 64);
+            a += __shfl_xor(a, 32, 64);
+            if (g == t) sNQ[16 * t + c16] = l2 ? rsqrtf(a + 1e-6f) : 1.f;
+        }
     }
     lds_sync();
     // ---- gates: inclusive scan over the chunk, one token per lane; the tables; the bound on the chunk's transition ----
@@ -191,14 +195,14 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
         const float xl = __shfl(x, 63, 64);      // rows past the end carry the last valid sum
         const float ex = fast_exp2(x);
         const float k2 = sK2[lane];
-        const float nk = l2 ? rsqrtf(k2 + 1e-6f) : 1.f, nq = sNQ[lane];
+        const float nk = l2 ? rsqrtf(k2 + 1e-6f) : 1.f, nq = q_norms_here ? sNQ[lane] : 1.f;
         beta_tok = b;
         sG[lane] = x;
         sBN[lane] = b * nk;
         sNK[lane] = nk;
         float* tab = (float*)(p.ws.Rec + (ci * HV + hv) * REC_BYTES + REC_TAB);
         tab[TAB_DEC + lane] = fast_exp2(xl - x) * nk;        // multiplies v_new rows on their way into k^T v_new
-        tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows
+        tab[TAB_SG + lane] = p.scale * ex * nq;              // multiplies (q S) rows (nq = 1: the scan adds 1/|q_t|)
         tab[TAB_EG + lane] = ex * nk;                        // multiplies (k S) rows
         if (lane == 63) tab[TAB_GLAST] = x;
         float* tab2 = (float*)(p.ws.Rec + (ci * HV + hv) * REC_BYTES + REC_TAB2);
@@ -336,9 +340,9 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
     }
 }
 
-template <typename T, bool L2, bool WANT_P>
+template <typename T, bool WANT_P>
 static int launch_prepare_as(const ChunkParams& p, int64_t units, hipStream_t stream) {
-    auto kern = gdn_chunk_prepare_kernel<T, L2, WANT_P>;
+    auto kern = gdn_chunk_prepare_kernel<T, WANT_P>;
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, PREP_SMEM, attr_done, "hipFuncSetAttribute(prepare)")) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)((units + PW_WAVES - 1) / PW_WAVES)), dim3(64 * PW_WAVES), PREP_SMEM, stream, p, units);
@@ -349,9 +353,7 @@ template <typename T>
 int launch_prepare(const ChunkParams& p, int64_t num_chunks, hipStream_t stream) {
     const int64_t units = num_chunks * p.HV;
     if (units <= 0) return GDN_OK;
-    const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;
-    if (p.want_P) return l2 ? launch_prepare_as<T, true, true>(p, units, stream) : launch_prepare_as<T, false, true>(p, units, stream);
-    return l2 ? launch_prepare_as<T, true, false>(p, units, stream) : launch_prepare_as<T, false, false>(p, units, stream);
+    return p.want_P ? launch_prepare_as<T, true>(p, units, stream) : launch_prepare_as<T, false>(p, units, stream);
 }
 template int launch_prepare<bf16_t>(const ChunkParams&, int64_t, hipStream_t);
 template int launch_prepare<f16_t>(const ChunkParams&, int64_t, hipStream_t);

@@ -42,6 +42,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int H = p.H, HV = p.HV;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    const bool l2q = p.flags & GDN_FLAG_QK_L2NORM;        // q is l2-normalised where P is formed (row factors)
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which (sequence, value head, block of value columns): the workgroups that read the same k and q rows take
@@ -127,7 +128,12 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
 #pragma unroll
                 for (int s8 = 0; s8 < 8; ++s8) qb[s8] = sQ[(s8 >> 2) * 1024 + tt * 256 + 16 * (s8 & 3) + a_off];
                 const int t = 16 * tt + c16;
-                const float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                float gt = t2[TAB2_G + t], st_ = t2[TAB2_NQS + t];
+                if (l2q) {                        // q is normalised here: P, and the table that scales the (q S) rows
+                    const float nq = row_rnorm<T>(qb, c16);
+                    st_ *= nq;
+                    if (sp == 0 && g == 0) ((float*)(rec + W2_RTAB))[TAB_SG + t] *= nq;
+                }
                 V8 out;
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {

@@ -47,6 +47,7 @@ def _records(call, num_chunks, HV):
     (1, 256, 4, 4, 32, torch.float16, 1.0, False),
     (2, 200, 2, 4, 128, torch.bfloat16, 16.0, True),           # ragged last chunk, row factors of the l2 norm
     (1, 63, 1, 1, 16, torch.float16, 4.0, False),              # tests/ops/test_solve_tril.py:22
+    (2, 100, 2, 4, 64, torch.bfloat16, 4.0, True),            # head dims up to 64: the row factors 1/|q_t| are in the tables
     (1, 128, 1, 2, 32, torch.bfloat16, 2.0, 'long'),           # keys of length 1.7: beta |k|^2 > 2 stretches the state
 ])
 def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2, monkeypatch):
@@ -99,10 +100,12 @@ def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2,
                 assert not Xb[:n, n:].any() and torch.equal(Xb, torch.tril(Xb))          # lower triangular, tail columns zero
                 tab = rec[REC_TAB:REC_TAB + 1024].view(torch.float32).double()
                 rk = 1.0 / torch.sqrt((k[b, sl, hv // G].double() ** 2).sum(-1) + 1e-6) if l2 else torch.ones(n, dtype=torch.float64)
-                rq = 1.0 / torch.sqrt((q[b, sl, hv // G].double() ** 2).sum(-1) + 1e-6) if l2 else torch.ones(n, dtype=torch.float64)
                 assert abs(tab[192].item() - gc[-1].item()) < 1e-4 * max(1.0, abs(gc[-1].item()))          # G_last
                 assert torch.allclose(tab[128:128 + n], torch.exp2(gc) * rk, rtol=2e-5, atol=1e-30)          # 2^G (k rows)
-                assert torch.allclose(tab[64:64 + n], scale * torch.exp2(gc) * rq, rtol=2e-5, atol=1e-30)    # scale 2^G (q rows)
+                # scale 2^G (q rows); the row factors 1/|q_t| of the l2 norm are the scan's (it has q in LDS), not the records',
+                # except for head dims up to 64
+                rq = 1.0 / torch.sqrt((q[b, sl, hv // G].double() ** 2).sum(-1) + 1e-6) if (l2 and K <= 64) else torch.ones(n, dtype=torch.float64)
+                assert torch.allclose(tab[64:64 + n], scale * torch.exp2(gc) * rq, rtol=2e-5, atol=1e-30)
                 assert torch.allclose(tab[0:n], torch.exp2(gc[-1] - gc) * rk, rtol=2e-5, atol=1e-30)         # 2^(G_last - G)
                 tab2 = rec[REC_TAB2:REC_TAB2 + 1024].view(torch.float32).double()                            # what P is formed from
                 assert torch.allclose(tab2[0:n], gc, rtol=1e-5, atol=1e-5)
