@@ -139,7 +139,8 @@ static int chunk_entry(
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH; p.K = (int)K; p.V = (int)V;
-    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags; p.NH = N * HV;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags & ~FLAG_Q_NORM_IN_SCAN; p.NH = N * HV;
+    if (q_norm_in_scan(flags, K, V, num_chunks * HV)) p.flags |= FLAG_Q_NORM_IN_SCAN;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_chunk<bf16_t>(p, num_chunks, stages, s)
                                        : launch_chunk<f16_t>(p, num_chunks, stages, s);
 }

@@ -69,13 +69,22 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 //   tab2 fp32 [256]       [0..63] G_t (log2 units), [64..127] scale, [128..191] 1/|k_t|: what P needs
 // The row factors 1/|q_t| of the l2 normalisation are not in the records: the prepare kernel does not read q.  The scan
 // kernels take them from the q tiles in LDS where they form P (row_rnorm below), scale P with them and multiply them
-// into [64..127] of their LDS copy of `tab` before anything reads it.  (Head dims up to 64 are the exception: there the
+// into [64..127] of their LDS copy of `tab` before anything reads it.  (Not always: see FLAG_Q_NORM_IN_SCAN; without it the
 // prepare kernel reads q for its norms and both tables carry 1/|q_t|, scale/|q_t|.)
 constexpr int REC_X = 0, REC_P = 5120, REC_TAB = 10240, REC_TAB2 = 11264;
 constexpr int64_t REC_BYTES = 12288;
 constexpr int REC_PIECES_X = 5, REC_PIECES_P = 5, REC_PIECE_TAB = 10, REC_PIECE_TAB2 = 11;      // in 1 KB pieces: Xb = 0..4, P = 5..9, tab = 10, tab2 = 11
 constexpr int TAB_DEC = 0, TAB_SG = 64, TAB_EG = 128, TAB_GLAST = 192;
 constexpr int TAB2_G = 0, TAB2_NQS = 64, TAB2_NK = 128;
+// Who applies the row factors 1/|q_t| of the in-kernel l2 norm (a bit of ChunkParams::flags that the entry points set, above
+// the caller's flags): the scan kernels, which have q in LDS anyway - except for head dims up to 64 (the scan's step is short
+// and P is on its critical path) and for wide keys on few units (every 64-column workgroup of a head would form the norms
+// again, while a prepare kernel that does not fill the chip reads q for nothing).
+constexpr uint32_t FLAG_Q_NORM_IN_SCAN = 1u << 30;
+inline bool q_norm_in_scan(uint32_t flags, int64_t K, int64_t V, int64_t units) {
+    if (!(flags & GDN_FLAG_QK_L2NORM) || (K <= 64 && V <= 64)) return false;
+    return K <= 128 || units >= 4096;
+}
 // 1/|q_t| of the token row that this lane's q fragments belong to (lane (c16, g) holds 8 features per fragment of row c16
 // of a t-tile).  On the matrix cores: the tile's q q^T, whose diagonal element (c16, c16) lands in lane (c16, g = c16 / 4),
 // register c16 % 4, and is handed to the other three lanes of the row by one cross-lane read.

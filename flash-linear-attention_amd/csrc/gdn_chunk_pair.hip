@@ -61,7 +61,7 @@ __global__ __launch_bounds__(PAIR_THREADS) void gdn_chunk_pair_kernel(ChunkParam
     const int tm = w >> 2, cw = w & 3;
     const int H = p.H, HV = p.HV;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-    const bool l2q = p.flags & GDN_FLAG_QK_L2NORM;        // q is l2-normalised where P is formed (row factors)
+    const bool l2q = p.flags & FLAG_Q_NORM_IN_SCAN;       // q is l2-normalised where P is formed (row factors)
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which runs: workgroups that read the same k rows take consecutive slots of one XCD ----

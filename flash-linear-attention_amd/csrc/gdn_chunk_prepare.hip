@@ -72,8 +72,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
         valid = (int)min((int64_t)CH, p.T - it * CH);
     }
     const bool l2 = p.flags & GDN_FLAG_QK_L2NORM;      // k is l2-normalised here, as row factors (q: by the scan, or below for P)
-    // (head dims up to 64: the scan's step is short and P is on its critical path, so 1/|q_t| comes from here, in the tables)
-    const bool q_norms_here = l2 && p.K <= 64 && p.V <= 64;
+    const bool q_norms_here = l2 && !(p.flags & FLAG_Q_NORM_IN_SCAN);       // 1/|q_t| into the tables (else the scan applies it)
 
     // ---- loads: the gate inputs of token `lane`, then the k rows as operand fragments ----
     float rg = 0.f, rb = 0.f;

@@ -75,7 +75,7 @@ __global__ __launch_bounds__(WIDE_THREADS) void gdn_chunk_wide_kernel(ChunkParam
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);       // scalar: the roles below branch on it
     const int H = p.H, HV = p.HV;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-    const bool l2q = !SMALL && (p.flags & GDN_FLAG_QK_L2NORM);      // q is l2-normalised where P is formed (row factors; head dims up to 64: in the records' tables)
+    const bool l2q = p.flags & FLAG_Q_NORM_IN_SCAN;       // q is l2-normalised where P is formed (row factors)
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which (sequence, head, segment) and what to start from / write to ----

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int H = p.H, HV = p.HV;
     const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-    const bool l2q = p.flags & GDN_FLAG_QK_L2NORM;        // q is l2-normalised where P is formed (row factors)
+    const bool l2q = p.flags & FLAG_Q_NORM_IN_SCAN;       // q is l2-normalised where P is formed (row factors)
     const bool vfirst = p.flags & GDN_FLAG_STATE_V_FIRST;
 
     // ---- which (sequence, value head, block of value columns): the workgroups that read the same k and q rows take

@@ -103,8 +103,8 @@ def test_prepare_stage_against_closed_forms(B, T, H, HV, K, dtype, gate_div, l2,
                 assert abs(tab[192].item() - gc[-1].item()) < 1e-4 * max(1.0, abs(gc[-1].item()))          # G_last
                 assert torch.allclose(tab[128:128 + n], torch.exp2(gc) * rk, rtol=2e-5, atol=1e-30)          # 2^G (k rows)
                 # scale 2^G (q rows); the row factors 1/|q_t| of the l2 norm are the scan's (it has q in LDS), not the records',
-                # except for head dims up to 64
-                rq = 1.0 / torch.sqrt((q[b, sl, hv // G].double() ** 2).sum(-1) + 1e-6) if (l2 and K <= 64) else torch.ones(n, dtype=torch.float64)
+                # except for head dims up to 64 and wide keys on few (chunk, head) units
+                rq = 1.0 / torch.sqrt((q[b, sl, hv // G].double() ** 2).sum(-1) + 1e-6) if (l2 and (K <= 64 or (K > 128 and B * NT * HV < 4096))) else torch.ones(n, dtype=torch.float64)
                 assert torch.allclose(tab[64:64 + n], scale * torch.exp2(gc) * rq, rtol=2e-5, atol=1e-30)
                 assert torch.allclose(tab[0:n], torch.exp2(gc[-1] - gc) * rk, rtol=2e-5, atol=1e-30)         # 2^(G_last - G)
                 tab2 = rec[REC_TAB2:REC_TAB2 + 1024].view(torch.float32).double()                            # what P is formed from
