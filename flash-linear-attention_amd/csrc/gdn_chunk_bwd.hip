@@ -1,0 +1,845 @@
+// Backward pass of the chunked gated delta rule (gfx950, 64-token chunks, K = V = 128; the host pads smaller head dims).
+// Replaces the reference's backward pipeline fla/ops/gated_delta_rule/chunk.py:125-257 (recompute_w_u_fwd,
+// chunk_gated_delta_rule_fwd_h, chunk_bwd_dv_local, chunk_gated_delta_rule_bwd_dhu, chunk_bwd_dqkwg, prepare_wy_repr_bwd,
+// reverse chunk_local_cumsum) by five kernels:
+//
+//   prepare   per (chunk, v-head)      gam = cumsum(g), A = (I + diag(beta) stril(k k^T o D))^-1, w = A (beta e^gam k), u = A (beta v),
+//                                      P^T with P = scale tril(q k^T o D);  D_ij = e^(gam_i - gam_j)
+//   state     per (sequence, v-head, 32 value columns), chunks in order:   S_c (state in front of chunk c), v_new = u - w S_c
+//   dstate    the same units, chunks in reverse order:   dS_c (gradient of the state behind chunk c),
+//                                      dv_new = P^T do + (k e^(gam_last - gam)) dS_c,  dS <- e^gam_last dS + scale (q e^gam)^T do - w^T dv_new
+//   dqkw      per (chunk, v-head)      dq, the parts of dk and dgam that come from the output and the state update, dw = -dv_new S^T
+//   wy        per (chunk, v-head)      through w, u, A back to k, v, beta, gam; dg = reverse cumulative sum of dgam
+//
+// All matrix products run on the matrix cores from row-major LDS tiles.  A product's two operands have the same register
+// layout (lane (c16, g) holds index c16 and the 8 contraction indices 8g .. 8g+7 of a 32-wide step), so there are just two
+// ways to fetch an operand fragment from a row-major tile: `frag_rows` (the contraction runs along a row: one 16-byte read)
+// and `frag_cols` (the contraction runs down a column: two transposing LDS reads).  The result of run(a, b) holds, in lane
+// (c16, g), column c16 (b's index) and rows 4g .. 4g+3 (a's index): whichever side carries the features gets them four in a
+// row per lane, which is what an 8-byte store into a row-major [token][feature] array wants.
+#include "gdn_chunk_common.h"
+
+namespace gdn {
+
+constexpr int BD = 128;              // head dims of these kernels
+constexpr int P128 = BD + 8;         // LDS pitch, in elements, of a [64][128] tile
+constexpr int P64 = CH + 8;          // ... of a [64][64] tile
+constexpr int VB = 32;               // value columns per workgroup of the two scans
+constexpr int PVB = VB + 8;
+constexpr int VS = BD / VB;
+constexpr int PL = CH + 4;           // pitch of the fp32 matrix L
+
+// Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels),
+// A [64][64], P^T [64][64], w [64][128], u -> v_new [64][128], S [128][128] ([K][V]), dS [128][128], dv_new [64][128],
+// dw [64][128], all in the operand type.
+struct BwdWs {
+    float* Gam; float* Dgam;
+    void* Am; void* PT; void* Wm; void* Vn; void* Hs; void* dHs; void* dVn; void* dWm;
+};
+inline size_t bwd_ws_layout(int64_t units, char* base, BwdWs* ws) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
+    const size_t u = (size_t)units;
+    void* Gam = take(u * 64 * 4); void* Dgam = take(u * 64 * 4);
+    void* Am = take(u * 64 * 64 * 2); void* PT = take(u * 64 * 64 * 2);
+    void* Wm = take(u * 64 * BD * 2); void* Vn = take(u * 64 * BD * 2);
+    void* Hs = take(u * BD * BD * 2); void* dHs = take(u * BD * BD * 2);
+    void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * BD * 2);
+    if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm};
+    return off;
+}
+
+struct BwdParams {
+    const void* q; const void* k; const void* v; const void* g; const void* beta;
+    const float* h0; const void* dout; const float* dht;
+    void* dq; void* dk; void* dv; float* dg; float* dbeta; float* dh0;
+    const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
+    BwdWs ws;
+    int64_t T; int H, HV; int64_t N; int64_t NT;
+    float scale; int gb_dtype; uint32_t flags;
+};
+
+// ---- geometry ------------------------------------------------------------------------------
+struct ChunkAt { int64_t tok0; int valid; };
+__device__ __forceinline__ ChunkAt chunk_at(const BwdParams& p, int64_t ci) {
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    if (p.cu_seqlens) {
+        const int64_t n = load_index(p.chunk_table, 2 * ci, cu32), it = load_index(p.chunk_table, 2 * ci + 1, cu32);
+        const int64_t bos = load_index(p.cu_seqlens, n, cu32), eos = load_index(p.cu_seqlens, n + 1, cu32);
+        const int64_t t0 = bos + it * CH;
+        return ChunkAt{t0, (int)min((int64_t)CH, eos - t0)};
+    }
+    const int64_t b = ci / p.NT, it = ci % p.NT;
+    return ChunkAt{b * p.T + it * CH, (int)min((int64_t)CH, p.T - it * CH)};
+}
+struct SeqAt { int64_t bos, len, cbase, nc; };
+__device__ __forceinline__ SeqAt seq_at(const BwdParams& p, int64_t n) {
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    SeqAt s;
+    if (p.cu_seqlens) {
+        s.bos = load_index(p.cu_seqlens, n, cu32);
+        s.len = load_index(p.cu_seqlens, n + 1, cu32) - s.bos;
+        s.cbase = load_index(p.chunk_offsets, n, cu32);
+    } else {
+        s.bos = n * p.T; s.len = p.T; s.cbase = n * p.NT;
+    }
+    s.nc = (s.len + CH - 1) / CH;
+    return s;
+}
+
+// ---- tiles ---------------------------------------------------------------------------------
+// 64 rows of NCOLS elements from global memory (row r at g + r * stride; rows from `valid` on read as zero) into a
+// row-major LDS tile, by all 256 threads.  Loads first, stores after: the loads of one tile are in flight together.
+template <int NCOLS, typename T>
+__device__ __forceinline__ void load_tile(T* s, int pitch, const T* g, int64_t stride, int valid, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+    u32x4 x[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        x[i] = u32x4{0u, 0u, 0u, 0u};
+        if (idx < TOTAL && row < valid) x[i] = *(const u32x4*)(g + row * stride + pc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = x[i];
+    }
+}
+
+// operand fragment whose contraction runs along a row: index r0 + c16, contraction c0 + 8g + e
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V8 frag_rows(const T* s, int pitch, int r0, int c0, int lane) {
+    return *(const typename Mma<T>::V8*)(s + (r0 + (lane & 15)) * pitch + c0 + 8 * (lane >> 4));
+}
+// operand fragment whose contraction runs down a column: index c0 + c16, contraction r0 + 8g + e
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V8 frag_cols(const T* s, int pitch, int r0, int c0, int lane) {
+    const int a = lane & 15;
+    const T* at = s + (r0 + 8 * (lane >> 4) + (a >> 2)) * pitch + c0 + 4 * (a & 3);
+    return join<typename Mma<T>::V8>(Mma<T>::tr_read(at), Mma<T>::tr_read(at + 4 * pitch));
+}
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::V4 pack4(f32x4 x) {
+    return typename Mma<T>::V4{(T)x[0], (T)x[1], (T)x[2], (T)x[3]};
+}
+__device__ __forceinline__ float sum_over_g(float x) {          // over the four lanes that share c16
+    x += __shfl_xor(x, 16, 64);
+    return x + __shfl_xor(x, 32, 64);
+}
+__device__ __forceinline__ float sum_over_c16(float x) {        // over the sixteen lanes that share g
+    x += __shfl_xor(x, 1, 64); x += __shfl_xor(x, 2, 64); x += __shfl_xor(x, 4, 64);
+    return x + __shfl_xor(x, 8, 64);
+}
+#define ZERO4 (f32x4{0.f, 0.f, 0.f, 0.f})
+
+// ---------------------------------------------------------------------------------------------
+// prepare
+// ---------------------------------------------------------------------------------------------
+constexpr size_t BWD_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PL + 128) * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
+    float* sL = (float*)(sA + 64 * P64); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int64_t u = blockIdx.x, ci = u / p.HV;
+    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+    const ChunkAt c = chunk_at(p, ci);
+
+    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    load_tile<BD>(sV, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    if (w == 0) {
+        float x = 0.f, b = 0.f;
+        if (lane < c.valid) {
+            x = p.g ? load_scalar(p.g, (c.tok0 + lane) * p.HV + hv, p.gb_dtype) : 0.f;
+            b = load_scalar(p.beta, (c.tok0 + lane) * p.HV + hv, p.gb_dtype);
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float y = __shfl_up(x, off, 64);
+            if (lane >= off) x += y;
+        }
+        sGam[lane] = x; sBeta[lane] = b;
+        p.ws.Gam[u * 64 + lane] = x;
+    }
+    __syncthreads();
+
+    // strip of 16 token rows per wave: L (fp32, for the substitution) and P^T
+    {
+        T* PTu = (T*)p.ws.PT + u * 64 * 64;
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            f32x4 kk = ZERO4, qk = ZERO4;
+            if (tj <= w) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const V8 b = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+                    kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), b, kk);
+                    qk = Mma<T>::run(frag_rows(sQ, P128, 16 * w, 32 * s, lane), b, qk);
+                }
+            }
+            const int j = 16 * tj + c16;
+            const float gj = sGam[j];
+            f32x4 pt;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * w + 4 * g + r;
+                const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
+                if (tj <= w) sL[i * PL + j] = i > j ? sBeta[i] * kk[r] * d : 0.f;
+                pt[r] = p.scale * qk[r] * d;
+            }
+            *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
+        }
+    }
+    __syncthreads();
+
+    // A = (I + L)^-1 by forward substitution: lane c owns column c, A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c]
+    if (w == 0) {
+        float a[64];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            float acc[4] = {i == lane ? 1.f : 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j4 = 0; 4 * j4 < i; ++j4) {
+                const f32x4 l = *(const f32x4*)(sL + i * PL + 4 * j4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (4 * j4 + e < i) acc[e] -= l[e] * a[4 * j4 + e];
+            }
+            a[i] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+            sA[i * P64 + lane] = (T)a[i];
+        }
+    }
+    // meanwhile the other waves turn k into beta e^gam k and v into beta v, in place
+    else {
+        for (int idx = tid - 64; idx < 64 * 16; idx += 192) {
+            const int row = idx >> 4, pc = idx & 15;
+            const float bk = sBeta[row] * __expf(sGam[row]), bv = sBeta[row];
+            V8 x = *(V8*)(sK + row * P128 + pc * 8), y = *(V8*)(sV + row * P128 + pc * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { x[e] = (T)((float)x[e] * bk); y[e] = (T)((float)y[e] * bv); }
+            *(V8*)(sK + row * P128 + pc * 8) = x;
+            *(V8*)(sV + row * P128 + pc * 8) = y;
+        }
+    }
+    __syncthreads();
+    {
+        T* Au = (T*)p.ws.Am + u * 64 * 64;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+            *(u32x4*)(Au + row * 64 + pc * 8) = *(const u32x4*)(sA + row * P64 + pc * 8);
+        }
+    }
+    // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
+    {
+        T* Wu = (T*)p.ws.Wm + u * 64 * BD;
+        T* Uu = (T*)p.ws.Vn + u * 64 * BD;
+        const int i = 16 * w + c16;
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            f32x4 aw = ZERO4, au = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (2 * s > w) continue;                        // A is lower triangular
+                const V8 b = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+                aw = Mma<T>::run(frag_cols(sK, P128, 32 * s, 16 * n, lane), b, aw);
+                au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), b, au);
+            }
+            *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
+            *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// state scan: S_c and v_new.  The state slice [128][32] lives in registers, transposed tiles: wave w holds key rows
+// 32w .. 32w+31 as two tiles (a2), lane (c16, g) key 16(2w+a2) + c16 and value columns 16b + 4g .. +3.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t BWD_STATE_SMEM = (2 * 64 * P128 + 128 * PVB + 64 * PVB) * 2 + 64 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sW = (T*)smem; T* sK = sW + 64 * P128; T* sS = sK + 64 * P128; T* sVn = sS + 128 * PVB;
+    float* sGam = (float*)(sVn + 64 * PVB);
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int vs = blockIdx.x % VS, hv = (blockIdx.x / VS) % p.HV, hq = hv / (p.HV / p.H);
+    const int64_t n = blockIdx.x / (VS * p.HV);
+    const SeqAt sq = seq_at(p, n);
+    const int vcol0 = vs * VB;
+
+    f32x4 S[2][2];
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int kk = 16 * (2 * w + a2) + c16;
+            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+        }
+    for (int64_t ic = 0; ic < sq.nc; ++ic) {
+        const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
+        const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
+        load_tile<BD>(sW, P128, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        load_tile<BD>(sK, P128, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        if (tid < 64) sGam[tid] = p.ws.Gam[u * 64 + tid];
+        T* Hu = (T*)p.ws.Hs + u * BD * BD;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int kk = 16 * (2 * w + a2) + c16;
+                const V4 s4 = pack4<T>(S[a2][b]);
+                *(V4*)(sS + kk * PVB + 16 * b + 4 * g) = s4;
+                *(V4*)(Hu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
+            }
+        __syncthreads();
+        const float glast = sGam[63];
+        {
+            // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
+            const int i = 16 * w + c16;
+            const float dec = __expf(glast - sGam[i]);
+            T* Vu = (T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                f32x4 acc = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    acc = Mma<T>::run(frag_cols(sS, PVB, 32 * s, 16 * b, lane), frag_rows(sW, P128, 16 * w, 32 * s, lane), acc);
+                const V4 u4 = *(const V4*)(Vu + 16 * b + 4 * g);
+                f32x4 vn;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[r] - acc[r];
+                const V4 vn4 = pack4<T>(vn);
+                *(V4*)(Vu + 16 * b + 4 * g) = vn4;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vn[r] = (float)vn4[r] * dec;
+                *(V4*)(sVn + i * PVB + 16 * b + 4 * g) = pack4<T>(vn);
+            }
+        }
+        __syncthreads();
+        {
+            const float eg = __expf(glast);
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    f32x4 acc = S[a2][b] * eg;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        acc = Mma<T>::run(frag_cols(sVn, PVB, 32 * s, 16 * b, lane),
+                                          frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
+                    S[a2][b] = acc;
+                }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// reverse scan: dS_c and dv_new; same ownership of the state slice as above
+// ---------------------------------------------------------------------------------------------
+constexpr size_t BWD_DSTATE_SMEM = (3 * 64 * P128 + 64 * P64 + 3 * 64 * PVB + 128 * PVB) * 2 + 64 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sW = sQ + 64 * P128; T* sPT = sW + 64 * P128;
+    T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PVB; T* sDvn = sDOg + 64 * PVB; T* sDS = sDvn + 64 * PVB;
+    float* sGam = (float*)(sDS + 128 * PVB);
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int vs = blockIdx.x % VS, hv = (blockIdx.x / VS) % p.HV, hq = hv / (p.HV / p.H);
+    const int64_t n = blockIdx.x / (VS * p.HV);
+    const SeqAt sq = seq_at(p, n);
+    const int vcol0 = vs * VB;
+
+    f32x4 dS[2][2];
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int kk = 16 * (2 * w + a2) + c16;
+            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+        }
+    for (int64_t ic = sq.nc - 1; ic >= 0; --ic) {
+        const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
+        const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
+        load_tile<BD>(sK, P128, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        load_tile<BD>(sQ, P128, (const T*)p.q + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        load_tile<BD>(sW, P128, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        load_tile<CH>(sPT, P64, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
+        load_tile<VB>(sDO, PVB, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
+        if (tid < 64) sGam[tid] = p.ws.Gam[u * 64 + tid];
+        T* dHu = (T*)p.ws.dHs + u * BD * BD;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int kk = 16 * (2 * w + a2) + c16;
+                const V4 s4 = pack4<T>(dS[a2][b]);
+                *(V4*)(sDS + kk * PVB + 16 * b + 4 * g) = s4;
+                *(V4*)(dHu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
+            }
+        __syncthreads();
+        const float glast = sGam[63];
+        {
+            // scale e^gam_i do_i, for the state's gradient
+            const int row = tid >> 2, pc = tid & 3;
+            const float f = p.scale * __expf(sGam[row]);
+            V8 x = *(const V8*)(sDO + row * PVB + pc * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
+            *(V8*)(sDOg + row * PVB + pc * 8) = x;
+        }
+        {
+            // dv_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
+            const int j = 16 * w + c16;
+            const float dec = __expf(glast - sGam[j]);
+            T* dVu = (T*)p.ws.dVn + u * 64 * BD + j * BD + vcol0;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                f32x4 a1 = ZERO4, a2v = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s + 31 < 16 * w) continue;         // P^T[j][i] = 0 for i < j
+                    a1 = Mma<T>::run(frag_cols(sDO, PVB, 32 * s, 16 * b, lane), frag_rows(sPT, P64, 16 * w, 32 * s, lane), a1);
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    a2v = Mma<T>::run(frag_cols(sDS, PVB, 32 * s, 16 * b, lane), frag_rows(sK, P128, 16 * w, 32 * s, lane), a2v);
+                f32x4 dvn = a1 + a2v * dec;
+                *(V4*)(dVu + 16 * b + 4 * g) = pack4<T>(dvn);
+                *(V4*)(sDvn + j * PVB + 16 * b + 4 * g) = pack4<T>(-dvn);
+            }
+        }
+        __syncthreads();
+        {
+            const float eg = __expf(glast);
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    f32x4 acc = dS[a2][b] * eg;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        acc = Mma<T>::run(frag_cols(sDOg, PVB, 32 * s, 16 * b, lane),
+                                          frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
+                        acc = Mma<T>::run(frag_cols(sDvn, PVB, 32 * s, 16 * b, lane),
+                                          frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
+                    }
+                    dS[a2][b] = acc;
+                }
+        }
+        __syncthreads();
+    }
+    if (p.dh0) {
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int kk = 16 * (2 * w + a2) + c16;
+                *(f32x4*)(p.dh0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dq, dw and the first parts of dk and dgam.  Wave w owns key features 32w .. 32w+31 (two tiles a2) of all 64 tokens
+// (four tiles t): lane (c16, g) holds token 16t + c16 and features 16(2w+a2) + 4g .. +3.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t BWD_DQKW_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + 128 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_dqkw_kernel(BwdParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sDP = sDvn + 64 * P128;
+    float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;
+    T* sK = sVn; T* sQ = sDvn;                                   // second phase
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int64_t u = blockIdx.x, ci = u / p.HV;
+    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+    const ChunkAt c = chunk_at(p, ci);
+
+    load_tile<BD>(sDO, P128, (const T*)p.dout + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    load_tile<BD>(sVn, P128, (const T*)p.ws.Vn + u * 64 * BD, BD, 64, tid);
+    load_tile<BD>(sDvn, P128, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+    if (tid < 64) { sGam[tid] = p.ws.Gam[u * 64 + tid]; sDg[tid] = 0.f; }
+    __syncthreads();
+
+    f32x4 G1[2][4], dWt[2][4], dKS[2][4];
+    float sdot = 0.f;
+    {
+        const T* Hu = (const T*)p.ws.Hs + u * BD * BD;
+        const T* dHu = (const T*)p.ws.dHs + u * BD * BD;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[a2][t] = dKS[a2][t] = ZERO4;
+            const int kk = 16 * (2 * w + a2) + c16;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const V8 sf = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
+                const V8 df = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sdot += (float)sf[e] * (float)df[e];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    G1[a2][t] = Mma<T>::run(sf, frag_rows(sDO, P128, 16 * t, 32 * s, lane), G1[a2][t]);
+                    dWt[a2][t] = Mma<T>::run(sf, frag_rows(sDvn, P128, 16 * t, 32 * s, lane), dWt[a2][t]);
+                    dKS[a2][t] = Mma<T>::run(df, frag_rows(sVn, P128, 16 * t, 32 * s, lane), dKS[a2][t]);
+                }
+            }
+        }
+    }
+    // dP o D for this wave's 16 token rows, as an operand tile
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+        f32x4 acc = ZERO4;
+        if (tj <= w) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                acc = Mma<T>::run(frag_rows(sDO, P128, 16 * w, 32 * s, lane), frag_rows(sVn, P128, 16 * tj, 32 * s, lane), acc);
+        }
+        const int j = 16 * tj + c16;
+        const float gj = sGam[j];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = 16 * w + 4 * g + r;
+            sDP[i * P64 + j] = (T)(i >= j ? p.scale * acc[r] * __expf(sGam[i] - gj) : 0.f);
+        }
+    }
+    {
+        T* dWu = (T*)p.ws.dWm + u * 64 * BD;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[a2][t]);
+    }
+    __syncthreads();
+    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    __syncthreads();
+
+    const float glast = sGam[63];
+    float dglast = __expf(glast) * sdot;
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2) {
+        const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int x = 16 * t + c16;
+            const float gx = sGam[x];
+            f32x4 dq = G1[a2][t] * (p.scale * __expf(gx));
+            f32x4 dk = dKS[a2][t] * __expf(glast - gx);
+            const V4 q4 = *(const V4*)(sQ + x * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dglast += (float)k4[r] * dk[r];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (32 * s <= 16 * t + 15)                      // dP[i][j] = 0 for j > i
+                    dq = Mma<T>::run(frag_cols(sK, P128, 32 * s, n16, lane), frag_rows(sDP, P64, 16 * t, 32 * s, lane), dq);
+                if (32 * s + 31 >= 16 * t)                      // ... and for i < j
+                    dk = Mma<T>::run(frag_cols(sQ, P128, 32 * s, n16, lane), frag_cols(sDP, P64, 32 * s, 16 * t, lane), dk);
+            }
+            float dgx = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dgx += (float)q4[r] * dq[r] - (float)k4[r] * dk[r];
+            dgx = sum_over_g(dgx);
+            if (g == 0) atomicAdd(&sDg[x], dgx);
+            if (x < c.valid) {
+                *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq);
+                *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk);
+            }
+        }
+    }
+    dglast = sum_over_c16(sum_over_g(dglast));
+    if (lane == 0) atomicAdd(&sDg[63], dglast);
+    __syncthreads();
+    if (tid < 64) p.ws.Dgam[u * 64 + tid] = sDg[tid];
+}
+
+// ---------------------------------------------------------------------------------------------
+// back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
+// ---------------------------------------------------------------------------------------------
+constexpr size_t BWD_WY_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 256 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_wy_kernel(BwdParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* X0 = (T*)smem; T* X1 = X0 + 64 * P128; T* sA = X1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
+    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 64;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int64_t u = blockIdx.x, ci = u / p.HV;
+    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+    const ChunkAt c = chunk_at(p, ci);
+
+    load_tile<BD>(X0, P128, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+    load_tile<BD>(X1, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    load_tile<CH>(sA, P64, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
+    if (tid < 64) {
+        sGam[tid] = p.ws.Gam[u * 64 + tid];
+        sBeta[tid] = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        sDg[tid] = p.ws.Dgam[u * 64 + tid];
+        sDb[tid] = 0.f;
+    }
+    __syncthreads();
+
+    // dX = du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), dv = beta (A^T du)
+    f32x4 dX[4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+        dX[tj] = ZERO4;
+        if (tj <= w) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                dX[tj] = Mma<T>::run(frag_rows(X0, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tj, 32 * s, lane), dX[tj]);
+        }
+    }
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2) {
+        const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            f32x4 acc = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (32 * s + 31 < 16 * t) continue;             // A[i][j] = 0 for i < j
+                acc = Mma<T>::run(frag_cols(X0, P128, 32 * s, n16, lane), frag_cols(sA, P64, 32 * s, 16 * t, lane), acc);
+            }
+            const int j = 16 * t + c16;
+            const V4 v4 = *(const V4*)(X1 + j * P128 + n16 + 4 * g);
+            float db = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) db += acc[r] * (float)v4[r];
+            db = sum_over_g(db);
+            if (g == 0) atomicAdd(&sDb[j], db);
+            if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(acc * sBeta[j]);
+        }
+    }
+    __syncthreads();
+    load_tile<BD>(X0, P128, (const T*)p.ws.dWm + u * 64 * BD, BD, 64, tid);
+    load_tile<BD>(X1, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    __syncthreads();
+
+    // dX += dw (e^gam k)^T;  dA = stril(dX diag(beta)) as an operand tile
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+        f32x4 acc = ZERO4;
+        if (tj <= w) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                acc = Mma<T>::run(frag_rows(X0, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tj, 32 * s, lane), acc);
+        }
+        const int j = 16 * tj + c16;
+        const float ej = __expf(sGam[j]), bj = sBeta[j];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = 16 * w + 4 * g + r;
+            sM1[i * P64 + j] = (T)(i > j ? (dX[tj][r] + ej * acc[r]) * bj : 0.f);
+        }
+    }
+    // d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
+    f32x4 dk[2][4];
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2) {
+        const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            f32x4 acc = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (32 * s + 31 < 16 * t) continue;
+                acc = Mma<T>::run(frag_cols(X0, P128, 32 * s, n16, lane), frag_cols(sA, P64, 32 * s, 16 * t, lane), acc);
+            }
+            const int j = 16 * t + c16;
+            const V4 k4 = *(const V4*)(X1 + j * P128 + n16 + 4 * g);
+            float dot = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dot += acc[r] * (float)k4[r];
+            dot = sum_over_g(dot);
+            const float ej = __expf(sGam[j]), bj = sBeta[j];
+            if (g == 0) { atomicAdd(&sDb[j], ej * dot); atomicAdd(&sDg[j], bj * ej * dot); }
+            dk[a2][t] = acc * (bj * ej);
+        }
+    }
+    __syncthreads();
+    // Y = dA A^T
+#pragma unroll
+    for (int tl = 0; tl < 4; ++tl) {
+        f32x4 acc = ZERO4;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            acc = Mma<T>::run(frag_rows(sM1, P64, 16 * w, 32 * s, lane), frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+        const int l = 16 * tl + c16;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+    }
+    __syncthreads();
+    // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
+    {
+        float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            f32x4 acc = ZERO4, kk = ZERO4;
+            if (tl <= w) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    acc = Mma<T>::run(frag_cols(sA, P64, 32 * s, 16 * w, lane), frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    kk = Mma<T>::run(frag_rows(X1, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tl, 32 * s, lane), kk);
+            }
+            const int l = 16 * tl + c16;
+            const float gl = sGam[l];
+            float colF = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * w + 4 * g + r;
+                float E = 0.f;
+                if (i > l) {
+                    const float d = __expf(sGam[i] - gl), dL = -acc[r];
+                    dbi[r] += dL * kk[r] * d;
+                    E = dL * sBeta[i] * d;
+                    const float F = E * kk[r];
+                    rowF[r] += F;
+                    colF += F;
+                }
+                sM1[i * P64 + l] = (T)E;
+            }
+            colF = sum_over_g(colF);
+            if (g == 0 && tl <= w) atomicAdd(&sDg[l], -colF);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
+            if (c16 == 0) { atomicAdd(&sDb[16 * w + 4 * g + r], a); atomicAdd(&sDg[16 * w + 4 * g + r], b); }
+        }
+    }
+    __syncthreads();
+    // dk += E k + E^T k, on top of what the previous kernel left
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2) {
+        const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            f32x4 acc = dk[a2][t];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const V8 af = frag_cols(X1, P128, 32 * s, n16, lane);
+                if (32 * s <= 16 * t + 15) acc = Mma<T>::run(af, frag_rows(sM1, P64, 16 * t, 32 * s, lane), acc);     // E[i][l], l < i
+                if (32 * s + 31 >= 16 * t) acc = Mma<T>::run(af, frag_cols(sM1, P64, 32 * s, 16 * t, lane), acc);     // E[i][l], i > l
+            }
+            const int x = 16 * t + c16;
+            if (x < c.valid) {
+                T* at = (T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g;
+                const V4 old = *(const V4*)at;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[r] += (float)old[r];
+                *(V4*)at = pack4<T>(acc);
+            }
+        }
+    }
+    if (w == 0) {
+        float x = sDg[lane];
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float y = __shfl_down(x, off, 64);
+            if (lane + off < 64) x += y;
+        }
+        if (lane < c.valid) {
+            p.dg[(c.tok0 + lane) * p.HV + hv] = x;
+            p.dbeta[(c.tok0 + lane) * p.HV + hv] = sDb[lane];
+        }
+    }
+}
+
+template <typename T>
+static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream) {
+    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)(p.N * p.HV * VS);
+    static SmemAttrDone done[5];
+    struct K { const void* f; size_t smem; const char* name; unsigned grid; };
+    const K ks[5] = {
+        {(const void*)gdn_bwd_prepare_kernel<T>, BWD_PREP_SMEM, "gdn_bwd_prepare_kernel", units},
+        {(const void*)gdn_bwd_state_kernel<T>, BWD_STATE_SMEM, "gdn_bwd_state_kernel", runs},
+        {(const void*)gdn_bwd_dstate_kernel<T>, BWD_DSTATE_SMEM, "gdn_bwd_dstate_kernel", runs},
+        {(const void*)gdn_bwd_dqkw_kernel<T>, BWD_DQKW_SMEM, "gdn_bwd_dqkw_kernel", units},
+        {(const void*)gdn_bwd_wy_kernel<T>, BWD_WY_SMEM, "gdn_bwd_wy_kernel", units},
+    };
+    for (int i = 0; i < 5; ++i) {
+        if (int rc = ensure_dynamic_smem(ks[i].f, ks[i].smem, done[i], ks[i].name)) return rc;
+        void* args[] = {(void*)&p};
+        if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
+        if (int rc = check_launch(ks[i].name)) return rc;
+    }
+    return GDN_OK;
+}
+
+}  // namespace gdn
+
+extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV) {
+    if (num_chunks < 0 || HV < 1) return 0;
+    return gdn::bwd_ws_layout(num_chunks * HV, nullptr, nullptr);
+}
+
+extern "C" int gdn_chunk_bwd(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    using namespace gdn;
+    const char* who = "gdn_chunk_bwd";
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
+    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
+                  who, (long long)K, (long long)V);
+    GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
+    GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
+                  "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * VS < (1ll << 31), GDN_ERR_UNSUPPORTED,
+                  "%s: too many heads or chunks for one launch", who);
+    if (cu_seqlens) {
+        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
+        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
+    } else {
+        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
+        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0 || num_chunks == 0) {
+        if (dh0) return launch_state_copy(dht, dh0, N * HV * K * V, s);
+        return GDN_OK;
+    }
+    GDN_CHECK_ARG(q && k && v && beta && dout && dq && dk && dv && dg && dbeta, GDN_ERR_INVALID,
+                  "%s: q, k, v, beta, do, dq, dk, dv, dg, dbeta must not be NULL", who);
+    for (const void* x : {q, k, v, dout, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dv, (const void*)dh0})
+        GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
+    GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
+    BwdParams p;
+    const size_t need = bwd_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
+    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
+                  need, workspace_bytes);
+    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
+    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0;
+    p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t>(p, num_chunks, s) : launch_bwd<f16_t>(p, num_chunks, s);
+}

@@ -243,7 +243,7 @@ def chunk_gated_delta_rule(
     cp_context=None,
     **kwargs,
 ):
-    r"""Chunked gated delta rule (prefill), forward only.
+    r"""Chunked gated delta rule (prefill; differentiable: inputs that require a gradient get one).
 
     Args:
         q, k: ``[B, T, H, K]``.  v: ``[B, T, HV, V]`` with ``HV % H == 0`` (grouped value heads).
@@ -305,6 +305,14 @@ def chunk_gated_delta_rule(
     if scale is None:
         scale = k.shape[-1] ** -0.5
 
+    if torch.is_grad_enabled() and any(
+            x is not None and x.requires_grad for x in (q, k, v, g, beta, initial_state, A_log, dt_bias)):
+        # training: the same forward kernels inside an autograd function (chunk.py:260-395)
+        from fla_hip.ops.gated_delta_rule.chunk_bwd import ChunkGatedDeltaRuleFunction
+        return ChunkGatedDeltaRuleFunction.apply(
+            q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first, cu_seqlens, cu_seqlens_cpu,
+            chunk_indices, use_qk_l2norm_in_kernel, use_gate_in_kernel, A_log, dt_bias,
+            use_beta_sigmoid_in_kernel, allow_neg_eigval, chunk_size)
     # the prologues the reference runs as separate launches before its chunk pipeline
     # (chunk.py:278-288, gate.py:63-106) happen inside the first kernel
     return chunk_gated_delta_rule_fwd(

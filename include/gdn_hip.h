@@ -206,6 +206,35 @@ int gdn_chunk_fwd_scan(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Backward pass of the chunked operator.  Replaces chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:125-257):
+ * recompute_w_u_fwd (fla/ops/gated_delta_rule/wy_fast.py:236-296), chunk_gated_delta_rule_fwd_h and
+ * chunk_gated_delta_rule_bwd_dhu (fla/ops/common/chunk_delta_h.py:563-744, 747-828), chunk_bwd_dv_local and
+ * chunk_bwd_dqkwg (fla/ops/common/chunk_o.py:647-697, 700-779), prepare_wy_repr_bwd (wy_fast.py:298-351) and the
+ * reverse chunk_local_cumsum of dg (fla/ops/utils/cumsum.py).  Nothing is kept from the forward call: A, w, u, the
+ * per-chunk states and v_new are computed again, into the workspace.
+ *   q, k [B,T,H,K]; v, dout [B,T,HV,V] (qkv_dtype: bf16 or f16); g (log decay, may be NULL), beta [B,T,HV] (gb_dtype),
+ *   both as the recurrence uses them: the activations of the forward call (l2 norm, gate, sigmoid) and their
+ *   derivatives are the caller's, as in the reference (chunk.py:278-288, 385-393)
+ *   h0, dht [N,HV,K,V] fp32 or NULL
+ *   dq, dk [B,T,HV,K], dv [B,T,HV,V] in qkv_dtype: per VALUE head; with grouped heads the caller adds the HV/H
+ *   gradients that belong to one q/k head; dg, dbeta [B,T,HV] fp32; dh0 [N,HV,K,V] fp32 or NULL
+ *   cu_seqlens, chunk_table, chunk_offsets ([N+1] here), N, num_chunks: as for gdn_chunk_fwd
+ *   workspace: at least gdn_chunk_bwd_workspace_bytes(num_chunks, HV) bytes, 256-byte aligned
+ *   flags: GDN_FLAG_CU_INT32 only.  K = V = 128 only: the Python host zero-pads smaller head dims.
+ *   T == 0: dh0 = dht (zeros without dht), nothing else is written.
+ */
+size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV);
+int gdn_chunk_bwd(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * gdn_chunk_fwd minus the workspace: the kernels use a fixed array of GDN_CHUNK_STATIC_WORKSPACE_BYTES that the

@@ -77,10 +77,11 @@ def l2norm(x: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
 
 def gdn_gate(g: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor | None = None) -> torch.Tensor:
     """g = -exp(A_log) * softplus(g + dt_bias) (fla/ops/gated_delta_rule/gate.py:21-46)."""
-    g = g.float()
+    dt = torch.float64 if g.dtype == torch.float64 else torch.float32
+    g = g.to(dt)
     if dt_bias is not None:
-        g = g + dt_bias.float()
-    return -A_log.float().exp() * F.softplus(g)
+        g = g + dt_bias.to(dt)
+    return -A_log.to(dt).exp() * F.softplus(g)
 
 
 def kda_gate(g: torch.Tensor, A_log: torch.Tensor | None = None, dt_bias: torch.Tensor | None = None,
@@ -430,3 +431,138 @@ def make_varlen_lengths(total: int, n_seq: int, lo: int, hi: int, seed: int = 42
         L[i % n_seq] += 1
     assert int(L.sum()) == total and int(L.min()) >= 1
     return [int(x) for x in L]
+
+
+# --------------------------------------------------------------------------- #
+# backward
+# --------------------------------------------------------------------------- #
+def gated_delta_rule_grads(
+    q, k, v, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
+    use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, A_log=None, dt_bias=None,
+    use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, state_v_first=False,
+    dtype=torch.float64,
+):
+    """Gradients of  sum(o * do) + sum(ht * dht)  with respect to q, k, v, g, beta, the initial state and
+    (with the gate activation) A_log and dt_bias, by reverse-mode differentiation of the token recurrence
+    above: what the reference's own tests take as the truth for its backward pass
+    (tests/ops/test_gdn.py:160-176, autograd through the naive implementation).  Returns a dict with
+    the keys dq, dk, dv, dg, dbeta, dh0, dA_log, ddt_bias (None where there is no such input)."""
+    leaves = {}
+
+    def leaf(name, x):
+        if x is None:
+            return None
+        leaves[name] = x.detach().to(dtype).clone().requires_grad_(True)
+        return leaves[name]
+
+    q_, k_, v_, g_, b_ = leaf('dq', q), leaf('dk', k), leaf('dv', v), leaf('dg', g), leaf('dbeta', beta)
+    h0_ = leaf('dh0', initial_state)
+    A_ = leaf('dA_log', A_log) if use_gate_in_kernel else None
+    dt_ = leaf('ddt_bias', dt_bias) if use_gate_in_kernel else None
+    o, ht = recurrent_gated_delta_rule(
+        q_, k_, v_, g_, b_, scale=scale, initial_state=h0_, output_final_state=dht is not None, cu_seqlens=cu_seqlens,
+        use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel, use_gate_in_kernel=use_gate_in_kernel, A_log=A_, dt_bias=dt_,
+        use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel, allow_neg_eigval=allow_neg_eigval,
+        state_v_first=state_v_first, dtype=dtype)
+    loss = (o * do.to(dtype)).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.to(dtype)).sum()
+    names = list(leaves)
+    grads = torch.autograd.grad(loss, [leaves[n] for n in names], allow_unused=True)
+    out = dict.fromkeys(('dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0', 'dA_log', 'ddt_bias'))
+    out.update(dict(zip(names, grads)))
+    return out
+
+
+def chunk_backward_one_sequence(q, k, v, g, beta, scale, S0, do, dSt=None, chunk_size=64, dtype=torch.float64):
+    """The reference's chunked backward pass, stage by stage, for ONE sequence with the q/k heads already
+    expanded: q, k [T,HV,K]; v, do [T,HV,V]; g, beta [T,HV]; S0 [HV,K,V]; dSt [HV,K,V] or None.
+    Natural-log gates (gam_r = cumsum(g) inside the chunk).  Returns the gradients and every intermediate.
+
+    Stages (fla/ops/gated_delta_rule/chunk.py:125-257):
+      recompute  A, w = A (beta e^gam k), u = A (beta v); states S_c and v_new = u - w S_c    wy_fast.py:72-106, chunk_delta_h.py:174-348
+      reverse scan over chunks (chunk_delta_h.py:369-560, chunk_o.py:465-560):
+        dv_new = P^T do + (k e^(gam_last - gam)) dS_next,      P = scale tril(q k^T e^(gam_i - gam_j))
+        dS     = e^gam_last dS_next + scale (q e^gam)^T do - w^T dv_new
+      per chunk (chunk_o.py:172-357):
+        dq = scale e^gam (do S^T) + (dP o D) k,  dk = (dP o D)^T q + e^(gam_last - gam) (v_new dS_next^T),
+        dw = -dv_new S^T,   dP = scale tril(do v_new^T),  D_ij = e^(gam_i - gam_j)
+        dgam from every factor e^gam above; dgam_last also from e^gam_last <S, dS_next>
+      WY factors backwards (wy_fast.py:123-296):  X = A diag(beta)
+        dX = tril(dw (e^gam k)^T + du v^T),  d(e^gam k) = X^T dw,  dv = X^T du,
+        dL = -stril(A^T (dX diag(beta)) A^T),  L = diag(beta) stril(k k^T o D)
+      dg = reverse cumulative sum of dgam inside the chunk (cumsum.py, reverse=True)."""
+    T, HV, K = k.shape
+    V = v.shape[-1]
+    C = chunk_size
+    q, k, v, g, beta, do = (x.to(dtype) for x in (q, k, v, g, beta, do))
+    NT = (T + C - 1) // C
+    fwd = []
+    S = S0.to(dtype).clone()
+    for ic in range(NT):
+        c0, c1 = ic * C, min(ic * C + C, T)
+        r = c1 - c0
+        kc, qc, vc, doc = (x[c0:c1].transpose(0, 1) for x in (k, q, v, do))      # [HV,r,*]
+        bc = beta[c0:c1].transpose(0, 1)
+        gam = g[c0:c1].transpose(0, 1).cumsum(-1)                               # [HV,r]
+        diff = gam[:, :, None] - gam[:, None, :]
+        incl = torch.ones(r, r, dtype=torch.bool).tril(0)
+        strict = torch.ones(r, r, dtype=torch.bool).tril(-1)
+        D = torch.where(incl, torch.exp(torch.where(incl, diff, torch.zeros_like(diff))), torch.zeros_like(diff))
+        KK = kc @ kc.transpose(-1, -2)
+        M = torch.where(strict, KK * D, torch.zeros_like(D))
+        eye = torch.eye(r, dtype=dtype).expand(HV, r, r)
+        A = torch.linalg.solve_triangular(eye + bc[:, :, None] * M, eye.clone(), upper=False, unitriangular=True)
+        eg = gam.exp()
+        w = A @ (kc * (bc * eg)[:, :, None])
+        u = A @ (vc * bc[:, :, None])
+        vn = u - w @ S
+        P = scale * (qc @ kc.transpose(-1, -2)) * D
+        glast = gam[:, -1]
+        kb = kc * torch.exp(glast[:, None] - gam)[:, :, None]
+        fwd.append(dict(c0=c0, c1=c1, kc=kc, qc=qc, vc=vc, doc=doc, bc=bc, gam=gam, D=D, M=M, A=A, w=w, u=u, vn=vn, P=P,
+                        S=S.clone(), glast=glast, kb=kb, eg=eg, incl=incl, strict=strict))
+        S = S * glast.exp()[:, None, None] + kb.transpose(-1, -2) @ vn
+    dS = torch.zeros(HV, K, V, dtype=dtype) if dSt is None else dSt.to(dtype).clone()
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    dg, dbeta = torch.zeros_like(g), torch.zeros_like(beta)
+    stages = [None] * NT
+    for ic in reversed(range(NT)):
+        f = fwd[ic]
+        kc, qc, vc, doc, bc, gam, D, M, A, w, vn, P, Sc, glast, kb, eg = (f[n] for n in (
+            'kc', 'qc', 'vc', 'doc', 'bc', 'gam', 'D', 'M', 'A', 'w', 'vn', 'P', 'S', 'glast', 'kb', 'eg'))
+        dSn = dS
+        dvn = P.transpose(-1, -2) @ doc + kb @ dSn
+        dS = dSn * glast.exp()[:, None, None] + scale * (qc * eg[:, :, None]).transpose(-1, -2) @ doc - w.transpose(-1, -2) @ dvn
+        # per chunk
+        dPm = torch.where(f['incl'], scale * (doc @ vn.transpose(-1, -2)) * D, torch.zeros_like(D))
+        dq_c = scale * eg[:, :, None] * (doc @ Sc.transpose(-1, -2)) + dPm @ kc
+        dk_P = dPm.transpose(-1, -2) @ qc
+        dk_S = torch.exp(glast[:, None] - gam)[:, :, None] * (vn @ dSn.transpose(-1, -2))
+        dw = -dvn @ Sc.transpose(-1, -2)
+        dgam = (qc * dq_c).sum(-1) - (kc * (dk_P + dk_S)).sum(-1)
+        dgam[:, -1] += glast.exp() * (Sc * dSn).sum((-1, -2)) + (kc * dk_S).sum((-1, -2))
+        # WY factors
+        X = A * bc[:, None, :]
+        kd = kc * eg[:, :, None]
+        dX = torch.where(f['incl'], dw @ kd.transpose(-1, -2) + dvn @ vc.transpose(-1, -2), torch.zeros_like(D))
+        dkd = X.transpose(-1, -2) @ dw
+        dv_c = X.transpose(-1, -2) @ dvn
+        dk_c = dq_c.new_zeros(kc.shape) + dk_P + dk_S + dkd * eg[:, :, None]
+        dgam = dgam + (kd * dkd).sum(-1)
+        db = (dX * A).sum(-2)
+        dA = dX * bc[:, None, :]
+        dL = torch.where(f['strict'], -(A.transpose(-1, -2) @ dA @ A.transpose(-1, -2)), torch.zeros_like(D))
+        db = db + (dL * M).sum(-1)
+        E = dL * bc[:, :, None] * D
+        dk_c = dk_c + E @ kc + E.transpose(-1, -2) @ kc
+        F_ = E * (kc @ kc.transpose(-1, -2))
+        dgam = dgam + F_.sum(-1) - F_.sum(-2)
+        c0, c1 = f['c0'], f['c1']
+        dq[c0:c1] = dq_c.transpose(0, 1)
+        dk[c0:c1] = dk_c.transpose(0, 1)
+        dv[c0:c1] = dv_c.transpose(0, 1)
+        dbeta[c0:c1] = db.transpose(0, 1)
+        dg[c0:c1] = dgam.flip(-1).cumsum(-1).flip(-1).transpose(0, 1)
+        stages[ic] = dict(A=A, w=w, u=f['u'], S=Sc, vn=vn, P=P, dvn=dvn, dSn=dSn, dw=dw, dgam=dgam)
+    return dict(dq=dq, dk=dk, dv=dv, dg=dg, dbeta=dbeta, dh0=dS, stages=stages)

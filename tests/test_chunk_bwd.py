@@ -1,0 +1,241 @@
+"""Backward of chunk_gated_delta_rule.
+
+CPU part: the oracle's gradients (reverse-mode differentiation of the token recurrence) are pinned by central
+finite differences of the recurrence itself, and the stage-by-stage restatement of the reference's chunked
+backward pass is pinned against those gradients.
+GPU part: gradients from the HIP kernels (autograd through the product's operator, C ABI underneath) against
+the oracle's on the same seeded inputs; cases and tolerances follow the reference's tests
+(tests/ops/test_gdn.py:108-200 dq, dk, dv, dh0 0.008, dbeta, dg 0.02; :281-370; :712-803 packed sequences)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+TOL = dict(dq=0.008, dk=0.008, dv=0.008, dbeta=0.02, dg=0.02, dh0=0.008)
+
+
+# --------------------------------------------------------------------------------------------
+# oracle pins (CPU)
+# --------------------------------------------------------------------------------------------
+def _loss(q, k, v, g, beta, h0, do, dht, **kw):
+    o, ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                         dtype=torch.float64, **kw)
+    return float((o * do).sum() + (ht * dht).sum())
+
+
+@pytest.mark.parametrize('kw', [
+    dict(),
+    dict(use_qk_l2norm_in_kernel=True),
+    dict(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True),
+    dict(use_gate_in_kernel=True),
+    dict(cu_seqlens=[0, 5, 12]),
+    dict(state_v_first=True),
+])
+def test_oracle_grads_match_finite_differences(kw):
+    B, T, H, HV, K, V = (1, 12, 2, 4, 6, 5) if 'cu_seqlens' in kw else (2, 9, 2, 4, 6, 5)
+    N = 2
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=7, h0_std=0.5, N=N, dtype=torch.float64)
+    q, k = q * 1.7, k * 0.8                              # not unit rows: the l2 norm must matter
+    gen = torch.Generator().manual_seed(8)
+    g, beta = g.double(), beta.double()
+    A_log = dt_bias = None
+    if kw.get('use_gate_in_kernel'):
+        g = torch.randn(B, T, HV, generator=gen, dtype=torch.float64)
+        A_log = torch.randn(HV, generator=gen, dtype=torch.float64) * 0.3
+        dt_bias = torch.randn(HV, generator=gen, dtype=torch.float64) * 0.3
+        kw = dict(kw, A_log=A_log, dt_bias=dt_bias)
+    if kw.get('use_beta_sigmoid_in_kernel'):
+        beta = torch.randn(B, T, HV, generator=gen, dtype=torch.float64)
+    h0 = h0.double()
+    if kw.get('state_v_first'):
+        h0 = h0.transpose(-1, -2).contiguous()
+    do = torch.randn(B, T, HV, V, generator=gen, dtype=torch.float64)
+    dht = torch.randn(*h0.shape, generator=gen, dtype=torch.float64)
+    grads = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, **kw)
+    inputs = dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=h0)
+    if A_log is not None:
+        inputs.update(dA_log=A_log, ddt_bias=dt_bias)
+    eps = 1e-6
+    for name, x in inputs.items():
+        d = torch.randn(x.shape, generator=gen, dtype=torch.float64)
+
+        def at(step):
+            args = {n: (t + step * d if n == name else t) for n, t in inputs.items()}
+            kw2 = dict(kw)
+            if A_log is not None:
+                kw2.update(A_log=args['dA_log'], dt_bias=args['ddt_bias'])
+            return _loss(args['dq'], args['dk'], args['dv'], args['dg'], args['dbeta'], args['dh0'], do, dht, **kw2)
+        fd = (at(eps) - at(-eps)) / (2 * eps)
+        an = float((grads[name] * d).sum())
+        assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), f'{name}: finite difference {fd} vs gradient {an}'
+
+
+@pytest.mark.parametrize('T,HV,K,V,C', [(150, 2, 16, 24, 64), (64, 1, 8, 8, 64), (37, 3, 12, 8, 16), (100, 2, 8, 8, 32)])
+def test_oracle_chunked_backward_matches_recurrence_grads(T, HV, K, V, C):
+    q, k, v, g, beta, h0 = O.make_inputs(1, T, HV, HV, K, V, seed=T, h0_std=0.5, dtype=torch.float64)
+    gen = torch.Generator().manual_seed(T + 1)
+    do = torch.randn(1, T, HV, V, generator=gen, dtype=torch.float64)
+    dht = torch.randn(1, HV, K, V, generator=gen, dtype=torch.float64)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, scale=0.3, initial_state=h0)
+    got = O.chunk_backward_one_sequence(q[0], k[0], v[0], g[0], beta[0], 0.3, h0[0], do[0], dht[0], chunk_size=C)
+    for n in TOL:
+        assert O.get_err_ratio(ref[n][0], got[n]) < 1e-12, n
+
+
+# --------------------------------------------------------------------------------------------
+# HIP kernels against the oracle (GPU)
+# --------------------------------------------------------------------------------------------
+def _op():
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    return chunk_gated_delta_rule
+
+
+def _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=None, **kw):
+    dev = 'cuda'
+    leaves = {n: (None if x is None else x.to(dev).requires_grad_(True))
+              for n, x in dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=h0).items()}
+    extra = {}
+    for n in ('A_log', 'dt_bias'):
+        if kw.get(n) is not None:
+            extra['d' + n] = kw[n] = kw[n].to(dev).requires_grad_(True)
+    cu_t = None if cu is None else torch.tensor(cu, dtype=torch.int64, device=dev)
+    o, ht = _op()(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dg'], leaves['dbeta'], initial_state=leaves['dh0'],
+                  output_final_state=dht is not None, cu_seqlens=cu_t, **kw)
+    loss = (o.float() * do.to(dev).float()).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.to(dev)).sum()
+    loss.backward()
+    out = {n: (None if x is None else x.grad) for n, x in leaves.items()}
+    out.update({n: x.grad for n, x in extra.items()})
+    return o, ht, out
+
+
+def _compare(ref, got, tol=TOL, names=None):
+    for n in names or [n for n in ref if ref[n] is not None]:
+        x = got[n].detach().float().cpu()
+        assert x.shape == ref[n].shape, f'{n}: shape {tuple(x.shape)} vs {tuple(ref[n].shape)}'
+        assert not torch.isnan(x).any(), f'{n}: NaN'
+        if O.get_abs_err(ref[n], x) <= 1e-6:       # (fla/utils/_testing.py:28-34: gradients that vanish, e.g. dg under extreme decay)
+            continue
+        r = O.get_err_ratio(ref[n], x)
+        assert r <= tol.get(n, 0.02), f'{n}: rel-rmse {r:.3e} > {tol.get(n, 0.02)}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_div,mask_p,l2,dtype', [
+    (1, 64, 1, 1, 128, None, 1.0, 0, False, torch.bfloat16),
+    (2, 75, 4, 4, 64, 1, 0.01, 0, False, torch.float16),          # the reference's matrix (shorter where it is long)
+    (2, 500, 3, 3, 60, 1, 1, 0, False, torch.float16),
+    (2, 300, 3, 3, 64, 0.1, 1, 0.5, False, torch.float16),
+    (1, 512, 4, 4, 100, 1, 0.1, 0, False, torch.float16),
+    (2, 256, 4, 4, 128, 0.1, 1, 1.0, False, torch.float16),
+    (2, 512, 4, 4, 128, 0.1, 1, 0, True, torch.float16),
+    (1, 700, 4, 4, 128, 0.1, 10, 0, False, torch.float16),
+    (2, 256, 2, 4, 64, 1, 1, 0, False, torch.float16),
+    (2, 512, 2, 8, 64, 1, 0.1, 0, True, torch.float16),
+    (2, 200, 2, 4, 128, None, 4.0, 0, False, torch.bfloat16),
+    (1, 130, 2, 2, 128, None, 4.0, 0, True, torch.bfloat16),
+])
+def test_chunk_backward(B, T, H, HV, D, scale, gate_div, mask_p, l2, dtype):
+    gen = torch.Generator().manual_seed(42)
+    q = torch.rand(B, T, H, D, generator=gen)
+    k = torch.rand(B, T, H, D, generator=gen)
+    if not l2:
+        q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    q, k = q.to(dtype), k.to(dtype)
+    v = torch.rand(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    g = F.logsigmoid(torch.rand(B, T, HV, generator=gen)) / gate_div
+    g = g * (torch.rand(B, T, HV, generator=gen) > mask_p)
+    h0 = torch.randn(B, HV, D, D, generator=gen) * 0.3
+    do = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    dht = torch.randn(B, HV, D, D, generator=gen)
+    kw = dict(scale=scale, use_qk_l2norm_in_kernel=l2)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, dtype=torch.float32, **kw)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, **kw)
+    assert got['dq'].dtype == dtype and got['dv'].dtype == dtype and got['dg'].dtype == g.dtype
+    _compare(ref, got)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('H,HV,D,mask_p,cu', [
+    (4, 4, 60, 0, [0, 15]),
+    (4, 4, 64, 0, [0, 256, 500, 1000]),
+    (4, 4, 64, 0.5, [0, 256, 500, 1000]),
+    (2, 2, 100, 0, [0, 15, 100, 300, 700]),
+    (2, 4, 64, 0, [0, 256, 500, 1000]),
+    (2, 8, 128, 0, [0, 1, 65, 200, 264]),
+])
+def test_chunk_backward_packed(H, HV, D, mask_p, cu):
+    gen = torch.Generator().manual_seed(42)
+    T, N = cu[-1], len(cu) - 1
+    dtype = torch.float16
+    q = torch.randn(1, T, H, D, generator=gen).to(dtype)
+    k = F.normalize(torch.randn(1, T, H, D, generator=gen), p=2, dim=-1).to(dtype)
+    v = torch.randn(1, T, HV, D, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.rand(1, T, HV, generator=gen))
+    g = g * (torch.rand(1, T, HV, generator=gen) > mask_p)
+    beta = torch.rand(1, T, HV, generator=gen).sigmoid()
+    h0 = torch.randn(N, HV, D, D, generator=gen)
+    do = torch.randn(1, T, HV, D, generator=gen).to(dtype)
+    dht = torch.rand(N, HV, D, D, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, dtype=torch.float32)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu)
+    _compare(ref, got, tol=dict(dq=0.007, dk=0.008, dv=0.007, dbeta=0.015, dg=0.015, dh0=0.007))
+    # every sequence's gradients are those of the sequence alone
+    if N > 1:
+        s, e = cu[1], cu[2]
+        _, _, alone = _grads_gpu(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e], h0[1:2], do[:, s:e], dht[1:2])
+        for n in ('dq', 'dk', 'dv'):
+            assert O.get_err_ratio(got[n][:, s:e].float().cpu(), alone[n].float().cpu()) < 2e-3, n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('what', ['beta_sigmoid', 'beta_sigmoid_neg', 'gate', 'gate_no_bias', 'v_first', 'no_h0', 'no_dht',
+                                  'wide_v', 'fp32'])
+def test_chunk_backward_options(what):
+    B, T, H, HV, D = 2, 200, 2, 4, 128
+    V = 256 if what == 'wide_v' else D
+    dtype = torch.float32 if what == 'fp32' else torch.bfloat16
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, D, V, seed=11, gate_div=4.0, h0_std=0.3, dtype=dtype)
+    gen = torch.Generator().manual_seed(12)
+    do = torch.randn(B, T, HV, V, generator=gen).to(dtype)
+    dht = torch.randn(B, HV, D, V, generator=gen)
+    kw = {}
+    if what.startswith('beta_sigmoid'):
+        beta = torch.randn(B, T, HV, generator=gen)
+        kw = dict(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=what.endswith('neg'))
+    if what.startswith('gate'):
+        g = torch.randn(B, T, HV, generator=gen)
+        kw = dict(use_gate_in_kernel=True, A_log=torch.randn(HV, generator=gen) * 0.5,
+                  dt_bias=None if what == 'gate_no_bias' else torch.randn(HV, generator=gen) * 0.5)
+    if what == 'v_first':
+        h0, dht = h0.transpose(-1, -2).contiguous(), dht.transpose(-1, -2).contiguous()
+        kw = dict(state_v_first=True)
+    if what == 'no_h0':
+        h0 = None
+    if what == 'no_dht':
+        dht = None
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, dtype=torch.float32,
+                                   **{n: x for n, x in kw.items()})
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, **dict(kw))
+    _compare(ref, got)
+
+
+@pytest.mark.gpu
+def test_chunk_backward_c_entry_checks():
+    from fla_hip import _lib
+    lib = _lib.load()
+    assert lib.gdn_chunk_bwd_workspace_bytes(4, 2) > 0
+    x = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16, device='cuda')
+    f = torch.zeros(1, 64, 1, device='cuda')
+    ws = torch.zeros(lib.gdn_chunk_bwd_workspace_bytes(1, 1), dtype=torch.uint8, device='cuda')
+    args = [x.data_ptr()] * 3 + [f.data_ptr()] * 2 + [None, x.data_ptr(), None] + [x.data_ptr()] * 3 + [f.data_ptr()] * 2 + [None]
+    rc = lib.gdn_chunk_bwd(*args, None, None, None, ws.data_ptr(), ws.numel(), 1, 64, 1, 1, 64, 64, 1, 1, 1.0,
+                           _lib.DTYPE_BF16, _lib.DTYPE_F32, 0, None)
+    assert rc == _lib.GDN_ERR_UNSUPPORTED and 'K = V = 128' in _lib.last_error()
+    with pytest.raises(NotImplementedError):
+        from fla_hip.ops.gated_delta_rule.chunk_bwd import chunk_gated_delta_rule_bwd
+        w = torch.zeros(1, 64, 1, 256, dtype=torch.bfloat16, device='cuda')
+        chunk_gated_delta_rule_bwd(w, w, w, f, f, 1.0, None, w, None)
