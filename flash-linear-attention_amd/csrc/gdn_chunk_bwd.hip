@@ -24,9 +24,6 @@ namespace gdn {
 constexpr int BD = 128;              // head dims of these kernels
 constexpr int P128 = BD + 8;         // LDS pitch, in elements, of a [64][128] tile
 constexpr int P64 = CH + 8;          // ... of a [64][64] tile
-constexpr int VB = 32;               // value columns per workgroup of the two scans
-constexpr int PVB = VB + 8;
-constexpr int VS = BD / VB;
 constexpr int PL = CH + 4;           // pitch of the fp32 matrix L
 
 // Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels),
@@ -258,194 +255,258 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// state scan: S_c and v_new.  The state slice [128][32] lives in registers, transposed tiles: wave w holds key rows
-// 32w .. 32w+31 as two tiles (a2), lane (c16, g) key 16(2w+a2) + c16 and value columns 16b + 4g .. +3.
+// The two scans.  A workgroup owns VBT value columns of one (sequence, v-head): the state slice [128][VBT] lives in
+// registers as transposed tiles - wave w holds key rows 32w .. 32w+31 as two tiles (a2), lane (c16, g) key
+// 16(2w+a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
+// current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
-constexpr size_t BWD_STATE_SMEM = (2 * 64 * P128 + 128 * PVB + 64 * PVB) * 2 + 64 * 4;
+template <int NCOLS>
+struct TileRegs { u32x4 x[(64 * (NCOLS / 8) + 255) / 256]; };
+template <int NCOLS, typename T>
+__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS>& r, const T* g, int64_t stride, int valid, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        r.x[i] = u32x4{0u, 0u, 0u, 0u};
+        if (idx < TOTAL && row < valid) r.x[i] = *(const u32x4*)(g + row * stride + pc * 8);
+    }
+}
+template <int NCOLS, typename T>
+__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS>& r, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = r.x[i];
+    }
+}
+template <int VBT> constexpr size_t bwd_state_smem() { return (2 * 64 * P128 + 128 * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
+template <int VBT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * P128 + 64 * P64 + 3 * 64 * (VBT + 8) + 128 * (VBT + 8)) * 2 + 64 * 4; }
 
-template <typename T>
+template <typename T, int VBT>
 __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
+    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
     extern __shared__ __align__(16) char smem[];
-    T* sW = (T*)smem; T* sK = sW + 64 * P128; T* sS = sK + 64 * P128; T* sVn = sS + 128 * PVB;
-    float* sGam = (float*)(sVn + 64 * PVB);
+    T* sW = (T*)smem; T* sK = sW + 64 * P128; T* sS = sK + 64 * P128; T* sVn = sS + 128 * PV;
+    float* sGam = (float*)(sVn + 64 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int vs = blockIdx.x % VS, hv = (blockIdx.x / VS) % p.HV, hq = hv / (p.HV / p.H);
-    const int64_t n = blockIdx.x / (VS * p.HV);
+    const int vs = blockIdx.x % NVS, hv = (blockIdx.x / NVS) % p.HV, hq = hv / (p.HV / p.H);
+    const int64_t n = blockIdx.x / (NVS * p.HV);
     const SeqAt sq = seq_at(p, n);
-    const int vcol0 = vs * VB;
+    const int vcol0 = vs * VBT;
 
-    f32x4 S[2][2];
+    f32x4 S[2][NB];
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (2 * w + a2) + c16;
             S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    for (int64_t ic = 0; ic < sq.nc; ++ic) {
+    TileRegs<BD> rW, rK;
+    V4 rU[NB];
+    float rGam = 0.f;
+    auto fetch = [&](int64_t ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        load_tile<BD>(sW, P128, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
-        load_tile<BD>(sK, P128, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
-        if (tid < 64) sGam[tid] = p.ws.Gam[u * 64 + tid];
+        fetch_tile<BD>(rW, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rK, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
+    };
+    if (sq.nc > 0) fetch(0);
+    for (int64_t ic = 0; ic < sq.nc; ++ic) {
+        const int64_t u = (sq.cbase + ic) * p.HV + hv;
+        put_tile<BD>(sW, P128, rW, tid);
+        put_tile<BD>(sK, P128, rK, tid);
+        if (tid < 64) sGam[tid] = rGam;
+        V4 u4[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) u4[b] = rU[b];
         T* Hu = (T*)p.ws.Hs + u * BD * BD;
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (2 * w + a2) + c16;
                 const V4 s4 = pack4<T>(S[a2][b]);
-                *(V4*)(sS + kk * PVB + 16 * b + 4 * g) = s4;
+                *(V4*)(sS + kk * PV + 16 * b + 4 * g) = s4;
                 *(V4*)(Hu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
             }
-        __syncthreads();
+        lds_barrier();
+        if (ic + 1 < sq.nc) fetch(ic + 1);
         const float glast = sGam[63];
         {
             // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int i = 16 * w + c16;
             const float dec = __expf(glast - sGam[i]);
             T* Vu = (T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0;
+            V8 wf[4];
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int s = 0; s < 4; ++s) wf[s] = frag_rows(sW, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
                 f32x4 acc = ZERO4;
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    acc = Mma<T>::run(frag_cols(sS, PVB, 32 * s, 16 * b, lane), frag_rows(sW, P128, 16 * w, 32 * s, lane), acc);
-                const V4 u4 = *(const V4*)(Vu + 16 * b + 4 * g);
+                for (int s = 0; s < 4; ++s) acc = Mma<T>::run(frag_cols(sS, PV, 32 * s, 16 * b, lane), wf[s], acc);
                 f32x4 vn;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[r] - acc[r];
+                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
                 const V4 vn4 = pack4<T>(vn);
                 *(V4*)(Vu + 16 * b + 4 * g) = vn4;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)vn4[r] * dec;
-                *(V4*)(sVn + i * PVB + 16 * b + 4 * g) = pack4<T>(vn);
+                *(V4*)(sVn + i * PV + 16 * b + 4 * g) = pack4<T>(vn);
             }
         }
-        __syncthreads();
+        lds_barrier();
         {
             const float eg = __expf(glast);
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < 2; ++a2) {
+                V8 kf[2];
 #pragma unroll
-                for (int b = 0; b < 2; ++b) {
+                for (int s = 0; s < 2; ++s) kf[s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
                     f32x4 acc = S[a2][b] * eg;
 #pragma unroll
-                    for (int s = 0; s < 2; ++s)
-                        acc = Mma<T>::run(frag_cols(sVn, PVB, 32 * s, 16 * b, lane),
-                                          frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
+                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(frag_cols(sVn, PV, 32 * s, 16 * b, lane), kf[s], acc);
                     S[a2][b] = acc;
                 }
+            }
         }
-        __syncthreads();
+        lds_barrier();
     }
 }
 
-// ---------------------------------------------------------------------------------------------
-// reverse scan: dS_c and dv_new; same ownership of the state slice as above
-// ---------------------------------------------------------------------------------------------
-constexpr size_t BWD_DSTATE_SMEM = (3 * 64 * P128 + 64 * P64 + 3 * 64 * PVB + 128 * PVB) * 2 + 64 * 4;
-
-template <typename T>
+template <typename T, int VBT>
 __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
+    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sW = sQ + 64 * P128; T* sPT = sW + 64 * P128;
-    T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PVB; T* sDvn = sDOg + 64 * PVB; T* sDS = sDvn + 64 * PVB;
-    float* sGam = (float*)(sDS + 128 * PVB);
+    T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
+    float* sGam = (float*)(sDS + 128 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int vs = blockIdx.x % VS, hv = (blockIdx.x / VS) % p.HV, hq = hv / (p.HV / p.H);
-    const int64_t n = blockIdx.x / (VS * p.HV);
+    const int vs = blockIdx.x % NVS, hv = (blockIdx.x / NVS) % p.HV, hq = hv / (p.HV / p.H);
+    const int64_t n = blockIdx.x / (NVS * p.HV);
     const SeqAt sq = seq_at(p, n);
-    const int vcol0 = vs * VB;
+    const int vcol0 = vs * VBT;
 
-    f32x4 dS[2][2];
+    f32x4 dS[2][NB];
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (2 * w + a2) + c16;
             dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    for (int64_t ic = sq.nc - 1; ic >= 0; --ic) {
+    TileRegs<BD> rK, rQ, rW;
+    TileRegs<CH> rPT;
+    TileRegs<VBT> rDO;
+    float rGam = 0.f;
+    auto fetch = [&](int64_t ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        load_tile<BD>(sK, P128, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
-        load_tile<BD>(sQ, P128, (const T*)p.q + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
-        load_tile<BD>(sW, P128, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
-        load_tile<CH>(sPT, P64, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
-        load_tile<VB>(sDO, PVB, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
-        if (tid < 64) sGam[tid] = p.ws.Gam[u * 64 + tid];
+        fetch_tile<BD>(rK, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        fetch_tile<BD>(rQ, (const T*)p.q + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        fetch_tile<BD>(rW, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        fetch_tile<CH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
+        fetch_tile<VBT>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
+        if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+    };
+    if (sq.nc > 0) fetch(sq.nc - 1);
+    for (int64_t ic = sq.nc - 1; ic >= 0; --ic) {
+        const int64_t u = (sq.cbase + ic) * p.HV + hv;
+        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<BD>(sQ, P128, rQ, tid);
+        put_tile<BD>(sW, P128, rW, tid);
+        put_tile<CH>(sPT, P64, rPT, tid);
+        put_tile<VBT>(sDO, PV, rDO, tid);
+        if (tid < 64) sGam[tid] = rGam;
         T* dHu = (T*)p.ws.dHs + u * BD * BD;
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (2 * w + a2) + c16;
                 const V4 s4 = pack4<T>(dS[a2][b]);
-                *(V4*)(sDS + kk * PVB + 16 * b + 4 * g) = s4;
+                *(V4*)(sDS + kk * PV + 16 * b + 4 * g) = s4;
                 *(V4*)(dHu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
             }
-        __syncthreads();
+        lds_barrier();
+        if (ic > 0) fetch(ic - 1);
         const float glast = sGam[63];
-        {
-            // scale e^gam_i do_i, for the state's gradient
-            const int row = tid >> 2, pc = tid & 3;
+        // scale e^gam_i do_i, for the state's gradient
+        for (int idx = tid; idx < 64 * (VBT / 8); idx += 256) {
+            const int row = idx / (VBT / 8), pc = idx % (VBT / 8);
             const float f = p.scale * __expf(sGam[row]);
-            V8 x = *(const V8*)(sDO + row * PVB + pc * 8);
+            V8 x = *(const V8*)(sDO + row * PV + pc * 8);
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
-            *(V8*)(sDOg + row * PVB + pc * 8) = x;
+            *(V8*)(sDOg + row * PV + pc * 8) = x;
         }
         {
             // dv_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int j = 16 * w + c16;
             const float dec = __expf(glast - sGam[j]);
             T* dVu = (T*)p.ws.dVn + u * 64 * BD + j * BD + vcol0;
+            V8 kf[4], pf[2];
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int s = 0; s < 4; ++s) kf[s] = frag_rows(sK, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) pf[s] = frag_rows(sPT, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
                 f32x4 a1 = ZERO4, a2v = ZERO4;
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     if (32 * s + 31 < 16 * w) continue;         // P^T[j][i] = 0 for i < j
-                    a1 = Mma<T>::run(frag_cols(sDO, PVB, 32 * s, 16 * b, lane), frag_rows(sPT, P64, 16 * w, 32 * s, lane), a1);
+                    a1 = Mma<T>::run(frag_cols(sDO, PV, 32 * s, 16 * b, lane), pf[s], a1);
                 }
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    a2v = Mma<T>::run(frag_cols(sDS, PVB, 32 * s, 16 * b, lane), frag_rows(sK, P128, 16 * w, 32 * s, lane), a2v);
+                for (int s = 0; s < 4; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, 16 * b, lane), kf[s], a2v);
                 f32x4 dvn = a1 + a2v * dec;
                 *(V4*)(dVu + 16 * b + 4 * g) = pack4<T>(dvn);
-                *(V4*)(sDvn + j * PVB + 16 * b + 4 * g) = pack4<T>(-dvn);
+                *(V4*)(sDvn + j * PV + 16 * b + 4 * g) = pack4<T>(-dvn);
             }
         }
-        __syncthreads();
+        lds_barrier();
         {
             const float eg = __expf(glast);
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < 2; ++a2) {
+                V8 qf[2], wf[2];
 #pragma unroll
-                for (int b = 0; b < 2; ++b) {
+                for (int s = 0; s < 2; ++s) {
+                    qf[s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    wf[s] = frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane);
+                }
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
                     f32x4 acc = dS[a2][b] * eg;
 #pragma unroll
                     for (int s = 0; s < 2; ++s) {
-                        acc = Mma<T>::run(frag_cols(sDOg, PVB, 32 * s, 16 * b, lane),
-                                          frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
-                        acc = Mma<T>::run(frag_cols(sDvn, PVB, 32 * s, 16 * b, lane),
-                                          frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane), acc);
+                        acc = Mma<T>::run(frag_cols(sDOg, PV, 32 * s, 16 * b, lane), qf[s], acc);
+                        acc = Mma<T>::run(frag_cols(sDvn, PV, 32 * s, 16 * b, lane), wf[s], acc);
                     }
                     dS[a2][b] = acc;
                 }
+            }
         }
-        __syncthreads();
+        lds_barrier();
     }
     if (p.dh0) {
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (2 * w + a2) + c16;
                 *(f32x4*)(p.dh0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
             }
@@ -767,20 +828,36 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy_kernel(BwdParams p) {
     }
 }
 
+template <typename T, int VBT>
+static void scan_kernels(const void** state, const void** dstate, size_t* smem_state, size_t* smem_dstate) {
+    *state = (const void*)gdn_bwd_state_kernel<T, VBT>; *dstate = (const void*)gdn_bwd_dstate_kernel<T, VBT>;
+    *smem_state = bwd_state_smem<VBT>(); *smem_dstate = bwd_dstate_smem<VBT>();
+}
+
 template <typename T>
 static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream) {
-    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)(p.N * p.HV * VS);
-    static SmemAttrDone done[5];
+    // Value columns per workgroup of the scans: as few as it takes to give every (sequence, head) run its own CU
+    // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.
+    const int64_t runs1 = p.N * p.HV;
+    const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
+    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)(runs1 * (BD / vbt));
+    static SmemAttrDone done[3][5];
+    const void *state, *dstate;
+    size_t smem_state, smem_dstate;
+    if (vbt == 32) scan_kernels<T, 32>(&state, &dstate, &smem_state, &smem_dstate);
+    else if (vbt == 64) scan_kernels<T, 64>(&state, &dstate, &smem_state, &smem_dstate);
+    else scan_kernels<T, 128>(&state, &dstate, &smem_state, &smem_dstate);
     struct K { const void* f; size_t smem; const char* name; unsigned grid; };
     const K ks[5] = {
         {(const void*)gdn_bwd_prepare_kernel<T>, BWD_PREP_SMEM, "gdn_bwd_prepare_kernel", units},
-        {(const void*)gdn_bwd_state_kernel<T>, BWD_STATE_SMEM, "gdn_bwd_state_kernel", runs},
-        {(const void*)gdn_bwd_dstate_kernel<T>, BWD_DSTATE_SMEM, "gdn_bwd_dstate_kernel", runs},
+        {state, smem_state, "gdn_bwd_state_kernel", runs},
+        {dstate, smem_dstate, "gdn_bwd_dstate_kernel", runs},
         {(const void*)gdn_bwd_dqkw_kernel<T>, BWD_DQKW_SMEM, "gdn_bwd_dqkw_kernel", units},
         {(const void*)gdn_bwd_wy_kernel<T>, BWD_WY_SMEM, "gdn_bwd_wy_kernel", units},
     };
+    const int vi = vbt == 32 ? 0 : vbt == 64 ? 1 : 2;
     for (int i = 0; i < 5; ++i) {
-        if (int rc = ensure_dynamic_smem(ks[i].f, ks[i].smem, done[i], ks[i].name)) return rc;
+        if (int rc = ensure_dynamic_smem(ks[i].f, ks[i].smem, done[vi][i], ks[i].name)) return rc;
         void* args[] = {(void*)&p};
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
@@ -813,7 +890,7 @@ extern "C" int gdn_chunk_bwd(
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
     GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
                   "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
-    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * VS < (1ll << 31), GDN_ERR_UNSUPPORTED,
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
                   "%s: too many heads or chunks for one launch", who);
     if (cu_seqlens) {
         GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);

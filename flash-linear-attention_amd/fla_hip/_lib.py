@@ -97,6 +97,8 @@ SIGNATURES['gdn_chunk_bwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_l2norm_fwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p])
+SIGNATURES['gdn_l2norm_bwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p])
 SIGNATURES['gdn_calib_rmw'] = (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p])
 CHUNK_STATIC_WORKSPACE_BYTES = 64 << 20
 

@@ -36,10 +36,14 @@ def chunk_gated_delta_rule_bwd(
     cu_seqlens_cpu: torch.Tensor | None = None,
     chunk_indices: torch.Tensor | None = None,
     chunk_size: int = 64,
+    q_rstd: torch.Tensor | None = None,
+    k_rstd: torch.Tensor | None = None,
 ):
     """q, k ``[B,T,H,K]``, v, do ``[B,T,HV,V]``, g (log decay), beta ``[B,T,HV]`` as the recurrence uses them.
     Returns ``(dq, dk, dv, dbeta, dg, dh0)``: dq, dk, dv in q's dtype, dbeta, dg fp32, dh0 fp32 (None without
-    ``initial_state``)."""
+    ``initial_state``).  With ``q_rstd``, ``k_rstd`` (the factors ``l2norm_fwd`` returns next to the normalised rows
+    passed as q and k) dq and dk are the gradients of the rows before normalisation: the reference's ``l2norm_bwd``
+    (chunk.py:385-387) happens in the kernel that also adds up the value heads of a q/k head."""
     dev = require_gpu(q, k, v, beta, do)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
@@ -63,7 +67,7 @@ def chunk_gated_delta_rule_bwd(
         h2, d2 = split(initial_state), split(dht)
         dq, dk, dv2, db2, dg2, dh2 = chunk_gated_delta_rule_bwd(
             q, k, v2, g2, beta.repeat_interleave(nb, dim=2), scale, h2, do2, d2, state_v_first,
-            cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size)
+            cu_seqlens, cu_seqlens_cpu, chunk_indices, chunk_size, q_rstd, k_rstd)
         # (dq, dk come back per q/k head: already summed over the value heads)
         dv = dv2.reshape(B, T, HV, nb * _DIM)[..., :V]
         db, dg = db2.reshape(B, T, HV, nb).sum(-1), dg2.reshape(B, T, HV, nb).sum(-1)
@@ -124,28 +128,45 @@ def chunk_gated_delta_rule_bwd(
         ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
         B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
         current_stream_ptr(dev)))
-    if HV != H:
-        # grouped value heads: a q/k head collects the gradients of its HV/H value heads
-        dq = dq.view(B, T, H, HV // H, _DIM).float().sum(3)
-        dk = dk.view(B, T, H, HV // H, _DIM).float().sum(3)
-    dq, dk, dv = dq[..., :K].to(out_dtype), dk[..., :K].to(out_dtype), dv[..., :V].to(out_dtype)
+    dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
+    dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
+    dv = dv[..., :V].to(out_dtype)
     if dh0 is not None:
         dh0 = dh0[..., :K, :V]
         dh0 = (dh0.transpose(-1, -2) if state_v_first else dh0).contiguous()
     return dq, dk, dv, db, dg, dh0
 
 
-def _l2norm(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """rows divided by sqrt(sum x^2 + 1e-6), in x's dtype, and the factors (fla/modules/l2norm.py:84-109)"""
-    xf = x.float()
-    rstd = torch.rsqrt(xf.square().sum(-1, keepdim=True) + 1e-6)
-    return (xf * rstd).to(x.dtype), rstd
+def _finish(lib, dxh: torch.Tensor, y: torch.Tensor, rstd: torch.Tensor | None, H: int, K: int, out_dtype) -> torch.Tensor:
+    """dq or dk per value head ``[B,T,HV,128]`` -> per q/k head ``[B,T,H,K]``: the sum over the value heads of a
+    q/k head and, with ``rstd``, the way back through the l2 normalisation (``y``: the normalised rows, 128 wide)."""
+    B, T, HV, D = dxh.shape
+    if rstd is None and HV == H and K == D:
+        return dxh.to(out_dtype)
+    dx = torch.empty(B, T, H, K, dtype=dxh.dtype, device=dxh.device)
+    if K % 8:                                       # (rows of the kernel are multiples of 8 elements)
+        KP = (K + 7) // 8 * 8
+        dx = torch.empty(B, T, H, KP, dtype=dxh.dtype, device=dxh.device)
+    _lib.check(lib.gdn_l2norm_bwd(ptr(dxh), ptr(y) if rstd is not None else None, ptr(rstd), ptr(dx), B * T * H, HV // H, D,
+                                  dx.shape[-1], dtype_code(dxh.dtype), current_stream_ptr(dxh.device)))
+    return dx[..., :K].to(out_dtype)
 
 
-def _l2norm_bwd(y: torch.Tensor, rstd: torch.Tensor, dy: torch.Tensor) -> torch.Tensor:
-    """(fla/modules/l2norm.py:112-146)  dx = (dy - y <dy, y>) * rstd"""
-    yf, dyf = y.float(), dy.float()
-    return (dyf - yf * (dyf * yf).sum(-1, keepdim=True)) * rstd
+def l2norm_fwd(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Rows divided by sqrt(sum x^2 + 1e-6), in x's dtype (fp32 input: bf16), and the factors ``[..., 1]`` fp32
+    (fla/modules/l2norm.py:222-262).  Rows whose length is not a multiple of 8 come back zero-padded to one."""
+    require_gpu(x)
+    work = x.dtype if x.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    if x.shape[-1] > 256:
+        raise NotImplementedError('l2norm_fwd: rows of up to 256 elements')
+    x = _pad_last(x, (x.shape[-1] + 7) // 8 * 8)
+    D = x.shape[-1]
+    xw = aligned16(x.to(work).contiguous())
+    y = torch.empty_like(xw)
+    rstd = torch.empty(*x.shape[:-1], 1, dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().gdn_l2norm_fwd(ptr(xw), ptr(y), ptr(rstd), xw.numel() // D, D, D, dtype_code(work),
+                                          current_stream_ptr(x.device)))
+    return y, rstd
 
 
 class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
@@ -170,9 +191,10 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         q, k, v, g, beta_raw, h0, cu_seqlens, cu_seqlens_cpu, chunk_indices, A_log, dt_bias = ctx.saved_tensors
         scale, state_v_first, l2, gate, bsig, neg, chunk_size = ctx.opts
         q_rstd = k_rstd = None
+        K = q.shape[-1]
         if l2:
-            q, q_rstd = _l2norm(q)
-            k, k_rstd = _l2norm(k)
+            q, q_rstd = l2norm_fwd(q)
+            k, k_rstd = l2norm_fwd(k)
         beta = beta_raw
         if bsig:
             beta = torch.sigmoid(beta_raw.float()) * (2.0 if neg else 1.0)
@@ -183,10 +205,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             g = -A_log.float().exp() * F.softplus(x)
         dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(
             q, k, v, g, beta, scale, h0, do.contiguous(), dht, state_v_first, cu_seqlens, cu_seqlens_cpu,
-            chunk_indices, chunk_size)
-        if l2:
-            dq = _l2norm_bwd(q, q_rstd, dq)
-            dk = _l2norm_bwd(k, k_rstd, dk)
+            chunk_indices, chunk_size, q_rstd, k_rstd)
         if bsig:
             s = torch.sigmoid(beta_raw.float())
             db = db * s * (1 - s) * (2.0 if neg else 1.0)
@@ -201,5 +220,5 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             dg = dg.to(g_in.dtype)
         else:
             dg = None
-        return (dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), dg, db.to(beta_raw.dtype), None, dh0, None, None, None,
+        return (dq[..., :K].to(q.dtype), dk[..., :K].to(k.dtype), dv.to(v.dtype), dg, db.to(beta_raw.dtype), None, dh0, None, None, None,
                 None, None, None, None, dA_log, ddt_bias, None, None, None)

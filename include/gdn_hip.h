@@ -235,6 +235,18 @@ int gdn_chunk_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Row-wise l2 normalisation around gdn_chunk_bwd.  gdn_l2norm_fwd replaces l2norm_fwd (fla/modules/l2norm.py:222-262):
+ * y[row] = x[row] / sqrt(sum x^2 + 1e-6) in x's dtype (bf16 or f16), rstd[row] = that factor; rows of D elements in,
+ * rows of Dout >= D elements out (zeros from D on: the backward kernels want 128).  gdn_l2norm_bwd replaces l2norm_bwd
+ * (fla/modules/l2norm.py:265-300) and the sum over grouped heads in front of it (chunk_gated_delta_rule_bwd returns dq, dk
+ * per value head): dx[row] = (dy - y <dy, y>) rstd[row] with dy = sum over g < G of dyh[row][g]; rows of Din elements in
+ * (dyh, y), the first Dout <= Din of them out; y == rstd == NULL: the sum alone.  Row lengths: multiples of 8 up to 256.
+ */
+int gdn_l2norm_fwd(const void* x, void* y, float* rstd, int64_t rows, int64_t D, int64_t Dout, int dtype, void* stream);
+int gdn_l2norm_bwd(const void* dyh, const void* y, const float* rstd, void* dx, int64_t rows, int64_t G, int64_t Din,
+                   int64_t Dout, int dtype, void* stream);
+
+/*
  * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * gdn_chunk_fwd minus the workspace: the kernels use a fixed array of GDN_CHUNK_STATIC_WORKSPACE_BYTES that the
