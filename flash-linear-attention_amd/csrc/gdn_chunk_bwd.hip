@@ -104,6 +104,28 @@ __device__ __forceinline__ void load_tile(T* s, int pitch, const T* g, int64_t s
     }
 }
 
+// The same in two halves, for loops that fetch the next tile while they work on the current one.
+template <int NCOLS>
+struct TileRegs { u32x4 x[(64 * (NCOLS / 8) + 255) / 256]; };
+template <int NCOLS, typename T>
+__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS>& r, const T* g, int64_t stride, int valid, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        r.x[i] = u32x4{0u, 0u, 0u, 0u};
+        if (idx < TOTAL && row < valid) r.x[i] = *(const u32x4*)(g + row * stride + pc * 8);
+    }
+}
+template <int NCOLS, typename T>
+__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS>& r, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
+        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = r.x[i];
+    }
+}
 // operand fragment whose contraction runs along a row: index r0 + c16, contraction c0 + 8g + e
 template <typename T>
 __device__ __forceinline__ typename Mma<T>::V8 frag_rows(const T* s, int pitch, int r0, int c0, int lane) {
@@ -128,6 +150,11 @@ __device__ __forceinline__ float sum_over_c16(float x) {        // over the sixt
     x += __shfl_xor(x, 1, 64); x += __shfl_xor(x, 2, 64); x += __shfl_xor(x, 4, 64);
     return x + __shfl_xor(x, 8, 64);
 }
+// x summed over the four lanes of a quad (lanes 4n .. 4n+3), in every one of them
+__device__ __forceinline__ float sum_over_quad(float x) {
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // [2,3,0,1]
+}
 #define ZERO4 (f32x4{0.f, 0.f, 0.f, 0.f})
 
 // ---------------------------------------------------------------------------------------------
@@ -136,85 +163,77 @@ __device__ __forceinline__ float sum_over_c16(float x) {        // over the sixt
 constexpr size_t BWD_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PL + 128) * 4;
 
 template <typename T>
-__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
     float* sL = (float*)(sA + 64 * P64); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t u = blockIdx.x, ci = u / p.HV;
-    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-    const ChunkAt c = chunk_at(p, ci);
 
-    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    load_tile<BD>(sV, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-    if (w == 0) {
-        float x = 0.f, b = 0.f;
-        if (lane < c.valid) {
-            x = p.g ? load_scalar(p.g, (c.tok0 + lane) * p.HV + hv, p.gb_dtype) : 0.f;
-            b = load_scalar(p.beta, (c.tok0 + lane) * p.HV + hv, p.gb_dtype);
+    // Units in turn; the next unit's rows are fetched into registers while this one is worked on.
+    TileRegs<BD> rK, rQ, rV;
+    float rG = 0.f, rB = 0.f;
+    auto fetch = [&](int64_t u) {
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        rG = rB = 0.f;
+        if (w == 0 && lane < c.valid) {
+            rG = p.g ? load_scalar(p.g, (c.tok0 + lane) * p.HV + hv, p.gb_dtype) : 0.f;
+            rB = load_scalar(p.beta, (c.tok0 + lane) * p.HV + hv, p.gb_dtype);
         }
+    };
+    fetch(blockIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<BD>(sQ, P128, rQ, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        if (w == 0) {
+            float x = rG;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const float y = __shfl_up(x, off, 64);
-            if (lane >= off) x += y;
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_up(x, off, 64);
+                if (lane >= off) x += y;
+            }
+            sGam[lane] = x; sBeta[lane] = rB;
+            p.ws.Gam[u * 64 + lane] = x;
         }
-        sGam[lane] = x; sBeta[lane] = b;
-        p.ws.Gam[u * 64 + lane] = x;
-    }
-    __syncthreads();
+        lds_barrier();
+        if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-    // strip of 16 token rows per wave: L (fp32, for the substitution) and P^T
-    {
-        T* PTu = (T*)p.ws.PT + u * 64 * 64;
+        // strip of 16 token rows per wave: L (fp32, for the substitution; entry (i, j) at [i][j % 4][j / 4]) and P^T
+        {
+            T* PTu = (T*)p.ws.PT + u * 64 * 64;
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            f32x4 kk = ZERO4, qk = ZERO4;
-            if (tj <= w) {
+            for (int tj = 0; tj < 4; ++tj) {
+                f32x4 kk = ZERO4, qk = ZERO4;
+                if (tj <= w) {
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const V8 b = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
-                    kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), b, kk);
-                    qk = Mma<T>::run(frag_rows(sQ, P128, 16 * w, 32 * s, lane), b, qk);
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 b = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+                        kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), b, kk);
+                        qk = Mma<T>::run(frag_rows(sQ, P128, 16 * w, 32 * s, lane), b, qk);
+                    }
                 }
-            }
-            const int j = 16 * tj + c16;
-            const float gj = sGam[j];
-            f32x4 pt;
+                const int j = 16 * tj + c16;
+                const float gj = sGam[j];
+                f32x4 pt;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int i = 16 * w + 4 * g + r;
-                const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
-                if (tj <= w) sL[i * PL + j] = i > j ? sBeta[i] * kk[r] * d : 0.f;
-                pt[r] = p.scale * qk[r] * d;
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
+                    if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = i > j ? sBeta[i] * kk[r] * d : 0.f;
+                    pt[r] = p.scale * qk[r] * d;
+                }
+                *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
             }
-            *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
         }
-    }
-    __syncthreads();
-
-    // A = (I + L)^-1 by forward substitution: lane c owns column c, A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c]
-    if (w == 0) {
-        float a[64];
-#pragma unroll
-        for (int i = 0; i < 64; ++i) {
-            float acc[4] = {i == lane ? 1.f : 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int j4 = 0; 4 * j4 < i; ++j4) {
-                const f32x4 l = *(const f32x4*)(sL + i * PL + 4 * j4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (4 * j4 + e < i) acc[e] -= l[e] * a[4 * j4 + e];
-            }
-            a[i] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-            sA[i * P64 + lane] = (T)a[i];
-        }
-    }
-    // meanwhile the other waves turn k into beta e^gam k and v into beta v, in place
-    else {
-        for (int idx = tid - 64; idx < 64 * 16; idx += 192) {
+        lds_barrier();
+        // k -> beta e^gam k and v -> beta v, in place
+        for (int idx = tid; idx < 64 * 16; idx += 256) {
             const int row = idx >> 4, pc = idx & 15;
             const float bk = sBeta[row] * __expf(sGam[row]), bv = sBeta[row];
             V8 x = *(V8*)(sK + row * P128 + pc * 8), y = *(V8*)(sV + row * P128 + pc * 8);
@@ -223,34 +242,60 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p) {
             *(V8*)(sK + row * P128 + pc * 8) = x;
             *(V8*)(sV + row * P128 + pc * 8) = y;
         }
-    }
-    __syncthreads();
-    {
-        T* Au = (T*)p.ws.Am + u * 64 * 64;
+        // A = (I + L)^-1 by forward substitution, A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c]: a quad of lanes per
+        // column c (16 columns per wave), lane gq of the quad keeps A[j][c] for j = gq mod 4 and adds up their part of the sum
+        {
+            const int c = 16 * w + (lane >> 2), gq = lane & 3;
+            float a[16];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
-            *(u32x4*)(Au + row * 64 + pc * 8) = *(const u32x4*)(sA + row * P64 + pc * 8);
-        }
-    }
-    // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
-    {
-        T* Wu = (T*)p.ws.Wm + u * 64 * BD;
-        T* Uu = (T*)p.ws.Vn + u * 64 * BD;
-        const int i = 16 * w + c16;
+            for (int m = 0; m < 16; ++m) a[m] = 0.f;
 #pragma unroll
-        for (int n = 0; n < 8; ++n) {
-            f32x4 aw = ZERO4, au = ZERO4;
+            for (int i = 0; i < 64; ++i) {
+                float part0 = 0.f, part1 = 0.f;
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (2 * s > w) continue;                        // A is lower triangular
-                const V8 b = frag_rows(sA, P64, 16 * w, 32 * s, lane);
-                aw = Mma<T>::run(frag_cols(sK, P128, 32 * s, 16 * n, lane), b, aw);
-                au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), b, au);
+                for (int m4 = 0; 16 * m4 < i; ++m4) {           // entries j = 4m + gq < i; those from i on are stored as zeros
+                    const f32x4 l = *(const f32x4*)(sL + i * PL + gq * 16 + 4 * m4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (4 * (4 * m4 + e) < i) {
+                            if (e & 1) part1 += l[e] * a[4 * m4 + e];
+                            else part0 += l[e] * a[4 * m4 + e];
+                        }
+                    }
+                }
+                const float ai = (i == c ? 1.f : 0.f) - sum_over_quad(part0 + part1);
+                if (gq == (i & 3)) { a[i >> 2] = ai; sA[i * P64 + c] = (T)ai; }
             }
-            *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
-            *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
         }
+        lds_barrier();
+        {
+            T* Au = (T*)p.ws.Am + u * 64 * 64;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+                *(u32x4*)(Au + row * 64 + pc * 8) = *(const u32x4*)(sA + row * P64 + pc * 8);
+            }
+        }
+        // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
+        {
+            T* Wu = (T*)p.ws.Wm + u * 64 * BD;
+            T* Uu = (T*)p.ws.Vn + u * 64 * BD;
+            const int i = 16 * w + c16;
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                f32x4 aw = ZERO4, au = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (2 * s > w) continue;                    // A is lower triangular
+                    const V8 b = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+                    aw = Mma<T>::run(frag_cols(sK, P128, 32 * s, 16 * n, lane), b, aw);
+                    au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), b, au);
+                }
+                *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
+                *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
+            }
+        }
+        lds_barrier();
     }
 }
 
@@ -260,27 +305,6 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p) {
 // 16(2w+a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
 // current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
-template <int NCOLS>
-struct TileRegs { u32x4 x[(64 * (NCOLS / 8) + 255) / 256]; };
-template <int NCOLS, typename T>
-__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS>& r, const T* g, int64_t stride, int valid, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        r.x[i] = u32x4{0u, 0u, 0u, 0u};
-        if (idx < TOTAL && row < valid) r.x[i] = *(const u32x4*)(g + row * stride + pc * 8);
-    }
-}
-template <int NCOLS, typename T>
-__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS>& r, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = r.x[i];
-    }
-}
 template <int VBT> constexpr size_t bwd_state_smem() { return (2 * 64 * P128 + 128 * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
 template <int VBT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * P128 + 64 * P64 + 3 * 64 * (VBT + 8) + 128 * (VBT + 8)) * 2 + 64 * 4; }
 
@@ -517,314 +541,340 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
 // dq, dw and the first parts of dk and dgam.  Wave w owns key features 32w .. 32w+31 (two tiles a2) of all 64 tokens
 // (four tiles t): lane (c16, g) holds token 16t + c16 and features 16(2w+a2) + 4g .. +3.
 // ---------------------------------------------------------------------------------------------
-constexpr size_t BWD_DQKW_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + 128 * 4;
+// One workgroup per CU walks over the units and fetches everything the next unit needs (five tiles and its fragments
+// of S and dS) into registers while it works on the current one.
+constexpr size_t BWD_DQKW_SMEM = (5 * 64 * P128 + 64 * P64) * 2 + 128 * 4;
 
 template <typename T>
-__global__ __launch_bounds__(256, 2) void gdn_bwd_dqkw_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
-    T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sDP = sDvn + 64 * P128;
+    T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sK = sDvn + 64 * P128; T* sQ = sK + 64 * P128;
+    T* sDP = sQ + 64 * P128;
     float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;
-    T* sK = sVn; T* sQ = sDvn;                                   // second phase
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t u = blockIdx.x, ci = u / p.HV;
-    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-    const ChunkAt c = chunk_at(p, ci);
 
-    load_tile<BD>(sDO, P128, (const T*)p.dout + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-    load_tile<BD>(sVn, P128, (const T*)p.ws.Vn + u * 64 * BD, BD, 64, tid);
-    load_tile<BD>(sDvn, P128, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
-    if (tid < 64) { sGam[tid] = p.ws.Gam[u * 64 + tid]; sDg[tid] = 0.f; }
-    __syncthreads();
-
-    f32x4 G1[2][4], dWt[2][4], dKS[2][4];
-    float sdot = 0.f;
-    {
+    TileRegs<BD> rDO, rVn, rDvn, rK, rQ;
+    V8 rS[2][4], rdS[2][4];
+    float rGam = 0.f;
+    auto fetch = [&](int64_t u) {
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rDO, (const T*)p.dout + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        fetch_tile<BD>(rVn, (const T*)p.ws.Vn + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
         const T* Hu = (const T*)p.ws.Hs + u * BD * BD;
         const T* dHu = (const T*)p.ws.dHs + u * BD * BD;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[a2][t] = dKS[a2][t] = ZERO4;
-            const int kk = 16 * (2 * w + a2) + c16;
+        for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                const V8 sf = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
-                const V8 df = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sdot += (float)sf[e] * (float)df[e];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    G1[a2][t] = Mma<T>::run(sf, frag_rows(sDO, P128, 16 * t, 32 * s, lane), G1[a2][t]);
-                    dWt[a2][t] = Mma<T>::run(sf, frag_rows(sDvn, P128, 16 * t, 32 * s, lane), dWt[a2][t]);
-                    dKS[a2][t] = Mma<T>::run(df, frag_rows(sVn, P128, 16 * t, 32 * s, lane), dKS[a2][t]);
-                }
+                const int kk = 16 * (2 * w + a2) + c16;
+                rS[a2][s] = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
+                rdS[a2][s] = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
             }
-        }
-    }
-    // dP o D for this wave's 16 token rows, as an operand tile
-#pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-        f32x4 acc = ZERO4;
-        if (tj <= w) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                acc = Mma<T>::run(frag_rows(sDO, P128, 16 * w, 32 * s, lane), frag_rows(sVn, P128, 16 * tj, 32 * s, lane), acc);
-        }
-        const int j = 16 * tj + c16;
-        const float gj = sGam[j];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int i = 16 * w + 4 * g + r;
-            sDP[i * P64 + j] = (T)(i >= j ? p.scale * acc[r] * __expf(sGam[i] - gj) : 0.f);
-        }
-    }
-    {
-        T* dWu = (T*)p.ws.dWm + u * 64 * BD;
+        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+    };
+    fetch(blockIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        put_tile<BD>(sDO, P128, rDO, tid);
+        put_tile<BD>(sVn, P128, rVn, tid);
+        put_tile<BD>(sDvn, P128, rDvn, tid);
+        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<BD>(sQ, P128, rQ, tid);
+        if (tid < 64) { sGam[tid] = rGam; sDg[tid] = 0.f; }
+        V8 sf[2][4], df[2][4];
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[a2][t]);
-    }
-    __syncthreads();
-    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    __syncthreads();
+            for (int s = 0; s < 4; ++s) { sf[a2][s] = rS[a2][s]; df[a2][s] = rdS[a2][s]; }
+        lds_barrier();
+        if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-    const float glast = sGam[63];
-    float dglast = __expf(glast) * sdot;
+        f32x4 G1[2][4], dKS[2][4];
+        float sdot = 0.f;
+        {
+            T* dWu = (T*)p.ws.dWm + u * 64 * BD;
 #pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2) {
-        const int n16 = 16 * (2 * w + a2);
+            for (int a2 = 0; a2 < 2; ++a2) {
+                f32x4 dWt[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int x = 16 * t + c16;
-            const float gx = sGam[x];
-            f32x4 dq = G1[a2][t] * (p.scale * __expf(gx));
-            f32x4 dk = dKS[a2][t] * __expf(glast - gx);
-            const V4 q4 = *(const V4*)(sQ + x * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+                for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[t] = dKS[a2][t] = ZERO4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dglast += (float)k4[r] * dk[r];
+                for (int s = 0; s < 4; ++s) {
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (32 * s <= 16 * t + 15)                      // dP[i][j] = 0 for j > i
-                    dq = Mma<T>::run(frag_cols(sK, P128, 32 * s, n16, lane), frag_rows(sDP, P64, 16 * t, 32 * s, lane), dq);
-                if (32 * s + 31 >= 16 * t)                      // ... and for i < j
-                    dk = Mma<T>::run(frag_cols(sQ, P128, 32 * s, n16, lane), frag_cols(sDP, P64, 32 * s, 16 * t, lane), dk);
-            }
-            float dgx = 0.f;
+                    for (int e = 0; e < 8; ++e) sdot += (float)sf[a2][s][e] * (float)df[a2][s][e];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dgx += (float)q4[r] * dq[r] - (float)k4[r] * dk[r];
-            dgx = sum_over_g(dgx);
-            if (g == 0) atomicAdd(&sDg[x], dgx);
-            if (x < c.valid) {
-                *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq);
-                *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk);
+                    for (int t = 0; t < 4; ++t) {
+                        G1[a2][t] = Mma<T>::run(sf[a2][s], frag_rows(sDO, P128, 16 * t, 32 * s, lane), G1[a2][t]);
+                        dWt[t] = Mma<T>::run(sf[a2][s], frag_rows(sDvn, P128, 16 * t, 32 * s, lane), dWt[t]);
+                        dKS[a2][t] = Mma<T>::run(df[a2][s], frag_rows(sVn, P128, 16 * t, 32 * s, lane), dKS[a2][t]);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[t]);
             }
         }
+        // dP o D for this wave's 16 token rows, as an operand tile
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            f32x4 acc = ZERO4;
+            if (tj <= w) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+                    acc = Mma<T>::run(frag_rows(sDO, P128, 16 * w, 32 * s, lane), frag_rows(sVn, P128, 16 * tj, 32 * s, lane), acc);
+            }
+            const int j = 16 * tj + c16;
+            const float gj = sGam[j];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * w + 4 * g + r;
+                sDP[i * P64 + j] = (T)(i >= j ? p.scale * acc[r] * __expf(sGam[i] - gj) : 0.f);
+            }
+        }
+        lds_barrier();
+
+        const float glast = sGam[63];
+        float dglast = __expf(glast) * sdot;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+            const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                const float gx = sGam[x];
+                f32x4 dq = G1[a2][t] * (p.scale * __expf(gx));
+                f32x4 dk = dKS[a2][t] * __expf(glast - gx);
+                const V4 q4 = *(const V4*)(sQ + x * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dglast += (float)k4[r] * dk[r];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s <= 16 * t + 15)                  // dP[i][j] = 0 for j > i
+                        dq = Mma<T>::run(frag_cols(sK, P128, 32 * s, n16, lane), frag_rows(sDP, P64, 16 * t, 32 * s, lane), dq);
+                    if (32 * s + 31 >= 16 * t)                  // ... and for i < j
+                        dk = Mma<T>::run(frag_cols(sQ, P128, 32 * s, n16, lane), frag_cols(sDP, P64, 32 * s, 16 * t, lane), dk);
+                }
+                float dgx = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dgx += (float)q4[r] * dq[r] - (float)k4[r] * dk[r];
+                dgx = sum_over_g(dgx);
+                if (g == 0) atomicAdd(&sDg[x], dgx);
+                if (x < c.valid) {
+                    *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq);
+                    *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk);
+                }
+            }
+        }
+        dglast = sum_over_c16(sum_over_g(dglast));
+        if (lane == 0) atomicAdd(&sDg[63], dglast);
+        lds_barrier();
+        if (tid < 64) p.ws.Dgam[u * 64 + tid] = sDg[tid];
+        lds_barrier();
     }
-    dglast = sum_over_c16(sum_over_g(dglast));
-    if (lane == 0) atomicAdd(&sDg[63], dglast);
-    __syncthreads();
-    if (tid < 64) p.ws.Dgam[u * 64 + tid] = sDg[tid];
 }
 
 // ---------------------------------------------------------------------------------------------
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
-constexpr size_t BWD_WY_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 256 * 4;
+// One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.
+constexpr size_t BWD_WY_SMEM = (4 * 64 * P128 + 3 * 64 * P64) * 2 + 256 * 4;
 
 template <typename T>
-__global__ __launch_bounds__(256, 2) void gdn_bwd_wy_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
-    T* X0 = (T*)smem; T* X1 = X0 + 64 * P128; T* sA = X1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
+    T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * P128;
+    T* sA = sK + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
     float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t u = blockIdx.x, ci = u / p.HV;
-    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-    const ChunkAt c = chunk_at(p, ci);
 
-    load_tile<BD>(X0, P128, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
-    load_tile<BD>(X1, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-    load_tile<CH>(sA, P64, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
-    if (tid < 64) {
-        sGam[tid] = p.ws.Gam[u * 64 + tid];
-        sBeta[tid] = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
-        sDg[tid] = p.ws.Dgam[u * 64 + tid];
-        sDb[tid] = 0.f;
-    }
-    __syncthreads();
-
-    // dX = du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), dv = beta (A^T du)
-    f32x4 dX[4];
-#pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-        dX[tj] = ZERO4;
-        if (tj <= w) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                dX[tj] = Mma<T>::run(frag_rows(X0, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tj, 32 * s, lane), dX[tj]);
+    TileRegs<BD> rDvn, rV, rDW, rK;
+    TileRegs<CH> rA;
+    V4 rDk[2][4];                                               // what the previous kernel left in dk, at this lane's places
+    float rGam = 0.f, rBeta = 0.f, rDg = 0.f;
+    auto fetch = [&](int64_t u) {
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
+        fetch_tile<BD>(rDW, (const T*)p.ws.dWm + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        if (tid < 64) {
+            rGam = p.ws.Gam[u * 64 + tid];
+            rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+            rDg = p.ws.Dgam[u * 64 + tid];
         }
-    }
 #pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2) {
-        const int n16 = 16 * (2 * w + a2);
+        for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            f32x4 acc = ZERO4;
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (32 * s + 31 < 16 * t) continue;             // A[i][j] = 0 for i < j
-                acc = Mma<T>::run(frag_cols(X0, P128, 32 * s, n16, lane), frag_cols(sA, P64, 32 * s, 16 * t, lane), acc);
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                rDk[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+                if (x < c.valid) rDk[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + 16 * (2 * w + a2) + 4 * g);
             }
-            const int j = 16 * t + c16;
-            const V4 v4 = *(const V4*)(X1 + j * P128 + n16 + 4 * g);
-            float db = 0.f;
+    };
+    fetch(blockIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        put_tile<BD>(sDvn, P128, rDvn, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        put_tile<CH>(sA, P64, rA, tid);
+        put_tile<BD>(sDW, P128, rDW, tid);
+        put_tile<BD>(sK, P128, rK, tid);
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; sDg[tid] = rDg; sDb[tid] = 0.f; }
+        V4 dk_old[2][4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) db += acc[r] * (float)v4[r];
-            db = sum_over_g(db);
-            if (g == 0) atomicAdd(&sDb[j], db);
-            if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(acc * sBeta[j]);
-        }
-    }
-    __syncthreads();
-    load_tile<BD>(X0, P128, (const T*)p.ws.dWm + u * 64 * BD, BD, 64, tid);
-    load_tile<BD>(X1, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    __syncthreads();
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) dk_old[a2][t] = rDk[a2][t];
+        lds_barrier();
+        if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-    // dX += dw (e^gam k)^T;  dA = stril(dX diag(beta)) as an operand tile
+        // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta))
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-        f32x4 acc = ZERO4;
-        if (tj <= w) {
+        for (int tj = 0; tj < 4; ++tj) {
+            f32x4 dXv = ZERO4, dXw = ZERO4;
+            if (tj <= w) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
-                acc = Mma<T>::run(frag_rows(X0, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tj, 32 * s, lane), acc);
-        }
-        const int j = 16 * tj + c16;
-        const float ej = __expf(sGam[j]), bj = sBeta[j];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int i = 16 * w + 4 * g + r;
-            sM1[i * P64 + j] = (T)(i > j ? (dX[tj][r] + ej * acc[r]) * bj : 0.f);
-        }
-    }
-    // d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
-    f32x4 dk[2][4];
-#pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2) {
-        const int n16 = 16 * (2 * w + a2);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            f32x4 acc = ZERO4;
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (32 * s + 31 < 16 * t) continue;
-                acc = Mma<T>::run(frag_cols(X0, P128, 32 * s, n16, lane), frag_cols(sA, P64, 32 * s, 16 * t, lane), acc);
+                for (int s = 0; s < 4; ++s) {
+                    dXv = Mma<T>::run(frag_rows(sDvn, P128, 16 * w, 32 * s, lane), frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
+                    dXw = Mma<T>::run(frag_rows(sDW, P128, 16 * w, 32 * s, lane), frag_rows(sK, P128, 16 * tj, 32 * s, lane), dXw);
+                }
             }
-            const int j = 16 * t + c16;
-            const V4 k4 = *(const V4*)(X1 + j * P128 + n16 + 4 * g);
-            float dot = 0.f;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) dot += acc[r] * (float)k4[r];
-            dot = sum_over_g(dot);
+            const int j = 16 * tj + c16;
             const float ej = __expf(sGam[j]), bj = sBeta[j];
-            if (g == 0) { atomicAdd(&sDb[j], ej * dot); atomicAdd(&sDg[j], bj * ej * dot); }
-            dk[a2][t] = acc * (bj * ej);
-        }
-    }
-    __syncthreads();
-    // Y = dA A^T
-#pragma unroll
-    for (int tl = 0; tl < 4; ++tl) {
-        f32x4 acc = ZERO4;
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-            acc = Mma<T>::run(frag_rows(sM1, P64, 16 * w, 32 * s, lane), frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
-        const int l = 16 * tl + c16;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
-    }
-    __syncthreads();
-    // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
-    {
-        float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int tl = 0; tl < 4; ++tl) {
-            f32x4 acc = ZERO4, kk = ZERO4;
-            if (tl <= w) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    acc = Mma<T>::run(frag_cols(sA, P64, 32 * s, 16 * w, lane), frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
-#pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    kk = Mma<T>::run(frag_rows(X1, P128, 16 * w, 32 * s, lane), frag_rows(X1, P128, 16 * tl, 32 * s, lane), kk);
-            }
-            const int l = 16 * tl + c16;
-            const float gl = sGam[l];
-            float colF = 0.f;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 16 * w + 4 * g + r;
-                float E = 0.f;
-                if (i > l) {
-                    const float d = __expf(sGam[i] - gl), dL = -acc[r];
-                    dbi[r] += dL * kk[r] * d;
-                    E = dL * sBeta[i] * d;
-                    const float F = E * kk[r];
-                    rowF[r] += F;
-                    colF += F;
+                sM1[i * P64 + j] = (T)(i > j ? (dXv[r] + ej * dXw[r]) * bj : 0.f);
+            }
+        }
+        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
+        f32x4 dk[2][4];
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+            const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                f32x4 av = ZERO4, ak = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s + 31 < 16 * t) continue;         // A[i][j] = 0 for i < j
+                    const V8 af = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                    av = Mma<T>::run(frag_cols(sDvn, P128, 32 * s, n16, lane), af, av);
+                    ak = Mma<T>::run(frag_cols(sDW, P128, 32 * s, n16, lane), af, ak);
                 }
-                sM1[i * P64 + l] = (T)E;
-            }
-            colF = sum_over_g(colF);
-            if (g == 0 && tl <= w) atomicAdd(&sDg[l], -colF);
-        }
+                const int j = 16 * t + c16;
+                const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + j * P128 + n16 + 4 * g);
+                float dbv = 0.f, dot = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
-            if (c16 == 0) { atomicAdd(&sDb[16 * w + 4 * g + r], a); atomicAdd(&sDg[16 * w + 4 * g + r], b); }
-        }
-    }
-    __syncthreads();
-    // dk += E k + E^T k, on top of what the previous kernel left
-#pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2) {
-        const int n16 = 16 * (2 * w + a2);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            f32x4 acc = dk[a2][t];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const V8 af = frag_cols(X1, P128, 32 * s, n16, lane);
-                if (32 * s <= 16 * t + 15) acc = Mma<T>::run(af, frag_rows(sM1, P64, 16 * t, 32 * s, lane), acc);     // E[i][l], l < i
-                if (32 * s + 31 >= 16 * t) acc = Mma<T>::run(af, frag_cols(sM1, P64, 32 * s, 16 * t, lane), acc);     // E[i][l], i > l
-            }
-            const int x = 16 * t + c16;
-            if (x < c.valid) {
-                T* at = (T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g;
-                const V4 old = *(const V4*)at;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] += (float)old[r];
-                *(V4*)at = pack4<T>(acc);
+                for (int r = 0; r < 4; ++r) { dbv += av[r] * (float)v4[r]; dot += ak[r] * (float)k4[r]; }
+                dbv = sum_over_g(dbv);
+                dot = sum_over_g(dot);
+                const float ej = __expf(sGam[j]), bj = sBeta[j];
+                if (g == 0) { atomicAdd(&sDb[j], dbv + ej * dot); atomicAdd(&sDg[j], bj * ej * dot); }
+                if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj);
+                dk[a2][t] = ak * (bj * ej);
             }
         }
-    }
-    if (w == 0) {
-        float x = sDg[lane];
+        lds_barrier();
+        // Y = dA A^T
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const float y = __shfl_down(x, off, 64);
-            if (lane + off < 64) x += y;
+        for (int tl = 0; tl < 4; ++tl) {
+            f32x4 acc = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+                acc = Mma<T>::run(frag_rows(sM1, P64, 16 * w, 32 * s, lane), frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+            const int l = 16 * tl + c16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
         }
-        if (lane < c.valid) {
-            p.dg[(c.tok0 + lane) * p.HV + hv] = x;
-            p.dbeta[(c.tok0 + lane) * p.HV + hv] = sDb[lane];
+        lds_barrier();
+        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
+        {
+            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4, kk = ZERO4;
+                if (tl <= w) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        acc = Mma<T>::run(frag_cols(sA, P64, 32 * s, 16 * w, lane), frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), frag_rows(sK, P128, 16 * tl, 32 * s, lane), kk);
+                }
+                const int l = 16 * tl + c16;
+                const float gl = sGam[l];
+                float colF = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    float E = 0.f;
+                    if (i > l) {
+                        const float d = __expf(sGam[i] - gl), dL = -acc[r];
+                        dbi[r] += dL * kk[r] * d;
+                        E = dL * sBeta[i] * d;
+                        const float F = E * kk[r];
+                        rowF[r] += F;
+                        colF += F;
+                    }
+                    sM1[i * P64 + l] = (T)E;
+                }
+                colF = sum_over_g(colF);
+                if (g == 0 && tl <= w) atomicAdd(&sDg[l], -colF);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
+                if (c16 == 0) { atomicAdd(&sDb[16 * w + 4 * g + r], a); atomicAdd(&sDg[16 * w + 4 * g + r], b); }
+            }
         }
+        lds_barrier();
+        // dk += E k + E^T k, on top of what the previous kernel left
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2) {
+            const int n16 = 16 * (2 * w + a2);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                f32x4 acc = dk[a2][t];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const V8 af = frag_cols(sK, P128, 32 * s, n16, lane);
+                    if (32 * s <= 16 * t + 15) acc = Mma<T>::run(af, frag_rows(sM1, P64, 16 * t, 32 * s, lane), acc);     // E[i][l], l < i
+                    if (32 * s + 31 >= 16 * t) acc = Mma<T>::run(af, frag_cols(sM1, P64, 32 * s, 16 * t, lane), acc);     // E[i][l], i > l
+                }
+                const int x = 16 * t + c16;
+                if (x < c.valid) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
+                    *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(acc);
+                }
+            }
+        }
+        if (w == 0) {
+            float x = sDg[lane];
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_down(x, off, 64);
+                if (lane + off < 64) x += y;
+            }
+            if (lane < c.valid) {
+                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
+                p.dbeta[(c.tok0 + lane) * p.HV + hv] = sDb[lane];
+            }
+        }
+        lds_barrier();
     }
 }
 
@@ -849,16 +899,17 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
     else scan_kernels<T, 128>(&state, &dstate, &smem_state, &smem_dstate);
     struct K { const void* f; size_t smem; const char* name; unsigned grid; };
     const K ks[5] = {
-        {(const void*)gdn_bwd_prepare_kernel<T>, BWD_PREP_SMEM, "gdn_bwd_prepare_kernel", units},
+        {(const void*)gdn_bwd_prepare_kernel<T>, BWD_PREP_SMEM, "gdn_bwd_prepare_kernel", units < 512u ? units : 512u},
         {state, smem_state, "gdn_bwd_state_kernel", runs},
         {dstate, smem_dstate, "gdn_bwd_dstate_kernel", runs},
-        {(const void*)gdn_bwd_dqkw_kernel<T>, BWD_DQKW_SMEM, "gdn_bwd_dqkw_kernel", units},
-        {(const void*)gdn_bwd_wy_kernel<T>, BWD_WY_SMEM, "gdn_bwd_wy_kernel", units},
+        {(const void*)gdn_bwd_dqkw_kernel<T>, BWD_DQKW_SMEM, "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
+        {(const void*)gdn_bwd_wy_kernel<T>, BWD_WY_SMEM, "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
     const int vi = vbt == 32 ? 0 : vbt == 64 ? 1 : 2;
     for (int i = 0; i < 5; ++i) {
         if (int rc = ensure_dynamic_smem(ks[i].f, ks[i].smem, done[vi][i], ks[i].name)) return rc;
-        void* args[] = {(void*)&p};
+        int64_t nunits = units;
+        void* args[] = {(void*)&p, (void*)&nunits};             // (the kernels that walk over the units take their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
     }
@@ -888,7 +939,7 @@ extern "C" int gdn_chunk_bwd(
     GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
                   who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
-    GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
+    GDN_CHECK_ARG((flags & ~(uint32_t)(GDN_FLAG_CU_INT32 | (7u << 27))) == 0, GDN_ERR_UNSUPPORTED,
                   "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
                   "%s: too many heads or chunks for one launch", who);
