@@ -1,14 +1,15 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
 configuration the >= 50 %-of-MFMA-roofline target is quoted on.  A step is one call of
 chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries, under
 "other_workloads", the decode step (B=256: us/step and state GB/s), the other prefill
-configurations and the layer's two memory-bound steps either side of the operator (causal
-convolution, gated norm), and:
+configurations, the layer's two memory-bound steps either side of the operator (causal
+convolution, gated norm), the reference's published shapes (forward, and forward + backward through
+autograd: the `*_fwd_bwd` rows), and:
   roofline      dominant stage (the launches of one C entry point), algorithmic FLOPs (or bytes)
                 per call / its mean duration measured with HIP events on the launch stream
   cpu_baseline  the CPU oracle (torch fp32, all host cores) on a bounded sample of the workload
@@ -232,6 +233,26 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     return out
 
 
+def bench_train(w, steps, warmup, device):
+    """Forward and backward of the operator through autograd on one of the published shapes, as the reference times its
+    'fwdbwd' mode (benchmarks/ops/run.py:340-384: the op, then backward of its output with a fixed do)."""
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    _, d = make_prefill_inputs(w, device)
+    leaves = [d[n].requires_grad_(True) for n in ('q', 'k', 'v', 'g', 'beta')]
+    do = torch.randn_like(d['v'])
+    l2norm = w.get('l2norm', False)
+
+    def step():
+        o, _ = chunk_gated_delta_rule(*leaves, use_qk_l2norm_in_kernel=l2norm)
+        o.backward(do)
+        for x in leaves:
+            x.grad = None
+
+    per_call, _ = _time_calls(step, steps, warmup)
+    return dict(workload=w['name'] + '; forward and backward through autograd', ms_per_step=round(per_call * 1e3, 4),
+                tokens_per_s=round(w['B'] * w['T'] / per_call, 1))
+
+
 def cpu_baseline_prefill(w, cpu):
     """Oracle (torch fp32 chunked form) on the first tokens of the same inputs; the sample
     length is chosen from a short calibration run so that the timed run takes ~10-20 s."""
@@ -435,7 +456,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
@@ -464,6 +485,13 @@ def main():
         return
     for key, val in WORKLOADS.items():
         val['key'] = key
+    if args.workload.startswith('train_'):
+        name = args.workload[len('train_'):]
+        r = bench_train(dict(PUBLISHED[name], key=name), args.steps, args.warmup, device)
+        print(json.dumps(dict(metric='gdn_chunk_fwd_bwd_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
+                              n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
+                              data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
+        return
     if args.workload in PUBLISHED:
         w = dict(PUBLISHED[args.workload], key=args.workload, stages=False)
         r = bench_prefill(w, args.steps, args.warmup, device, False)
@@ -510,6 +538,11 @@ def main():
             extra[name] = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), tokens_per_s=round(r['value'], 1),
                                call_ms_quantiles=r['call_ms_quantiles'], roofline=r['roofline'])
             torch.cuda.empty_cache()
+        # training step (forward + backward) on the published shapes the backward kernels cover (head dims up to 128)
+        for name, ww in PUBLISHED.items():
+            if ww.get('K', 128) <= 128 and ww.get('V', 128) <= 128:
+                extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
+                torch.cuda.empty_cache()
         line['other_workloads'] = extra
     print(json.dumps(line))
 
