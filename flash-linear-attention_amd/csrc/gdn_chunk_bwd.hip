@@ -596,79 +596,116 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         lds_barrier();
         if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-        f32x4 G1[2][4], dKS[2][4];
+        // Operand fragments are fetched from LDS once per use across the two feature tiles of this wave.
+        f32x4 G1[2][4], dKS[2][4], dWt[2][4], dPt[4];
         float sdot = 0.f;
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[a2][t] = dKS[a2][t] = ZERO4;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dPt[t] = ZERO4;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sdot += (float)sf[a2][s][e] * (float)df[a2][s][e];
+            const V8 own = frag_rows(sDO, P128, 16 * w, 32 * s, lane);        // this wave's 16 token rows of do, for dP
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const V8 bdo = frag_rows(sDO, P128, 16 * t, 32 * s, lane), bdv = frag_rows(sDvn, P128, 16 * t, 32 * s, lane),
+                         bvn = frag_rows(sVn, P128, 16 * t, 32 * s, lane);
+#pragma unroll
+                for (int a2 = 0; a2 < 2; ++a2) {
+                    G1[a2][t] = Mma<T>::run(sf[a2][s], bdo, G1[a2][t]);
+                    dWt[a2][t] = Mma<T>::run(sf[a2][s], bdv, dWt[a2][t]);
+                    dKS[a2][t] = Mma<T>::run(df[a2][s], bvn, dKS[a2][t]);
+                }
+                if (t <= w) dPt[t] = Mma<T>::run(own, bvn, dPt[t]);
+            }
+        }
         {
             T* dWu = (T*)p.ws.dWm + u * 64 * BD;
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {
-                f32x4 dWt[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[t] = dKS[a2][t] = ZERO4;
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) sdot += (float)sf[a2][s][e] * (float)df[a2][s][e];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        G1[a2][t] = Mma<T>::run(sf[a2][s], frag_rows(sDO, P128, 16 * t, 32 * s, lane), G1[a2][t]);
-                        dWt[t] = Mma<T>::run(sf[a2][s], frag_rows(sDvn, P128, 16 * t, 32 * s, lane), dWt[t]);
-                        dKS[a2][t] = Mma<T>::run(df[a2][s], frag_rows(sVn, P128, 16 * t, 32 * s, lane), dKS[a2][t]);
-                    }
-                }
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[t]);
-            }
+                    *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[a2][t]);
         }
         // dP o D for this wave's 16 token rows, as an operand tile
+        {
+            float gi[4];
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            f32x4 acc = ZERO4;
-            if (tj <= w) {
+            for (int r = 0; r < 4; ++r) gi[r] = sGam[16 * w + 4 * g + r];
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
-                    acc = Mma<T>::run(frag_rows(sDO, P128, 16 * w, 32 * s, lane), frag_rows(sVn, P128, 16 * tj, 32 * s, lane), acc);
-            }
-            const int j = 16 * tj + c16;
-            const float gj = sGam[j];
+            for (int tj = 0; tj < 4; ++tj) {
+                const int j = 16 * tj + c16;
+                const float gj = sGam[j];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int i = 16 * w + 4 * g + r;
-                sDP[i * P64 + j] = (T)(i >= j ? p.scale * acc[r] * __expf(sGam[i] - gj) : 0.f);
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    sDP[i * P64 + j] = (T)(i >= j ? p.scale * dPt[tj][r] * __expf(gi[r] - gj) : 0.f);
+                }
             }
         }
         lds_barrier();
 
         const float glast = sGam[63];
         float dglast = __expf(glast) * sdot;
+        {
+            V8 fk[2][2], fq[2][2];
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2) {
-            const int n16 = 16 * (2 * w + a2);
+            for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    fk[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    fq[a2][s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
+                }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int x = 16 * t + c16;
                 const float gx = sGam[x];
-                f32x4 dq = G1[a2][t] * (p.scale * __expf(gx));
-                f32x4 dk = dKS[a2][t] * __expf(glast - gx);
-                const V4 q4 = *(const V4*)(sQ + x * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+                const float fqs = p.scale * __expf(gx), fks = __expf(glast - gx);
+                f32x4 dq[2], dk[2];
+                V4 q4[2], k4[2];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) dglast += (float)k4[r] * dk[r];
+                for (int a2 = 0; a2 < 2; ++a2) {
+                    const int n16 = 16 * (2 * w + a2);
+                    dq[a2] = G1[a2][t] * fqs;
+                    dk[a2] = dKS[a2][t] * fks;
+                    q4[a2] = *(const V4*)(sQ + x * P128 + n16 + 4 * g);
+                    k4[a2] = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dglast += (float)k4[a2][r] * dk[a2][r];
+                }
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    if (32 * s <= 16 * t + 15)                  // dP[i][j] = 0 for j > i
-                        dq = Mma<T>::run(frag_cols(sK, P128, 32 * s, n16, lane), frag_rows(sDP, P64, 16 * t, 32 * s, lane), dq);
-                    if (32 * s + 31 >= 16 * t)                  // ... and for i < j
-                        dk = Mma<T>::run(frag_cols(sQ, P128, 32 * s, n16, lane), frag_cols(sDP, P64, 32 * s, 16 * t, lane), dk);
+                    if (32 * s <= 16 * t + 15) {                // dP[i][j] = 0 for j > i
+                        const V8 e = frag_rows(sDP, P64, 16 * t, 32 * s, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; ++a2) dq[a2] = Mma<T>::run(fk[a2][s], e, dq[a2]);
+                    }
+                    if (32 * s + 31 >= 16 * t) {                // ... and for i < j
+                        const V8 e = frag_cols(sDP, P64, 32 * s, 16 * t, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; ++a2) dk[a2] = Mma<T>::run(fq[a2][s], e, dk[a2]);
+                    }
                 }
                 float dgx = 0.f;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) dgx += (float)q4[r] * dq[r] - (float)k4[r] * dk[r];
+                for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dgx += (float)q4[a2][r] * dq[a2][r] - (float)k4[a2][r] * dk[a2][r];
                 dgx = sum_over_g(dgx);
                 if (g == 0) atomicAdd(&sDg[x], dgx);
                 if (x < c.valid) {
-                    *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq);
-                    *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk);
+#pragma unroll
+                    for (int a2 = 0; a2 < 2; ++a2) {
+                        const int n16 = 16 * (2 * w + a2);
+                        *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq[a2]);
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk[a2]);
+                    }
                 }
             }
         }
@@ -740,80 +777,117 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         lds_barrier();
         if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-        // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta))
+        // Operand fragments are fetched from LDS once and kept: what does not change across an inner loop is loaded outside it.
+        // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta));
+        // k k^T of the same rows and columns is formed along the way, for the last step but one
+        f32x4 kkT[4];
+        {
+            V8 fa[4], fw[4], fk[4];
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            f32x4 dXv = ZERO4, dXw = ZERO4;
-            if (tj <= w) {
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    dXv = Mma<T>::run(frag_rows(sDvn, P128, 16 * w, 32 * s, lane), frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
-                    dXw = Mma<T>::run(frag_rows(sDW, P128, 16 * w, 32 * s, lane), frag_rows(sK, P128, 16 * tj, 32 * s, lane), dXw);
-                }
+            for (int s = 0; s < 4; ++s) {
+                fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
+                fw[s] = frag_rows(sDW, P128, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sK, P128, 16 * w, 32 * s, lane);
             }
-            const int j = 16 * tj + c16;
-            const float ej = __expf(sGam[j]), bj = sBeta[j];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int i = 16 * w + 4 * g + r;
-                sM1[i * P64 + j] = (T)(i > j ? (dXv[r] + ej * dXw[r]) * bj : 0.f);
+            for (int tj = 0; tj < 4; ++tj) {
+                f32x4 dXv = ZERO4, dXw = ZERO4;
+                kkT[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 bk = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+                        dXv = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
+                        dXw = Mma<T>::run(fw[s], bk, dXw);
+                        kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
+                    }
+                }
+                const int j = 16 * tj + c16;
+                const float ej = __expf(sGam[j]), bj = sBeta[j];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    sM1[i * P64 + j] = (T)(i > j ? (dXv[r] + ej * dXw[r]) * bj : 0.f);
+                }
             }
         }
         // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
         f32x4 dk[2][4];
-#pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2) {
-            const int n16 = 16 * (2 * w + a2);
+        {
+            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
+            float ej[4], bj[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                f32x4 av = ZERO4, ak = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                ej[t] = __expf(sGam[16 * t + c16]);
+                bj[t] = sBeta[16 * t + c16];
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2) {
+                const int n16 = 16 * (2 * w + a2);
+                V8 fdv[2], fdw[2];
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    if (32 * s + 31 < 16 * t) continue;         // A[i][j] = 0 for i < j
-                    const V8 af = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                    av = Mma<T>::run(frag_cols(sDvn, P128, 32 * s, n16, lane), af, av);
-                    ak = Mma<T>::run(frag_cols(sDW, P128, 32 * s, n16, lane), af, ak);
+                    fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
+                    fdw[s] = frag_cols(sDW, P128, 32 * s, n16, lane);
                 }
-                const int j = 16 * t + c16;
-                const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + j * P128 + n16 + 4 * g);
-                float dbv = 0.f, dot = 0.f;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) { dbv += av[r] * (float)v4[r]; dot += ak[r] * (float)k4[r]; }
-                dbv = sum_over_g(dbv);
-                dot = sum_over_g(dot);
-                const float ej = __expf(sGam[j]), bj = sBeta[j];
-                if (g == 0) { atomicAdd(&sDb[j], dbv + ej * dot); atomicAdd(&sDg[j], bj * ej * dot); }
-                if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj);
-                dk[a2][t] = ak * (bj * ej);
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 av = ZERO4, ak = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
+                        av = Mma<T>::run(fdv[s], fA[t][s], av);
+                        ak = Mma<T>::run(fdw[s], fA[t][s], ak);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + j * P128 + n16 + 4 * g);
+                    float dbv = 0.f, dot = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) { dbv += av[r] * (float)v4[r]; dot += ak[r] * (float)k4[r]; }
+                    dbv = sum_over_g(dbv);
+                    dot = sum_over_g(dot);
+                    if (g == 0) { atomicAdd(&sDb[j], dbv + ej[t] * dot); atomicAdd(&sDg[j], bj[t] * ej[t] * dot); }
+                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                    dk[a2][t] = ak * (bj[t] * ej[t]);
+                }
             }
         }
         lds_barrier();
         // Y = dA A^T
+        {
+            V8 fd[2];
 #pragma unroll
-        for (int tl = 0; tl < 4; ++tl) {
-            f32x4 acc = ZERO4;
+            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
-                acc = Mma<T>::run(frag_rows(sM1, P64, 16 * w, 32 * s, lane), frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
-            const int l = 16 * tl + c16;
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+                const int l = 16 * tl + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+            }
         }
         lds_barrier();
         // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
         {
-            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f};
+            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
+            V8 fAt[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
-                f32x4 acc = ZERO4, kk = ZERO4;
+                f32x4 acc = ZERO4;
                 if (tl <= w) {
 #pragma unroll
-                    for (int s = 0; s < 2; ++s)
-                        acc = Mma<T>::run(frag_cols(sA, P64, 32 * s, 16 * w, lane), frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-                        kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), frag_rows(sK, P128, 16 * tl, 32 * s, lane), kk);
+                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
                 }
+                const f32x4 kk = kkT[tl];
                 const int l = 16 * tl + c16;
                 const float gl = sGam[l];
                 float colF = 0.f;
@@ -822,9 +896,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     const int i = 16 * w + 4 * g + r;
                     float E = 0.f;
                     if (i > l) {
-                        const float d = __expf(sGam[i] - gl), dL = -acc[r];
+                        const float d = __expf(gi[r] - gl), dL = -acc[r];
                         dbi[r] += dL * kk[r] * d;
-                        E = dL * sBeta[i] * d;
+                        E = dL * bi[r] * d;
                         const float F = E * kk[r];
                         rowF[r] += F;
                         colF += F;
@@ -842,23 +916,36 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         }
         lds_barrier();
         // dk += E k + E^T k, on top of what the previous kernel left
+        {
+            V8 fk[2][2];
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2) {
-            const int n16 = 16 * (2 * w + a2);
+            for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                f32x4 acc = dk[a2][t];
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const V8 af = frag_cols(sK, P128, 32 * s, n16, lane);
-                    if (32 * s <= 16 * t + 15) acc = Mma<T>::run(af, frag_rows(sM1, P64, 16 * t, 32 * s, lane), acc);     // E[i][l], l < i
-                    if (32 * s + 31 >= 16 * t) acc = Mma<T>::run(af, frag_cols(sM1, P64, 32 * s, 16 * t, lane), acc);     // E[i][l], i > l
+                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
+                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
+                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
+                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
                 }
                 const int x = 16 * t + c16;
                 if (x < c.valid) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
-                    *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(acc);
+                    for (int a2 = 0; a2 < 2; ++a2) {
+                        f32x4 acc = dk[a2][t];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(acc);
+                    }
                 }
             }
         }
