@@ -226,6 +226,60 @@ def test_chunk_backward_options(what):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('seed', range(24))
+def test_chunk_backward_random(seed):
+    """Seeded random combinations of head dims, grouping, packing, state layout, prologues and dtype."""
+    import random
+    rnd = random.Random(1000 + seed)
+    D = rnd.choice([16, 32, 40, 64, 96, 128])
+    V = rnd.choice([D, 64, 128, 192]) if seed % 4 == 0 else D
+    H = rnd.choice([1, 2, 3])
+    HV = H * rnd.choice([1, 1, 2, 4])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    packed = rnd.random() < 0.4
+    if packed:
+        N = rnd.randint(1, 4)
+        cu = [0]
+        for _ in range(N):
+            cu.append(cu[-1] + rnd.choice([1, 7, 63, 64, 65, 130, 200]))
+        B, T = 1, cu[-1]
+    else:
+        B, T, cu = rnd.randint(1, 3), rnd.choice([1, 5, 64, 100, 129, 257]), None
+        N = B
+    kw = {}
+    gen = torch.Generator().manual_seed(2000 + seed)
+    q, k = torch.randn(B, T, H, D, generator=gen), torch.randn(B, T, H, D, generator=gen)
+    if rnd.random() < 0.5:
+        kw['use_qk_l2norm_in_kernel'] = True
+    else:
+        q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    q, k = q.to(dtype), k.to(dtype)
+    v = torch.randn(B, T, HV, V, generator=gen).to(dtype)
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / rnd.choice([1.0, 4.0, 16.0])
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    if rnd.random() < 0.3:
+        beta = torch.randn(B, T, HV, generator=gen)
+        kw.update(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=rnd.random() < 0.5)
+    if rnd.random() < 0.3:
+        g = torch.randn(B, T, HV, generator=gen)
+        kw.update(use_gate_in_kernel=True, A_log=torch.randn(HV, generator=gen) * 0.5,
+                  dt_bias=torch.randn(HV, generator=gen) * 0.5 if rnd.random() < 0.5 else None)
+    vfirst = rnd.random() < 0.3
+    h0 = torch.randn(N, HV, D, V, generator=gen) * 0.3 if rnd.random() < 0.7 else None
+    dht = torch.randn(N, HV, D, V, generator=gen) if rnd.random() < 0.7 else None
+    if vfirst:
+        kw['state_v_first'] = True
+        h0 = None if h0 is None else h0.transpose(-1, -2).contiguous()
+        dht = None if dht is None else dht.transpose(-1, -2).contiguous()
+    do = torch.randn(B, T, HV, V, generator=gen).to(dtype)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, dtype=torch.float32, **kw)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu, **dict(kw))
+    # (single tokens and very short sequences: the rounding of a handful of bf16 products is all there is to compare)
+    tol = TOL if T >= 64 else {n: 2 * x for n, x in TOL.items()}
+    _compare(ref, got, tol=tol)
+
+
+@pytest.mark.gpu
 def test_chunk_backward_c_entry_checks():
     from fla_hip import _lib
     lib = _lib.load()
