@@ -317,8 +317,12 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
     T* sW = (T*)smem; T* sK = sW + 64 * P128; T* sS = sK + 64 * P128; T* sVn = sS + 128 * PV;
     float* sGam = (float*)(sVn + 64 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int vs = blockIdx.x % NVS, hv = (blockIdx.x / NVS) % p.HV, hq = hv / (p.HV / p.H);
-    const int64_t n = blockIdx.x / (NVS * p.HV);
+    // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
+    // an L2 for the rows of k, q and w that all of them read.
+    const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
+    if (run >= p.N * p.HV) return;
+    const int vs = (blockIdx.x / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
+    const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
 
@@ -390,19 +394,23 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
         lds_barrier();
         {
             const float eg = __expf(glast);
+            V8 kf[2][2];
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {
-                V8 kf[2];
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                for (int s = 0; s < 2; ++s) kf[s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
+                for (int s = 0; s < 2; ++s) kf[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    f32x4 acc = S[a2][b] * eg;
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(frag_cols(sVn, PV, 32 * s, 16 * b, lane), kf[s], acc);
-                    S[a2][b] = acc;
+                for (int b = 0; b < NB; ++b) S[a2][b] *= eg;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const V8 fv = frag_cols(sVn, PV, 32 * s, 16 * b, lane);
+#pragma unroll
+                    for (int a2 = 0; a2 < 2; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
                 }
-            }
         }
         lds_barrier();
     }
@@ -418,8 +426,12 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
     float* sGam = (float*)(sDS + 128 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int vs = blockIdx.x % NVS, hv = (blockIdx.x / NVS) % p.HV, hq = hv / (p.HV / p.H);
-    const int64_t n = blockIdx.x / (NVS * p.HV);
+    // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
+    // an L2 for the rows of k, q and w that all of them read.
+    const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
+    if (run >= p.N * p.HV) return;
+    const int vs = (blockIdx.x / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
+    const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
 
@@ -504,25 +516,29 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
         lds_barrier();
         {
             const float eg = __expf(glast);
+            V8 qf[2][2], wf[2][2];
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {
-                V8 qf[2], wf[2];
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    qf[s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
-                    wf[s] = frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    qf[a2][s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    wf[a2][s] = frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane);
                 }
 #pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    f32x4 acc = dS[a2][b] * eg;
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        acc = Mma<T>::run(frag_cols(sDOg, PV, 32 * s, 16 * b, lane), qf[s], acc);
-                        acc = Mma<T>::run(frag_cols(sDvn, PV, 32 * s, 16 * b, lane), wf[s], acc);
+                for (int b = 0; b < NB; ++b) dS[a2][b] *= eg;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const V8 fo = frag_cols(sDOg, PV, 32 * s, 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, 16 * b, lane);
+#pragma unroll
+                    for (int a2 = 0; a2 < 2; ++a2) {
+                        dS[a2][b] = Mma<T>::run(fo, qf[a2][s], dS[a2][b]);
+                        dS[a2][b] = Mma<T>::run(fv, wf[a2][s], dS[a2][b]);
                     }
-                    dS[a2][b] = acc;
                 }
-            }
         }
         lds_barrier();
     }
@@ -977,7 +993,7 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
     // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.
     const int64_t runs1 = p.N * p.HV;
     const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
-    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)(runs1 * (BD / vbt));
+    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)((runs1 + 7) / 8 * 8 * (BD / vbt));
     static SmemAttrDone done[3][5];
     const void *state, *dstate;
     size_t smem_state, smem_dstate;
