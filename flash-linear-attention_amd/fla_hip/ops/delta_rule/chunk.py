@@ -1,8 +1,9 @@
-"""``chunk_delta_rule``: the delta rule without gates (DeltaNet), forward only, with the signature,
+"""``chunk_delta_rule``: the delta rule without gates (DeltaNet), with the signature,
 validation and error types of fla/ops/delta_rule/chunk.py:223-349.  It is the gated operator with
 g = 0 (the reference runs the same state and output kernels with ``g=None``,
 fla/ops/delta_rule/chunk.py:39-62), so it runs on the same HIP kernels: the library takes
-``g = NULL`` and skips nothing but the gate load."""
+``g = NULL`` and skips nothing but the gate load.  Differentiable like the gated operator (backward through
+``gdn_chunk_bwd`` with ``g = NULL``; the reference's own backward is fla/ops/delta_rule/chunk.py:65-140)."""
 from __future__ import annotations
 
 import torch
@@ -54,6 +55,11 @@ def chunk_delta_rule(
                 f'The number of initial states is expected to be equal to the number of input sequences, '
                 f'i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.')
     scale = k.shape[-1] ** -0.5 if scale is None else scale
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, beta, initial_state)):
+        from fla_hip.ops.gated_delta_rule.chunk_bwd import ChunkGatedDeltaRuleFunction
+        return ChunkGatedDeltaRuleFunction.apply(
+            q, k, v, None, beta, scale, initial_state, output_final_state, False, cu_seqlens, cu_seqlens_cpu, None,
+            use_qk_l2norm_in_kernel, False, None, None, False, False, chunk_size)
     return chunk_gated_delta_rule_fwd(
         q, k, v, None, beta, scale, initial_state, output_final_state, False,
         cu_seqlens, cu_seqlens_cpu, None, chunk_size, None, None, use_qk_l2norm_in_kernel, False, False)

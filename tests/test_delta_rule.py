@@ -94,3 +94,35 @@ def test_chunk_delta_rule_packed_and_validation():
     with pytest.raises(ValueError):
         chunk_delta_rule(q.to(dev), k.to(dev), v.to(dev), beta.to(dev), initial_state=h0[:3].to(dev),
                          cu_seqlens=torch.tensor(cu, device=dev))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,D,scale,l2,dtype', [
+    (2, 100, 4, 60, 0.1, False, torch.float16),
+    (2, 500, 3, 128, 0.1, False, torch.float16),
+    (1, 300, 2, 128, 1, True, torch.bfloat16),
+])
+def test_chunk_delta_rule_backward(B, T, H, D, scale, l2, dtype):
+    """Gradients through the operator against reverse-mode differentiation of the oracle's recurrence without a gate
+    (the reference checks its backward the same way, bars 0.008: tests/ops/test_delta.py:60-86)."""
+    from fla_hip.ops.delta_rule import chunk_delta_rule
+    gen = torch.Generator().manual_seed(7)
+    q, k = torch.randn(B, T, H, D, generator=gen), torch.randn(B, T, H, D, generator=gen)
+    if not l2:
+        q, k = F.normalize(q, dim=-1), F.normalize(k, dim=-1)
+    q, k = q.to(dtype), k.to(dtype)
+    v = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, H, generator=gen).sigmoid()
+    h0 = torch.randn(B, H, D, D, generator=gen) * 0.3
+    do = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    dht = torch.randn(B, H, D, D, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, None, beta, do, dht, scale=scale, initial_state=h0, use_qk_l2norm_in_kernel=l2,
+                                   dtype=torch.float32)
+    dev = 'cuda'
+    leaves = [x.to(dev).requires_grad_(True) for x in (q, k, v, beta, h0)]
+    o, ht = chunk_delta_rule(leaves[0], leaves[1], leaves[2], leaves[3], scale=scale, initial_state=leaves[4],
+                             output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    ((o.float() * do.to(dev).float()).sum() + (ht * dht.to(dev)).sum()).backward()
+    for name, x in zip(('dq', 'dk', 'dv', 'dbeta', 'dh0'), leaves):
+        r = O.get_err_ratio(ref[name], x.grad.float().cpu())
+        assert r <= 0.008, f'{name}: rel-rmse {r:.3e}'
