@@ -12,7 +12,7 @@ import torch
 import torch.nn as nn
 
 from fla_hip import _lib
-from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, ptr, require_gpu
+from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, forward_only, ptr, require_gpu
 from fla_hip.utils import input_guard
 
 MAX_KERNEL_SIZE = 8
@@ -40,6 +40,7 @@ def _rows(x: torch.Tensor, D: int) -> torch.Tensor:
 
 def _launch_fwd(x, weight, bias, residual, initial_state, want_y, want_state, activation, cu_seqlens, W):
     dev = require_gpu(x)
+    forward_only('causal_conv1d', x, residual)
     B, T, D = x.shape
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     if cu_seqlens is not None and B != 1:
@@ -132,6 +133,7 @@ def causal_conv1d_update(
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """One new token per sequence: ``x`` is ``[N, D]``, ``[1, N, D]`` or ``[N, 1, D]``; ``cache`` ``[N, D, W]`` is
     updated in place (shifted left by one, ``x`` appended) and returned."""
+    forward_only('causal_conv1d_update', x, residual)
     if weight is None:
         raise ValueError('causal_conv1d_update needs a weight of shape [D, W]')
     dev = require_gpu(x)

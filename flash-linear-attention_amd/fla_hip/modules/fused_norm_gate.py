@@ -8,7 +8,7 @@ import torch
 import torch.nn as nn
 
 from fla_hip import _lib
-from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, ptr, require_gpu
+from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, forward_only, ptr, require_gpu
 
 
 def _gate_code(activation: str) -> int:
@@ -34,6 +34,7 @@ def layer_norm_gated_fwd(
     """``x``, ``g`` are ``[T, D]``.  Returns ``(y, mean, rstd, residual_out)`` like the reference: ``mean`` is ``None``
     for RMS norm and ``residual_out`` is ``x`` itself when no residual stream was asked for."""
     dev = require_gpu(x, g)
+    forward_only('layer_norm_gated', x, g, residual)
     if x.dim() != 2 or g.shape != x.shape:
         raise ValueError(f'x and g must be [T, D] and alike, got {tuple(x.shape)} and {tuple(g.shape)}')
     T, D = x.shape

@@ -66,3 +66,10 @@ def unify_gate_beta(g, beta):
 
 def current_stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def forward_only(what: str, *activations: torch.Tensor | None) -> None:
+    """Operators without a backward refuse activations that require a gradient (in grad mode) instead of returning a
+    result that silently carries none.  Parameters are not looked at: inference outside ``torch.no_grad()`` is fine."""
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in activations):
+        raise NotImplementedError(f'{what} has no backward in fla_hip: run it under torch.no_grad() or on detached inputs')
