@@ -21,27 +21,27 @@
 
 namespace gdn {
 
-constexpr int BD = 128;              // head dims of these kernels
-constexpr int P128 = BD + 8;         // LDS pitch, in elements, of a [64][128] tile
+constexpr int BD = 128;              // value columns of these kernels; key features: KD = 128 KT with KT = 1 or 2 (a template argument)
+constexpr int P128 = BD + 8;         // LDS pitch, in elements, of a [64][128] tile ([64][KD] tiles: KD + 8)
 constexpr int P64 = CH + 8;          // ... of a [64][64] tile
 constexpr int PL = CH + 4;           // pitch of the fp32 matrix L
 
 // Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels),
-// A [64][64], P^T [64][64], w [64][128], u -> v_new [64][128], S [128][128] ([K][V]), dS [128][128], dv_new [64][128],
-// dw [64][128], all in the operand type.
+// A [64][64], P^T [64][64], w [64][KD], u -> v_new [64][128], S [KD][128] ([K][V]), dS [KD][128], dv_new [64][128],
+// dw [64][KD], all in the operand type.
 struct BwdWs {
     float* Gam; float* Dgam;
     void* Am; void* PT; void* Wm; void* Vn; void* Hs; void* dHs; void* dVn; void* dWm;
 };
-inline size_t bwd_ws_layout(int64_t units, char* base, BwdWs* ws) {
+inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
     const size_t u = (size_t)units;
     void* Gam = take(u * 64 * 4); void* Dgam = take(u * 64 * 4);
     void* Am = take(u * 64 * 64 * 2); void* PT = take(u * 64 * 64 * 2);
-    void* Wm = take(u * 64 * BD * 2); void* Vn = take(u * 64 * BD * 2);
-    void* Hs = take(u * BD * BD * 2); void* dHs = take(u * BD * BD * 2);
-    void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * BD * 2);
+    void* Wm = take(u * 64 * KD * 2); void* Vn = take(u * 64 * BD * 2);
+    void* Hs = take(u * KD * BD * 2); void* dHs = take(u * KD * BD * 2);
+    void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * KD * 2);
     if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm};
     return off;
 }
@@ -160,25 +160,27 @@ __device__ __forceinline__ float sum_over_quad(float x) {
 // ---------------------------------------------------------------------------------------------
 // prepare
 // ---------------------------------------------------------------------------------------------
-constexpr size_t BWD_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PL + 128) * 4;
+template <int KT> constexpr size_t bwd_prep_smem() { return (2 * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + (64 * PL + 128) * 4; }
 
-template <typename T>
-__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
+template <typename T, int KT>
+__global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
+    constexpr int KD = BD * KT, PK = KD + 8;
     extern __shared__ __align__(16) char smem[];
-    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
+    T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sV = sQ + 64 * PK; T* sA = sV + 64 * P128;
     float* sL = (float*)(sA + 64 * P64); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
     // Units in turn; the next unit's rows are fetched into registers while this one is worked on.
-    TileRegs<BD> rK, rQ, rV;
+    TileRegs<KD> rK, rQ;
+    TileRegs<BD> rV;
     float rG = 0.f, rB = 0.f;
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
-        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         rG = rB = 0.f;
         if (w == 0 && lane < c.valid) {
@@ -188,8 +190,8 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, in
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
-        put_tile<BD>(sK, P128, rK, tid);
-        put_tile<BD>(sQ, P128, rQ, tid);
+        put_tile<KD>(sK, PK, rK, tid);
+        put_tile<KD>(sQ, PK, rQ, tid);
         put_tile<BD>(sV, P128, rV, tid);
         if (w == 0) {
             float x = rG;
@@ -212,10 +214,10 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, in
                 f32x4 kk = ZERO4, qk = ZERO4;
                 if (tj <= w) {
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const V8 b = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
-                        kk = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), b, kk);
-                        qk = Mma<T>::run(frag_rows(sQ, P128, 16 * w, 32 * s, lane), b, qk);
+                    for (int s = 0; s < 4 * KT; ++s) {
+                        const V8 b = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
+                        kk = Mma<T>::run(frag_rows(sK, PK, 16 * w, 32 * s, lane), b, kk);
+                        qk = Mma<T>::run(frag_rows(sQ, PK, 16 * w, 32 * s, lane), b, qk);
                     }
                 }
                 const int j = 16 * tj + c16;
@@ -233,14 +235,14 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, in
         }
         lds_barrier();
         // k -> beta e^gam k and v -> beta v, in place
-        for (int idx = tid; idx < 64 * 16; idx += 256) {
-            const int row = idx >> 4, pc = idx & 15;
-            const float bk = sBeta[row] * __expf(sGam[row]), bv = sBeta[row];
-            V8 x = *(V8*)(sK + row * P128 + pc * 8), y = *(V8*)(sV + row * P128 + pc * 8);
+        for (int idx = tid; idx < 64 * 16 * (KT + 1); idx += 256) {
+            const int row = idx / (16 * (KT + 1)), pc = idx % (16 * (KT + 1));      // the row's pieces of k, then those of v
+            T* at = pc < 16 * KT ? sK + row * PK + pc * 8 : sV + row * P128 + (pc - 16 * KT) * 8;
+            const float f = pc < 16 * KT ? sBeta[row] * __expf(sGam[row]) : sBeta[row];
+            V8 x = *(V8*)at;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { x[e] = (T)((float)x[e] * bk); y[e] = (T)((float)y[e] * bv); }
-            *(V8*)(sK + row * P128 + pc * 8) = x;
-            *(V8*)(sV + row * P128 + pc * 8) = y;
+            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
+            *(V8*)at = x;
         }
         // A = (I + L)^-1 by forward substitution, A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c]: a quad of lanes per
         // column c (16 columns per wave), lane gq of the quad keeps A[j][c] for j = gq mod 4 and adds up their part of the sum
@@ -278,20 +280,30 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, in
         }
         // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
         {
-            T* Wu = (T*)p.ws.Wm + u * 64 * BD;
+            T* Wu = (T*)p.ws.Wm + u * 64 * KD;
             T* Uu = (T*)p.ws.Vn + u * 64 * BD;
             const int i = 16 * w + c16;
+            V8 fa[2];
 #pragma unroll
-            for (int n = 0; n < 8; ++n) {
-                f32x4 aw = ZERO4, au = ZERO4;
+            for (int s = 0; s < 2; ++s) fa[s] = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int n = 0; n < 8 * KT; ++n) {
+                f32x4 aw = ZERO4;
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     if (2 * s > w) continue;                    // A is lower triangular
-                    const V8 b = frag_rows(sA, P64, 16 * w, 32 * s, lane);
-                    aw = Mma<T>::run(frag_cols(sK, P128, 32 * s, 16 * n, lane), b, aw);
-                    au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), b, au);
+                    aw = Mma<T>::run(frag_cols(sK, PK, 32 * s, 16 * n, lane), fa[s], aw);
                 }
-                *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
+                *(V4*)(Wu + i * KD + 16 * n + 4 * g) = pack4<T>(aw);
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                f32x4 au = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (2 * s > w) continue;
+                    au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), fa[s], au);
+                }
                 *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
             }
         }
@@ -305,16 +317,16 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, in
 // 16(2w+a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
 // current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
-template <int VBT> constexpr size_t bwd_state_smem() { return (2 * 64 * P128 + 128 * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
-template <int VBT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * P128 + 64 * P64 + 3 * 64 * (VBT + 8) + 128 * (VBT + 8)) * 2 + 64 * 4; }
+template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
+template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
-template <typename T, int VBT>
+template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
-    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
+    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
     extern __shared__ __align__(16) char smem[];
-    T* sW = (T*)smem; T* sK = sW + 64 * P128; T* sS = sK + 64 * P128; T* sVn = sS + 128 * PV;
+    T* sW = (T*)smem; T* sK = sW + 64 * PK; T* sS = sK + 64 * PK; T* sVn = sS + KD * PV;
     float* sGam = (float*)(sVn + 64 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
@@ -326,22 +338,22 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
 
-    f32x4 S[2][NB];
+    f32x4 S[NA][NB];
 #pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2)
+    for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const int kk = 16 * (2 * w + a2) + c16;
-            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+            const int kk = 16 * (NA * w + a2) + c16;
+            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    TileRegs<BD> rW, rK;
+    TileRegs<KD> rW, rK;
     V4 rU[NB];
     float rGam = 0.f;
     auto fetch = [&](int64_t ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        fetch_tile<BD>(rW, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
-        fetch_tile<BD>(rK, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
+        fetch_tile<KD>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
 #pragma unroll
         for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
@@ -349,18 +361,18 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
     if (sq.nc > 0) fetch(0);
     for (int64_t ic = 0; ic < sq.nc; ++ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
-        put_tile<BD>(sW, P128, rW, tid);
-        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<KD>(sW, PK, rW, tid);
+        put_tile<KD>(sK, PK, rK, tid);
         if (tid < 64) sGam[tid] = rGam;
         V4 u4[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) u4[b] = rU[b];
-        T* Hu = (T*)p.ws.Hs + u * BD * BD;
+        T* Hu = (T*)p.ws.Hs + u * KD * BD;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+        for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const int kk = 16 * (2 * w + a2) + c16;
+                const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(S[a2][b]);
                 *(V4*)(sS + kk * PV + 16 * b + 4 * g) = s4;
                 *(V4*)(Hu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
@@ -373,14 +385,14 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
             const int i = 16 * w + c16;
             const float dec = __expf(glast - sGam[i]);
             T* Vu = (T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0;
-            V8 wf[4];
+            V8 wf[4 * KT];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) wf[s] = frag_rows(sW, P128, 16 * w, 32 * s, lane);
+            for (int s = 0; s < 4 * KT; ++s) wf[s] = frag_rows(sW, PK, 16 * w, 32 * s, lane);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 f32x4 acc = ZERO4;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) acc = Mma<T>::run(frag_cols(sS, PV, 32 * s, 16 * b, lane), wf[s], acc);
+                for (int s = 0; s < 4 * KT; ++s) acc = Mma<T>::run(frag_cols(sS, PV, 32 * s, 16 * b, lane), wf[s], acc);
                 f32x4 vn;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
@@ -394,13 +406,13 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
         lds_barrier();
         {
             const float eg = __expf(glast);
-            V8 kf[2][2];
+            V8 kf[NA][2];
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
-                for (int s = 0; s < 2; ++s) kf[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
+                for (int s = 0; s < 2; ++s) kf[a2][s] = frag_cols(sK, PK, 32 * s, 16 * (NA * w + a2), lane);
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
                 for (int b = 0; b < NB; ++b) S[a2][b] *= eg;
 #pragma unroll
@@ -409,22 +421,22 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
                 for (int s = 0; s < 2; ++s) {
                     const V8 fv = frag_cols(sVn, PV, 32 * s, 16 * b, lane);
 #pragma unroll
-                    for (int a2 = 0; a2 < 2; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
+                    for (int a2 = 0; a2 < NA; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
                 }
         }
         lds_barrier();
     }
 }
 
-template <typename T, int VBT>
+template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
-    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
+    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
     extern __shared__ __align__(16) char smem[];
-    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sW = sQ + 64 * P128; T* sPT = sW + 64 * P128;
+    T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sW = sQ + 64 * PK; T* sPT = sW + 64 * PK;
     T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
-    float* sGam = (float*)(sDS + 128 * PV);
+    float* sGam = (float*)(sDS + KD * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
@@ -435,24 +447,24 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
 
-    f32x4 dS[2][NB];
+    f32x4 dS[NA][NB];
 #pragma unroll
-    for (int a2 = 0; a2 < 2; ++a2)
+    for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const int kk = 16 * (2 * w + a2) + c16;
-            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+            const int kk = 16 * (NA * w + a2) + c16;
+            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    TileRegs<BD> rK, rQ, rW;
+    TileRegs<KD> rK, rQ, rW;
     TileRegs<CH> rPT;
     TileRegs<VBT> rDO;
     float rGam = 0.f;
     auto fetch = [&](int64_t ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        fetch_tile<BD>(rK, (const T*)p.k + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
-        fetch_tile<BD>(rQ, (const T*)p.q + (tok0 * p.H + hq) * BD, (int64_t)p.H * BD, valid, tid);
-        fetch_tile<BD>(rW, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        fetch_tile<KD>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        fetch_tile<KD>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
         fetch_tile<CH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
         fetch_tile<VBT>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
@@ -460,18 +472,18 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     if (sq.nc > 0) fetch(sq.nc - 1);
     for (int64_t ic = sq.nc - 1; ic >= 0; --ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
-        put_tile<BD>(sK, P128, rK, tid);
-        put_tile<BD>(sQ, P128, rQ, tid);
-        put_tile<BD>(sW, P128, rW, tid);
+        put_tile<KD>(sK, PK, rK, tid);
+        put_tile<KD>(sQ, PK, rQ, tid);
+        put_tile<KD>(sW, PK, rW, tid);
         put_tile<CH>(sPT, P64, rPT, tid);
         put_tile<VBT>(sDO, PV, rDO, tid);
         if (tid < 64) sGam[tid] = rGam;
-        T* dHu = (T*)p.ws.dHs + u * BD * BD;
+        T* dHu = (T*)p.ws.dHs + u * KD * BD;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+        for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const int kk = 16 * (2 * w + a2) + c16;
+                const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(dS[a2][b]);
                 *(V4*)(sDS + kk * PV + 16 * b + 4 * g) = s4;
                 *(V4*)(dHu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
@@ -493,9 +505,9 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
             const int j = 16 * w + c16;
             const float dec = __expf(glast - sGam[j]);
             T* dVu = (T*)p.ws.dVn + u * 64 * BD + j * BD + vcol0;
-            V8 kf[4], pf[2];
+            V8 kf[4 * KT], pf[2];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) kf[s] = frag_rows(sK, P128, 16 * w, 32 * s, lane);
+            for (int s = 0; s < 4 * KT; ++s) kf[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
 #pragma unroll
             for (int s = 0; s < 2; ++s) pf[s] = frag_rows(sPT, P64, 16 * w, 32 * s, lane);
 #pragma unroll
@@ -507,7 +519,7 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
                     a1 = Mma<T>::run(frag_cols(sDO, PV, 32 * s, 16 * b, lane), pf[s], a1);
                 }
 #pragma unroll
-                for (int s = 0; s < 4; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, 16 * b, lane), kf[s], a2v);
+                for (int s = 0; s < 4 * KT; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, 16 * b, lane), kf[s], a2v);
                 f32x4 dvn = a1 + a2v * dec;
                 *(V4*)(dVu + 16 * b + 4 * g) = pack4<T>(dvn);
                 *(V4*)(sDvn + j * PV + 16 * b + 4 * g) = pack4<T>(-dvn);
@@ -516,16 +528,16 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
         lds_barrier();
         {
             const float eg = __expf(glast);
-            V8 qf[2][2], wf[2][2];
+            V8 qf[NA][2], wf[NA][2];
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    qf[a2][s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
-                    wf[a2][s] = frag_cols(sW, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    qf[a2][s] = frag_cols(sQ, PK, 32 * s, 16 * (NA * w + a2), lane);
+                    wf[a2][s] = frag_cols(sW, PK, 32 * s, 16 * (NA * w + a2), lane);
                 }
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
                 for (int b = 0; b < NB; ++b) dS[a2][b] *= eg;
 #pragma unroll
@@ -534,7 +546,7 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
                 for (int s = 0; s < 2; ++s) {
                     const V8 fo = frag_cols(sDOg, PV, 32 * s, 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, 16 * b, lane);
 #pragma unroll
-                    for (int a2 = 0; a2 < 2; ++a2) {
+                    for (int a2 = 0; a2 < NA; ++a2) {
                         dS[a2][b] = Mma<T>::run(fo, qf[a2][s], dS[a2][b]);
                         dS[a2][b] = Mma<T>::run(fv, wf[a2][s], dS[a2][b]);
                     }
@@ -544,34 +556,37 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
     }
     if (p.dh0) {
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+        for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const int kk = 16 * (2 * w + a2) + c16;
-                *(f32x4*)(p.dh0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
+                const int kk = 16 * (NA * w + a2) + c16;
+                *(f32x4*)(p.dh0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
             }
     }
 }
 
 // ---------------------------------------------------------------------------------------------
-// dq, dw and the first parts of dk and dgam.  Wave w owns key features 32w .. 32w+31 (two tiles a2) of all 64 tokens
-// (four tiles t): lane (c16, g) holds token 16t + c16 and features 16(2w+a2) + 4g .. +3.
+// dq, dw and the first parts of dk and dgam.  Per block kb of 128 key features wave w owns features 128kb + 32w .. + 31
+// (two tiles a2) of all 64 tokens (four tiles t): lane (c16, g) holds token 16t + c16 and features
+// 128kb + 16(2w+a2) + 4g .. +3.
 // ---------------------------------------------------------------------------------------------
-// One workgroup per CU walks over the units and fetches everything the next unit needs (five tiles and its fragments
-// of S and dS) into registers while it works on the current one.
-constexpr size_t BWD_DQKW_SMEM = (5 * 64 * P128 + 64 * P64) * 2 + 128 * 4;
+// One workgroup per CU walks over the units and fetches everything the next unit needs (five tiles and, with one block of key
+// features, its fragments of S and dS) into registers while it works on the current one.
+template <int KT> constexpr size_t bwd_dqkw_smem() { return (3 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 64 * P64) * 2 + 128 * 4; }
 
-template <typename T>
+template <typename T, int KT>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
+    constexpr int KD = BD * KT, PK = KD + 8;
     extern __shared__ __align__(16) char smem[];
-    T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sK = sDvn + 64 * P128; T* sQ = sK + 64 * P128;
-    T* sDP = sQ + 64 * P128;
+    T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sK = sDvn + 64 * P128; T* sQ = sK + 64 * PK;
+    T* sDP = sQ + 64 * PK;
     float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
-    TileRegs<BD> rDO, rVn, rDvn, rK, rQ;
+    TileRegs<BD> rDO, rVn, rDvn;
+    TileRegs<KD> rK, rQ;
     V8 rS[2][4], rdS[2][4];
     float rGam = 0.f;
     auto fetch = [&](int64_t u) {
@@ -580,103 +595,128 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         fetch_tile<BD>(rDO, (const T*)p.dout + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         fetch_tile<BD>(rVn, (const T*)p.ws.Vn + u * 64 * BD, BD, 64, tid);
         fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
-        const T* Hu = (const T*)p.ws.Hs + u * BD * BD;
-        const T* dHu = (const T*)p.ws.dHs + u * BD * BD;
+        if constexpr (KT == 1) {
+            const T* Hu = (const T*)p.ws.Hs + u * KD * BD;
+            const T* dHu = (const T*)p.ws.dHs + u * KD * BD;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int kk = 16 * (2 * w + a2) + c16;
-                rS[a2][s] = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
-                rdS[a2][s] = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
-            }
-        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+                for (int s = 0; s < 4; ++s) {
+                    const int kk = 16 * (2 * w + a2) + c16;
+                    rS[a2][s] = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
+                    rdS[a2][s] = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
+                }
+        }
+        if constexpr (KT == 1) {
+            fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+            fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        }
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
         const int hv = (int)(u % p.HV);
         const ChunkAt c = chunk_at(p, u / p.HV);
+        if constexpr (KT > 1) {                                 // (no registers to spare for fetching the wide tiles ahead)
+            const int hq = hv / (p.HV / p.H);
+            fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+            fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        }
         put_tile<BD>(sDO, P128, rDO, tid);
         put_tile<BD>(sVn, P128, rVn, tid);
         put_tile<BD>(sDvn, P128, rDvn, tid);
-        put_tile<BD>(sK, P128, rK, tid);
-        put_tile<BD>(sQ, P128, rQ, tid);
+        put_tile<KD>(sK, PK, rK, tid);
+        put_tile<KD>(sQ, PK, rQ, tid);
         if (tid < 64) { sGam[tid] = rGam; sDg[tid] = 0.f; }
         V8 sf[2][4], df[2][4];
+        if constexpr (KT == 1) {
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) { sf[a2][s] = rS[a2][s]; df[a2][s] = rdS[a2][s]; }
+                for (int s = 0; s < 4; ++s) { sf[a2][s] = rS[a2][s]; df[a2][s] = rdS[a2][s]; }
+        }
         lds_barrier();
         if (u + gridDim.x < units) fetch(u + gridDim.x);
 
-        // Operand fragments are fetched from LDS once per use across the two feature tiles of this wave.
-        f32x4 G1[2][4], dKS[2][4], dWt[2][4], dPt[4];
-        float sdot = 0.f;
+        float sdot = 0.f, dglast = 0.f;
+#pragma unroll 1
+        for (int kb = 0; kb < KT; ++kb) {                       // (a real loop: one block's accumulators at a time)
+            if (KT > 1) {
+                // (two blocks of key features: no registers to spare for fetching these ahead, they come straight from memory)
+                const T* Hu = (const T*)p.ws.Hs + u * KD * BD;
+                const T* dHu = (const T*)p.ws.dHs + u * KD * BD;
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+                for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[a2][t] = dKS[a2][t] = ZERO4;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) dPt[t] = ZERO4;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
+                    for (int s = 0; s < 4; ++s) {
+                        const int kk = BD * kb + 16 * (2 * w + a2) + c16;
+                        sf[a2][s] = *(const V8*)(Hu + kk * BD + 32 * s + 8 * g);
+                        df[a2][s] = *(const V8*)(dHu + kk * BD + 32 * s + 8 * g);
+                    }
+            }
+            // Operand fragments are fetched from LDS once per use across the two feature tiles of this wave.
+            f32x4 G1[2][4], dKS[2][4], dWt[2][4], dPt[4];
 #pragma unroll
             for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sdot += (float)sf[a2][s][e] * (float)df[a2][s][e];
-            const V8 own = frag_rows(sDO, P128, 16 * w, 32 * s, lane);        // this wave's 16 token rows of do, for dP
+                for (int t = 0; t < 4; ++t) G1[a2][t] = dWt[a2][t] = dKS[a2][t] = ZERO4;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const V8 bdo = frag_rows(sDO, P128, 16 * t, 32 * s, lane), bdv = frag_rows(sDvn, P128, 16 * t, 32 * s, lane),
-                         bvn = frag_rows(sVn, P128, 16 * t, 32 * s, lane);
+            for (int t = 0; t < 4; ++t) dPt[t] = ZERO4;
 #pragma unroll
-                for (int a2 = 0; a2 < 2; ++a2) {
-                    G1[a2][t] = Mma<T>::run(sf[a2][s], bdo, G1[a2][t]);
-                    dWt[a2][t] = Mma<T>::run(sf[a2][s], bdv, dWt[a2][t]);
-                    dKS[a2][t] = Mma<T>::run(df[a2][s], bvn, dKS[a2][t]);
-                }
-                if (t <= w) dPt[t] = Mma<T>::run(own, bvn, dPt[t]);
-            }
-        }
-        {
-            T* dWu = (T*)p.ws.dWm + u * 64 * BD;
+            for (int s = 0; s < 4; ++s) {
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+                for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    *(V4*)(dWu + (16 * t + c16) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[a2][t]);
-        }
-        // dP o D for this wave's 16 token rows, as an operand tile
-        {
-            float gi[4];
+                    for (int e = 0; e < 8; ++e) sdot += (float)sf[a2][s][e] * (float)df[a2][s][e];
+                V8 own;
+                if (kb == 0) own = frag_rows(sDO, P128, 16 * w, 32 * s, lane);      // this wave's 16 token rows of do, for dP
 #pragma unroll
-            for (int r = 0; r < 4; ++r) gi[r] = sGam[16 * w + 4 * g + r];
+                for (int t = 0; t < 4; ++t) {
+                    const V8 bdo = frag_rows(sDO, P128, 16 * t, 32 * s, lane), bdv = frag_rows(sDvn, P128, 16 * t, 32 * s, lane),
+                             bvn = frag_rows(sVn, P128, 16 * t, 32 * s, lane);
 #pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                const int j = 16 * tj + c16;
-                const float gj = sGam[j];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    sDP[i * P64 + j] = (T)(i >= j ? p.scale * dPt[tj][r] * __expf(gi[r] - gj) : 0.f);
+                    for (int a2 = 0; a2 < 2; ++a2) {
+                        G1[a2][t] = Mma<T>::run(sf[a2][s], bdo, G1[a2][t]);
+                        dWt[a2][t] = Mma<T>::run(sf[a2][s], bdv, dWt[a2][t]);
+                        dKS[a2][t] = Mma<T>::run(df[a2][s], bvn, dKS[a2][t]);
+                    }
+                    if (kb == 0 && t <= w) dPt[t] = Mma<T>::run(own, bvn, dPt[t]);
                 }
             }
-        }
-        lds_barrier();
+            {
+                T* dWu = (T*)p.ws.dWm + u * 64 * KD;
+#pragma unroll
+                for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        *(V4*)(dWu + (16 * t + c16) * KD + BD * kb + 16 * (2 * w + a2) + 4 * g) = pack4<T>(-dWt[a2][t]);
+            }
+            if (kb == 0) {
+                // dP o D for this wave's 16 token rows, as an operand tile
+                float gi[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) gi[r] = sGam[16 * w + 4 * g + r];
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj) {
+                    const int j = 16 * tj + c16;
+                    const float gj = sGam[j];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int i = 16 * w + 4 * g + r;
+                        sDP[i * P64 + j] = (T)(i >= j ? p.scale * dPt[tj][r] * __expf(gi[r] - gj) : 0.f);
+                    }
+                }
+                lds_barrier();
+            }
 
-        const float glast = sGam[63];
-        float dglast = __expf(glast) * sdot;
-        {
+            const float glast = sGam[63];
             V8 fk[2][2], fq[2][2];
 #pragma unroll
             for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    fk[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
-                    fq[a2][s] = frag_cols(sQ, P128, 32 * s, 16 * (2 * w + a2), lane);
+                    fk[a2][s] = frag_cols(sK, PK, 32 * s, BD * kb + 16 * (2 * w + a2), lane);
+                    fq[a2][s] = frag_cols(sQ, PK, 32 * s, BD * kb + 16 * (2 * w + a2), lane);
                 }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -687,11 +727,11 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
                 V4 q4[2], k4[2];
 #pragma unroll
                 for (int a2 = 0; a2 < 2; ++a2) {
-                    const int n16 = 16 * (2 * w + a2);
+                    const int n16 = BD * kb + 16 * (2 * w + a2);
                     dq[a2] = G1[a2][t] * fqs;
                     dk[a2] = dKS[a2][t] * fks;
-                    q4[a2] = *(const V4*)(sQ + x * P128 + n16 + 4 * g);
-                    k4[a2] = *(const V4*)(sK + x * P128 + n16 + 4 * g);
+                    q4[a2] = *(const V4*)(sQ + x * PK + n16 + 4 * g);
+                    k4[a2] = *(const V4*)(sK + x * PK + n16 + 4 * g);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) dglast += (float)k4[a2][r] * dk[a2][r];
                 }
@@ -718,13 +758,14 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
                 if (x < c.valid) {
 #pragma unroll
                     for (int a2 = 0; a2 < 2; ++a2) {
-                        const int n16 = 16 * (2 * w + a2);
-                        *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dq[a2]);
-                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(dk[a2]);
+                        const int n16 = BD * kb + 16 * (2 * w + a2);
+                        *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(dq[a2]);
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(dk[a2]);
                     }
                 }
             }
         }
+        dglast += __expf(sGam[63]) * sdot;
         dglast = sum_over_c16(sum_over_g(dglast));
         if (lane == 0) atomicAdd(&sDg[63], dglast);
         lds_barrier();
@@ -737,21 +778,24 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
 // One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.
-constexpr size_t BWD_WY_SMEM = (4 * 64 * P128 + 3 * 64 * P64) * 2 + 256 * 4;
+template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 256 * 4; }
 
-template <typename T>
+template <typename T, int KT>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
+    constexpr int KD = BD * KT, PK = KD + 8, NA = 2 * KT;      // NA tiles of 16 key features per wave: two in every block of 128
     extern __shared__ __align__(16) char smem[];
-    T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * P128;
-    T* sA = sK + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
+    T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * PK;
+    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
     float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 64;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    auto feat = [&](int a) { return BD * (a >> 1) + 16 * (2 * w + (a & 1)); };       // first key feature of this wave's tile a
 
-    TileRegs<BD> rDvn, rV, rDW, rK;
+    TileRegs<BD> rDvn, rV;
+    TileRegs<KD> rDW, rK;
     TileRegs<CH> rA;
-    V4 rDk[2][4];                                               // what the previous kernel left in dk, at this lane's places
+    V4 rDk[NA][4];                                               // what the previous kernel left in dk, at this lane's places
     float rGam = 0.f, rBeta = 0.f, rDg = 0.f;
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
@@ -759,20 +803,20 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
-        fetch_tile<BD>(rDW, (const T*)p.ws.dWm + u * 64 * BD, BD, 64, tid);
-        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if (tid < 64) {
             rGam = p.ws.Gam[u * 64 + tid];
             rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
             rDg = p.ws.Dgam[u * 64 + tid];
         }
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+        for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int x = 16 * t + c16;
                 rDk[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-                if (x < c.valid) rDk[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + 16 * (2 * w + a2) + 4 * g);
+                if (x < c.valid) rDk[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g);
             }
     };
     fetch(blockIdx.x);
@@ -782,12 +826,12 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<BD>(sV, P128, rV, tid);
         put_tile<CH>(sA, P64, rA, tid);
-        put_tile<BD>(sDW, P128, rDW, tid);
-        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<KD>(sDW, PK, rDW, tid);
+        put_tile<KD>(sK, PK, rK, tid);
         if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; sDg[tid] = rDg; sDb[tid] = 0.f; }
-        V4 dk_old[2][4];
+        V4 dk_old[NA][4];
 #pragma unroll
-        for (int a2 = 0; a2 < 2; ++a2)
+        for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
             for (int t = 0; t < 4; ++t) dk_old[a2][t] = rDk[a2][t];
         lds_barrier();
@@ -798,12 +842,13 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         // k k^T of the same rows and columns is formed along the way, for the last step but one
         f32x4 kkT[4];
         {
-            V8 fa[4], fw[4], fk[4];
+            V8 fa[4], fw[4 * KT], fk[4 * KT];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
-                fw[s] = frag_rows(sDW, P128, 16 * w, 32 * s, lane);
-                fk[s] = frag_rows(sK, P128, 16 * w, 32 * s, lane);
+            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int s = 0; s < 4 * KT; ++s) {
+                fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
             }
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
@@ -811,9 +856,10 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                 kkT[tj] = ZERO4;
                 if (tj <= w) {
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const V8 bk = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
-                        dXv = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
+                    for (int s = 0; s < 4; ++s) dXv = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
+#pragma unroll
+                    for (int s = 0; s < 4 * KT; ++s) {
+                        const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
                         dXw = Mma<T>::run(fw[s], bk, dXw);
                         kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
                     }
@@ -828,7 +874,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
             }
         }
         // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
-        f32x4 dk[2][4];
+        f32x4 dk[NA][4];
         {
             V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
             float ej[4], bj[4];
@@ -841,32 +887,50 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                 bj[t] = sBeta[16 * t + c16];
             }
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {
+            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
                 const int n16 = 16 * (2 * w + a2);
-                V8 fdv[2], fdw[2];
+                V8 fdv[2];
 #pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
-                    fdw[s] = frag_cols(sDW, P128, 32 * s, n16, lane);
-                }
+                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    f32x4 av = ZERO4, ak = ZERO4;
+                    f32x4 av = ZERO4;
 #pragma unroll
                     for (int s = 0; s < 2; ++s) {
                         if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
                         av = Mma<T>::run(fdv[s], fA[t][s], av);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
+                    float dbv = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
+                    dbv = sum_over_g(dbv);
+                    if (g == 0) atomicAdd(&sDb[j], dbv);
+                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                }
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
+                const int n16 = feat(a2);
+                V8 fdw[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 ak = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;
                         ak = Mma<T>::run(fdw[s], fA[t][s], ak);
                     }
                     const int j = 16 * t + c16;
-                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g), k4 = *(const V4*)(sK + j * P128 + n16 + 4 * g);
-                    float dbv = 0.f, dot = 0.f;
+                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
+                    float dot = 0.f;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) { dbv += av[r] * (float)v4[r]; dot += ak[r] * (float)k4[r]; }
-                    dbv = sum_over_g(dbv);
+                    for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
                     dot = sum_over_g(dot);
-                    if (g == 0) { atomicAdd(&sDb[j], dbv + ej[t] * dot); atomicAdd(&sDg[j], bj[t] * ej[t] * dot); }
-                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                    if (g == 0) { atomicAdd(&sDb[j], ej[t] * dot); atomicAdd(&sDg[j], bj[t] * ej[t] * dot); }
                     dk[a2][t] = ak * (bj[t] * ej[t]);
                 }
             }
@@ -933,11 +997,11 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         lds_barrier();
         // dk += E k + E^T k, on top of what the previous kernel left
         {
-            V8 fk[2][2];
+            V8 fk[NA][2];
 #pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2)
+            for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
-                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, P128, 32 * s, 16 * (2 * w + a2), lane);
+                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -945,22 +1009,22 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
                         const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
 #pragma unroll
-                        for (int a2 = 0; a2 < 2; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
                     }
                     if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
                         const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
 #pragma unroll
-                        for (int a2 = 0; a2 < 2; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
                     }
                 }
                 const int x = 16 * t + c16;
                 if (x < c.valid) {
 #pragma unroll
-                    for (int a2 = 0; a2 < 2; ++a2) {
+                    for (int a2 = 0; a2 < NA; ++a2) {
                         f32x4 acc = dk[a2][t];
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
-                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + 16 * (2 * w + a2) + 4 * g) = pack4<T>(acc);
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
                     }
                 }
             }
@@ -981,36 +1045,36 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     }
 }
 
-template <typename T, int VBT>
-static void scan_kernels(const void** state, const void** dstate, size_t* smem_state, size_t* smem_dstate) {
-    *state = (const void*)gdn_bwd_state_kernel<T, VBT>; *dstate = (const void*)gdn_bwd_dstate_kernel<T, VBT>;
-    *smem_state = bwd_state_smem<VBT>(); *smem_dstate = bwd_dstate_smem<VBT>();
-}
-
-template <typename T>
+template <typename T, int KT>
 static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream) {
     // Value columns per workgroup of the scans: as few as it takes to give every (sequence, head) run its own CU
-    // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.
+    // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.  With two
+    // blocks of key features the reverse scan's tiles leave room for 32 columns only.
     const int64_t runs1 = p.N * p.HV;
     const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
-    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)((runs1 + 7) / 8 * 8 * (BD / vbt));
-    static SmemAttrDone done[3][5];
-    const void *state, *dstate;
-    size_t smem_state, smem_dstate;
-    if (vbt == 32) scan_kernels<T, 32>(&state, &dstate, &smem_state, &smem_dstate);
-    else if (vbt == 64) scan_kernels<T, 64>(&state, &dstate, &smem_state, &smem_dstate);
-    else scan_kernels<T, 128>(&state, &dstate, &smem_state, &smem_dstate);
+    const int vbt_d = KT == 1 ? vbt : 32;
+    const unsigned units = (unsigned)(num_chunks * p.HV);
+    auto runs = [&](int v) { return (unsigned)((runs1 + 7) / 8 * 8 * (BD / v)); };
     struct K { const void* f; size_t smem; const char* name; unsigned grid; };
+    K state, dstate;
+    if (vbt == 32) state = {(const void*)gdn_bwd_state_kernel<T, 32, KT>, bwd_state_smem<32, KT>(), "gdn_bwd_state_kernel", runs(32)};
+    else if (vbt == 64) state = {(const void*)gdn_bwd_state_kernel<T, 64, KT>, bwd_state_smem<64, KT>(), "gdn_bwd_state_kernel", runs(64)};
+    else state = {(const void*)gdn_bwd_state_kernel<T, 128, KT>, bwd_state_smem<128, KT>(), "gdn_bwd_state_kernel", runs(128)};
+    if (vbt_d == 32) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 32, KT>, bwd_dstate_smem<32, KT>(), "gdn_bwd_dstate_kernel", runs(32)};
+    else if constexpr (KT == 1) {
+        if (vbt_d == 64) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, KT>, bwd_dstate_smem<64, KT>(), "gdn_bwd_dstate_kernel", runs(64)};
+        else dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, KT>, bwd_dstate_smem<128, KT>(), "gdn_bwd_dstate_kernel", runs(128)};
+    }
     const K ks[5] = {
-        {(const void*)gdn_bwd_prepare_kernel<T>, BWD_PREP_SMEM, "gdn_bwd_prepare_kernel", units < 512u ? units : 512u},
-        {state, smem_state, "gdn_bwd_state_kernel", runs},
-        {dstate, smem_dstate, "gdn_bwd_dstate_kernel", runs},
-        {(const void*)gdn_bwd_dqkw_kernel<T>, BWD_DQKW_SMEM, "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
-        {(const void*)gdn_bwd_wy_kernel<T>, BWD_WY_SMEM, "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
+        {(const void*)gdn_bwd_prepare_kernel<T, KT>, bwd_prep_smem<KT>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
+        state,
+        dstate,
+        {(const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
+        {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
-    const int vi = vbt == 32 ? 0 : vbt == 64 ? 1 : 2;
     for (int i = 0; i < 5; ++i) {
-        if (int rc = ensure_dynamic_smem(ks[i].f, ks[i].smem, done[vi][i], ks[i].name)) return rc;
+        // (the limit on dynamic LDS belongs to the function: asked for on every call, it is a cheap host-side setting)
+        if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
         int64_t nunits = units;
         void* args[] = {(void*)&p, (void*)&nunits};             // (the kernels that walk over the units take their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
@@ -1021,9 +1085,9 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
 
 }  // namespace gdn
 
-extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV) {
-    if (num_chunks < 0 || HV < 1) return 0;
-    return gdn::bwd_ws_layout(num_chunks * HV, nullptr, nullptr);
+extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t K) {
+    if (num_chunks < 0 || HV < 1 || (K != 128 && K != 256)) return 0;
+    return gdn::bwd_ws_layout(num_chunks * HV, K, nullptr, nullptr);
 }
 
 extern "C" int gdn_chunk_bwd(
@@ -1039,8 +1103,8 @@ extern "C" int gdn_chunk_bwd(
     const char* who = "gdn_chunk_bwd";
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
-    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
-                  who, (long long)K, (long long)V);
+    GDN_CHECK_ARG((K == BD || K == 2 * BD) && V == BD, GDN_ERR_UNSUPPORTED,
+                  "%s: K = 128 or 256 and V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros", who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
     GDN_CHECK_ARG((flags & ~(uint32_t)(GDN_FLAG_CU_INT32 | (7u << 27))) == 0, GDN_ERR_UNSUPPORTED,
                   "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
@@ -1064,7 +1128,7 @@ extern "C" int gdn_chunk_bwd(
         GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
     GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
     BwdParams p;
-    const size_t need = bwd_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
+    const size_t need = bwd_ws_layout(num_chunks * HV, K, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
@@ -1072,5 +1136,6 @@ extern "C" int gdn_chunk_bwd(
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
-    return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t>(p, num_chunks, s) : launch_bwd<f16_t>(p, num_chunks, s);
+    if (K == BD) return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 1>(p, num_chunks, s) : launch_bwd<f16_t, 1>(p, num_chunks, s);
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 2>(p, num_chunks, s) : launch_bwd<f16_t, 2>(p, num_chunks, s);
 }

@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -88,7 +88,7 @@ for _name in ('gdn_chunk_fwd', 'gdn_chunk_fwd_prepare', 'gdn_chunk_fwd_scan'):
     SIGNATURES[_name] = (c_int, _CHUNK_ARGS)
 
 SIGNATURES['gdn_chunk_fwd_static'] = (c_int, _CHUNK_ARGS[:13] + _CHUNK_ARGS[15:])     # no workspace, no size
-SIGNATURES['gdn_chunk_bwd_workspace_bytes'] = (c_size_t, [c_int64, c_int64])
+SIGNATURES['gdn_chunk_bwd_workspace_bytes'] = (c_size_t, [c_int64, c_int64, c_int64])
 SIGNATURES['gdn_chunk_bwd'] = (c_int, [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k v g beta
     c_void_p, c_void_p, c_void_p,                      # h0 dout dht

@@ -14,7 +14,7 @@ from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, current_stre
 from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
-_DIM = 128          # head dims of the backward kernels; smaller ones are zero-padded
+_DIM = 128          # value columns of the backward kernels; key features: 128 or 256 (other head dims are zero-padded)
 
 
 def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
@@ -47,8 +47,9 @@ def chunk_gated_delta_rule_bwd(
     dev = require_gpu(q, k, v, beta, do)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
-    if K > _DIM:
-        raise NotImplementedError(f'the backward kernels cover head dims up to {_DIM} (got K={K})')
+    if K > 2 * _DIM:
+        raise NotImplementedError(f'the backward kernels cover key head dims up to {2 * _DIM} (got K={K})')
+    KD = _DIM if K <= _DIM else 2 * _DIM
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     nb = (V + _DIM - 1) // _DIM
     if nb > 1:
@@ -82,7 +83,7 @@ def chunk_gated_delta_rule_bwd(
 
     out_dtype = q.dtype
     work = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
-    qw, kw = (aligned16(_pad_last(x.to(work), _DIM).contiguous()) for x in (q, k))
+    qw, kw = (aligned16(_pad_last(x.to(work), KD).contiguous()) for x in (q, k))
     vw, dow = (aligned16(_pad_last(x.to(work), _DIM).contiguous()) for x in (v, do))
     gw = None if g is None else as_f32(g).contiguous()
     bw = as_f32(beta).contiguous()
@@ -93,7 +94,7 @@ def chunk_gated_delta_rule_bwd(
         s = as_f32(s)
         if state_v_first:
             s = s.transpose(-1, -2)
-        return aligned16(F.pad(s, (0, _DIM - V, 0, _DIM - K)).contiguous())
+        return aligned16(F.pad(s, (0, _DIM - V, 0, KD - K)).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
     flags = 0
@@ -113,20 +114,20 @@ def chunk_gated_delta_rule_bwd(
         num_chunks = B * ((T + _CHUNK - 1) // _CHUNK)
 
     # rows past a sequence's end inside its last chunk are never written: start from zeros only where that matters
-    dq = torch.empty(B, T, HV, _DIM, dtype=work, device=dev)
-    dk = torch.empty(B, T, HV, _DIM, dtype=work, device=dev)
+    dq = torch.empty(B, T, HV, KD, dtype=work, device=dev)
+    dk = torch.empty(B, T, HV, KD, dtype=work, device=dev)
     dv = torch.empty(B, T, HV, _DIM, dtype=work, device=dev)
     dg = torch.empty(B, T, HV, dtype=torch.float32, device=dev)
     db = torch.empty(B, T, HV, dtype=torch.float32, device=dev)
-    dh0 = torch.empty(N, HV, _DIM, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
+    dh0 = torch.empty(N, HV, KD, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
     lib = _lib.load()
-    ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV)
+    ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, KD)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     _lib.check(lib.gdn_chunk_bwd(
         ptr(qw), ptr(kw), ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
         ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
         ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
-        B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
+        B, T, H, HV, KD, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
         current_stream_ptr(dev)))
     dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
     dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
@@ -138,8 +139,8 @@ def chunk_gated_delta_rule_bwd(
 
 
 def _finish(lib, dxh: torch.Tensor, y: torch.Tensor, rstd: torch.Tensor | None, H: int, K: int, out_dtype) -> torch.Tensor:
-    """dq or dk per value head ``[B,T,HV,128]`` -> per q/k head ``[B,T,H,K]``: the sum over the value heads of a
-    q/k head and, with ``rstd``, the way back through the l2 normalisation (``y``: the normalised rows, 128 wide)."""
+    """dq or dk per value head ``[B,T,HV,KD]`` -> per q/k head ``[B,T,H,K]``: the sum over the value heads of a
+    q/k head and, with ``rstd``, the way back through the l2 normalisation (``y``: the normalised rows, KD wide)."""
     B, T, HV, D = dxh.shape
     if rstd is None and HV == H and K == D:
         return dxh.to(out_dtype)

@@ -41,9 +41,6 @@ def make_backends(BaseBackend):
                 return False, 'not a gfx950 device'
             if cp_context is not None:
                 return False, 'context parallelism is not supported'
-            if k.shape[-1] > 128 and _needs_grad(q, k, v, g, beta, kwargs.get('initial_state'), kwargs.get('A_log'),
-                                                  kwargs.get('dt_bias')):
-                return False, 'the backward kernels cover key head dims up to 128: a tensor requires grad'
             if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
                 return False, f'dtype {q.dtype}'
             if k.shape[-1] > 256:

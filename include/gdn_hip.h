@@ -219,11 +219,12 @@ int gdn_chunk_fwd_scan(
  *   dq, dk [B,T,HV,K], dv [B,T,HV,V] in qkv_dtype: per VALUE head; with grouped heads the caller adds the HV/H
  *   gradients that belong to one q/k head; dg, dbeta [B,T,HV] fp32; dh0 [N,HV,K,V] fp32 or NULL
  *   cu_seqlens, chunk_table, chunk_offsets ([N+1] here), N, num_chunks: as for gdn_chunk_fwd
- *   workspace: at least gdn_chunk_bwd_workspace_bytes(num_chunks, HV) bytes, 256-byte aligned
- *   flags: GDN_FLAG_CU_INT32 only.  K = V = 128 only: the Python host zero-pads smaller head dims.
+ *   workspace: at least gdn_chunk_bwd_workspace_bytes(num_chunks, HV, K) bytes (0: unsupported K), 256-byte aligned
+ *   flags: GDN_FLAG_CU_INT32 only.  K = 128 or 256 (the reference's limit, fla/ops/common/chunk_delta_h.py:712) and V = 128 only: the Python host
+ *   zero-pads other head dims and splits V > 128 into value heads of 128 columns.
  *   T == 0: dh0 = dht (zeros without dht), nothing else is written.
  */
-size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV);
+size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t K);
 int gdn_chunk_bwd(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,

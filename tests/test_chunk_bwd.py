@@ -194,6 +194,37 @@ def test_chunk_backward_packed(H, HV, D, mask_p, cu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,K,V,l2,cu', [
+    (2, 200, 2, 4, 256, 128, True, None),
+    (1, 130, 2, 2, 256, 256, False, None),
+    (1, 300, 1, 2, 192, 128, True, None),
+    (1, 257, 2, 2, 256, 512, True, None),                  # the reference layer's default head shape (head_dim 256, expand_v 2)
+    (1, 0, 2, 4, 160, 64, False, [0, 100, 101, 300]),
+    (3, 100, 12, 24, 256, 128, True, None),                 # 72 runs: the forward scan takes 64 columns per workgroup
+])
+def test_chunk_backward_wide_keys(B, T, H, HV, K, V, l2, cu):
+    """Key head dims above 128 (two blocks of 128 key features in every backward kernel)."""
+    if cu is not None:
+        T = cu[-1]
+    N = B if cu is None else len(cu) - 1
+    gen = torch.Generator().manual_seed(5)
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    if not l2:
+        q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
+    q, k = q.bfloat16(), k.bfloat16()
+    v = torch.randn(B, T, HV, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / 4
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    h0 = torch.randn(N, HV, K, V, generator=gen) * 0.3
+    do = torch.randn(B, T, HV, V, generator=gen).bfloat16()
+    dht = torch.randn(N, HV, K, V, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, use_qk_l2norm_in_kernel=l2,
+                                   dtype=torch.float32)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu, use_qk_l2norm_in_kernel=l2)
+    _compare(ref, got)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize('what', ['beta_sigmoid', 'beta_sigmoid_neg', 'gate', 'gate_no_bias', 'v_first', 'no_h0', 'no_dht',
                                   'wide_v', 'fp32'])
 def test_chunk_backward_options(what):
@@ -283,15 +314,16 @@ def test_chunk_backward_random(seed):
 def test_chunk_backward_c_entry_checks():
     from fla_hip import _lib
     lib = _lib.load()
-    assert lib.gdn_chunk_bwd_workspace_bytes(4, 2) > 0
+    assert lib.gdn_chunk_bwd_workspace_bytes(4, 2, 128) > 0 and lib.gdn_chunk_bwd_workspace_bytes(4, 2, 256) > lib.gdn_chunk_bwd_workspace_bytes(4, 2, 128)
+    assert lib.gdn_chunk_bwd_workspace_bytes(4, 2, 192) == 0
     x = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16, device='cuda')
     f = torch.zeros(1, 64, 1, device='cuda')
-    ws = torch.zeros(lib.gdn_chunk_bwd_workspace_bytes(1, 1), dtype=torch.uint8, device='cuda')
+    ws = torch.zeros(lib.gdn_chunk_bwd_workspace_bytes(1, 1, 128), dtype=torch.uint8, device='cuda')
     args = [x.data_ptr()] * 3 + [f.data_ptr()] * 2 + [None, x.data_ptr(), None] + [x.data_ptr()] * 3 + [f.data_ptr()] * 2 + [None]
     rc = lib.gdn_chunk_bwd(*args, None, None, None, ws.data_ptr(), ws.numel(), 1, 64, 1, 1, 64, 64, 1, 1, 1.0,
                            _lib.DTYPE_BF16, _lib.DTYPE_F32, 0, None)
-    assert rc == _lib.GDN_ERR_UNSUPPORTED and 'K = V = 128' in _lib.last_error()
+    assert rc == _lib.GDN_ERR_UNSUPPORTED and 'K = 128 or 256' in _lib.last_error()
     with pytest.raises(NotImplementedError):
         from fla_hip.ops.gated_delta_rule.chunk_bwd import chunk_gated_delta_rule_bwd
-        w = torch.zeros(1, 64, 1, 256, dtype=torch.bfloat16, device='cuda')
+        w = torch.zeros(1, 64, 1, 264, dtype=torch.bfloat16, device='cuda')
         chunk_gated_delta_rule_bwd(w, w, w, f, f, 1.0, None, w, None)

@@ -338,10 +338,8 @@ def test_upstream_backends_take_gpu_inference_calls_and_leave_the_rest():
     dq, dk, dv, dg, db = (t.cuda() for t in (q, k, v, g, beta))
     o, ht = chunk_gated_delta_rule(dq, dk, dv, dg, db, output_final_state=False)
     assert isinstance(o, torch.Tensor) and ht is None and O.get_err_ratio(ref, o.float().cpu()) < 5e-3
-    o_t = chunk_gated_delta_rule(dq.requires_grad_(), dk, dv, dg, db)[0]                          # training: key head dims up to 128
+    o_t = chunk_gated_delta_rule(dq.requires_grad_(), dk, dv, dg, db)[0]                          # training goes through the backward kernels
     assert isinstance(o_t, torch.Tensor) and o_t.requires_grad
-    wide = torch.zeros(1, 130, 2, 192, device='cuda', dtype=torch.bfloat16)
-    assert chunk_gated_delta_rule(wide.requires_grad_(), wide, dv, dg, db)[0] == 'default'        # ... wider keys stay upstream
     assert chunk_gated_delta_rule(q, k, v, g, beta)[0] == 'default'                               # CPU stays upstream
     with torch.no_grad():
         assert isinstance(chunk_gated_delta_rule(dq, dk, dv, dg, db)[0], torch.Tensor)
