@@ -538,11 +538,10 @@ def main():
             extra[name] = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), tokens_per_s=round(r['value'], 1),
                                call_ms_quantiles=r['call_ms_quantiles'], roofline=r['roofline'])
             torch.cuda.empty_cache()
-        # training step (forward + backward) on the published shapes the backward kernels cover (head dims up to 128)
+        # training step (forward + backward) on the same shapes
         for name, ww in PUBLISHED.items():
-            if ww.get('K', 128) <= 128 and ww.get('V', 128) <= 128:
-                extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
-                torch.cuda.empty_cache()
+            extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
+            torch.cuda.empty_cache()
         line['other_workloads'] = extra
     print(json.dumps(line))
 

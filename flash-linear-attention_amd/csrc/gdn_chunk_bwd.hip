@@ -1,4 +1,4 @@
-// Backward pass of the chunked gated delta rule (gfx950, 64-token chunks, K = V = 128; the host pads smaller head dims).
+// Backward pass of the chunked gated delta rule (gfx950, 64-token chunks, 128 or 256 key features, 128 value columns; the host pads other head dims).
 // Replaces the reference's backward pipeline fla/ops/gated_delta_rule/chunk.py:125-257 (recompute_w_u_fwd,
 // chunk_gated_delta_rule_fwd_h, chunk_bwd_dv_local, chunk_gated_delta_rule_bwd_dhu, chunk_bwd_dqkwg, prepare_wy_repr_bwd,
 // reverse chunk_local_cumsum) by five kernels:
@@ -312,9 +312,9 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 }
 
 // ---------------------------------------------------------------------------------------------
-// The two scans.  A workgroup owns VBT value columns of one (sequence, v-head): the state slice [128][VBT] lives in
-// registers as transposed tiles - wave w holds key rows 32w .. 32w+31 as two tiles (a2), lane (c16, g) key
-// 16(2w+a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
+// The two scans.  A workgroup owns VBT value columns of one (sequence, v-head): the state slice [KD][VBT] lives in
+// registers as transposed tiles - wave w holds key rows KD/4 w .. as NA = KD/64 tiles (a2), lane (c16, g) key
+// 16(NA w + a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
 // current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
 template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
