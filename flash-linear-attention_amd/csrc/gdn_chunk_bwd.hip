@@ -572,7 +572,7 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
 // ---------------------------------------------------------------------------------------------
 // One workgroup per CU walks over the units and fetches everything the next unit needs (five tiles and, with one block of key
 // features, its fragments of S and dS) into registers while it works on the current one.
-template <int KT> constexpr size_t bwd_dqkw_smem() { return (3 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 64 * P64) * 2 + 128 * 4; }
+template <int KT> constexpr size_t bwd_dqkw_smem() { return (3 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 64 * P64) * 2 + 320 * 4; }
 
 template <typename T, int KT>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64_t units) {
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
     extern __shared__ __align__(16) char smem[];
     T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sK = sDvn + 64 * P128; T* sQ = sK + 64 * PK;
     T* sDP = sQ + 64 * PK;
-    float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;
+    float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;    // sDg [4][64]: a row per wave, added up in a fixed order (same bits every run)
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
     TileRegs<BD> rDO, rVn, rDvn;
@@ -627,7 +627,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
-        if (tid < 64) { sGam[tid] = rGam; sDg[tid] = 0.f; }
+        if (tid < 64) sGam[tid] = rGam;
+        sDg[tid] = 0.f;
         V8 sf[2][4], df[2][4];
         if constexpr (KT == 1) {
 #pragma unroll
@@ -754,7 +755,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 #pragma unroll
                     for (int r = 0; r < 4; ++r) dgx += (float)q4[a2][r] * dq[a2][r] - (float)k4[a2][r] * dk[a2][r];
                 dgx = sum_over_g(dgx);
-                if (g == 0) atomicAdd(&sDg[x], dgx);
+                if (g == 0) atomicAdd(&sDg[64 * w + x], dgx);
                 if (x < c.valid) {
 #pragma unroll
                     for (int a2 = 0; a2 < 2; ++a2) {
@@ -767,9 +768,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         }
         dglast += __expf(sGam[63]) * sdot;
         dglast = sum_over_c16(sum_over_g(dglast));
-        if (lane == 0) atomicAdd(&sDg[63], dglast);
+        if (lane == 0) atomicAdd(&sDg[64 * w + 63], dglast);
         lds_barrier();
-        if (tid < 64) p.ws.Dgam[u * 64 + tid] = sDg[tid];
+        if (tid < 64) p.ws.Dgam[u * 64 + tid] = (sDg[tid] + sDg[64 + tid]) + (sDg[128 + tid] + sDg[192 + tid]);
         lds_barrier();
     }
 }
@@ -778,7 +779,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
 // One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.
-template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 256 * 4; }
+template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 640 * 4; }
 
 template <typename T, int KT>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
@@ -788,7 +789,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     extern __shared__ __align__(16) char smem[];
     T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * PK;
     T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
-    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 64;
+    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    // (sDg, sDb [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     auto feat = [&](int a) { return BD * (a >> 1) + 16 * (2 * w + (a & 1)); };       // first key feature of this wave's tile a
 
@@ -828,7 +830,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         put_tile<CH>(sA, P64, rA, tid);
         put_tile<KD>(sDW, PK, rDW, tid);
         put_tile<KD>(sK, PK, rK, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; sDg[tid] = rDg; sDb[tid] = 0.f; }
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; }
+        sDg[tid] = tid < 64 ? rDg : 0.f;
+        sDb[tid] = 0.f;
         V4 dk_old[NA][4];
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -906,7 +910,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                     for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
                     dbv = sum_over_g(dbv);
-                    if (g == 0) atomicAdd(&sDb[j], dbv);
+                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
                     if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
                 }
             }
@@ -930,7 +934,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                     for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
                     dot = sum_over_g(dot);
-                    if (g == 0) { atomicAdd(&sDb[j], ej[t] * dot); atomicAdd(&sDg[j], bj[t] * ej[t] * dot); }
+                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
                     dk[a2][t] = ak * (bj[t] * ej[t]);
                 }
             }
@@ -986,12 +990,12 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     sM1[i * P64 + l] = (T)E;
                 }
                 colF = sum_over_g(colF);
-                if (g == 0 && tl <= w) atomicAdd(&sDg[l], -colF);
+                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
-                if (c16 == 0) { atomicAdd(&sDb[16 * w + 4 * g + r], a); atomicAdd(&sDg[16 * w + 4 * g + r], b); }
+                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
             }
         }
         lds_barrier();
@@ -1030,7 +1034,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
             }
         }
         if (w == 0) {
-            float x = sDg[lane];
+            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
                 const float y = __shfl_down(x, off, 64);
@@ -1038,7 +1042,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
             }
             if (lane < c.valid) {
                 p.dg[(c.tok0 + lane) * p.HV + hv] = x;
-                p.dbeta[(c.tok0 + lane) * p.HV + hv] = sDb[lane];
+                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
             }
         }
         lds_barrier();

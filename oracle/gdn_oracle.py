@@ -20,6 +20,9 @@ reference checkout):
 * ``fla/utils/_testing.py:19-41``                error metric
 * ``fla/ops/kda/naive.py:12-66``, ``fla/ops/kda/gate.py:27-94``, ``fla/ops/kda/fused_recurrent.py:150-181``
   the KDA operator's token recurrence (a decay per key feature) and its gate activations
+* ``fla/ops/gated_delta_rule/chunk.py:125-257``, ``fla/ops/common/chunk_delta_h.py:369-560``, ``fla/ops/common/chunk_o.py:172-357``,
+  ``fla/ops/gated_delta_rule/wy_fast.py:123-296``  the chunked backward pass, stage by stage (``chunk_backward_one_sequence``);
+  the gradients themselves are reverse-mode differentiation of the token recurrence (``gated_delta_rule_grads``)
 
 Parity pins (all in ``tests/test_oracle.py``): scalar brute force written as
 independent pure-python loops on tiny shapes, closed forms for one decode step
@@ -30,6 +33,8 @@ fixtures under ``tests/golden/`` (a second set of scalar fixtures pins the
 optional arguments gk, gv, beta per value column and the pooled states of
 speculative decoding).  The KDA recurrence is the gk branch of the token recurrence (pinned by those
 fixtures); its gate activations are pinned by values that the formulas fix (``test_kda_gate_pins``).
+The gradients (``gated_delta_rule_grads``) are pinned by central finite differences of the recurrence in fp64 for every input
+and every prologue, and the stage-by-stage backward agrees with them to 1e-12 (``tests/test_chunk_bwd.py``).
 No function here is "parity unpinned".
 
 Everything is computed in ``dtype`` (float32 by default, float64 for tight

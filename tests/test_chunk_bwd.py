@@ -311,6 +311,69 @@ def test_chunk_backward_random(seed):
 
 
 @pytest.mark.gpu
+def test_chunk_backward_empty_sequences_and_no_tokens():
+    """Packed input with sequences of length zero: their dh0 is their dht, nobody else's gradient moves."""
+    H, D = 2, 128
+    cu = [0, 0, 70, 70, 134]
+    T, N = cu[-1], len(cu) - 1
+    gen = torch.Generator().manual_seed(3)
+    q, k, v, g, beta, _ = O.make_inputs(1, T, H, H, D, D, seed=3, gate_div=4.0, dtype=torch.bfloat16)
+    h0 = torch.randn(N, H, D, D, generator=gen) * 0.3
+    do = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(N, H, D, D, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, dtype=torch.float32)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu)
+    _compare(ref, got)
+    assert torch.equal(got['dh0'][0].cpu(), dht[0]) and torch.equal(got['dh0'][2].cpu(), dht[2])
+    # no token at all
+    e = torch.zeros(1, 0, H, D, dtype=torch.bfloat16)
+    z = torch.zeros(1, 0, H)
+    o, ht, got = _grads_gpu(e, e, e, z, z, h0[:1], e, dht[:1])
+    assert o.shape == (1, 0, H, D) and torch.equal(got['dh0'].cpu(), dht[:1]) and got['dq'].shape == e.shape
+
+
+@pytest.mark.gpu
+def test_chunk_backward_full_size_properties():
+    """At the size of a published shape (B=1 T=8192 H=32 of 96, D=128) the CPU oracle is out of reach; what the algebra fixes is not:
+    two runs give the same bits, gradients are linear in (do, dht) - doubling both doubles every gradient bit for bit - and a sequence cut in two,
+    chained through the state forward and through its gradient backward, gives the gradients of the whole."""
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    dev = 'cuda'
+    B, T, H, D = 1, 8192, 32, 128
+    gen = torch.Generator().manual_seed(9)
+    q = F.normalize(torch.randn(B, T, H, D, generator=gen), dim=-1).bfloat16().to(dev)
+    k = F.normalize(torch.randn(B, T, H, D, generator=gen), dim=-1).bfloat16().to(dev)
+    v = torch.randn(B, T, H, D, generator=gen).bfloat16().to(dev)
+    g = (F.logsigmoid(torch.randn(B, T, H, generator=gen)) / 4).to(dev)
+    beta = torch.rand(B, T, H, generator=gen).sigmoid().to(dev)
+    h0 = (torch.randn(B, H, D, D, generator=gen) * 0.3).to(dev)
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16().to(dev)
+    dht = torch.randn(B, H, D, D, generator=gen).to(dev)
+
+    def grads(sl, h_in, do_, dht_):
+        xs = [x[:, sl].detach().clone().requires_grad_(True) for x in (q, k, v, g, beta)] + [h_in.detach().clone().requires_grad_(True)]
+        o, ht = chunk_gated_delta_rule(*xs[:5], initial_state=xs[5], output_final_state=True)
+        ((o.float() * do_[:, sl].float()).sum() + (ht * dht_).sum()).backward()
+        return [x.grad for x in xs], ht.detach()
+
+    whole, _ = grads(slice(0, T), h0, do, dht)
+    again, _ = grads(slice(0, T), h0, do, dht)
+    twice, _ = grads(slice(0, T), h0, do * 2, dht * 2)
+    for name, a, b, c in zip(('dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0'), whole, twice, again):
+        assert torch.equal(a, c), f'{name}: two runs differ'
+        assert torch.equal((a.float() * 2).to(a.dtype), b), f'{name}: not linear in (do, dht)'
+    cut = 4096 + 64 * 3
+    _, h_mid = grads(slice(0, cut), h0, do, torch.zeros_like(dht))
+    second, _ = grads(slice(cut, T), h_mid, do, dht)
+    first, _ = grads(slice(0, cut), h0, do, second[5])
+    for i, name in enumerate(('dq', 'dk', 'dv', 'dg', 'dbeta')):
+        joined = torch.cat([first[i], second[i]], dim=1)
+        r = O.get_err_ratio(whole[i].float().cpu(), joined.float().cpu())
+        assert r < 4e-3, f'{name}: {r:.3e}'
+    assert O.get_err_ratio(whole[5].cpu(), first[5].cpu()) < 4e-3
+
+
+@pytest.mark.gpu
 def test_chunk_backward_c_entry_checks():
     from fla_hip import _lib
     lib = _lib.load()
