@@ -106,25 +106,31 @@ __device__ __forceinline__ void load_tile(T* s, int pitch, const T* g, int64_t s
 
 // The same in two halves, for loops that fetch the next tile while they work on the current one.
 template <int NCOLS>
-struct TileRegs { u32x4 x[(64 * (NCOLS / 8) + 255) / 256]; };
+struct TileRegs { u32x4 x[64 * (NCOLS / 8) / 256]; };
 template <int NCOLS, typename T>
 __device__ __forceinline__ void fetch_tile(TileRegs<NCOLS>& r, const T* g, int64_t stride, int valid, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL / 256, RPI = 256 / PPR;      // a thread's pieces lie RPI rows apart
+    static_assert(TOTAL % 256 == 0, "whole rounds of 256 threads");
+    const int row0 = tid / PPR, pc = tid % PPR;
+    const char* at = (const char*)(g + (int64_t)row0 * stride + pc * 8);
+    const int64_t step = (int64_t)RPI * stride * (int64_t)sizeof(T);
+    if (valid >= 64) {                                          // (the same for the whole workgroup) full chunk: plain loads
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        r.x[i] = u32x4{0u, 0u, 0u, 0u};
-        if (idx < TOTAL && row < valid) r.x[i] = *(const u32x4*)(g + row * stride + pc * 8);
+        for (int i = 0; i < N; ++i) r.x[i] = *(const u32x4*)(at + i * step);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            r.x[i] = u32x4{0u, 0u, 0u, 0u};
+            if (row0 + RPI * i < valid) r.x[i] = *(const u32x4*)(at + i * step);
+        }
     }
 }
 template <int NCOLS, typename T>
 __device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS>& r, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
+    constexpr int PPR = NCOLS / 8, N = 64 * PPR / 256, RPI = 256 / PPR;
+    T* at = s + (tid / PPR) * pitch + (tid % PPR) * 8;
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = r.x[i];
-    }
+    for (int i = 0; i < N; ++i) *(u32x4*)(at + i * RPI * pitch) = r.x[i];
 }
 // operand fragment whose contraction runs along a row: index r0 + c16, contraction c0 + 8g + e
 template <typename T>
@@ -320,15 +326,14 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
 template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
-template <typename T, int VBT, int KT>
-__global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
+template <typename T, int VBT, int KT, int AHEAD>
+__device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
-    extern __shared__ __align__(16) char smem[];
     T* sW = (T*)smem; T* sK = sW + 64 * PK; T* sS = sK + 64 * PK; T* sVn = sS + KD * PV;
     float* sGam = (float*)(sVn + 64 * PV);
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
     const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
@@ -346,10 +351,13 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
             const int kk = 16 * (NA * w + a2) + c16;
             S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    TileRegs<KD> rW, rK;
-    V4 rU[NB];
-    float rGam = 0.f;
-    auto fetch = [&](int64_t ic) {
+    // two sets of registers take turns: the tiles of chunk c + 2 are requested while chunk c is worked on (one chunk of
+    // lead does not cover the way to memory and back: a step would then last as long as that way)
+    struct Ahead { TileRegs<KD> rW, rK; V4 rU[NB]; float rGam; };
+    Ahead RA, RB;
+    RA.rGam = RB.rGam = 0.f;
+    auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
+        auto& rW = R.rW; auto& rK = R.rK; auto& rU = R.rU; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
         fetch_tile<KD>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
@@ -358,8 +366,8 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
     };
-    if (sq.nc > 0) fetch(0);
-    for (int64_t ic = 0; ic < sq.nc; ++ic) {
+    auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
+        auto& rW = R.rW; auto& rK = R.rK; auto& rU = R.rU; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
         put_tile<KD>(sW, PK, rW, tid);
         put_tile<KD>(sK, PK, rK, tid);
@@ -378,7 +386,7 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
                 *(V4*)(Hu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
-        if (ic + 1 < sq.nc) fetch(ic + 1);
+        if (ic + AHEAD < sq.nc) fetch(R, ic + AHEAD);
         const float glast = sGam[63];
         {
             // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
@@ -425,19 +433,34 @@ __global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
                 }
         }
         lds_barrier();
+    };
+    if (sq.nc > 0) fetch(RA, 0);
+    if constexpr (AHEAD == 1) {
+        for (int64_t ic = 0; ic < sq.nc; ++ic) step(RA, ic);
+    } else {
+        if (sq.nc > 1) fetch(RB, 1);
+        for (int64_t ic = 0; ic < sq.nc; ic += 2) {
+            step(RA, ic);
+            if (ic + 1 < sq.nc) step(RB, ic + 1);
+        }
     }
 }
 
 template <typename T, int VBT, int KT>
-__global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
+    extern __shared__ __align__(16) char smem[];
+    bwd_state_body<T, VBT, KT, 2>(p, smem, threadIdx.x);
+}
+
+template <typename T, int VBT, int KT, int AHEAD>
+__device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
-    extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sW = sQ + 64 * PK; T* sPT = sW + 64 * PK;
     T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
     float* sGam = (float*)(sDS + KD * PV);
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
     const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
@@ -455,11 +478,12 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
             const int kk = 16 * (NA * w + a2) + c16;
             dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
         }
-    TileRegs<KD> rK, rQ, rW;
-    TileRegs<CH> rPT;
-    TileRegs<VBT> rDO;
-    float rGam = 0.f;
-    auto fetch = [&](int64_t ic) {
+    // two sets of registers take turns, as in the forward scan
+    struct Ahead { TileRegs<KD> rK, rQ, rW; TileRegs<CH> rPT; TileRegs<VBT> rDO; float rGam; };
+    Ahead RA, RB;
+    RA.rGam = RB.rGam = 0.f;
+    auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
+        auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
         fetch_tile<KD>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
@@ -469,8 +493,8 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
         fetch_tile<VBT>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
     };
-    if (sq.nc > 0) fetch(sq.nc - 1);
-    for (int64_t ic = sq.nc - 1; ic >= 0; --ic) {
+    auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
+        auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
@@ -489,7 +513,7 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
                 *(V4*)(dHu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
-        if (ic > 0) fetch(ic - 1);
+        if (ic >= AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
         // scale e^gam_i do_i, for the state's gradient
         for (int idx = tid; idx < 64 * (VBT / 8); idx += 256) {
@@ -553,6 +577,16 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
                 }
         }
         lds_barrier();
+    };
+    if (sq.nc > 0) fetch(RA, sq.nc - 1);
+    if constexpr (AHEAD == 1) {
+        for (int64_t ic = sq.nc - 1; ic >= 0; --ic) step(RA, ic);
+    } else {
+        if (sq.nc > 1) fetch(RB, sq.nc - 2);
+        for (int64_t ic = sq.nc - 1; ic >= 0; ic -= 2) {
+            step(RA, ic);
+            if (ic > 0) step(RB, ic - 1);
+        }
     }
     if (p.dh0) {
 #pragma unroll
@@ -563,6 +597,26 @@ __global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
                 *(f32x4*)(p.dh0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
             }
     }
+}
+
+template <typename T, int VBT, int KT>
+__global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
+    extern __shared__ __align__(16) char smem[];
+    bwd_dstate_body<T, VBT, KT, KT == 1 ? 2 : 1>(p, smem, threadIdx.x);          // (two blocks of key features: registers for one set only)
+}
+
+// Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
+// Neither needs anything from the other, both take three barriers per chunk, and a step of either leaves most of a CU idle
+// (one wave per SIMD waiting for its own LDS reads and matrix instructions): side by side, two per SIMD, they take about the
+// time of the longer one.  Used where both sets of LDS tiles fit a CU (32 value columns per workgroup, one block of key features).
+template <int VBT, int KT> constexpr size_t bwd_scans_smem() { return bwd_state_smem<VBT, KT>() + bwd_dstate_smem<VBT, KT>(); }
+
+template <typename T, int VBT, int KT>
+__global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
+    extern __shared__ __align__(16) char smem[];
+    static_assert(bwd_state_smem<VBT, KT>() % 16 == 0, "the second set of tiles starts 16-byte aligned");
+    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1>(p, smem, threadIdx.x);
+    else bwd_dstate_body<T, VBT, KT, 1>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1069,6 +1123,15 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
         if (vbt_d == 64) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, KT>, bwd_dstate_smem<64, KT>(), "gdn_bwd_dstate_kernel", runs(64)};
         else dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, KT>, bwd_dstate_smem<128, KT>(), "gdn_bwd_dstate_kernel", runs(128)};
     }
+    unsigned threads[5] = {256, 256, 256, 256, 256};
+    if constexpr (KT == 1) {
+        if (vbt == 32 && !(p.flags & (1u << 28))) {
+            // both scans side by side in one launch (the second entry then has nothing to launch)
+            state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
+            threads[1] = 512;
+            dstate.grid = 0;
+        }
+    }
     const K ks[5] = {
         {(const void*)gdn_bwd_prepare_kernel<T, KT>, bwd_prep_smem<KT>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
@@ -1077,11 +1140,12 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
         {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
     for (int i = 0; i < 5; ++i) {
+        if (ks[i].grid == 0) continue;
         // (the limit on dynamic LDS belongs to the function: asked for on every call, it is a cheap host-side setting)
         if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
         int64_t nunits = units;
         void* args[] = {(void*)&p, (void*)&nunits};             // (the kernels that walk over the units take their number)
-        if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
+        if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(threads[i]), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
     }
     return GDN_OK;
