@@ -105,30 +105,31 @@ __device__ __forceinline__ void load_tile(T* s, int pitch, const T* g, int64_t s
 }
 
 // The same in two halves, for loops that fetch the next tile while they work on the current one.
-template <int NCOLS>
-struct TileRegs { u32x4 x[64 * (NCOLS / 8) / 256]; };
-template <int NCOLS, typename T>
-__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS>& r, const T* g, int64_t stride, int valid, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL / 256, RPI = 256 / PPR;      // a thread's pieces lie RPI rows apart
-    static_assert(TOTAL % 256 == 0, "whole rounds of 256 threads");
+template <int NCOLS, int NTH = 256>
+struct TileRegs { u32x4 x[64 * (NCOLS / 8) >= NTH ? 64 * (NCOLS / 8) / NTH : 1]; };
+template <int NCOLS, int NTH = 256, typename T>
+__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS, NTH>& r, const T* g, int64_t stride, int valid, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL >= NTH ? TOTAL / NTH : 1, RPI = NTH / PPR;      // a thread's pieces lie RPI rows apart
+    static_assert(TOTAL % NTH == 0 || TOTAL < NTH, "whole rounds of the workgroup's threads, or less than one");
     const int row0 = tid / PPR, pc = tid % PPR;
     const char* at = (const char*)(g + (int64_t)row0 * stride + pc * 8);
     const int64_t step = (int64_t)RPI * stride * (int64_t)sizeof(T);
-    if (valid >= 64) {                                          // (the same for the whole workgroup) full chunk: plain loads
+    if (valid >= 64 && TOTAL >= NTH) {                          // (the same for the whole workgroup) full chunk: plain loads
 #pragma unroll
         for (int i = 0; i < N; ++i) r.x[i] = *(const u32x4*)(at + i * step);
     } else {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             r.x[i] = u32x4{0u, 0u, 0u, 0u};
-            if (row0 + RPI * i < valid) r.x[i] = *(const u32x4*)(at + i * step);
+            if (row0 + RPI * i < valid && tid < TOTAL) r.x[i] = *(const u32x4*)(at + i * step);
         }
     }
 }
-template <int NCOLS, typename T>
-__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS>& r, int tid) {
-    constexpr int PPR = NCOLS / 8, N = 64 * PPR / 256, RPI = 256 / PPR;
+template <int NCOLS, int NTH = 256, typename T>
+__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS, NTH>& r, int tid) {
+    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL >= NTH ? TOTAL / NTH : 1, RPI = NTH / PPR;
     T* at = s + (tid / PPR) * pitch + (tid % PPR) * 8;
+    if (TOTAL < NTH && tid >= TOTAL) return;
 #pragma unroll
     for (int i = 0; i < N; ++i) *(u32x4*)(at + i * RPI * pitch) = r.x[i];
 }
@@ -326,14 +327,15 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
 template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
-template <typename T, int VBT, int KT, int AHEAD>
+template <typename T, int VBT, int KT, int AHEAD, int NW>
 __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
-    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
+    // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
+    constexpr int PV = VBT + 8, VBQ = VBT / (NW / 4), NB = VBQ / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT, NTH = 64 * NW;
     T* sW = (T*)smem; T* sK = sW + 64 * PK; T* sS = sK + 64 * PK; T* sVn = sS + KD * PV;
     float* sGam = (float*)(sVn + 64 * PV);
-    const int lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
     const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
@@ -349,28 +351,28 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (NA * w + a2) + c16;
-            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
-    // two sets of registers take turns: the tiles of chunk c + 2 are requested while chunk c is worked on (one chunk of
-    // lead does not cover the way to memory and back: a step would then last as long as that way)
-    struct Ahead { TileRegs<KD> rW, rK; V4 rU[NB]; float rGam; };
+    // (AHEAD = 2: two sets of registers take turns and the tiles of chunk c + 2 are requested while chunk c is worked on;
+    // measured: no faster than one chunk of lead - a step is bound by the CU's load path, not by the way to memory)
+    struct Ahead { TileRegs<KD, NTH> rW, rK; V4 rU[NB]; float rGam; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rW = R.rW; auto& rK = R.rK; auto& rU = R.rU; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        fetch_tile<KD>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<KD>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        fetch_tile<KD, NTH>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
+        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + vq0 + 16 * b + 4 * g);
     };
     auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rW = R.rW; auto& rK = R.rK; auto& rU = R.rU; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
-        put_tile<KD>(sW, PK, rW, tid);
-        put_tile<KD>(sK, PK, rK, tid);
+        put_tile<KD, NTH>(sW, PK, rW, tid);
+        put_tile<KD, NTH>(sK, PK, rK, tid);
         if (tid < 64) sGam[tid] = rGam;
         V4 u4[NB];
 #pragma unroll
@@ -382,8 +384,8 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
             for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(S[a2][b]);
-                *(V4*)(sS + kk * PV + 16 * b + 4 * g) = s4;
-                *(V4*)(Hu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
+                *(V4*)(sS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
+                *(V4*)(Hu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
         if (ic + AHEAD < sq.nc) fetch(R, ic + AHEAD);
@@ -400,15 +402,15 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
             for (int b = 0; b < NB; ++b) {
                 f32x4 acc = ZERO4;
 #pragma unroll
-                for (int s = 0; s < 4 * KT; ++s) acc = Mma<T>::run(frag_cols(sS, PV, 32 * s, 16 * b, lane), wf[s], acc);
+                for (int s = 0; s < 4 * KT; ++s) acc = Mma<T>::run(frag_cols(sS, PV, 32 * s, vq0 + 16 * b, lane), wf[s], acc);
                 f32x4 vn;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
                 const V4 vn4 = pack4<T>(vn);
-                *(V4*)(Vu + 16 * b + 4 * g) = vn4;
+                *(V4*)(Vu + vq0 + 16 * b + 4 * g) = vn4;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)vn4[r] * dec;
-                *(V4*)(sVn + i * PV + 16 * b + 4 * g) = pack4<T>(vn);
+                *(V4*)(sVn + i * PV + vq0 + 16 * b + 4 * g) = pack4<T>(vn);
             }
         }
         lds_barrier();
@@ -427,7 +429,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const V8 fv = frag_cols(sVn, PV, 32 * s, 16 * b, lane);
+                    const V8 fv = frag_cols(sVn, PV, 32 * s, vq0 + 16 * b, lane);
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
                 }
@@ -446,21 +448,25 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
     }
 }
 
+// (all 128 value columns of a head: eight waves, two per SIMD, share one set of tiles)
+template <int VBT> constexpr int scan_waves() { return VBT == BD ? 8 : 4; }
+
 template <typename T, int VBT, int KT>
-__global__ __launch_bounds__(256) void gdn_bwd_state_kernel(BwdParams p) {
+__global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_state_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_state_body<T, VBT, KT, 2>(p, smem, threadIdx.x);
+    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x);
 }
 
-template <typename T, int VBT, int KT, int AHEAD>
+template <typename T, int VBT, int KT, int AHEAD, int NW>
 __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
-    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT;       // NA key tiles per wave
+    // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
+    constexpr int PV = VBT + 8, VBQ = VBT / (NW / 4), NB = VBQ / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT, NTH = 64 * NW;
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sW = sQ + 64 * PK; T* sPT = sW + 64 * PK;
     T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
     float* sGam = (float*)(sDS + KD * PV);
-    const int lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
     const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
@@ -476,31 +482,31 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (NA * w + a2) + c16;
-            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
-    // two sets of registers take turns, as in the forward scan
-    struct Ahead { TileRegs<KD> rK, rQ, rW; TileRegs<CH> rPT; TileRegs<VBT> rDO; float rGam; };
+    // (two sets of registers for AHEAD = 2, as in the forward scan)
+    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        fetch_tile<KD>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
-        fetch_tile<KD>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
-        fetch_tile<KD>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<CH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
-        fetch_tile<VBT>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
+        fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        fetch_tile<KD, NTH>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        fetch_tile<KD, NTH>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
+        fetch_tile<VBT, NTH>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
     };
     auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
-        put_tile<KD>(sK, PK, rK, tid);
-        put_tile<KD>(sQ, PK, rQ, tid);
-        put_tile<KD>(sW, PK, rW, tid);
-        put_tile<CH>(sPT, P64, rPT, tid);
-        put_tile<VBT>(sDO, PV, rDO, tid);
+        put_tile<KD, NTH>(sK, PK, rK, tid);
+        put_tile<KD, NTH>(sQ, PK, rQ, tid);
+        put_tile<KD, NTH>(sW, PK, rW, tid);
+        put_tile<CH, NTH>(sPT, P64, rPT, tid);
+        put_tile<VBT, NTH>(sDO, PV, rDO, tid);
         if (tid < 64) sGam[tid] = rGam;
         T* dHu = (T*)p.ws.dHs + u * KD * BD;
 #pragma unroll
@@ -509,14 +515,14 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(dS[a2][b]);
-                *(V4*)(sDS + kk * PV + 16 * b + 4 * g) = s4;
-                *(V4*)(dHu + kk * BD + vcol0 + 16 * b + 4 * g) = s4;
+                *(V4*)(sDS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
+                *(V4*)(dHu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
         if (ic >= AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
         // scale e^gam_i do_i, for the state's gradient
-        for (int idx = tid; idx < 64 * (VBT / 8); idx += 256) {
+        for (int idx = tid; idx < 64 * (VBT / 8); idx += NTH) {
             const int row = idx / (VBT / 8), pc = idx % (VBT / 8);
             const float f = p.scale * __expf(sGam[row]);
             V8 x = *(const V8*)(sDO + row * PV + pc * 8);
@@ -540,13 +546,13 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     if (32 * s + 31 < 16 * w) continue;         // P^T[j][i] = 0 for i < j
-                    a1 = Mma<T>::run(frag_cols(sDO, PV, 32 * s, 16 * b, lane), pf[s], a1);
+                    a1 = Mma<T>::run(frag_cols(sDO, PV, 32 * s, vq0 + 16 * b, lane), pf[s], a1);
                 }
 #pragma unroll
-                for (int s = 0; s < 4 * KT; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, 16 * b, lane), kf[s], a2v);
+                for (int s = 0; s < 4 * KT; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, vq0 + 16 * b, lane), kf[s], a2v);
                 f32x4 dvn = a1 + a2v * dec;
-                *(V4*)(dVu + 16 * b + 4 * g) = pack4<T>(dvn);
-                *(V4*)(sDvn + j * PV + 16 * b + 4 * g) = pack4<T>(-dvn);
+                *(V4*)(dVu + vq0 + 16 * b + 4 * g) = pack4<T>(dvn);
+                *(V4*)(sDvn + j * PV + vq0 + 16 * b + 4 * g) = pack4<T>(-dvn);
             }
         }
         lds_barrier();
@@ -568,7 +574,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const V8 fo = frag_cols(sDOg, PV, 32 * s, 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, 16 * b, lane);
+                    const V8 fo = frag_cols(sDOg, PV, 32 * s, vq0 + 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, vq0 + 16 * b, lane);
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) {
                         dS[a2][b] = Mma<T>::run(fo, qf[a2][s], dS[a2][b]);
@@ -594,15 +600,15 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (NA * w + a2) + c16;
-                *(f32x4*)(p.dh0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + 16 * b + 4 * g) = dS[a2][b];
+                *(f32x4*)(p.dh0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) = dS[a2][b];
             }
     }
 }
 
 template <typename T, int VBT, int KT>
-__global__ __launch_bounds__(256) void gdn_bwd_dstate_kernel(BwdParams p) {
+__global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_dstate_body<T, VBT, KT, KT == 1 ? 2 : 1>(p, smem, threadIdx.x);          // (two blocks of key features: registers for one set only)
+    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x);
 }
 
 // Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
@@ -615,8 +621,8 @@ template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
     static_assert(bwd_state_smem<VBT, KT>() % 16 == 0, "the second set of tiles starts 16-byte aligned");
-    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1>(p, smem, threadIdx.x);
-    else bwd_dstate_body<T, VBT, KT, 1>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256);
+    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x);
+    else bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1123,9 +1129,9 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
         if (vbt_d == 64) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, KT>, bwd_dstate_smem<64, KT>(), "gdn_bwd_dstate_kernel", runs(64)};
         else dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, KT>, bwd_dstate_smem<128, KT>(), "gdn_bwd_dstate_kernel", runs(128)};
     }
-    unsigned threads[5] = {256, 256, 256, 256, 256};
+    unsigned threads[5] = {256, vbt == BD ? 512u : 256u, vbt_d == BD ? 512u : 256u, 256, 256};
     if constexpr (KT == 1) {
-        if (vbt == 32 && !(p.flags & (1u << 28))) {
+        if (vbt == 32) {
             // both scans side by side in one launch (the second entry then has nothing to launch)
             state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
             threads[1] = 512;
@@ -1174,7 +1180,7 @@ extern "C" int gdn_chunk_bwd(
     GDN_CHECK_ARG((K == BD || K == 2 * BD) && V == BD, GDN_ERR_UNSUPPORTED,
                   "%s: K = 128 or 256 and V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros", who, (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
-    GDN_CHECK_ARG((flags & ~(uint32_t)(GDN_FLAG_CU_INT32 | (7u << 27))) == 0, GDN_ERR_UNSUPPORTED,
+    GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
                   "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
                   "%s: too many heads or chunks for one launch", who);
