@@ -99,7 +99,7 @@ def _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=None, **kw):
     for n in ('A_log', 'dt_bias'):
         if kw.get(n) is not None:
             extra['d' + n] = kw[n] = kw[n].to(dev).requires_grad_(True)
-    cu_t = None if cu is None else torch.tensor(cu, dtype=torch.int64, device=dev)
+    cu_t = None if cu is None else torch.tensor(cu, dtype=kw.pop('idx_dtype', torch.int64), device=dev)
     o, ht = _op()(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dg'], leaves['dbeta'], initial_state=leaves['dh0'],
                   output_final_state=dht is not None, cu_seqlens=cu_t, **kw)
     loss = (o.float() * do.to(dev).float()).sum()
@@ -183,7 +183,7 @@ def test_chunk_backward_packed(H, HV, D, mask_p, cu):
     do = torch.randn(1, T, HV, D, generator=gen).to(dtype)
     dht = torch.rand(N, HV, D, D, generator=gen)
     ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, dtype=torch.float32)
-    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu)
+    o, ht, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu, idx_dtype=torch.int32 if D == 64 else torch.int64)
     _compare(ref, got, tol=dict(dq=0.007, dk=0.008, dv=0.007, dbeta=0.015, dg=0.015, dh0=0.007))
     # every sequence's gradients are those of the sequence alone
     if N > 1:
