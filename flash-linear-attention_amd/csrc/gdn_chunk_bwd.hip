@@ -17,14 +17,9 @@
 // and `frag_cols` (the contraction runs down a column: two transposing LDS reads).  The result of run(a, b) holds, in lane
 // (c16, g), column c16 (b's index) and rows 4g .. 4g+3 (a's index): whichever side carries the features gets them four in a
 // row per lane, which is what an 8-byte store into a row-major [token][feature] array wants.
-#include "gdn_chunk_common.h"
+#include "gdn_tiles.h"
 
 namespace gdn {
-
-constexpr int BD = 128;              // value columns of these kernels; key features: KD = 128 KT with KT = 1 or 2 (a template argument)
-constexpr int P128 = BD + 8;         // LDS pitch, in elements, of a [64][128] tile ([64][KD] tiles: KD + 8)
-constexpr int P64 = CH + 8;          // ... of a [64][64] tile
-constexpr int PL = CH + 4;           // pitch of the fp32 matrix L
 
 // Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels),
 // A [64][64], P^T [64][64], w [64][KD], u -> v_new [64][128], S [KD][128] ([K][V]), dS [KD][128], dv_new [64][128],
@@ -55,114 +50,6 @@ struct BwdParams {
     int64_t T; int H, HV; int64_t N; int64_t NT;
     float scale; int gb_dtype; uint32_t flags;
 };
-
-// ---- geometry ------------------------------------------------------------------------------
-struct ChunkAt { int64_t tok0; int valid; };
-__device__ __forceinline__ ChunkAt chunk_at(const BwdParams& p, int64_t ci) {
-    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-    if (p.cu_seqlens) {
-        const int64_t n = load_index(p.chunk_table, 2 * ci, cu32), it = load_index(p.chunk_table, 2 * ci + 1, cu32);
-        const int64_t bos = load_index(p.cu_seqlens, n, cu32), eos = load_index(p.cu_seqlens, n + 1, cu32);
-        const int64_t t0 = bos + it * CH;
-        return ChunkAt{t0, (int)min((int64_t)CH, eos - t0)};
-    }
-    const int64_t b = ci / p.NT, it = ci % p.NT;
-    return ChunkAt{b * p.T + it * CH, (int)min((int64_t)CH, p.T - it * CH)};
-}
-struct SeqAt { int64_t bos, len, cbase, nc; };
-__device__ __forceinline__ SeqAt seq_at(const BwdParams& p, int64_t n) {
-    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
-    SeqAt s;
-    if (p.cu_seqlens) {
-        s.bos = load_index(p.cu_seqlens, n, cu32);
-        s.len = load_index(p.cu_seqlens, n + 1, cu32) - s.bos;
-        s.cbase = load_index(p.chunk_offsets, n, cu32);
-    } else {
-        s.bos = n * p.T; s.len = p.T; s.cbase = n * p.NT;
-    }
-    s.nc = (s.len + CH - 1) / CH;
-    return s;
-}
-
-// ---- tiles ---------------------------------------------------------------------------------
-// 64 rows of NCOLS elements from global memory (row r at g + r * stride; rows from `valid` on read as zero) into a
-// row-major LDS tile, by all 256 threads.  Loads first, stores after: the loads of one tile are in flight together.
-template <int NCOLS, typename T>
-__device__ __forceinline__ void load_tile(T* s, int pitch, const T* g, int64_t stride, int valid, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = (TOTAL + 255) / 256;
-    u32x4 x[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        x[i] = u32x4{0u, 0u, 0u, 0u};
-        if (idx < TOTAL && row < valid) x[i] = *(const u32x4*)(g + row * stride + pc * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int idx = tid + 256 * i, row = idx / PPR, pc = idx % PPR;
-        if (idx < TOTAL) *(u32x4*)(s + row * pitch + pc * 8) = x[i];
-    }
-}
-
-// The same in two halves, for loops that fetch the next tile while they work on the current one.
-template <int NCOLS, int NTH = 256>
-struct TileRegs { u32x4 x[64 * (NCOLS / 8) >= NTH ? 64 * (NCOLS / 8) / NTH : 1]; };
-template <int NCOLS, int NTH = 256, typename T>
-__device__ __forceinline__ void fetch_tile(TileRegs<NCOLS, NTH>& r, const T* g, int64_t stride, int valid, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL >= NTH ? TOTAL / NTH : 1, RPI = NTH / PPR;      // a thread's pieces lie RPI rows apart
-    static_assert(TOTAL % NTH == 0 || TOTAL < NTH, "whole rounds of the workgroup's threads, or less than one");
-    const int row0 = tid / PPR, pc = tid % PPR;
-    const char* at = (const char*)(g + (int64_t)row0 * stride + pc * 8);
-    const int64_t step = (int64_t)RPI * stride * (int64_t)sizeof(T);
-    if (valid >= 64 && TOTAL >= NTH) {                          // (the same for the whole workgroup) full chunk: plain loads
-#pragma unroll
-        for (int i = 0; i < N; ++i) r.x[i] = *(const u32x4*)(at + i * step);
-    } else {
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            r.x[i] = u32x4{0u, 0u, 0u, 0u};
-            if (row0 + RPI * i < valid && tid < TOTAL) r.x[i] = *(const u32x4*)(at + i * step);
-        }
-    }
-}
-template <int NCOLS, int NTH = 256, typename T>
-__device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS, NTH>& r, int tid) {
-    constexpr int PPR = NCOLS / 8, TOTAL = 64 * PPR, N = TOTAL >= NTH ? TOTAL / NTH : 1, RPI = NTH / PPR;
-    T* at = s + (tid / PPR) * pitch + (tid % PPR) * 8;
-    if (TOTAL < NTH && tid >= TOTAL) return;
-#pragma unroll
-    for (int i = 0; i < N; ++i) *(u32x4*)(at + i * RPI * pitch) = r.x[i];
-}
-// operand fragment whose contraction runs along a row: index r0 + c16, contraction c0 + 8g + e
-template <typename T>
-__device__ __forceinline__ typename Mma<T>::V8 frag_rows(const T* s, int pitch, int r0, int c0, int lane) {
-    return *(const typename Mma<T>::V8*)(s + (r0 + (lane & 15)) * pitch + c0 + 8 * (lane >> 4));
-}
-// operand fragment whose contraction runs down a column: index c0 + c16, contraction r0 + 8g + e
-template <typename T>
-__device__ __forceinline__ typename Mma<T>::V8 frag_cols(const T* s, int pitch, int r0, int c0, int lane) {
-    const int a = lane & 15;
-    const T* at = s + (r0 + 8 * (lane >> 4) + (a >> 2)) * pitch + c0 + 4 * (a & 3);
-    return join<typename Mma<T>::V8>(Mma<T>::tr_read(at), Mma<T>::tr_read(at + 4 * pitch));
-}
-template <typename T>
-__device__ __forceinline__ typename Mma<T>::V4 pack4(f32x4 x) {
-    return typename Mma<T>::V4{(T)x[0], (T)x[1], (T)x[2], (T)x[3]};
-}
-__device__ __forceinline__ float sum_over_g(float x) {          // over the four lanes that share c16
-    x += __shfl_xor(x, 16, 64);
-    return x + __shfl_xor(x, 32, 64);
-}
-__device__ __forceinline__ float sum_over_c16(float x) {        // over the sixteen lanes that share g
-    x += __shfl_xor(x, 1, 64); x += __shfl_xor(x, 2, 64); x += __shfl_xor(x, 4, 64);
-    return x + __shfl_xor(x, 8, 64);
-}
-// x summed over the four lanes of a quad (lanes 4n .. 4n+3), in every one of them
-__device__ __forceinline__ float sum_over_quad(float x) {
-    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // [2,3,0,1]
-}
-#define ZERO4 (f32x4{0.f, 0.f, 0.f, 0.f})
 
 // ---------------------------------------------------------------------------------------------
 // prepare
