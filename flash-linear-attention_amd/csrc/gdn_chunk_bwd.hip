@@ -138,31 +138,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
             *(V8*)at = x;
         }
-        // A = (I + L)^-1 by forward substitution, A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c]: a quad of lanes per
-        // column c (16 columns per wave), lane gq of the quad keeps A[j][c] for j = gq mod 4 and adds up their part of the sum
-        {
-            const int c = 16 * w + (lane >> 2), gq = lane & 3;
-            float a[16];
-#pragma unroll
-            for (int m = 0; m < 16; ++m) a[m] = 0.f;
-#pragma unroll
-            for (int i = 0; i < 64; ++i) {
-                float part0 = 0.f, part1 = 0.f;
-#pragma unroll
-                for (int m4 = 0; 16 * m4 < i; ++m4) {           // entries j = 4m + gq < i; those from i on are stored as zeros
-                    const f32x4 l = *(const f32x4*)(sL + i * PL + gq * 16 + 4 * m4);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (4 * (4 * m4 + e) < i) {
-                            if (e & 1) part1 += l[e] * a[4 * m4 + e];
-                            else part0 += l[e] * a[4 * m4 + e];
-                        }
-                    }
-                }
-                const float ai = (i == c ? 1.f : 0.f) - sum_over_quad(part0 + part1);
-                if (gq == (i & 3)) { a[i >> 2] = ai; sA[i * P64 + c] = (T)ai; }
-            }
-        }
+        solve_unit_lower<T>(sL, sA, w, lane);
         lds_barrier();
         {
             T* Au = (T*)p.ws.Am + u * 64 * 64;

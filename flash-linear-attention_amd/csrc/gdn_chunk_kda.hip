@@ -1,0 +1,465 @@
+// Chunked forward of the KDA operator (the gated delta rule with a decay per key feature), 64-token chunks, K, V <= 128
+// (zero-padded to 128 by the host).  Replaces chunk_kda_fwd (fla/ops/kda/chunk_fwd.py:20-134): the gate activation and
+// chunk-local cumsum (fla/ops/kda/gate.py), the intra-chunk stage (fla/ops/kda/chunk_intra.py), recompute_w_u_fwd
+// (fla/ops/kda/wy_fast.py), chunk_gated_delta_rule_fwd_h and chunk_gla_fwd_o_gk.  Two kernels:
+//
+//   prepare  per (chunk, v-head): Gam = cumsum of the log decays inside the chunk [64][K];
+//            M_ij = sum_k k_ik k_jk e^(Gam_ik - Gam_jk) (i > j),  P_ij = scale sum_k q_ik k_jk e^(Gam_ik - Gam_jk) (i >= j);
+//            A = (I + diag(beta) M)^-1,  w = A (beta k e^Gam),  u = A (beta v);
+//            also qg = scale q e^Gam, kg = k e^(Gam_last - Gam), e^Gam_last: what the scan needs, so that it never sees a gate
+//   scan     per (sequence, v-head, VBT value columns), chunks in order, state slice in registers:
+//            v_new = u - w S;  o = qg S + P v_new;  S <- diag(e^Gam_last) S + kg^T v_new
+//
+// The exponent Gam_ik - Gam_jk is only ever non-positive for i >= j, but it cannot be split into a factor of row i and a
+// factor of row j without overflow unless a reference row lies between them.  Blocks of 16 rows: for j in an earlier
+// block than i the reference is the last row in front of i's block, e^(Gam_i - ref) e^(ref - Gam_j) with both exponents <= 0,
+// and the products run on the matrix cores; inside a 16 x 16 diagonal block every pair gets its own exponentials
+// (the reference does the same, fla/ops/kda/chunk_intra.py: sub-chunks of 16).
+#include "gdn_tiles.h"
+
+namespace gdn {
+
+constexpr int PG = BD + 4;           // pitch of the fp32 gate tile
+
+struct KdaWs { void* Wm; void* Um; void* QG; void* KG; void* Pm; float* EGL; };
+inline size_t kda_ws_layout(int64_t units, char* base, KdaWs* ws) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
+    const size_t u = (size_t)units;
+    void* Wm = take(u * 64 * BD * 2); void* Um = take(u * 64 * BD * 2);
+    void* QG = take(u * 64 * BD * 2); void* KG = take(u * 64 * BD * 2);
+    void* Pm = take(u * 64 * 64 * 2); void* EGL = take(u * BD * 4);
+    if (ws) *ws = KdaWs{Wm, Um, QG, KG, Pm, (float*)EGL};
+    return off;
+}
+
+struct KdaParams {
+    const void* q; const void* k; const void* v; const float* g; const void* beta;
+    const float* A_log; const float* gk_bias; float gk_lower; int gk_act;      // gate activation, as in the token recurrence
+    const float* h0; float* ht; void* o;
+    const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
+    KdaWs ws;
+    int64_t T; int H, HV; int64_t N; int64_t NT;
+    float scale; int gb_dtype; uint32_t flags;
+};
+
+// ---------------------------------------------------------------------------------------------
+// prepare
+// ---------------------------------------------------------------------------------------------
+constexpr size_t KDA_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PG + 64 * PL + 64) * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
+    float* sG = (float*)(sA + 64 * P64); float* sL = sG + 64 * PG; float* sBeta = sL + 64 * PL;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int64_t u = blockIdx.x, ci = u / p.HV;
+    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+    const ChunkAt c = chunk_at(p, ci);
+
+    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+    load_tile<BD>(sV, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    {
+        // gates: a thread per key feature and half of the chunk's rows; running sums inside the half first
+        const int col = tid & 127, half = tid >> 7;
+        const float a_k = p.gk_act ? (p.A_log ? __expf(p.A_log[hv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
+        const float bias = (p.gk_act && p.gk_bias) ? p.gk_bias[hv * BD + col] : 0.f;
+        float x[32];
+#pragma unroll
+        for (int r = 0; r < 32; ++r) {
+            const int row = 32 * half + r;
+            x[r] = row < c.valid ? p.g[((c.tok0 + row) * p.HV + hv) * BD + col] : 0.f;
+        }
+        float run = 0.f;
+#pragma unroll
+        for (int r = 0; r < 32; ++r) {
+            const int row = 32 * half + r;
+            float gt = x[r];
+            if (p.gk_act && row < c.valid) {
+                gt += bias;
+                gt = p.gk_act == 2 ? p.gk_lower * sigmoid_f(a_k * gt) : -a_k * softplus_f(gt);
+            }
+            run += gt;
+            sG[row * PG + col] = run;
+        }
+    }
+    if (tid < 64) {
+        float b = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        if ((p.flags & GDN_FLAG_BETA_SIGMOID) && tid < c.valid) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
+        sBeta[tid] = b;
+    }
+    __syncthreads();
+    {
+        // second half of the rows: add the first half's total
+        const int col = tid & 127, half = tid >> 7;
+        if (half == 1) {
+            const float tot = sG[31 * PG + col];
+#pragma unroll
+            for (int r = 0; r < 32; ++r) sG[(32 + r) * PG + col] += tot;
+        }
+    }
+    if (p.flags & GDN_FLAG_QK_L2NORM) {
+        // rows of q and k divided by sqrt(sum x^2 + 1e-6): 16 consecutive lanes hold the 16 pieces of a row
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = (tid >> 4) + 16 * i, pc = tid & 15;
+#pragma unroll
+            for (int which = 0; which < 2; ++which) {
+                T* at = (which ? sQ : sK) + row * P128 + pc * 8;
+                V8 x = *(V8*)at;
+                float ss = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += (float)x[e] * (float)x[e];
+                const float r = rsqrtf(sum_over_c16(ss) + 1e-6f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * r);
+                *(V8*)at = x;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- M (as L = diag(beta) M, for the substitution) and P, this wave's 16 rows ----
+    {
+        T* Pu = (T*)p.ws.Pm + u * 64 * 64;
+        const int i = 16 * w + c16;                             // the row this lane's operand fragments belong to
+        // rows of this block against rows of earlier blocks: reference = the row in front of the block
+        if (w > 0) {
+            V8 kd[4], qd[4];
+            float ref[4][8];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float* gi = sG + i * PG + 32 * s + 8 * g;
+                const float* gr = sG + (16 * w - 1) * PG + 32 * s + 8 * g;
+                const V8 kx = frag_rows(sK, P128, 16 * w, 32 * s, lane), qx = frag_rows(sQ, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    ref[s][e] = gr[e];
+                    const float f = __expf(gi[e] - gr[e]);
+                    kd[s][e] = (T)((float)kx[e] * f);
+                    qd[s][e] = (T)((float)qx[e] * f);
+                }
+            }
+#pragma unroll
+            for (int tj = 0; tj < 3; ++tj) {
+                if (tj >= w) break;
+                f32x4 m = ZERO4, pt = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float* gj = sG + (16 * tj + c16) * PG + 32 * s + 8 * g;
+                    V8 kn = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
+                    m = Mma<T>::run(kd[s], kn, m);             // lane: column j = 16tj + c16, rows i = 16w + 4g + r
+                    pt = Mma<T>::run(kn, qd[s], pt);           // lane: column i = 16w + c16, rows j = 16tj + 4g + r
+                }
+                const int j = 16 * tj + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int ir = 16 * w + 4 * g + r;
+                    sL[ir * PL + (j & 3) * 16 + (j >> 2)] = sBeta[ir] * m[r];
+                }
+                *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(pt * p.scale);
+            }
+        }
+        // the diagonal block: lane (il, jq) takes row il and columns 4jq .. 4jq+3 of the block, every pair with its own exponentials
+        {
+            const int il = lane >> 2, jq = lane & 3, row = 16 * w + il;
+            float m[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int kc = 0; kc < BD / 8; ++kc) {
+                const V8 ki = *(const V8*)(sK + row * P128 + 8 * kc), qi = *(const V8*)(sQ + row * P128 + 8 * kc);
+                const f32x4 gi0 = *(const f32x4*)(sG + row * PG + 8 * kc), gi1 = *(const f32x4*)(sG + row * PG + 8 * kc + 4);
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int jl = 4 * jq + jj;
+                    if (jl > il) continue;                      // (upper triangle: nothing)
+                    const int rj = 16 * w + jl;
+                    const V8 kj = *(const V8*)(sK + rj * P128 + 8 * kc);
+                    const f32x4 gj0 = *(const f32x4*)(sG + rj * PG + 8 * kc), gj1 = *(const f32x4*)(sG + rj * PG + 8 * kc + 4);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float d = __expf((e < 4 ? gi0[e & 3] : gi1[e & 3]) - (e < 4 ? gj0[e & 3] : gj1[e & 3]));
+                        const float kk = (float)kj[e] * d;
+                        m[jj] += (float)ki[e] * kk;
+                        pq[jj] += (float)qi[e] * kk;
+                    }
+                }
+            }
+            f32x4 pt;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int jl = 4 * jq + jj, j = 16 * w + jl;
+                sL[row * PL + (j & 3) * 16 + (j >> 2)] = jl < il ? sBeta[row] * m[jj] : 0.f;
+                pt[jj] = jl <= il ? p.scale * pq[jj] : 0.f;
+            }
+            *(V4*)(Pu + row * 64 + 16 * w + 4 * jq) = pack4<T>(pt);
+            // blocks to the right of the diagonal: zeros
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj)
+                if (tj > w) *(V4*)(Pu + row * 64 + 16 * tj + 4 * jq) = pack4<T>(ZERO4);
+        }
+    }
+    __syncthreads();
+    solve_unit_lower<T>(sL, sA, w, lane);
+    __syncthreads();
+    {
+        // what the scan needs of q and k, and k, v as the factors of w, u
+        T* QGu = (T*)p.ws.QG + u * 64 * BD;
+        T* KGu = (T*)p.ws.KG + u * 64 * BD;
+        for (int idx = tid; idx < 64 * 16; idx += 256) {
+            const int row = idx >> 4, pc = idx & 15;
+            const float* gi = sG + row * PG + pc * 8;
+            const float* gl = sG + 63 * PG + pc * 8;
+            V8 kx = *(V8*)(sK + row * P128 + pc * 8), qx = *(V8*)(sQ + row * P128 + pc * 8), vx = *(V8*)(sV + row * P128 + pc * 8);
+            V8 kg, qg;
+            const float b = sBeta[row];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float eg = __expf(gi[e]);
+                kg[e] = (T)((float)kx[e] * __expf(gl[e] - gi[e]));
+                qg[e] = (T)((float)qx[e] * (p.scale * eg));
+                kx[e] = (T)((float)kx[e] * (b * eg));
+                vx[e] = (T)((float)vx[e] * b);
+            }
+            *(V8*)(KGu + row * BD + pc * 8) = kg;
+            *(V8*)(QGu + row * BD + pc * 8) = qg;
+            *(V8*)(sK + row * P128 + pc * 8) = kx;
+            *(V8*)(sV + row * P128 + pc * 8) = vx;
+        }
+        if (tid < BD) p.ws.EGL[u * BD + tid] = __expf(sG[63 * PG + tid]);
+    }
+    __syncthreads();
+    {
+        // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
+        T* Wu = (T*)p.ws.Wm + u * 64 * BD;
+        T* Uu = (T*)p.ws.Um + u * 64 * BD;
+        const int i = 16 * w + c16;
+        V8 fa[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) fa[s] = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            f32x4 aw = ZERO4, au = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (2 * s > w) continue;                        // A is lower triangular
+                aw = Mma<T>::run(frag_cols(sK, P128, 32 * s, 16 * n, lane), fa[s], aw);
+                au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), fa[s], au);
+            }
+            *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
+            *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// scan: the state slice [128][VBT] lives in registers as transposed tiles (wave w: key rows 32w .. 32w+31 as two tiles a2,
+// lane (c16, g): key 16(2w+a2) + c16, value columns 16b + 4g .. +3); the next chunk's tiles are fetched into registers
+// while the current chunk is computed.
+// ---------------------------------------------------------------------------------------------
+template <int VBT> constexpr size_t kda_scan_smem() { return (3 * 64 * P128 + 64 * P64 + BD * (VBT + 8) + 64 * (VBT + 8)) * 2 + (BD + 64) * 4; }
+
+template <typename T, int VBT>
+__global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
+    extern __shared__ __align__(16) char smem[];
+    T* sW = (T*)smem; T* sKG = sW + 64 * P128; T* sQG = sKG + 64 * P128; T* sP = sQG + 64 * P128;
+    T* sS = sP + 64 * P64; T* sVn = sS + BD * PV;
+    float* sE = (float*)(sVn + 64 * PV);
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;       // (slices of one head on one XCD)
+    if (run >= p.N * p.HV) return;
+    const int vs = (blockIdx.x / 8) % NVS, hv = (int)(run % p.HV);
+    const int64_t n = run / p.HV;
+    const SeqAt sq = seq_at(p, n);
+    const int vcol0 = vs * VBT;
+
+    f32x4 S[2][NB];
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int kk = 16 * (2 * w + a2) + c16;
+            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) : ZERO4;
+        }
+    TileRegs<BD> rW, rKG, rQG;
+    TileRegs<CH> rP;
+    V4 rU[NB];
+    float rE = 0.f;
+    auto fetch = [&](int64_t ic) {
+        const int64_t u = (sq.cbase + ic) * p.HV + hv;
+        fetch_tile<BD>(rW, (const T*)p.ws.Wm + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rKG, (const T*)p.ws.KG + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rQG, (const T*)p.ws.QG + u * 64 * BD, BD, 64, tid);
+        fetch_tile<CH>(rP, (const T*)p.ws.Pm + u * 64 * 64, 64, 64, tid);
+        if (tid < BD) rE = p.ws.EGL[u * BD + tid];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Um + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
+    };
+    if (sq.nc > 0) fetch(0);
+    for (int64_t ic = 0; ic < sq.nc; ++ic) {
+        const int64_t tok0 = sq.bos + ic * CH;
+        const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
+        put_tile<BD>(sW, P128, rW, tid);
+        put_tile<BD>(sKG, P128, rKG, tid);
+        put_tile<BD>(sQG, P128, rQG, tid);
+        put_tile<CH>(sP, P64, rP, tid);
+        if (tid < BD) sE[tid] = rE;
+        V4 u4[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) u4[b] = rU[b];
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                *(V4*)(sS + (16 * (2 * w + a2) + c16) * PV + 16 * b + 4 * g) = pack4<T>(S[a2][b]);
+        lds_barrier();
+        if (ic + 1 < sq.nc) fetch(ic + 1);
+        f32x4 oacc[NB];
+        {
+            // v_new^T and (qg S)^T tiles: value columns on the rows, this wave's 16 tokens on the columns
+            const int i = 16 * w + c16;
+            V8 wf[4], qf[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) { wf[s] = frag_rows(sW, P128, 16 * w, 32 * s, lane); qf[s] = frag_rows(sQG, P128, 16 * w, 32 * s, lane); }
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                f32x4 acc = ZERO4;
+                oacc[b] = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const V8 fs = frag_cols(sS, PV, 32 * s, 16 * b, lane);
+                    acc = Mma<T>::run(fs, wf[s], acc);
+                    oacc[b] = Mma<T>::run(fs, qf[s], oacc[b]);
+                }
+                f32x4 vn;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
+                *(V4*)(sVn + i * PV + 16 * b + 4 * g) = pack4<T>(vn);
+            }
+        }
+        lds_barrier();
+        {
+            // o += P v_new;  S <- diag(e^Gam_last) S + kg^T v_new
+            const int i = 16 * w + c16;
+            V8 pf[2], kf[2][2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                pf[s] = frag_rows(sP, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+                for (int a2 = 0; a2 < 2; ++a2) kf[a2][s] = frag_cols(sKG, P128, 32 * s, 16 * (2 * w + a2), lane);
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2) {
+                const float e = sE[16 * (2 * w + a2) + c16];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) S[a2][b] *= e;
+            }
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const V8 fv = frag_cols(sVn, PV, 32 * s, 16 * b, lane);
+                    if (32 * s <= 16 * w + 15) oacc[b] = Mma<T>::run(fv, pf[s], oacc[b]);      // P[i][j] = 0 for j > i
+#pragma unroll
+                    for (int a2 = 0; a2 < 2; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
+                }
+                if (i < valid) *(V4*)((T*)p.o + ((tok0 + i) * p.HV + hv) * BD + vcol0 + 16 * b + 4 * g) = pack4<T>(oacc[b]);
+            }
+        }
+        lds_barrier();
+    }
+    if (p.ht) {
+#pragma unroll
+        for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int kk = 16 * (2 * w + a2) + c16;
+                *(f32x4*)(p.ht + ((n * p.HV + hv) * BD + kk) * BD + vcol0 + 16 * b + 4 * g) = S[a2][b];
+            }
+    }
+}
+
+template <typename T>
+static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream) {
+    const int64_t runs1 = p.N * p.HV;
+    const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
+    const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)((runs1 + 7) / 8 * 8 * (BD / vbt));
+    struct K { const void* f; size_t smem; const char* name; unsigned grid; };
+    K scan;
+    if (vbt == 32) scan = {(const void*)gdn_kda_scan_kernel<T, 32>, kda_scan_smem<32>(), "gdn_kda_scan_kernel", runs};
+    else if (vbt == 64) scan = {(const void*)gdn_kda_scan_kernel<T, 64>, kda_scan_smem<64>(), "gdn_kda_scan_kernel", runs};
+    else scan = {(const void*)gdn_kda_scan_kernel<T, 128>, kda_scan_smem<128>(), "gdn_kda_scan_kernel", runs};
+    const K ks[2] = {{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units}, scan};
+    for (int i = 0; i < 2; ++i) {
+        if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
+        void* args[] = {(void*)&p};
+        if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
+        if (int rc = check_launch(ks[i].name)) return rc;
+    }
+    return GDN_OK;
+}
+
+}  // namespace gdn
+
+extern "C" size_t gdn_chunk_kda_workspace_bytes(int64_t num_chunks, int64_t HV) {
+    if (num_chunks < 0 || HV < 1) return 0;
+    return gdn::kda_ws_layout(num_chunks * HV, nullptr, nullptr);
+}
+
+extern "C" int gdn_chunk_kda_fwd(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    using namespace gdn;
+    const char* who = "gdn_chunk_kda_fwd";
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
+    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
+                  who, (long long)K, (long long)V);
+    GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v must be bf16 or f16", who);
+    GDN_CHECK_ARG(gate_mode >= 0 && gate_mode <= 2, GDN_ERR_INVALID, "%s: gate_mode must be 0, 1 or 2", who);
+    GDN_CHECK_ARG(gate_mode != 0 || (!A_log && !dt_bias), GDN_ERR_INVALID, "%s: A_log / dt_bias without a gate activation", who);
+    const uint32_t known = GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM | GDN_FLAG_BETA_SIGMOID | GDN_FLAG_NEG_EIGVAL;
+    GDN_CHECK_ARG((flags & ~known) == 0, GDN_ERR_UNSUPPORTED, "%s: unknown flag (the state layout is the caller's)", who);
+    GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
+                  "%s: too many heads or chunks for one launch", who);
+    if (cu_seqlens) {
+        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
+        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
+    } else {
+        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
+        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0 || num_chunks == 0) {
+        if (ht) return launch_state_copy(h0, ht, N * HV * K * V, s);
+        return GDN_OK;
+    }
+    GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
+    for (const void* x : {q, k, v, (const void*)g, (const void*)h0, (const void*)ht, (const void*)o})
+        GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
+    GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
+    KdaParams p;
+    const size_t need = kda_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
+    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
+                  need, workspace_bytes);
+    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.gk_bias = dt_bias; p.gk_lower = lower_bound; p.gk_act = gate_mode;
+    p.h0 = h0; p.ht = ht; p.o = o;
+    p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_kda<bf16_t>(p, num_chunks, s) : launch_kda<f16_t>(p, num_chunks, s);
+}

@@ -128,4 +128,34 @@ __device__ __forceinline__ float sum_over_quad(float x) {
 #define ZERO4 (f32x4{0.f, 0.f, 0.f, 0.f})
 
 
+// A = (I + L)^-1 for a strictly lower triangular 64 x 64 L, by forward substitution in fp32:
+// A[i][c] = [i == c] - sum_{j < i} L[i][j] A[j][c].  Four waves, wave w the columns 16w .. 16w+15: a quad of lanes per
+// column c, lane gq of the quad keeps A[j][c] for j = gq mod 4 and adds up its part of the sum.  sL holds entry (i, j)
+// at [i][j % 4][j / 4] (pitch PL; zeros from the diagonal on within the 16 x 16 diagonal blocks); A goes to sA (pitch
+// P64) in the operand type.  The caller's barriers separate it from the writers of sL and the readers of sA.
+template <typename T>
+__device__ __forceinline__ void solve_unit_lower(const float* sL, T* sA, int w, int lane) {
+    const int c = 16 * w + (lane >> 2), gq = lane & 3;
+    float a[16];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) a[m] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 64; ++i) {
+        float part0 = 0.f, part1 = 0.f;
+#pragma unroll
+        for (int m4 = 0; 16 * m4 < i; ++m4) {                   // entries j = 4m + gq < i; those from i on are stored as zeros
+            const f32x4 l = *(const f32x4*)(sL + i * PL + gq * 16 + 4 * m4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (4 * (4 * m4 + e) < i) {
+                    if (e & 1) part1 += l[e] * a[4 * m4 + e];
+                    else part0 += l[e] * a[4 * m4 + e];
+                }
+            }
+        }
+        const float ai = (i == c ? 1.f : 0.f) - sum_over_quad(part0 + part1);
+        if (gq == (i & 3)) { a[i >> 2] = ai; sA[i * P64 + c] = (T)ai; }
+    }
+}
+
 }  // namespace gdn

@@ -1,0 +1,205 @@
+"""``chunk_kda``: chunked prefill of the KDA operator (the gated delta rule with a decay per key feature), forward
+only, with the signature, validation and error types of fla/ops/kda/chunk.py:178-443.  The reference's launches
+(gate activation + chunk-local cumsum, the intra-chunk stage, ``recompute_w_u_fwd``, the state recurrence and the output,
+fla/ops/kda/chunk_fwd.py:20-134) are one call into libgdn_hip.so (``gdn_chunk_kda_fwd``): a chunk-parallel kernel and a
+sequential one.  The activations the reference fuses (l2 norm of q and k, gate, beta sigmoid) happen inside the first."""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from fla_hip import _lib
+from fla_hip.ops.gated_delta_rule._common import (
+    aligned16,
+    as_f32,
+    current_stream_ptr,
+    dtype_code,
+    forward_only,
+    ptr,
+    require_gpu,
+)
+from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
+
+_CHUNK = 64
+_DIM = 128          # head dims of the kernels; smaller ones are zero-padded
+
+
+def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
+    return x if x.shape[-1] == size else F.pad(x, (0, size - x.shape[-1]))
+
+
+def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first=False, cu_seqlens=None,
+                  cu_seqlens_cpu=None, A_log=None, dt_bias=None, lower_bound=None, gate_mode=0,
+                  use_qk_l2norm_in_kernel=False, use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False):
+    """Returns ``(o [B,T,HV,V] in q's dtype, final_state fp32 or None)``; ``gate_mode`` 0: g is the log decay,
+    1: ``-exp(A_log) softplus(g + dt_bias)``, 2: ``lower_bound sigmoid(exp(A_log) (g + dt_bias))``."""
+    dev = require_gpu(q, k, v, g, beta)
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if K > _DIM:
+        raise NotImplementedError(f'the chunked KDA kernels cover key head dims up to {_DIM} (got K={K})')
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    nb = (V + _DIM - 1) // _DIM
+    if nb > 1:
+        # value columns are independent: a head with V > 128 is nb heads of 128 columns that share q, k, g, beta
+        v2 = _pad_last(v, nb * _DIM).reshape(B, T, HV * nb, _DIM)
+        h2 = None
+        if initial_state is not None:
+            if state_v_first:
+                h2 = F.pad(initial_state, (0, 0, 0, nb * _DIM - V)).reshape(N, HV * nb, _DIM, K)
+            else:
+                h2 = _pad_last(initial_state, nb * _DIM).reshape(N, HV, K, nb, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV * nb, K, _DIM)
+        o2, ht2 = chunk_kda_fwd(
+            q, k, v2, g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2), scale, h2, output_final_state,
+            state_v_first, cu_seqlens, cu_seqlens_cpu, None if A_log is None else A_log.reshape(-1).repeat_interleave(nb),
+            None if dt_bias is None else dt_bias.reshape(HV, K).repeat_interleave(nb, dim=0), lower_bound, gate_mode,
+            use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)
+        o = o2.reshape(B, T, HV, nb * _DIM)[..., :V].contiguous()
+        ht = None
+        if ht2 is not None:
+            if state_v_first:
+                ht = ht2.reshape(N, HV, nb * _DIM, K)[:, :, :V]
+            else:
+                ht = ht2.reshape(N, HV, nb, K, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV, K, nb * _DIM)[..., :V]
+            ht = ht.contiguous()
+        return o, ht
+
+    out_dtype = q.dtype
+    work = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    qw, kw, vw = (aligned16(_pad_last(x.to(work), _DIM).contiguous()) for x in (q, k, v))
+    gw = aligned16(_pad_last(as_f32(g), _DIM).contiguous())
+    bw = as_f32(beta).contiguous()
+    if A_log is not None:
+        A_log = A_log.detach().to(device=dev, dtype=torch.float32).reshape(-1).contiguous()
+        if A_log.numel() != HV:
+            raise ValueError(f'A_log must have {HV} entries, got {A_log.numel()}')
+    if dt_bias is not None:
+        if dt_bias.numel() != HV * K:
+            raise ValueError(f'dt_bias must have HV * K = {HV * K} elements, got {dt_bias.numel()}')
+        dt_bias = _pad_last(dt_bias.detach().to(device=dev, dtype=torch.float32).reshape(HV, K), _DIM).contiguous()
+    h0 = None
+    if initial_state is not None:
+        h0 = as_f32(initial_state)
+        if state_v_first:
+            h0 = h0.transpose(-1, -2)
+        h0 = aligned16(F.pad(h0, (0, _DIM - V, 0, _DIM - K)).contiguous())
+
+    flags = 0
+    if use_qk_l2norm_in_kernel:
+        flags |= _lib.FLAG_QK_L2NORM
+    if use_beta_sigmoid_in_kernel:
+        flags |= _lib.FLAG_BETA_SIGMOID | (_lib.FLAG_NEG_EIGVAL if allow_neg_eigval else 0)
+    chunk_table = chunk_offsets = None
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype not in (torch.int32, torch.int64):
+            cu_seqlens = cu_seqlens.long()
+        cu_seqlens = cu_seqlens.to(dev)
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        chunk_table = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        chunk_table = chunk_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        chunk_offsets = prepare_scan_tables(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        num_chunks = chunk_table.shape[0]
+    else:
+        num_chunks = B * ((T + _CHUNK - 1) // _CHUNK)
+
+    o = torch.empty(B, T, HV, _DIM, dtype=work, device=dev)
+    ht = torch.empty(N, HV, _DIM, _DIM, dtype=torch.float32, device=dev) if output_final_state else None
+    lib = _lib.load()
+    ws_bytes = lib.gdn_chunk_kda_workspace_bytes(num_chunks, HV)
+    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _lib.check(lib.gdn_chunk_kda_fwd(
+        ptr(qw), ptr(kw), ptr(vw), ptr(gw), ptr(bw), ptr(A_log), ptr(dt_bias),
+        0.0 if lower_bound is None else float(lower_bound), gate_mode, ptr(h0), ptr(ht), ptr(o),
+        ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
+        B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
+        current_stream_ptr(dev)))
+    o = o[..., :V].to(out_dtype)
+    if ht is not None:
+        ht = ht[..., :K, :V]
+        ht = (ht.transpose(-1, -2) if state_v_first else ht).contiguous()
+    return o, ht
+
+
+@torch.compiler.disable
+def chunk_kda(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    scale: float | None = None,
+    initial_state: torch.Tensor | None = None,
+    output_final_state: bool = False,
+    use_qk_l2norm_in_kernel: bool = False,
+    use_gate_in_kernel: bool = False,
+    use_beta_sigmoid_in_kernel: bool = False,
+    allow_neg_eigval: bool = False,
+    safe_gate: bool = False,
+    lower_bound: float | None = None,
+    disable_recompute: bool = False,
+    return_intermediate_states: bool = False,
+    state_v_first: bool = False,
+    cu_seqlens: torch.LongTensor | None = None,
+    cu_seqlens_cpu: torch.LongTensor | None = None,
+    cp_context=None,
+    **kwargs,
+):
+    r"""Chunked KDA (prefill), forward only.
+
+    Args:
+        q, k: ``[B, T, H, K]``; v: ``[B, T, HV, V]`` with ``HV % H == 0``.
+        g: ``[B, T, HV, K]`` log decay per key feature, or the raw gate input with ``use_gate_in_kernel=True``
+            (``A_log [HV]`` and optional ``dt_bias [HV * K]`` as keywords: ``-exp(A_log) softplus(g + dt_bias)``, or with
+            ``lower_bound`` (``safe_gate``) ``lower_bound sigmoid(exp(A_log) (g + dt_bias))``).
+        beta: ``[B, T, HV]`` (logits with ``use_beta_sigmoid_in_kernel``; ``allow_neg_eigval`` doubles the sigmoid).
+        scale: defaults to ``K ** -0.5``.  initial_state: ``[N, HV, K, V]`` (``[N, HV, V, K]`` with ``state_v_first``).
+        safe_gate: accepted; the kernels form the intra-chunk decays pair by pair inside blocks of 16 rows whatever the
+            gate's range, so it changes nothing here.  disable_recompute: accepted, nothing is saved (forward only).
+        return_intermediate_states, cp_context: not part of this build.
+        cu_seqlens: ``[N + 1]`` boundaries of packed sequences (then ``B == 1``).
+
+    Returns:
+        ``(o [B, T, HV, V] in q's dtype, final_state or None)``.
+    """
+    if cp_context is not None:
+        raise NotImplementedError('context parallelism (cp_context) is outside this single-GPU build')
+    if return_intermediate_states:
+        raise NotImplementedError('return_intermediate_states: the per-chunk states never reach memory here')
+    if 'transpose_state_layout' in kwargs:
+        state_v_first = kwargs.pop('transpose_state_layout')
+    if cu_seqlens is not None:
+        if q.shape[0] != 1:
+            raise ValueError(
+                f'The batch size is expected to be 1 rather than {q.shape[0]} when using `cu_seqlens`.'
+                f'Please flatten variable-length inputs before processing.')
+        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+            raise ValueError(
+                f'The number of initial states is expected to be equal to the number of input sequences, '
+                f'i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.')
+    H, HV = q.shape[2], v.shape[2]
+    if q.shape[2] != k.shape[2] or HV % H != 0:
+        raise ValueError(f'q and k must share their heads and HV={HV} must be a multiple of H={H}')
+    if g.shape != (*v.shape[:3], k.shape[-1]):
+        raise ValueError(f'g must have shape {(*v.shape[:3], k.shape[-1])}, got {tuple(g.shape)}')
+    chunk_size = kwargs.pop('chunk_size', 64)
+    if chunk_size not in (16, 32, 64):
+        raise ValueError(f'`chunk_size` must be 16, 32, or 64, got {chunk_size}.')
+    if allow_neg_eigval and not use_beta_sigmoid_in_kernel:
+        raise ValueError('`allow_neg_eigval=True` requires `use_beta_sigmoid_in_kernel=True`.')
+    if safe_gate and lower_bound is None:
+        raise ValueError('`safe_gate=True` requires `lower_bound`.')
+    A_log, dt_bias = kwargs.get('A_log'), kwargs.get('dt_bias')
+    gate_mode = 0
+    if use_gate_in_kernel:
+        if A_log is None and lower_bound is None:
+            raise AssertionError('A_log must be provided when use_gate_in_kernel=True (unless lower_bound is set).')
+        gate_mode = 2 if lower_bound is not None else 1
+    else:
+        A_log = dt_bias = None
+    forward_only('chunk_kda', q, k, v, g, beta, initial_state)
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    return chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first, cu_seqlens,
+                         cu_seqlens_cpu, A_log, dt_bias, lower_bound, gate_mode, use_qk_l2norm_in_kernel,
+                         use_beta_sigmoid_in_kernel, allow_neg_eigval)

@@ -1,7 +1,7 @@
 """``fused_recurrent_kda``: the token recurrence of the KDA operator (the gated delta rule with a decay per key
 feature), forward only, with the signatures of fla/ops/kda/fused_recurrent.py:236-260 (``fused_recurrent_kda_fwd``, the
 serving form with state pools) and :341-492 (``fused_recurrent_kda``).  Both run the token-recurrence kernel of the gated
-delta rule through ``gdn_fused_recurrent_kda_fwd``; the chunked KDA prefill (``chunk_kda``) has no kernel here."""
+delta rule through ``gdn_fused_recurrent_kda_fwd``; the chunked prefill is ``chunk_kda`` (chunk.py)."""
 from __future__ import annotations
 
 import warnings

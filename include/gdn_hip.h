@@ -248,6 +248,31 @@ int gdn_l2norm_bwd(const void* dyh, const void* y, const float* rstd, void* dx, 
                    int64_t Dout, int dtype, void* stream);
 
 /*
+ * Chunked forward of the KDA operator (a decay per key feature).  Replaces chunk_kda_fwd (fla/ops/kda/chunk_fwd.py:20-134):
+ * the gate activation and chunk-local cumsum (fla/ops/kda/gate.py:27-94), chunk_kda_fwd_intra (fla/ops/kda/chunk_intra.py),
+ * recompute_w_u_fwd (fla/ops/kda/wy_fast.py), chunk_gated_delta_rule_fwd_h with gk (fla/ops/common/chunk_delta_h.py:687-744) and
+ * chunk_gla_fwd_o_gk (fla/ops/gla/chunk.py).
+ *   q, k [B,T,H,K]; v [B,T,HV,V] (bf16 or f16); g [B,T,HV,K] fp32: log decay per key feature, or the raw gate input with
+ *   gate_mode 1 (g <- -exp(A_log[hv]) softplus(g + dt_bias[hv][k])) or 2 (g <- lower_bound sigmoid(exp(A_log[hv]) (g + dt_bias[hv][k])));
+ *   A_log [HV] or NULL (then exp(A_log) reads as e in mode 1 and as 1 in mode 2, as in the token recurrence), dt_bias [HV,K] or NULL
+ *   beta [B,T,HV] (gb_dtype); h0, ht [N,HV,K,V] fp32 or NULL; o [B,T,HV,V] in qkv_dtype
+ *   cu_seqlens, chunk_table, chunk_offsets ([N+1]), N, num_chunks: as for gdn_chunk_fwd
+ *   workspace: at least gdn_chunk_kda_workspace_bytes(num_chunks, HV) bytes, 256-byte aligned
+ *   flags: GDN_FLAG_CU_INT32, GDN_FLAG_QK_L2NORM, GDN_FLAG_BETA_SIGMOID, GDN_FLAG_NEG_EIGVAL.  K = V = 128 only: the Python host
+ *   zero-pads smaller head dims and splits V > 128 into value heads of 128 columns.  T == 0: ht = h0 (zeros without h0).
+ */
+size_t gdn_chunk_kda_workspace_bytes(int64_t num_chunks, int64_t HV);
+int gdn_chunk_kda_fwd(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * gdn_chunk_fwd minus the workspace: the kernels use a fixed array of GDN_CHUNK_STATIC_WORKSPACE_BYTES that the

@@ -216,3 +216,154 @@ def test_upstream_kda_backend_takes_gpu_inference_calls_and_leaves_the_rest():
     assert fused_recurrent_kda_fwd(q, k, v, g, beta, initial_state=h0)[0] == 'default'                       # CPU stays upstream
     assert fused_recurrent_kda_fwd(dq.requires_grad_(), dk, dv, dg, db, initial_state=dh)[0] == 'default'    # training stays upstream
     assert fused_recurrent_kda_fwd(dq.detach(), dk, dv, dg, db, initial_state=dh.bfloat16())[0] == 'default'
+
+
+# --------------------------------------------------------------------------------------------
+# chunked prefill (chunk_kda) against the oracle's token recurrence
+# --------------------------------------------------------------------------------------------
+def _chunk_inputs(B, T, H, HV, D, gate_div, mask_p, gate_in_kernel, safe_gate, dtype, seed=42, V=None):
+    gen = torch.Generator().manual_seed(seed)
+    V = D if V is None else V
+    q = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    k = torch.rand(B, T, H, D, generator=gen).to(dtype)
+    v = torch.rand(B, T, HV, V, generator=gen).to(dtype)
+    g = torch.randn(B, T, HV, D, generator=gen)
+    A_log = dt_bias = None
+    if gate_in_kernel:
+        A_log = torch.randn(HV, generator=gen)
+        dt_bias = torch.randn(HV * D, generator=gen)
+    else:
+        g = F.logsigmoid(g) / gate_div
+        g = g * (torch.rand(B, T, HV, D, generator=gen) > mask_p)
+        if safe_gate:
+            g = g.clamp(-5, 0)
+    beta = torch.randn(B, T, HV, generator=gen).sigmoid()
+    h0 = torch.randn(B, HV, D, V, generator=gen)
+    return q, k, v, g, beta, h0, A_log, dt_bias
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_div,mask_p,l2,gate_in_kernel,dtype,safe_gate', [
+    (1, 63, 1, 1, 64, 1, 1, 0, False, False, torch.float16, True),          # the reference's matrix, tests/ops/test_kda.py:535-560
+    (2, 500, 3, 3, 60, 1, 1, 0, False, False, torch.float16, True),
+    (2, 1000, 3, 3, 64, 0.1, 1, 0.5, False, False, torch.float16, False),
+    (3, 1024, 4, 4, 100, 1, 0.1, 0, False, False, torch.float16, False),
+    (4, 1024, 4, 4, 128, 0.1, 1, 0, False, False, torch.float16, True),
+    (4, 1024, 4, 4, 128, 0.1, 1, 0, True, False, torch.float16, True),
+    (2, 1500, 4, 4, 128, 0.1, 10, 0, False, True, torch.float16, False),
+    (4, 2048, 8, 8, 64, 0.1, 1, 0, False, True, torch.float16, True),
+    (2, 1024, 2, 4, 64, 0.1, 1, 0, False, False, torch.float16, False),
+    (2, 1024, 2, 8, 64, 0.1, 1, 0, False, True, torch.float16, False),
+    (2, 1024, 4, 8, 128, 0.1, 1, 0, True, True, torch.float16, False),
+    (2, 1024, 2, 4, 64, 0.1, 1, 0, True, True, torch.bfloat16, True),
+    (2, 1024, 2, 8, 128, 0.1, 1, 0, True, True, torch.bfloat16, False),
+])
+def test_chunk_kda_reference_matrix(B, T, H, HV, D, scale, gate_div, mask_p, l2, gate_in_kernel, dtype, safe_gate):
+    from fla_hip.ops.kda import chunk_kda
+    q, k, v, g, beta, h0, A_log, dt_bias = _chunk_inputs(B, T, H, HV, D, gate_div, mask_p, gate_in_kernel, safe_gate, dtype)
+    lower_bound = -5.0 if safe_gate else None
+    if not l2:
+        q, k = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, scale, h0, True, use_qk_l2norm_in_kernel=l2,
+                                    use_gate_in_kernel=gate_in_kernel, A_log=A_log, dt_bias=dt_bias, lower_bound=lower_bound)
+    dev = 'cuda'
+    d = lambda x: None if x is None else x.to(dev)
+    o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), scale=scale, initial_state=d(h0), output_final_state=True,
+                      use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel, A_log=d(A_log), dt_bias=d(dt_bias),
+                      safe_gate=safe_gate, lower_bound=lower_bound)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and o.shape == v.shape
+    # (the reference's bars for o and the final state: tests/ops/test_kda.py:640-641)
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.005
+    assert O.get_err_ratio(ref_ht, ht.cpu()) < 0.005
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('H,D,mask_p,cu,gate_in_kernel,safe_gate', [
+    (4, 60, 0.1, [0, 15], True, False),
+    (4, 64, 0.9, [0, 256, 500, 1000], True, False),
+    (4, 128, 0.5, [0, 256, 500, 1000], False, False),
+    (4, 100, 0, [0, 15, 100, 300, 1200, 2000], True, False),
+    (2, 128, 0, [0, 1, 65, 65, 200], False, True),
+])
+def test_chunk_kda_packed(H, D, mask_p, cu, gate_in_kernel, safe_gate):
+    """Packed sequences (tests/ops/test_kda.py:839-960), one of them empty, int32 boundaries, every sequence alone = packed."""
+    from fla_hip.ops.kda import chunk_kda
+    T, N = cu[-1], len(cu) - 1
+    dtype = torch.float16
+    q, k, v, g, beta, _, A_log, dt_bias = _chunk_inputs(1, T, H, H, D, 1.0, mask_p, gate_in_kernel, safe_gate, dtype, seed=7)
+    gen = torch.Generator().manual_seed(8)
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    lower_bound = -5.0 if safe_gate else None
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=gate_in_kernel, lower_bound=lower_bound)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, A_log=A_log, dt_bias=dt_bias, **kw)
+    dev = 'cuda'
+    d = lambda x: None if x is None else x.to(dev)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), initial_state=d(h0), output_final_state=True, cu_seqlens=cu_t,
+                      A_log=d(A_log), dt_bias=d(dt_bias), safe_gate=safe_gate, **kw)
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.005 and O.get_err_ratio(ref_ht, ht.cpu()) < 0.005
+    for n in range(N):
+        s, e = cu[n], cu[n + 1]
+        if e == s:
+            assert torch.equal(ht[n].cpu(), h0[n])
+            continue
+        o1, ht1 = chunk_kda(d(q[:, s:e]), d(k[:, s:e]), d(v[:, s:e]), d(g[:, s:e]), d(beta[:, s:e]), initial_state=d(h0[n:n + 1]),
+                            output_final_state=True, A_log=d(A_log), dt_bias=d(dt_bias), safe_gate=safe_gate, **kw)
+        assert torch.equal(o1[0], o[0, s:e]) and torch.equal(ht1[0], ht[n])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('what', ['v_first', 'beta_sigmoid', 'beta_sigmoid_neg', 'wide_v', 'no_h0', 'strong_decay', 'bf16_hand_over'])
+def test_chunk_kda_options(what):
+    from fla_hip.ops.kda import chunk_kda, fused_recurrent_kda
+    B, T, H, HV, D = 2, 200, 2, 4, 128
+    V = 256 if what == 'wide_v' else D
+    dtype = torch.bfloat16
+    q, k, v, g, beta, h0, _, _ = _chunk_inputs(B, T, H, HV, D, 0.05 if what == 'strong_decay' else 4.0, 0, False, False, dtype, seed=3, V=V)
+    kw = dict(use_qk_l2norm_in_kernel=True)
+    gen = torch.Generator().manual_seed(4)
+    if what.startswith('beta_sigmoid'):
+        beta = torch.randn(B, T, HV, generator=gen)
+        kw.update(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=what.endswith('neg'))
+    if what == 'no_h0':
+        h0 = None
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, **kw)
+    dev = 'cuda'
+    d = lambda x: None if x is None else x.to(dev)
+    if what == 'v_first':
+        o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), initial_state=d(h0.transpose(-1, -2).contiguous()), output_final_state=True,
+                          state_v_first=True, **kw)
+        ht = ht.transpose(-1, -2)
+    else:
+        o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), initial_state=d(h0), output_final_state=True, **kw)
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.005 and O.get_err_ratio(ref_ht, ht.cpu()) < 0.005
+    if what == 'bf16_hand_over':
+        # prefill in two calls chained through the state, then a token of the recurrence: the same as one pass of the oracle
+        o1, h1 = chunk_kda(d(q[:, :130]), d(k[:, :130]), d(v[:, :130]), d(g[:, :130]), d(beta[:, :130]), initial_state=d(h0),
+                           output_final_state=True, **kw)
+        o2, h2 = chunk_kda(d(q[:, 130:199]), d(k[:, 130:199]), d(v[:, 130:199]), d(g[:, 130:199]), d(beta[:, 130:199]),
+                           initial_state=h1, output_final_state=True, **kw)
+        o3, h3 = fused_recurrent_kda(d(q[:, 199:]), d(k[:, 199:]), d(v[:, 199:]), d(g[:, 199:]), d(beta[:, 199:]), initial_state=h2,
+                                     output_final_state=True, **kw)
+        joined = torch.cat([o1, o2, o3], dim=1)
+        assert O.get_err_ratio(ref_o, joined.float().cpu()) < 0.005 and O.get_err_ratio(ref_ht, h3.cpu()) < 0.005
+
+
+@pytest.mark.gpu
+def test_chunk_kda_validation():
+    from fla_hip.ops.kda import chunk_kda
+    x = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16, device='cuda')
+    g = torch.zeros(1, 64, 2, 64, device='cuda')
+    b = torch.zeros(1, 64, 2, device='cuda')
+    with pytest.raises(ValueError):
+        chunk_kda(x, x, x, g, b, allow_neg_eigval=True)
+    with pytest.raises(ValueError):
+        chunk_kda(x, x, x, g, b, safe_gate=True)
+    with pytest.raises(ValueError):
+        chunk_kda(x, x, x, g[..., :32], b)
+    with pytest.raises(NotImplementedError):
+        chunk_kda(x, x, x, g, b, return_intermediate_states=True)
+    with pytest.raises(NotImplementedError):
+        chunk_kda(x.requires_grad_(), x, x, g, b)
+    o, ht = chunk_kda(x[:, :0].detach(), x[:, :0].detach(), x[:, :0].detach(), g[:, :0], b[:, :0], output_final_state=True)
+    assert o.shape == (1, 0, 2, 64) and torch.count_nonzero(ht) == 0
