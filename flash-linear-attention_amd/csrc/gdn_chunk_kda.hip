@@ -49,36 +49,48 @@ struct KdaParams {
 constexpr size_t KDA_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PG + 64 * PL + 64) * 4;
 
 template <typename T>
-__global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
+__global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
     float* sG = (float*)(sA + 64 * P64); float* sL = sG + 64 * PG; float* sBeta = sL + 64 * PL;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int64_t u = blockIdx.x, ci = u / p.HV;
-    const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-    const ChunkAt c = chunk_at(p, ci);
 
-    load_tile<BD>(sK, P128, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    load_tile<BD>(sQ, P128, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-    load_tile<BD>(sV, P128, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-    {
-        // gates: a thread per key feature and half of the chunk's rows; running sums inside the half first
+    // One workgroup per CU walks over the units; the next unit's rows and gates are fetched into registers meanwhile.
+    TileRegs<BD> rK, rQ, rV;
+    float rG[32], rB = 0.f;                                     // gates: a thread per key feature and half of the chunk's rows
+    auto fetch = [&](int64_t u) {
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         const int col = tid & 127, half = tid >> 7;
-        const float a_k = p.gk_act ? (p.A_log ? __expf(p.A_log[hv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
-        const float bias = (p.gk_act && p.gk_bias) ? p.gk_bias[hv * BD + col] : 0.f;
-        float x[32];
 #pragma unroll
         for (int r = 0; r < 32; ++r) {
             const int row = 32 * half + r;
-            x[r] = row < c.valid ? p.g[((c.tok0 + row) * p.HV + hv) * BD + col] : 0.f;
+            rG[r] = row < c.valid ? p.g[((c.tok0 + row) * p.HV + hv) * BD + col] : 0.f;
         }
+        rB = (tid < 64 && tid < c.valid) ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+    };
+    fetch(blockIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+    const int hv = (int)(u % p.HV);
+    const ChunkAt c = chunk_at(p, u / p.HV);
+    put_tile<BD>(sK, P128, rK, tid);
+    put_tile<BD>(sQ, P128, rQ, tid);
+    put_tile<BD>(sV, P128, rV, tid);
+    {
+        // running sums of the gates inside each half of the rows first
+        const int col = tid & 127, half = tid >> 7;
+        const float a_k = p.gk_act ? (p.A_log ? __expf(p.A_log[hv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
+        const float bias = (p.gk_act && p.gk_bias) ? p.gk_bias[hv * BD + col] : 0.f;
         float run = 0.f;
 #pragma unroll
         for (int r = 0; r < 32; ++r) {
             const int row = 32 * half + r;
-            float gt = x[r];
+            float gt = rG[r];
             if (p.gk_act && row < c.valid) {
                 gt += bias;
                 gt = p.gk_act == 2 ? p.gk_lower * sigmoid_f(a_k * gt) : -a_k * softplus_f(gt);
@@ -88,11 +100,12 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
         }
     }
     if (tid < 64) {
-        float b = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        float b = rB;
         if ((p.flags & GDN_FLAG_BETA_SIGMOID) && tid < c.valid) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
         sBeta[tid] = b;
     }
-    __syncthreads();
+    lds_barrier();
+    if (u + gridDim.x < units) fetch(u + gridDim.x);
     {
         // second half of the rows: add the first half's total
         const int col = tid & 127, half = tid >> 7;
@@ -121,52 +134,86 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // ---- M (as L = diag(beta) M, for the substitution) and P, this wave's 16 rows ----
     {
         T* Pu = (T*)p.ws.Pm + u * 64 * 64;
         const int i = 16 * w + c16;                             // the row this lane's operand fragments belong to
-        // rows of this block against rows of earlier blocks: reference = the row in front of the block
-        if (w > 0) {
-            V8 kd[4], qd[4];
-            float ref[4][8];
+        // rows of this block against rows of earlier blocks: reference = the row in front of the block (zeros for block 0)
+        V8 kd[4], qd[4];
+        float ref[4][8];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const float* gi = sG + i * PG + 32 * s + 8 * g;
-                const float* gr = sG + (16 * w - 1) * PG + 32 * s + 8 * g;
-                const V8 kx = frag_rows(sK, P128, 16 * w, 32 * s, lane), qx = frag_rows(sQ, P128, 16 * w, 32 * s, lane);
+        for (int s = 0; s < 4; ++s) {
+            const float* gi = sG + i * PG + 32 * s + 8 * g;
+            const float* gr = sG + (16 * w - 1) * PG + 32 * s + 8 * g;
+            const V8 kx = frag_rows(sK, P128, 16 * w, 32 * s, lane), qx = frag_rows(sQ, P128, 16 * w, 32 * s, lane);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    ref[s][e] = gr[e];
-                    const float f = __expf(gi[e] - gr[e]);
-                    kd[s][e] = (T)((float)kx[e] * f);
-                    qd[s][e] = (T)((float)qx[e] * f);
-                }
-            }
-#pragma unroll
-            for (int tj = 0; tj < 3; ++tj) {
-                if (tj >= w) break;
-                f32x4 m = ZERO4, pt = ZERO4;
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const float* gj = sG + (16 * tj + c16) * PG + 32 * s + 8 * g;
-                    V8 kn = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
-                    m = Mma<T>::run(kd[s], kn, m);             // lane: column j = 16tj + c16, rows i = 16w + 4g + r
-                    pt = Mma<T>::run(kn, qd[s], pt);           // lane: column i = 16w + c16, rows j = 16tj + 4g + r
-                }
-                const int j = 16 * tj + c16;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int ir = 16 * w + 4 * g + r;
-                    sL[ir * PL + (j & 3) * 16 + (j >> 2)] = sBeta[ir] * m[r];
-                }
-                *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(pt * p.scale);
+            for (int e = 0; e < 8; ++e) {
+                ref[s][e] = w > 0 ? gr[e] : 0.f;
+                const float f = __expf(gi[e] - ref[s][e]);
+                kd[s][e] = (T)((float)kx[e] * f);
+                qd[s][e] = (T)((float)qx[e] * f);
             }
         }
-        // the diagonal block: lane (il, jq) takes row il and columns 4jq .. 4jq+3 of the block, every pair with its own exponentials
+#pragma unroll
+        for (int tj = 0; tj < 3; ++tj) {
+            if (tj >= w) break;
+            f32x4 m = ZERO4, pt = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float* gj = sG + (16 * tj + c16) * PG + 32 * s + 8 * g;
+                V8 kn = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
+                m = Mma<T>::run(kd[s], kn, m);                 // lane: column j = 16tj + c16, rows i = 16w + 4g + r
+                pt = Mma<T>::run(kn, qd[s], pt);               // lane: column i = 16w + c16, rows j = 16tj + 4g + r
+            }
+            const int j = 16 * tj + c16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int ir = 16 * w + 4 * g + r;
+                sL[ir * PL + (j & 3) * 16 + (j >> 2)] = sBeta[ir] * m[r];
+            }
+            *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(pt * p.scale);
+        }
+        // blocks to the right of the diagonal: zeros
+#pragma unroll
+        for (int tj = 1; tj < 4; ++tj)
+            if (tj > w) *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(ZERO4);
+        // The diagonal block.  Where the decay across the block stays within what the operand type can hold as a factor
+        // e^(ref - Gam_j) >= 1 (the usual case), the same reference serves and the block is one more tile on the matrix
+        // cores; otherwise every pair of rows gets its own exponentials.
+        float span = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int col = lane + 64 * h;
+            span = fminf(span, sG[(16 * w + 15) * PG + col] - (w > 0 ? sG[(16 * w - 1) * PG + col] : 0.f));
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) span = fminf(span, __shfl_xor(span, off, 64));
+        constexpr float SPAN_OK = std::is_same<T, bf16_t>::value ? -80.f : -8.f;
+        if (span >= SPAN_OK) {
+            f32x4 m = ZERO4, pt = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float* gj = sG + i * PG + 32 * s + 8 * g;
+                V8 kn = frag_rows(sK, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
+                m = Mma<T>::run(kd[s], kn, m);                 // lane: column j = 16w + c16, rows i = 16w + 4g + r
+                pt = Mma<T>::run(kn, qd[s], pt);               // lane: column i = 16w + c16, rows j = 16w + 4g + r
+            }
+            const int j = 16 * w + c16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int ir = 16 * w + 4 * g + r;
+                sL[ir * PL + (j & 3) * 16 + (j >> 2)] = ir > j ? sBeta[ir] * m[r] : 0.f;
+                pt[r] = (16 * w + 4 * g + r) <= i ? pt[r] * p.scale : 0.f;
+            }
+            *(V4*)(Pu + i * 64 + 16 * w + 4 * g) = pack4<T>(pt);
+        } else
+        // (lane (il, jq) takes row il and columns 4jq .. 4jq+3 of the block)
         {
             const int il = lane >> 2, jq = lane & 3, row = 16 * w + il;
             float m[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
@@ -197,15 +244,11 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
                 pt[jj] = jl <= il ? p.scale * pq[jj] : 0.f;
             }
             *(V4*)(Pu + row * 64 + 16 * w + 4 * jq) = pack4<T>(pt);
-            // blocks to the right of the diagonal: zeros
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj)
-                if (tj > w) *(V4*)(Pu + row * 64 + 16 * tj + 4 * jq) = pack4<T>(ZERO4);
         }
     }
-    __syncthreads();
+    lds_barrier();
     solve_unit_lower<T>(sL, sA, w, lane);
-    __syncthreads();
+    lds_barrier();
     {
         // what the scan needs of q and k, and k, v as the factors of w, u
         T* QGu = (T*)p.ws.QG + u * 64 * BD;
@@ -232,7 +275,7 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
         }
         if (tid < BD) p.ws.EGL[u * BD + tid] = __expf(sG[63 * PG + tid]);
     }
-    __syncthreads();
+    lds_barrier();
     {
         // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
         T* Wu = (T*)p.ws.Wm + u * 64 * BD;
@@ -253,6 +296,8 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p) {
             *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
             *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
         }
+    }
+    lds_barrier();
     }
 }
 
@@ -396,10 +441,11 @@ static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream
     if (vbt == 32) scan = {(const void*)gdn_kda_scan_kernel<T, 32>, kda_scan_smem<32>(), "gdn_kda_scan_kernel", runs};
     else if (vbt == 64) scan = {(const void*)gdn_kda_scan_kernel<T, 64>, kda_scan_smem<64>(), "gdn_kda_scan_kernel", runs};
     else scan = {(const void*)gdn_kda_scan_kernel<T, 128>, kda_scan_smem<128>(), "gdn_kda_scan_kernel", runs};
-    const K ks[2] = {{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units}, scan};
+    const K ks[2] = {{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 256u ? units : 256u}, scan};
     for (int i = 0; i < 2; ++i) {
         if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
-        void* args[] = {(void*)&p};
+        int64_t nunits = units;
+        void* args[] = {(void*)&p, (void*)&nunits};             // (the prepare kernel walks over the units and takes their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
     }
