@@ -253,6 +253,19 @@ def bench_train(w, steps, warmup, device):
                 tokens_per_s=round(w['B'] * w['T'] / per_call, 1))
 
 
+def bench_kda(steps, warmup, device):
+    """Chunked prefill of the sibling KDA operator (a decay per key feature) on one of the published GDN shapes."""
+    from fla_hip.ops.kda import chunk_kda
+    B, T, H, D = 1, 8192, 96, 128
+    gen = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(B, T, H, D, generator=gen).bfloat16().to(device) for _ in range(3))
+    g = (F.logsigmoid(torch.randn(B, T, H, D, generator=gen)) / 4).to(device)
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=gen)).to(device)
+    per_call, _ = _time_calls(lambda: chunk_kda(q, k, v, g, beta, use_qk_l2norm_in_kernel=True), steps, warmup)
+    return dict(workload=f'chunk_kda forward B={B} T={T} H={H} K=V={D} bf16, fp32 log decays per key feature, in-kernel l2 norm',
+                ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
+
+
 def cpu_baseline_prefill(w, cpu):
     """Oracle (torch fp32 chunked form) on the first tokens of the same inputs; the sample
     length is chosen from a short calibration run so that the timed run takes ~10-20 s."""
@@ -542,6 +555,7 @@ def main():
         for name, ww in PUBLISHED.items():
             extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
             torch.cuda.empty_cache()
+        extra['chunk_kda_b1_t8192_h96_d128'] = bench_kda(max(10, args.steps // 4), max(3, args.warmup // 4), device)
         line['other_workloads'] = extra
     print(json.dumps(line))
 

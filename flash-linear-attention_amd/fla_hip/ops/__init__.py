@@ -1,5 +1,5 @@
 from fla_hip.ops.delta_rule import chunk_delta_rule, fused_recurrent_delta_rule
-from fla_hip.ops.kda import fused_recurrent_kda
+from fla_hip.ops.kda import chunk_kda, fused_recurrent_kda
 from fla_hip.ops.gated_delta_rule import (
     chunk_gated_delta_rule,
     chunk_gdn,
@@ -8,4 +8,4 @@ from fla_hip.ops.gated_delta_rule import (
 )
 
 __all__ = ['chunk_delta_rule', 'fused_recurrent_delta_rule', 'chunk_gated_delta_rule', 'chunk_gdn', 'fused_recurrent_gated_delta_rule', 'fused_recurrent_gdn',
-           'fused_recurrent_kda']
+           'chunk_kda', 'fused_recurrent_kda']

@@ -6,7 +6,7 @@ whole operator and ``fla/modules/backends/triton_ascend`` for module functions).
     fla_hip.upstream.register()        # needs `fla` importable; registers for 'gated_delta_rule', 'modules' and 'kda'
 
 Upstream's ``@dispatch`` then offers every call of ``chunk_gated_delta_rule``, ``causal_conv1d_fwd``,
-``causal_conv1d_update_states``, ``causal_conv1d_update``, ``layer_norm_gated_fwd`` and ``fused_recurrent_kda_fwd``
+``causal_conv1d_update_states``, ``causal_conv1d_update``, ``layer_norm_gated_fwd``, ``chunk_kda`` and ``fused_recurrent_kda_fwd``
 (the KDA operator's token recurrence, ``fla/ops/kda/fused_recurrent.py:236``) to the verifier below first;
 a rejected call (other device, gradients needed, a shape outside the kernels) falls through to upstream's own
 implementation.  The classes are built on whatever ``BaseBackend`` they are given, so the same code serves this
@@ -119,7 +119,7 @@ def make_backends(BaseBackend):
 
 
 def make_kda_backend(BaseBackend):
-    """Backend for the 'kda' registry: the token recurrence only (the chunked KDA prefill stays upstream)."""
+    """Backend for the 'kda' registry: the token recurrence and the chunked prefill (forward; training stays upstream)."""
 
     class HipGfx950KDABackend(BaseBackend):
         backend_type = 'hip_gfx950'
@@ -144,6 +144,23 @@ def make_kda_backend(BaseBackend):
         def fused_recurrent_kda_fwd(self, *args, **kwargs):
             from fla_hip.ops.kda import fused_recurrent_kda_fwd
             return fused_recurrent_kda_fwd(*args, **kwargs)
+
+        def chunk_kda_verifier(self, q, k, v, g, beta, *args, cp_context=None, return_intermediate_states=False, **kwargs):
+            if not _on_gfx950(q):
+                return False, 'not a gfx950 device'
+            if cp_context is not None or return_intermediate_states:
+                return False, 'context parallelism and intermediate states are not supported'
+            if _needs_grad(q, k, v, g, beta, kwargs.get('initial_state'), kwargs.get('A_log'), kwargs.get('dt_bias')):
+                return False, 'forward only: a tensor requires grad'
+            if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+                return False, f'dtype {q.dtype}'
+            if k.shape[-1] > 128:
+                return False, 'key head dim above 128'
+            return True, None
+
+        def chunk_kda(self, *args, **kwargs):
+            from fla_hip.ops.kda import chunk_kda
+            return chunk_kda(*args, **kwargs)
 
     return HipGfx950KDABackend
 

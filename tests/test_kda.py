@@ -217,6 +217,21 @@ def test_upstream_kda_backend_takes_gpu_inference_calls_and_leaves_the_rest():
     assert fused_recurrent_kda_fwd(dq.requires_grad_(), dk, dv, dg, db, initial_state=dh)[0] == 'default'    # training stays upstream
     assert fused_recurrent_kda_fwd(dq.detach(), dk, dv, dg, db, initial_state=dh.bfloat16())[0] == 'default'
 
+    @dispatch('upstream_test_kda')
+    def chunk_kda(q, k, v, g, beta, scale=None, initial_state=None, output_final_state=False, **kwargs):
+        return 'default', None
+
+    q, k, v, g, beta, h0 = _inputs(1, 150, 2, 4, 64)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, use_qk_l2norm_in_kernel=True)
+    dq, dk, dv, dg, db, dh = _cuda(q, k, v, g, beta, h0)
+    o, ht = chunk_kda(dq.bfloat16(), dk.bfloat16(), dv.bfloat16(), dg, db, initial_state=dh, output_final_state=True,
+                      use_qk_l2norm_in_kernel=True)
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.01 and O.get_err_ratio(ref_ht, ht.cpu()) < 0.01
+    assert chunk_kda(q, k, v, g, beta)[0] == 'default'                                                        # CPU stays upstream
+    assert chunk_kda(dq.bfloat16().requires_grad_(), dk.bfloat16(), dv.bfloat16(), dg, db)[0] == 'default'    # training stays upstream
+    wide = torch.zeros(1, 150, 2, 192, device='cuda', dtype=torch.bfloat16)
+    assert chunk_kda(wide, wide, dv.bfloat16(), torch.zeros(1, 150, 4, 192, device='cuda'), db)[0] == 'default'
+
 
 # --------------------------------------------------------------------------------------------
 # chunked prefill (chunk_kda) against the oracle's token recurrence
