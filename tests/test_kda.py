@@ -382,3 +382,56 @@ def test_chunk_kda_validation():
         chunk_kda(x.requires_grad_(), x, x, g, b)
     o, ht = chunk_kda(x[:, :0].detach(), x[:, :0].detach(), x[:, :0].detach(), g[:, :0], b[:, :0], output_final_state=True)
     assert o.shape == (1, 0, 2, 64) and torch.count_nonzero(ht) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('seed', range(16))
+def test_chunk_kda_random(seed):
+    """Seeded random combinations of head dims, grouping, packing, gate form and range, prologues, state layout and dtype."""
+    import random
+    from fla_hip.ops.kda import chunk_kda
+    rnd = random.Random(500 + seed)
+    D = rnd.choice([16, 40, 64, 96, 128])
+    V = rnd.choice([D, 64, 192]) if seed % 4 == 0 else D
+    H = rnd.choice([1, 2, 3])
+    HV = H * rnd.choice([1, 1, 2, 4])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    if rnd.random() < 0.4:
+        cu = [0]
+        for _ in range(rnd.randint(1, 4)):
+            cu.append(cu[-1] + rnd.choice([1, 7, 63, 64, 65, 130, 200]))
+        B, T, N = 1, cu[-1], len(cu) - 1
+    else:
+        B, T, cu = rnd.randint(1, 3), rnd.choice([1, 5, 64, 100, 129, 257]), None
+        N = B
+    gen = torch.Generator().manual_seed(600 + seed)
+    q, k = torch.randn(B, T, H, D, generator=gen).to(dtype), torch.randn(B, T, H, D, generator=gen).to(dtype)
+    v = torch.randn(B, T, HV, V, generator=gen).to(dtype)
+    kw = dict(use_qk_l2norm_in_kernel=True)
+    A_log = dt_bias = None
+    mode = rnd.choice(['plain', 'strong', 'softplus', 'lower_bound'])
+    g = torch.randn(B, T, HV, D, generator=gen)
+    if mode in ('plain', 'strong'):
+        g = F.logsigmoid(g) / (0.05 if mode == 'strong' else rnd.choice([1.0, 8.0]))
+    else:
+        A_log = torch.randn(HV, generator=gen) * 0.5
+        dt_bias = torch.randn(HV * D, generator=gen) * 0.5 if rnd.random() < 0.6 else None
+        kw.update(use_gate_in_kernel=True)
+        if mode == 'lower_bound':
+            kw.update(lower_bound=-5.0, safe_gate=True)
+    beta = torch.rand(B, T, HV, generator=gen).sigmoid()
+    if rnd.random() < 0.3:
+        beta = torch.randn(B, T, HV, generator=gen)
+        kw.update(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=rnd.random() < 0.5)
+    h0 = torch.randn(N, HV, D, V, generator=gen) * 0.5 if rnd.random() < 0.7 else None
+    okw = {n: x for n, x in kw.items() if n != 'safe_gate'}
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, A_log=A_log, dt_bias=dt_bias, **okw)
+    d = lambda x: None if x is None else x.cuda()
+    vfirst = h0 is not None and rnd.random() < 0.3
+    h_in = h0.transpose(-1, -2).contiguous() if vfirst else h0
+    o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), initial_state=d(h_in), output_final_state=True, state_v_first=vfirst,
+                      cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'), A_log=d(A_log), dt_bias=d(dt_bias), **kw)
+    if vfirst:
+        ht = ht.transpose(-1, -2)
+    bar = 0.005 if T >= 64 else 0.01
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < bar and O.get_err_ratio(ref_ht, ht.cpu()) < bar
