@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -469,7 +469,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
@@ -498,6 +498,12 @@ def main():
         return
     for key, val in WORKLOADS.items():
         val['key'] = key
+    if args.workload == 'chunk_kda':
+        r = bench_kda(args.steps, args.warmup, device)
+        print(json.dumps(dict(metric='kda_chunk_prefill_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
+                              n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
+                              data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
+        return
     if args.workload.startswith('train_'):
         name = args.workload[len('train_'):]
         r = bench_train(dict(PUBLISHED[name], key=name), args.steps, args.warmup, device)
