@@ -1,6 +1,8 @@
 // Error channel and version of the C ABI.
 #include "gdn_common.h"
 #include <algorithm>
+#include <mutex>
+#include <unordered_map>
 
 namespace gdn {
 static thread_local char g_err[512] = {0};
@@ -9,6 +11,13 @@ void set_error(const char* fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+int ensure_dynamic_smem_for(const void* kernel, size_t bytes, const char* what) {
+    static std::mutex lock;
+    static std::unordered_map<const void*, SmemAttrDone> table;
+    std::lock_guard<std::mutex> hold(lock);
+    return ensure_dynamic_smem(kernel, bytes, table[kernel], what);
 }
 
 // dst = src (or zero when src is NULL), `count` floats, count a multiple of 4 and both 16-byte aligned or anything

@@ -1010,8 +1010,7 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
     };
     for (int i = 0; i < 5; ++i) {
         if (ks[i].grid == 0) continue;
-        // (the limit on dynamic LDS belongs to the function: asked for on every call, it is a cheap host-side setting)
-        if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
+        if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
         int64_t nunits = units;
         void* args[] = {(void*)&p, (void*)&nunits};             // (the kernels that walk over the units take their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(threads[i]), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);

@@ -443,7 +443,7 @@ static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream
     else scan = {(const void*)gdn_kda_scan_kernel<T, 128>, kda_scan_smem<128>(), "gdn_kda_scan_kernel", runs};
     const K ks[2] = {{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 256u ? units : 256u}, scan};
     for (int i = 0; i < 2; ++i) {
-        if (hipFuncSetAttribute(ks[i].f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ks[i].smem) != hipSuccess) return check_launch(ks[i].name);
+        if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
         int64_t nunits = units;
         void* args[] = {(void*)&p, (void*)&nunits};             // (the prepare kernel walks over the units and takes their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);

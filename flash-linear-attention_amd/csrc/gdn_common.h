@@ -44,6 +44,9 @@ inline int ensure_dynamic_smem(const void* kernel, size_t bytes, SmemAttrDone& d
     return GDN_OK;
 }
 
+// The same for launchers that pick among many kernels at run time: the table is kept here, one entry per kernel.
+int ensure_dynamic_smem_for(const void* kernel, size_t bytes, const char* what);
+
 // ---- element types -------------------------------------------------------
 typedef __bf16 bf16_t;
 typedef _Float16 f16_t;
