@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -266,6 +266,19 @@ def bench_kda(steps, warmup, device):
                 ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
 
 
+def bench_comba(steps, warmup, device):
+    """Chunked prefill of the sibling comba operator (a second key for the prediction) on one of the published GDN shapes."""
+    from fla_hip.ops.comba import chunk_comba
+    B, T, H, D = 1, 8192, 96, 128
+    gen = torch.Generator().manual_seed(42)
+    q, k, v, p = (torch.randn(B, T, H, D, generator=gen).bfloat16().to(device) for _ in range(4))
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen)).to(device)
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=gen)).to(device)
+    per_call, _ = _time_calls(lambda: chunk_comba(q, k, v, p, g, beta, use_qk_l2norm_in_kernel=True), steps, warmup)
+    return dict(workload=f'chunk_comba forward B={B} T={T} H={H} K=V={D} bf16, fp32 log decays, in-kernel l2 norm of q, k, p',
+                ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
+
+
 def cpu_baseline_prefill(w, cpu):
     """Oracle (torch fp32 chunked form) on the first tokens of the same inputs; the sample
     length is chosen from a short calibration run so that the timed run takes ~10-20 s."""
@@ -469,7 +482,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'chunk_comba', 'layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
@@ -501,6 +514,12 @@ def main():
     if args.workload == 'chunk_kda':
         r = bench_kda(args.steps, args.warmup, device)
         print(json.dumps(dict(metric='kda_chunk_prefill_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
+                              n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
+                              data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
+        return
+    if args.workload == 'chunk_comba':
+        r = bench_comba(args.steps, args.warmup, device)
+        print(json.dumps(dict(metric='comba_chunk_prefill_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
                               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
                               data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
         return
@@ -562,6 +581,7 @@ def main():
             extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
             torch.cuda.empty_cache()
         extra['chunk_kda_b1_t8192_h96_d128'] = bench_kda(max(10, args.steps // 4), max(3, args.warmup // 4), device)
+        extra['chunk_comba_b1_t8192_h96_d128'] = bench_comba(max(10, args.steps // 4), max(3, args.warmup // 4), device)
         line['other_workloads'] = extra
     print(json.dumps(line))
 

@@ -15,6 +15,10 @@
 // block than i the reference is the last row in front of i's block, e^(Gam_i - ref) e^(ref - Gam_j) with both exponents <= 0,
 // and the products run on the matrix cores; inside a 16 x 16 diagonal block every pair gets its own exponentials
 // (the reference does the same, fla/ops/kda/chunk_intra.py: sub-chunks of 16).
+//
+// The comba operator (one decay per token and head, a second key p for the prediction, which sees the state before the
+// token's decay; fla/ops/comba/chunk.py:22-90) has a prepare kernel of its own that writes the same per-chunk operands,
+// and shares the scan:  M_ij = (p_i . k_j) e^(Gam0_i - Gam_j) with Gam0 = Gam - g,  w = A (beta p e^Gam0).
 #include "gdn_tiles.h"
 
 namespace gdn {
@@ -35,6 +39,7 @@ inline size_t kda_ws_layout(int64_t units, char* base, KdaWs* ws) {
 
 struct KdaParams {
     const void* q; const void* k; const void* v; const float* g; const void* beta;
+    const void* pk; const void* gs;                                             // comba: the second key, the log decay per token and head
     const float* A_log; const float* gk_bias; float gk_lower; int gk_act;      // gate activation, as in the token recurrence
     const float* h0; float* ht; void* o;
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
@@ -302,6 +307,187 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
 }
 
 // ---------------------------------------------------------------------------------------------
+// prepare, comba
+// ---------------------------------------------------------------------------------------------
+constexpr size_t COMBA_PREP_SMEM = (4 * 64 * P128 + 64 * P64) * 2 + 3 * 64 * 4;
+static_assert(64 * PL * 4 <= 64 * P128 * 2, "the matrix L takes the place of the q tile");
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, int64_t units) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    extern __shared__ __align__(16) char smem[];
+    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sP = sQ + 64 * P128; T* sV = sP + 64 * P128; T* sA = sV + 64 * P128;
+    float* sGam = (float*)(sA + 64 * P64); float* sGam0 = sGam + 64; float* sBeta = sGam0 + 64;
+    float* sL = (float*)sQ;                                     // once q has been used
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+
+    // Two workgroups per CU walk over the units; the next unit's rows and gates are fetched into registers meanwhile.
+    TileRegs<BD> rK, rQ, rP, rV;
+    float rG = 0.f, rB = 0.f;
+    auto fetch_v = [&](int64_t u) {                             // (on its own, later than the rest: fewer registers live across the substitution)
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    };
+    auto fetch = [&](int64_t u) {
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        fetch_tile<BD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
+        const bool have = tid < 64 && tid < c.valid;
+        rG = have ? load_scalar(p.gs, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        rB = have ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+    };
+    fetch(blockIdx.x);
+    fetch_v(blockIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+    put_tile<BD>(sK, P128, rK, tid);
+    put_tile<BD>(sQ, P128, rQ, tid);
+    put_tile<BD>(sP, P128, rP, tid);
+    put_tile<BD>(sV, P128, rV, tid);
+    if (w == 0) {
+        float run = rG;                                         // running sum over the chunk's tokens (rows past the end add 0)
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float t = __shfl_up(run, off, 64);
+            if (lane >= off) run += t;
+        }
+        sGam[lane] = run;
+        sGam0[lane] = run - rG;
+        sBeta[lane] = rB;
+    }
+    lds_barrier();
+    if (u + gridDim.x < units) fetch(u + gridDim.x);
+    if (p.flags & GDN_FLAG_QK_L2NORM) {
+        // rows of q, k and p divided by sqrt(sum x^2 + 1e-6): 16 consecutive lanes hold the 16 pieces of a row
+#pragma unroll 2
+        for (int i = 0; i < 4; ++i) {
+            const int row = (tid >> 4) + 16 * i, pc = tid & 15;
+#pragma unroll
+            for (int which = 0; which < 3; ++which) {
+                T* at = (which == 0 ? sK : which == 1 ? sQ : sP) + row * P128 + pc * 8;
+                V8 x = *(V8*)at;
+                float ss = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss += (float)x[e] * (float)x[e];
+                const float r = rsqrtf(sum_over_c16(ss) + 1e-6f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * r);
+                *(V8*)at = x;
+            }
+        }
+        lds_barrier();
+    }
+    const float gl = sGam[63];
+    {
+        // P, this wave's 16 rows; and what the scan needs of q and k
+        T* Pu = (T*)p.ws.Pm + u * 64 * 64;
+        const int i = 16 * w + c16;
+        V8 qf[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) qf[s] = frag_rows(sQ, P128, 16 * w, 32 * s, lane);
+        const float gam_i = sGam[i];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            if (tj > w) { *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(ZERO4); continue; }
+            f32x4 pt = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                pt = Mma<T>::run(frag_rows(sK, P128, 16 * tj, 32 * s, lane), qf[s], pt);     // lane: column i = 16w + c16, rows j = 16tj + 4g + r
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int jr = 16 * tj + 4 * g + r;
+                pt[r] = jr <= i ? p.scale * pt[r] * __expf(gam_i - sGam[jr]) : 0.f;
+            }
+            *(V4*)(Pu + i * 64 + 16 * tj + 4 * g) = pack4<T>(pt);
+        }
+        T* QGu = (T*)p.ws.QG + u * 64 * BD;
+        T* KGu = (T*)p.ws.KG + u * 64 * BD;
+#pragma unroll 2                                        // (unrolled fully, the kernel spills registers)
+        for (int it = 0; it < 4; ++it) {
+            const int row = (tid >> 4) + 16 * it, pc = tid & 15;
+            V8 kx = *(V8*)(sK + row * P128 + pc * 8), qx = *(V8*)(sQ + row * P128 + pc * 8);
+            const float fk = __expf(gl - sGam[row]), fq = p.scale * __expf(sGam[row]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kx[e] = (T)((float)kx[e] * fk);
+                qx[e] = (T)((float)qx[e] * fq);
+            }
+            *(V8*)(KGu + row * BD + pc * 8) = kx;
+            *(V8*)(QGu + row * BD + pc * 8) = qx;
+        }
+        if (tid < BD) p.ws.EGL[u * BD + tid] = __expf(gl);
+    }
+    lds_barrier();                                              // q is done with: L takes its place
+    {
+        // L = diag(beta) M for the substitution, this wave's 16 rows
+        V8 pf[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) pf[s] = frag_rows(sP, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            if (tj > w) continue;
+            f32x4 m = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                m = Mma<T>::run(pf[s], frag_rows(sK, P128, 16 * tj, 32 * s, lane), m);       // lane: column j = 16tj + c16, rows i = 16w + 4g + r
+            const int j = 16 * tj + c16;
+            const float gam_j = sGam[j];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int ir = 16 * w + 4 * g + r;
+                sL[ir * PL + (j & 3) * 16 + (j >> 2)] = ir > j ? sBeta[ir] * m[r] * __expf(sGam0[ir] - gam_j) : 0.f;
+            }
+        }
+    }
+    lds_barrier();
+    solve_unit_lower<T>(sL, sA, w, lane);
+    {
+        // p, v as the factors of w, u
+#pragma unroll 2                                        // (unrolled fully, the kernel spills registers)
+        for (int it = 0; it < 4; ++it) {
+            const int row = (tid >> 4) + 16 * it, pc = tid & 15;
+            V8 px = *(V8*)(sP + row * P128 + pc * 8), vx = *(V8*)(sV + row * P128 + pc * 8);
+            const float b = sBeta[row], fp = b * __expf(sGam0[row]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                px[e] = (T)((float)px[e] * fp);
+                vx[e] = (T)((float)vx[e] * b);
+            }
+            *(V8*)(sP + row * P128 + pc * 8) = px;
+            *(V8*)(sV + row * P128 + pc * 8) = vx;
+        }
+    }
+    lds_barrier();
+    if (u + gridDim.x < units) fetch_v(u + gridDim.x);
+    {
+        // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
+        T* Wu = (T*)p.ws.Wm + u * 64 * BD;
+        T* Uu = (T*)p.ws.Um + u * 64 * BD;
+        const int i = 16 * w + c16;
+        V8 fa[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) fa[s] = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+            f32x4 aw = ZERO4, au = ZERO4;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (2 * s > w) continue;                        // A is lower triangular
+                aw = Mma<T>::run(frag_cols(sP, P128, 32 * s, 16 * n, lane), fa[s], aw);
+                au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), fa[s], au);
+            }
+            *(V4*)(Wu + i * BD + 16 * n + 4 * g) = pack4<T>(aw);
+            *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
+        }
+    }
+    lds_barrier();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // scan: the state slice [128][VBT] lives in registers as transposed tiles (wave w: key rows 32w .. 32w+31 as two tiles a2,
 // lane (c16, g): key 16(2w+a2) + c16, value columns 16b + 4g .. +3); the next chunk's tiles are fetched into registers
 // while the current chunk is computed.
@@ -432,7 +618,7 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
 }
 
 template <typename T>
-static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream) {
+static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream, bool comba = false) {
     const int64_t runs1 = p.N * p.HV;
     const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
     const unsigned units = (unsigned)(num_chunks * p.HV), runs = (unsigned)((runs1 + 7) / 8 * 8 * (BD / vbt));
@@ -441,13 +627,37 @@ static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream
     if (vbt == 32) scan = {(const void*)gdn_kda_scan_kernel<T, 32>, kda_scan_smem<32>(), "gdn_kda_scan_kernel", runs};
     else if (vbt == 64) scan = {(const void*)gdn_kda_scan_kernel<T, 64>, kda_scan_smem<64>(), "gdn_kda_scan_kernel", runs};
     else scan = {(const void*)gdn_kda_scan_kernel<T, 128>, kda_scan_smem<128>(), "gdn_kda_scan_kernel", runs};
-    const K ks[2] = {{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 256u ? units : 256u}, scan};
+    const K prep = comba ? K{(const void*)gdn_comba_prepare_kernel<T>, COMBA_PREP_SMEM, "gdn_comba_prepare_kernel", units < 512u ? units : 512u}
+                         : K{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 256u ? units : 256u};
+    const K ks[2] = {prep, scan};
     for (int i = 0; i < 2; ++i) {
         if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
         int64_t nunits = units;
         void* args[] = {(void*)&p, (void*)&nunits};             // (the prepare kernel walks over the units and takes their number)
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(256), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
+    }
+    return GDN_OK;
+}
+
+
+// checks shared by the two entry points
+static int check_shapes(const char* who, int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N, int64_t num_chunks,
+                        const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets, int qkv_dtype, uint32_t flags, uint32_t known) {
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
+    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
+                  who, (long long)K, (long long)V);
+    GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v must be bf16 or f16", who);
+    GDN_CHECK_ARG((flags & ~known) == 0, GDN_ERR_UNSUPPORTED, "%s: unknown flag (the state layout is the caller's)", who);
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
+                  "%s: too many heads or chunks for one launch", who);
+    if (cu_seqlens) {
+        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
+        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
+    } else {
+        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
+        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
     }
     return GDN_OK;
 }
@@ -470,25 +680,11 @@ extern "C" int gdn_chunk_kda_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
     const char* who = "gdn_chunk_kda_fwd";
-    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
-    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
-    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
-                  who, (long long)K, (long long)V);
-    GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v must be bf16 or f16", who);
+    const uint32_t known = GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM | GDN_FLAG_BETA_SIGMOID | GDN_FLAG_NEG_EIGVAL;
+    if (int rc = check_shapes(who, B, T, H, HV, K, V, N, num_chunks, cu_seqlens, chunk_table, chunk_offsets, qkv_dtype, flags, known)) return rc;
     GDN_CHECK_ARG(gate_mode >= 0 && gate_mode <= 2, GDN_ERR_INVALID, "%s: gate_mode must be 0, 1 or 2", who);
     GDN_CHECK_ARG(gate_mode != 0 || (!A_log && !dt_bias), GDN_ERR_INVALID, "%s: A_log / dt_bias without a gate activation", who);
-    const uint32_t known = GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM | GDN_FLAG_BETA_SIGMOID | GDN_FLAG_NEG_EIGVAL;
-    GDN_CHECK_ARG((flags & ~known) == 0, GDN_ERR_UNSUPPORTED, "%s: unknown flag (the state layout is the caller's)", who);
     GDN_CHECK_ARG(!(flags & GDN_FLAG_NEG_EIGVAL) || (flags & GDN_FLAG_BETA_SIGMOID), GDN_ERR_INVALID, "%s: GDN_FLAG_NEG_EIGVAL needs GDN_FLAG_BETA_SIGMOID", who);
-    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
-                  "%s: too many heads or chunks for one launch", who);
-    if (cu_seqlens) {
-        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
-        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
-    } else {
-        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
-        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
-    }
     hipStream_t s = (hipStream_t)stream;
     if (T == 0 || num_chunks == 0) {
         if (ht) return launch_state_copy(h0, ht, N * HV * K * V, s);
@@ -502,10 +698,46 @@ extern "C" int gdn_chunk_kda_fwd(
     const size_t need = kda_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
-    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.gk_bias = dt_bias; p.gk_lower = lower_bound; p.gk_act = gate_mode;
+    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.pk = nullptr; p.gs = nullptr; p.A_log = A_log; p.gk_bias = dt_bias; p.gk_lower = lower_bound; p.gk_act = gate_mode;
     p.h0 = h0; p.ht = ht; p.o = o;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_kda<bf16_t>(p, num_chunks, s) : launch_kda<f16_t>(p, num_chunks, s);
+}
+
+extern "C" int gdn_chunk_comba_fwd(
+    const void* q, const void* k, const void* v, const void* p_key, const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    using namespace gdn;
+    const char* who = "gdn_chunk_comba_fwd";
+    if (int rc = check_shapes(who, B, T, H, HV, K, V, N, num_chunks, cu_seqlens, chunk_table, chunk_offsets, qkv_dtype, flags,
+                              GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM)) return rc;
+    GDN_CHECK_ARG(gb_dtype == GDN_DTYPE_F32 || gb_dtype == GDN_DTYPE_BF16 || gb_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED,
+                  "%s: g and beta must be f32, bf16 or f16", who);
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0 || num_chunks == 0) {
+        if (ht) return launch_state_copy(h0, ht, N * HV * K * V, s);
+        return GDN_OK;
+    }
+    GDN_CHECK_ARG(q && k && v && p_key && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, p, g, beta, o must not be NULL", who);
+    for (const void* x : {q, k, v, p_key, (const void*)h0, (const void*)ht, (const void*)o})
+        GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
+    GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
+    KdaParams p;
+    const size_t need = kda_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
+    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
+                  need, workspace_bytes);
+    p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.pk = p_key; p.gs = g;
+    p.A_log = nullptr; p.gk_bias = nullptr; p.gk_lower = 0.f; p.gk_act = 0;
+    p.h0 = h0; p.ht = ht; p.o = o;
+    p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_kda<bf16_t>(p, num_chunks, s, true) : launch_kda<f16_t>(p, num_chunks, s, true);
 }

@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -103,6 +103,13 @@ SIGNATURES['gdn_chunk_kda_workspace_bytes'] = (c_size_t, [c_int64, c_int64])
 SIGNATURES['gdn_chunk_kda_fwd'] = (c_int, [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k v g beta
     c_void_p, c_void_p, c_float, c_int,                # A_log dt_bias lower_bound gate_mode
+    c_void_p, c_void_p, c_void_p,                      # h0 ht o
+    c_void_p, c_void_p, c_void_p,                      # cu_seqlens chunk_table chunk_offsets
+    c_void_p, c_size_t,                                # workspace workspace_bytes
+    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
+    c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_chunk_comba_fwd'] = (c_int, [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # q k v p g beta
     c_void_p, c_void_p, c_void_p,                      # h0 ht o
     c_void_p, c_void_p, c_void_p,                      # cu_seqlens chunk_table chunk_offsets
     c_void_p, c_size_t,                                # workspace workspace_bytes

@@ -273,6 +273,24 @@ int gdn_chunk_kda_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Chunked forward of the comba operator (one decay per token and head; the prediction uses a second key p and the state
+ * before the token's decay).  Replaces chunk_comba_fwd (fla/ops/comba/chunk.py:22-90): chunk_comba_cumsum_scalar_fwd
+ * (fla/ops/comba/utils.py), chunk_scaled_dot_comba_pkt_fwd and the triangular solve (fla/ops/comba/wy_fast.py), recompute_w_u_fwd,
+ * chunk_gated_delta_rule_fwd_h and chunk_fwd_o; the sequential part is gdn_chunk_kda_fwd's.
+ *   q, k, p [B,T,H,K]; v [B,T,HV,V] (bf16 or f16); g (natural-log decay), beta [B,T,HV] (gb_dtype);
+ *   h0, ht [N,HV,K,V] fp32 or NULL; o [B,T,HV,V] in qkv_dtype; the rest as for gdn_chunk_kda_fwd, whose workspace size it shares.
+ *   flags: GDN_FLAG_CU_INT32, GDN_FLAG_QK_L2NORM (normalises q, k and p, fla/ops/comba/chunk.py:202-205).  K = V = 128 only.
+ */
+int gdn_chunk_comba_fwd(
+    const void* q, const void* k, const void* v, const void* p, const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * gdn_chunk_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
  * gdn_chunk_fwd minus the workspace: the kernels use a fixed array of GDN_CHUNK_STATIC_WORKSPACE_BYTES that the

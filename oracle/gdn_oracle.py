@@ -20,6 +20,8 @@ reference checkout):
 * ``fla/utils/_testing.py:19-41``                error metric
 * ``fla/ops/kda/naive.py:12-66``, ``fla/ops/kda/gate.py:27-94``, ``fla/ops/kda/fused_recurrent.py:150-181``
   the KDA operator's token recurrence (a decay per key feature) and its gate activations
+* ``fla/ops/comba/fused_recurrent.py:85-105``, ``fla/ops/comba/naive.py:70-171``  the comba operator (a second key for the
+  prediction, made before the token's decay): token recurrence and chunked form
 * ``fla/ops/gated_delta_rule/chunk.py:125-257``, ``fla/ops/common/chunk_delta_h.py:369-560``, ``fla/ops/common/chunk_o.py:172-357``,
   ``fla/ops/gated_delta_rule/wy_fast.py:123-296``  the chunked backward pass, stage by stage (``chunk_backward_one_sequence``);
   the gradients themselves are reverse-mode differentiation of the token recurrence (``gated_delta_rule_grads``)
@@ -35,6 +37,8 @@ speculative decoding).  The KDA recurrence is the gk branch of the token recurre
 fixtures); its gate activations are pinned by values that the formulas fix (``test_kda_gate_pins``).
 The gradients (``gated_delta_rule_grads``) are pinned by central finite differences of the recurrence in fp64 for every input
 and every prologue, and the stage-by-stage backward agrees with them to 1e-12 (``tests/test_chunk_bwd.py``).
+The comba recurrence is pinned by scalar loops, by its chunked form (library triangular solve) and by its reduction to the
+delta rule at p = k, g = 0 (``test_comba_*`` in ``tests/test_oracle.py``).
 No function here is "parity unpinned".
 
 Everything is computed in ``dtype`` (float32 by default, float64 for tight
@@ -225,6 +229,73 @@ def recurrent_kda(
         q, k, v, None, beta, scale, initial_state, output_final_state, cu_seqlens, gk=gk,
         use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel,
         allow_neg_eigval=allow_neg_eigval, state_v_first=state_v_first, dtype=dtype)
+
+
+def recurrent_comba(
+    q, k, v, p, g, beta=None, scale=None, initial_state=None, output_final_state=False, cu_seqlens=None,
+    use_qk_l2norm_in_kernel=False, dtype=torch.float32,
+):
+    """Token recurrence of the comba operator as its kernels run it (fla/ops/comba/fused_recurrent.py:85-105; the chunked
+    form fla/ops/comba/naive.py:70-171, which the reference's tests take as the truth, is the same map): the prediction
+    uses a second key p and the state BEFORE this token's decay,
+        v' = beta (v - S^T p);  S <- e^g S + k v'^T;  o = S^T (q scale).
+    q, k, p: [B,T,H,K]; v: [B,T,HV,V]; g, beta: [B,T,HV]; p defaults to k.  With use_qk_l2norm_in_kernel q, k and p
+    are normalised (fused_recurrent.py:90-93)."""
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if scale is None:
+        scale = K ** -0.5
+    if p is None:
+        p = k
+    qf, kf, pf, vf = q.to(dtype), k.to(dtype), p.to(dtype), v.to(dtype)
+    if use_qk_l2norm_in_kernel:
+        qf, kf, pf = (x / torch.sqrt((x * x).sum(-1, keepdim=True) + 1e-6) for x in (qf, kf, pf))
+    qf, kf, pf = _expand_heads(qf, HV), _expand_heads(kf, HV), _expand_heads(pf, HV)
+    bf = torch.ones(B, T, HV, dtype=dtype) if beta is None else beta.to(dtype)
+    gf = g.to(dtype)
+    if cu_seqlens is None:
+        bounds = [(b, 0, T) for b in range(B)]
+    else:
+        cu = [int(x) for x in cu_seqlens]
+        bounds = [(0, s, e) for s, e in zip(cu[:-1], cu[1:])]
+    o = torch.zeros(B, T, HV, V, dtype=dtype)
+    ht = torch.zeros(len(bounds), HV, K, V, dtype=dtype)
+    for n, (b, s, e) in enumerate(bounds):
+        S = initial_state[n].to(dtype).clone() if initial_state is not None else torch.zeros(HV, K, V, dtype=dtype)
+        for t in range(s, e):
+            vp = bf[b, t][:, None] * (vf[b, t] - torch.einsum('hkv,hk->hv', S, pf[b, t]))
+            S = S * gf[b, t].exp()[:, None, None] + kf[b, t][:, :, None] * vp[:, None, :]
+            o[b, t] = torch.einsum('hkv,hk->hv', S, qf[b, t] * scale)
+        ht[n] = S
+    return o, (ht if output_final_state else None)
+
+
+def chunk_comba_one_sequence(q, k, v, p, g, beta, scale, S0, chunk_size=64, dtype=torch.float32):
+    """The comba operator in chunked form for one sequence and head (fla/ops/comba/naive.py:113-160; the kernels'
+    stage order fla/ops/comba/chunk.py:22-90): with Gam the in-chunk cumsum of g and Gam0 = Gam - g,
+        M_ij = (p_i . k_j) e^(Gam0_i - Gam_j) (i > j);  A = (I + diag(beta) M)^-1;  w = A (beta p e^Gam0);  u = A (beta v);
+    then, as for the gated delta rule, v_new = u - w S;  o = scale (q e^Gam) S + scale tril(q k^T e^(Gam_i - Gam_j)) v_new;
+    S <- e^Gam_last S + (k e^(Gam_last - Gam))^T v_new.
+    q, k, p: [T,K]; v: [T,V]; g, beta: [T]; S0: [K,V].  Returns (o [T,V], S [K,V])."""
+    T, K = k.shape
+    q, k, v, p, g, beta = (x.to(dtype) for x in (q, k, v, p, g, beta))
+    S = S0.to(dtype).clone()
+    o = torch.zeros(T, v.shape[1], dtype=dtype)
+    for t0 in range(0, T, chunk_size):
+        sl = slice(t0, min(T, t0 + chunk_size))
+        qc, kc, vc, pc, gc, bc = q[sl], k[sl], v[sl], p[sl], g[sl], beta[sl]
+        n = qc.shape[0]
+        gam = gc.cumsum(0)
+        gam0 = gam - gc
+        M = (pc @ kc.T) * (gam0[:, None] - gam[None, :]).tril(-1).exp().tril(-1)
+        A = torch.linalg.solve_triangular(torch.eye(n, dtype=dtype) + bc[:, None] * M, torch.eye(n, dtype=dtype), upper=False)
+        w = A @ (pc * (bc * gam0.exp())[:, None])
+        u = A @ (vc * bc[:, None])
+        v_new = u - w @ S
+        P = scale * (qc @ kc.T) * (gam[:, None] - gam[None, :]).tril().exp().tril()
+        o[sl] = scale * (qc * gam.exp()[:, None]) @ S + P @ v_new
+        S = S * gam[-1].exp() + (kc * (gam[-1] - gam).exp()[:, None]).T @ v_new
+    return o, S
 
 
 def recurrent_gated_delta_rule_pooled(

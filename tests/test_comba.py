@@ -1,0 +1,234 @@
+"""The comba operator (chunk_comba, fused_recurrent_comba) on the HIP kernels, through gdn_chunk_comba_fwd, against the
+CPU oracle.  Shapes, input recipes and bars of the reference's own tests (tests/ops/test_comba.py: chunk 22-... fp16,
+normalised q, k, p, gates logsigmoid(rand) / normalizer with a share mask_p of them zeroed, o and ht within 0.005; the
+recurrent entry point fp32 and fp16 within 0.002; packed sequences with a random fp16 initial state)."""
+import ctypes
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from fla_hip.ops.comba import chunk_comba, fused_recurrent_comba
+    return chunk_comba, fused_recurrent_comba
+
+
+def _check(name, ref, got, ratio):
+    got = got.detach().float().cpu()
+    assert got.shape == ref.shape, f'{name}: shape {tuple(got.shape)} vs {tuple(ref.shape)}'
+    assert not torch.isnan(got).any(), f'{name}: NaN'
+    r, m = O.get_err_ratio(ref, got), O.max_abs_ratio(ref, got)
+    assert r <= ratio and m <= 1e-2, f'{name}: rel-rmse {r:.3e} max-abs ratio {m:.3e}'
+
+
+def _inputs(B, T, H, HV, D, dtype, normalizer=1.0, mask_p=0.0, seed=42, normalise=True, h0_std=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q, k, p = (torch.randn(B, T, H, D, generator=gen) for _ in range(3))
+    if normalise:
+        q, k, p = (F.normalize(x, p=2, dim=-1) for x in (q, k, p))
+    q, k, p = q.to(dtype), k.to(dtype), p.to(dtype)
+    v = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    beta = torch.rand(B, T, HV, generator=gen).to(dtype).sigmoid()
+    g = F.logsigmoid(torch.rand(B, T, HV, generator=gen)) / normalizer
+    g = g * (torch.rand(B, T, HV, generator=gen) > mask_p)
+    h0 = torch.randn(B, HV, D, D, generator=gen) * h0_std
+    return q, k, v, p, g, beta, h0
+
+
+def _cuda(*xs):
+    return [None if x is None else x.cuda() for x in xs]
+
+
+@pytest.mark.parametrize('B,T,H,D,scale,normalizer,mask_p,l2,dtype', [
+    (1, 63, 1, 64, 1, 1, 0, False, torch.float16),
+    (2, 1000, 3, 60, 1, 1, 0, False, torch.float16),
+    (2, 1024, 3, 64, 0.1, 1, 0.5, False, torch.float16),
+    (2, 1024, 4, 100, 1, 0.1, 0, False, torch.float16),
+    (2, 1024, 4, 128, 0.1, 1, 0, True, torch.float16),
+    (2, 1024, 4, 128, 0.1, 1, 0.5, False, torch.float16),
+    (2, 1024, 4, 128, 0.1, 10, 0, False, torch.float16),
+    (4, 2048, 8, 64, 0.1, 1, 0, True, torch.float16),
+    (2, 1024, 4, 128, 0.1, 1, 0.5, True, torch.bfloat16),
+])
+def test_chunk_comba_reference_matrix(B, T, H, D, scale, normalizer, mask_p, l2, dtype):
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, H, D, dtype, normalizer, mask_p, normalise=not l2)
+    h0 = torch.zeros_like(h0)                                   # (the reference's chunk test starts from a zero state)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, scale, h0, True, use_qk_l2norm_in_kernel=l2)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    o, ht = _ops()[0](dq, dk, dv, dp, dg, db, scale=scale, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht, 5e-3)
+
+
+@pytest.mark.parametrize('H,D,mask_p,cu,idx', [
+    (4, 64, 0, [0, 15], torch.int32),
+    (4, 64, 0, [0, 256, 500, 1000], torch.int32),
+    (4, 64, 0.5, [0, 256, 500, 1000], torch.int64),
+    (4, 100, 0, [0, 15, 100, 300, 1200, 2000], torch.int32),
+    (2, 128, 0, [0, 64, 64, 200, 201], torch.int64),            # an empty sequence and one of a single token
+])
+def test_chunk_comba_packed_sequences(H, D, mask_p, cu, idx):
+    T, N = cu[-1], len(cu) - 1
+    q, k, v, p, g, beta, _ = _inputs(1, T, H, H, D, torch.float16, 1.0, mask_p)
+    q = torch.randn(1, T, H, D, generator=torch.Generator().manual_seed(1)).half()      # (as there: q is not normalised)
+    h0 = torch.randn(N, H, D, D, generator=torch.Generator().manual_seed(2)).half()
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, None, h0, True, cu_seqlens=cu)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    cu_t = torch.tensor(cu, dtype=idx, device='cuda')
+    o, ht = _ops()[0](dq, dk, dv, dp, dg, db, initial_state=dh, output_final_state=True, cu_seqlens=cu_t)
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht, 5e-3)
+    # the same through a host copy of the boundaries
+    o2, ht2 = _ops()[0](dq, dk, dv, dp, dg, db, initial_state=dh, output_final_state=True, cu_seqlens=cu_t,
+                        cu_seqlens_cpu=torch.tensor(cu, dtype=idx))
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)
+
+
+@pytest.mark.parametrize('B,T,H,D,scale,normalizer,dtype', [
+    (1, 63, 1, 64, 1, 1, torch.float32),
+    (2, 1024, 4, 60, 1, 1, torch.float32),
+    (2, 1024, 8, 128, 1, 0.1, torch.float32),
+    (2, 1024, 8, 128, 0.1, 1, torch.float32),
+    (2, 1024, 8, 128, 1, 10, torch.float32),
+    (4, 2048, 8, 64, 0.1, 1, torch.float32),
+    (2, 1024, 8, 128, 1, 0.1, torch.float16),
+    (2, 1024, 8, 128, 1, 10, torch.float16),
+])
+def test_fused_recurrent_comba_reference_matrix(B, T, H, D, scale, normalizer, dtype):
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, H, D, dtype, normalizer)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, scale, h0, True)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    keep = dh.clone()
+    o, ht = _ops()[1](dq, dk, dp, dv, dg, db, scale=scale, initial_state=dh, output_final_state=True)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and torch.equal(dh, keep)
+    _check('o', ref_o, o, 2e-3)
+    _check('ht', ref_ht, ht, 2e-3)
+
+
+def test_comba_options_and_reductions():
+    """Defaults (p = k, beta = 1, no state), grouped value heads, value heads wider than the kernels' 128 columns, the split
+    of a sequence at a chunk boundary handing the state over, and p = k with g = 0 against the delta rule operator."""
+    chunk, recurrent = _ops()
+    B, T, H, HV, D = 2, 300, 2, 4, 128
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, HV, D, torch.bfloat16, seed=7)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, None, h0, True)
+    o, ht = chunk(dq, dk, dv, dp, dg, db, initial_state=dh, output_final_state=True)
+    _check('gva o', ref_o, o, 5e-3)
+    _check('gva ht', ref_ht, ht, 5e-3)
+    o_r, ht_r = recurrent(dq, dk, dp, dv, dg, db, initial_state=dh, output_final_state=True)
+    assert torch.equal(o, o_r) and torch.equal(ht, ht_r)
+
+    ref_o, _ = O.recurrent_comba(q, k, v, None, g, None)
+    o, none = chunk(dq, dk, dv, None, dg)
+    assert none is None
+    _check('defaults o', ref_o, o, 5e-3)
+
+    o_a, ht_a = chunk(dq[:, :128], dk[:, :128], dv[:, :128], dp[:, :128], dg[:, :128], db[:, :128], initial_state=dh, output_final_state=True)
+    o_b, ht_b = chunk(dq[:, 128:], dk[:, 128:], dv[:, 128:], dp[:, 128:], dg[:, 128:], db[:, 128:], initial_state=ht_a, output_final_state=True)
+    o, ht = chunk(dq, dk, dv, dp, dg, db, initial_state=dh, output_final_state=True)
+    assert torch.equal(torch.cat([o_a, o_b], 1), o) and torch.equal(ht_b, ht)
+
+    gen = torch.Generator().manual_seed(9)
+    v2 = torch.randn(B, T, HV, 200, generator=gen).bfloat16()
+    h2 = torch.randn(B, HV, D, 200, generator=gen)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v2, p, g, beta, 0.2, h2, True)
+    o, ht = chunk(dq, dk, v2.cuda(), dp, dg, db, scale=0.2, initial_state=h2.cuda(), output_final_state=True)
+    _check('wide v o', ref_o, o, 5e-3)
+    _check('wide v ht', ref_ht, ht, 5e-3)
+
+    from fla_hip.ops.delta_rule import chunk_delta_rule
+    zero = torch.zeros_like(dg)
+    qh, kh, vh, bh = dq[:, :, :, :], dk, dv[:, :, :H], db[:, :, :H]
+    o_c, ht_c = chunk(qh, kh, vh, None, zero[:, :, :H], bh, initial_state=dh[:, :H], output_final_state=True)
+    o_d, ht_d = chunk_delta_rule(qh, kh, vh, bh, initial_state=dh[:, :H], output_final_state=True)
+    _check('delta rule o', o_d.float().cpu(), o_c, 5e-3)
+    _check('delta rule ht', ht_d.float().cpu(), ht_c, 5e-3)
+
+
+def test_comba_validation():
+    chunk, recurrent = _ops()
+    q, k, v, p, g, beta, h0 = _cuda(*_inputs(2, 64, 2, 2, 64, torch.bfloat16))
+    with pytest.raises(ValueError, match='batch size'):
+        chunk(q, k, v, p, g, beta, cu_seqlens=torch.tensor([0, 64], device='cuda'))
+    with pytest.raises(ValueError, match='number of initial states'):
+        chunk(q[:1], k[:1], v[:1], p[:1], g[:1], beta[:1], initial_state=h0, cu_seqlens=torch.tensor([0, 64], device='cuda'))
+    with pytest.raises(ValueError, match='share one shape'):
+        chunk(q, k, v, p[..., :32], g, beta)
+    with pytest.raises(ValueError, match='g and beta'):
+        chunk(q, k, v, p, g[..., :1], beta)
+    with pytest.raises(NotImplementedError, match='no backward'):
+        chunk(q.clone().requires_grad_(), k, v, p, g, beta)
+    with pytest.raises(NotImplementedError, match='per value column'):
+        recurrent(q, k, p, v, g, beta[..., None].expand(-1, -1, -1, 64))
+    with pytest.raises(RuntimeError, match='ROCm GPU'):
+        chunk(*(x.cpu() for x in (q, k, v, p, g, beta)))
+    big = torch.zeros(1, 64, 1, 256, dtype=torch.bfloat16, device='cuda')
+    with pytest.raises(NotImplementedError, match='key head dims'):
+        chunk(big, big, big, big, g[:1, :, :1], beta[:1, :, :1])
+    # no tokens: the state passes through
+    e = [x[:, :0] for x in (q, k, v, p, g, beta)]
+    o, ht = chunk(*e, initial_state=h0, output_final_state=True)
+    assert o.shape == (2, 0, 2, 64) and torch.equal(ht, h0)
+
+
+def test_comba_c_entry_checks():
+    from fla_hip import _lib
+    lib = _lib.load()
+    x = torch.zeros(1, 64, 1, 128, dtype=torch.bfloat16, device='cuda')
+    s = torch.zeros(1, 64, 1, device='cuda')
+    o = torch.empty_like(x)
+    ws = torch.empty(lib.gdn_chunk_kda_workspace_bytes(1, 1), dtype=torch.uint8, device='cuda')
+
+    def call(K=128, V=128, flags=0, ws_bytes=None, p=x, num_chunks=1, qkv=_lib.DTYPE_BF16):
+        return lib.gdn_chunk_comba_fwd(
+            x.data_ptr(), x.data_ptr(), x.data_ptr(), None if p is None else p.data_ptr(), s.data_ptr(), s.data_ptr(), None, None, o.data_ptr(),
+            None, None, None, ws.data_ptr(), ws.numel() if ws_bytes is None else ws_bytes,
+            1, 64, 1, 1, K, V, 1, num_chunks, 1.0, qkv, _lib.DTYPE_F32, flags, 0)
+
+    assert call() == _lib.GDN_OK
+    assert call(K=64) == _lib.GDN_ERR_UNSUPPORTED
+    assert call(flags=_lib.FLAG_BETA_SIGMOID) == _lib.GDN_ERR_UNSUPPORTED
+    assert call(ws_bytes=16) == _lib.GDN_ERR_WORKSPACE
+    assert call(p=None) == _lib.GDN_ERR_INVALID
+    assert call(num_chunks=2) == _lib.GDN_ERR_INVALID
+    assert call(qkv=_lib.DTYPE_F32) == _lib.GDN_ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('seed', range(12))
+def test_chunk_comba_random_combinations(seed):
+    """Seeded random shapes and options (lengths off the chunk grid, packed or padded batches, grouped heads, narrow head
+    dims, l2 norm in the kernel, extreme and masked gates, either 16-bit type) against the oracle."""
+    gen = torch.Generator().manual_seed(1000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    H = r(1, 3); HV = H * r(1, 2); D = [32, 60, 64, 100, 128][r(0, 4)]
+    dtype = [torch.bfloat16, torch.float16][r(0, 1)]
+    l2 = bool(r(0, 1)); packed = bool(r(0, 1))
+    normalizer = [0.1, 1.0, 10.0][r(0, 2)]; mask_p = [0.0, 0.5][r(0, 1)]
+    if packed:
+        lens = [r(0, 200) for _ in range(r(1, 4))]
+        if sum(lens) == 0:
+            lens[0] = 5
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        B, T, N = 1, cu[-1], len(lens)
+    else:
+        B, T, cu = r(1, 3), r(1, 260), None
+        N = B
+    q, k, v, p, g, beta, _ = _inputs(B, T, H, HV, D, dtype, normalizer, mask_p, seed=seed, normalise=not l2)
+    h0 = torch.randn(N, HV, D, D, generator=gen) if r(0, 1) else None
+    scale = [None, 0.1, 1.0][r(0, 2)]
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, scale, h0, True, cu_seqlens=cu, use_qk_l2norm_in_kernel=l2)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    o, ht = _ops()[0](dq, dk, dv, dp, dg, db, scale=scale, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=l2,
+                      cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'))
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht, 5e-3)

@@ -297,3 +297,81 @@ def test_error_metric_definition():
 def test_varlen_length_recipe():
     L = O.make_varlen_lengths(65536, 32, 256, 4096, seed=42)
     assert len(L) == 32 and sum(L) == 65536 and min(L) >= 1
+
+
+# --------------------------------------------------------------------------- #
+# comba (a second key p for the prediction, taken before the token's decay)
+# --------------------------------------------------------------------------- #
+def _comba_inputs(B, T, H, K, V, seed, gate_div=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, T, H, K, generator=gen, dtype=torch.float64), dim=-1)
+    k = F.normalize(torch.randn(B, T, H, K, generator=gen, dtype=torch.float64), dim=-1)
+    p = F.normalize(torch.randn(B, T, H, K, generator=gen, dtype=torch.float64), dim=-1)
+    v = torch.randn(B, T, H, V, generator=gen, dtype=torch.float64)
+    g = F.logsigmoid(torch.rand(B, T, H, generator=gen, dtype=torch.float64)) / gate_div
+    beta = torch.rand(B, T, H, generator=gen, dtype=torch.float64).sigmoid()
+    h0 = torch.randn(B, H, K, V, generator=gen, dtype=torch.float64)
+    return q, k, v, p, g, beta, h0
+
+
+def test_comba_recurrence_against_scalar_loops():
+    """The token recurrence written again as loops over single numbers (fla/ops/comba/fused_recurrent.py:85-105: predict
+    with p on the undecayed state, then decay, then write k).  A prediction taken after the decay, or with k, fails it."""
+    B, T, H, K, V = 1, 5, 2, 3, 2
+    q, k, v, p, g, beta, h0 = _comba_inputs(B, T, H, K, V, seed=3)
+    scale = 0.7
+    o, ht = O.recurrent_comba(q, k, v, p, g, beta, scale, h0, True, dtype=torch.float64)
+    for h in range(H):
+        S = [[float(h0[0, h, a, c]) for c in range(V)] for a in range(K)]
+        for t in range(T):
+            pred = [sum(S[a][c] * float(p[0, t, h, a]) for a in range(K)) for c in range(V)]
+            vn = [float(beta[0, t, h]) * (float(v[0, t, h, c]) - pred[c]) for c in range(V)]
+            eg = math.exp(float(g[0, t, h]))
+            for a in range(K):
+                for c in range(V):
+                    S[a][c] = eg * S[a][c] + float(k[0, t, h, a]) * vn[c]
+            for c in range(V):
+                want = scale * sum(S[a][c] * float(q[0, t, h, a]) for a in range(K))
+                assert abs(float(o[0, t, h, c]) - want) < 1e-12
+        for a in range(K):
+            for c in range(V):
+                assert abs(float(ht[0, h, a, c]) - S[a][c]) < 1e-12
+
+
+def test_comba_reductions_and_chunk_form():
+    """p = k and g = 0 is the plain delta rule; the chunked form (in-chunk inverse, fla/ops/comba/naive.py:113-160) is the
+    same map as the recurrence for every chunk size; l2 norm in the kernel equals normalising q, k and p beforehand."""
+    B, T, H, K, V = 2, 150, 2, 16, 12
+    q, k, v, p, g, beta, h0 = _comba_inputs(B, T, H, K, V, seed=5, gate_div=0.5)
+    zero = torch.zeros_like(g)
+    o1, s1 = O.recurrent_comba(q, k, v, None, zero, beta, None, h0, True, dtype=torch.float64)
+    o2, s2 = O.recurrent_gated_delta_rule(q, k, v, zero, beta, None, h0, True, dtype=torch.float64)
+    assert (o1 - o2).abs().max() < 1e-12 and (s1 - s2).abs().max() < 1e-12
+    # with p = k and a decay, comba differs from the gated delta rule only in what the prediction sees: e^-g times it
+    o3, _ = O.recurrent_comba(q[:, :1], k[:, :1], v[:, :1], None, g[:, :1], beta[:, :1], 1.0, h0, True, dtype=torch.float64)
+    pred = torch.einsum('bhkv,bhk->bhv', h0, k[:, 0])
+    S1 = h0 * g[:, 0].exp()[..., None, None] + k[:, 0, :, :, None] * (beta[:, 0, :, None] * (v[:, 0] - pred))[:, :, None, :]
+    assert (o3[:, 0] - torch.einsum('bhkv,bhk->bhv', S1, q[:, 0])).abs().max() < 1e-12
+
+    ref_o, ref_s = O.recurrent_comba(q, k, v, p, g, beta, 0.3, h0, True, dtype=torch.float64)
+    for chunk in (16, 64):
+        for b in range(B):
+            for h in range(H):
+                oc, sc = O.chunk_comba_one_sequence(q[b, :, h], k[b, :, h], v[b, :, h], p[b, :, h], g[b, :, h], beta[b, :, h],
+                                                    0.3, h0[b, h], chunk, torch.float64)
+                assert (oc - ref_o[b, :, h]).abs().max() < 1e-10 and (sc - ref_s[b, h]).abs().max() < 1e-10
+    raw = [x * 3.0 for x in (q, k, p)]
+    o4, s4 = O.recurrent_comba(raw[0], raw[1], v, raw[2], g, beta, 0.3, h0, True, use_qk_l2norm_in_kernel=True, dtype=torch.float64)
+    assert (o4 - ref_o).abs().max() < 1e-6 and (s4 - ref_s).abs().max() < 1e-6
+    # packed sequences and grouped value heads
+    cu = [0, 40, 150]
+    qp, kp, vp, pp, gp, bp = (x[:1] for x in (q, k, v, p, g, beta))
+    o5, s5 = O.recurrent_comba(qp, kp, vp, pp, gp, bp, 0.3, h0, True, cu_seqlens=cu, dtype=torch.float64)
+    for n in range(2):
+        sl = slice(cu[n], cu[n + 1])
+        on, sn = O.recurrent_comba(qp[:, sl], kp[:, sl], vp[:, sl], pp[:, sl], gp[:, sl], bp[:, sl], 0.3, h0[n:n + 1], True, dtype=torch.float64)
+        assert torch.equal(o5[:, sl], on) and torch.equal(s5[n:n + 1], sn)
+    o6, _ = O.recurrent_comba(q[:, :, :1], k[:, :, :1], v, p[:, :, :1], g, beta, 0.3, h0, dtype=torch.float64)
+    o7, _ = O.recurrent_comba(q[:, :, :1].expand(-1, -1, 2, -1), k[:, :, :1].expand(-1, -1, 2, -1), v, p[:, :, :1].expand(-1, -1, 2, -1),
+                              g, beta, 0.3, h0, dtype=torch.float64)
+    assert torch.equal(o6, o7)
