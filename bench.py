@@ -382,7 +382,7 @@ def bench_layer_steps(steps, warmup, device, with_cpu):
     """The two memory-bound steps either side of the operator in the layer at the default prefill size: the causal
     convolution (+ SiLU) over the joined q|k|v projection (8192 channels, kernel size 4) and the gated RMS norm over
     the 32 value heads of 128 features.  Algorithmic bytes: every input element read once, every output written once."""
-    from fla_hip.modules import causal_conv1d, rms_norm_gated
+    from fla_hip.modules import causal_conv1d, causal_conv1d_bwd, layer_norm_gated_bwd, layer_norm_gated_fwd, rms_norm_gated
     T, H, HV, W = 32768, 16, 32, 4
     D = 2 * H * K + HV * V
     gen = torch.Generator(device=device).manual_seed(42)
@@ -391,13 +391,23 @@ def bench_layer_steps(steps, warmup, device, with_cpu):
     o = torch.randn(T * HV, V, generator=gen, device=device).bfloat16()
     gate = torch.randn(T * HV, V, generator=gen, device=device).bfloat16()
     wn = torch.randn(V, generator=gen, device=device).bfloat16()
+    dy_x, dy_o = torch.randn_like(x), torch.randn_like(o)
+    _, _, rstd, _ = layer_norm_gated_fwd(o, gate, wn, None, 'swish', 1e-5, is_rms_norm=True)
     out = {}
     cases = (('conv_qkv', 'causal_conv1d_fwd_kernel', 2 * T * D * 2,
               f'causal conv + SiLU, T={T}, {D} channels (q|k|v), kernel size {W}, bf16',
               lambda: causal_conv1d(x, wt, activation='silu')),
              ('norm_gate', 'norm_gated_rows_kernel', 3 * T * HV * V * 2,
               f'gated RMS norm (swish), {T}x{HV} rows of {V} features, bf16',
-              lambda: rms_norm_gated(o, gate, wn, None, 'swish', eps=1e-5)))
+              lambda: rms_norm_gated(o, gate, wn, None, 'swish', eps=1e-5)),
+             # the backward passes (training): x, dy read and dx written; x, g, dy read and dx, dg written.  The time is the
+             # whole call: the kernel and the sum over the rows of partial parameter gradients it leaves
+             ('conv_qkv_bwd', 'causal_conv1d_bwd_kernel', 3 * T * D * 2,
+              f'backward of the causal conv + SiLU, T={T}, {D} channels, kernel size {W}, bf16',
+              lambda: causal_conv1d_bwd(x, dy_x, None, wt, activation='silu')),
+             ('norm_gate_bwd', 'norm_gated_bwd_kernel', 5 * T * HV * V * 2,
+              f'backward of the gated RMS norm (swish), {T}x{HV} rows of {V} features, bf16',
+              lambda: layer_norm_gated_bwd(dy_o, o, gate, wn, None, 'swish', 1e-5, None, rstd, is_rms_norm=True)))
     for key, kernel, nbytes, name, fn in cases:
         wall, t_kernel = _time_calls(fn, steps, warmup)
         achieved = nbytes / t_kernel / 1e9

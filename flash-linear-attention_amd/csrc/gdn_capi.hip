@@ -80,5 +80,5 @@ extern "C" int gdn_calib_rmw(float* data, int64_t n_floats, int xcd_run, int wor
     return check_launch("calib_rmw_kernel");
 }
 
-extern "C" int gdn_hip_abi_version(void) { return 12; }
+extern "C" int gdn_hip_abi_version(void) { return 13; }
 extern "C" const char* gdn_last_error(void) { return gdn::g_err; }

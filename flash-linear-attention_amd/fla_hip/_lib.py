@@ -9,7 +9,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get('FLA_HIP_LIBRARY') or os.path.join(_HERE, '_C', 'libgdn_hip.so')
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 GDN_OK = 0
 GDN_ERR_INVALID = -1
@@ -115,8 +115,20 @@ SIGNATURES['gdn_chunk_comba_fwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_causal_conv1d_bwd'] = (c_int, [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # x weight bias initial_state dy dht
+    c_void_p, c_void_p, c_void_p, c_void_p,            # dx dw_part db_part dh0
+    c_void_p, c_void_p,                                # cu_seqlens tile_table
+    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T D W N num_tiles stride_x_n stride_x_t
+    c_int, c_int, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_norm_gated_bwd'] = (c_int, [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # dy x g weight bias
+    c_void_p, c_void_p, c_void_p,                      # mean rstd dresidual
+    c_void_p, c_void_p, c_void_p, c_void_p,            # dx dg dw_part db_part
+    c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p])   # T D ld parts ...
 SIGNATURES['gdn_calib_rmw'] = (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p])
 CHUNK_STATIC_WORKSPACE_BYTES = 64 << 20
+CONV_BWD_TILES_PER_PART = 4
 
 _lib = None
 _lock = threading.Lock()

@@ -1,4 +1,4 @@
-"""Gated DeltaNet layer for inference: projections, causal short convolutions, the gated delta rule, gated RMS
+"""Gated DeltaNet layer: projections, causal short convolutions, the gated delta rule, gated RMS
 norm, output projection - the immediate caller of this package's kernels, with the constructor arguments,
 parameter names (so upstream checkpoints load with ``load_state_dict``) and call signature of the reference's
 ``GatedDeltaNet`` (fla/layers/gated_deltanet.py:28-364), and its cache contract: ``past_key_values[layer_idx]``
@@ -10,7 +10,9 @@ upstream's ``fla.models.utils.Cache`` objects are used the same way.
 Prompts longer than 64 tokens run the chunk kernels, shorter calls (decode) the token recurrence; both read and
 write the same state layout, so a prefill hands over to decode through the cache without any conversion.
 The linear projections are torch matmuls; everything between them runs in this package's HIP kernels.
-Forward only: no autograd graph is built through the kernels."""
+In training mode (``.train()``) the call is differentiable: the convolutions, the chunked operator and the gated norm
+each have backward kernels, and every call runs the chunk kernels as in the reference (fla/layers/gated_deltanet.py:237-239).
+In eval mode no autograd graph is built (the token recurrence of decode has no backward)."""
 from __future__ import annotations
 
 import math
@@ -122,7 +124,6 @@ class GatedDeltaNet(nn.Module):
             self.o_norm = nn.RMSNorm(self.head_v_dim, eps=norm_eps, dtype=torch.float32)
         self.o_proj = nn.Linear(self.value_dim, hidden_size, bias=False)
 
-    @torch.no_grad()
     def forward(
         self,
         hidden_states: torch.Tensor,
@@ -133,13 +134,19 @@ class GatedDeltaNet(nn.Module):
         **kwargs,
     ):
         if self.training:
-            raise RuntimeError('fla_hip.layers.GatedDeltaNet is inference only: call .eval() first')
+            return self._forward(hidden_states, attention_mask, past_key_values, use_cache, **kwargs)
+        with torch.no_grad():
+            return self._forward(hidden_states, attention_mask, past_key_values, use_cache, **kwargs)
+
+    def _forward(self, hidden_states, attention_mask, past_key_values, use_cache, **kwargs):
         if attention_mask is not None:
             assert attention_mask.dim() == 2, 'attention_mask must be a 0-1 matrix [batch_size, seq_len] (0 = padding)'
         if past_key_values is not None and self.layer_idx is None:
             raise ValueError(f'{self.__class__.__name__} requires `layer_idx` when `past_key_values` is provided.')
         batch_size, q_len, _ = hidden_states.shape
-        mode = 'fused_recurrent' if q_len <= 64 else self.mode
+        mode = 'fused_recurrent' if (q_len <= 64 and not self.training) else self.mode
+        if self.training and mode != 'chunk':
+            raise AssertionError('Only chunk mode is supported in training.')
 
         last_state = None
         if past_key_values is not None and len(past_key_values) > self.layer_idx:

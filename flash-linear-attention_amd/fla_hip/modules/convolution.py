@@ -1,8 +1,9 @@
-"""Causal depthwise short convolution, forward only, with the reference's interface:
-``causal_conv1d`` (fla/modules/conv/causal_conv1d.py:16-129), ``causal_conv1d_fwd``,
-``causal_conv1d_update_states``, ``causal_conv1d_update`` (fla/modules/conv/triton/ops.py:37-96,
-:252-296, :301-363) and the ``ShortConvolution`` layer (fla/modules/conv/short_conv.py:24-250).
-All compute is done by ``gdn_causal_conv1d_fwd`` / ``gdn_causal_conv1d_update`` of the HIP library."""
+"""Causal depthwise short convolution with the reference's interface:
+``causal_conv1d`` (fla/modules/conv/causal_conv1d.py:16-129), ``causal_conv1d_fwd``, ``causal_conv1d_bwd``,
+``causal_conv1d_update_states``, ``causal_conv1d_update`` (fla/modules/conv/triton/ops.py:37-96, :147-249,
+:252-296, :301-363), the autograd function that ties forward and backward together (:366-428) and the
+``ShortConvolution`` layer (fla/modules/conv/short_conv.py:24-250).  All compute is done by ``gdn_causal_conv1d_fwd``,
+``gdn_causal_conv1d_bwd`` and ``gdn_causal_conv1d_update`` of the HIP library; the one-token update is forward only."""
 from __future__ import annotations
 
 import os
@@ -10,9 +11,11 @@ import warnings
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, forward_only, ptr, require_gpu
+from fla_hip.ops.utils.index import prepare_chunk_indices
 from fla_hip.utils import input_guard
 
 MAX_KERNEL_SIZE = 8
@@ -103,6 +106,122 @@ def causal_conv1d_fwd(
     return y.view(shape), final_state
 
 
+def causal_conv1d_bwd(
+    x: torch.Tensor,
+    dy: torch.Tensor,
+    dht: torch.Tensor | None,
+    weight: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
+    residual: torch.Tensor | None = None,
+    initial_state: torch.Tensor | None = None,
+    activation: str | None = None,
+    cu_seqlens: torch.Tensor | None = None,
+    cu_seqlens_cpu: torch.LongTensor | None = None,
+    chunk_indices: torch.LongTensor | None = None,
+    BT: int = 64,
+    layout_fallback: bool = False,
+):
+    """Gradients ``(dx, dw, db, dr, dh0)`` of ``causal_conv1d_fwd`` for the output gradient ``dy`` and the gradient ``dht``
+    of the final state (``None``: none); ``dr`` is ``dy`` itself when there was a residual, ``dh0`` has the initial
+    state's dtype.  ``chunk_indices`` (tiles of 64 tokens), ``BT`` and ``layout_fallback`` as in the forward."""
+    if weight is None:
+        raise ValueError('causal_conv1d_bwd needs the weight of shape [D, W]')
+    dev = require_gpu(x, dy)
+    shape = x.shape
+    D, W = weight.shape
+    x = _rows(x, D)
+    B, T, _ = x.shape
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    dy = dy.reshape(B, T, D).to(x.dtype).contiguous()
+    vec = 16 // x.element_size()
+    pad = (-D) % vec
+    if pad or x.data_ptr() % 16 or x.stride(1) % vec or x.stride(0) % vec:
+        # the kernel takes 16 bytes of channels per thread: bring odd layouts to that form
+        x = F.pad(x, (0, pad)) if pad else x.clone(memory_format=torch.contiguous_format)
+        dy = F.pad(dy, (0, pad))
+        weight_k = F.pad(weight, (0, 0, 0, pad))
+        bias_k = None if bias is None else F.pad(bias, (0, pad))
+        h0_k = None if initial_state is None else F.pad(initial_state, (0, 0, 0, pad))
+        dht_k = None if dht is None else F.pad(dht, (0, 0, 0, pad))
+    else:
+        weight_k, bias_k, h0_k, dht_k = weight, bias, initial_state, dht
+    Dk = D + pad
+    weight_k = weight_k.contiguous()
+    if bias_k is not None:
+        bias_k = bias_k.to(weight_k.dtype).contiguous()
+    if h0_k is not None:
+        h0_k = h0_k.contiguous()
+    if dht_k is not None:
+        dht_k = dht_k.to(x.dtype).contiguous()
+    flags = 0
+    tile_table = None
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        elif cu_seqlens.dtype != torch.int64:
+            raise ValueError(f'cu_seqlens must be int32 or int64, got {cu_seqlens.dtype}')
+        cu_seqlens = cu_seqlens.to(dev).contiguous()
+        if chunk_indices is None or BT != 64:
+            chunk_indices = prepare_chunk_indices(cu_seqlens, 64, cu_seqlens_cpu=cu_seqlens_cpu)
+        tile_table = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        num_tiles = tile_table.shape[0]
+        dx = torch.zeros(B, T, Dk, dtype=x.dtype, device=dev)   # tokens outside the sequences keep a zero gradient
+    else:
+        num_tiles = B * ((T + 63) // 64)
+        dx = torch.empty(B, T, Dk, dtype=x.dtype, device=dev)
+    parts = (num_tiles + _lib.CONV_BWD_TILES_PER_PART - 1) // _lib.CONV_BWD_TILES_PER_PART
+    dw_part = torch.empty(max(parts, 1), Dk, W, dtype=torch.float32, device=dev)
+    db_part = torch.empty(max(parts, 1), Dk, dtype=torch.float32, device=dev) if bias_k is not None else None
+    if parts == 0:
+        dw_part.zero_()
+        if db_part is not None:
+            db_part.zero_()
+    dh0 = torch.empty(N, Dk, W, dtype=torch.float32, device=dev) if initial_state is not None else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().gdn_causal_conv1d_bwd(
+            ptr(x), ptr(weight_k), ptr(bias_k), ptr(h0_k), ptr(dy), ptr(dht_k), ptr(dx), ptr(dw_part), ptr(db_part), ptr(dh0),
+            ptr(cu_seqlens), ptr(tile_table), B, T, Dk, W, N, num_tiles,
+            x.stride(0) if B > 1 else T * max(x.stride(1), Dk), x.stride(1) if T > 1 else Dk,
+            dtype_code(x.dtype), dtype_code(weight_k.dtype),
+            dtype_code(h0_k.dtype) if h0_k is not None else _lib.DTYPE_F32,
+            _activation_code(activation), flags, current_stream_ptr(dev)))
+    dw = dw_part.sum(0)[:D].to(weight.dtype)
+    db = db_part.sum(0)[:D].to(bias.dtype) if bias is not None else None
+    if pad:
+        dx = dx[..., :D].contiguous()
+    if dh0 is not None:
+        dh0 = dh0[:, :D].to(initial_state.dtype)
+    dr = dy[..., :D].reshape(shape) if residual is not None else None
+    return dx.view(shape), dw, db, dr, dh0
+
+
+class CausalConv1dFunction(torch.autograd.Function):
+    """Forward and backward kernels as one differentiable function (fla/modules/conv/triton/ops.py:366-428)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, residual, initial_state, output_final_state, activation, cu_seqlens, cu_seqlens_cpu,
+                chunk_indices):
+        ctx.activation = activation
+        ctx.cu_seqlens = cu_seqlens
+        ctx.cu_seqlens_cpu = cu_seqlens_cpu
+        ctx.chunk_indices = chunk_indices
+        ctx.save_for_backward(x, weight, bias, residual, initial_state)
+        return causal_conv1d_fwd(
+            x=x, weight=weight, bias=bias, residual=residual, initial_state=initial_state,
+            output_final_state=output_final_state, activation=activation, cu_seqlens=cu_seqlens, cu_seqlens_cpu=cu_seqlens_cpu)
+
+    @staticmethod
+    def backward(ctx, dy, dht=None):
+        x, weight, bias, residual, initial_state = ctx.saved_tensors
+        dx, dw, db, dr, dh0 = causal_conv1d_bwd(
+            x=x, dy=dy, dht=dht, weight=weight, bias=bias, residual=residual, initial_state=initial_state,
+            activation=ctx.activation, cu_seqlens=ctx.cu_seqlens, cu_seqlens_cpu=ctx.cu_seqlens_cpu,
+            chunk_indices=ctx.chunk_indices)
+        if residual is not None and dr.dtype != residual.dtype:
+            dr = dr.to(residual.dtype)
+        return dx, dw, db, dr, dh0, None, None, None, None, None
+
+
 @input_guard(no_guard_contiguous=['x'])
 def causal_conv1d_update_states(
     x: torch.Tensor,
@@ -191,11 +310,19 @@ def causal_conv1d(
     **kwargs,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """Causal 1D convolution over ``x [B, T, D]`` with ``weight [D, W]``; returns ``(y, final_state)``.
-    Every value of ``backend`` the reference accepts (`triton`, `cuda`, `mix`) runs the same HIP kernel."""
+    Every value of ``backend`` the reference accepts (`triton`, `cuda`, `mix`) runs the same HIP kernels.  Differentiable
+    in x, weight, bias, residual and initial_state."""
     if cp_context is not None:
         raise NotImplementedError('context parallelism (cp_context) spans several GPUs and is not supported')
     if backend not in ('triton', 'cuda', 'mix'):
         raise ValueError(f'Unsupported backend: {backend}')
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias, residual, initial_state)):
+        if weight is None:
+            raise ValueError('causal_conv1d_fwd needs a weight of shape [D, W]')
+        if weight.shape[1] > MAX_KERNEL_SIZE:
+            raise NotImplementedError(f'kernel sizes above {MAX_KERNEL_SIZE} are not supported (got {weight.shape[1]})')
+        return CausalConv1dFunction.apply(x, weight, bias, residual, initial_state, bool(output_final_state), activation,
+                                          cu_seqlens, cu_seqlens_cpu, chunk_indices)
     return causal_conv1d_fwd(
         x=x, weight=weight, bias=bias, residual=residual, initial_state=initial_state,
         output_final_state=output_final_state, activation=activation,
@@ -204,7 +331,7 @@ def causal_conv1d(
 
 class ShortConvolution(nn.Conv1d):
     """Depthwise causal convolution layer with the reference's parameters and call signature
-    (fla/modules/conv/short_conv.py:24-250); inference only."""
+    (fla/modules/conv/short_conv.py:24-250); the prefill form is differentiable, the one-token step is not."""
 
     def __init__(
         self,

@@ -79,6 +79,18 @@ def make_backends(BaseBackend):
             from fla_hip.modules import causal_conv1d_fwd
             return causal_conv1d_fwd(*args, **kwargs)
 
+        def causal_conv1d_bwd_verifier(self, x, dy, dht, weight=None, *args, **kwargs):
+            # (upstream calls this from its autograd function's backward, for a forward that may have run here)
+            if weight is None or weight.shape[-1] > 8:
+                return False, 'kernel size above 8 (or no weight)'
+            if kwargs.get('activation') not in (None, 'silu', 'swish'):
+                return False, 'activation'
+            return self._conv_ok(x, weight)
+
+        def causal_conv1d_bwd(self, *args, **kwargs):
+            from fla_hip.modules import causal_conv1d_bwd
+            return causal_conv1d_bwd(*args, **kwargs)
+
         def causal_conv1d_update_states_verifier(self, x, state_len, initial_state=None, cu_seqlens=None):
             if state_len > 8:
                 return False, 'kernel size above 8'
@@ -114,6 +126,25 @@ def make_backends(BaseBackend):
         def layer_norm_gated_fwd(self, *args, **kwargs):
             from fla_hip.modules import layer_norm_gated_fwd
             return layer_norm_gated_fwd(*args, **kwargs)
+
+        def layer_norm_gated_bwd_verifier(self, dy, x, g, weight, bias, activation='swish', eps=1e-5, mean=None, rstd=None,
+                                          dresidual=None, has_residual=False, is_rms_norm=False, x_dtype=None,
+                                          recompute_output=False):
+            if not _on_gfx950(x):
+                return False, 'not a gfx950 device'
+            if recompute_output:
+                return False, 'recompute_output (the fused norm + linear layer)'
+            if x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or x.dim() != 2:
+                return False, 'needs [T, D] rows of bf16, fp16 or fp32'
+            if x.shape[1] > 2048:
+                return False, 'feature dim above 2048'
+            if activation not in ('swish', 'silu', 'sigmoid'):
+                return False, 'activation'
+            return True, None
+
+        def layer_norm_gated_bwd(self, *args, **kwargs):
+            from fla_hip.modules import layer_norm_gated_bwd
+            return layer_norm_gated_bwd(*args, **kwargs)
 
     return HipGfx950Backend, HipGfx950ModulesBackend
 

@@ -368,6 +368,42 @@ int gdn_norm_gated_fwd(
     int x_dtype, int w_dtype, int res_dtype, int res_out_dtype, int activation, int is_rms_norm, void* stream);
 
 /*
+ * Backward of gdn_causal_conv1d_fwd.  Replaces causal_conv1d_bwd (fla/modules/conv/triton/ops.py:147-249: kernel
+ * fla/modules/conv/triton/kernels.py:142-353, and compute_dh0_triton, ops.py:100-144).
+ *   x, weight, bias, initial_state, cu_seqlens, strides, dtypes, activation, flags: the forward's arguments (the output before
+ *   the activation is recomputed from them); dy [B,T,D] x_dtype contiguous: gradient of y (the residual's gradient is dy itself);
+ *   dht [N,D,W] x_dtype or NULL: gradient of final_state
+ *   dx [B,T,D] x_dtype contiguous (packed input: tokens outside [cu_seqlens[0], cu_seqlens[N]) are not written)
+ *   dw_part [parts,D,W], db_part [parts,D] (NULL without bias) fp32 with parts = ceil(num_tiles / GDN_CONV_BWD_TILES_PER_PART):
+ *   one row of partial sums per run of that many 64-token tiles, to be added up by the caller (parts == 0: nothing is written);
+ *   dh0 [N,D,W] fp32 or NULL (needs initial_state)
+ *   tile_table [num_tiles,2]: (sequence, tile inside it) per 64-token tile of a packed input, in cu_seqlens' integer type
+ *   (the chunk table of gdn_chunk_fwd); dense input: NULL and num_tiles = B * ceil(T / 64)
+ *   Requires D % (16 / sizeof(element)) == 0 and 16-byte aligned rows.
+ */
+#define GDN_CONV_BWD_TILES_PER_PART 4
+int gdn_causal_conv1d_bwd(
+    const void* x, const void* weight, const void* bias, const void* initial_state, const void* dy, const void* dht,
+    void* dx, float* dw_part, float* db_part, float* dh0,
+    const void* cu_seqlens, const void* tile_table,
+    int64_t B, int64_t T, int64_t D, int64_t W, int64_t N, int64_t num_tiles, int64_t stride_x_n, int64_t stride_x_t,
+    int x_dtype, int w_dtype, int state_dtype, int activation, uint32_t flags, void* stream);
+
+/*
+ * Backward of gdn_norm_gated_fwd.  Replaces layer_norm_gated_bwd (fla/modules/fused_norm_gate.py:541-650, kernels :192-453).
+ *   dy, x, g, dx, dg: T rows of D features x_dtype, ld elements apart (ld >= D a multiple of 16 / sizeof(element), up to 2048;
+ *   dy must read as zero from D on); x is what was normalised (the forward's residual_out when there was a residual);
+ *   mean (NULL for rms norm), rstd [T] fp32 from the forward; dresidual (rows like dy) or NULL: gradient of residual_out, added to dx
+ *   dw_part, db_part [parts,ld] fp32 (NULL without weight / bias): one row of partial sums per workgroup, to be added up by the caller
+ */
+int gdn_norm_gated_bwd(
+    const void* dy, const void* x, const void* g, const void* weight, const void* bias,
+    const float* mean, const float* rstd, const void* dresidual,
+    void* dx, void* dg, float* dw_part, float* db_part,
+    int64_t T, int64_t D, int64_t ld, int64_t parts,
+    int x_dtype, int w_dtype, int activation, int is_rms_norm, void* stream);
+
+/*
  * Measurement aid with no counterpart in the reference (bench.py --workload calib_rmw): the memory traffic and the
  * dependency of a decode step without its arithmetic.  Every 64 KB block of `data` (n_floats a multiple of 16384)
  * is read, reduced across its workgroup and written back in place.  xcd_run > 0: every XCD works on runs of that

@@ -108,3 +108,35 @@ def norm_gated(x, g, weight=None, bias=None, residual=None, eps=1e-5, activation
     gg = g.to(dtype)
     y = y * gg * torch.sigmoid(gg) if activation in ('swish', 'silu') else y * torch.sigmoid(gg)
     return y, r, mean, rstd
+
+
+def conv_grads(x, weight, bias, residual, initial_state, dy, dht=None, activation=None, cu_seqlens=None, dtype=torch.float64):
+    """Gradients of ``causal_conv1d`` for the output gradients (dy, dht): reverse-mode differentiation of the oracle's own
+    forward in ``dtype`` (fla/modules/conv/triton/ops.py:147-249 computes the same quantities).  Returns a dict with
+    dx, dw, db, dr, dh0 (None where the input is absent)."""
+    leaves = {}
+    for name, t in (('x', x), ('w', weight), ('b', bias), ('r', residual), ('h0', initial_state)):
+        leaves[name] = None if t is None else t.detach().to(dtype).clone().requires_grad_(True)
+    y, final = causal_conv1d(leaves['x'], leaves['w'], leaves['b'], leaves['r'], leaves['h0'], dht is not None,
+                             activation, cu_seqlens, dtype)
+    loss = (y * dy.to(dtype)).sum()
+    if dht is not None:
+        loss = loss + (final * dht.to(dtype)).sum()
+    loss.backward()
+    return {('d' + k): (None if v is None else v.grad) for k, v in leaves.items()}
+
+
+def norm_gated_grads(x, g, weight, bias, residual, dy, dres_out=None, eps=1e-5, activation='swish', is_rms_norm=False,
+                     dtype=torch.float64):
+    """Gradients of ``norm_gated`` for the gradient dy of y and (prenorm) dres_out of the residual stream r:
+    reverse-mode differentiation of the oracle's own forward (fla/modules/fused_norm_gate.py:541-650 computes the same).
+    Returns a dict with dx, dg, dw, db, dr."""
+    leaves = {}
+    for name, t in (('x', x), ('g', g), ('w', weight), ('b', bias), ('r', residual)):
+        leaves[name] = None if t is None else t.detach().to(dtype).clone().requires_grad_(True)
+    y, r, _, _ = norm_gated(leaves['x'], leaves['g'], leaves['w'], leaves['b'], leaves['r'], eps, activation, is_rms_norm, dtype)
+    loss = (y * dy.to(dtype)).sum()
+    if dres_out is not None:
+        loss = loss + (r * dres_out.to(dtype)).sum()
+    loss.backward()
+    return {('d' + k): (None if v is None else v.grad) for k, v in leaves.items()}

@@ -299,10 +299,13 @@ def test_upstream_backends_follow_the_plugin_interface():
     x = torch.zeros(1, 4, 1, 8)
     assert chunk_gated_delta_rule(x, x, x, x[..., 0], x[..., 0]) == 'default' and calls == ['default']
     be = mod_cls()
-    for name in ('causal_conv1d_fwd', 'causal_conv1d_update_states', 'causal_conv1d_update', 'layer_norm_gated_fwd'):
+    for name in ('causal_conv1d_fwd', 'causal_conv1d_bwd', 'causal_conv1d_update_states', 'causal_conv1d_update', 'layer_norm_gated_fwd',
+                 'layer_norm_gated_bwd'):
         assert callable(getattr(be, name)) and callable(getattr(be, name + '_verifier'))
     assert be.verify('causal_conv1d_fwd', x[0], torch.zeros(8, 4))[0] is False
     assert be.verify('layer_norm_gated_fwd', x[0, :, 0], x[0, :, 0], None, None)[0] is False
+    assert be.verify('causal_conv1d_bwd', x[0], x[0], None, torch.zeros(8, 4))[0] is False
+    assert be.verify('layer_norm_gated_bwd', x[0, :, 0], x[0, :, 0], x[0, :, 0], None, None)[0] is False
     os.environ['FLA_HIP_GFX950'] = '0'
     try:
         assert not op_cls.is_enabled()
@@ -352,3 +355,20 @@ def test_upstream_backends_take_gpu_inference_calls_and_leave_the_rest():
     out = layer_norm_gated_fwd(x[0], x[1], None, None, is_rms_norm=True)
     assert len(out) == 4 and out[0].shape == x[0].shape and out[1] is None
     assert layer_norm_gated_fwd(x[0], x[1], None, None, activation='relu') == 'default'
+
+    # the backward entries upstream's autograd functions call (fla/modules/conv/triton/ops.py:411-428, fla/modules/fused_norm_gate.py:712-733)
+    @dispatch('upstream_test_modules')
+    def causal_conv1d_bwd(x, dy, dht, weight=None, bias=None, residual=None, initial_state=None, activation=None, **kwargs):
+        return ('default',) * 5
+
+    @dispatch('upstream_test_modules')
+    def layer_norm_gated_bwd(dy, x, g, weight, bias, activation='swish', eps=1e-5, mean=None, rstd=None, dresidual=None,
+                             has_residual=False, is_rms_norm=False, x_dtype=None, recompute_output=False):
+        return ('default',) * 5
+
+    dx, dw, db_, dr, dh0 = causal_conv1d_bwd(x, torch.randn_like(x), None, weight=w, activation='silu')
+    assert dx.shape == x.shape and dw.shape == w.shape and db_ is None and dr is None and dh0 is None
+    assert causal_conv1d_bwd(x, torch.randn_like(x), None, weight=w, activation='gelu')[0] == 'default'
+    grads = layer_norm_gated_bwd(x[0], x[0], x[1], None, None, rstd=out[2], is_rms_norm=True)
+    assert grads[0].shape == x[0].shape and grads[2] is None and grads[4] is None
+    assert layer_norm_gated_bwd(x[0], x[0], x[1], None, None, rstd=out[2], is_rms_norm=True, recompute_output=True)[0] == 'default'

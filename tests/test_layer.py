@@ -117,13 +117,67 @@ def test_padding_mask_equals_each_sequence_alone():
     assert torch.equal(out_p, want)
 
 
-def test_layer_refuses_training_and_missing_layer_idx():
+def _oracle_loss(layer, x, dy, cu=None):
+    """The layer as a composition of the oracles in fp64 on the CPU, differentiable: returns the gradients of
+    sum(out * dy) with respect to the input and every parameter (by name)."""
+    DT = torch.float64
+    p = {k: v.detach().to(DT).cpu().requires_grad_(True) for k, v in layer.state_dict().items()}
+    xs = x.detach().to(DT).cpu().requires_grad_(True)
+    lin = lambda name: F.linear(xs, p[f'{name}.weight'])
+    conv = lambda t, name: M.causal_conv1d(t, p[f'{name}.weight'].squeeze(1), p.get(f'{name}.bias'), activation='silu',
+                                           cu_seqlens=cu, dtype=DT)[0]
+    q, k, v = conv(lin('q_proj'), 'q_conv1d'), conv(lin('k_proj'), 'k_conv1d'), conv(lin('v_proj'), 'v_conv1d')
+    H, HV, K, V = layer.num_heads, layer.num_v_heads, layer.head_k_dim, layer.head_v_dim
+    q, k, v = q.unflatten(-1, (H, K)), k.unflatten(-1, (H, K)), v.unflatten(-1, (HV, V))
+    g = O.gdn_gate(lin('a_proj'), p['A_log'], p['dt_bias'])
+    beta = torch.sigmoid(lin('b_proj')) * (2.0 if layer.allow_neg_eigval else 1.0)
+    o, _ = O.recurrent_gated_delta_rule(O.l2norm(q), O.l2norm(k), v, g, beta, None, None, False, cu_seqlens=cu, dtype=DT)
+    gate = lin('g_proj').unflatten(-1, (HV, V))
+    y, *_ = M.norm_gated(o.reshape(-1, V), gate.reshape(-1, V), p['o_norm.weight'], None, None, layer.o_norm.eps, 'swish', True, DT)
+    out = F.linear(y.reshape(*o.shape[:2], HV * V), p['o_proj.weight'])
+    (out * dy.to(DT).cpu()).sum().backward()
+    return out.detach(), xs.grad, {k: v.grad for k, v in p.items()}
+
+
+@pytest.mark.parametrize('packed', [False, True])
+def test_layer_trains(packed):
+    """Training mode: the gradient of every parameter and of the input through the convolutions' , the chunked operator's and
+    the gated norm's backward kernels against reverse-mode differentiation of the oracles' composition.  Everything between
+    the projections is bf16 on the GPU, so the bar is that of a bf16 pipeline (2e-2 rel-RMSE; gate parameters, whose
+    gradients are small sums of many terms, 4e-2)."""
+    layer = _layer(seed=6).train()
+    gen = torch.Generator().manual_seed(7)
+    if packed:
+        x = torch.randn(1, 230, 256, generator=gen).to(BF)
+        cu = [0, 70, 71, 230]
+        kw = dict(cu_seqlens=torch.tensor(cu, device=DEV, dtype=torch.int32))
+    else:
+        x = torch.randn(2, 150, 256, generator=gen).to(BF)
+        cu, kw = None, {}
+    dy = torch.randn(*x.shape[:2], 256, generator=gen).to(BF)
+    xd = x.to(DEV).requires_grad_(True)
+    out, _, _ = layer(xd, **kw)
+    out.backward(dy.to(DEV))
+    ref_out, ref_dx, ref = _oracle_loss(layer, x, dy, cu)
+    assert O.get_err_ratio(ref_out, out.detach().double().cpu()) < 1e-2
+    assert O.get_err_ratio(ref_dx, xd.grad.double().cpu()) < 2e-2
+    for name, prm in layer.named_parameters():
+        assert prm.grad is not None, name
+        bar = 4e-2 if name in ('A_log', 'dt_bias') else 2e-2
+        err = O.get_err_ratio(ref[name], prm.grad.double().cpu())
+        assert err < bar, f'{name}: rel-RMSE {err:.3e}'
+    # a short call trains too (the chunk kernels take it), and eval mode builds no graph
+    layer.zero_grad()
+    short, _, _ = layer(xd[:, :8])
+    short.sum().backward()
+    assert layer.q_proj.weight.grad is not None
+    assert not layer.eval()(xd)[0].requires_grad
+
+
+def test_layer_missing_layer_idx():
     from fla_hip.layers import GatedDeltaNet, LayerCache
     layer = _layer()
     x = torch.randn(1, 8, 256, device=DEV, dtype=BF)
-    with pytest.raises(RuntimeError):
-        layer.train()(x)
-    layer.eval()
     layer.layer_idx = None
     with pytest.raises(ValueError):
         layer(x, past_key_values=LayerCache())

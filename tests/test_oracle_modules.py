@@ -142,3 +142,81 @@ def test_norm_gated_special_cases():
     assert torch.allclose(y, (w + b).expand(T, D) * 0.5, atol=1e-12)
     y, *_ = M.norm_gated(x, g, w, b, None, 1e-5, 'sigmoid', False, dtype=DT)
     assert torch.allclose(y, b.expand(T, D) * 0.5, atol=1e-12)
+
+
+# --------------------------------------------------------------------------- #
+# gradients
+# --------------------------------------------------------------------------- #
+def _fd(fn, t, eps=1e-6):
+    """Central finite differences of the scalar fn() with respect to every element of the fp64 tensor t."""
+    out = torch.zeros_like(t)
+    flat, oflat = t.view(-1), out.view(-1)
+    for i in range(flat.numel()):
+        keep = flat[i].item()
+        flat[i] = keep + eps
+        up = fn()
+        flat[i] = keep - eps
+        down = fn()
+        flat[i] = keep
+        oflat[i] = (up - down) / (2 * eps)
+    return out
+
+
+@pytest.mark.parametrize('activation', [None, 'silu'])
+@pytest.mark.parametrize('packed', [False, True])
+def test_conv_gradients_against_finite_differences(activation, packed):
+    """Every gradient the convolution's backward returns (input, taps, bias, residual, initial state), with the gradient of
+    the final state flowing in, against central differences of the forward in fp64; sequences shorter than the kernel
+    hand part of the initial state on to the final state."""
+    gen = torch.Generator().manual_seed(5)
+    W, D = 4, 3
+    if packed:
+        cu, B, T = [0, 2, 2, 9], 1, 9
+    else:
+        cu, B, T = None, 2, 5
+    N = B if cu is None else len(cu) - 1
+    x, w, b, r, h0 = (torch.randn(*s, generator=gen, dtype=torch.float64) for s in ((B, T, D), (D, W), (D,), (B, T, D), (N, D, W)))
+    dy = torch.randn(B, T, D, generator=gen, dtype=torch.float64)
+    dht = torch.randn(N, D, W, generator=gen, dtype=torch.float64)
+    grads = M.conv_grads(x, w, b, r, h0, dy, dht, activation, cu)
+
+    def loss():
+        y, final = M.causal_conv1d(x, w, b, r, h0, True, activation, cu, torch.float64)
+        return ((y * dy).sum() + (final * dht).sum()).item()
+
+    for name, t in (('dx', x), ('dw', w), ('db', b), ('dr', r), ('dh0', h0)):
+        assert (grads[name] - _fd(loss, t)).abs().max() < 1e-7, name
+    assert torch.equal(grads['dr'], dy)                         # the residual's gradient is dy itself
+    assert (grads['dh0'][:, :, 0].abs().max() == 0) == (not packed)      # entry 0 only matters to a sequence without tokens
+
+
+def test_conv_gradient_closed_forms():
+    """One tap and no activation: dx = w dy, dw = sum dy x; two taps: the gradient of x[t] collects dy[t] w[1] + dy[t+1] w[0]."""
+    gen = torch.Generator().manual_seed(6)
+    x, dy = torch.randn(1, 6, 2, generator=gen, dtype=torch.float64), torch.randn(1, 6, 2, generator=gen, dtype=torch.float64)
+    w1 = torch.randn(2, 1, generator=gen, dtype=torch.float64)
+    g1 = M.conv_grads(x, w1, None, None, None, dy)
+    assert torch.allclose(g1['dx'], dy * w1[:, 0]) and torch.allclose(g1['dw'][:, 0], (dy * x).sum((0, 1)))
+    w2 = torch.randn(2, 2, generator=gen, dtype=torch.float64)
+    g2 = M.conv_grads(x, w2, None, None, None, dy)
+    want = dy * w2[:, 1]
+    want[:, :-1] += dy[:, 1:] * w2[:, 0]
+    assert torch.allclose(g2['dx'], want)
+
+
+@pytest.mark.parametrize('activation', ['swish', 'sigmoid'])
+@pytest.mark.parametrize('is_rms', [False, True])
+def test_norm_gated_gradients_against_finite_differences(activation, is_rms):
+    gen = torch.Generator().manual_seed(7)
+    T, D = 3, 5
+    x, g, r, dy, dres = (torch.randn(T, D, generator=gen, dtype=torch.float64) for _ in range(5))
+    w, b = torch.randn(D, generator=gen, dtype=torch.float64), torch.randn(D, generator=gen, dtype=torch.float64)
+    grads = M.norm_gated_grads(x, g, w, b, r, dy, dres, 1e-5, activation, is_rms)
+
+    def loss():
+        y, rr, _, _ = M.norm_gated(x, g, w, b, r, 1e-5, activation, is_rms, torch.float64)
+        return ((y * dy).sum() + (rr * dres).sum()).item()
+
+    for name, t in (('dx', x), ('dg', g), ('dw', w), ('db', b), ('dr', r)):
+        assert (grads[name] - _fd(loss, t)).abs().max() < 1e-7, name
+    assert torch.equal(grads['dx'], grads['dr'])                # x and the residual enter as their sum
