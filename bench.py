@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|layer_train|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -279,6 +279,28 @@ def bench_comba(steps, warmup, device):
                 ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
 
 
+def bench_layer_train(steps, warmup, device):
+    """One training step (forward and backward) of the Gated DeltaNet layer with the reference's default sizes
+    (fla/layers/gated_deltanet.py:88-107: hidden 2048, 6 heads of K = 256, V = 512, convolutions of size 4) on one prompt:
+    torch matmuls for the projections, this library's kernels for everything between them, both ways."""
+    from fla_hip.layers import GatedDeltaNet
+    T = 32768
+    torch.manual_seed(0)
+    layer = GatedDeltaNet(hidden_size=2048, expand_v=2, head_dim=256, num_heads=6, layer_idx=0).to(device).bfloat16().train()
+    x = torch.randn(1, T, 2048, device=device, dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(1, T, 2048, device=device, dtype=torch.bfloat16)
+
+    def step():
+        out, _, _ = layer(x)
+        out.backward(dy)
+        x.grad = None
+        layer.zero_grad(set_to_none=True)
+
+    per_call, _ = _time_calls(step, steps, warmup)
+    return dict(workload=f'GatedDeltaNet layer (hidden 2048, H=6, K=256, V=512, conv 4) forward + backward, one prompt of {T} tokens, bf16',
+                ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(T / per_call, 1))
+
+
 def cpu_baseline_prefill(w, cpu):
     """Oracle (torch fp32 chunked form) on the first tokens of the same inputs; the sample
     length is chosen from a short calibration run so that the timed run takes ~10-20 s."""
@@ -492,7 +514,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'chunk_comba', 'layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'chunk_comba', 'layer_train', 'layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
@@ -524,6 +546,12 @@ def main():
     if args.workload == 'chunk_kda':
         r = bench_kda(args.steps, args.warmup, device)
         print(json.dumps(dict(metric='kda_chunk_prefill_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
+                              n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
+                              data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
+        return
+    if args.workload == 'layer_train':
+        r = bench_layer_train(args.steps, args.warmup, device)
+        print(json.dumps(dict(metric='gdn_layer_fwd_bwd_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
                               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'], dtype='bf16',
                               data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
         return
@@ -591,6 +619,8 @@ def main():
             extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
             torch.cuda.empty_cache()
         extra['chunk_kda_b1_t8192_h96_d128'] = bench_kda(max(10, args.steps // 4), max(3, args.warmup // 4), device)
+        extra['layer_train_t32768'] = bench_layer_train(max(5, args.steps // 10), 3, device)
+        torch.cuda.empty_cache()
         extra['chunk_comba_b1_t8192_h96_d128'] = bench_comba(max(10, args.steps // 4), max(3, args.warmup // 4), device)
         line['other_workloads'] = extra
     print(json.dumps(line))
