@@ -13,8 +13,10 @@ namespace gdn {
 //   dz[t] = dy[t] act'(z[t]);  dx[t] = sum_j w[j] dz[t + (W-1) - j]  (+ dht where t is one of the last W positions);
 //   dw[j] = sum_t dz[t] x[t - (W-1) + j];  db = sum_t dz[t];  positions in front of the sequence belong to the initial state
 // ---------------------------------------------------------------------------------------------
-constexpr int CB_TOK = 8, CB_CX = 32, CB_TY = 8;       // a thread: 8 bytes of channels x 8 tokens; a workgroup: 32 channel groups x 64 tokens
-constexpr int CB_BYTES = 8;                            // (measured against 16 bytes of channels and 16 tokens per thread: more registers, fewer waves, no faster)
+constexpr int CB_TOK = 8, CB_CX = 32, CB_TY = 8;       // a thread: 2 channels x 8 positions; a workgroup: 32 channel pairs x 64 tokens
+constexpr int CB_VEC = 2;                              // Two channels keep a thread at 134 registers (three waves per SIMD); measured for bf16 at
+                                                       // 32768 x 3072: 4 channels (232 registers, two waves) 240 us, 2 channels 207 us; 8 channels or 16
+                                                       // positions per thread: one wave per SIMD, 330 - 400 us; four waves by a register cap: spills, slower.
 constexpr int CB_MAX_W = 8;
 
 struct ConvBwdParams {
@@ -36,7 +38,7 @@ __device__ __forceinline__ float silu_grad(float z) {
 // the dz its last inputs feed), and the output gradients at its positions and the W-1 behind them.
 template <typename T, int W>
 struct ConvBwdRows {
-    typedef T vec_t __attribute__((ext_vector_type(CB_BYTES / sizeof(T))));
+    typedef T vec_t __attribute__((ext_vector_type(CB_VEC)));
     vec_t x[CB_TOK + 2 * (W - 1)];     // x[k]: position t0 - (W-1) + k
     vec_t dy[CB_TOK + W - 1];          // dy[i]: position t0 + i
 };
@@ -59,7 +61,7 @@ __device__ __forceinline__ ConvBwdTile conv_bwd_tile(const ConvBwdParams& p, int
 // state where a position lies in front of the sequence.
 template <typename T, int W>
 __device__ __forceinline__ void conv_bwd_fetch(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, ConvBwdRows<T, W>& r) {
-    constexpr int VEC = CB_BYTES / sizeof(T), NX = CB_TOK + 2 * (W - 1), NZ = CB_TOK + W - 1;
+    constexpr int VEC = CB_VEC, NX = CB_TOK + 2 * (W - 1), NZ = CB_TOK + W - 1;
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int D = (int)p.D;
     const int64_t t0 = g.it * (CB_TOK * CB_TY) + ty * CB_TOK;
@@ -93,9 +95,9 @@ __device__ __forceinline__ void conv_bwd_fetch(const ConvBwdParams& p, const Con
 // unrolled, so the window moves by renaming): dz[s] = dy[s] act'(z[s]);  dx[u] = sum_j w[j] dz[u + (W-1) - j].
 template <typename T, int W>
 __device__ __forceinline__ void conv_bwd_walk(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, const ConvBwdRows<T, W>& r,
-                                              const float (&wgt)[W][CB_BYTES / sizeof(T)], const float (&bias)[CB_BYTES / sizeof(T)],
-                                              float (&dwacc)[W][CB_BYTES / sizeof(T)], float (&dbacc)[CB_BYTES / sizeof(T)]) {
-    constexpr int VEC = CB_BYTES / sizeof(T);
+                                              const float (&wgt)[W][CB_VEC], const float (&bias)[CB_VEC],
+                                              float (&dwacc)[W][CB_VEC], float (&dbacc)[CB_VEC]) {
+    constexpr int VEC = CB_VEC;
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int D = (int)p.D;
     const int64_t t0 = g.it * (CB_TOK * CB_TY) + ty * CB_TOK, len = g.len;
@@ -152,7 +154,7 @@ __device__ __forceinline__ void conv_bwd_walk(const ConvBwdParams& p, const Conv
 // registers across them: one row of partial sums per such run.
 template <typename T, int W>
 __global__ __launch_bounds__(CB_CX * CB_TY, 2) void causal_conv1d_bwd_kernel(ConvBwdParams p) {
-    constexpr int VEC = CB_BYTES / sizeof(T);
+    constexpr int VEC = CB_VEC;
     __shared__ float red[W + 1][CB_TY][CB_CX * VEC];
     const int cx = threadIdx.x, ty = threadIdx.y;
     const int D = (int)p.D;
@@ -257,7 +259,7 @@ __global__ __launch_bounds__(256) void causal_conv1d_dh0_kernel(ConvBwdParams p)
 
 template <typename T>
 static int launch_conv_bwd(const ConvBwdParams& p, hipStream_t stream) {
-    constexpr int VEC = CB_BYTES / sizeof(T);
+    constexpr int VEC = CB_VEC;
     if (p.dx && p.num_tiles > 0) {
         const int64_t parts = (p.num_tiles + GDN_CONV_BWD_TILES_PER_PART - 1) / GDN_CONV_BWD_TILES_PER_PART;
         const int64_t blocks = ((p.D + CB_CX * VEC - 1) / (CB_CX * VEC)) * parts;
@@ -445,10 +447,10 @@ extern "C" int gdn_causal_conv1d_bwd(
     GDN_CHECK_ARG(x && weight && dy && dx && dw_part, GDN_ERR_INVALID, "%s: x, weight, dy, dx and dw_part are required", who);
     GDN_CHECK_ARG(!bias == !db_part, GDN_ERR_INVALID, "%s: db_part goes with bias", who);
     GDN_CHECK_ARG(!dh0 || initial_state, GDN_ERR_INVALID, "%s: dh0 needs initial_state", who);
-    const int64_t vec = x_dtype == GDN_DTYPE_F32 ? 4 : 8;
     GDN_CHECK_ARG(D < (1ll << 31) && stride_x_t >= D, GDN_ERR_INVALID, "%s: token stride %lld below D", who, (long long)stride_x_t);
-    GDN_CHECK_ARG(D % vec == 0 && stride_x_t % vec == 0 && stride_x_n % vec == 0 && aligned16(x) && aligned16(dy) && aligned16(dx), GDN_ERR_UNSUPPORTED,
-                  "%s: rows must start on 16-byte boundaries and D must be a multiple of %lld", who, (long long)vec);
+    const uintptr_t pair = (uintptr_t)CB_VEC * (x_dtype == GDN_DTYPE_F32 ? 4 : 2);     // a thread reads its two channels in one piece
+    GDN_CHECK_ARG(D % CB_VEC == 0 && stride_x_t % CB_VEC == 0 && stride_x_n % CB_VEC == 0 && (uintptr_t)x % pair == 0 && (uintptr_t)dy % pair == 0 &&
+                  (uintptr_t)dx % pair == 0, GDN_ERR_UNSUPPORTED, "%s: D and the strides of x must be even and rows must start on %d-byte boundaries", who, (int)pair);
     ConvBwdParams p{};
     p.x = x; p.weight = weight; p.bias = bias; p.initial_state = initial_state; p.dy = dy; p.dht = dht;
     p.dx = dx; p.dw_part = dw_part; p.db_part = db_part; p.dh0 = dh0;

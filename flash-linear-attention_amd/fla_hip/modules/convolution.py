@@ -133,10 +133,9 @@ def causal_conv1d_bwd(
     B, T, _ = x.shape
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     dy = dy.reshape(B, T, D).to(x.dtype).contiguous()
-    vec = 16 // x.element_size()
-    pad = (-D) % vec
-    if pad or x.data_ptr() % 16 or x.stride(1) % vec or x.stride(0) % vec:
-        # the kernel takes 16 bytes of channels per thread: bring odd layouts to that form
+    pad = D % 2
+    if pad or x.data_ptr() % (2 * x.element_size()) or x.stride(1) % 2 or x.stride(0) % 2:
+        # the kernel takes two adjacent channels per thread: bring odd layouts to that form
         x = F.pad(x, (0, pad)) if pad else x.clone(memory_format=torch.contiguous_format)
         dy = F.pad(dy, (0, pad))
         weight_k = F.pad(weight, (0, 0, 0, pad))

@@ -61,6 +61,8 @@ def test_flag_and_status_constants_match_the_header():
         assert getattr(_lib, 'FLAG_' + name) == value, name
     m = re.search(r'#define\s+GDN_CHUNK_STATIC_WORKSPACE_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)', header)
     assert int(m.group(1)) << int(m.group(2)) == _lib.CHUNK_STATIC_WORKSPACE_BYTES
+    m = re.search(r'#define\s+GDN_CONV_BWD_TILES_PER_PART\s+(\d+)', header)
+    assert int(m.group(1)) == _lib.CONV_BWD_TILES_PER_PART
     for name, value in re.findall(r'#define\s+(GDN_ERR_\w+|GDN_OK)\s+\(?(-?\d+)\)?', header):
         assert getattr(_lib, name) == int(value), name
 

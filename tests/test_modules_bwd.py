@@ -81,7 +81,8 @@ DENSE = [
     (2, 128, 128, 4, None, False, False, torch.float16),
     (2, 500, 1024, 4, 'silu', True, True, torch.bfloat16),
     (3, 77, 200, 2, 'silu', False, False, torch.bfloat16),
-    (1, 33, 100, 7, None, True, False, torch.bfloat16),        # channels not a multiple of 8: padded on the host
+    (1, 33, 100, 7, None, True, False, torch.bfloat16),
+    (2, 50, 77, 4, 'silu', True, True, torch.bfloat16),        # an odd number of channels: padded on the host
     (2, 40, 64, 1, 'silu', True, False, torch.float16),
     (2, 40, 64, 8, 'silu', False, True, torch.float32),
 ]
@@ -276,7 +277,7 @@ def test_modules_backward_c_entry_checks():
     assert conv(W=9) == _lib.GDN_ERR_UNSUPPORTED
     assert conv(tiles=2) == _lib.GDN_ERR_INVALID
     assert conv(dw=None) == _lib.GDN_ERR_INVALID
-    assert conv(D=60, stride=60) == _lib.GDN_ERR_UNSUPPORTED
+    assert conv(D=63, stride=63) == _lib.GDN_ERR_UNSUPPORTED               # channels go in pairs
 
     rstd = torch.ones(64, device=DEV)
     xr = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
