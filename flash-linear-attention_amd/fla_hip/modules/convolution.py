@@ -123,7 +123,8 @@ def causal_conv1d_bwd(
 ):
     """Gradients ``(dx, dw, db, dr, dh0)`` of ``causal_conv1d_fwd`` for the output gradient ``dy`` and the gradient ``dht``
     of the final state (``None``: none); ``dr`` is ``dy`` itself when there was a residual, ``dh0`` has the initial
-    state's dtype.  ``chunk_indices`` (tiles of 64 tokens), ``BT`` and ``layout_fallback`` as in the forward."""
+    state's dtype.  ``chunk_indices``, ``BT`` and ``layout_fallback`` steer the reference's tiling only and are accepted for
+    compatibility, as in the forward."""
     if weight is None:
         raise ValueError('causal_conv1d_bwd needs the weight of shape [D, W]')
     dev = require_gpu(x, dy)
@@ -160,9 +161,9 @@ def causal_conv1d_bwd(
         elif cu_seqlens.dtype != torch.int64:
             raise ValueError(f'cu_seqlens must be int32 or int64, got {cu_seqlens.dtype}')
         cu_seqlens = cu_seqlens.to(dev).contiguous()
-        if chunk_indices is None or BT != 64:
-            chunk_indices = prepare_chunk_indices(cu_seqlens, 64, cu_seqlens_cpu=cu_seqlens_cpu)
-        tile_table = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        # (a caller's chunk_indices may have been made for another tile size: the kernel's 64-token tiles are derived here)
+        tile_table = prepare_chunk_indices(cu_seqlens, 64, cu_seqlens_cpu=cu_seqlens_cpu)
+        tile_table = tile_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
         num_tiles = tile_table.shape[0]
         dx = torch.zeros(B, T, Dk, dtype=x.dtype, device=dev)   # tokens outside the sequences keep a zero gradient
     else:

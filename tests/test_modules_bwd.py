@@ -295,3 +295,44 @@ def test_modules_backward_c_entry_checks():
     assert norm(rs=None) == _lib.GDN_ERR_INVALID
     assert norm(rms=0) == _lib.GDN_ERR_INVALID                  # layer norm without the means
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('seed', range(16))
+def test_conv_backward_random_configuration(seed):
+    """Seeded random shapes and options: kernel sizes 1..8, odd and even channel counts, dense or packed with sequences from
+    empty to several tiles long, with or without bias / residual / initial state and final-state gradient, all three dtypes."""
+    gen = torch.Generator().manual_seed(2000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    W = r(1, 8)
+    D = [2, 6, 33, 64, 130, 256, 500][r(0, 6)]
+    dtype = [torch.float32, torch.float16, torch.bfloat16][r(0, 2)]
+    activation = [None, 'silu'][r(0, 1)]
+    has_bias, has_residual, state = bool(r(0, 1)), bool(r(0, 1)), bool(r(0, 1))
+    if r(0, 1):
+        lens = [[0, 1, 2, W - 1, W, 63, 64, 65, 130, 200][r(0, 9)] for _ in range(r(1, 5))]
+        if sum(lens) == 0:
+            lens[-1] = 3
+        cu = [0]
+        for n in lens:
+            cu.append(cu[-1] + n)
+        case = _conv_case(1, cu[-1], D, W, dtype, has_bias, has_residual, state=state, N=len(lens), seed=seed)
+        _check_conv(case, activation, cu, [torch.int32, torch.int64][r(0, 1)])
+    else:
+        B, T = r(1, 3), [1, 2, 7, 64, 65, 129, 300][r(0, 6)]
+        _check_conv(_conv_case(B, T, D, W, dtype, has_bias, has_residual, state=state, seed=seed), activation)
+
+
+@pytest.mark.parametrize('seed', range(16))
+def test_norm_gated_backward_random_configuration(seed):
+    gen = torch.Generator().manual_seed(3000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))
+    D = [8, 50, 64, 100, 128, 256, 384, 520, 1024, 2048][r(0, 9)]
+    rows = [1, 3, 40, 257, 1000][r(0, 4)]
+    dtype = [torch.float32, torch.float16, torch.bfloat16][r(0, 2)]
+    is_rms = bool(r(0, 1))
+    affine = bool(r(0, 1))
+    bias = affine and not is_rms and bool(r(0, 1))
+    residual = bool(r(0, 1))
+    prenorm = residual and bool(r(0, 1))
+    _check_norm((rows,), D, dtype, affine, bias, ['swish', 'sigmoid'][r(0, 1)], is_rms, residual=residual, prenorm=prenorm,
+                fp32_stream=prenorm and bool(r(0, 1)), seed=seed)
