@@ -191,7 +191,7 @@ template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * 
 template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
 template <typename T, int VBT, int KT, int AHEAD, int NW>
-__device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid) {
+__device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
@@ -201,9 +201,9 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
-    const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
+    const int64_t run = (int64_t)(bid / (8 * NVS)) * 8 + bid % 8;
     if (run >= p.N * p.HV) return;
-    const int vs = (blockIdx.x / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
+    const int vs = (bid / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
     const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
@@ -317,11 +317,11 @@ template <int VBT> constexpr int scan_waves() { return VBT == BD ? 8 : 4; }
 template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_state_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x);
+    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x, blockIdx.x);
 }
 
 template <typename T, int VBT, int KT, int AHEAD, int NW>
-__device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid) {
+__device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
@@ -332,9 +332,9 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.
-    const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;
+    const int64_t run = (int64_t)(bid / (8 * NVS)) * 8 + bid % 8;
     if (run >= p.N * p.HV) return;
-    const int vs = (blockIdx.x / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
+    const int vs = (bid / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
     const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
@@ -471,7 +471,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x);
+    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x, blockIdx.x);
 }
 
 // Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
@@ -484,8 +484,21 @@ template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
     static_assert(bwd_state_smem<VBT, KT>() % 16 == 0, "the second set of tiles starts 16-byte aligned");
-    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x);
-    else bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256);
+    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x);
+    else bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256, blockIdx.x);
+}
+
+// Both scans in one launch, in workgroups of their own: the first `nstate` workgroups walk forwards, the others backwards.
+// For calls whose two scans together leave CUs without a workgroup (few heads, long sequences) and whose tiles do not fit a
+// CU side by side (two blocks of key features): the launch then takes the time of the longer scan instead of their sum.
+template <int VBT, int KT> constexpr size_t bwd_scans_apart_smem() {
+    return bwd_state_smem<VBT, KT>() > bwd_dstate_smem<VBT, KT>() ? bwd_state_smem<VBT, KT>() : bwd_dstate_smem<VBT, KT>();
+}
+template <typename T, int VBT, int KT>
+__global__ __launch_bounds__(256) void gdn_bwd_scans_apart_kernel(BwdParams p, int64_t nstate) {
+    extern __shared__ __align__(16) char smem[];
+    if (blockIdx.x >= nstate) bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x - (unsigned)nstate);
+    else bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1001,6 +1014,13 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
             dstate.grid = 0;
         }
     }
+    int64_t second_arg[5] = {units, units, units, units, units};    // (the kernels that walk over the units take their number)
+    if (vbt == 32 && vbt_d == 32 && dstate.grid != 0 && state.grid + dstate.grid <= 256u) {
+        // both scans in one launch, each in workgroups of its own (the second entry then has nothing to launch)
+        second_arg[1] = state.grid;
+        state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, KT>, bwd_scans_apart_smem<32, KT>(), "gdn_bwd_scans_apart_kernel", state.grid + dstate.grid};
+        dstate.grid = 0;
+    }
     const K ks[5] = {
         {(const void*)gdn_bwd_prepare_kernel<T, KT>, bwd_prep_smem<KT>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
@@ -1011,8 +1031,7 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
     for (int i = 0; i < 5; ++i) {
         if (ks[i].grid == 0) continue;
         if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
-        int64_t nunits = units;
-        void* args[] = {(void*)&p, (void*)&nunits};             // (the kernels that walk over the units take their number)
+        void* args[] = {(void*)&p, (void*)&second_arg[i]};
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(threads[i]), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
     }
