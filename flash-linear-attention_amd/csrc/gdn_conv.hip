@@ -266,7 +266,7 @@ extern "C" int gdn_causal_conv1d_fwd(
     void* y, void* final_state, const void* cu_seqlens,
     int64_t B, int64_t T, int64_t D, int64_t W, int64_t N, int64_t stride_x_n, int64_t stride_x_t,
     int x_dtype, int w_dtype, int state_dtype, int activation, uint32_t flags, void* stream) {
-    GDN_CHECK_ARG(x && (y || final_state), GDN_ERR_INVALID, "gdn_causal_conv1d_fwd: x and one of y, final_state are required");
+    GDN_CHECK_ARG((x && (y || final_state)) || B * T == 0, GDN_ERR_INVALID, "gdn_causal_conv1d_fwd: x and one of y, final_state are required");
     GDN_CHECK_ARG(!y || weight, GDN_ERR_INVALID, "gdn_causal_conv1d_fwd: y needs a weight");
     GDN_CHECK_ARG(B >= 0 && T >= 0 && D >= 1 && N >= 0, GDN_ERR_INVALID, "gdn_causal_conv1d_fwd: bad sizes B=%lld T=%lld D=%lld N=%lld",
                   (long long)B, (long long)T, (long long)D, (long long)N);

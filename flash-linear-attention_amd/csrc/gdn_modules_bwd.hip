@@ -444,7 +444,7 @@ extern "C" int gdn_causal_conv1d_bwd(
     GDN_CHECK_ARG(!cu_seqlens || tile_table || num_tiles == 0, GDN_ERR_INVALID, "%s: packed input needs the table of 64-token tiles", who);
     GDN_CHECK_ARG(cu_seqlens || num_tiles == B * ((T + 63) / 64), GDN_ERR_INVALID, "%s: num_tiles does not match B and T", who);
     if (B * T == 0 && !dh0) return GDN_OK;
-    GDN_CHECK_ARG(x && weight && dy && dx && dw_part, GDN_ERR_INVALID, "%s: x, weight, dy, dx and dw_part are required", who);
+    GDN_CHECK_ARG(weight && (B * T == 0 || (x && dy && dx && dw_part)), GDN_ERR_INVALID, "%s: x, weight, dy, dx and dw_part are required", who);
     GDN_CHECK_ARG(!bias == !db_part, GDN_ERR_INVALID, "%s: db_part goes with bias", who);
     GDN_CHECK_ARG(!dh0 || initial_state, GDN_ERR_INVALID, "%s: dh0 needs initial_state", who);
     GDN_CHECK_ARG(D < (1ll << 31) && stride_x_t >= D, GDN_ERR_INVALID, "%s: token stride %lld below D", who, (long long)stride_x_t);
@@ -479,8 +479,8 @@ extern "C" int gdn_norm_gated_bwd(
     const int64_t vec = x_dtype == GDN_DTYPE_F32 ? 4 : 8;
     GDN_CHECK_ARG(ld % vec == 0 && ld <= 2048, GDN_ERR_UNSUPPORTED, "%s: the row pitch must be a multiple of %lld up to 2048 (got %lld)", who,
                   (long long)vec, (long long)ld);
-    GDN_CHECK_ARG(dy && x && g && rstd && dx && dg, GDN_ERR_INVALID, "%s: dy, x, g, rstd, dx and dg are required", who);
-    GDN_CHECK_ARG(is_rms_norm || mean, GDN_ERR_INVALID, "%s: layer norm needs the rows' means", who);
+    GDN_CHECK_ARG(T == 0 || (dy && x && g && rstd && dx && dg), GDN_ERR_INVALID, "%s: dy, x, g, rstd, dx and dg are required", who);
+    GDN_CHECK_ARG(T == 0 || is_rms_norm || mean, GDN_ERR_INVALID, "%s: layer norm needs the rows' means", who);
     GDN_CHECK_ARG(!weight == !dw_part && !bias == !db_part, GDN_ERR_INVALID, "%s: dw_part goes with weight and db_part with bias", who);
     GDN_CHECK_ARG(aligned16(dy) && aligned16(x) && aligned16(g) && aligned16(dx) && aligned16(dg) && aligned16(dresidual), GDN_ERR_UNSUPPORTED,
                   "%s: tensors must be 16-byte aligned", who);

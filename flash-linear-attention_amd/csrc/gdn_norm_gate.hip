@@ -236,7 +236,7 @@ extern "C" int gdn_norm_gated_fwd(
     int64_t T, int64_t D, float eps,
     int x_dtype, int w_dtype, int res_dtype, int res_out_dtype, int activation, int is_rms_norm, void* stream) {
     auto is_dtype = [](int d) { return d == GDN_DTYPE_BF16 || d == GDN_DTYPE_F16 || d == GDN_DTYPE_F32; };
-    GDN_CHECK_ARG(x && g && y, GDN_ERR_INVALID, "gdn_norm_gated_fwd: x, g and y are required");
+    GDN_CHECK_ARG((x && g && y) || T == 0, GDN_ERR_INVALID, "gdn_norm_gated_fwd: x, g and y are required");
     GDN_CHECK_ARG(T >= 0 && D >= 1 && T < (1ll << 31), GDN_ERR_INVALID, "gdn_norm_gated_fwd: bad sizes T=%lld D=%lld", (long long)T, (long long)D);
     GDN_CHECK_ARG(D <= 65536 / (x_dtype == GDN_DTYPE_F32 ? 4 : 2), GDN_ERR_UNSUPPORTED,
                   "gdn_norm_gated_fwd: rows of 64 KB and more are not supported (D=%lld)", (long long)D);

@@ -336,3 +336,22 @@ def test_norm_gated_backward_random_configuration(seed):
     prenorm = residual and bool(r(0, 1))
     _check_norm((rows,), D, dtype, affine, bias, ['swish', 'sigmoid'][r(0, 1)], is_rms, residual=residual, prenorm=prenorm,
                 fp32_stream=prenorm and bool(r(0, 1)), seed=seed)
+
+
+def test_modules_backward_without_tokens():
+    """No tokens at all: zero parameter gradients, an initial state that is handed straight on to the final state."""
+    mods = _mods()
+    x = torch.zeros(2, 0, 64, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    w = torch.randn(64, 4, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    b = torch.randn(64, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    h0 = torch.randn(2, 64, 4, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    y, final = mods.causal_conv1d(x, w, b, None, h0, True, 'silu')
+    assert y.shape == (2, 0, 64) and torch.equal(final, h0.detach())
+    dht = torch.randn_like(final)
+    (final.float() * dht.float()).sum().backward()
+    assert torch.equal(h0.grad, dht) and not w.grad.any() and not b.grad.any() and x.grad.shape == x.shape
+    xn = torch.zeros(0, 128, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    wn = torch.randn(128, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    out = mods.rms_norm_gated(xn, xn.detach(), wn, None)
+    out.sum().backward()
+    assert xn.grad.shape == xn.shape and not wn.grad.any()
