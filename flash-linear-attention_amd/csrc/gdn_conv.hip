@@ -297,7 +297,7 @@ extern "C" int gdn_causal_conv1d_update(
     const void* x, void* cache, const void* residual, const void* weight, const void* bias, void* y,
     int64_t N, int64_t D, int64_t W, int64_t stride_x_n, int64_t stride_y_n,
     int x_dtype, int w_dtype, int cache_dtype, int activation, void* stream) {
-    GDN_CHECK_ARG(x && y, GDN_ERR_INVALID, "gdn_causal_conv1d_update: x and y are required");
+    GDN_CHECK_ARG((x && y) || N == 0, GDN_ERR_INVALID, "gdn_causal_conv1d_update: x and y are required");
     GDN_CHECK_ARG(N >= 0 && D >= 1, GDN_ERR_INVALID, "gdn_causal_conv1d_update: bad sizes N=%lld D=%lld", (long long)N, (long long)D);
     GDN_CHECK_ARG(W >= 1 && W <= CONV_MAX_W, GDN_ERR_UNSUPPORTED, "gdn_causal_conv1d_update: kernel size %lld outside 1..%d", (long long)W, CONV_MAX_W);
     GDN_CHECK_ARG(is_dtype(x_dtype) && is_dtype(w_dtype) && is_dtype(cache_dtype), GDN_ERR_UNSUPPORTED, "gdn_causal_conv1d_update: unknown dtype");

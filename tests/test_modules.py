@@ -446,3 +446,18 @@ def test_norm_gated_random_configuration(seed):
         _close('residual_out', r, rout, res.dtype)
     else:
         assert rout is gx or rout.data_ptr() == gx.data_ptr()
+
+
+def test_modules_without_tokens_or_sequences():
+    mods = _mods()
+    x = torch.zeros(2, 0, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.randn(64, 4, device=DEV, dtype=torch.bfloat16)
+    h0 = torch.randn(2, 64, 4, device=DEV, dtype=torch.bfloat16)
+    y, final = mods.causal_conv1d(x, w, None, None, h0, True, 'silu')
+    assert y.shape == (2, 0, 64) and torch.equal(final, h0)
+    y, cache = mods.causal_conv1d_update(torch.zeros(0, 64, device=DEV, dtype=torch.bfloat16),
+                                         torch.zeros(0, 64, 4, device=DEV, dtype=torch.bfloat16), weight=w)
+    assert y.shape[0] == 0 and cache.shape == (0, 64, 4)
+    out = mods.rms_norm_gated(torch.zeros(0, 128, device=DEV, dtype=torch.bfloat16), torch.zeros(0, 128, device=DEV, dtype=torch.bfloat16),
+                              torch.ones(128, device=DEV, dtype=torch.bfloat16), None)
+    assert out.shape == (0, 128)
