@@ -11,6 +11,7 @@ import torch.nn.functional as F
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
     aligned16,
+    check_operand_shapes,
     as_f32,
     current_stream_ptr,
     dtype_code,
@@ -33,6 +34,9 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
     """Returns ``(o [B,T,HV,V] in q's dtype, final_state [N,HV,K,V] fp32 or None)``.  The kernels take 16-bit operands
     (the state and all sums are fp32); inputs of another dtype are converted to ``fp32_as`` first."""
     dev = require_gpu(q, k, v, p, g, beta)
+    check_operand_shapes(q, k, v, g=g, beta=beta)
+    if p.shape != q.shape:
+        raise ValueError(f'q, k and p must share one shape, got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(p.shape)}')
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if K > _DIM:

@@ -64,6 +64,40 @@ def unify_gate_beta(g, beta):
     return as_f32(g), as_f32(beta), _lib.DTYPE_F32
 
 
+def check_operand_shapes(q, k, v, g=None, beta=None, gk=None, gv=None, beta_per_column: bool = False) -> None:
+    """The kernels index every operand from B, T, H, K of q and HV, V of v: anything of another shape would be read out
+    of bounds, so it is refused here.  q, k ``[B,T,H,K]``; v ``[B,T,HV,V]``; g, beta ``[B,T,HV]`` (a trailing dimension of 1
+    is let through; beta ``[B,T,HV,V]`` where the operator takes one per value column); gk ``[B,T,HV,K]``; gv ``[B,T,HV,V]``."""
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError(f'q, k, v must be [B, T, heads, dim], got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}')
+    if k.shape != q.shape:
+        raise ValueError(f'q and k must have the same shape, got {tuple(q.shape)} and {tuple(k.shape)}')
+    if v.shape[:2] != q.shape[:2]:
+        raise ValueError(f'v must share batch and sequence length with q, got {tuple(v.shape)} and {tuple(q.shape)}')
+    B, T, H, K = q.shape
+    HV, V = v.shape[2], v.shape[3]
+    if HV % H != 0:
+        raise ValueError(f'num_v_heads (HV={HV}) must be divisible by num_heads (H={H})')
+
+    def per_head(x, name, last=None):
+        want = (B, T, HV) if last is None else (B, T, HV, last)
+        ok = tuple(x.shape) == want or (last is None and tuple(x.shape) == (B, T, HV, 1))
+        if not ok:
+            raise ValueError(f'{name} must have shape {want}, got {tuple(x.shape)}')
+
+    if g is not None:
+        per_head(g, 'g')
+    if beta is not None:
+        if beta_per_column and beta.dim() == 4 and beta.shape[-1] != 1:
+            per_head(beta, 'beta', V)
+        else:
+            per_head(beta, 'beta')
+    if gk is not None:
+        per_head(gk, 'gk', K)
+    if gv is not None:
+        per_head(gv, 'gv', V)
+
+
 def current_stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 

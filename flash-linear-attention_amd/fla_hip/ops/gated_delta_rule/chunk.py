@@ -16,6 +16,7 @@ import torch
 from fla_hip import _lib
 from fla_hip.ops.backends import dispatch
 from fla_hip.ops.gated_delta_rule._common import (
+    check_operand_shapes,
     aligned16,
     as_f32,
     current_stream_ptr,
@@ -62,6 +63,7 @@ class ChunkLaunch:
                  cu_seqlens=None, cu_seqlens_cpu=None, chunk_indices=None, chunk_size=64,
                  A_log=None, dt_bias=None, qk_l2norm=False, beta_sigmoid=False, neg_eigval=False):
         dev = require_gpu(q, k, v, beta) if g is None else require_gpu(q, k, v, g, beta)
+        check_operand_shapes(q, k, v, g=g, beta=beta)
         B, T, H, K = k.shape
         HV, V = v.shape[2], v.shape[3]
         N = B if cu_seqlens is None else len(cu_seqlens) - 1

@@ -10,7 +10,7 @@ import torch
 import torch.nn.functional as F
 
 from fla_hip import _lib
-from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, current_stream_ptr, dtype_code, ptr, require_gpu
+from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, check_operand_shapes, current_stream_ptr, dtype_code, ptr, require_gpu
 from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
@@ -45,6 +45,9 @@ def chunk_gated_delta_rule_bwd(
     passed as q and k) dq and dk are the gradients of the rows before normalisation: the reference's ``l2norm_bwd``
     (chunk.py:385-387) happens in the kernel that also adds up the value heads of a q/k head."""
     dev = require_gpu(q, k, v, beta, do)
+    check_operand_shapes(q, k, v, g=g, beta=beta)
+    if do.shape != v.shape:
+        raise ValueError(f'do must have the shape of v, got {tuple(do.shape)} and {tuple(v.shape)}')
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if K > 2 * _DIM:

@@ -9,6 +9,7 @@ import torch
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
+    check_operand_shapes,
     aligned16,
     as_f32,
     current_stream_ptr,
@@ -58,6 +59,7 @@ def fused_recurrent_gated_delta_rule_fwd(
     (mode 0: log decays; 1, 2: raw, activated in the kernel with ``A_log [HV]``, ``dt_bias [HV, K]`` and
     ``lower_bound``), and ``g``, ``gv`` must be absent."""
     dev = require_gpu(q, k, v)
+    check_operand_shapes(q, k, v, g=g, beta=beta, gk=gk, gv=gv, beta_per_column=True)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     N = B if cu_seqlens is None else len(cu_seqlens) - 1

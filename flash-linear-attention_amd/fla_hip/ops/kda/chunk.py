@@ -11,6 +11,7 @@ import torch.nn.functional as F
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
     aligned16,
+    check_operand_shapes,
     as_f32,
     current_stream_ptr,
     dtype_code,
@@ -34,6 +35,7 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
     """Returns ``(o [B,T,HV,V] in q's dtype, final_state fp32 or None)``; ``gate_mode`` 0: g is the log decay,
     1: ``-exp(A_log) softplus(g + dt_bias)``, 2: ``lower_bound sigmoid(exp(A_log) (g + dt_bias))``."""
     dev = require_gpu(q, k, v, g, beta)
+    check_operand_shapes(q, k, v, beta=beta, gk=g)
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if K > _DIM:

@@ -374,3 +374,25 @@ def test_upstream_backends_take_gpu_inference_calls_and_leave_the_rest():
     grads = layer_norm_gated_bwd(x[0], x[0], x[1], None, None, rstd=out[2], is_rms_norm=True)
     assert grads[0].shape == x[0].shape and grads[2] is None and grads[4] is None
     assert layer_norm_gated_bwd(x[0], x[0], x[1], None, None, rstd=out[2], is_rms_norm=True, recompute_output=True)[0] == 'default'
+
+
+def test_operand_shapes_are_checked_before_anything_reaches_a_kernel():
+    """g, beta, gk, gv of a shape other than the one q and v imply would be read out of bounds by the kernels: the host
+    refuses them (the helper itself needs no GPU)."""
+    import torch
+    from fla_hip.ops.gated_delta_rule._common import check_operand_shapes
+    q = torch.zeros(2, 8, 2, 16)
+    v = torch.zeros(2, 8, 4, 32)
+    g = torch.zeros(2, 8, 4)
+    check_operand_shapes(q, q, v, g=g, beta=g, gk=torch.zeros(2, 8, 4, 16), gv=torch.zeros(2, 8, 4, 32))
+    check_operand_shapes(q, q, v, g=g[..., None], beta=torch.zeros(2, 8, 4, 32), beta_per_column=True)
+    for bad in (dict(g=torch.zeros(2, 8, 2)), dict(beta=torch.zeros(2, 8, 4, 32)), dict(gk=g), dict(gk=torch.zeros(2, 8, 4, 32)),
+                dict(gv=torch.zeros(2, 8, 4, 16)), dict(beta=torch.zeros(2, 7, 4))):
+        with pytest.raises(ValueError, match='must have shape'):
+            check_operand_shapes(q, q, v, **bad)
+    with pytest.raises(ValueError, match='same shape'):
+        check_operand_shapes(q, q[..., :8], v)
+    with pytest.raises(ValueError, match='batch and sequence'):
+        check_operand_shapes(q, q, v[:, :4])
+    with pytest.raises(ValueError, match='divisible'):
+        check_operand_shapes(q, q, v[:, :, :3])
