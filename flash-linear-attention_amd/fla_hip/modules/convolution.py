@@ -52,6 +52,8 @@ def _launch_fwd(x, weight, bias, residual, initial_state, want_y, want_state, ac
         if tuple(initial_state.shape) != (N, D, W):
             raise ValueError(f'initial_state must be [{N}, {D}, {W}], got {tuple(initial_state.shape)}')
         initial_state = initial_state.contiguous()
+    if bias is not None and bias.numel() != D:
+        raise ValueError(f'bias must have {D} entries, got {bias.numel()}')
     flags = 0
     if cu_seqlens is not None:
         if cu_seqlens.dtype == torch.int32:
@@ -133,6 +135,11 @@ def causal_conv1d_bwd(
     x = _rows(x, D)
     B, T, _ = x.shape
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    if cu_seqlens is not None and B != 1:
+        raise ValueError(f'The batch size is expected to be 1 rather than {B} when using `cu_seqlens`.')
+    for name, t, want in (('bias', bias, (D,)), ('initial_state', initial_state, (N, D, W)), ('dht', dht, (N, D, W))):
+        if t is not None and tuple(t.shape) != want:
+            raise ValueError(f'{name} must have shape {want}, got {tuple(t.shape)}')
     dy = dy.reshape(B, T, D).to(x.dtype).contiguous()
     pad = D % 2
     if pad or x.data_ptr() % (2 * x.element_size()) or x.stride(1) % 2 or x.stride(0) % 2:

@@ -63,6 +63,8 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
     gw, bw = as_f32(g).contiguous(), as_f32(beta).contiguous()
     h0 = None
     if initial_state is not None:
+        if tuple(initial_state.shape) != (N, HV, K, V):
+            raise ValueError(f'initial_state must have shape {(N, HV, K, V)}, got {tuple(initial_state.shape)}')
         h0 = aligned16(F.pad(as_f32(initial_state), (0, _DIM - V, 0, _DIM - K)).contiguous())
 
     flags = _lib.FLAG_QK_L2NORM if use_qk_l2norm_in_kernel else 0

@@ -94,6 +94,9 @@ def chunk_gated_delta_rule_bwd(
     def state_in(s):
         if s is None:
             return None
+        want = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+        if tuple(s.shape) != want:
+            raise ValueError(f'initial_state and dht must have shape {want}, got {tuple(s.shape)}')
         s = as_f32(s)
         if state_v_first:
             s = s.transpose(-1, -2)

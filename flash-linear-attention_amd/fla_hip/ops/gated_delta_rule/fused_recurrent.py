@@ -66,6 +66,10 @@ def fused_recurrent_gated_delta_rule_fwd(
     q, k, v = unify_qkv(q, k, v)
     g, beta, gb_code = unify_gate_beta(g, beta)
     gk, gv, A_log, dt_bias = as_f32(gk), as_f32(gv), as_f32(A_log), as_f32(dt_bias)
+    if A_log is not None and A_log.numel() != HV:
+        raise ValueError(f'A_log must have {HV} entries, got {A_log.numel()}')
+    if dt_bias is not None and dt_bias.numel() != (HV * K if kda_gate_mode is not None else HV):
+        raise ValueError(f'dt_bias must have {HV * K if kda_gate_mode is not None else HV} entries, got {dt_bias.numel()}')
 
     # The kernel moves 16-byte pieces of state rows.  Head dims that are not multiples of 4 are zero-padded
     # here (zero key features and zero value columns change nothing else) and the results cut back.

@@ -81,6 +81,9 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
         dt_bias = _pad_last(dt_bias.detach().to(device=dev, dtype=torch.float32).reshape(HV, K), _DIM).contiguous()
     h0 = None
     if initial_state is not None:
+        want = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+        if tuple(initial_state.shape) != want:
+            raise ValueError(f'initial_state must have shape {want}, got {tuple(initial_state.shape)}')
         h0 = as_f32(initial_state)
         if state_v_first:
             h0 = h0.transpose(-1, -2)
