@@ -15,7 +15,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import current_stream_ptr, dtype_code, forward_only, ptr, require_gpu
-from fla_hip.ops.utils.index import prepare_chunk_indices
+from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices
 from fla_hip.utils import input_guard
 
 MAX_KERNEL_SIZE = 8
@@ -169,6 +169,7 @@ def causal_conv1d_bwd(
             raise ValueError(f'cu_seqlens must be int32 or int64, got {cu_seqlens.dtype}')
         cu_seqlens = cu_seqlens.to(dev).contiguous()
         # (a caller's chunk_indices may have been made for another tile size: the kernel's 64-token tiles are derived here)
+        check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
         tile_table = prepare_chunk_indices(cu_seqlens, 64, cu_seqlens_cpu=cu_seqlens_cpu)
         tile_table = tile_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
         num_tiles = tile_table.shape[0]

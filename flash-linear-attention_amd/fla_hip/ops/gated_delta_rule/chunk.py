@@ -25,7 +25,7 @@ from fla_hip.ops.gated_delta_rule._common import (
     require_gpu,
     unify_gate_beta,
 )
-from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
 from fla_hip.utils import input_guard
 
 # The HIP kernels work on 64-token chunks.  The result of the operator does not depend on
@@ -104,8 +104,10 @@ class ChunkLaunch:
                 cu_seqlens = cu_seqlens.to(dev)
             if cu_seqlens.dtype == torch.int32:
                 flags |= _lib.FLAG_CU_INT32
-            if chunk_indices is None or chunk_size != _KERNEL_CHUNK:
-                chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+            check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
+            # (a caller's chunk_indices are not taken over: the kernels index with them, so they are derived here from the
+            # boundaries just checked - memoised per cu_seqlens tensor, as the reference's are)
+            chunk_indices = prepare_chunk_indices(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
             chunk_indices = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
             # chunk offsets per sequence, followed by the longest-first order of the sequences
             chunk_offsets = prepare_scan_tables(cu_seqlens, _KERNEL_CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)

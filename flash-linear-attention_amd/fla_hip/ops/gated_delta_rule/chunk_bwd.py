@@ -11,7 +11,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, check_operand_shapes, current_stream_ptr, dtype_code, ptr, require_gpu
-from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
 _DIM = 128          # value columns of the backward kernels; key features: 128 or 256 (other head dims are zero-padded)
@@ -111,8 +111,8 @@ def chunk_gated_delta_rule_bwd(
         cu_seqlens = cu_seqlens.to(dev)
         if cu_seqlens.dtype == torch.int32:
             flags |= _lib.FLAG_CU_INT32
-        if chunk_indices is None or chunk_size != _CHUNK:
-            chunk_indices = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
+        chunk_indices = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)      # (derived here, never taken over)
         chunk_table = chunk_indices.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
         chunk_offsets = prepare_scan_tables(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
         num_chunks = chunk_table.shape[0]

@@ -19,7 +19,7 @@ from fla_hip.ops.gated_delta_rule._common import (
     ptr,
     require_gpu,
 )
-from fla_hip.ops.utils.index import prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
 _DIM = 128          # head dims of the kernels; smaller ones are zero-padded
@@ -101,6 +101,7 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
         cu_seqlens = cu_seqlens.to(dev)
         if cu_seqlens.dtype == torch.int32:
             flags |= _lib.FLAG_CU_INT32
+        check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
         chunk_table = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
         chunk_table = chunk_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
         chunk_offsets = prepare_scan_tables(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)

@@ -15,10 +15,27 @@ def prepare_lens(cu_seqlens: torch.Tensor) -> torch.Tensor:
     return cu_seqlens[1:] - cu_seqlens[:-1]
 
 
-def _host_lens(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None) -> torch.Tensor:
+@tensor_cache
+def _host_cu(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None = None) -> torch.Tensor:
+    """The boundaries as int64 on the host (one device-to-host copy per ``cu_seqlens`` tensor, none with ``cu_seqlens_cpu``)."""
     src = cu_seqlens_cpu if cu_seqlens_cpu is not None else cu_seqlens
-    src = src.detach().to('cpu', torch.int64)
+    return src.detach().to('cpu', torch.int64)
+
+
+def _host_lens(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None) -> torch.Tensor:
+    src = _host_cu(cu_seqlens, cu_seqlens_cpu)
     return src[1:] - src[:-1]
+
+
+def check_cu_seqlens(cu_seqlens: torch.Tensor, total_tokens: int, cu_seqlens_cpu: torch.Tensor | None = None) -> None:
+    """The kernels take token positions from ``cu_seqlens`` as they are: boundaries that decrease, start below zero or end
+    beyond the packed tensor would send them out of bounds.  Checked on the host copy the chunk tables are built from."""
+    src = _host_cu(cu_seqlens, cu_seqlens_cpu)
+    if src.dim() != 1 or src.numel() < 2:
+        raise ValueError(f'cu_seqlens must hold N + 1 >= 2 boundaries, got shape {tuple(src.shape)}')
+    if int(src[0]) < 0 or bool((src[1:] < src[:-1]).any()) or int(src[-1]) > total_tokens:
+        raise ValueError(f'cu_seqlens must be non-decreasing within [0, {total_tokens}] (the packed length), '
+                         f'got {src.tolist() if src.numel() <= 16 else [int(src[0]), "...", int(src[-1])]}')
 
 
 @tensor_cache

@@ -396,3 +396,38 @@ def test_operand_shapes_are_checked_before_anything_reaches_a_kernel():
         check_operand_shapes(q, q, v[:, :4])
     with pytest.raises(ValueError, match='divisible'):
         check_operand_shapes(q, q, v[:, :, :3])
+
+
+def test_cu_seqlens_are_checked_on_the_host_copy():
+    import torch
+    from fla_hip.ops.utils.index import check_cu_seqlens
+    check_cu_seqlens(torch.tensor([0, 3, 3, 10]), 10)
+    check_cu_seqlens(torch.tensor([2, 5], dtype=torch.int32), 10)                   # tokens outside all sequences are allowed
+    check_cu_seqlens(torch.tensor([0, 99]), 10, cu_seqlens_cpu=torch.tensor([0, 10]))      # (the host copy is what is read)
+    for bad in ([0, 11], [-1, 4], [0, 6, 5, 10], [0]):
+        with pytest.raises(ValueError, match='cu_seqlens must'):
+            check_cu_seqlens(torch.tensor(bad), 10)
+
+
+@pytest.mark.gpu
+def test_packed_calls_refuse_boundaries_beyond_the_input():
+    import torch
+    from fla_hip.modules import causal_conv1d
+    from fla_hip.ops.comba import chunk_comba
+    from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_hip.ops.kda import chunk_kda
+    q = torch.randn(1, 100, 2, 64, device='cuda', dtype=torch.bfloat16)
+    g = -torch.rand(1, 100, 2, device='cuda')
+    cu = torch.tensor([0, 50, 101], device='cuda')
+    with pytest.raises(ValueError, match='cu_seqlens must'):
+        chunk_gated_delta_rule(q, q, q, g, g.exp(), cu_seqlens=cu)
+    with pytest.raises(ValueError, match='cu_seqlens must'):
+        chunk_gated_delta_rule(q.clone().requires_grad_(), q, q, g, g.exp(), cu_seqlens=torch.tensor([0, 60, 40, 100], device='cuda'))
+    with pytest.raises(ValueError, match='cu_seqlens must'):
+        chunk_kda(q, q, q, g[..., None].expand(-1, -1, -1, 64).contiguous(), g.exp(), cu_seqlens=cu)
+    with pytest.raises(ValueError, match='cu_seqlens must'):
+        chunk_comba(q, q, q, q, g, g.exp(), cu_seqlens=cu)
+    x = torch.randn(1, 100, 64, device='cuda', dtype=torch.bfloat16, requires_grad=True)
+    y, _ = causal_conv1d(x, torch.randn(64, 4, device='cuda', dtype=torch.bfloat16), cu_seqlens=torch.tensor([0, 100], device='cuda'))
+    y.sum().backward()
+    assert x.grad is not None
