@@ -27,15 +27,25 @@ def _host_lens(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None) ->
     return src[1:] - src[:-1]
 
 
-def check_cu_seqlens(cu_seqlens: torch.Tensor, total_tokens: int, cu_seqlens_cpu: torch.Tensor | None = None) -> None:
-    """The kernels take token positions from ``cu_seqlens`` as they are: boundaries that decrease, start below zero or end
-    beyond the packed tensor would send them out of bounds.  Checked on the host copy the chunk tables are built from."""
+@tensor_cache
+def _cu_summary(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None = None) -> tuple:
     src = _host_cu(cu_seqlens, cu_seqlens_cpu)
     if src.dim() != 1 or src.numel() < 2:
-        raise ValueError(f'cu_seqlens must hold N + 1 >= 2 boundaries, got shape {tuple(src.shape)}')
-    if int(src[0]) < 0 or bool((src[1:] < src[:-1]).any()) or int(src[-1]) > total_tokens:
-        raise ValueError(f'cu_seqlens must be non-decreasing within [0, {total_tokens}] (the packed length), '
-                         f'got {src.tolist() if src.numel() <= 16 else [int(src[0]), "...", int(src[-1])]}')
+        return (tuple(src.shape),)
+    shown = src.tolist() if src.numel() <= 16 else [int(src[0]), '...', int(src[-1])]
+    return int(src[0]), int(src[-1]), not bool((src[1:] < src[:-1]).any()), shown
+
+
+def check_cu_seqlens(cu_seqlens: torch.Tensor, total_tokens: int, cu_seqlens_cpu: torch.Tensor | None = None) -> None:
+    """The kernels take token positions from ``cu_seqlens`` as they are: boundaries that decrease, start below zero or end
+    beyond the packed tensor would send them out of bounds.  Checked on the host copy the chunk tables are built from
+    (memoised per tensor, like the tables)."""
+    summary = _cu_summary(cu_seqlens, cu_seqlens_cpu)
+    if len(summary) == 1:
+        raise ValueError(f'cu_seqlens must hold N + 1 >= 2 boundaries, got shape {summary[0]}')
+    first, last, monotone, shown = summary
+    if first < 0 or not monotone or last > total_tokens:
+        raise ValueError(f'cu_seqlens must be non-decreasing within [0, {total_tokens}] (the packed length), got {shown}')
 
 
 @tensor_cache
