@@ -101,10 +101,14 @@ __device__ __forceinline__ float row_rnorm(const typename Mma<T>::V8 (&qb)[N], i
 // the chunk's transition S -> 2^G_last S - k~^T (Xb 2^G k) S can stretch any state:
 //   bound = sum_t [ log2 gamma_t + log2 max(1, |1 - beta_t |k_t|^2|) ]      (each token's factor gamma_t (I - beta_t k_t k_t^T))
 // A run of chunks whose bounds add up to at most WARM_LOG2 forgets what came before it to within 2^WARM_LOG2 of that
-// state's size: the state in front of the run would have to be 2^24 times the size of the state behind it for the
-// dropped part to reach the rounding of the fp32 state (2^-24 of its own size).  So a time segment may start from a
-// ZERO state that many chunks early instead of from the exact state that a first pass and a merge would have to compute.
-constexpr float WARM_LOG2 = -48.f;
+// state's size: the state in front of the run would have to be 2^8 times the size of the state behind it for the
+// dropped part to reach the rounding of the fp32 state (2^-24 of its own size), and 2^24 times its size to reach the
+// operator's error bar (5e-3, set by the 16-bit operands).  So a time segment may start from a ZERO state that many
+// chunks early instead of from the exact state that a first pass and a merge would have to compute.  (Measured against
+// -48: warm-ups a third shorter, config 3 0.317 instead of 0.32 ms; with wide keys, where a head that cannot start warm is
+// evaluated whole, more heads qualify: the forward of the layer's default shape with a random A_log 0.5 instead of 1.95 ms.
+// -24 would take config 3 to 0.304 ms and leave no margin over the fp32 rounding.)
+constexpr float WARM_LOG2 = -32.f;
 constexpr int WARM_CAP_MAX = 64;
 __host__ __device__ constexpr int p_slot(int tt, int sp) { return tt < 2 ? tt : 2 + 2 * (tt - 2) + sp; }
 __host__ __device__ constexpr bool frag_half(int tt, int sp) { return (tt == 0 && sp == 0) || (tt == 2 && sp == 1); }
