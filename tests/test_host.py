@@ -7,6 +7,7 @@ import re
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import gdn_oracle as O
 
@@ -250,6 +251,33 @@ def test_naive_forms_match_oracle():
     o3, h3 = naive_chunk_gated_delta_rule(q, k, v, g, beta, chunk_size=16, scale=0.3)
     ref_o3, _ = O.recurrent_gated_delta_rule(q, k, v, g, beta, 0.3, dtype=torch.float64)
     assert h3 is None and O.get_err_ratio(ref_o3, o3) < 1e-5
+
+
+def test_naive_comba_forms():
+    """The chunked plain-torch form is the oracle's recurrence (predict before the decay); the token loop of that name decays
+    first, as the reference's does, and equals the chunked form only where there is no decay."""
+    from fla_hip.ops.comba import naive_chunk_comba, naive_recurrent_comba
+    gen = torch.Generator().manual_seed(17)
+    q, k, p = (F.normalize(torch.randn(2, 150, 2, 16, generator=gen), dim=-1) for _ in range(3))
+    v = torch.randn(2, 150, 2, 8, generator=gen)
+    g = F.logsigmoid(torch.randn(2, 150, 2, generator=gen))
+    beta = torch.rand(2, 150, 2, generator=gen)
+    h0 = torch.randn(2, 2, 16, 8, generator=gen)
+    ref_o, ref_h = O.recurrent_comba(q, k, v, p, g, beta, None, h0, True, dtype=torch.float64)
+    for cs in (64, 16):
+        o, h = naive_chunk_comba(q, k, v, p, g, beta, chunk_size=cs, initial_state=h0, output_final_state=True)
+        assert o.shape == ref_o.shape and O.get_err_ratio(ref_o, o) < 1e-5 and O.get_err_ratio(ref_h, h) < 1e-5
+    o_r, h_r = naive_recurrent_comba(q, k, v, p, beta, g, initial_state=h0, output_final_state=True)
+    assert O.get_err_ratio(ref_o, o_r) > 1e-3                                         # (a different map)
+    zero = torch.zeros_like(g)
+    o_r0, h_r0 = naive_recurrent_comba(q, k, v, p, beta, zero, initial_state=h0, output_final_state=True)
+    ref0, refh0 = O.recurrent_comba(q, k, v, p, zero, beta, None, h0, True, dtype=torch.float64)
+    assert O.get_err_ratio(ref0, o_r0) < 1e-5 and O.get_err_ratio(refh0, h_r0) < 1e-5
+    # its decay-first step in scalars: S <- e^g S, then the delta rule with p
+    S = h0[0, 0].double() * g[0, 0, 0].exp().double()
+    d = beta[0, 0, 0].double() * (v[0, 0, 0].double() - S.T @ p[0, 0, 0].double())
+    S = S + torch.outer(k[0, 0, 0].double(), d)
+    assert torch.allclose(o_r[0, 0, 0].double(), (S.T @ q[0, 0, 0].double()) * 16 ** -0.5, atol=1e-5)
 
 
 def test_assert_close_metric():
