@@ -17,6 +17,7 @@ constexpr int CB_TOK = 8, CB_CX = 32, CB_TY = 8;       // a thread: 2 channels x
 constexpr int CB_VEC = 2;                              // Two channels keep a thread at 134 registers (three waves per SIMD); measured for bf16 at
                                                        // 32768 x 3072: 4 channels (232 registers, two waves) 240 us, 2 channels 207 us; 8 channels or 16
                                                        // positions per thread: one wave per SIMD, 330 - 400 us; four waves by a register cap: spills, slower.
+                                                       // (8 tiles per workgroup, GDN_CONV_BWD_TILES_PER_PART: 202 us against 207 us with 4.)
 constexpr int CB_MAX_W = 8;
 
 struct ConvBwdParams {

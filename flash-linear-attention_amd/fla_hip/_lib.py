@@ -128,7 +128,7 @@ SIGNATURES['gdn_norm_gated_bwd'] = (c_int, [
     c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_void_p])   # T D ld parts ...
 SIGNATURES['gdn_calib_rmw'] = (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p])
 CHUNK_STATIC_WORKSPACE_BYTES = 64 << 20
-CONV_BWD_TILES_PER_PART = 4
+CONV_BWD_TILES_PER_PART = 8
 
 _lib = None
 _lock = threading.Lock()

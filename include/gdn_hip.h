@@ -381,7 +381,7 @@ int gdn_norm_gated_fwd(
  *   (the chunk table of gdn_chunk_fwd); dense input: NULL and num_tiles = B * ceil(T / 64)
  *   Requires an even D, even strides of x and rows that start on a boundary of two elements.
  */
-#define GDN_CONV_BWD_TILES_PER_PART 4
+#define GDN_CONV_BWD_TILES_PER_PART 8
 int gdn_causal_conv1d_bwd(
     const void* x, const void* weight, const void* bias, const void* initial_state, const void* dy, const void* dht,
     void* dx, float* dw_part, float* db_part, float* dh0,
