@@ -6,15 +6,17 @@ Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, 
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
 configuration the >= 50 %-of-MFMA-roofline target is quoted on.  A step is one call of
 chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries, under
-"other_workloads", the decode step (B=256: us/step and state GB/s), the other prefill
-configurations, the layer's two memory-bound steps either side of the operator (causal
-convolution, gated norm), the reference's published shapes (forward, and forward + backward through
-autograd: the `*_fwd_bwd` rows), and:
+"other_workloads" and in short form (ms per call, fraction of the bounding roofline), the reference's published
+shapes (forward, and forward + backward through autograd: the `*_fwd_bwd` rows), the sibling operators, the layer's two
+memory-bound steps either side of the operator (causal convolution, gated norm), the default workload again with exact
+start states forced and with gates that hardly decay, and last the other BASELINE configurations (packed prefill, B=4
+prefill, the decode step at B=256: us/step and state GB/s); and:
   roofline      dominant stage (the launches of one C entry point), algorithmic FLOPs (or bytes)
                 per call / its mean duration measured with HIP events on the launch stream
   cpu_baseline  the CPU oracle (torch fp32, all host cores) on a bounded sample of the workload
 Before the W warm-up steps of a workload the GPU is kept busy with the same step for 80 ms (untimed), so that the timed
-steps run at the clocks of sustained load and not at those of the first milliseconds after an idle period.
+steps run at the clocks of sustained load and not at those of the first milliseconds after an idle period;
+"ms_per_step_cold" is the default workload timed without that (5 + 20 calls straight after an idle half second).
 --workload layer_steps runs only the convolution and the gated norm; --workload calib_copy runs a plain 1 GiB device copy: the kernel of known size against which the
 FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled; --workload calib_rmw an in-place read-modify-write of the decode states' 2 x 512 MiB
 with torch's elementwise kernel: the stream the decode step is compared with.
@@ -74,6 +76,13 @@ WORKLOADS = {
     'decode_bf16_states': dict(kind='decode', N=256, H=16, HV=32, state_dtype='bf16',
                                name='the decode step of configs[4] with the states kept in bf16 (an option of this library: '
                                     'fp32 step, one rounding per step; 2 x 256 MiB of state traffic)'),
+    # configs[2] again, so that the headline's dependence on the gates is a number: with the exact start states of the
+    # time segments forced (first pass, merge, second pass), and with gates that hardly decay (logsigmoid / 1024:
+    # no segment can start from a zero state, so the automatic choice takes the exact path by itself)
+    'prefill_exact': dict(kind='prefill', B=1, T=32768, H=16, HV=32, h0=True, varlen=False, scan_mode='segments-exact',
+                          name='configs[2] with exact start states of the time segments (FLA_HIP_SCAN_MODE=segments-exact)'),
+    'prefill_weak_decay': dict(kind='prefill', B=1, T=32768, H=16, HV=32, h0=True, varlen=False, gate_div=1024.0,
+                               name='configs[2] with g = logsigmoid(N(0,1)) / 1024, automatic choice'),
 }
 
 
@@ -108,8 +117,18 @@ def _ensure_built():
         __graft_entry__.build()
 
 
+def varlen_lengths(total, n_seq, lo, hi, seed=42):
+    """configs[3]: lengths drawn uniformly in [lo, hi] from a seed, rescaled (floor) to sum to `total`, the remainder handed
+    out one token at a time to the first sequences."""
+    gen = torch.Generator().manual_seed(seed)
+    L = torch.randint(lo, hi + 1, (n_seq,), generator=gen).double()
+    L = torch.floor(L * total / L.sum()).long()
+    for i in range(total - int(L.sum())):
+        L[i % n_seq] += 1
+    return [int(x) for x in L]
+
+
 def make_prefill_inputs(w, device):
-    from oracle import gdn_oracle as O
     gen = torch.Generator().manual_seed(42)
     B, T, H, HV = w['B'], w['T'], w['H'], w['HV']
     K, V = w.get('K', 128), w.get('V', 128)
@@ -118,12 +137,12 @@ def make_prefill_inputs(w, device):
         q, k = F.normalize(q, p=2, dim=-1), F.normalize(k, p=2, dim=-1)
     q, k = q.bfloat16(), k.bfloat16()
     v = torch.randn(B, T, HV, V, generator=gen).bfloat16()
-    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / 16
+    g = F.logsigmoid(torch.randn(B, T, HV, generator=gen)) / w.get('gate_div', 16.0)
     beta = torch.sigmoid(torch.randn(B, T, HV, generator=gen))
     cu = None
     N = B
     if w['varlen']:
-        lens = O.make_varlen_lengths(T, 32, 256, 4096, seed=42)
+        lens = varlen_lengths(T, 32, 256, 4096, seed=42)
         cu = [0]
         for x in lens:
             cu.append(cu[-1] + x)
@@ -157,7 +176,24 @@ def spin_up(fn):
     torch.cuda.synchronize()
 
 
-def bench_prefill(w, steps, warmup, device, with_cpu):
+def bench_prefill(w, steps, warmup, device, with_cpu, cold=False):
+    """One prefill workload.  `cold`: also time 20 calls (after 5) straight after the idle period of the input generation,
+    before the untimed load that brings the clocks to those of sustained work ('ms_per_step_cold')."""
+    mode = w.get('scan_mode')
+    saved = os.environ.get('FLA_HIP_SCAN_MODE')
+    if mode:
+        os.environ['FLA_HIP_SCAN_MODE'] = mode       # (read by the operator when it builds its launch)
+    try:
+        return _bench_prefill(w, steps, warmup, device, with_cpu, cold)
+    finally:
+        if mode:
+            if saved is None:
+                os.environ.pop('FLA_HIP_SCAN_MODE', None)
+            else:
+                os.environ['FLA_HIP_SCAN_MODE'] = saved
+
+
+def _bench_prefill(w, steps, warmup, device, with_cpu, cold):
     from fla_hip.ops.gated_delta_rule import chunk_gated_delta_rule
     from fla_hip.ops.gated_delta_rule.chunk import ChunkLaunch
     cpu, d = make_prefill_inputs(w, device)
@@ -172,6 +208,18 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
                                       output_final_state=final, use_qk_l2norm_in_kernel=l2norm,
                                       cu_seqlens=d['cu_t'], cu_seqlens_cpu=d['cu_cpu'])
 
+    ms_cold = None
+    if cold:
+        torch.cuda.synchronize()
+        time.sleep(0.5)
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        ms_cold = (time.perf_counter() - t0) / 20 * 1e3
     spin_up(step)
     for _ in range(warmup):
         step()
@@ -216,8 +264,7 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
     torch.cuda.synchronize()
     t_prep = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e-3
     t_scan = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e-3
-    scan_name = ('gdn_chunk_fwd_scan: gdn_chunk_wide_kernel / gdn_chunk_pair_kernel '
-                 '(+ gdn_segment_merge_kernel when time is cut into segments)')
+    scan_name = 'gdn_chunk_fwd_scan (all launches of the sequential stage)'
     dom = (scan_name, F_SCAN, t_scan) if t_scan >= t_prep else ('gdn_chunk_fwd_prepare: gdn_chunk_prepare_kernel', F_PREP, t_prep)
     achieved = units * dom[1] / dom[2] / 1e12
     roofline = dict(bound='mfma', achieved=round(achieved, 2), peak=PEAK_BF16_TFLOPS, unit='TFLOP/s',
@@ -226,6 +273,8 @@ def bench_prefill(w, steps, warmup, device, with_cpu):
                     kernels_us=dict(gdn_chunk_fwd_prepare=round(t_prep * 1e6, 1), gdn_chunk_fwd_scan=round(t_scan * 1e6, 1)),
                     whole_op=whole)
     out = dict(value=tokens * steps / elapsed, ms_per_step=ms_per_step, roofline=roofline, call_ms_quantiles=quant)
+    if ms_cold is not None:
+        out['ms_per_step_cold'] = round(ms_cold, 4)
 
     if with_cpu:
         out['cpu_baseline'] = cpu_baseline_prefill(w, cpu)
@@ -323,8 +372,8 @@ def cpu_baseline_prefill(w, cpu):
     t = statistics.median(ts)
     toks = T_s * cpu['q'].shape[0]
     return dict(value=round(toks / t, 1), unit='tokens/s', cores=torch.get_num_threads(), kind='port',
-                sample=f'oracle chunk_gated_delta_rule (torch fp32 CPU) on the first {T_s} tokens per sequence of the same '
-                       f'inputs, median of {reps} runs of {t:.1f} s, dense (not packed) layout', seconds=round(sum(ts), 2))
+                sample=f'oracle chunk_gated_delta_rule (torch fp32 CPU), first {T_s} tokens of the same inputs, '
+                       f'median of {reps} runs of {t:.1f} s', seconds=round(sum(ts), 2))
 
 
 def bench_decode(w, steps, warmup, device, with_cpu):
@@ -577,53 +626,61 @@ def main():
                               call_ms_quantiles=r['call_ms_quantiles'])))
         return
     w = WORKLOADS[args.workload]
-    fn = bench_prefill if w['kind'] == 'prefill' else bench_decode
-    res = fn(w, args.steps, args.warmup, device, not args.no_cpu_baseline)
     if w['kind'] == 'prefill':
+        res = bench_prefill(w, args.steps, args.warmup, device, not args.no_cpu_baseline, cold=True)
         line = dict(metric='gdn_chunk_prefill_tokens_per_s', value=round(res['value'], 1), unit='tokens/s', higher_is_better=True)
     else:
+        res = bench_decode(w, args.steps, args.warmup, device, not args.no_cpu_baseline)
         line = dict(metric='gdn_decode_us_per_step', value=round(res['value'], 2), unit='us/step', higher_is_better=False)
     line.update(n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(res['ms_per_step'], 4), scaling='weak',
                 vs_baseline=None, dtype='bf16', data='synthetic', config=dict(workload=w['name'], chunk_size=64),
                 roofline=res['roofline'])
-    if 'cpu_baseline' in res:
-        line['cpu_baseline'] = res['cpu_baseline']
-    if 'call_ms_quantiles' in res:
-        line['call_ms_quantiles'] = res['call_ms_quantiles']
+    for key in ('ms_per_step_cold', 'cpu_baseline', 'call_ms_quantiles'):
+        if key in res:
+            line[key] = res[key]
     if not args.no_extra:
+        # The other rows are kept short (the whole line stays well under 8 KB) and the BASELINE configurations come last.
+        # Keys: ms = wall time per call, frac = fraction of the roofline that bounds the row (prefill rows: the whole
+        # operator's algorithmic FLOPs against the bf16 matrix-core peak; streaming rows: algorithmic bytes against 8 TB/s),
+        # frac_stage / us = the same for the dominant stage alone and the durations of the two stages (HIP events).
         extra = {}
+        half, quarter = (max(10, args.steps // 2), max(3, args.warmup // 2)), (max(10, args.steps // 4), max(3, args.warmup // 4))
+        for name, ww in PUBLISHED.items():
+            r = bench_prefill(dict(ww, key=name, stages=False), *half, device, False)
+            extra[name] = dict(ms=round(r['ms_per_step'], 4), frac=r['roofline']['frac'])
+            torch.cuda.empty_cache()
+        for name, ww in PUBLISHED.items():       # training step (forward + backward) on the same shapes
+            extra[name + '_fwd_bwd'] = dict(ms=bench_train(dict(ww, key=name), *quarter, device)['ms_per_step'])
+            torch.cuda.empty_cache()
+        extra['chunk_kda_b1_t8192_h96_d128'] = dict(ms=bench_kda(*quarter, device)['ms_per_step'])
+        extra['chunk_comba_b1_t8192_h96_d128'] = dict(ms=bench_comba(*quarter, device)['ms_per_step'])
+        extra['layer_train_t32768'] = dict(ms=bench_layer_train(max(5, args.steps // 10), 3, device)['ms_per_step'])
+        torch.cuda.empty_cache()
+        for key, r in bench_layer_steps(args.steps, args.warmup, device, False).items():
+            extra[key] = dict(ms=r['ms_per_step'], GBps=r['roofline']['achieved'], frac=r['roofline']['frac'])
         for name, ww in WORKLOADS.items():
             if name == args.workload:
                 continue
-            f2 = bench_prefill if ww['kind'] == 'prefill' else bench_decode
-            r = f2(ww, args.steps, args.warmup, device, name == 'decode' and not args.no_cpu_baseline)
-            e = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), roofline=r['roofline'])
             if ww['kind'] == 'prefill':
-                e['tokens_per_s'] = round(r['value'], 1)
-                e['call_ms_quantiles'] = r['call_ms_quantiles']
+                r = bench_prefill(ww, args.steps, args.warmup, device, False)
+                rf = r['roofline']
+                e = dict(ms=round(r['ms_per_step'], 4), tokens_per_s=round(r['value'], 1), frac=rf['whole_op']['frac'],
+                         frac_stage=rf['frac'], us=rf['kernels_us'], traffic=rf['traffic'])
             else:
-                e['us_per_step'] = round(r['value'], 2)
-                e['state_GBps'] = r['roofline']['achieved']
-            if 'cpu_baseline' in r:
-                e['cpu_baseline'] = r['cpu_baseline']
+                r = bench_decode(ww, args.steps, args.warmup, device, name == 'decode' and not args.no_cpu_baseline)
+                rf = r['roofline']
+                e = dict(us_per_step=round(r['value'], 2), state_GBps=rf['achieved'], frac=rf['frac'], kernel_us=rf['kernel_us'],
+                         bytes_per_launch=rf['bytes_per_launch'], traffic=rf['traffic'])
+                if 'cpu_baseline' in r:
+                    e['cpu_baseline'] = {k2: r['cpu_baseline'][k2] for k2 in ('value', 'unit', 'cores', 'kind')}
             extra[name] = e
             torch.cuda.empty_cache()
-        extra.update(bench_layer_steps(args.steps, args.warmup, device, not args.no_cpu_baseline))
-        for name, ww in PUBLISHED.items():
-            r = bench_prefill(dict(ww, key=name, stages=False), max(10, args.steps // 2), max(3, args.warmup // 2), device, False)
-            extra[name] = dict(workload=ww['name'], ms_per_step=round(r['ms_per_step'], 4), tokens_per_s=round(r['value'], 1),
-                               call_ms_quantiles=r['call_ms_quantiles'], roofline=r['roofline'])
-            torch.cuda.empty_cache()
-        # training step (forward + backward) on the same shapes
-        for name, ww in PUBLISHED.items():
-            extra[name + '_fwd_bwd'] = bench_train(dict(ww, key=name), max(10, args.steps // 4), max(3, args.warmup // 4), device)
-            torch.cuda.empty_cache()
-        extra['chunk_kda_b1_t8192_h96_d128'] = bench_kda(max(10, args.steps // 4), max(3, args.warmup // 4), device)
-        extra['layer_train_t32768'] = bench_layer_train(max(5, args.steps // 10), 3, device)
-        torch.cuda.empty_cache()
-        extra['chunk_comba_b1_t8192_h96_d128'] = bench_comba(max(10, args.steps // 4), max(3, args.warmup // 4), device)
+        # BASELINE configs[1], [3], [4] last
+        for name in ('varlen', 'prefill_b4', 'decode'):
+            if name in extra:
+                extra[name] = extra.pop(name)
         line['other_workloads'] = extra
-    print(json.dumps(line))
+    print(json.dumps(line, separators=(',', ':')))
 
 
 if __name__ == '__main__':

@@ -1,6 +1,6 @@
-// C entry points of the chunked prefill (64-token chunks, K = V = 128): argument checks,
-// workspace layout and the choice of kernels.  The kernels live in gdn_chunk_prepare.hip
-// (chunk-parallel stage) and gdn_chunk_wide.hip (sequential stage).
+// C entry points of the chunked prefill (64-token chunks; head dims that are multiples of 8, K <= 256): argument
+// checks, workspace layout and the choice of kernels.  The kernels live in gdn_chunk_prepare.hip (chunk-parallel
+// stage) and gdn_chunk_wide.hip, gdn_chunk_pair.hip, gdn_chunk_wide256.hip (sequential stage).
 #include "gdn_chunk_common.h"
 
 namespace gdn {

@@ -109,7 +109,9 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
     int64_t slot = in;
     if (p.state_slots) {
         int64_t first = 0;
-        if (slot_per_token && p.num_accepted) first = load_index(p.num_accepted, in, slot32) - 1;
+        // (a count outside 1 .. row width would index past this sequence's row of the table: held to the row)
+        if (slot_per_token && p.num_accepted)
+            first = min(max(load_index(p.num_accepted, in, slot32) - 1, (int64_t)0), p.slots_stride - 1);
         slot = load_index(p.state_slots, slot_per_token ? in * p.slots_stride + first : in, slot32);
     }
     const int64_t head_off = (int64_t)ihv * K * V, state_stride = (int64_t)HV * K * V;
@@ -279,7 +281,8 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
             }
         }
         // a state per token: into the slot named for (n, t), or into entry `tok` of a per-token state tensor
-        if (p.ht && (slot_per_token || state_per_token)) {
+        // (a token past the row width of the slot table has no slot: its state is kept in registers and not stored)
+        if (p.ht && (state_per_token || (slot_per_token && t < p.slots_stride))) {
             const int64_t dst = state_per_token ? tok : load_index(p.state_slots, in * p.slots_stride + t, slot32);
             store_state(p.ht + dst * state_stride + head_off);
         }

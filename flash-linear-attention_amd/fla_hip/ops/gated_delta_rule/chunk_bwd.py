@@ -11,7 +11,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, check_operand_shapes, current_stream_ptr, dtype_code, ptr, require_gpu
-from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.utils.index import check_cu_seqlens, cu_bounds, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
 _DIM = 128          # value columns of the backward kernels; key features: 128 or 256 (other head dims are zero-padded)
@@ -119,12 +119,19 @@ def chunk_gated_delta_rule_bwd(
     else:
         num_chunks = B * ((T + _CHUNK - 1) // _CHUNK)
 
-    # rows past a sequence's end inside its last chunk are never written: start from zeros only where that matters
-    dq = torch.empty(B, T, HV, KD, dtype=work, device=dev)
-    dk = torch.empty(B, T, HV, KD, dtype=work, device=dev)
-    dv = torch.empty(B, T, HV, _DIM, dtype=work, device=dev)
-    dg = torch.empty(B, T, HV, dtype=torch.float32, device=dev)
-    db = torch.empty(B, T, HV, dtype=torch.float32, device=dev)
+    # The kernels write the tokens inside [cu_seqlens[0], cu_seqlens[-1]) only.  Tokens of a packed tensor outside every
+    # sequence get zero gradients (what autograd hands on, e.g. to a projection's weight gradient, must not be
+    # uninitialised memory); the boundaries are known from the host summary that check_cu_seqlens has just memoised.
+    alloc = torch.empty
+    if cu_seqlens is not None:
+        first, last = cu_bounds(cu_seqlens, cu_seqlens_cpu)
+        if first != 0 or last != T:
+            alloc = torch.zeros
+    dq = alloc(B, T, HV, KD, dtype=work, device=dev)
+    dk = alloc(B, T, HV, KD, dtype=work, device=dev)
+    dv = alloc(B, T, HV, _DIM, dtype=work, device=dev)
+    dg = alloc(B, T, HV, dtype=torch.float32, device=dev)
+    db = alloc(B, T, HV, dtype=torch.float32, device=dev)
     dh0 = torch.empty(N, HV, KD, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
     lib = _lib.load()
     ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, KD)

@@ -19,6 +19,7 @@ from fla_hip.ops.gated_delta_rule._common import (
     unify_gate_beta,
     unify_qkv,
 )
+from fla_hip.ops.utils.index import max_seq_len
 from fla_hip.utils import input_guard
 
 
@@ -126,8 +127,11 @@ def fused_recurrent_gated_delta_rule_fwd(
         elif ssm_state_indices.ndim == 2:
             if ssm_state_indices.shape[0] != N:
                 raise ValueError(f'ssm_state_indices must have {N} rows, got {tuple(ssm_state_indices.shape)}')
-            if cu_seqlens is None and ssm_state_indices.shape[1] < T:
-                raise ValueError(f'ssm_state_indices needs a slot for each of the {T} tokens of a sequence, '
+            # a slot per token: the kernel reads row n at column t for every token t of sequence n (packed input: the
+            # longest sequence decides, from the host copy of the boundaries, memoised per cu_seqlens tensor)
+            longest = T if cu_seqlens is None else max_seq_len(cu_seqlens)
+            if ssm_state_indices.shape[1] < longest:
+                raise ValueError(f'ssm_state_indices needs a slot for each of the {longest} tokens of a sequence, '
                                  f'got {tuple(ssm_state_indices.shape)}')
             if inplace_final_state:
                 flags |= _lib.FLAG_SLOT_PER_TOKEN

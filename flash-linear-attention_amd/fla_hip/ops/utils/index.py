@@ -3,7 +3,9 @@
 
 The tables are tiny integer arrays; they are built on the HOST from ``cu_seqlens_cpu`` when
 the caller supplies it (no device sync), otherwise from one device-to-host copy of
-``cu_seqlens``, and then uploaded.  Results are memoised by tensor identity."""
+``cu_seqlens``, and then uploaded.  Results are memoised by tensor identity and version (an in-place
+update of ``cu_seqlens`` recomputes); ``cu_seqlens_cpu``, when given, must mirror ``cu_seqlens``: it is
+the copy that is checked and the tables are built from, while the kernels index with the device tensor."""
 from __future__ import annotations
 
 import torch
@@ -46,6 +48,18 @@ def check_cu_seqlens(cu_seqlens: torch.Tensor, total_tokens: int, cu_seqlens_cpu
     first, last, monotone, shown = summary
     if first < 0 or not monotone or last > total_tokens:
         raise ValueError(f'cu_seqlens must be non-decreasing within [0, {total_tokens}] (the packed length), got {shown}')
+
+
+def cu_bounds(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None = None) -> tuple[int, int]:
+    """First and last boundary (tokens outside [first, last) belong to no sequence); from the memoised host summary."""
+    summary = _cu_summary(cu_seqlens, cu_seqlens_cpu)
+    return summary[0], summary[1]
+
+
+def max_seq_len(cu_seqlens: torch.Tensor, cu_seqlens_cpu: torch.Tensor | None = None) -> int:
+    """Length of the longest packed sequence (host copy, memoised)."""
+    lens = _host_lens(cu_seqlens, cu_seqlens_cpu)
+    return int(lens.max()) if lens.numel() else 0
 
 
 @tensor_cache

@@ -41,7 +41,9 @@ def make_backends(BaseBackend):
                 return False, 'not a gfx950 device'
             if cp_context is not None:
                 return False, 'context parallelism is not supported'
-            if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            # (fp32 operands are left to upstream, which multiplies them as tf32: the chunk kernels here take 16-bit
+            # operands and would round fp32 inputs to bf16 first - a silent loss of precision for such a caller)
+            if q.dtype not in (torch.bfloat16, torch.float16):
                 return False, f'dtype {q.dtype}'
             if k.shape[-1] > 256:
                 return False, 'key head dim above 256'           # (upstream asserts the same: chunk_delta_h.py:712)
@@ -183,7 +185,7 @@ def make_kda_backend(BaseBackend):
                 return False, 'context parallelism and intermediate states are not supported'
             if _needs_grad(q, k, v, g, beta, kwargs.get('initial_state'), kwargs.get('A_log'), kwargs.get('dt_bias')):
                 return False, 'forward only: a tensor requires grad'
-            if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            if q.dtype not in (torch.bfloat16, torch.float16):      # (fp32 operands: upstream's tf32 path, as above)
                 return False, f'dtype {q.dtype}'
             if k.shape[-1] > 128:
                 return False, 'key head dim above 128'

@@ -24,20 +24,26 @@ FLA_TENSOR_CACHE_SIZE = int(os.environ.get('FLA_TENSOR_CACHE_SIZE', '4'))
 def tensor_cache(fn: Callable[..., Any]) -> Callable[..., Any]:
     """Memoise the last few results by ARGUMENT IDENTITY (``is``), as the reference does for
     its index helpers: calling again with the very same tensor objects returns the cached
-    result; equal-valued but distinct tensors recompute."""
+    result; equal-valued but distinct tensors recompute.  A tensor argument that has been written
+    in place since (its version counter moved: a serving loop that refills a persistent
+    ``cu_seqlens`` buffer) recomputes as well - what is cached here includes bounds checks."""
     entries: deque = deque(maxlen=FLA_TENSOR_CACHE_SIZE)
+
+    def versions(args, kwargs):
+        return tuple(x._version for x in (*args, *kwargs.values()) if isinstance(x, torch.Tensor))
 
     @functools.wraps(fn)
     def wrapper(*args, **kwargs):
         if FLA_DISABLE_TENSOR_CACHE or os.environ.get('FLA_DISABLE_TENSOR_CACHE') == '1':
             return fn(*args, **kwargs)
-        for a0, k0, r0 in entries:
+        for a0, k0, v0, r0 in entries:
             if len(a0) == len(args) and k0.keys() == kwargs.keys() \
                     and all(x is y for x, y in zip(args, a0)) \
-                    and all(kwargs[key] is k0[key] for key in kwargs):
+                    and all(kwargs[key] is k0[key] for key in kwargs) \
+                    and v0 == versions(args, kwargs):
                 return r0
         out = fn(*args, **kwargs)
-        entries.append((args, kwargs, out))
+        entries.append((args, kwargs, versions(args, kwargs), out))
         return out
 
     return wrapper

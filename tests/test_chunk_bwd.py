@@ -194,6 +194,29 @@ def test_chunk_backward_packed(H, HV, D, mask_p, cu):
 
 
 @pytest.mark.gpu
+def test_chunk_backward_packed_tokens_outside_every_sequence_get_zero_gradients():
+    # boundaries that start after token 0 and end before the last one: the padding tokens belong to no sequence, the
+    # kernels never write them, and what autograd hands on for them must be zero (not whatever the allocator held)
+    cu, T, H, HV, D = [70, 200, 390], 460, 2, 4, 64
+    gen = torch.Generator().manual_seed(5)
+    q, k, v, g, beta, h0 = O.make_inputs(1, T, H, HV, D, D, seed=5, h0_std=0.5, N=2, dtype=torch.bfloat16)
+    do = torch.randn(1, T, HV, D, generator=gen).bfloat16()
+    dht = torch.randn(2, HV, D, D, generator=gen)
+    # poison the caching allocator's free blocks so that an uninitialised buffer would show
+    junk = [torch.full((1, T, HV, D), float('nan'), device='cuda', dtype=dt) for dt in (torch.bfloat16, torch.float32) for _ in range(4)]
+    del junk
+    _, _, got = _grads_gpu(q, k, v, g, beta, h0, do, dht, cu=cu)
+    for n in ('dq', 'dk', 'dv', 'dg', 'dbeta'):
+        x = got[n].float().cpu()
+        assert not torch.isnan(x).any(), n
+        assert not x[:, :cu[0]].any() and not x[:, cu[-1]:].any(), f'{n}: tokens outside the sequences'
+    sl = slice(cu[0], cu[-1])
+    ref = O.gated_delta_rule_grads(q[:, sl], k[:, sl], v[:, sl], g[:, sl], beta[:, sl], do[:, sl], dht, initial_state=h0,
+                                   cu_seqlens=[c - cu[0] for c in cu], dtype=torch.float32)
+    _compare(ref, {n: (x[:, sl] if n != 'dh0' else x) for n, x in got.items()})
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize('B,T,H,HV,K,V,l2,cu', [
     (2, 200, 2, 4, 256, 128, True, None),
     (1, 130, 2, 2, 256, 256, False, None),

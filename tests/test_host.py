@@ -98,6 +98,24 @@ def test_tensor_cache_is_by_identity():
     assert len(calls) == 2
     f(a, n=2)                            # different call shape: recomputed
     assert len(calls) == 3
+    # a tensor written in place since (a persistent buffer refilled by a serving loop) is not the tensor that was cached
+    b = torch.ones(3)
+    f(b, 2)
+    f(b, 2)
+    assert len(calls) == 4
+    b.add_(1)
+    assert f(b, 2).tolist() == [4.0, 4.0, 4.0] and len(calls) == 5
+
+
+def test_cu_seqlens_check_follows_in_place_updates():
+    from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices
+    cu = torch.tensor([0, 100, 200])
+    check_cu_seqlens(cu, 200)
+    assert prepare_chunk_indices(cu, 64).shape[0] == 4
+    cu.copy_(torch.tensor([0, 100, 300]))            # same tensor object, new boundaries: checked and tabulated again
+    with pytest.raises(ValueError):
+        check_cu_seqlens(cu, 200)
+    assert prepare_chunk_indices(cu, 64).shape[0] == 6
 
 
 def test_input_guard_makes_contiguous():
@@ -374,6 +392,8 @@ def test_upstream_backends_take_gpu_inference_calls_and_leave_the_rest():
     o_t = chunk_gated_delta_rule(dq.requires_grad_(), dk, dv, dg, db)[0]                          # training goes through the backward kernels
     assert isinstance(o_t, torch.Tensor) and o_t.requires_grad
     assert chunk_gated_delta_rule(q, k, v, g, beta)[0] == 'default'                               # CPU stays upstream
+    # fp32 operands stay upstream too (it multiplies them as tf32; the chunk kernels here would round them to bf16)
+    assert chunk_gated_delta_rule(dq.detach().float(), dk.float(), dv.float(), dg, db)[0] == 'default'
     with torch.no_grad():
         assert isinstance(chunk_gated_delta_rule(dq, dk, dv, dg, db)[0], torch.Tensor)
     x = torch.randn(2, 40, 64, device='cuda', dtype=torch.bfloat16)
