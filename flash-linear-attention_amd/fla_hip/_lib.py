@@ -99,6 +99,12 @@ SIGNATURES['gdn_chunk_bwd'] = (c_int, [
     c_float, c_int, c_int, c_uint32, c_void_p])
 SIGNATURES['gdn_l2norm_fwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p])
 SIGNATURES['gdn_l2norm_bwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p])
+SIGNATURES['gdn_fused_recurrent_delta_bwd_value_block'] = (c_int64, [c_int64])
+SIGNATURES['gdn_fused_recurrent_delta_bwd'] = (c_int, [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # q k v beta dout h0 dht
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # dq_part dk_part dv db dh0 u_workspace cu_seqlens
+    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,                      # B T H K V N
+    c_float, c_int, c_int, c_uint32, c_void_p])
 SIGNATURES['gdn_chunk_kda_workspace_bytes'] = (c_size_t, [c_int64, c_int64])
 SIGNATURES['gdn_chunk_kda_fwd'] = (c_int, [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k v g beta

@@ -105,6 +105,26 @@ int gdn_fused_recurrent_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Replaces fla/ops/delta_rule/fused_recurrent.py:313-385 (fused_recurrent_delta_rule_bwd and its kernel :111-266): the
+ * backward of the token recurrence of the delta rule without gates,
+ *   u_t = v_t - S^T k_t;  S <- S + k_t (beta_t u_t)^T;  o_t = scale S^T q_t.
+ *   q, k [B,T,H,K], v, dout [B,T,H,V] in qkv_dtype (bf16, f16 or f32); beta [B,T,H] (NULL = ones) or, with
+ *   GDN_FLAG_BETA_VECTOR, [B,T,H,V], in gb_dtype; h0, dht [N,H,K,V] fp32 or NULL; cu_seqlens as in the forward.
+ *   Outputs, all fp32: dq_part, dk_part [NVB,B,T,H,K] (partial over the NVB = V / gdn_fused_recurrent_delta_bwd_value_block(K)
+ *   blocks of value columns: the caller adds them, as the reference does, :375-378), dv [B,T,H,V], db [NVB,B,T,H] (with
+ *   GDN_FLAG_BETA_VECTOR [B,T,H,V]), dh0 [N,H,K,V] or NULL.  u_workspace [B,T,H,V] fp32 receives the residuals u_t (the
+ *   reference keeps them from its forward kernel, :292-295; here the backward forms them again).
+ *   K a multiple of 16 up to 256, V a multiple of the value block (32 for K <= 128, else 16); every tensor 16-byte aligned.
+ *   Tokens outside every sequence (packed input) are not written.
+ */
+int64_t gdn_fused_recurrent_delta_bwd_value_block(int64_t K);
+int gdn_fused_recurrent_delta_bwd(
+    const void* q, const void* k, const void* v, const void* beta, const void* dout, const float* h0, const float* dht,
+    float* dq_part, float* dk_part, float* dv, float* db, float* dh0, float* u_workspace, const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, int qkv_dtype, int gb_dtype, uint32_t flags,
+    void* stream);
+
+/*
  * Replaces fla/ops/kda/fused_recurrent.py:236-338 (fused_recurrent_kda_fwd and its kernel :37-233): the token recurrence of
  * the KDA operator, i.e. the gated delta rule with a decay per key feature,
  *   S <- diag(e^{g_t}) S;  d = beta_t (v_t - S^T k_t);  S <- S + k_t d^T;  o_t = scale S^T q_t.

@@ -126,3 +126,88 @@ def test_chunk_delta_rule_backward(B, T, H, D, scale, l2, dtype):
     for name, x in zip(('dq', 'dk', 'dv', 'dbeta', 'dh0'), leaves):
         r = O.get_err_ratio(ref[name], x.grad.float().cpu())
         assert r <= 0.008, f'{name}: rel-rmse {r:.3e}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,K,V,scale,l2,dtype,what', [
+    (1, 63, 1, 64, 64, 1, False, torch.float16, ''),
+    (2, 100, 4, 60, 60, 0.1, False, torch.float16, ''),
+    (2, 300, 3, 128, 128, 0.1, False, torch.float16, ''),
+    (2, 256, 4, 128, 128, 1, True, torch.float16, ''),
+    (2, 200, 2, 64, 128, 0.1, False, torch.float32, ''),
+    (1, 150, 2, 256, 64, 0.1, True, torch.bfloat16, ''),
+    (2, 130, 2, 100, 72, 0.1, False, torch.float32, 'beta_vector'),
+    (2, 130, 2, 192, 40, 0.1, False, torch.float16, 'beta_vector'),
+    (2, 90, 2, 64, 64, 0.1, False, torch.float32, 'no_beta'),
+    (2, 90, 2, 64, 64, 0.1, True, torch.float32, 'no_h0'),
+])
+def test_fused_recurrent_delta_rule_backward(B, T, H, K, V, scale, l2, dtype, what):
+    """Gradients through fused_recurrent_delta_rule (the kernel behind fla/ops/delta_rule/fused_recurrent.py:313-441, which
+    the reference's own tests use as the truth for its chunked operator, tests/ops/test_delta.py:60-86) against
+    reverse-mode differentiation of the oracle's recurrence without a gate.  The kernel computes in fp32 from the inputs
+    as given, so the bar is far below the reference's 0.008."""
+    from fla_hip.ops.delta_rule import fused_recurrent_delta_rule
+    gen = torch.Generator().manual_seed(11)
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    if not l2:
+        q, k = F.normalize(q, dim=-1), F.normalize(k, dim=-1)
+    q, k = q.to(dtype), k.to(dtype)
+    v = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    beta = torch.rand(B, T, H, V if what == 'beta_vector' else 1, generator=gen).sigmoid()
+    beta = None if what == 'no_beta' else (beta if what == 'beta_vector' else beta[..., 0])
+    h0 = None if what == 'no_h0' else torch.randn(B, H, K, V, generator=gen) * 0.3
+    do = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    dht = torch.randn(B, H, K, V, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, None, beta, do, dht, scale=scale, initial_state=h0, use_qk_l2norm_in_kernel=l2,
+                                   dtype=torch.float64)
+    dev = 'cuda'
+    names = ('dq', 'dk', 'dv', 'dbeta', 'dh0')
+    leaves = [None if x is None else x.to(dev).requires_grad_(True) for x in (q, k, v, beta, h0)]
+    o, ht = fused_recurrent_delta_rule(leaves[0], leaves[1], leaves[2], leaves[3], scale=scale, initial_state=leaves[4],
+                                       output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    ((o.float() * do.to(dev).float()).sum() + (ht * dht.to(dev)).sum()).backward()
+    for name, x in zip(names, leaves):
+        if x is None:
+            continue
+        assert x.grad.shape == x.shape and x.grad.dtype == x.dtype
+        got = x.grad.double().cpu()
+        assert not torch.isnan(got).any(), name
+        r = O.get_err_ratio(ref[name], got)
+        # (16-bit gradients carry their own rounding: 2^-9 relative for bf16)
+        bar = 2e-5 if dtype == torch.float32 else 3e-3 if dtype == torch.bfloat16 and name in ('dq', 'dk', 'dv') else 1e-3
+        assert r <= bar, f'{name}: rel-rmse {r:.3e} > {bar}'
+
+
+@pytest.mark.gpu
+def test_fused_recurrent_delta_rule_backward_packed():
+    # packed sequences with tokens in front of the first and behind the last one (zero gradients there), an empty and a
+    # one-token sequence; every sequence's gradients are those of the sequence alone
+    from fla_hip.ops.delta_rule import fused_recurrent_delta_rule
+    cu, T, H, D = [30, 30, 31, 200, 333], 350, 2, 64
+    N = len(cu) - 1
+    gen = torch.Generator().manual_seed(12)
+    q = F.normalize(torch.randn(1, T, H, D, generator=gen), dim=-1)
+    k = F.normalize(torch.randn(1, T, H, D, generator=gen), dim=-1)
+    v = torch.randn(1, T, H, D, generator=gen)
+    beta = torch.rand(1, T, H, generator=gen).sigmoid()
+    h0 = torch.randn(N, H, D, D, generator=gen) * 0.3
+    do, dht = torch.randn(1, T, H, D, generator=gen), torch.randn(N, H, D, D, generator=gen)
+    sl = slice(cu[0], cu[-1])
+    ref = O.gated_delta_rule_grads(q[:, sl], k[:, sl], v[:, sl], None, beta[:, sl], do[:, sl], dht, initial_state=h0,
+                                   cu_seqlens=[c - cu[0] for c in cu], dtype=torch.float64)
+    dev = 'cuda'
+    for idx in (torch.int32, torch.int64):
+        junk = [torch.full((1, T, H, D), float('nan'), device=dev) for _ in range(6)]       # what an uninitialised buffer would show
+        del junk
+        leaves = [x.to(dev).requires_grad_(True) for x in (q, k, v, beta, h0)]
+        o, ht = fused_recurrent_delta_rule(*leaves[:4], initial_state=leaves[4], output_final_state=True,
+                                           cu_seqlens=torch.tensor(cu, dtype=idx, device=dev))
+        ((o[:, sl] * do[:, sl].to(dev)).sum() + (ht * dht.to(dev)).sum()).backward()
+        for name, x in zip(('dq', 'dk', 'dv', 'dbeta'), leaves):
+            got = x.grad.double().cpu()
+            assert not torch.isnan(got).any(), name
+            assert not got[:, :cu[0]].any() and not got[:, cu[-1]:].any(), f'{name}: tokens outside the sequences'
+            r = O.get_err_ratio(ref[name], got[:, sl])
+            assert r <= 2e-5, f'{name}: rel-rmse {r:.3e}'
+        assert O.get_err_ratio(ref['dh0'], leaves[4].grad.double().cpu()) <= 2e-5
+        assert torch.equal(leaves[4].grad[0].cpu(), dht[0])          # the empty sequence hands its state gradient through
