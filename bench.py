@@ -108,6 +108,11 @@ PUBLISHED = {
                                                  name="one prompt of 32768 tokens in the reference layer's default head shape: H=6 K=256 V=512 bf16, "
                                                       'use_qk_l2norm_in_kernel, final state returned'),
 }
+# ... and the same prompt with exact start states of the time segments forced: what a head pays whose gates decay too
+# slowly for a warm start (first pass over 256-row states and transitions, merge, second pass)
+PUBLISHED['layer_default_b1_t32768_h6_k256_v512_exact'] = dict(
+    PUBLISHED['layer_default_b1_t32768_h6_k256_v512'], scan_mode='segments-exact',
+    name=PUBLISHED['layer_default_b1_t32768_h6_k256_v512']['name'] + ', exact start states of the time segments')
 
 
 def _ensure_built():

@@ -79,10 +79,13 @@ static bool chunk_dims_ok(int64_t K, int64_t V) {
 }
 
 // bytes of workspace for the plan that launch_chunk will choose
-static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int64_t HV, int64_t K, bool packed, uint32_t flags,
-                                   char* base, gdn::ChunkWs* ws) {
+static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V, bool packed,
+                                   uint32_t flags, char* base, gdn::ChunkWs* ws) {
     using namespace gdn;
-    if (K > 128) flags = (flags & ~GDN_FLAG_SCAN_SEGMENTS) | GDN_FLAG_SCAN_WIDE;       // wide keys: no time segments
+    if (K > 128) {                      // wide keys: segment matrices of their own size, none for whole sequences
+        const int nseg = plan_segments256(N, H, HV, V, (T + CH - 1) / CH, !packed, flags);
+        return ws_layout(num_chunks, HV, nseg > 1 ? (int64_t)nseg * N * HV : 0, base, ws, seg256_floats(V));
+    }
     const int nseg = plan_segments(N, HV, (T + CH - 1) / CH, num_chunks, !packed, flags);
     return ws_layout(num_chunks, HV, (int64_t)nseg * N * HV, base, ws);
 }
@@ -90,7 +93,7 @@ static size_t chunk_workspace_need(int64_t N, int64_t T, int64_t num_chunks, int
 extern "C" size_t gdn_chunk_workspace_bytes(int64_t N, int64_t T, int64_t num_chunks, int64_t H, int64_t HV, int64_t K, int64_t V,
                                             int packed, uint32_t flags) {
     if (!chunk_dims_ok(K, V) || num_chunks < 0 || N < 1 || T < 0 || H < 1 || HV < 1) return 0;
-    return chunk_workspace_need(N, T, num_chunks, HV, K, packed != 0, flags, nullptr, nullptr);
+    return chunk_workspace_need(N, T, num_chunks, H, HV, K, V, packed != 0, flags, nullptr, nullptr);
 }
 
 static int chunk_entry(
@@ -133,7 +136,7 @@ static int chunk_entry(
         return GDN_OK;
     }
     ChunkParams p;
-    const size_t need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, (char*)workspace, &p.ws);
+    const size_t need = chunk_workspace_need(N, T, num_chunks, H, HV, K, V, cu_seqlens != nullptr, flags, (char*)workspace, &p.ws);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o;
@@ -207,10 +210,10 @@ extern "C" int gdn_chunk_fwd_static(
     GDN_CHECK_ARG(chunk_dims_ok(K, V) && N >= 1 && T >= 0 && HV >= 1 && num_chunks >= 0, GDN_ERR_INVALID,
                   "%s: bad dimensions", who);
     // The plan with time segments needs room for their matrices; when only that does not fit, whole sequences do.
-    size_t need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, nullptr, nullptr);
+    size_t need = chunk_workspace_need(N, T, num_chunks, H, HV, K, V, cu_seqlens != nullptr, flags, nullptr, nullptr);
     if (need > GDN_CHUNK_STATIC_WORKSPACE_BYTES && !(flags & GDN_FLAG_SCAN_SEGMENTS)) {
         flags |= GDN_FLAG_SCAN_WIDE;
-        need = chunk_workspace_need(N, T, num_chunks, HV, K, cu_seqlens != nullptr, flags, nullptr, nullptr);
+        need = chunk_workspace_need(N, T, num_chunks, H, HV, K, V, cu_seqlens != nullptr, flags, nullptr, nullptr);
     }
     GDN_CHECK_ARG(need <= GDN_CHUNK_STATIC_WORKSPACE_BYTES, GDN_ERR_WORKSPACE,
                   "%s: this input needs %zu bytes of workspace, the built-in one holds %zu (%lld records of one chunk and "

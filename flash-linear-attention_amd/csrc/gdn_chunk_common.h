@@ -140,6 +140,7 @@ struct ChunkWs {
     char* Rec;           // [NC][HV] records
 };
 
+
 constexpr int64_t SEG_SLOTS_MAX = 640;            // upper bound on (sequences * heads * segments) when segmenting
 
 inline size_t ws_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -166,12 +167,31 @@ inline int plan_segments(int64_t N, int64_t HV, int64_t NT, int64_t num_chunks, 
     return segments ? nseg : 0;
 }
 
+// Wide keys (128 < K <= 256): a workgroup owns 64 value columns of a (sequence, value head) for all key rows, and time
+// is cut into segments where whole sequences leave CUs without a workgroup: never more workgroups than CUs, segments of
+// 8 chunks or more, and at least 24 chunks saved per workgroup (a warm-up of typical length must pay).  1 = whole sequences.
+constexpr int W2_VB = 64;                                 // value columns per workgroup
+constexpr int W2_KD = 256;                                // key rows of the segment matrices
+inline int plan_segments256(int64_t N, int64_t H, int64_t HV, int64_t V, int64_t NT, bool dense, uint32_t flags) {
+    const int64_t runs = N * HV * ((V + W2_VB - 1) / W2_VB);
+    if (!dense || (flags & GDN_FLAG_SCAN_WIDE) || runs <= 0) return 1;
+    int nseg = (int)std::min<int64_t>(256 / runs, NT / ((flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
+    while (nseg >= 2 && (int64_t)nseg * N * HV > SEG_SLOTS_MAX) --nseg;
+    if (nseg >= 2 && ((flags & GDN_FLAG_SCAN_SEGMENTS) || NT - NT / nseg >= 24)) return nseg;
+    return 1;
+}
+// floats per (sequence, value head, segment) of the wide-key segment matrices: S_loc and S_in [256][VP], M [256][256]
+__host__ __device__ inline size_t seg256_floats(int64_t V) {
+    const size_t VP = (size_t)((V + W2_VB - 1) / W2_VB) * W2_VB;
+    return 2 * (size_t)W2_KD * VP + (size_t)W2_KD * W2_KD;
+}
+
 // Workspace: the segment matrices (S_loc, M, S_in per (sequence, head, segment); none without segments),
-// the transition bounds, then the records.
-inline size_t ws_layout(int64_t NC, int64_t HV, int64_t seg_slots, char* base, ChunkWs* ws) {
+// the transition bounds, then the records.  `seg_floats`: floats per slot (3 matrices of 128 x 128 by default).
+inline size_t ws_layout(int64_t NC, int64_t HV, int64_t seg_slots, char* base, ChunkWs* ws, size_t seg_floats = 3 * 16384) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
-    void* Seg = take(3 * (size_t)seg_slots * 16384 * 4);
+    void* Seg = take((size_t)seg_slots * seg_floats * 4);
     void* Bound = take((size_t)NC * HV * 4);
     void* Rec = take((size_t)NC * HV * REC_BYTES);
     if (ws) { ws->Seg = (float*)Seg; ws->Bound = (float*)Bound; ws->Rec = (char*)Rec; }

@@ -14,6 +14,12 @@
 // have two, q and P have ONE: q of the next chunk is requested after the barrier that ends this chunk's last read of
 // it and awaited in the middle of the next step - a step multiplies by k first (the products that head the chain to the
 // next state) and turns to q, P and the output when an LDS counter says that q has landed.
+//
+// Long dense sequences on few heads are cut into time segments.  A segment starts warm where the decay allows it (see
+// WARM_LOG2); a head with a segment that cannot start warm takes exact start states, S_out = M S_in + S_loc per segment as in
+// gdn_chunk_wide.hip: pass 1 (FULL = false: no q, P, output) runs every segment but the last from zero (S_loc, 64 value
+// columns per workgroup) and from the identity with v = 0 (the 256 x 256 transition M, 64 of its columns per
+// workgroup), gdn_segment_merge256_kernel chains them in fp32, pass 2 starts every segment from its merged state.
 #include "gdn_chunk_common.h"
 
 namespace gdn {
@@ -30,9 +36,8 @@ constexpr int W2_PCOUNT = W2_OT + 64 * W2_OT_PITCH;
 constexpr size_t W2_SMEM = W2_PCOUNT + 16;                // 159 760 B
 constexpr int W2_CW = 4;                                  // compute waves
 constexpr int W2_THREADS = (W2_CW + 4) * 64;
-constexpr int W2_VB = 64;                                 // value columns per workgroup
 
-template <typename T>
+template <typename T, bool FULL>
 __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkParams p, int NVB, SegmentPlan sp) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -47,36 +52,56 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
 
     // ---- which (sequence, value head, block of value columns): the workgroups that read the same k and q rows take
     // consecutive slots of one XCD (block index mod 8) ----
-    const int G = HV / H, GV = G * NVB;
+    // Pass 1 (FULL = false) adds, per value head, four workgroups for the 64-column blocks of the transition M.
+    const int G = HV / H, NMB = FULL ? 0 : W2_KD / W2_VB, GV = G * (NVB + NMB);
+    const int VP = NVB * W2_VB;                                      // value columns of the segment buffers
     const int64_t slot = blockIdx.x >> 3;
     const int xcd = blockIdx.x & 7;
     const int64_t group = (slot / GV) * 8 + xcd;                     // (sequence, q/k head, time segment)
     const int nseg = sp.nseg;                                        // 1: whole sequences
-    if (group >= p.N * H * nseg) return;
-    const int seg = (int)(group % nseg);
-    int64_t n = (group / nseg) / H;
+    const int nrun = FULL ? nseg : nseg - 1;                         // (pass 1: every segment but the last)
+    if (group >= p.N * H * nrun) return;
+    const int seg = (int)(group % nrun);
+    int64_t n = (group / nrun) / H;
     if (p.flags & GDN_FLAG_SEQ_ORDER) n = load_index(p.chunk_offsets, p.N + 1 + n, cu32);
-    const int h = (int)((group / nseg) % H);
+    const int h = (int)((group / nrun) % H);
     const int member = (int)(slot % GV);
-    const int hv = h * G + member / NVB;
-    const int v0 = (member % NVB) * W2_VB;
+    const bool m_run = !FULL && member >= G * NVB;                   // a block of columns of the transition matrix
+    const int hv = h * G + (m_run ? (member - G * NVB) / NMB : member / NVB);
+    const int v0 = (m_run ? (member - G * NVB) % NMB : member % NVB) * W2_VB;
     const int64_t inh = n * HV + hv;
-    // Time segments (long dense sequences on few heads) start warm: a zero state a few chunks early, where the bound on
-    // the chunks' transitions makes the true state irrelevant (see WARM_LOG2), and no output until the segment proper.
-    // A head with a segment that cannot start this way is evaluated whole by the workgroups of its segment 0; those of
-    // its other segments have nothing to do.
+    // Time segments start warm: a zero state a few chunks early, where the bound on the chunks' transitions makes the true
+    // state irrelevant (see WARM_LOG2), and no output until the segment proper.  A head with a segment that cannot start
+    // this way takes the exact start states of the first pass and the merge.
     int warm = 0;
-    bool whole = nseg == 1;
+    bool exact = false;
     if (nseg > 1) {
-        const float* bnd = sp.bound + n * p.NT * HV + hv;
         int wch = 0;
-        whole = needs_exact_segments(sp, bnd, HV, lane, seg, &wch);
-        if (whole && seg > 0) return;
-        if (!whole && seg > 0) warm = __builtin_amdgcn_readfirstlane(wch);
+        exact = !sp.bound || needs_exact_segments(sp, sp.bound + n * p.NT * HV + hv, HV, lane, seg, &wch);
+        if (!exact && seg > 0) warm = __builtin_amdgcn_readfirstlane(wch);
     }
-    const bool from_start = whole || (int64_t)seg * sp.seg_chunks - warm == 0, to_end = whole || seg == nseg - 1;
-    const float* src = p.h0 && from_start ? p.h0 + inh * (int64_t)(K * V) : nullptr;
-    float* dst = p.ht && to_end ? p.ht + inh * (int64_t)(K * V) : nullptr;
+    if (!FULL && (!exact || (m_run && seg == 0))) return;            // (the first segment starts from the true state: no transition needed)
+    // where the state comes from and goes to: the caller's tensors ([K][V] or [V][K], K x V entries), or the segment
+    // buffers ([256][VP], for M [256][256])
+    const size_t seg_floats = seg256_floats(V);
+    float* seg_base = nseg > 1 ? p.ws.Seg + (size_t)(inh * nseg + seg) * seg_floats : nullptr;
+    const bool from_start = nseg == 1 || (int64_t)seg * sp.seg_chunks - warm == 0, to_end = nseg == 1 || seg == nseg - 1;
+    const float* src = nullptr;
+    float* dst = nullptr;
+    int init = 0;                                                    // 0: from src (NULL: zero), 1: identity
+    bool src_user = false, dst_user = false;
+    if (FULL) {
+        if (from_start) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
+        else if (exact) src = seg_base + (size_t)W2_KD * VP + (size_t)W2_KD * W2_KD;       // S_in of this segment
+        if (to_end && p.ht) { dst = p.ht + inh * (int64_t)(K * V); dst_user = true; }
+    } else if (m_run) {
+        init = 1;
+        dst = seg_base + (size_t)W2_KD * VP;                         // M of this segment
+    } else {
+        if (seg == 0) { src = p.h0 ? p.h0 + inh * (int64_t)(K * V) : nullptr; src_user = true; }
+        dst = seg_base;                                              // S_loc of this segment
+    }
+    const bool v_zero = m_run;
 
     int64_t bos, len, boh;
     if (p.cu_seqlens) {
@@ -89,8 +114,8 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         boh = n * p.NT;
     }
     const int64_t nt = (len + CH - 1) / CH;
-    const int64_t it0 = whole ? 0 : (int64_t)seg * sp.seg_chunks - warm;           // first chunk of this run (warm-up included)
-    const int64_t it1 = whole ? nt : min(nt, (int64_t)(seg + 1) * sp.seg_chunks);
+    const int64_t it0 = nseg == 1 ? 0 : (int64_t)seg * sp.seg_chunks - warm;       // first chunk of this run (warm-up included)
+    const int64_t it1 = nseg == 1 ? nt : min(nt, (int64_t)(seg + 1) * sp.seg_chunks);
     const int64_t nsteps = it1 - it0;                                               // step i works on chunk it0 + i
     const int64_t lastc = it1 - 1;
     char* otile = smem + W2_OT;
@@ -116,6 +141,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         // P = scale tril(q k^T 2^(G_t - G_t')) of a chunk from its q and k tiles (see gdn_chunk_wide.hip), contraction
         // over both halves of the key features
         auto produce_P = [&](const char* kbuf, const char* rec, int q_target) {
+            if constexpr (!FULL) return;
             while (*qcount < q_target) __builtin_amdgcn_s_sleep(1);          // q of this chunk has landed
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_setprio(3);
@@ -203,18 +229,18 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             // ---- q (one buffer) and the record (two).  q of chunk i+1 is requested right after the barrier B1 of step i,
             // which ends the last read of q of chunk i, and is awaited inside step i+1: the compute waves multiply by k
             // first and turn to q, and the copy waves to P, only when the counter says that it has landed ----
-            gather_qk((const T*)p.q, it0, lds0 + W2_Q);
+            if constexpr (FULL) gather_qk((const T*)p.q, it0, lds0 + W2_Q);
             copy_rec(it0, lds0 + W2_REC);
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 copy_rec(min(it0 + i + 1, lastc), lds0 + W2_REC + (int)((i + 1) & 1) * W2_REC_BYTES);      // 7 operations
                 wait_vm_at_most<7>();                                       // everything older than these: q of chunk i
-                if (lane == 0) __hip_atomic_fetch_add((int*)qcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (FULL && lane == 0) __hip_atomic_fetch_add((int*)qcount, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();                                       // the record of chunk i+1
-                if (i + 1 < nsteps) gather_qk((const T*)p.q, it0 + i + 1, lds0 + W2_Q);
+                if (FULL && i + 1 < nsteps) gather_qk((const T*)p.q, it0 + i + 1, lds0 + W2_Q);
                 lds_barrier();                                              // B2
             }
         } else if (w == W2_CW + 2) {
@@ -231,11 +257,11 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
                     gather_1k_to_lds_masked(base, (uint32_t)row * row_bytes + 16 * c, lds_tile + j * 1024, mask);
                 }
             };
-            gather_v(it0, lds0 + W2_V);
+            if (!v_zero) gather_v(it0, lds0 + W2_V);                        // (v is not read where it counts as zero)
             wait_vm_at_most<0>();
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
-                gather_v(min(it0 + i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
+                if (!v_zero) gather_v(min(it0 + i + 1, lastc), lds0 + W2_V + (int)((i + 1) & 1) * 16384);
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
                 lds_barrier();                                              // B1
                 wait_vm_at_most<0>();
@@ -258,13 +284,15 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             lds_barrier();                                                  // B0
             for (int64_t i = 0; i < nsteps; ++i) {
                 produce_P(smem + W2_KB + (int)(i & 1) * 32768, smem + W2_REC + (int)(i & 1) * W2_REC_BYTES, (int)i + 1);
-                if (i > warm) store_rows(it0 + i - 1);             // (the chunks of a warm-up leave no output)
+                if (FULL && i > warm) store_rows(it0 + i - 1);     // (the chunks of a warm-up leave no output)
                 lds_barrier();                                              // B1
+                if constexpr (FULL) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) orow[j] = *(const u32x4*)(otile + (8 * j + orow_r) * W2_OT_PITCH + opiece * 16);
+                    for (int j = 0; j < 8; ++j) orow[j] = *(const u32x4*)(otile + (8 * j + orow_r) * W2_OT_PITCH + opiece * 16);
+                }
                 lds_barrier();                                              // B2 (waits for the tile reads)
             }
-            if (nsteps > warm) store_rows(lastc);
+            if (FULL && nsteps > warm) store_rows(lastc);
         }
         wait_vm_at_most<0>();                               // no copy may land in LDS after this workgroup has gone
         return;
@@ -276,14 +304,21 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     // state tile m (0..15), row 4g + r: key feature 32 (m/2) + 8g + 4 (m%2) + r; column: value v0 + 16w + c16
     f32x4 S[16];
     const int vc = v0 + 16 * w + c16;
-    const int sk = vfirst ? 1 : V, sv = vfirst ? K : 1;
+    // the caller's state is [K][V] or [V][K]; the buffers of the segment passes are [256][VP] (M: [256][256])
+    const int buf_pitch = m_run ? W2_KD : VP;
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
         const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
-        if (src && kk < K && vc < V) {
-            const float* e = src + (int64_t)kk * sk + (int64_t)vc * sv;
-            s = f32x4{e[0], e[sk], e[2 * sk], e[3 * sk]};
+        if (init == 1) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] = (kk + r == vc) ? 1.f : 0.f;
+        } else if (src) {
+            const int sk = src_user ? (vfirst ? 1 : V) : buf_pitch, sv = src_user ? (vfirst ? K : 1) : 1;
+            if (kk < (src_user ? K : W2_KD) && vc < (src_user ? V : buf_pitch)) {
+                const float* e = src + (int64_t)kk * sk + (int64_t)vc * sv;
+                s = f32x4{e[0], e[sk], e[2 * sk], e[3 * sk]};
+            }
         }
         S[m] = s;
     }
@@ -314,11 +349,11 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         auto fidx = [&](int f) { return ((f & 7) >> 2) * 1024 + (f >> 3) * 256 + 16 * (f & 3) + a_off; };
         V8 ak[4], aq[4];
         auto Fk = [&](int f) { if (f < 32) ak[f & 3] = sK[fidx(f)]; };
-        auto Fq = [&](int f) { if (f < 32) aq[f & 3] = sQ[fidx(f)]; };
+        auto Fq = [&](int f) { if constexpr (FULL) { if (f < 32) aq[f & 3] = sQ[fidx(f)]; } };
         f32x4 ks[4], ao[4];
         V8 Sb[8];
         auto Mk = [&](int f) { ks[f >> 3] = Mma<T>::run(ak[f & 3], Sb[f & 7], (f & 7) ? ks[f >> 3] : f32x4{0.f, 0.f, 0.f, 0.f}); };
-        auto Mq = [&](int f) { ao[f >> 3] = Mma<T>::run(Sb[f & 7], aq[f & 3], (f & 7) ? ao[f >> 3] : f32x4{0.f, 0.f, 0.f, 0.f}); };
+        auto Mq = [&](int f) { if constexpr (FULL) ao[f >> 3] = Mma<T>::run(Sb[f & 7], aq[f & 3], (f & 7) ? ao[f >> 3] : f32x4{0.f, 0.f, 0.f, 0.f}); };
         auto KK = [&](int r) { Fk(2 * r + 2); Fk(2 * r + 3); Mk(2 * r); Mk(2 * r + 1); };       // region r of the k products
         auto QQ = [&](int r) { Fq(2 * r + 2); Fq(2 * r + 3); Mq(2 * r); Mq(2 * r + 1); };       // region r of the q products
         V4 vv[4];
@@ -329,8 +364,10 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ax[tt][sp2] = load_frag<T>(sX, tt, sp2, lane);
         };
         auto FP = [&](int tt) {
+            if constexpr (FULL) {
 #pragma unroll
-            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) ap[tt][sp2] = load_frag<T>(sP, tt, sp2, lane);
+            }
         };
         // k^T operands of the state update, u = 16 sp2 + m (t-tile pair sp2, key tile m), in a ring of 8, fetched 6 ahead
         V8 kt[8];
@@ -345,7 +382,10 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         auto TD = [&](int tt) {
             const f32x4 eg = *(const f32x4*)(sTab + TAB_EG + 16 * tt + 4 * g) * gamma;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) Db[tt >> 1][(tt & 1) * 4 + r] = from_f32<T>(to_f32(vv[tt][r]) - eg[r] * ks[tt][r]);
+            for (int r = 0; r < 4; ++r) {
+                const float x = (!FULL && v_zero) ? 0.f : to_f32(vv[tt][r]);      // (full runs always have their v)
+                Db[tt >> 1][(tt & 1) * 4 + r] = from_f32<T>(x - eg[r] * ks[tt][r]);
+            }
         };
         f32x4 vn[4], oacc[4];
         auto TXa = [&](int tt) {
@@ -362,16 +402,20 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
             }
         };
         auto TPa = [&](int tt) {
-            const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
-            oacc[tt] = ao[tt] * gam;
+            if constexpr (FULL) {
+                const float gam = sTab[TAB_SG + 16 * tt + c16] * gamma;
+                oacc[tt] = ao[tt] * gam;
 #pragma unroll
-            for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) oacc[tt] = Mma<T>::run(Vn[sp2], ap[tt][sp2], oacc[tt]);
+                for (int sp2 = 0; sp2 <= (tt >> 1); ++sp2) oacc[tt] = Mma<T>::run(Vn[sp2], ap[tt][sp2], oacc[tt]);
+            }
         };
         auto TPb = [&](int tt) {
-            V4 o4;
+            if constexpr (FULL) {
+                V4 o4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(oacc[tt][r]);
-            *(V4*)(otile + (16 * tt + c16) * W2_OT_PITCH + (16 * w + 4 * g) * 2) = o4;
+                for (int r = 0; r < 4; ++r) o4[r] = from_f32<T>(oacc[tt][r]);
+                *(V4*)(otile + (16 * tt + c16) * W2_OT_PITCH + (16 * w + 4 * g) * 2) = o4;
+            }
         };
         auto UU = [&](int j) {                   // two products of the state update, and the operands of two later ones
             FK(2 * j + 6); FK(2 * j + 7);
@@ -414,7 +458,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         KK(9); TXa(0); TXa(1); fence();
         KK(10); TXb(0); TXb(1); fence();
         KK(11); UU(0); fence();
-        while (*qcount < istep + 1) __builtin_amdgcn_s_sleep(1);      // q of this chunk (normally long there)
+        if constexpr (FULL) { while (*qcount < istep + 1) __builtin_amdgcn_s_sleep(1); }      // q of this chunk (normally long there)
         asm volatile("" ::: "memory");                                // (no read of the tile may move in front of the poll)
         Fq(0); Fq(1);
         KK(12); UU(1); TD(2); FX(2); fence();
@@ -424,7 +468,7 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
         TD(3); UU(5); QQ(3); fence();
         TXa(2); TXa(3); UU(6); QQ(4); fence();
         TXb(2); TXb(3); UU(7); QQ(5); fence();
-        while (*pcount < 4 * (istep + 1)) __builtin_amdgcn_s_sleep(1);      // P of this chunk
+        if constexpr (FULL) { while (*pcount < 4 * (istep + 1)) __builtin_amdgcn_s_sleep(1); }      // P of this chunk
         asm volatile("" ::: "memory");
         FP(0); FP(1);
         UU(8); QQ(6); fence();
@@ -452,11 +496,12 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
 
     if (dst) {
         const float gamma = fast_exp2(lg);
+        const int sk = dst_user ? (vfirst ? 1 : V) : buf_pitch, sv = dst_user ? (vfirst ? K : 1) : 1;
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
             const int kk = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
             const f32x4 s = S[m] * gamma;
-            if (kk < K && vc < V) {
+            if (kk < (dst_user ? K : W2_KD) && vc < (dst_user ? V : buf_pitch)) {
                 float* e = dst + (int64_t)kk * sk + (int64_t)vc * sv;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) e[r * sk] = s[r];
@@ -465,32 +510,133 @@ __global__ __launch_bounds__(W2_THREADS) void gdn_chunk_wide256_kernel(ChunkPara
     }
 }
 
-template <typename T>
-int launch_wide256(const ChunkParams& p, hipStream_t stream) {
-    auto kern = gdn_chunk_wide256_kernel<T>;
+// S_in[j+1] = M_j S_in[j] + S_loc,j for j = 1 .. nseg-2, with S_in[1] = S_loc,0 (the run of segment 0 started from the true
+// initial state), for the 256-row states of wide keys.  fp32 throughout (fp32 matrix cores): one workgroup per (sequence,
+// head, slab of 16 value columns) keeps the slab transposed in LDS and stages M_j by halves of 128 rows; wave w takes
+// the key tiles 2w, 2w+1 of a half.  Buffers per (sequence, head, segment): S_loc [256][VP], M [256][256], S_in [256][VP].
+constexpr int M2P = W2_KD + 4;                     // pitch of the staged rows (floats): conflict-free 16-byte reads
+constexpr size_t MERGE256_SMEM = (128 * M2P + 16 * M2P) * 4;
+
+__global__ __launch_bounds__(256) void gdn_segment_merge256_kernel(SegmentPlan sp, float* seg, int64_t NH, int HV, int64_t NT, int VP,
+                                                                   size_t seg_floats) {
+    extern __shared__ __align__(16) char smem[];
+    float* sM = (float*)smem;                      // [128 rows of a half][M2P]
+    float* sSt = sM + 128 * M2P;                   // [16 columns][M2P]: the current S_in slab, transposed
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
+    const int slabs = VP / 16;
+    const int64_t inh = blockIdx.x / slabs;
+    const int v0 = (int)(blockIdx.x % slabs) * 16;
+    if (inh >= NH) return;
+    if (sp.bound && !needs_exact_segments(sp, sp.bound + (inh / HV) * NT * HV + inh % HV, HV, lane)) return;      // all segments start warm
+    const int nseg = sp.nseg;
+    auto sloc = [&](int j) { return seg + (size_t)(inh * nseg + j) * seg_floats; };
+    auto mseg = [&](int j) { return sloc(j) + (size_t)W2_KD * VP; };
+    auto sin = [&](int j) { return mseg(j) + (size_t)W2_KD * W2_KD; };
+    // this wave's part of a slab: per half the key tiles 2w, 2w+1 in C/D layout (column c16, rows 4g .. 4g+3)
+    auto row_of = [&](int half, int i) { return 128 * half + 16 * (2 * w + i) + 4 * g; };
+    f32x4 x[2][2];
+    auto publish = [&](int j) {                    // x becomes S_in[j]: to the other waves (transposed) and to memory
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                *(f32x4*)(sSt + c16 * M2P + row_of(half, i)) = x[half][i];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sin(j)[(size_t)(row_of(half, i) + r) * VP + v0 + c16] = x[half][i][r];
+            }
+    };
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) x[half][i][r] = sloc(0)[(size_t)(row_of(half, i) + r) * VP + v0 + c16];
+    publish(1);
+    for (int j = 1; j + 1 < nseg; ++j) {
+        f32x4 y[2][2];
+        for (int half = 0; half < 2; ++half) {
+            __syncthreads();                        // the slab is complete; the last reads of the previous half are done
+            const float* M = mseg(j) + (size_t)128 * half * W2_KD;
+            for (int i0 = 0; i0 < 32; i0 += 8) {
+                f32x4 pre[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int idx = tid + 256 * (i0 + i);                   // 64 pieces of 16 bytes per row
+                    pre[i] = *(const f32x4*)(M + (size_t)(idx >> 6) * W2_KD + (idx & 63) * 4);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int idx = tid + 256 * (i0 + i);
+                    *(f32x4*)(sM + (idx >> 6) * M2P + (idx & 63) * 4) = pre[i];
+                }
+            }
+            __syncthreads();                        // this half of M_j is in LDS
+            f32x4 acc[2][2];                        // two accumulation chains per tile (even / odd blocks)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) acc[i][0] = acc[i][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const f32x4 b = *(const f32x4*)(sSt + c16 * M2P + 16 * q + 4 * g);
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const f32x4 a = *(const f32x4*)(sM + (16 * (2 * w + i) + c16) * M2P + 16 * q + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][q & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], acc[i][q & 1], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                f32x4 sl;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sl[r] = sloc(j)[(size_t)(row_of(half, i) + r) * VP + v0 + c16];
+                y[half][i] = acc[i][0] + acc[i][1] + sl;
+            }
+        }
+        __syncthreads();                            // all waves have read the slab S_in[j]
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) x[half][i] = y[half][i];
+        publish(j + 1);
+    }
+}
+
+template <typename T, bool FULL>
+static int launch_wide256_kind(const ChunkParams& p, int NVB, const SegmentPlan& sp, int64_t blocks, hipStream_t stream) {
+    auto kern = gdn_chunk_wide256_kernel<T, FULL>;
     static SmemAttrDone attr_done;       // per instantiation
     if (int rc = ensure_dynamic_smem((const void*)kern, W2_SMEM, attr_done, "hipFuncSetAttribute(wide256)")) return rc;
+    if (blocks >= (1ll << 31)) { set_error("gdn_chunk_fwd: too many workgroups for one launch"); return GDN_ERR_UNSUPPORTED; }
+    if (blocks <= 0) return GDN_OK;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(W2_THREADS), W2_SMEM, stream, p, NVB, sp);
+    return check_launch("gdn_chunk_wide256_kernel");
+}
+
+template <typename T>
+int launch_wide256(const ChunkParams& p, hipStream_t stream) {
     const int NVB = (p.V + W2_VB - 1) / W2_VB;
-    const int64_t GV = (int64_t)(p.HV / p.H) * NVB;
-    // Time segments where whole sequences leave CUs without a workgroup: never more workgroups than CUs, segments of 8
-    // chunks or more, and at least 24 chunks saved per workgroup (a warm-up of typical length must pay)
+    const int64_t G = p.HV / p.H;
     SegmentPlan sp = {};
-    sp.nseg = 1;
+    sp.nseg = plan_segments256(p.N, p.H, p.HV, p.V, p.NT, p.cu_seqlens == nullptr, p.flags);
     sp.seg_chunks = 1 << 30;
-    const int64_t runs = p.N * p.H * GV;
-    if (!p.cu_seqlens && !(p.flags & (GDN_FLAG_SCAN_WIDE | GDN_FLAG_SCAN_NO_WARM)) && runs > 0) {
-        const int nseg = (int)std::min<int64_t>(256 / runs, p.NT / ((p.flags & GDN_FLAG_SCAN_SEGMENTS) ? 4 : 8));
-        if (nseg >= 2 && ((p.flags & GDN_FLAG_SCAN_SEGMENTS) || p.NT - p.NT / nseg >= 24)) {
-            sp.nseg = nseg;
-            sp.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
+    if (sp.nseg > 1) {
+        sp.seg_chunks = (int)((p.NT + sp.nseg - 1) / sp.nseg);
+        // Segments start warm where the decay allows it; the first pass and the merge then only serve the heads that need
+        // exact start states, and their workgroups for the other heads return at once.
+        if (!(p.flags & GDN_FLAG_SCAN_NO_WARM)) {
             sp.bound = p.ws.Bound;
             sp.warm_cap = std::min(WARM_CAP_MAX, sp.seg_chunks + sp.seg_chunks / 4 + 6);
         }
+        // pass 1: per (sequence, q/k head, segment but the last) the S runs of its value heads' column blocks, then the M runs
+        if (int rc = launch_wide256_kind<T, false>(p, NVB, sp, (p.N * p.H * (sp.nseg - 1) + 7) / 8 * 8 * G * (NVB + W2_KD / W2_VB), stream)) return rc;
+        static SmemAttrDone attr_done;
+        if (int rc = ensure_dynamic_smem((const void*)gdn_segment_merge256_kernel, MERGE256_SMEM, attr_done, "hipFuncSetAttribute(merge256)")) return rc;
+        const int VP = NVB * W2_VB;
+        hipLaunchKernelGGL(gdn_segment_merge256_kernel, dim3((unsigned)(p.NH * (VP / 16))), dim3(256), MERGE256_SMEM, stream, sp, p.ws.Seg,
+                           p.NH, p.HV, p.NT, VP, seg256_floats(p.V));
+        if (int rc = check_launch("gdn_segment_merge256_kernel")) return rc;
     }
-    const int64_t blocks = (p.N * p.H * sp.nseg + 7) / 8 * 8 * GV;
-    if (blocks >= (1ll << 31)) { set_error("gdn_chunk_fwd: too many workgroups for one launch"); return GDN_ERR_UNSUPPORTED; }
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(W2_THREADS), W2_SMEM, stream, p, NVB, sp);
-    return check_launch("gdn_chunk_wide256_kernel");
+    return launch_wide256_kind<T, true>(p, NVB, sp, (p.N * p.H * sp.nseg + 7) / 8 * 8 * G * NVB, stream);
 }
 
 template int launch_wide256<bf16_t>(const ChunkParams&, hipStream_t);

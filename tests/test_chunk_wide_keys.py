@@ -127,9 +127,10 @@ def test_wide_keys_outputs_fully_written_and_deterministic():
 @pytest.mark.parametrize('case', ['fast', 'slow', 'mixed'])
 def test_wide_keys_time_segments_that_start_warm(monkeypatch, case):
     """A long dense sequence on few heads is cut into time segments that start warm (a zero state a few chunks early, decided
-    per head on the device from the bound on the chunks' transitions); a head that decays too slowly for that is evaluated
-    whole by the workgroups of its first segment and equals the run without segments bit for bit."""
-    B, T, H, HV, K, V = 1, 4096, 2, 4, 256, 128                # 16 workgroups per segment: 8 segments of 8 chunks
+    per head on the device from the bound on the chunks' transitions); a head that decays too slowly for that takes the exact
+    start states of a first pass and a merge (fla/ops/common/intracard_cp.py:139-180 does the same inside one card), bit
+    for bit what the run with exact start states forced for every head gives it."""
+    B, T, H, HV, K, V = 1, 8192, 2, 4, 256, 256                # 16 workgroups per segment: 16 segments of 8 chunks in either mode
     q, k, v, _, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=31, h0_std=0.5, dtype=torch.bfloat16)
     per_token = {'fast': [0.1] * 4, 'slow': [1e-3] * 4, 'mixed': [0.1, 1e-3, 0.3, 0.005]}[case]
     gen = torch.Generator().manual_seed(32)
@@ -138,13 +139,48 @@ def test_wide_keys_time_segments_that_start_warm(monkeypatch, case):
     o_s, h_s = _run(q, k, v, g, beta, h0)
     _check('o', ref_o, o_s)
     _check('ht', ref_ht, h_s)
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'segments-exact')
+    o_e, h_e = _run(q, k, v, g, beta, h0)
+    _check('o (exact start states)', ref_o, o_e)
+    _check('ht (exact start states)', ref_ht, h_e)
     monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'wide')
     o_w, h_w = _run(q, k, v, g, beta, h0)
     slow_heads = {'fast': [], 'slow': [0, 1, 2, 3], 'mixed': [1, 3]}[case]
     for hv in range(HV):
-        same = torch.equal(o_s[:, :, hv], o_w[:, :, hv]) and torch.equal(h_s[:, hv], h_w[:, hv])
+        same = torch.equal(o_s[:, :, hv], o_e[:, :, hv]) and torch.equal(h_s[:, hv], h_e[:, hv])
+        # (the first segment starts from the true state in every form)
+        assert torch.equal(o_s[:, :512, hv], o_w[:, :512, hv]) and torch.equal(o_e[:, :512, hv], o_w[:, :512, hv]), hv
         if hv in slow_heads:
-            assert same, f'head {hv} cannot start warm and must be evaluated whole'
+            assert same, f'head {hv} cannot start warm and must take the exact start states'
         else:
-            # (the first segment starts from the true state either way; the later ones from a different, equally good one)
-            assert torch.equal(o_s[:, :512, hv], o_w[:, :512, hv]) and not same, hv
+            assert not same, hv                                 # a different, equally good start
+        # (two evaluations with 16-bit operands, each within the bar of the oracle)
+        assert O.get_err_ratio(o_w[:, :, hv].float().cpu(), o_e[:, :, hv].float().cpu()) < 7e-3, hv
+
+
+def test_wide_keys_exact_segments_layer_shape(monkeypatch):
+    """The reference layer's default head shape (K = 256, V = 512) on a prompt long enough for time segments, with gates that
+    hardly decay (no segment can start warm: first pass, merge of 256-row states, second pass), V-first states and a final state."""
+    B, T, H, HV, K, V = 1, 8192, 2, 2, 256, 512                # 16 segments of 8 chunks in either mode
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=41, gate_div=512.0, h0_std=0.5, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    o, ht = _run(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), state_v_first=True)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht.transpose(-1, -2))
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'segments-exact')
+    o_e, h_e = _run(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), state_v_first=True)
+    assert torch.equal(o, o_e) and torch.equal(ht, h_e)           # the automatic choice took that path by itself
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'wide')
+    o_w, h_w = _run(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), state_v_first=True)
+    assert not torch.equal(o, o_w)
+    _check('o (whole sequences)', ref_o, o_w)
+    # K below 256 and value columns past the last block: rows and columns of the segment buffers that no run writes
+    B, T, H, HV, K, V = 1, 2048, 1, 2, 192, 200
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, K, V, seed=42, gate_div=512.0, h0_std=0.5, dtype=torch.bfloat16)
+    ref_o, ref_ht = O.chunk_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    junk = [torch.full((1 << 22,), float('nan'), device='cuda') for _ in range(8)]
+    del junk
+    monkeypatch.setenv('FLA_HIP_SCAN_MODE', 'segments-exact')
+    o, ht = _run(q, k, v, g, beta, h0)
+    _check('o (K = 192, V = 200)', ref_o, o)
+    _check('ht (K = 192, V = 200)', ref_ht, ht)
