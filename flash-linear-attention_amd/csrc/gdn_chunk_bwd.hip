@@ -11,6 +11,12 @@
 //   dqkw      per (chunk, v-head)      dq, the parts of dk and dgam that come from the output and the state update, dw = -dv_new S^T
 //   wy        per (chunk, v-head)      through w, u, A back to k, v, beta, gam; dg = reverse cumulative sum of dgam
 //
+// The comba operator (fla/ops/comba/chunk.py:92-178) predicts with a second key p and the state BEFORE the token's decay:
+// with gam0 = gam - g its chunk form has A = (I + diag(beta) stril(p k^T o D0))^-1, D0_ij = e^(gam0_i - gam_j), and
+// w = A (beta e^gam0 p); everything between w, u and the state is the gated delta rule's.  So the two scans and the dqkw
+// kernel serve it unchanged, and `prepare` and `wy` have a COMBA form (one more tile: the rows of p; a second gradient,
+// dgam0, whose reverse cumulative sum enters dg without its own token).
+//
 // All matrix products run on the matrix cores from row-major LDS tiles.  A product's two operands have the same register
 // layout (lane (c16, g) holds index c16 and the 8 contraction indices 8g .. 8g+7 of a 32-wide step), so there are just two
 // ways to fetch an operand fragment from a row-major tile: `frag_rows` (the contraction runs along a row: one 16-byte read)
@@ -21,23 +27,23 @@
 
 namespace gdn {
 
-// Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels),
+// Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels), gam0 [64] fp32 (comba),
 // A [64][64], P^T [64][64], w [64][KD], u -> v_new [64][128], S [KD][128] ([K][V]), dS [KD][128], dv_new [64][128],
 // dw [64][KD], all in the operand type.
 struct BwdWs {
-    float* Gam; float* Dgam;
+    float* Gam; float* Dgam; float* Gam0;
     void* Am; void* PT; void* Wm; void* Vn; void* Hs; void* dHs; void* dVn; void* dWm;
 };
 inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
     const size_t u = (size_t)units;
-    void* Gam = take(u * 64 * 4); void* Dgam = take(u * 64 * 4);
+    void* Gam = take(u * 64 * 4); void* Dgam = take(u * 64 * 4); void* Gam0 = take(u * 64 * 4);
     void* Am = take(u * 64 * 64 * 2); void* PT = take(u * 64 * 64 * 2);
     void* Wm = take(u * 64 * KD * 2); void* Vn = take(u * 64 * BD * 2);
     void* Hs = take(u * KD * BD * 2); void* dHs = take(u * KD * BD * 2);
     void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * KD * 2);
-    if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm};
+    if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, (float*)Gam0, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm};
     return off;
 }
 
@@ -45,6 +51,7 @@ struct BwdParams {
     const void* q; const void* k; const void* v; const void* g; const void* beta;
     const float* h0; const void* dout; const float* dht;
     void* dq; void* dk; void* dv; float* dg; float* dbeta; float* dh0;
+    const void* pk; void* dp;            // (comba) the second key, the one the prediction is made with, and its gradient
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     BwdWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;
@@ -54,20 +61,24 @@ struct BwdParams {
 // ---------------------------------------------------------------------------------------------
 // prepare
 // ---------------------------------------------------------------------------------------------
-template <int KT> constexpr size_t bwd_prep_smem() { return (2 * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + (64 * PL + 128) * 4; }
+template <int KT, bool COMBA = false> constexpr size_t bwd_prep_smem() {
+    return ((2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + (64 * PL + 192) * 4;
+}
 
-template <typename T, int KT>
-__global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
+template <typename T, int KT, bool COMBA = false>
+__global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int KD = BD * KT, PK = KD + 8;
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sV = sQ + 64 * PK; T* sA = sV + 64 * P128;
-    float* sL = (float*)(sA + 64 * P64); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64;
+    T* sP = sA + 64 * P64;                                       // (comba) rows of the second key
+    float* sL = (float*)(sP + (COMBA ? 64 * PK : 0)); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64; float* sGam0 = sBeta + 64;
+    T* sRows = COMBA ? sP : sK;                                  // the rows that enter L from the left and w
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
     // Units in turn; the next unit's rows are fetched into registers while this one is worked on.
-    TileRegs<KD> rK, rQ;
+    TileRegs<KD> rK, rQ, rP;
     TileRegs<BD> rV;
     float rG = 0.f, rB = 0.f;
     auto fetch = [&](int64_t u) {
@@ -75,6 +86,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         const ChunkAt c = chunk_at(p, u / p.HV);
         fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         rG = rB = 0.f;
         if (w == 0 && lane < c.valid) {
@@ -87,6 +99,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
         put_tile<BD>(sV, P128, rV, tid);
+        if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
         if (w == 0) {
             float x = rG;
 #pragma unroll
@@ -95,7 +108,9 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
                 if (lane >= off) x += y;
             }
             sGam[lane] = x; sBeta[lane] = rB;
+            sGam0[lane] = COMBA ? x - rG : x;                    // (comba) the sum in front of this token: the prediction sees the state before its decay
             p.ws.Gam[u * 64 + lane] = x;
+            if constexpr (COMBA) p.ws.Gam0[u * 64 + lane] = x - rG;
         }
         lds_barrier();
         if (u + gridDim.x < units) fetch(u + gridDim.x);
@@ -110,7 +125,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 #pragma unroll
                     for (int s = 0; s < 4 * KT; ++s) {
                         const V8 b = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
-                        kk = Mma<T>::run(frag_rows(sK, PK, 16 * w, 32 * s, lane), b, kk);
+                        kk = Mma<T>::run(frag_rows(sRows, PK, 16 * w, 32 * s, lane), b, kk);
                         qk = Mma<T>::run(frag_rows(sQ, PK, 16 * w, 32 * s, lane), b, qk);
                     }
                 }
@@ -121,18 +136,19 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
                 for (int r = 0; r < 4; ++r) {
                     const int i = 16 * w + 4 * g + r;
                     const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
-                    if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = i > j ? sBeta[i] * kk[r] * d : 0.f;
+                    const float d0 = !COMBA ? d : i > j ? __expf(sGam0[i] - gj) : 0.f;
+                    if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = i > j ? sBeta[i] * kk[r] * d0 : 0.f;
                     pt[r] = p.scale * qk[r] * d;
                 }
                 *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
             }
         }
         lds_barrier();
-        // k -> beta e^gam k and v -> beta v, in place
+        // k -> beta e^gam k (comba: p -> beta e^gam0 p) and v -> beta v, in place
         for (int idx = tid; idx < 64 * 16 * (KT + 1); idx += 256) {
             const int row = idx / (16 * (KT + 1)), pc = idx % (16 * (KT + 1));      // the row's pieces of k, then those of v
-            T* at = pc < 16 * KT ? sK + row * PK + pc * 8 : sV + row * P128 + (pc - 16 * KT) * 8;
-            const float f = pc < 16 * KT ? sBeta[row] * __expf(sGam[row]) : sBeta[row];
+            T* at = pc < 16 * KT ? sRows + row * PK + pc * 8 : sV + row * P128 + (pc - 16 * KT) * 8;
+            const float f = pc < 16 * KT ? sBeta[row] * __expf(sGam0[row]) : sBeta[row];
             V8 x = *(V8*)at;
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
@@ -162,7 +178,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     if (2 * s > w) continue;                    // A is lower triangular
-                    aw = Mma<T>::run(frag_cols(sK, PK, 32 * s, 16 * n, lane), fa[s], aw);
+                    aw = Mma<T>::run(frag_cols(sRows, PK, 32 * s, 16 * n, lane), fa[s], aw);
                 }
                 *(V4*)(Wu + i * KD + 16 * n + 4 * g) = pack4<T>(aw);
             }
@@ -715,26 +731,33 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
 // One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.
-template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 640 * 4; }
+// COMBA: L = diag(beta) stril(p k^T o D0), w = X (e^gam0 p): the rows of p take the place of k's wherever k stood on the
+// left of k k^T or under e^gam, their gradient goes to dp, and the exponent of the row side is gam0, with a gradient of its own.
+template <int KT, bool COMBA = false> constexpr size_t bwd_wy_smem() {
+    return (2 * 64 * P128 + (2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + (640 + 320) * 4;
+}
 
-template <typename T, int KT>
+template <typename T, int KT, bool COMBA = false>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int KD = BD * KT, PK = KD + 8, NA = 2 * KT;      // NA tiles of 16 key features per wave: two in every block of 128
     extern __shared__ __align__(16) char smem[];
     T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * PK;
-    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
-    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
-    // (sDg, sDb [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
+    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64; T* sP = sM2 + 64 * P64;
+    float* sGam = (float*)(sP + (COMBA ? 64 * PK : 0)); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    float* sDg0 = sDb + 256; float* sGam0 = sDg0 + 256;
+    // (sDg, sDb, sDg0 [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
+    T* sRows = COMBA ? sP : sK;
+    float* sGamRow = COMBA ? sGam0 : sGam; float* sDgRow = COMBA ? sDg0 : sDg;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     auto feat = [&](int a) { return BD * (a >> 1) + 16 * (2 * w + (a & 1)); };       // first key feature of this wave's tile a
 
     TileRegs<BD> rDvn, rV;
-    TileRegs<KD> rDW, rK;
+    TileRegs<KD> rDW, rK, rP;
     TileRegs<CH> rA;
     V4 rDk[NA][4];                                               // what the previous kernel left in dk, at this lane's places
-    float rGam = 0.f, rBeta = 0.f, rDg = 0.f;
+    float rGam = 0.f, rBeta = 0.f, rDg = 0.f, rGam0 = 0.f;
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -743,10 +766,12 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
         fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
         fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if (tid < 64) {
             rGam = p.ws.Gam[u * 64 + tid];
             rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
             rDg = p.ws.Dgam[u * 64 + tid];
+            if constexpr (COMBA) rGam0 = p.ws.Gam0[u * 64 + tid];
         }
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -766,9 +791,11 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         put_tile<CH>(sA, P64, rA, tid);
         put_tile<KD>(sDW, PK, rDW, tid);
         put_tile<KD>(sK, PK, rK, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; }
+        if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; sGam0[tid] = rGam0; }
         sDg[tid] = tid < 64 ? rDg : 0.f;
         sDb[tid] = 0.f;
+        sDg0[tid] = 0.f;
         V4 dk_old[NA][4];
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -779,7 +806,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 
         // Operand fragments are fetched from LDS once and kept: what does not change across an inner loop is loaded outside it.
         // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta));
-        // k k^T of the same rows and columns is formed along the way, for the last step but one
+        // k k^T (comba: p k^T) of the same rows and columns is formed along the way, for the last step but one
         f32x4 kkT[4];
         {
             V8 fa[4], fw[4 * KT], fk[4 * KT];
@@ -788,7 +815,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) {
                 fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
-                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sRows, PK, 16 * w, 32 * s, lane);
             }
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
@@ -800,12 +827,13 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                     for (int s = 0; s < 4 * KT; ++s) {
                         const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
-                        dXw = Mma<T>::run(fw[s], bk, dXw);
+                        if constexpr (COMBA) dXw = Mma<T>::run(fw[s], frag_rows(sP, PK, 16 * tj, 32 * s, lane), dXw);
+                        else dXw = Mma<T>::run(fw[s], bk, dXw);
                         kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
                     }
                 }
                 const int j = 16 * tj + c16;
-                const float ej = __expf(sGam[j]), bj = sBeta[j];
+                const float ej = __expf(sGamRow[j]), bj = sBeta[j];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int i = 16 * w + 4 * g + r;
@@ -813,8 +841,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                 }
             }
         }
-        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
-        f32x4 dk[NA][4];
+        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam  (comba: d(e^gam0 p), into dp, dbeta, dgam0)
+        f32x4 dk[NA][4], dpk[COMBA ? NA : 1][4];
         {
             V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
             float ej[4], bj[4];
@@ -823,7 +851,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
                     if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                ej[t] = __expf(sGam[16 * t + c16]);
+                ej[t] = __expf(sGamRow[16 * t + c16]);
                 bj[t] = sBeta[16 * t + c16];
             }
 #pragma unroll
@@ -865,13 +893,14 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                         ak = Mma<T>::run(fdw[s], fA[t][s], ak);
                     }
                     const int j = 16 * t + c16;
-                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
+                    const V4 k4 = *(const V4*)(sRows + j * PK + n16 + 4 * g);
                     float dot = 0.f;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
                     dot = sum_over_g(dot);
-                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
-                    dk[a2][t] = ak * (bj[t] * ej[t]);
+                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDgRow[64 * w + j], bj[t] * ej[t] * dot); }
+                    if constexpr (COMBA) { dpk[a2][t] = ak * (bj[t] * ej[t]); dk[a2][t] = ZERO4; }
+                    else dk[a2][t] = ak * (bj[t] * ej[t]);
                 }
             }
         }
@@ -896,7 +925,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         {
             float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
+            for (int r = 0; r < 4; ++r) { gi[r] = sGamRow[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
             V8 fAt[2];
 #pragma unroll
             for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
@@ -931,17 +960,20 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
-                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
+                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDgRow[64 * w + 16 * w + 4 * g + r], b); }
             }
         }
         lds_barrier();
-        // dk += E k + E^T k, on top of what the previous kernel left
+        // dk += E k + E^T k, on top of what the previous kernel left  (comba: dp += E k, dk += E^T p)
         {
-            V8 fk[NA][2];
+            V8 fk[NA][2], fp[COMBA ? NA : 1][2];
 #pragma unroll
             for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
-                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
+                for (int s = 0; s < 2; ++s) {
+                    fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
+                    if constexpr (COMBA) fp[a2][s] = frag_cols(sP, PK, 32 * s, feat(a2), lane);
+                }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -949,12 +981,18 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
                         const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
 #pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        for (int a2 = 0; a2 < NA; ++a2) {
+                            if constexpr (COMBA) dpk[a2][t] = Mma<T>::run(fk[a2][s], e, dpk[a2][t]);
+                            else dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        }
                     }
                     if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
                         const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
 #pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        for (int a2 = 0; a2 < NA; ++a2) {
+                            if constexpr (COMBA) dk[a2][t] = Mma<T>::run(fp[a2][s], e, dk[a2][t]);
+                            else dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                        }
                     }
                 }
                 const int x = 16 * t + c16;
@@ -965,17 +1003,22 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
                         *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
+                        if constexpr (COMBA) *(V4*)((T*)p.dp + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(dpk[a2][t]);
                     }
                 }
             }
         }
         if (w == 0) {
             float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
+            // (comba) dg_t = sum_{s >= t} dgam_s + sum_{s > t} dgam0_s: one reverse cumulative sum of both, less the token's own dgam0
+            float own0 = 0.f;
+            if constexpr (COMBA) { own0 = (sDg0[lane] + sDg0[64 + lane]) + (sDg0[128 + lane] + sDg0[192 + lane]); x += own0; }
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
                 const float y = __shfl_down(x, off, 64);
                 if (lane + off < 64) x += y;
             }
+            x -= own0;
             if (lane < c.valid) {
                 p.dg[(c.tok0 + lane) * p.HV + hv] = x;
                 p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
@@ -985,7 +1028,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     }
 }
 
-template <typename T, int KT>
+template <typename T, int KT, bool COMBA = false>
 static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream) {
     // Value columns per workgroup of the scans: as few as it takes to give every (sequence, head) run its own CU
     // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.  With two
@@ -1022,11 +1065,11 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
         dstate.grid = 0;
     }
     const K ks[5] = {
-        {(const void*)gdn_bwd_prepare_kernel<T, KT>, bwd_prep_smem<KT>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
+        {(const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 && !COMBA ? 512u : 256u) ? units : (KT == 1 && !COMBA ? 512u : 256u)},
         state,
         dstate,
         {(const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
-        {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
+        {(const void*)gdn_bwd_wy_kernel<T, KT, COMBA>, bwd_wy_smem<KT, COMBA>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
     for (int i = 0; i < 5; ++i) {
         if (ks[i].grid == 0) continue;
@@ -1045,21 +1088,23 @@ extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, 
     return gdn::bwd_ws_layout(num_chunks * HV, K, nullptr, nullptr);
 }
 
-extern "C" int gdn_chunk_bwd(
-    const void* q, const void* k, const void* v, const void* g, const void* beta,
+// Both operators' entry: `pk` (and `dp`) non-NULL selects comba.
+static int chunk_bwd_entry(
+    const char* who, bool comba,
+    const void* q, const void* k, const void* pk, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,
-    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    const char* who = "gdn_chunk_bwd";
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
     GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
-    GDN_CHECK_ARG((K == BD || K == 2 * BD) && V == BD, GDN_ERR_UNSUPPORTED,
-                  "%s: K = 128 or 256 and V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros", who, (long long)K, (long long)V);
+    GDN_CHECK_ARG((K == BD || (K == 2 * BD && !comba)) && V == BD, GDN_ERR_UNSUPPORTED,
+                  "%s: K = 128%s and V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros", who, comba ? "" : " or 256",
+                  (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
     GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
                   "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
@@ -1079,7 +1124,8 @@ extern "C" int gdn_chunk_bwd(
     }
     GDN_CHECK_ARG(q && k && v && beta && dout && dq && dk && dv && dg && dbeta, GDN_ERR_INVALID,
                   "%s: q, k, v, beta, do, dq, dk, dv, dg, dbeta must not be NULL", who);
-    for (const void* x : {q, k, v, dout, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dv, (const void*)dh0})
+    GDN_CHECK_ARG(!comba || (pk && dp && g), GDN_ERR_INVALID, "%s: p, g and dp must not be NULL", who);
+    for (const void* x : {q, k, pk, v, dout, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dp, (const void*)dv, (const void*)dh0})
         GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
     GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
     BwdParams p;
@@ -1087,10 +1133,39 @@ extern "C" int gdn_chunk_bwd(
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
-    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0;
+    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0; p.pk = pk; p.dp = dp;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    if (comba) return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 1, true>(p, num_chunks, s) : launch_bwd<f16_t, 1, true>(p, num_chunks, s);
     if (K == BD) return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 1>(p, num_chunks, s) : launch_bwd<f16_t, 1>(p, num_chunks, s);
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 2>(p, num_chunks, s) : launch_bwd<f16_t, 2>(p, num_chunks, s);
+}
+
+extern "C" int gdn_chunk_bwd(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    return chunk_bwd_entry("gdn_chunk_bwd", false, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
+                           cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
+                           scale, qkv_dtype, gb_dtype, flags, stream);
+}
+
+extern "C" int gdn_chunk_comba_bwd(
+    const void* q, const void* k, const void* p, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    return chunk_bwd_entry("gdn_chunk_comba_bwd", true, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
+                           cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
+                           scale, qkv_dtype, gb_dtype, flags, stream);
 }

@@ -97,6 +97,14 @@ SIGNATURES['gdn_chunk_bwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_chunk_comba_bwd'] = (c_int, [
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k p v g beta
+    c_void_p, c_void_p, c_void_p,                      # h0 dout dht
+    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,      # dq dk dp dv dg dbeta dh0
+    c_void_p, c_void_p, c_void_p,                      # cu_seqlens chunk_table chunk_offsets
+    c_void_p, c_size_t,                                # workspace workspace_bytes
+    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
+    c_float, c_int, c_int, c_uint32, c_void_p])
 SIGNATURES['gdn_l2norm_fwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p])
 SIGNATURES['gdn_l2norm_bwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p])
 SIGNATURES['gdn_fused_recurrent_delta_bwd_value_block'] = (c_int64, [c_int64])

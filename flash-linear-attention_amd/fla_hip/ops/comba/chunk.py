@@ -1,8 +1,11 @@
 """``chunk_comba``: chunked prefill of the comba operator (the gated delta rule whose prediction uses a second key ``p`` and
-the state before the token's decay), forward only, with the signature and validation of fla/ops/comba/chunk.py:292-406.
-The reference's launches (``chunk_comba_cumsum_scalar_fwd``, ``chunk_scaled_dot_comba_pkt_fwd``, the triangular solve,
-``recompute_w_u_fwd``, ``chunk_gated_delta_rule_fwd_h``, ``chunk_fwd_o``; fla/ops/comba/chunk.py:22-90) are one call into
-libgdn_hip.so (``gdn_chunk_comba_fwd``): a chunk-parallel kernel and the sequential kernel of the chunked KDA forward."""
+the state before the token's decay), with the signature and validation of fla/ops/comba/chunk.py:292-406.
+The reference's forward launches (``chunk_comba_cumsum_scalar_fwd``, ``chunk_scaled_dot_comba_pkt_fwd``, the triangular
+solve, ``recompute_w_u_fwd``, ``chunk_gated_delta_rule_fwd_h``, ``chunk_fwd_o``; fla/ops/comba/chunk.py:22-90) are one call
+into libgdn_hip.so (``gdn_chunk_comba_fwd``): a chunk-parallel kernel and the sequential kernel of the chunked KDA forward.
+Its backward (``chunk_comba_bwd``, chunk.py:92-178, inside ``ChunkCombaFunction``, :181-289) is one call as well
+(``gdn_chunk_comba_bwd``): the kernels of the gated delta rule's backward, two of them in their comba form; nothing is
+kept from the forward call but its inputs."""
 from __future__ import annotations
 
 import torch
@@ -15,11 +18,11 @@ from fla_hip.ops.gated_delta_rule._common import (
     as_f32,
     current_stream_ptr,
     dtype_code,
-    forward_only,
     ptr,
     require_gpu,
 )
-from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.gated_delta_rule.chunk_bwd import _finish, l2norm_fwd
+from fla_hip.ops.utils.index import check_cu_seqlens, cu_bounds, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
 _DIM = 128          # head dims of the kernels; smaller ones are zero-padded
@@ -99,6 +102,124 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
     return o, ht
 
 
+def chunk_comba_bwd(q, k, v, p, g, beta, scale, initial_state, do, dht, cu_seqlens=None, cu_seqlens_cpu=None,
+                    q_rstd=None, k_rstd=None, p_rstd=None):
+    """q, k, p ``[B,T,H,K]``, v, do ``[B,T,HV,V]``, g (log decay), beta ``[B,T,HV]`` as the recurrence uses them.
+    Returns ``(dq, dk, dv, dp, dbeta, dg, dh0)``: dq, dk, dv, dp in q's dtype, dbeta, dg fp32, dh0 fp32 (None without
+    ``initial_state``).  With the ``*_rstd`` factors (what ``l2norm_fwd`` returns next to the normalised rows passed as
+    q, k, p) dq, dk, dp are the gradients of the rows before normalisation (fla/ops/comba/chunk.py:277-280)."""
+    dev = require_gpu(q, k, v, p, g, beta, do)
+    check_operand_shapes(q, k, v, g=g, beta=beta)
+    if do.shape != v.shape:
+        raise ValueError(f'do must have the shape of v, got {tuple(do.shape)} and {tuple(v.shape)}')
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if K > _DIM:
+        raise NotImplementedError(f'the chunked comba kernels cover key head dims up to {_DIM} (got K={K})')
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    nb = (V + _DIM - 1) // _DIM
+    if nb > 1:
+        # value columns are independent: a head with V > 128 is nb heads of 128 columns that share q, k, p, g, beta
+        def split(s):       # [N, HV, K, V] -> [N, HV*nb, K, 128]
+            if s is None:
+                return None
+            return _pad_last(s, nb * _DIM).reshape(N, HV, K, nb, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV * nb, K, _DIM)
+        v2 = _pad_last(v, nb * _DIM).reshape(B, T, HV * nb, _DIM)
+        do2 = _pad_last(do, nb * _DIM).reshape(B, T, HV * nb, _DIM)
+        dq, dk, dv2, dp, db2, dg2, dh2 = chunk_comba_bwd(
+            q, k, v2, p, g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2), scale, split(initial_state), do2,
+            split(dht), cu_seqlens, cu_seqlens_cpu, q_rstd, k_rstd, p_rstd)
+        dv = dv2.reshape(B, T, HV, nb * _DIM)[..., :V].contiguous()
+        db, dg = db2.reshape(B, T, HV, nb).sum(-1), dg2.reshape(B, T, HV, nb).sum(-1)
+        dh0 = None
+        if dh2 is not None:
+            dh0 = dh2.reshape(N, HV, nb, K, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV, K, nb * _DIM)[..., :V].contiguous()
+        return dq, dk, dv, dp, db, dg, dh0
+
+    out_dtype = q.dtype
+    work = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    qw, kw, pw, vw, dow = (aligned16(_pad_last(x.to(work), _DIM).contiguous()) for x in (q, k, p, v, do))
+    gw, bw = as_f32(g).contiguous(), as_f32(beta).contiguous()
+
+    def state_in(s):
+        if s is None:
+            return None
+        if tuple(s.shape) != (N, HV, K, V):
+            raise ValueError(f'initial_state and dht must have shape {(N, HV, K, V)}, got {tuple(s.shape)}')
+        return aligned16(F.pad(as_f32(s), (0, _DIM - V, 0, _DIM - K)).contiguous())
+    h0, dhtw = state_in(initial_state), state_in(dht)
+
+    flags = 0
+    chunk_table = chunk_offsets = None
+    alloc = torch.empty
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype not in (torch.int32, torch.int64):
+            cu_seqlens = cu_seqlens.long()
+        cu_seqlens = cu_seqlens.to(dev)
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
+        chunk_table = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        chunk_table = chunk_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        chunk_offsets = prepare_scan_tables(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        num_chunks = chunk_table.shape[0]
+        # tokens of a packed tensor outside every sequence are never written: they get zero gradients
+        first, last = cu_bounds(cu_seqlens, cu_seqlens_cpu)
+        if first != 0 or last != T:
+            alloc = torch.zeros
+    else:
+        num_chunks = B * ((T + _CHUNK - 1) // _CHUNK)
+
+    dq, dk, dp = (alloc(B, T, HV, _DIM, dtype=work, device=dev) for _ in range(3))
+    dv = alloc(B, T, HV, _DIM, dtype=work, device=dev)
+    dg = alloc(B, T, HV, dtype=torch.float32, device=dev)
+    db = alloc(B, T, HV, dtype=torch.float32, device=dev)
+    dh0 = torch.empty(N, HV, _DIM, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
+    lib = _lib.load()
+    ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, _DIM)
+    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _lib.check(lib.gdn_chunk_comba_bwd(
+        ptr(qw), ptr(kw), ptr(pw), ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
+        ptr(dq), ptr(dk), ptr(dp), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
+        ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
+        B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
+        current_stream_ptr(dev)))
+    dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
+    dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
+    dp = _finish(lib, dp, pw, p_rstd, H, K, out_dtype)
+    dv = dv[..., :V].to(out_dtype)
+    if dh0 is not None:
+        dh0 = dh0[..., :K, :V].contiguous()
+    return dq, dk, dv, dp, db, dg, dh0
+
+
+class ChunkCombaFunction(torch.autograd.Function):
+    """Forward through ``gdn_chunk_comba_fwd``, backward through ``gdn_chunk_comba_bwd`` (fla/ops/comba/chunk.py:181-289)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, p, g, beta, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel, cu_seqlens,
+                cu_seqlens_cpu):
+        o, ht = chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel,
+                                cu_seqlens, cu_seqlens_cpu)
+        ctx.save_for_backward(q, k, v, p, g, beta, initial_state, cu_seqlens, cu_seqlens_cpu)
+        ctx.opts = (scale, use_qk_l2norm_in_kernel)
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        q, k, v, p, g, beta, h0, cu_seqlens, cu_seqlens_cpu = ctx.saved_tensors
+        scale, l2 = ctx.opts
+        q_rstd = k_rstd = p_rstd = None
+        qn, kn, pn = q, k, p
+        if l2:
+            (qn, q_rstd), (kn, k_rstd), (pn, p_rstd) = l2norm_fwd(q), l2norm_fwd(k), l2norm_fwd(p)
+        dq, dk, dv, dp, db, dg, dh0 = chunk_comba_bwd(qn, kn, v, pn, g, beta, scale, h0, do.contiguous(), dht, cu_seqlens,
+                                                      cu_seqlens_cpu, q_rstd, k_rstd, p_rstd)
+        K = q.shape[-1]
+        return (dq[..., :K].to(q.dtype), dk[..., :K].to(k.dtype), dv.to(v.dtype), dp[..., :K].to(p.dtype), dg.to(g.dtype),
+                db.to(beta.dtype), None, dh0, None, None, None, None)
+
+
 def check_comba_args(q, k, v, p, g, beta, initial_state, cu_seqlens):
     """The reference's checks (fla/ops/comba/chunk.py:376-388) and the shapes the kernels rely on."""
     if cu_seqlens is not None:
@@ -134,7 +255,7 @@ def chunk_comba(
     cu_seqlens: torch.LongTensor | None = None,
     cu_seqlens_cpu: torch.LongTensor | None = None,
 ):
-    r"""Chunked comba (prefill), forward only.
+    r"""Chunked comba (prefill); differentiable in q, k, v, p, g, beta and ``initial_state``.
 
     Args:
         q, k, p: ``[B, T, H, K]``; ``p`` (the key the prediction is made with) defaults to ``k``.
@@ -152,8 +273,10 @@ def chunk_comba(
     if beta is None:
         beta = torch.ones_like(g)
     check_comba_args(q, k, v, p, g, beta, initial_state, cu_seqlens)
-    forward_only('chunk_comba', q, k, v, p, g, beta, initial_state)
     if scale is None:
         scale = k.shape[-1] ** -0.5
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, p, g, beta, initial_state)):
+        return ChunkCombaFunction.apply(q, k, v, p, g, beta, scale, initial_state, output_final_state,
+                                        use_qk_l2norm_in_kernel, cu_seqlens, cu_seqlens_cpu)
     return chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel,
                            cu_seqlens, cu_seqlens_cpu)

@@ -256,6 +256,27 @@ int gdn_chunk_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Backward pass of the chunked comba operator.  Replaces chunk_comba_bwd (fla/ops/comba/chunk.py:92-178): the
+ * gated delta rule's backward with the comba forms of recompute_w_u_fwd and prepare_wy_repr_bwd
+ * (fla/ops/comba/wy_fast.py), which form A and w from the second key p and the decay in front of each token
+ * (g0 = cumsum(g) - g, fla/ops/comba/utils.py), and the two reverse cumulative sums of dg (chunk.py:163-177).
+ * Arguments as for gdn_chunk_bwd, and:
+ *   p [B,T,H,K] in qkv_dtype: the key the prediction is made with, as the recurrence uses it (after its l2 norm, if any)
+ *   dp [B,T,HV,K] in qkv_dtype, per value head like dq and dk
+ *   g must not be NULL; K = 128 only (smaller head dims zero-padded by the caller), V = 128
+ *   workspace: gdn_chunk_bwd_workspace_bytes(num_chunks, HV, 128)
+ */
+int gdn_chunk_comba_bwd(
+    const void* q, const void* k, const void* p, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Row-wise l2 normalisation around gdn_chunk_bwd.  gdn_l2norm_fwd replaces l2norm_fwd (fla/modules/l2norm.py:222-262):
  * y[row] = x[row] / sqrt(sum x^2 + 1e-6) in x's dtype (bf16 or f16), rstd[row] = that factor; rows of D elements in,
  * rows of Dout >= D elements out (zeros from D on: the backward kernels want 128).  gdn_l2norm_bwd replaces l2norm_bwd

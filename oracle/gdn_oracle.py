@@ -38,7 +38,8 @@ fixtures); its gate activations are pinned by values that the formulas fix (``te
 The gradients (``gated_delta_rule_grads``) are pinned by central finite differences of the recurrence in fp64 for every input
 and every prologue, and the stage-by-stage backward agrees with them to 1e-12 (``tests/test_chunk_bwd.py``).
 The comba recurrence is pinned by scalar loops, by its chunked form (library triangular solve) and by its reduction to the
-delta rule at p = k, g = 0 (``test_comba_*`` in ``tests/test_oracle.py``).
+delta rule at p = k, g = 0 (``test_comba_*`` in ``tests/test_oracle.py``).  Its gradients (``comba_grads``) are pinned by central finite
+differences of that recurrence in fp64 for every input (``test_comba_grads_match_finite_differences``).
 No function here is "parity unpinned".
 
 Everything is computed in ``dtype`` (float32 by default, float64 for tight
@@ -546,6 +547,28 @@ def gated_delta_rule_grads(
     names = list(leaves)
     grads = torch.autograd.grad(loss, [leaves[n] for n in names], allow_unused=True)
     out = dict.fromkeys(('dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0', 'dA_log', 'ddt_bias'))
+    out.update(dict(zip(names, grads)))
+    return out
+
+
+def comba_grads(q, k, v, p, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
+                use_qk_l2norm_in_kernel=False, dtype=torch.float64):
+    """Gradients of  sum(o * do) + sum(ht * dht)  of the comba operator with respect to q, k, v, p, g, beta and the
+    initial state, by reverse-mode differentiation of ``recurrent_comba``: what the reference's tests take as the
+    truth for chunk_comba's backward pass (tests/ops/test_comba.py:92-150, autograd through fla/ops/comba/naive.py,
+    the same map).  Returns a dict with the keys dq, dk, dv, dp, dg, dbeta, dh0 (None where there is no such input)."""
+    leaves = {}
+    for name, x in dict(dq=q, dk=k, dv=v, dp=p, dg=g, dbeta=beta, dh0=initial_state).items():
+        leaves[name] = None if x is None else x.detach().to(dtype).clone().requires_grad_(True)
+    o, ht = recurrent_comba(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dp'], leaves['dg'], leaves['dbeta'], scale=scale,
+                            initial_state=leaves['dh0'], output_final_state=dht is not None, cu_seqlens=cu_seqlens,
+                            use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel, dtype=dtype)
+    loss = (o * do.to(dtype)).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.to(dtype)).sum()
+    names = [n for n, x in leaves.items() if x is not None]
+    grads = torch.autograd.grad(loss, [leaves[n] for n in names], allow_unused=True)
+    out = dict.fromkeys(leaves)
     out.update(dict(zip(names, grads)))
     return out
 

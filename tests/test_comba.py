@@ -164,7 +164,7 @@ def test_comba_validation():
     with pytest.raises(ValueError, match='g and beta'):
         chunk(q, k, v, p, g[..., :1], beta)
     with pytest.raises(NotImplementedError, match='no backward'):
-        chunk(q.clone().requires_grad_(), k, v, p, g, beta)
+        recurrent(q.clone().requires_grad_(), k, p, v, g, beta)
     with pytest.raises(NotImplementedError, match='per value column'):
         recurrent(q, k, p, v, g, beta[..., None].expand(-1, -1, -1, 64))
     with pytest.raises(RuntimeError, match='ROCm GPU'):
@@ -232,3 +232,108 @@ def test_chunk_comba_random_combinations(seed):
                       cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'))
     _check('o', ref_o, o, 5e-3)
     _check('ht', ref_ht, ht, 5e-3)
+
+
+# --------------------------------------------------------------------------------------------
+# backward of chunk_comba (gdn_chunk_comba_bwd) against the oracle's gradients
+# --------------------------------------------------------------------------------------------
+# (tests/ops/test_comba.py:198-206 and :290-297 of the reference)
+GRAD_TOL = dict(dq=0.005, dk=0.008, dv=0.005, dp=0.008, dg=0.02, dbeta=0.005, dh0=0.008)
+GRAD_TOL_PACKED = dict(dq=0.007, dk=0.008, dv=0.007, dp=0.008, dg=0.015, dbeta=0.015, dh0=0.007)
+
+
+def _comba_grads_gpu(q, k, v, p, g, beta, h0, do, dht, scale, cu=None, l2=False, idx_dtype=torch.int64):
+    chunk_comba, _ = _ops()
+    leaves = {n: (None if x is None else x.cuda().requires_grad_(True))
+              for n, x in dict(dq=q, dk=k, dv=v, dp=p, dg=g, dbeta=beta, dh0=h0).items()}
+    cu_t = None if cu is None else torch.tensor(cu, dtype=idx_dtype, device='cuda')
+    o, ht = chunk_comba(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dp'], leaves['dg'], leaves['dbeta'], scale=scale,
+                        initial_state=leaves['dh0'], output_final_state=True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu_t)
+    ((o.float() * do.cuda().float()).sum() + (ht * dht.cuda()).sum()).backward()
+    return o, ht, {n: (None if x is None else x.grad) for n, x in leaves.items()}
+
+
+def _compare_grads(ref, got, tol):
+    for n, r in ref.items():
+        if r is None:
+            continue
+        x = got[n].detach().float().cpu()
+        assert x.shape == r.shape, f'{n}: shape {tuple(x.shape)} vs {tuple(r.shape)}'
+        assert not torch.isnan(x).any(), f'{n}: NaN'
+        if O.get_abs_err(r, x) <= 1e-6:            # (fla/utils/_testing.py:28-34: gradients that vanish)
+            continue
+        e = O.get_err_ratio(r, x)
+        assert e <= tol[n], f'{n}: rel-rmse {e:.3e} > {tol[n]}'
+
+
+@pytest.mark.parametrize('B,T,H,HV,D,scale,normalizer,mask_p,l2,dtype', [
+    (1, 63, 1, 1, 64, 1, 1, 0, False, torch.float16),               # the reference's matrix (shorter where it is long)
+    (2, 500, 3, 3, 60, 1, 1, 0, False, torch.float16),
+    (2, 300, 3, 3, 64, 0.1, 1, 0.5, False, torch.float16),
+    (2, 256, 4, 4, 100, 1, 0.1, 0, False, torch.float16),
+    (2, 512, 4, 4, 128, 0.1, 1, 0, True, torch.float16),
+    (2, 256, 4, 4, 128, 0.1, 1, 0.5, False, torch.float16),
+    (2, 256, 4, 4, 128, 0.1, 10, 0, False, torch.float16),
+    (2, 200, 8, 8, 64, 0.1, 1, 0, True, torch.float16),
+    (2, 200, 2, 4, 128, None, 4.0, 0, False, torch.bfloat16),       # grouped value heads
+    (1, 130, 2, 6, 128, None, 4.0, 0, True, torch.bfloat16),
+    (3, 100, 12, 24, 128, None, 4.0, 0, False, torch.bfloat16),     # 72 runs: the scans take 64 value columns per workgroup
+    (2, 70, 80, 80, 128, None, 4.0, 0, False, torch.bfloat16),      # 160 runs: all 128
+])
+def test_chunk_comba_backward(B, T, H, HV, D, scale, normalizer, mask_p, l2, dtype):
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, HV, D, dtype, normalizer, mask_p, normalise=not l2, h0_std=0.5)
+    gen = torch.Generator().manual_seed(43)
+    do = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    dht = torch.randn(B, HV, D, D, generator=gen)
+    ref = O.comba_grads(q, k, v, p, g, beta, do, dht, scale=scale, initial_state=h0, use_qk_l2norm_in_kernel=l2, dtype=torch.float32)
+    o, ht, got = _comba_grads_gpu(q, k, v, p, g, beta, h0, do, dht, scale, l2=l2)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, scale, h0, True, use_qk_l2norm_in_kernel=l2)
+    _check('o', ref_o, o, 0.005)
+    _check('ht', ref_ht, ht, 0.005)
+    _compare_grads(ref, got, GRAD_TOL)
+    for n, x in dict(dq=q, dk=k, dv=v, dp=p, dg=g, dbeta=beta, dh0=h0).items():
+        assert got[n].dtype == x.dtype and got[n].shape == x.shape, n
+
+
+@pytest.mark.parametrize('H,D,mask_p,cu,idx_dtype', [
+    (4, 64, 0, [0, 15], torch.int32),
+    (4, 64, 0, [0, 256, 500, 1000], torch.int32),
+    (4, 64, 0.5, [0, 256, 500, 1000], torch.int64),
+    (4, 100, 0, [0, 15, 100, 300, 1200, 2000], torch.int32),
+    (2, 128, 0, [0, 64, 64, 129, 400], torch.int64),                # an empty sequence, a chunk boundary
+])
+def test_chunk_comba_backward_packed(H, D, mask_p, cu, idx_dtype):
+    T, N = cu[-1], len(cu) - 1
+    q, k, v, p, g, beta, _ = _inputs(1, T, H, H, D, torch.float16, 1.0, mask_p)
+    gen = torch.Generator().manual_seed(44)
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    do = torch.randn(1, T, H, D, generator=gen).half()
+    dht = torch.rand(N, H, D, D, generator=gen)
+    ref = O.comba_grads(q, k, v, p, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, dtype=torch.float32)
+    _, _, got = _comba_grads_gpu(q, k, v, p, g, beta, h0, do, dht, None, cu=cu, idx_dtype=idx_dtype)
+    _compare_grads(ref, got, GRAD_TOL_PACKED)
+
+
+def test_chunk_comba_backward_wide_values_and_outside_tokens():
+    """V = 256 (two heads of 128 columns inside), and a packed tensor whose sequences leave tokens out at both ends:
+    those get zero gradients."""
+    B, T, H, K, V = 1, 200, 2, 64, 256
+    gen = torch.Generator().manual_seed(45)
+    q, k, p = (F.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).bfloat16() for _ in range(3))
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.rand(B, T, H, generator=gen))
+    beta = torch.rand(B, T, H, generator=gen).sigmoid()
+    cu = [10, 90, 180]
+    h0 = torch.randn(2, H, K, V, generator=gen) * 0.5
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(2, H, K, V, generator=gen)
+    sl = slice(cu[0], cu[-1])
+    ref = O.comba_grads(q[:, sl], k[:, sl], v[:, sl], p[:, sl], g[:, sl], beta[:, sl], do[:, sl], dht, initial_state=h0,
+                        cu_seqlens=[c - cu[0] for c in cu], dtype=torch.float32)
+    _, _, got = _comba_grads_gpu(q, k, v, p, g, beta, h0, do, dht, None, cu=cu)
+    for n in ('dq', 'dk', 'dv', 'dp', 'dg', 'dbeta'):
+        x = got[n]
+        assert not x[:, :cu[0]].any() and not x[:, cu[-1]:].any(), f'{n}: tokens outside every sequence must get zero'
+        got[n] = x[:, sl]
+    _compare_grads(ref, got, GRAD_TOL)
+

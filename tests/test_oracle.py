@@ -375,3 +375,30 @@ def test_comba_reductions_and_chunk_form():
     o7, _ = O.recurrent_comba(q[:, :, :1].expand(-1, -1, 2, -1), k[:, :, :1].expand(-1, -1, 2, -1), v, p[:, :, :1].expand(-1, -1, 2, -1),
                               g, beta, 0.3, h0, dtype=torch.float64)
     assert torch.equal(o6, o7)
+
+
+@pytest.mark.parametrize('kw', [dict(), dict(use_qk_l2norm_in_kernel=True), dict(cu_seqlens=[0, 4, 11])])
+def test_comba_grads_match_finite_differences(kw):
+    """``comba_grads`` (reverse mode through the recurrence) against central differences of the recurrence itself, along a
+    random direction in every input; grouped value heads, rows that are not unit vectors, an initial state."""
+    B, T, H, HV, K, V = (1, 11, 2, 4, 5, 3) if 'cu_seqlens' in kw else (2, 8, 2, 4, 5, 3)
+    gen = torch.Generator().manual_seed(11)
+    f64 = dict(generator=gen, dtype=torch.float64)
+    q, k, p = (torch.randn(B, T, H, K, **f64) * s for s in (1.3, 0.6, 0.9))
+    v = torch.randn(B, T, HV, V, **f64)
+    g = F.logsigmoid(torch.randn(B, T, HV, **f64))
+    beta = torch.rand(B, T, HV, **f64)
+    h0 = torch.randn(2, HV, K, V, **f64) * 0.5
+    do, dht = torch.randn(B, T, HV, V, **f64), torch.randn(2, HV, K, V, **f64)
+    grads = O.comba_grads(q, k, v, p, g, beta, do, dht, scale=0.4, initial_state=h0, **kw)
+    inputs = dict(dq=q, dk=k, dv=v, dp=p, dg=g, dbeta=beta, dh0=h0)
+
+    def loss(a):
+        o, ht = O.recurrent_comba(a['dq'], a['dk'], a['dv'], a['dp'], a['dg'], a['dbeta'], 0.4, a['dh0'], True, dtype=torch.float64, **kw)
+        return float((o * do).sum() + (ht * dht).sum())
+    eps = 1e-6
+    for name, x in inputs.items():
+        d = torch.randn(x.shape, **f64)
+        fd = (loss({**inputs, name: x + eps * d}) - loss({**inputs, name: x - eps * d})) / (2 * eps)
+        an = float((grads[name] * d).sum())
+        assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), f'{name}: finite difference {fd} vs gradient {an}'
