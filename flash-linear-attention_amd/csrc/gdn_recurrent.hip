@@ -8,12 +8,16 @@
 // float4 pieces, every global access is a 16-byte piece of a contiguous row, so one wave
 // instruction reads whole rows - the step is a pure HBM stream of the state (read once,
 // written once, in place if the caller aliases ht to h0).
+//
+// The comba operator (fla/ops/comba/fused_recurrent.py:85-105) is the same recurrence with a second key p for the
+// prediction, taken on the state BEFORE the token's decay:  d = beta_t (v_t - S^T p_t);  S <- e^{g_t} S + k_t d^T.
 #include "gdn_common.h"
 
 namespace gdn {
 
 struct RecurrentParams {
     const void* q; const void* k; const void* v;
+    const void* pk;                      // comba: the key the prediction is made with (NULL otherwise)
     const void* g; const void* beta; const float* gk; const float* gv;
     const float* A_log; const float* dt_bias;
     const float* h0; float* ht; void* o;
@@ -59,8 +63,9 @@ __device__ __forceinline__ float wave_sum(float x) {
 }
 
 // KMAX: compile-time bound on K (rows padded with zeros), VB: value block per workgroup.
-template <typename T, int KMAX, int VB, bool VFIRST>
+template <typename T, int KMAX, int VB, bool VFIRST, bool COMBA = false>
 __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
+    static_assert(!(COMBA && VFIRST), "the comba recurrence is built for the K-first layout");
     // lanes along the contiguous dim (float4 each), the rest of the 256 threads along rows
     constexpr int CONT = VFIRST ? KMAX : VB;        // extent of the contiguous dim handled
     constexpr int TC = CONT / 4;                    // threads along the contiguous dim
@@ -134,8 +139,8 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
         }
     };
 
-    __shared__ float sh_q[2][KMAX], sh_k[2][KMAX];
-    __shared__ float sh_red[2][4][4];                       // per-wave partial sums for |q|^2, |k|^2, q.k
+    __shared__ float sh_q[2][KMAX], sh_k[2][KMAX], sh_p[2][COMBA ? KMAX : 1];
+    __shared__ float sh_red[2][4][4];                       // per-wave partial sums for |q|^2, |k|^2, q.k, |p|^2
     __shared__ float sh_part[2][4][2][VFIRST ? 4 : VB];     // K-first: per-wave column sums for S^T k and S^T q
 
     const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
@@ -155,6 +160,12 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
         if (tid < KMAX) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
         float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
         if ((tid & 63) == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
+        if constexpr (COMBA) {
+            const float pv = tid < K ? to_f32(((const T*)p.pk)[(tok * H + ih) * K + tid]) : 0.f;
+            if (tid < KMAX) sh_p[pb][tid] = pv;
+            const float spp = wave_sum(pv * pv);
+            if ((tid & 63) == 0) sh_red[pb][wave][3] = spp;
+        }
         // per-token scalars / per-column vectors (independent of the state)
         float eg = 1.f;
         if (p.g) {
@@ -166,21 +177,23 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
         sqq = sh_red[pb][0][0] + sh_red[pb][1][0] + sh_red[pb][2][0] + sh_red[pb][3][0];
         skk = sh_red[pb][0][1] + sh_red[pb][1][1] + sh_red[pb][2][1] + sh_red[pb][3][1];
         sqk = sh_red[pb][0][2] + sh_red[pb][1][2] + sh_red[pb][2][2] + sh_red[pb][3][2];
-        float rq = p.scale, rk = 1.f;
+        float rq = p.scale, rk = 1.f, rp = 1.f;
         if (p.flags & GDN_FLAG_QK_L2NORM) {
             rq *= 1.f / sqrtf(sqq + 1e-6f);
             rk = 1.f / sqrtf(skk + 1e-6f);
+            if constexpr (COMBA) rp = 1.f / sqrtf(sh_red[pb][0][3] + sh_red[pb][1][3] + sh_red[pb][2][3] + sh_red[pb][3][3] + 1e-6f);
         }
         const float qk = sqk * rq * rk;             // (scale q).k after normalisation
 
         if constexpr (!VFIRST) {
             // ---------------- K-first: rows are k, this thread owns 4 value columns ----------------
-            float kr[R], qr[R];
+            float kr[R], qr[R], pr[COMBA ? R : 1];
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 const int row = r0 + RP * i;
                 kr[i] = row < KMAX ? sh_k[pb][row] * rk : 0.f;
                 qr[i] = row < KMAX ? sh_q[pb][row] * rq : 0.f;
+                if constexpr (COMBA) pr[i] = row < KMAX ? sh_p[pb][row] * rp : 0.f;
             }
             f32x4 dgv = {1.f, 1.f, 1.f, 1.f};
             if (p.gv && cont_ok) {
@@ -191,13 +204,14 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
             f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < R; ++i) {
+                if constexpr (COMBA) sk += S[i] * pr[i];     // the prediction sees the state before this token's decay
                 f32x4 s = S[i] * dgv;
                 if (p.gk) {
                     const int row = r0 + RP * i;
                     if (row < K) s *= __expf(gate_k(p, tok, ihv, row, a_k));
                 }
                 S[i] = s;
-                sk += s * kr[i];
+                if constexpr (!COMBA) sk += s * kr[i];
                 sq += s * qr[i];
             }
             // reduce over the row groups that share this thread's columns: inside the wave, then across waves
@@ -572,6 +586,10 @@ static int launch_vb(const RecurrentParams& p0, int64_t n_states, int vb, hipStr
     dim3 grid((unsigned)place(p, n_states * p.NVB, (int64_t)p.HV * p.NVB)), block(256);
     void (*kern)(RecurrentParams) = vb == 128 ? gdn_recurrent_kernel<T, KMAX, 128, VFIRST>
                                    : vb == 64 ? gdn_recurrent_kernel<T, KMAX, 64, VFIRST> : gdn_recurrent_kernel<T, KMAX, 32, VFIRST>;
+    if constexpr (!VFIRST) {
+        if (p.pk) kern = vb == 128 ? gdn_recurrent_kernel<T, KMAX, 128, false, true>
+                       : vb == 64 ? gdn_recurrent_kernel<T, KMAX, 64, false, true> : gdn_recurrent_kernel<T, KMAX, 32, false, true>;
+    }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, p);
     return check_launch("gdn_recurrent_kernel");
 }
@@ -586,7 +604,7 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         return check_launch("gdn_decode_bf16_kernel");
     }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
-    if (p.K == 128 && p.V == 128 && !vfirst && !p.gk && !p.gv && n_states >= 1024 &&
+    if (p.K == 128 && p.V == 128 && !vfirst && !p.gk && !p.gv && !p.pk && n_states >= 1024 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
         RecurrentParams pd = p;
         const int64_t grid = place(pd, n_states, p.HV);
@@ -626,7 +644,7 @@ static int recurrent_entry(
     const void* cu_seqlens, const void* state_slots, const void* num_accepted, int64_t slots_stride,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream,
-    int gk_act, const float* gk_bias, float gk_lower) {
+    int gk_act, const float* gk_bias, float gk_lower, const void* pk = nullptr) {
     using namespace gdn;
     GDN_CHECK_ARG(T == 0 || (q && k && v && o), GDN_ERR_INVALID, "%s: q, k, v, o must not be NULL", who);
     GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && K >= 1 && V >= 1 && N >= 1, GDN_ERR_INVALID,
@@ -663,7 +681,7 @@ static int recurrent_entry(
         return GDN_OK;
     }
     RecurrentParams p;
-    p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.gk = gk; p.gv = gv;
+    p.q = q; p.k = k; p.v = v; p.pk = pk; p.g = g; p.beta = beta; p.gk = gk; p.gv = gv;
     p.A_log = A_log; p.dt_bias = dt_bias; p.h0 = h0; p.ht = ht; p.o = o; p.cu_seqlens = cu_seqlens; p.state_slots = state_slots;
     p.num_accepted = num_accepted; p.slots_stride = slots_stride;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.K = (int)K; p.V = (int)V; p.NVB = 1;
@@ -706,4 +724,20 @@ extern "C" int gdn_fused_recurrent_kda_fwd(
     GDN_CHECK_ARG(!(flags & GDN_FLAG_STATE_BF16), GDN_ERR_UNSUPPORTED, "%s: bf16 states are not supported with a decay per key feature", who);
     return recurrent_entry(who, q, k, v, nullptr, beta, g, nullptr, A_log, nullptr, h0, ht, o, cu_seqlens, state_slots,
                            num_accepted, slots_stride, B, T, H, HV, K, V, N, scale, qkv_dtype, gb_dtype, flags, stream, gate_mode, dt_bias, lower_bound);
+}
+
+// The comba operator's token recurrence: a second key p [B,T,H,K] for the prediction, made before the token's decay.
+extern "C" int gdn_fused_recurrent_comba_fwd(
+    const void* q, const void* k, const void* p, const void* v,
+    const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    const char* who = "gdn_fused_recurrent_comba_fwd";
+    GDN_CHECK_ARG(T == 0 || (p && g), GDN_ERR_INVALID, "%s: p and g must not be NULL", who);
+    GDN_CHECK_ARG((flags & ~(uint32_t)(GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM | GDN_FLAG_BETA_VECTOR)) == 0, GDN_ERR_UNSUPPORTED,
+                  "%s: only GDN_FLAG_CU_INT32, GDN_FLAG_QK_L2NORM (q, k and p) and GDN_FLAG_BETA_VECTOR are understood here", who);
+    return recurrent_entry(who, q, k, v, g, beta, nullptr, nullptr, nullptr, nullptr, h0, ht, o, cu_seqlens, nullptr, nullptr, 0,
+                           B, T, H, HV, K, V, N, scale, qkv_dtype, gb_dtype, flags, stream, 0, nullptr, 0.f, p);
 }

@@ -59,6 +59,13 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_int64,             # cu_seqlens state_slots num_accepted slots_stride
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
         c_float, c_int, c_int, c_uint32, c_void_p]),
+    'gdn_fused_recurrent_comba_fwd': (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p,            # q k p v
+        c_void_p, c_void_p,                                # g beta
+        c_void_p, c_void_p, c_void_p,                      # h0 ht o
+        c_void_p,                                          # cu_seqlens
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N
+        c_float, c_int, c_int, c_uint32, c_void_p]),
     'gdn_chunk_workspace_bytes': (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_uint32]),
     'gdn_causal_conv1d_fwd': (c_int, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # x weight bias residual initial_state

@@ -145,6 +145,24 @@ int gdn_fused_recurrent_kda_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Replaces fla/ops/comba/fused_recurrent.py:123-170 (fused_recurrent_comba_fwd and its kernel :37-120): the token recurrence
+ * of the comba operator in fp32,
+ *   d = beta_t (v_t - S^T p_t);  S <- e^{g_t} S + k_t d^T;  o_t = scale S^T q_t
+ * (the prediction uses the second key p and the state before the token's decay).
+ *   q, k, p [B,T,H,K], v, o [B,T,HV,V] (qkv_dtype: bf16, f16 or f32), g [B,T,HV] (log decay), beta [B,T,HV] or, with
+ *   GDN_FLAG_BETA_VECTOR, [B,T,HV,V] (gb_dtype; NULL: ones), h0, ht [N,HV,K,V] fp32 or NULL, cu_seqlens [N+1] or NULL.
+ *   flags: GDN_FLAG_QK_L2NORM (q, k and p are normalised, :90-93), GDN_FLAG_BETA_VECTOR, GDN_FLAG_CU_INT32.
+ *   K <= 256, K and V multiples of 4.  On the kernel of gdn_fused_recurrent_fwd.
+ */
+int gdn_fused_recurrent_comba_fwd(
+    const void* q, const void* k, const void* p, const void* v,
+    const void* g, const void* beta,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Bytes of device workspace gdn_chunk_fwd needs for the same N, T, num_chunks (64-token chunks; dense:
  * B*ceil(T/64); packed: sum over sequences of ceil(len/64)), head counts, packed (cu_seqlens given) and flags
  * (the scan flags change the plan and with it the size).  Returns 0 for unsupported (K,V).

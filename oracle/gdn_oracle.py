@@ -240,7 +240,7 @@ def recurrent_comba(
     form fla/ops/comba/naive.py:70-171, which the reference's tests take as the truth, is the same map): the prediction
     uses a second key p and the state BEFORE this token's decay,
         v' = beta (v - S^T p);  S <- e^g S + k v'^T;  o = S^T (q scale).
-    q, k, p: [B,T,H,K]; v: [B,T,HV,V]; g, beta: [B,T,HV]; p defaults to k.  With use_qk_l2norm_in_kernel q, k and p
+    q, k, p: [B,T,H,K]; v: [B,T,HV,V]; g: [B,T,HV]; beta: [B,T,HV] or, one per value column, [B,T,HV,V]; p defaults to k.  With use_qk_l2norm_in_kernel q, k and p
     are normalised (fused_recurrent.py:90-93)."""
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
@@ -264,7 +264,8 @@ def recurrent_comba(
     for n, (b, s, e) in enumerate(bounds):
         S = initial_state[n].to(dtype).clone() if initial_state is not None else torch.zeros(HV, K, V, dtype=dtype)
         for t in range(s, e):
-            vp = bf[b, t][:, None] * (vf[b, t] - torch.einsum('hkv,hk->hv', S, pf[b, t]))
+            bt = bf[b, t] if bf.dim() == 4 else bf[b, t][:, None]          # a beta per value column (fused_recurrent.py:68-71, 97-100)
+            vp = bt * (vf[b, t] - torch.einsum('hkv,hk->hv', S, pf[b, t]))
             S = S * gf[b, t].exp()[:, None, None] + kf[b, t][:, :, None] * vp[:, None, :]
             o[b, t] = torch.einsum('hkv,hk->hv', S, qf[b, t] * scale)
         ht[n] = S

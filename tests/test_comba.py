@@ -1,5 +1,5 @@
-"""The comba operator (chunk_comba, fused_recurrent_comba) on the HIP kernels, through gdn_chunk_comba_fwd, against the
-CPU oracle.  Shapes, input recipes and bars of the reference's own tests (tests/ops/test_comba.py: chunk 22-... fp16,
+"""The comba operator (chunk_comba through gdn_chunk_comba_fwd / gdn_chunk_comba_bwd, fused_recurrent_comba through the
+token kernel, gdn_fused_recurrent_comba_fwd) on the HIP kernels against the CPU oracle.  Shapes, input recipes and bars of the reference's own tests (tests/ops/test_comba.py: chunk 22-... fp16,
 normalised q, k, p, gates logsigmoid(rand) / normalizer with a share mask_p of them zeroed, o and ht within 0.005; the
 recurrent entry point fp32 and fp16 within 0.002; packed sequences with a random fp16 initial state)."""
 import ctypes
@@ -123,7 +123,19 @@ def test_comba_options_and_reductions():
     _check('gva o', ref_o, o, 5e-3)
     _check('gva ht', ref_ht, ht, 5e-3)
     o_r, ht_r = recurrent(dq, dk, dp, dv, dg, db, initial_state=dh, output_final_state=True)
-    assert torch.equal(o, o_r) and torch.equal(ht, ht_r)
+    _check('gva o, token kernel', ref_o, o_r, 2e-3)
+    _check('gva ht, token kernel', ref_ht, ht_r, 2e-3)
+    # a beta per value column, fp32 inputs, the l2 norm of q, k and p in the kernel (token kernel only)
+    gen = torch.Generator().manual_seed(8)
+    bv = torch.rand(B, T, HV, D, generator=gen)
+    q32, k32, p32 = (torch.randn(B, T, H, D, generator=gen) for _ in range(3))
+    v32 = v.float()
+    ref_o, ref_ht = O.recurrent_comba(q32, k32, v32, p32, g, bv, 0.5, h0, True, use_qk_l2norm_in_kernel=True)
+    o_r, ht_r = recurrent(q32.cuda(), k32.cuda(), p32.cuda(), v32.cuda(), dg, bv.cuda(), scale=0.5, initial_state=dh,
+                          output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert o_r.dtype == torch.float32
+    _check('vector beta o', ref_o, o_r, 1e-4)
+    _check('vector beta ht', ref_ht, ht_r, 1e-4)
 
     ref_o, _ = O.recurrent_comba(q, k, v, None, g, None)
     o, none = chunk(dq, dk, dv, None, dg)
@@ -165,8 +177,8 @@ def test_comba_validation():
         chunk(q, k, v, p, g[..., :1], beta)
     with pytest.raises(NotImplementedError, match='no backward'):
         recurrent(q.clone().requires_grad_(), k, p, v, g, beta)
-    with pytest.raises(NotImplementedError, match='per value column'):
-        recurrent(q, k, p, v, g, beta[..., None].expand(-1, -1, -1, 64))
+    with pytest.raises(ValueError, match='beta'):
+        recurrent(q, k, p, v, g, beta[..., None].expand(-1, -1, -1, 32))
     with pytest.raises(RuntimeError, match='ROCm GPU'):
         chunk(*(x.cpu() for x in (q, k, v, p, g, beta)))
     big = torch.zeros(1, 64, 1, 256, dtype=torch.bfloat16, device='cuda')

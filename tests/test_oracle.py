@@ -375,6 +375,12 @@ def test_comba_reductions_and_chunk_form():
     o7, _ = O.recurrent_comba(q[:, :, :1].expand(-1, -1, 2, -1), k[:, :, :1].expand(-1, -1, 2, -1), v, p[:, :, :1].expand(-1, -1, 2, -1),
                               g, beta, 0.3, h0, dtype=torch.float64)
     assert torch.equal(o6, o7)
+    # a beta per value column: every column is a recurrence of its own with that column's beta
+    bv = torch.rand(B, T, H, V, dtype=torch.float64)
+    o8, s8 = O.recurrent_comba(q, k, v, p, g, bv, 0.3, h0, True, dtype=torch.float64)
+    for c in (0, V - 1):
+        oc, sc = O.recurrent_comba(q, k, v[..., c:c + 1], p, g, bv[..., c], 0.3, h0[..., c:c + 1], True, dtype=torch.float64)
+        assert (o8[..., c:c + 1] - oc).abs().max() < 1e-12 and (s8[..., c:c + 1] - sc).abs().max() < 1e-12
 
 
 @pytest.mark.parametrize('kw', [dict(), dict(use_qk_l2norm_in_kernel=True), dict(cu_seqlens=[0, 4, 11])])
