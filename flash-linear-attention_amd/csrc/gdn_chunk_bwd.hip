@@ -23,16 +23,20 @@
 // and `frag_cols` (the contraction runs down a column: two transposing LDS reads).  The result of run(a, b) holds, in lane
 // (c16, g), column c16 (b's index) and rows 4g .. 4g+3 (a's index): whichever side carries the features gets them four in a
 // row per lane, which is what an 8-byte store into a row-major [token][feature] array wants.
-#include "gdn_tiles.h"
+#include "gdn_chunk_kda.h"
 
 namespace gdn {
 
 // Per (chunk, v-head) unit, in separate arrays: gam [64] fp32, dgam [64] fp32 (partial, between the last two kernels), gam0 [64] fp32 (comba),
 // A [64][64], P^T [64][64], w [64][KD], u -> v_new [64][128], S [KD][128] ([K][V]), dS [KD][128], dv_new [64][128],
 // dw [64][KD], all in the operand type.
+// The KDA operator (a decay per key feature) adds: Gk, the running sums of the log decays [64][128] fp32; QG = scale q e^Gk,
+// KG = k e^(Gk_last - Gk) [64][128] and P [64][64] in the operand type, EGL = e^Gk_last [128] fp32 (all four as the forward's
+// chunk-parallel kernel writes them); dPs = scale tril(do v_new^T) [64][64]; dGk [64][128] fp32 (partial, between the last two kernels).
 struct BwdWs {
     float* Gam; float* Dgam; float* Gam0;
     void* Am; void* PT; void* Wm; void* Vn; void* Hs; void* dHs; void* dVn; void* dWm;
+    float* Gk; void* QG; void* KG; void* Pm; float* EGL; void* dPs; float* dGk;
 };
 inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     size_t off = 0;
@@ -43,7 +47,22 @@ inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     void* Wm = take(u * 64 * KD * 2); void* Vn = take(u * 64 * BD * 2);
     void* Hs = take(u * KD * BD * 2); void* dHs = take(u * KD * BD * 2);
     void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * KD * 2);
-    if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, (float*)Gam0, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm};
+    if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, (float*)Gam0, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm,
+                        nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    return off;
+}
+inline size_t kda_bwd_ws_layout(int64_t units, char* base, BwdWs* ws) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
+    const size_t u = (size_t)units;
+    void* Am = take(u * 64 * 64 * 2); void* Pm = take(u * 64 * 64 * 2); void* dPs = take(u * 64 * 64 * 2);
+    void* Wm = take(u * 64 * BD * 2); void* Vn = take(u * 64 * BD * 2);
+    void* QG = take(u * 64 * BD * 2); void* KG = take(u * 64 * BD * 2);
+    void* Hs = take(u * BD * BD * 2); void* dHs = take(u * BD * BD * 2);
+    void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * BD * 2);
+    void* Gk = take(u * 64 * BD * 4); void* dGk = take(u * 64 * BD * 4); void* EGL = take(u * BD * 4);
+    if (ws) *ws = BwdWs{nullptr, nullptr, nullptr, Am, nullptr, Wm, Vn, Hs, dHs, dVn, dWm,
+                        (float*)Gk, QG, KG, Pm, (float*)EGL, dPs, (float*)dGk};
     return off;
 }
 
@@ -52,6 +71,7 @@ struct BwdParams {
     const float* h0; const void* dout; const float* dht;
     void* dq; void* dk; void* dv; float* dg; float* dbeta; float* dh0;
     const void* pk; void* dp;            // (comba) the second key, the one the prediction is made with, and its gradient
+    float* dgk;                          // (KDA) gradient of the log decays [B,T,HV,128] fp32
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     BwdWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;
@@ -206,7 +226,8 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
 template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
 template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
-template <typename T, int VBT, int KT, int AHEAD, int NW>
+// KDA: the rows of k arrive with their decay to the end of the chunk on them (KG), and the state decays per key feature (EGL).
+template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
 __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -234,7 +255,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
         }
     // (AHEAD = 2: two sets of registers take turns and the tiles of chunk c + 2 are requested while chunk c is worked on;
     // measured: no faster than one chunk of lead - a step is bound by the CU's load path, not by the way to memory)
-    struct Ahead { TileRegs<KD, NTH> rW, rK; V4 rU[NB]; float rGam; };
+    struct Ahead { TileRegs<KD, NTH> rW, rK; V4 rU[NB]; float rGam; float rE[NA]; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
@@ -242,8 +263,14 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
         fetch_tile<KD, NTH>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
-        if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+        if constexpr (KDA) {
+            fetch_tile<KD, NTH>(rK, (const T*)p.ws.KG + u * 64 * KD, KD, 64, tid);
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2) R.rE[a2] = p.ws.EGL[u * KD + 16 * (NA * w + a2) + c16];
+        } else {
+            fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+            if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + vq0 + 16 * b + 4 * g);
     };
@@ -256,6 +283,9 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
         V4 u4[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) u4[b] = rU[b];
+        float egk[NA];
+#pragma unroll
+        for (int a2 = 0; a2 < NA; ++a2) egk[a2] = R.rE[a2];
         T* Hu = (T*)p.ws.Hs + u * KD * BD;
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -272,7 +302,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
         {
             // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int i = 16 * w + c16;
-            const float dec = __expf(glast - sGam[i]);
+            const float dec = KDA ? 1.f : __expf(glast - sGam[i]);
             T* Vu = (T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0;
             V8 wf[4 * KT];
 #pragma unroll
@@ -303,7 +333,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
             for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
-                for (int b = 0; b < NB; ++b) S[a2][b] *= eg;
+                for (int b = 0; b < NB; ++b) S[a2][b] *= KDA ? egk[a2] : eg;
 #pragma unroll
             for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -330,13 +360,15 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 // (all 128 value columns of a head: eight waves, two per SIMD, share one set of tiles)
 template <int VBT> constexpr int scan_waves() { return VBT == BD ? 8 : 4; }
 
-template <typename T, int VBT, int KT>
+template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_state_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x, blockIdx.x);
+    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x);
 }
 
-template <typename T, int VBT, int KT, int AHEAD, int NW>
+// KDA: k and q arrive as KG and QG (decays and the scale on them), P row-major instead of transposed, the gradient of the
+// state decays per key feature.
+template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
 __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -364,19 +396,27 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
     // (two sets of registers for AHEAD = 2, as in the forward scan)
-    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; };
+    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv, tok0 = sq.bos + ic * CH;
         const int valid = (int)min((int64_t)CH, sq.len - ic * CH);
-        fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
-        fetch_tile<KD, NTH>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+        if constexpr (KDA) {
+            fetch_tile<KD, NTH>(rK, (const T*)p.ws.KG + u * 64 * KD, KD, 64, tid);
+            fetch_tile<KD, NTH>(rQ, (const T*)p.ws.QG + u * 64 * KD, KD, 64, tid);
+            fetch_tile<CH, NTH>(rPT, (const T*)p.ws.Pm + u * 64 * 64, 64, 64, tid);
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2) R.rE[a2] = p.ws.EGL[u * KD + 16 * (NA * w + a2) + c16];
+        } else {
+            fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+            fetch_tile<KD, NTH>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
+            fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
+            if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+        }
         fetch_tile<KD, NTH>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
         fetch_tile<VBT, NTH>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
-        if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
     };
     auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
@@ -387,6 +427,9 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         put_tile<CH, NTH>(sPT, P64, rPT, tid);
         put_tile<VBT, NTH>(sDO, PV, rDO, tid);
         if (tid < 64) sGam[tid] = rGam;
+        float egk[NA];
+#pragma unroll
+        for (int a2 = 0; a2 < NA; ++a2) egk[a2] = R.rE[a2];
         T* dHu = (T*)p.ws.dHs + u * KD * BD;
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -400,7 +443,8 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         lds_barrier();
         if (ic >= AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
-        // scale e^gam_i do_i, for the state's gradient
+        // scale e^gam_i do_i, for the state's gradient  (KDA: the factors are on the rows of q already)
+        if constexpr (!KDA)
         for (int idx = tid; idx < 64 * (VBT / 8); idx += NTH) {
             const int row = idx / (VBT / 8), pc = idx % (VBT / 8);
             const float f = p.scale * __expf(sGam[row]);
@@ -412,13 +456,13 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         {
             // dv_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int j = 16 * w + c16;
-            const float dec = __expf(glast - sGam[j]);
+            const float dec = KDA ? 1.f : __expf(glast - sGam[j]);
             T* dVu = (T*)p.ws.dVn + u * 64 * BD + j * BD + vcol0;
             V8 kf[4 * KT], pf[2];
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) kf[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) pf[s] = frag_rows(sPT, P64, 16 * w, 32 * s, lane);
+            for (int s = 0; s < 2; ++s) pf[s] = KDA ? frag_cols(sPT, P64, 32 * s, 16 * w, lane) : frag_rows(sPT, P64, 16 * w, 32 * s, lane);
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 f32x4 a1 = ZERO4, a2v = ZERO4;
@@ -448,12 +492,12 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
             for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
-                for (int b = 0; b < NB; ++b) dS[a2][b] *= eg;
+                for (int b = 0; b < NB; ++b) dS[a2][b] *= KDA ? egk[a2] : eg;
 #pragma unroll
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const V8 fo = frag_cols(sDOg, PV, 32 * s, vq0 + 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, vq0 + 16 * b, lane);
+                    const V8 fo = frag_cols(KDA ? sDO : sDOg, PV, 32 * s, vq0 + 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, vq0 + 16 * b, lane);
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) {
                         dS[a2][b] = Mma<T>::run(fo, qf[a2][s], dS[a2][b]);
@@ -484,10 +528,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     }
 }
 
-template <typename T, int VBT, int KT>
+template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>()>(p, smem, threadIdx.x, blockIdx.x);
+    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x);
 }
 
 // Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
@@ -496,12 +540,12 @@ __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(
 // time of the longer one.  Used where both sets of LDS tiles fit a CU (32 value columns per workgroup, one block of key features).
 template <int VBT, int KT> constexpr size_t bwd_scans_smem() { return bwd_state_smem<VBT, KT>() + bwd_dstate_smem<VBT, KT>(); }
 
-template <typename T, int VBT, int KT>
+template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
     static_assert(bwd_state_smem<VBT, KT>() % 16 == 0, "the second set of tiles starts 16-byte aligned");
-    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x);
-    else bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256, blockIdx.x);
+    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4, KDA>(p, smem, threadIdx.x, blockIdx.x);
+    else bwd_dstate_body<T, VBT, KT, 1, 4, KDA>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256, blockIdx.x);
 }
 
 // Both scans in one launch, in workgroups of their own: the first `nstate` workgroups walk forwards, the others backwards.
@@ -1081,6 +1125,8 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
     return GDN_OK;
 }
 
+#include "gdn_chunk_kda_bwd.h"      // (inside the namespace: it builds on the types and the two scans above)
+
 }  // namespace gdn
 
 extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t K) {
@@ -1168,4 +1214,68 @@ extern "C" int gdn_chunk_comba_bwd(
     return chunk_bwd_entry("gdn_chunk_comba_bwd", true, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
+}
+
+extern "C" size_t gdn_chunk_kda_bwd_workspace_bytes(int64_t num_chunks, int64_t HV) {
+    if (num_chunks < 0 || HV < 1) return 0;
+    return gdn::kda_bwd_ws_layout(num_chunks * HV, nullptr, nullptr);
+}
+
+extern "C" int gdn_chunk_kda_bwd(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    using namespace gdn;
+    const char* who = "gdn_chunk_kda_bwd";
+    GDN_CHECK_ARG(B >= 1 && T >= 0 && H >= 1 && HV >= 1 && N >= 1 && num_chunks >= 0, GDN_ERR_INVALID, "%s: bad dimension", who);
+    GDN_CHECK_ARG(HV % H == 0, GDN_ERR_INVALID, "%s: HV=%lld not divisible by H=%lld", who, (long long)HV, (long long)H);
+    GDN_CHECK_ARG(K == BD && V == BD, GDN_ERR_UNSUPPORTED, "%s: K = V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros",
+                  who, (long long)K, (long long)V);
+    GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
+    GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
+                  "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
+    GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
+                  "%s: too many heads or chunks for one launch", who);
+    if (cu_seqlens) {
+        GDN_CHECK_ARG(B == 1, GDN_ERR_INVALID, "%s: with cu_seqlens B must be 1", who);
+        GDN_CHECK_ARG((chunk_table || num_chunks == 0) && chunk_offsets, GDN_ERR_INVALID, "%s: packed input needs chunk_table and chunk_offsets", who);
+    } else {
+        GDN_CHECK_ARG(N == B, GDN_ERR_INVALID, "%s: without cu_seqlens N must equal B", who);
+        GDN_CHECK_ARG(num_chunks == B * ((T + CH - 1) / CH), GDN_ERR_INVALID, "%s: num_chunks does not match B and T", who);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0 || num_chunks == 0) {
+        if (dh0) return launch_state_copy(dht, dh0, N * HV * K * V, s);
+        return GDN_OK;
+    }
+    GDN_CHECK_ARG(q && k && v && g && beta && dout && dq && dk && dv && dg && dbeta, GDN_ERR_INVALID,
+                  "%s: q, k, v, g, beta, do, dq, dk, dv, dg, dbeta must not be NULL", who);
+    for (const void* x : {q, k, v, dout, (const void*)g, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dv,
+                          (const void*)dg, (const void*)dh0})
+        GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
+    GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
+    BwdParams p;
+    const size_t need = kda_bwd_ws_layout(num_chunks * HV, (char*)workspace, &p.ws);
+    GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
+                  need, workspace_bytes);
+    p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
+    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = nullptr; p.dbeta = dbeta; p.dh0 = dh0; p.pk = nullptr; p.dp = nullptr; p.dgk = dg;
+    p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
+    p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
+    p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    // the forward's chunk-parallel kernel again, writing into this workspace (u where the scan will put v_new)
+    KdaParams kp;
+    kp.q = q; kp.k = k; kp.v = v; kp.g = g; kp.beta = beta; kp.pk = nullptr; kp.gs = nullptr;
+    kp.A_log = nullptr; kp.gk_bias = nullptr; kp.gk_lower = 0.f; kp.gk_act = 0;
+    kp.h0 = nullptr; kp.ht = nullptr; kp.o = nullptr;
+    kp.cu_seqlens = cu_seqlens; kp.chunk_table = chunk_table; kp.chunk_offsets = chunk_offsets;
+    kp.ws = KdaWs{p.ws.Wm, p.ws.Vn, p.ws.QG, p.ws.KG, p.ws.Pm, p.ws.EGL, p.ws.Am, p.ws.Gk};
+    kp.T = T; kp.H = (int)H; kp.HV = (int)HV; kp.N = N; kp.NT = p.NT;
+    kp.scale = scale; kp.gb_dtype = gb_dtype; kp.flags = flags;
+    return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd_kda<bf16_t>(p, kp, num_chunks, qkv_dtype, s) : launch_bwd_kda<f16_t>(p, kp, num_chunks, qkv_dtype, s);
 }

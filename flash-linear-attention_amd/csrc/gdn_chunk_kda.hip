@@ -19,34 +19,9 @@
 // The comba operator (one decay per token and head, a second key p for the prediction, which sees the state before the
 // token's decay; fla/ops/comba/chunk.py:22-90) has a prepare kernel of its own that writes the same per-chunk operands,
 // and shares the scan:  M_ij = (p_i . k_j) e^(Gam0_i - Gam_j) with Gam0 = Gam - g,  w = A (beta p e^Gam0).
-#include "gdn_tiles.h"
+#include "gdn_chunk_kda.h"
 
 namespace gdn {
-
-constexpr int PG = BD + 4;           // pitch of the fp32 gate tile
-
-struct KdaWs { void* Wm; void* Um; void* QG; void* KG; void* Pm; float* EGL; };
-inline size_t kda_ws_layout(int64_t units, char* base, KdaWs* ws) {
-    size_t off = 0;
-    auto take = [&](size_t bytes) { size_t o = off; off += ws_align(bytes); return base ? (void*)(base + o) : nullptr; };
-    const size_t u = (size_t)units;
-    void* Wm = take(u * 64 * BD * 2); void* Um = take(u * 64 * BD * 2);
-    void* QG = take(u * 64 * BD * 2); void* KG = take(u * 64 * BD * 2);
-    void* Pm = take(u * 64 * 64 * 2); void* EGL = take(u * BD * 4);
-    if (ws) *ws = KdaWs{Wm, Um, QG, KG, Pm, (float*)EGL};
-    return off;
-}
-
-struct KdaParams {
-    const void* q; const void* k; const void* v; const float* g; const void* beta;
-    const void* pk; const void* gs;                                             // comba: the second key, the log decay per token and head
-    const float* A_log; const float* gk_bias; float gk_lower; int gk_act;      // gate activation, as in the token recurrence
-    const float* h0; float* ht; void* o;
-    const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
-    KdaWs ws;
-    int64_t T; int H, HV; int64_t N; int64_t NT;
-    float scale; int gb_dtype; uint32_t flags;
-};
 
 // ---------------------------------------------------------------------------------------------
 // prepare
@@ -254,6 +229,20 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
     lds_barrier();
     solve_unit_lower<T>(sL, sA, w, lane);
     lds_barrier();
+    if (p.ws.Am) {                                              // (for the backward pass)
+        T* Au = (T*)p.ws.Am + u * 64 * 64;
+        float* Gu = p.ws.Gk + u * 64 * BD;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+            *(u32x4*)(Au + row * 64 + pc * 8) = *(const u32x4*)(sA + row * P64 + pc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = tid + 256 * i, row = idx >> 5, pc = idx & 31;
+            *(f32x4*)(Gu + row * BD + pc * 4) = *(const f32x4*)(sG + row * PG + pc * 4);
+        }
+    }
     {
         // what the scan needs of q and k, and k, v as the factors of w, u
         T* QGu = (T*)p.ws.QG + u * 64 * BD;
@@ -640,6 +629,16 @@ static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream
     return GDN_OK;
 }
 
+
+int launch_kda_prepare(const KdaParams& p, int64_t num_chunks, int qkv_dtype, hipStream_t stream) {
+    const unsigned units = (unsigned)(num_chunks * p.HV);
+    const void* f = qkv_dtype == GDN_DTYPE_BF16 ? (const void*)gdn_kda_prepare_kernel<bf16_t> : (const void*)gdn_kda_prepare_kernel<f16_t>;
+    if (int rc = ensure_dynamic_smem_for(f, KDA_PREP_SMEM, "gdn_kda_prepare_kernel")) return rc;
+    int64_t nunits = units;
+    void* args[] = {(void*)&p, (void*)&nunits};
+    if (hipLaunchKernel(f, dim3(units < 256u ? units : 256u), dim3(256), args, KDA_PREP_SMEM, stream) != hipSuccess) return check_launch("gdn_kda_prepare_kernel");
+    return check_launch("gdn_kda_prepare_kernel");
+}
 
 // checks shared by the two entry points
 static int check_shapes(const char* who, int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V, int64_t N, int64_t num_chunks,

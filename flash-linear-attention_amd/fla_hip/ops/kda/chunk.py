@@ -1,8 +1,11 @@
-"""``chunk_kda``: chunked prefill of the KDA operator (the gated delta rule with a decay per key feature), forward
-only, with the signature, validation and error types of fla/ops/kda/chunk.py:178-443.  The reference's launches
+"""``chunk_kda``: chunked prefill of the KDA operator (the gated delta rule with a decay per key feature), with the
+signature, validation and error types of fla/ops/kda/chunk.py:178-443.  The reference's forward launches
 (gate activation + chunk-local cumsum, the intra-chunk stage, ``recompute_w_u_fwd``, the state recurrence and the output,
 fla/ops/kda/chunk_fwd.py:20-134) are one call into libgdn_hip.so (``gdn_chunk_kda_fwd``): a chunk-parallel kernel and a
-sequential one.  The activations the reference fuses (l2 norm of q and k, gate, beta sigmoid) happen inside the first."""
+sequential one.  The activations the reference fuses (l2 norm of q and k, gate, beta sigmoid) happen inside the first.
+Its backward (``chunk_kda_bwd``, fla/ops/kda/chunk_bwd.py, behind ``ChunkKDAFunction``, chunk.py:23-175) is one call as well
+(``gdn_chunk_kda_bwd``); nothing is kept from the forward call but its inputs, and the activations' derivatives are
+elementwise work around that call."""
 from __future__ import annotations
 
 import torch
@@ -15,11 +18,11 @@ from fla_hip.ops.gated_delta_rule._common import (
     as_f32,
     current_stream_ptr,
     dtype_code,
-    forward_only,
     ptr,
     require_gpu,
 )
-from fla_hip.ops.utils.index import check_cu_seqlens, prepare_chunk_indices, prepare_scan_tables
+from fla_hip.ops.gated_delta_rule.chunk_bwd import _finish, l2norm_fwd
+from fla_hip.ops.utils.index import check_cu_seqlens, cu_bounds, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
 _DIM = 128          # head dims of the kernels; smaller ones are zero-padded
@@ -127,6 +130,175 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
     return o, ht
 
 
+def chunk_kda_bwd(q, k, v, g, beta, scale, initial_state, do, dht, state_v_first=False, cu_seqlens=None, cu_seqlens_cpu=None,
+                  q_rstd=None, k_rstd=None):
+    """q, k ``[B,T,H,K]``, v, do ``[B,T,HV,V]``, g ``[B,T,HV,K]`` (log decays), beta ``[B,T,HV]`` as the recurrence uses them.
+    Returns ``(dq, dk, dv, dbeta, dg, dh0)``: dq, dk, dv in q's dtype, dbeta ``[B,T,HV]`` and dg ``[B,T,HV,K]`` fp32, dh0 fp32
+    (None without ``initial_state``).  With ``q_rstd``, ``k_rstd`` (what ``l2norm_fwd`` returns next to the normalised rows
+    passed as q and k) dq and dk are the gradients of the rows before normalisation."""
+    dev = require_gpu(q, k, v, g, beta, do)
+    check_operand_shapes(q, k, v, beta=beta, gk=g)
+    if do.shape != v.shape:
+        raise ValueError(f'do must have the shape of v, got {tuple(do.shape)} and {tuple(v.shape)}')
+    B, T, H, K = k.shape
+    HV, V = v.shape[2], v.shape[3]
+    if K > _DIM:
+        raise NotImplementedError(f'the chunked KDA kernels cover key head dims up to {_DIM} (got K={K})')
+    N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    nb = (V + _DIM - 1) // _DIM
+    if nb > 1:
+        # value columns are independent: a head with V > 128 is nb heads of 128 columns that share q, k, g, beta
+        def split(s):       # [N, HV, K, V] -> [N, HV*nb, K, 128]  (V-first: [N, HV, V, K] -> [N, HV*nb, 128, K])
+            if s is None:
+                return None
+            if state_v_first:
+                return F.pad(s, (0, 0, 0, nb * _DIM - V)).reshape(N, HV * nb, _DIM, K)
+            return _pad_last(s, nb * _DIM).reshape(N, HV, K, nb, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV * nb, K, _DIM)
+        v2 = _pad_last(v, nb * _DIM).reshape(B, T, HV * nb, _DIM)
+        do2 = _pad_last(do, nb * _DIM).reshape(B, T, HV * nb, _DIM)
+        dq, dk, dv2, db2, dg2, dh2 = chunk_kda_bwd(
+            q, k, v2, g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2), scale, split(initial_state), do2,
+            split(dht), state_v_first, cu_seqlens, cu_seqlens_cpu, q_rstd, k_rstd)
+        dv = dv2.reshape(B, T, HV, nb * _DIM)[..., :V].contiguous()
+        db, dg = db2.reshape(B, T, HV, nb).sum(-1), dg2.reshape(B, T, HV, nb, K).sum(-2)
+        dh0 = None
+        if dh2 is not None:
+            if state_v_first:
+                dh0 = dh2.reshape(N, HV, nb * _DIM, K)[:, :, :V]
+            else:
+                dh0 = dh2.reshape(N, HV, nb, K, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV, K, nb * _DIM)[..., :V]
+            dh0 = dh0.contiguous()
+        return dq, dk, dv, db, dg, dh0
+
+    out_dtype = q.dtype
+    work = q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    qw, kw, vw, dow = (aligned16(_pad_last(x.to(work), _DIM).contiguous()) for x in (q, k, v, do))
+    gw = aligned16(_pad_last(as_f32(g), _DIM).contiguous())
+    bw = as_f32(beta).contiguous()
+
+    def state_in(s):
+        if s is None:
+            return None
+        want = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+        if tuple(s.shape) != want:
+            raise ValueError(f'initial_state and dht must have shape {want}, got {tuple(s.shape)}')
+        s = as_f32(s)
+        if state_v_first:
+            s = s.transpose(-1, -2)
+        return aligned16(F.pad(s, (0, _DIM - V, 0, _DIM - K)).contiguous())
+    h0, dhtw = state_in(initial_state), state_in(dht)
+
+    flags = 0
+    chunk_table = chunk_offsets = None
+    alloc = torch.empty
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype not in (torch.int32, torch.int64):
+            cu_seqlens = cu_seqlens.long()
+        cu_seqlens = cu_seqlens.to(dev)
+        if cu_seqlens.dtype == torch.int32:
+            flags |= _lib.FLAG_CU_INT32
+        check_cu_seqlens(cu_seqlens, T, cu_seqlens_cpu)
+        chunk_table = prepare_chunk_indices(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        chunk_table = chunk_table.to(device=dev, dtype=cu_seqlens.dtype).contiguous()
+        chunk_offsets = prepare_scan_tables(cu_seqlens, _CHUNK, cu_seqlens_cpu=cu_seqlens_cpu)
+        num_chunks = chunk_table.shape[0]
+        # tokens of a packed tensor outside every sequence are never written: they get zero gradients
+        first, last = cu_bounds(cu_seqlens, cu_seqlens_cpu)
+        if first != 0 or last != T:
+            alloc = torch.zeros
+    else:
+        num_chunks = B * ((T + _CHUNK - 1) // _CHUNK)
+
+    dq, dk, dv = (alloc(B, T, HV, _DIM, dtype=work, device=dev) for _ in range(3))
+    dg = alloc(B, T, HV, _DIM, dtype=torch.float32, device=dev)
+    db = alloc(B, T, HV, dtype=torch.float32, device=dev)
+    dh0 = torch.empty(N, HV, _DIM, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
+    lib = _lib.load()
+    ws_bytes = lib.gdn_chunk_kda_bwd_workspace_bytes(num_chunks, HV)
+    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    _lib.check(lib.gdn_chunk_kda_bwd(
+        ptr(qw), ptr(kw), ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
+        ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
+        ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
+        B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
+        current_stream_ptr(dev)))
+    dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
+    dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
+    dv = dv[..., :V].to(out_dtype)
+    dg = dg[..., :K]
+    if dh0 is not None:
+        dh0 = dh0[..., :K, :V]
+        dh0 = (dh0.transpose(-1, -2) if state_v_first else dh0).contiguous()
+    return dq, dk, dv, db, dg, dh0
+
+
+def _kda_gate(g, A_log, dt_bias, lower_bound):
+    """The gate activation in fp32 (fla/ops/kda/gate.py:27-94) and what its derivative needs: returns
+    ``(log decay, x = g + dt_bias, a = exp(A_log) per head or None)``."""
+    HV, K = g.shape[-2:]
+    x = g.float()
+    if dt_bias is not None:
+        x = x + dt_bias.float().reshape(HV, K)
+    a = None if A_log is None else A_log.float().exp().reshape(HV, 1)
+    if lower_bound is not None:
+        return lower_bound * torch.sigmoid(x if a is None else a * x), x, a
+    return -(a if a is not None else torch.e) * F.softplus(x), x, a
+
+
+class ChunkKDAFunction(torch.autograd.Function):
+    """Forward through ``gdn_chunk_kda_fwd``, backward through ``gdn_chunk_kda_bwd`` (fla/ops/kda/chunk.py:23-175)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel,
+                gate_mode, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, cu_seqlens, cu_seqlens_cpu, lower_bound):
+        o, ht = chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first, cu_seqlens,
+                              cu_seqlens_cpu, A_log, dt_bias, lower_bound, gate_mode, use_qk_l2norm_in_kernel,
+                              use_beta_sigmoid_in_kernel, allow_neg_eigval)
+        ctx.save_for_backward(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, cu_seqlens_cpu)
+        ctx.opts = (scale, use_qk_l2norm_in_kernel, gate_mode, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, lower_bound)
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        q, k, v, g_in, beta_raw, A_log, dt_bias, h0, cu_seqlens, cu_seqlens_cpu = ctx.saved_tensors
+        scale, l2, gate_mode, bsig, neg, state_v_first, lower_bound = ctx.opts
+        q_rstd = k_rstd = None
+        qn, kn = q, k
+        if l2:
+            (qn, q_rstd), (kn, k_rstd) = l2norm_fwd(q), l2norm_fwd(k)
+        beta = beta_raw
+        if bsig:
+            beta = torch.sigmoid(beta_raw.float()) * (2.0 if neg else 1.0)
+        g = g_in
+        if gate_mode:
+            g, x, a = _kda_gate(g_in, A_log, dt_bias, lower_bound if gate_mode == 2 else None)
+        dq, dk, dv, db, dg, dh0 = chunk_kda_bwd(qn, kn, v, g, beta, scale, h0, do.contiguous(), dht, state_v_first,
+                                                cu_seqlens, cu_seqlens_cpu, q_rstd, k_rstd)
+        if bsig:
+            s = torch.sigmoid(beta_raw.float())
+            db = db * s * (1 - s) * (2.0 if neg else 1.0)
+        dA_log = ddt_bias = None
+        if gate_mode:
+            # (fla/ops/kda/gate.py)  softplus form: dg/dx = -a sigmoid(x), dg/dA_log = g;  bounded form, s = sigmoid(a x):
+            # dg/dx = lower_bound s (1 - s) a, dg/dA_log = lower_bound s (1 - s) a x
+            if gate_mode == 2:
+                s = torch.sigmoid(x if a is None else a * x)
+                ds = dg * (lower_bound * s * (1 - s))
+                if A_log is not None:
+                    dA_log = (ds * a * x).sum((0, 1, 3)).to(A_log.dtype).reshape(A_log.shape)
+                    ds = ds * a
+                dg = ds
+            else:
+                if A_log is not None:
+                    dA_log = (dg * g).sum((0, 1, 3)).to(A_log.dtype).reshape(A_log.shape)
+                dg = dg * (-(a if a is not None else torch.e) * torch.sigmoid(x))
+            if dt_bias is not None:
+                ddt_bias = dg.sum((0, 1)).to(dt_bias.dtype).reshape(dt_bias.shape)
+        K = q.shape[-1]
+        return (dq[..., :K].to(q.dtype), dk[..., :K].to(k.dtype), dv.to(v.dtype), dg.to(g_in.dtype), db.to(beta_raw.dtype), dA_log, ddt_bias,
+                None, dh0, None, None, None, None, None, None, None, None, None)
+
+
 @torch.compiler.disable
 def chunk_kda(
     q: torch.Tensor,
@@ -151,7 +323,7 @@ def chunk_kda(
     cp_context=None,
     **kwargs,
 ):
-    r"""Chunked KDA (prefill), forward only.
+    r"""Chunked KDA (prefill); differentiable in q, k, v, g, beta, ``A_log``, ``dt_bias`` and ``initial_state``.
 
     Args:
         q, k: ``[B, T, H, K]``; v: ``[B, T, HV, V]`` with ``HV % H == 0``.
@@ -161,7 +333,8 @@ def chunk_kda(
         beta: ``[B, T, HV]`` (logits with ``use_beta_sigmoid_in_kernel``; ``allow_neg_eigval`` doubles the sigmoid).
         scale: defaults to ``K ** -0.5``.  initial_state: ``[N, HV, K, V]`` (``[N, HV, V, K]`` with ``state_v_first``).
         safe_gate: accepted; the kernels form the intra-chunk decays pair by pair inside blocks of 16 rows whatever the
-            gate's range, so it changes nothing here.  disable_recompute: accepted, nothing is saved (forward only).
+            gate's range, so it changes nothing here.  disable_recompute: accepted; the backward pass always computes the
+            forward's intermediates again.
         return_intermediate_states, cp_context: not part of this build.
         cu_seqlens: ``[N + 1]`` boundaries of packed sequences (then ``B == 1``).
 
@@ -203,9 +376,12 @@ def chunk_kda(
         gate_mode = 2 if lower_bound is not None else 1
     else:
         A_log = dt_bias = None
-    forward_only('chunk_kda', q, k, v, g, beta, initial_state)
     if scale is None:
         scale = k.shape[-1] ** -0.5
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, g, beta, A_log, dt_bias, initial_state)):
+        return ChunkKDAFunction.apply(q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state,
+                                      use_qk_l2norm_in_kernel, gate_mode, use_beta_sigmoid_in_kernel, allow_neg_eigval,
+                                      state_v_first, cu_seqlens, cu_seqlens_cpu, lower_bound)
     return chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first, cu_seqlens,
                          cu_seqlens_cpu, A_log, dt_bias, lower_bound, gate_mode, use_qk_l2norm_in_kernel,
                          use_beta_sigmoid_in_kernel, allow_neg_eigval)

@@ -295,6 +295,30 @@ int gdn_chunk_comba_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * Backward pass of the chunked KDA operator.  Replaces chunk_kda_bwd (fla/ops/kda/chunk_bwd.py, called from
+ * ChunkKDAFunction.backward, fla/ops/kda/chunk.py:124-175): the forward's intermediates are computed again (the
+ * chunk-parallel kernel of gdn_chunk_kda_fwd, then the state scan), then the reverse scan, dq / dk / dw and the way back
+ * through w, u and the two matrices with a decay per pair of rows and key feature (the reference's
+ * chunk_kda_bwd_intra / chunk_kda_bwd_wy_dqkg_fused), and the reverse chunk-local cumulative sum of dg.
+ * Arguments as for gdn_chunk_bwd, except:
+ *   g [B,T,HV,K] fp32: the log decay per key feature as the recurrence uses it (after the gate activation, whose
+ *   derivative is the caller's, like those of the l2 norm and of the beta sigmoid); must not be NULL
+ *   dg [B,T,HV,K] fp32
+ *   K = V = 128 only (smaller head dims zero-padded by the caller; V > 128 as value heads of 128 columns)
+ *   workspace: gdn_chunk_kda_bwd_workspace_bytes(num_chunks, HV)
+ */
+size_t gdn_chunk_kda_bwd_workspace_bytes(int64_t num_chunks, int64_t HV);
+int gdn_chunk_kda_bwd(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Row-wise l2 normalisation around gdn_chunk_bwd.  gdn_l2norm_fwd replaces l2norm_fwd (fla/modules/l2norm.py:222-262):
  * y[row] = x[row] / sqrt(sum x^2 + 1e-6) in x's dtype (bf16 or f16), rstd[row] = that factor; rows of D elements in,
  * rows of Dout >= D elements out (zeros from D on: the backward kernels want 128).  gdn_l2norm_bwd replaces l2norm_bwd

@@ -38,7 +38,8 @@ fixtures); its gate activations are pinned by values that the formulas fix (``te
 The gradients (``gated_delta_rule_grads``) are pinned by central finite differences of the recurrence in fp64 for every input
 and every prologue, and the stage-by-stage backward agrees with them to 1e-12 (``tests/test_chunk_bwd.py``).
 The comba recurrence is pinned by scalar loops, by its chunked form (library triangular solve) and by its reduction to the
-delta rule at p = k, g = 0 (``test_comba_*`` in ``tests/test_oracle.py``).  Its gradients (``comba_grads``) are pinned by central finite
+delta rule at p = k, g = 0 (``test_comba_*`` in ``tests/test_oracle.py``).  Its gradients (``comba_grads``) and those of the KDA recurrence
+(``kda_grads``, every gate activation) are pinned by central finite
 differences of that recurrence in fp64 for every input (``test_comba_grads_match_finite_differences``).
 No function here is "parity unpinned".
 
@@ -101,14 +102,15 @@ def kda_gate(g: torch.Tensor, A_log: torch.Tensor | None = None, dt_bias: torch.
     ``lower_bound * sigmoid(exp(A_log[hv]) * g)``.  Without A_log the factor is 1 under the sigmoid and exp(1) in
     front of the softplus (the recurrent kernel's constant, fla/ops/kda/fused_recurrent.py:168-181)."""
     HV, K = g.shape[-2:]
-    x = g.float()
+    dt = torch.float64 if g.dtype == torch.float64 else torch.float32       # (fp64 for the finite-difference pins)
+    x = g.to(dt)
     if dt_bias is not None:
-        x = x + dt_bias.float().reshape(HV, K)
+        x = x + dt_bias.to(dt).reshape(HV, K)
     if lower_bound is not None:
         if A_log is not None:
-            x = x * A_log.float().exp().reshape(HV, 1)
+            x = x * A_log.to(dt).exp().reshape(HV, 1)
         return lower_bound * torch.sigmoid(x)
-    a = A_log.float().exp().reshape(HV, 1) if A_log is not None else math.e
+    a = A_log.to(dt).exp().reshape(HV, 1) if A_log is not None else math.e
     return -a * F.softplus(x)
 
 
@@ -546,6 +548,33 @@ def gated_delta_rule_grads(
     if dht is not None:
         loss = loss + (ht * dht.to(dtype)).sum()
     names = list(leaves)
+    grads = torch.autograd.grad(loss, [leaves[n] for n in names], allow_unused=True)
+    out = dict.fromkeys(('dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0', 'dA_log', 'ddt_bias'))
+    out.update(dict(zip(names, grads)))
+    return out
+
+
+def kda_grads(q, k, v, g, beta, do, dht=None, scale=None, initial_state=None, cu_seqlens=None,
+              use_qk_l2norm_in_kernel=False, use_gate_in_kernel=False, A_log=None, dt_bias=None, lower_bound=None,
+              use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, state_v_first=False, dtype=torch.float64):
+    """Gradients of  sum(o * do) + sum(ht * dht)  of the KDA operator with respect to q, k, v, g, beta, the initial state
+    and (with the gate activation) A_log and dt_bias, by reverse-mode differentiation of ``recurrent_kda``: what the
+    reference's tests take as the truth for chunk_kda's backward pass (tests/ops/test_kda.py, autograd through
+    fla/ops/kda/naive.py).  Returns a dict with the keys dq, dk, dv, dg, dbeta, dh0, dA_log, ddt_bias."""
+    leaves = {}
+    gate = dict(dA_log=A_log, ddt_bias=dt_bias) if use_gate_in_kernel else {}
+    for name, x in dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=initial_state, **gate).items():
+        leaves[name] = None if x is None else x.detach().to(dtype).clone().requires_grad_(True)
+    o, ht = recurrent_kda(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dg'], leaves['dbeta'], scale=scale,
+                          initial_state=leaves['dh0'], output_final_state=dht is not None, cu_seqlens=cu_seqlens,
+                          use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel, use_gate_in_kernel=use_gate_in_kernel,
+                          A_log=leaves.get('dA_log'), dt_bias=leaves.get('ddt_bias'), lower_bound=lower_bound,
+                          use_beta_sigmoid_in_kernel=use_beta_sigmoid_in_kernel, allow_neg_eigval=allow_neg_eigval,
+                          state_v_first=state_v_first, dtype=dtype)
+    loss = (o * do.to(dtype)).sum()
+    if dht is not None:
+        loss = loss + (ht * dht.to(dtype)).sum()
+    names = [n for n, x in leaves.items() if x is not None]
     grads = torch.autograd.grad(loss, [leaves[n] for n in names], allow_unused=True)
     out = dict.fromkeys(('dq', 'dk', 'dv', 'dg', 'dbeta', 'dh0', 'dA_log', 'ddt_bias'))
     out.update(dict(zip(names, grads)))

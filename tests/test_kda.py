@@ -435,3 +435,134 @@ def test_chunk_kda_random(seed):
         ht = ht.transpose(-1, -2)
     bar = 0.005 if T >= 64 else 0.01
     assert O.get_err_ratio(ref_o, o.float().cpu()) < bar and O.get_err_ratio(ref_ht, ht.cpu()) < bar
+
+
+# --------------------------------------------------------------------------------------------
+# backward of chunk_kda (gdn_chunk_kda_bwd) against the oracle's gradients
+# --------------------------------------------------------------------------------------------
+# (tests/ops/test_kda.py:651-661 of the reference; its 0.003 for dA only warns there, :659: held to 0.01 here)
+GRAD_TOL = dict(dq=0.008, dk=0.008, dv=0.008, dg=0.02, dbeta=0.02, dh0=0.008, dA_log=0.01, ddt_bias=0.008)
+
+
+def _kda_grads_gpu(q, k, v, g, beta, h0, A_log, dt_bias, do, dht, cu=None, **kw):
+    from fla_hip.ops.kda import chunk_kda
+    leaves = {n: (None if x is None else x.cuda().requires_grad_(True))
+              for n, x in dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=h0, dA_log=A_log, ddt_bias=dt_bias).items()}
+    cu_t = None if cu is None else torch.tensor(cu, dtype=kw.pop('idx_dtype', torch.int64), device='cuda')
+    o, ht = chunk_kda(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dg'], leaves['dbeta'], initial_state=leaves['dh0'],
+                      output_final_state=True, A_log=leaves['dA_log'], dt_bias=leaves['ddt_bias'], cu_seqlens=cu_t, **kw)
+    ((o.float() * do.cuda().float()).sum() + (ht * dht.cuda()).sum()).backward()
+    return o, ht, {n: (None if x is None else x.grad) for n, x in leaves.items()}
+
+
+def _compare_grads(ref, got, tol=GRAD_TOL):
+    for n, r in ref.items():
+        if r is None:
+            continue
+        x = got[n].detach().float().cpu()
+        assert x.shape == r.shape, f'{n}: shape {tuple(x.shape)} vs {tuple(r.shape)}'
+        assert not torch.isnan(x).any(), f'{n}: NaN'
+        if O.get_abs_err(r, x) <= 1e-6:            # (fla/utils/_testing.py:28-34: gradients that vanish)
+            continue
+        e = O.get_err_ratio(r, x)
+        assert e <= tol[n], f'{n}: rel-rmse {e:.3e} > {tol[n]}'
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,D,scale,gate_div,mask_p,l2,gate_in_kernel,dtype,safe_gate', [
+    (1, 63, 1, 1, 64, 1, 1, 0, False, False, torch.float16, True),          # the reference's matrix (shorter where it is long)
+    (2, 500, 3, 3, 60, 1, 1, 0, False, False, torch.float16, True),
+    (2, 300, 3, 3, 64, 0.1, 1, 0.5, False, False, torch.float16, False),
+    (2, 256, 4, 4, 100, 1, 0.1, 0, False, False, torch.float16, False),
+    (2, 256, 4, 4, 128, 0.1, 1, 0, False, False, torch.float16, True),
+    (2, 256, 4, 4, 128, 0.1, 1, 0, True, False, torch.float16, True),
+    (2, 300, 4, 4, 128, 0.1, 10, 0, False, True, torch.float16, False),
+    (2, 256, 8, 8, 64, 0.1, 1, 0, False, True, torch.float16, True),
+    (2, 256, 2, 4, 64, 0.1, 1, 0, False, False, torch.float16, False),
+    (2, 256, 2, 8, 64, 0.1, 1, 0, False, True, torch.float16, False),
+    (2, 256, 4, 8, 128, 0.1, 1, 0, True, True, torch.float16, False),
+    (2, 256, 2, 4, 64, 0.1, 1, 0, True, True, torch.bfloat16, True),
+    (2, 256, 2, 4, 64, 0.1, 1, 0, False, True, torch.bfloat16, False),
+    (2, 256, 2, 8, 128, 0.1, 1, 0, True, True, torch.bfloat16, False),
+    (3, 100, 12, 24, 128, 0.1, 4.0, 0, False, False, torch.bfloat16, False),     # 72 runs: the scans take 64 value columns per workgroup
+    (2, 70, 80, 80, 128, 0.1, 4.0, 0, False, False, torch.bfloat16, False),      # 160 runs: all 128
+])
+def test_chunk_kda_backward(B, T, H, HV, D, scale, gate_div, mask_p, l2, gate_in_kernel, dtype, safe_gate):
+    q, k, v, g, beta, h0, A_log, dt_bias = _chunk_inputs(B, T, H, HV, D, gate_div, mask_p, gate_in_kernel, safe_gate, dtype)
+    lower_bound = -5.0 if safe_gate else None
+    if not l2:
+        q, k = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    if gate_in_kernel:
+        g = g.to(dtype)
+    gen = torch.Generator().manual_seed(43)
+    do = torch.randn(B, T, HV, D, generator=gen).to(dtype)
+    dht = torch.randn(B, HV, D, D, generator=gen)
+    kw = dict(scale=scale, use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel, lower_bound=lower_bound)
+    ref = O.kda_grads(q, k, v, g, beta, do, dht, initial_state=h0, A_log=A_log, dt_bias=dt_bias, dtype=torch.float32, **kw)
+    o, ht, got = _kda_grads_gpu(q, k, v, g, beta, h0, A_log, dt_bias, do, dht, safe_gate=safe_gate, **kw)
+    _compare_grads(ref, got)
+    for n, x in dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=h0, dA_log=A_log, ddt_bias=dt_bias).items():
+        if x is not None:
+            assert got[n].dtype == x.dtype and got[n].shape == x.shape, n
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('H,D,mask_p,cu,gate_in_kernel,safe_gate,idx_dtype', [
+    (4, 60, 0.1, [0, 15], True, False, torch.int32),
+    (4, 64, 0.9, [0, 256, 500, 1000], True, False, torch.int64),
+    (4, 128, 0.5, [0, 256, 500, 1000], False, False, torch.int32),
+    (4, 100, 0, [0, 15, 100, 300, 1200, 2000], True, False, torch.int64),
+    (2, 128, 0, [0, 1, 65, 65, 200], False, True, torch.int64),
+])
+def test_chunk_kda_backward_packed(H, D, mask_p, cu, gate_in_kernel, safe_gate, idx_dtype):
+    T, N = cu[-1], len(cu) - 1
+    q, k, v, g, beta, _, A_log, dt_bias = _chunk_inputs(1, T, H, H, D, 1.0, mask_p, gate_in_kernel, safe_gate, torch.bfloat16)
+    q, k = F.normalize(q.float(), p=2, dim=-1).bfloat16(), F.normalize(k.float(), p=2, dim=-1).bfloat16()
+    lower_bound = -5.0 if safe_gate else None
+    gen = torch.Generator().manual_seed(44)
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    do = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    dht = torch.rand(N, H, D, D, generator=gen)
+    kw = dict(use_gate_in_kernel=gate_in_kernel, lower_bound=lower_bound)
+    ref = O.kda_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, A_log=A_log, dt_bias=dt_bias, dtype=torch.float32, **kw)
+    _, _, got = _kda_grads_gpu(q, k, v, g, beta, h0, A_log, dt_bias, do, dht, cu=cu, idx_dtype=idx_dtype, safe_gate=safe_gate, **kw)
+    _compare_grads(ref, got)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('what', ['v_first', 'beta_sigmoid', 'beta_sigmoid_neg', 'wide_v', 'no_h0', 'strong_decay', 'outside_tokens'])
+def test_chunk_kda_backward_options(what):
+    B, T, H, HV, D = 2, 200, 2, 4, 64
+    V = 200 if what == 'wide_v' else D
+    q, k, v, g, beta, h0, _, _ = _chunk_inputs(B, T, H, HV, D, 0.02 if what == 'strong_decay' else 1.0, 0, False, False, torch.bfloat16, seed=5, V=V)
+    q, k = F.normalize(q.float(), p=2, dim=-1).bfloat16(), F.normalize(k.float(), p=2, dim=-1).bfloat16()
+    gen = torch.Generator().manual_seed(45)
+    do = torch.randn(B, T, HV, V, generator=gen).bfloat16()
+    kw, cu = {}, None
+    if what == 'v_first':
+        h0 = h0.transpose(-1, -2).contiguous()
+        kw = dict(state_v_first=True)
+    if what.startswith('beta_sigmoid'):
+        beta = torch.randn(B, T, HV, generator=gen)
+        kw = dict(use_beta_sigmoid_in_kernel=True, allow_neg_eigval=what.endswith('neg'))
+    if what == 'no_h0':
+        h0 = None
+    dht = torch.randn(B, HV, V, D, generator=gen) if what == 'v_first' else torch.randn(B, HV, D, V, generator=gen)
+    if what == 'outside_tokens':
+        # a packed tensor whose sequences leave tokens out at both ends: those get zero gradients
+        cu = [10, 90, 180]
+        q, k, v, g, beta, do = (x[:1] for x in (q, k, v, g, beta, do))
+        sl = slice(cu[0], cu[-1])
+        ref = O.kda_grads(q[:, sl], k[:, sl], v[:, sl], g[:, sl], beta[:, sl], do[:, sl], dht, initial_state=h0,
+                          cu_seqlens=[c - cu[0] for c in cu], dtype=torch.float32)
+        _, _, got = _kda_grads_gpu(q, k, v, g, beta, h0, None, None, do, dht, cu=cu)
+        for n in ('dq', 'dk', 'dv', 'dg', 'dbeta'):
+            x = got[n]
+            assert not x[:, :cu[0]].any() and not x[:, cu[-1]:].any(), f'{n}: tokens outside every sequence must get zero'
+            got[n] = x[:, sl]
+        _compare_grads(ref, got)
+        return
+    ref = O.kda_grads(q, k, v, g, beta, do, dht, initial_state=h0, dtype=torch.float32, **kw)
+    _, _, got = _kda_grads_gpu(q, k, v, g, beta, h0, None, None, do, dht, **kw)
+    _compare_grads(ref, got)
+

@@ -408,3 +408,48 @@ def test_comba_grads_match_finite_differences(kw):
         fd = (loss({**inputs, name: x + eps * d}) - loss({**inputs, name: x - eps * d})) / (2 * eps)
         an = float((grads[name] * d).sum())
         assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), f'{name}: finite difference {fd} vs gradient {an}'
+
+
+@pytest.mark.parametrize('kw', [
+    dict(),
+    dict(use_qk_l2norm_in_kernel=True, use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True),
+    dict(use_gate_in_kernel=True),
+    dict(use_gate_in_kernel=True, lower_bound=-3.0),
+    dict(use_gate_in_kernel=True, lower_bound=-3.0, no_A=True),
+    dict(cu_seqlens=[0, 4, 11], state_v_first=True),
+])
+def test_kda_grads_match_finite_differences(kw):
+    """``kda_grads`` (reverse mode through the recurrence) against central differences of the recurrence itself, along a
+    random direction in every input and gate parameter."""
+    kw = dict(kw)
+    no_A = kw.pop('no_A', False)
+    B, T, H, HV, K, V = (1, 11, 2, 4, 5, 3) if 'cu_seqlens' in kw else (2, 8, 2, 4, 5, 3)
+    gen = torch.Generator().manual_seed(13)
+    f64 = dict(generator=gen, dtype=torch.float64)
+    q, k = torch.randn(B, T, H, K, **f64) * 1.3, torch.randn(B, T, H, K, **f64) * 0.6
+    v = torch.randn(B, T, HV, V, **f64)
+    gate = kw.get('use_gate_in_kernel', False)
+    g = torch.randn(B, T, HV, K, **f64) if gate else F.logsigmoid(torch.randn(B, T, HV, K, **f64))
+    beta = torch.randn(B, T, HV, **f64) if kw.get('use_beta_sigmoid_in_kernel') else torch.rand(B, T, HV, **f64)
+    h0 = torch.randn(2, HV, V, K, **f64) * 0.5 if kw.get('state_v_first') else torch.randn(2, HV, K, V, **f64) * 0.5
+    do, dht = torch.randn(B, T, HV, V, **f64), torch.randn(*h0.shape, **f64)
+    inputs = dict(dq=q, dk=k, dv=v, dg=g, dbeta=beta, dh0=h0)
+    if gate:
+        if not no_A:
+            inputs['dA_log'] = torch.randn(HV, **f64) * 0.3
+        inputs['ddt_bias'] = torch.randn(HV * K, **f64) * 0.3
+
+    grads = O.kda_grads(q, k, v, g, beta, do, dht, scale=0.4, initial_state=h0, A_log=inputs.get('dA_log'),
+                        dt_bias=inputs.get('ddt_bias'), dtype=torch.float64, **kw)
+
+    def loss(a):
+        o, ht = O.recurrent_kda(a['dq'], a['dk'], a['dv'], a['dg'], a['dbeta'], scale=0.4, initial_state=a['dh0'],
+                                output_final_state=True, A_log=a.get('dA_log'), dt_bias=a.get('ddt_bias'), dtype=torch.float64, **kw)
+        return float((o * do).sum() + (ht * dht).sum())
+    eps = 1e-6
+    for name, x in inputs.items():
+        d = torch.randn(x.shape, **f64)
+        fd = (loss({**inputs, name: x + eps * d}) - loss({**inputs, name: x - eps * d})) / (2 * eps)
+        an = float((grads[name] * d).sum())
+        assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), f'{name}: finite difference {fd} vs gradient {an}'
+
