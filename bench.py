@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|layer_train|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|train_chunk_kda|train_chunk_comba|layer_train|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -307,29 +307,48 @@ def bench_train(w, steps, warmup, device):
                 tokens_per_s=round(w['B'] * w['T'] / per_call, 1))
 
 
-def bench_kda(steps, warmup, device):
-    """Chunked prefill of the sibling KDA operator (a decay per key feature) on one of the published GDN shapes."""
+def _train_step(op, leaves, do, **kw):
+    def step():
+        o, _ = op(*leaves, **kw)
+        o.backward(do)
+        for x in leaves:
+            x.grad = None
+    return step
+
+
+def bench_kda(steps, warmup, device, train=False):
+    """Chunked prefill of the sibling KDA operator (a decay per key feature) on one of the published GDN shapes; with
+    ``train`` a training step (forward and backward through autograd)."""
     from fla_hip.ops.kda import chunk_kda
     B, T, H, D = 1, 8192, 96, 128
     gen = torch.Generator().manual_seed(42)
     q, k, v = (torch.randn(B, T, H, D, generator=gen).bfloat16().to(device) for _ in range(3))
     g = (F.logsigmoid(torch.randn(B, T, H, D, generator=gen)) / 4).to(device)
     beta = torch.sigmoid(torch.randn(B, T, H, generator=gen)).to(device)
-    per_call, _ = _time_calls(lambda: chunk_kda(q, k, v, g, beta, use_qk_l2norm_in_kernel=True), steps, warmup)
-    return dict(workload=f'chunk_kda forward B={B} T={T} H={H} K=V={D} bf16, fp32 log decays per key feature, in-kernel l2 norm',
+    call = lambda: chunk_kda(q, k, v, g, beta, use_qk_l2norm_in_kernel=True)
+    if train:
+        leaves = [x.requires_grad_(True) for x in (q, k, v, g, beta)]
+        call = _train_step(chunk_kda, leaves, torch.randn_like(v), use_qk_l2norm_in_kernel=True)
+    per_call, _ = _time_calls(call, steps, warmup)
+    return dict(workload=f'chunk_kda {"forward and backward" if train else "forward"} B={B} T={T} H={H} K=V={D} bf16, fp32 log decays per key feature, in-kernel l2 norm',
                 ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
 
 
-def bench_comba(steps, warmup, device):
-    """Chunked prefill of the sibling comba operator (a second key for the prediction) on one of the published GDN shapes."""
+def bench_comba(steps, warmup, device, train=False):
+    """Chunked prefill of the sibling comba operator (a second key for the prediction) on one of the published GDN shapes; with
+    ``train`` a training step (forward and backward through autograd)."""
     from fla_hip.ops.comba import chunk_comba
     B, T, H, D = 1, 8192, 96, 128
     gen = torch.Generator().manual_seed(42)
     q, k, v, p = (torch.randn(B, T, H, D, generator=gen).bfloat16().to(device) for _ in range(4))
     g = F.logsigmoid(torch.randn(B, T, H, generator=gen)).to(device)
     beta = torch.sigmoid(torch.randn(B, T, H, generator=gen)).to(device)
-    per_call, _ = _time_calls(lambda: chunk_comba(q, k, v, p, g, beta, use_qk_l2norm_in_kernel=True), steps, warmup)
-    return dict(workload=f'chunk_comba forward B={B} T={T} H={H} K=V={D} bf16, fp32 log decays, in-kernel l2 norm of q, k, p',
+    call = lambda: chunk_comba(q, k, v, p, g, beta, use_qk_l2norm_in_kernel=True)
+    if train:
+        leaves = [x.requires_grad_(True) for x in (q, k, v, p, g, beta)]
+        call = _train_step(chunk_comba, leaves, torch.randn_like(v), use_qk_l2norm_in_kernel=True)
+    per_call, _ = _time_calls(call, steps, warmup)
+    return dict(workload=f'chunk_comba {"forward and backward" if train else "forward"} B={B} T={T} H={H} K=V={D} bf16, fp32 log decays, in-kernel l2 norm of q, k, p',
                 ms_per_step=round(per_call * 1e3, 4), tokens_per_s=round(B * T / per_call, 1))
 
 
@@ -568,7 +587,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
-    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'chunk_comba', 'layer_train', 'layer_steps', 'calib_copy', 'calib_rmw'])
+    ap.add_argument('--workload', default='prefill', choices=list(WORKLOADS) + list(PUBLISHED) + ['train_' + n for n in PUBLISHED] + ['chunk_kda', 'chunk_comba', 'train_chunk_kda', 'train_chunk_comba', 'layer_train', 'layer_steps', 'calib_copy', 'calib_rmw'])
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-extra', action='store_true', help='skip the other workloads')
     ap.add_argument('--no-spin-up', action='store_true', help='no untimed load in front of the warm-up steps (clocks as after an idle period)')
@@ -597,6 +616,12 @@ def main():
         return
     for key, val in WORKLOADS.items():
         val['key'] = key
+    if args.workload in ('train_chunk_kda', 'train_chunk_comba'):
+        r = (bench_kda if args.workload.endswith('kda') else bench_comba)(args.steps, args.warmup, device, train=True)
+        print(json.dumps(dict(metric=args.workload[len('train_'):] + '_fwd_bwd_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s',
+                              higher_is_better=True, n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=r['ms_per_step'],
+                              dtype='bf16', data='synthetic', config=dict(workload=r['workload'], chunk_size=64))))
+        return
     if args.workload == 'chunk_kda':
         r = bench_kda(args.steps, args.warmup, device)
         print(json.dumps(dict(metric='kda_chunk_prefill_tokens_per_s', value=r['tokens_per_s'], unit='tokens/s', higher_is_better=True,
@@ -658,7 +683,11 @@ def main():
             extra[name + '_fwd_bwd'] = dict(ms=bench_train(dict(ww, key=name), *quarter, device)['ms_per_step'])
             torch.cuda.empty_cache()
         extra['chunk_kda_b1_t8192_h96_d128'] = dict(ms=bench_kda(*quarter, device)['ms_per_step'])
+        extra['chunk_kda_b1_t8192_h96_d128_fwd_bwd'] = dict(ms=bench_kda(*quarter, device, train=True)['ms_per_step'])
+        torch.cuda.empty_cache()
         extra['chunk_comba_b1_t8192_h96_d128'] = dict(ms=bench_comba(*quarter, device)['ms_per_step'])
+        extra['chunk_comba_b1_t8192_h96_d128_fwd_bwd'] = dict(ms=bench_comba(*quarter, device, train=True)['ms_per_step'])
+        torch.cuda.empty_cache()
         extra['layer_train_t32768'] = dict(ms=bench_layer_train(max(5, args.steps // 10), 3, device)['ms_per_step'])
         torch.cuda.empty_cache()
         for key, r in bench_layer_steps(args.steps, args.warmup, device, False).items():

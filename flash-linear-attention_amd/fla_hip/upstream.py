@@ -8,8 +8,8 @@ whole operator and ``fla/modules/backends/triton_ascend`` for module functions).
 Upstream's ``@dispatch`` then offers every call of ``chunk_gated_delta_rule``, ``causal_conv1d_fwd``,
 ``causal_conv1d_update_states``, ``causal_conv1d_update``, ``layer_norm_gated_fwd``, ``chunk_kda`` and ``fused_recurrent_kda_fwd``
 (the KDA operator's token recurrence, ``fla/ops/kda/fused_recurrent.py:236``) to the verifier below first;
-a rejected call (other device, gradients needed, a shape outside the kernels) falls through to upstream's own
-implementation.  The classes are built on whatever ``BaseBackend`` they are given, so the same code serves this
+a rejected call (other device, a shape outside the kernels, gradients through an entry point that is forward only here) falls
+through to upstream's own implementation.  The classes are built on whatever ``BaseBackend`` they are given, so the same code serves this
 package's mirror of the registry (used by the tests)."""
 from __future__ import annotations
 
@@ -152,7 +152,7 @@ def make_backends(BaseBackend):
 
 
 def make_kda_backend(BaseBackend):
-    """Backend for the 'kda' registry: the token recurrence and the chunked prefill (forward; training stays upstream)."""
+    """Backend for the 'kda' registry: the token recurrence (inference calls) and the chunked operator (forward and backward)."""
 
     class HipGfx950KDABackend(BaseBackend):
         backend_type = 'hip_gfx950'
@@ -183,8 +183,7 @@ def make_kda_backend(BaseBackend):
                 return False, 'not a gfx950 device'
             if cp_context is not None or return_intermediate_states:
                 return False, 'context parallelism and intermediate states are not supported'
-            if _needs_grad(q, k, v, g, beta, kwargs.get('initial_state'), kwargs.get('A_log'), kwargs.get('dt_bias')):
-                return False, 'forward only: a tensor requires grad'
+            # (calls that need gradients are taken too: chunk_kda here is differentiable in every input upstream's is)
             if q.dtype not in (torch.bfloat16, torch.float16):      # (fp32 operands: upstream's tf32 path, as above)
                 return False, f'dtype {q.dtype}'
             if k.shape[-1] > 128:

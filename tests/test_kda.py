@@ -228,7 +228,10 @@ def test_upstream_kda_backend_takes_gpu_inference_calls_and_leaves_the_rest():
                       use_qk_l2norm_in_kernel=True)
     assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.01 and O.get_err_ratio(ref_ht, ht.cpu()) < 0.01
     assert chunk_kda(q, k, v, g, beta)[0] == 'default'                                                        # CPU stays upstream
-    assert chunk_kda(dq.bfloat16().requires_grad_(), dk.bfloat16(), dv.bfloat16(), dg, db)[0] == 'default'    # training stays upstream
+    qg = dq.bfloat16().requires_grad_()
+    o2, _ = chunk_kda(qg, dk.bfloat16(), dv.bfloat16(), dg, db, initial_state=dh, use_qk_l2norm_in_kernel=True)      # training calls too
+    o2.float().square().sum().backward()
+    assert torch.equal(o2, o) and qg.grad is not None and bool(qg.grad.float().abs().sum() > 0)
     wide = torch.zeros(1, 150, 2, 192, device='cuda', dtype=torch.bfloat16)
     assert chunk_kda(wide, wide, dv.bfloat16(), torch.zeros(1, 150, 4, 192, device='cuda'), db)[0] == 'default'
 
