@@ -1272,7 +1272,7 @@ extern "C" int gdn_chunk_kda_bwd(
     KdaParams kp;
     kp.q = q; kp.k = k; kp.v = v; kp.g = g; kp.beta = beta; kp.pk = nullptr; kp.gs = nullptr;
     kp.A_log = nullptr; kp.gk_bias = nullptr; kp.gk_lower = 0.f; kp.gk_act = 0;
-    kp.h0 = nullptr; kp.ht = nullptr; kp.o = nullptr;
+    kp.h0 = nullptr; kp.ht = nullptr; kp.o = nullptr; kp.hs = nullptr;
     kp.cu_seqlens = cu_seqlens; kp.chunk_table = chunk_table; kp.chunk_offsets = chunk_offsets;
     kp.ws = KdaWs{p.ws.Wm, p.ws.Vn, p.ws.QG, p.ws.KG, p.ws.Pm, p.ws.EGL, p.ws.Am, p.ws.Gk};
     kp.T = T; kp.H = (int)H; kp.HV = (int)HV; kp.N = N; kp.NT = p.NT;

@@ -26,6 +26,7 @@ struct KdaParams {
     const void* pk; const void* gs;                                             // comba: the second key, the log decay per token and head
     const float* A_log; const float* gk_bias; float gk_lower; int gk_act;      // gate activation, as in the token recurrence
     const float* h0; float* ht; void* o;
+    void* hs;                           // the state in front of every chunk [num_chunks][HV][128][128] in the operand type, or NULL
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     KdaWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;

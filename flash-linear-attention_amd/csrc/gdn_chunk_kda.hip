@@ -537,8 +537,11 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-            for (int b = 0; b < NB; ++b)
-                *(V4*)(sS + (16 * (2 * w + a2) + c16) * PV + 16 * b + 4 * g) = pack4<T>(S[a2][b]);
+            for (int b = 0; b < NB; ++b) {
+                const V4 s4 = pack4<T>(S[a2][b]);
+                *(V4*)(sS + (16 * (2 * w + a2) + c16) * PV + 16 * b + 4 * g) = s4;
+                if (p.hs) *(V4*)((T*)p.hs + (((sq.cbase + ic) * p.HV + hv) * BD + 16 * (2 * w + a2) + c16) * BD + vcol0 + 16 * b + 4 * g) = s4;
+            }
         lds_barrier();
         if (ic + 1 < sq.nc) fetch(ic + 1);
         f32x4 oacc[NB];
@@ -668,17 +671,17 @@ extern "C" size_t gdn_chunk_kda_workspace_bytes(int64_t num_chunks, int64_t HV) 
     return gdn::kda_ws_layout(num_chunks * HV, nullptr, nullptr);
 }
 
-extern "C" int gdn_chunk_kda_fwd(
+static int kda_fwd_entry(
+    const char* who,
     const void* q, const void* k, const void* v, const float* g, const void* beta,
     const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
-    const float* h0, float* ht, void* o,
+    const float* h0, float* ht, void* o, void* states,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
     void* workspace, size_t workspace_bytes,
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
     using namespace gdn;
-    const char* who = "gdn_chunk_kda_fwd";
     const uint32_t known = GDN_FLAG_CU_INT32 | GDN_FLAG_QK_L2NORM | GDN_FLAG_BETA_SIGMOID | GDN_FLAG_NEG_EIGVAL;
     if (int rc = check_shapes(who, B, T, H, HV, K, V, N, num_chunks, cu_seqlens, chunk_table, chunk_offsets, qkv_dtype, flags, known)) return rc;
     GDN_CHECK_ARG(gate_mode >= 0 && gate_mode <= 2, GDN_ERR_INVALID, "%s: gate_mode must be 0, 1 or 2", who);
@@ -690,7 +693,7 @@ extern "C" int gdn_chunk_kda_fwd(
         return GDN_OK;
     }
     GDN_CHECK_ARG(q && k && v && g && beta && o, GDN_ERR_INVALID, "%s: q, k, v, g, beta, o must not be NULL", who);
-    for (const void* x : {q, k, v, (const void*)g, (const void*)h0, (const void*)ht, (const void*)o})
+    for (const void* x : {q, k, v, (const void*)g, (const void*)h0, (const void*)ht, (const void*)o, (const void*)states})
         GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
     GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
     KdaParams p;
@@ -698,11 +701,39 @@ extern "C" int gdn_chunk_kda_fwd(
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.pk = nullptr; p.gs = nullptr; p.A_log = A_log; p.gk_bias = dt_bias; p.gk_lower = lower_bound; p.gk_act = gate_mode;
-    p.h0 = h0; p.ht = ht; p.o = o;
+    p.h0 = h0; p.ht = ht; p.o = o; p.hs = states;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_kda<bf16_t>(p, num_chunks, s) : launch_kda<f16_t>(p, num_chunks, s);
+}
+
+extern "C" int gdn_chunk_kda_fwd(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    return kda_fwd_entry("gdn_chunk_kda_fwd", q, k, v, g, beta, A_log, dt_bias, lower_bound, gate_mode, h0, ht, o, nullptr, cu_seqlens, chunk_table,
+                         chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks, scale, qkv_dtype, gb_dtype, flags, stream);
+}
+
+// ... and the state in front of every chunk, states [num_chunks][HV][K][V] in qkv_dtype (the reference's h with return_intermediate_states)
+extern "C" int gdn_chunk_kda_fwd_states(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o, void* states,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    GDN_CHECK_ARG(states || T == 0 || num_chunks == 0, GDN_ERR_INVALID, "gdn_chunk_kda_fwd_states: states must not be NULL");
+    return kda_fwd_entry("gdn_chunk_kda_fwd_states", q, k, v, g, beta, A_log, dt_bias, lower_bound, gate_mode, h0, ht, o, states, cu_seqlens, chunk_table,
+                         chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks, scale, qkv_dtype, gb_dtype, flags, stream);
 }
 
 extern "C" int gdn_chunk_comba_fwd(
@@ -734,7 +765,7 @@ extern "C" int gdn_chunk_comba_fwd(
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.pk = p_key; p.gs = g;
     p.A_log = nullptr; p.gk_bias = nullptr; p.gk_lower = 0.f; p.gk_act = 0;
-    p.h0 = h0; p.ht = ht; p.o = o;
+    p.h0 = h0; p.ht = ht; p.o = o; p.hs = nullptr;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;

@@ -131,6 +131,7 @@ SIGNATURES['gdn_chunk_kda_fwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_chunk_kda_fwd_states'] = (c_int, SIGNATURES['gdn_chunk_kda_fwd'][1][:12] + [c_void_p] + SIGNATURES['gdn_chunk_kda_fwd'][1][12:])
 SIGNATURES['gdn_chunk_comba_fwd'] = (c_int, [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # q k v p g beta
     c_void_p, c_void_p, c_void_p,                      # h0 ht o

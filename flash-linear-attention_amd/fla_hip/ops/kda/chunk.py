@@ -34,9 +34,11 @@ def _pad_last(x: torch.Tensor, size: int) -> torch.Tensor:
 
 def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first=False, cu_seqlens=None,
                   cu_seqlens_cpu=None, A_log=None, dt_bias=None, lower_bound=None, gate_mode=0,
-                  use_qk_l2norm_in_kernel=False, use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False):
+                  use_qk_l2norm_in_kernel=False, use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, return_states=False):
     """Returns ``(o [B,T,HV,V] in q's dtype, final_state fp32 or None)``; ``gate_mode`` 0: g is the log decay,
-    1: ``-exp(A_log) softplus(g + dt_bias)``, 2: ``lower_bound sigmoid(exp(A_log) (g + dt_bias))``."""
+    1: ``-exp(A_log) softplus(g + dt_bias)``, 2: ``lower_bound sigmoid(exp(A_log) (g + dt_bias))``.  With ``return_states``
+    a third result: the state in front of every chunk, ``[B, NT, HV, K, V]`` (``[1, chunks of all sequences, ...]`` for packed
+    input; ``[..., V, K]`` with ``state_v_first``) in the kernels' operand dtype."""
     dev = require_gpu(q, k, v, g, beta)
     check_operand_shapes(q, k, v, beta=beta, gk=g)
     B, T, H, K = k.shape
@@ -54,11 +56,11 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
                 h2 = F.pad(initial_state, (0, 0, 0, nb * _DIM - V)).reshape(N, HV * nb, _DIM, K)
             else:
                 h2 = _pad_last(initial_state, nb * _DIM).reshape(N, HV, K, nb, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV * nb, K, _DIM)
-        o2, ht2 = chunk_kda_fwd(
+        o2, ht2, *hs2 = chunk_kda_fwd(
             q, k, v2, g.repeat_interleave(nb, dim=2), beta.repeat_interleave(nb, dim=2), scale, h2, output_final_state,
             state_v_first, cu_seqlens, cu_seqlens_cpu, None if A_log is None else A_log.reshape(-1).repeat_interleave(nb),
             None if dt_bias is None else dt_bias.reshape(HV, K).repeat_interleave(nb, dim=0), lower_bound, gate_mode,
-            use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval)
+            use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval, return_states)
         o = o2.reshape(B, T, HV, nb * _DIM)[..., :V].contiguous()
         ht = None
         if ht2 is not None:
@@ -67,6 +69,14 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
             else:
                 ht = ht2.reshape(N, HV, nb, K, _DIM).permute(0, 1, 3, 2, 4).reshape(N, HV, K, nb * _DIM)[..., :V]
             ht = ht.contiguous()
+        if return_states:
+            hs = hs2[0]
+            B1, NC = hs.shape[:2]
+            if state_v_first:
+                hs = hs.reshape(B1, NC, HV, nb * _DIM, K)[:, :, :, :V]
+            else:
+                hs = hs.reshape(B1, NC, HV, nb, K, _DIM).permute(0, 1, 2, 4, 3, 5).reshape(B1, NC, HV, K, nb * _DIM)[..., :V]
+            return o, ht, hs.contiguous()
         return o, ht
 
     out_dtype = q.dtype
@@ -117,9 +127,11 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
     lib = _lib.load()
     ws_bytes = lib.gdn_chunk_kda_workspace_bytes(num_chunks, HV)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    _lib.check(lib.gdn_chunk_kda_fwd(
+    hs = torch.empty(num_chunks, HV, _DIM, _DIM, dtype=work, device=dev) if return_states else None
+    entry, states = (lib.gdn_chunk_kda_fwd_states, (ptr(hs),)) if return_states else (lib.gdn_chunk_kda_fwd, ())
+    _lib.check(entry(
         ptr(qw), ptr(kw), ptr(vw), ptr(gw), ptr(bw), ptr(A_log), ptr(dt_bias),
-        0.0 if lower_bound is None else float(lower_bound), gate_mode, ptr(h0), ptr(ht), ptr(o),
+        0.0 if lower_bound is None else float(lower_bound), gate_mode, ptr(h0), ptr(ht), ptr(o), *states,
         ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
         B, T, H, HV, _DIM, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
         current_stream_ptr(dev)))
@@ -127,6 +139,10 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
     if ht is not None:
         ht = ht[..., :K, :V]
         ht = (ht.transpose(-1, -2) if state_v_first else ht).contiguous()
+    if return_states:
+        hs = hs[..., :K, :V]
+        hs = (hs.transpose(-1, -2) if state_v_first else hs).contiguous()
+        return o, ht, hs.reshape(B if cu_seqlens is None else 1, -1, *hs.shape[1:]).to(out_dtype)
     return o, ht
 
 
@@ -335,7 +351,8 @@ def chunk_kda(
         safe_gate: accepted; the kernels form the intra-chunk decays pair by pair inside blocks of 16 rows whatever the
             gate's range, so it changes nothing here.  disable_recompute: accepted; the backward pass always computes the
             forward's intermediates again.
-        return_intermediate_states, cp_context: not part of this build.
+        return_intermediate_states: in inference mode a third result, the state in front of every chunk
+            ``[B, NT, HV, K, V]`` in q's dtype (fla/ops/kda/chunk.py:98-100).  cp_context: not part of this build.
         cu_seqlens: ``[N + 1]`` boundaries of packed sequences (then ``B == 1``).
 
     Returns:
@@ -343,8 +360,6 @@ def chunk_kda(
     """
     if cp_context is not None:
         raise NotImplementedError('context parallelism (cp_context) is outside this single-GPU build')
-    if return_intermediate_states:
-        raise NotImplementedError('return_intermediate_states: the per-chunk states never reach memory here')
     if 'transpose_state_layout' in kwargs:
         state_v_first = kwargs.pop('transpose_state_layout')
     if cu_seqlens is not None:
@@ -378,6 +393,13 @@ def chunk_kda(
         A_log = dt_bias = None
     if scale is None:
         scale = k.shape[-1] ** -0.5
+    if return_intermediate_states:
+        # (the reference's conditions, fla/ops/kda/chunk.py:98-100)
+        assert torch.is_inference_mode_enabled(), 'return_intermediate_states is only allowed in inference mode'
+        assert disable_recompute is False, 'return_intermediate_states must be used with disable_recompute=False'
+        return chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, state_v_first, cu_seqlens,
+                             cu_seqlens_cpu, A_log, dt_bias, lower_bound, gate_mode, use_qk_l2norm_in_kernel,
+                             use_beta_sigmoid_in_kernel, allow_neg_eigval, return_states=True)
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, g, beta, A_log, dt_bias, initial_state)):
         return ChunkKDAFunction.apply(q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state,
                                       use_qk_l2norm_in_kernel, gate_mode, use_beta_sigmoid_in_kernel, allow_neg_eigval,

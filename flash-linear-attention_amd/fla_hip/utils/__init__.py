@@ -30,20 +30,24 @@ def tensor_cache(fn: Callable[..., Any]) -> Callable[..., Any]:
     entries: deque = deque(maxlen=FLA_TENSOR_CACHE_SIZE)
 
     def versions(args, kwargs):
-        return tuple(x._version for x in (*args, *kwargs.values()) if isinstance(x, torch.Tensor))
+        # (tensors created in inference mode keep no version counter: calls with one are not memoised)
+        return tuple(None if x.is_inference() else x._version for x in (*args, *kwargs.values()) if isinstance(x, torch.Tensor))
 
     @functools.wraps(fn)
     def wrapper(*args, **kwargs):
         if FLA_DISABLE_TENSOR_CACHE or os.environ.get('FLA_DISABLE_TENSOR_CACHE') == '1':
             return fn(*args, **kwargs)
+        now = versions(args, kwargs)
+        if None in now:
+            return fn(*args, **kwargs)
         for a0, k0, v0, r0 in entries:
             if len(a0) == len(args) and k0.keys() == kwargs.keys() \
                     and all(x is y for x, y in zip(args, a0)) \
                     and all(kwargs[key] is k0[key] for key in kwargs) \
-                    and v0 == versions(args, kwargs):
+                    and v0 == now:
                 return r0
         out = fn(*args, **kwargs)
-        entries.append((args, kwargs, versions(args, kwargs), out))
+        entries.append((args, kwargs, now, out))
         return out
 
     return wrapper

@@ -356,6 +356,22 @@ int gdn_chunk_kda_fwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * gdn_chunk_kda_fwd that also leaves the state in front of every chunk: what chunk_kda returns as `h` with
+ * return_intermediate_states (fla/ops/kda/chunk.py:98-100, fla/ops/kda/chunk_fwd.py:130-131; the array
+ * chunk_gated_delta_rule_fwd_h fills, fla/ops/common/chunk_delta_h.py:714-718).
+ *   states [num_chunks, HV, K, V] in qkv_dtype (chunks in packed order: [B, NT, ...] for equal lengths), written by the scan
+ */
+int gdn_chunk_kda_fwd_states(
+    const void* q, const void* k, const void* v, const float* g, const void* beta,
+    const float* A_log, const float* dt_bias, float lower_bound, int gate_mode,
+    const float* h0, float* ht, void* o, void* states,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Chunked forward of the comba operator (one decay per token and head; the prediction uses a second key p and the state
  * before the token's decay).  Replaces chunk_comba_fwd (fla/ops/comba/chunk.py:22-90): chunk_comba_cumsum_scalar_fwd
  * (fla/ops/comba/utils.py), chunk_scaled_dot_comba_pkt_fwd and the triangular solve (fla/ops/comba/wy_fast.py), recompute_w_u_fwd,

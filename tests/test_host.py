@@ -105,6 +105,12 @@ def test_tensor_cache_is_by_identity():
     assert len(calls) == 4
     b.add_(1)
     assert f(b, 2).tolist() == [4.0, 4.0, 4.0] and len(calls) == 5
+    # tensors made in inference mode have no version counter: calls with one are computed every time
+    with torch.inference_mode():
+        c = torch.ones(3)
+        f(c, 2)
+        c.add_(1)
+        assert f(c, 2).tolist() == [4.0, 4.0, 4.0] and len(calls) == 7
 
 
 def test_cu_seqlens_check_follows_in_place_updates():

@@ -379,10 +379,8 @@ def test_chunk_kda_validation():
         chunk_kda(x, x, x, g, b, safe_gate=True)
     with pytest.raises(ValueError):
         chunk_kda(x, x, x, g[..., :32], b)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(AssertionError, match='inference mode'):
         chunk_kda(x, x, x, g, b, return_intermediate_states=True)
-    with pytest.raises(NotImplementedError):
-        chunk_kda(x.requires_grad_(), x, x, g, b)
     o, ht = chunk_kda(x[:, :0].detach(), x[:, :0].detach(), x[:, :0].detach(), g[:, :0], b[:, :0], output_final_state=True)
     assert o.shape == (1, 0, 2, 64) and torch.count_nonzero(ht) == 0
 
@@ -568,4 +566,37 @@ def test_chunk_kda_backward_options(what):
     ref = O.kda_grads(q, k, v, g, beta, do, dht, initial_state=h0, dtype=torch.float32, **kw)
     _, _, got = _kda_grads_gpu(q, k, v, g, beta, h0, None, None, do, dht, **kw)
     _compare_grads(ref, got)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('packed,vfirst,V', [(False, False, 64), (True, False, 64), (False, True, 64), (False, False, 200)])
+def test_chunk_kda_return_intermediate_states(packed, vfirst, V):
+    """``return_intermediate_states`` (inference mode): the state in front of every chunk, against the oracle's final state of
+    the tokens before that chunk (shapes and dtype as tests/ops/test_kda.py:1139-1211 of the reference)."""
+    from fla_hip.ops.kda import chunk_kda
+    B, T, H, HV, D = (1, 330, 2, 4, 64) if packed else (2, 200, 2, 4, 64)
+    q, k, v, g, beta, h0, _, _ = _chunk_inputs(B, T, H, HV, D, 1.0, 0, False, False, torch.bfloat16, seed=11, V=V)
+    cu = [0, 70, 70, 200, 330] if packed else None
+    N = len(cu) - 1 if packed else B
+    h0 = torch.randn(N, HV, D, V, generator=torch.Generator().manual_seed(12))
+    d = lambda x: x.cuda()
+    with torch.inference_mode():
+        o, ht, h = chunk_kda(d(q), d(k), d(v), d(g), d(beta), initial_state=d(h0.transpose(-1, -2).contiguous() if vfirst else h0),
+                             output_final_state=True, use_qk_l2norm_in_kernel=True, return_intermediate_states=True,
+                             state_v_first=vfirst, cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'))
+    bounds = [(0, s, e) for s, e in zip(cu[:-1], cu[1:])] if packed else [(b, 0, T) for b in range(B)]
+    chunks = sum((e - s + 63) // 64 for _, s, e in bounds)
+    nb = 1 if packed else B
+    assert h.dtype == torch.bfloat16 and h.shape == (nb, chunks // nb, HV, *((V, D) if vfirst else (D, V)))
+    hf = h.float().cpu().reshape(chunks, *h.shape[2:])
+    c = 0
+    for n, (b, s, e) in enumerate(bounds):
+        for t0 in range(s, e, 64):
+            sl = slice(s, t0)
+            _, ref = O.recurrent_kda(q[b:b + 1, sl], k[b:b + 1, sl], v[b:b + 1, sl], g[b:b + 1, sl], beta[b:b + 1, sl], None, h0[n:n + 1], True,
+                                     use_qk_l2norm_in_kernel=True)
+            got = hf[c].transpose(-1, -2) if vfirst else hf[c]
+            assert O.get_err_ratio(ref[0], got) < 0.005, (n, t0)
+            c += 1
+    assert c == chunks
 
