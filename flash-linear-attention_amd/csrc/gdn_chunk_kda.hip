@@ -26,41 +26,67 @@ namespace gdn {
 // ---------------------------------------------------------------------------------------------
 // prepare
 // ---------------------------------------------------------------------------------------------
-constexpr size_t KDA_PREP_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PG + 64 * PL + 64) * 4;
+// Two workgroups share a CU (80 KB of LDS each; a workgroup's phases are chains of dependent steps - the substitution above all -
+// that leave most of a CU idle): only k is kept as a tile; a wave reads nothing of q but its own 16 rows, which stay in
+// registers as operand fragments from the load to the store of qg; v arrives late, in the place of the matrix L.
+static_assert(64 * PL * 4 == 64 * P128 * 2, "the rows of v take the place of the matrix L");
+constexpr size_t KDA_PREP_SMEM = (2 * 64 * P128 + 64 * P64) * 2 + (64 * PG + 64) * 4;
 
 template <typename T>
-__global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, int64_t units) {
+__global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     extern __shared__ __align__(16) char smem[];
-    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
-    float* sG = (float*)(sA + 64 * P64); float* sL = sG + 64 * PG; float* sBeta = sL + 64 * PL;
+    T* sK = (T*)smem; T* sV = sK + 64 * P128; T* sA = sV + 64 * P128;
+    float* sL = (float*)sV;
+    float* sG = (float*)(sA + 64 * P64); float* sBeta = sG + 64 * PG;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
-    // One workgroup per CU walks over the units; the next unit's rows and gates are fetched into registers meanwhile.
-    TileRegs<BD> rK, rQ, rV;
+    // A workgroup walks over the units; the next unit's rows and gates are fetched into registers meanwhile.
+    TileRegs<BD> rK, rV;
+    V8 rQ[4];                                                   // q: row 16w + c16, features 32s + 8g .. + 7
     float rG[32], rB = 0.f;                                     // gates: a thread per key feature and half of the chunk's rows
+    auto fetch_v = [&](int64_t u) {
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + (int)(u % p.HV)) * BD, (int64_t)p.HV * BD, c.valid, tid);
+    };
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
         fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-        fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
-        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) rQ[s][e] = (T)0.f;
+            if (16 * w + c16 < c.valid) rQ[s] = *(const V8*)((const T*)p.q + ((c.tok0 + 16 * w + c16) * p.H + hq) * BD + 32 * s + 8 * g);
+        }
+        rB = (tid < 64 && tid < c.valid) ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+    };
+    auto fetch_g = [&](int64_t u) {
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
         const int col = tid & 127, half = tid >> 7;
 #pragma unroll
         for (int r = 0; r < 32; ++r) {
             const int row = 32 * half + r;
             rG[r] = row < c.valid ? p.g[((c.tok0 + row) * p.HV + hv) * BD + col] : 0.f;
         }
-        rB = (tid < 64 && tid < c.valid) ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
     };
     fetch(blockIdx.x);
+    const int tid_outer = tid;
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+    // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through: hoisted out
+    // of this loop, the addresses of its fully unrolled body would fill the register file before the loop starts, and spill)
+    int tid_opaque = tid_outer;
+    asm volatile("" : "+v"(tid_opaque));
+    const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
     const int hv = (int)(u % p.HV);
     const ChunkAt c = chunk_at(p, u / p.HV);
+    fetch_g(u);                                                 // (the gates are not fetched ahead: no 32 registers to carry them round the loop)
     put_tile<BD>(sK, P128, rK, tid);
-    put_tile<BD>(sQ, P128, rQ, tid);
-    put_tile<BD>(sV, P128, rV, tid);
+    V8 qx[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) qx[s] = rQ[s];
     {
         // running sums of the gates inside each half of the rows first
         const int col = tid & 127, half = tid >> 7;
@@ -77,6 +103,7 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
             }
             run += gt;
             sG[row * PG + col] = run;
+            __builtin_amdgcn_sched_barrier(0);                  // (one row at a time: 32 activations in flight at once cost 100 registers)
         }
     }
     if (tid < 64) {
@@ -85,7 +112,7 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
         sBeta[tid] = b;
     }
     lds_barrier();
-    if (u + gridDim.x < units) fetch(u + gridDim.x);
+    fetch_v(u);
     {
         // second half of the rows: add the first half's total
         const int col = tid & 127, half = tid >> 7;
@@ -96,23 +123,31 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
         }
     }
     if (p.flags & GDN_FLAG_QK_L2NORM) {
-        // rows of q and k divided by sqrt(sum x^2 + 1e-6): 16 consecutive lanes hold the 16 pieces of a row
+        // rows of q and k divided by sqrt(sum x^2 + 1e-6).  k: 16 consecutive lanes hold the 16 pieces of a row
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = (tid >> 4) + 16 * i, pc = tid & 15;
+            T* at = sK + row * P128 + pc * 8;
+            V8 x = *(V8*)at;
+            float ss = 0.f;
 #pragma unroll
-            for (int which = 0; which < 2; ++which) {
-                T* at = (which ? sQ : sK) + row * P128 + pc * 8;
-                V8 x = *(V8*)at;
-                float ss = 0.f;
+            for (int e = 0; e < 8; ++e) ss += (float)x[e] * (float)x[e];
+            const float r = rsqrtf(sum_over_c16(ss) + 1e-6f);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) ss += (float)x[e] * (float)x[e];
-                const float r = rsqrtf(sum_over_c16(ss) + 1e-6f);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * r);
-                *(V8*)at = x;
-            }
+            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * r);
+            *(V8*)at = x;
         }
+        // q: the four lanes that share c16 hold a row
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += (float)qx[s][e] * (float)qx[s][e];
+        const float r = rsqrtf(sum_over_g(ss) + 1e-6f);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qx[s][e] = (T)((float)qx[s][e] * r);
     }
     lds_barrier();
 
@@ -122,18 +157,17 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
         const int i = 16 * w + c16;                             // the row this lane's operand fragments belong to
         // rows of this block against rows of earlier blocks: reference = the row in front of the block (zeros for block 0)
         V8 kd[4], qd[4];
-        float ref[4][8];
+        const float* gref = sG + (16 * w - 1) * PG + 8 * g;         // the reference row, read where it is used (w > 0)
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const float* gi = sG + i * PG + 32 * s + 8 * g;
             const float* gr = sG + (16 * w - 1) * PG + 32 * s + 8 * g;
-            const V8 kx = frag_rows(sK, P128, 16 * w, 32 * s, lane), qx = frag_rows(sQ, P128, 16 * w, 32 * s, lane);
+            const V8 kx = frag_rows(sK, P128, 16 * w, 32 * s, lane);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                ref[s][e] = w > 0 ? gr[e] : 0.f;
-                const float f = __expf(gi[e] - ref[s][e]);
+                const float f = __expf(gi[e] - (w > 0 ? gr[e] : 0.f));
                 kd[s][e] = (T)((float)kx[e] * f);
-                qd[s][e] = (T)((float)qx[e] * f);
+                qd[s][e] = (T)((float)qx[s][e] * f);
             }
         }
 #pragma unroll
@@ -145,7 +179,7 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
                 const float* gj = sG + (16 * tj + c16) * PG + 32 * s + 8 * g;
                 V8 kn = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
+                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(gref[32 * s + e] - gj[e]));        // (tj < w: w > 0)
                 m = Mma<T>::run(kd[s], kn, m);                 // lane: column j = 16tj + c16, rows i = 16w + 4g + r
                 pt = Mma<T>::run(kn, qd[s], pt);               // lane: column i = 16w + c16, rows j = 16tj + 4g + r
             }
@@ -180,7 +214,7 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
                 const float* gj = sG + i * PG + 32 * s + 8 * g;
                 V8 kn = frag_rows(sK, P128, 16 * w, 32 * s, lane);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf(ref[s][e] - gj[e]));
+                for (int e = 0; e < 8; ++e) kn[e] = (T)((float)kn[e] * __expf((w > 0 ? gref[32 * s + e] : 0.f) - gj[e]));
                 m = Mma<T>::run(kd[s], kn, m);                 // lane: column j = 16w + c16, rows i = 16w + 4g + r
                 pt = Mma<T>::run(kn, qd[s], pt);               // lane: column i = 16w + c16, rows j = 16w + 4g + r
             }
@@ -193,37 +227,33 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
             }
             *(V4*)(Pu + i * 64 + 16 * w + 4 * g) = pack4<T>(pt);
         } else
-        // (lane (il, jq) takes row il and columns 4jq .. 4jq+3 of the block)
+        // (lane (c16, g) takes row i against every row j of the block over the features of its own fragments; the four lanes that
+        // share a row add up)
         {
-            const int il = lane >> 2, jq = lane & 3, row = 16 * w + il;
-            float m[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
-            for (int kc = 0; kc < BD / 8; ++kc) {
-                const V8 ki = *(const V8*)(sK + row * P128 + 8 * kc), qi = *(const V8*)(sQ + row * P128 + 8 * kc);
-                const f32x4 gi0 = *(const f32x4*)(sG + row * PG + 8 * kc), gi1 = *(const f32x4*)(sG + row * PG + 8 * kc + 4);
+#pragma unroll 1
+            for (int jl = 0; jl < 16; ++jl) {
+                const int rj = 16 * w + jl;
+                float mj = 0.f, pj = 0.f;
+                if (jl <= c16) {
 #pragma unroll
-                for (int jj = 0; jj < 4; ++jj) {
-                    const int jl = 4 * jq + jj;
-                    if (jl > il) continue;                      // (upper triangle: nothing)
-                    const int rj = 16 * w + jl;
-                    const V8 kj = *(const V8*)(sK + rj * P128 + 8 * kc);
-                    const f32x4 gj0 = *(const f32x4*)(sG + rj * PG + 8 * kc), gj1 = *(const f32x4*)(sG + rj * PG + 8 * kc + 4);
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 ki = frag_rows(sK, P128, 16 * w, 32 * s, lane), kj = *(const V8*)(sK + rj * P128 + 32 * s + 8 * g);
+                        const float* gi = sG + i * PG + 32 * s + 8 * g;
+                        const float* gj = sG + rj * PG + 32 * s + 8 * g;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float d = __expf((e < 4 ? gi0[e & 3] : gi1[e & 3]) - (e < 4 ? gj0[e & 3] : gj1[e & 3]));
-                        const float kk = (float)kj[e] * d;
-                        m[jj] += (float)ki[e] * kk;
-                        pq[jj] += (float)qi[e] * kk;
+                        for (int e = 0; e < 8; ++e) {
+                            const float kk = (float)kj[e] * __expf(gi[e] - gj[e]);
+                            mj += (float)ki[e] * kk;
+                            pj += (float)qx[s][e] * kk;
+                        }
                     }
                 }
+                mj = sum_over_g(mj); pj = sum_over_g(pj);
+                if (g == 0) {
+                    sL[i * PL + (rj & 3) * 16 + (rj >> 2)] = jl < c16 ? sBeta[i] * mj : 0.f;
+                    Pu[i * 64 + rj] = (T)(jl <= c16 ? p.scale * pj : 0.f);
+                }
             }
-            f32x4 pt;
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const int jl = 4 * jq + jj, j = 16 * w + jl;
-                sL[row * PL + (j & 3) * 16 + (j >> 2)] = jl < il ? sBeta[row] * m[jj] : 0.f;
-                pt[jj] = jl <= il ? p.scale * pq[jj] : 0.f;
-            }
-            *(V4*)(Pu + row * 64 + 16 * w + 4 * jq) = pack4<T>(pt);
         }
     }
     lds_barrier();
@@ -247,29 +277,42 @@ __global__ __launch_bounds__(256, 1) void gdn_kda_prepare_kernel(KdaParams p, in
         // what the scan needs of q and k, and k, v as the factors of w, u
         T* QGu = (T*)p.ws.QG + u * 64 * BD;
         T* KGu = (T*)p.ws.KG + u * 64 * BD;
-        for (int idx = tid; idx < 64 * 16; idx += 256) {
-            const int row = idx >> 4, pc = idx & 15;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {                        // (the pieces of v: those this thread fetched)
+            const int idx = tid + 256 * it, row = idx >> 4, pc = idx & 15;
             const float* gi = sG + row * PG + pc * 8;
             const float* gl = sG + 63 * PG + pc * 8;
-            V8 kx = *(V8*)(sK + row * P128 + pc * 8), qx = *(V8*)(sQ + row * P128 + pc * 8), vx = *(V8*)(sV + row * P128 + pc * 8);
-            V8 kg, qg;
+            V8 kx = *(V8*)(sK + row * P128 + pc * 8), vx = __builtin_bit_cast(V8, rV.x[it]);
+            V8 kg;
             const float b = sBeta[row];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float eg = __expf(gi[e]);
                 kg[e] = (T)((float)kx[e] * __expf(gl[e] - gi[e]));
-                qg[e] = (T)((float)qx[e] * (p.scale * eg));
                 kx[e] = (T)((float)kx[e] * (b * eg));
                 vx[e] = (T)((float)vx[e] * b);
             }
             *(V8*)(KGu + row * BD + pc * 8) = kg;
-            *(V8*)(QGu + row * BD + pc * 8) = qg;
             *(V8*)(sK + row * P128 + pc * 8) = kx;
-            *(V8*)(sV + row * P128 + pc * 8) = vx;
+            *(V8*)(sV + row * P128 + pc * 8) = vx;                                  // (in the place of L: the substitution is over)
+        }
+        {
+            const int i = 16 * w + c16;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float* gi = sG + i * PG + 32 * s + 8 * g;
+                V8 qg;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qg[e] = (T)((float)qx[s][e] * (p.scale * __expf(gi[e])));
+                *(V8*)(QGu + i * BD + 32 * s + 8 * g) = qg;
+            }
         }
         if (tid < BD) p.ws.EGL[u * BD + tid] = __expf(sG[63 * PG + tid]);
     }
     lds_barrier();
+    // (the next unit's rows and gates: requested this late because the phases above have no registers to spare under the cap
+    // that lets two workgroups share a CU)
+    if (u + gridDim.x < units) fetch(u + gridDim.x);
     {
         // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
         T* Wu = (T*)p.ws.Wm + u * 64 * BD;
@@ -620,7 +663,7 @@ static int launch_kda(const KdaParams& p, int64_t num_chunks, hipStream_t stream
     else if (vbt == 64) scan = {(const void*)gdn_kda_scan_kernel<T, 64>, kda_scan_smem<64>(), "gdn_kda_scan_kernel", runs};
     else scan = {(const void*)gdn_kda_scan_kernel<T, 128>, kda_scan_smem<128>(), "gdn_kda_scan_kernel", runs};
     const K prep = comba ? K{(const void*)gdn_comba_prepare_kernel<T>, COMBA_PREP_SMEM, "gdn_comba_prepare_kernel", units < 512u ? units : 512u}
-                         : K{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 256u ? units : 256u};
+                         : K{(const void*)gdn_kda_prepare_kernel<T>, KDA_PREP_SMEM, "gdn_kda_prepare_kernel", units < 512u ? units : 512u};
     const K ks[2] = {prep, scan};
     for (int i = 0; i < 2; ++i) {
         if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
@@ -639,7 +682,7 @@ int launch_kda_prepare(const KdaParams& p, int64_t num_chunks, int qkv_dtype, hi
     if (int rc = ensure_dynamic_smem_for(f, KDA_PREP_SMEM, "gdn_kda_prepare_kernel")) return rc;
     int64_t nunits = units;
     void* args[] = {(void*)&p, (void*)&nunits};
-    if (hipLaunchKernel(f, dim3(units < 256u ? units : 256u), dim3(256), args, KDA_PREP_SMEM, stream) != hipSuccess) return check_launch("gdn_kda_prepare_kernel");
+    if (hipLaunchKernel(f, dim3(units < 512u ? units : 512u), dim3(256), args, KDA_PREP_SMEM, stream) != hipSuccess) return check_launch("gdn_kda_prepare_kernel");
     return check_launch("gdn_kda_prepare_kernel");
 }
 
