@@ -69,7 +69,11 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kda_kernel(BwdParams p, i
         }
     };
     fetch(blockIdx.x);
+    const int tid_outer = tid;
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        int tid_opaque = tid_outer;                             // (see gdn_bwd_wy_kda_kernel)
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         const int hv = (int)(u % p.HV);
         const ChunkAt c = chunk_at(p, u / p.HV);
         put_tile<BD>(sDO, P128, rDO, tid);
@@ -228,7 +232,14 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
         if (tid < 64) rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
     };
     fetch(blockIdx.x);
+    const int tid_outer = tid;
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would fill the register file and spill)
+        int tid_opaque = tid_outer;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        auto feat = [&](int a) { return 16 * (2 * w + a); };
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
         put_tile<BD>(sDvn, P128, rDvn, tid);
