@@ -46,11 +46,13 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
     TileRegs<BD> rK, rV;
     V8 rQ[4];                                                   // q: row 16w + c16, features 32s + 8g .. + 7
     float rG[32], rB = 0.f;                                     // gates: a thread per key feature and half of the chunk's rows
-    auto fetch_v = [&](int64_t u) {
+    // (the lane number is an argument: inside the loop over the units it is the opaque copy, see there)
+    auto fetch_v = [&](int64_t u, int tid) {
         const ChunkAt c = chunk_at(p, u / p.HV);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + (int)(u % p.HV)) * BD, (int64_t)p.HV * BD, c.valid, tid);
     };
-    auto fetch = [&](int64_t u) {
+    auto fetch = [&](int64_t u, int tid) {
+        const int lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
         fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
         }
         rB = (tid < 64 && tid < c.valid) ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
     };
-    auto fetch_g = [&](int64_t u) {
+    auto fetch_g = [&](int64_t u, int tid) {
         const int hv = (int)(u % p.HV);
         const ChunkAt c = chunk_at(p, u / p.HV);
         const int col = tid & 127, half = tid >> 7;
@@ -72,7 +74,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
             rG[r] = row < c.valid ? p.g[((c.tok0 + row) * p.HV + hv) * BD + col] : 0.f;
         }
     };
-    fetch(blockIdx.x);
+    fetch(blockIdx.x, tid);
     const int tid_outer = tid;
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
     // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through: hoisted out
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
     const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
     const int hv = (int)(u % p.HV);
     const ChunkAt c = chunk_at(p, u / p.HV);
-    fetch_g(u);                                                 // (the gates are not fetched ahead: no 32 registers to carry them round the loop)
+    fetch_g(u, tid);                                                 // (the gates are not fetched ahead: no 32 registers to carry them round the loop)
     put_tile<BD>(sK, P128, rK, tid);
     V8 qx[4];
 #pragma unroll
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
         sBeta[tid] = b;
     }
     lds_barrier();
-    fetch_v(u);
+    fetch_v(u, tid);
     {
         // second half of the rows: add the first half's total
         const int col = tid & 127, half = tid >> 7;
@@ -257,7 +259,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
         }
     }
     lds_barrier();
-    solve_unit_lower<T>(sL, sA, w, lane);
+    solve_unit_lower_blocks<T>(sL, (float*)sA, sA, w, lane);
     lds_barrier();
     if (p.ws.Am) {                                              // (for the backward pass)
         T* Au = (T*)p.ws.Am + u * 64 * 64;
@@ -310,9 +312,6 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
         if (tid < BD) p.ws.EGL[u * BD + tid] = __expf(sG[63 * PG + tid]);
     }
     lds_barrier();
-    // (the next unit's rows and gates: requested this late because the phases above have no registers to spare under the cap
-    // that lets two workgroups share a CU)
-    if (u + gridDim.x < units) fetch(u + gridDim.x);
     {
         // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
         T* Wu = (T*)p.ws.Wm + u * 64 * BD;
@@ -334,6 +333,9 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
             *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
         }
     }
+    // (the next unit's rows: requested this late because the phases above have no registers to spare under the cap that lets two
+    // workgroups share a CU; the other workgroup covers the wait)
+    if (u + gridDim.x < units) fetch(u + gridDim.x, tid);
     lds_barrier();
     }
 }

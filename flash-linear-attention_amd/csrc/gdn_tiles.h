@@ -158,4 +158,69 @@ __device__ __forceinline__ void solve_unit_lower(const float* sL, T* sA, int w, 
     }
 }
 
+// The same inverse by blocks of 16, for the same four waves (all of them must call it: it holds two barriers).  Wave a first
+// inverts the diagonal block a on its own (X_a (I + L_aa) = I by rows from the right: lane c16 owns row c16, 16 short steps
+// without any exchange between lanes) and leaves X_a in LDS; then wave b computes block column b of A from
+//     A_bb = X_b,   A_ab = -X_a sum_{b <= m < a} L_am A_mb   (a > b)
+// on the matrix cores in fp32 (v_mfma_f32_16x16x4_f32): the left factors L_am and X_a come from LDS, the right factors are
+// the blocks just computed, which an accumulator holds in the layout a right factor needs.  64 dependent steps become 16
+// plus at most nine 16 x 16 products.  sX: 1024 floats of scratch, which may be the memory of sA itself.
+template <typename T>
+__device__ __forceinline__ void solve_unit_lower_blocks(const float* sL, float* sX, T* sA, int w, int lane) {
+    const int c16 = lane & 15, g = lane >> 4;
+    {
+        float x[16], acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int i = 15; i >= 0; --i) {
+            x[i] = ((i == c16) ? 1.f : 0.f) - acc[i];
+            // row i of the diagonal block: entry j = 4q + e at [e][4w + q]
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (e >= i) continue;
+                const f32x4 l = *(const f32x4*)(sL + (16 * w + i) * PL + e * 16 + 4 * w);
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (4 * q + e < i) acc[4 * q + e] += l[q] * x[i];
+            }
+        }
+        if (g == 0) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *(f32x4*)(sX + w * 256 + c16 * 16 + 4 * q) = f32x4{x[4 * q], x[4 * q + 1], x[4 * q + 2], x[4 * q + 3]};
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    f32x4 A[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        A[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (a < w) continue;
+        if (a == w) {
+            const float* t = sX + a * 256;
+            A[a] = f32x4{t[(4 * g) * 16 + c16], t[(4 * g + 1) * 16 + c16], t[(4 * g + 2) * 16 + c16], t[(4 * g + 3) * 16 + c16]};
+            continue;
+        }
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < a; ++m) {
+            if (m < w) continue;
+            // left factor L_am by rows: entry (16a + c16, 16m + 4g + e) at [e][4m + g]
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                t = __builtin_amdgcn_mfma_f32_16x16x4f32(sL[(16 * a + c16) * PL + e * 16 + 4 * m + g], A[m][e], t, 0, 0, 0);
+        }
+        const f32x4 xa = *(const f32x4*)(sX + a * 256 + c16 * 16 + 4 * g);
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[e], t[e], r, 0, 0, 0);
+        A[a] = -r;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");     // (every wave has read the X tiles: sA may take their place)
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sA[(16 * a + 4 * g + r) * P64 + 16 * w + c16] = (T)A[a][r];
+}
+
 }  // namespace gdn
