@@ -116,6 +116,11 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
+        int tid_opaque = threadIdx.x;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
         put_tile<BD>(sV, P128, rV, tid);
@@ -174,7 +179,7 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
             *(V8*)at = x;
         }
-        solve_unit_lower<T>(sL, sA, w, lane);
+        solve_unit_lower_blocks<T>(sL, (float*)sA, sA, w, lane);
         lds_barrier();
         {
             T* Au = (T*)p.ws.Am + u * 64 * 64;

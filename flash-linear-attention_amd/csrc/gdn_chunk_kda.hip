@@ -377,6 +377,11 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
     fetch(blockIdx.x);
     fetch_v(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+    // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through: hoisted
+    // out of this loop, the addresses of its unrolled body would fill the register file and spill)
+    int tid_opaque = threadIdx.x;
+    asm volatile("" : "+v"(tid_opaque));
+    const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
     put_tile<BD>(sK, P128, rK, tid);
     put_tile<BD>(sQ, P128, rQ, tid);
     put_tile<BD>(sP, P128, rP, tid);
@@ -477,7 +482,7 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
         }
     }
     lds_barrier();
-    solve_unit_lower<T>(sL, sA, w, lane);
+    solve_unit_lower_blocks<T>(sL, (float*)sA, sA, w, lane);
     {
         // p, v as the factors of w, u
 #pragma unroll 2                                        // (unrolled fully, the kernel spills registers)
