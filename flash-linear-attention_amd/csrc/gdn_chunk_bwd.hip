@@ -33,10 +33,13 @@ namespace gdn {
 // The KDA operator (a decay per key feature) adds: Gk, the running sums of the log decays [64][128] fp32; QG = scale q e^Gk,
 // KG = k e^(Gk_last - Gk) [64][128] and P [64][64] in the operand type, EGL = e^Gk_last [128] fp32 (all four as the forward's
 // chunk-parallel kernel writes them); dPs = scale tril(do v_new^T) [64][64]; dGk [64][128] fp32 (partial, between the last two kernels).
+// Um: u [64][128], read by the forward scan (which leaves v_new in Vn: a scan cut into time segments reads the u of chunks that belong
+// to another workgroup, so it must not be overwritten); Bound: one float per unit, see gdn_chunk_common.h (WARM_LOG2).
 struct BwdWs {
     float* Gam; float* Dgam; float* Gam0;
     void* Am; void* PT; void* Wm; void* Vn; void* Hs; void* dHs; void* dVn; void* dWm;
     float* Gk; void* QG; void* KG; void* Pm; float* EGL; void* dPs; float* dGk;
+    void* Um; float* Bound;
 };
 inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     size_t off = 0;
@@ -47,8 +50,9 @@ inline size_t bwd_ws_layout(int64_t units, int64_t KD, char* base, BwdWs* ws) {
     void* Wm = take(u * 64 * KD * 2); void* Vn = take(u * 64 * BD * 2);
     void* Hs = take(u * KD * BD * 2); void* dHs = take(u * KD * BD * 2);
     void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * KD * 2);
+    void* Um = take(u * 64 * BD * 2); void* Bound = take(u * 4);
     if (ws) *ws = BwdWs{(float*)Gam, (float*)Dgam, (float*)Gam0, Am, PT, Wm, Vn, Hs, dHs, dVn, dWm,
-                        nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+                        nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, Um, (float*)Bound};
     return off;
 }
 inline size_t kda_bwd_ws_layout(int64_t units, char* base, BwdWs* ws) {
@@ -62,7 +66,7 @@ inline size_t kda_bwd_ws_layout(int64_t units, char* base, BwdWs* ws) {
     void* dVn = take(u * 64 * BD * 2); void* dWm = take(u * 64 * BD * 2);
     void* Gk = take(u * 64 * BD * 4); void* dGk = take(u * 64 * BD * 4); void* EGL = take(u * BD * 4);
     if (ws) *ws = BwdWs{nullptr, nullptr, nullptr, Am, nullptr, Wm, Vn, Hs, dHs, dVn, dWm,
-                        (float*)Gk, QG, KG, Pm, (float*)EGL, dPs, (float*)dGk};
+                        (float*)Gk, QG, KG, Pm, (float*)EGL, dPs, (float*)dGk, Vn, nullptr};       // (u and v_new share their place: whole sequences only)
     return off;
 }
 
@@ -76,7 +80,52 @@ struct BwdParams {
     BwdWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;
     float scale; int gb_dtype; uint32_t flags;
+    // The two scans cut into `nseg` time segments of `seg_chunks` chunks (1: whole sequences): a segment starts from a zero state up
+    // to `warm_cap` chunks outside its range where the chunks' transition bounds say that this is forgotten by the time its own
+    // range begins (gdn_chunk_common.h, WARM_LOG2); a head with a segment that cannot is walked whole by the workgroups of segment 0.
+    int nseg, seg_chunks, warm_cap;
 };
+
+// The mirror image of warm_chunks() for the scan that runs backwards: how many chunks AFTER chunk it1 - 1 a run must start from a
+// zero state so that at it1 - 1 it has forgotten the difference to the true state.  When the end of the sequence comes first the
+// answer is nc - it1 (the run starts from the true gradient of the final state and is exact).  -1: not within `cap` chunks.
+__device__ __forceinline__ int warm_chunks_rev(const float* bound, int HV, int64_t it1, int64_t nc, int cap, int lane) {
+    const bool in = lane < cap && it1 + lane < nc;
+    float x = in ? bound[(it1 + lane) * HV] : 0.f;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float y = __shfl_up(x, off, 64);
+        if (lane >= off) x += y;
+    }
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(in && x <= WARM_LOG2);
+    if (hit) return __builtin_ctzll(hit) + 1;
+    return nc - it1 <= cap ? (int)(nc - it1) : -1;
+}
+
+// What a workgroup of the two scans does with time segments: `whole`: segment 0 walks the sequence, the others leave;
+// otherwise the forward scan walks chunks [f0 - fw, f1) and keeps its results from f0 on, the reverse scan walks [f0, f1 + rw)
+// downwards and keeps its results below f1.  The same in every wave of a workgroup (both scans need both answers: side by side
+// in one workgroup they must take the same number of barriers).
+struct ScanPlan { bool whole; int64_t f0, f1; int fw, rw; };
+__device__ __forceinline__ ScanPlan scan_plan(const BwdParams& p, const SeqAt& sq, int hv, int seg, int lane) {
+    ScanPlan sp{false, 0, sq.nc, 0, 0};
+    if (p.nseg <= 1) return sp;
+    const float* bound = p.ws.Bound + sq.cbase * p.HV + hv;
+    sp.f0 = (int64_t)seg * p.seg_chunks;
+    sp.f1 = seg == p.nseg - 1 ? sq.nc : (int64_t)(seg + 1) * p.seg_chunks;
+    for (int s = 1; s < p.nseg; ++s) {
+        const int64_t at = (int64_t)s * p.seg_chunks;           // the boundary between segments s - 1 and s
+        const int fw = warm_chunks(bound, p.HV, at, p.warm_cap, lane), rw = warm_chunks_rev(bound, p.HV, at, sq.nc, p.warm_cap, lane);
+        sp.whole |= fw < 0 || rw < 0;
+        if (s == seg) sp.fw = fw;
+        if (s == seg + 1) sp.rw = rw;
+    }
+    if (sp.whole) { sp.f0 = 0; sp.f1 = sq.nc; sp.fw = sp.rw = 0; }
+    return sp;
+}
+
+// steps of the longer of the two scans of a workgroup
+__device__ __forceinline__ int64_t pad_steps_of(const ScanPlan& sp) { return (sp.f1 - sp.f0) + (sp.fw > sp.rw ? sp.fw : sp.rw); }
 
 // ---------------------------------------------------------------------------------------------
 // prepare
@@ -138,6 +187,20 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
             if constexpr (COMBA) p.ws.Gam0[u * 64 + lane] = x - rG;
         }
         lds_barrier();
+        if (!COMBA && p.nseg > 1 && w == 0) {
+            // how much this chunk's transition can stretch a state, in log2 units: every token's factor gamma_t (I - beta_t k_t k_t^T)
+            float k2 = 0.f;
+            for (int pc = 0; pc < KD / 8; ++pc) {
+                const V8 kx = *(const V8*)(sK + lane * PK + pc * 8);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) k2 += (float)kx[e] * (float)kx[e];
+            }
+            float lb = fabsf(1.f - sBeta[lane] * k2);
+            lb = lb > 1.f ? __log2f(lb) : 0.f;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) lb += __shfl_xor(lb, off, 64);
+            if (lane == 63) p.ws.Bound[u] = sGam[63] * 1.44269504f + lb;
+        }
         if (u + gridDim.x < units) fetch(u + gridDim.x);
 
         // strip of 16 token rows per wave: L (fp32, for the substitution; entry (i, j) at [i][j % 4][j / 4]) and P^T
@@ -192,7 +255,7 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
         // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
         {
             T* Wu = (T*)p.ws.Wm + u * 64 * KD;
-            T* Uu = (T*)p.ws.Vn + u * 64 * BD;
+            T* Uu = (T*)p.ws.Um + u * 64 * BD;
             const int i = 16 * w + c16;
             V8 fa[2];
 #pragma unroll
@@ -233,7 +296,7 @@ template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 *
 
 // KDA: the rows of k arrive with their decay to the end of the chunk on them (KG), and the state decays per key feature (EGL).
 template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
-__device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
+__device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, const int tid, const unsigned bid_all, const unsigned nwg) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
@@ -242,13 +305,18 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
     float* sGam = (float*)(sVn + 64 * PV);
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
-    // an L2 for the rows of k, q and w that all of them read.
+    // an L2 for the rows of k, q and w that all of them read.  With time segments (nwg workgroups each) a segment's come in a row.
+    const int seg = p.nseg > 1 ? (int)(bid_all / (nwg / p.nseg)) : 0;
+    const unsigned bid = p.nseg > 1 ? bid_all % (nwg / p.nseg) : bid_all;
     const int64_t run = (int64_t)(bid / (8 * NVS)) * 8 + bid % 8;
     if (run >= p.N * p.HV) return;
     const int vs = (bid / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
     const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
+    const ScanPlan plan = scan_plan(p, sq, hv, seg, lane);
+    if (plan.whole && seg != 0) return;
+    const int64_t c_first = plan.f0 - plan.fw, c_keep = plan.f0, c_end = plan.f1;     // walks [c_first, c_end), results kept from c_keep on
 
     f32x4 S[NA][NB];
 #pragma unroll
@@ -256,7 +324,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (NA * w + a2) + c16;
-            S[a2][b] = p.h0 ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
+            S[a2][b] = (p.h0 && c_first == 0) ? *(const f32x4*)(p.h0 + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
     // (AHEAD = 2: two sets of registers take turns and the tiles of chunk c + 2 are requested while chunk c is worked on;
     // measured: no faster than one chunk of lead - a step is bound by the CU's load path, not by the way to memory)
@@ -277,11 +345,12 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
             if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
         }
 #pragma unroll
-        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Vn + u * 64 * BD + (16 * w + c16) * BD + vcol0 + vq0 + 16 * b + 4 * g);
+        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Um + u * 64 * BD + (16 * w + c16) * BD + vcol0 + vq0 + 16 * b + 4 * g);
     };
     auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rW = R.rW; auto& rK = R.rK; auto& rU = R.rU; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
+        const bool keep = ic >= c_keep;                         // (chunks of the warm-up belong to another segment: nothing of them is stored)
         put_tile<KD, NTH>(sW, PK, rW, tid);
         put_tile<KD, NTH>(sK, PK, rK, tid);
         if (tid < 64) sGam[tid] = rGam;
@@ -299,10 +368,10 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
                 const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(S[a2][b]);
                 *(V4*)(sS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
-                *(V4*)(Hu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
+                if (keep) *(V4*)(Hu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
-        if (ic + AHEAD < sq.nc) fetch(R, ic + AHEAD);
+        if (ic + AHEAD < c_end) fetch(R, ic + AHEAD);
         const float glast = sGam[63];
         {
             // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
@@ -321,7 +390,7 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
                 const V4 vn4 = pack4<T>(vn);
-                *(V4*)(Vu + vq0 + 16 * b + 4 * g) = vn4;
+                if (keep) *(V4*)(Vu + vq0 + 16 * b + 4 * g) = vn4;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)vn4[r] * dec;
                 *(V4*)(sVn + i * PV + vq0 + 16 * b + 4 * g) = pack4<T>(vn);
@@ -350,16 +419,18 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
         }
         lds_barrier();
     };
-    if (sq.nc > 0) fetch(RA, 0);
+    if (c_end > c_first) fetch(RA, c_first);
     if constexpr (AHEAD == 1) {
-        for (int64_t ic = 0; ic < sq.nc; ++ic) step(RA, ic);
+        for (int64_t ic = c_first; ic < c_end; ++ic) step(RA, ic);
     } else {
-        if (sq.nc > 1) fetch(RB, 1);
-        for (int64_t ic = 0; ic < sq.nc; ic += 2) {
+        if (c_end > c_first + 1) fetch(RB, c_first + 1);
+        for (int64_t ic = c_first; ic < c_end; ic += 2) {
             step(RA, ic);
-            if (ic + 1 < sq.nc) step(RB, ic + 1);
+            if (ic + 1 < c_end) step(RB, ic + 1);
         }
     }
+    // (side by side with the reverse scan in one workgroup: as many barriers as the longer of the two takes)
+    for (int64_t i = (c_end - c_first); i < pad_steps_of(plan); ++i) { lds_barrier(); lds_barrier(); lds_barrier(); }
 }
 
 // (all 128 value columns of a head: eight waves, two per SIMD, share one set of tiles)
@@ -368,13 +439,13 @@ template <int VBT> constexpr int scan_waves() { return VBT == BD ? 8 : 4; }
 template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_state_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x);
+    bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x, gridDim.x);
 }
 
 // KDA: k and q arrive as KG and QG (decays and the scale on them), P row-major instead of transposed, the gradient of the
 // state decays per key feature.
 template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
-__device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid, const unsigned bid) {
+__device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, const int tid, const unsigned bid_all, const unsigned nwg) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
@@ -384,13 +455,18 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     float* sGam = (float*)(sDS + KD * PV);
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
-    // an L2 for the rows of k, q and w that all of them read.
+    // an L2 for the rows of k, q and w that all of them read.  With time segments (nwg workgroups each) a segment's come in a row.
+    const int seg = p.nseg > 1 ? (int)(bid_all / (nwg / p.nseg)) : 0;
+    const unsigned bid = p.nseg > 1 ? bid_all % (nwg / p.nseg) : bid_all;
     const int64_t run = (int64_t)(bid / (8 * NVS)) * 8 + bid % 8;
     if (run >= p.N * p.HV) return;
     const int vs = (bid / 8) % NVS, hv = (int)(run % p.HV), hq = hv / (p.HV / p.H);
     const int64_t n = run / p.HV;
     const SeqAt sq = seq_at(p, n);
     const int vcol0 = vs * VBT;
+    const ScanPlan plan = scan_plan(p, sq, hv, seg, lane);
+    if (plan.whole && seg != 0) return;
+    const int64_t c_lo = plan.f0, c_keep = plan.f1, c_top = plan.f1 + plan.rw;       // walks [c_lo, c_top) downwards, results kept below c_keep
 
     f32x4 dS[NA][NB];
 #pragma unroll
@@ -398,7 +474,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const int kk = 16 * (NA * w + a2) + c16;
-            dS[a2][b] = p.dht ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
+            dS[a2][b] = (p.dht && c_top == sq.nc) ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
     // (two sets of registers for AHEAD = 2, as in the forward scan)
     struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; };
@@ -426,6 +502,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     auto step = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
         auto& rK = R.rK; auto& rQ = R.rQ; auto& rW = R.rW; auto& rPT = R.rPT; auto& rDO = R.rDO; auto& rGam = R.rGam;
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
+        const bool keep = ic < c_keep;                          // (chunks of the warm-up belong to another segment: nothing of them is stored)
         put_tile<KD, NTH>(sK, PK, rK, tid);
         put_tile<KD, NTH>(sQ, PK, rQ, tid);
         put_tile<KD, NTH>(sW, PK, rW, tid);
@@ -443,10 +520,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
                 const int kk = 16 * (NA * w + a2) + c16;
                 const V4 s4 = pack4<T>(dS[a2][b]);
                 *(V4*)(sDS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
-                *(V4*)(dHu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
+                if (keep) *(V4*)(dHu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
             }
         lds_barrier();
-        if (ic >= AHEAD) fetch(R, ic - AHEAD);
+        if (ic >= c_lo + AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
         // scale e^gam_i do_i, for the state's gradient  (KDA: the factors are on the rows of q already)
         if constexpr (!KDA)
@@ -479,7 +556,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
                 for (int s = 0; s < 4 * KT; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, vq0 + 16 * b, lane), kf[s], a2v);
                 f32x4 dvn = a1 + a2v * dec;
-                *(V4*)(dVu + vq0 + 16 * b + 4 * g) = pack4<T>(dvn);
+                if (keep) *(V4*)(dVu + vq0 + 16 * b + 4 * g) = pack4<T>(dvn);
                 *(V4*)(sDvn + j * PV + vq0 + 16 * b + 4 * g) = pack4<T>(-dvn);
             }
         }
@@ -512,17 +589,18 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         }
         lds_barrier();
     };
-    if (sq.nc > 0) fetch(RA, sq.nc - 1);
+    if (c_top > c_lo) fetch(RA, c_top - 1);
     if constexpr (AHEAD == 1) {
-        for (int64_t ic = sq.nc - 1; ic >= 0; --ic) step(RA, ic);
+        for (int64_t ic = c_top - 1; ic >= c_lo; --ic) step(RA, ic);
     } else {
-        if (sq.nc > 1) fetch(RB, sq.nc - 2);
-        for (int64_t ic = sq.nc - 1; ic >= 0; ic -= 2) {
+        if (c_top > c_lo + 1) fetch(RB, c_top - 2);
+        for (int64_t ic = c_top - 1; ic >= c_lo; ic -= 2) {
             step(RA, ic);
-            if (ic > 0) step(RB, ic - 1);
+            if (ic > c_lo) step(RB, ic - 1);
         }
     }
-    if (p.dh0) {
+    for (int64_t i = (c_top - c_lo); i < pad_steps_of(plan); ++i) { lds_barrier(); lds_barrier(); lds_barrier(); }
+    if (p.dh0 && c_lo == 0) {
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
 #pragma unroll
@@ -536,7 +614,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
-    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x);
+    bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x, gridDim.x);
 }
 
 // Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
@@ -549,8 +627,8 @@ template <typename T, int VBT, int KT, bool KDA = false>
 __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
     extern __shared__ __align__(16) char smem[];
     static_assert(bwd_state_smem<VBT, KT>() % 16 == 0, "the second set of tiles starts 16-byte aligned");
-    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4, KDA>(p, smem, threadIdx.x, blockIdx.x);
-    else bwd_dstate_body<T, VBT, KT, 1, 4, KDA>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256, blockIdx.x);
+    if (threadIdx.x < 256) bwd_state_body<T, VBT, KT, 1, 4, KDA>(p, smem, threadIdx.x, blockIdx.x, gridDim.x);
+    else bwd_dstate_body<T, VBT, KT, 1, 4, KDA>(p, smem + bwd_state_smem<VBT, KT>(), threadIdx.x - 256, blockIdx.x, gridDim.x);
 }
 
 // Both scans in one launch, in workgroups of their own: the first `nstate` workgroups walk forwards, the others backwards.
@@ -562,8 +640,8 @@ template <int VBT, int KT> constexpr size_t bwd_scans_apart_smem() {
 template <typename T, int VBT, int KT>
 __global__ __launch_bounds__(256) void gdn_bwd_scans_apart_kernel(BwdParams p, int64_t nstate) {
     extern __shared__ __align__(16) char smem[];
-    if (blockIdx.x >= nstate) bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x - (unsigned)nstate);
-    else bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x);
+    if (blockIdx.x >= nstate) bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x - (unsigned)nstate, gridDim.x - (unsigned)nstate);
+    else bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x, (unsigned)nstate);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1078,7 +1156,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 }
 
 template <typename T, int KT, bool COMBA = false>
-static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream) {
+static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t stream) {
+    BwdParams p = p_in;
     // Value columns per workgroup of the scans: as few as it takes to give every (sequence, head) run its own CU
     // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.  With two
     // blocks of key features the reverse scan's tiles leave room for 32 columns only.
@@ -1104,6 +1183,22 @@ static int launch_bwd(const BwdParams& p, int64_t num_chunks, hipStream_t stream
             state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
             threads[1] = 512;
             dstate.grid = 0;
+        }
+    }
+    // Time segments for the two scans (one block of key features, dense input): long sequences on few heads leave CUs without a
+    // workgroup; never more workgroups than CUs, segments of 8 chunks or more, and at least 24 steps saved per workgroup
+    // (a warm-up of typical length must pay).  GDN_FLAG_SCAN_WIDE asks for whole sequences, GDN_FLAG_SCAN_SEGMENTS for segments of 4.
+    p.nseg = 1; p.seg_chunks = (int)p.NT; p.warm_cap = 0;
+    if constexpr (KT == 1 && !COMBA) {
+        if (!p.cu_seqlens && vbt == 32 && !(p.flags & GDN_FLAG_SCAN_WIDE)) {
+            const bool force = p.flags & GDN_FLAG_SCAN_SEGMENTS;
+            int nseg = (int)std::min<int64_t>(256 / runs(32), p.NT / (force ? 4 : 8));
+            if (nseg >= 2 && (force || p.NT - p.NT / nseg >= 24)) {
+                p.nseg = nseg;
+                p.seg_chunks = (int)((p.NT + nseg - 1) / nseg);
+                p.warm_cap = std::min(WARM_CAP_MAX, p.seg_chunks + p.seg_chunks / 4 + 6);
+                state.grid *= nseg;                             // (vbt = 32: the two scans side by side)
+            }
         }
     }
     int64_t second_arg[5] = {units, units, units, units, units};    // (the kernels that walk over the units take their number)
@@ -1157,8 +1252,8 @@ static int chunk_bwd_entry(
                   "%s: K = 128%s and V = 128 only (got K=%lld V=%lld); pad smaller head dims with zeros", who, comba ? "" : " or 256",
                   (long long)K, (long long)V);
     GDN_CHECK_ARG(qkv_dtype == GDN_DTYPE_BF16 || qkv_dtype == GDN_DTYPE_F16, GDN_ERR_UNSUPPORTED, "%s: q/k/v/do must be bf16 or f16", who);
-    GDN_CHECK_ARG((flags & ~(uint32_t)GDN_FLAG_CU_INT32) == 0, GDN_ERR_UNSUPPORTED,
-                  "%s: only GDN_FLAG_CU_INT32 is understood here (activations and the state layout are the caller's)", who);
+    GDN_CHECK_ARG((flags & ~(uint32_t)(GDN_FLAG_CU_INT32 | GDN_FLAG_SCAN_WIDE | GDN_FLAG_SCAN_SEGMENTS)) == 0, GDN_ERR_UNSUPPORTED,
+                  "%s: only GDN_FLAG_CU_INT32 and the two flags that steer the scans' time segments are understood here (activations and the state layout are the caller's)", who);
     GDN_CHECK_ARG(HV <= 65535 && num_chunks * HV < (1ll << 31) && N * HV * 4 < (1ll << 31), GDN_ERR_UNSUPPORTED,
                   "%s: too many heads or chunks for one launch", who);
     if (cu_seqlens) {
@@ -1188,6 +1283,7 @@ static int chunk_bwd_entry(
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    p.nseg = 1; p.seg_chunks = (int)p.NT; p.warm_cap = 0;
     if (comba) return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 1, true>(p, num_chunks, s) : launch_bwd<f16_t, 1, true>(p, num_chunks, s);
     if (K == BD) return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 1>(p, num_chunks, s) : launch_bwd<f16_t, 1>(p, num_chunks, s);
     return qkv_dtype == GDN_DTYPE_BF16 ? launch_bwd<bf16_t, 2>(p, num_chunks, s) : launch_bwd<f16_t, 2>(p, num_chunks, s);
@@ -1273,6 +1369,7 @@ extern "C" int gdn_chunk_kda_bwd(
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
+    p.nseg = 1; p.seg_chunks = (int)p.NT; p.warm_cap = 0;
     // the forward's chunk-parallel kernel again, writing into this workspace (u where the scan will put v_new)
     KdaParams kp;
     kp.q = q; kp.k = k; kp.v = v; kp.g = g; kp.beta = beta; kp.pk = nullptr; kp.gs = nullptr;

@@ -6,6 +6,8 @@ again).  The activations the forward kernels apply themselves (l2 norm of q and 
 their derivatives are elementwise work around that call, as in the reference (chunk.py:278-288, 385-393)."""
 from __future__ import annotations
 
+import os
+
 import torch
 import torch.nn.functional as F
 
@@ -103,7 +105,9 @@ def chunk_gated_delta_rule_bwd(
         return aligned16(F.pad(s, (0, _DIM - V, 0, KD - K)).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
-    flags = 0
+    # FLA_HIP_BWD_SCAN_MODE forces one form of the two scans (default: automatic): whole sequences ('wide') or time segments
+    # wherever they are possible at all ('segments')
+    flags = {'wide': _lib.FLAG_SCAN_WIDE, 'segments': _lib.FLAG_SCAN_SEGMENTS}.get(os.environ.get('FLA_HIP_BWD_SCAN_MODE', 'auto'), 0)
     chunk_table = chunk_offsets = None
     if cu_seqlens is not None:
         if cu_seqlens.dtype not in (torch.int32, torch.int64):

@@ -413,3 +413,32 @@ def test_chunk_backward_c_entry_checks():
         from fla_hip.ops.gated_delta_rule.chunk_bwd import chunk_gated_delta_rule_bwd
         w = torch.zeros(1, 64, 1, 264, dtype=torch.bfloat16, device='cuda')
         chunk_gated_delta_rule_bwd(w, w, w, f, f, 1.0, None, w, None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,gate_div,h0_std,forced', [
+    (1, 2048, 2, 4, 2.0, 0.5, False),       # 16 workgroups of the scans: 4 segments of 8 chunks, automatic
+    (2, 1100, 2, 2, 1.0, 0.5, True),        # ragged last chunk, segments of 4 chunks forced
+    (1, 1024, 1, 2, 512.0, 0.5, True),      # hardly any decay: no segment may start warm, segment 0's workgroups walk the sequence
+    (1, 1536, 2, 2, 16.0, None, True),      # slower decay: warm-ups of several chunks, the first and last reach the ends of the sequence
+])
+def test_chunk_backward_time_segments(B, T, H, HV, gate_div, h0_std, forced, monkeypatch):
+    """The two scans cut into time segments that start from a zero state where the chunks' transition bounds allow it:
+    against the oracle, and against the same call with whole sequences (equal up to what a warm start forgets, 2^-32)."""
+    D = 128
+    q, k, v, g, beta, h0 = O.make_inputs(B, T, H, HV, D, D, seed=T, gate_div=gate_div, h0_std=h0_std)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    gen = torch.Generator().manual_seed(T + 1)
+    do = torch.randn(B, T, HV, D, generator=gen).bfloat16()
+    dht = torch.randn(B, HV, D, D, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, dtype=torch.float32)
+    got = {}
+    for mode in ('segments' if forced else 'auto', 'wide'):
+        monkeypatch.setenv('FLA_HIP_BWD_SCAN_MODE', mode)
+        _, _, got[mode] = _grads_gpu(q, k, v, g, beta, h0, do, dht)
+        _compare(ref, got[mode])
+    a, b = got['segments' if forced else 'auto'], got['wide']
+    for n in a:
+        if a[n] is not None:
+            assert O.get_err_ratio(b[n].float().cpu(), a[n].float().cpu()) < 2e-3, n
+
