@@ -130,19 +130,23 @@ __device__ __forceinline__ int64_t pad_steps_of(const ScanPlan& sp) { return (sp
 // ---------------------------------------------------------------------------------------------
 // prepare
 // ---------------------------------------------------------------------------------------------
+// (comba: a third tile of rows, those of p; the matrix L then takes the place of the q tile once q has been used, which keeps a
+// workgroup at 80 KB: two per CU)
 template <int KT, bool COMBA = false> constexpr size_t bwd_prep_smem() {
-    return ((2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + (64 * PL + 192) * 4;
+    return ((2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + ((COMBA ? 0 : 64 * PL) + 192) * 4;
 }
 
 template <typename T, int KT, bool COMBA = false>
-__global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
+__global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int KD = BD * KT, PK = KD + 8;
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sV = sQ + 64 * PK; T* sA = sV + 64 * P128;
     T* sP = sA + 64 * P64;                                       // (comba) rows of the second key
-    float* sL = (float*)(sP + (COMBA ? 64 * PK : 0)); float* sGam = sL + 64 * PL; float* sBeta = sGam + 64; float* sGam0 = sBeta + 64;
+    static_assert(!COMBA || 64 * PL * 4 <= 64 * PK * 2, "the matrix L fits the q tile");
+    float* sL = COMBA ? (float*)sQ : (float*)sP;
+    float* sGam = COMBA ? (float*)(sP + 64 * PK) : sL + 64 * PL; float* sBeta = sGam + 64; float* sGam0 = sBeta + 64;
     T* sRows = COMBA ? sP : sK;                                  // the rows that enter L from the left and w
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
@@ -206,6 +210,7 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
         // strip of 16 token rows per wave: L (fp32, for the substitution; entry (i, j) at [i][j % 4][j / 4]) and P^T
         {
             T* PTu = (T*)p.ws.PT + u * 64 * 64;
+            f32x4 lrow[COMBA ? 4 : 1];                          // (comba) this wave's entries of L, until q's tile is free for them
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
                 f32x4 kk = ZERO4, qk = ZERO4;
@@ -225,10 +230,22 @@ __global__ __launch_bounds__(256, KT == 1 && !COMBA ? 2 : 1) void gdn_bwd_prepar
                     const int i = 16 * w + 4 * g + r;
                     const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
                     const float d0 = !COMBA ? d : i > j ? __expf(sGam0[i] - gj) : 0.f;
-                    if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = i > j ? sBeta[i] * kk[r] * d0 : 0.f;
+                    const float l = i > j ? sBeta[i] * kk[r] * d0 : 0.f;
+                    if constexpr (COMBA) lrow[tj][r] = l;
+                    else if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = l;
                     pt[r] = p.scale * qk[r] * d;
                 }
                 *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
+            }
+            if constexpr (COMBA) {
+                lds_barrier();                                  // (every wave has read its rows of q)
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj) {
+                    const int j = 16 * tj + c16;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (tj <= w) sL[(16 * w + 4 * g + r) * PL + (j & 3) * 16 + (j >> 2)] = lrow[tj][r];
+                }
             }
         }
         lds_barrier();
@@ -1209,7 +1226,7 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         dstate.grid = 0;
     }
     const K ks[5] = {
-        {(const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 && !COMBA ? 512u : 256u) ? units : (KT == 1 && !COMBA ? 512u : 256u)},
+        {(const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
         dstate,
         {(const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
