@@ -213,6 +213,7 @@ class ChunkCombaFunction(torch.autograd.Function):
         qn, kn, pn = q, k, p
         if l2:
             (qn, q_rstd), (kn, k_rstd), (pn, p_rstd) = l2norm_fwd(q), l2norm_fwd(k), l2norm_fwd(p)
+            qn, kn, pn = (x[..., :q.shape[-1]] for x in (qn, kn, pn))     # (l2norm_fwd pads rows to a multiple of 8)
         dq, dk, dv, dp, db, dg, dh0 = chunk_comba_bwd(qn, kn, v, pn, g, beta, scale, h0, do.contiguous(), dht, cu_seqlens,
                                                       cu_seqlens_cpu, q_rstd, k_rstd, p_rstd)
         K = q.shape[-1]

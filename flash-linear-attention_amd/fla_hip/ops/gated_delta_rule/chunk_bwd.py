@@ -213,6 +213,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         if l2:
             q, q_rstd = l2norm_fwd(q)
             k, k_rstd = l2norm_fwd(k)
+            q, k = q[..., :K], k[..., :K]                  # (l2norm_fwd pads rows to a multiple of 8)
         beta = beta_raw
         if bsig:
             beta = torch.sigmoid(beta_raw.float()) * (2.0 if neg else 1.0)

@@ -282,6 +282,7 @@ class ChunkKDAFunction(torch.autograd.Function):
         qn, kn = q, k
         if l2:
             (qn, q_rstd), (kn, k_rstd) = l2norm_fwd(q), l2norm_fwd(k)
+            qn, kn = qn[..., :q.shape[-1]], kn[..., :k.shape[-1]]       # (l2norm_fwd pads rows to a multiple of 8)
         beta = beta_raw
         if bsig:
             beta = torch.sigmoid(beta_raw.float()) * (2.0 if neg else 1.0)
