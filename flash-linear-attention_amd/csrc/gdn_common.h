@@ -89,4 +89,47 @@ __device__ __forceinline__ float sigmoid_stream(float x) {
     return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
+// Asynchronous copy of 64 x 16 bytes from global memory straight into LDS: lane l fetches the
+// 16 bytes at gbase + voff (gbase wave-uniform, voff per lane) and they land at the
+// wave-uniform LDS byte offset `lds_off` + 16 l.  Issued from inline assembly on purpose: the
+// compiler then keeps no account of it, and completion is awaited explicitly with s_waitcnt
+// vmcnt before the barrier that publishes the data.
+__device__ __forceinline__ void gather_1k_to_lds(const char* gbase, uint32_t voff, uint32_t lds_off) {
+    lds_off = __builtin_amdgcn_readfirstlane(lds_off);          // wave-uniform by construction; make them scalars
+    const uint64_t g = (uint64_t)gbase;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+    const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_off), "v"(voff), "s"(gs));
+}
+
+// The same copy for the lanes named by `mask` only (the others leave their 16 bytes of LDS as they are).
+// The instruction is issued whatever the mask, so counts of outstanding operations do not depend on it.
+__device__ __forceinline__ void gather_1k_to_lds_masked(const char* gbase, uint32_t voff, uint32_t lds_off, uint64_t mask) {
+    lds_off = __builtin_amdgcn_readfirstlane(lds_off);
+    const uint64_t g = (uint64_t)gbase;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)g), hi = __builtin_amdgcn_readfirstlane((uint32_t)(g >> 32));
+    const uint64_t gs = ((uint64_t)hi << 32) | lo;
+    const uint32_t mlo = __builtin_amdgcn_readfirstlane((uint32_t)mask), mhi = __builtin_amdgcn_readfirstlane((uint32_t)(mask >> 32));
+    mask = ((uint64_t)mhi << 32) | mlo;                         // wave-uniform by construction; make it scalar registers
+    uint64_t saved;
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_and_saveexec_b64 %0, %4\n\t"
+                 "global_load_lds_dwordx4 %2, %3\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved) : "s"(lds_off), "v"(voff), "s"(gs), "s"(mask) : "scc");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm_at_most() {
+    static_assert(N >= 0 && N <= 63, "the vector-memory counter has 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Workgroup barrier that only waits for this wave's LDS traffic.  __syncthreads() also drains
+// the vector-memory counter, which would serialise the global prefetch of later chunks
+// behind every barrier of the current one.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 }  // namespace gdn

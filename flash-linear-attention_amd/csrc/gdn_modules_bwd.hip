@@ -4,6 +4,7 @@
 // fla/modules/fused_norm_gate.py:541-650, kernels :192-453).  Both stream their operands once; the gradients of the
 // parameters leave each workgroup as a row of partial sums in fp32 that the caller adds up (the reference does the same).
 #include "gdn_common.h"
+#include <type_traits>
 
 namespace gdn {
 
@@ -13,11 +14,15 @@ namespace gdn {
 //   dz[t] = dy[t] act'(z[t]);  dx[t] = sum_j w[j] dz[t + (W-1) - j]  (+ dht where t is one of the last W positions);
 //   dw[j] = sum_t dz[t] x[t - (W-1) + j];  db = sum_t dz[t];  positions in front of the sequence belong to the initial state
 // ---------------------------------------------------------------------------------------------
-constexpr int CB_TOK = 8, CB_CX = 32, CB_TY = 8;       // a thread: 2 channels x 8 positions; a workgroup: 32 channel pairs x 64 tokens
-constexpr int CB_VEC = 2;                              // Two channels keep a thread at 134 registers (three waves per SIMD); measured for bf16 at
-                                                       // 32768 x 3072: 4 channels (232 registers, two waves) 240 us, 2 channels 207 us; 8 channels or 16
-                                                       // positions per thread: one wave per SIMD, 330 - 400 us; four waves by a register cap: spills, slower.
-                                                       // (8 tiles per workgroup, GDN_CONV_BWD_TILES_PER_PART: 202 us against 207 us with 4.)
+constexpr int CB_TOK = 4, CB_CX = 64, CB_TY = 4;       // a thread: 4 channels x 4 positions at a time; a wave: 256 channels; a workgroup: 4 waves
+constexpr int CB_TILE = 64;                            // positions of a tile (the unit of the table for packed input)
+constexpr int CB_VEC = 4;                              // Measured for bf16 at 32768 x 8192 (whole call): 4 channels x 4 positions (183 registers, two waves per
+                                                       // SIMD) 331 us; 2 channels x 8 positions (150 registers, three waves) 338 us, with the next but one strip
+                                                       // requested as well (168 registers) 380 us, with 16 / 4 tiles per workgroup instead of 8: 356 / 389 us.  Forms it replaced: a workgroup per tile of 64
+                                                       // positions, every thread evaluating the W-1 dz behind its own positions again, 404 us; the same with those dz
+                                                       // handed over through LDS (one barrier per tile) 420 - 450 us; tiles copied asynchronously into LDS two ahead
+                                                       // (two barriers per tile) 472 us.  What counted was a loop without tested accesses: with them in the loop the
+                                                       // compiler waits for the newest load before every use, and nothing is in flight while a wave computes.
 constexpr int CB_MAX_W = 8;
 
 struct ConvBwdParams {
@@ -35,13 +40,21 @@ __device__ __forceinline__ float silu_grad(float z) {
     return s * (1.f + z * (1.f - s));
 }
 
-// What a thread needs of one tile: the inputs at its 8 positions, the W-1 in front (for z) and the W-1 behind them (for
-// the dz its last inputs feed), and the output gradients at its positions and the W-1 behind them.
+// A number that is the same in every lane, moved to scalar registers: what is derived from it (the rows' base addresses,
+// the step from row to row) is then scalar arithmetic, and a row is addressed as scalar base + one 32-bit lane offset.
+__device__ __forceinline__ int64_t uniform_i64(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// What a thread needs of one tile: the inputs at its 8 positions and the W-1 in front of them (for z), and the output
+// gradients at its positions.  The dz of the W-1 positions behind its own, which its last inputs feed as well, come from the
+// thread that owns them (through LDS), not from a second evaluation of the activation.
 template <typename T, int W>
 struct ConvBwdRows {
     typedef T vec_t __attribute__((ext_vector_type(CB_VEC)));
-    vec_t x[CB_TOK + 2 * (W - 1)];     // x[k]: position t0 - (W-1) + k
-    vec_t dy[CB_TOK + W - 1];          // dy[i]: position t0 + i
+    vec_t x[CB_TOK + W - 1];           // x[k]: position t0 - (W-1) + k
+    vec_t dy[CB_TOK];                  // dy[i]: position t0 + i
 };
 struct ConvBwdTile { int64_t n, it, bos, len; };
 
@@ -54,153 +67,358 @@ __device__ __forceinline__ ConvBwdTile conv_bwd_tile(const ConvBwdParams& p, int
     } else {
         g.n = tile / p.NT; g.it = tile % p.NT; g.bos = g.n * p.T; g.len = p.T;
     }
+    g.n = uniform_i64(g.n); g.it = uniform_i64(g.it); g.bos = uniform_i64(g.bos); g.len = uniform_i64(g.len);
     return g;
 }
 
-// Tiles inside their sequence with W-1 positions in front and W behind them are read without a test, so that all the loads
-// of a thread are in flight together; the others (starts and ends of sequences) test every row, and read the initial
-// state where a position lies in front of the sequence.
-template <typename T, int W>
-__device__ __forceinline__ void conv_bwd_fetch(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, ConvBwdRows<T, W>& r) {
-    constexpr int VEC = CB_VEC, NX = CB_TOK + 2 * (W - 1), NZ = CB_TOK + W - 1;
+// The input at position s of the tile's sequence as the convolution sees it: the initial state in front of the sequence,
+// zero behind it.
+template <typename T>
+__device__ __forceinline__ float conv_bwd_input(const ConvBwdParams& p, const ConvBwdTile& g, const T* xs, int c, int W, int64_t s) {
+    if (s >= 0) return s < g.len ? (float)xs[s * p.stride_t] : 0.f;
+    if (s < -(int64_t)(W - 1) || !p.initial_state) return 0.f;
+    return load_scalar(p.initial_state, (g.n * p.D + c) * (int64_t)W + (W + s), p.state_dtype);
+}
+
+// Tiles that lie inside their sequence with W-1 positions in front are read without a test, so that all the loads of a
+// thread are in flight together; the others (starts and ends of sequences) test every row, and read the initial state
+// where a position lies in front of the sequence.
+// With `held` (the strip behind this one in the same tile) the last W-1 rows of x are that strip's first W-1.
+template <typename T, int W, bool HELD = false>
+__device__ __forceinline__ void conv_bwd_fetch(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, ConvBwdRows<T, W>& r,
+                                               const ConvBwdRows<T, W>& held) {
+    constexpr int VEC = CB_VEC, NX = CB_TOK + W - 1, nx = HELD ? CB_TOK : NX;
+    if constexpr (HELD) {
+#pragma unroll
+        for (int m = 0; m < W - 1; ++m) r.x[CB_TOK + m] = held.x[m];
+    }
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int D = (int)p.D;
-    const int64_t t0 = g.it * (CB_TOK * CB_TY) + ty * CB_TOK;
-    const T* xs = (const T*)p.x + (p.cu_seqlens ? g.bos * p.stride_t : g.n * p.stride_n) + c0;
-    const T* dys = (const T*)p.dy + g.bos * D + c0;
-    if (g.it > 0 && (g.it + 1) * (CB_TOK * CB_TY) + W <= g.len) {
+    if (g.it > 0 && (g.it + 1) * CB_TILE <= g.len) {
+        // rows of the tile: a base that is the same for every lane (scalar registers, scalar arithmetic from row to row)
+        // and one 32-bit offset per lane (the entry point bounds the strides accordingly)
+        const char* xrow = (const char*)((const T*)p.x + (p.cu_seqlens ? g.bos * p.stride_t : g.n * p.stride_n)
+                                         + (g.it * CB_TILE - (W - 1)) * p.stride_t);
+        const char* dyrow = (const char*)((const T*)p.dy + (g.bos + g.it * CB_TILE) * D);
+        const uint32_t xoff = (uint32_t)((ty * CB_TOK) * (int)p.stride_t + c0) * (uint32_t)sizeof(T);
+        const uint32_t dyoff = (uint32_t)((ty * CB_TOK) * D + c0) * (uint32_t)sizeof(T);
 #pragma unroll
-        for (int k = 0; k < NX; ++k) r.x[k] = *(const vec_t*)(xs + (t0 - (W - 1) + k) * p.stride_t);
+        for (int k = 0; k < NX; ++k)
+            if (k < nx) r.x[k] = *(const vec_t*)(xrow + (int64_t)k * p.stride_t * (int64_t)sizeof(T) + xoff);
 #pragma unroll
-        for (int i = 0; i < NZ; ++i) r.dy[i] = *(const vec_t*)(dys + (t0 + i) * D);
+        for (int i = 0; i < CB_TOK; ++i) r.dy[i] = *(const vec_t*)(dyrow + (int64_t)i * D * (int64_t)sizeof(T) + dyoff);
         return;
     }
+    const int64_t t0 = g.it * CB_TILE + ty * CB_TOK;
+    const T* xs = (const T*)p.x + (p.cu_seqlens ? g.bos * p.stride_t : g.n * p.stride_n) + c0;
+    const T* dys = (const T*)p.dy + g.bos * D + c0;
 #pragma unroll
     for (int k = 0; k < NX; ++k) {
         const int64_t s = t0 - (W - 1) + k;
+        if (k >= nx) continue;
         r.x[k] = vec_t{};
         if (s >= 0 && s < g.len) r.x[k] = *(const vec_t*)(xs + s * p.stride_t);
-        else if (s < 0 && s >= -(W - 1) && p.initial_state) {
+        else if (s < 0 && p.initial_state) {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) r.x[k][e] = (T)load_scalar(p.initial_state, (g.n * D + c0 + e) * (int64_t)W + (W + s), p.state_dtype);
+            for (int e = 0; e < VEC; ++e) r.x[k][e] = (T)conv_bwd_input<T>(p, g, xs + e, c0 + e, W, s);
         }
     }
 #pragma unroll
-    for (int i = 0; i < NZ; ++i) {
+    for (int i = 0; i < CB_TOK; ++i) {
         r.dy[i] = vec_t{};
         if (t0 + i < g.len) r.dy[i] = *(const vec_t*)(dys + (t0 + i) * D);
     }
 }
 
-// The thread's 8 positions and the W-1 behind them in order, with the last W values of dz in registers (the loop is
-// unrolled, so the window moves by renaming): dz[s] = dy[s] act'(z[s]);  dx[u] = sum_j w[j] dz[u + (W-1) - j].
+// dz[s] = dy[s] act'(z[s]) at the thread's 8 positions, with the sums for the parameters.
+template <typename T, int W, bool ACT>
+__device__ __forceinline__ void conv_bwd_dz(const ConvBwdRows<T, W>& r, const float (&wgt)[W][CB_VEC],
+                                            const float (&bias)[CB_VEC], float (&dz)[CB_TOK + W - 1][CB_VEC],
+                                            float (&dwacc)[W][CB_VEC], float (&dbacc)[CB_VEC]) {
+#pragma unroll
+    for (int i = 0; i < CB_TOK; ++i)
+#pragma unroll
+        for (int e = 0; e < CB_VEC; ++e) {
+            float xf[W];
+#pragma unroll
+            for (int j = 0; j < W; ++j) xf[j] = (float)r.x[i + j][e];
+            float d = (float)r.dy[i][e];                        // (zero past the end of the sequence)
+            if constexpr (ACT) {
+                float z = bias[e];
+#pragma unroll
+                for (int j = 0; j < W; ++j) z += wgt[j][e] * xf[j];
+                d *= silu_grad(z);
+            }
+            dz[i][e] = d;
+#pragma unroll
+            for (int j = 0; j < W; ++j) dwacc[j][e] += d * xf[j];
+            dbacc[e] += d;
+        }
+}
+
+// dz at the W-1 positions from t1 on, evaluated from memory: only where no thread has just formed them (the strip a wave
+// starts with).
 template <typename T, int W>
-__device__ __forceinline__ void conv_bwd_walk(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, const ConvBwdRows<T, W>& r,
-                                              const float (&wgt)[W][CB_VEC], const float (&bias)[CB_VEC],
-                                              float (&dwacc)[W][CB_VEC], float (&dbacc)[CB_VEC]) {
+__device__ __forceinline__ void conv_bwd_dz_behind(const ConvBwdParams& p, const ConvBwdTile& g, int64_t t1, int c0, const float (&wgt)[W][CB_VEC],
+                                                   const float (&bias)[CB_VEC], float (&out)[W > 1 ? W - 1 : 1][CB_VEC]) {
+    const int D = (int)p.D;
+    const T* xs = (const T*)p.x + (p.cu_seqlens ? g.bos * p.stride_t : g.n * p.stride_n) + c0;
+    const T* dys = (const T*)p.dy + g.bos * D + c0;
+#pragma unroll
+    for (int i = 0; i < W - 1; ++i)
+#pragma unroll
+        for (int e = 0; e < CB_VEC; ++e) {
+            float d = 0.f;
+            if (t1 + i < g.len) {
+                d = (float)dys[(t1 + i) * D + e];
+                if (p.act) {
+                    float z = bias[e];
+#pragma unroll
+                    for (int j = 0; j < W; ++j) z += wgt[j][e] * conv_bwd_input<T>(p, g, xs + e, c0 + e, W, t1 + i - (W - 1) + j);
+                    d *= silu_grad(z);
+                }
+            }
+            out[i][e] = d;
+        }
+}
+
+// dx[u] = sum_j w[j] dz[u + (W-1) - j] at the thread's 8 positions (+ dht where u is one of the sequence's last W).
+template <typename T, int W>
+__device__ __forceinline__ void conv_bwd_dx(const ConvBwdParams& p, const ConvBwdTile& g, int ty, int c0, const float (&wgt)[W][CB_VEC],
+                                            const float (&dz)[CB_TOK + W - 1][CB_VEC]) {
     constexpr int VEC = CB_VEC;
     typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const int D = (int)p.D;
-    const int64_t t0 = g.it * (CB_TOK * CB_TY) + ty * CB_TOK, len = g.len;
+    const int64_t t0 = g.it * CB_TILE + ty * CB_TOK, len = g.len;
+    if ((g.it + 1) * CB_TILE <= len - (p.dht ? W : 0)) {   // a whole tile that the final state does not reach
+        char* row = (char*)((T*)p.dx + (g.bos + g.it * CB_TILE) * D);
+        const uint32_t off = (uint32_t)((ty * CB_TOK) * D + c0) * (uint32_t)sizeof(T);
+#pragma unroll
+        for (int i = 0; i < CB_TOK; ++i) {
+            vec_t out;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                float a = 0.f;
+#pragma unroll
+                for (int j = 0; j < W; ++j) a += wgt[j][e] * dz[i + (W - 1) - j][e];
+                out[e] = (T)a;
+            }
+            *(vec_t*)(row + (int64_t)i * D * (int64_t)sizeof(T) + off) = out;
+        }
+        return;
+    }
     T* dxs = (T*)p.dx + g.bos * D + c0;
-    float dzw[W][VEC];                                          // dzw[j]: dz at position s - j
 #pragma unroll
-    for (int j = 0; j < W; ++j)
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) dzw[j][e] = 0.f;
-#pragma unroll
-    for (int i = 0; i < CB_TOK + W - 1; ++i) {
-        const int64_t s = t0 + i;
-#pragma unroll
-        for (int j = W - 1; j > 0; --j)
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) dzw[j][e] = dzw[j - 1][e];
+    for (int i = 0; i < CB_TOK; ++i) {
+        const int64_t u = t0 + i;
+        if (u >= len) continue;
+        const bool in_final = p.dht && u >= len - W;            // this input is also entry u - (len - W) of the final state
+        vec_t out;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            float d = (float)r.dy[i][e];                        // (zero past the end of the sequence)
-            if (p.act) {
-                float z = bias[e];
+            float a = 0.f;
 #pragma unroll
-                for (int j = 0; j < W; ++j) z += wgt[j][e] * (float)r.x[i + j][e];
-                d *= silu_grad(z);
-            }
-            dzw[0][e] = d;
-            if (i < CB_TOK) {                                   // (positions past this thread's own belong to the next thread's sums)
-#pragma unroll
-                for (int j = 0; j < W; ++j) dwacc[j][e] += d * (float)r.x[i + j][e];
-                dbacc[e] += d;
-            }
+            for (int j = 0; j < W; ++j) a += wgt[j][e] * dz[i + (W - 1) - j][e];
+            if (in_final) a += (float)((const T*)p.dht)[(g.n * D + c0 + e) * (int64_t)W + (u - (len - W))];
+            out[e] = (T)a;
         }
-        if (i >= W - 1) {
-            const int64_t u = s - (W - 1);
-            if (u < len) {
-                const bool in_final = p.dht && u >= len - W;    // this input is also entry u - (len - W) of the final state
+        *(vec_t*)(dxs + u * D) = out;
+    }
+}
+
+// A workgroup takes GDN_CONV_BWD_TILES_PER_PART consecutive tiles of its channels and keeps the sums for the parameters in
+// registers across them: one row of partial sums per such run.  Each of its four waves owns a quarter of the run's
+// positions and walks over it in strips of CB_TOK positions, LAST FIRST, with the rows of the next strip on their way into
+// registers while it works on the current one; the waves never wait for each other and nothing passes through LDS.
+// Walking backwards, a thread has just formed the W-1 dz behind its positions itself (only a wave's first strip evaluates
+// them from memory), and inside a tile it already holds the W-1 rows of x in front of the strip it leaves.
+template <typename T, int W>
+__global__ __launch_bounds__(CB_CX * CB_TY, 2) void causal_conv1d_bwd_kernel(ConvBwdParams p) {
+    constexpr int VEC = CB_VEC, H = W > 1 ? W - 1 : 1, STRIPS = CB_TILE / CB_TOK;      // strips of a tile
+    static_assert(CB_CX == 64 && STRIPS % CB_TY == 0, "one wave per row of the block; the waves share a run evenly");
+    __shared__ float red[W + 1][CB_TY][CB_CX * VEC];
+    const int cx = threadIdx.x, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.y);
+    const int D = (int)p.D;
+    const int64_t cblocks = (p.D + CB_CX * VEC - 1) / (CB_CX * VEC);
+    const int64_t part = blockIdx.x / cblocks;
+    const int c0 = (int)((blockIdx.x % cblocks) * CB_CX + cx) * VEC;
+    const bool live = c0 < D;
+
+    float dwacc[W][VEC], dbacc[VEC], wgt[W][VEC], bias[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        dbacc[e] = 0.f;
+        bias[e] = live && p.bias ? load_scalar(p.bias, c0 + e, p.w_dtype) : 0.f;
+#pragma unroll
+        for (int j = 0; j < W; ++j) {
+            dwacc[j][e] = 0.f;
+            wgt[j][e] = live ? load_scalar(p.weight, (int64_t)(c0 + e) * W + j, p.w_dtype) : 0.f;
+        }
+    }
+    const int64_t tile0 = part * GDN_CONV_BWD_TILES_PER_PART, tile_end = min(p.num_tiles, tile0 + GDN_CONV_BWD_TILES_PER_PART);
+    const int per_wave = (int)(tile_end - tile0) * (STRIPS / CB_TY);     // strips per wave
+    const int s_last = (wave + 1) * per_wave - 1;               // strip s of the run: tile tile0 + s / STRIPS, positions CB_TOK (s % STRIPS) ...
+    const ConvBwdTile ga = conv_bwd_tile(p, tile0 + (s_last - (per_wave - 1)) / STRIPS), gb = conv_bwd_tile(p, tile0 + s_last / STRIPS);
+    // The wave's strips lie in one sequence, the first of them W-1 positions or more from its start, the last one clear of
+    // the positions that also feed the final state: nothing to test in the loop, whose waits for loads the compiler then
+    // counts exactly (with the tested accesses of the other loop in it, it waits for the newest load before every use).
+    const bool plain = ga.n == gb.n && gb.it - ga.it == (s_last / STRIPS) - ((s_last - (per_wave - 1)) / STRIPS) && ga.it > 0 &&
+                       (gb.it + 1) * CB_TILE <= gb.len - (p.dht ? W : 0) && per_wave > 1;
+    if (live && plain) {
+        typedef T vec_t __attribute__((ext_vector_type(VEC)));
+        int64_t pos = gb.it * CB_TILE + (s_last % STRIPS) * CB_TOK;      // first position of the strip in hand
+        const int64_t xstep = p.stride_t * (int64_t)sizeof(T), dstep = (int64_t)D * (int64_t)sizeof(T);
+        const uint32_t coff = (uint32_t)c0 * (uint32_t)sizeof(T);
+        const char* xseq = (const char*)((const T*)p.x + (p.cu_seqlens ? gb.bos * p.stride_t : gb.n * p.stride_n));
+        const char* dyseq = (const char*)((const T*)p.dy + gb.bos * D);
+        char* dxseq = (char*)((T*)p.dx + gb.bos * D);
+        vec_t xr[CB_TOK + W - 1], dyr[CB_TOK], xn[CB_TOK], dyn[CB_TOK];
+#pragma unroll
+        for (int k = 0; k < CB_TOK + W - 1; ++k) xr[k] = *(const vec_t*)(xseq + (pos - (W - 1) + k) * xstep + coff);
+#pragma unroll
+        for (int i = 0; i < CB_TOK; ++i) dyr[i] = *(const vec_t*)(dyseq + (pos + i) * dstep + coff);
+        float first[H][VEC];                                    // the first W-1 dz of the strip behind the one in hand
+        if constexpr (W > 1) {
+            // from rows of their own: x up to position pos + CB_TOK - 1 is in hand, past the end of the sequence everything is zero
+            vec_t xb[W - 1], dyb[W - 1];
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i) {
+                xb[i] = vec_t{}; dyb[i] = vec_t{};
+                if (pos + CB_TOK + i < gb.len) {
+                    xb[i] = *(const vec_t*)(xseq + (pos + CB_TOK + i) * xstep + coff);
+                    dyb[i] = *(const vec_t*)(dyseq + (pos + CB_TOK + i) * dstep + coff);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float d = (float)dyb[i][e];
+                    if (p.act) {
+                        float z = bias[e];
+#pragma unroll
+                        for (int j = 0; j < W; ++j) {           // input at position pos + CB_TOK + i - (W-1) + j
+                            const int k = CB_TOK + i + j;       // as an index into xr (position pos - (W-1) + k)
+                            z += wgt[j][e] * (k < CB_TOK + W - 1 ? (float)xr[k < CB_TOK + W - 1 ? k : 0][e] : (float)xb[k - (CB_TOK + W - 1) < W - 1 ? k - (CB_TOK + W - 1) : 0][e]);
+                        }
+                        d *= silu_grad(z);
+                    }
+                    first[i][e] = d;
+                }
+        }
+        auto step = [&](auto ahead, auto act) {
+            if constexpr (decltype(ahead)::value) {
+#pragma unroll
+                for (int k = 0; k < CB_TOK; ++k) xn[k] = *(const vec_t*)(xseq + (pos - CB_TOK - (W - 1) + k) * xstep + coff);
+#pragma unroll
+                for (int i = 0; i < CB_TOK; ++i) dyn[i] = *(const vec_t*)(dyseq + (pos - CB_TOK + i) * dstep + coff);
+            }
+            float dz[CB_TOK + W - 1][VEC];
+#pragma unroll
+            for (int i = 0; i < CB_TOK; ++i)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float xf[W];
+#pragma unroll
+                    for (int j = 0; j < W; ++j) xf[j] = (float)xr[i + j][e];
+                    float d = (float)dyr[i][e];
+                    if constexpr (decltype(act)::value) {
+                        float z = bias[e];
+#pragma unroll
+                        for (int j = 0; j < W; ++j) z += wgt[j][e] * xf[j];
+                        d *= silu_grad(z);
+                    }
+                    dz[i][e] = d;
+#pragma unroll
+                    for (int j = 0; j < W; ++j) dwacc[j][e] += d * xf[j];
+                    dbacc[e] += d;
+                }
+#pragma unroll
+            for (int i = 0; i < W - 1; ++i)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    dz[CB_TOK + i][e] = first[i][e];
+                    first[i][e] = dz[i][e];
+                }
+#pragma unroll
+            for (int i = 0; i < CB_TOK; ++i) {
                 vec_t out;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     float a = 0.f;
 #pragma unroll
-                    for (int j = 0; j < W; ++j) a += wgt[j][e] * dzw[j][e];
-                    if (in_final) a += (float)((const T*)p.dht)[(g.n * D + c0 + e) * (int64_t)W + (u - (len - W))];
+                    for (int j = 0; j < W; ++j) a += wgt[j][e] * dz[i + (W - 1) - j][e];
                     out[e] = (T)a;
                 }
-                *(vec_t*)(dxs + u * D) = out;
+                *(vec_t*)(dxseq + (pos + i) * dstep + coff) = out;
             }
-        }
-    }
-}
-
-// A workgroup takes GDN_CONV_BWD_TILES_PER_PART consecutive tiles of its channels, one after the other, with the rows of the
-// next tile on their way into registers while it works on the current one, and keeps the sums for the parameters in
-// registers across them: one row of partial sums per such run.
-template <typename T, int W>
-__global__ __launch_bounds__(CB_CX * CB_TY, 2) void causal_conv1d_bwd_kernel(ConvBwdParams p) {
-    constexpr int VEC = CB_VEC;
-    __shared__ float red[W + 1][CB_TY][CB_CX * VEC];
-    const int cx = threadIdx.x, ty = threadIdx.y;
-    const int D = (int)p.D;
-    const int64_t cblocks = (p.D + CB_CX * VEC - 1) / (CB_CX * VEC);
-    const int64_t part = blockIdx.x / cblocks;
-    const int c0 = (int)((blockIdx.x % cblocks) * CB_CX + cx) * VEC;
-
-    float dwacc[W][VEC], dbacc[VEC];
+            if constexpr (decltype(ahead)::value) {
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-        dbacc[e] = 0.f;
+                for (int m = W - 2; m >= 0; --m) xr[CB_TOK + m] = xr[m];       // (last first: the two ranges overlap when W - 1 > CB_TOK)
 #pragma unroll
-        for (int j = 0; j < W; ++j) dwacc[j][e] = 0.f;
-    }
-    if (c0 < D) {
-        float wgt[W][VEC], bias[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-#pragma unroll
-            for (int j = 0; j < W; ++j) wgt[j][e] = load_scalar(p.weight, (int64_t)(c0 + e) * W + j, p.w_dtype);
-            bias[e] = p.bias ? load_scalar(p.bias, c0 + e, p.w_dtype) : 0.f;
-        }
-        const int64_t tile0 = part * GDN_CONV_BWD_TILES_PER_PART, tile_end = min(p.num_tiles, tile0 + GDN_CONV_BWD_TILES_PER_PART);
-        ConvBwdRows<T, W> next;
-        ConvBwdTile gnext = conv_bwd_tile(p, tile0);
-        conv_bwd_fetch<T, W>(p, gnext, ty, c0, next);
+                for (int k = 0; k < CB_TOK; ++k) { xr[k] = xn[k]; dyr[k] = dyn[k]; }
+                pos -= CB_TOK;
+            }
+        };
+        if (p.act) {
 #pragma unroll 1
-        for (int64_t tile = tile0; tile < tile_end; ++tile) {
+            for (int n = 0; n + 1 < per_wave; ++n) step(std::true_type{}, std::true_type{});
+            step(std::false_type{}, std::true_type{});
+        } else {
+#pragma unroll 1
+            for (int n = 0; n + 1 < per_wave; ++n) step(std::true_type{}, std::false_type{});
+            step(std::false_type{}, std::false_type{});
+        }
+    } else if (live) {
+        int s = s_last;
+        ConvBwdRows<T, W> next;
+        ConvBwdTile gnext = gb;
+        conv_bwd_fetch<T, W>(p, gnext, s % STRIPS, c0, next, next);
+        float first[H][VEC];                                    // the first W-1 dz of the strip taken before this one
+#pragma unroll 1
+        for (int n = 0; n < per_wave; ++n, --s) {
             const ConvBwdRows<T, W> cur = next;
             const ConvBwdTile g = gnext;
-            if (tile + 1 < tile_end) {
-                gnext = conv_bwd_tile(p, tile + 1);
-                conv_bwd_fetch<T, W>(p, gnext, ty, c0, next);
+            const int ty = s % STRIPS;
+            if (n + 1 < per_wave) {
+                if (ty > 0) conv_bwd_fetch<T, W, true>(p, g, ty - 1, c0, next, cur);
+                else {
+                    gnext = conv_bwd_tile(p, tile0 + (s - 1) / STRIPS);
+                    conv_bwd_fetch<T, W>(p, gnext, STRIPS - 1, c0, next, cur);
+                }
             }
-            __builtin_amdgcn_sched_barrier(0);                  // (the loads are issued here, not where the scheduler finds room for them)
-            conv_bwd_walk<T, W>(p, g, ty, c0, cur, wgt, bias, dwacc, dbacc);
+            float dz[CB_TOK + W - 1][VEC];
+            if (p.act) conv_bwd_dz<T, W, true>(cur, wgt, bias, dz, dwacc, dbacc);
+            else conv_bwd_dz<T, W, false>(cur, wgt, bias, dz, dwacc, dbacc);
+            if constexpr (W > 1) {
+                // the strip behind this one, if the sequence goes on there: what the last step left, or (first step) from memory
+                const int64_t strip_end = g.it * CB_TILE + (ty + 1) * CB_TOK;
+                if (strip_end >= g.len) {
+#pragma unroll
+                    for (int i = 0; i < W - 1; ++i)
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) first[i][e] = 0.f;
+                } else if (n == 0) {
+                    conv_bwd_dz_behind<T, W>(p, g, strip_end, c0, wgt, bias, first);
+                }
+#pragma unroll
+                for (int i = 0; i < W - 1; ++i)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        dz[CB_TOK + i][e] = first[i][e];
+                        first[i][e] = dz[i][e];
+                    }
+            }
+            conv_bwd_dx<T, W>(p, g, ty, c0, wgt, dz);
         }
     }
     // sums over the workgroup's tokens (W taps and the bias), in a fixed order
 #pragma unroll
     for (int q = 0; q <= W; ++q)
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) red[q][ty][cx * VEC + e] = q < W ? dwacc[q < W ? q : 0][e] : dbacc[e];
+        for (int e = 0; e < VEC; ++e) red[q][threadIdx.y][cx * VEC + e] = q < W ? dwacc[q < W ? q : 0][e] : dbacc[e];
     __syncthreads();
-    for (int q = ty; q <= W; q += CB_TY) {
+    for (int q = threadIdx.y; q <= W; q += CB_TY) {
         if (c0 >= D || (q == W && !p.db_part)) continue;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -449,9 +667,11 @@ extern "C" int gdn_causal_conv1d_bwd(
     GDN_CHECK_ARG(!bias == !db_part, GDN_ERR_INVALID, "%s: db_part goes with bias", who);
     GDN_CHECK_ARG(!dh0 || initial_state, GDN_ERR_INVALID, "%s: dh0 needs initial_state", who);
     GDN_CHECK_ARG(D < (1ll << 31) && stride_x_t >= D, GDN_ERR_INVALID, "%s: token stride %lld below D", who, (long long)stride_x_t);
-    const uintptr_t pair = (uintptr_t)CB_VEC * (x_dtype == GDN_DTYPE_F32 ? 4 : 2);     // a thread reads its two channels in one piece
+    GDN_CHECK_ARG(stride_x_t <= (1ll << 24), GDN_ERR_UNSUPPORTED, "%s: token stride %lld above 2^24 elements (a lane's offset inside a tile of 64 tokens is kept in 32 bits)",
+                  who, (long long)stride_x_t);
+    const uintptr_t pair = (uintptr_t)CB_VEC * (x_dtype == GDN_DTYPE_F32 ? 4 : 2);     // a thread reads its channels in one piece
     GDN_CHECK_ARG(D % CB_VEC == 0 && stride_x_t % CB_VEC == 0 && stride_x_n % CB_VEC == 0 && (uintptr_t)x % pair == 0 && (uintptr_t)dy % pair == 0 &&
-                  (uintptr_t)dx % pair == 0, GDN_ERR_UNSUPPORTED, "%s: D and the strides of x must be even and rows must start on %d-byte boundaries", who, (int)pair);
+                  (uintptr_t)dx % pair == 0, GDN_ERR_UNSUPPORTED, "%s: D and the strides of x must be multiples of %d and rows must start on %d-byte boundaries", who, CB_VEC, (int)pair);
     ConvBwdParams p{};
     p.x = x; p.weight = weight; p.bias = bias; p.initial_state = initial_state; p.dy = dy; p.dht = dht;
     p.dx = dx; p.dw_part = dw_part; p.db_part = db_part; p.dh0 = dh0;

@@ -141,9 +141,9 @@ def causal_conv1d_bwd(
         if t is not None and tuple(t.shape) != want:
             raise ValueError(f'{name} must have shape {want}, got {tuple(t.shape)}')
     dy = dy.reshape(B, T, D).to(x.dtype).contiguous()
-    pad = D % 2
-    if pad or x.data_ptr() % (2 * x.element_size()) or x.stride(1) % 2 or x.stride(0) % 2:
-        # the kernel takes two adjacent channels per thread: bring odd layouts to that form
+    pad = -D % 4
+    if pad or x.data_ptr() % (4 * x.element_size()) or x.stride(1) % 4 or x.stride(0) % 4:
+        # the kernel takes four adjacent channels per thread: bring other layouts to that form
         x = F.pad(x, (0, pad)) if pad else x.clone(memory_format=torch.contiguous_format)
         dy = F.pad(dy, (0, pad))
         weight_k = F.pad(weight, (0, 0, 0, pad))

@@ -478,7 +478,7 @@ int gdn_norm_gated_fwd(
  *   dh0 [N,D,W] fp32 or NULL (needs initial_state)
  *   tile_table [num_tiles,2]: (sequence, tile inside it) per 64-token tile of a packed input, in cu_seqlens' integer type
  *   (the chunk table of gdn_chunk_fwd); dense input: NULL and num_tiles = B * ceil(T / 64)
- *   Requires an even D, even strides of x and rows that start on a boundary of two elements.
+ *   Requires D and the strides of x to be multiples of 4 and rows that start on a boundary of four elements.
  */
 #define GDN_CONV_BWD_TILES_PER_PART 8
 int gdn_causal_conv1d_bwd(
