@@ -153,7 +153,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
     // Units in turn; the next unit's rows are fetched into registers while this one is worked on.
     TileRegs<KD> rK, rQ, rP;
     TileRegs<BD> rV;
-    float rG = 0.f, rB = 0.f;
+    uint32_t rG = 0, rB = 0;                                     // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -161,10 +161,10 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-        rG = rB = 0.f;
+        rG = rB = 0;
         if (w == 0 && lane < c.valid) {
-            rG = p.g ? load_scalar(p.g, (c.tok0 + lane) * p.HV + hv, p.gb_dtype) : 0.f;
-            rB = load_scalar(p.beta, (c.tok0 + lane) * p.HV + hv, p.gb_dtype);
+            rG = p.g ? load_scalar_bits(p.g, (c.tok0 + lane) * p.HV + hv, p.gb_dtype) : 0;
+            rB = load_scalar_bits(p.beta, (c.tok0 + lane) * p.HV + hv, p.gb_dtype);
         }
     };
     fetch(blockIdx.x);
@@ -179,16 +179,17 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         put_tile<BD>(sV, P128, rV, tid);
         if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
         if (w == 0) {
-            float x = rG;
+            const float g_own = scalar_of_bits(rG, p.gb_dtype);
+            float x = g_own;
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
                 const float y = __shfl_up(x, off, 64);
                 if (lane >= off) x += y;
             }
-            sGam[lane] = x; sBeta[lane] = rB;
-            sGam0[lane] = COMBA ? x - rG : x;                    // (comba) the sum in front of this token: the prediction sees the state before its decay
+            sGam[lane] = x; sBeta[lane] = scalar_of_bits(rB, p.gb_dtype);
+            sGam0[lane] = COMBA ? x - g_own : x;                 // (comba) the sum in front of this token: the prediction sees the state before its decay
             p.ws.Gam[u * 64 + lane] = x;
-            if constexpr (COMBA) p.ws.Gam0[u * 64 + lane] = x - rG;
+            if constexpr (COMBA) p.ws.Gam0[u * 64 + lane] = x - g_own;
         }
         lds_barrier();
         if (!COMBA && p.nseg > 1 && w == 0) {
@@ -901,7 +902,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     TileRegs<KD> rDW, rK, rP;
     TileRegs<CH> rA;
     V4 rDk[NA][4];                                               // what the previous kernel left in dk, at this lane's places
-    float rGam = 0.f, rBeta = 0.f, rDg = 0.f, rGam0 = 0.f;
+    float rGam = 0.f, rDg = 0.f, rGam0 = 0.f;
+    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -913,7 +915,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if (tid < 64) {
             rGam = p.ws.Gam[u * 64 + tid];
-            rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
             rDg = p.ws.Dgam[u * 64 + tid];
             if constexpr (COMBA) rGam0 = p.ws.Gam0[u * 64 + tid];
         }
@@ -936,7 +938,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         put_tile<KD>(sDW, PK, rDW, tid);
         put_tile<KD>(sK, PK, rK, tid);
         if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = rBeta; sGam0[tid] = rGam0; }
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); sGam0[tid] = rGam0; }
         sDg[tid] = tid < 64 ? rDg : 0.f;
         sDb[tid] = 0.f;
         sDg0[tid] = 0.f;

@@ -45,7 +45,8 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
     // A workgroup walks over the units; the next unit's rows and gates are fetched into registers meanwhile.
     TileRegs<BD> rK, rV;
     V8 rQ[4];                                                   // q: row 16w + c16, features 32s + 8g .. + 7
-    float rG[32], rB = 0.f;                                     // gates: a thread per key feature and half of the chunk's rows
+    float rG[32];                                               // gates: a thread per key feature and half of the chunk's rows
+    uint32_t rB = 0;                                            // (raw bits: converted when the unit's turn comes)
     // (the lane number is an argument: inside the loop over the units it is the opaque copy, see there)
     auto fetch_v = [&](int64_t u, int tid) {
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
             for (int e = 0; e < 8; ++e) rQ[s][e] = (T)0.f;
             if (16 * w + c16 < c.valid) rQ[s] = *(const V8*)((const T*)p.q + ((c.tok0 + 16 * w + c16) * p.H + hq) * BD + 32 * s + 8 * g);
         }
-        rB = (tid < 64 && tid < c.valid) ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        rB = (tid < 64 && tid < c.valid) ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
     };
     auto fetch_g = [&](int64_t u, int tid) {
         const int hv = (int)(u % p.HV);
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256, 2) void gdn_kda_prepare_kernel(KdaParams p, in
         }
     }
     if (tid < 64) {
-        float b = rB;
+        float b = scalar_of_bits(rB, p.gb_dtype);
         if ((p.flags & GDN_FLAG_BETA_SIGMOID) && tid < c.valid) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
         sBeta[tid] = b;
     }
@@ -358,7 +359,7 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
 
     // Two workgroups per CU walk over the units; the next unit's rows and gates are fetched into registers meanwhile.
     TileRegs<BD> rK, rQ, rP, rV;
-    float rG = 0.f, rB = 0.f;
+    uint32_t rG = 0, rB = 0;                                    // (raw bits: converted when the unit's turn comes)
     auto fetch_v = [&](int64_t u) {                             // (on its own, later than the rest: fewer registers live across the substitution)
         const int hv = (int)(u % p.HV);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -371,8 +372,8 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
         fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
         fetch_tile<BD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
         const bool have = tid < 64 && tid < c.valid;
-        rG = have ? load_scalar(p.gs, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
-        rB = have ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        rG = have ? load_scalar_bits(p.gs, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
+        rB = have ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
     };
     fetch(blockIdx.x);
     fetch_v(blockIdx.x);
@@ -387,15 +388,16 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
     put_tile<BD>(sP, P128, rP, tid);
     put_tile<BD>(sV, P128, rV, tid);
     if (w == 0) {
-        float run = rG;                                         // running sum over the chunk's tokens (rows past the end add 0)
+        const float g_own = scalar_of_bits(rG, p.gb_dtype);
+        float run = g_own;                                      // running sum over the chunk's tokens (rows past the end add 0)
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const float t = __shfl_up(run, off, 64);
             if (lane >= off) run += t;
         }
         sGam[lane] = run;
-        sGam0[lane] = run - rG;
-        sBeta[lane] = rB;
+        sGam0[lane] = run - g_own;
+        sBeta[lane] = scalar_of_bits(rB, p.gb_dtype);
     }
     lds_barrier();
     if (u + gridDim.x < units) fetch(u + gridDim.x);

@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
     TileRegs<BD> rDvn, rV, rDW, rK, rQ;
     TileRegs<CH> rA, rDPs;
     f32x4 rG[8];
-    float rBeta = 0.f;
+    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
             const int idx = tid + 256 * i;
             rG[i] = *(const f32x4*)(p.ws.Gk + u * 64 * BD + (idx >> 5) * BD + (idx & 31) * 4);
         }
-        if (tid < 64) rBeta = tid < c.valid ? load_scalar(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0.f;
+        if (tid < 64) rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
     };
     fetch(blockIdx.x);
     const int tid_outer = tid;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
             const int idx = tid + 256 * i;
             *(f32x4*)(sG + (idx >> 5) * PG + (idx & 31) * 4) = rG[i];
         }
-        if (tid < 64) sBeta[tid] = rBeta;
+        if (tid < 64) sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype);
         sDb[tid] = 0.f;
         lds_barrier();
         if (u + gridDim.x < units) fetch(u + gridDim.x);

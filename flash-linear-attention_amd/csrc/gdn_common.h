@@ -73,6 +73,18 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i, int dtype
     return (float)((const f16_t*)p)[i];
 }
 
+// The same number as raw bits (16-bit types in the low half), to be converted where it is used: a load whose result is
+// converted on the spot makes the wave wait there for it and for every load requested before it, which undoes a prefetch.
+__device__ __forceinline__ uint32_t load_scalar_bits(const void* p, int64_t i, int dtype) {
+    if (dtype == GDN_DTYPE_F32) return ((const uint32_t*)p)[i];
+    return ((const uint16_t*)p)[i];
+}
+__device__ __forceinline__ float scalar_of_bits(uint32_t bits, int dtype) {
+    if (dtype == GDN_DTYPE_F32) return __builtin_bit_cast(float, bits);
+    if (dtype == GDN_DTYPE_BF16) return __builtin_bit_cast(float, bits << 16);
+    return (float)__builtin_bit_cast(f16_t, (uint16_t)bits);
+}
+
 __device__ __forceinline__ int64_t load_index(const void* p, int64_t i, bool is_i32) {
     return is_i32 ? (int64_t)((const int32_t*)p)[i] : ((const int64_t*)p)[i];
 }
