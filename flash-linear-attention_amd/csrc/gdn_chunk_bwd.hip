@@ -310,7 +310,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 // current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
 template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
-template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 3 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
+template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 2 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
 // KDA: the rows of k arrive with their decay to the end of the chunk on them (KG), and the state decays per key feature (EGL).
 template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
@@ -469,7 +469,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
     constexpr int PV = VBT + 8, VBQ = VBT / (NW / 4), NB = VBQ / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT, NTH = 64 * NW;
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sW = sQ + 64 * PK; T* sPT = sW + 64 * PK;
-    T* sDO = sPT + 64 * P64; T* sDOg = sDO + 64 * PV; T* sDvn = sDOg + 64 * PV; T* sDS = sDvn + 64 * PV;
+    T* sDO = sPT + 64 * P64; T* sDvn = sDO + 64 * PV; T* sDS = sDvn + 64 * PV;
     float* sGam = (float*)(sDS + KD * PV);
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
@@ -495,7 +495,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             dS[a2][b] = (p.dht && c_top == sq.nc) ? *(const f32x4*)(p.dht + ((n * p.HV + hv) * KD + kk) * BD + vcol0 + vq0 + 16 * b + 4 * g) : ZERO4;
         }
     // (two sets of registers for AHEAD = 2, as in the forward scan)
-    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; };
+    // (the rows of q meet the state's gradient as scale e^gam_i q_i: a thread scales its pieces of the tile on their way into LDS, with
+    // the gam of their rows fetched beside them)
+    constexpr int QN = 64 * (KD / 8) / NTH, QPPR = KD / 8, QRPI = NTH / QPPR;
+    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; float rGq[QN]; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
@@ -513,6 +516,8 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             fetch_tile<KD, NTH>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
             fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
             if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+#pragma unroll
+            for (int i = 0; i < QN; ++i) R.rGq[i] = p.ws.Gam[u * 64 + tid / QPPR + QRPI * i];
         }
         fetch_tile<KD, NTH>(rW, (const T*)p.ws.Wm + u * 64 * KD, KD, 64, tid);
         fetch_tile<VBT, NTH>(rDO, (const T*)p.dout + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, valid, tid);
@@ -522,6 +527,16 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
         const bool keep = ic < c_keep;                          // (chunks of the warm-up belong to another segment: nothing of them is stored)
         put_tile<KD, NTH>(sK, PK, rK, tid);
+        if constexpr (!KDA) {                                   // (KDA: the factors are on the rows of q already)
+#pragma unroll
+            for (int i = 0; i < QN; ++i) {
+                const float f = p.scale * __expf(R.rGq[i]);
+                V8 x = __builtin_bit_cast(V8, rQ.x[i]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
+                rQ.x[i] = __builtin_bit_cast(u32x4, x);
+            }
+        }
         put_tile<KD, NTH>(sQ, PK, rQ, tid);
         put_tile<KD, NTH>(sW, PK, rW, tid);
         put_tile<CH, NTH>(sPT, P64, rPT, tid);
@@ -543,16 +558,6 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         lds_barrier();
         if (ic >= c_lo + AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
-        // scale e^gam_i do_i, for the state's gradient  (KDA: the factors are on the rows of q already)
-        if constexpr (!KDA)
-        for (int idx = tid; idx < 64 * (VBT / 8); idx += NTH) {
-            const int row = idx / (VBT / 8), pc = idx % (VBT / 8);
-            const float f = p.scale * __expf(sGam[row]);
-            V8 x = *(const V8*)(sDO + row * PV + pc * 8);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
-            *(V8*)(sDOg + row * PV + pc * 8) = x;
-        }
         {
             // dv_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int j = 16 * w + c16;
@@ -597,7 +602,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
-                    const V8 fo = frag_cols(KDA ? sDO : sDOg, PV, 32 * s, vq0 + 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, vq0 + 16 * b, lane);
+                    const V8 fo = frag_cols(sDO, PV, 32 * s, vq0 + 16 * b, lane), fv = frag_cols(sDvn, PV, 32 * s, vq0 + 16 * b, lane);
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) {
                         dS[a2][b] = Mma<T>::run(fo, qf[a2][s], dS[a2][b]);
@@ -1197,9 +1202,11 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
     }
     unsigned threads[5] = {256, vbt == BD ? 512u : 256u, vbt_d == BD ? 512u : 256u, 256, 256};
     if constexpr (KT == 1) {
-        if (vbt == 32) {
-            // both scans side by side in one launch (the second entry then has nothing to launch)
-            state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
+        // both scans side by side in one launch (the second entry then has nothing to launch)
+        static_assert(bwd_scans_smem<64, 1>() <= 160 * 1024, "the two scans' tiles of 64 value columns share a CU's LDS");
+        if (vbt == 32) state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
+        if (vbt == 64) state = {(const void*)gdn_bwd_scans_kernel<T, 64, KT>, bwd_scans_smem<64, KT>(), "gdn_bwd_scans_kernel", runs(64)};
+        if (vbt <= 64) {
             threads[1] = 512;
             dstate.grid = 0;
         }

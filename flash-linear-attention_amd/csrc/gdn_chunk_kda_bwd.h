@@ -601,8 +601,8 @@ static int launch_bwd_kda(const BwdParams& p, const KdaParams& kp, int64_t num_c
         state = {(const void*)gdn_bwd_scans_kernel<T, 32, 1, true>, bwd_scans_smem<32, 1>(), "gdn_bwd_scans_kernel", runs(32), 512};
         dstate = {nullptr, 0, "", 0, 0};
     } else if (vbt == 64) {
-        state = {(const void*)gdn_bwd_state_kernel<T, 64, 1, true>, bwd_state_smem<64, 1>(), "gdn_bwd_state_kernel", runs(64), 256};
-        dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, 1, true>, bwd_dstate_smem<64, 1>(), "gdn_bwd_dstate_kernel", runs(64), 256};
+        state = {(const void*)gdn_bwd_scans_kernel<T, 64, 1, true>, bwd_scans_smem<64, 1>(), "gdn_bwd_scans_kernel", runs(64), 512};
+        dstate = {nullptr, 0, "", 0, 0};
     } else {
         state = {(const void*)gdn_bwd_state_kernel<T, 128, 1, true>, bwd_state_smem<128, 1>(), "gdn_bwd_state_kernel", runs(128), 512};
         dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, 1, true>, bwd_dstate_smem<128, 1>(), "gdn_bwd_dstate_kernel", runs(128), 512};

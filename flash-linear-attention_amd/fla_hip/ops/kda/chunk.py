@@ -44,7 +44,18 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if K > _DIM:
-        raise NotImplementedError(f'the chunked KDA kernels cover key head dims up to {_DIM} (got K={K})')
+        # Wide keys (the reference takes K up to 256, fla/ops/kda/chunk.py:409): the chunked kernels hold one block of 128 key
+        # features, so the forward goes token by token on the recurrence kernel, which holds two - the same mathematics and the
+        # same options, far slower on long prompts.  No states in front of the chunks (there are no chunks) and no backward.
+        if K > 2 * _DIM or return_states:
+            raise NotImplementedError(f'chunk_kda with key head dims above {_DIM}: forward only, without intermediate states, '
+                                      f'up to {2 * _DIM} (got K={K}, return_intermediate_states={return_states})')
+        from fla_hip.ops.gated_delta_rule.fused_recurrent import fused_recurrent_gated_delta_rule_fwd
+        o, ht = fused_recurrent_gated_delta_rule_fwd(
+            q, k, v, None, g, None, beta, A_log, dt_bias, scale, initial_state, output_final_state,
+            use_qk_l2norm_in_kernel, use_beta_sigmoid_in_kernel, allow_neg_eigval, state_v_first, cu_seqlens,
+            False, None, None, kda_gate_mode=gate_mode, lower_bound=0.0 if lower_bound is None else lower_bound)
+        return o.to(q.dtype), ht
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     nb = (V + _DIM - 1) // _DIM
     if nb > 1:
@@ -402,6 +413,8 @@ def chunk_kda(
                              cu_seqlens_cpu, A_log, dt_bias, lower_bound, gate_mode, use_qk_l2norm_in_kernel,
                              use_beta_sigmoid_in_kernel, allow_neg_eigval, return_states=True)
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, g, beta, A_log, dt_bias, initial_state)):
+        if k.shape[-1] > _DIM:
+            raise NotImplementedError(f'chunk_kda with key head dims above {_DIM} is forward only (got K={k.shape[-1]})')
         return ChunkKDAFunction.apply(q, k, v, g, beta, A_log, dt_bias, scale, initial_state, output_final_state,
                                       use_qk_l2norm_in_kernel, gate_mode, use_beta_sigmoid_in_kernel, allow_neg_eigval,
                                       state_v_first, cu_seqlens, cu_seqlens_cpu, lower_bound)

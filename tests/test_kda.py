@@ -368,6 +368,49 @@ def test_chunk_kda_options(what):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,HV,D,V,l2,gate_in_kernel,safe_gate,vfirst,packed,dtype', [
+    (2, 200, 2, 2, 256, 64, False, False, False, False, False, torch.bfloat16),
+    (1, 300, 2, 4, 192, 128, True, True, False, True, False, torch.float16),
+    (1, 260, 1, 2, 160, 200, False, True, True, False, True, torch.bfloat16),
+])
+def test_chunk_kda_wide_keys_forward(B, T, H, HV, D, V, l2, gate_in_kernel, safe_gate, vfirst, packed, dtype):
+    """Key head dims above 128 (the reference allows up to 256, fla/ops/kda/chunk.py:409): forward only, on the token kernel."""
+    from fla_hip.ops.kda import chunk_kda
+    q, k, v, g, beta, h0, A_log, dt_bias = _chunk_inputs(B, T, H, HV, D, 1, 0, gate_in_kernel, safe_gate, dtype, V=V)
+    lower_bound = -5.0 if safe_gate else None
+    if not l2:
+        q, k = F.normalize(q.float(), p=2, dim=-1).to(dtype), F.normalize(k.float(), p=2, dim=-1).to(dtype)
+    cu = [0, 70, 71, T] if packed else None
+    if packed:
+        h0 = torch.randn(3, HV, D, V, generator=torch.Generator().manual_seed(7))
+    if packed:
+        outs = [O.recurrent_kda(q[:, a:b], k[:, a:b], v[:, a:b], g[:, a:b], beta[:, a:b], 0.1, h0[i:i + 1], True,
+                                use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel, A_log=A_log, dt_bias=dt_bias,
+                                lower_bound=lower_bound) for i, (a, b) in enumerate(zip(cu[:-1], cu[1:]))]
+        ref_o, ref_ht = torch.cat([x[0] for x in outs], 1), torch.cat([x[1] for x in outs], 0)
+    else:
+        ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, 0.1, h0, True, use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel,
+                                        A_log=A_log, dt_bias=dt_bias, lower_bound=lower_bound)
+    d = lambda x: None if x is None else x.cuda()
+    h0_in = h0.transpose(-1, -2).contiguous() if vfirst else h0
+    o, ht = chunk_kda(d(q), d(k), d(v), d(g), d(beta), scale=0.1, initial_state=d(h0_in), output_final_state=True,
+                      use_qk_l2norm_in_kernel=l2, use_gate_in_kernel=gate_in_kernel, A_log=d(A_log), dt_bias=d(dt_bias),
+                      safe_gate=safe_gate, lower_bound=lower_bound, state_v_first=vfirst,
+                      cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'))
+    assert o.dtype == dtype and ht.dtype == torch.float32 and o.shape == v.shape
+    ht = ht.transpose(-1, -2) if vfirst else ht
+    assert O.get_err_ratio(ref_o, o.float().cpu()) < 0.005
+    assert O.get_err_ratio(ref_ht, ht.cpu()) < 0.005
+    # what this width does not have says so
+    with pytest.raises(NotImplementedError, match='forward only'):
+        chunk_kda(d(q).requires_grad_(True), d(k), d(v), d(g), d(beta), scale=0.1)
+    with torch.inference_mode():
+        with pytest.raises(NotImplementedError, match='intermediate'):
+            chunk_kda(d(q), d(k), d(v), d(g), d(beta), scale=0.1, return_intermediate_states=True,
+                      cu_seqlens=None if cu is None else torch.tensor(cu, device='cuda'))
+
+
+@pytest.mark.gpu
 def test_chunk_kda_validation():
     from fla_hip.ops.kda import chunk_kda
     x = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16, device='cuda')
