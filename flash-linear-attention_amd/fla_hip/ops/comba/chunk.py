@@ -43,7 +43,14 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
     B, T, H, K = k.shape
     HV, V = v.shape[2], v.shape[3]
     if K > _DIM:
-        raise NotImplementedError(f'the chunked comba kernels cover key head dims up to {_DIM} (got K={K})')
+        # Wide keys: the chunked kernels hold one block of 128 key features, so the forward goes token by token on the
+        # recurrence kernel, which holds two (the same mathematics, far slower on long prompts); no backward at this width.
+        if K > 2 * _DIM:
+            raise NotImplementedError(f'chunk_comba covers key head dims up to {2 * _DIM} (got K={K})')
+        from fla_hip.ops.comba.fused_recurrent import fused_recurrent_comba_fwd
+        o, ht = fused_recurrent_comba_fwd(q, k, p, v, g, beta, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel,
+                                          cu_seqlens)
+        return o.to(q.dtype), ht
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     nb = (V + _DIM - 1) // _DIM
     if nb > 1:
@@ -277,6 +284,8 @@ def chunk_comba(
     if scale is None:
         scale = k.shape[-1] ** -0.5
     if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, p, g, beta, initial_state)):
+        if k.shape[-1] > _DIM:
+            raise NotImplementedError(f'chunk_comba with key head dims above {_DIM} is forward only (got K={k.shape[-1]})')
         return ChunkCombaFunction.apply(q, k, v, p, g, beta, scale, initial_state, output_final_state,
                                         use_qk_l2norm_in_kernel, cu_seqlens, cu_seqlens_cpu)
     return chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_state, use_qk_l2norm_in_kernel,

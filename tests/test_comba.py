@@ -66,6 +66,28 @@ def test_chunk_comba_reference_matrix(B, T, H, D, scale, normalizer, mask_p, l2,
     _check('ht', ref_ht, ht, 5e-3)
 
 
+@pytest.mark.parametrize('B,T,H,HV,D,l2,cu,dtype', [
+    (2, 200, 2, 2, 256, False, None, torch.bfloat16),
+    (1, 300, 2, 4, 192, True, None, torch.float16),
+    (1, 260, 1, 2, 160, False, [0, 70, 71, 260], torch.bfloat16),
+])
+def test_chunk_comba_wide_keys_forward(B, T, H, HV, D, l2, cu, dtype):
+    """Key head dims above 128: forward only, token by token on the recurrence kernel."""
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, HV, D, dtype, normalise=not l2)
+    if cu is not None:
+        h0 = torch.randn(len(cu) - 1, HV, D, D, generator=torch.Generator().manual_seed(3))
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, 0.1, h0, True, use_qk_l2norm_in_kernel=l2, cu_seqlens=cu)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    cu_t = None if cu is None else torch.tensor(cu, device='cuda')
+    o, ht = _ops()[0](dq, dk, dv, dp, dg, db, scale=0.1, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=l2,
+                      cu_seqlens=cu_t)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and o.shape == v.shape
+    _check('o', ref_o, o, 5e-3)
+    _check('ht', ref_ht, ht, 5e-3)
+    with pytest.raises(NotImplementedError, match='forward only'):
+        _ops()[0](dq.requires_grad_(True), dk, dv, dp, dg, db, scale=0.1, cu_seqlens=cu_t)
+
+
 @pytest.mark.parametrize('H,D,mask_p,cu,idx', [
     (4, 64, 0, [0, 15], torch.int32),
     (4, 64, 0, [0, 256, 500, 1000], torch.int32),
@@ -181,7 +203,7 @@ def test_comba_validation():
         recurrent(q, k, p, v, g, beta[..., None].expand(-1, -1, -1, 32))
     with pytest.raises(RuntimeError, match='ROCm GPU'):
         chunk(*(x.cpu() for x in (q, k, v, p, g, beta)))
-    big = torch.zeros(1, 64, 1, 256, dtype=torch.bfloat16, device='cuda')
+    big = torch.zeros(1, 64, 1, 264, dtype=torch.bfloat16, device='cuda')
     with pytest.raises(NotImplementedError, match='key head dims'):
         chunk(big, big, big, big, g[:1, :, :1], beta[:1, :, :1])
     # no tokens: the state passes through
