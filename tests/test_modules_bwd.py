@@ -131,6 +131,18 @@ def test_conv_backward_with_states(activation, dtype):
     _close('dh0', ref['dh0'], dh0, dtype)
 
 
+@pytest.mark.parametrize('W', [2, 4, 7])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+def test_conv_backward_long_runs(W, dtype):
+    """Several runs of eight tiles per workgroup, so that most waves take the loop for runs inside one sequence: dense rows
+    whose boundaries fall inside a run, and packed sequences that start, end and hand over a final-state gradient inside runs
+    (lengths that are and are not multiples of the tile and of the strip)."""
+    _check_conv(_conv_case(2, 1600, 96, W, dtype, True, False, state=True), 'silu')
+    cu = [0, 700, 701, 1340, 1344, 2368, 3000]
+    _check_conv(_conv_case(1, 3000, 72, W, dtype, False, True, state=True, N=6), 'silu', cu, torch.int32)
+    _check_conv(_conv_case(1, 3000, 72, W, dtype, True, False, state=False), None, cu, torch.int64)
+
+
 def test_conv_backward_reads_a_slice_in_place_and_is_deterministic():
     gen = torch.Generator().manual_seed(3)
     wide = torch.randn(2, 300, 3 * 256, generator=gen).bfloat16()
