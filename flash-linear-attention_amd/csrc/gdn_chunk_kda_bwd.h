@@ -256,7 +256,6 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
         if (tid < 64) sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype);
         sDb[tid] = 0.f;
         lds_barrier();
-        if (u + gridDim.x < units) fetch(u + gridDim.x);
         // this unit's rows of q (wanted late, no room for them in LDS yet) and what the previous kernel left of dGk
         fetch_tile<BD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * BD, (int64_t)p.H * BD, c.valid, tid);
         f32x4 dG[2][4];
@@ -401,6 +400,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
             }
         }
         lds_barrier();
+        // (the next unit's tiles are requested here, not at the top of the unit: there the requests queue behind the last unit's stores)
+        if (u + gridDim.x < units) fetch(u + gridDim.x);
         // the two matrices with a decay per pair and feature, a block of 16 rows at a time
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
