@@ -318,7 +318,9 @@ __global__ __launch_bounds__(256) void gdn_recurrent_kernel(RecurrentParams p) {
 // per CU = 208, 183, 191 us for 1 GiB of state traffic).
 constexpr size_t DECODE_LDS_PAD = 64 * 1024;
 
-template <typename T>
+// GK: a decay per key feature as well (the KDA operator's decode step): S' = diag(e^gk) e^g S + k d^T, so the two
+// reductions run over e^gk k and e^gk q, staged beside k and q, and the update takes a factor per row.
+template <typename T, bool GK = false>
 __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = tid & 31, r0 = tid >> 5;
@@ -341,11 +343,17 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 4 * c;
     const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
     // what a token brings, as it comes from memory
-    struct Token { T q, k; T v[4]; float g, b; };
+    struct Token { T q, k; T v[4]; float g, b, gk; };
+    const float a_k = GK && p.gk_act ? (p.A_log ? __expf(p.A_log[ihv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
+    const float gk_bias = GK && p.gk_act && p.gk_bias && tid < 128 ? p.gk_bias[ihv * 128 + tid] : 0.f;
     auto fetch = [&](int64_t tok) {
         Token x;
         x.q = x.k = from_f32<T>(0.f);
-        if (tid < 128) { x.q = q[(tok * H + ih) * 128 + tid]; x.k = k[(tok * H + ih) * 128 + tid]; }
+        x.gk = 0.f;
+        if (tid < 128) {
+            x.q = q[(tok * H + ih) * 128 + tid]; x.k = k[(tok * H + ih) * 128 + tid];
+            if constexpr (GK) x.gk = p.gk[(tok * HV + ihv) * 128 + tid];
+        }
         const T* pv = v + (tok * HV + ihv) * 128 + 4 * c;
 #pragma unroll
         for (int j = 0; j < 4; ++j) x.v[j] = pv[j];
@@ -365,6 +373,7 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
         if (p.h0) S[i] = __builtin_nontemporal_load((const f32x4*)(p.h0 + state_off + (r0 + 8 * i) * 128));
     }
     __shared__ float sh_q[2][128], sh_k[2][128];
+    __shared__ float sh_kr[GK ? 2 : 1][GK ? 128 : 1], sh_eg[GK ? 2 : 1][GK ? 128 : 1];     // (GK) k as it is, and e^gk per row
     __shared__ float sh_red[2][4][4];
     __shared__ f32x4 sh_part[2][4][2][32];
     const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
@@ -373,7 +382,19 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
         const int pb = (int)(t & 1);
         const int64_t tok = bos + t;
         const float qv = to_f32(cur.q), kv = to_f32(cur.k);
-        if (tid < 128) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
+        if constexpr (GK) {
+            if (tid < 128) {
+                float x = cur.gk;
+                if (p.gk_act) {
+                    x += gk_bias;
+                    x = p.gk_act == 2 ? p.gk_lower * sigmoid_f(a_k * x) : -a_k * softplus_f(x);
+                }
+                const float e = __expf(x);
+                sh_q[pb][tid] = qv * e; sh_k[pb][tid] = kv * e; sh_kr[pb][tid] = kv; sh_eg[pb][tid] = e;
+            }
+        } else {
+            if (tid < 128) { sh_q[pb][tid] = qv; sh_k[pb][tid] = kv; }
+        }
         float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
         if (lane == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
         float eg = 1.f;
@@ -412,7 +433,10 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
         const f32x4 d = bb * (vv - sk);
         const f32x4 dk = d * rk;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) S[i] = S[i] * eg + dk * sh_k[pb][r0 + 8 * i];
+        for (int i = 0; i < 16; ++i) {
+            if constexpr (GK) S[i] = S[i] * (eg * sh_eg[pb][r0 + 8 * i]) + dk * sh_kr[pb][r0 + 8 * i];
+            else S[i] = S[i] * eg + dk * sh_k[pb][r0 + 8 * i];
+        }
         if (r0 == 0) {
             const f32x4 ov = sq + d * qk;
             T* po = o + (tok * HV + ihv) * 128 + 4 * c;
@@ -604,13 +628,18 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         return check_launch("gdn_decode_bf16_kernel");
     }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
-    if (p.K == 128 && p.V == 128 && !vfirst && !p.gk && !p.gv && !p.pk && n_states >= 1024 &&
+    if (p.K == 128 && p.V == 128 && !vfirst && !p.gv && !p.pk && n_states >= 1024 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
         RecurrentParams pd = p;
         const int64_t grid = place(pd, n_states, p.HV);
-        static SmemAttrDone attr_done;                   // per instantiation
-        if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T>, DECODE_LDS_PAD, attr_done, "hipFuncSetAttribute(decode)")) return rc;
-        hipLaunchKernelGGL(gdn_decode_kernel<T>, dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        static SmemAttrDone attr_done, attr_done_gk;     // per instantiation
+        if (p.gk) {
+            if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T, true>, DECODE_LDS_PAD, attr_done_gk, "hipFuncSetAttribute(decode)")) return rc;
+            hipLaunchKernelGGL((gdn_decode_kernel<T, true>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        } else {
+            if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T, false>, DECODE_LDS_PAD, attr_done, "hipFuncSetAttribute(decode)")) return rc;
+            hipLaunchKernelGGL((gdn_decode_kernel<T, false>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        }
         return check_launch("gdn_decode_kernel");
     }
     // Value block per workgroup: whole rows when there are enough (sequence, head) pairs to

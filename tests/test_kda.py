@@ -118,6 +118,36 @@ def test_fused_recurrent_kda_gate_in_kernel(mode, H, HV, D, vfirst):
     _check('ht (host gate)', ht2.cpu(), ht, 1e-4)
 
 
+@pytest.mark.parametrize('mode', ['log-decay', 'softplus', 'bounded-no-A'])
+@pytest.mark.parametrize('T,dtype', [(1, torch.bfloat16), (3, torch.float32)])
+def test_fused_recurrent_kda_decode_kernel(mode, T, dtype):
+    """1024 states of K = V = 128 and more take the whole-state decode kernel in its form with a decay per key feature:
+    against the oracle, and against the general kernel (the same call on a V-first copy of the states)."""
+    B, H, HV, D = 128, 4, 8, 128
+    q, k, v, g, beta, h0 = _inputs(B, T, H, HV, D, dtype=dtype, raw_gate=mode != 'log-decay', seed=11)
+    gen = torch.Generator().manual_seed(12)
+    A_log = torch.log(1 + 15 * torch.rand(HV, generator=gen)) if mode == 'softplus' else None
+    dt_bias = torch.randn(HV * D, generator=gen) if mode != 'log-decay' else None
+    lower = -5.0 if mode.startswith('bounded') else None
+    if mode == 'softplus':
+        g = g - 4.0
+    kw = dict(use_qk_l2norm_in_kernel=True, use_gate_in_kernel=mode != 'log-decay', lower_bound=lower)
+    ref_o, ref_ht = O.recurrent_kda(q, k, v, g, beta, None, h0, True, A_log=A_log, dt_bias=dt_bias, **kw)
+    dq, dk, dv, dg, db, dh, dA, dbias = _cuda(q, k, v, g, beta, h0, A_log, dt_bias)
+    o, ht = _ops()[0](dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=dh, output_final_state=True, **kw)
+    _check('o', ref_o, o)
+    _check('ht', ref_ht, ht)
+    o2, ht2 = _ops()[0](dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=dh.transpose(-1, -2).contiguous(),
+                        output_final_state=True, state_v_first=True, **kw)
+    _check('o (general kernel)', o2.float().cpu(), o, 1e-4)
+    _check('ht (general kernel)', ht2.transpose(-1, -2).cpu(), ht, 1e-4)
+    # the serving form: states updated in place
+    from fla_hip.ops.kda import fused_recurrent_kda_fwd
+    pool = dh.clone()
+    o3, _ = fused_recurrent_kda_fwd(dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=pool, inplace_final_state=True, **kw)
+    assert torch.equal(o3, o) and torch.equal(pool, ht)
+
+
 @pytest.mark.parametrize('idx_dtype', [torch.int64, torch.int32])
 def test_fused_recurrent_kda_packed(idx_dtype):
     cu = [0, 15, 16, 100, 356, 357, 1000]
