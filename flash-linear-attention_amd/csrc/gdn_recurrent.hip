@@ -320,8 +320,11 @@ constexpr size_t DECODE_LDS_PAD = 64 * 1024;
 
 // GK: a decay per key feature as well (the KDA operator's decode step): S' = diag(e^gk) e^g S + k d^T, so the two
 // reductions run over e^gk k and e^gk q, staged beside k and q, and the update takes a factor per row.
-template <typename T, bool GK = false>
+// PK: a second key p that the prediction uses on the state as it was BEFORE this token's decay (the comba operator's
+// decode step): d = beta (v - S^T p), so that reduction runs over p and takes no e^g.
+template <typename T, bool GK = false, bool PK = false>
 __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
+    static_assert(!(GK && PK), "one of the two forms at a time");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = tid & 31, r0 = tid >> 5;
     const int64_t inh = xcd_block(p);
@@ -343,16 +346,17 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 4 * c;
     const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
     // what a token brings, as it comes from memory
-    struct Token { T q, k; T v[4]; float g, b, gk; };
+    struct Token { T q, k, pk; T v[4]; float g, b, gk; };
     const float a_k = GK && p.gk_act ? (p.A_log ? __expf(p.A_log[ihv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
     const float gk_bias = GK && p.gk_act && p.gk_bias && tid < 128 ? p.gk_bias[ihv * 128 + tid] : 0.f;
     auto fetch = [&](int64_t tok) {
         Token x;
-        x.q = x.k = from_f32<T>(0.f);
+        x.q = x.k = x.pk = from_f32<T>(0.f);
         x.gk = 0.f;
         if (tid < 128) {
             x.q = q[(tok * H + ih) * 128 + tid]; x.k = k[(tok * H + ih) * 128 + tid];
             if constexpr (GK) x.gk = p.gk[(tok * HV + ihv) * 128 + tid];
+            if constexpr (PK) x.pk = ((const T*)p.pk)[(tok * H + ih) * 128 + tid];
         }
         const T* pv = v + (tok * HV + ihv) * 128 + 4 * c;
 #pragma unroll
@@ -374,6 +378,7 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     }
     __shared__ float sh_q[2][128], sh_k[2][128];
     __shared__ float sh_kr[GK ? 2 : 1][GK ? 128 : 1], sh_eg[GK ? 2 : 1][GK ? 128 : 1];     // (GK) k as it is, and e^gk per row
+    __shared__ float sh_p[PK ? 2 : 1][PK ? 128 : 1];
     __shared__ float sh_red[2][4][4];
     __shared__ f32x4 sh_part[2][4][2][32];
     const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
@@ -397,6 +402,12 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
         }
         float sqq = wave_sum(qv * qv), skk = wave_sum(kv * kv), sqk = wave_sum(qv * kv);
         if (lane == 0) { sh_red[pb][wave][0] = sqq; sh_red[pb][wave][1] = skk; sh_red[pb][wave][2] = sqk; }
+        if constexpr (PK) {
+            const float pv = to_f32(cur.pk);
+            if (tid < 128) sh_p[pb][tid] = pv;
+            const float spp = wave_sum(pv * pv);
+            if (lane == 0) sh_red[pb][wave][3] = spp;
+        }
         float eg = 1.f;
         if (p.g) {
             float gt = cur.g;
@@ -411,24 +422,25 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
         sqq = sh_red[pb][0][0] + sh_red[pb][1][0];      // (q and k live in waves 0 and 1)
         skk = sh_red[pb][0][1] + sh_red[pb][1][1];
         sqk = sh_red[pb][0][2] + sh_red[pb][1][2];
-        float rq = p.scale, rk = 1.f;
+        float rq = p.scale, rk = 1.f, rp = 1.f;
         if (p.flags & GDN_FLAG_QK_L2NORM) {
             rq *= 1.f / sqrtf(sqq + 1e-6f);
             rk = 1.f / sqrtf(skk + 1e-6f);
+            if constexpr (PK) rp = 1.f / sqrtf(sh_red[pb][0][3] + sh_red[pb][1][3] + 1e-6f);
         }
         const float qk = sqk * rq * rk;
         // S^T k and S^T q over this thread's rows (k, q unscaled: the row factors come after the reduction)
         f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            sk += S[i] * sh_k[pb][r0 + 8 * i];
+            sk += S[i] * (PK ? sh_p[pb][r0 + 8 * i] : sh_k[pb][r0 + 8 * i]);
             sq += S[i] * sh_q[pb][r0 + 8 * i];
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) { sk[j] += __shfl_xor(sk[j], 32, 64); sq[j] += __shfl_xor(sq[j], 32, 64); }
         if (lane < 32) { sh_part[pb][wave][0][c] = sk; sh_part[pb][wave][1][c] = sq; }
         __syncthreads();
-        sk = (sh_part[pb][0][0][c] + sh_part[pb][1][0][c] + sh_part[pb][2][0][c] + sh_part[pb][3][0][c]) * (eg * rk);
+        sk = (sh_part[pb][0][0][c] + sh_part[pb][1][0][c] + sh_part[pb][2][0][c] + sh_part[pb][3][0][c]) * (PK ? rp : eg * rk);
         sq = (sh_part[pb][0][1][c] + sh_part[pb][1][1][c] + sh_part[pb][2][1][c] + sh_part[pb][3][1][c]) * (eg * rq);
         const f32x4 d = bb * (vv - sk);
         const f32x4 dk = d * rk;
@@ -628,12 +640,15 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         return check_launch("gdn_decode_bf16_kernel");
     }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
-    if (p.K == 128 && p.V == 128 && !vfirst && !p.gv && !p.pk && n_states >= 1024 &&
+    if (p.K == 128 && p.V == 128 && !vfirst && !p.gv && !(p.pk && p.gk) && n_states >= 1024 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
         RecurrentParams pd = p;
         const int64_t grid = place(pd, n_states, p.HV);
-        static SmemAttrDone attr_done, attr_done_gk;     // per instantiation
-        if (p.gk) {
+        static SmemAttrDone attr_done, attr_done_gk, attr_done_pk;     // per instantiation
+        if (p.pk) {
+            if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T, false, true>, DECODE_LDS_PAD, attr_done_pk, "hipFuncSetAttribute(decode)")) return rc;
+            hipLaunchKernelGGL((gdn_decode_kernel<T, false, true>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        } else if (p.gk) {
             if (int rc = ensure_dynamic_smem((const void*)gdn_decode_kernel<T, true>, DECODE_LDS_PAD, attr_done_gk, "hipFuncSetAttribute(decode)")) return rc;
             hipLaunchKernelGGL((gdn_decode_kernel<T, true>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
         } else {

@@ -13,6 +13,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
+    pad_last_two,
     aligned16,
     check_operand_shapes,
     as_f32,
@@ -75,7 +76,7 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
     if initial_state is not None:
         if tuple(initial_state.shape) != (N, HV, K, V):
             raise ValueError(f'initial_state must have shape {(N, HV, K, V)}, got {tuple(initial_state.shape)}')
-        h0 = aligned16(F.pad(as_f32(initial_state), (0, _DIM - V, 0, _DIM - K)).contiguous())
+        h0 = aligned16(pad_last_two(as_f32(initial_state), _DIM, _DIM).contiguous())
 
     flags = _lib.FLAG_QK_L2NORM if use_qk_l2norm_in_kernel else 0
     chunk_table = chunk_offsets = None
@@ -153,7 +154,7 @@ def chunk_comba_bwd(q, k, v, p, g, beta, scale, initial_state, do, dht, cu_seqle
             return None
         if tuple(s.shape) != (N, HV, K, V):
             raise ValueError(f'initial_state and dht must have shape {(N, HV, K, V)}, got {tuple(s.shape)}')
-        return aligned16(F.pad(as_f32(s), (0, _DIM - V, 0, _DIM - K)).contiguous())
+        return aligned16(pad_last_two(as_f32(s), _DIM, _DIM).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
     flags = 0

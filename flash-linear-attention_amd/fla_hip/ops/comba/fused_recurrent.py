@@ -10,6 +10,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
+    pad_last_two,
     aligned16,
     as_f32,
     check_operand_shapes,
@@ -54,7 +55,7 @@ def fused_recurrent_comba_fwd(q, k, p, v, g, beta, scale, initial_state, output_
     if initial_state is not None:
         if tuple(initial_state.shape) != (N, HV, K, V):
             raise ValueError(f'initial_state must have shape {(N, HV, K, V)}, got {tuple(initial_state.shape)}')
-        h0 = aligned16(F.pad(as_f32(initial_state), (0, VP - V, 0, KP - K)).contiguous())
+        h0 = aligned16(pad_last_two(as_f32(initial_state), KP, VP).contiguous())
     if cu_seqlens is not None:
         if cu_seqlens.dtype not in (torch.int32, torch.int64):
             cu_seqlens = cu_seqlens.long()

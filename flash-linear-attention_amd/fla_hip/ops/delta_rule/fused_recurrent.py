@@ -8,7 +8,7 @@ import torch
 import torch.nn.functional as F
 
 from fla_hip import _lib
-from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, current_stream_ptr, dtype_code, ptr, require_gpu
+from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, current_stream_ptr, dtype_code, pad_last_two, ptr, require_gpu
 from fla_hip.ops.gated_delta_rule.fused_recurrent import fused_recurrent_gated_delta_rule_fwd
 from fla_hip.ops.utils.index import check_cu_seqlens, cu_bounds
 
@@ -60,7 +60,7 @@ def fused_recurrent_delta_rule_bwd(
             return None
         if tuple(s.shape) != (N, H, K, V):
             raise ValueError(f'initial_state and dht must have shape {(N, H, K, V)}, got {tuple(s.shape)}')
-        return aligned16(F.pad(as_f32(s), (0, VP - V, 0, KP - K)).contiguous())
+        return aligned16(pad_last_two(as_f32(s), KP, VP).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
     # tokens of a packed tensor outside every sequence are never written: they get zero gradients

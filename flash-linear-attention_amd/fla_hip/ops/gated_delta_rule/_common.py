@@ -38,6 +38,13 @@ def as_f32(x: torch.Tensor | None) -> torch.Tensor | None:
     return x if x.dtype == torch.float32 else x.float()
 
 
+def pad_last_two(x: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """Zero-pads the last two dims up to ``rows x cols``; the tensor itself when nothing is missing (``F.pad`` by zero
+    would still copy it: a pool of states per decode step)."""
+    r, c = rows - x.shape[-2], cols - x.shape[-1]
+    return x if r == 0 and c == 0 else torch.nn.functional.pad(x, (0, c, 0, r))
+
+
 def aligned16(x: torch.Tensor | None) -> torch.Tensor | None:
     """The kernels read states with 16-byte vector loads."""
     if x is None or x.data_ptr() % 16 == 0:

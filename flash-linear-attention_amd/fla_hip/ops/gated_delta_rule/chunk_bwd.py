@@ -12,7 +12,7 @@ import torch
 import torch.nn.functional as F
 
 from fla_hip import _lib
-from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, check_operand_shapes, current_stream_ptr, dtype_code, ptr, require_gpu
+from fla_hip.ops.gated_delta_rule._common import aligned16, as_f32, check_operand_shapes, current_stream_ptr, dtype_code, pad_last_two, ptr, require_gpu
 from fla_hip.ops.utils.index import check_cu_seqlens, cu_bounds, prepare_chunk_indices, prepare_scan_tables
 
 _CHUNK = 64
@@ -102,7 +102,7 @@ def chunk_gated_delta_rule_bwd(
         s = as_f32(s)
         if state_v_first:
             s = s.transpose(-1, -2)
-        return aligned16(F.pad(s, (0, _DIM - V, 0, KD - K)).contiguous())
+        return aligned16(pad_last_two(s, KD, _DIM).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
     # FLA_HIP_BWD_SCAN_MODE forces one form of the two scans (default: automatic): whole sequences ('wide') or time segments

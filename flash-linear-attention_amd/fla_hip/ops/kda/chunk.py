@@ -13,6 +13,7 @@ import torch.nn.functional as F
 
 from fla_hip import _lib
 from fla_hip.ops.gated_delta_rule._common import (
+    pad_last_two,
     aligned16,
     check_operand_shapes,
     as_f32,
@@ -111,7 +112,7 @@ def chunk_kda_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, st
         h0 = as_f32(initial_state)
         if state_v_first:
             h0 = h0.transpose(-1, -2)
-        h0 = aligned16(F.pad(h0, (0, _DIM - V, 0, _DIM - K)).contiguous())
+        h0 = aligned16(pad_last_two(h0, _DIM, _DIM).contiguous())
 
     flags = 0
     if use_qk_l2norm_in_kernel:
@@ -212,7 +213,7 @@ def chunk_kda_bwd(q, k, v, g, beta, scale, initial_state, do, dht, state_v_first
         s = as_f32(s)
         if state_v_first:
             s = s.transpose(-1, -2)
-        return aligned16(F.pad(s, (0, _DIM - V, 0, _DIM - K)).contiguous())
+        return aligned16(pad_last_two(s, _DIM, _DIM).contiguous())
     h0, dhtw = state_in(initial_state), state_in(dht)
 
     flags = 0

@@ -133,6 +133,24 @@ def test_fused_recurrent_comba_reference_matrix(B, T, H, D, scale, normalizer, d
     _check('ht', ref_ht, ht, 2e-3)
 
 
+@pytest.mark.parametrize('T,l2,dtype', [(1, False, torch.bfloat16), (1, True, torch.float32), (3, True, torch.float16)])
+def test_fused_recurrent_comba_decode_kernel(T, l2, dtype):
+    """1024 states of K = V = 128 and more take the whole-state decode kernel in its form with a second key: against the
+    oracle, and against the general kernel (the same sequences in two calls of 512 states each)."""
+    B, H, HV, D = 128, 4, 8, 128
+    q, k, v, p, g, beta, h0 = _inputs(B, T, H, HV, D, dtype, normalise=not l2, seed=5)
+    ref_o, ref_ht = O.recurrent_comba(q, k, v, p, g, beta, 0.1, h0, True, use_qk_l2norm_in_kernel=l2)
+    dq, dk, dv, dp, dg, db, dh = _cuda(q, k, v, p, g, beta, h0)
+    rec = _ops()[1]
+    o, ht = rec(dq, dk, dp, dv, dg, db, scale=0.1, initial_state=dh, output_final_state=True, use_qk_l2norm_in_kernel=l2)
+    _check('o', ref_o, o, 2e-3 if dtype == torch.float32 else 5e-3)
+    _check('ht', ref_ht, ht, 2e-3 if dtype == torch.float32 else 5e-3)
+    halves = [rec(dq[a:b], dk[a:b], dp[a:b], dv[a:b], dg[a:b], db[a:b], scale=0.1, initial_state=dh[a:b], output_final_state=True,
+                  use_qk_l2norm_in_kernel=l2) for a, b in ((0, 64), (64, 128))]
+    _check('o (general kernel)', torch.cat([x[0] for x in halves]).float().cpu(), o, 1e-4)
+    _check('ht (general kernel)', torch.cat([x[1] for x in halves]).cpu(), ht, 1e-4)
+
+
 def test_comba_options_and_reductions():
     """Defaults (p = k, beta = 1, no state), grouped value heads, value heads wider than the kernels' 128 columns, the split
     of a sequence at a chunk boundary handing the state over, and p = k with g = 0 against the delta rule operator."""
