@@ -461,6 +461,107 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
     }
 }
 
+// The common decode shape with V-first states [V][K] (the layout serving engines keep, `state_v_first`): thread
+// (c = tid % 32, r0 = tid / 32) owns key features 4c .. 4c+3 of value rows r0 + 8i, so S^T k and S^T q are sums along a
+// row: four products per thread and row, then over the 32 lanes that share the row.  The token's rows are requested
+// before the state here as well (k and q as the thread's own four features, v through LDS), two workgroups share a CU.
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_decode_vfirst_kernel(RecurrentParams p) {
+    const int tid = threadIdx.x;
+    const int c = tid & 31, r0 = tid >> 5;
+    const int64_t inh = xcd_block(p);
+    if (inh < 0) return;
+    const int64_t in = inh / p.HV;
+    const int ihv = (int)(inh % p.HV);
+    const int H = p.H, HV = p.HV;
+    const int ih = ihv / (HV / H);
+    const bool cu32 = p.flags & GDN_FLAG_CU_INT32;
+    int64_t bos, len;
+    if (p.cu_seqlens) {
+        bos = load_index(p.cu_seqlens, in, cu32);
+        len = load_index(p.cu_seqlens, in + 1, cu32) - bos;
+    } else {
+        bos = in * p.T;
+        len = p.T;
+    }
+    const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
+    const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 4 * c;
+    const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
+    struct Token { T q[4], k[4]; T v; float g, b; };
+    auto fetch = [&](int64_t tok) {
+        Token x;
+        const T* pq = q + (tok * H + ih) * 128 + 4 * c;
+        const T* pk = k + (tok * H + ih) * 128 + 4 * c;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { x.q[j] = pq[j]; x.k[j] = pk[j]; }
+        x.v = from_f32<T>(0.f);
+        if (tid < 128) x.v = v[(tok * HV + ihv) * 128 + tid];
+        x.g = p.g ? load_scalar(p.g, tok * HV + ihv, p.gb_dtype) : 0.f;
+        x.b = p.beta ? load_scalar(p.beta, tok * HV + ihv, p.gb_dtype) : 1.f;
+        return x;
+    };
+    Token cur = {};
+    if (len > 0) cur = fetch(bos);
+    float a_neg = 0.f, dtb = 0.f;
+    if (p.A_log) { a_neg = -__expf(p.A_log[ihv]); if (p.dt_bias) dtb = p.dt_bias[ihv]; }
+    f32x4 S[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (p.h0) S[i] = __builtin_nontemporal_load((const f32x4*)(p.h0 + state_off + (r0 + 8 * i) * 128));
+    }
+    __shared__ float sh_v[2][128];
+    const float bmul = (p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f;
+    auto row_sum = [&](float x) {                               // over the 32 lanes that share a row
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) x += __shfl_xor(x, off, 64);
+        return x;
+    };
+
+    for (int64_t t = 0; t < len; ++t) {
+        const int pb = (int)(t & 1);
+        const int64_t tok = bos + t;
+        f32x4 qc, kc;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { qc[j] = to_f32(cur.q[j]); kc[j] = to_f32(cur.k[j]); }
+        if (tid < 128) sh_v[pb][tid] = to_f32(cur.v);
+        float eg = 1.f;
+        if (p.g) {
+            float gt = cur.g;
+            if (p.A_log) gt = a_neg * softplus_f(gt + dtb);
+            eg = __expf(gt);
+        }
+        float bb = cur.b;
+        if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
+        if (t + 1 < len) cur = fetch(tok + 1);          // the next token's rows travel during this one's arithmetic
+        const float sqq = row_sum(qc.x * qc.x + qc.y * qc.y + qc.z * qc.z + qc.w * qc.w);
+        const float skk = row_sum(kc.x * kc.x + kc.y * kc.y + kc.z * kc.z + kc.w * kc.w);
+        const float sqk = row_sum(qc.x * kc.x + qc.y * kc.y + qc.z * kc.z + qc.w * kc.w);
+        float rq = p.scale, rk = 1.f;
+        if (p.flags & GDN_FLAG_QK_L2NORM) {
+            rq *= 1.f / sqrtf(sqq + 1e-6f);
+            rk = 1.f / sqrtf(skk + 1e-6f);
+        }
+        const float qk = sqk * rq * rk;
+        kc *= rk; qc *= rq;
+        __syncthreads();                                // (v of this token is in LDS)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int row = r0 + 8 * i;
+            const f32x4 sdec = S[i] * eg;
+            const f32x4 a = sdec * kc, b = sdec * qc;
+            const float sk = row_sum((a.x + a.y) + (a.z + a.w)), sq = row_sum((b.x + b.y) + (b.z + b.w));
+            const float d = bb * (sh_v[pb][row] - sk);
+            S[i] = sdec + kc * d;
+            if (c == 0) o[(tok * HV + ihv) * 128 + row] = from_f32<T>(sq + d * qk);
+        }
+    }
+    if (p.ht) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) __builtin_nontemporal_store(S[i], (f32x4*)(p.ht + state_off + (r0 + 8 * i) * 128));
+    }
+}
+
 // The same step with the states held in bf16 in memory (half the traffic of a decode step): K = V = 128, K-first.  The
 // recurrence runs in fp32 registers; the state is rounded (to nearest even) once, when it is written back.  A thread owns
 // 8 value columns (16 bytes of a row) of key rows r0 + 16 i; a wave instruction covers four whole rows.  (Three to five
@@ -638,6 +739,15 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         const int64_t grid = place(pd, n_states, p.HV);
         hipLaunchKernelGGL(gdn_decode_bf16_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, pd);
         return check_launch("gdn_decode_bf16_kernel");
+    }
+    if (p.K == 128 && p.V == 128 && vfirst && !p.gk && !p.gv && !p.pk && n_states >= 1024 &&
+        !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
+        RecurrentParams pd = p;
+        const int64_t grid = place(pd, n_states, p.HV);
+        static SmemAttrDone attr_done_vf;
+        if (int rc = ensure_dynamic_smem((const void*)gdn_decode_vfirst_kernel<T>, DECODE_LDS_PAD, attr_done_vf, "hipFuncSetAttribute(decode)")) return rc;
+        hipLaunchKernelGGL(gdn_decode_vfirst_kernel<T>, dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        return check_launch("gdn_decode_vfirst_kernel");
     }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)
     if (p.K == 128 && p.V == 128 && !vfirst && !p.gv && !(p.pk && p.gk) && n_states >= 1024 &&

@@ -386,9 +386,10 @@ def test_no_tokens_returns_the_initial_state():
     assert torch.equal(ht, h0)
 
 
+@pytest.mark.parametrize('vfirst', [False, True])
 @pytest.mark.parametrize('case', ['plain', 'flags', 'packed', 'slots', 'f16', 'fp32'])
-def test_decode_kernel_for_the_common_shape(case):
-    """K = V = 128, K-first states, 1024 or more (sequence, head) states: the decode kernel written for that shape."""
+def test_decode_kernel_for_the_common_shape(case, vfirst):
+    """K = V = 128, 1024 or more (sequence, head) states: the decode kernels written for that shape, one per state layout."""
     H, HV, D = 8, 32, 128
     dtype = {'f16': torch.float16, 'fp32': torch.float32}.get(case, torch.bfloat16)
     kw, okw = {}, {}
@@ -416,21 +417,23 @@ def test_decode_kernel_for_the_common_shape(case):
     ref_o, ref_ht = O.recurrent_gated_delta_rule(q, k, v, g, beta, None, h0, True, cu_seqlens=cu, **okw)
     dev = 'cuda'
     cu_t = None if cu is None else torch.tensor(cu, device=dev)
+    lay = (lambda x: x.transpose(-1, -2).contiguous()) if vfirst else (lambda x: x)
+    kw = dict(kw, state_v_first=vfirst)
     if case == 'slots':
         pool = torch.randn(N + 5, HV, D, D, generator=gen)
         idx = torch.randperm(N + 5, generator=gen)[:N]
         pool[idx] = h0
-        dpool = pool.to(dev)
+        dpool = lay(pool).to(dev)
         o, _ = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=dpool, inplace_final_state=True,
                       ssm_state_indices=idx.to(dev), **kw)
         ht = dpool[idx.to(dev)]
         rest = [i for i in range(N + 5) if i not in idx.tolist()]
-        assert torch.equal(dpool[rest].cpu(), pool[rest])
+        assert torch.equal(dpool[rest].cpu(), lay(pool[rest]))
     else:
-        o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=h0.to(dev),
+        o, ht = _ops()(q.to(dev), k.to(dev), v.to(dev), g.to(dev), beta=beta.to(dev), initial_state=lay(h0).to(dev),
                        output_final_state=True, cu_seqlens=cu_t, **kw)
     _check('o', ref_o, o)
-    _check('ht', ref_ht, ht)
+    _check('ht', ref_ht, lay(ht))
 
 
 @pytest.mark.parametrize('case', ['plain', 'few', 'flags', 'packed', 'slots', 'f16'])
