@@ -465,7 +465,8 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_kernel(RecurrentParams p) {
 // (c = tid % 32, r0 = tid / 32) owns key features 4c .. 4c+3 of value rows r0 + 8i, so S^T k and S^T q are sums along a
 // row: four products per thread and row, then over the 32 lanes that share the row.  The token's rows are requested
 // before the state here as well (k and q as the thread's own four features, v through LDS), two workgroups share a CU.
-template <typename T>
+// GK: a decay per key feature as well (the KDA operator): here a factor per column, the thread's own four.
+template <typename T, bool GK = false>
 __global__ __launch_bounds__(256, 2) void gdn_decode_vfirst_kernel(RecurrentParams p) {
     const int tid = threadIdx.x;
     const int c = tid & 31, r0 = tid >> 5;
@@ -487,13 +488,18 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_vfirst_kernel(RecurrentPara
     const int64_t slot = p.state_slots ? load_index(p.state_slots, in, p.flags & GDN_FLAG_SLOT_INT32) : in;
     const int64_t state_off = (slot * HV + ihv) * (int64_t)16384 + 4 * c;
     const T* q = (const T*)p.q; const T* k = (const T*)p.k; const T* v = (const T*)p.v; T* o = (T*)p.o;
-    struct Token { T q[4], k[4]; T v; float g, b; };
+    struct Token { T q[4], k[4]; T v; float g, b; f32x4 gk; };
+    const float a_k = GK && p.gk_act ? (p.A_log ? __expf(p.A_log[ihv]) : (p.gk_act == 2 ? 1.f : __expf(1.f))) : 0.f;
+    f32x4 gk_bias = {0.f, 0.f, 0.f, 0.f};
+    if (GK && p.gk_act && p.gk_bias) gk_bias = *(const f32x4*)(p.gk_bias + ihv * 128 + 4 * c);
     auto fetch = [&](int64_t tok) {
         Token x;
         const T* pq = q + (tok * H + ih) * 128 + 4 * c;
         const T* pk = k + (tok * H + ih) * 128 + 4 * c;
 #pragma unroll
         for (int j = 0; j < 4; ++j) { x.q[j] = pq[j]; x.k[j] = pk[j]; }
+        x.gk = f32x4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GK) x.gk = *(const f32x4*)(p.gk + (tok * HV + ihv) * 128 + 4 * c);
         x.v = from_f32<T>(0.f);
         if (tid < 128) x.v = v[(tok * HV + ihv) * 128 + tid];
         x.g = p.g ? load_scalar(p.g, tok * HV + ihv, p.gb_dtype) : 0.f;
@@ -533,6 +539,18 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_vfirst_kernel(RecurrentPara
         }
         float bb = cur.b;
         if (p.flags & GDN_FLAG_BETA_SIGMOID) bb = bmul * sigmoid_f(bb);
+        f32x4 eg4 = {eg, eg, eg, eg};
+        if constexpr (GK) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float x = cur.gk[j];
+                if (p.gk_act) {
+                    x += gk_bias[j];
+                    x = p.gk_act == 2 ? p.gk_lower * sigmoid_f(a_k * x) : -a_k * softplus_f(x);
+                }
+                eg4[j] *= __expf(x);
+            }
+        }
         if (t + 1 < len) cur = fetch(tok + 1);          // the next token's rows travel during this one's arithmetic
         const float sqq = row_sum(qc.x * qc.x + qc.y * qc.y + qc.z * qc.z + qc.w * qc.w);
         const float skk = row_sum(kc.x * kc.x + kc.y * kc.y + kc.z * kc.z + kc.w * kc.w);
@@ -548,7 +566,7 @@ __global__ __launch_bounds__(256, 2) void gdn_decode_vfirst_kernel(RecurrentPara
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int row = r0 + 8 * i;
-            const f32x4 sdec = S[i] * eg;
+            const f32x4 sdec = S[i] * eg4;
             const f32x4 a = sdec * kc, b = sdec * qc;
             const float sk = row_sum((a.x + a.y) + (a.z + a.w)), sq = row_sum((b.x + b.y) + (b.z + b.w));
             const float d = bb * (sh_v[pb][row] - sk);
@@ -740,13 +758,18 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         hipLaunchKernelGGL(gdn_decode_bf16_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, pd);
         return check_launch("gdn_decode_bf16_kernel");
     }
-    if (p.K == 128 && p.V == 128 && vfirst && !p.gk && !p.gv && !p.pk && n_states >= 1024 &&
+    if (p.K == 128 && p.V == 128 && vfirst && !p.gv && !p.pk && n_states >= 1024 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
         RecurrentParams pd = p;
         const int64_t grid = place(pd, n_states, p.HV);
-        static SmemAttrDone attr_done_vf;
-        if (int rc = ensure_dynamic_smem((const void*)gdn_decode_vfirst_kernel<T>, DECODE_LDS_PAD, attr_done_vf, "hipFuncSetAttribute(decode)")) return rc;
-        hipLaunchKernelGGL(gdn_decode_vfirst_kernel<T>, dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        static SmemAttrDone attr_done_vf, attr_done_vf_gk;
+        if (p.gk) {
+            if (int rc = ensure_dynamic_smem((const void*)gdn_decode_vfirst_kernel<T, true>, DECODE_LDS_PAD, attr_done_vf_gk, "hipFuncSetAttribute(decode)")) return rc;
+            hipLaunchKernelGGL((gdn_decode_vfirst_kernel<T, true>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        } else {
+            if (int rc = ensure_dynamic_smem((const void*)gdn_decode_vfirst_kernel<T, false>, DECODE_LDS_PAD, attr_done_vf, "hipFuncSetAttribute(decode)")) return rc;
+            hipLaunchKernelGGL((gdn_decode_vfirst_kernel<T, false>), dim3((unsigned)grid), dim3(256), DECODE_LDS_PAD, stream, pd);
+        }
         return check_launch("gdn_decode_vfirst_kernel");
     }
     // the common decode shape has a kernel of its own (enough states to fill the chip with whole-state workgroups)

@@ -121,8 +121,8 @@ def test_fused_recurrent_kda_gate_in_kernel(mode, H, HV, D, vfirst):
 @pytest.mark.parametrize('mode', ['log-decay', 'softplus', 'bounded-no-A'])
 @pytest.mark.parametrize('T,dtype', [(1, torch.bfloat16), (3, torch.float32)])
 def test_fused_recurrent_kda_decode_kernel(mode, T, dtype):
-    """1024 states of K = V = 128 and more take the whole-state decode kernel in its form with a decay per key feature:
-    against the oracle, and against the general kernel (the same call on a V-first copy of the states)."""
+    """1024 states of K = V = 128 and more take the whole-state decode kernels in their form with a decay per key feature:
+    both state layouts against the oracle and against the general kernel (the same sequences in two calls of 512 states)."""
     B, H, HV, D = 128, 4, 8, 128
     q, k, v, g, beta, h0 = _inputs(B, T, H, HV, D, dtype=dtype, raw_gate=mode != 'log-decay', seed=11)
     gen = torch.Generator().manual_seed(12)
@@ -139,8 +139,13 @@ def test_fused_recurrent_kda_decode_kernel(mode, T, dtype):
     _check('ht', ref_ht, ht)
     o2, ht2 = _ops()[0](dq, dk, dv, dg, db, A_log=dA, dt_bias=dbias, initial_state=dh.transpose(-1, -2).contiguous(),
                         output_final_state=True, state_v_first=True, **kw)
-    _check('o (general kernel)', o2.float().cpu(), o, 1e-4)
-    _check('ht (general kernel)', ht2.transpose(-1, -2).cpu(), ht, 1e-4)
+    _check('o (V-first decode kernel)', o2.float().cpu(), o, 1e-4)
+    _check('ht (V-first decode kernel)', ht2.transpose(-1, -2).cpu(), ht, 1e-4)
+    # (512 states at a time go to the general kernel)
+    halves = [_ops()[0](dq[a:b], dk[a:b], dv[a:b], dg[a:b], db[a:b], A_log=dA, dt_bias=dbias, initial_state=dh[a:b],
+                        output_final_state=True, **kw) for a, b in ((0, 64), (64, 128))]
+    _check('o (general kernel)', torch.cat([x[0] for x in halves]).float().cpu(), o, 1e-4)
+    _check('ht (general kernel)', torch.cat([x[1] for x in halves]).cpu(), ht, 1e-4)
     # the serving form: states updated in place
     from fla_hip.ops.kda import fused_recurrent_kda_fwd
     pool = dh.clone()
