@@ -1,6 +1,6 @@
 """Benchmark of the gated delta rule inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|ref_*|train_ref_*|chunk_kda|chunk_comba|train_chunk_kda|train_chunk_comba|layer_train|layer_steps|calib_copy|calib_rmw]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|prefill_b4|varlen|decode|decode_bf16_states|decode_v_first|decode_kda|ref_*|train_ref_*|chunk_kda|chunk_comba|train_chunk_kda|train_chunk_comba|layer_train|layer_steps|calib_copy|calib_rmw]
 
 Prints ONE JSON line.  Default workload: chunked prefill, B=1, T=32768, Hqk=16, Hv=32,
 K=V=128, bf16 inputs, fp32 state (random initial state, final state returned) - the
@@ -76,6 +76,10 @@ WORKLOADS = {
     'decode_bf16_states': dict(kind='decode', N=256, H=16, HV=32, state_dtype='bf16',
                                name='the decode step of configs[4] with the states kept in bf16 (an option of this library: '
                                     'fp32 step, one rounding per step; 2 x 256 MiB of state traffic)'),
+    'decode_v_first': dict(kind='decode', N=256, H=16, HV=32, v_first=True,
+                           name='the decode step of configs[4] on V-first states [N,HV,V,K] (state_v_first, the layout serving engines keep)'),
+    'decode_kda': dict(kind='decode', N=256, H=16, HV=32, op='kda',
+                       name='the KDA operator\'s decode step (a decay per key feature) at the shape of configs[4]'),
     # configs[2] again, so that the headline's dependence on the gates is a number: with the exact start states of the
     # time segments forced (first pass, merge, second pass), and with gates that hardly decay (logsigmoid / 1024:
     # no segment can start from a zero state, so the automatic choice takes the exact path by itself)
@@ -407,7 +411,8 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     q = F.normalize(torch.randn(N, 1, H, K, generator=gen), p=2, dim=-1).bfloat16()
     k = F.normalize(torch.randn(N, 1, H, K, generator=gen), p=2, dim=-1).bfloat16()
     v = torch.randn(N, 1, HV, V, generator=gen).bfloat16()
-    g = F.logsigmoid(torch.randn(N, 1, HV, generator=gen))
+    kda = w.get('op') == 'kda'
+    g = F.logsigmoid(torch.randn(N, 1, HV, K, generator=gen) if kda else torch.randn(N, 1, HV, generator=gen))
     beta = torch.sigmoid(torch.randn(N, 1, HV, generator=gen))
     h0 = 0.1 * torch.randn(N, HV, K, V, generator=gen)
     bf16_states = w.get('state_dtype') == 'bf16'
@@ -418,9 +423,16 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     # pools of 256 MiB, so that a pool's lines have left the cache when its turn comes again)
     states = [h0.to(device) for _ in range(4 if bf16_states else 2)]
 
+    v_first = bool(w.get('v_first'))
+    if kda:
+        from fla_hip.ops.kda import fused_recurrent_kda_fwd
+
     def step(i):
+        if kda:
+            return fused_recurrent_kda_fwd(dq, dk, dv, dg, db, initial_state=states[i % len(states)], output_final_state=True,
+                                           inplace_final_state=True)
         return fused_recurrent_gated_delta_rule(dq, dk, dv, dg, beta=db, initial_state=states[i % len(states)],
-                                                output_final_state=True, inplace_final_state=True)
+                                                output_final_state=True, inplace_final_state=True, state_v_first=v_first)
 
     spin_up(step)
     for i in range(warmup):
@@ -439,7 +451,7 @@ def bench_decode(w, steps, warmup, device, with_cpu):
     achieved = state_bytes / t_kernel / 1e9
     roofline = dict(bound='hbm', achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit='GB/s',
                     frac=round(achieved / PEAK_HBM_GBS, 4), traffic=measured_traffic(w['key']),
-                    kernel='gdn_decode_bf16_kernel' if bf16_states else 'gdn_decode_kernel',
+                    kernel='gdn_decode_bf16_kernel' if bf16_states else 'gdn_decode_vfirst_kernel' if v_first else 'gdn_decode_kernel',
                     kernel_us=round(t_kernel * 1e6, 1), bytes_per_launch=state_bytes)
     out = dict(value=elapsed / steps * 1e6, ms_per_step=elapsed / steps * 1e3, roofline=roofline)
     if with_cpu:
