@@ -75,10 +75,12 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
     const bool q_norms_here = l2 && !(p.flags & FLAG_Q_NORM_IN_SCAN);       // 1/|q_t| into the tables (else the scan applies it)
 
     // ---- loads: the gate inputs of token `lane`, then the k rows as operand fragments ----
-    float rg = 0.f, rb = 0.f;
+    // (as raw bits, converted where they are used: a 16-bit value converted on the spot would hold the k rows' requests back
+    // until it has arrived)
+    uint32_t rg = 0, rb = 0;
     if (lane < valid) {
-        rg = p.g ? load_scalar(p.g, (tok0 + lane) * HV + hv, p.gb_dtype) : 0.f;      // (no gate: the plain delta rule)
-        rb = load_scalar(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
+        rg = p.g ? load_scalar_bits(p.g, (tok0 + lane) * HV + hv, p.gb_dtype) : 0;   // (no gate: the plain delta rule)
+        rb = load_scalar_bits(p.beta, (tok0 + lane) * HV + hv, p.gb_dtype);
     }
     f32x4 U[4][4];
 #pragma unroll
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(64 * PW_WAVES, (WANT_P ? 8 : 16) / PW_WAVES) void g
     // ---- gates: inclusive scan over the chunk, one token per lane; the tables; the bound on the chunk's transition ----
     float beta_tok;
     {
-        float x = rg, b = rb;
+        float x = scalar_of_bits(rg, p.gb_dtype), b = scalar_of_bits(rb, p.gb_dtype);
         if (lane < valid) {                      // optional activations of the raw gate / beta inputs
             if (p.A_log && p.g) x = -__expf(p.A_log[hv]) * softplus_f(x + (p.dt_bias ? p.dt_bias[hv] : 0.f));
             if (p.flags & GDN_FLAG_BETA_SIGMOID) b = sigmoid_f(b) * ((p.flags & GDN_FLAG_NEG_EIGVAL) ? 2.f : 1.f);
