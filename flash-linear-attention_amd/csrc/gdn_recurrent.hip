@@ -758,7 +758,7 @@ static int launch_t(const RecurrentParams& p, int64_t n_states, hipStream_t stre
         hipLaunchKernelGGL(gdn_decode_bf16_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, pd);
         return check_launch("gdn_decode_bf16_kernel");
     }
-    if (p.K == 128 && p.V == 128 && vfirst && !p.gv && !p.pk && n_states >= 1024 &&
+    if (p.K == 128 && p.V == 128 && vfirst && !p.gv && !p.pk && n_states >= 1024 && (uintptr_t)p.gk_bias % 16 == 0 &&
         !(p.flags & (GDN_FLAG_BETA_VECTOR | GDN_FLAG_SLOT_PER_TOKEN | GDN_FLAG_STATE_PER_TOKEN))) {
         RecurrentParams pd = p;
         const int64_t grid = place(pd, n_states, p.HV);
