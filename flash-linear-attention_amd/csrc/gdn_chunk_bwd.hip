@@ -1179,6 +1179,303 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     }
 }
 
+// The same kernel for one block of key features and one key (the gated delta rule itself) in 64 KB of LDS, so that two
+// workgroups share a CU: the unit is walked in two halves over the same two tile places - first dv_new and v (dX's first
+// term, dv and its share of dbeta), then dw and k (dX's second term, k k^T, the first part of dk) - with the second pair
+// on its way into registers during the first half and the next unit's first pair during the second.
+constexpr size_t BWD_WY2_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 640 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_t units) {
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    constexpr int KD = BD, PK = P128, NA = 2;
+    extern __shared__ __align__(16) char smem[];
+    T* sX0 = (T*)smem; T* sX1 = sX0 + 64 * P128;               // dv_new | v, then dw | k
+    T* sA = sX1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
+    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1;
+
+    TileRegs<BD> rDvn, rV, rDW, rK;
+    TileRegs<CH> rA;
+    float rGam = 0.f, rDg = 0.f;
+    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
+    auto fetch_first = [&](int64_t u, int tid) {
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
+        if (tid < 64) {
+            rGam = p.ws.Gam[u * 64 + tid];
+            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
+            rDg = p.ws.Dgam[u * 64 + tid];
+        }
+    };
+    fetch_first(blockIdx.x, threadIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
+        int tid_opaque = threadIdx.x;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        auto feat = [&](int a) { return 16 * (2 * w + a); };    // first key feature of this wave's tile a
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        put_tile<BD>(sDvn, P128, rDvn, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        put_tile<CH>(sA, P64, rA, tid);
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); }
+        sDg[tid] = tid < 64 ? rDg : 0.f;
+        sDb[tid] = 0.f;
+        // the second pair of this unit, and what the previous kernel left in dk at this lane's places
+        fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        V4 dk_old[NA][4];
+#pragma unroll
+        for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                dk_old[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+                if (x < c.valid) dk_old[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g);
+            }
+        lds_barrier();
+
+        // ---- first half: dX's first term du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), and dv = beta (A^T du) ----
+        f32x4 dXv[4];
+        {
+            V8 fa[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                dXv[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) dXv[tj] = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv[tj]);
+                }
+            }
+        }
+        {
+            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
+            float bj[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                bj[t] = sBeta[16 * t + c16];
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
+                const int n16 = 16 * (2 * w + a2);
+                V8 fdv[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 av = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
+                        av = Mma<T>::run(fdv[s], fA[t][s], av);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
+                    float dbv = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
+                    dbv = sum_over_g(dbv);
+                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
+                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                }
+            }
+        }
+        lds_barrier();                                          // (dv_new and v are done with)
+        put_tile<KD>(sDW, PK, rDW, tid);
+        put_tile<KD>(sK, PK, rK, tid);
+        lds_barrier();
+        if (u + gridDim.x < units) fetch_first(u + gridDim.x, tid);
+
+        // ---- second half: dX's second term dw (e^gam k)^T, dA = stril(dX diag(beta)), k k^T of the same rows and columns ----
+        f32x4 kkT[4];
+        {
+            V8 fw[4], fk[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
+            }
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                f32x4 dXw = ZERO4;
+                kkT[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
+                        dXw = Mma<T>::run(fw[s], bk, dXw);
+                        kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
+                    }
+                }
+                const int j = 16 * tj + c16;
+                const float ej = __expf(sGam[j]), bj = sBeta[j];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    sM1[i * P64 + j] = (T)(i > j ? (dXv[tj][r] + ej * dXw[r]) * bj : 0.f);
+                }
+            }
+        }
+        // d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
+        f32x4 dk[NA][4];
+        {
+            V8 fA[4][2];
+            float ej[4], bj[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                ej[t] = __expf(sGam[16 * t + c16]);
+                bj[t] = sBeta[16 * t + c16];
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
+                const int n16 = feat(a2);
+                V8 fdw[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 ak = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;
+                        ak = Mma<T>::run(fdw[s], fA[t][s], ak);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
+                    float dot = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
+                    dot = sum_over_g(dot);
+                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
+                    dk[a2][t] = ak * (bj[t] * ej[t]);
+                }
+            }
+        }
+        lds_barrier();
+        // Y = dA A^T
+        {
+            V8 fd[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+                const int l = 16 * tl + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+            }
+        }
+        lds_barrier();
+        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
+        {
+            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
+            V8 fAt[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+                if (tl <= w) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
+                }
+                const f32x4 kk = kkT[tl];
+                const int l = 16 * tl + c16;
+                const float gl = sGam[l];
+                float colF = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    float E = 0.f;
+                    if (i > l) {
+                        const float d = __expf(gi[r] - gl), dL = -acc[r];
+                        dbi[r] += dL * kk[r] * d;
+                        E = dL * bi[r] * d;
+                        const float F = E * kk[r];
+                        rowF[r] += F;
+                        colF += F;
+                    }
+                    sM1[i * P64 + l] = (T)E;
+                }
+                colF = sum_over_g(colF);
+                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
+                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
+            }
+        }
+        lds_barrier();
+        // dk += E k + E^T k, on top of what the previous kernel left
+        {
+            V8 fk[NA][2];
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
+                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
+                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
+                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
+                }
+                const int x = 16 * t + c16;
+                if (x < c.valid) {
+#pragma unroll
+                    for (int a2 = 0; a2 < NA; ++a2) {
+                        f32x4 acc = dk[a2][t];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
+                    }
+                }
+            }
+        }
+        if (w == 0) {
+            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_down(x, off, 64);
+                if (lane + off < 64) x += y;
+            }
+            if (lane < c.valid) {
+                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
+                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
+            }
+        }
+        lds_barrier();
+    }
+}
+
 template <typename T, int KT, bool COMBA = false>
 static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t stream) {
     BwdParams p = p_in;
@@ -1239,7 +1536,8 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         state,
         dstate,
         {(const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
-        {(const void*)gdn_bwd_wy_kernel<T, KT, COMBA>, bwd_wy_smem<KT, COMBA>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
+        (KT == 1 && !COMBA) ? K{(const void*)gdn_bwd_wy2_kernel<T>, BWD_WY2_SMEM, "gdn_bwd_wy2_kernel", units < 512u ? units : 512u}
+                            : K{(const void*)gdn_bwd_wy_kernel<T, KT, COMBA>, bwd_wy_smem<KT, COMBA>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
     for (int i = 0; i < 5; ++i) {
         if (ks[i].grid == 0) continue;
