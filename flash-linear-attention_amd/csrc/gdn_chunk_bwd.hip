@@ -76,6 +76,9 @@ struct BwdParams {
     void* dq; void* dk; void* dv; float* dg; float* dbeta; float* dh0;
     const void* pk; void* dp;            // (comba) the second key, the one the prediction is made with, and its gradient
     float* dgk;                          // (KDA) gradient of the log decays [B,T,HV,128] fp32
+    // q and k are rows after an l2 normalisation and these its factors [B,T,H] (H == HV, one block of key features): dq and dk
+    // come back as the gradients of the rows before it, dx = (dy - y (y . dy)) rstd (fla/modules/l2norm.py:265-298)
+    const float* q_rstd; const float* k_rstd;
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     BwdWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;
@@ -674,9 +677,10 @@ __global__ __launch_bounds__(256) void gdn_bwd_scans_apart_kernel(BwdParams p, i
 // ---------------------------------------------------------------------------------------------
 // One workgroup per CU walks over the units and fetches everything the next unit needs (five tiles and, with one block of key
 // features, its fragments of S and dS) into registers while it works on the current one.
-template <int KT> constexpr size_t bwd_dqkw_smem() { return (3 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 64 * P64) * 2 + 320 * 4; }
+// L2: dq goes back through the l2 normalisation of q before it is written (its rows wait in registers for the row sums of q . dq).
+template <int KT> constexpr size_t bwd_dqkw_smem() { return (3 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 64 * P64) * 2 + 640 * 4; }
 
-template <typename T, int KT>
+template <typename T, int KT, bool L2 = false>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -685,12 +689,14 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
     T* sDO = (T*)smem; T* sVn = sDO + 64 * P128; T* sDvn = sVn + 64 * P128; T* sK = sDvn + 64 * P128; T* sQ = sK + 64 * PK;
     T* sDP = sQ + 64 * PK;
     float* sGam = (float*)(sDP + 64 * P64); float* sDg = sGam + 64;    // sDg [4][64]: a row per wave, added up in a fixed order (same bits every run)
+    float* sQd = sDg + 256; float* sRq = sQd + 256;                    // (L2) q . dq per wave and token; the tokens' factors
+    static_assert(!L2 || KT == 1, "the rows of dq wait in the registers of one block of key features");
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
 
     TileRegs<BD> rDO, rVn, rDvn;
     TileRegs<KD> rK, rQ;
     V8 rS[2][4], rdS[2][4];
-    float rGam = 0.f;
+    float rGam = 0.f, rRq = 0.f;
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
@@ -714,6 +720,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
             fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         }
         if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
+        if constexpr (L2) rRq = tid < c.valid ? p.q_rstd[(c.tok0 + tid) * p.H + hq] : 0.f;
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
@@ -730,6 +737,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
         if (tid < 64) sGam[tid] = rGam;
+        if constexpr (L2) { if (tid < 64) sRq[tid] = rRq; }
         sDg[tid] = 0.f;
         V8 sf[2][4], df[2][4];
         if constexpr (KT == 1) {
@@ -742,6 +750,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         if (u + gridDim.x < units) fetch(u + gridDim.x);
 
         float sdot = 0.f, dglast = 0.f;
+        f32x4 dq_rows[L2 ? 2 : 1][4];
 #pragma unroll 1
         for (int kb = 0; kb < KT; ++kb) {                       // (a real loop: one block's accumulators at a time)
             if (KT > 1) {
@@ -851,18 +860,23 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
                         for (int a2 = 0; a2 < 2; ++a2) dk[a2] = Mma<T>::run(fq[a2][s], e, dk[a2]);
                     }
                 }
-                float dgx = 0.f;
+                float qdq = 0.f, kdk = 0.f;
 #pragma unroll
                 for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) dgx += (float)q4[a2][r] * dq[a2][r] - (float)k4[a2][r] * dk[a2][r];
-                dgx = sum_over_g(dgx);
+                    for (int r = 0; r < 4; ++r) { qdq += (float)q4[a2][r] * dq[a2][r]; kdk += (float)k4[a2][r] * dk[a2][r]; }
+                const float dgx = sum_over_g(qdq - kdk);
                 if (g == 0) atomicAdd(&sDg[64 * w + x], dgx);
+                if constexpr (L2) {
+                    qdq = sum_over_g(qdq);
+                    if (g == 0) sQd[64 * w + x] = qdq;
+                    dq_rows[0][t] = dq[0]; dq_rows[1][t] = dq[1];
+                }
                 if (x < c.valid) {
 #pragma unroll
                     for (int a2 = 0; a2 < 2; ++a2) {
                         const int n16 = BD * kb + 16 * (2 * w + a2);
-                        *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(dq[a2]);
+                        if constexpr (!L2) *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(dq[a2]);
                         *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(dk[a2]);
                     }
                 }
@@ -872,6 +886,24 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
         dglast = sum_over_c16(sum_over_g(dglast));
         if (lane == 0) atomicAdd(&sDg[64 * w + 63], dglast);
         lds_barrier();
+        if constexpr (L2) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                const float dot = (sQd[x] + sQd[64 + x]) + (sQd[128 + x] + sQd[192 + x]), rs = sRq[x];
+                if (x < c.valid) {
+#pragma unroll
+                    for (int a2 = 0; a2 < 2; ++a2) {
+                        const int n16 = 16 * (2 * w + a2);
+                        const V4 q4 = *(const V4*)(sQ + x * PK + n16 + 4 * g);
+                        f32x4 out;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) out[r] = (dq_rows[a2][t][r] - (float)q4[r] * dot) * rs;
+                        *(V4*)((T*)p.dq + ((c.tok0 + x) * p.HV + hv) * KD + n16 + 4 * g) = pack4<T>(out);
+                    }
+                }
+            }
+        }
         if (tid < 64) p.ws.Dgam[u * 64 + tid] = (sDg[tid] + sDg[64 + tid]) + (sDg[128 + tid] + sDg[192 + tid]);
         lds_barrier();
     }
@@ -1183,9 +1215,10 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 // workgroups share a CU: the unit is walked in two halves over the same two tile places - first dv_new and v (dX's first
 // term, dv and its share of dbeta), then dw and k (dX's second term, k k^T, the first part of dk) - with the second pair
 // on its way into registers during the first half and the next unit's first pair during the second.
-constexpr size_t BWD_WY2_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 640 * 4;
+// L2: dk goes back through the l2 normalisation of k before it is written.
+constexpr size_t BWD_WY2_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 960 * 4;
 
-template <typename T>
+template <typename T, bool L2 = false>
 __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -1194,11 +1227,12 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
     T* sX0 = (T*)smem; T* sX1 = sX0 + 64 * P128;               // dv_new | v, then dw | k
     T* sA = sX1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
     float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    float* sKd = sDb + 256; float* sRk = sKd + 256;              // (L2) k . dk per wave and token; the tokens' factors
     T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1;
 
     TileRegs<BD> rDvn, rV, rDW, rK;
     TileRegs<CH> rA;
-    float rGam = 0.f, rDg = 0.f;
+    float rGam = 0.f, rDg = 0.f, rRk = 0.f;
     uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch_first = [&](int64_t u, int tid) {
         const int hv = (int)(u % p.HV);
@@ -1210,6 +1244,7 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
             rGam = p.ws.Gam[u * 64 + tid];
             rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
             rDg = p.ws.Dgam[u * 64 + tid];
+            if constexpr (L2) rRk = tid < c.valid ? p.k_rstd[(c.tok0 + tid) * p.H + hv] : 0.f;
         }
     };
     fetch_first(blockIdx.x, threadIdx.x);
@@ -1225,7 +1260,7 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<BD>(sV, P128, rV, tid);
         put_tile<CH>(sA, P64, rA, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); }
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); if constexpr (L2) sRk[tid] = rRk; }
         sDg[tid] = tid < 64 ? rDg : 0.f;
         sDb[tid] = 0.f;
         // the second pair of this unit, and what the previous kernel left in dk at this lane's places
@@ -1449,13 +1484,41 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
                     }
                 }
                 const int x = 16 * t + c16;
-                if (x < c.valid) {
+                if constexpr (L2) {
+                    float kdk = 0.f;
+#pragma unroll
+                    for (int a2 = 0; a2 < NA; ++a2) {
+                        const V4 k4 = *(const V4*)(sK + x * PK + feat(a2) + 4 * g);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) { dk[a2][t][r] += (float)dk_old[a2][t][r]; kdk += (float)k4[r] * dk[a2][t][r]; }
+                    }
+                    kdk = sum_over_g(kdk);
+                    if (g == 0) sKd[64 * w + x] = kdk;
+                } else if (x < c.valid) {
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) {
                         f32x4 acc = dk[a2][t];
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
                         *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
+                    }
+                }
+            }
+        }
+        if constexpr (L2) {
+            lds_barrier();
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                const float dot = (sKd[x] + sKd[64 + x]) + (sKd[128 + x] + sKd[192 + x]), rs = sRk[x];
+                if (x < c.valid) {
+#pragma unroll
+                    for (int a2 = 0; a2 < NA; ++a2) {
+                        const V4 k4 = *(const V4*)(sK + x * PK + feat(a2) + 4 * g);
+                        f32x4 out;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) out[r] = (dk[a2][t][r] - (float)k4[r] * dot) * rs;
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(out);
                     }
                 }
             }
@@ -1531,12 +1594,13 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, KT>, bwd_scans_apart_smem<32, KT>(), "gdn_bwd_scans_apart_kernel", state.grid + dstate.grid};
         dstate.grid = 0;
     }
+    const bool l2 = KT == 1 && !COMBA && p.q_rstd;          // (the entry has checked that both factors come together, with H == HV)
     const K ks[5] = {
         {(const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
         dstate,
-        {(const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
-        (KT == 1 && !COMBA) ? K{(const void*)gdn_bwd_wy2_kernel<T>, BWD_WY2_SMEM, "gdn_bwd_wy2_kernel", units < 512u ? units : 512u}
+        {l2 ? (const void*)gdn_bwd_dqkw_kernel<T, 1, true> : (const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
+        (KT == 1 && !COMBA) ? K{l2 ? (const void*)gdn_bwd_wy2_kernel<T, true> : (const void*)gdn_bwd_wy2_kernel<T>, BWD_WY2_SMEM, "gdn_bwd_wy2_kernel", units < 512u ? units : 512u}
                             : K{(const void*)gdn_bwd_wy_kernel<T, KT, COMBA>, bwd_wy_smem<KT, COMBA>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
     };
     for (int i = 0; i < 5; ++i) {
@@ -1560,7 +1624,7 @@ extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, 
 
 // Both operators' entry: `pk` (and `dp`) non-NULL selects comba.
 static int chunk_bwd_entry(
-    const char* who, bool comba,
+    const char* who, bool comba, const float* q_rstd, const float* k_rstd,
     const void* q, const void* k, const void* pk, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,
     void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
@@ -1595,6 +1659,9 @@ static int chunk_bwd_entry(
     GDN_CHECK_ARG(q && k && v && beta && dout && dq && dk && dv && dg && dbeta, GDN_ERR_INVALID,
                   "%s: q, k, v, beta, do, dq, dk, dv, dg, dbeta must not be NULL", who);
     GDN_CHECK_ARG(!comba || (pk && dp && g), GDN_ERR_INVALID, "%s: p, g and dp must not be NULL", who);
+    GDN_CHECK_ARG(!q_rstd == !k_rstd, GDN_ERR_INVALID, "%s: q_rstd and k_rstd come together", who);
+    GDN_CHECK_ARG(!q_rstd || (H == HV && K == BD), GDN_ERR_UNSUPPORTED,
+                  "%s: the way back through the l2 normalisation is taken in here for H == HV and K = 128 only", who);
     for (const void* x : {q, k, pk, v, dout, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dp, (const void*)dv, (const void*)dh0})
         GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
     GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
@@ -1603,7 +1670,8 @@ static int chunk_bwd_entry(
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
-    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0; p.pk = pk; p.dp = dp;
+    p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0; p.pk = pk; p.dp = dp; p.dgk = nullptr;
+    p.q_rstd = q_rstd; p.k_rstd = k_rstd;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
@@ -1622,7 +1690,22 @@ extern "C" int gdn_chunk_bwd(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
-    return chunk_bwd_entry("gdn_chunk_bwd", false, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
+    return chunk_bwd_entry("gdn_chunk_bwd", false, nullptr, nullptr, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
+                           cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
+                           scale, qkv_dtype, gb_dtype, flags, stream);
+}
+
+extern "C" int gdn_chunk_bwd_qk_l2norm(
+    const void* q, const void* k, const float* q_rstd, const float* k_rstd, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    GDN_CHECK_ARG(T == 0 || num_chunks == 0 || (q_rstd && k_rstd), GDN_ERR_INVALID, "gdn_chunk_bwd_qk_l2norm: q_rstd and k_rstd must not be NULL");
+    return chunk_bwd_entry("gdn_chunk_bwd_qk_l2norm", false, q_rstd, k_rstd, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
@@ -1636,7 +1719,7 @@ extern "C" int gdn_chunk_comba_bwd(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
-    return chunk_bwd_entry("gdn_chunk_comba_bwd", true, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
+    return chunk_bwd_entry("gdn_chunk_comba_bwd", true, nullptr, nullptr, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
@@ -1690,6 +1773,7 @@ extern "C" int gdn_chunk_kda_bwd(
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
     p.dq = dq; p.dk = dk; p.dv = dv; p.dg = nullptr; p.dbeta = dbeta; p.dh0 = dh0; p.pk = nullptr; p.dp = nullptr; p.dgk = dg;
+    p.q_rstd = p.k_rstd = nullptr;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;

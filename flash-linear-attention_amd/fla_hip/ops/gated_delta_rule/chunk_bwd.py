@@ -140,12 +140,17 @@ def chunk_gated_delta_rule_bwd(
     lib = _lib.load()
     ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, KD)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    _lib.check(lib.gdn_chunk_bwd(
-        ptr(qw), ptr(kw), ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
-        ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
-        ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
-        B, T, H, HV, KD, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
-        current_stream_ptr(dev)))
+    tail = (ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
+            ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
+            ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
+            B, T, H, HV, KD, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
+            current_stream_ptr(dev))
+    if q_rstd is not None and k_rstd is not None and H == HV and KD == _DIM:
+        # the way back through the l2 normalisation inside the kernels that produce dq and dk
+        _lib.check(lib.gdn_chunk_bwd_qk_l2norm(ptr(qw), ptr(kw), ptr(as_f32(q_rstd).contiguous()), ptr(as_f32(k_rstd).contiguous()), *tail))
+        q_rstd = k_rstd = None
+    else:
+        _lib.check(lib.gdn_chunk_bwd(ptr(qw), ptr(kw), *tail))
     dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
     dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
     dv = dv[..., :V].to(out_dtype)

@@ -274,6 +274,27 @@ int gdn_chunk_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * gdn_chunk_bwd for q and k that are rows after an l2 normalisation (use_qk_l2norm_in_kernel): dq and dk come back as the
+ * gradients of the rows BEFORE it.  Replaces chunk_gated_delta_rule_bwd followed by the two l2norm_bwd calls of
+ * ChunkGatedDeltaRuleFunction.backward (fla/ops/gated_delta_rule/chunk.py:385-393; fla/modules/l2norm.py:265-298):
+ * dx = (dy - y (y . dy)) rstd per row, taken inside the kernels that produce dq and dk, from their fp32 results.
+ * Arguments as for gdn_chunk_bwd, and:
+ *   q, k: the normalised rows, as gdn_l2norm_fwd returns them
+ *   q_rstd, k_rstd [B,T,H] fp32: its factors 1/sqrt(sum x^2 + eps); both must be given
+ *   H == HV and K = 128 only (GDN_ERR_UNSUPPORTED otherwise: call gdn_chunk_bwd, then gdn_l2norm_bwd, which also
+ *   adds up the value heads of a q/k head).
+ */
+int gdn_chunk_bwd_qk_l2norm(
+    const void* q, const void* k, const float* q_rstd, const float* k_rstd, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Backward pass of the chunked comba operator.  Replaces chunk_comba_bwd (fla/ops/comba/chunk.py:92-178): the
  * gated delta rule's backward with the comba forms of recompute_w_u_fwd and prepare_wy_repr_bwd
  * (fla/ops/comba/wy_fast.py), which form A and w from the second key p and the decay in front of each token
