@@ -76,8 +76,11 @@ struct BwdParams {
     void* dq; void* dk; void* dv; float* dg; float* dbeta; float* dh0;
     const void* pk; void* dp;            // (comba) the second key, the one the prediction is made with, and its gradient
     float* dgk;                          // (KDA) gradient of the log decays [B,T,HV,128] fp32
-    // q and k are rows after an l2 normalisation and these its factors [B,T,H] (H == HV, one block of key features): dq and dk
-    // come back as the gradients of the rows before it, dx = (dy - y (y . dy)) rstd (fla/modules/l2norm.py:265-298)
+    // The l2 normalisation of q and k taken in here (H == HV, one block of key features): the rows as the caller has them; q and k
+    // above are then places in the workspace that the prepare kernel fills with the normalised rows, and these with the factors
+    // [tokens,H] (fla/modules/l2norm.py:222-262); dq and dk come back as the gradients of the rows before the normalisation,
+    // dx = (dy - y (y . dy)) rstd (fla/modules/l2norm.py:265-298).  NULL: q and k are what the recurrence uses.
+    const void* q_raw; const void* k_raw;
     const float* q_rstd; const float* k_rstd;
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     BwdWs ws;
@@ -139,7 +142,33 @@ template <int KT, bool COMBA = false> constexpr size_t bwd_prep_smem() {
     return ((2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + ((COMBA ? 0 : 64 * PL) + 192) * 4;
 }
 
-template <typename T, int KT, bool COMBA = false>
+// Rows of a tile on their way from memory to LDS (a row: 16 lanes next to each other, 8 features each) divided by their
+// length, as gdn_l2norm_fwd does it; the normalised rows and the factors are left for the kernels that follow.
+template <typename T>
+__device__ __forceinline__ void l2norm_tile_rows(TileRegs<BD>& r, T* out, float* rstd_out, int H, int valid, int tid) {
+    typedef typename Mma<T>::V8 V8;
+    const int row0 = tid >> 4, pc = tid & 15;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        V8 x = __builtin_bit_cast(V8, r.x[i]);
+        float f[8], ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { f[e] = (float)x[e]; ss += f[e] * f[e]; }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) ss += __shfl_xor(ss, off, 64);
+        const float rs = rsqrtf(ss + 1e-6f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (T)(f[e] * rs);
+        r.x[i] = __builtin_bit_cast(u32x4, x);
+        const int row = row0 + 16 * i;
+        if (row < valid) {
+            *(u32x4*)(out + (int64_t)row * H * BD + pc * 8) = r.x[i];
+            if (pc == 0) rstd_out[(int64_t)row * H] = rs;
+        }
+    }
+}
+
+template <typename T, int KT, bool COMBA = false, bool L2 = false>
 __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -160,8 +189,8 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
         const ChunkAt c = chunk_at(p, u / p.HV);
-        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
-        fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        fetch_tile<KD>(rK, (const T*)(L2 ? p.k_raw : p.k) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        fetch_tile<KD>(rQ, (const T*)(L2 ? p.q_raw : p.q) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         rG = rB = 0;
@@ -177,6 +206,13 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         int tid_opaque = threadIdx.x;
         asm volatile("" : "+v"(tid_opaque));
         const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        if constexpr (L2) {
+            static_assert(!L2 || (KT == 1 && !COMBA), "one block of key features, one key");
+            const int hv = (int)(u % p.HV);                      // (== the q/k head)
+            const ChunkAt c = chunk_at(p, u / p.HV);
+            l2norm_tile_rows<T>(rK, (T*)p.k + (c.tok0 * p.H + hv) * KD, (float*)p.k_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
+            l2norm_tile_rows<T>(rQ, (T*)p.q + (c.tok0 * p.H + hv) * KD, (float*)p.q_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
+        }
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
         put_tile<BD>(sV, P128, rV, tid);
@@ -1594,9 +1630,9 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, KT>, bwd_scans_apart_smem<32, KT>(), "gdn_bwd_scans_apart_kernel", state.grid + dstate.grid};
         dstate.grid = 0;
     }
-    const bool l2 = KT == 1 && !COMBA && p.q_rstd;          // (the entry has checked that both factors come together, with H == HV)
+    const bool l2 = KT == 1 && !COMBA && p.q_raw;           // (the entry has checked H == HV)
     const K ks[5] = {
-        {(const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
+        {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, false, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
         dstate,
         {l2 ? (const void*)gdn_bwd_dqkw_kernel<T, 1, true> : (const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
@@ -1624,7 +1660,7 @@ extern "C" size_t gdn_chunk_bwd_workspace_bytes(int64_t num_chunks, int64_t HV, 
 
 // Both operators' entry: `pk` (and `dp`) non-NULL selects comba.
 static int chunk_bwd_entry(
-    const char* who, bool comba, const float* q_rstd, const float* k_rstd,
+    const char* who, bool comba, bool l2,
     const void* q, const void* k, const void* pk, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,
     void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
@@ -1659,19 +1695,27 @@ static int chunk_bwd_entry(
     GDN_CHECK_ARG(q && k && v && beta && dout && dq && dk && dv && dg && dbeta, GDN_ERR_INVALID,
                   "%s: q, k, v, beta, do, dq, dk, dv, dg, dbeta must not be NULL", who);
     GDN_CHECK_ARG(!comba || (pk && dp && g), GDN_ERR_INVALID, "%s: p, g and dp must not be NULL", who);
-    GDN_CHECK_ARG(!q_rstd == !k_rstd, GDN_ERR_INVALID, "%s: q_rstd and k_rstd come together", who);
-    GDN_CHECK_ARG(!q_rstd || (H == HV && K == BD), GDN_ERR_UNSUPPORTED,
-                  "%s: the way back through the l2 normalisation is taken in here for H == HV and K = 128 only", who);
+    GDN_CHECK_ARG(!l2 || (H == HV && K == BD), GDN_ERR_UNSUPPORTED,
+                  "%s: the l2 normalisation is taken in here for H == HV and K = 128 only", who);
     for (const void* x : {q, k, pk, v, dout, (const void*)h0, (const void*)dht, (const void*)dq, (const void*)dk, (const void*)dp, (const void*)dv, (const void*)dh0})
         GDN_CHECK_ARG(((uintptr_t)x % 16) == 0, GDN_ERR_INVALID, "%s: tensors must be 16-byte aligned", who);
     GDN_CHECK_ARG(((uintptr_t)workspace % 256) == 0, GDN_ERR_INVALID, "%s: the workspace must be 256-byte aligned", who);
     BwdParams p;
-    const size_t need = bwd_ws_layout(num_chunks * HV, K, (char*)workspace, &p.ws);
+    size_t need = bwd_ws_layout(num_chunks * HV, K, (char*)workspace, &p.ws);
+    const size_t rows_bytes = ws_align((size_t)(B * T * H) * BD * 2), factors_bytes = ws_align((size_t)(B * T * H) * 4);
+    const size_t l2_at = need;
+    if (l2) need += 2 * rows_bytes + 2 * factors_bytes;
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
+    p.q_raw = p.k_raw = nullptr; p.q_rstd = p.k_rstd = nullptr;
+    if (l2) {
+        char* at = (char*)workspace + l2_at;
+        p.q_raw = q; p.k_raw = k;
+        q = at; k = at + rows_bytes;
+        p.q_rstd = (const float*)(at + 2 * rows_bytes); p.k_rstd = (const float*)(at + 2 * rows_bytes + factors_bytes);
+    }
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
     p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0; p.pk = pk; p.dp = dp; p.dgk = nullptr;
-    p.q_rstd = q_rstd; p.k_rstd = k_rstd;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;
@@ -1690,13 +1734,19 @@ extern "C" int gdn_chunk_bwd(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
-    return chunk_bwd_entry("gdn_chunk_bwd", false, nullptr, nullptr, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
+    return chunk_bwd_entry("gdn_chunk_bwd", false, false, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
 
+extern "C" size_t gdn_chunk_bwd_qk_l2norm_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t K, int64_t tokens) {
+    if (num_chunks < 0 || HV < 1 || K != 128 || tokens < 0) return 0;
+    return gdn::bwd_ws_layout(num_chunks * HV, K, nullptr, nullptr) + 2 * gdn::ws_align((size_t)(tokens * HV) * gdn::BD * 2) +
+           2 * gdn::ws_align((size_t)(tokens * HV) * 4);
+}
+
 extern "C" int gdn_chunk_bwd_qk_l2norm(
-    const void* q, const void* k, const float* q_rstd, const float* k_rstd, const void* v, const void* g, const void* beta,
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,
     void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
@@ -1704,8 +1754,7 @@ extern "C" int gdn_chunk_bwd_qk_l2norm(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
-    GDN_CHECK_ARG(T == 0 || num_chunks == 0 || (q_rstd && k_rstd), GDN_ERR_INVALID, "gdn_chunk_bwd_qk_l2norm: q_rstd and k_rstd must not be NULL");
-    return chunk_bwd_entry("gdn_chunk_bwd_qk_l2norm", false, q_rstd, k_rstd, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
+    return chunk_bwd_entry("gdn_chunk_bwd_qk_l2norm", false, true, q, k, nullptr, v, g, beta, h0, dout, dht, dq, dk, nullptr, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
@@ -1719,7 +1768,7 @@ extern "C" int gdn_chunk_comba_bwd(
     int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
     int64_t N, int64_t num_chunks,
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
-    return chunk_bwd_entry("gdn_chunk_comba_bwd", true, nullptr, nullptr, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
+    return chunk_bwd_entry("gdn_chunk_comba_bwd", true, false, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
                            cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
@@ -1773,7 +1822,7 @@ extern "C" int gdn_chunk_kda_bwd(
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
     p.dq = dq; p.dk = dk; p.dv = dv; p.dg = nullptr; p.dbeta = dbeta; p.dh0 = dh0; p.pk = nullptr; p.dp = nullptr; p.dgk = dg;
-    p.q_rstd = p.k_rstd = nullptr;
+    p.q_raw = p.k_raw = nullptr; p.q_rstd = p.k_rstd = nullptr;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;

@@ -104,9 +104,8 @@ SIGNATURES['gdn_chunk_bwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
-SIGNATURES['gdn_chunk_bwd_qk_l2norm'] = (c_int, [
-    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k q_rstd k_rstd v g beta
-    *SIGNATURES['gdn_chunk_bwd'][1][5:]])
+SIGNATURES['gdn_chunk_bwd_qk_l2norm_workspace_bytes'] = (c_size_t, [c_int64, c_int64, c_int64, c_int64])
+SIGNATURES['gdn_chunk_bwd_qk_l2norm'] = SIGNATURES['gdn_chunk_bwd']      # (q, k before their l2 normalisation)
 SIGNATURES['gdn_chunk_comba_bwd'] = (c_int, [
     c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,  # q k p v g beta
     c_void_p, c_void_p, c_void_p,                      # h0 dout dht

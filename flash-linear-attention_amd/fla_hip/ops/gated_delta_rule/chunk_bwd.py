@@ -40,12 +40,15 @@ def chunk_gated_delta_rule_bwd(
     chunk_size: int = 64,
     q_rstd: torch.Tensor | None = None,
     k_rstd: torch.Tensor | None = None,
+    qk_l2norm: bool = False,
 ):
     """q, k ``[B,T,H,K]``, v, do ``[B,T,HV,V]``, g (log decay), beta ``[B,T,HV]`` as the recurrence uses them.
     Returns ``(dq, dk, dv, dbeta, dg, dh0)``: dq, dk, dv in q's dtype, dbeta, dg fp32, dh0 fp32 (None without
     ``initial_state``).  With ``q_rstd``, ``k_rstd`` (the factors ``l2norm_fwd`` returns next to the normalised rows
     passed as q and k) dq and dk are the gradients of the rows before normalisation: the reference's ``l2norm_bwd``
-    (chunk.py:385-387) happens in the kernel that also adds up the value heads of a q/k head."""
+    (chunk.py:385-387) happens in the kernel that also adds up the value heads of a q/k head.  With ``qk_l2norm`` q and k
+    are the rows BEFORE their l2 normalisation and dq, dk the gradients of those: one C call (``gdn_chunk_bwd_qk_l2norm``)
+    where every value head has a q/k head of its own and K <= 128, ``l2norm_fwd`` and the route above otherwise."""
     dev = require_gpu(q, k, v, beta, do)
     check_operand_shapes(q, k, v, g=g, beta=beta)
     if do.shape != v.shape:
@@ -56,6 +59,11 @@ def chunk_gated_delta_rule_bwd(
         raise NotImplementedError(f'the backward kernels cover key head dims up to {2 * _DIM} (got K={K})')
     KD = _DIM if K <= _DIM else 2 * _DIM
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
+    inside = qk_l2norm and H == HV and KD == _DIM and V <= _DIM
+    if qk_l2norm and not inside:
+        q, q_rstd = l2norm_fwd(q)
+        k, k_rstd = l2norm_fwd(k)
+        q, k = q[..., :K], k[..., :K]                  # (l2norm_fwd pads rows to a multiple of 8)
     nb = (V + _DIM - 1) // _DIM
     if nb > 1:
         # value columns are independent: a head with V > 128 is nb heads of 128 columns that share q, k, g, beta
@@ -138,19 +146,14 @@ def chunk_gated_delta_rule_bwd(
     db = alloc(B, T, HV, dtype=torch.float32, device=dev)
     dh0 = torch.empty(N, HV, KD, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
     lib = _lib.load()
-    ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, KD)
+    ws_bytes = lib.gdn_chunk_bwd_qk_l2norm_workspace_bytes(num_chunks, HV, KD, B * T) if inside else lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, KD)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     tail = (ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
             ptr(dq), ptr(dk), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
             ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
             B, T, H, HV, KD, _DIM, N, num_chunks, float(scale), dtype_code(work), _lib.DTYPE_F32, flags,
             current_stream_ptr(dev))
-    if q_rstd is not None and k_rstd is not None and H == HV and KD == _DIM:
-        # the way back through the l2 normalisation inside the kernels that produce dq and dk
-        _lib.check(lib.gdn_chunk_bwd_qk_l2norm(ptr(qw), ptr(kw), ptr(as_f32(q_rstd).contiguous()), ptr(as_f32(k_rstd).contiguous()), *tail))
-        q_rstd = k_rstd = None
-    else:
-        _lib.check(lib.gdn_chunk_bwd(ptr(qw), ptr(kw), *tail))
+    _lib.check((lib.gdn_chunk_bwd_qk_l2norm if inside else lib.gdn_chunk_bwd)(ptr(qw), ptr(kw), *tail))
     dq = _finish(lib, dq, qw, q_rstd, H, K, out_dtype)
     dk = _finish(lib, dk, kw, k_rstd, H, K, out_dtype)
     dv = dv[..., :V].to(out_dtype)
@@ -213,12 +216,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
     def backward(ctx, do, dht):
         q, k, v, g, beta_raw, h0, cu_seqlens, cu_seqlens_cpu, chunk_indices, A_log, dt_bias = ctx.saved_tensors
         scale, state_v_first, l2, gate, bsig, neg, chunk_size = ctx.opts
-        q_rstd = k_rstd = None
         K = q.shape[-1]
-        if l2:
-            q, q_rstd = l2norm_fwd(q)
-            k, k_rstd = l2norm_fwd(k)
-            q, k = q[..., :K], k[..., :K]                  # (l2norm_fwd pads rows to a multiple of 8)
         beta = beta_raw
         if bsig:
             beta = torch.sigmoid(beta_raw.float()) * (2.0 if neg else 1.0)
@@ -229,7 +227,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             g = -A_log.float().exp() * F.softplus(x)
         dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(
             q, k, v, g, beta, scale, h0, do.contiguous(), dht, state_v_first, cu_seqlens, cu_seqlens_cpu,
-            chunk_indices, chunk_size, q_rstd, k_rstd)
+            chunk_indices, chunk_size, qk_l2norm=l2)
         if bsig:
             s = torch.sigmoid(beta_raw.float())
             db = db * s * (1 - s) * (2.0 if neg else 1.0)

@@ -274,18 +274,20 @@ int gdn_chunk_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
- * gdn_chunk_bwd for q and k that are rows after an l2 normalisation (use_qk_l2norm_in_kernel): dq and dk come back as the
- * gradients of the rows BEFORE it.  Replaces chunk_gated_delta_rule_bwd followed by the two l2norm_bwd calls of
- * ChunkGatedDeltaRuleFunction.backward (fla/ops/gated_delta_rule/chunk.py:385-393; fla/modules/l2norm.py:265-298):
- * dx = (dy - y (y . dy)) rstd per row, taken inside the kernels that produce dq and dk, from their fp32 results.
- * Arguments as for gdn_chunk_bwd, and:
- *   q, k: the normalised rows, as gdn_l2norm_fwd returns them
- *   q_rstd, k_rstd [B,T,H] fp32: its factors 1/sqrt(sum x^2 + eps); both must be given
- *   H == HV and K = 128 only (GDN_ERR_UNSUPPORTED otherwise: call gdn_chunk_bwd, then gdn_l2norm_bwd, which also
- *   adds up the value heads of a q/k head).
+ * gdn_chunk_bwd with the l2 normalisation of q and k taken inside (use_qk_l2norm_in_kernel): q and k are the rows as the
+ * caller has them, dq and dk the gradients of THOSE rows.  Replaces l2norm_fwd (twice), chunk_gated_delta_rule_bwd and
+ * l2norm_bwd (twice) of ChunkGatedDeltaRuleFunction.backward (fla/ops/gated_delta_rule/chunk.py:278-282, 385-393;
+ * fla/modules/l2norm.py:222-298): the first kernel divides the rows by sqrt(sum x^2 + 1e-6) on their way in and leaves
+ * them, with the factors, in the workspace for the kernels that follow; the kernels that produce dq and dk apply
+ * dx = (dy - y (y . dy)) rstd per row to their fp32 results before they write them.
+ * Arguments as for gdn_chunk_bwd, except:
+ *   workspace: at least gdn_chunk_bwd_qk_l2norm_workspace_bytes(num_chunks, HV, K, B * T) bytes (0: unsupported K)
+ *   H == HV and K = 128 only (GDN_ERR_UNSUPPORTED otherwise: call gdn_l2norm_fwd, gdn_chunk_bwd, then gdn_l2norm_bwd,
+ *   which also adds up the value heads of a q/k head).
  */
+size_t gdn_chunk_bwd_qk_l2norm_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t K, int64_t tokens);
 int gdn_chunk_bwd_qk_l2norm(
-    const void* q, const void* k, const float* q_rstd, const float* k_rstd, const void* v, const void* g, const void* beta,
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
     const float* h0, const void* dout, const float* dht,
     void* dq, void* dk, void* dv, float* dg, float* dbeta, float* dh0,
     const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
