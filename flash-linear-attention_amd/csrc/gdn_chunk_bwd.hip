@@ -699,11 +699,11 @@ __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
 template <int VBT, int KT> constexpr size_t bwd_scans_apart_smem() {
     return bwd_state_smem<VBT, KT>() > bwd_dstate_smem<VBT, KT>() ? bwd_state_smem<VBT, KT>() : bwd_dstate_smem<VBT, KT>();
 }
-template <typename T, int VBT, int KT>
-__global__ __launch_bounds__(256) void gdn_bwd_scans_apart_kernel(BwdParams p, int64_t nstate) {
+template <typename T, int VBT, int KT, bool KDA = false>
+__global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_scans_apart_kernel(BwdParams p, int64_t nstate) {
     extern __shared__ __align__(16) char smem[];
-    if (blockIdx.x >= nstate) bwd_dstate_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x - (unsigned)nstate, gridDim.x - (unsigned)nstate);
-    else bwd_state_body<T, VBT, KT, 1, 4>(p, smem, threadIdx.x, blockIdx.x, (unsigned)nstate);
+    if (blockIdx.x >= nstate) bwd_dstate_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x - (unsigned)nstate, gridDim.x - (unsigned)nstate);
+    else bwd_state_body<T, VBT, KT, 1, scan_waves<VBT>(), KDA>(p, smem, threadIdx.x, blockIdx.x, (unsigned)nstate);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1578,9 +1578,9 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
 template <typename T, int KT, bool COMBA = false>
 static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t stream) {
     BwdParams p = p_in;
-    // Value columns per workgroup of the scans: as few as it takes to give every (sequence, head) run its own CU
-    // (their LDS tiles allow one workgroup per CU): a step's length hardly depends on the width of the slice.  With two
-    // blocks of key features the reverse scan's tiles leave room for 32 columns only.
+    // Value columns per workgroup of the scans where the two run one after the other or side by side in one workgroup: as few as
+    // it takes to give every (sequence, head) run its own CU (their LDS tiles allow one workgroup per CU).  With two blocks of
+    // key features the reverse scan's tiles leave room for 32 columns only.
     const int64_t runs1 = p.N * p.HV;
     const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
     const int vbt_d = KT == 1 ? vbt : 32;
@@ -1598,11 +1598,10 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
     }
     unsigned threads[5] = {256, vbt == BD ? 512u : 256u, vbt_d == BD ? 512u : 256u, 256, 256};
     if constexpr (KT == 1) {
-        // both scans side by side in one launch (the second entry then has nothing to launch)
-        static_assert(bwd_scans_smem<64, 1>() <= 160 * 1024, "the two scans' tiles of 64 value columns share a CU's LDS");
-        if (vbt == 32) state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
-        if (vbt == 64) state = {(const void*)gdn_bwd_scans_kernel<T, 64, KT>, bwd_scans_smem<64, KT>(), "gdn_bwd_scans_kernel", runs(64)};
-        if (vbt <= 64) {
+        // both scans side by side in one launch (the second entry then has nothing to launch): what time segments run in, where
+        // every CU has a workgroup already
+        if (vbt == 32) {
+            state = {(const void*)gdn_bwd_scans_kernel<T, 32, KT>, bwd_scans_smem<32, KT>(), "gdn_bwd_scans_kernel", runs(32)};
             threads[1] = 512;
             dstate.grid = 0;
         }
@@ -1629,6 +1628,21 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         second_arg[1] = state.grid;
         state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, KT>, bwd_scans_apart_smem<32, KT>(), "gdn_bwd_scans_apart_kernel", state.grid + dstate.grid};
         dstate.grid = 0;
+    }
+    if constexpr (KT == 1) {
+        // Whole sequences on up to 128 runs: both scans in one launch, every workgroup with a CU to itself, as many value columns
+        // each as that allows.  What a CU moves per step bounds the step (some 22 GB/s per CU, loads and stores together, whatever
+        // shares the CU): 32 KB + c/2 for c columns of the forward scan, 56 KB + c/2 of the reverse one - side by side in one
+        // workgroup the two add up, apart the longer one counts.
+        if (p.nseg == 1 && runs1 <= 128) {
+            const int va = runs1 <= 32 ? 32 : runs1 <= 64 ? 64 : 128;
+            second_arg[1] = runs(va);
+            threads[1] = va == BD ? 512u : 256u;
+            if (va == 32) state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, KT>, bwd_scans_apart_smem<32, KT>(), "gdn_bwd_scans_apart_kernel", 2 * runs(32)};
+            else if (va == 64) state = {(const void*)gdn_bwd_scans_apart_kernel<T, 64, KT>, bwd_scans_apart_smem<64, KT>(), "gdn_bwd_scans_apart_kernel", 2 * runs(64)};
+            else state = {(const void*)gdn_bwd_scans_apart_kernel<T, 128, KT>, bwd_scans_apart_smem<128, KT>(), "gdn_bwd_scans_apart_kernel", 2 * runs(128)};
+            dstate.grid = 0;
+        }
     }
     const bool l2 = KT == 1 && !COMBA && p.q_raw;           // (the entry has checked H == HV)
     const K ks[5] = {

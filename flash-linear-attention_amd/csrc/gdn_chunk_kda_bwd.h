@@ -592,17 +592,18 @@ template <typename T>
 static int launch_bwd_kda(const BwdParams& p, const KdaParams& kp, int64_t num_chunks, int qkv_dtype, hipStream_t stream) {
     if (int rc = launch_kda_prepare(kp, num_chunks, qkv_dtype, stream)) return rc;
     const int64_t runs1 = p.N * p.HV;
-    const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
     const unsigned units = (unsigned)(num_chunks * p.HV);
     auto runs = [&](int v) { return (unsigned)((runs1 + 7) / 8 * 8 * (BD / v)); };
     struct K { const void* f; size_t smem; const char* name; unsigned grid, threads; };
     K state, dstate;
-    if (vbt == 32) {
-        // both scans side by side in one launch
-        state = {(const void*)gdn_bwd_scans_kernel<T, 32, 1, true>, bwd_scans_smem<32, 1>(), "gdn_bwd_scans_kernel", runs(32), 512};
-        dstate = {nullptr, 0, "", 0, 0};
-    } else if (vbt == 64) {
-        state = {(const void*)gdn_bwd_scans_kernel<T, 64, 1, true>, bwd_scans_smem<64, 1>(), "gdn_bwd_scans_kernel", runs(64), 512};
+    int64_t nstate = 0;
+    if (runs1 <= 128) {
+        // both scans in one launch, every workgroup with a CU to itself, as many value columns each as that allows
+        const int va = runs1 <= 32 ? 32 : runs1 <= 64 ? 64 : 128;
+        nstate = runs(va);
+        if (va == 32) state = {(const void*)gdn_bwd_scans_apart_kernel<T, 32, 1, true>, bwd_scans_apart_smem<32, 1>(), "gdn_bwd_scans_apart_kernel", 2 * runs(32), 256};
+        else if (va == 64) state = {(const void*)gdn_bwd_scans_apart_kernel<T, 64, 1, true>, bwd_scans_apart_smem<64, 1>(), "gdn_bwd_scans_apart_kernel", 2 * runs(64), 256};
+        else state = {(const void*)gdn_bwd_scans_apart_kernel<T, 128, 1, true>, bwd_scans_apart_smem<128, 1>(), "gdn_bwd_scans_apart_kernel", 2 * runs(128), 512};
         dstate = {nullptr, 0, "", 0, 0};
     } else {
         state = {(const void*)gdn_bwd_state_kernel<T, 128, 1, true>, bwd_state_smem<128, 1>(), "gdn_bwd_state_kernel", runs(128), 512};
@@ -617,7 +618,7 @@ static int launch_bwd_kda(const BwdParams& p, const KdaParams& kp, int64_t num_c
     for (int i = 0; i < 4; ++i) {
         if (ks[i].grid == 0) continue;
         if (int rc = ensure_dynamic_smem_for(ks[i].f, ks[i].smem, ks[i].name)) return rc;
-        void* args[] = {(void*)&p, (void*)&nunits};
+        void* args[] = {(void*)&p, i == 0 && nstate ? (void*)&nstate : (void*)&nunits};
         if (hipLaunchKernel(ks[i].f, dim3(ks[i].grid), dim3(ks[i].threads), args, ks[i].smem, stream) != hipSuccess) return check_launch(ks[i].name);
         if (int rc = check_launch(ks[i].name)) return rc;
     }
