@@ -948,34 +948,28 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 // ---------------------------------------------------------------------------------------------
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
-// One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.
-// COMBA: L = diag(beta) stril(p k^T o D0), w = X (e^gam0 p): the rows of p take the place of k's wherever k stood on the
-// left of k k^T or under e^gam, their gradient goes to dp, and the exponent of the row side is gam0, with a gradient of its own.
-template <int KT, bool COMBA = false> constexpr size_t bwd_wy_smem() {
-    return (2 * 64 * P128 + (2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + (640 + 320) * 4;
-}
+// One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.  (Two blocks of key
+// features; one block takes gdn_bwd_wy2_kernel below.)
+template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 640 * 4; }
 
-template <typename T, int KT, bool COMBA = false>
+template <typename T, int KT>
 __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
     constexpr int KD = BD * KT, PK = KD + 8, NA = 2 * KT;      // NA tiles of 16 key features per wave: two in every block of 128
     extern __shared__ __align__(16) char smem[];
     T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * PK;
-    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64; T* sP = sM2 + 64 * P64;
-    float* sGam = (float*)(sP + (COMBA ? 64 * PK : 0)); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
-    float* sDg0 = sDb + 256; float* sGam0 = sDg0 + 256;
-    // (sDg, sDb, sDg0 [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
-    T* sRows = COMBA ? sP : sK;
-    float* sGamRow = COMBA ? sGam0 : sGam; float* sDgRow = COMBA ? sDg0 : sDg;
+    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
+    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    // (sDg, sDb [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     auto feat = [&](int a) { return BD * (a >> 1) + 16 * (2 * w + (a & 1)); };       // first key feature of this wave's tile a
 
     TileRegs<BD> rDvn, rV;
-    TileRegs<KD> rDW, rK, rP;
+    TileRegs<KD> rDW, rK;
     TileRegs<CH> rA;
     V4 rDk[NA][4];                                               // what the previous kernel left in dk, at this lane's places
-    float rGam = 0.f, rDg = 0.f, rGam0 = 0.f;
+    float rGam = 0.f, rDg = 0.f;
     uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
         const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
@@ -985,12 +979,10 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
         fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
         fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
-        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if (tid < 64) {
             rGam = p.ws.Gam[u * 64 + tid];
             rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
             rDg = p.ws.Dgam[u * 64 + tid];
-            if constexpr (COMBA) rGam0 = p.ws.Gam0[u * 64 + tid];
         }
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -1010,11 +1002,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
         put_tile<CH>(sA, P64, rA, tid);
         put_tile<KD>(sDW, PK, rDW, tid);
         put_tile<KD>(sK, PK, rK, tid);
-        if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); sGam0[tid] = rGam0; }
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); }
         sDg[tid] = tid < 64 ? rDg : 0.f;
         sDb[tid] = 0.f;
-        sDg0[tid] = 0.f;
         V4 dk_old[NA][4];
 #pragma unroll
         for (int a2 = 0; a2 < NA; ++a2)
@@ -1025,7 +1015,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 
         // Operand fragments are fetched from LDS once and kept: what does not change across an inner loop is loaded outside it.
         // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta));
-        // k k^T (comba: p k^T) of the same rows and columns is formed along the way, for the last step but one
+        // k k^T of the same rows and columns is formed along the way, for the last step but one
         f32x4 kkT[4];
         {
             V8 fa[4], fw[4 * KT], fk[4 * KT];
@@ -1034,7 +1024,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) {
                 fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
-                fk[s] = frag_rows(sRows, PK, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
             }
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
@@ -1046,13 +1036,12 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                     for (int s = 0; s < 4 * KT; ++s) {
                         const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
-                        if constexpr (COMBA) dXw = Mma<T>::run(fw[s], frag_rows(sP, PK, 16 * tj, 32 * s, lane), dXw);
-                        else dXw = Mma<T>::run(fw[s], bk, dXw);
+                        dXw = Mma<T>::run(fw[s], bk, dXw);
                         kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
                     }
                 }
                 const int j = 16 * tj + c16;
-                const float ej = __expf(sGamRow[j]), bj = sBeta[j];
+                const float ej = __expf(sGam[j]), bj = sBeta[j];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int i = 16 * w + 4 * g + r;
@@ -1060,8 +1049,8 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                 }
             }
         }
-        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam  (comba: d(e^gam0 p), into dp, dbeta, dgam0)
-        f32x4 dk[NA][4], dpk[COMBA ? NA : 1][4];
+        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
+        f32x4 dk[NA][4];
         {
             V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
             float ej[4], bj[4];
@@ -1070,7 +1059,7 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
                     if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                ej[t] = __expf(sGamRow[16 * t + c16]);
+                ej[t] = __expf(sGam[16 * t + c16]);
                 bj[t] = sBeta[16 * t + c16];
             }
 #pragma unroll
@@ -1096,6 +1085,317 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
                     if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
                 }
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
+                const int n16 = feat(a2);
+                V8 fdw[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 ak = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;
+                        ak = Mma<T>::run(fdw[s], fA[t][s], ak);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
+                    float dot = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
+                    dot = sum_over_g(dot);
+                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
+                    dk[a2][t] = ak * (bj[t] * ej[t]);
+                }
+            }
+        }
+        lds_barrier();
+        // Y = dA A^T
+        {
+            V8 fd[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+                const int l = 16 * tl + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+            }
+        }
+        lds_barrier();
+        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
+        {
+            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
+            V8 fAt[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+                if (tl <= w) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
+                }
+                const f32x4 kk = kkT[tl];
+                const int l = 16 * tl + c16;
+                const float gl = sGam[l];
+                float colF = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    float E = 0.f;
+                    if (i > l) {
+                        const float d = __expf(gi[r] - gl), dL = -acc[r];
+                        dbi[r] += dL * kk[r] * d;
+                        E = dL * bi[r] * d;
+                        const float F = E * kk[r];
+                        rowF[r] += F;
+                        colF += F;
+                    }
+                    sM1[i * P64 + l] = (T)E;
+                }
+                colF = sum_over_g(colF);
+                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
+                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
+            }
+        }
+        lds_barrier();
+        // dk += E k + E^T k, on top of what the previous kernel left
+        {
+            V8 fk[NA][2];
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
+                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
+                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
+                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
+                    }
+                }
+                const int x = 16 * t + c16;
+                if (x < c.valid) {
+#pragma unroll
+                    for (int a2 = 0; a2 < NA; ++a2) {
+                        f32x4 acc = dk[a2][t];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
+                    }
+                }
+            }
+        }
+        if (w == 0) {
+            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_down(x, off, 64);
+                if (lane + off < 64) x += y;
+            }
+            if (lane < c.valid) {
+                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
+                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// The same kernel for one block of key features in at most 76 KB of LDS, so that two workgroups share a CU: the unit is walked
+// in two halves over the same two tile places - first dv_new and v (dX's first term, dv and its share of dbeta), then dw and k
+// (dX's second term, k k^T, the first part of dk; comba: with the rows of p in a third place) - with the second set on its way
+// into registers during the first half and the next unit's first pair during the second; Y = dA A^T takes dw's place once dw is done with.
+// L2: dk goes back through the l2 normalisation of k before it is written.
+template <bool COMBA = false> constexpr size_t bwd_wy2_smem() { return ((2 + (COMBA ? 1 : 0)) * 64 * P128 + 2 * 64 * P64) * 2 + (960 + 320) * 4; }
+
+template <typename T, bool L2 = false, bool COMBA = false>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_t units) {
+    static_assert(!(L2 && COMBA), "the l2 norm inside: the gated delta rule only");
+    static_assert(2 * bwd_wy2_smem<COMBA>() <= 160 * 1024, "two workgroups per CU");
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    constexpr int KD = BD, PK = P128, NA = 2;
+    extern __shared__ __align__(16) char smem[];
+    T* sX0 = (T*)smem; T* sX1 = sX0 + 64 * P128;               // dv_new | v, then dw | k
+    T* sA = sX1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sP = sM1 + 64 * P64;     // (comba) rows of the second key
+    float* sGam = (float*)(sP + (COMBA ? 64 * P128 : 0)); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    float* sKd = sDb + 256; float* sRk = sKd + 256;              // (L2) k . dk per wave and token; the tokens' factors
+    float* sDg0 = sRk + 64; float* sGam0 = sDg0 + 256;           // (comba)
+    T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1; T* sM2 = sX0;
+    T* sRows = COMBA ? sP : sK;
+    float* sGamRow = COMBA ? sGam0 : sGam; float* sDgRow = COMBA ? sDg0 : sDg;
+
+    TileRegs<BD> rDvn, rV, rDW, rK, rP;
+    TileRegs<CH> rA;
+    float rGam = 0.f, rDg = 0.f, rRk = 0.f, rGam0 = 0.f;
+    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
+    auto fetch_first = [&](int64_t u, int tid) {
+        const int hv = (int)(u % p.HV);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
+        if (tid < 64) {
+            rGam = p.ws.Gam[u * 64 + tid];
+            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
+            rDg = p.ws.Dgam[u * 64 + tid];
+            if constexpr (COMBA) rGam0 = p.ws.Gam0[u * 64 + tid];
+            if constexpr (L2) rRk = tid < c.valid ? p.k_rstd[(c.tok0 + tid) * p.H + hv] : 0.f;
+        }
+    };
+    fetch_first(blockIdx.x, threadIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
+        int tid_opaque = threadIdx.x;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        auto feat = [&](int a) { return 16 * (2 * w + a); };    // first key feature of this wave's tile a
+        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
+        const ChunkAt c = chunk_at(p, u / p.HV);
+        put_tile<BD>(sDvn, P128, rDvn, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        put_tile<CH>(sA, P64, rA, tid);
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); if constexpr (L2) sRk[tid] = rRk; if constexpr (COMBA) sGam0[tid] = rGam0; }
+        sDg[tid] = tid < 64 ? rDg : 0.f;
+        sDb[tid] = 0.f;
+        if constexpr (COMBA) sDg0[tid] = 0.f;
+        // the second pair of this unit, and what the previous kernel left in dk at this lane's places
+        fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
+        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        V4 dk_old[NA][4];
+#pragma unroll
+        for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int x = 16 * t + c16;
+                dk_old[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+                if (x < c.valid) dk_old[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g);
+            }
+        lds_barrier();
+
+        // ---- first half: dX's first term du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), and dv = beta (A^T du) ----
+        f32x4 dXv[4];
+        {
+            V8 fa[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                dXv[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) dXv[tj] = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv[tj]);
+                }
+            }
+        }
+        {
+            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
+            float bj[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                bj[t] = sBeta[16 * t + c16];
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
+                const int n16 = 16 * (2 * w + a2);
+                V8 fdv[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 av = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
+                        av = Mma<T>::run(fdv[s], fA[t][s], av);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
+                    float dbv = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
+                    dbv = sum_over_g(dbv);
+                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
+                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                }
+            }
+        }
+        lds_barrier();                                          // (dv_new and v are done with)
+        put_tile<KD>(sDW, PK, rDW, tid);
+        put_tile<KD>(sK, PK, rK, tid);
+        if constexpr (COMBA) put_tile<KD>(sP, PK, rP, tid);
+        lds_barrier();
+        if (u + gridDim.x < units) fetch_first(u + gridDim.x, tid);
+
+        // ---- second half: dX's second term dw (e^gam k)^T, dA = stril(dX diag(beta)), k k^T of the same rows and columns ----
+        // (comba: e^gam0 p in k's place wherever k stood on the left of k k^T or under e^gam)
+        f32x4 kkT[4];
+        {
+            V8 fw[4], fk[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
+                fk[s] = frag_rows(sRows, PK, 16 * w, 32 * s, lane);
+            }
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                f32x4 dXw = ZERO4;
+                kkT[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
+                        if constexpr (COMBA) dXw = Mma<T>::run(fw[s], frag_rows(sP, PK, 16 * tj, 32 * s, lane), dXw);
+                        else dXw = Mma<T>::run(fw[s], bk, dXw);
+                        kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
+                    }
+                }
+                const int j = 16 * tj + c16;
+                const float ej = __expf(sGamRow[j]), bj = sBeta[j];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    sM1[i * P64 + j] = (T)(i > j ? (dXv[tj][r] + ej * dXw[r]) * bj : 0.f);
+                }
+            }
+        }
+        // d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam  (comba: d(e^gam0 p), into dp, dbeta, dgam0)
+        f32x4 dk[NA][4], dpk[COMBA ? NA : 1][4];
+        {
+            V8 fA[4][2];
+            float ej[4], bj[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                ej[t] = __expf(sGamRow[16 * t + c16]);
+                bj[t] = sBeta[16 * t + c16];
             }
 #pragma unroll
             for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
@@ -1215,311 +1515,6 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
                     }
                 }
                 const int x = 16 * t + c16;
-                if (x < c.valid) {
-#pragma unroll
-                    for (int a2 = 0; a2 < NA; ++a2) {
-                        f32x4 acc = dk[a2][t];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
-                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
-                        if constexpr (COMBA) *(V4*)((T*)p.dp + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(dpk[a2][t]);
-                    }
-                }
-            }
-        }
-        if (w == 0) {
-            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
-            // (comba) dg_t = sum_{s >= t} dgam_s + sum_{s > t} dgam0_s: one reverse cumulative sum of both, less the token's own dgam0
-            float own0 = 0.f;
-            if constexpr (COMBA) { own0 = (sDg0[lane] + sDg0[64 + lane]) + (sDg0[128 + lane] + sDg0[192 + lane]); x += own0; }
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const float y = __shfl_down(x, off, 64);
-                if (lane + off < 64) x += y;
-            }
-            x -= own0;
-            if (lane < c.valid) {
-                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
-                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
-            }
-        }
-        lds_barrier();
-    }
-}
-
-// The same kernel for one block of key features and one key (the gated delta rule itself) in 64 KB of LDS, so that two
-// workgroups share a CU: the unit is walked in two halves over the same two tile places - first dv_new and v (dX's first
-// term, dv and its share of dbeta), then dw and k (dX's second term, k k^T, the first part of dk) - with the second pair
-// on its way into registers during the first half and the next unit's first pair during the second.
-// L2: dk goes back through the l2 normalisation of k before it is written.
-constexpr size_t BWD_WY2_SMEM = (2 * 64 * P128 + 3 * 64 * P64) * 2 + 960 * 4;
-
-template <typename T, bool L2 = false>
-__global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_t units) {
-    typedef typename Mma<T>::V8 V8;
-    typedef typename Mma<T>::V4 V4;
-    constexpr int KD = BD, PK = P128, NA = 2;
-    extern __shared__ __align__(16) char smem[];
-    T* sX0 = (T*)smem; T* sX1 = sX0 + 64 * P128;               // dv_new | v, then dw | k
-    T* sA = sX1 + 64 * P128; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
-    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
-    float* sKd = sDb + 256; float* sRk = sKd + 256;              // (L2) k . dk per wave and token; the tokens' factors
-    T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1;
-
-    TileRegs<BD> rDvn, rV, rDW, rK;
-    TileRegs<CH> rA;
-    float rGam = 0.f, rDg = 0.f, rRk = 0.f;
-    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
-    auto fetch_first = [&](int64_t u, int tid) {
-        const int hv = (int)(u % p.HV);
-        const ChunkAt c = chunk_at(p, u / p.HV);
-        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
-        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
-        if (tid < 64) {
-            rGam = p.ws.Gam[u * 64 + tid];
-            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
-            rDg = p.ws.Dgam[u * 64 + tid];
-            if constexpr (L2) rRk = tid < c.valid ? p.k_rstd[(c.tok0 + tid) * p.H + hv] : 0.f;
-        }
-    };
-    fetch_first(blockIdx.x, threadIdx.x);
-    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
-        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
-        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
-        int tid_opaque = threadIdx.x;
-        asm volatile("" : "+v"(tid_opaque));
-        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
-        auto feat = [&](int a) { return 16 * (2 * w + a); };    // first key feature of this wave's tile a
-        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-        const ChunkAt c = chunk_at(p, u / p.HV);
-        put_tile<BD>(sDvn, P128, rDvn, tid);
-        put_tile<BD>(sV, P128, rV, tid);
-        put_tile<CH>(sA, P64, rA, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); if constexpr (L2) sRk[tid] = rRk; }
-        sDg[tid] = tid < 64 ? rDg : 0.f;
-        sDb[tid] = 0.f;
-        // the second pair of this unit, and what the previous kernel left in dk at this lane's places
-        fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
-        V4 dk_old[NA][4];
-#pragma unroll
-        for (int a2 = 0; a2 < NA; ++a2)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int x = 16 * t + c16;
-                dk_old[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-                if (x < c.valid) dk_old[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g);
-            }
-        lds_barrier();
-
-        // ---- first half: dX's first term du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), and dv = beta (A^T du) ----
-        f32x4 dXv[4];
-        {
-            V8 fa[4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                dXv[tj] = ZERO4;
-                if (tj <= w) {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) dXv[tj] = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv[tj]);
-                }
-            }
-        }
-        {
-            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
-            float bj[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                bj[t] = sBeta[16 * t + c16];
-            }
-#pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
-                const int n16 = 16 * (2 * w + a2);
-                V8 fdv[2];
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    f32x4 av = ZERO4;
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
-                        av = Mma<T>::run(fdv[s], fA[t][s], av);
-                    }
-                    const int j = 16 * t + c16;
-                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
-                    float dbv = 0.f;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
-                    dbv = sum_over_g(dbv);
-                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
-                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
-                }
-            }
-        }
-        lds_barrier();                                          // (dv_new and v are done with)
-        put_tile<KD>(sDW, PK, rDW, tid);
-        put_tile<KD>(sK, PK, rK, tid);
-        lds_barrier();
-        if (u + gridDim.x < units) fetch_first(u + gridDim.x, tid);
-
-        // ---- second half: dX's second term dw (e^gam k)^T, dA = stril(dX diag(beta)), k k^T of the same rows and columns ----
-        f32x4 kkT[4];
-        {
-            V8 fw[4], fk[4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
-                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
-            }
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                f32x4 dXw = ZERO4;
-                kkT[tj] = ZERO4;
-                if (tj <= w) {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
-                        dXw = Mma<T>::run(fw[s], bk, dXw);
-                        kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
-                    }
-                }
-                const int j = 16 * tj + c16;
-                const float ej = __expf(sGam[j]), bj = sBeta[j];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    sM1[i * P64 + j] = (T)(i > j ? (dXv[tj][r] + ej * dXw[r]) * bj : 0.f);
-                }
-            }
-        }
-        // d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
-        f32x4 dk[NA][4];
-        {
-            V8 fA[4][2];
-            float ej[4], bj[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                ej[t] = __expf(sGam[16 * t + c16]);
-                bj[t] = sBeta[16 * t + c16];
-            }
-#pragma unroll
-            for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
-                const int n16 = feat(a2);
-                V8 fdw[2];
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    f32x4 ak = ZERO4;
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        if (32 * s + 31 < 16 * t) continue;
-                        ak = Mma<T>::run(fdw[s], fA[t][s], ak);
-                    }
-                    const int j = 16 * t + c16;
-                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
-                    float dot = 0.f;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
-                    dot = sum_over_g(dot);
-                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
-                    dk[a2][t] = ak * (bj[t] * ej[t]);
-                }
-            }
-        }
-        lds_barrier();
-        // Y = dA A^T
-        {
-            V8 fd[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                f32x4 acc = ZERO4;
-#pragma unroll
-                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
-                const int l = 16 * tl + c16;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
-            }
-        }
-        lds_barrier();
-        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
-        {
-            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
-            V8 fAt[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                f32x4 acc = ZERO4;
-                if (tl <= w) {
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
-                }
-                const f32x4 kk = kkT[tl];
-                const int l = 16 * tl + c16;
-                const float gl = sGam[l];
-                float colF = 0.f;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    float E = 0.f;
-                    if (i > l) {
-                        const float d = __expf(gi[r] - gl), dL = -acc[r];
-                        dbi[r] += dL * kk[r] * d;
-                        E = dL * bi[r] * d;
-                        const float F = E * kk[r];
-                        rowF[r] += F;
-                        colF += F;
-                    }
-                    sM1[i * P64 + l] = (T)E;
-                }
-                colF = sum_over_g(colF);
-                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
-                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
-            }
-        }
-        lds_barrier();
-        // dk += E k + E^T k, on top of what the previous kernel left
-        {
-            V8 fk[NA][2];
-#pragma unroll
-            for (int a2 = 0; a2 < NA; ++a2)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
-                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
-#pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
-                    }
-                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
-                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
-#pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
-                    }
-                }
-                const int x = 16 * t + c16;
                 if constexpr (L2) {
                     float kdk = 0.f;
 #pragma unroll
@@ -1537,6 +1532,7 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
                         *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
+                        if constexpr (COMBA) *(V4*)((T*)p.dp + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(dpk[a2][t]);
                     }
                 }
             }
@@ -1561,11 +1557,15 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
         }
         if (w == 0) {
             float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
+            // (comba) dg_t = sum_{s >= t} dgam_s + sum_{s > t} dgam0_s: one reverse cumulative sum of both, less the token's own dgam0
+            float own0 = 0.f;
+            if constexpr (COMBA) { own0 = (sDg0[lane] + sDg0[64 + lane]) + (sDg0[128 + lane] + sDg0[192 + lane]); x += own0; }
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
                 const float y = __shfl_down(x, off, 64);
                 if (lane + off < 64) x += y;
             }
+            x -= own0;
             if (lane < c.valid) {
                 p.dg[(c.tok0 + lane) * p.HV + hv] = x;
                 p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
@@ -1645,13 +1645,15 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         }
     }
     const bool l2 = KT == 1 && !COMBA && p.q_raw;           // (the entry has checked H == HV)
+    K wy;
+    if constexpr (KT == 1) wy = {l2 ? (const void*)gdn_bwd_wy2_kernel<T, true> : (const void*)gdn_bwd_wy2_kernel<T, false, COMBA>, bwd_wy2_smem<COMBA>(), "gdn_bwd_wy2_kernel", units < 512u ? units : 512u};
+    else wy = {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u};
     const K ks[5] = {
         {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, false, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
         dstate,
         {l2 ? (const void*)gdn_bwd_dqkw_kernel<T, 1, true> : (const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
-        (KT == 1 && !COMBA) ? K{l2 ? (const void*)gdn_bwd_wy2_kernel<T, true> : (const void*)gdn_bwd_wy2_kernel<T>, BWD_WY2_SMEM, "gdn_bwd_wy2_kernel", units < 512u ? units : 512u}
-                            : K{(const void*)gdn_bwd_wy_kernel<T, KT, COMBA>, bwd_wy_smem<KT, COMBA>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u},
+        wy,
     };
     for (int i = 0; i < 5; ++i) {
         if (ks[i].grid == 0) continue;
