@@ -80,8 +80,8 @@ struct BwdParams {
     // above are then places in the workspace that the prepare kernel fills with the normalised rows, and these with the factors
     // [tokens,H] (fla/modules/l2norm.py:222-262); dq and dk come back as the gradients of the rows before the normalisation,
     // dx = (dy - y (y . dy)) rstd (fla/modules/l2norm.py:265-298).  NULL: q and k are what the recurrence uses.
-    const void* q_raw; const void* k_raw;
-    const float* q_rstd; const float* k_rstd;
+    const void* q_raw; const void* k_raw; const void* pk_raw;    // (pk_raw, p_rstd: comba's second key, the same way)
+    const float* q_rstd; const float* k_rstd; const float* p_rstd;
     const void* cu_seqlens; const void* chunk_table; const void* chunk_offsets;
     BwdWs ws;
     int64_t T; int H, HV; int64_t N; int64_t NT;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         const ChunkAt c = chunk_at(p, u / p.HV);
         fetch_tile<KD>(rK, (const T*)(L2 ? p.k_raw : p.k) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<KD>(rQ, (const T*)(L2 ? p.q_raw : p.q) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
-        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)p.pk + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
+        if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)(L2 ? p.pk_raw : p.pk) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         rG = rB = 0;
         if (w == 0 && lane < c.valid) {
@@ -207,11 +207,12 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         asm volatile("" : "+v"(tid_opaque));
         const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         if constexpr (L2) {
-            static_assert(!L2 || (KT == 1 && !COMBA), "one block of key features, one key");
+            static_assert(!L2 || KT == 1, "one block of key features");
             const int hv = (int)(u % p.HV);                      // (== the q/k head)
             const ChunkAt c = chunk_at(p, u / p.HV);
             l2norm_tile_rows<T>(rK, (T*)p.k + (c.tok0 * p.H + hv) * KD, (float*)p.k_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
             l2norm_tile_rows<T>(rQ, (T*)p.q + (c.tok0 * p.H + hv) * KD, (float*)p.q_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
+            if constexpr (COMBA) l2norm_tile_rows<T>(rP, (T*)p.pk + (c.tok0 * p.H + hv) * KD, (float*)p.p_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
         }
         put_tile<KD>(sK, PK, rK, tid);
         put_tile<KD>(sQ, PK, rQ, tid);
@@ -1226,11 +1227,10 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
 // (dX's second term, k k^T, the first part of dk; comba: with the rows of p in a third place) - with the second set on its way
 // into registers during the first half and the next unit's first pair during the second; Y = dA A^T takes dw's place once dw is done with.
 // L2: dk goes back through the l2 normalisation of k before it is written.
-template <bool COMBA = false> constexpr size_t bwd_wy2_smem() { return ((2 + (COMBA ? 1 : 0)) * 64 * P128 + 2 * 64 * P64) * 2 + (960 + 320) * 4; }
+template <bool COMBA = false> constexpr size_t bwd_wy2_smem() { return ((2 + (COMBA ? 1 : 0)) * 64 * P128 + 2 * 64 * P64) * 2 + (960 + 640) * 4; }
 
 template <typename T, bool L2 = false, bool COMBA = false>
 __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_t units) {
-    static_assert(!(L2 && COMBA), "the l2 norm inside: the gated delta rule only");
     static_assert(2 * bwd_wy2_smem<COMBA>() <= 160 * 1024, "two workgroups per CU");
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
@@ -1241,13 +1241,14 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
     float* sGam = (float*)(sP + (COMBA ? 64 * P128 : 0)); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
     float* sKd = sDb + 256; float* sRk = sKd + 256;              // (L2) k . dk per wave and token; the tokens' factors
     float* sDg0 = sRk + 64; float* sGam0 = sDg0 + 256;           // (comba)
+    float* sPd = sGam0 + 64; float* sRp = sPd + 256;             // (comba, L2) p . dp per wave and token; the tokens' factors
     T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1; T* sM2 = sX0;
     T* sRows = COMBA ? sP : sK;
     float* sGamRow = COMBA ? sGam0 : sGam; float* sDgRow = COMBA ? sDg0 : sDg;
 
     TileRegs<BD> rDvn, rV, rDW, rK, rP;
     TileRegs<CH> rA;
-    float rGam = 0.f, rDg = 0.f, rRk = 0.f, rGam0 = 0.f;
+    float rGam = 0.f, rDg = 0.f, rRk = 0.f, rGam0 = 0.f, rRp = 0.f;
     uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch_first = [&](int64_t u, int tid) {
         const int hv = (int)(u % p.HV);
@@ -1261,6 +1262,7 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
             rDg = p.ws.Dgam[u * 64 + tid];
             if constexpr (COMBA) rGam0 = p.ws.Gam0[u * 64 + tid];
             if constexpr (L2) rRk = tid < c.valid ? p.k_rstd[(c.tok0 + tid) * p.H + hv] : 0.f;
+            if constexpr (L2 && COMBA) rRp = tid < c.valid ? p.p_rstd[(c.tok0 + tid) * p.H + hv] : 0.f;
         }
     };
     fetch_first(blockIdx.x, threadIdx.x);
@@ -1276,7 +1278,7 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<BD>(sV, P128, rV, tid);
         put_tile<CH>(sA, P64, rA, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); if constexpr (L2) sRk[tid] = rRk; if constexpr (COMBA) sGam0[tid] = rGam0; }
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); if constexpr (L2) sRk[tid] = rRk; if constexpr (COMBA) sGam0[tid] = rGam0; if constexpr (L2 && COMBA) sRp[tid] = rRp; }
         sDg[tid] = tid < 64 ? rDg : 0.f;
         sDb[tid] = 0.f;
         if constexpr (COMBA) sDg0[tid] = 0.f;
@@ -1525,6 +1527,17 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
                     }
                     kdk = sum_over_g(kdk);
                     if (g == 0) sKd[64 * w + x] = kdk;
+                    if constexpr (COMBA) {
+                        float pdp = 0.f;
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) {
+                            const V4 p4 = *(const V4*)(sP + x * PK + feat(a2) + 4 * g);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) pdp += (float)p4[r] * dpk[a2][t][r];
+                        }
+                        pdp = sum_over_g(pdp);
+                        if (g == 0) sPd[64 * w + x] = pdp;
+                    }
                 } else if (x < c.valid) {
 #pragma unroll
                     for (int a2 = 0; a2 < NA; ++a2) {
@@ -1551,6 +1564,19 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
 #pragma unroll
                         for (int r = 0; r < 4; ++r) out[r] = (dk[a2][t][r] - (float)k4[r] * dot) * rs;
                         *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(out);
+                    }
+                }
+                if constexpr (COMBA) {
+                    const float dotp = (sPd[x] + sPd[64 + x]) + (sPd[128 + x] + sPd[192 + x]), rp = sRp[x];
+                    if (x < c.valid) {
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) {
+                            const V4 p4 = *(const V4*)(sP + x * PK + feat(a2) + 4 * g);
+                            f32x4 out;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) out[r] = (dpk[a2][t][r] - (float)p4[r] * dotp) * rp;
+                            *(V4*)((T*)p.dp + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(out);
+                        }
                     }
                 }
             }
@@ -1644,12 +1670,12 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
             dstate.grid = 0;
         }
     }
-    const bool l2 = KT == 1 && !COMBA && p.q_raw;           // (the entry has checked H == HV)
+    const bool l2 = KT == 1 && p.q_raw;                     // (the entry has checked H == HV)
     K wy;
-    if constexpr (KT == 1) wy = {l2 ? (const void*)gdn_bwd_wy2_kernel<T, true> : (const void*)gdn_bwd_wy2_kernel<T, false, COMBA>, bwd_wy2_smem<COMBA>(), "gdn_bwd_wy2_kernel", units < 512u ? units : 512u};
+    if constexpr (KT == 1) wy = {l2 ? (const void*)gdn_bwd_wy2_kernel<T, true, COMBA> : (const void*)gdn_bwd_wy2_kernel<T, false, COMBA>, bwd_wy2_smem<COMBA>(), "gdn_bwd_wy2_kernel", units < 512u ? units : 512u};
     else wy = {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u};
     const K ks[5] = {
-        {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, false, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
+        {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, COMBA && KT == 1, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
         dstate,
         {l2 ? (const void*)gdn_bwd_dqkw_kernel<T, 1, true> : (const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
@@ -1720,15 +1746,21 @@ static int chunk_bwd_entry(
     size_t need = bwd_ws_layout(num_chunks * HV, K, (char*)workspace, &p.ws);
     const size_t rows_bytes = ws_align((size_t)(B * T * H) * BD * 2), factors_bytes = ws_align((size_t)(B * T * H) * 4);
     const size_t l2_at = need;
-    if (l2) need += 2 * rows_bytes + 2 * factors_bytes;
+    if (l2) need += (comba ? 3 : 2) * (rows_bytes + factors_bytes);
     GDN_CHECK_ARG(workspace && workspace_bytes >= need, GDN_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who,
                   need, workspace_bytes);
-    p.q_raw = p.k_raw = nullptr; p.q_rstd = p.k_rstd = nullptr;
+    p.q_raw = p.k_raw = p.pk_raw = nullptr; p.q_rstd = p.k_rstd = p.p_rstd = nullptr;
     if (l2) {
         char* at = (char*)workspace + l2_at;
         p.q_raw = q; p.k_raw = k;
         q = at; k = at + rows_bytes;
         p.q_rstd = (const float*)(at + 2 * rows_bytes); p.k_rstd = (const float*)(at + 2 * rows_bytes + factors_bytes);
+        if (comba) {
+            at += 2 * (rows_bytes + factors_bytes);
+            p.pk_raw = pk;
+            pk = at;
+            p.p_rstd = (const float*)(at + rows_bytes);
+        }
     }
     p.q = q; p.k = k; p.v = v; p.g = g; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
     p.dq = dq; p.dk = dk; p.dv = dv; p.dg = dg; p.dbeta = dbeta; p.dh0 = dh0; p.pk = pk; p.dp = dp; p.dgk = nullptr;
@@ -1789,6 +1821,26 @@ extern "C" int gdn_chunk_comba_bwd(
                            scale, qkv_dtype, gb_dtype, flags, stream);
 }
 
+extern "C" size_t gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t tokens) {
+    if (num_chunks < 0 || HV < 1 || tokens < 0) return 0;
+    return gdn::bwd_ws_layout(num_chunks * HV, gdn::BD, nullptr, nullptr) + 3 * gdn::ws_align((size_t)(tokens * HV) * gdn::BD * 2) +
+           3 * gdn::ws_align((size_t)(tokens * HV) * 4);
+}
+
+extern "C" int gdn_chunk_comba_bwd_qk_l2norm(
+    const void* q, const void* k, const void* p, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream) {
+    return chunk_bwd_entry("gdn_chunk_comba_bwd_qk_l2norm", true, true, q, k, p, v, g, beta, h0, dout, dht, dq, dk, dp, dv, dg, dbeta, dh0,
+                           cu_seqlens, chunk_table, chunk_offsets, workspace, workspace_bytes, B, T, H, HV, K, V, N, num_chunks,
+                           scale, qkv_dtype, gb_dtype, flags, stream);
+}
+
 extern "C" size_t gdn_chunk_kda_bwd_workspace_bytes(int64_t num_chunks, int64_t HV) {
     if (num_chunks < 0 || HV < 1) return 0;
     return gdn::kda_bwd_ws_layout(num_chunks * HV, nullptr, nullptr);
@@ -1838,7 +1890,7 @@ extern "C" int gdn_chunk_kda_bwd(
                   need, workspace_bytes);
     p.q = q; p.k = k; p.v = v; p.g = nullptr; p.beta = beta; p.h0 = h0; p.dout = dout; p.dht = dht;
     p.dq = dq; p.dk = dk; p.dv = dv; p.dg = nullptr; p.dbeta = dbeta; p.dh0 = dh0; p.pk = nullptr; p.dp = nullptr; p.dgk = dg;
-    p.q_raw = p.k_raw = nullptr; p.q_rstd = p.k_rstd = nullptr;
+    p.q_raw = p.k_raw = p.pk_raw = nullptr; p.q_rstd = p.k_rstd = p.p_rstd = nullptr;
     p.cu_seqlens = cu_seqlens; p.chunk_table = chunk_table; p.chunk_offsets = chunk_offsets;
     p.T = T; p.H = (int)H; p.HV = (int)HV; p.N = N; p.NT = (T + CH - 1) / CH;
     p.scale = scale; p.gb_dtype = gb_dtype; p.flags = flags;

@@ -114,6 +114,8 @@ SIGNATURES['gdn_chunk_comba_bwd'] = (c_int, [
     c_void_p, c_size_t,                                # workspace workspace_bytes
     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,   # B T H HV K V N num_chunks
     c_float, c_int, c_int, c_uint32, c_void_p])
+SIGNATURES['gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes'] = (c_size_t, [c_int64, c_int64, c_int64])
+SIGNATURES['gdn_chunk_comba_bwd_qk_l2norm'] = SIGNATURES['gdn_chunk_comba_bwd']      # (q, k, p before their l2 normalisation)
 SIGNATURES['gdn_chunk_kda_bwd_workspace_bytes'] = (c_size_t, [c_int64, c_int64])
 SIGNATURES['gdn_chunk_kda_bwd'] = SIGNATURES['gdn_chunk_bwd']        # (g: [B,T,HV,K] fp32, dg likewise)
 SIGNATURES['gdn_l2norm_fwd'] = (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p])

@@ -111,11 +111,14 @@ def chunk_comba_fwd(q, k, v, p, g, beta, scale, initial_state, output_final_stat
 
 
 def chunk_comba_bwd(q, k, v, p, g, beta, scale, initial_state, do, dht, cu_seqlens=None, cu_seqlens_cpu=None,
-                    q_rstd=None, k_rstd=None, p_rstd=None):
+                    q_rstd=None, k_rstd=None, p_rstd=None, qk_l2norm=False):
     """q, k, p ``[B,T,H,K]``, v, do ``[B,T,HV,V]``, g (log decay), beta ``[B,T,HV]`` as the recurrence uses them.
     Returns ``(dq, dk, dv, dp, dbeta, dg, dh0)``: dq, dk, dv, dp in q's dtype, dbeta, dg fp32, dh0 fp32 (None without
     ``initial_state``).  With the ``*_rstd`` factors (what ``l2norm_fwd`` returns next to the normalised rows passed as
-    q, k, p) dq, dk, dp are the gradients of the rows before normalisation (fla/ops/comba/chunk.py:277-280)."""
+    q, k, p) dq, dk, dp are the gradients of the rows before normalisation (fla/ops/comba/chunk.py:277-280).  With
+    ``qk_l2norm`` q, k, p are the rows BEFORE their l2 normalisation and dq, dk, dp the gradients of those: one C call
+    (``gdn_chunk_comba_bwd_qk_l2norm``) where every value head has a q/k head of its own, ``l2norm_fwd`` and the route above
+    otherwise."""
     dev = require_gpu(q, k, v, p, g, beta, do)
     check_operand_shapes(q, k, v, g=g, beta=beta)
     if do.shape != v.shape:
@@ -126,6 +129,10 @@ def chunk_comba_bwd(q, k, v, p, g, beta, scale, initial_state, do, dht, cu_seqle
         raise NotImplementedError(f'the chunked comba kernels cover key head dims up to {_DIM} (got K={K})')
     N = B if cu_seqlens is None else len(cu_seqlens) - 1
     nb = (V + _DIM - 1) // _DIM
+    inside = qk_l2norm and H == HV and nb == 1
+    if qk_l2norm and not inside:
+        (q, q_rstd), (k, k_rstd), (p, p_rstd) = l2norm_fwd(q), l2norm_fwd(k), l2norm_fwd(p)
+        q, k, p = (x[..., :K] for x in (q, k, p))          # (l2norm_fwd pads rows to a multiple of 8)
     if nb > 1:
         # value columns are independent: a head with V > 128 is nb heads of 128 columns that share q, k, p, g, beta
         def split(s):       # [N, HV, K, V] -> [N, HV*nb, K, 128]
@@ -184,9 +191,9 @@ def chunk_comba_bwd(q, k, v, p, g, beta, scale, initial_state, do, dht, cu_seqle
     db = alloc(B, T, HV, dtype=torch.float32, device=dev)
     dh0 = torch.empty(N, HV, _DIM, _DIM, dtype=torch.float32, device=dev) if initial_state is not None else None
     lib = _lib.load()
-    ws_bytes = lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, _DIM)
+    ws_bytes = lib.gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(num_chunks, HV, B * T) if inside else lib.gdn_chunk_bwd_workspace_bytes(num_chunks, HV, _DIM)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    _lib.check(lib.gdn_chunk_comba_bwd(
+    _lib.check((lib.gdn_chunk_comba_bwd_qk_l2norm if inside else lib.gdn_chunk_comba_bwd)(
         ptr(qw), ptr(kw), ptr(pw), ptr(vw), ptr(gw), ptr(bw), ptr(h0), ptr(dow), ptr(dhtw),
         ptr(dq), ptr(dk), ptr(dp), ptr(dv), ptr(dg), ptr(db), ptr(dh0),
         ptr(cu_seqlens), ptr(chunk_table), ptr(chunk_offsets), ptr(workspace), ws_bytes,
@@ -217,13 +224,8 @@ class ChunkCombaFunction(torch.autograd.Function):
     def backward(ctx, do, dht):
         q, k, v, p, g, beta, h0, cu_seqlens, cu_seqlens_cpu = ctx.saved_tensors
         scale, l2 = ctx.opts
-        q_rstd = k_rstd = p_rstd = None
-        qn, kn, pn = q, k, p
-        if l2:
-            (qn, q_rstd), (kn, k_rstd), (pn, p_rstd) = l2norm_fwd(q), l2norm_fwd(k), l2norm_fwd(p)
-            qn, kn, pn = (x[..., :q.shape[-1]] for x in (qn, kn, pn))     # (l2norm_fwd pads rows to a multiple of 8)
-        dq, dk, dv, dp, db, dg, dh0 = chunk_comba_bwd(qn, kn, v, pn, g, beta, scale, h0, do.contiguous(), dht, cu_seqlens,
-                                                      cu_seqlens_cpu, q_rstd, k_rstd, p_rstd)
+        dq, dk, dv, dp, db, dg, dh0 = chunk_comba_bwd(q, k, v, p, g, beta, scale, h0, do.contiguous(), dht, cu_seqlens,
+                                                      cu_seqlens_cpu, qk_l2norm=l2)
         K = q.shape[-1]
         return (dq[..., :K].to(q.dtype), dk[..., :K].to(k.dtype), dv.to(v.dtype), dp[..., :K].to(p.dtype), dg.to(g.dtype),
                 db.to(beta.dtype), None, dh0, None, None, None, None)

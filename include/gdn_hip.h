@@ -318,6 +318,25 @@ int gdn_chunk_comba_bwd(
     float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
 
 /*
+ * gdn_chunk_comba_bwd with the l2 normalisation of q, k and p taken inside, as gdn_chunk_bwd_qk_l2norm does it for q and k:
+ * q, k, p are the rows as the caller has them, dq, dk, dp the gradients of those rows.  Replaces the three l2norm_fwd and
+ * three l2norm_bwd launches around chunk_comba_bwd in ChunkCombaFunction.backward (fla/ops/comba/chunk.py:277-280).
+ * Arguments as for gdn_chunk_comba_bwd, except:
+ *   workspace: at least gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(num_chunks, HV, B * T) bytes
+ *   H == HV only (GDN_ERR_UNSUPPORTED otherwise).
+ */
+size_t gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(int64_t num_chunks, int64_t HV, int64_t tokens);
+int gdn_chunk_comba_bwd_qk_l2norm(
+    const void* q, const void* k, const void* p, const void* v, const void* g, const void* beta,
+    const float* h0, const void* dout, const float* dht,
+    void* dq, void* dk, void* dp, void* dv, float* dg, float* dbeta, float* dh0,
+    const void* cu_seqlens, const void* chunk_table, const void* chunk_offsets,
+    void* workspace, size_t workspace_bytes,
+    int64_t B, int64_t T, int64_t H, int64_t HV, int64_t K, int64_t V,
+    int64_t N, int64_t num_chunks,
+    float scale, int qkv_dtype, int gb_dtype, uint32_t flags, void* stream);
+
+/*
  * Backward pass of the chunked KDA operator.  Replaces chunk_kda_bwd (fla/ops/kda/chunk_bwd.py, called from
  * ChunkKDAFunction.backward, fla/ops/kda/chunk.py:124-175): the forward's intermediates are computed again (the
  * chunk-parallel kernel of gdn_chunk_kda_fwd, then the state scan), then the reverse scan, dq / dk / dw and the way back

@@ -389,3 +389,47 @@ def test_chunk_comba_backward_wide_values_and_outside_tokens():
         got[n] = x[:, sl]
     _compare_grads(ref, got, GRAD_TOL)
 
+
+
+@pytest.mark.parametrize('B,T,H,K,cu', [(2, 200, 3, 128, None), (1, 333, 2, 100, [0, 1, 130, 333])])
+def test_chunk_comba_backward_l2norm_inside_the_kernels(B, T, H, K, cu):
+    """One value head per q/k head: the l2 normalisation of q, k and p, forward and back, is taken inside the backward's
+    kernels (C entry gdn_chunk_comba_bwd_qk_l2norm): against the separate route (gdn_l2norm_fwd, gdn_chunk_comba_bwd, then
+    gdn_l2norm_bwd on its rounded output) and against the oracle's gradients of the rows before normalisation."""
+    from fla_hip.ops.comba import chunk as M
+    gen = torch.Generator().manual_seed(6)
+    N = B if cu is None else len(cu) - 1
+    q, k, p = (torch.randn(B, T, H, K, generator=gen).bfloat16() for _ in range(3))
+    v, do = (torch.randn(B, T, H, 128, generator=gen).bfloat16() for _ in range(2))
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen)) / 2
+    beta = torch.rand(B, T, H, generator=gen)
+    h0, dht = 0.5 * torch.randn(N, H, K, 128, generator=gen), torch.randn(N, H, K, 128, generator=gen)
+    ref = O.comba_grads(q, k, v, p, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, use_qk_l2norm_in_kernel=True, dtype=torch.float32)
+    cu_t = None if cu is None else torch.tensor(cu, device='cuda')
+    rest = (g.cuda(), beta.cuda(), K ** -0.5, h0.cuda(), do.cuda(), dht.cuda(), cu_t, None)
+    inside = M.chunk_comba_bwd(q.cuda(), k.cuda(), v.cuda(), p.cuda(), *rest, qk_l2norm=True)
+    (qn, q_rstd), (kn, k_rstd), (pn, p_rstd) = (M.l2norm_fwd(x.cuda()) for x in (q, k, p))
+    apart = M.chunk_comba_bwd(qn[..., :K], kn[..., :K], v.cuda(), pn[..., :K], *rest, q_rstd, k_rstd, p_rstd)
+    for i, name in ((0, 'dq'), (1, 'dk'), (3, 'dp')):
+        a, b = inside[i], apart[i]
+        assert a.shape == b.shape == (B, T, H, K)
+        r = O.get_err_ratio(b.float().cpu(), a.float().cpu())
+        assert r < 5e-3, f'{name}: inside the kernels against the separate route {r:.3e}'
+        e = O.get_err_ratio(ref[name], a.float().cpu())
+        assert e <= GRAD_TOL[name], f'{name}: rel-rmse {e:.3e} against the oracle'
+    for i, name in ((2, 'dv'), (4, 'dbeta'), (5, 'dg'), (6, 'dh0')):      # (the normalised rows may differ in their last bit)
+        r = O.get_err_ratio(apart[i].float().cpu(), inside[i].float().cpu())
+        assert r < 2e-3, f'{name}: {r:.3e}'
+    from fla_hip import _lib
+    lib = _lib.load()
+    assert lib.gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(1, 2, 64) > lib.gdn_chunk_bwd_qk_l2norm_workspace_bytes(1, 2, 128, 64)
+    x = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device='cuda')
+    x1 = torch.zeros(1, 64, 1, 128, dtype=torch.bfloat16, device='cuda')
+    f = torch.zeros(1, 64, 2, device='cuda')
+    ws = torch.zeros(lib.gdn_chunk_comba_bwd_qk_l2norm_workspace_bytes(1, 2, 64), dtype=torch.uint8, device='cuda')
+    tail = [x.data_ptr(), f.data_ptr(), f.data_ptr(), None, x.data_ptr(), None] + [x.data_ptr()] * 4 + [f.data_ptr()] * 2 + [None]
+    dims = lambda h: (None, None, None, ws.data_ptr(), ws.numel(), 1, 64, h, 2, 128, 128, 1, 1, 1.0, _lib.DTYPE_BF16, _lib.DTYPE_F32, 0, None)
+    rc = lib.gdn_chunk_comba_bwd_qk_l2norm(x1.data_ptr(), x1.data_ptr(), x1.data_ptr(), *tail, *dims(1))
+    assert rc == _lib.GDN_ERR_UNSUPPORTED and 'H == HV' in _lib.last_error()
+    assert lib.gdn_chunk_comba_bwd_qk_l2norm(x.data_ptr(), x.data_ptr(), x.data_ptr(), *tail, *dims(2)) == _lib.GDN_OK
+    torch.cuda.synchronize()
