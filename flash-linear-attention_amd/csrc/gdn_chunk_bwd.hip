@@ -681,9 +681,10 @@ __global__ __launch_bounds__(64 * scan_waves<VBT>()) void gdn_bwd_dstate_kernel(
 }
 
 // Both scans in one workgroup of eight waves: waves 0-3 walk the chunks forwards (S, v_new), waves 4-7 backwards (dS, dv_new).
-// Neither needs anything from the other, both take three barriers per chunk, and a step of either leaves most of a CU idle
-// (one wave per SIMD waiting for its own LDS reads and matrix instructions): side by side, two per SIMD, they take about the
-// time of the longer one.  Used where both sets of LDS tiles fit a CU (32 value columns per workgroup, one block of key features).
+// Neither needs anything from the other and both take three barriers per chunk.  What a CU can move per step bounds both, so
+// side by side they take little less than one after the other: this form serves time segments, whose workgroups already fill
+// every CU (32 value columns per workgroup, one block of key features: both sets of LDS tiles fit a CU); whole sequences take
+// gdn_bwd_scans_apart_kernel below.
 template <int VBT, int KT> constexpr size_t bwd_scans_smem() { return bwd_state_smem<VBT, KT>() + bwd_dstate_smem<VBT, KT>(); }
 
 template <typename T, int VBT, int KT, bool KDA = false>
@@ -695,8 +696,8 @@ __global__ __launch_bounds__(512) void gdn_bwd_scans_kernel(BwdParams p) {
 }
 
 // Both scans in one launch, in workgroups of their own: the first `nstate` workgroups walk forwards, the others backwards.
-// For calls whose two scans together leave CUs without a workgroup (few heads, long sequences) and whose tiles do not fit a
-// CU side by side (two blocks of key features): the launch then takes the time of the longer scan instead of their sum.
+// For calls whose two scans together need no more workgroups than there are CUs: the launch then takes the time of the
+// longer scan instead of their sum.
 template <int VBT, int KT> constexpr size_t bwd_scans_apart_smem() {
     return bwd_state_smem<VBT, KT>() > bwd_dstate_smem<VBT, KT>() ? bwd_state_smem<VBT, KT>() : bwd_dstate_smem<VBT, KT>();
 }
