@@ -136,8 +136,10 @@ def _compare(ref, got, tol=TOL, names=None):
     (2, 512, 2, 8, 64, 1, 0.1, 0, True, torch.float16),
     (2, 200, 2, 4, 128, None, 4.0, 0, False, torch.bfloat16),
     (1, 130, 2, 2, 128, None, 4.0, 0, True, torch.bfloat16),
-    (3, 100, 12, 24, 128, None, 4.0, 0, True, torch.bfloat16),       # 72 runs: the scans take 64 value columns per workgroup
-    (2, 70, 80, 80, 128, None, 4.0, 0, False, torch.bfloat16),       # 160 runs: all 128
+    (3, 100, 12, 24, 128, None, 4.0, 0, True, torch.bfloat16),       # 72 runs: the two scans apart, 128 value columns per workgroup
+    (2, 70, 80, 80, 128, None, 4.0, 0, False, torch.bfloat16),       # 160 runs: one scan after the other, 128 columns
+    (2, 130, 20, 20, 128, None, 4.0, 0, True, torch.bfloat16),       # 40 runs: apart at 64 columns; the l2 norm inside the kernels
+    (1, 100, 72, 72, 100, None, 4.0, 0, True, torch.float16),        # 72 runs apart at 128 columns, the l2 norm inside, K padded
 ])
 def test_chunk_backward(B, T, H, HV, D, scale, gate_div, mask_p, l2, dtype):
     gen = torch.Generator().manual_seed(42)
