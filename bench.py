@@ -9,7 +9,7 @@ chunk_gated_delta_rule on inputs already resident in HBM.  The same line carries
 "other_workloads" and in short form (ms per call, fraction of the bounding roofline), the reference's published
 shapes (forward, and forward + backward through autograd: the `*_fwd_bwd` rows), the sibling operators, the layer's two
 memory-bound steps either side of the operator (causal convolution, gated norm), the default workload again with exact
-start states forced and with gates that hardly decay, and last the other BASELINE configurations (packed prefill, B=4
+start states forced and with gates that hardly decay, and last the benchmark's other configurations (packed prefill, B=4
 prefill, the decode step at B=256: us/step and state GB/s); and:
   roofline      dominant stage (the launches of one C entry point), algorithmic FLOPs (or bytes)
                 per call / its mean duration measured with HIP events on the launch stream
@@ -681,7 +681,7 @@ def main():
         if key in res:
             line[key] = res[key]
     if not args.no_extra:
-        # The other rows are kept short (the whole line stays well under 8 KB) and the BASELINE configurations come last.
+        # The other rows are kept short (the whole line stays well under 8 KB) and the benchmark's other configurations come last.
         # Keys: ms = wall time per call, frac = fraction of the roofline that bounds the row (prefill rows: the whole
         # operator's algorithmic FLOPs against the bf16 matrix-core peak; streaming rows: algorithmic bytes against 8 TB/s),
         # frac_stage / us = the same for the dominant stage alone and the durations of the two stages (HIP events).
@@ -721,7 +721,7 @@ def main():
                     e['cpu_baseline'] = {k2: r['cpu_baseline'][k2] for k2 in ('value', 'unit', 'cores', 'kind')}
             extra[name] = e
             torch.cuda.empty_cache()
-        # BASELINE configs[1], [3], [4] last
+        # the benchmark's packed prefill, B=4 prefill and decode configurations last
         for name in ('varlen', 'prefill_b4', 'decode'):
             if name in extra:
                 extra[name] = extra.pop(name)
