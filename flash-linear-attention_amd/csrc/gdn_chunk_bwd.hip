@@ -187,8 +187,9 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
     TileRegs<BD> rV;
     uint32_t rG = 0, rB = 0;                                     // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
-        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv, hq = at.hq;
+        const ChunkAt c = at.c;
         fetch_tile<KD>(rK, (const T*)(L2 ? p.k_raw : p.k) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         fetch_tile<KD>(rQ, (const T*)(L2 ? p.q_raw : p.q) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         if constexpr (COMBA) fetch_tile<KD>(rP, (const T*)(L2 ? p.pk_raw : p.pk) + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
@@ -208,8 +209,9 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         if constexpr (L2) {
             static_assert(!L2 || KT == 1, "one block of key features");
-            const int hv = (int)(u % p.HV);                      // (== the q/k head)
-            const ChunkAt c = chunk_at(p, u / p.HV);
+            const UnitAt at = unit_at(p, u);
+            const int hv = at.hv;                      // (== the q/k head)
+            const ChunkAt c = at.c;
             l2norm_tile_rows<T>(rK, (T*)p.k + (c.tok0 * p.H + hv) * KD, (float*)p.k_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
             l2norm_tile_rows<T>(rQ, (T*)p.q + (c.tok0 * p.H + hv) * KD, (float*)p.q_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
             if constexpr (COMBA) l2norm_tile_rows<T>(rP, (T*)p.pk + (c.tok0 * p.H + hv) * KD, (float*)p.p_rstd + c.tok0 * p.H + hv, p.H, c.valid, tid);
@@ -736,8 +738,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
     V8 rS[2][4], rdS[2][4];
     float rGam = 0.f, rRq = 0.f;
     auto fetch = [&](int64_t u) {
-        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv, hq = at.hq;
+        const ChunkAt c = at.c;
         fetch_tile<BD>(rDO, (const T*)p.dout + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         fetch_tile<BD>(rVn, (const T*)p.ws.Vn + u * 64 * BD, BD, 64, tid);
         fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
@@ -762,10 +765,11 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
-        const int hv = (int)(u % p.HV);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv;
+        const ChunkAt c = at.c;
         if constexpr (KT > 1) {                                 // (no registers to spare for fetching the wide tiles ahead)
-            const int hq = hv / (p.HV / p.H);
+            const int hq = at.hq;
             fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
             fetch_tile<KD>(rQ, (const T*)p.q + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
         }
@@ -974,8 +978,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     float rGam = 0.f, rDg = 0.f;
     uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch = [&](int64_t u) {
-        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv, hq = at.hq;
+        const ChunkAt c = at.c;
         fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
@@ -997,8 +1002,9 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t
     };
     fetch(blockIdx.x);
     for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
-        const int hv = (int)(u % p.HV);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv;
+        const ChunkAt c = at.c;
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<BD>(sV, P128, rV, tid);
         put_tile<CH>(sA, P64, rA, tid);
@@ -1252,8 +1258,9 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
     float rGam = 0.f, rDg = 0.f, rRk = 0.f, rGam0 = 0.f, rRp = 0.f;
     uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
     auto fetch_first = [&](int64_t u, int tid) {
-        const int hv = (int)(u % p.HV);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv;
+        const ChunkAt c = at.c;
         fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
         fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
         fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
@@ -1274,8 +1281,9 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
         asm volatile("" : "+v"(tid_opaque));
         const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         auto feat = [&](int a) { return 16 * (2 * w + a); };    // first key feature of this wave's tile a
-        const int hv = (int)(u % p.HV), hq = hv / (p.HV / p.H);
-        const ChunkAt c = chunk_at(p, u / p.HV);
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv, hq = at.hq;
+        const ChunkAt c = at.c;
         put_tile<BD>(sDvn, P128, rDvn, tid);
         put_tile<BD>(sV, P128, rV, tid);
         put_tile<CH>(sA, P64, rA, tid);

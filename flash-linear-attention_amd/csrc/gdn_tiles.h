@@ -28,8 +28,17 @@ __device__ __forceinline__ ChunkAt chunk_at(const P& p, int64_t ci) {
         const int64_t t0 = bos + it * CH;
         return ChunkAt{t0, (int)min((int64_t)CH, eos - t0)};
     }
-    const int64_t b = ci / p.NT, it = ci % p.NT;
-    return ChunkAt{b * p.T + it * CH, (int)min((int64_t)CH, p.T - it * CH)};
+    // (32-bit: the entries refuse calls with 2^31 chunks or more, and a 64-bit division costs some hundred instructions)
+    const uint32_t b = (uint32_t)ci / (uint32_t)p.NT, it = (uint32_t)ci - b * (uint32_t)p.NT;
+    return ChunkAt{(int64_t)b * p.T + (int64_t)it * CH, (int)min((int64_t)CH, p.T - (int64_t)it * CH)};
+}
+// Unit u = chunk * HV + v-head of the kernels that walk over the units: its v-head, q/k head and chunk.  (32-bit arithmetic,
+// as above: these kernels are bound by the rate at which one or two waves per SIMD issue instructions.)
+struct UnitAt { int hv, hq; ChunkAt c; };
+template <typename P>
+__device__ __forceinline__ UnitAt unit_at(const P& p, int64_t u) {
+    const uint32_t HV = (uint32_t)p.HV, ch = (uint32_t)u / HV, hv = (uint32_t)u - ch * HV, G = HV / (uint32_t)p.H;
+    return UnitAt{(int)hv, (int)(G == 1 ? hv : hv / G), chunk_at(p, ch)};
 }
 struct SeqAt { int64_t bos, len, cbase, nc; };
 template <typename P>
