@@ -426,11 +426,10 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (NA * w + a2) + c16;
-                const V4 s4 = pack4<T>(S[a2][b]);
-                *(V4*)(sS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
-                if (keep) *(V4*)(Hu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
+                *(V4*)(sS + kk * PV + vq0 + 16 * b + 4 * g) = pack4<T>(S[a2][b]);
             }
         lds_barrier();
+        if (keep) copy_rows_out<KD, VBT, NTH>(Hu + vcol0, BD, sS, PV, tid);     // (whole rows of the tile: 16 bytes a lane)
         if (ic + AHEAD < c_end) fetch(R, ic + AHEAD);
         const float glast = sGam[63];
         {
@@ -593,11 +592,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 const int kk = 16 * (NA * w + a2) + c16;
-                const V4 s4 = pack4<T>(dS[a2][b]);
-                *(V4*)(sDS + kk * PV + vq0 + 16 * b + 4 * g) = s4;
-                if (keep) *(V4*)(dHu + kk * BD + vcol0 + vq0 + 16 * b + 4 * g) = s4;
+                *(V4*)(sDS + kk * PV + vq0 + 16 * b + 4 * g) = pack4<T>(dS[a2][b]);
             }
         lds_barrier();
+        if (keep) copy_rows_out<KD, VBT, NTH>(dHu + vcol0, BD, sDS, PV, tid);
         if (ic >= c_lo + AHEAD) fetch(R, ic - AHEAD);
         const float glast = sGam[63];
         {
