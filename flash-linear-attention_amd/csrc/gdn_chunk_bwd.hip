@@ -351,7 +351,12 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
 // 16(NA w + a2) + c16 and value columns 16b + 4g .. +3.  The next chunk's tiles are fetched into registers while the
 // current chunk is computed, and the barriers wait for LDS traffic only, so those loads stay in flight across them.
 // ---------------------------------------------------------------------------------------------
-template <int VBT, int KT> constexpr size_t bwd_state_smem() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 64 * (VBT + 8)) * 2 + 64 * 4; }
+// (the forward scan keeps v_new twice where a CU's LDS has the room: as the operand of the state update, with the decay to the end
+// of the chunk on it, and as it is stored, so that it can leave as whole rows)
+template <int VBT, int KT> constexpr bool state_out_tile() { return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + 2 * 64 * (VBT + 8)) * 2 + 64 * 4 <= 160 * 1024; }
+template <int VBT, int KT> constexpr size_t bwd_state_smem() {
+    return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + (state_out_tile<VBT, KT>() ? 2 : 1) * 64 * (VBT + 8)) * 2 + 64 * 4;
+}
 template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 2 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
 
 // KDA: the rows of k arrive with their decay to the end of the chunk on them (KG), and the state decays per key feature (EGL).
@@ -362,7 +367,9 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
     constexpr int PV = VBT + 8, VBQ = VBT / (NW / 4), NB = VBQ / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT, NTH = 64 * NW;
     T* sW = (T*)smem; T* sK = sW + 64 * PK; T* sS = sK + 64 * PK; T* sVn = sS + KD * PV;
-    float* sGam = (float*)(sVn + 64 * PV);
+    constexpr bool OUT_TILE = state_out_tile<VBT, KT>();
+    T* sOut = sVn + 64 * PV;                                     // v_new as it is stored (sVn: with the decay to the end of the chunk on it)
+    float* sGam = (float*)(sOut + (OUT_TILE ? 64 * PV : 0));
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
     // an L2 for the rows of k, q and w that all of them read.  With time segments (nwg workgroups each) a segment's come in a row.
@@ -436,7 +443,6 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
             // v_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int i = 16 * w + c16;
             const float dec = KDA ? 1.f : __expf(glast - sGam[i]);
-            T* Vu = (T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0;
             V8 wf[4 * KT];
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) wf[s] = frag_rows(sW, PK, 16 * w, 32 * s, lane);
@@ -449,13 +455,15 @@ __device__ __forceinline__ void bwd_state_body(const BwdParams& p, char* smem, c
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
                 const V4 vn4 = pack4<T>(vn);
-                if (keep) *(V4*)(Vu + vq0 + 16 * b + 4 * g) = vn4;
+                if constexpr (OUT_TILE) *(V4*)(sOut + i * PV + vq0 + 16 * b + 4 * g) = vn4;
+                else if (keep) *(V4*)((T*)p.ws.Vn + u * 64 * BD + i * BD + vcol0 + vq0 + 16 * b + 4 * g) = vn4;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) vn[r] = (float)vn4[r] * dec;
                 *(V4*)(sVn + i * PV + vq0 + 16 * b + 4 * g) = pack4<T>(vn);
             }
         }
         lds_barrier();
+        if constexpr (OUT_TILE) { if (keep) copy_rows_out<64, VBT, NTH>((T*)p.ws.Vn + u * 64 * BD + vcol0, BD, sOut, PV, tid); }
         {
             const float eg = __expf(glast);
             V8 kf[NA][2];
@@ -579,6 +587,9 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             }
         }
         put_tile<KD, NTH>(sQ, PK, rQ, tid);
+        // (the rows of w change their sign on the way in - one bit per element - so that dv_new can stay in LDS as it is stored)
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(rW.x) / sizeof(rW.x[0])); ++i) rW.x[i] ^= u32x4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
         put_tile<KD, NTH>(sW, PK, rW, tid);
         put_tile<CH, NTH>(sPT, P64, rPT, tid);
         put_tile<VBT, NTH>(sDO, PV, rDO, tid);
@@ -602,7 +613,6 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
             // dv_new^T tiles: value columns on the rows, this wave's 16 tokens on the columns
             const int j = 16 * w + c16;
             const float dec = KDA ? 1.f : __expf(glast - sGam[j]);
-            T* dVu = (T*)p.ws.dVn + u * 64 * BD + j * BD + vcol0;
             V8 kf[4 * KT], pf[2];
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) kf[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
@@ -619,11 +629,11 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
                 for (int s = 0; s < 4 * KT; ++s) a2v = Mma<T>::run(frag_cols(sDS, PV, 32 * s, vq0 + 16 * b, lane), kf[s], a2v);
                 f32x4 dvn = a1 + a2v * dec;
-                if (keep) *(V4*)(dVu + vq0 + 16 * b + 4 * g) = pack4<T>(dvn);
-                *(V4*)(sDvn + j * PV + vq0 + 16 * b + 4 * g) = pack4<T>(-dvn);
+                *(V4*)(sDvn + j * PV + vq0 + 16 * b + 4 * g) = pack4<T>(dvn);
             }
         }
         lds_barrier();
+        if (keep) copy_rows_out<64, VBT, NTH>((T*)p.ws.dVn + u * 64 * BD + vcol0, BD, sDvn, PV, tid);
         {
             const float eg = __expf(glast);
             V8 qf[NA][2], wf[NA][2];
