@@ -533,7 +533,9 @@ __global__ __launch_bounds__(256, 2) void gdn_comba_prepare_kernel(KdaParams p, 
 // lane (c16, g): key 16(2w+a2) + c16, value columns 16b + 4g .. +3); the next chunk's tiles are fetched into registers
 // while the current chunk is computed.
 // ---------------------------------------------------------------------------------------------
-template <int VBT> constexpr size_t kda_scan_smem() { return (3 * 64 * P128 + 64 * P64 + BD * (VBT + 8) + 64 * (VBT + 8)) * 2 + (BD + 64) * 4; }
+// (u comes in, and o leaves, as whole rows through LDS tiles of their own: the lanes that hold them as matrix-instruction operands
+// and results would move 8-byte pieces of 16 rows per instruction)
+template <int VBT> constexpr size_t kda_scan_smem() { return (3 * 64 * P128 + 64 * P64 + BD * (VBT + 8) + 3 * 64 * (VBT + 8)) * 2 + (BD + 64) * 4; }
 
 template <typename T, int VBT>
 __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
@@ -542,8 +544,8 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
     constexpr int PV = VBT + 8, NB = VBT / 16, NVS = BD / VBT;
     extern __shared__ __align__(16) char smem[];
     T* sW = (T*)smem; T* sKG = sW + 64 * P128; T* sQG = sKG + 64 * P128; T* sP = sQG + 64 * P128;
-    T* sS = sP + 64 * P64; T* sVn = sS + BD * PV;
-    float* sE = (float*)(sVn + 64 * PV);
+    T* sS = sP + 64 * P64; T* sVn = sS + BD * PV; T* sU = sVn + 64 * PV; T* sO = sU + 64 * PV;
+    float* sE = (float*)(sO + 64 * PV);
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
     const int64_t run = (int64_t)(blockIdx.x / (8 * NVS)) * 8 + blockIdx.x % 8;       // (slices of one head on one XCD)
     if (run >= p.N * p.HV) return;
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
         }
     TileRegs<BD> rW, rKG, rQG;
     TileRegs<CH> rP;
-    V4 rU[NB];
+    TileRegs<VBT> rU;
     float rE = 0.f;
     auto fetch = [&](int64_t ic) {
         const int64_t u = (sq.cbase + ic) * p.HV + hv;
@@ -571,8 +573,7 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
         fetch_tile<BD>(rQG, (const T*)p.ws.QG + u * 64 * BD, BD, 64, tid);
         fetch_tile<CH>(rP, (const T*)p.ws.Pm + u * 64 * 64, 64, 64, tid);
         if (tid < BD) rE = p.ws.EGL[u * BD + tid];
-#pragma unroll
-        for (int b = 0; b < NB; ++b) rU[b] = *(const V4*)((const T*)p.ws.Um + u * 64 * BD + (16 * w + c16) * BD + vcol0 + 16 * b + 4 * g);
+        fetch_tile<VBT>(rU, (const T*)p.ws.Um + u * 64 * BD + vcol0, BD, 64, tid);
     };
     if (sq.nc > 0) fetch(0);
     for (int64_t ic = 0; ic < sq.nc; ++ic) {
@@ -582,10 +583,8 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
         put_tile<BD>(sKG, P128, rKG, tid);
         put_tile<BD>(sQG, P128, rQG, tid);
         put_tile<CH>(sP, P64, rP, tid);
+        put_tile<VBT>(sU, PV, rU, tid);
         if (tid < BD) sE[tid] = rE;
-        V4 u4[NB];
-#pragma unroll
-        for (int b = 0; b < NB; ++b) u4[b] = rU[b];
 #pragma unroll
         for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
@@ -613,9 +612,10 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
                     acc = Mma<T>::run(fs, wf[s], acc);
                     oacc[b] = Mma<T>::run(fs, qf[s], oacc[b]);
                 }
+                const V4 u4 = *(const V4*)(sU + i * PV + 16 * b + 4 * g);
                 f32x4 vn;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[b][r] - acc[r];
+                for (int r = 0; r < 4; ++r) vn[r] = (float)u4[r] - acc[r];
                 *(V4*)(sVn + i * PV + 16 * b + 4 * g) = pack4<T>(vn);
             }
         }
@@ -645,10 +645,11 @@ __global__ __launch_bounds__(256) void gdn_kda_scan_kernel(KdaParams p) {
 #pragma unroll
                     for (int a2 = 0; a2 < 2; ++a2) S[a2][b] = Mma<T>::run(fv, kf[a2][s], S[a2][b]);
                 }
-                if (i < valid) *(V4*)((T*)p.o + ((tok0 + i) * p.HV + hv) * BD + vcol0 + 16 * b + 4 * g) = pack4<T>(oacc[b]);
+                *(V4*)(sO + i * PV + 16 * b + 4 * g) = pack4<T>(oacc[b]);
             }
         }
         lds_barrier();
+        copy_rows_out<64, VBT, 256>((T*)p.o + (tok0 * p.HV + hv) * BD + vcol0, (int64_t)p.HV * BD, sO, PV, tid, valid);
     }
     if (p.ht) {
 #pragma unroll

@@ -107,8 +107,9 @@ __device__ __forceinline__ void put_tile(T* s, int pitch, const TileRegs<NCOLS, 
 }
 // ROWS rows of NCOLS elements of an LDS tile out to global memory (row r at g + r * stride), 16 bytes a lane along the rows:
 // whole cache lines per group of lanes, where the lanes that hold a result as matrix-instruction output would write 8-byte pieces.
+// (`valid`: rows from there on are left alone)
 template <int ROWS, int NCOLS, int NTH, typename T>
-__device__ __forceinline__ void copy_rows_out(T* g, int64_t stride, const T* s, int pitch, int tid) {
+__device__ __forceinline__ void copy_rows_out(T* g, int64_t stride, const T* s, int pitch, int tid, int valid = ROWS) {
     constexpr int PPR = NCOLS / 8, TOTAL = ROWS * PPR, N = TOTAL / NTH;
     static_assert(TOTAL % NTH == 0, "whole rounds of the workgroup's threads");
     u32x4 x[N];
@@ -120,7 +121,7 @@ __device__ __forceinline__ void copy_rows_out(T* g, int64_t stride, const T* s, 
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const int idx = tid + NTH * i;
-        *(u32x4*)(g + (int64_t)(idx / PPR) * stride + (idx % PPR) * 8) = x[i];
+        if (idx / PPR < valid) *(u32x4*)(g + (int64_t)(idx / PPR) * stride + (idx % PPR) * 8) = x[i];
     }
 }
 // operand fragment whose contraction runs along a row: index r0 + c16, contraction c0 + 8g + e
