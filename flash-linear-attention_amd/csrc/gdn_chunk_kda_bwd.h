@@ -561,12 +561,13 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kda_kernel(BwdParams p, int
                     f32x4 acc = dk[a2][t];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
-                    if (x < c.valid) *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * BD + feat(a2) + 4 * g) = pack4<T>(acc);
+                    *(V4*)(sT + x * P128 + feat(a2) + 4 * g) = pack4<T>(acc);     // (the operand rows are done with: dk leaves from here as whole rows)
                     *(f32x4*)(sG + x * PG + feat(a2) + 4 * g) = dG[a2][t];
                 }
             }
         }
         lds_barrier();
+        copy_rows_out<64, BD, 256>((T*)p.dk + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, sT, P128, tid, c.valid);
         {
             // dg = reverse cumulative sum of dGk: a thread per key feature and half of the rows
             const int f = tid & 127, half = tid >> 7;
