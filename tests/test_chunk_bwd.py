@@ -469,6 +469,46 @@ def test_chunk_backward_l2norm_inside_the_kernels(B, T, H, K, cu):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize('B,T,H,K,V,cu,dtype,with_h0', [
+    (1, 400, 2, 128, 128, [0, 64, 64, 129, 400], torch.bfloat16, True),     # an empty sequence, chunk boundaries
+    (1, 1, 1, 128, 128, None, torch.bfloat16, True),                          # one token
+    (2, 65, 3, 40, 72, None, torch.float16, True),                            # small head dims, one token past a chunk
+    (1, 300, 2, 128, 128, [10, 100, 290], torch.bfloat16, False),             # tokens outside every sequence
+    (1, 130, 130, 64, 64, None, torch.bfloat16, True),                        # 130 runs: one scan after the other
+])
+def test_chunk_backward_l2norm_inside_edge_cases(B, T, H, K, V, cu, dtype, with_h0):
+    """The route with the l2 normalisation inside the backward's kernels (autograd, use_qk_l2norm_in_kernel, H == HV) on the edges."""
+    op = _op()
+    gen = torch.Generator().manual_seed(3)
+    N = B if cu is None else len(cu) - 1
+    q, k = (torch.randn(B, T, H, K, generator=gen).to(dtype) for _ in range(2))
+    v, do = (torch.randn(B, T, H, V, generator=gen).to(dtype) for _ in range(2))
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen)) / 2
+    beta = torch.rand(B, T, H, generator=gen)
+    h0 = 0.5 * torch.randn(N, H, K, V, generator=gen) if with_h0 else None
+    dht = torch.randn(N, H, K, V, generator=gen)
+    ref = O.gated_delta_rule_grads(q, k, v, g, beta, do, dht, initial_state=h0, cu_seqlens=cu, use_qk_l2norm_in_kernel=True, dtype=torch.float32)
+    dev = lambda x: None if x is None else x.cuda().requires_grad_(True)
+    leaves = dict(dq=dev(q), dk=dev(k), dv=dev(v), dg=dev(g), dbeta=dev(beta), dh0=dev(h0))
+    cu_t = None if cu is None else torch.tensor(cu, device='cuda')
+    o, ht = op(leaves['dq'], leaves['dk'], leaves['dv'], leaves['dg'], leaves['dbeta'], initial_state=leaves['dh0'], output_final_state=True,
+               cu_seqlens=cu_t, use_qk_l2norm_in_kernel=True)
+    ((o.float() * do.cuda().float()).sum() + (ht * dht.cuda()).sum()).backward()
+    for n, r in ref.items():
+        if r is None or leaves.get(n) is None:
+            continue
+        x = leaves[n].grad.float().cpu()
+        assert x.shape == r.shape and not torch.isnan(x).any(), n
+        if O.get_abs_err(r, x) <= 1e-5:             # (gradients that vanish; exactly zero in the oracle: one token on an empty state)
+            continue
+        e = O.get_err_ratio(r, x)
+        assert e <= TOL[n], f'{n}: rel-rmse {e:.3e} > {TOL[n]}'
+    if cu is not None and cu[0] > 0:                 # (tokens outside every sequence get zero gradients)
+        for n in ('dq', 'dk', 'dv'):
+            assert not leaves[n].grad[:, :cu[0]].any() and not leaves[n].grad[:, cu[-1]:].any(), n
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize('B,T,H,HV,gate_div,h0_std,forced', [
     (1, 2048, 2, 4, 2.0, 0.5, False),       # 16 workgroups of the scans: 4 segments of 8 chunks, automatic
     (2, 1100, 2, 2, 1.0, 0.5, True),        # ragged last chunk, segments of 4 chunks forced
