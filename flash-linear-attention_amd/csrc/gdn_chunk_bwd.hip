@@ -357,7 +357,12 @@ template <int VBT, int KT> constexpr bool state_out_tile() { return (2 * 64 * (B
 template <int VBT, int KT> constexpr size_t bwd_state_smem() {
     return (2 * 64 * (BD * KT + 8) + BD * KT * (VBT + 8) + (state_out_tile<VBT, KT>() ? 2 : 1) * 64 * (VBT + 8)) * 2 + 64 * 4;
 }
-template <int VBT, int KT> constexpr size_t bwd_dstate_smem() { return (3 * 64 * (BD * KT + 8) + 64 * P64 + 2 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4; }
+// (two blocks of key features at 64 columns: no room for the tile of P^T - a wave's two operand fragments of it come straight from
+// memory, a step ahead like the tiles)
+template <int VBT, int KT> constexpr bool dstate_pt_direct() { return KT == 2 && VBT == 64; }
+template <int VBT, int KT> constexpr size_t bwd_dstate_smem() {
+    return (3 * 64 * (BD * KT + 8) + (dstate_pt_direct<VBT, KT>() ? 0 : 64 * P64) + 2 * 64 * (VBT + 8) + BD * KT * (VBT + 8)) * 2 + 64 * 4;
+}
 
 // KDA: the rows of k arrive with their decay to the end of the chunk on them (KG), and the state decays per key feature (EGL).
 template <typename T, int VBT, int KT, int AHEAD, int NW, bool KDA = false>
@@ -517,8 +522,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     typedef typename Mma<T>::V4 V4;
     // NW waves in groups of four: a group takes VBQ of the workgroup's value columns (NB tiles per wave), every wave NA key tiles
     constexpr int PV = VBT + 8, VBQ = VBT / (NW / 4), NB = VBQ / 16, NVS = BD / VBT, KD = BD * KT, PK = KD + 8, NA = 2 * KT, NTH = 64 * NW;
+    constexpr bool PT_DIRECT = dstate_pt_direct<VBT, KT>();
+    static_assert(!PT_DIRECT || (!KDA && NW == 4), "fragments of P^T as the four waves of the gated delta rule read them");
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sW = sQ + 64 * PK; T* sPT = sW + 64 * PK;
-    T* sDO = sPT + 64 * P64; T* sDvn = sDO + 64 * PV; T* sDS = sDvn + 64 * PV;
+    T* sDO = sPT + (PT_DIRECT ? 0 : 64 * P64); T* sDvn = sDO + 64 * PV; T* sDS = sDvn + 64 * PV;
     float* sGam = (float*)(sDS + KD * PV);
     const int lane = tid & 63, w = (tid >> 6) & 3, vq0 = (tid >> 8) * VBQ, c16 = lane & 15, g = lane >> 4;
     // Workgroups go to the 8 XCDs in turn: the slices of one (sequence, head) take the same residue, so that they share
@@ -547,7 +554,7 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
     // (the rows of q meet the state's gradient as scale e^gam_i q_i: a thread scales its pieces of the tile on their way into LDS, with
     // the gam of their rows fetched beside them)
     constexpr int QN = 64 * (KD / 8) / NTH, QPPR = KD / 8, QRPI = NTH / QPPR;
-    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; float rGq[QN]; };
+    struct Ahead { TileRegs<KD, NTH> rK, rQ, rW; TileRegs<CH, NTH> rPT; V8 rPf[2]; TileRegs<VBT, NTH> rDO; float rGam; float rE[NA]; float rGq[QN]; };
     Ahead RA, RB;
     RA.rGam = RB.rGam = 0.f;
     auto fetch = [&](Ahead& R, int64_t ic) __attribute__((always_inline)) {
@@ -563,7 +570,11 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
         } else {
             fetch_tile<KD, NTH>(rK, (const T*)p.k + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
             fetch_tile<KD, NTH>(rQ, (const T*)p.q + (tok0 * p.H + hq) * KD, (int64_t)p.H * KD, valid, tid);
-            fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
+            if constexpr (PT_DIRECT) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * w) R.rPf[s] = *(const V8*)((const T*)p.ws.PT + u * 64 * 64 + (16 * w + c16) * 64 + 32 * s + 8 * g);
+            } else fetch_tile<CH, NTH>(rPT, (const T*)p.ws.PT + u * 64 * 64, 64, 64, tid);
             if (tid < 64) rGam = p.ws.Gam[u * 64 + tid];
 #pragma unroll
             for (int i = 0; i < QN; ++i) R.rGq[i] = p.ws.Gam[u * 64 + tid / QPPR + QRPI * i];
@@ -591,7 +602,9 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
         for (int i = 0; i < (int)(sizeof(rW.x) / sizeof(rW.x[0])); ++i) rW.x[i] ^= u32x4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
         put_tile<KD, NTH>(sW, PK, rW, tid);
-        put_tile<CH, NTH>(sPT, P64, rPT, tid);
+        if constexpr (!PT_DIRECT) put_tile<CH, NTH>(sPT, P64, rPT, tid);
+        V8 pf_now[2];
+        if constexpr (PT_DIRECT) { pf_now[0] = R.rPf[0]; pf_now[1] = R.rPf[1]; }
         put_tile<VBT, NTH>(sDO, PV, rDO, tid);
         if (tid < 64) sGam[tid] = rGam;
         float egk[NA];
@@ -617,7 +630,10 @@ __device__ __forceinline__ void bwd_dstate_body(const BwdParams& p, char* smem, 
 #pragma unroll
             for (int s = 0; s < 4 * KT; ++s) kf[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) pf[s] = KDA ? frag_cols(sPT, P64, 32 * s, 16 * w, lane) : frag_rows(sPT, P64, 16 * w, 32 * s, lane);
+            for (int s = 0; s < 2; ++s) {
+                if constexpr (PT_DIRECT) pf[s] = pf_now[s];
+                else pf[s] = KDA ? frag_cols(sPT, P64, 32 * s, 16 * w, lane) : frag_rows(sPT, P64, 16 * w, 32 * s, lane);
+            }
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 f32x4 a1 = ZERO4, a2v = ZERO4;
@@ -1623,10 +1639,11 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
     BwdParams p = p_in;
     // Value columns per workgroup of the scans where the two run one after the other or side by side in one workgroup: as few as
     // it takes to give every (sequence, head) run its own CU (their LDS tiles allow one workgroup per CU).  With two blocks of
-    // key features the reverse scan's tiles leave room for 32 columns only.
+    // key features the reverse scan's tiles leave room for 64 columns at most (taken where 64-column slices fill the chip: each
+    // slice reads the head's rows of k, q and w again, 96 KB a step).
     const int64_t runs1 = p.N * p.HV;
     const int vbt = runs1 <= 64 ? 32 : runs1 <= 128 ? 64 : 128;
-    const int vbt_d = KT == 1 ? vbt : 32;
+    const int vbt_d = KT == 1 ? vbt : runs1 >= 128 ? 64 : 32;
     const unsigned units = (unsigned)(num_chunks * p.HV);
     auto runs = [&](int v) { return (unsigned)((runs1 + 7) / 8 * 8 * (BD / v)); };
     struct K { const void* f; size_t smem; const char* name; unsigned grid; };
@@ -1635,10 +1652,8 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
     else if (vbt == 64) state = {(const void*)gdn_bwd_state_kernel<T, 64, KT>, bwd_state_smem<64, KT>(), "gdn_bwd_state_kernel", runs(64)};
     else state = {(const void*)gdn_bwd_state_kernel<T, 128, KT>, bwd_state_smem<128, KT>(), "gdn_bwd_state_kernel", runs(128)};
     if (vbt_d == 32) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 32, KT>, bwd_dstate_smem<32, KT>(), "gdn_bwd_dstate_kernel", runs(32)};
-    else if constexpr (KT == 1) {
-        if (vbt_d == 64) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, KT>, bwd_dstate_smem<64, KT>(), "gdn_bwd_dstate_kernel", runs(64)};
-        else dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, KT>, bwd_dstate_smem<128, KT>(), "gdn_bwd_dstate_kernel", runs(128)};
-    }
+    else if (vbt_d == 64) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 64, KT>, bwd_dstate_smem<64, KT>(), "gdn_bwd_dstate_kernel", runs(64)};
+    else if constexpr (KT == 1) dstate = {(const void*)gdn_bwd_dstate_kernel<T, 128, KT>, bwd_dstate_smem<128, KT>(), "gdn_bwd_dstate_kernel", runs(128)};
     unsigned threads[5] = {256, vbt == BD ? 512u : 256u, vbt_d == BD ? 512u : 256u, 256, 256};
     if constexpr (KT == 1) {
         // both scans side by side in one launch (the second entry then has nothing to launch): what time segments run in, where

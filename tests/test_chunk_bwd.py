@@ -226,6 +226,8 @@ def test_chunk_backward_packed_tokens_outside_every_sequence_get_zero_gradients(
     (1, 257, 2, 2, 256, 512, True, None),                  # the reference layer's default head shape (head_dim 256, expand_v 2)
     (1, 0, 2, 4, 160, 64, False, [0, 100, 101, 300]),
     (3, 100, 12, 24, 256, 128, True, None),                 # 72 runs: the forward scan takes 64 columns per workgroup
+    (2, 130, 16, 32, 256, 256, False, None),                # 128 runs: the reverse scan takes 64 columns, P^T straight from memory
+    (1, 70, 136, 136, 200, 64, True, None),                 # 136 runs, a ragged chunk
 ])
 def test_chunk_backward_wide_keys(B, T, H, HV, K, V, l2, cu):
     """Key head dims above 128 (two blocks of 128 key features in every backward kernel)."""
