@@ -978,282 +978,12 @@ __global__ __launch_bounds__(256, 1) void gdn_bwd_dqkw_kernel(BwdParams p, int64
 // ---------------------------------------------------------------------------------------------
 // back through w = X (e^gam k), u = X v, X = A diag(beta), A = (I + diag(beta) stril(k k^T o D))^-1
 // ---------------------------------------------------------------------------------------------
-// One workgroup per CU walks over the units, the next unit's tiles on their way into registers meanwhile.  (Two blocks of key
-// features; one block takes gdn_bwd_wy2_kernel below.)
-template <int KT> constexpr size_t bwd_wy_smem() { return (2 * 64 * P128 + 2 * 64 * (BD * KT + 8) + 3 * 64 * P64) * 2 + 640 * 4; }
-
-template <typename T, int KT>
-__global__ __launch_bounds__(256, 1) void gdn_bwd_wy_kernel(BwdParams p, int64_t units) {
-    typedef typename Mma<T>::V8 V8;
-    typedef typename Mma<T>::V4 V4;
-    constexpr int KD = BD * KT, PK = KD + 8, NA = 2 * KT;      // NA tiles of 16 key features per wave: two in every block of 128
-    extern __shared__ __align__(16) char smem[];
-    T* sDvn = (T*)smem; T* sV = sDvn + 64 * P128; T* sDW = sV + 64 * P128; T* sK = sDW + 64 * PK;
-    T* sA = sK + 64 * PK; T* sM1 = sA + 64 * P64; T* sM2 = sM1 + 64 * P64;
-    float* sGam = (float*)(sM2 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
-    // (sDg, sDb [4][64]: a row per wave, added up in a fixed order at the end - the same bits every run)
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    auto feat = [&](int a) { return BD * (a >> 1) + 16 * (2 * w + (a & 1)); };       // first key feature of this wave's tile a
-
-    TileRegs<BD> rDvn, rV;
-    TileRegs<KD> rDW, rK;
-    TileRegs<CH> rA;
-    V4 rDk[NA][4];                                               // what the previous kernel left in dk, at this lane's places
-    float rGam = 0.f, rDg = 0.f;
-    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
-    auto fetch = [&](int64_t u) {
-        const UnitAt at = unit_at(p, u);
-        const int hv = at.hv, hq = at.hq;
-        const ChunkAt c = at.c;
-        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
-        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
-        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
-        fetch_tile<KD>(rDW, (const T*)p.ws.dWm + u * 64 * KD, KD, 64, tid);
-        fetch_tile<KD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD, (int64_t)p.H * KD, c.valid, tid);
-        if (tid < 64) {
-            rGam = p.ws.Gam[u * 64 + tid];
-            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + hv, p.gb_dtype) : 0;
-            rDg = p.ws.Dgam[u * 64 + tid];
-        }
-#pragma unroll
-        for (int a2 = 0; a2 < NA; ++a2)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int x = 16 * t + c16;
-                rDk[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-                if (x < c.valid) rDk[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g);
-            }
-    };
-    fetch(blockIdx.x);
-    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
-        const UnitAt at = unit_at(p, u);
-        const int hv = at.hv;
-        const ChunkAt c = at.c;
-        put_tile<BD>(sDvn, P128, rDvn, tid);
-        put_tile<BD>(sV, P128, rV, tid);
-        put_tile<CH>(sA, P64, rA, tid);
-        put_tile<KD>(sDW, PK, rDW, tid);
-        put_tile<KD>(sK, PK, rK, tid);
-        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); }
-        sDg[tid] = tid < 64 ? rDg : 0.f;
-        sDb[tid] = 0.f;
-        V4 dk_old[NA][4];
-#pragma unroll
-        for (int a2 = 0; a2 < NA; ++a2)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) dk_old[a2][t] = rDk[a2][t];
-        lds_barrier();
-        if (u + gridDim.x < units) fetch(u + gridDim.x);
-
-        // Operand fragments are fetched from LDS once and kept: what does not change across an inner loop is loaded outside it.
-        // dX = du v^T + dw (e^gam k)^T (this wave's 16 rows i; lane: column j, rows 4g + r);  dA = stril(dX diag(beta));
-        // k k^T of the same rows and columns is formed along the way, for the last step but one
-        f32x4 kkT[4];
-        {
-            V8 fa[4], fw[4 * KT], fk[4 * KT];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
-#pragma unroll
-            for (int s = 0; s < 4 * KT; ++s) {
-                fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
-                fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
-            }
-#pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                f32x4 dXv = ZERO4, dXw = ZERO4;
-                kkT[tj] = ZERO4;
-                if (tj <= w) {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) dXv = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv);
-#pragma unroll
-                    for (int s = 0; s < 4 * KT; ++s) {
-                        const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
-                        dXw = Mma<T>::run(fw[s], bk, dXw);
-                        kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
-                    }
-                }
-                const int j = 16 * tj + c16;
-                const float ej = __expf(sGam[j]), bj = sBeta[j];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    sM1[i * P64 + j] = (T)(i > j ? (dXv[r] + ej * dXw[r]) * bj : 0.f);
-                }
-            }
-        }
-        // dv = beta (A^T du);  d(e^gam k) = beta (A^T dw): into dk, dbeta, dgam
-        f32x4 dk[NA][4];
-        {
-            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
-            float ej[4], bj[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
-                ej[t] = __expf(sGam[16 * t + c16]);
-                bj[t] = sBeta[16 * t + c16];
-            }
-#pragma unroll
-            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
-                const int n16 = 16 * (2 * w + a2);
-                V8 fdv[2];
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    f32x4 av = ZERO4;
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
-                        av = Mma<T>::run(fdv[s], fA[t][s], av);
-                    }
-                    const int j = 16 * t + c16;
-                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
-                    float dbv = 0.f;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
-                    dbv = sum_over_g(dbv);
-                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
-                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
-                }
-            }
-#pragma unroll
-            for (int a2 = 0; a2 < NA; ++a2) {                   // key features feat(a2) ..
-                const int n16 = feat(a2);
-                V8 fdw[2];
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    f32x4 ak = ZERO4;
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) {
-                        if (32 * s + 31 < 16 * t) continue;
-                        ak = Mma<T>::run(fdw[s], fA[t][s], ak);
-                    }
-                    const int j = 16 * t + c16;
-                    const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
-                    float dot = 0.f;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
-                    dot = sum_over_g(dot);
-                    if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
-                    dk[a2][t] = ak * (bj[t] * ej[t]);
-                }
-            }
-        }
-        lds_barrier();
-        // Y = dA A^T
-        {
-            V8 fd[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                f32x4 acc = ZERO4;
-#pragma unroll
-                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
-                const int l = 16 * tl + c16;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
-            }
-        }
-        lds_barrier();
-        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
-        {
-            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
-            V8 fAt[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                f32x4 acc = ZERO4;
-                if (tl <= w) {
-#pragma unroll
-                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
-                }
-                const f32x4 kk = kkT[tl];
-                const int l = 16 * tl + c16;
-                const float gl = sGam[l];
-                float colF = 0.f;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 16 * w + 4 * g + r;
-                    float E = 0.f;
-                    if (i > l) {
-                        const float d = __expf(gi[r] - gl), dL = -acc[r];
-                        dbi[r] += dL * kk[r] * d;
-                        E = dL * bi[r] * d;
-                        const float F = E * kk[r];
-                        rowF[r] += F;
-                        colF += F;
-                    }
-                    sM1[i * P64 + l] = (T)E;
-                }
-                colF = sum_over_g(colF);
-                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
-                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
-            }
-        }
-        lds_barrier();
-        // dk += E k + E^T k, on top of what the previous kernel left
-        {
-            V8 fk[NA][2];
-#pragma unroll
-            for (int a2 = 0; a2 < NA; ++a2)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
-                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
-#pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
-                    }
-                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
-                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
-#pragma unroll
-                        for (int a2 = 0; a2 < NA; ++a2) dk[a2][t] = Mma<T>::run(fk[a2][s], e, dk[a2][t]);
-                    }
-                }
-                const int x = 16 * t + c16;
-                if (x < c.valid) {
-#pragma unroll
-                    for (int a2 = 0; a2 < NA; ++a2) {
-                        f32x4 acc = dk[a2][t];
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
-                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + feat(a2) + 4 * g) = pack4<T>(acc);
-                    }
-                }
-            }
-        }
-        if (w == 0) {
-            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const float y = __shfl_down(x, off, 64);
-                if (lane + off < 64) x += y;
-            }
-            if (lane < c.valid) {
-                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
-                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
-            }
-        }
-        lds_barrier();
-    }
-}
-
-// The same kernel for one block of key features in at most 76 KB of LDS, so that two workgroups share a CU: the unit is walked
+// Workgroups walk over the units (chunk, v-head), the next unit's tiles on their way into registers meanwhile: dX = tril(dw (e^gam k)^T
+// + du v^T), dA = stril(dX diag(beta)); dv = beta (A^T du); d(e^gam k) = beta (A^T dw), into dk, dbeta, dgam; Y = dA A^T,
+// dL = -stril(A^T Y), E = diag(beta) dL o D; dk += E k + E^T k; dbeta, dgam from L = diag(beta) stril(k k^T o D); dg = the reverse
+// cumulative sum of dgam inside the chunk.  sDg, sDb [4][64]: a row per wave, added up in a fixed order at the end - the same
+// bits every run.
+// One block of key features in at most 76 KB of LDS, so that two workgroups share a CU: the unit is walked
 // in two halves over the same two tile places - first dv_new and v (dX's first term, dv and its share of dbeta), then dw and k
 // (dX's second term, k k^T, the first part of dk; comba: with the rows of p in a third place) - with the second set on its way
 // into registers during the first half and the next unit's first pair during the second; Y = dA A^T takes dw's place once dw is done with.
@@ -1634,6 +1364,320 @@ __global__ __launch_bounds__(256, 2) void gdn_bwd_wy2_kernel(BwdParams p, int64_
     }
 }
 
+// The same in two halves for two blocks of key features, still two workgroups per CU: the second half takes dw and k one block of
+// 128 features at a time through the same two tile places (the products with dw and k add up over the blocks; d(e^gam k) of a
+// block needs that block only), and the last step goes over the blocks again, k's first block fetched a second time.
+constexpr size_t BWD_WY2W_SMEM = (2 * 64 * P128 + 2 * 64 * P64) * 2 + 640 * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_wy2w_kernel(BwdParams p, int64_t units) {
+    static_assert(2 * BWD_WY2W_SMEM <= 160 * 1024, "two workgroups per CU");
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    constexpr int KD = 2 * BD, PK = P128, NA = 2;
+    extern __shared__ __align__(16) char smem[];
+    T* sX0 = (T*)smem; T* sX1 = sX0 + 64 * P128;               // dv_new | v, then a block of dw | k
+    T* sA = sX1 + 64 * P128; T* sM1 = sA + 64 * P64;
+    float* sGam = (float*)(sM1 + 64 * P64); float* sBeta = sGam + 64; float* sDg = sBeta + 64; float* sDb = sDg + 256;
+    T* sDvn = sX0; T* sV = sX1; T* sDW = sX0; T* sK = sX1; T* sM2 = sX0;
+
+    TileRegs<BD> rDvn, rV, rDW, rK;
+    TileRegs<CH> rA;
+    float rGam = 0.f, rDg = 0.f;
+    uint32_t rBeta = 0;                                          // (raw bits: converted when the unit's turn comes)
+    auto fetch_first = [&](int64_t u, int tid) {
+        const UnitAt at = unit_at(p, u);
+        const ChunkAt c = at.c;
+        fetch_tile<BD>(rDvn, (const T*)p.ws.dVn + u * 64 * BD, BD, 64, tid);
+        fetch_tile<BD>(rV, (const T*)p.v + (c.tok0 * p.HV + at.hv) * BD, (int64_t)p.HV * BD, c.valid, tid);
+        fetch_tile<CH>(rA, (const T*)p.ws.Am + u * 64 * 64, 64, 64, tid);
+        if (tid < 64) {
+            rGam = p.ws.Gam[u * 64 + tid];
+            rBeta = tid < c.valid ? load_scalar_bits(p.beta, (c.tok0 + tid) * p.HV + at.hv, p.gb_dtype) : 0;
+            rDg = p.ws.Dgam[u * 64 + tid];
+        }
+    };
+    fetch_first(blockIdx.x, threadIdx.x);
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
+        int tid_opaque = threadIdx.x;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        auto feat = [&](int a) { return 16 * (2 * w + a); };    // first key feature, inside a block, of this wave's tile a
+        const UnitAt at = unit_at(p, u);
+        const int hv = at.hv, hq = at.hq;
+        const ChunkAt c = at.c;
+        auto fetch_dw = [&](int kb) { fetch_tile<BD>(rDW, (const T*)p.ws.dWm + u * 64 * KD + BD * kb, KD, 64, tid); };
+        auto fetch_k = [&](int kb) { fetch_tile<BD>(rK, (const T*)p.k + (c.tok0 * p.H + hq) * KD + BD * kb, (int64_t)p.H * KD, c.valid, tid); };
+        put_tile<BD>(sDvn, P128, rDvn, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        put_tile<CH>(sA, P64, rA, tid);
+        if (tid < 64) { sGam[tid] = rGam; sBeta[tid] = scalar_of_bits(rBeta, p.gb_dtype); }
+        sDg[tid] = tid < 64 ? rDg : 0.f;
+        sDb[tid] = 0.f;
+        fetch_dw(0);
+        fetch_k(0);
+        lds_barrier();
+
+        // ---- first half: dX's first term du v^T (this wave's 16 rows i; lane: column j, rows 4g + r), and dv = beta (A^T du) ----
+        f32x4 dXv[4];
+        {
+            V8 fa[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) fa[s] = frag_rows(sDvn, P128, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                dXv[tj] = ZERO4;
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) dXv[tj] = Mma<T>::run(fa[s], frag_rows(sV, P128, 16 * tj, 32 * s, lane), dXv[tj]);
+                }
+            }
+        }
+        {
+            V8 fA[4][2];                                        // A^T operand of token tile t, step s (zero where A is)
+            float bj[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                bj[t] = sBeta[16 * t + c16];
+            }
+#pragma unroll
+            for (int a2 = 0; a2 < 2; ++a2) {                    // value columns 16(2w+a2) ..
+                const int n16 = 16 * (2 * w + a2);
+                V8 fdv[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fdv[s] = frag_cols(sDvn, P128, 32 * s, n16, lane);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    f32x4 av = ZERO4;
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        if (32 * s + 31 < 16 * t) continue;     // A[i][j] = 0 for i < j
+                        av = Mma<T>::run(fdv[s], fA[t][s], av);
+                    }
+                    const int j = 16 * t + c16;
+                    const V4 v4 = *(const V4*)(sV + j * P128 + n16 + 4 * g);
+                    float dbv = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dbv += av[r] * (float)v4[r];
+                    dbv = sum_over_g(dbv);
+                    if (g == 0) atomicAdd(&sDb[64 * w + j], dbv);
+                    if (j < c.valid) *(V4*)((T*)p.dv + ((c.tok0 + j) * p.HV + hv) * BD + n16 + 4 * g) = pack4<T>(av * bj[t]);
+                }
+            }
+        }
+
+        // ---- second half, a block of key features at a time: dX's second term dw (e^gam k)^T and k k^T add up over the blocks;
+        // d(e^gam k) = beta (A^T dw) of a block goes into that block's dk, and into dbeta, dgam ----
+        f32x4 dXw[4], kkT[4], dk[2][NA][4];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) dXw[tj] = kkT[tj] = ZERO4;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            lds_barrier();                                      // (the two tile places are done with)
+            put_tile<BD>(sDW, PK, rDW, tid);
+            put_tile<BD>(sK, PK, rK, tid);
+            lds_barrier();
+            if (kb == 0) { fetch_dw(1); fetch_k(1); }
+            else {
+                if (u + gridDim.x < units) fetch_first(u + gridDim.x, tid);
+                fetch_k(0);                                     // (for the last step)
+            }
+            {
+                V8 fw[4], fk[4];
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    fw[s] = frag_rows(sDW, PK, 16 * w, 32 * s, lane);
+                    fk[s] = frag_rows(sK, PK, 16 * w, 32 * s, lane);
+                }
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj) {
+                    if (tj <= w) {
+#pragma unroll
+                        for (int s = 0; s < 4; ++s) {
+                            const V8 bk = frag_rows(sK, PK, 16 * tj, 32 * s, lane);
+                            dXw[tj] = Mma<T>::run(fw[s], bk, dXw[tj]);
+                            kkT[tj] = Mma<T>::run(fk[s], bk, kkT[tj]);
+                        }
+                    }
+                }
+            }
+            {
+                V8 fA[4][2];
+                float ej[4], bj[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s)
+                        if (32 * s + 31 >= 16 * t) fA[t][s] = frag_cols(sA, P64, 32 * s, 16 * t, lane);
+                    ej[t] = __expf(sGam[16 * t + c16]);
+                    bj[t] = sBeta[16 * t + c16];
+                }
+#pragma unroll
+                for (int a2 = 0; a2 < NA; ++a2) {               // key features 128 kb + feat(a2) ..
+                    const int n16 = feat(a2);
+                    V8 fdw[2];
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) fdw[s] = frag_cols(sDW, PK, 32 * s, n16, lane);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        f32x4 ak = ZERO4;
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {
+                            if (32 * s + 31 < 16 * t) continue;
+                            ak = Mma<T>::run(fdw[s], fA[t][s], ak);
+                        }
+                        const int j = 16 * t + c16;
+                        const V4 k4 = *(const V4*)(sK + j * PK + n16 + 4 * g);
+                        float dot = 0.f;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) dot += ak[r] * (float)k4[r];
+                        dot = sum_over_g(dot);
+                        if (g == 0) { atomicAdd(&sDb[64 * w + j], ej[t] * dot); atomicAdd(&sDg[64 * w + j], bj[t] * ej[t] * dot); }
+                        dk[kb][a2][t] = ak * (bj[t] * ej[t]);
+                    }
+                }
+            }
+        }
+        // dA = stril(dX diag(beta))
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            const int j = 16 * tj + c16;
+            const float ej = __expf(sGam[j]), bj = sBeta[j];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * w + 4 * g + r;
+                sM1[i * P64 + j] = (T)(i > j ? (dXv[tj][r] + ej * dXw[tj][r]) * bj : 0.f);
+            }
+        }
+        lds_barrier();
+        // Y = dA A^T  (into dw's place)
+        {
+            V8 fd[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fd[s] = frag_rows(sM1, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fd[s], frag_rows(sA, P64, 16 * tl, 32 * s, lane), acc);
+                const int l = 16 * tl + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sM2[(16 * w + 4 * g + r) * P64 + l] = (T)acc[r];
+            }
+        }
+        lds_barrier();
+        // dL = -stril(A^T Y);  E = diag(beta) dL o D as an operand tile;  dbeta, dgam from L = diag(beta) stril(k k^T o D)
+        {
+            float dbi[4] = {0.f, 0.f, 0.f, 0.f}, rowF[4] = {0.f, 0.f, 0.f, 0.f}, gi[4], bi[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { gi[r] = sGam[16 * w + 4 * g + r]; bi[r] = sBeta[16 * w + 4 * g + r]; }
+            V8 fAt[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fAt[s] = frag_cols(sA, P64, 32 * s, 16 * w, lane);
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 acc = ZERO4;
+                if (tl <= w) {
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) acc = Mma<T>::run(fAt[s], frag_cols(sM2, P64, 32 * s, 16 * tl, lane), acc);
+                }
+                const f32x4 kk = kkT[tl];
+                const int l = 16 * tl + c16;
+                const float gl = sGam[l];
+                float colF = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    float E = 0.f;
+                    if (i > l) {
+                        const float d = __expf(gi[r] - gl), dL = -acc[r];
+                        dbi[r] += dL * kk[r] * d;
+                        E = dL * bi[r] * d;
+                        const float F = E * kk[r];
+                        rowF[r] += F;
+                        colF += F;
+                    }
+                    sM1[i * P64 + l] = (T)E;
+                }
+                colF = sum_over_g(colF);
+                if (g == 0 && tl <= w) atomicAdd(&sDg[64 * w + l], -colF);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float a = sum_over_c16(dbi[r]), b = sum_over_c16(rowF[r]);
+                if (c16 == 0) { atomicAdd(&sDb[64 * w + 16 * w + 4 * g + r], a); atomicAdd(&sDg[64 * w + 16 * w + 4 * g + r], b); }
+            }
+        }
+        // dk += E k + E^T k, on top of what the previous kernel left: the second block (its rows of k are in place), then the first
+#pragma unroll
+        for (int kb = 1; kb >= 0; --kb) {
+            V4 dk_old[NA][4];
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int x = 16 * t + c16;
+                    dk_old[a2][t] = V4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+                    if (x < c.valid) dk_old[a2][t] = *(const V4*)((const T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + BD * kb + feat(a2) + 4 * g);
+                }
+            lds_barrier();                                      // (E is complete; second round: the second block's rows are done with)
+            if (kb == 0) {
+                put_tile<BD>(sK, PK, rK, tid);
+                lds_barrier();
+            }
+            V8 fk[NA][2];
+#pragma unroll
+            for (int a2 = 0; a2 < NA; ++a2)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) fk[a2][s] = frag_cols(sK, PK, 32 * s, feat(a2), lane);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (32 * s <= 16 * t + 15) {                // E[i][l], l < i
+                        const V8 e = frag_rows(sM1, P64, 16 * t, 32 * s, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[kb][a2][t] = Mma<T>::run(fk[a2][s], e, dk[kb][a2][t]);
+                    }
+                    if (32 * s + 31 >= 16 * t) {                // E[i][l], i > l
+                        const V8 e = frag_cols(sM1, P64, 32 * s, 16 * t, lane);
+#pragma unroll
+                        for (int a2 = 0; a2 < NA; ++a2) dk[kb][a2][t] = Mma<T>::run(fk[a2][s], e, dk[kb][a2][t]);
+                    }
+                }
+                const int x = 16 * t + c16;
+                if (x < c.valid) {
+#pragma unroll
+                    for (int a2 = 0; a2 < NA; ++a2) {
+                        f32x4 acc = dk[kb][a2][t];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[r] += (float)dk_old[a2][t][r];
+                        *(V4*)((T*)p.dk + ((c.tok0 + x) * p.HV + hv) * KD + BD * kb + feat(a2) + 4 * g) = pack4<T>(acc);
+                    }
+                }
+            }
+        }
+        if (w == 0) {
+            float x = (sDg[lane] + sDg[64 + lane]) + (sDg[128 + lane] + sDg[192 + lane]);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_down(x, off, 64);
+                if (lane + off < 64) x += y;
+            }
+            if (lane < c.valid) {
+                p.dg[(c.tok0 + lane) * p.HV + hv] = x;
+                p.dbeta[(c.tok0 + lane) * p.HV + hv] = (sDb[lane] + sDb[64 + lane]) + (sDb[128 + lane] + sDb[192 + lane]);
+            }
+        }
+        lds_barrier();
+    }
+}
+
 template <typename T, int KT, bool COMBA = false>
 static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t stream) {
     BwdParams p = p_in;
@@ -1705,7 +1749,7 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
     const bool l2 = KT == 1 && p.q_raw;                     // (the entry has checked H == HV)
     K wy;
     if constexpr (KT == 1) wy = {l2 ? (const void*)gdn_bwd_wy2_kernel<T, true, COMBA> : (const void*)gdn_bwd_wy2_kernel<T, false, COMBA>, bwd_wy2_smem<COMBA>(), "gdn_bwd_wy2_kernel", units < 512u ? units : 512u};
-    else wy = {(const void*)gdn_bwd_wy_kernel<T, KT>, bwd_wy_smem<KT>(), "gdn_bwd_wy_kernel", units < 256u ? units : 256u};
+    else wy = {(const void*)gdn_bwd_wy2w_kernel<T>, BWD_WY2W_SMEM, "gdn_bwd_wy2w_kernel", units < 512u ? units : 512u};
     const K ks[5] = {
         {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, COMBA && KT == 1, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
         state,
