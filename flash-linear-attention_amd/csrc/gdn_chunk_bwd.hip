@@ -138,8 +138,8 @@ __device__ __forceinline__ int64_t pad_steps_of(const ScanPlan& sp) { return (sp
 // ---------------------------------------------------------------------------------------------
 // (comba: a third tile of rows, those of p; the matrix L then takes the place of the q tile once q has been used, which keeps a
 // workgroup at 80 KB: two per CU)
-template <int KT, bool COMBA = false> constexpr size_t bwd_prep_smem() {
-    return ((2 + (COMBA ? 1 : 0)) * 64 * (BD * KT + 8) + 64 * P128 + 64 * P64) * 2 + ((COMBA ? 0 : 64 * PL) + 192) * 4;
+template <bool COMBA = false> constexpr size_t bwd_prep_smem() {
+    return ((2 + (COMBA ? 1 : 0)) * 64 * P128 + 64 * P128 + 64 * P64) * 2 + ((COMBA ? 0 : 64 * PL) + 192) * 4;
 }
 
 // Rows of a tile on their way from memory to LDS (a row: 16 lanes next to each other, 8 features each) divided by their
@@ -168,11 +168,11 @@ __device__ __forceinline__ void l2norm_tile_rows(TileRegs<BD>& r, T* out, float*
     }
 }
 
-template <typename T, int KT, bool COMBA = false, bool L2 = false>
-__global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
+template <typename T, bool COMBA = false, bool L2 = false>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare_kernel(BwdParams p, int64_t units) {
     typedef typename Mma<T>::V8 V8;
     typedef typename Mma<T>::V4 V4;
-    constexpr int KD = BD * KT, PK = KD + 8;
+    constexpr int KT = 1, KD = BD * KT, PK = KD + 8;             // (one block of key features; two: gdn_bwd_prepare2w_kernel)
     extern __shared__ __align__(16) char smem[];
     T* sK = (T*)smem; T* sQ = sK + 64 * PK; T* sV = sQ + 64 * PK; T* sA = sV + 64 * P128;
     T* sP = sA + 64 * P64;                                       // (comba) rows of the second key
@@ -208,7 +208,6 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
         asm volatile("" : "+v"(tid_opaque));
         const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
         if constexpr (L2) {
-            static_assert(!L2 || KT == 1, "one block of key features");
             const UnitAt at = unit_at(p, u);
             const int hv = at.hv;                      // (== the q/k head)
             const ChunkAt c = at.c;
@@ -327,6 +326,180 @@ __global__ __launch_bounds__(256, KT == 1 ? 2 : 1) void gdn_bwd_prepare_kernel(B
                 for (int s = 0; s < 2; ++s) {
                     if (2 * s > w) continue;                    // A is lower triangular
                     aw = Mma<T>::run(frag_cols(sRows, PK, 32 * s, 16 * n, lane), fa[s], aw);
+                }
+                *(V4*)(Wu + i * KD + 16 * n + 4 * g) = pack4<T>(aw);
+            }
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                f32x4 au = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (2 * s > w) continue;
+                    au = Mma<T>::run(frag_cols(sV, P128, 32 * s, 16 * n, lane), fa[s], au);
+                }
+                *(V4*)(Uu + i * BD + 16 * n + 4 * g) = pack4<T>(au);
+            }
+        }
+        lds_barrier();
+    }
+}
+
+// Two blocks of key features in 80 KB, two workgroups per CU: k and q pass through two tile places a block of 128 features at a
+// time (k k^T and q k^T add up over the blocks in registers); for w = A (beta e^gam k), which needs every block of k again, the
+// second block is still in place and the first is fetched a second time, into q's place.
+constexpr size_t BWD_PREP2W_SMEM = (3 * 64 * P128 + 64 * P64) * 2 + (64 * PL + 192) * 4;
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gdn_bwd_prepare2w_kernel(BwdParams p, int64_t units) {
+    static_assert(2 * BWD_PREP2W_SMEM <= 160 * 1024, "two workgroups per CU");
+    typedef typename Mma<T>::V8 V8;
+    typedef typename Mma<T>::V4 V4;
+    constexpr int KD = 2 * BD;
+    extern __shared__ __align__(16) char smem[];
+    T* sK = (T*)smem; T* sQ = sK + 64 * P128; T* sV = sQ + 64 * P128; T* sA = sV + 64 * P128;
+    float* sL = (float*)(sA + 64 * P64);
+    float* sGam = sL + 64 * PL; float* sBeta = sGam + 64;
+    T* sK0 = sQ;                                                 // k's first block, once q is done with
+
+    TileRegs<BD> rK, rQ, rV;
+    uint32_t rG = 0, rB = 0;                                     // (raw bits: converted when the unit's turn comes)
+    auto fetch_k = [&](const UnitAt& at, int kb, int tid) {
+        fetch_tile<BD>(rK, (const T*)p.k + (at.c.tok0 * p.H + at.hq) * KD + BD * kb, (int64_t)p.H * KD, at.c.valid, tid);
+    };
+    auto fetch_q = [&](const UnitAt& at, int kb, int tid) {
+        fetch_tile<BD>(rQ, (const T*)p.q + (at.c.tok0 * p.H + at.hq) * KD + BD * kb, (int64_t)p.H * KD, at.c.valid, tid);
+    };
+    auto fetch_rest = [&](const UnitAt& at, int tid) {           // v and the two scalars per token
+        fetch_tile<BD>(rV, (const T*)p.v + (at.c.tok0 * p.HV + at.hv) * BD, (int64_t)p.HV * BD, at.c.valid, tid);
+        rG = rB = 0;
+        if (tid < at.c.valid) {                                  // (wave 0)
+            rG = p.g ? load_scalar_bits(p.g, (at.c.tok0 + tid) * p.HV + at.hv, p.gb_dtype) : 0;
+            rB = load_scalar_bits(p.beta, (at.c.tok0 + tid) * p.HV + at.hv, p.gb_dtype);
+        }
+    };
+    {
+        const UnitAt at = unit_at(p, blockIdx.x);
+        fetch_k(at, 0, threadIdx.x); fetch_q(at, 0, threadIdx.x); fetch_rest(at, threadIdx.x);
+    }
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        // (everything derived from the lane number is derived again per unit from a copy the compiler cannot see through:
+        // hoisted out of this loop, the addresses of its unrolled body would sit in registers, or spill, for its whole length)
+        int tid_opaque = threadIdx.x;
+        asm volatile("" : "+v"(tid_opaque));
+        const int tid = tid_opaque, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6), c16 = lane & 15, g = lane >> 4;
+        const UnitAt at = unit_at(p, u);
+        const bool more = u + gridDim.x < units;
+        const UnitAt nx = unit_at(p, more ? u + gridDim.x : u);
+        put_tile<BD>(sK, P128, rK, tid);
+        put_tile<BD>(sQ, P128, rQ, tid);
+        put_tile<BD>(sV, P128, rV, tid);
+        if (w == 0) {
+            float x = scalar_of_bits(rG, p.gb_dtype);
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const float y = __shfl_up(x, off, 64);
+                if (lane >= off) x += y;
+            }
+            sGam[lane] = x; sBeta[lane] = scalar_of_bits(rB, p.gb_dtype);
+            p.ws.Gam[u * 64 + lane] = x;
+        }
+        lds_barrier();
+        fetch_k(at, 1, tid); fetch_q(at, 1, tid);
+
+        // strip of 16 token rows per wave: k k^T and q k^T, a block of features at a time
+        f32x4 kk[4], qk[4];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) kk[tj] = qk[tj] = ZERO4;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            if (kb == 1) {
+                lds_barrier();                                  // (the first block is done with)
+                put_tile<BD>(sK, P128, rK, tid);
+                put_tile<BD>(sQ, P128, rQ, tid);
+                lds_barrier();
+                fetch_k(at, 0, tid);                            // (again, for w)
+                if (more) { fetch_q(nx, 0, tid); fetch_rest(nx, tid); }
+            }
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                if (tj <= w) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const V8 b = frag_rows(sK, P128, 16 * tj, 32 * s, lane);
+                        kk[tj] = Mma<T>::run(frag_rows(sK, P128, 16 * w, 32 * s, lane), b, kk[tj]);
+                        qk[tj] = Mma<T>::run(frag_rows(sQ, P128, 16 * w, 32 * s, lane), b, qk[tj]);
+                    }
+                }
+            }
+        }
+        // L (fp32, for the substitution; entry (i, j) at [i][j % 4][j / 4]) and P^T
+        {
+            T* PTu = (T*)p.ws.PT + u * 64 * 64;
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                const int j = 16 * tj + c16;
+                const float gj = sGam[j];
+                f32x4 pt;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * w + 4 * g + r;
+                    const float d = i >= j ? __expf(sGam[i] - gj) : 0.f;
+                    if (tj <= w) sL[i * PL + (j & 3) * 16 + (j >> 2)] = i > j ? sBeta[i] * kk[tj][r] * d : 0.f;
+                    pt[r] = p.scale * qk[tj][r] * d;
+                }
+                *(V4*)(PTu + j * 64 + 16 * w + 4 * g) = pack4<T>(pt);
+            }
+        }
+        lds_barrier();
+        // k -> beta e^gam k, v -> beta v: the second block of k and v in place, the first block of k on its way into q's place
+        {
+            const int row0 = tid >> 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float f = sBeta[row0 + 16 * i] * __expf(sGam[row0 + 16 * i]);
+                V8 x = __builtin_bit_cast(V8, rK.x[i]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
+                rK.x[i] = __builtin_bit_cast(u32x4, x);
+            }
+            put_tile<BD>(sK0, P128, rK, tid);
+            if (more) fetch_k(nx, 0, tid);
+        }
+        for (int idx = tid; idx < 64 * 32; idx += 256) {
+            const int row = idx >> 5, pc = idx & 31;            // the row's pieces of k's second block, then those of v
+            T* at2 = pc < 16 ? sK + row * P128 + pc * 8 : sV + row * P128 + (pc - 16) * 8;
+            const float f = pc < 16 ? sBeta[row] * __expf(sGam[row]) : sBeta[row];
+            V8 x = *(V8*)at2;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * f);
+            *(V8*)at2 = x;
+        }
+        solve_unit_lower_blocks<T>(sL, (float*)sA, sA, w, lane);
+        lds_barrier();
+        {
+            T* Au = (T*)p.ws.Am + u * 64 * 64;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int idx = tid + 256 * i, row = idx >> 3, pc = idx & 7;
+                *(u32x4*)(Au + row * 64 + pc * 8) = *(const u32x4*)(sA + row * P64 + pc * 8);
+            }
+        }
+        // w^T and u^T tiles: features on the rows, this wave's 16 tokens on the columns
+        {
+            T* Wu = (T*)p.ws.Wm + u * 64 * KD;
+            T* Uu = (T*)p.ws.Um + u * 64 * BD;
+            const int i = 16 * w + c16;
+            V8 fa[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fa[s] = frag_rows(sA, P64, 16 * w, 32 * s, lane);
+#pragma unroll
+            for (int n = 0; n < 16; ++n) {
+                const T* src = n < 8 ? sK0 : sK;
+                f32x4 aw = ZERO4;
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    if (2 * s > w) continue;                    // A is lower triangular
+                    aw = Mma<T>::run(frag_cols(src, P128, 32 * s, 16 * (n & 7), lane), fa[s], aw);
                 }
                 *(V4*)(Wu + i * KD + 16 * n + 4 * g) = pack4<T>(aw);
             }
@@ -1747,11 +1920,14 @@ static int launch_bwd(const BwdParams& p_in, int64_t num_chunks, hipStream_t str
         }
     }
     const bool l2 = KT == 1 && p.q_raw;                     // (the entry has checked H == HV)
+    K prep;
+    if constexpr (KT == 1) prep = {l2 ? (const void*)gdn_bwd_prepare_kernel<T, COMBA, true> : (const void*)gdn_bwd_prepare_kernel<T, COMBA>, bwd_prep_smem<COMBA>(), "gdn_bwd_prepare_kernel", units < 512u ? units : 512u};
+    else prep = {(const void*)gdn_bwd_prepare2w_kernel<T>, BWD_PREP2W_SMEM, "gdn_bwd_prepare2w_kernel", units < 512u ? units : 512u};
     K wy;
     if constexpr (KT == 1) wy = {l2 ? (const void*)gdn_bwd_wy2_kernel<T, true, COMBA> : (const void*)gdn_bwd_wy2_kernel<T, false, COMBA>, bwd_wy2_smem<COMBA>(), "gdn_bwd_wy2_kernel", units < 512u ? units : 512u};
     else wy = {(const void*)gdn_bwd_wy2w_kernel<T>, BWD_WY2W_SMEM, "gdn_bwd_wy2w_kernel", units < 512u ? units : 512u};
     const K ks[5] = {
-        {l2 ? (const void*)gdn_bwd_prepare_kernel<T, 1, COMBA && KT == 1, true> : (const void*)gdn_bwd_prepare_kernel<T, KT, COMBA>, bwd_prep_smem<KT, COMBA>(), "gdn_bwd_prepare_kernel", units < (KT == 1 ? 512u : 256u) ? units : (KT == 1 ? 512u : 256u)},
+        prep,
         state,
         dstate,
         {l2 ? (const void*)gdn_bwd_dqkw_kernel<T, 1, true> : (const void*)gdn_bwd_dqkw_kernel<T, KT>, bwd_dqkw_smem<KT>(), "gdn_bwd_dqkw_kernel", units < 256u ? units : 256u},
